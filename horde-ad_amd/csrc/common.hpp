@@ -1,0 +1,189 @@
+// Shared host-side definitions of the gfx950 backend: context, buffer, array
+// view, dimension collapsing and launch helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "hordead_gpu.h"
+
+// Largest number of dimensions a kernel sees after adjacent dimensions that
+// are contiguous in every operand have been merged.
+#define HG_KDIMS 10
+
+struct hgpu_buffer {
+  hgpu_ctx* ctx;
+  void* ptr;
+  size_t bytes;      // size of the block handed out by the allocator
+  std::atomic<int> refs;
+};
+
+struct hgpu_array {
+  hgpu_ctx* ctx;
+  std::atomic<int> refs;
+  hgpu_buffer* buf;  // nullptr for zero-size arrays
+  int dtype;
+  int rank;
+  int64_t shape[HGPU_MAX_RANK];
+  int64_t strides[HGPU_MAX_RANK];  // in elements
+  int64_t offset;                  // in elements, from buf->ptr
+};
+
+struct hgpu_ctx {
+  int device;
+  hipStream_t stream;
+  std::mutex mu;                 // guards allocator state and `err`
+  std::multimap<size_t, void*> cache;
+  uint64_t in_use = 0, reserved = 0, n_device_allocs = 0;
+  int64_t fail_after = -1;
+  std::string err;
+  void* staging = nullptr;       // pinned host staging block
+  size_t staging_bytes = 0;
+  std::mutex launch_mu;          // serialises enqueue order across host threads
+  int num_cu = 256;
+  // JIT cache of fused elementwise kernels, keyed by generated source.
+  std::map<std::string, void*> jit_cache;
+};
+
+namespace hg {
+
+inline size_t dtype_size(int dt) {
+  switch (dt) {
+    case HGPU_F64: case HGPU_I64: return 8;
+    case HGPU_F32: case HGPU_I32: return 4;
+    case HGPU_I16: return 2;
+    case HGPU_I8: case HGPU_BOOL: return 1;
+  }
+  return 0;
+}
+inline bool dtype_is_float(int dt) { return dt == HGPU_F64 || dt == HGPU_F32; }
+inline bool dtype_is_int(int dt) { return dt >= HGPU_I64 && dt <= HGPU_I8; }
+
+int fail(hgpu_ctx* ctx, int code, const char* fmt, ...);
+int check_hip(hgpu_ctx* ctx, hipError_t e, const char* what);
+
+// Allocator (runtime.hip).
+int buffer_alloc(hgpu_ctx* ctx, size_t bytes, hgpu_buffer** out);
+void buffer_retain(hgpu_buffer* b);
+void buffer_release(hgpu_buffer* b);
+
+// Array construction helpers (runtime.hip).
+hgpu_array* new_view(hgpu_ctx* ctx, hgpu_buffer* buf, int dtype, int rank, const int64_t* shape,
+                     const int64_t* strides, int64_t offset);
+int new_dense(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, hgpu_array** out);
+int new_zeros(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, hgpu_array** out);
+inline int64_t nelem(const hgpu_array* a) {
+  int64_t n = 1;
+  for (int i = 0; i < a->rank; ++i) n *= a->shape[i];
+  return n;
+}
+inline void* data_ptr(const hgpu_array* a) {
+  if (!a->buf) return nullptr;
+  return (char*)a->buf->ptr + a->offset * (int64_t)dtype_size(a->dtype);
+}
+bool is_dense(const hgpu_array* a);
+bool same_shape(const hgpu_array* a, const hgpu_array* b);
+
+// Up to four operands viewed over one iteration space.  `nd` dimensions of
+// extent `shape`, operand k advancing by `st[k][d]` elements along dim d.
+struct Dims {
+  int nd;
+  int64_t shape[HG_KDIMS];
+  int64_t st[4][HG_KDIMS];
+};
+
+// Builds the merged iteration space of `nops` operands that share `shape`.
+// Size-1 dims vanish; adjacent dims merge when every operand's strides allow.
+// Returns false when more than HG_KDIMS dims remain.
+bool collapse(int rank, const int64_t* shape, int nops, const int64_t* const* strides, Dims* out);
+
+inline void dense_strides(int rank, const int64_t* shape, int64_t* st) {
+  int64_t s = 1;
+  for (int i = rank - 1; i >= 0; --i) { st[i] = s; s *= shape[i]; }
+}
+
+inline unsigned grid_for(int64_t n, int block, int max_blocks) {
+  int64_t g = (n + block - 1) / block;
+  if (g < 1) g = 1;
+  if (g > max_blocks) g = max_blocks;
+  return (unsigned)g;
+}
+
+// Zeroes `bytes` bytes (rounded up to 16) with a fill kernel (ewise.hip).
+int zero_fill(hgpu_ctx* ctx, void* p, size_t bytes);
+// Strided copy between two views of equal shape (ewise.hip).
+int copy_view(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const void* src,
+              const int64_t* sst, void* dst, const int64_t* dst_st);
+
+struct LaunchGuard {
+  hgpu_ctx* ctx;
+  explicit LaunchGuard(hgpu_ctx* c) : ctx(c) {
+    c->launch_mu.lock();
+    (void)hipSetDevice(c->device);
+  }
+  ~LaunchGuard() { ctx->launch_mu.unlock(); }
+};
+
+}  // namespace hg
+
+#define HG_DISPATCH_DTYPE(dt, T, ...)                                   \
+  switch (dt) {                                                         \
+    case HGPU_F64: { using T = double; __VA_ARGS__; break; }            \
+    case HGPU_F32: { using T = float; __VA_ARGS__; break; }             \
+    case HGPU_I64: { using T = int64_t; __VA_ARGS__; break; }           \
+    case HGPU_I32: { using T = int32_t; __VA_ARGS__; break; }           \
+    case HGPU_I16: { using T = int16_t; __VA_ARGS__; break; }           \
+    case HGPU_I8: { using T = int8_t; __VA_ARGS__; break; }             \
+    case HGPU_BOOL: { using T = uint8_t; __VA_ARGS__; break; }          \
+    default: break;                                                     \
+  }
+
+#define HG_CHECK_LAUNCH(ctx, what)                                      \
+  do {                                                                  \
+    hipError_t e__ = hipGetLastError();                                 \
+    if (e__ != hipSuccess) return hg::check_hip(ctx, e__, what);        \
+  } while (0)
+
+// Device-side decomposition of a linear index over a merged iteration space.
+#ifdef __HIPCC__
+namespace hg {
+template <int NOPS>
+__device__ __forceinline__ void decompose(const Dims& d, int64_t lin, int64_t* off) {
+#pragma unroll
+  for (int k = 0; k < NOPS; ++k) off[k] = 0;
+  if (lin < (int64_t)0x7fffffff) {
+    uint32_t r = (uint32_t)lin;
+    for (int i = d.nd - 1; i > 0; --i) {
+      uint32_t s = (uint32_t)d.shape[i];
+      uint32_t q = r / s;
+      uint32_t c = r - q * s;
+      r = q;
+#pragma unroll
+      for (int k = 0; k < NOPS; ++k) off[k] += (int64_t)c * d.st[k][i];
+    }
+#pragma unroll
+    for (int k = 0; k < NOPS; ++k) off[k] += (int64_t)r * d.st[k][0];
+  } else {
+    int64_t r = lin;
+    for (int i = d.nd - 1; i > 0; --i) {
+      int64_t s = d.shape[i];
+      int64_t q = r / s;
+      int64_t c = r - q * s;
+      r = q;
+#pragma unroll
+      for (int k = 0; k < NOPS; ++k) off[k] += c * d.st[k][i];
+    }
+#pragma unroll
+    for (int k = 0; k < NOPS; ++k) off[k] += r * d.st[k][0];
+  }
+}
+}  // namespace hg
+#endif

@@ -1,0 +1,309 @@
+// Reductions and contractions over strided views:
+//   out[o] = sum_r a[o,r] * b[o,r]
+// which, with free views, is horde-ad's tssum / tssumN / tssum0 / tsdot0 /
+// tsdot1In / tsmatvecmul / tsmatmul2 (src/HordeAd/Core/OpsConcrete.hs:215-242).
+//
+// This file holds the general path, bound by HBM bandwidth:
+//   * lane-per-output: adjacent lanes own adjacent outputs and walk the
+//     reduced index space with an odometer (coalesced when the kept innermost
+//     dimension has unit stride: sums over outer dimensions);
+//   * wave-per-output: the 64 lanes of a wavefront stride over the innermost
+//     reduced dimension and combine with a shuffle tree (coalesced when the
+//     reduced innermost dimension has unit stride: dot1In, sum0, dot0).
+// Long reductions with few outputs are split into S chunks whose partial sums
+// (double / int64 accumulators) are combined by a second launch, so the
+// summation order is fixed by the shape alone: results are reproducible from
+// run to run.  GEMM-shaped contractions are routed to the MFMA kernels first.
+#include "common.hpp"
+
+using namespace hg;
+
+namespace hg {
+// gemm.hip: returns HGPU_OK and sets *handled when the contraction was
+// recognised as a matrix product and executed on the matrix cores.
+int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled);
+}
+
+namespace {
+
+constexpr int kBlock = 256;
+
+template <typename T> struct acc_of { using type = int64_t; };
+template <> struct acc_of<double> { using type = double; };
+template <> struct acc_of<float> { using type = double; };
+
+template <typename A>
+__device__ __forceinline__ A wave_sum(A v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    if constexpr (sizeof(A) == 8) {
+      unsigned long long u = *reinterpret_cast<unsigned long long*>(&v);
+      unsigned lo = __shfl_down((unsigned)(u & 0xffffffffu), off, 64);
+      unsigned hi = __shfl_down((unsigned)(u >> 32), off, 64);
+      unsigned long long w = ((unsigned long long)hi << 32) | lo;
+      v += *reinterpret_cast<A*>(&w);
+    } else {
+      v += __shfl_down(v, off, 64);
+    }
+  }
+  return v;
+}
+
+// Work item = (output o, chunk s); s-th chunk covers reduced linear indices
+// [s*chunk, min(R, (s+1)*chunk)).  out is dense [n_out, S].
+template <typename TI, typename TO, bool HASB>
+__global__ void __launch_bounds__(kBlock) k_contract_lane(Dims keep, Dims red, int64_t n_out, int64_t R, int S, int64_t chunk,
+                                                           const TI* __restrict__ a, const TI* __restrict__ b, TO* __restrict__ out) {
+  using A = typename acc_of<TI>::type;
+  int64_t items = n_out * S;
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x; item < items; item += step) {
+    int64_t o = item % n_out, s = item / n_out;
+    int64_t ko[2];
+    decompose<2>(keep, o, ko);
+    int64_t r0 = s * chunk, r1 = r0 + chunk;
+    if (r1 > R) r1 = R;
+    // odometer over the reduced dims, started at r0
+    int64_t idx[HG_KDIMS];
+    int64_t oa = ko[0], ob = ko[1];
+    {
+      int64_t r = r0;
+      for (int i = red.nd - 1; i >= 0; --i) {
+        int64_t q = i > 0 ? r / red.shape[i] : 0;
+        int64_t c = i > 0 ? r - q * red.shape[i] : r;
+        idx[i] = c;
+        oa += c * red.st[0][i];
+        ob += c * red.st[1][i];
+        r = q;
+      }
+    }
+    A acc = 0;
+    const int last = red.nd - 1;
+    for (int64_t r = r0; r < r1; ++r) {
+      A x = (A)a[oa];
+      if (HASB) x *= (A)b[ob];
+      acc += x;
+      // advance
+      int i = last;
+      idx[i]++;
+      oa += red.st[0][i];
+      ob += red.st[1][i];
+      while (i > 0 && idx[i] == red.shape[i]) {
+        oa -= idx[i] * red.st[0][i];
+        ob -= idx[i] * red.st[1][i];
+        idx[i] = 0;
+        --i;
+        idx[i]++;
+        oa += red.st[0][i];
+        ob += red.st[1][i];
+      }
+    }
+    out[o * S + s] = (TO)acc;
+  }
+}
+
+// One wavefront per work item.  `red` has its innermost dim split off:
+// Lin = extent, (sa_in, sb_in) = strides; `red` keeps the outer reduced dims
+// with Q = their product.  Chunks split Q when Q > 1, else Lin.
+template <typename TI, typename TO, bool HASB>
+__global__ void __launch_bounds__(kBlock) k_contract_wave(Dims keep, Dims red, int64_t n_out, int64_t Q, int64_t Lin, int64_t sa_in, int64_t sb_in,
+                                                           int S, int64_t chunk, const TI* __restrict__ a, const TI* __restrict__ b, TO* __restrict__ out) {
+  using A = typename acc_of<TI>::type;
+  const int lane = threadIdx.x & 63;
+  int64_t wave = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+  int64_t nwaves = ((int64_t)gridDim.x * kBlock) >> 6;
+  int64_t items = n_out * S;
+  for (int64_t item = wave; item < items; item += nwaves) {
+    int64_t o = item / S;
+    int s = (int)(item - o * S);
+    int64_t ko[2];
+    decompose<2>(keep, o, ko);
+    int64_t q0 = 0, q1 = Q, j0 = 0, j1 = Lin;
+    if (Q > 1) { q0 = s * chunk; q1 = q0 + chunk; if (q1 > Q) q1 = Q; }
+    else { j0 = s * chunk; j1 = j0 + chunk; if (j1 > Lin) j1 = Lin; }
+    A acc = 0;
+    for (int64_t q = q0; q < q1; ++q) {
+      int64_t ro[2];
+      decompose<2>(red, q, ro);
+      const TI* pa = a + ko[0] + ro[0];
+      const TI* pb = HASB ? b + ko[1] + ro[1] : nullptr;
+      for (int64_t j = j0 + lane; j < j1; j += 64) {
+        A x = (A)pa[j * sa_in];
+        if (HASB) x *= (A)pb[j * sb_in];
+        acc += x;
+      }
+    }
+    acc = wave_sum<A>(acc);
+    if (lane == 0) out[item] = (TO)acc;
+  }
+}
+
+// First (want_max = 0: minimal, 1: maximal) element along the last dim.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_argminmax(Dims keep, int64_t n_out, int64_t L, int64_t sl, int want_max, const T* __restrict__ a, int64_t* __restrict__ out) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t o = (int64_t)blockIdx.x * kBlock + threadIdx.x; o < n_out; o += step) {
+    int64_t ko[1];
+    decompose<1>(keep, o, ko);
+    const T* p = a + ko[0];
+    T best = p[0];
+    int64_t bi = 0;
+    for (int64_t j = 1; j < L; ++j) {
+      T x = p[j * sl];
+      bool better = want_max ? (x > best) : (x < best);
+      if (better) { best = x; bi = j; }
+    }
+    out[o] = bi;
+  }
+}
+
+template <typename TI, typename TO>
+int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red_full, int64_t n_out, int64_t R, int S, const void* a, const void* b, void* out) {
+  LaunchGuard lg(ctx);
+  int maxb = ctx->num_cu * 8;
+  if (use_wave) {
+    Dims red = red_full;
+    int last = red.nd - 1;
+    int64_t Lin = red.shape[last], sa = red.st[0][last], sb = red.st[1][last];
+    int64_t Q = R / Lin;
+    if (red.nd > 1) { red.nd -= 1; } else { red.shape[0] = 1; red.st[0][0] = red.st[1][0] = 0; }
+    int64_t span = Q > 1 ? Q : Lin;
+    int64_t chunk = (span + S - 1) / S;
+    int64_t items = n_out * S;
+    unsigned g = grid_for(items * 64, kBlock, maxb);
+    if (b) hipLaunchKernelGGL((k_contract_wave<TI, TO, true>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red, n_out, Q, Lin, sa, sb, S, chunk, (const TI*)a, (const TI*)b, (TO*)out);
+    else hipLaunchKernelGGL((k_contract_wave<TI, TO, false>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red, n_out, Q, Lin, sa, sb, S, chunk, (const TI*)a, (const TI*)nullptr, (TO*)out);
+  } else {
+    int64_t chunk = (R + S - 1) / S;
+    unsigned g = grid_for(n_out * S, kBlock, maxb);
+    if (b) hipLaunchKernelGGL((k_contract_lane<TI, TO, true>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red_full, n_out, R, S, chunk, (const TI*)a, (const TI*)b, (TO*)out);
+    else hipLaunchKernelGGL((k_contract_lane<TI, TO, false>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red_full, n_out, R, S, chunk, (const TI*)a, (const TI*)nullptr, (TO*)out);
+  }
+  HG_CHECK_LAUNCH(ctx, "contract");
+  return HGPU_OK;
+}
+
+int64_t min_abs_nonzero(const Dims& d, int dim) {
+  int64_t m = INT64_MAX;
+  for (int k = 0; k < 2; ++k) {
+    int64_t s = d.st[k][dim];
+    if (s < 0) s = -s;
+    if (s != 0 && s < m) m = s;
+  }
+  return m;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (n_keep < 0 || n_keep > a->rank) return fail(ctx, HGPU_ERR_INVALID, "contract: n_keep %d of rank %d", n_keep, a->rank);
+  if (b) {
+    if (b->dtype != a->dtype) return fail(ctx, HGPU_ERR_INVALID, "contract: dtypes differ");
+    if (!same_shape(a, b)) return fail(ctx, HGPU_ERR_INVALID, "contract: shapes differ");
+  }
+  if (a->dtype == HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "contract: Bool arrays have no sum");
+  hgpu_array* o = nullptr;
+  int64_t n_out = 1, R = 1;
+  for (int i = 0; i < n_keep; ++i) n_out *= a->shape[i];
+  for (int i = n_keep; i < a->rank; ++i) R *= a->shape[i];
+  int rc;
+  if (n_out == 0 || R == 0) {
+    rc = new_zeros(ctx, a->dtype, n_keep, a->shape, &o);
+    if (rc) return rc;
+    *out = o;
+    return HGPU_OK;
+  }
+  rc = new_dense(ctx, a->dtype, n_keep, a->shape, &o);
+  if (rc) return rc;
+
+  bool handled = false;
+  rc = try_gemm(ctx, a, b, n_keep, o, &handled);
+  if (rc) { hgpu_release(o); return rc; }
+  if (handled) { *out = o; return HGPU_OK; }
+
+  int64_t zero[HGPU_MAX_RANK] = {0};
+  const int64_t* bst = b ? b->strides : zero;
+  const int64_t* ks[2] = {a->strides, bst};
+  const int64_t* rs[2] = {a->strides + n_keep, bst + n_keep};
+  Dims keep, red;
+  if (!collapse(n_keep, a->shape, 2, ks, &keep) || !collapse(a->rank - n_keep, a->shape + n_keep, 2, rs, &red)) {
+    hgpu_release(o);
+    return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract: more than %d merged dims", HG_KDIMS);
+  }
+  // Which way is memory contiguous: along the kept or along the reduced index?
+  int64_t sr = min_abs_nonzero(red, red.nd - 1);
+  int64_t sk = min_abs_nonzero(keep, keep.nd - 1);
+  int64_t Lin = red.shape[red.nd - 1];
+  bool use_wave;
+  if (n_out < 2048) use_wave = true;
+  else if (sr <= sk && Lin >= 16) use_wave = true;
+  else use_wave = false;
+  // Enough work items to fill the device, chunks of at least 2048 elements.
+  int64_t want_items = (int64_t)ctx->num_cu * (use_wave ? 16 : 1024);
+  int64_t S = 1;
+  if (n_out < want_items) {
+    S = (want_items + n_out - 1) / n_out;
+    int64_t span = use_wave ? ((R / Lin) > 1 ? (R / Lin) : Lin) : R;
+    int64_t per = use_wave ? ((R / Lin) > 1 ? 2048 / (Lin < 2048 ? Lin : 2048) : 2048) : 256;
+    if (per < 1) per = 1;
+    int64_t maxS = span / per;
+    if (maxS < 1) maxS = 1;
+    if (S > maxS) S = maxS;
+    if (S > 4096) S = 4096;
+  }
+  const void* pa = data_ptr(a);
+  const void* pb = b ? data_ptr(b) : nullptr;
+  if (S == 1) {
+    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, use_wave, keep, red, n_out, R, 1, pa, pb, data_ptr(o))));
+  } else {
+    // stage 1: partials [n_out, S] in the accumulator type; stage 2 sums them.
+    int accdt = dtype_is_float(a->dtype) ? HGPU_F64 : HGPU_I64;
+    int64_t psh[2] = {n_out, S};
+    hgpu_array* part = nullptr;
+    rc = new_dense(ctx, accdt, 2, psh, &part);
+    if (rc) { hgpu_release(o); return rc; }
+    HG_DISPATCH_DTYPE(a->dtype, T, { using A = typename acc_of<T>::type; rc = (launch_stage<T, A>(ctx, use_wave, keep, red, n_out, R, (int)S, pa, pb, data_ptr(part))); });
+    if (!rc) {
+      Dims k2, r2;
+      int64_t z1[1] = {0};
+      const int64_t* ks2[2] = {part->strides, z1};
+      const int64_t* rs2[2] = {part->strides + 1, z1};
+      collapse(1, psh, 2, ks2, &k2);
+      collapse(1, psh + 1, 2, rs2, &r2);
+      bool wave2 = n_out < 65536;
+      HG_DISPATCH_DTYPE(a->dtype, T, { using A = typename acc_of<T>::type; rc = (launch_stage<A, T>(ctx, wave2, k2, r2, n_out, S, 1, data_ptr(part), nullptr, data_ptr(o))); });
+    }
+    hgpu_release(part);
+  }
+  if (rc) { hgpu_release(o); return rc; }
+  *out = o;
+  return HGPU_OK;
+}
+
+int hgpu_argminmax_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (a->rank < 1) return fail(ctx, HGPU_ERR_INVALID, "argminmax: rank 0");
+  int64_t L = a->shape[a->rank - 1];
+  if (L < 1) return fail(ctx, HGPU_ERR_INVALID, "argminmax: empty last dim");
+  hgpu_array* o = nullptr;
+  int rc = new_dense(ctx, HGPU_I64, a->rank - 1, a->shape, &o);
+  if (rc) return rc;
+  int64_t n_out = nelem(o);
+  if (n_out > 0) {
+    const int64_t* ks[1] = {a->strides};
+    Dims keep;
+    if (!collapse(a->rank - 1, a->shape, 1, ks, &keep)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "argminmax: too many dims"); }
+    LaunchGuard lg(ctx);
+    unsigned g = grid_for(n_out, kBlock, ctx->num_cu * 8);
+    HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "argminmax"); }
+  }
+  *out = o;
+  return HGPU_OK;
+}
+
+}  // extern "C"

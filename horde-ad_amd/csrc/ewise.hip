@@ -1,0 +1,524 @@
+// Elementwise kernels over strided views: the Num / Fractional / Floating /
+// IntegralH instances of arrays that horde-ad's `Concrete` backend takes from
+// ox-arrays (src/HordeAd/Core/CarriersConcrete.hs:40-56,333-343), comparisons,
+// conversions, and the copying structural operations (append, pad, oneHot).
+//
+// Every kernel walks the OUTPUT in linear order, one element per lane per
+// grid-stride step, so stores are always coalesced; loads are coalesced
+// whenever the operand's innermost merged dimension has unit stride.  When all
+// operands are dense (or one-element broadcasts) the index decomposition is
+// skipped and each lane moves 16-byte vectors.
+#include "common.hpp"
+
+using namespace hg;
+
+namespace {
+
+constexpr int kBlock = 256;
+
+template <typename T> struct is_fp { static constexpr bool value = false; };
+template <> struct is_fp<double> { static constexpr bool value = true; };
+template <> struct is_fp<float> { static constexpr bool value = true; };
+
+template <typename T>
+__device__ __forceinline__ T apply1(int op, T x) {
+  if constexpr (is_fp<T>::value) {
+    switch (op) {
+      case HGPU_NEG: return -x;
+      case HGPU_ABS: return fabs(x);
+      case HGPU_SIGNUM: return x > T(0) ? T(1) : (x < T(0) ? T(-1) : x);
+      case HGPU_RECIP: return T(1) / x;
+      case HGPU_EXP: return exp(x);
+      case HGPU_LOG: return log(x);
+      case HGPU_SQRT: return sqrt(x);
+      case HGPU_SIN: return sin(x);
+      case HGPU_COS: return cos(x);
+      case HGPU_TAN: return tan(x);
+      case HGPU_ASIN: return asin(x);
+      case HGPU_ACOS: return acos(x);
+      case HGPU_ATAN: return atan(x);
+      case HGPU_SINH: return sinh(x);
+      case HGPU_COSH: return cosh(x);
+      case HGPU_TANH: return tanh(x);
+      case HGPU_ASINH: return asinh(x);
+      case HGPU_ACOSH: return acosh(x);
+      case HGPU_ATANH: return atanh(x);
+    }
+    return x;
+  } else {
+    switch (op) {
+      case HGPU_NEG: return (T)(-x);
+      case HGPU_ABS: return x < 0 ? (T)(-x) : x;
+      case HGPU_SIGNUM: return x > 0 ? T(1) : (x < 0 ? T(-1) : T(0));
+      case HGPU_NOT: return (T)(x == 0 ? 1 : 0);
+    }
+    return x;
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ T apply2(int op, T x, T y) {
+  if constexpr (is_fp<T>::value) {
+    switch (op) {
+      case HGPU_ADD: return x + y;
+      case HGPU_MUL: return x * y;
+      case HGPU_SUB: return x - y;
+      case HGPU_DIV: return x / y;
+      case HGPU_POW: return pow(x, y);
+      case HGPU_LOGBASE: return log(y) / log(x);  // logBase x y = log y / log x
+      case HGPU_ATAN2: return atan2(x, y);
+      case HGPU_MIN: return x <= y ? x : y;
+      case HGPU_MAX: return x >= y ? x : y;
+    }
+    return x;
+  } else {
+    switch (op) {
+      case HGPU_ADD: return (T)(x + y);
+      case HGPU_MUL: return (T)(x * y);
+      case HGPU_SUB: return (T)(x - y);
+      case HGPU_QUOT: return y == 0 ? x : (T)(x / y);  // quot a 1 = a
+      case HGPU_REM: return y == 0 ? T(0) : (T)(x % y);  // array rule: rem a 1 = 0
+      case HGPU_REM_SCALAR: return y == 0 ? x : (T)(x % y);
+      case HGPU_MIN: return x <= y ? x : y;
+      case HGPU_MAX: return x >= y ? x : y;
+      case HGPU_AND: return (T)((x != 0 && y != 0) ? 1 : 0);
+    }
+    return x;
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ uint8_t applycmp(int op, T x, T y) {
+  switch (op) {
+    case HGPU_LEQ: return x <= y;
+    case HGPU_EQ: return x == y;
+    case HGPU_LT: return x < y;
+  }
+  return 0;
+}
+
+// ---- generic strided kernels (operand 0 is the dense output) --------------
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_ewise1(int op, Dims d, int64_t n, const T* __restrict__ a, T* __restrict__ o) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) {
+    int64_t off[1];
+    decompose<1>(d, i, off);
+    o[i] = apply1<T>(op, a[off[0]]);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_ewise2(int op, Dims d, int64_t n, const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ o) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) {
+    int64_t off[2];
+    decompose<2>(d, i, off);
+    o[i] = apply2<T>(op, a[off[0]], b[off[1]]);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_cmp(int op, Dims d, int64_t n, const T* __restrict__ a, const T* __restrict__ b, uint8_t* __restrict__ o) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) {
+    int64_t off[2];
+    decompose<2>(d, i, off);
+    o[i] = applycmp<T>(op, a[off[0]], b[off[1]]);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_select(Dims d, int64_t n, const uint8_t* __restrict__ c, const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ o) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) {
+    int64_t off[3];
+    decompose<3>(d, i, off);
+    o[i] = c[off[0]] ? a[off[1]] : b[off[2]];
+  }
+}
+
+template <typename S, typename D>
+__device__ __forceinline__ D conv1(S x, int mode) {
+  if constexpr (is_fp<S>::value && !is_fp<D>::value) {
+    if (mode == HGPU_CONV_FLOOR) return (D)(int64_t)floor((double)x);
+    return (D)(int64_t)x;
+  } else {
+    return (D)x;
+  }
+}
+
+template <typename S, typename D>
+__global__ void __launch_bounds__(kBlock) k_convert(int mode, Dims d, int64_t n, const S* __restrict__ a, D* __restrict__ o) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) {
+    int64_t off[1];
+    decompose<1>(d, i, off);
+    o[i] = conv1<S, D>(a[off[0]], mode);
+  }
+}
+
+// Copy between two strided views of one shape (operand 0 = source, 1 = dest).
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_copy(Dims d, int64_t n, const T* __restrict__ a, T* __restrict__ o) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) {
+    int64_t off[2];
+    decompose<2>(d, i, off);
+    o[off[1]] = a[off[0]];
+  }
+}
+
+// ---- dense fast paths: 16-byte vectors, flags say which operands broadcast --
+
+template <typename T> struct Vec16 { static constexpr int N = 16 / sizeof(T); T v[N]; };
+
+template <typename T, bool BA, bool BB>
+__global__ void __launch_bounds__(kBlock) k_ewise2_dense(int op, int64_t n, const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ o) {
+  constexpr int N = Vec16<T>::N;
+  int64_t nv = n / N;
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  T sa = BA ? a[0] : T(0), sb = BB ? b[0] : T(0);
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nv; i += step) {
+    Vec16<T> va, vb, vo;
+    if (!BA) va = reinterpret_cast<const Vec16<T>*>(a)[i];
+    if (!BB) vb = reinterpret_cast<const Vec16<T>*>(b)[i];
+#pragma unroll
+    for (int k = 0; k < N; ++k) vo.v[k] = apply2<T>(op, BA ? sa : va.v[k], BB ? sb : vb.v[k]);
+    reinterpret_cast<Vec16<T>*>(o)[i] = vo;
+  }
+  int64_t t = nv * N + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (t < n) o[t] = apply2<T>(op, BA ? sa : a[t], BB ? sb : b[t]);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_ewise1_dense(int op, int64_t n, const T* __restrict__ a, T* __restrict__ o) {
+  constexpr int N = Vec16<T>::N;
+  int64_t nv = n / N;
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nv; i += step) {
+    Vec16<T> va = reinterpret_cast<const Vec16<T>*>(a)[i], vo;
+#pragma unroll
+    for (int k = 0; k < N; ++k) vo.v[k] = apply1<T>(op, va.v[k]);
+    reinterpret_cast<Vec16<T>*>(o)[i] = vo;
+  }
+  int64_t t = nv * N + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (t < n) o[t] = apply1<T>(op, a[t]);
+}
+
+__global__ void __launch_bounds__(kBlock) k_zero16(int64_t n16, uint4* __restrict__ o) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n16; i += step) o[i] = make_uint4(0, 0, 0, 0);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_iota(int64_t n, T* __restrict__ o) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) o[i] = (T)i;
+}
+
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// 0 = general view, 1 = dense, 2 = every stride zero (one element broadcast).
+inline int layout_class(const hgpu_array* a) {
+  bool all0 = true;
+  for (int i = 0; i < a->rank; ++i)
+    if (a->shape[i] != 1 && a->strides[i] != 0) all0 = false;
+  if (all0) return 2;
+  return is_dense(a) ? 1 : 0;
+}
+
+inline int max_blocks(hgpu_ctx* ctx) { return ctx->num_cu * 8; }
+
+}  // namespace
+
+namespace hg {
+
+int zero_fill(hgpu_ctx* ctx, void* p, size_t bytes) {
+  // Blocks come from the allocator in multiples of 256 bytes, so rounding the
+  // length up to 16 stays inside the block.
+  int64_t n16 = (int64_t)((bytes + 15) / 16);
+  if (n16 == 0) return HGPU_OK;
+  LaunchGuard lg(ctx);
+  hipLaunchKernelGGL(k_zero16, dim3(grid_for(n16, kBlock, max_blocks(ctx))), dim3(kBlock), 0, ctx->stream, n16, (uint4*)p);
+  HG_CHECK_LAUNCH(ctx, "zero_fill");
+  return HGPU_OK;
+}
+
+int copy_view(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const void* src, const int64_t* sst,
+              void* dst, const int64_t* dst_st) {
+  int64_t n = 1;
+  for (int i = 0; i < rank; ++i) n *= shape[i];
+  if (n == 0) return HGPU_OK;
+  const int64_t* sts[2] = {sst, dst_st};
+  Dims d;
+  if (!collapse(rank, shape, 2, sts, &d)) return fail(ctx, HGPU_ERR_UNSUPPORTED, "copy: more than %d merged dims", HG_KDIMS);
+  LaunchGuard lg(ctx);
+  unsigned g = grid_for(n, kBlock, max_blocks(ctx));
+  switch (dtype_size(dtype)) {
+    case 8: hipLaunchKernelGGL(k_copy<uint64_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint64_t*)src, (uint64_t*)dst); break;
+    case 4: hipLaunchKernelGGL(k_copy<uint32_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint32_t*)src, (uint32_t*)dst); break;
+    case 2: hipLaunchKernelGGL(k_copy<uint16_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint16_t*)src, (uint16_t*)dst); break;
+    default: hipLaunchKernelGGL(k_copy<uint8_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint8_t*)src, (uint8_t*)dst); break;
+  }
+  HG_CHECK_LAUNCH(ctx, "copy_view");
+  return HGPU_OK;
+}
+
+}  // namespace hg
+
+extern "C" {
+
+int hgpu_materialize(hgpu_ctx* ctx, const hgpu_array* a, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  hgpu_array* o = nullptr;
+  int rc = new_dense(ctx, a->dtype, a->rank, a->shape, &o);
+  if (rc) return rc;
+  rc = copy_view(ctx, a->dtype, a->rank, a->shape, data_ptr(a), a->strides, data_ptr(o), o->strides);
+  if (rc) { hgpu_release(o); return rc; }
+  *out = o;
+  return HGPU_OK;
+}
+
+int hgpu_pad(hgpu_ctx* ctx, const hgpu_array* a, const int64_t* lo, const int64_t* hi, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  int64_t sh[HGPU_MAX_RANK];
+  for (int i = 0; i < a->rank; ++i) {
+    if (lo[i] < 0 || hi[i] < 0) return fail(ctx, HGPU_ERR_INVALID, "pad: negative padding");
+    sh[i] = a->shape[i] + lo[i] + hi[i];
+  }
+  hgpu_array* o = nullptr;
+  int rc = new_zeros(ctx, a->dtype, a->rank, sh, &o);
+  if (rc) return rc;
+  int64_t off = 0;
+  for (int i = 0; i < a->rank; ++i) off += lo[i] * o->strides[i];
+  if (nelem(a) > 0)
+    rc = copy_view(ctx, a->dtype, a->rank, a->shape, data_ptr(a), a->strides,
+                   (char*)data_ptr(o) + off * (int64_t)dtype_size(a->dtype), o->strides);
+  if (rc) { hgpu_release(o); return rc; }
+  *out = o;
+  return HGPU_OK;
+}
+
+int hgpu_ewise1(hgpu_ctx* ctx, int op, const hgpu_array* a, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (op < 0 || op >= HGPU_OP1_COUNT) return fail(ctx, HGPU_ERR_INVALID, "ewise1: unknown opcode %d", op);
+  bool fp = dtype_is_float(a->dtype);
+  if (op >= HGPU_RECIP && op <= HGPU_ATANH && !fp) return fail(ctx, HGPU_ERR_INVALID, "ewise1: floating opcode %d on a non-floating array", op);
+  if (op == HGPU_NOT && a->dtype != HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "ewise1: NOT on a non-Bool array");
+  if (a->dtype == HGPU_BOOL && op != HGPU_NOT) return fail(ctx, HGPU_ERR_INVALID, "ewise1: arithmetic on a Bool array");
+  hgpu_array* o = nullptr;
+  int rc = new_dense(ctx, a->dtype, a->rank, a->shape, &o);
+  if (rc) return rc;
+  int64_t n = nelem(o);
+  if (n > 0) {
+    LaunchGuard lg(ctx);
+    if (layout_class(a) == 1 && aligned16(data_ptr(a))) {
+      unsigned g = grid_for(n, kBlock * 4, max_blocks(ctx));
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_ewise1_dense<T>, dim3(g), dim3(kBlock), 0, ctx->stream, op, n, (const T*)data_ptr(a), (T*)data_ptr(o)));
+    } else {
+      const int64_t* sts[1] = {a->strides};
+      Dims d;
+      if (!collapse(a->rank, a->shape, 1, sts, &d)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "ewise1: too many dims"); }
+      unsigned g = grid_for(n, kBlock, max_blocks(ctx));
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_ewise1<T>, dim3(g), dim3(kBlock), 0, ctx->stream, op, d, n, (const T*)data_ptr(a), (T*)data_ptr(o)));
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "ewise1"); }
+  }
+  *out = o;
+  return HGPU_OK;
+}
+
+static int check_binary(hgpu_ctx* ctx, const char* who, const hgpu_array* a, const hgpu_array* b) {
+  if (a->dtype != b->dtype) return fail(ctx, HGPU_ERR_INVALID, "%s: dtypes %d and %d differ", who, a->dtype, b->dtype);
+  if (!same_shape(a, b)) return fail(ctx, HGPU_ERR_INVALID, "%s: shapes differ", who);
+  return HGPU_OK;
+}
+
+int hgpu_ewise2(hgpu_ctx* ctx, int op, const hgpu_array* a, const hgpu_array* b, hgpu_array** out) {
+  if (!ctx || !a || !b || !out) return HGPU_ERR_INVALID;
+  if (op < 0 || op >= HGPU_OP2_COUNT) return fail(ctx, HGPU_ERR_INVALID, "ewise2: unknown opcode %d", op);
+  int rc = check_binary(ctx, "ewise2", a, b);
+  if (rc) return rc;
+  bool fp = dtype_is_float(a->dtype);
+  if (op >= HGPU_DIV && op <= HGPU_ATAN2 && !fp) return fail(ctx, HGPU_ERR_INVALID, "ewise2: floating opcode %d on a non-floating array", op);
+  if (op >= HGPU_QUOT && op <= HGPU_REM_SCALAR && !dtype_is_int(a->dtype)) return fail(ctx, HGPU_ERR_INVALID, "ewise2: integral opcode %d on a non-integral array", op);
+  if (op == HGPU_AND && a->dtype != HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "ewise2: AND on a non-Bool array");
+  if (a->dtype == HGPU_BOOL && op != HGPU_AND) return fail(ctx, HGPU_ERR_INVALID, "ewise2: arithmetic on a Bool array");
+  hgpu_array* o = nullptr;
+  rc = new_dense(ctx, a->dtype, a->rank, a->shape, &o);
+  if (rc) return rc;
+  int64_t n = nelem(o);
+  if (n > 0) {
+    LaunchGuard lg(ctx);
+    int la = layout_class(a), lb = layout_class(b);
+    bool fast = la != 0 && lb != 0 && !(la == 2 && lb == 2) && (la == 2 || aligned16(data_ptr(a))) && (lb == 2 || aligned16(data_ptr(b)));
+    if (fast) {
+      unsigned g = grid_for(n, kBlock * 4, max_blocks(ctx));
+      HG_DISPATCH_DTYPE(a->dtype, T, {
+        const T* pa = (const T*)data_ptr(a);
+        const T* pb = (const T*)data_ptr(b);
+        T* po = (T*)data_ptr(o);
+        if (la == 2) hipLaunchKernelGGL((k_ewise2_dense<T, true, false>), dim3(g), dim3(kBlock), 0, ctx->stream, op, n, pa, pb, po);
+        else if (lb == 2) hipLaunchKernelGGL((k_ewise2_dense<T, false, true>), dim3(g), dim3(kBlock), 0, ctx->stream, op, n, pa, pb, po);
+        else hipLaunchKernelGGL((k_ewise2_dense<T, false, false>), dim3(g), dim3(kBlock), 0, ctx->stream, op, n, pa, pb, po);
+      });
+    } else {
+      const int64_t* sts[2] = {a->strides, b->strides};
+      Dims d;
+      if (!collapse(a->rank, a->shape, 2, sts, &d)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "ewise2: too many dims"); }
+      unsigned g = grid_for(n, kBlock, max_blocks(ctx));
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_ewise2<T>, dim3(g), dim3(kBlock), 0, ctx->stream, op, d, n, (const T*)data_ptr(a), (const T*)data_ptr(b), (T*)data_ptr(o)));
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "ewise2"); }
+  }
+  *out = o;
+  return HGPU_OK;
+}
+
+int hgpu_compare(hgpu_ctx* ctx, int cmp, const hgpu_array* a, const hgpu_array* b, hgpu_array** out) {
+  if (!ctx || !a || !b || !out) return HGPU_ERR_INVALID;
+  if (cmp < HGPU_LEQ || cmp > HGPU_LT) return fail(ctx, HGPU_ERR_INVALID, "compare: unknown opcode %d", cmp);
+  int rc = check_binary(ctx, "compare", a, b);
+  if (rc) return rc;
+  hgpu_array* o = nullptr;
+  rc = new_dense(ctx, HGPU_BOOL, a->rank, a->shape, &o);
+  if (rc) return rc;
+  int64_t n = nelem(o);
+  if (n > 0) {
+    const int64_t* sts[2] = {a->strides, b->strides};
+    Dims d;
+    if (!collapse(a->rank, a->shape, 2, sts, &d)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "compare: too many dims"); }
+    LaunchGuard lg(ctx);
+    unsigned g = grid_for(n, kBlock, max_blocks(ctx));
+    HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_cmp<T>, dim3(g), dim3(kBlock), 0, ctx->stream, cmp, d, n, (const T*)data_ptr(a), (const T*)data_ptr(b), (uint8_t*)data_ptr(o)));
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "compare"); }
+  }
+  *out = o;
+  return HGPU_OK;
+}
+
+int hgpu_select(hgpu_ctx* ctx, const hgpu_array* c, const hgpu_array* a, const hgpu_array* b, hgpu_array** out) {
+  if (!ctx || !c || !a || !b || !out) return HGPU_ERR_INVALID;
+  if (c->dtype != HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "select: condition is not Bool");
+  int rc = check_binary(ctx, "select", a, b);
+  if (rc) return rc;
+  if (!same_shape(c, a)) return fail(ctx, HGPU_ERR_INVALID, "select: condition shape differs");
+  hgpu_array* o = nullptr;
+  rc = new_dense(ctx, a->dtype, a->rank, a->shape, &o);
+  if (rc) return rc;
+  int64_t n = nelem(o);
+  if (n > 0) {
+    const int64_t* sts[3] = {c->strides, a->strides, b->strides};
+    Dims d;
+    if (!collapse(a->rank, a->shape, 3, sts, &d)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "select: too many dims"); }
+    LaunchGuard lg(ctx);
+    unsigned g = grid_for(n, kBlock, max_blocks(ctx));
+    HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_select<T>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint8_t*)data_ptr(c), (const T*)data_ptr(a), (const T*)data_ptr(b), (T*)data_ptr(o)));
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "select"); }
+  }
+  *out = o;
+  return HGPU_OK;
+}
+
+int hgpu_convert(hgpu_ctx* ctx, const hgpu_array* a, int dtype, int mode, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (dtype_size(dtype) == 0) return fail(ctx, HGPU_ERR_INVALID, "convert: unknown dtype %d", dtype);
+  if (mode == HGPU_CONV_FLOOR && !(dtype_is_float(a->dtype) && dtype_is_int(dtype)))
+    return fail(ctx, HGPU_ERR_INVALID, "convert: floor needs a floating source and an integral target");
+  hgpu_array* o = nullptr;
+  int rc = new_dense(ctx, dtype, a->rank, a->shape, &o);
+  if (rc) return rc;
+  int64_t n = nelem(o);
+  if (n > 0) {
+    const int64_t* sts[1] = {a->strides};
+    Dims d;
+    if (!collapse(a->rank, a->shape, 1, sts, &d)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "convert: too many dims"); }
+    LaunchGuard lg(ctx);
+    unsigned g = grid_for(n, kBlock, max_blocks(ctx));
+    HG_DISPATCH_DTYPE(a->dtype, S, {
+      HG_DISPATCH_DTYPE(dtype, D, hipLaunchKernelGGL((k_convert<S, D>), dim3(g), dim3(kBlock), 0, ctx->stream, mode, d, n, (const S*)data_ptr(a), (D*)data_ptr(o)));
+    });
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "convert"); }
+  }
+  *out = o;
+  return HGPU_OK;
+}
+
+int hgpu_iota(hgpu_ctx* ctx, int64_t n, int dtype, hgpu_array** out) {
+  if (!ctx || !out) return HGPU_ERR_INVALID;
+  if (n < 0 || dtype_size(dtype) == 0 || dtype == HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "iota: bad arguments");
+  hgpu_array* o = nullptr;
+  int rc = new_dense(ctx, dtype, 1, &n, &o);
+  if (rc) return rc;
+  if (n > 0) {
+    LaunchGuard lg(ctx);
+    unsigned g = grid_for(n, kBlock, max_blocks(ctx));
+    HG_DISPATCH_DTYPE(dtype, T, hipLaunchKernelGGL(k_iota<T>, dim3(g), dim3(kBlock), 0, ctx->stream, n, (T*)data_ptr(o)));
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "iota"); }
+  }
+  *out = o;
+  return HGPU_OK;
+}
+
+int hgpu_concat(hgpu_ctx* ctx, int n, const hgpu_array* const* parts, hgpu_array** out) {
+  if (!ctx || !parts || !out || n < 1) return HGPU_ERR_INVALID;
+  const hgpu_array* p0 = parts[0];
+  if (p0->rank < 1) return fail(ctx, HGPU_ERR_INVALID, "concat: rank 0");
+  int64_t sh[HGPU_MAX_RANK];
+  for (int i = 0; i < p0->rank; ++i) sh[i] = p0->shape[i];
+  sh[0] = 0;
+  for (int k = 0; k < n; ++k) {
+    const hgpu_array* p = parts[k];
+    if (!p || p->rank != p0->rank || p->dtype != p0->dtype) return fail(ctx, HGPU_ERR_INVALID, "concat: part %d has another rank or dtype", k);
+    for (int i = 1; i < p0->rank; ++i)
+      if (p->shape[i] != p0->shape[i]) return fail(ctx, HGPU_ERR_INVALID, "concat: part %d differs in dim %d", k, i);
+    sh[0] += p->shape[0];
+  }
+  hgpu_array* o = nullptr;
+  int rc = new_dense(ctx, p0->dtype, p0->rank, sh, &o);
+  if (rc) return rc;
+  int64_t row = 0;
+  for (int k = 0; k < n && !rc; ++k) {
+    const hgpu_array* p = parts[k];
+    if (nelem(p) > 0)
+      rc = copy_view(ctx, p->dtype, p->rank, p->shape, data_ptr(p), p->strides,
+                     (char*)data_ptr(o) + row * o->strides[0] * (int64_t)dtype_size(p->dtype), o->strides);
+    row += p->shape[0];
+  }
+  if (rc) { hgpu_release(o); return rc; }
+  *out = o;
+  return HGPU_OK;
+}
+
+int hgpu_onehot(hgpu_ctx* ctx, const hgpu_array* v, int n, const int64_t* ix, const int64_t* shp, hgpu_array** out) {
+  if (!ctx || !v || !out || n < 0 || n + v->rank > HGPU_MAX_RANK) return HGPU_ERR_INVALID;
+  int64_t sh[HGPU_MAX_RANK];
+  bool oob = false;
+  for (int i = 0; i < n; ++i) {
+    sh[i] = shp[i];
+    if (ix[i] < 0 || ix[i] >= shp[i]) oob = true;
+  }
+  for (int i = 0; i < v->rank; ++i) sh[n + i] = v->shape[i];
+  hgpu_array* o = nullptr;
+  int rc = new_zeros(ctx, v->dtype, n + v->rank, sh, &o);
+  if (rc) return rc;
+  if (!oob && nelem(v) > 0) {
+    int64_t off = 0;
+    for (int i = 0; i < n; ++i) off += ix[i] * o->strides[i];
+    rc = copy_view(ctx, v->dtype, v->rank, v->shape, data_ptr(v), v->strides,
+                   (char*)data_ptr(o) + off * (int64_t)dtype_size(v->dtype), o->strides + n);
+  }
+  if (rc) { hgpu_release(o); return rc; }
+  *out = o;
+  return HGPU_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,564 @@
+// Context, caching allocator, upload/download, and the metadata-only view
+// operations of the backend.  The view operations mirror what ox-arrays does
+// with strides for the `Concrete` instance of horde-ad
+// (src/HordeAd/Core/OpsConcrete.hs:243-246,641-652): no element is touched.
+#include "common.hpp"
+
+namespace hg {
+
+int fail(hgpu_ctx* ctx, int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  if (ctx) {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    ctx->err = buf;
+  }
+  return code;
+}
+
+int check_hip(hgpu_ctx* ctx, hipError_t e, const char* what) {
+  if (e == hipSuccess) return HGPU_OK;
+  return fail(ctx, e == hipErrorOutOfMemory ? HGPU_ERR_OOM : HGPU_ERR_DEVICE, "%s: %s", what,
+              hipGetErrorString(e));
+}
+
+static size_t round_block(size_t bytes) {
+  if (bytes < 256) return 256;
+  if (bytes <= (1u << 20)) {  // powers of two up to 1 MiB
+    size_t p = 256;
+    while (p < bytes) p <<= 1;
+    return p;
+  }
+  const size_t mib = 1u << 20;  // then multiples of 1 MiB
+  return (bytes + mib - 1) / mib * mib;
+}
+
+static void drop_cache_locked(hgpu_ctx* ctx) {
+  for (auto& kv : ctx->cache) {
+    (void)hipFree(kv.second);
+    ctx->reserved -= kv.first;
+  }
+  ctx->cache.clear();
+}
+
+int buffer_alloc(hgpu_ctx* ctx, size_t bytes, hgpu_buffer** out) {
+  size_t blk = round_block(bytes);
+  void* p = nullptr;
+  {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    auto it = ctx->cache.find(blk);
+    if (it != ctx->cache.end()) {
+      p = it->second;
+      ctx->cache.erase(it);
+    } else {
+      if (ctx->fail_after >= 0 && (int64_t)ctx->n_device_allocs >= ctx->fail_after) {
+        ctx->err = "device allocation failed (injected)";
+        return HGPU_ERR_OOM;
+      }
+      (void)hipSetDevice(ctx->device);
+      hipError_t e = hipMalloc(&p, blk);
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        // Cached blocks may still be read by enqueued kernels: drain first.
+        (void)hipStreamSynchronize(ctx->stream);
+        drop_cache_locked(ctx);
+        e = hipMalloc(&p, blk);
+      }
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        char msg[160];
+        snprintf(msg, sizeof msg, "device allocation of %zu bytes failed: %s", blk, hipGetErrorString(e));
+        ctx->err = msg;
+        return HGPU_ERR_OOM;
+      }
+      ctx->reserved += blk;
+      ctx->n_device_allocs++;
+    }
+    ctx->in_use += blk;
+  }
+  hgpu_buffer* b = new hgpu_buffer;
+  b->ctx = ctx;
+  b->ptr = p;
+  b->bytes = blk;
+  b->refs.store(1);
+  *out = b;
+  return HGPU_OK;
+}
+
+void buffer_retain(hgpu_buffer* b) {
+  if (b) b->refs.fetch_add(1);
+}
+
+void buffer_release(hgpu_buffer* b) {
+  if (!b) return;
+  if (b->refs.fetch_sub(1) == 1) {
+    hgpu_ctx* ctx = b->ctx;
+    {
+      // The block goes back to the cache at once: all work that reads it is
+      // already enqueued on the in-order stream, and whatever reuses it is
+      // enqueued behind that work.
+      std::lock_guard<std::mutex> g(ctx->mu);
+      ctx->cache.emplace(b->bytes, b->ptr);
+      ctx->in_use -= b->bytes;
+    }
+    delete b;
+  }
+}
+
+hgpu_array* new_view(hgpu_ctx* ctx, hgpu_buffer* buf, int dtype, int rank, const int64_t* shape,
+                     const int64_t* strides, int64_t offset) {
+  hgpu_array* a = new hgpu_array;
+  a->ctx = ctx;
+  a->refs.store(1);
+  a->buf = buf;
+  buffer_retain(buf);
+  a->dtype = dtype;
+  a->rank = rank;
+  for (int i = 0; i < rank; ++i) {
+    a->shape[i] = shape[i];
+    a->strides[i] = strides[i];
+  }
+  a->offset = offset;
+  return a;
+}
+
+int new_dense(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, hgpu_array** out) {
+  if (rank < 0 || rank > HGPU_MAX_RANK) return fail(ctx, HGPU_ERR_INVALID, "rank %d out of range", rank);
+  int64_t n = 1;
+  for (int i = 0; i < rank; ++i) {
+    if (shape[i] < 0) return fail(ctx, HGPU_ERR_INVALID, "negative extent");
+    n *= shape[i];
+  }
+  int64_t st[HGPU_MAX_RANK];
+  dense_strides(rank, shape, st);
+  hgpu_buffer* buf = nullptr;
+  if (n > 0) {
+    int rc = buffer_alloc(ctx, (size_t)n * dtype_size(dtype), &buf);
+    if (rc) return rc;
+  }
+  *out = new_view(ctx, buf, dtype, rank, shape, st, 0);
+  buffer_release(buf);  // the view holds the only reference
+  return HGPU_OK;
+}
+
+int new_zeros(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, hgpu_array** out) {
+  int rc = new_dense(ctx, dtype, rank, shape, out);
+  if (rc) return rc;
+  int64_t n = nelem(*out);
+  if (n > 0) {
+    // A fill kernel, not hipMemsetAsync: callers may capture the stream.
+    rc = zero_fill(ctx, data_ptr(*out), (size_t)n * dtype_size(dtype));
+    if (rc) {
+      hgpu_release(*out);
+      *out = nullptr;
+      return rc;
+    }
+  }
+  return HGPU_OK;
+}
+
+bool is_dense(const hgpu_array* a) {
+  int64_t s = 1;
+  for (int i = a->rank - 1; i >= 0; --i) {
+    if (a->shape[i] != 1 && a->strides[i] != s) return false;
+    s *= a->shape[i];
+  }
+  return true;
+}
+
+bool same_shape(const hgpu_array* a, const hgpu_array* b) {
+  if (a->rank != b->rank) return false;
+  for (int i = 0; i < a->rank; ++i)
+    if (a->shape[i] != b->shape[i]) return false;
+  return true;
+}
+
+bool collapse(int rank, const int64_t* shape, int nops, const int64_t* const* strides, Dims* out) {
+  Dims d;
+  d.nd = 0;
+  for (int i = 0; i < rank; ++i) {
+    if (shape[i] == 1) continue;
+    bool merged = false;
+    if (d.nd > 0) {
+      int p = d.nd - 1;
+      bool ok = true;
+      for (int k = 0; k < nops; ++k)
+        if (d.st[k][p] != strides[k][i] * shape[i]) { ok = false; break; }
+      if (ok) {
+        d.shape[p] *= shape[i];
+        for (int k = 0; k < nops; ++k) d.st[k][p] = strides[k][i];
+        merged = true;
+      }
+    }
+    if (!merged) {
+      if (d.nd == HG_KDIMS) return false;
+      d.shape[d.nd] = shape[i];
+      for (int k = 0; k < nops; ++k) d.st[k][d.nd] = strides[k][i];
+      d.nd++;
+    }
+  }
+  if (d.nd == 0) {
+    d.nd = 1;
+    d.shape[0] = 1;
+    for (int k = 0; k < nops; ++k) d.st[k][0] = 0;
+  }
+  for (int i = d.nd; i < HG_KDIMS; ++i) {
+    d.shape[i] = 1;
+    for (int k = 0; k < 4; ++k) d.st[k][i] = 0;
+  }
+  for (int k = nops; k < 4; ++k)
+    for (int i = 0; i < HG_KDIMS; ++i) d.st[k][i] = 0;
+  *out = d;
+  return true;
+}
+
+static int ensure_staging(hgpu_ctx* ctx, size_t bytes) {
+  if (ctx->staging_bytes >= bytes) return HGPU_OK;
+  if (ctx->staging) (void)hipHostFree(ctx->staging);
+  ctx->staging = nullptr;
+  ctx->staging_bytes = 0;
+  hipError_t e = hipHostMalloc(&ctx->staging, bytes, hipHostMallocDefault);
+  if (e != hipSuccess) return check_hip(ctx, e, "hipHostMalloc");
+  ctx->staging_bytes = bytes;
+  return HGPU_OK;
+}
+
+}  // namespace hg
+
+using namespace hg;
+
+extern "C" {
+
+int hgpu_init(int device, hgpu_ctx** out) {
+  if (!out) return HGPU_ERR_INVALID;
+  *out = nullptr;
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n) {
+    (void)hipGetLastError();
+    return HGPU_ERR_DEVICE;
+  }
+  if (hipSetDevice(device) != hipSuccess) return HGPU_ERR_DEVICE;
+  hgpu_ctx* ctx = new hgpu_ctx;
+  ctx->device = device;
+  if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
+    delete ctx;
+    return HGPU_ERR_DEVICE;
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->num_cu = prop.multiProcessorCount;
+  *out = ctx;
+  return HGPU_OK;
+}
+
+int hgpu_shutdown(hgpu_ctx* ctx) {
+  if (!ctx) return HGPU_ERR_INVALID;
+  (void)hipSetDevice(ctx->device);
+  (void)hipStreamSynchronize(ctx->stream);
+  {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    drop_cache_locked(ctx);
+  }
+  if (ctx->staging) (void)hipHostFree(ctx->staging);
+  ctx->staging = nullptr;
+  ctx->staging_bytes = 0;
+  // The context itself stays allocated: arrays released later (finalizers)
+  // still find their allocator.
+  return HGPU_OK;
+}
+
+int hgpu_sync(hgpu_ctx* ctx) {
+  if (!ctx) return HGPU_ERR_INVALID;
+  (void)hipSetDevice(ctx->device);
+  return check_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+const char* hgpu_last_error(hgpu_ctx* ctx) {
+  static thread_local std::string copy;
+  if (!ctx) return "no context";
+  std::lock_guard<std::mutex> g(ctx->mu);
+  copy = ctx->err;
+  return copy.c_str();
+}
+
+int hgpu_mem_stats(hgpu_ctx* ctx, uint64_t* in_use, uint64_t* reserved, uint64_t* n_allocs) {
+  if (!ctx) return HGPU_ERR_INVALID;
+  std::lock_guard<std::mutex> g(ctx->mu);
+  if (in_use) *in_use = ctx->in_use;
+  if (reserved) *reserved = ctx->reserved;
+  if (n_allocs) *n_allocs = ctx->n_device_allocs;
+  return HGPU_OK;
+}
+
+void* hgpu_stream(hgpu_ctx* ctx) { return ctx ? (void*)ctx->stream : nullptr; }
+
+int hgpu_inject_alloc_failure(hgpu_ctx* ctx, int64_t limit) {
+  if (!ctx) return HGPU_ERR_INVALID;
+  std::lock_guard<std::mutex> g(ctx->mu);
+  if (limit < 0) {
+    ctx->fail_after = -1;
+  } else {
+    ctx->fail_after = (int64_t)ctx->n_device_allocs + limit;
+    // Cached blocks would satisfy requests without a device allocation.
+    (void)hipStreamSynchronize(ctx->stream);
+    drop_cache_locked(ctx);
+  }
+  return HGPU_OK;
+}
+
+int hgpu_upload(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const void* host, hgpu_array** out) {
+  if (!ctx || !out) return HGPU_ERR_INVALID;
+  *out = nullptr;
+  if (dtype_size(dtype) == 0) return fail(ctx, HGPU_ERR_INVALID, "unknown dtype %d", dtype);
+  hgpu_array* a = nullptr;
+  int rc = new_dense(ctx, dtype, rank, shape, &a);
+  if (rc) return rc;
+  size_t bytes = (size_t)nelem(a) * dtype_size(dtype);
+  if (bytes > 0) {
+    if (!host) {
+      hgpu_release(a);
+      return fail(ctx, HGPU_ERR_INVALID, "null host pointer");
+    }
+    LaunchGuard lg(ctx);
+    // Pageable source: hipMemcpyAsync stages it and the host block may be
+    // reused by the caller as soon as we return, so wait for the copy.
+    hipError_t e = hipMemcpyAsync(data_ptr(a), host, bytes, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+      hgpu_release(a);
+      return check_hip(ctx, e, "upload");
+    }
+  }
+  *out = a;
+  return HGPU_OK;
+}
+
+int hgpu_download(hgpu_ctx* ctx, const hgpu_array* a, void* host) {
+  if (!ctx || !a) return HGPU_ERR_INVALID;
+  int64_t n = nelem(a);
+  if (n == 0) return HGPU_OK;
+  if (!host) return fail(ctx, HGPU_ERR_INVALID, "null host pointer");
+  size_t bytes = (size_t)n * dtype_size(a->dtype);
+  hgpu_array* dense = nullptr;
+  const hgpu_array* src = a;
+  if (!is_dense(a)) {
+    int rc = hgpu_materialize(ctx, a, &dense);
+    if (rc) return rc;
+    src = dense;
+  }
+  hipError_t e;
+  {
+    LaunchGuard lg(ctx);
+    e = hipMemcpyAsync(host, data_ptr(src), bytes, hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  }
+  if (dense) hgpu_release(dense);
+  return check_hip(ctx, e, "download");
+}
+
+int hgpu_read_scalar(hgpu_ctx* ctx, const hgpu_array* a, void* host) {
+  if (!ctx || !a || !host) return HGPU_ERR_INVALID;
+  if (nelem(a) != 1) return fail(ctx, HGPU_ERR_INVALID, "read_scalar of an array with %lld elements", (long long)nelem(a));
+  LaunchGuard lg(ctx);
+  hipError_t e = hipMemcpyAsync(host, data_ptr(a), dtype_size(a->dtype), hipMemcpyDeviceToHost, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  return check_hip(ctx, e, "read_scalar");
+}
+
+int hgpu_retain(hgpu_array* a) {
+  if (!a) return HGPU_ERR_INVALID;
+  a->refs.fetch_add(1);
+  return HGPU_OK;
+}
+
+int hgpu_release(hgpu_array* a) {
+  if (!a) return HGPU_OK;
+  if (a->refs.fetch_sub(1) == 1) {
+    buffer_release(a->buf);
+    delete a;
+  }
+  return HGPU_OK;
+}
+
+int hgpu_rank(const hgpu_array* a) { return a ? a->rank : -1; }
+int hgpu_dtype_of(const hgpu_array* a) { return a ? a->dtype : -1; }
+int64_t hgpu_size(const hgpu_array* a) { return a ? nelem(a) : -1; }
+int hgpu_shape(const hgpu_array* a, int64_t* s) {
+  if (!a || !s) return HGPU_ERR_INVALID;
+  for (int i = 0; i < a->rank; ++i) s[i] = a->shape[i];
+  return HGPU_OK;
+}
+int hgpu_strides(const hgpu_array* a, int64_t* s) {
+  if (!a || !s) return HGPU_ERR_INVALID;
+  for (int i = 0; i < a->rank; ++i) s[i] = a->strides[i];
+  return HGPU_OK;
+}
+int hgpu_is_dense(const hgpu_array* a) { return a && is_dense(a) ? 1 : 0; }
+
+/* -------------------------------------------------------------------- views */
+
+int hgpu_transpose(hgpu_ctx* ctx, const hgpu_array* a, int nperm, const int* perm, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (nperm < 0 || nperm > a->rank) return fail(ctx, HGPU_ERR_INVALID, "transpose: permutation longer than rank");
+  int64_t sh[HGPU_MAX_RANK], st[HGPU_MAX_RANK];
+  bool seen[HGPU_MAX_RANK] = {false};
+  for (int i = 0; i < a->rank; ++i) {
+    int s = i;
+    if (i < nperm) {
+      s = perm[i];
+      if (s < 0 || s >= nperm || seen[s]) return fail(ctx, HGPU_ERR_INVALID, "transpose: not a permutation");
+      seen[s] = true;
+    }
+    sh[i] = a->shape[s];
+    st[i] = a->strides[s];
+  }
+  *out = new_view(ctx, a->buf, a->dtype, a->rank, sh, st, a->offset);
+  return HGPU_OK;
+}
+
+// Tries to express `shape` as a view of a; fills strides on success.
+static bool reshape_view(const hgpu_array* a, int rank, const int64_t* shape, int64_t* st) {
+  // Merge a's dims into maximal contiguous runs, then split them.
+  int64_t rsh[HGPU_MAX_RANK], rst[HGPU_MAX_RANK];
+  int nr = 0;
+  for (int i = 0; i < a->rank; ++i) {
+    if (a->shape[i] == 1) continue;
+    if (nr > 0 && rst[nr - 1] == a->strides[i] * a->shape[i]) {
+      rsh[nr - 1] *= a->shape[i];
+      rst[nr - 1] = a->strides[i];
+    } else {
+      rsh[nr] = a->shape[i];
+      rst[nr] = a->strides[i];
+      nr++;
+    }
+  }
+  int r = 0;
+  int64_t rem = nr > 0 ? rsh[0] : 1;  // elements of the current run not yet consumed (outer part)
+  for (int i = 0; i < rank; ++i) {
+    int64_t s = shape[i];
+    if (s == 1) { st[i] = 0; continue; }
+    if (r >= nr) return false;
+    if (rem % s != 0) return false;
+    rem /= s;
+    st[i] = rst[r] * rem;
+    if (rem == 1) {
+      r++;
+      rem = r < nr ? rsh[r] : 1;
+    }
+  }
+  return r == nr;
+}
+
+int hgpu_reshape(hgpu_ctx* ctx, const hgpu_array* a, int rank, const int64_t* shape, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (rank < 0 || rank > HGPU_MAX_RANK) return fail(ctx, HGPU_ERR_INVALID, "reshape: bad rank");
+  int64_t n = 1;
+  for (int i = 0; i < rank; ++i) n *= shape[i];
+  if (n != nelem(a)) return fail(ctx, HGPU_ERR_INVALID, "reshape: %lld elements into %lld", (long long)nelem(a), (long long)n);
+  int64_t st[HGPU_MAX_RANK];
+  if (n == 0) {
+    dense_strides(rank, shape, st);
+    *out = new_view(ctx, nullptr, a->dtype, rank, shape, st, 0);
+    return HGPU_OK;
+  }
+  if (reshape_view(a, rank, shape, st)) {
+    *out = new_view(ctx, a->buf, a->dtype, rank, shape, st, a->offset);
+    return HGPU_OK;
+  }
+  hgpu_array* d = nullptr;
+  int rc = hgpu_materialize(ctx, a, &d);
+  if (rc) return rc;
+  dense_strides(rank, shape, st);
+  *out = new_view(ctx, d->buf, d->dtype, rank, shape, st, d->offset);
+  hgpu_release(d);
+  return HGPU_OK;
+}
+
+int hgpu_slice(hgpu_ctx* ctx, const hgpu_array* a, int dim, int64_t start, int64_t len, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (dim < 0 || dim >= a->rank) return fail(ctx, HGPU_ERR_INVALID, "slice: dim %d of rank %d", dim, a->rank);
+  if (start < 0 || len < 0 || start + len > a->shape[dim])
+    return fail(ctx, HGPU_ERR_INVALID, "slice: [%lld,+%lld) outside extent %lld", (long long)start, (long long)len, (long long)a->shape[dim]);
+  int64_t sh[HGPU_MAX_RANK];
+  for (int i = 0; i < a->rank; ++i) sh[i] = a->shape[i];
+  sh[dim] = len;
+  *out = new_view(ctx, len == 0 ? nullptr : a->buf, a->dtype, a->rank, sh, a->strides, a->offset + start * a->strides[dim]);
+  return HGPU_OK;
+}
+
+int hgpu_reverse(hgpu_ctx* ctx, const hgpu_array* a, int dim, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (dim < 0 || dim >= a->rank) return fail(ctx, HGPU_ERR_INVALID, "reverse: dim %d of rank %d", dim, a->rank);
+  int64_t st[HGPU_MAX_RANK];
+  for (int i = 0; i < a->rank; ++i) st[i] = a->strides[i];
+  int64_t off = a->offset;
+  if (a->shape[dim] > 0) off += (a->shape[dim] - 1) * a->strides[dim];
+  st[dim] = -st[dim];
+  *out = new_view(ctx, a->buf, a->dtype, a->rank, a->shape, st, off);
+  return HGPU_OK;
+}
+
+int hgpu_replicate(hgpu_ctx* ctx, const hgpu_array* a, int np, const int64_t* pre, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (np < 0 || np + a->rank > HGPU_MAX_RANK) return fail(ctx, HGPU_ERR_INVALID, "replicate: rank too large");
+  int64_t sh[HGPU_MAX_RANK], st[HGPU_MAX_RANK];
+  bool empty = false;
+  for (int i = 0; i < np; ++i) {
+    if (pre[i] < 0) return fail(ctx, HGPU_ERR_INVALID, "replicate: negative extent");
+    sh[i] = pre[i];
+    st[i] = 0;
+    if (pre[i] == 0) empty = true;
+  }
+  for (int i = 0; i < a->rank; ++i) {
+    sh[np + i] = a->shape[i];
+    st[np + i] = a->strides[i];
+  }
+  *out = new_view(ctx, empty ? nullptr : a->buf, a->dtype, np + a->rank, sh, st, a->offset);
+  return HGPU_OK;
+}
+
+int hgpu_index_prefix(hgpu_ctx* ctx, const hgpu_array* a, int n, const int64_t* ix, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (n < 0 || n > a->rank) return fail(ctx, HGPU_ERR_INVALID, "index: %d indices into rank %d", n, a->rank);
+  int64_t off = a->offset;
+  bool oob = false;
+  for (int i = 0; i < n; ++i) {
+    if (ix[i] < 0 || ix[i] >= a->shape[i]) oob = true;
+    off += ix[i] * a->strides[i];
+  }
+  if (oob) return new_zeros(ctx, a->dtype, a->rank - n, a->shape + n, out);
+  *out = new_view(ctx, a->buf, a->dtype, a->rank - n, a->shape + n, a->strides + n, off);
+  return HGPU_OK;
+}
+
+int hgpu_as_strided(hgpu_ctx* ctx, const hgpu_array* a, int rank, const int64_t* shape, const int64_t* strides,
+                    int64_t offset, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (rank < 0 || rank > HGPU_MAX_RANK) return fail(ctx, HGPU_ERR_INVALID, "as_strided: bad rank");
+  int64_t lo = a->offset + offset, hi = lo;
+  bool empty = false;
+  for (int i = 0; i < rank; ++i) {
+    if (shape[i] < 0) return fail(ctx, HGPU_ERR_INVALID, "as_strided: negative extent");
+    if (shape[i] == 0) { empty = true; continue; }
+    int64_t span = (shape[i] - 1) * strides[i];
+    if (span > 0) hi += span; else lo += span;
+  }
+  if (!empty) {
+    if (!a->buf) return fail(ctx, HGPU_ERR_INVALID, "as_strided: view of an empty array");
+    // The addressed range must stay inside the elements a itself addresses.
+    int64_t alo = a->offset, ahi = a->offset;
+    for (int i = 0; i < a->rank; ++i) {
+      int64_t span = (a->shape[i] - 1) * a->strides[i];
+      if (span > 0) ahi += span; else alo += span;
+    }
+    if (lo < alo || hi > ahi)
+      return fail(ctx, HGPU_ERR_INVALID, "as_strided: elements [%lld,%lld] outside the source view [%lld,%lld]",
+                  (long long)lo, (long long)hi, (long long)alo, (long long)ahi);
+  }
+  *out = new_view(ctx, empty ? nullptr : a->buf, a->dtype, rank, shape, strides, a->offset + offset);
+  return HGPU_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,289 @@
+/* hordead_gpu.h -- C ABI of the MI355X (gfx950) tensor backend for horde-ad.
+ *
+ * This is the boundary a `Gpu` carrier of horde-ad's tensor classes binds with
+ * `foreign import ccall`: one entry point per array primitive that the
+ * `BaseTensor Concrete` instance (src/HordeAd/Core/OpsConcrete.hs:97-775)
+ * obtains from ox-arrays or from its own Haskell index loops.  Everything is
+ * plain C: opaque handles, pointers, sizes, an `int` status.  No exception,
+ * no C++ type and no torch type crosses it.
+ *
+ * Model
+ *   - `hgpu_ctx`   one device + one in-order HIP stream + a caching allocator.
+ *   - `hgpu_array` an immutable strided VIEW (dtype, rank, shape, element
+ *                  strides, element offset) of a reference-counted device
+ *                  buffer.  Strides may be 0 (replicate) or negative (reverse),
+ *                  exactly the freedom ox-arrays' arrays have
+ *                  (src/HordeAd/Core/CarriersConcrete.hs:150-155).
+ *   - Logical element order is row-major over `shape`; every compute entry
+ *     point returns a dense row-major array.
+ *   - All work is enqueued on the context's stream; only `hgpu_download`,
+ *     `hgpu_read_scalar`, `hgpu_compare_all` and `hgpu_sync` wait for it.
+ *   - `hgpu_release` may be called from any thread (it is what a Haskell
+ *     `ForeignPtr` finalizer calls); the buffer returns to the allocator and
+ *     may be reused by later enqueued work, which the in-order stream makes
+ *     safe.
+ *
+ * Status codes: 0 = ok; otherwise `hgpu_last_error` holds a message.  Indices
+ * out of bounds in index/gather/scatter/onehot are NOT errors: they have the
+ * reference's defined semantics (zeros / skipped), see each entry point.
+ */
+#ifndef HORDEAD_GPU_H
+#define HORDEAD_GPU_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct hgpu_ctx hgpu_ctx;
+typedef struct hgpu_array hgpu_array;
+
+#define HGPU_MAX_RANK 16
+
+enum hgpu_status {
+  HGPU_OK = 0,
+  HGPU_ERR_INVALID = 1,     /* shape/dtype/argument mismatch (the reference calls `error`) */
+  HGPU_ERR_OOM = 2,         /* device allocation failed */
+  HGPU_ERR_DEVICE = 3,      /* a HIP call failed */
+  HGPU_ERR_UNSUPPORTED = 4  /* valid request this build has no kernel for */
+};
+
+/* Scalar types: the reference's whitelist (src/HordeAd/Core/Types.hs:135-150,
+ * OpsConcrete.hs:1043-1058).  Haskell `Int` is I64; `CInt` is I32; Bool is one
+ * byte holding 0 or 1. */
+enum hgpu_dtype {
+  HGPU_F64 = 0, HGPU_F32 = 1, HGPU_I64 = 2, HGPU_I32 = 3,
+  HGPU_I16 = 4, HGPU_I8 = 5, HGPU_BOOL = 6
+};
+
+/* Unary opcodes: OpCodeNum1 / OpCode1 (src/HordeAd/Core/AstInterpret.hs:394-421). */
+enum hgpu_op1 {
+  HGPU_NEG = 0, HGPU_ABS, HGPU_SIGNUM,
+  HGPU_RECIP, HGPU_EXP, HGPU_LOG, HGPU_SQRT, HGPU_SIN, HGPU_COS, HGPU_TAN,
+  HGPU_ASIN, HGPU_ACOS, HGPU_ATAN, HGPU_SINH, HGPU_COSH, HGPU_TANH,
+  HGPU_ASINH, HGPU_ACOSH, HGPU_ATANH,
+  HGPU_NOT,           /* notB on Bool (AstInterpret.hs:329-335) */
+  HGPU_OP1_COUNT
+};
+
+/* Binary opcodes: + and * (AstInterpret.hs:187-188), OpCode2 (:423-429),
+ * OpCodeIntegral2 (:431-435) with the divisor-0 rule of Types.hs:394-419
+ * (quotH a 0 = a on scalars; arrays replace a 0 divisor by 1,
+ * CarriersConcrete.hs:40-56,140-144 -- the two rules agree: quot a 1 = a, and
+ * differ for remH: scalar remH a 0 = a, array remH a 0 = rem a 1 = 0; the
+ * array rule is HGPU_REM, the scalar rule is HGPU_REM_SCALAR). */
+enum hgpu_op2 {
+  HGPU_ADD = 0, HGPU_MUL, HGPU_SUB,
+  HGPU_DIV, HGPU_POW, HGPU_LOGBASE, HGPU_ATAN2,
+  HGPU_QUOT, HGPU_REM, HGPU_REM_SCALAR,
+  HGPU_MIN, HGPU_MAX,
+  HGPU_AND,           /* &&* on Bool (AstInterpret.hs:336-344) */
+  HGPU_OP2_COUNT
+};
+
+/* Comparison opcodes (Types.hs:442-452). */
+enum hgpu_cmp { HGPU_LEQ = 0, HGPU_EQ = 1, HGPU_LT = 2 };
+
+/* Conversion modes for hgpu_convert. */
+enum hgpu_conv {
+  HGPU_CONV_CAST = 0,   /* realToFrac / fromIntegral (OpsConcrete.hs:456-532) */
+  HGPU_CONV_FLOOR = 1   /* floor: float -> integer (OpsConcrete.hs:455) */
+};
+
+/* ---------------------------------------------------------------- context */
+
+/* Creates a context on HIP device `device` (one stream, default priority).
+ * No reference counterpart: `Concrete` needs no state (OpsConcrete.hs:97). */
+int hgpu_init(int device, hgpu_ctx** ctx);
+/* Waits for the stream and frees every cached device block.  Arrays still
+ * alive keep their buffers until released. */
+int hgpu_shutdown(hgpu_ctx* ctx);
+/* Blocks until all enqueued work is complete. */
+int hgpu_sync(hgpu_ctx* ctx);
+/* Message of the last failed call made on this context by any thread. */
+const char* hgpu_last_error(hgpu_ctx* ctx);
+/* Allocator statistics: bytes held by live arrays, bytes reserved from the
+ * device (live + cached), number of device allocations made so far. */
+int hgpu_mem_stats(hgpu_ctx* ctx, uint64_t* in_use, uint64_t* reserved, uint64_t* n_device_allocs);
+/* The stream all work is enqueued on, as a `hipStream_t` cast to void*. */
+void* hgpu_stream(hgpu_ctx* ctx);
+/* When `limit` >= 0, the next `limit`-th device allocation and all later ones
+ * fail with HGPU_ERR_OOM (host-forced fault injection for tests of the error
+ * path); a negative value switches it off. */
+int hgpu_inject_alloc_failure(hgpu_ctx* ctx, int64_t limit);
+
+/* ----------------------------------------------------------------- memory */
+
+/* tkconcrete/tsconcrete/tconcrete (OpsConcrete.hs:120-124): identity on the
+ * CPU, an upload here.  `host` holds prod(shape) elements in row-major order
+ * and is borrowed for the call only. */
+int hgpu_upload(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape,
+                const void* host, hgpu_array** out);
+/* Nested.stoVector (OpsConcrete.hs:144-164, `tstoListLinear`): writes the
+ * logical row-major contents of the view to `host`; waits for the stream. */
+int hgpu_download(hgpu_ctx* ctx, const hgpu_array* a, void* host);
+/* Reads the single element of a one-element array (unConcrete on a scalar,
+ * `kfromS`); waits for the stream.  `host` receives one value of a's dtype. */
+int hgpu_read_scalar(hgpu_ctx* ctx, const hgpu_array* a, void* host);
+int hgpu_retain(hgpu_array* a);
+int hgpu_release(hgpu_array* a);
+
+/* sshape/rshape/xshape/tftk (OpsConcrete.hs:99-106): host metadata only. */
+int hgpu_rank(const hgpu_array* a);
+int hgpu_dtype_of(const hgpu_array* a);
+int64_t hgpu_size(const hgpu_array* a);
+int hgpu_shape(const hgpu_array* a, int64_t* shape_out);
+int hgpu_strides(const hgpu_array* a, int64_t* strides_out);
+/* 1 when the view is dense row-major (what `stoVector` can return without a copy). */
+int hgpu_is_dense(const hgpu_array* a);
+
+/* ------------------------------------------------- views (no element traffic) */
+
+/* tstranspose (OpsConcrete.hs:647-649): result dim i = source dim perm[i] for
+ * i < nperm; the remaining dims keep their place. */
+int hgpu_transpose(hgpu_ctx* ctx, const hgpu_array* a, int nperm, const int* perm, hgpu_array** out);
+/* tsreshape (OpsConcrete.hs:650-652): a view when the strides allow it, else a
+ * dense copy. */
+int hgpu_reshape(hgpu_ctx* ctx, const hgpu_array* a, int rank, const int64_t* shape, hgpu_array** out);
+/* tsslice (OpsConcrete.hs:641-643) generalised to any dim: elements
+ * [start, start+len) of dimension `dim`. */
+int hgpu_slice(hgpu_ctx* ctx, const hgpu_array* a, int dim, int64_t start, int64_t len, hgpu_array** out);
+/* tsreverse (OpsConcrete.hs:644-646) generalised to any dim. */
+int hgpu_reverse(hgpu_ctx* ctx, const hgpu_array* a, int dim, hgpu_array** out);
+/* tsreplicateN / tsreplicate0N (OpsConcrete.hs:243-246): new leading dims of
+ * stride 0. */
+int hgpu_replicate(hgpu_ctx* ctx, const hgpu_array* a, int nprefix, const int64_t* prefix_shape, hgpu_array** out);
+/* tsindex / tindexZSScalar (OpsConcrete.hs:1477-1490): fixes the first n dims.
+ * Any index out of bounds gives an all-zero array of the remaining shape. */
+int hgpu_index_prefix(hgpu_ctx* ctx, const hgpu_array* a, int n, const int64_t* ix, hgpu_array** out);
+/* A gather whose index function is affine in the position and provably in
+ * bounds (tgatherZSScalar, OpsConcrete.hs:1654-1665, with f linear): the result
+ * is a view of a's buffer with the given shape, strides (in elements) and
+ * offset relative to a's first element.  Refused (HGPU_ERR_INVALID) when any
+ * addressed element would lie outside a's buffer. */
+int hgpu_as_strided(hgpu_ctx* ctx, const hgpu_array* a, int rank, const int64_t* shape,
+                    const int64_t* strides, int64_t offset, hgpu_array** out);
+
+/* ----------------------------------------------------------------- compute */
+
+/* Dense copy of a view in logical order (what ox-arrays does before handing a
+ * strided array to a C kernel that wants a vector). */
+int hgpu_materialize(hgpu_ctx* ctx, const hgpu_array* a, hgpu_array** out);
+/* Zero-extends every dimension d by lo[d] elements in front and hi[d] behind
+ * (the zero rows a gather with out-of-bounds indices produces,
+ * OpsConcrete.hs:1488-1490; also slice's VJP, DeltaEval.hs:569-575). */
+int hgpu_pad(hgpu_ctx* ctx, const hgpu_array* a, const int64_t* lo, const int64_t* hi, hgpu_array** out);
+
+/* Elementwise Num/Fractional/Floating/IntegralH instances of arrays
+ * (CarriersConcrete.hs:40-56,333-343), dispatched from AstN1S/AstR1S/AstPlusS/
+ * AstTimesS/AstR2S/AstI2S (AstInterpret.hs:187-194).  Operands have equal
+ * shape and dtype. */
+int hgpu_ewise1(hgpu_ctx* ctx, int op1, const hgpu_array* a, hgpu_array** out);
+int hgpu_ewise2(hgpu_ctx* ctx, int op2, const hgpu_array* a, const hgpu_array* b, hgpu_array** out);
+/* Elementwise comparison giving a BOOL array: the lane-batched form of
+ * AstLeqK / AstLeqS (AstInterpret.hs:345-366). */
+int hgpu_compare(hgpu_ctx* ctx, int cmp, const hgpu_array* a, const hgpu_array* b, hgpu_array** out);
+/* Whole-array comparison, one Bool: EqH/OrdH Concrete (CarriersConcrete.hs:
+ * 310-331) -- lexicographic over the row-major element sequence.  Waits. */
+int hgpu_compare_all(hgpu_ctx* ctx, int cmp, const hgpu_array* a, const hgpu_array* b, int* result);
+/* Elementwise conditional, cond BOOL: the lane-batched form of kcond / ifH
+ * (OpsConcrete.hs:113-119). */
+int hgpu_select(hgpu_ctx* ctx, const hgpu_array* cond, const hgpu_array* a, const hgpu_array* b, hgpu_array** out);
+/* tsfloor / tsfromIntegral / tscast / tkcast (OpsConcrete.hs:352-368,455-532). */
+int hgpu_convert(hgpu_ctx* ctx, const hgpu_array* a, int dtype, int mode, hgpu_array** out);
+
+/* out[o] = sum_r a[o,r] * b[o,r]  (b == NULL: b = 1), o ranging over the first
+ * n_keep dims and r over the rest.  With the free views above this one entry
+ * point is tssum / tssumN / tssum0 (OpsConcrete.hs:215-230, b NULL, summed dims
+ * transposed behind), tsdot0 (:231-232), tsdot1In (:233-235), tsmatvecmul
+ * (:236) and tsmatmul2 (:237-242, which the reference itself defines as
+ * dot1In over replicated and transposed views).  Floating-point summation
+ * order is unspecified (as it is in ox-arrays); integers are exact. */
+int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array** out);
+
+/* tsargMin / tsargMax (OpsConcrete.hs:533-534, targMinS :1712-1746): index of
+ * the first minimal / maximal element along the LAST dim; result I64 of shape
+ * init(shape). */
+int hgpu_argminmax_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_array** out);
+/* tsiota (OpsConcrete.hs:535-536): [0, 1, ..., n-1] of the given dtype. */
+int hgpu_iota(hgpu_ctx* ctx, int64_t n, int dtype, hgpu_array** out);
+/* tsappend / trconcat (OpsConcrete.hs:623-625,638-640): concatenation along
+ * dim 0 of n arrays that agree on all other dims. */
+int hgpu_concat(hgpu_ctx* ctx, int n, const hgpu_array* const* parts, hgpu_array** out);
+
+/* tsgather / tgatherZSScalar (OpsConcrete.hs:1621-1665):
+ *   out[m.., n..] = src[ix[0][m..], ..., ix[n_ix-1][m..], n..]
+ * where every ix[j] is an I64 array (any view) of shape shm, and shn is the
+ * rest of src's shape after its first n_ix dims.  A position with any index
+ * out of bounds yields zeros (OpsConcrete.hs:923-926,1488-1490,1504-1506).
+ * Pure data movement: bit-exact. */
+int hgpu_gather(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array* const* ix,
+                int rank_m, const int64_t* shm, hgpu_array** out);
+/* tsscatter / tscatterZSScalar (OpsConcrete.hs:1581-1619):
+ *   out = 0;  out[ix[0][m..], ..., ix[n_ix-1][m..], n..] += src[m.., n..]
+ * src has shape shm ++ shn (rank_m leading dims are shm), out has shape
+ * shp ++ shn with shp given (n_ix dims).  Positions with an index out of
+ * bounds are skipped (OpsConcrete.hs:944-950).  Integers exact; floating
+ * point sums may be associated differently from the reference's ascending
+ * row-major order.  `flags`: bit 0 = the caller guarantees distinct
+ * positions map to distinct destinations (plain stores suffice). */
+int hgpu_scatter_add(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array* const* ix,
+                     int rank_m, const int64_t* shp, int flags, hgpu_array** out);
+/* tsoneHot / toneHotS (OpsConcrete.hs:1516-1525): zeros of shape shp ++ shape(v)
+ * with v written at prefix index ix; all zeros when ix is out of bounds. */
+int hgpu_onehot(hgpu_ctx* ctx, const hgpu_array* v, int n, const int64_t* ix, const int64_t* shp, hgpu_array** out);
+
+/* ------------------------------------------------------------- api table */
+
+/* The same entry points as a table of function pointers, so that host code
+ * written against the table can be pointed at another provider of this ABI
+ * (the test suite points it at a CPU checker). */
+typedef struct hgpu_api {
+  int (*init)(int, hgpu_ctx**);
+  int (*shutdown)(hgpu_ctx*);
+  int (*sync)(hgpu_ctx*);
+  const char* (*last_error)(hgpu_ctx*);
+  int (*upload)(hgpu_ctx*, int, int, const int64_t*, const void*, hgpu_array**);
+  int (*download)(hgpu_ctx*, const hgpu_array*, void*);
+  int (*read_scalar)(hgpu_ctx*, const hgpu_array*, void*);
+  int (*retain)(hgpu_array*);
+  int (*release)(hgpu_array*);
+  int (*rank)(const hgpu_array*);
+  int (*dtype_of)(const hgpu_array*);
+  int64_t (*size)(const hgpu_array*);
+  int (*shape)(const hgpu_array*, int64_t*);
+  int (*strides)(const hgpu_array*, int64_t*);
+  int (*is_dense)(const hgpu_array*);
+  int (*transpose)(hgpu_ctx*, const hgpu_array*, int, const int*, hgpu_array**);
+  int (*reshape)(hgpu_ctx*, const hgpu_array*, int, const int64_t*, hgpu_array**);
+  int (*slice)(hgpu_ctx*, const hgpu_array*, int, int64_t, int64_t, hgpu_array**);
+  int (*reverse)(hgpu_ctx*, const hgpu_array*, int, hgpu_array**);
+  int (*replicate)(hgpu_ctx*, const hgpu_array*, int, const int64_t*, hgpu_array**);
+  int (*index_prefix)(hgpu_ctx*, const hgpu_array*, int, const int64_t*, hgpu_array**);
+  int (*as_strided)(hgpu_ctx*, const hgpu_array*, int, const int64_t*, const int64_t*, int64_t, hgpu_array**);
+  int (*materialize)(hgpu_ctx*, const hgpu_array*, hgpu_array**);
+  int (*pad)(hgpu_ctx*, const hgpu_array*, const int64_t*, const int64_t*, hgpu_array**);
+  int (*ewise1)(hgpu_ctx*, int, const hgpu_array*, hgpu_array**);
+  int (*ewise2)(hgpu_ctx*, int, const hgpu_array*, const hgpu_array*, hgpu_array**);
+  int (*compare)(hgpu_ctx*, int, const hgpu_array*, const hgpu_array*, hgpu_array**);
+  int (*compare_all)(hgpu_ctx*, int, const hgpu_array*, const hgpu_array*, int*);
+  int (*select)(hgpu_ctx*, const hgpu_array*, const hgpu_array*, const hgpu_array*, hgpu_array**);
+  int (*convert)(hgpu_ctx*, const hgpu_array*, int, int, hgpu_array**);
+  int (*contract)(hgpu_ctx*, const hgpu_array*, const hgpu_array*, int, hgpu_array**);
+  int (*argminmax_last)(hgpu_ctx*, const hgpu_array*, int, hgpu_array**);
+  int (*iota)(hgpu_ctx*, int64_t, int, hgpu_array**);
+  int (*concat)(hgpu_ctx*, int, const hgpu_array* const*, hgpu_array**);
+  int (*gather)(hgpu_ctx*, const hgpu_array*, int, const hgpu_array* const*, int, const int64_t*, hgpu_array**);
+  int (*scatter_add)(hgpu_ctx*, const hgpu_array*, int, const hgpu_array* const*, int, const int64_t*, int, hgpu_array**);
+  int (*onehot)(hgpu_ctx*, const hgpu_array*, int, const int64_t*, const int64_t*, hgpu_array**);
+} hgpu_api;
+
+/* The table of this library's own entry points. */
+const hgpu_api* hgpu_get_api(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HORDEAD_GPU_H */

@@ -1,0 +1,350 @@
+"""Parity of the gfx950 library with the CPU checker, primitive by primitive,
+through the C ABI.  Data movement, integers, indices and Bool results must be
+bit-exact; floating point is held to the stated normwise relative tolerance
+(fp64 1e-10, fp32 1e-5 -- reductions are associated differently on the device).
+"""
+import numpy as np
+import pytest
+
+from conftest import Pair, assert_same, capi
+
+pytestmark = pytest.mark.gpu
+
+RNG = np.random.default_rng(99)
+TOL = {np.dtype(np.float64): 1e-10, np.dtype(np.float32): 1e-5}
+ALL = [np.float64, np.float32, np.int64, np.int32, np.int16, np.int8]
+
+
+def rnd(shape, dtype):
+    k = np.dtype(dtype).kind
+    if k == "f":
+        return RNG.uniform(-2, 2, shape).astype(dtype)
+    if k == "b":
+        return RNG.integers(0, 2, shape).astype(bool)
+    return RNG.integers(-50, 50, shape).astype(dtype)
+
+
+def random_view(both, dtype, rank=None, max_extent=7, steps=4):
+    """Uploads a random dense array to both providers and derives the same random
+    chain of views (transpose / slice / reverse / replicate) on each."""
+    rank = rank or int(RNG.integers(1, 5))
+    shape = [int(RNG.integers(1, max_extent)) for _ in range(rank)]
+    p = both.upload(rnd(shape, dtype))
+    for _ in range(steps):
+        shape = list(p.shape)
+        kind = int(RNG.integers(0, 4))
+        if kind == 0 and len(shape) >= 2:
+            n = int(RNG.integers(2, len(shape) + 1))
+            p = p.transpose([int(i) for i in RNG.permutation(n)])
+        elif kind == 1 and shape:
+            d = int(RNG.integers(0, len(shape)))
+            if shape[d] > 1:
+                s = int(RNG.integers(0, shape[d] - 1))
+                ln = int(RNG.integers(1, shape[d] - s + 1))
+                p = p.slice(d, s, ln)
+        elif kind == 2 and shape:
+            p = p.reverse(int(RNG.integers(0, len(shape))))
+        elif kind == 3 and len(shape) < 5:
+            p = p.replicate([int(RNG.integers(1, 4))])
+    return p
+
+
+def like(both, p, dtype, view=True):
+    """Another operand of p's shape: a fresh dense array, or a stride-0 broadcast."""
+    shape = p.shape
+    if view and len(shape) >= 1 and RNG.integers(0, 3) == 0:
+        return both.upload(rnd(shape[1:], dtype)).replicate([shape[0]])
+    return both.upload(rnd(shape, dtype))
+
+
+def test_upload_download_views(both):
+    for dt in ALL + [np.bool_]:
+        for _ in range(6):
+            p = random_view(both, dt)
+            assert_same(p, what="view download")
+            assert_same(p.materialize())
+    p = both.upload(rnd((3, 0, 4), np.float64))
+    assert_same(p.transpose([2, 0, 1]))
+    assert_same(both.upload(np.float32(2.5)).replicate([3, 2]))
+
+
+def test_reshape_view_or_copy(both, gpu):
+    x = rnd((4, 6, 5), np.float64)
+    p = both.upload(x)
+    for shp in ([24, 5], [4, 30], [2, 2, 3, 2, 5], [120], [4, 6, 5, 1]):
+        assert_same(p.reshape(shp))
+    t = p.transpose([1, 0])
+    for shp in ([6, 20], [24, 5], [6, 2, 2, 5]):
+        assert_same(t.reshape(shp))
+    # a reshape that the strides allow costs no allocation
+    a = gpu.upload(x)
+    n0 = gpu.mem_stats()[2]
+    v = a.transpose([1, 0]).reshape([6, 2, 2, 5])
+    assert gpu.mem_stats()[2] == n0 and not v.is_dense
+    r = both.upload(rnd((3,), np.float64)).replicate([4])
+    assert_same(r.reshape([12]))
+    assert_same(r.reshape([2, 6]))
+    assert_same(p.reverse(2).reshape([24, 5]))
+    assert_same(p.reverse(2).reshape([4, 30]))
+
+
+def test_index_pad_onehot_as_strided(both):
+    p = random_view(both, np.float64, rank=4, steps=3)
+    sh = p.shape
+    assert_same(p.index_prefix([sh[0] - 1, 0]))
+    assert_same(p.index_prefix([sh[0], 0]))       # out of bounds: zeros
+    assert_same(p.index_prefix([0, -1]))
+    assert_same(p.index_prefix([]))
+    assert_same(p.pad([1, 0, 2, 0], [0, 3, 0, 1]))
+    assert_same(p.onehot([1, 2], [3, 4]))
+    assert_same(p.onehot([3, 2], [3, 4]))          # out of bounds: all zeros
+    v = both.upload(rnd((11,), np.float32))
+    assert_same(v.as_strided([8, 4], [1, 1], 0))
+    assert_same(v.as_strided([4, 3], [2, -1], 2))
+    for a in v.arrays:
+        with pytest.raises(capi.HgpuError):
+            a.as_strided([9, 4], [1, 1], 0)
+        with pytest.raises(capi.HgpuError):
+            a.as_strided([2], [1], -1)
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_unary_float(both, dt):
+    ops = ["neg", "abs", "signum", "recip", "exp", "sin", "cos", "tan", "atan", "sinh", "cosh", "tanh", "asinh"]
+    for op in ops:
+        p = random_view(both, dt)
+        assert_same(p.ewise1(op), TOL[np.dtype(dt)], op)
+    x = rnd((5, 33), dt)
+    pos = both.upload(np.abs(x) + dt(0.25))
+    unit = both.upload((x / dt(2.5)).astype(dt))
+    for op in ("sqrt", "log"):
+        assert_same(pos.ewise1(op), TOL[np.dtype(dt)], op)
+    for op in ("asin", "acos", "atanh"):
+        assert_same(unit.ewise1(op), TOL[np.dtype(dt)], op)
+    assert_same(both.upload(np.abs(x) + dt(1.25)).ewise1("acosh"), TOL[np.dtype(dt)], "acosh")
+    # dense fast path incl. a tail that is not a multiple of the vector width
+    d = both.upload(rnd((1031,), dt))
+    assert_same(d.ewise1("sin"), TOL[np.dtype(dt)])
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_binary_float(both, dt):
+    tol = TOL[np.dtype(dt)]
+    for op in ("add", "mul", "sub", "div", "atan2", "min", "max"):
+        for _ in range(3):
+            p = random_view(both, dt)
+            q = like(both, p, dt)
+            assert_same(p.ewise2(op, q), tol, op)
+    x = rnd((4, 9), dt)
+    px, py = both.upload(np.abs(x) + dt(0.5)), both.upload(np.abs(x[::-1]) + dt(0.5))
+    assert_same(px.ewise2("pow", both.upload(x)), tol, "pow")
+    assert_same(px.ewise2("logbase", py), 100 * tol, "logbase")
+    # dense paths: dense*dense, dense*broadcast scalar, odd length
+    a, b = both.upload(rnd((3001,), dt)), both.upload(rnd((3001,), dt))
+    s = both.upload(dt(1.5)).replicate([3001])
+    assert_same(a.ewise2("mul", b), tol)
+    assert_same(a.ewise2("add", s), tol)
+    assert_same(s.ewise2("sub", a), tol)
+    assert_same(s.ewise2("mul", s), tol)
+
+
+@pytest.mark.parametrize("dt", [np.int64, np.int32, np.int16, np.int8])
+def test_integer_exact(both, dt):
+    for op in ("add", "mul", "sub", "quot", "rem", "rem_scalar", "min", "max"):
+        p = random_view(both, dt)
+        q = like(both, p, dt)       # contains zeros: the divisor-0 rules apply
+        assert_same(p.ewise2(op, q), 0.0, op)
+    for op in ("neg", "abs", "signum"):
+        assert_same(random_view(both, dt).ewise1(op), 0.0, op)
+    for a in random_view(both, dt).arrays:
+        with pytest.raises(capi.HgpuError):
+            a.ewise1("exp")
+
+
+def test_compare_select_bool(both):
+    for dt in ALL:
+        p = random_view(both, dt)
+        q = like(both, p, dt)
+        for c in ("leq", "eq", "lt"):
+            m = p.compare(c, q)
+            assert_same(m)
+            assert_same(m.ewise1("not"))
+            assert_same(m.ewise2("and", p.compare("leq", p)))
+            assert_same(m.select(p, q))
+        assert p.compare_all("eq", p) == [True, True]
+        assert p.compare_all("lt", p) == [False, False]
+        r = p.compare_all("leq", q)
+        assert r[0] == r[1]
+        r = p.compare_all("lt", q)
+        assert r[0] == r[1]
+    a = both.upload(np.array([1, 2, 3, 4], np.int64))
+    b = both.upload(np.array([1, 2, 4, 0], np.int64))
+    assert a.compare_all("leq", b) == [True, True] and b.compare_all("leq", a) == [False, False]
+
+
+def test_convert(both):
+    f = both.upload(np.array([-2.5, -0.5, 0.0, 0.5, 2.5, 7.99, 1e6 + 0.75]))
+    for dt in (capi.I64, capi.I32):
+        assert_same(f.convert(dt, 1))
+    assert_same(f.convert(capi.F32, 0))
+    for src in ALL:
+        p = random_view(both, src)
+        for dst in (capi.F64, capi.F32, capi.I64, capi.I32, capi.I16, capi.I8):
+            if np.dtype(src).kind == "f" and dst >= capi.I64:
+                continue  # float -> int goes through floor
+            assert_same(p.convert(dst, 0), 0.0, (src, dst))
+
+
+@pytest.mark.parametrize("dt", ALL)
+def test_contract_random_views(both, dt):
+    tol = TOL.get(np.dtype(dt), 0.0)
+    for _ in range(12):
+        p = random_view(both, dt)
+        k = int(RNG.integers(0, len(p.shape) + 1))
+        assert_same(p.contract(None, k), tol, ("sum", p.shape, k))
+        q = like(both, p, dt)
+        assert_same(p.contract(q, k), tol, ("dot", p.shape, k))
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32, np.int32])
+def test_contract_shapes_of_the_workloads(both, dt):
+    tol = TOL.get(np.dtype(dt), 0.0)
+    # long flat reductions (split into chunks + second pass)
+    x = both.upload(rnd((300007,), dt))
+    assert_same(x.contract(None, 0), tol)
+    assert_same(x.contract(x, 0), tol)
+    # sum over the outer dim of a matrix (lane-per-output) and over the inner dim (wave-per-output)
+    m = both.upload(rnd((513, 130), dt))
+    assert_same(m.transpose([1, 0]).contract(None, 1), tol)
+    assert_same(m.contract(None, 1), tol)
+    # few outputs, long rows
+    w = both.upload(rnd((3, 70001), dt))
+    assert_same(w.contract(w, 1), tol)
+    # tsmatmul2 as the reference defines it: dot1In over replicated + transposed views
+    m1, m2 = both.upload(rnd((37, 65), dt)), both.upload(rnd((65, 29), dt))
+    lhs = m1.replicate([29]).transpose([1, 0])
+    rhs = m2.replicate([37]).transpose([0, 2, 1])
+    assert_same(lhs.contract(rhs, 2), tol)
+    # tssumN over two leading dims after transposition
+    t = both.upload(rnd((6, 7, 40, 9), dt))
+    assert_same(t.transpose([2, 3, 0, 1]).contract(None, 2), tol)
+    # empty reductions give zeros
+    assert_same(both.upload(rnd((4, 0), dt)).contract(None, 1))
+    assert_same(both.upload(rnd((0, 4), dt)).contract(None, 1))
+
+
+def test_argminmax_iota_concat(both):
+    for dt in ALL:
+        p = random_view(both, dt, rank=3)
+        assert_same(p.argminmax_last(True))
+        assert_same(p.argminmax_last(False))
+    t = both.upload(np.array([[3, 1, 1, 3], [0, 0, 5, 5]], np.int32))   # ties: first occurrence
+    assert_same(t.argminmax_last(True))
+    assert_same(t.argminmax_last(False))
+    for dt in (capi.F64, capi.F32, capi.I64, capi.I32):
+        assert_same(both.iota(1000, dt))
+    assert_same(both.iota(0, capi.I64))
+    parts = [random_view(both, np.float32, rank=1, steps=0)]
+    base = parts[0].shape
+    parts = [both.upload(rnd((k,) + base[1:], np.float32)) for k in (2, 0, 5)] + [both.upload(rnd((3,) + base[1:], np.float32)).reverse(0)]
+    assert_same(both.concat(parts))
+
+
+def ix_arrays(both, shm, extents, oob=True, view=False):
+    out = []
+    for e in extents:
+        lo, hi = (-1, e + 1) if oob else (0, e)
+        if view and len(shm) >= 2 and RNG.integers(0, 2) == 0:
+            out.append(both.upload(RNG.integers(lo, hi, shm[1:]).astype(np.int64)).replicate([shm[0]]))
+        else:
+            out.append(both.upload(RNG.integers(lo, hi, shm).astype(np.int64)))
+    return out
+
+
+@pytest.mark.parametrize("dt", ALL + [np.bool_])
+def test_gather_exact(both, dt):
+    for _ in range(8):
+        src = random_view(both, dt, rank=int(RNG.integers(1, 5)))
+        n_ix = int(RNG.integers(0, len(src.shape) + 1))
+        shm = [int(RNG.integers(1, 6)) for _ in range(int(RNG.integers(0, 4)))]
+        ix = ix_arrays(both, shm, src.shape[:n_ix], view=True)
+        assert_same(both.gather(src, ix, shm), 0.0, (src.shape, n_ix, shm))
+    src = both.upload(rnd((4, 5), dt))
+    assert_same(both.gather(src, ix_arrays(both, [0, 3], [4]), [0, 3]))
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32, np.int64, np.int32])
+def test_scatter(both, dt):
+    tol = TOL.get(np.dtype(dt), 0.0)
+    for _ in range(8):
+        src = random_view(both, dt, rank=int(RNG.integers(1, 5)))
+        rank_m = int(RNG.integers(0, len(src.shape) + 1))
+        shp = [int(RNG.integers(1, 6)) for _ in range(int(RNG.integers(0, 3)))]
+        ix = ix_arrays(both, list(src.shape[:rank_m]), shp, view=True)
+        assert_same(both.scatter_add(src, ix, rank_m, shp), tol, (src.shape, rank_m, shp))
+    # heavy collisions: 20000 positions into 7 cells
+    src = both.upload(rnd((20000, 2), dt))
+    ix = ix_arrays(both, [20000], [7])
+    assert_same(both.scatter_add(src, ix, 1, [7]), tol)
+    # distinct destinations, caller-guaranteed: plain stores
+    perm = both.upload(RNG.permutation(500).astype(np.int64))
+    src = both.upload(rnd((500, 3), dt))
+    assert_same(both.scatter_add(src, [perm], 1, [500], flags=1))
+
+
+def test_scatter_small_ints(both, gpu):
+    perm = both.upload(RNG.permutation(64).astype(np.int64))
+    for dt in (np.int16, np.int8):
+        src = both.upload(rnd((64,), dt))
+        assert_same(both.scatter_add(src, [perm], 1, [64], flags=1))
+        with pytest.raises(capi.HgpuError) as e:
+            gpu.scatter_add(src.arrays[0], [perm.arrays[0]], 1, [64])
+        assert e.value.code == 4
+
+
+def test_gather_scatter_adjoint_large(both):
+    """<gather x f, y> == <x, scatter y f> on a conv-sized window pattern."""
+    x = both.upload(rnd((48, 48), np.float64))
+    shm = [48, 5]
+    i = np.add.outer(np.arange(48), np.arange(5)).astype(np.int64)   # i + k, runs out of bounds
+    ix = [both.upload(i)]
+    y = both.upload(rnd((48, 5, 48), np.float64))
+    g = both.gather(x, ix, shm)
+    s = both.scatter_add(y, ix, 2, [48])
+    assert_same(g)
+    assert_same(s, 1e-10)
+    lhs = g.contract(y, 0).numpy()
+    rhs = x.contract(s, 0).numpy()
+    assert abs(lhs[0] - rhs[0]) <= 1e-10 * abs(lhs[0])
+    assert abs(lhs[0] - lhs[1]) <= 1e-10 * abs(lhs[1])
+
+
+def test_errors_and_allocator(gpu):
+    a = gpu.upload(rnd((4, 5), np.float64))
+    b = gpu.upload(rnd((4, 6), np.float64))
+    with pytest.raises(capi.HgpuError) as e:
+        a.ewise2("add", b)
+    assert e.value.code == 1 and "shape" in str(e.value)
+    with pytest.raises(capi.HgpuError):
+        a.ewise2("add", gpu.upload(rnd((4, 5), np.float32)))
+    with pytest.raises(capi.HgpuError):
+        a.contract(b, 1)
+    with pytest.raises(capi.HgpuError):
+        a.transpose([0, 0])
+    with pytest.raises(capi.HgpuError):
+        a.slice(1, 3, 4)
+    # blocks are recycled: repeating the same op needs no new device allocation
+    c = a.ewise1("sin")
+    del c
+    n0 = gpu.mem_stats()[2]
+    for _ in range(10):
+        c = a.ewise1("sin")
+        del c
+    assert gpu.mem_stats()[2] == n0
+    # a device allocation that fails surfaces as a status, not a crash
+    gpu.check(gpu.lib.inject_alloc_failure(gpu.h, 0))
+    with pytest.raises(capi.HgpuError) as e:
+        a.ewise1("cos")
+    assert e.value.code == 2
+    gpu.check(gpu.lib.inject_alloc_failure(gpu.h, -1))
+    assert np.allclose(a.ewise1("cos").numpy(), np.cos(a.numpy()))
