@@ -1,0 +1,179 @@
+// extern "C" surface of the host layer (include/hordead_host.h): handles in,
+// status codes out; C++ exceptions stop here.
+#include "hordead_host.h"
+
+#include <cstring>
+
+#include "host.hpp"
+
+using namespace hordead;
+
+struct hh_ctx {
+  Backend be;
+  Tape tape;
+  std::string err;
+  bool owns_ctx = true;
+  hh_ctx() : tape(&be) {}
+};
+struct hh_val { D d; };
+struct hh_ix { Ix x; };
+
+namespace {
+
+template <typename F>
+int guarded(hh_ctx* c, F f) {
+  try {
+    f();
+    return HGPU_OK;
+  } catch (const HostError& e) {
+    if (c) c->err = e.what();
+    return e.code;
+  } catch (const std::exception& e) {
+    if (c) c->err = e.what();
+    return HGPU_ERR_INVALID;
+  }
+}
+
+Shape mk(int n, const int64_t* p) { return n > 0 ? Shape(p, p + n) : Shape(); }
+hh_val* box(const D& d) { return new hh_val{d}; }
+hh_ix* boxi(const Ix& x) { return new hh_ix{x}; }
+std::vector<Ix> ixs(int n, hh_ix* const* p) {
+  std::vector<Ix> v;
+  for (int i = 0; i < n; ++i) v.push_back(p[i]->x);
+  return v;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hh_create(const hgpu_api* api, int device, hh_ctx** out) {
+  if (!api || !out) return HGPU_ERR_INVALID;
+  hh_ctx* c = new hh_ctx;
+  c->be.api = api;
+  c->be.ctx = nullptr;
+  int rc = api->init(device, &c->be.ctx);
+  if (rc) { delete c; return rc; }
+  *out = c;
+  return HGPU_OK;
+}
+
+int hh_create_gpu(int device, hh_ctx** out) { return hh_create(hgpu_get_api(), device, out); }
+
+int hh_destroy(hh_ctx* c) {
+  if (!c) return HGPU_OK;
+  c->tape.recs.clear();
+  c->be.iota_cache.clear();
+  c->be.const_cache.clear();
+  c->be.api->shutdown(c->be.ctx);
+  // The context object stays: values released later still point at it.
+  return HGPU_OK;
+}
+
+const char* hh_last_error(hh_ctx* c) { return c ? c->err.c_str() : "no context"; }
+int hh_sync(hh_ctx* c) { return guarded(c, [&] { c->be.check(c->be.api->sync(c->be.ctx)); }); }
+hgpu_ctx* hh_array_ctx(hh_ctx* c) { return c ? c->be.ctx : nullptr; }
+int hh_tape_reset(hh_ctx* c) { c->tape.recs.clear(); return HGPU_OK; }
+
+int hh_upload(hh_ctx* c, int dtype, int rank, const int64_t* shape, const void* host, int rg, hh_val** out) {
+  return guarded(c, [&] {
+    T t = upload(&c->be, dtype, mk(rank, shape), host);
+    *out = box(rg ? c->tape.input(t) : d_const(t));
+  });
+}
+
+int hh_from_array(hh_ctx* c, hgpu_array* a, int rg, hh_val** out) {
+  return guarded(c, [&] {
+    c->be.check(c->be.api->retain(a));
+    T t(&c->be, a);
+    *out = box(rg ? c->tape.input(t) : d_const(t));
+  });
+}
+
+int hh_constant(hh_ctx* c, int dtype, double value, int rank, const int64_t* shape, hh_val** out) {
+  return guarded(c, [&] { *out = box(d_const(broadcast_scalar(constant(&c->be, dtype, value), mk(rank, shape)))); });
+}
+
+int hh_array(hh_val* v, hgpu_array** out) {
+  if (!v || !out) return HGPU_ERR_INVALID;
+  v->d.primal.be()->api->retain(v->d.primal.h());
+  *out = v->d.primal.h();
+  return HGPU_OK;
+}
+
+int hh_download(hh_ctx* c, hh_val* v, void* host) {
+  return guarded(c, [&] { c->be.check(c->be.api->download(c->be.ctx, v->d.primal.h(), host)); });
+}
+int hh_val_rank(hh_val* v) { return v->d.primal.rank(); }
+int hh_val_dtype(hh_val* v) { return v->d.primal.dtype(); }
+int hh_val_shape(hh_val* v, int64_t* s) {
+  Shape sh = v->d.primal.shape();
+  std::copy(sh.begin(), sh.end(), s);
+  return HGPU_OK;
+}
+int hh_free(hh_val* v) { delete v; return HGPU_OK; }
+
+int hh_backward(hh_ctx* c, hh_val* out, hh_val* dt, int n, hh_val* const* inputs, hh_val** grads) {
+  return guarded(c, [&] {
+    std::vector<D> ins;
+    for (int i = 0; i < n; ++i) ins.push_back(inputs[i]->d);
+    std::vector<T> g = c->tape.backward(out->d, dt->d.primal, ins);
+    for (int i = 0; i < n; ++i) grads[i] = box(d_const(g[(size_t)i]));
+  });
+}
+
+#define HH_OP(body) return guarded(c, [&] { *out = box(body); })
+
+int hh_ewise1(hh_ctx* c, int op, hh_val* a, hh_val** out) { HH_OP(d_ewise1(c->tape, op, a->d)); }
+int hh_ewise2(hh_ctx* c, int op, hh_val* a, hh_val* b, hh_val** out) { HH_OP(d_ewise2(c->tape, op, a->d, b->d)); }
+int hh_compare(hh_ctx* c, int cmp, hh_val* a, hh_val* b, hh_val** out) { HH_OP(d_const(compare(cmp, a->d.primal, b->d.primal))); }
+int hh_compare_all(hh_ctx* c, int cmp, hh_val* a, hh_val* b, int* result) {
+  return guarded(c, [&] { *result = compare_all(cmp, a->d.primal, b->d.primal) ? 1 : 0; });
+}
+int hh_select(hh_ctx* c, hh_val* cond, hh_val* a, hh_val* b, hh_val** out) { HH_OP(d_select(c->tape, cond->d.primal, a->d, b->d)); }
+int hh_convert(hh_ctx* c, hh_val* a, int dtype, int mode, hh_val** out) { HH_OP(d_convert(c->tape, a->d, dtype, mode)); }
+int hh_tssumN(hh_ctx* c, hh_val* t, int k, hh_val** out) { HH_OP(d_tssumN(c->tape, t->d, k)); }
+int hh_tssum0(hh_ctx* c, hh_val* t, hh_val** out) { HH_OP(d_tssum0(c->tape, t->d)); }
+int hh_tsdot0(hh_ctx* c, hh_val* a, hh_val* b, hh_val** out) { HH_OP(d_tsdot0(c->tape, a->d, b->d)); }
+int hh_tsdot1In(hh_ctx* c, hh_val* a, hh_val* b, hh_val** out) { HH_OP(d_tsdot1In(c->tape, a->d, b->d)); }
+int hh_tsmatvecmul(hh_ctx* c, hh_val* m, hh_val* v, hh_val** out) {
+  HH_OP(d_tsdot1In(c->tape, m->d, d_tsreplicateN(c->tape, v->d, {m->d.primal.shape().at(0)})));
+}
+int hh_tsmatmul2(hh_ctx* c, hh_val* a, hh_val* b, hh_val** out) { HH_OP(d_tsmatmul2(c->tape, a->d, b->d)); }
+int hh_tsreplicateN(hh_ctx* c, hh_val* t, int n, const int64_t* shm, hh_val** out) { HH_OP(d_tsreplicateN(c->tape, t->d, mk(n, shm))); }
+int hh_tsappend(hh_ctx* c, hh_val* a, hh_val* b, hh_val** out) { HH_OP(d_tsappend(c->tape, a->d, b->d)); }
+int hh_tsslice(hh_ctx* c, hh_val* t, int64_t i, int64_t n, hh_val** out) { HH_OP(d_tsslice(c->tape, t->d, i, n)); }
+int hh_tsreverse(hh_ctx* c, hh_val* t, hh_val** out) { HH_OP(d_tsreverse(c->tape, t->d)); }
+int hh_tstranspose(hh_ctx* c, hh_val* t, int n, const int* perm, hh_val** out) {
+  HH_OP(d_tstranspose(c->tape, t->d, n > 0 ? std::vector<int>(perm, perm + n) : std::vector<int>()));
+}
+int hh_tsreshape(hh_ctx* c, hh_val* t, int rank, const int64_t* shape, hh_val** out) { HH_OP(d_tsreshape(c->tape, t->d, mk(rank, shape))); }
+int hh_tsindex(hh_ctx* c, hh_val* t, int n, const int64_t* ix, hh_val** out) { HH_OP(d_tsindex(c->tape, t->d, mk(n, ix))); }
+int hh_tsargminmax(hh_ctx* c, hh_val* t, int want_max, hh_val** out) { HH_OP(d_const(argminmax_last(t->d.primal, want_max != 0))); }
+int hh_tsiota(hh_ctx* c, int64_t n, int dtype, hh_val** out) { HH_OP(d_const(tsiota(&c->be, n, dtype))); }
+
+#define HH_IX(body) return guarded(c, [&] { *out = boxi(body); })
+
+int hh_ix_var(hh_ctx* c, int rank_m, const int64_t* shm, int d, hh_ix** out) { HH_IX(ix_var(&c->be, mk(rank_m, shm), d)); }
+int hh_ix_const(hh_ctx* c, int rank_m, const int64_t* shm, int dtype, double v, hh_ix** out) { HH_IX(ix_const(&c->be, mk(rank_m, shm), dtype, v)); }
+int hh_ix_lift(hh_ctx* c, int rank_m, const int64_t* shm, hh_val* s, hh_ix** out) { HH_IX(ix_lift(mk(rank_m, shm), s->d.primal)); }
+int hh_ix_op1(hh_ctx* c, int op, hh_ix* a, hh_ix** out) { HH_IX(ix_op1(&c->be, op, a->x)); }
+int hh_ix_op2(hh_ctx* c, int op, hh_ix* a, hh_ix* b, hh_ix** out) { HH_IX(ix_op2(&c->be, op, a->x, b->x)); }
+int hh_ix_compare(hh_ctx* c, int cmp, hh_ix* a, hh_ix* b, hh_ix** out) { HH_IX(ix_compare(&c->be, cmp, a->x, b->x)); }
+int hh_ix_select(hh_ctx* c, hh_ix* cond, hh_ix* a, hh_ix* b, hh_ix** out) { HH_IX(ix_select(&c->be, cond->x, a->x, b->x)); }
+int hh_ix_convert(hh_ctx* c, hh_ix* a, int dtype, int mode, hh_ix** out) { HH_IX(ix_convert(&c->be, a->x, dtype, mode)); }
+int hh_ix_index0(hh_ctx* c, hh_val* t, int n, hh_ix* const* ix, hh_ix** out) { HH_IX(ix_index0(&c->be, t->d.primal, ixs(n, ix))); }
+int hh_ix_argminmax(hh_ctx* c, hh_val* t, int n, hh_ix* const* ix, int want_max, hh_ix** out) {
+  HH_IX(ix_argminmax(&c->be, t->d.primal, ixs(n, ix), want_max != 0));
+}
+int hh_ix_free(hh_ix* x) { delete x; return HGPU_OK; }
+int hh_ix_is_affine(hh_ix* x) { return x && x->x.affine ? 1 : 0; }
+
+int hh_tsgather(hh_ctx* c, hh_val* src, int rank_m, const int64_t* shm, int n_ix, hh_ix* const* ix, hh_val** out) {
+  HH_OP(d_tsgather(c->tape, src->d, mk(rank_m, shm), ixs(n_ix, ix)));
+}
+int hh_tsscatter(hh_ctx* c, hh_val* src, int rank_m, int n_ix, const int64_t* shp, hh_ix* const* ix, hh_val** out) {
+  HH_OP(d_tsscatter(c->tape, src->d, rank_m, mk(n_ix, shp), ixs(n_ix, ix)));
+}
+
+}  // extern "C"

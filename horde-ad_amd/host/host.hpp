@@ -1,0 +1,210 @@
+// Host layer above the C ABI of include/hordead_gpu.h: the `Gpu` carrier and
+// its tensor-class operations, named after the methods of horde-ad's
+// `BaseTensor` class (src/HordeAd/Core/Ops.hs:297-1255) whose `Concrete`
+// instance (src/HordeAd/Core/OpsConcrete.hs:97-775) they stand beside.
+//
+// The layer is written against the table `hgpu_api`, never against a concrete
+// library, so the same object code drives the gfx950 library in production and
+// any other provider of the ABI a test hands in.
+#pragma once
+#include <cstdint>
+#include <functional>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "hordead_gpu.h"
+
+namespace hordead {
+
+using Shape = std::vector<int64_t>;
+
+struct HostError : std::runtime_error {
+  int code;
+  HostError(int c, const std::string& m) : std::runtime_error(m), code(c) {}
+};
+
+class T;
+struct ArrHolder;
+
+// One provider of the array ABI plus a context on it.
+struct Backend {
+  const hgpu_api* api;
+  hgpu_ctx* ctx;
+  std::map<std::pair<int, int64_t>, std::shared_ptr<ArrHolder>> iota_cache;   // (dtype, n)
+  std::map<std::pair<int, uint64_t>, std::shared_ptr<ArrHolder>> const_cache; // (dtype, value bits)
+  void check(int rc) const;
+};
+
+struct ArrHolder {
+  Backend* be;
+  hgpu_array* h;
+  // Small integer arrays that came from the host keep their values: index
+  // functions that look constants up in them can then be folded on the host.
+  std::shared_ptr<std::vector<int64_t>> host_i64;
+  ArrHolder(Backend* b, hgpu_array* a) : be(b), h(a) {}
+  ~ArrHolder() { if (h) be->api->release(h); }
+  ArrHolder(const ArrHolder&) = delete;
+};
+
+// `Gpu (TKS sh r)`: an immutable strided view on the device.  Scalars
+// (`TKScalar r`) are rank-0 views, so that they never force a device sync.
+class T {
+ public:
+  T() {}
+  T(Backend* be, hgpu_array* h) : p_(std::make_shared<ArrHolder>(be, h)) {}
+  explicit T(std::shared_ptr<ArrHolder> p) : p_(std::move(p)) {}
+  const std::shared_ptr<ArrHolder>& holder() const { return p_; }
+  bool valid() const { return (bool)p_; }
+  Backend* be() const { return p_->be; }
+  hgpu_array* h() const { return p_->h; }
+  int rank() const { return be()->api->rank(h()); }
+  int dtype() const { return be()->api->dtype_of(h()); }
+  int64_t size() const { return be()->api->size(h()); }
+  Shape shape() const;
+  Shape strides() const;
+  const std::shared_ptr<std::vector<int64_t>>& host_i64() const { return p_->host_i64; }
+  void set_host_i64(std::shared_ptr<std::vector<int64_t>> v) { p_->host_i64 = std::move(v); }
+
+ private:
+  std::shared_ptr<ArrHolder> p_;
+};
+
+// ---- array primitives (one ABI call each) ---------------------------------
+T upload(Backend* be, int dtype, const Shape& shape, const void* host);
+T constant(Backend* be, int dtype, double value);                 // cached rank-0 array
+T constant_i(Backend* be, int dtype, int64_t value);
+T iota(Backend* be, int64_t n, int dtype);                         // cached
+T transpose(const T& a, const std::vector<int>& perm);
+T reshape(const T& a, const Shape& shape);
+T slice(const T& a, int dim, int64_t start, int64_t len);
+T reverse(const T& a, int dim);
+T replicate(const T& a, const Shape& prefix);
+T index_prefix(const T& a, const Shape& ix);
+T as_strided(const T& a, const Shape& shape, const Shape& strides, int64_t offset);
+T materialize(const T& a);
+T pad(const T& a, const Shape& lo, const Shape& hi);
+T ewise1(int op, const T& a);
+T ewise2(int op, const T& a, const T& b);
+T compare(int cmp, const T& a, const T& b);
+bool compare_all(int cmp, const T& a, const T& b);
+T select(const T& c, const T& a, const T& b);
+T convert(const T& a, int dtype, int mode);
+T contract(const T& a, const T* b, int n_keep);
+T argminmax_last(const T& a, bool want_max);
+T concat(const std::vector<T>& parts);
+T gather_raw(const T& src, const std::vector<T>& ix, const Shape& shm);
+T scatter_raw(const T& src, const std::vector<T>& ix, int rank_m, const Shape& shp, int flags);
+T onehot(const T& v, const Shape& ix, const Shape& shp);
+T zeros(Backend* be, int dtype, const Shape& shape);               // stride-0 view of a cached 0
+T broadcast_scalar(const T& s, const Shape& shape);                // tsreplicate0N
+
+// ---- BaseTensor-named operations (Ops.hs line of each method in the .cpp) --
+T tssum(const T& t);                       // sum over the outermost dim
+T tssumN(const T& t, int k);               // sum over the k outermost dims
+T tssum0(const T& t);
+T tsdot0(const T& a, const T& b);
+T tsdot1In(const T& a, const T& b);        // contraction over the innermost dim
+T tsmatvecmul(const T& m, const T& v);
+T tsmatmul2(const T& m1, const T& m2);
+T tsreplicate(const T& t, int64_t k);
+T tsreplicateN(const T& t, const Shape& shm);
+T tsreplicate0N(const T& scalar, const Shape& sh);
+T tsappend(const T& a, const T& b);
+T tsslice(const T& t, int64_t i, int64_t n);
+T tsreverse(const T& t);
+T tstranspose(const T& t, const std::vector<int>& perm);
+T tsreshape(const T& t, const Shape& sh);
+T tsindex(const T& t, const Shape& ix);    // concrete (host) indices
+T tsoneHot(const T& v, const Shape& ix, const Shape& shp);
+T tsfloor(const T& t, int dtype);
+T tsfromIntegral(const T& t, int dtype);
+T tscast(const T& t, int dtype);
+T tsargMin(const T& t);
+T tsargMax(const T& t);
+T tsiota(Backend* be, int64_t n, int dtype);
+
+// ---- lane-batched scalars: the `IntOf Gpu` an index function is applied to --
+//
+// horde-ad hands gather/scatter/build an index FUNCTION over scalars
+// (Ops.hs:689-705); `Concrete` calls it once per position
+// (OpsConcrete.hs:1581-1665).  Here the function is called ONCE with symbolic
+// position variables; every scalar it computes is an `Ix`: a value for all
+// positions of the space `shm` at a time -- an affine form in the position
+// variables when that is provable (then gathers become strided views), or a
+// device array of shape shm otherwise.
+struct Ix {
+  Shape shm;                   // the position space this value ranges over
+  bool affine = false;
+  int64_t c0 = 0;              // affine: c0 + sum_d coef[d] * m_d
+  std::vector<int64_t> coef;
+  T arr;                       // otherwise: array of shape shm (any dtype, any strides)
+  int dtype = HGPU_I64;
+};
+
+Ix ix_var(Backend* be, const Shape& shm, int d);
+Ix ix_const(Backend* be, const Shape& shm, int dtype, double v);
+Ix ix_lift(const Shape& shm, const T& scalar);            // a rank-0 tensor seen from every position
+T ix_array(Backend* be, const Ix& x);                     // as a device array of shape shm
+Ix ix_op1(Backend* be, int op, const Ix& a);
+Ix ix_op2(Backend* be, int op, const Ix& a, const Ix& b);
+Ix ix_compare(Backend* be, int cmp, const Ix& a, const Ix& b);
+Ix ix_select(Backend* be, const Ix& c, const Ix& a, const Ix& b);   // kcond / ifH
+Ix ix_convert(Backend* be, const Ix& a, int dtype, int mode);
+Ix ix_index0(Backend* be, const T& t, const std::vector<Ix>& ix);   // tsindex0 at batched indices
+// kargMin / kargMax (t !$ ix): arg-extremum of the last dim of the batched partial index
+Ix ix_argminmax(Backend* be, const T& t, const std::vector<Ix>& ix, bool want_max);
+
+// tsgather (Ops.hs:701-705) / tsscatter (Ops.hs:689-693) with the index
+// function already applied to the symbolic positions.
+T tsgather(const T& src, const Shape& shm, const std::vector<Ix>& ix);
+T tsscatter(const T& src, int rank_m, const Shape& shp, const std::vector<Ix>& ix);
+
+// ---- dual numbers: reverse-mode differentiation over the carrier -----------
+//
+// Mirror of `ADVal target` + `gradientFromDelta` (OpsADVal.hs:44-60,
+// DeltaEval.hs:64-78,391-595) for the operations above: every operation on a
+// `D` runs the primal operation on the carrier and records the transposition
+// rule; `backward` plays the records in reverse.
+struct Tape;
+struct D {
+  T primal;
+  int node = -1;               // index into the tape; -1 = no derivative flows
+};
+
+struct Tape {
+  struct Rec {
+    std::function<void(const T& cot, std::vector<T>& slots)> back;
+  };
+  Backend* be;
+  std::vector<Rec> recs;
+  explicit Tape(Backend* b) : be(b) {}
+  D input(const T& t);                                     // differentiable leaf
+  int push(std::function<void(const T&, std::vector<T>&)> f);
+  // Cotangents of `inputs` given d(out) = dt.
+  std::vector<T> backward(const D& out, const T& dt, const std::vector<D>& inputs);
+};
+
+D d_const(const T& t);
+D d_ewise1(Tape& tp, int op, const D& a);
+D d_ewise2(Tape& tp, int op, const D& a, const D& b);
+D d_select(Tape& tp, const T& cond, const D& a, const D& b);
+D d_convert(Tape& tp, const D& a, int dtype, int mode);
+D d_tssumN(Tape& tp, const D& t, int k);
+D d_tssum0(Tape& tp, const D& t);
+D d_tsdot0(Tape& tp, const D& a, const D& b);
+D d_tsdot1In(Tape& tp, const D& a, const D& b);
+D d_tsmatmul2(Tape& tp, const D& a, const D& b);
+D d_tsreplicateN(Tape& tp, const D& t, const Shape& shm);
+D d_tsappend(Tape& tp, const D& a, const D& b);
+D d_tsslice(Tape& tp, const D& t, int64_t i, int64_t n);
+D d_tsreverse(Tape& tp, const D& t);
+D d_tstranspose(Tape& tp, const D& t, const std::vector<int>& perm);
+D d_tsreshape(Tape& tp, const D& t, const Shape& sh);
+D d_tsindex(Tape& tp, const D& t, const Shape& ix);
+D d_tsgather(Tape& tp, const D& src, const Shape& shm, const std::vector<Ix>& ix);
+D d_tsscatter(Tape& tp, const D& src, int rank_m, const Shape& shp, const std::vector<Ix>& ix);
+
+}  // namespace hordead

@@ -1,0 +1,547 @@
+// The `Gpu` carrier's array operations: thin wrappers over the ABI table, the
+// BaseTensor-named methods built from them, and the lane-batched evaluation of
+// index functions that turns gathers with affine indices into strided views.
+#include <algorithm>
+#include <cstring>
+#include <numeric>
+
+#include "host.hpp"
+
+namespace hordead {
+
+void Backend::check(int rc) const {
+  if (rc != HGPU_OK) throw HostError(rc, api->last_error(ctx));
+}
+
+Shape T::shape() const {
+  Shape s((size_t)rank());
+  if (!s.empty()) be()->api->shape(h(), s.data());
+  return s;
+}
+Shape T::strides() const {
+  Shape s((size_t)rank());
+  if (!s.empty()) be()->api->strides(h(), s.data());
+  return s;
+}
+
+static int64_t prod(const Shape& s, size_t from = 0) {
+  int64_t n = 1;
+  for (size_t i = from; i < s.size(); ++i) n *= s[i];
+  return n;
+}
+static const int64_t* ptr_or_dummy(const Shape& s) {
+  static const int64_t dummy = 0;
+  return s.empty() ? &dummy : s.data();
+}
+
+// ---------------------------------------------------------------- primitives
+
+T upload(Backend* be, int dtype, const Shape& shape, const void* host) {
+  hgpu_array* o = nullptr;
+  be->check(be->api->upload(be->ctx, dtype, (int)shape.size(), ptr_or_dummy(shape), host, &o));
+  T t(be, o);
+  // keep small integer tables on the host as well (see ArrHolder::host_i64)
+  int64_t n = prod(shape);
+  if (dtype == HGPU_I64 && n > 0 && n <= 65536) {
+    auto v = std::make_shared<std::vector<int64_t>>((size_t)n);
+    std::memcpy(v->data(), host, (size_t)n * 8);
+    t.set_host_i64(v);
+  }
+  return t;
+}
+
+static T upload_scalar(Backend* be, int dtype, double v, int64_t vi, bool integral) {
+  union { double d; float f; int64_t i64; int32_t i32; int16_t i16; int8_t i8; uint8_t b; } u;
+  std::memset(&u, 0, sizeof u);
+  switch (dtype) {
+    case HGPU_F64: u.d = integral ? (double)vi : v; break;
+    case HGPU_F32: u.f = integral ? (float)vi : (float)v; break;
+    case HGPU_I64: u.i64 = integral ? vi : (int64_t)v; break;
+    case HGPU_I32: u.i32 = (int32_t)(integral ? vi : (int64_t)v); break;
+    case HGPU_I16: u.i16 = (int16_t)(integral ? vi : (int64_t)v); break;
+    case HGPU_I8: u.i8 = (int8_t)(integral ? vi : (int64_t)v); break;
+    case HGPU_BOOL: u.b = (integral ? vi : (int64_t)v) != 0; break;
+    default: throw HostError(HGPU_ERR_INVALID, "unknown dtype");
+  }
+  return upload(be, dtype, {}, &u);
+}
+
+T constant(Backend* be, int dtype, double value) {
+  uint64_t bits;
+  std::memcpy(&bits, &value, 8);
+  auto key = std::make_pair(dtype, bits);
+  auto it = be->const_cache.find(key);
+  if (it != be->const_cache.end()) return T(it->second);
+  T t = upload_scalar(be, dtype, value, 0, false);
+  be->const_cache[key] = t.holder();
+  return t;
+}
+
+T constant_i(Backend* be, int dtype, int64_t value) {
+  if (dtype == HGPU_F64 || dtype == HGPU_F32) return constant(be, dtype, (double)value);
+  auto key = std::make_pair(dtype + 100, (uint64_t)value);
+  auto it = be->const_cache.find(key);
+  if (it != be->const_cache.end()) return T(it->second);
+  T t = upload_scalar(be, dtype, 0, value, true);
+  be->const_cache[key] = t.holder();
+  return t;
+}
+
+T iota(Backend* be, int64_t n, int dtype) {
+  auto key = std::make_pair(dtype, n);
+  auto it = be->iota_cache.find(key);
+  if (it != be->iota_cache.end()) return T(it->second);
+  hgpu_array* o = nullptr;
+  be->check(be->api->iota(be->ctx, n, dtype, &o));
+  T t(be, o);
+  be->iota_cache[key] = t.holder();
+  return t;
+}
+
+#define HD_OUT(call)                      \
+  hgpu_array* o__ = nullptr;              \
+  Backend* be__ = a.be();                 \
+  be__->check(be__->api->call);           \
+  return T(be__, o__)
+
+T transpose(const T& a, const std::vector<int>& perm) {
+  static const int dummy = 0;
+  HD_OUT(transpose(be__->ctx, a.h(), (int)perm.size(), perm.empty() ? &dummy : perm.data(), &o__));
+}
+T reshape(const T& a, const Shape& s) { HD_OUT(reshape(be__->ctx, a.h(), (int)s.size(), ptr_or_dummy(s), &o__)); }
+T slice(const T& a, int dim, int64_t start, int64_t len) { HD_OUT(slice(be__->ctx, a.h(), dim, start, len, &o__)); }
+T reverse(const T& a, int dim) { HD_OUT(reverse(be__->ctx, a.h(), dim, &o__)); }
+T replicate(const T& a, const Shape& pre) {
+  if (pre.empty()) return a;
+  HD_OUT(replicate(be__->ctx, a.h(), (int)pre.size(), pre.data(), &o__));
+}
+T index_prefix(const T& a, const Shape& ix) { HD_OUT(index_prefix(be__->ctx, a.h(), (int)ix.size(), ptr_or_dummy(ix), &o__)); }
+T as_strided(const T& a, const Shape& shape, const Shape& strides, int64_t offset) {
+  HD_OUT(as_strided(be__->ctx, a.h(), (int)shape.size(), ptr_or_dummy(shape), ptr_or_dummy(strides), offset, &o__));
+}
+T materialize(const T& a) { HD_OUT(materialize(be__->ctx, a.h(), &o__)); }
+T pad(const T& a, const Shape& lo, const Shape& hi) { HD_OUT(pad(be__->ctx, a.h(), ptr_or_dummy(lo), ptr_or_dummy(hi), &o__)); }
+T ewise1(int op, const T& a) { HD_OUT(ewise1(be__->ctx, op, a.h(), &o__)); }
+T ewise2(int op, const T& a, const T& b) { HD_OUT(ewise2(be__->ctx, op, a.h(), b.h(), &o__)); }
+T compare(int cmp, const T& a, const T& b) { HD_OUT(compare(be__->ctx, cmp, a.h(), b.h(), &o__)); }
+bool compare_all(int cmp, const T& a, const T& b) {
+  int r = 0;
+  a.be()->check(a.be()->api->compare_all(a.be()->ctx, cmp, a.h(), b.h(), &r));
+  return r != 0;
+}
+T select(const T& c, const T& a, const T& b) { HD_OUT(select(be__->ctx, c.h(), a.h(), b.h(), &o__)); }
+T convert(const T& a, int dtype, int mode) {
+  if (a.dtype() == dtype && mode == HGPU_CONV_CAST) return a;
+  HD_OUT(convert(be__->ctx, a.h(), dtype, mode, &o__));
+}
+T contract(const T& a, const T* b, int n_keep) { HD_OUT(contract(be__->ctx, a.h(), b ? b->h() : nullptr, n_keep, &o__)); }
+T argminmax_last(const T& a, bool want_max) { HD_OUT(argminmax_last(be__->ctx, a.h(), want_max ? 1 : 0, &o__)); }
+T concat(const std::vector<T>& parts) {
+  if (parts.empty()) throw HostError(HGPU_ERR_INVALID, "concat of nothing");
+  std::vector<const hgpu_array*> hs;
+  for (auto& p : parts) hs.push_back(p.h());
+  const T& a = parts[0];
+  HD_OUT(concat(be__->ctx, (int)hs.size(), hs.data(), &o__));
+}
+T gather_raw(const T& a, const std::vector<T>& ix, const Shape& shm) {
+  std::vector<const hgpu_array*> hs;
+  for (auto& p : ix) hs.push_back(p.h());
+  const hgpu_array* dummy = nullptr;
+  HD_OUT(gather(be__->ctx, a.h(), (int)hs.size(), hs.empty() ? &dummy : hs.data(), (int)shm.size(), ptr_or_dummy(shm), &o__));
+}
+T scatter_raw(const T& a, const std::vector<T>& ix, int rank_m, const Shape& shp, int flags) {
+  std::vector<const hgpu_array*> hs;
+  for (auto& p : ix) hs.push_back(p.h());
+  const hgpu_array* dummy = nullptr;
+  HD_OUT(scatter_add(be__->ctx, a.h(), (int)hs.size(), hs.empty() ? &dummy : hs.data(), rank_m, ptr_or_dummy(shp), flags, &o__));
+}
+T onehot(const T& a, const Shape& ix, const Shape& shp) {
+  HD_OUT(onehot(be__->ctx, a.h(), (int)ix.size(), ptr_or_dummy(ix), ptr_or_dummy(shp), &o__));
+}
+
+T broadcast_scalar(const T& s, const Shape& shape) {
+  if (s.size() != 1) throw HostError(HGPU_ERR_INVALID, "broadcast_scalar: not a scalar");
+  Shape st(shape.size(), 0);
+  for (auto e : shape)
+    if (e == 0) return replicate(reshape(s, {}), shape);
+  return as_strided(s, shape, st, 0);
+}
+
+T zeros(Backend* be, int dtype, const Shape& shape) { return broadcast_scalar(constant_i(be, dtype, 0), shape); }
+
+// ------------------------------------------------- BaseTensor-named methods
+
+static std::vector<int> rotate_left(int rank, int k) {  // [k..rank-1, 0..k-1]
+  std::vector<int> p((size_t)rank);
+  for (int i = 0; i < rank; ++i) p[(size_t)i] = (i + k) % rank;
+  return p;
+}
+
+// Ops.hs:511-516, OpsConcrete.hs:215-228
+T tssumN(const T& t, int k) {
+  int r = t.rank();
+  if (k < 0 || k > r) throw HostError(HGPU_ERR_INVALID, "tssumN: more summed dims than rank");
+  if (k == 0) return t;
+  return contract(k == r ? t : transpose(t, rotate_left(r, k)), nullptr, r - k);
+}
+T tssum(const T& t) { return tssumN(t, 1); }
+T tssum0(const T& t) { return contract(t, nullptr, 0); }                      // Ops.hs:517, OpsConcrete.hs:229
+T tsdot0(const T& a, const T& b) { return contract(a, &b, 0); }                // Ops.hs:519, OpsConcrete.hs:231
+T tsdot1In(const T& a, const T& b) {                                           // Ops.hs:522, OpsConcrete.hs:233
+  if (a.rank() < 1) throw HostError(HGPU_ERR_INVALID, "tsdot1In: rank 0");
+  return contract(a, &b, a.rank() - 1);
+}
+T tsmatvecmul(const T& m, const T& v) {                                        // OpsConcrete.hs:236
+  return tsdot1In(m, tsreplicate(v, m.shape().at(0)));
+}
+T tsmatmul2(const T& m1, const T& m2) {                                        // OpsConcrete.hs:237-242
+  Shape s1 = m1.shape(), s2 = m2.shape();
+  if (s1.size() != 2 || s2.size() != 2 || s1[1] != s2[0]) throw HostError(HGPU_ERR_INVALID, "tsmatmul2: shapes do not agree");
+  T lhs = transpose(tsreplicate(m1, s2[1]), {1, 0});       // [m, p, n]
+  T rhs = transpose(tsreplicate(m2, s1[0]), {0, 2, 1});    // [m, p, n]
+  return tsdot1In(lhs, rhs);
+}
+T tsreplicate(const T& t, int64_t k) { return replicate(t, {k}); }            // Ops.hs:548
+T tsreplicateN(const T& t, const Shape& shm) { return replicate(t, shm); }     // OpsConcrete.hs:243
+T tsreplicate0N(const T& s, const Shape& sh) { return broadcast_scalar(s, sh); }  // OpsConcrete.hs:245
+T tsappend(const T& a, const T& b) { return concat({a, b}); }                  // OpsConcrete.hs:638
+T tsslice(const T& t, int64_t i, int64_t n) { return slice(t, 0, i, n); }      // OpsConcrete.hs:641
+T tsreverse(const T& t) { return reverse(t, 0); }                              // OpsConcrete.hs:644
+T tstranspose(const T& t, const std::vector<int>& perm) { return transpose(t, perm); }  // OpsConcrete.hs:647
+T tsreshape(const T& t, const Shape& sh) { return reshape(t, sh); }            // OpsConcrete.hs:650
+T tsindex(const T& t, const Shape& ix) { return index_prefix(t, ix); }         // OpsConcrete.hs:1477
+T tsoneHot(const T& v, const Shape& ix, const Shape& shp) { return onehot(v, ix, shp); }  // OpsConcrete.hs:1516
+T tsfloor(const T& t, int dtype) { return convert(t, dtype, HGPU_CONV_FLOOR); }            // OpsConcrete.hs:455
+T tsfromIntegral(const T& t, int dtype) { return convert(t, dtype, HGPU_CONV_CAST); }      // OpsConcrete.hs:456
+T tscast(const T& t, int dtype) { return convert(t, dtype, HGPU_CONV_CAST); }              // OpsConcrete.hs:518
+T tsargMin(const T& t) { return argminmax_last(t, false); }                    // OpsConcrete.hs:533
+T tsargMax(const T& t) { return argminmax_last(t, true); }                     // OpsConcrete.hs:534
+T tsiota(Backend* be, int64_t n, int dtype) { return iota(be, n, dtype); }     // OpsConcrete.hs:535
+
+// ----------------------------------------------------- lane-batched scalars
+
+Ix ix_var(Backend*, const Shape& shm, int d) {
+  if (d < 0 || d >= (int)shm.size()) throw HostError(HGPU_ERR_INVALID, "ix_var: no such position variable");
+  Ix x;
+  x.shm = shm;
+  x.affine = true;
+  x.coef.assign(shm.size(), 0);
+  x.coef[(size_t)d] = 1;
+  return x;
+}
+
+Ix ix_const(Backend* be, const Shape& shm, int dtype, double v) {
+  Ix x;
+  x.shm = shm;
+  x.dtype = dtype;
+  if (dtype == HGPU_I64) {
+    x.affine = true;
+    x.coef.assign(shm.size(), 0);
+    x.c0 = (int64_t)v;
+  } else {
+    x.arr = broadcast_scalar(constant(be, dtype, v), shm);
+  }
+  return x;
+}
+
+Ix ix_lift(const Shape& shm, const T& scalar) {
+  Ix x;
+  x.shm = shm;
+  x.dtype = scalar.dtype();
+  x.arr = broadcast_scalar(scalar, shm);
+  return x;
+}
+
+static bool is_const(const Ix& x) {
+  if (!x.affine) return false;
+  for (size_t d = 0; d < x.coef.size(); ++d)
+    if (x.coef[d] != 0 && x.shm[d] > 1) return false;
+  return true;
+}
+
+T ix_array(Backend* be, const Ix& x) {
+  if (!x.affine) return x.arr;
+  T acc;
+  bool c0_done = false;
+  for (size_t d = 0; d < x.coef.size(); ++d) {
+    if (x.coef[d] == 0 || x.shm[d] <= 1) continue;
+    T v = iota(be, x.shm[d], HGPU_I64);
+    if (x.coef[d] != 1) v = ewise2(HGPU_MUL, v, broadcast_scalar(constant_i(be, HGPU_I64, x.coef[d]), {x.shm[d]}));
+    if (!c0_done && x.c0 != 0) {
+      v = ewise2(HGPU_ADD, v, broadcast_scalar(constant_i(be, HGPU_I64, x.c0), {x.shm[d]}));
+      c0_done = true;
+    }
+    Shape st(x.shm.size(), 0);
+    st[d] = 1;
+    T view = as_strided(v, x.shm, st, 0);
+    acc = acc.valid() ? ewise2(HGPU_ADD, acc, view) : view;
+  }
+  if (!acc.valid()) return broadcast_scalar(constant_i(be, HGPU_I64, x.c0), x.shm);
+  if (!c0_done && x.c0 != 0) acc = ewise2(HGPU_ADD, acc, broadcast_scalar(constant_i(be, HGPU_I64, x.c0), x.shm));
+  return acc;
+}
+
+static Ix from_array(const Shape& shm, const T& arr) {
+  Ix x;
+  x.shm = shm;
+  x.arr = arr;
+  x.dtype = arr.dtype();
+  return x;
+}
+
+static void same_space(const Ix& a, const Ix& b) {
+  if (a.shm != b.shm) throw HostError(HGPU_ERR_INVALID, "index values of different position spaces");
+  if (a.dtype != b.dtype) throw HostError(HGPU_ERR_INVALID, "index values of different scalar types");
+}
+
+Ix ix_op1(Backend* be, int op, const Ix& a) {
+  if (a.affine && op == HGPU_NEG) {
+    Ix r = a;
+    r.c0 = -r.c0;
+    for (auto& c : r.coef) c = -c;
+    return r;
+  }
+  return from_array(a.shm, ewise1(op, ix_array(be, a)));
+}
+
+Ix ix_op2(Backend* be, int op, const Ix& a, const Ix& b) {
+  same_space(a, b);
+  if (a.affine && b.affine) {
+    if (op == HGPU_ADD || op == HGPU_SUB) {
+      Ix r = a;
+      int64_t s = op == HGPU_ADD ? 1 : -1;
+      r.c0 += s * b.c0;
+      for (size_t d = 0; d < r.coef.size(); ++d) r.coef[d] += s * b.coef[d];
+      return r;
+    }
+    if (op == HGPU_MUL && (is_const(a) || is_const(b))) {
+      const Ix& k = is_const(a) ? a : b;
+      Ix r = is_const(a) ? b : a;
+      r.c0 *= k.c0;
+      for (auto& c : r.coef) c *= k.c0;
+      return r;
+    }
+    if (is_const(a) && is_const(b)) {  // fold the remaining integer operations (Types.hs:394-419)
+      int64_t x = a.c0, y = b.c0, v = 0;
+      bool folded = true;
+      switch (op) {
+        case HGPU_QUOT: v = y == 0 ? x : x / y; break;
+        case HGPU_REM: case HGPU_REM_SCALAR: v = y == 0 ? x : x % y; break;
+        case HGPU_MIN: v = std::min(x, y); break;
+        case HGPU_MAX: v = std::max(x, y); break;
+        default: folded = false;
+      }
+      if (folded) {
+        Ix r = a;
+        r.c0 = v;
+        std::fill(r.coef.begin(), r.coef.end(), 0);
+        return r;
+      }
+    }
+  }
+  return from_array(a.shm, ewise2(op, ix_array(be, a), ix_array(be, b)));
+}
+
+Ix ix_compare(Backend* be, int cmp, const Ix& a, const Ix& b) {
+  same_space(a, b);
+  return from_array(a.shm, compare(cmp, ix_array(be, a), ix_array(be, b)));
+}
+
+Ix ix_select(Backend* be, const Ix& c, const Ix& a, const Ix& b) {
+  same_space(a, b);
+  if (c.shm != a.shm || c.dtype != HGPU_BOOL) throw HostError(HGPU_ERR_INVALID, "ix_select: condition is not a Bool of the same space");
+  return from_array(a.shm, select(ix_array(be, c), ix_array(be, a), ix_array(be, b)));
+}
+
+Ix ix_convert(Backend* be, const Ix& a, int dtype, int mode) {
+  if (a.dtype == dtype) return a;
+  return from_array(a.shm, convert(ix_array(be, a), dtype, mode));
+}
+
+// Range of an affine index over its position box.
+static void affine_range(const Ix& x, int64_t* lo, int64_t* hi) {
+  *lo = *hi = x.c0;
+  for (size_t d = 0; d < x.coef.size(); ++d) {
+    int64_t span = x.coef[d] * (x.shm[d] - 1);
+    if (span > 0) *hi += span; else *lo += span;
+  }
+}
+
+// out[m.., n..] = src[ix(m).., n..] as a view of src (zero-extended first when
+// some index leaves the bounds): tgatherZSScalar with an affine index function.
+// Returns an invalid T when a view is not sensible.
+static T affine_view(const T& src0, const Shape& shm, const std::vector<Ix>& ix) {
+  Backend* be = src0.be();
+  T src = src0;
+  Shape ssh = src.shape();
+  size_t n_ix = ix.size();
+  Shape oshape = shm;
+  oshape.insert(oshape.end(), ssh.begin() + (long)n_ix, ssh.end());
+  if (prod(oshape) == 0) return zeros(be, src.dtype(), oshape);
+  for (size_t j = 0; j < n_ix; ++j)
+    if (ssh[j] == 0) return zeros(be, src.dtype(), oshape);
+  std::vector<int64_t> c0(n_ix);
+  Shape lo_pad(ssh.size(), 0), hi_pad(ssh.size(), 0);
+  bool need_pad = false;
+  int64_t padded = 1;
+  for (size_t j = 0; j < n_ix; ++j) {
+    int64_t lo, hi;
+    affine_range(ix[j], &lo, &hi);
+    c0[j] = ix[j].c0;
+    if (lo < 0) { lo_pad[j] = -lo; need_pad = true; }
+    if (hi > ssh[j] - 1) { hi_pad[j] = hi - (ssh[j] - 1); need_pad = true; }
+    padded *= ssh[j] + lo_pad[j] + hi_pad[j];
+  }
+  if (need_pad) {
+    int64_t plain = 1;
+    for (size_t j = 0; j < n_ix; ++j) plain *= ssh[j];
+    if (padded > 4 * plain + 4096) return T();  // mostly out of bounds: not worth a zero-extended copy
+    src = pad(src, lo_pad, hi_pad);
+    for (size_t j = 0; j < n_ix; ++j) c0[j] += lo_pad[j];
+  }
+  Shape sst = src.strides();
+  Shape ost(oshape.size(), 0);
+  int64_t offset = 0;
+  for (size_t j = 0; j < n_ix; ++j) {
+    offset += c0[j] * sst[j];
+    for (size_t d = 0; d < shm.size(); ++d) ost[d] += ix[j].coef[d] * sst[j];
+  }
+  for (size_t i = n_ix; i < ssh.size(); ++i) ost[shm.size() + (i - n_ix)] = sst[i];
+  return as_strided(src, oshape, ost, offset);
+}
+
+static bool all_affine(const std::vector<Ix>& ix) {
+  for (auto& x : ix)
+    if (!x.affine) return false;
+  return true;
+}
+
+static void check_ix(const Shape& shm, const std::vector<Ix>& ix) {
+  for (auto& x : ix) {
+    if (x.shm != shm) throw HostError(HGPU_ERR_INVALID, "index function built over another position space");
+    if (x.dtype != HGPU_I64) throw HostError(HGPU_ERR_INVALID, "index component is not an Int");
+  }
+}
+
+// Ops.hs:701-705; OpsConcrete.hs:1621-1665
+T tsgather(const T& src, const Shape& shm, const std::vector<Ix>& ix) {
+  if ((int)ix.size() > src.rank()) throw HostError(HGPU_ERR_INVALID, "tsgather: more indices than dims");
+  check_ix(shm, ix);
+  Backend* be = src.be();
+  if (all_affine(ix)) {
+    T v = affine_view(src, shm, ix);
+    if (v.valid()) return v;
+  }
+  std::vector<T> arrs;
+  for (auto& x : ix) arrs.push_back(ix_array(be, x));
+  return gather_raw(src, arrs, shm);
+}
+
+// True when distinct positions provably go to distinct destinations: every
+// component, read as a mixed-radix number in the variables it uses, determines
+// those variables, and together the components use every variable.
+static bool provably_injective(const Shape& shm, const std::vector<Ix>& ix) {
+  if (!all_affine(ix)) return false;
+  std::vector<bool> covered(shm.size(), false);
+  for (auto& x : ix) {
+    std::vector<std::pair<int64_t, size_t>> terms;
+    for (size_t d = 0; d < shm.size(); ++d)
+      if (x.coef[d] != 0 && shm[d] > 1) terms.push_back({std::llabs(x.coef[d]), d});
+    std::sort(terms.begin(), terms.end());
+    int64_t reach = 0;  // largest value the smaller terms can sum to
+    bool ok = true;
+    for (auto& t : terms) {
+      if (t.first <= reach) { ok = false; break; }
+      reach += t.first * (shm[t.second] - 1);
+    }
+    if (ok)
+      for (auto& t : terms) covered[t.second] = true;
+  }
+  for (size_t d = 0; d < shm.size(); ++d)
+    if (shm[d] > 1 && !covered[d]) return false;
+  return true;
+}
+
+// Ops.hs:689-693; OpsConcrete.hs:1581-1619
+T tsscatter(const T& src, int rank_m, const Shape& shp, const std::vector<Ix>& ix) {
+  if (rank_m > src.rank() || ix.size() != shp.size()) throw HostError(HGPU_ERR_INVALID, "tsscatter: ranks do not agree");
+  Shape ssh = src.shape();
+  Shape shm(ssh.begin(), ssh.begin() + rank_m);
+  check_ix(shm, ix);
+  Backend* be = src.be();
+  std::vector<T> arrs;
+  for (auto& x : ix) arrs.push_back(ix_array(be, x));
+  return scatter_raw(src, arrs, rank_m, shp, provably_injective(shm, ix) ? 1 : 0);
+}
+
+// tsindex0 at lane-batched indices (AstIndexK, AstInterpret.hs:181-185)
+Ix ix_index0(Backend* be, const T& t, const std::vector<Ix>& ix) {
+  if ((int)ix.size() != t.rank()) throw HostError(HGPU_ERR_INVALID, "ix_index0: needs one index per dim");
+  if (ix.empty()) throw HostError(HGPU_ERR_INVALID, "ix_index0: rank 0");
+  const Shape& shm = ix[0].shm;
+  check_ix(shm, ix);
+  if (all_affine(ix)) {
+    // A lookup in a host-known integer table that is itself affine in its
+    // indices, with all lookups in bounds, is again an affine form
+    // (e.g. the window tables [0..2n-1] reshaped [n,2]: tbl[i,k] = 2i + k).
+    if (t.host_i64() && t.dtype() == HGPU_I64) {
+      Shape tsh = t.shape(), tst = t.strides();
+      bool dense = true;
+      int64_t s = 1;
+      for (int i = (int)tsh.size() - 1; i >= 0; --i) { if (tsh[(size_t)i] != 1 && tst[(size_t)i] != s) dense = false; s *= tsh[(size_t)i]; }
+      bool inb = true;
+      for (size_t j = 0; j < ix.size(); ++j) {
+        int64_t lo, hi;
+        affine_range(ix[j], &lo, &hi);
+        if (lo < 0 || hi >= tsh[j]) inb = false;
+      }
+      const std::vector<int64_t>& tab = *t.host_i64();
+      if (dense && inb && (int64_t)tab.size() == prod(tsh) && !tab.empty()) {
+        std::vector<int64_t> a(tsh.size(), 0);
+        Shape dst(tsh.size());
+        int64_t q = 1;
+        for (int i = (int)tsh.size() - 1; i >= 0; --i) { dst[(size_t)i] = q; q *= tsh[(size_t)i]; }
+        for (size_t j = 0; j < tsh.size(); ++j)
+          if (tsh[j] > 1) a[j] = tab[(size_t)dst[j]] - tab[0];
+        bool affine_tab = true;
+        std::vector<int64_t> idx(tsh.size(), 0);
+        for (size_t lin = 0; lin < tab.size() && affine_tab; ++lin) {
+          int64_t want = tab[0];
+          for (size_t j = 0; j < tsh.size(); ++j) want += a[j] * idx[j];
+          if (tab[lin] != want) affine_tab = false;
+          for (int j = (int)tsh.size() - 1; j >= 0; --j) {
+            if (++idx[(size_t)j] < tsh[(size_t)j]) break;
+            idx[(size_t)j] = 0;
+          }
+        }
+        if (affine_tab) {
+          Ix r;
+          r.shm = shm;
+          r.affine = true;
+          r.c0 = tab[0];
+          r.coef.assign(shm.size(), 0);
+          for (size_t j = 0; j < ix.size(); ++j) {
+            r.c0 += a[j] * ix[j].c0;
+            for (size_t d = 0; d < shm.size(); ++d) r.coef[d] += a[j] * ix[j].coef[d];
+          }
+          return r;
+        }
+      }
+    }
+    T v = affine_view(t, shm, ix);
+    if (v.valid()) return from_array(shm, v);
+  }
+  std::vector<T> arrs;
+  for (auto& x : ix) arrs.push_back(ix_array(be, x));
+  return from_array(shm, gather_raw(t, arrs, shm));
+}
+
+Ix ix_argminmax(Backend*, const T& t, const std::vector<Ix>& ix, bool want_max) {
+  if ((int)ix.size() + 1 != t.rank()) throw HostError(HGPU_ERR_INVALID, "ix_argminmax: the partial index must leave one dim");
+  if (ix.empty()) throw HostError(HGPU_ERR_INVALID, "ix_argminmax: no position space");
+  const Shape& shm = ix[0].shm;
+  T part = tsgather(t, shm, ix);  // shm ++ [n]
+  return from_array(shm, argminmax_last(part, want_max));
+}
+
+}  // namespace hordead

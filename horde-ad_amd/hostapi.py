@@ -1,0 +1,330 @@
+"""ctypes binding of include/hordead_host.h (libhordead_host.so).
+
+`Host` is a context of the host layer on some provider of the array ABI, `V` a
+tensor value whose methods carry the names of horde-ad's tensor operations
+(`ssum`, `sgather`, `smatmul2`, ...; reference export list:
+src/HordeAd/OpsTensor.hs:16-78), and `IxV` a lane-batched scalar with Python
+operators, so that an index function is written as a lambda exactly like the
+reference's `\\[i, k] -> [i + k]` and is called once, symbolically.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import capi
+from .capi import _DT2NP, _NP2DT, CMP, OP1, OP2, HgpuError, _larr
+
+P, PP, I, L = C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_int64
+LP, IP = C.POINTER(C.c_int64), C.POINTER(C.c_int)
+D = C.c_double
+SIG = {
+    "create_gpu": (I, [I, PP]), "create": (I, [P, I, PP]), "destroy": (I, [P]),
+    "last_error": (C.c_char_p, [P]), "sync": (I, [P]), "array_ctx": (P, [P]), "tape_reset": (I, [P]),
+    "upload": (I, [P, I, I, LP, P, I, PP]), "from_array": (I, [P, P, I, PP]),
+    "constant": (I, [P, I, D, I, LP, PP]), "array": (I, [P, PP]), "download": (I, [P, P, P]),
+    "val_rank": (I, [P]), "val_dtype": (I, [P]), "val_shape": (I, [P, LP]), "free": (I, [P]),
+    "backward": (I, [P, P, P, I, PP, PP]),
+    "ewise1": (I, [P, I, P, PP]), "ewise2": (I, [P, I, P, P, PP]), "compare": (I, [P, I, P, P, PP]),
+    "compare_all": (I, [P, I, P, P, IP]), "select": (I, [P, P, P, P, PP]), "convert": (I, [P, P, I, I, PP]),
+    "tssumN": (I, [P, P, I, PP]), "tssum0": (I, [P, P, PP]), "tsdot0": (I, [P, P, P, PP]),
+    "tsdot1In": (I, [P, P, P, PP]), "tsmatvecmul": (I, [P, P, P, PP]), "tsmatmul2": (I, [P, P, P, PP]),
+    "tsreplicateN": (I, [P, P, I, LP, PP]), "tsappend": (I, [P, P, P, PP]), "tsslice": (I, [P, P, L, L, PP]),
+    "tsreverse": (I, [P, P, PP]), "tstranspose": (I, [P, P, I, IP, PP]), "tsreshape": (I, [P, P, I, LP, PP]),
+    "tsindex": (I, [P, P, I, LP, PP]), "tsargminmax": (I, [P, P, I, PP]), "tsiota": (I, [P, L, I, PP]),
+    "ix_var": (I, [P, I, LP, I, PP]), "ix_const": (I, [P, I, LP, I, D, PP]), "ix_lift": (I, [P, I, LP, P, PP]),
+    "ix_op1": (I, [P, I, P, PP]), "ix_op2": (I, [P, I, P, P, PP]), "ix_compare": (I, [P, I, P, P, PP]),
+    "ix_select": (I, [P, P, P, P, PP]), "ix_convert": (I, [P, P, I, I, PP]),
+    "ix_index0": (I, [P, P, I, PP, PP]), "ix_argminmax": (I, [P, P, I, PP, I, PP]), "ix_free": (I, [P]),
+    "ix_is_affine": (I, [P]),
+    "tsgather": (I, [P, P, I, LP, I, PP, PP]), "tsscatter": (I, [P, P, I, I, LP, PP, PP]),
+}
+
+_dll = None
+
+
+def _lib():
+    global _dll
+    if _dll is None:
+        import os
+        if not os.path.exists(capi.HOST_LIB):
+            raise FileNotFoundError(f"{capi.HOST_LIB} is not built; run __graft_entry__.build()")
+        dll = C.CDLL(capi.HOST_LIB)
+        for name, (res, args) in SIG.items():
+            fn = getattr(dll, "hh_" + name)
+            fn.restype, fn.argtypes = res, args
+        _dll = dll
+    return _dll
+
+
+class Host:
+    """A host-layer context: on the gfx950 library by default, or on the provider
+    whose ABI table `api_lib.get_api()` returns."""
+
+    def __init__(self, api_lib=None, device=0):
+        self.dll = _lib()
+        h = C.c_void_p()
+        if api_lib is None:
+            rc = self.dll.hh_create_gpu(device, C.byref(h))
+        else:
+            self._api_lib = api_lib  # keep the provider loaded
+            rc = self.dll.hh_create(api_lib.get_api(), device, C.byref(h))
+        if rc:
+            raise HgpuError(rc, "cannot create a host-layer context (no usable device?)")
+        self.h = h
+
+    def check(self, rc):
+        if rc:
+            raise HgpuError(rc, self.dll.hh_last_error(self.h).decode())
+
+    def _out(self, fn, *args):
+        o = C.c_void_p()
+        self.check(fn(self.h, *args, C.byref(o)))
+        return V(self, o)
+
+    def sync(self):
+        self.check(self.dll.hh_sync(self.h))
+
+    def tape_reset(self):
+        self.check(self.dll.hh_tape_reset(self.h))
+
+    def destroy(self):
+        self.dll.hh_destroy(self.h)
+
+    # -- values
+    def concrete(self, x, requires_grad=False):
+        x = np.asarray(x)
+        if not x.flags.c_contiguous:
+            x = x.copy(order="C")
+        return self._out(self.dll.hh_upload, _NP2DT[x.dtype], x.ndim, _larr(x.shape),
+                         x.ctypes.data_as(C.c_void_p), int(requires_grad))
+
+    def param(self, x):
+        return self.concrete(x, requires_grad=True)
+
+    def srepl(self, shape, value, dtype=capi.F64):
+        """sconcrete (sreplicate shape value)"""
+        return self._out(self.dll.hh_constant, dtype, float(value), len(shape), _larr(shape))
+
+    def siota(self, n, dtype=capi.I64):
+        return self._out(self.dll.hh_tsiota, n, dtype)
+
+    def grad(self, out, inputs, dt=None):
+        """Cotangents of `inputs` for d(out) = dt (default: ones, as `grad` uses)."""
+        if dt is None:
+            dt = self.srepl(out.shape, 1.0, out.dtype)
+        arr = (C.c_void_p * len(inputs))(*[v.h for v in inputs])
+        outs = (C.c_void_p * len(inputs))()
+        self.check(self.dll.hh_backward(self.h, out.h, dt.h, len(inputs), arr, outs))
+        return [V(self, C.c_void_p(o)) for o in outs]
+
+    # -- index functions
+    def ix_space(self, shm):
+        return [IxV(self, self._ixo(self.dll.hh_ix_var, len(shm), _larr(shm), d), tuple(shm)) for d in range(len(shm))]
+
+    def _ixo(self, fn, *args):
+        o = C.c_void_p()
+        self.check(fn(self.h, *args, C.byref(o)))
+        return o
+
+    def _apply_index_fn(self, shm, f):
+        shm = tuple(int(s) for s in shm)
+        vars_ = self.ix_space(shm)
+        res = f(*vars_)
+        res = [r if isinstance(r, IxV) else IxV.const(self, shm, int(r)) for r in res]
+        return shm, res
+
+
+def _ixarr(ixs):
+    return (C.c_void_p * max(len(ixs), 1))(*[x.h for x in ixs])
+
+
+class IxV:
+    """A scalar inside an index function, for all positions at once."""
+
+    def __init__(self, host, h, shm):
+        self.host, self.h, self.shm = host, h, shm
+
+    def __del__(self):
+        try:
+            self.host.dll.hh_ix_free(self.h)
+        except Exception:
+            pass
+
+    @staticmethod
+    def const(host, shm, value, dtype=capi.I64):
+        return IxV(host, host._ixo(host.dll.hh_ix_const, len(shm), _larr(shm), dtype, float(value)), shm)
+
+    def _coerce(self, o, dtype=capi.I64):
+        return o if isinstance(o, IxV) else IxV.const(self.host, self.shm, o, dtype)
+
+    def _op2(self, op, o, dtype=capi.I64):
+        o = self._coerce(o, dtype)
+        return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_op2, OP2[op], self.h, o.h), self.shm)
+
+    def _rop2(self, op, o, dtype=capi.I64):
+        return self._coerce(o, dtype)._op2(op, self)
+
+    @property
+    def is_affine(self):
+        return bool(self.host.dll.hh_ix_is_affine(self.h))
+
+    def __add__(self, o): return self._op2("add", o)
+    def __radd__(self, o): return self._rop2("add", o)
+    def __sub__(self, o): return self._op2("sub", o)
+    def __rsub__(self, o): return self._rop2("sub", o)
+    def __mul__(self, o): return self._op2("mul", o)
+    def __rmul__(self, o): return self._rop2("mul", o)
+    def __neg__(self): return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_op1, OP1["neg"], self.h), self.shm)
+    def quotH(self, o): return self._op2("quot", o)
+    def remH(self, o): return self._op2("rem_scalar", o)      # scalar rule: remH a 0 = a (Types.hs:402-419)
+    def minH(self, o): return self._op2("min", o)
+    def maxH(self, o): return self._op2("max", o)
+    def op1(self, name): return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_op1, OP1[name], self.h), self.shm)
+
+    def _cmp(self, c, o, dtype):
+        o = self._coerce(o, dtype)
+        return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_compare, CMP[c], self.h, o.h), self.shm)
+
+    def leq(self, o, dtype=capi.I64): return self._cmp("leq", o, dtype)     # <=.
+    def lt(self, o, dtype=capi.I64): return self._cmp("lt", o, dtype)       # <.
+    def eq(self, o, dtype=capi.I64): return self._cmp("eq", o, dtype)       # ==.
+
+    def convert(self, dtype, mode=0):
+        return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_convert, self.h, dtype, mode), self.shm)
+
+
+def ifH(cond, a, b):
+    """ifH / kcond on lane-batched scalars."""
+    a = a if isinstance(a, IxV) else IxV.const(cond.host, cond.shm, a)
+    b = b if isinstance(b, IxV) else IxV.const(cond.host, cond.shm, b)
+    return IxV(cond.host, cond.host._ixo(cond.host.dll.hh_ix_select, cond.h, a.h, b.h), cond.shm)
+
+
+class V:
+    """A tensor value of the `Gpu` carrier (possibly carrying a tape node)."""
+
+    def __init__(self, host, h):
+        self.host, self.h = host, h
+
+    def __del__(self):
+        try:
+            if self.h:
+                self.host.dll.hh_free(self.h)
+                self.h = None
+        except Exception:
+            pass
+
+    @property
+    def shape(self):
+        r = self.host.dll.hh_val_rank(self.h)
+        buf = (C.c_int64 * max(r, 1))()
+        self.host.dll.hh_val_shape(self.h, buf)
+        return tuple(buf[i] for i in range(r))
+
+    @property
+    def dtype(self):
+        return self.host.dll.hh_val_dtype(self.h)
+
+    def numpy(self):
+        out = np.empty(self.shape, dtype=_DT2NP[self.dtype])
+        self.host.check(self.host.dll.hh_download(self.host.h, self.h, out.ctypes.data_as(C.c_void_p)))
+        return out
+
+    def _o(self, fn, *args):
+        return self.host._out(fn, *args)
+
+    def _lift(self, o):
+        if isinstance(o, V):
+            return o
+        return self.host.srepl(self.shape, o, self.dtype)
+
+    # -- Num / Fractional / Floating
+    def op1(self, name): return self._o(self.host.dll.hh_ewise1, OP1[name], self.h)
+    def op2(self, name, o): return self._o(self.host.dll.hh_ewise2, OP2[name], self.h, self._lift(o).h)
+    def __add__(self, o): return self.op2("add", o)
+    def __radd__(self, o): return self._lift(o).op2("add", self)
+    def __sub__(self, o): return self.op2("sub", o)
+    def __rsub__(self, o): return self._lift(o).op2("sub", self)
+    def __mul__(self, o): return self.op2("mul", o)
+    def __rmul__(self, o): return self._lift(o).op2("mul", self)
+    def __truediv__(self, o): return self.op2("div", o)
+    def __rtruediv__(self, o): return self._lift(o).op2("div", self)
+    def __pow__(self, o): return self.op2("pow", o)
+    def __neg__(self): return self.op1("neg")
+    def atan2H(self, o): return self.op2("atan2", o)
+    def quotH(self, o): return self.op2("quot", o)
+    def remH(self, o): return self.op2("rem", o)
+
+    # -- comparisons, conditionals, conversions
+    def leq(self, o): return self._o(self.host.dll.hh_compare, CMP["leq"], self.h, self._lift(o).h)
+    def lt(self, o): return self._o(self.host.dll.hh_compare, CMP["lt"], self.h, self._lift(o).h)
+    def eq(self, o): return self._o(self.host.dll.hh_compare, CMP["eq"], self.h, self._lift(o).h)
+
+    def compare_all(self, cmp, o):
+        r = C.c_int()
+        self.host.check(self.host.dll.hh_compare_all(self.host.h, CMP[cmp], self.h, o.h, C.byref(r)))
+        return bool(r.value)
+
+    def select(self, a, b):
+        """Elementwise ifH on a Bool tensor."""
+        return self._o(self.host.dll.hh_select, self.h, a.h, b.h)
+
+    def scast(self, dtype): return self._o(self.host.dll.hh_convert, self.h, dtype, 0)
+    def sfromIntegral(self, dtype): return self._o(self.host.dll.hh_convert, self.h, dtype, 0)
+    def sfloor(self, dtype=capi.I64): return self._o(self.host.dll.hh_convert, self.h, dtype, 1)
+
+    # -- reductions and contractions
+    def ssum(self): return self._o(self.host.dll.hh_tssumN, self.h, 1)
+    def ssumN(self, k): return self._o(self.host.dll.hh_tssumN, self.h, k)
+    def ssum0(self): return self._o(self.host.dll.hh_tssum0, self.h)
+    def sdot0(self, o): return self._o(self.host.dll.hh_tsdot0, self.h, o.h)
+    def sdot1In(self, o): return self._o(self.host.dll.hh_tsdot1In, self.h, o.h)
+    def smatvecmul(self, v): return self._o(self.host.dll.hh_tsmatvecmul, self.h, v.h)
+    def smatmul2(self, o): return self._o(self.host.dll.hh_tsmatmul2, self.h, o.h)
+    def sargMax(self): return self._o(self.host.dll.hh_tsargminmax, self.h, 1)
+    def sargMin(self): return self._o(self.host.dll.hh_tsargminmax, self.h, 0)
+
+    # -- structure
+    def sreplicate(self, k): return self._o(self.host.dll.hh_tsreplicateN, self.h, 1, _larr([k]))
+    def sreplicateN(self, shm): return self._o(self.host.dll.hh_tsreplicateN, self.h, len(shm), _larr(shm))
+    sreplicate0N = sreplicateN
+    def sappend(self, o): return self._o(self.host.dll.hh_tsappend, self.h, o.h)
+    def sslice(self, i, n): return self._o(self.host.dll.hh_tsslice, self.h, i, n)
+    def sreverse(self): return self._o(self.host.dll.hh_tsreverse, self.h)
+    def stranspose(self, perm): return self._o(self.host.dll.hh_tstranspose, self.h, len(perm), (C.c_int * max(len(perm), 1))(*perm))
+    def str_(self): return self.stranspose([1, 0])
+    def sreshape(self, shape): return self._o(self.host.dll.hh_tsreshape, self.h, len(shape), _larr(shape))
+    def sindex(self, ix): return self._o(self.host.dll.hh_tsindex, self.h, len(ix), _larr(ix))   # `!$` with concrete indices
+
+    # -- indexing with index functions
+    def sgather(self, shm, f):
+        """sgather @shm self (\\[i...] -> [ix...])"""
+        shm, ix = self.host._apply_index_fn(shm, f)
+        return self._o(self.host.dll.hh_tsgather, self.h, len(shm), _larr(shm), len(ix), _ixarr(ix))
+
+    def sscatter(self, rank_m, shp, f):
+        """sscatter @shm self (\\[i...] -> [ix...]) with shm = the first rank_m dims; result shp ++ rest"""
+        shm, ix = self.host._apply_index_fn(self.shape[:rank_m], f)
+        if len(ix) != len(shp):
+            raise HgpuError(1, "sscatter: the index function must return one index per dim of shp")
+        return self._o(self.host.dll.hh_tsscatter, self.h, rank_m, len(ix), _larr(shp), _ixarr(ix))
+
+    # inside index functions
+    def sindex0(self, ix):
+        """self `sindex0` [ix...] with lane-batched indices"""
+        first = next(x for x in ix if isinstance(x, IxV))
+        ix = [x if isinstance(x, IxV) else IxV.const(self.host, first.shm, x) for x in ix]
+        return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_index0, self.h, len(ix), _ixarr(ix)), first.shm)
+
+    def kargMax(self, ix, want_max=True):
+        """kargMax (self !$ [ix...])"""
+        first = next(x for x in ix if isinstance(x, IxV))
+        ix = [x if isinstance(x, IxV) else IxV.const(self.host, first.shm, x) for x in ix]
+        return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_argminmax, self.h, len(ix), _ixarr(ix), int(want_max)), first.shm)
+
+    def kargMin(self, ix):
+        return self.kargMax(ix, want_max=False)
+
+    def lift(self, shm):
+        """A rank-0 tensor as a scalar of the position space shm."""
+        return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_lift, len(shm), _larr(shm), self.h), tuple(shm))

@@ -1,0 +1,118 @@
+/* hordead_host.h -- C ABI of the host layer: the `Gpu` carrier's tensor-class
+ * operations as horde-ad's interpreter would call them, one call per AST node.
+ *
+ * Where hordead_gpu.h is the array library (strided views + kernels), this
+ * layer is what `instance BaseTensor Gpu` binds method by method
+ * (reference class: src/HordeAd/Core/Ops.hs:297-1255; the instance it stands
+ * beside: src/HordeAd/Core/OpsConcrete.hs:97-775).  It adds what an array
+ * library cannot know:
+ *   - index FUNCTIONS (tsgather / tsscatter / tsindex0 inside them) evaluated
+ *     once over all positions with lane-batched scalars (`hh_ix`), so that an
+ *     affine index function becomes a strided view and anything else becomes
+ *     index arrays (reference: one call of the closure per position,
+ *     OpsConcrete.hs:1581-1665, AstInterpret.hs:242-283);
+ *   - dual numbers: values carry a tape node, and `hh_backward` transposes the
+ *     recorded operations (reference: OpsADVal.hs:44-60, DeltaEval.hs:391-595).
+ *
+ * Every function returns an hgpu_status code; `hh_last_error` has the message.
+ * Shape mismatches are HGPU_ERR_INVALID (the reference calls `error`).
+ */
+#ifndef HORDEAD_HOST_H
+#define HORDEAD_HOST_H
+
+#include "hordead_gpu.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct hh_ctx hh_ctx;   /* a provider context + the tape of the gradient in progress */
+typedef struct hh_val hh_val;   /* a tensor value (primal array view + tape node) */
+typedef struct hh_ix hh_ix;     /* a lane-batched scalar: `IntOf Gpu` inside an index function */
+
+/* Context on the gfx950 library (device `device`). */
+int hh_create_gpu(int device, hh_ctx** out);
+/* Context on any provider of the array ABI. */
+int hh_create(const hgpu_api* api, int device, hh_ctx** out);
+int hh_destroy(hh_ctx* ctx);
+const char* hh_last_error(hh_ctx* ctx);
+int hh_sync(hh_ctx* ctx);
+hgpu_ctx* hh_array_ctx(hh_ctx* ctx);
+/* Forgets the recorded operations; values made before stay usable as constants. */
+int hh_tape_reset(hh_ctx* ctx);
+
+/* tsconcrete (OpsConcrete.hs:120-124): a value from host data; `requires_grad`
+ * makes it a differentiable input (an `ADVal` with a fresh input delta,
+ * OpsADVal.hs:62-73). */
+int hh_upload(hh_ctx* ctx, int dtype, int rank, const int64_t* shape, const void* host, int requires_grad, hh_val** out);
+/* The same from an array already on the device (the array is retained). */
+int hh_from_array(hh_ctx* ctx, hgpu_array* a, int requires_grad, hh_val** out);
+/* sconcrete (sreplicate sh x): a constant of the given shape, no element traffic. */
+int hh_constant(hh_ctx* ctx, int dtype, double value, int rank, const int64_t* shape, hh_val** out);
+/* The primal array of a value (a new reference the caller releases). */
+int hh_array(hh_val* v, hgpu_array** out);
+int hh_download(hh_ctx* ctx, hh_val* v, void* host);
+int hh_val_rank(hh_val* v);
+int hh_val_dtype(hh_val* v);
+int hh_val_shape(hh_val* v, int64_t* shape);
+int hh_free(hh_val* v);
+
+/* gradientFromDelta (DeltaEval.hs:64-78): cotangents of `inputs` for d(out)=dt. */
+int hh_backward(hh_ctx* ctx, hh_val* out, hh_val* dt, int n, hh_val* const* inputs, hh_val** grads);
+
+/* Elementwise Num/Floating/IntegralH/RealFloatH methods (AstInterpret.hs:187-194). */
+int hh_ewise1(hh_ctx* ctx, int op1, hh_val* a, hh_val** out);
+int hh_ewise2(hh_ctx* ctx, int op2, hh_val* a, hh_val* b, hh_val** out);
+/* Elementwise comparison -> Bool tensor (AstLeqS, AstInterpret.hs:353-366). */
+int hh_compare(hh_ctx* ctx, int cmp, hh_val* a, hh_val* b, hh_val** out);
+/* Whole-tensor comparison -> one Bool on the host (AstLeq, EqH/OrdH). */
+int hh_compare_all(hh_ctx* ctx, int cmp, hh_val* a, hh_val* b, int* result);
+/* Elementwise conditional on a Bool tensor (what tsmap0N/tszipWith0N of ifH compute). */
+int hh_select(hh_ctx* ctx, hh_val* cond, hh_val* a, hh_val* b, hh_val** out);
+/* tscast / tsfromIntegral (mode HGPU_CONV_CAST), tsfloor (HGPU_CONV_FLOOR). */
+int hh_convert(hh_ctx* ctx, hh_val* a, int dtype, int mode, hh_val** out);
+int hh_tssumN(hh_ctx* ctx, hh_val* t, int k, hh_val** out);              /* Ops.hs:514; tssum is k = 1 */
+int hh_tssum0(hh_ctx* ctx, hh_val* t, hh_val** out);                     /* Ops.hs:517 */
+int hh_tsdot0(hh_ctx* ctx, hh_val* a, hh_val* b, hh_val** out);          /* Ops.hs:519 */
+int hh_tsdot1In(hh_ctx* ctx, hh_val* a, hh_val* b, hh_val** out);        /* Ops.hs:522 */
+int hh_tsmatvecmul(hh_ctx* ctx, hh_val* m, hh_val* v, hh_val** out);     /* Ops.hs:538 */
+int hh_tsmatmul2(hh_ctx* ctx, hh_val* a, hh_val* b, hh_val** out);       /* Ops.hs:543 */
+int hh_tsreplicateN(hh_ctx* ctx, hh_val* t, int n, const int64_t* shm, hh_val** out);   /* Ops.hs:552; also tsreplicate0N */
+int hh_tsappend(hh_ctx* ctx, hh_val* a, hh_val* b, hh_val** out);        /* Ops.hs:825 */
+int hh_tsslice(hh_ctx* ctx, hh_val* t, int64_t i, int64_t n, hh_val** out);   /* Ops.hs:828 */
+int hh_tsreverse(hh_ctx* ctx, hh_val* t, hh_val** out);                  /* Ops.hs:831 */
+int hh_tstranspose(hh_ctx* ctx, hh_val* t, int n, const int* perm, hh_val** out);   /* Ops.hs:833 */
+int hh_tsreshape(hh_ctx* ctx, hh_val* t, int rank, const int64_t* shape, hh_val** out);   /* Ops.hs:837 */
+int hh_tsindex(hh_ctx* ctx, hh_val* t, int n, const int64_t* ix, hh_val** out);   /* Ops.hs:667, host indices */
+int hh_tsargminmax(hh_ctx* ctx, hh_val* t, int want_max, hh_val** out);  /* Ops.hs:792 */
+int hh_tsiota(hh_ctx* ctx, int64_t n, int dtype, hh_val** out);          /* Ops.hs:795 */
+
+/* Index functions.  A position space is a shape `shm`; `hh_ix_var` is its d-th
+ * position variable.  All hh_ix of one function must share the space. */
+int hh_ix_var(hh_ctx* ctx, int rank_m, const int64_t* shm, int d, hh_ix** out);
+int hh_ix_const(hh_ctx* ctx, int rank_m, const int64_t* shm, int dtype, double value, hh_ix** out);
+/* A rank-0 tensor value used as a scalar inside an index function. */
+int hh_ix_lift(hh_ctx* ctx, int rank_m, const int64_t* shm, hh_val* scalar, hh_ix** out);
+int hh_ix_op1(hh_ctx* ctx, int op1, hh_ix* a, hh_ix** out);              /* AstN1K / AstR1K */
+int hh_ix_op2(hh_ctx* ctx, int op2, hh_ix* a, hh_ix* b, hh_ix** out);    /* AstPlusK / AstTimesK / AstR2K / AstI2K */
+int hh_ix_compare(hh_ctx* ctx, int cmp, hh_ix* a, hh_ix* b, hh_ix** out);   /* AstLeqK */
+int hh_ix_select(hh_ctx* ctx, hh_ix* c, hh_ix* a, hh_ix* b, hh_ix** out);   /* AstCondK -> kcond (ifH) */
+int hh_ix_convert(hh_ctx* ctx, hh_ix* a, int dtype, int mode, hh_ix** out); /* AstFromIntegralK / AstCastK / AstFloorK */
+/* AstIndexK (AstInterpret.hs:181-185): t `sindex0` [ix...], one index per dim of t. */
+int hh_ix_index0(hh_ctx* ctx, hh_val* t, int n, hh_ix* const* ix, hh_ix** out);
+/* AstArgMinK / AstArgMaxK of a partial index: kargMax (t !$ [ix...]); the
+ * partial index must leave exactly the last dim of t. */
+int hh_ix_argminmax(hh_ctx* ctx, hh_val* t, int n, hh_ix* const* ix, int want_max, hh_ix** out);
+int hh_ix_free(hh_ix* x);
+/* 1 when the value is an affine form of the position variables (diagnostic). */
+int hh_ix_is_affine(hh_ix* x);
+
+/* tsgather (Ops.hs:701-705): out[m.., n..] = src[ix(m).., n..], zeros out of bounds. */
+int hh_tsgather(hh_ctx* ctx, hh_val* src, int rank_m, const int64_t* shm, int n_ix, hh_ix* const* ix, hh_val** out);
+/* tsscatter (Ops.hs:689-693): out[ix(m).., n..] += src[m.., n..]; shp has n_ix dims. */
+int hh_tsscatter(hh_ctx* ctx, hh_val* src, int rank_m, int n_ix, const int64_t* shp, hh_ix* const* ix, hh_val** out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HORDEAD_HOST_H */
