@@ -1,0 +1,165 @@
+#!/usr/bin/env python3
+"""Gradient throughput of the gfx950 backend on the synthetic configs.
+
+One "step" = one full forward + reverse gradient of a config's objective on one
+batch of synthetic input that is already resident in HBM (uploads happen before
+the timed region; every step ends with a stream sync, the equivalent of the
+reference forcing every gradient leaf, bench/ConvVjpBench.hs:174-175).
+
+Prints ONE JSON line.  `value` is gradient samples/s of the headline config
+(the CNN); the other configs ride along under "configs".  "roofline" prices the
+dominant kernel of the headline config: its ALGORITHMIC bytes (or flops) per
+launch divided by its average launch duration, measured here with HIP events
+on the library's stream.  "cpu_baseline" is the CPU checker (a single-threaded
+dense restatement of the reference's array semantics) timed on a bounded
+sample of the same workload.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3}
+MFMA_KERNELS = ("gemm",)          # kernel families priced against the matrix-core peak
+DTYPE_NAME = {0: "f64", 1: "f32"}
+# CPU-baseline sample sizes (batch) chosen so the checker runs ~10-30 s in total
+CPU_SAMPLE = {"c0": dict(n=1024, m=1024), "c1": dict(batch=250), "c2": dict(batch=64),
+              "c3": dict(batch=12), "c4": dict(batch=64)}
+
+
+def array_ctx(capi, host):
+    """The array-library context behind a host-layer context, as a capi.Ctx."""
+    ctx = capi.Ctx.__new__(capi.Ctx)
+    ctx.lib = capi.Lib()
+    ctx.h = C.c_void_p(host.dll.hh_array_ctx(host.h))
+    return ctx
+
+
+def time_steps(host, wl, ps, ds, steps, warmup):
+    for _ in range(warmup):
+        wl.gradient(host, ps, ds)
+        host.sync()
+    host.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss, grads = wl.gradient(host, ps, ds)
+        host.sync()
+    host.sync()
+    dt = time.perf_counter() - t0
+    return dt / steps, float(loss.numpy())
+
+
+def profile(capi, host, wl, ps, ds, reps=2):
+    actx = array_ctx(capi, host)
+    actx.profile(True)
+    for _ in range(reps):
+        wl.gradient(host, ps, ds)
+        host.sync()
+    rep = actx.profile_report()
+    actx.profile(False)
+    return {k: (v[0] / reps, v[1] / reps, v[2] / reps, v[3] / reps) for k, v in rep.items()}
+
+
+def roofline_of(rep, dtype_name):
+    """Prices the kernel family with the largest share of device time."""
+    if not rep:
+        return None, {}
+    name = max(rep, key=lambda k: rep[k][1])
+    launches, ms, by, fl = rep[name]
+    if launches == 0 or ms <= 0:
+        return None, {}
+    avg_ms = ms / launches
+    if name.startswith(MFMA_KERNELS):
+        ach = fl / launches / (avg_ms * 1e-3) / 1e12
+        peak = MFMA_PEAK_TFLOPS[dtype_name]
+        roof = {"bound": "mfma", "achieved": ach, "peak": peak, "unit": "TFLOP/s", "frac": ach / peak}
+    else:
+        ach = by / launches / (avg_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS}
+    roof.update({"kernel": name, "launches_per_step": launches, "avg_launch_ms": avg_ms,
+                 "share_of_device_time": ms / sum(v[1] for v in rep.values()), "traffic": None})
+    shares = {k: round(v[1], 4) for k, v in sorted(rep.items(), key=lambda kv: -kv[1][1])}
+    return roof, shares
+
+
+def cpu_baseline(pkg, key, mk):
+    capi, H = pkg.capi, pkg.hostapi
+    if not os.path.exists(entry.ORACLE_LIB):
+        return None
+    host = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    wl = mk(**CPU_SAMPLE[key])
+    ps, ds = wl.upload(host)
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        wl.gradient(host, ps, ds)
+        n += 1
+        if time.perf_counter() - t0 > 8.0 or n >= 3:
+            break
+    dt = (time.perf_counter() - t0) / n
+    return {"value": wl.batch / dt, "unit": "samples/s", "cores": 1, "kind": "port",
+            "sample": f"{wl.name} at {CPU_SAMPLE[key]} ({wl.batch} samples per gradient, {n} gradients, {dt:.3f} s each)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="c3", help="headline config: c0..c4")
+    ap.add_argument("--only", action="store_true", help="measure the headline config only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    pkg = entry.load_package()
+    capi, H, W = pkg.capi, pkg.hostapi, pkg.workloads
+    host = H.Host()      # raises when the HIP library is missing or no device is usable
+
+    keys = [args.workload] if args.only else [args.workload] + [k for k in W.CONFIGS if k != args.workload]
+    results = {}
+    for key in keys:
+        wl = W.CONFIGS[key]()
+        ps, ds = wl.upload(host)
+        host.sync()
+        sec, loss = time_steps(host, wl, ps, ds, args.steps, args.warmup)
+        rep = profile(capi, host, wl, ps, ds)
+        dn = DTYPE_NAME[wl.dtype]
+        roof, shares = roofline_of(rep, dn)
+        dev_ms = sum(v[1] for v in rep.values())
+        results[key] = {"workload": wl.name, "dtype": dn, "batch": wl.batch, "ms_per_step": sec * 1e3,
+                        "samples_per_s": wl.batch / sec, "gradients_per_s": 1.0 / sec, "loss": loss,
+                        "device_ms_per_step": dev_ms, "algorithmic_gflop": wl.flops / 1e9,
+                        "achieved_tflops": wl.flops / sec / 1e12, "roofline": roof, "kernel_ms": shares}
+        if wl.bytes:
+            results[key]["algorithmic_gb"] = wl.bytes / 1e9
+            results[key]["achieved_gbs_whole_step"] = wl.bytes / sec / 1e9
+        del ps, ds
+
+    head = results[args.workload]
+    cpu = None if args.no_cpu else cpu_baseline(pkg, args.workload, W.CONFIGS[args.workload])
+    line = {
+        "metric": "gradient samples/sec at 1 GPU", "value": head["samples_per_s"], "unit": "samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
+        "data": "synthetic",
+        "config": {"workload": f"{head['workload']}: forward + reverse gradient, batch {head['batch']}, {head['dtype']}"},
+        "roofline": head["roofline"], "cpu_baseline": cpu,
+        "configs": {k: v for k, v in results.items() if k != args.workload},
+        "headline_detail": {k: v for k, v in head.items() if k != "roofline"},
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

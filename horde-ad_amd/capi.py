@@ -53,6 +53,7 @@ SIGNATURES = {
 GPU_ONLY = {
     "mem_stats": (I, [P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "stream": (P, [P]), "inject_alloc_failure": (I, [P, L]),
+    "profile_enable": (I, [P, I]), "profile_report": (I, [P, C.c_char_p, C.c_size_t]),
 }
 
 
@@ -111,6 +112,19 @@ class Ctx:
         a, b, c = C.c_uint64(), C.c_uint64(), C.c_uint64()
         self.check(self.lib.mem_stats(self.h, C.byref(a), C.byref(b), C.byref(c)))
         return a.value, b.value, c.value
+
+    def profile(self, on):
+        self.check(self.lib.profile_enable(self.h, int(on)))
+
+    def profile_report(self):
+        """{kernel family: (launches, total_ms, algorithmic_bytes, algorithmic_flops)}"""
+        buf = C.create_string_buffer(1 << 16)
+        self.check(self.lib.profile_report(self.h, buf, len(buf)))
+        out = {}
+        for line in buf.value.decode().splitlines():
+            name, cnt, ms, by, fl = line.split()
+            out[name] = (int(cnt), float(ms), float(by), float(fl))
+        return out
 
     def _wrap(self, h):
         return Array(self, h)

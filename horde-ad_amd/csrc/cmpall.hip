@@ -60,7 +60,7 @@ extern "C" int hgpu_compare_all(hgpu_ctx* ctx, int cmp, const hgpu_array* a, con
   int host = 0;
   hipError_t e;
   {
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, "compare_all", 2.0 * n * dtype_size(a->dtype), (double)n);
     hipLaunchKernelGGL(k_set_u64, dim3(1), dim3(1), 0, ctx->stream, first, ~0ull);
     unsigned g = grid_for(n, kBlock, ctx->num_cu * 8);
     HG_DISPATCH_DTYPE(a->dtype, T, {

@@ -51,6 +51,10 @@ struct hgpu_ctx {
   int num_cu = 256;
   // JIT cache of fused elementwise kernels, keyed by generated source.
   std::map<std::string, void*> jit_cache;
+  // Optional per-launch timing (hgpu_profile_enable): one event pair per launch.
+  struct ProfRec { const char* name; hipEvent_t a, b; double bytes, flops; };
+  bool profiling = false;
+  std::vector<ProfRec> prof;
 };
 
 namespace hg {
@@ -123,13 +127,28 @@ int zero_fill(hgpu_ctx* ctx, void* p, size_t bytes);
 int copy_view(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const void* src,
               const int64_t* sst, void* dst, const int64_t* dst_st);
 
+// Serialises enqueueing and, when profiling is on, brackets the launches made
+// while it lives with an event pair labelled `name`; `bytes` / `flops` are the
+// ALGORITHMIC traffic and work of those launches.
 struct LaunchGuard {
   hgpu_ctx* ctx;
-  explicit LaunchGuard(hgpu_ctx* c) : ctx(c) {
+  bool timed = false;
+  explicit LaunchGuard(hgpu_ctx* c, const char* name = nullptr, double bytes = 0, double flops = 0) : ctx(c) {
     c->launch_mu.lock();
     (void)hipSetDevice(c->device);
+    if (c->profiling && name) {
+      hgpu_ctx::ProfRec r{name, nullptr, nullptr, bytes, flops};
+      if (hipEventCreate(&r.a) == hipSuccess && hipEventCreate(&r.b) == hipSuccess) {
+        (void)hipEventRecord(r.a, c->stream);
+        c->prof.push_back(r);
+        timed = true;
+      }
+    }
   }
-  ~LaunchGuard() { ctx->launch_mu.unlock(); }
+  ~LaunchGuard() {
+    if (timed) (void)hipEventRecord(ctx->prof.back().b, ctx->stream);
+    ctx->launch_mu.unlock();
+  }
 };
 
 }  // namespace hg

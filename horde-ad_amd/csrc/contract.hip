@@ -159,7 +159,8 @@ __global__ void __launch_bounds__(kBlock) k_argminmax(Dims keep, int64_t n_out, 
 
 template <typename TI, typename TO>
 int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red_full, int64_t n_out, int64_t R, int S, const void* a, const void* b, void* out) {
-  LaunchGuard lg(ctx);
+  LaunchGuard lg(ctx, b ? (use_wave ? "contract_dot_wave" : "contract_dot_lane") : (use_wave ? "contract_sum_wave" : "contract_sum_lane"),
+                 (double)n_out * R * sizeof(TI) * (b ? 2 : 1) + (double)n_out * S * sizeof(TO), (double)n_out * R * (b ? 2 : 1));
   int maxb = ctx->num_cu * 8;
   if (use_wave) {
     Dims red = red_full;
@@ -296,7 +297,7 @@ int hgpu_argminmax_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_a
     const int64_t* ks[1] = {a->strides};
     Dims keep;
     if (!collapse(a->rank - 1, a->shape, 1, ks, &keep)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "argminmax: too many dims"); }
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, "argminmax", (double)n_out * (L * dtype_size(a->dtype) + 8), (double)n_out * L);
     unsigned g = grid_for(n_out, kBlock, ctx->num_cu * 8);
     HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
     hipError_t e = hipGetLastError();

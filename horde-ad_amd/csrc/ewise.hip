@@ -240,7 +240,7 @@ int zero_fill(hgpu_ctx* ctx, void* p, size_t bytes) {
   // length up to 16 stays inside the block.
   int64_t n16 = (int64_t)((bytes + 15) / 16);
   if (n16 == 0) return HGPU_OK;
-  LaunchGuard lg(ctx);
+  LaunchGuard lg(ctx, "zero_fill", (double)bytes, 0);
   hipLaunchKernelGGL(k_zero16, dim3(grid_for(n16, kBlock, max_blocks(ctx))), dim3(kBlock), 0, ctx->stream, n16, (uint4*)p);
   HG_CHECK_LAUNCH(ctx, "zero_fill");
   return HGPU_OK;
@@ -254,7 +254,7 @@ int copy_view(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const vo
   const int64_t* sts[2] = {sst, dst_st};
   Dims d;
   if (!collapse(rank, shape, 2, sts, &d)) return fail(ctx, HGPU_ERR_UNSUPPORTED, "copy: more than %d merged dims", HG_KDIMS);
-  LaunchGuard lg(ctx);
+  LaunchGuard lg(ctx, "copy_view", 2.0 * n * dtype_size(dtype), 0);
   unsigned g = grid_for(n, kBlock, max_blocks(ctx));
   switch (dtype_size(dtype)) {
     case 8: hipLaunchKernelGGL(k_copy<uint64_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint64_t*)src, (uint64_t*)dst); break;
@@ -313,7 +313,7 @@ int hgpu_ewise1(hgpu_ctx* ctx, int op, const hgpu_array* a, hgpu_array** out) {
   if (rc) return rc;
   int64_t n = nelem(o);
   if (n > 0) {
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, "ewise1", 2.0 * n * dtype_size(a->dtype), (double)n);
     if (layout_class(a) == 1 && aligned16(data_ptr(a))) {
       unsigned g = grid_for(n, kBlock * 4, max_blocks(ctx));
       HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_ewise1_dense<T>, dim3(g), dim3(kBlock), 0, ctx->stream, op, n, (const T*)data_ptr(a), (T*)data_ptr(o)));
@@ -352,7 +352,7 @@ int hgpu_ewise2(hgpu_ctx* ctx, int op, const hgpu_array* a, const hgpu_array* b,
   if (rc) return rc;
   int64_t n = nelem(o);
   if (n > 0) {
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, "ewise2", 3.0 * n * dtype_size(a->dtype), (double)n);
     int la = layout_class(a), lb = layout_class(b);
     bool fast = la != 0 && lb != 0 && !(la == 2 && lb == 2) && (la == 2 || aligned16(data_ptr(a))) && (lb == 2 || aligned16(data_ptr(b)));
     if (fast) {
@@ -392,7 +392,7 @@ int hgpu_compare(hgpu_ctx* ctx, int cmp, const hgpu_array* a, const hgpu_array* 
     const int64_t* sts[2] = {a->strides, b->strides};
     Dims d;
     if (!collapse(a->rank, a->shape, 2, sts, &d)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "compare: too many dims"); }
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, "compare", n * (2.0 * dtype_size(a->dtype) + 1), (double)n);
     unsigned g = grid_for(n, kBlock, max_blocks(ctx));
     HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_cmp<T>, dim3(g), dim3(kBlock), 0, ctx->stream, cmp, d, n, (const T*)data_ptr(a), (const T*)data_ptr(b), (uint8_t*)data_ptr(o)));
     hipError_t e = hipGetLastError();
@@ -416,7 +416,7 @@ int hgpu_select(hgpu_ctx* ctx, const hgpu_array* c, const hgpu_array* a, const h
     const int64_t* sts[3] = {c->strides, a->strides, b->strides};
     Dims d;
     if (!collapse(a->rank, a->shape, 3, sts, &d)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "select: too many dims"); }
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, "select", n * (3.0 * dtype_size(a->dtype) + 1), (double)n);
     unsigned g = grid_for(n, kBlock, max_blocks(ctx));
     HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_select<T>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint8_t*)data_ptr(c), (const T*)data_ptr(a), (const T*)data_ptr(b), (T*)data_ptr(o)));
     hipError_t e = hipGetLastError();
@@ -439,7 +439,7 @@ int hgpu_convert(hgpu_ctx* ctx, const hgpu_array* a, int dtype, int mode, hgpu_a
     const int64_t* sts[1] = {a->strides};
     Dims d;
     if (!collapse(a->rank, a->shape, 1, sts, &d)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "convert: too many dims"); }
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, "convert", (double)n * (dtype_size(a->dtype) + dtype_size(dtype)), (double)n);
     unsigned g = grid_for(n, kBlock, max_blocks(ctx));
     HG_DISPATCH_DTYPE(a->dtype, S, {
       HG_DISPATCH_DTYPE(dtype, D, hipLaunchKernelGGL((k_convert<S, D>), dim3(g), dim3(kBlock), 0, ctx->stream, mode, d, n, (const S*)data_ptr(a), (D*)data_ptr(o)));
@@ -458,7 +458,7 @@ int hgpu_iota(hgpu_ctx* ctx, int64_t n, int dtype, hgpu_array** out) {
   int rc = new_dense(ctx, dtype, 1, &n, &o);
   if (rc) return rc;
   if (n > 0) {
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, "iota", (double)n * dtype_size(dtype), 0);
     unsigned g = grid_for(n, kBlock, max_blocks(ctx));
     HG_DISPATCH_DTYPE(dtype, T, hipLaunchKernelGGL(k_iota<T>, dim3(g), dim3(kBlock), 0, ctx->stream, n, (T*)data_ptr(o)));
     hipError_t e = hipGetLastError();

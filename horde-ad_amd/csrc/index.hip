@@ -214,7 +214,7 @@ int hgpu_gather(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array
   Dims inner;
   if (!collapse(rank_n, src->shape + n_ix, 1, is, &inner)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "gather: too many inner dims"); }
   {
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, "gather", 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, 0);
     unsigned g = grid_for(M * N, kBlock, ctx->num_cu * 8);
     switch (dtype_size(src->dtype)) {
       case 8: hipLaunchKernelGGL(k_gather<uint64_t>, dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, (const uint64_t*)data_ptr(src), (uint64_t*)data_ptr(o)); break;
@@ -257,7 +257,7 @@ int hgpu_scatter_add(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_
   bool inj = (flags & 1) != 0;
   bool launched = false;
   {
-    LaunchGuard lg(ctx);
+    LaunchGuard lg(ctx, inj ? "scatter_store" : "scatter_atomic", 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, (double)M * N);
     unsigned g = grid_for(M * N, kBlock, ctx->num_cu * 8);
     HG_DISPATCH_DTYPE(src->dtype, T, {
       if constexpr (atomic_ok<T>::value) {

@@ -308,6 +308,41 @@ int hgpu_inject_alloc_failure(hgpu_ctx* ctx, int64_t limit) {
   return HGPU_OK;
 }
 
+int hgpu_profile_enable(hgpu_ctx* ctx, int on) {
+  if (!ctx) return HGPU_ERR_INVALID;
+  std::lock_guard<std::mutex> g(ctx->launch_mu);
+  (void)hipStreamSynchronize(ctx->stream);
+  for (auto& r : ctx->prof) { (void)hipEventDestroy(r.a); (void)hipEventDestroy(r.b); }
+  ctx->prof.clear();
+  ctx->profiling = on != 0;
+  return HGPU_OK;
+}
+
+int hgpu_profile_report(hgpu_ctx* ctx, char* buf, size_t n) {
+  if (!ctx || !buf || n == 0) return HGPU_ERR_INVALID;
+  std::lock_guard<std::mutex> g(ctx->launch_mu);
+  (void)hipStreamSynchronize(ctx->stream);
+  struct Agg { long count = 0; double ms = 0, bytes = 0, flops = 0; };
+  std::map<std::string, Agg> agg;
+  for (auto& r : ctx->prof) {
+    float ms = 0;
+    if (hipEventElapsedTime(&ms, r.a, r.b) != hipSuccess) continue;
+    Agg& a = agg[r.name];
+    a.count++;
+    a.ms += ms;
+    a.bytes += r.bytes;
+    a.flops += r.flops;
+  }
+  std::string out;
+  char line[256];
+  for (auto& kv : agg) {
+    snprintf(line, sizeof line, "%s %ld %.6f %.0f %.0f\n", kv.first.c_str(), kv.second.count, kv.second.ms, kv.second.bytes, kv.second.flops);
+    out += line;
+  }
+  snprintf(buf, n, "%s", out.c_str());
+  return HGPU_OK;
+}
+
 int hgpu_upload(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const void* host, hgpu_array** out) {
   if (!ctx || !out) return HGPU_ERR_INVALID;
   *out = nullptr;

@@ -57,7 +57,9 @@ D d_const(const T& t) {
   return d;
 }
 
-static T mul(const T& a, const T& b) { return ewise2(HGPU_MUL, a, b); }
+// Products made by transposition rules stay pending: most are summed at once
+// by the rule of a `replicate` further up, which then is a single contraction.
+static T mul(const T& a, const T& b) { return lazy_mul(a, b); }
 static T add(const T& a, const T& b) { return ewise2(HGPU_ADD, a, b); }
 static T neg(const T& a) { return ewise1(HGPU_NEG, a); }
 static T recip(const T& a) { return ewise1(HGPU_RECIP, a); }
@@ -242,6 +244,41 @@ D d_tsdot1In(Tape& tp, const D& a, const D& b) {
     if (an >= 0) accum(s, an, mul(v, cc));
     if (bn >= 0) accum(s, bn, mul(u, cc));
   });
+  return r;
+}
+
+// The cotangent of a contraction over the n innermost dims, broadcast back.
+static T expand_inner_n(const T& c, const Shape& inner) {
+  int r = c.rank(), n = (int)inner.size();
+  std::vector<int> perm((size_t)(r + n));
+  for (int i = 0; i < r; ++i) perm[(size_t)i] = i + n;
+  for (int i = 0; i < n; ++i) perm[(size_t)(r + i)] = i;
+  return transpose(replicate(c, inner), perm);
+}
+
+D d_tsdotNIn(Tape& tp, const D& a, const D& b, int n) {
+  D r;
+  r.primal = tsdotNIn(a.primal, b.primal, n);
+  if (a.node < 0 && b.node < 0) return r;
+  T u = a.primal, v = b.primal;
+  int an = a.node, bn = b.node;
+  Shape sh = u.shape();
+  Shape inner(sh.end() - n, sh.end());
+  r.node = tp.push([an, bn, u, v, inner](const T& c, std::vector<T>& s) {
+    T cc = expand_inner_n(c, inner);
+    if (an >= 0) accum(s, an, mul(v, cc));
+    if (bn >= 0) accum(s, bn, mul(u, cc));
+  });
+  return r;
+}
+
+// tD (Ops.hs, `tD stk primal dual`): used by lossSoftMaxCrossEntropyS
+// (External/CommonShapedOps.hs:89-111) to pair a primal with a hand-made dual.
+D d_tD(const D& primal, const D& dual) {
+  if (primal.primal.shape() != dual.primal.shape()) throw HostError(HGPU_ERR_INVALID, "tD: primal and dual parts differ in shape");
+  D r;
+  r.primal = primal.primal;
+  r.node = dual.node;
   return r;
 }
 

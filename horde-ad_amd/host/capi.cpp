@@ -136,6 +136,10 @@ int hh_tssumN(hh_ctx* c, hh_val* t, int k, hh_val** out) { HH_OP(d_tssumN(c->tap
 int hh_tssum0(hh_ctx* c, hh_val* t, hh_val** out) { HH_OP(d_tssum0(c->tape, t->d)); }
 int hh_tsdot0(hh_ctx* c, hh_val* a, hh_val* b, hh_val** out) { HH_OP(d_tsdot0(c->tape, a->d, b->d)); }
 int hh_tsdot1In(hh_ctx* c, hh_val* a, hh_val* b, hh_val** out) { HH_OP(d_tsdot1In(c->tape, a->d, b->d)); }
+int hh_tsdotNIn(hh_ctx* c, hh_val* a, hh_val* b, int n, hh_val** out) { HH_OP(d_tsdotNIn(c->tape, a->d, b->d, n)); }
+int hh_as_input(hh_ctx* c, hh_val* v, hh_val** out) { HH_OP(c->tape.input(v->d.primal)); }
+int hh_tprimalPart(hh_ctx* c, hh_val* v, hh_val** out) { HH_OP(d_const(v->d.primal)); }
+int hh_tD(hh_ctx* c, hh_val* primal, hh_val* dual, hh_val** out) { HH_OP(d_tD(primal->d, dual->d)); }
 int hh_tsmatvecmul(hh_ctx* c, hh_val* m, hh_val* v, hh_val** out) {
   HH_OP(d_tsdot1In(c->tape, m->d, d_tsreplicateN(c->tape, v->d, {m->d.primal.shape().at(0)})));
 }

@@ -44,9 +44,14 @@ struct ArrHolder {
   // Small integer arrays that came from the host keep their values: index
   // functions that look constants up in them can then be folded on the host.
   std::shared_ptr<std::vector<int64_t>> host_i64;
+  // A pending elementwise product fa * fb (h == nullptr until it is needed as
+  // an array).  Views of it stay pending, and summing it is a contraction of
+  // the two factors, so `tssumN (u * v)` never writes the product to memory.
+  std::shared_ptr<ArrHolder> fa, fb;
   ArrHolder(Backend* b, hgpu_array* a) : be(b), h(a) {}
   ~ArrHolder() { if (h) be->api->release(h); }
   ArrHolder(const ArrHolder&) = delete;
+  void force();
 };
 
 // `Gpu (TKS sh r)`: an immutable strided view on the device.  Scalars
@@ -59,10 +64,22 @@ class T {
   const std::shared_ptr<ArrHolder>& holder() const { return p_; }
   bool valid() const { return (bool)p_; }
   Backend* be() const { return p_->be; }
-  hgpu_array* h() const { return p_->h; }
-  int rank() const { return be()->api->rank(h()); }
-  int dtype() const { return be()->api->dtype_of(h()); }
-  int64_t size() const { return be()->api->size(h()); }
+  hgpu_array* h() const {
+    if (!p_->h) p_->force();
+    return p_->h;
+  }
+  bool pending_product() const { return p_ && !p_->h && p_->fa; }
+  T factor_a() const { return T(p_->fa); }
+  T factor_b() const { return T(p_->fb); }
+  // metadata never forces a pending product: the first factor has the same
+  hgpu_array* meta_h() const {
+    const ArrHolder* q = p_.get();
+    while (!q->h && q->fa) q = q->fa.get();
+    return q->h;
+  }
+  int rank() const { return be()->api->rank(meta_h()); }
+  int dtype() const { return be()->api->dtype_of(meta_h()); }
+  int64_t size() const { return be()->api->size(meta_h()); }
   Shape shape() const;
   Shape strides() const;
   const std::shared_ptr<std::vector<int64_t>>& host_i64() const { return p_->host_i64; }
@@ -88,6 +105,7 @@ T materialize(const T& a);
 T pad(const T& a, const Shape& lo, const Shape& hi);
 T ewise1(int op, const T& a);
 T ewise2(int op, const T& a, const T& b);
+T lazy_mul(const T& a, const T& b);                                // a * b, not yet written to memory
 T compare(int cmp, const T& a, const T& b);
 bool compare_all(int cmp, const T& a, const T& b);
 T select(const T& c, const T& a, const T& b);
@@ -107,6 +125,7 @@ T tssumN(const T& t, int k);               // sum over the k outermost dims
 T tssum0(const T& t);
 T tsdot0(const T& a, const T& b);
 T tsdot1In(const T& a, const T& b);        // contraction over the innermost dim
+T tsdotNIn(const T& a, const T& b, int n); // contraction over the n innermost dims
 T tsmatvecmul(const T& m, const T& v);
 T tsmatmul2(const T& m1, const T& m2);
 T tsreplicate(const T& t, int64_t k);
@@ -196,6 +215,8 @@ D d_tssumN(Tape& tp, const D& t, int k);
 D d_tssum0(Tape& tp, const D& t);
 D d_tsdot0(Tape& tp, const D& a, const D& b);
 D d_tsdot1In(Tape& tp, const D& a, const D& b);
+D d_tsdotNIn(Tape& tp, const D& a, const D& b, int n);
+D d_tD(const D& primal, const D& dual);                 // tD: primal part of one, dual part of the other
 D d_tsmatmul2(Tape& tp, const D& a, const D& b);
 D d_tsreplicateN(Tape& tp, const D& t, const Shape& shm);
 D d_tsappend(Tape& tp, const D& a, const D& b);

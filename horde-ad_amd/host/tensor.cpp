@@ -15,7 +15,7 @@ void Backend::check(int rc) const {
 
 Shape T::shape() const {
   Shape s((size_t)rank());
-  if (!s.empty()) be()->api->shape(h(), s.data());
+  if (!s.empty()) be()->api->shape(meta_h(), s.data());
   return s;
 }
 Shape T::strides() const {
@@ -104,18 +104,49 @@ T iota(Backend* be, int64_t n, int dtype) {
   be__->check(be__->api->call);           \
   return T(be__, o__)
 
+void ArrHolder::force() {
+  if (h || !fa) return;
+  T p = ewise2(HGPU_MUL, T(fa), T(fb));
+  be->check(be->api->retain(p.h()));
+  h = p.h();
+  fa.reset();
+  fb.reset();
+}
+
+T lazy_mul(const T& a, const T& b) {
+  if (a.dtype() != b.dtype() || a.shape() != b.shape()) return ewise2(HGPU_MUL, a, b);  // reports the mismatch
+  auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
+  p->fa = a.holder();
+  p->fb = b.holder();
+  return T(p);
+}
+
+#define HD_VIEW_OF_PRODUCT(expr_a, expr_b) \
+  if (a.pending_product()) { T a0 = a.factor_a(), b0 = a.factor_b(); return lazy_mul(expr_a, expr_b); }
+
 T transpose(const T& a, const std::vector<int>& perm) {
+  HD_VIEW_OF_PRODUCT(transpose(a0, perm), transpose(b0, perm))
   static const int dummy = 0;
   HD_OUT(transpose(be__->ctx, a.h(), (int)perm.size(), perm.empty() ? &dummy : perm.data(), &o__));
 }
 T reshape(const T& a, const Shape& s) { HD_OUT(reshape(be__->ctx, a.h(), (int)s.size(), ptr_or_dummy(s), &o__)); }
-T slice(const T& a, int dim, int64_t start, int64_t len) { HD_OUT(slice(be__->ctx, a.h(), dim, start, len, &o__)); }
-T reverse(const T& a, int dim) { HD_OUT(reverse(be__->ctx, a.h(), dim, &o__)); }
+T slice(const T& a, int dim, int64_t start, int64_t len) {
+  HD_VIEW_OF_PRODUCT(slice(a0, dim, start, len), slice(b0, dim, start, len))
+  HD_OUT(slice(be__->ctx, a.h(), dim, start, len, &o__));
+}
+T reverse(const T& a, int dim) {
+  HD_VIEW_OF_PRODUCT(reverse(a0, dim), reverse(b0, dim))
+  HD_OUT(reverse(be__->ctx, a.h(), dim, &o__));
+}
 T replicate(const T& a, const Shape& pre) {
   if (pre.empty()) return a;
+  HD_VIEW_OF_PRODUCT(replicate(a0, pre), replicate(b0, pre))
   HD_OUT(replicate(be__->ctx, a.h(), (int)pre.size(), pre.data(), &o__));
 }
-T index_prefix(const T& a, const Shape& ix) { HD_OUT(index_prefix(be__->ctx, a.h(), (int)ix.size(), ptr_or_dummy(ix), &o__)); }
+T index_prefix(const T& a, const Shape& ix) {
+  HD_VIEW_OF_PRODUCT(index_prefix(a0, ix), index_prefix(b0, ix))
+  HD_OUT(index_prefix(be__->ctx, a.h(), (int)ix.size(), ptr_or_dummy(ix), &o__));
+}
 T as_strided(const T& a, const Shape& shape, const Shape& strides, int64_t offset) {
   HD_OUT(as_strided(be__->ctx, a.h(), (int)shape.size(), ptr_or_dummy(shape), ptr_or_dummy(strides), offset, &o__));
 }
@@ -134,7 +165,13 @@ T convert(const T& a, int dtype, int mode) {
   if (a.dtype() == dtype && mode == HGPU_CONV_CAST) return a;
   HD_OUT(convert(be__->ctx, a.h(), dtype, mode, &o__));
 }
-T contract(const T& a, const T* b, int n_keep) { HD_OUT(contract(be__->ctx, a.h(), b ? b->h() : nullptr, n_keep, &o__)); }
+T contract(const T& a, const T* b, int n_keep) {
+  if (!b && a.pending_product()) {  // sum (u * v) = the contraction of u and v
+    T fa = a.factor_a(), fb = a.factor_b();
+    return contract(fa, &fb, n_keep);
+  }
+  HD_OUT(contract(be__->ctx, a.h(), b ? b->h() : nullptr, n_keep, &o__));
+}
 T argminmax_last(const T& a, bool want_max) { HD_OUT(argminmax_last(be__->ctx, a.h(), want_max ? 1 : 0, &o__)); }
 T concat(const std::vector<T>& parts) {
   if (parts.empty()) throw HostError(HGPU_ERR_INVALID, "concat of nothing");
@@ -190,6 +227,12 @@ T tsdot0(const T& a, const T& b) { return contract(a, &b, 0); }                /
 T tsdot1In(const T& a, const T& b) {                                           // Ops.hs:522, OpsConcrete.hs:233
   if (a.rank() < 1) throw HostError(HGPU_ERR_INVALID, "tsdot1In: rank 0");
   return contract(a, &b, a.rank() - 1);
+}
+// ssumN @sh (sdot1In u v) in one pass: the form conv layers reach the backend in
+// (test/simplified/TestMnistPP.hs:735, `t259 = ssumN @[3, 4] (sdot1In ...)`).
+T tsdotNIn(const T& a, const T& b, int n) {
+  if (n < 0 || n > a.rank()) throw HostError(HGPU_ERR_INVALID, "tsdotNIn: more contracted dims than rank");
+  return contract(a, &b, a.rank() - n);
 }
 T tsmatvecmul(const T& m, const T& v) {                                        // OpsConcrete.hs:236
   return tsdot1In(m, tsreplicate(v, m.shape().at(0)));

@@ -27,7 +27,7 @@ SIG = {
     "ewise1": (I, [P, I, P, PP]), "ewise2": (I, [P, I, P, P, PP]), "compare": (I, [P, I, P, P, PP]),
     "compare_all": (I, [P, I, P, P, IP]), "select": (I, [P, P, P, P, PP]), "convert": (I, [P, P, I, I, PP]),
     "tssumN": (I, [P, P, I, PP]), "tssum0": (I, [P, P, PP]), "tsdot0": (I, [P, P, P, PP]),
-    "tsdot1In": (I, [P, P, P, PP]), "tsmatvecmul": (I, [P, P, P, PP]), "tsmatmul2": (I, [P, P, P, PP]),
+    "tsdot1In": (I, [P, P, P, PP]), "tsdotNIn": (I, [P, P, P, I, PP]), "tD": (I, [P, P, P, PP]), "tprimalPart": (I, [P, P, PP]), "as_input": (I, [P, P, PP]), "tsmatvecmul": (I, [P, P, P, PP]), "tsmatmul2": (I, [P, P, P, PP]),
     "tsreplicateN": (I, [P, P, I, LP, PP]), "tsappend": (I, [P, P, P, PP]), "tsslice": (I, [P, P, L, L, PP]),
     "tsreverse": (I, [P, P, PP]), "tstranspose": (I, [P, P, I, IP, PP]), "tsreshape": (I, [P, P, I, LP, PP]),
     "tsindex": (I, [P, P, I, LP, PP]), "tsargminmax": (I, [P, P, I, PP]), "tsiota": (I, [P, L, I, PP]),
@@ -240,7 +240,13 @@ class V:
 
     # -- Num / Fractional / Floating
     def op1(self, name): return self._o(self.host.dll.hh_ewise1, OP1[name], self.h)
-    def op2(self, name, o): return self._o(self.host.dll.hh_ewise2, OP2[name], self.h, self._lift(o).h)
+    def op2(self, name, o):
+        o = self._lift(o)   # keeps the lifted constant alive across the call
+        return self._o(self.host.dll.hh_ewise2, OP2[name], self.h, o.h)
+
+    def _cmp(self, c, o):
+        o = self._lift(o)
+        return self._o(self.host.dll.hh_compare, CMP[c], self.h, o.h)
     def __add__(self, o): return self.op2("add", o)
     def __radd__(self, o): return self._lift(o).op2("add", self)
     def __sub__(self, o): return self.op2("sub", o)
@@ -256,9 +262,9 @@ class V:
     def remH(self, o): return self.op2("rem", o)
 
     # -- comparisons, conditionals, conversions
-    def leq(self, o): return self._o(self.host.dll.hh_compare, CMP["leq"], self.h, self._lift(o).h)
-    def lt(self, o): return self._o(self.host.dll.hh_compare, CMP["lt"], self.h, self._lift(o).h)
-    def eq(self, o): return self._o(self.host.dll.hh_compare, CMP["eq"], self.h, self._lift(o).h)
+    def leq(self, o): return self._cmp("leq", o)
+    def lt(self, o): return self._cmp("lt", o)
+    def eq(self, o): return self._cmp("eq", o)
 
     def compare_all(self, cmp, o):
         r = C.c_int()
@@ -279,6 +285,10 @@ class V:
     def ssum0(self): return self._o(self.host.dll.hh_tssum0, self.h)
     def sdot0(self, o): return self._o(self.host.dll.hh_tsdot0, self.h, o.h)
     def sdot1In(self, o): return self._o(self.host.dll.hh_tsdot1In, self.h, o.h)
+    def sdotNIn(self, o, n): return self._o(self.host.dll.hh_tsdotNIn, self.h, o.h, n)
+    def as_input(self): return self._o(self.host.dll.hh_as_input, self.h)
+    def sprimalPart(self): return self._o(self.host.dll.hh_tprimalPart, self.h)
+    def tD(self, dual): return self._o(self.host.dll.hh_tD, self.h, dual.h)
     def smatvecmul(self, v): return self._o(self.host.dll.hh_tsmatvecmul, self.h, v.h)
     def smatmul2(self, o): return self._o(self.host.dll.hh_tsmatmul2, self.h, o.h)
     def sargMax(self): return self._o(self.host.dll.hh_tsargminmax, self.h, 1)

@@ -1,0 +1,250 @@
+"""The five benchmark objectives as user programs over the carrier.
+
+Each function mirrors a definition of the reference, written in the form the
+reference's vectoriser leaves it in (builds over the batch eliminated, index
+functions kept), and calls the host layer one tensor operation at a time -- the
+way horde-ad's interpreter drives a `BaseTensor` instance:
+
+  reluS, lossSoftMaxCrossEntropyS, conv2dPreservingS, maxPool2dUnpaddedS
+      src/HordeAd/External/CommonShapedOps.hs:42-44, 89-111, 136-157, 241-260
+  convMnistLayerS / convMnistTwoS / convMnistLossFusedS
+      example/MnistCnnShaped2.hs:45-64, 67-108, 111-136
+  afcnnMnist2 (batched), rnnMnistLayerR / rnnMnistTwoR / rnnMnistZeroR
+      example/MnistFcnnRanked2.hs:52-66, example/MnistRnnRanked2.hs:62-110
+  foo (the elementwise objective)
+      test/simplified/TestAdaptorSimplified.hs:610-624
+
+Inputs are synthetic, drawn from numpy's counter-based Philox generator with
+fixed seeds, so that every provider of the array ABI sees the same numbers.
+"""
+import numpy as np
+
+from . import capi
+
+F64, F32 = capi.F64, capi.F32
+NP = {F64: np.float64, F32: np.float32}
+
+
+def _rng(seed):
+    return np.random.Generator(np.random.Philox(seed))
+
+
+def uniform(seed, shape, lo, hi, dtype):
+    return _rng(seed).uniform(lo, hi, shape).astype(NP[dtype])
+
+
+def pixels(seed, shape, dtype):
+    """Uniform integers 0..255 scaled by 1/255."""
+    return (_rng(seed).integers(0, 256, shape).astype(np.float64) / 255.0).astype(NP[dtype])
+
+
+def one_hot_labels(seed, n_classes, batch, dtype):
+    """[n_classes, batch] one-hot columns, classes uniform."""
+    cls = _rng(seed).integers(0, n_classes, batch)
+    out = np.zeros((n_classes, batch), NP[dtype])
+    out[cls, np.arange(batch)] = 1
+    return out
+
+
+# --------------------------------------------------------------- shared pieces
+
+def reluS(v):
+    """oneIfGtZero * v with oneIfGtZero = smap0N (\\x -> ifH (x <=. 0) 0 1) v."""
+    h = v.host
+    mask = v.sprimalPart().leq(0.0)
+    one_if = mask.select(h.srepl(v.shape, 0.0, v.dtype), h.srepl(v.shape, 1.0, v.dtype))
+    return one_if * v
+
+
+def sminimum(u):
+    """sindex0 tf [kargMin tf] on the flattened tensor."""
+    n = int(np.prod(u.shape))
+    tf = u.sreshape([n])
+    arg = tf.sargMin()
+    return tf.sgather((), lambda: [arg.lift(())])
+
+
+def lossSoftMaxCrossEntropyS(expected, d):
+    u = d.sprimalPart()
+    exp_u = (u - sminimum(u).sreplicate0N(u.shape)).op1("exp")
+    recip_sum = exp_u.ssum0().op1("recip")
+    soft = recip_sum.sreplicate0N(u.shape) * exp_u
+    primal = -(soft.op1("log").sdot0(expected))
+    dual = (soft - expected).sdot0(d)
+    return primal.tD(dual)
+
+
+def conv2dPreservingS(ker, arr):
+    """out[img, co, h, w] = sum_{ci, p, q} arr[img, ci, h + p, w + q] * ker[co, ci, p, q],
+    reading zeros beyond the image (slicezS)."""
+    co, ci, kh, kw = ker.shape
+    b, ci2, h, w = arr.shape
+    assert ci == ci2
+    win = arr.stranspose([2, 3, 0, 1]).sgather((h, kh, w, kw), lambda i, p, j, q: [i + p, j + q])
+    # win: [h, kh, w, kw, b, ci]
+    lhs = win.sreplicate(co).stranspose([5, 0, 1, 3, 6, 2, 4])          # [b, co, h, w, ci, kh, kw]
+    rhs = ker.sreplicateN([b, h, w]).stranspose([0, 3, 1, 2])           # [b, co, h, w, ci, kh, kw]
+    return lhs.sdotNIn(rhs, 3)
+
+
+def maxPool2dUnpaddedS(arr):
+    """ksize = stride = 2: smaximum of every 2x2 window."""
+    b, c, h, w = arr.shape
+    h2, w2 = h // 2, w // 2
+    win = arr.stranspose([2, 3, 0, 1]).sgather((h2, 2, w2, 2), lambda i, p, j, q: [2 * i + p, 2 * j + q])
+    win = win.stranspose([4, 5, 0, 2, 1, 3]).sreshape([b, c, h2, w2, 4])
+    wp = win.sprimalPart()
+    return win.sgather((b, c, h2, w2), lambda i, j, k, l: [i, j, k, l, wp.kargMax([i, j, k, l])])
+
+
+def convMnistLayerS(ker, inp, bias):
+    b, _, h, w = inp.shape
+    y = conv2dPreservingS(ker, inp)
+    bias_stretched = bias.sreplicateN([b, h, w]).stranspose([0, 3, 1, 2])
+    return maxPool2dUnpaddedS(reluS(y + bias_stretched))
+
+
+def convMnistTwoS(inp, params):
+    (k1, b1), (k2, b2), (wd, bd), (wr, br) = params
+    b = inp.shape[0]
+    t1 = convMnistLayerS(k1, inp, b1)
+    t2 = convMnistLayerS(k2, t1, b2)
+    m1 = t2.sreshape([b, int(np.prod(t2.shape[1:]))])
+    dense = wd.smatmul2(m1.str_()) + bd.sreplicate(b).str_()
+    return wr.smatmul2(reluS(dense)) + br.sreplicate(b).str_()
+
+
+# ------------------------------------------------------------------- configs
+
+class Workload:
+    """name, dtype, batch, numpy inputs (params first), and the objective."""
+
+    def __init__(self, name, dtype, batch, params, data, objective, flops, bytes_):
+        self.name, self.dtype, self.batch = name, dtype, batch
+        self.params, self.data, self.objective = params, data, objective
+        self.flops, self.bytes = flops, bytes_
+
+    def upload(self, host):
+        ps = [host.param(p) for p in self.params]
+        ds = [host.concrete(d) for d in self.data]
+        return ps, ds
+
+    def gradient(self, host, ps, ds):
+        """One forward + reverse pass: (loss, [d loss / d param])."""
+        host.tape_reset()
+        ps = [p.as_input() for p in ps]    # parameters are fresh tape inputs for every gradient
+        loss = self.objective(ps, ds)
+        return loss, host.grad(loss, ps)
+
+
+def c0_elementwise(n=4096, m=4096, dtype=F64):
+    """sum (atan2 z (x * sin y) + z * (x * sin y)); gradient w.r.t. x, y, z."""
+    def away(a):
+        return np.where(np.abs(a) < 0.1, np.where(a < 0, a - 0.1, a + 0.1), a).astype(NP[dtype])
+    x, y, z = (uniform(s, (n, m), -2, 2, dtype) for s in (1, 2, 3))
+    x, z = away(x), away(z)
+
+    def objective(ps, ds):
+        x, y, z = ps
+        w = x * y.op1("sin")
+        return (z.atan2H(w) + z * w).ssum0()
+
+    el = n * m
+    return Workload("c0_elementwise", dtype, el, [x, y, z], [], objective, flops=20.0 * el, bytes_=6.0 * el * np.dtype(NP[dtype]).itemsize)
+
+
+def _dense_net(name, dtype, batch, widths, act, seeds, init):
+    n_in = widths[0]
+    x = pixels(seeds[0], (n_in, batch), dtype)
+    labels = one_hot_labels(seeds[1], widths[-1], batch, dtype)
+    rng = _rng(seeds[2])
+    params = []
+    for fan_in, fan_out in zip(widths[:-1], widths[1:]):
+        r = init(fan_in, fan_out)
+        params.append(rng.uniform(-r, r, (fan_out, fan_in)).astype(NP[dtype]))
+        params.append(rng.uniform(-r, r, (fan_out,)).astype(NP[dtype]))
+
+    def objective(ps, ds):
+        xx, lab = ds
+        hcur = xx
+        n_layers = len(ps) // 2
+        for li in range(n_layers):
+            w, bias = ps[2 * li], ps[2 * li + 1]
+            hcur = w.smatmul2(hcur) + bias.sreplicate(batch).str_()
+            if li < n_layers - 1:
+                hcur = hcur.op1("tanh") if act == "tanh" else reluS(hcur)
+        loss = lossSoftMaxCrossEntropyS(lab, hcur)
+        return loss.host.srepl((), 1.0 / batch, dtype) * loss
+
+    mm = sum(a * b for a, b in zip(widths[:-1], widths[1:]))
+    dx = sum(a * b for a, b in zip(widths[1:-1], widths[2:]))
+    flops = 2.0 * batch * (2 * mm + dx)
+    return Workload(name, dtype, batch, params, [x, labels], objective, flops=flops, bytes_=None)
+
+
+def c1_fcnn(batch=5000, dtype=F64, widths=(784, 300, 100, 10)):
+    return _dense_net("c1_fcnn", dtype, batch, widths, "tanh", (11, 12, 13), lambda i, o: 0.5)
+
+
+def c2_wide(batch=8192, dtype=F32, widths=(784, 2048, 2048, 10)):
+    return _dense_net("c2_wide", dtype, batch, widths, "relu", (11, 12, 21), lambda i, o: float(np.sqrt(6.0 / (i + o))))
+
+
+def c3_cnn(batch=1000, dtype=F64, h=28, w=28, ksize=5, c_out=16, n_hidden=128, n_classes=10):
+    inp = pixels(31, (batch, 1, h, w), dtype)
+    labels = one_hot_labels(32, n_classes, batch, dtype)
+    rng = _rng(33)
+    flat = c_out * (h // 4) * (w // 4)
+    shapes = [(c_out, 1, ksize, ksize), (c_out,), (c_out, c_out, ksize, ksize), (c_out,),
+              (n_hidden, flat), (n_hidden,), (n_classes, n_hidden), (n_classes,)]
+    params = [rng.uniform(-0.4, 0.4, s).astype(NP[dtype]) for s in shapes]
+
+    def objective(ps, ds):
+        x, lab = ds
+        result = convMnistTwoS(x, list(zip(ps[0::2], ps[1::2])))
+        loss = lossSoftMaxCrossEntropyS(lab, result)
+        return loss.host.srepl((), 1.0 / batch, dtype) * loss
+
+    k2 = ksize * ksize
+    conv1 = 2.0 * batch * c_out * h * w * k2
+    conv2 = 2.0 * batch * c_out * c_out * (h // 2) * (w // 2) * k2
+    dense = 2.0 * batch * flat * n_hidden
+    ro = 2.0 * batch * n_hidden * n_classes
+    flops = 2 * conv1 + 3 * conv2 + 3 * dense + 3 * ro
+    return Workload("c3_cnn", dtype, batch, params, [inp, labels], objective, flops=flops, bytes_=None)
+
+
+def c4_rnn(batch=5000, dtype=F32, steps=28, n_in=28, width=128, n_classes=10):
+    xs = pixels(41, (steps, n_in, batch), dtype)
+    labels = one_hot_labels(43, n_classes, batch, dtype)
+    rng = _rng(42)
+    shapes = [(width, n_in), (width, width), (width,), (width, width), (width, width), (width,),
+              (n_classes, width), (n_classes,)]
+    params = [rng.uniform(-0.1, 0.1, s).astype(NP[dtype]) for s in shapes]
+
+    def layer(s, x, wx, ws, b):
+        return (wx.smatmul2(x) + ws.smatmul2(s) + b.sreplicate(batch).str_()).op1("tanh")
+
+    def objective(ps, ds):
+        xs_, lab = ds
+        wx, ws, b, wx2, ws2, b2, w3, b3 = ps
+        host = wx.host
+        s = host.srepl((2 * width, batch), 0.0, dtype)           # zeroStateR
+        out = None
+        for t in range(steps):                                    # unrollLastR: foldl' over runravelToList
+            x = xs_.sindex([t])
+            s1, s2 = s.sslice(0, width), s.sslice(width, width)
+            v1 = layer(s1, x, wx, ws, b)
+            v2 = layer(s2, v1, wx2, ws2, b2)
+            s = v1.sappend(v2)
+            out = s.sslice(width, width)
+        result = w3.smatmul2(out) + b3.sreplicate(batch).str_()
+        loss = lossSoftMaxCrossEntropyS(lab, result)
+        return host.srepl((), 1.0 / batch, dtype) * loss
+
+    per_step = 2.0 * batch * (width * n_in + 3 * width * width)
+    flops = 3 * steps * per_step + 3 * 2.0 * batch * width * n_classes
+    return Workload("c4_rnn", dtype, batch, params, [xs, labels], objective, flops=flops, bytes_=None)
+
+
+CONFIGS = {"c0": c0_elementwise, "c1": c1_fcnn, "c2": c2_wide, "c3": c3_cnn, "c4": c4_rnn}

@@ -114,6 +114,13 @@ void* hgpu_stream(hgpu_ctx* ctx);
  * path); a negative value switches it off. */
 int hgpu_inject_alloc_failure(hgpu_ctx* ctx, int64_t limit);
 
+/* Per-launch timing for benchmarks: while enabled every kernel launch is
+ * bracketed by a HIP event pair on the context's stream.  The report has one
+ * line per kernel family: "name launches total_ms algorithmic_bytes
+ * algorithmic_flops".  Enabling (or disabling) clears the records. */
+int hgpu_profile_enable(hgpu_ctx* ctx, int on);
+int hgpu_profile_report(hgpu_ctx* ctx, char* buf, size_t n);
+
 /* ----------------------------------------------------------------- memory */
 
 /* tkconcrete/tsconcrete/tconcrete (OpsConcrete.hs:120-124): identity on the

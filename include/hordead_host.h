@@ -75,6 +75,17 @@ int hh_tssumN(hh_ctx* ctx, hh_val* t, int k, hh_val** out);              /* Ops.
 int hh_tssum0(hh_ctx* ctx, hh_val* t, hh_val** out);                     /* Ops.hs:517 */
 int hh_tsdot0(hh_ctx* ctx, hh_val* a, hh_val* b, hh_val** out);          /* Ops.hs:519 */
 int hh_tsdot1In(hh_ctx* ctx, hh_val* a, hh_val* b, hh_val** out);        /* Ops.hs:522 */
+/* ssumN @sh (sdot1In a b) as one contraction over the n innermost dims
+ * (the shape conv layers reach the backend in, TestMnistPP.hs:735 `t259`). */
+int hh_tsdotNIn(hh_ctx* ctx, hh_val* a, hh_val* b, int n, hh_val** out);
+/* The same array as a fresh differentiable input of the current tape (what
+ * crevOnParams does with the parameters for every gradient, OpsADVal.hs:62-73). */
+int hh_as_input(hh_ctx* ctx, hh_val* v, hh_val** out);
+/* tprimalPart (OpsConcrete.hs:761): the value without its dual part. */
+int hh_tprimalPart(hh_ctx* ctx, hh_val* v, hh_val** out);
+/* tD: the primal part of `primal` with the dual part (tape node) of `dual`
+ * (lossSoftMaxCrossEntropyS, External/CommonShapedOps.hs:89-111). */
+int hh_tD(hh_ctx* ctx, hh_val* primal, hh_val* dual, hh_val** out);
 int hh_tsmatvecmul(hh_ctx* ctx, hh_val* m, hh_val* v, hh_val** out);     /* Ops.hs:538 */
 int hh_tsmatmul2(hh_ctx* ctx, hh_val* a, hh_val* b, hh_val** out);       /* Ops.hs:543 */
 int hh_tsreplicateN(hh_ctx* ctx, hh_val* t, int n, const int64_t* shm, hh_val** out);   /* Ops.hs:552; also tsreplicate0N */

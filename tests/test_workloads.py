@@ -1,0 +1,127 @@
+"""The five objectives through the host layer.
+
+CPU half (no GPU): the host layer driving the CPU checker is compared with the
+independent numpy gradients of tests/ref_numpy.py and with known answers held
+by the reference's own tests -- this pins the operation sequences, the
+transposition rules and the index-function machinery.
+
+GPU half: the same programs on the gfx950 library against the checker on the
+same seeded inputs: fp64 to 1e-10, fp32 to 1e-5 (normwise relative; device
+reductions associate differently from the checker's sequential double sums).
+"""
+import numpy as np
+import pytest
+
+import ref_numpy as ref
+from conftest import capi, entry, pkg
+
+H, W = pkg.hostapi, pkg.workloads
+
+SMALL = {
+    "c0": (W.c0_elementwise, dict(n=17, m=9)),
+    "c1": (W.c1_fcnn, dict(batch=11, widths=(12, 7, 5, 3))),
+    "c2": (W.c2_wide, dict(batch=9, widths=(12, 9, 8, 4))),
+    "c3": (W.c3_cnn, dict(batch=3, h=8, w=12, ksize=3, c_out=2, n_hidden=5, n_classes=4)),
+    "c4": (W.c4_rnn, dict(batch=4, steps=5, n_in=5, width=6, n_classes=3)),
+}
+MEDIUM = {
+    "c0": (W.c0_elementwise, dict(n=301, m=257)),
+    "c1": (W.c1_fcnn, dict(batch=130, widths=(784, 300, 100, 10))),
+    "c2": (W.c2_wide, dict(batch=96, widths=(784, 256, 192, 10))),
+    "c3": (W.c3_cnn, dict(batch=6, h=28, w=28, ksize=5, c_out=16, n_hidden=128, n_classes=10)),
+    "c4": (W.c4_rnn, dict(batch=70, steps=28, n_in=28, width=128, n_classes=10)),
+}
+TOL = {capi.F64: 1e-10, capi.F32: 1e-5}
+
+
+@pytest.fixture(scope="module")
+def host_cpu():
+    return H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+
+
+@pytest.fixture(scope="module")
+def host_gpu():
+    return H.Host()
+
+
+def numpy_reference(name, wl):
+    if name == "c0":
+        return ref.c0(*wl.params)
+    if name in ("c1", "c2"):
+        return ref.dense_net(wl.params, wl.data[0], wl.data[1], "tanh" if name == "c1" else "relu")
+    if name == "c3":
+        return ref.cnn(wl.params, *wl.data)
+    return ref.rnn(wl.params, *wl.data)
+
+
+def run(host, wl):
+    ps, ds = wl.upload(host)
+    loss, grads = wl.gradient(host, ps, ds)
+    return float(loss.numpy()), [g.numpy() for g in grads]
+
+
+def close(a, b, tol):
+    scale = max(float(np.max(np.abs(b))), 1e-300)
+    return float(np.max(np.abs(a - b))) <= tol * scale
+
+
+@pytest.mark.parametrize("name", list(SMALL))
+def test_host_on_checker_matches_numpy(host_cpu, name):
+    mk, kw = SMALL[name]
+    wl = mk(**kw)
+    loss, grads = run(host_cpu, wl)
+    rloss, rgrads = numpy_reference(name, wl)
+    tol = 1e-11 if wl.dtype == capi.F64 else 2e-5
+    assert abs(loss - rloss) <= tol * abs(rloss)
+    assert len(grads) == len(rgrads)
+    for i, (g, r) in enumerate(zip(grads, rgrads)):
+        assert g.shape == r.shape, i
+        assert close(g, r, tol), (name, i)
+
+
+def test_foo_known_answers(host_cpu):
+    """foo (x, y, z) = atan2H z (x * sin y) + z * (x * sin y) at (1.1, 2.2, 3.3):
+    value and gradient as the reference's tests expect them
+    (test/simplified/TestAdaptorSimplified.hs:610-674, 749-759)."""
+    for dt, tol, want in [(np.float64, 1e-13, (2.4396285219055063, -1.953374825727421, 0.9654825811012627)),
+                          (np.float32, 1e-6, (2.4396284, -1.9533751, 0.96548253))]:
+        x, y, z = (host_cpu.param(np.array(v, dt)) for v in (1.1, 2.2, 3.3))
+        w = x * y.op1("sin")
+        f = z.atan2H(w) + z * w
+        if dt == np.float64:
+            assert abs(float(f.numpy()) - 4.242393641025528) < 1e-13
+        got = [float(g.numpy()) for g in host_cpu.grad(f, [x, y, z])]
+        assert np.allclose(got, want, rtol=tol, atol=0)
+    # summed over a [3, 534, 3] broadcast of the same point the gradient is unchanged per element
+    xs = [host_cpu.param(np.full((3, 5, 3), v)) for v in (1.1, 2.2, 3.3)]
+    w = xs[0] * xs[1].op1("sin")
+    f = (xs[2].atan2H(w) + xs[2] * w).ssum0()
+    for g, wv in zip(host_cpu.grad(f, xs), (2.4396285219055063, -1.953374825727421, 0.9654825811012627)):
+        assert np.allclose(g.numpy(), wv, rtol=1e-13)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("size", ["small", "medium"])
+@pytest.mark.parametrize("name", list(SMALL))
+def test_gpu_matches_checker(host_gpu, host_cpu, name, size):
+    mk, kw = (SMALL if size == "small" else MEDIUM)[name]
+    wl = mk(**kw)
+    gl, gg = run(host_gpu, wl)
+    cl, cg = run(host_cpu, wl)
+    tol = TOL[wl.dtype]
+    assert abs(gl - cl) <= tol * abs(cl), (gl, cl)
+    for i, (g, c) in enumerate(zip(gg, cg)):
+        assert g.shape == c.shape and g.dtype == c.dtype
+        assert close(g, c, tol), (name, size, i, float(np.max(np.abs(g - c))) / max(float(np.max(np.abs(c))), 1e-300))
+
+
+@pytest.mark.gpu
+def test_gpu_c0_full_size_properties(host_gpu):
+    """At the benchmark's full size the checker is too slow; the gradient of the
+    elementwise objective is checked against numpy's closed form instead."""
+    wl = W.c0_elementwise()
+    loss, grads = run(host_gpu, wl)
+    rloss, rgrads = ref.c0(*wl.params)
+    assert abs(loss - rloss) <= 1e-10 * abs(rloss)
+    for g, r in zip(grads, rgrads):
+        assert close(g, r, 1e-10)
