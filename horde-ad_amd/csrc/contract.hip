@@ -157,6 +157,53 @@ __global__ void __launch_bounds__(kBlock) k_argminmax(Dims keep, int64_t n_out, 
   }
 }
 
+// The same with one wavefront per row, for long rows: every lane scans a
+// strided subsequence keeping its first extremum, then lanes combine; on equal
+// values the smaller index wins, which keeps "first occurrence".
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_argminmax_wave(Dims keep, int64_t n_out, int64_t L, int64_t sl, int want_max, const T* __restrict__ a, int64_t* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  int64_t wave = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
+  int64_t nwaves = ((int64_t)gridDim.x * kBlock) >> 6;
+  for (int64_t o = wave; o < n_out; o += nwaves) {
+    int64_t ko[1];
+    decompose<1>(keep, o, ko);
+    const T* p = a + ko[0];
+    bool have = lane < L;
+    T best = have ? p[(int64_t)lane * sl] : T(0);
+    int64_t bi = lane;
+    for (int64_t j = lane + 64; j < L; j += 64) {
+      T x = p[j * sl];
+      bool better = want_max ? (x > best) : (x < best);
+      if (better) { best = x; bi = j; }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      int o_have = __shfl_down((int)have, off, 64);
+      long long o_bi = __shfl_down((long long)bi, off, 64);
+      T o_best;
+      if constexpr (sizeof(T) == 8) {
+        unsigned long long u = *reinterpret_cast<unsigned long long*>(&best);
+        unsigned lo = __shfl_down((unsigned)(u & 0xffffffffu), off, 64);
+        unsigned hi = __shfl_down((unsigned)(u >> 32), off, 64);
+        unsigned long long w = ((unsigned long long)hi << 32) | lo;
+        o_best = *reinterpret_cast<T*>(&w);
+      } else if constexpr (sizeof(T) == 4) {
+        unsigned u = *reinterpret_cast<unsigned*>(&best);
+        unsigned w = __shfl_down(u, off, 64);
+        o_best = *reinterpret_cast<T*>(&w);
+      } else {
+        int w = __shfl_down((int)best, off, 64);
+        o_best = (T)w;
+      }
+      if (o_have) {
+        bool better = !have || (want_max ? (o_best > best) : (o_best < best)) || (o_best == best && o_bi < bi);
+        if (better) { best = o_best; bi = o_bi; have = true; }
+      }
+    }
+    if (lane == 0) out[o] = bi;
+  }
+}
+
 template <typename TI, typename TO>
 int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red_full, int64_t n_out, int64_t R, int S, const void* a, const void* b, void* out) {
   LaunchGuard lg(ctx, b ? (use_wave ? "contract_dot_wave" : "contract_dot_lane") : (use_wave ? "contract_sum_wave" : "contract_sum_lane"),
@@ -298,8 +345,13 @@ int hgpu_argminmax_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_a
     Dims keep;
     if (!collapse(a->rank - 1, a->shape, 1, ks, &keep)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "argminmax: too many dims"); }
     LaunchGuard lg(ctx, "argminmax", (double)n_out * (L * dtype_size(a->dtype) + 8), (double)n_out * L);
-    unsigned g = grid_for(n_out, kBlock, ctx->num_cu * 8);
-    HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
+    if (L >= 256 && n_out < (int64_t)ctx->num_cu * 64) {
+      unsigned g = grid_for(n_out * 64, kBlock, ctx->num_cu * 8);
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_wave<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
+    } else {
+      unsigned g = grid_for(n_out, kBlock, ctx->num_cu * 8);
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "argminmax"); }
   }

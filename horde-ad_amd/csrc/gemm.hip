@@ -1,12 +1,383 @@
-// Matrix-core (MFMA) path of hgpu_contract: recognises contractions that are
-// matrix products over strided views and runs them on gfx950's matrix cores.
+// Matrix-core (MFMA) path of hgpu_contract.
+//
+// horde-ad's `Concrete` backend computes matmul2 as "dot over the innermost
+// dim of two broadcast views" (src/HordeAd/Core/OpsConcrete.hs:237-242) and
+// convolutions as the same contraction over gathered windows
+// (test/simplified/TestMnistPP.hs:735).  Seen through strides these are all ONE
+// pattern:  every kept dim advances only A (an "M" dim), only B (an "N" dim) or
+// both (a batch dim), and every reduced dim advances both (a "K" dim).  Then
+//     A[m, k] sits at  offAm(m) + offAk(k),   B[n, k] at  offBn(n) + offBk(k),
+//     C[m, n] at  offCm(m) + offCn(n),
+// with m, n, k multi-indices -- a matrix product whose operands are addressed
+// through separable offset maps.  No operand is copied or re-laid-out: the
+// im2col "patch matrix" of a convolution exists only as such a map.
+//
+// Kernel: 256 threads = 4 wavefronts in a 2x2 grid, block tile 128x128,
+// K-step 16; each wavefront owns a 64x64 sub-tile = 4x4 MFMA tiles of 16x16
+// (v_mfma_f64_16x16x4_f64 / v_mfma_f32_16x16x4_f32, accumulators in registers).
+// Operand tiles are staged through LDS in [k][m] order (one element of padding
+// per row keeps both the transposing stores and the MFMA-fragment loads free
+// of bank conflicts); the global loads of tile t+1 are issued before the MFMAs
+// of tile t.  Lanes run along whichever of m or k is contiguous in memory, so
+// loads coalesce for both plain and transposed operands.  Tiles are numbered
+// so that each XCD (blockIdx mod 8) works on a contiguous run of tiles and its
+// L2 sees neighbouring rows of A.  Small outputs with long K are split along K
+// into partial products summed by a second launch (fixed order: reproducible).
 #include "common.hpp"
+
+using namespace hg;
+
+namespace {
+
+constexpr int BM = 128, BN = 128, BK = 16, NT = 256;
+constexpr int GD = 5;  // dims per index group after merging
+
+struct Group {
+  int nd;
+  int64_t shape[GD];
+  int64_t sa[GD], sb[GD], sc[GD];
+};
+
+struct GemmParams {
+  Group m, n, k, bt;
+  int64_t M, N, K, BT;
+  int split;          // K chunks
+  int64_t kchunk;     // K elements per chunk (multiple of BK)
+  int64_t c_split_stride;  // elements between partial outputs
+};
+
+__device__ __forceinline__ void group_off(const Group& g, int64_t lin, int64_t* oa, int64_t* ob, int64_t* oc) {
+  int64_t a = 0, b = 0, c = 0;
+  int64_t r = lin;
+  for (int i = g.nd - 1; i >= 0; --i) {
+    int64_t idx;
+    if (i > 0) {
+      int64_t q = r / g.shape[i];
+      idx = r - q * g.shape[i];
+      r = q;
+    } else {
+      idx = r;
+    }
+    a += idx * g.sa[i];
+    b += idx * g.sb[i];
+    c += idx * g.sc[i];
+  }
+  *oa = a;
+  *ob = b;
+  *oc = c;
+}
+
+__global__ void k_koff(Group k, int64_t K, int64_t* __restrict__ ka, int64_t* __restrict__ kb) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < K) {
+    int64_t a, b, c;
+    group_off(k, i, &a, &b, &c);
+    ka[i] = a;
+    kb[i] = b;
+  }
+}
+
+template <typename T> struct Mfma;
+template <> struct Mfma<double> {
+  using V4 = __attribute__((ext_vector_type(4))) double;
+  static __device__ __forceinline__ V4 run(double a, double b, V4 c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+};
+template <> struct Mfma<float> {
+  using V4 = __attribute__((ext_vector_type(4))) float;
+  static __device__ __forceinline__ V4 run(float a, float b, V4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+};
+
+// A_KC / B_KC: the operand's innermost K dim has unit stride (lanes run along k);
+// otherwise lanes run along m (resp. n).
+template <typename T, bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                             const int64_t* __restrict__ koffA, const int64_t* __restrict__ koffB) {
+  using V4 = typename Mfma<T>::V4;
+  __shared__ T As[BK][BM + 1];
+  __shared__ T Bs[BK][BN + 1];
+
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // XCD-aware tile numbering: blocks b, b+8, b+16, ... share an XCD; give each
+  // XCD a contiguous range of tiles.
+  const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int64_t ntiles = tiles_m * tiles_n;
+  int64_t bid = blockIdx.x;
+  {
+    const int64_t per = (ntiles + 7) / 8;
+    int64_t xcd = bid & 7, local = bid >> 3;
+    int64_t tile = xcd * per + local;
+    // the last XCDs may own fewer tiles: fall back to the identity for them
+    bid = (ntiles >= 64 && (ntiles & 7) == 0) ? tile : bid;
+  }
+  const int64_t tile_m = bid / tiles_n, tile_n = bid - tile_m * tiles_n;
+  const int64_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+  int64_t bta, btb, btc;
+  group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
+  const int s = blockIdx.y;
+  const int64_t kbeg = (int64_t)s * p.kchunk;
+  int64_t kend = kbeg + p.kchunk;
+  if (kend > p.K) kend = p.K;
+
+  // this thread's 8 (row, k) slots of each operand tile
+  int aml[8], akl[8], bnl[8], bkl[8];
+  int64_t aoff[8], boff[8];
+  bool aok[8], bok[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if (A_KC) { aml[i] = (t >> 4) + 16 * i; akl[i] = t & 15; }
+    else { aml[i] = t & 127; akl[i] = (t >> 7) + 2 * i; }
+    if (B_KC) { bnl[i] = (t >> 4) + 16 * i; bkl[i] = t & 15; }
+    else { bnl[i] = t & 127; bkl[i] = (t >> 7) + 2 * i; }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    int64_t m = m0 + aml[i], n = n0 + bnl[i];
+    aok[i] = m < p.M;
+    bok[i] = n < p.N;
+    int64_t oa = 0, ob = 0, oc = 0;
+    if (A_KC || i == 0) {
+      if (aok[i]) group_off(p.m, m, &oa, &ob, &oc);
+      aoff[i] = oa + bta;
+    } else {
+      aoff[i] = aoff[0];
+    }
+    oa = ob = oc = 0;
+    if (B_KC || i == 0) {
+      if (bok[i]) group_off(p.n, n, &oa, &ob, &oc);
+      boff[i] = ob + btb;
+    } else {
+      boff[i] = boff[0];
+    }
+  }
+
+  V4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = V4{0, 0, 0, 0};
+
+  T ra[8], rb[8];
+  auto load_tile = [&](int64_t k0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int64_t ka = k0 + akl[i], kb = k0 + bkl[i];
+      ra[i] = (aok[i] && ka < kend) ? A[aoff[i] + koffA[ka]] : T(0);
+      rb[i] = (bok[i] && kb < kend) ? B[boff[i] + koffB[kb]] : T(0);
+    }
+  };
+
+  if (kbeg < kend) load_tile(kbeg);
+  for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      As[akl[i]][aml[i]] = ra[i];
+      Bs[bkl[i]][bnl[i]] = rb[i];
+    }
+    __syncthreads();
+    if (k0 + BK < kend) load_tile(k0 + BK);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 4) {
+      const int kr = kk + (lane >> 4);
+      T fa[4], fb[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        fa[i] = As[kr][wm * 64 + i * 16 + (lane & 15)];
+        fb[i] = Bs[kr][wn * 64 + i * 16 + (lane & 15)];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+
+  // D[row = 4 * (lane / 16) + r][col = lane % 16] of each 16x16 tile
+  T* Cout = C + btc + (int64_t)s * p.c_split_stride;
+  int64_t coln[4];
+  bool colok[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int64_t n = n0 + wn * 64 + j * 16 + (lane & 15);
+    colok[j] = n < p.N;
+    int64_t oa = 0, ob = 0, oc = 0;
+    if (colok[j]) group_off(p.n, n, &oa, &ob, &oc);
+    coln[j] = oc;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      int64_t m = m0 + wm * 64 + i * 16 + 4 * (lane >> 4) + r;
+      if (m < p.M) {
+        int64_t oa, ob, oc;
+        group_off(p.m, m, &oa, &ob, &oc);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (colok[j]) Cout[oc + coln[j]] = acc[i][j][r];
+      }
+    }
+  }
+}
+
+// Sums the split-K partials: out[i] = sum_s part[s * stride + i] for every element of the dense output.
+template <typename T>
+__global__ void __launch_bounds__(256) k_sum_partials(int64_t n, int S, int64_t stride, const T* __restrict__ part, T* __restrict__ out) {
+  int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
+    T acc = part[i];
+    for (int s = 1; s < S; ++s) acc += part[(int64_t)s * stride + i];
+    out[i] = acc;
+  }
+}
+
+// Appends dim (extent e, strides a, b, c) to a group, merging with the previous dim when all strides allow.
+bool push_dim(Group& g, int64_t e, int64_t a, int64_t b, int64_t c) {
+  if (e == 1) return true;
+  if (g.nd > 0) {
+    int p = g.nd - 1;
+    if (g.sa[p] == a * e && g.sb[p] == b * e && g.sc[p] == c * e) {
+      g.shape[p] *= e;
+      g.sa[p] = a;
+      g.sb[p] = b;
+      g.sc[p] = c;
+      return true;
+    }
+  }
+  if (g.nd == GD) return false;
+  g.shape[g.nd] = e;
+  g.sa[g.nd] = a;
+  g.sb[g.nd] = b;
+  g.sc[g.nd] = c;
+  g.nd++;
+  return true;
+}
+
+void finish(Group& g) {
+  if (g.nd == 0) {
+    g.nd = 1;
+    g.shape[0] = 1;
+    g.sa[0] = g.sb[0] = g.sc[0] = 0;
+  }
+  for (int i = g.nd; i < GD; ++i) {
+    g.shape[i] = 1;
+    g.sa[i] = g.sb[i] = g.sc[i] = 0;
+  }
+}
+
+int64_t total(const Group& g) {
+  int64_t n = 1;
+  for (int i = 0; i < g.nd; ++i) n *= g.shape[i];
+  return n;
+}
+
+template <typename T>
+void launch(hgpu_ctx* ctx, const GemmParams& p, bool akc, bool bkc, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
+  if (akc && bkc) hipLaunchKernelGGL((k_gemm<T, true, true>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+  else if (akc) hipLaunchKernelGGL((k_gemm<T, true, false>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+  else if (bkc) hipLaunchKernelGGL((k_gemm<T, false, true>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+  else hipLaunchKernelGGL((k_gemm<T, false, false>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+}
+
+}  // namespace
 
 namespace hg {
 
 int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled) {
-  (void)ctx; (void)a; (void)b; (void)n_keep; (void)out;
   *handled = false;
+  if (!b) return HGPU_OK;
+  if (a->dtype != HGPU_F64 && a->dtype != HGPU_F32) return HGPU_OK;
+  GemmParams p;
+  p.m.nd = p.n.nd = p.k.nd = p.bt.nd = 0;
+  // classify the kept dims (output strides are the dense ones of `out`)
+  for (int i = 0; i < n_keep; ++i) {
+    int64_t e = a->shape[i], sa = a->strides[i], sb = b->strides[i], sc = out->strides[i];
+    if (e == 1) continue;
+    bool ok;
+    if (sa != 0 && sb == 0) ok = push_dim(p.m, e, sa, 0, sc);
+    else if (sa == 0 && sb != 0) ok = push_dim(p.n, e, 0, sb, sc);
+    else if (sa != 0 && sb != 0) ok = push_dim(p.bt, e, sa, sb, sc);
+    else return HGPU_OK;  // an output dim neither operand depends on
+    if (!ok) return HGPU_OK;
+  }
+  for (int i = n_keep; i < a->rank; ++i) {
+    int64_t e = a->shape[i], sa = a->strides[i], sb = b->strides[i];
+    if (e == 1) continue;
+    if (sa == 0 || sb == 0) return HGPU_OK;  // a plain sum hidden in the contraction
+    if (!push_dim(p.k, e, sa, sb, 0)) return HGPU_OK;
+  }
+  finish(p.m);
+  finish(p.n);
+  finish(p.k);
+  finish(p.bt);
+  p.M = total(p.m);
+  p.N = total(p.n);
+  p.K = total(p.k);
+  p.BT = total(p.bt);
+  // Worth the matrix cores only when there is reuse on both sides.
+  if (p.K < 4 || p.M * p.N < 256) return HGPU_OK;
+  if (p.BT > 65535) return HGPU_OK;
+  if ((double)p.M * p.N * p.K * p.BT < 2.0e6) return HGPU_OK;
+
+  int64_t tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  if (tiles > 0x7fffffff) return HGPU_OK;
+  // split K when the tiles alone cannot fill the device
+  int split = 1;
+  int64_t want = (int64_t)ctx->num_cu * 2;
+  if (tiles * p.BT < want && p.K >= 8 * BK) {
+    split = (int)((want + tiles * p.BT - 1) / (tiles * p.BT));
+    int64_t max_split = p.K / (4 * BK);
+    if (split > max_split) split = (int)max_split;
+    if (split > 64) split = 64;
+    if (split < 1) split = 1;
+  }
+  p.split = split;
+  p.kchunk = ((p.K + split - 1) / split + BK - 1) / BK * BK;
+  p.split = (int)((p.K + p.kchunk - 1) / p.kchunk);
+  split = p.split;
+
+  size_t es = dtype_size(a->dtype);
+  int64_t out_n = nelem(out);
+  hgpu_buffer* koff = nullptr;
+  int rc = buffer_alloc(ctx, (size_t)p.K * 16, &koff);
+  if (rc) return rc;
+  hgpu_buffer* part = nullptr;
+  if (split > 1) {
+    rc = buffer_alloc(ctx, (size_t)out_n * split * es, &part);
+    if (rc) { buffer_release(koff); return rc; }
+  }
+  p.c_split_stride = split > 1 ? out_n : 0;
+  int64_t* ka = (int64_t*)koff->ptr;
+  int64_t* kb = ka + p.K;
+  bool akc = p.k.sa[p.k.nd - 1] == 1;
+  bool bkc = p.k.sb[p.k.nd - 1] == 1;
+  dim3 grid((unsigned)tiles, (unsigned)split, (unsigned)p.BT);
+  {
+    double flops = 2.0 * p.M * p.N * p.K * p.BT;
+    double bytes = ((double)p.M * p.K + (double)p.N * p.K + (double)p.M * p.N) * p.BT * es;
+    LaunchGuard lg(ctx, a->dtype == HGPU_F64 ? "gemm_f64" : "gemm_f32", bytes, flops);
+    hipLaunchKernelGGL(k_koff, dim3((unsigned)((p.K + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, ka, kb);
+    if (a->dtype == HGPU_F64) {
+      double* cdst = split > 1 ? (double*)part->ptr : (double*)data_ptr(out);
+      launch<double>(ctx, p, akc, bkc, grid, (const double*)data_ptr(a), (const double*)data_ptr(b), cdst, ka, kb);
+      if (split > 1)
+        hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 256, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
+    } else {
+      float* cdst = split > 1 ? (float*)part->ptr : (float*)data_ptr(out);
+      launch<float>(ctx, p, akc, bkc, grid, (const float*)data_ptr(a), (const float*)data_ptr(b), cdst, ka, kb);
+      if (split > 1)
+        hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 256, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
+    }
+  }
+  hipError_t e = hipGetLastError();
+  buffer_release(koff);
+  if (part) buffer_release(part);
+  if (e != hipSuccess) return check_hip(ctx, e, "gemm");
+  *handled = true;
   return HGPU_OK;
 }
 

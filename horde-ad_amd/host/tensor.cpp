@@ -140,7 +140,8 @@ T reverse(const T& a, int dim) {
 }
 T replicate(const T& a, const Shape& pre) {
   if (pre.empty()) return a;
-  HD_VIEW_OF_PRODUCT(replicate(a0, pre), replicate(b0, pre))
+  // a pending product is written out before it is replicated: only shrinking
+  // or permuting views of it are worth keeping pending
   HD_OUT(replicate(be__->ctx, a.h(), (int)pre.size(), pre.data(), &o__));
 }
 T index_prefix(const T& a, const Shape& ix) {

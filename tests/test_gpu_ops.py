@@ -349,3 +349,53 @@ def test_errors_and_allocator(gpu):
     assert e.value.code == 2
     gpu.check(gpu.lib.inject_alloc_failure(gpu.h, -1))
     assert np.allclose(a.ewise1("cos").numpy(), np.cos(a.numpy()))
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_contract_on_the_matrix_cores(both, gpu, dt):
+    """Contractions whose strides make them matrix products run on the MFMA
+    kernel; operands stay views (replicated, transposed, windowed)."""
+    tol = TOL[np.dtype(dt)]
+
+    def matmul_views(m1, m2):
+        m, n = m1.shape
+        p = m2.shape[1]
+        return m1.replicate([p]).transpose([1, 0]), m2.replicate([m]).transpose([0, 2, 1])
+
+    for (m, n, p) in [(130, 70, 129), (257, 33, 64), (16, 300, 16), (1, 520, 700), (300, 4, 300), (128, 128, 128), (10, 128, 2500)]:
+        a, b = both.upload(rnd((m, n), dt)), both.upload(rnd((n, p), dt))
+        lhs, rhs = matmul_views(a, b)
+        assert_same(lhs.contract(rhs, 2), tol, ("matmul", m, n, p))
+        # transposed operands: A^T stored, B^T stored
+        at, bt = both.upload(rnd((n, m), dt)).transpose([1, 0]), both.upload(rnd((p, n), dt)).transpose([1, 0])
+        lhs, rhs = matmul_views(at, bt)
+        assert_same(lhs.contract(rhs, 2), tol, ("matmul^T", m, n, p))
+    # long K with a small output: split along K
+    a, b = both.upload(rnd((24, 40000), dt)), both.upload(rnd((40000, 20), dt))
+    lhs, rhs = matmul_views(a, b)
+    assert_same(lhs.contract(rhs, 2), 10 * tol, "split-K")
+    # a batch dim on both operands
+    x, y = both.upload(rnd((5, 40, 30), dt)), both.upload(rnd((5, 30, 50), dt))
+    lhs = x.replicate([50]).transpose([1, 2, 0])            # [5, 40, 50, 30]
+    rhs = y.replicate([40]).transpose([1, 0, 3, 2])          # [5, 40, 50, 30]
+    assert_same(lhs.contract(rhs, 3), tol, "batched")
+    # convolution as a contraction over a window view: out[b, co, h, w]
+    img, ker = both.upload(rnd((3, 4, 12, 10), dt)), both.upload(rnd((6, 4, 3, 3), dt))
+    padded = img.pad([0, 0, 0, 0], [0, 0, 2, 2])
+    st = padded.strides
+    win = padded.as_strided([3, 12, 10, 4, 3, 3], [st[0], st[2], st[3], st[1], st[2], st[3]], 0)
+    lhs = win.replicate([6]).transpose([1, 0, 2, 3])          # [b, co, h, w, ci, kh, kw]
+    rhs = ker.replicate([3, 12, 10]).transpose([0, 3, 1, 2])  # [b, co, h, w, ci, kh, kw]
+    assert_same(lhs.contract(rhs, 4), tol, "conv")
+    # the kernel-gradient contraction: K = (b, h, w) on both operands
+    dout = both.upload(rnd((3, 6, 12, 10), dt))
+    lhs = win.replicate([6]).transpose([0, 4, 5, 6, 1, 2, 3])             # [co, ci, kh, kw, b, h, w]
+    rhs = dout.replicate([4, 3, 3]).transpose([4, 0, 1, 2, 3, 5, 6])      # [co, ci, kh, kw, b, h, w]
+    assert_same(lhs.contract(rhs, 4), tol, "conv dK")
+    rep = None
+    gpu.profile(True)
+    a, b = gpu.upload(rnd((256, 64), dt)), gpu.upload(rnd((64, 256), dt))
+    a.replicate([256]).transpose([1, 0]).contract(b.replicate([256]).transpose([0, 2, 1]), 2)
+    rep = gpu.profile_report()
+    gpu.profile(False)
+    assert any(k.startswith("gemm") for k in rep), rep
