@@ -81,10 +81,14 @@ template <typename T> struct Mfma;
 template <> struct Mfma<double> {
   using V4 = __attribute__((ext_vector_type(4))) double;
   static __device__ __forceinline__ V4 run(double a, double b, V4 c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+  // accumulator register r of a lane holds D[4 r + lane / 16][lane % 16]
+  static __device__ __forceinline__ int row(int lane, int r) { return 4 * r + (lane >> 4); }
 };
 template <> struct Mfma<float> {
   using V4 = __attribute__((ext_vector_type(4))) float;
   static __device__ __forceinline__ V4 run(float a, float b, V4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  // accumulator register r of a lane holds D[4 (lane / 16) + r][lane % 16]
+  static __device__ __forceinline__ int row(int lane, int r) { return 4 * (lane >> 4) + r; }
 };
 
 // A_KC / B_KC: the operand's innermost K dim has unit stride (lanes run along k);
@@ -196,7 +200,7 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__
     __syncthreads();
   }
 
-  // D[row = 4 * (lane / 16) + r][col = lane % 16] of each 16x16 tile
+  // each lane holds 4 rows of one column of every 16x16 tile (Mfma<T>::row)
   T* Cout = C + btc + (int64_t)s * p.c_split_stride;
   int64_t coln[4];
   bool colok[4];
@@ -212,7 +216,7 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__
   for (int i = 0; i < 4; ++i) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      int64_t m = m0 + wm * 64 + i * 16 + 4 * (lane >> 4) + r;
+      int64_t m = m0 + wm * 64 + i * 16 + Mfma<T>::row(lane, r);
       if (m < p.M) {
         int64_t oa, ob, oc;
         group_off(p.m, m, &oa, &ob, &oc);

@@ -382,7 +382,7 @@ def test_contract_on_the_matrix_cores(both, gpu, dt):
     # convolution as a contraction over a window view: out[b, co, h, w]
     img, ker = both.upload(rnd((3, 4, 12, 10), dt)), both.upload(rnd((6, 4, 3, 3), dt))
     padded = img.pad([0, 0, 0, 0], [0, 0, 2, 2])
-    st = padded.strides
+    st = padded.arrays[0].strides    # dense on both providers
     win = padded.as_strided([3, 12, 10, 4, 3, 3], [st[0], st[2], st[3], st[1], st[2], st[3]], 0)
     lhs = win.replicate([6]).transpose([1, 0, 2, 3])          # [b, co, h, w, ci, kh, kw]
     rhs = ker.replicate([3, 12, 10]).transpose([0, 3, 1, 2])  # [b, co, h, w, ci, kh, kw]
