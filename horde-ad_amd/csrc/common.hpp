@@ -10,6 +10,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -54,6 +55,8 @@ struct hgpu_ctx {
   // Optional per-launch timing (hgpu_profile_enable): one event pair per launch.
   struct ProfRec { const char* name; hipEvent_t a, b; double bytes, flops; };
   bool profiling = false;
+  bool profile_shapes = false;           // hgpu_profile_enable(ctx, 2): labels carry the problem shape
+  std::set<std::string> label_pool;
   std::vector<ProfRec> prof;
 };
 

@@ -251,9 +251,18 @@ int copy_view(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const vo
   int64_t n = 1;
   for (int i = 0; i < rank; ++i) n *= shape[i];
   if (n == 0) return HGPU_OK;
-  const int64_t* sts[2] = {sst, dst_st};
+  // A copy may visit the elements in any order: walk the dims in the
+  // destination's memory order (largest stride first) so that stores coalesce.
+  int order[HGPU_MAX_RANK];
+  for (int i = 0; i < rank; ++i) order[i] = i;
+  auto mag = [&](int dim) { return dst_st[dim] < 0 ? -dst_st[dim] : dst_st[dim]; };
+  for (int i = 1; i < rank; ++i)
+    for (int j = i; j > 0 && mag(order[j]) > mag(order[j - 1]); --j) { int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t; }
+  int64_t psh[HGPU_MAX_RANK], pss[HGPU_MAX_RANK], pds[HGPU_MAX_RANK];
+  for (int i = 0; i < rank; ++i) { psh[i] = shape[order[i]]; pss[i] = sst[order[i]]; pds[i] = dst_st[order[i]]; }
+  const int64_t* sts[2] = {pss, pds};
   Dims d;
-  if (!collapse(rank, shape, 2, sts, &d)) return fail(ctx, HGPU_ERR_UNSUPPORTED, "copy: more than %d merged dims", HG_KDIMS);
+  if (!collapse(rank, psh, 2, sts, &d)) return fail(ctx, HGPU_ERR_UNSUPPORTED, "copy: more than %d merged dims", HG_KDIMS);
   LaunchGuard lg(ctx, "copy_view", 2.0 * n * dtype_size(dtype), 0);
   unsigned g = grid_for(n, kBlock, max_blocks(ctx));
   switch (dtype_size(dtype)) {
@@ -288,9 +297,26 @@ int hgpu_pad(hgpu_ctx* ctx, const hgpu_array* a, const int64_t* lo, const int64_
     if (lo[i] < 0 || hi[i] < 0) return fail(ctx, HGPU_ERR_INVALID, "pad: negative padding");
     sh[i] = a->shape[i] + lo[i] + hi[i];
   }
-  hgpu_array* o = nullptr;
-  int rc = new_zeros(ctx, a->dtype, a->rank, sh, &o);
+  // The result keeps the operand's order of dims IN MEMORY (a transposed view is
+  // padded into a transposed array): the copy is coalesced on both sides and
+  // whatever was contiguous stays contiguous for the consumer.
+  int order[HGPU_MAX_RANK];
+  for (int i = 0; i < a->rank; ++i) order[i] = i;
+  auto key = [&](int d) -> int64_t {
+    int64_t s = a->strides[d] < 0 ? -a->strides[d] : a->strides[d];
+    return (s == 0 || a->shape[d] == 1) ? INT64_MAX : s;   // replicated dims go outermost
+  };
+  for (int i = 1; i < a->rank; ++i)   // stable insertion sort, largest stride first
+    for (int j = i; j > 0 && key(order[j]) > key(order[j - 1]); --j) { int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t; }
+  int64_t psh[HGPU_MAX_RANK];
+  for (int i = 0; i < a->rank; ++i) psh[i] = sh[order[i]];
+  hgpu_array* phys = nullptr;
+  int rc = new_zeros(ctx, a->dtype, a->rank, psh, &phys);
   if (rc) return rc;
+  int64_t st[HGPU_MAX_RANK];
+  for (int i = 0; i < a->rank; ++i) st[order[i]] = phys->strides[i];
+  hgpu_array* o = new_view(ctx, phys->buf, a->dtype, a->rank, sh, st, 0);
+  hgpu_release(phys);
   int64_t off = 0;
   for (int i = 0; i < a->rank; ++i) off += lo[i] * o->strides[i];
   if (nelem(a) > 0)

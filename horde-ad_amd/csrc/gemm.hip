@@ -12,9 +12,11 @@
 // through separable offset maps.  No operand is copied or re-laid-out: the
 // im2col "patch matrix" of a convolution exists only as such a map.
 //
-// Kernel: 256 threads = 4 wavefronts in a 2x2 grid, block tile 128x128,
-// K-step 16; each wavefront owns a 64x64 sub-tile = 4x4 MFMA tiles of 16x16
-// (v_mfma_f64_16x16x4_f64 / v_mfma_f32_16x16x4_f32, accumulators in registers).
+// Kernel: 256 threads = 4 wavefronts, K-step 16; the block tile ranges from
+// 128x128 (wavefronts 2x2, each 4x4 MFMA tiles of 16x16) down to 256x16 / 16x256
+// and 32x32 for skinny or tiny outputs (a convolution with 16 output channels
+// has N = 16).  v_mfma_f64_16x16x4_f64 / v_mfma_f32_16x16x4_f32, accumulators
+// in registers.
 // Operand tiles are staged through LDS in [k][m] order (one element of padding
 // per row keeps both the transposing stores and the MFMA-fragment loads free
 // of bank conflicts); the global loads of tile t+1 are issued before the MFMAs
@@ -29,7 +31,7 @@ using namespace hg;
 
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 16, NT = 256;
+constexpr int BK = 16, NT = 256;
 constexpr int GD = 5;  // dims per index group after merging
 
 struct Group {
@@ -91,31 +93,30 @@ template <> struct Mfma<float> {
   static __device__ __forceinline__ int row(int lane, int r) { return 4 * (lane >> 4) + r; }
 };
 
-// A_KC / B_KC: the operand's innermost K dim has unit stride (lanes run along k);
-// otherwise lanes run along m (resp. n).
-template <typename T, bool A_KC, bool B_KC>
+// Block tile BM x BN = (WGM * TM * 16) x (WGN * TN * 16): the 4 wavefronts form a
+// WGM x WGN grid and each owns TM x TN MFMA tiles.  A_KC / B_KC: the operand's
+// innermost K dim has unit stride (lanes run along k); otherwise lanes run
+// along m (resp. n).
+template <typename T, int WGM, int WGN, int TM, int TN, bool A_KC, bool B_KC>
 __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                              const int64_t* __restrict__ koffA, const int64_t* __restrict__ koffB) {
   using V4 = typename Mfma<T>::V4;
+  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
+  constexpr int NA = BM * BK / NT, NB = BN * BK / NT;   // operand elements each thread stages per K-step
+  static_assert(WGM * WGN == 4 && NA >= 1 && NB >= 1, "tile shape");
   __shared__ T As[BK][BM + 1];
   __shared__ T Bs[BK][BN + 1];
 
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
 
   // XCD-aware tile numbering: blocks b, b+8, b+16, ... share an XCD; give each
   // XCD a contiguous range of tiles.
   const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int64_t ntiles = tiles_m * tiles_n;
   int64_t bid = blockIdx.x;
-  {
-    const int64_t per = (ntiles + 7) / 8;
-    int64_t xcd = bid & 7, local = bid >> 3;
-    int64_t tile = xcd * per + local;
-    // the last XCDs may own fewer tiles: fall back to the identity for them
-    bid = (ntiles >= 64 && (ntiles & 7) == 0) ? tile : bid;
-  }
+  if (ntiles >= 64 && (ntiles & 7) == 0) bid = (bid & 7) * (ntiles >> 3) + (bid >> 3);
   const int64_t tile_m = bid / tiles_n, tile_n = bid - tile_m * tiles_n;
   const int64_t m0 = tile_m * BM, n0 = tile_n * BN;
 
@@ -126,31 +127,32 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__
   int64_t kend = kbeg + p.kchunk;
   if (kend > p.K) kend = p.K;
 
-  // this thread's 8 (row, k) slots of each operand tile
-  int aml[8], akl[8], bnl[8], bkl[8];
-  int64_t aoff[8], boff[8];
-  bool aok[8], bok[8];
+  // this thread's (row, k) slots of each operand tile
+  int aml[NA], akl[NA], bnl[NB], bkl[NB];
+  int64_t aoff[NA], boff[NB];
+  bool aok[NA], bok[NB];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < NA; ++i) {
     if (A_KC) { aml[i] = (t >> 4) + 16 * i; akl[i] = t & 15; }
-    else { aml[i] = t & 127; akl[i] = (t >> 7) + 2 * i; }
-    if (B_KC) { bnl[i] = (t >> 4) + 16 * i; bkl[i] = t & 15; }
-    else { bnl[i] = t & 127; bkl[i] = (t >> 7) + 2 * i; }
-  }
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    int64_t m = m0 + aml[i], n = n0 + bnl[i];
+    else { aml[i] = t % BM; akl[i] = t / BM + (NT / BM) * i; }
+    int64_t m = m0 + aml[i];
     aok[i] = m < p.M;
-    bok[i] = n < p.N;
-    int64_t oa = 0, ob = 0, oc = 0;
     if (A_KC || i == 0) {
+      int64_t oa = 0, ob = 0, oc = 0;
       if (aok[i]) group_off(p.m, m, &oa, &ob, &oc);
       aoff[i] = oa + bta;
     } else {
       aoff[i] = aoff[0];
     }
-    oa = ob = oc = 0;
+  }
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    if (B_KC) { bnl[i] = (t >> 4) + 16 * i; bkl[i] = t & 15; }
+    else { bnl[i] = t % BN; bkl[i] = t / BN + (NT / BN) * i; }
+    int64_t n = n0 + bnl[i];
+    bok[i] = n < p.N;
     if (B_KC || i == 0) {
+      int64_t oa = 0, ob = 0, oc = 0;
       if (bok[i]) group_off(p.n, n, &oa, &ob, &oc);
       boff[i] = ob + btb;
     } else {
@@ -158,18 +160,22 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__
     }
   }
 
-  V4 acc[4][4];
+  V4 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = V4{0, 0, 0, 0};
+    for (int j = 0; j < TN; ++j) acc[i][j] = V4{0, 0, 0, 0};
 
-  T ra[8], rb[8];
+  T ra[NA], rb[NB];
   auto load_tile = [&](int64_t k0) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      int64_t ka = k0 + akl[i], kb = k0 + bkl[i];
+    for (int i = 0; i < NA; ++i) {
+      int64_t ka = k0 + akl[i];
       ra[i] = (aok[i] && ka < kend) ? A[aoff[i] + koffA[ka]] : T(0);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      int64_t kb = k0 + bkl[i];
       rb[i] = (bok[i] && kb < kend) ? B[boff[i] + koffB[kb]] : T(0);
     }
   };
@@ -177,51 +183,49 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__
   if (kbeg < kend) load_tile(kbeg);
   for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      As[akl[i]][aml[i]] = ra[i];
-      Bs[bkl[i]][bnl[i]] = rb[i];
-    }
+    for (int i = 0; i < NA; ++i) As[akl[i]][aml[i]] = ra[i];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) Bs[bkl[i]][bnl[i]] = rb[i];
     __syncthreads();
     if (k0 + BK < kend) load_tile(k0 + BK);
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 4) {
       const int kr = kk + (lane >> 4);
-      T fa[4], fb[4];
+      T fa[TM], fb[TN];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        fa[i] = As[kr][wm * 64 + i * 16 + (lane & 15)];
-        fb[i] = Bs[kr][wn * 64 + i * 16 + (lane & 15)];
-      }
+      for (int i = 0; i < TM; ++i) fa[i] = As[kr][(wm * TM + i) * 16 + (lane & 15)];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int j = 0; j < TN; ++j) fb[j] = Bs[kr][(wn * TN + j) * 16 + (lane & 15)];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
     }
     __syncthreads();
   }
 
   // each lane holds 4 rows of one column of every 16x16 tile (Mfma<T>::row)
   T* Cout = C + btc + (int64_t)s * p.c_split_stride;
-  int64_t coln[4];
-  bool colok[4];
+  int64_t coln[TN];
+  bool colok[TN];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    int64_t n = n0 + wn * 64 + j * 16 + (lane & 15);
+  for (int j = 0; j < TN; ++j) {
+    int64_t n = n0 + (wn * TN + j) * 16 + (lane & 15);
     colok[j] = n < p.N;
     int64_t oa = 0, ob = 0, oc = 0;
     if (colok[j]) group_off(p.n, n, &oa, &ob, &oc);
     coln[j] = oc;
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < TM; ++i) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      int64_t m = m0 + wm * 64 + i * 16 + Mfma<T>::row(lane, r);
+      int64_t m = m0 + (wm * TM + i) * 16 + Mfma<T>::row(lane, r);
       if (m < p.M) {
         int64_t oa, ob, oc;
         group_off(p.m, m, &oa, &ob, &oc);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
           if (colok[j]) Cout[oc + coln[j]] = acc[i][j][r];
       }
     }
@@ -279,12 +283,46 @@ int64_t total(const Group& g) {
   return n;
 }
 
+struct TileCfg { int wgm, wgn, tm, tn; double eff; };
+// Candidate tiles, with a rough relative efficiency (operand reuse from LDS).
+const TileCfg kTiles[] = {
+    {2, 2, 4, 4, 1.00},  // 128 x 128
+    {2, 2, 4, 2, 0.85},  // 128 x 64
+    {2, 2, 2, 4, 0.85},  // 64 x 128
+    {4, 1, 4, 2, 0.70},  // 256 x 32
+    {1, 4, 2, 4, 0.70},  // 32 x 256
+    {4, 1, 4, 1, 0.50},  // 256 x 16
+    {1, 4, 1, 4, 0.50},  // 16 x 256
+    {2, 2, 2, 2, 0.65},  // 64 x 64
+    {2, 2, 1, 1, 0.35},  // 32 x 32
+    {4, 1, 1, 1, 0.30},  // 64 x 16
+    {1, 4, 1, 1, 0.30},  // 16 x 64
+};
+constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
+
+template <typename T, int WGM, int WGN, int TM, int TN>
+void launch_cfg(hgpu_ctx* ctx, const GemmParams& p, bool akc, bool bkc, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
+  if (akc && bkc) hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, true, true>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+  else if (akc) hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, true, false>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+  else if (bkc) hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, false, true>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+  else hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, false, false>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+}
+
 template <typename T>
-void launch(hgpu_ctx* ctx, const GemmParams& p, bool akc, bool bkc, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
-  if (akc && bkc) hipLaunchKernelGGL((k_gemm<T, true, true>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
-  else if (akc) hipLaunchKernelGGL((k_gemm<T, true, false>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
-  else if (bkc) hipLaunchKernelGGL((k_gemm<T, false, true>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
-  else hipLaunchKernelGGL((k_gemm<T, false, false>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+void launch(hgpu_ctx* ctx, int cfg, const GemmParams& p, bool akc, bool bkc, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
+  switch (cfg) {
+    case 0: launch_cfg<T, 2, 2, 4, 4>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 1: launch_cfg<T, 2, 2, 4, 2>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 2: launch_cfg<T, 2, 2, 2, 4>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 3: launch_cfg<T, 4, 1, 4, 2>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 4: launch_cfg<T, 1, 4, 2, 4>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 5: launch_cfg<T, 4, 1, 4, 1>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 6: launch_cfg<T, 1, 4, 1, 4>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 7: launch_cfg<T, 2, 2, 2, 2>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 8: launch_cfg<T, 2, 2, 1, 1>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 9: launch_cfg<T, 4, 1, 1, 1>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    default: launch_cfg<T, 1, 4, 1, 1>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+  }
 }
 
 }  // namespace
@@ -327,16 +365,39 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   if (p.BT > 65535) return HGPU_OK;
   if ((double)p.M * p.N * p.K * p.BT < 2.0e6) return HGPU_OK;
 
+  // tile shape: least padded work per unit of efficiency
+  int cfg = 0;
+  double best = 1e300;
+  for (int c = 0; c < kNumTiles; ++c) {
+    int64_t bm = kTiles[c].wgm * kTiles[c].tm * 16, bn = kTiles[c].wgn * kTiles[c].tn * 16;
+    double padded = (double)((p.M + bm - 1) / bm * bm) * (double)((p.N + bn - 1) / bn * bn);
+    double cost = padded / kTiles[c].eff;
+    // a tile shape that cannot occupy the device even with K split pays for the idle CUs
+    double blocks = (double)((p.M + bm - 1) / bm) * (double)((p.N + bn - 1) / bn) * (double)p.BT;
+    double can_split = (double)(p.K / (4 * BK));
+    double cap0 = (double)(p.M + p.N) * p.K / (2.0 * p.M * p.N);
+    if (can_split > cap0) can_split = cap0;
+    if (can_split > 512) can_split = 512;
+    if (can_split < 1) can_split = 1;
+    if (blocks * can_split < ctx->num_cu) cost *= ctx->num_cu / (blocks * can_split);
+    if (cost < best * 0.999) { best = cost; cfg = c; }
+  }
+  const int64_t BM = kTiles[cfg].wgm * kTiles[cfg].tm * 16, BN = kTiles[cfg].wgn * kTiles[cfg].tn * 16;
   int64_t tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   if (tiles > 0x7fffffff) return HGPU_OK;
   // split K when the tiles alone cannot fill the device
   int split = 1;
   int64_t want = (int64_t)ctx->num_cu * 2;
+  int64_t out_elems = p.M * p.N * p.BT;
   if (tiles * p.BT < want && p.K >= 8 * BK) {
     split = (int)((want + tiles * p.BT - 1) / (tiles * p.BT));
     int64_t max_split = p.K / (4 * BK);
     if (split > max_split) split = (int)max_split;
-    if (split > 64) split = 64;
+    // the partial products must stay small next to the operands
+    int64_t cap = out_elems > 0 ? (int64_t)((double)(p.M + p.N) * p.K * p.BT / (2.0 * out_elems)) : 1;
+    if (cap > 512) cap = 512;
+    if (cap < 1) cap = 1;
+    if (split > cap) split = (int)cap;
     if (split < 1) split = 1;
   }
   p.split = split;
@@ -363,16 +424,22 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   {
     double flops = 2.0 * p.M * p.N * p.K * p.BT;
     double bytes = ((double)p.M * p.K + (double)p.N * p.K + (double)p.M * p.N) * p.BT * es;
-    LaunchGuard lg(ctx, a->dtype == HGPU_F64 ? "gemm_f64" : "gemm_f32", bytes, flops);
+    const char* label = a->dtype == HGPU_F64 ? "gemm_f64" : "gemm_f32";
+    if (ctx->profiling && ctx->profile_shapes) {
+      char buf[128];
+      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,%s%s,t%lldx%lld]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, split, akc ? "k" : "m", bkc ? "k" : "n", (long long)BM, (long long)BN);
+      label = ctx->label_pool.insert(buf).first->c_str();
+    }
+    LaunchGuard lg(ctx, label, bytes, flops);
     hipLaunchKernelGGL(k_koff, dim3((unsigned)((p.K + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, ka, kb);
     if (a->dtype == HGPU_F64) {
       double* cdst = split > 1 ? (double*)part->ptr : (double*)data_ptr(out);
-      launch<double>(ctx, p, akc, bkc, grid, (const double*)data_ptr(a), (const double*)data_ptr(b), cdst, ka, kb);
+      launch<double>(ctx, cfg, p, akc, bkc, grid, (const double*)data_ptr(a), (const double*)data_ptr(b), cdst, ka, kb);
       if (split > 1)
         hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 256, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
     } else {
       float* cdst = split > 1 ? (float*)part->ptr : (float*)data_ptr(out);
-      launch<float>(ctx, p, akc, bkc, grid, (const float*)data_ptr(a), (const float*)data_ptr(b), cdst, ka, kb);
+      launch<float>(ctx, cfg, p, akc, bkc, grid, (const float*)data_ptr(a), (const float*)data_ptr(b), cdst, ka, kb);
       if (split > 1)
         hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 256, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
     }

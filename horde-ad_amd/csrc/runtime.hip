@@ -315,6 +315,7 @@ int hgpu_profile_enable(hgpu_ctx* ctx, int on) {
   for (auto& r : ctx->prof) { (void)hipEventDestroy(r.a); (void)hipEventDestroy(r.b); }
   ctx->prof.clear();
   ctx->profiling = on != 0;
+  ctx->profile_shapes = on == 2;
   return HGPU_OK;
 }
 

@@ -117,7 +117,8 @@ int hgpu_inject_alloc_failure(hgpu_ctx* ctx, int64_t limit);
 /* Per-launch timing for benchmarks: while enabled every kernel launch is
  * bracketed by a HIP event pair on the context's stream.  The report has one
  * line per kernel family: "name launches total_ms algorithmic_bytes
- * algorithmic_flops".  Enabling (or disabling) clears the records. */
+ * algorithmic_flops".  Enabling (or disabling) clears the records.  on = 2
+ * makes the matrix-product labels carry the problem shape. */
 int hgpu_profile_enable(hgpu_ctx* ctx, int on);
 int hgpu_profile_report(hgpu_ctx* ctx, char* buf, size_t n);
 
@@ -180,7 +181,9 @@ int hgpu_as_strided(hgpu_ctx* ctx, const hgpu_array* a, int rank, const int64_t*
 int hgpu_materialize(hgpu_ctx* ctx, const hgpu_array* a, hgpu_array** out);
 /* Zero-extends every dimension d by lo[d] elements in front and hi[d] behind
  * (the zero rows a gather with out-of-bounds indices produces,
- * OpsConcrete.hs:1488-1490; also slice's VJP, DeltaEval.hs:569-575). */
+ * OpsConcrete.hs:1488-1490; also slice's VJP, DeltaEval.hs:569-575).  Unlike
+ * the other compute entry points the result is dense in the operand's own
+ * order of dims in memory (a transposed view pads into a transposed array). */
 int hgpu_pad(hgpu_ctx* ctx, const hgpu_array* a, const int64_t* lo, const int64_t* hi, hgpu_array** out);
 
 /* Elementwise Num/Fractional/Floating/IntegralH instances of arrays
