@@ -47,7 +47,12 @@ struct ArrHolder {
   // A pending elementwise product fa * fb (h == nullptr until it is needed as
   // an array).  Views of it stay pending, and summing it is a contraction of
   // the two factors, so `tssumN (u * v)` never writes the product to memory.
+  // With keep >= 0 the pending value is instead the CONTRACTION of fa and fb
+  // over all but their first `keep` dims (the sum of a pending product): a
+  // scatter with an affine index function folds into it (the transposed
+  // convolution never writes its patch gradient to memory).
   std::shared_ptr<ArrHolder> fa, fb;
+  int keep = -1;
   ArrHolder(Backend* b, hgpu_array* a) : be(b), h(a) {}
   ~ArrHolder() { if (h) be->api->release(h); }
   ArrHolder(const ArrHolder&) = delete;
@@ -68,7 +73,9 @@ class T {
     if (!p_->h) p_->force();
     return p_->h;
   }
-  bool pending_product() const { return p_ && !p_->h && p_->fa; }
+  bool pending_product() const { return p_ && !p_->h && p_->fa && p_->keep < 0; }
+  bool pending_contraction() const { return p_ && !p_->h && p_->fa && p_->keep >= 0; }
+  int pending_keep() const { return p_->keep; }
   T factor_a() const { return T(p_->fa); }
   T factor_b() const { return T(p_->fb); }
   // metadata never forces a pending product: the first factor has the same
@@ -77,9 +84,13 @@ class T {
     while (!q->h && q->fa) q = q->fa.get();
     return q->h;
   }
-  int rank() const { return be()->api->rank(meta_h()); }
+  int rank() const { return pending_contraction() ? p_->keep : be()->api->rank(meta_h()); }
   int dtype() const { return be()->api->dtype_of(meta_h()); }
-  int64_t size() const { return be()->api->size(meta_h()); }
+  int64_t size() const {
+    int64_t n = 1;
+    for (auto e : shape()) n *= e;
+    return n;
+  }
   Shape shape() const;
   Shape strides() const;
   const std::shared_ptr<std::vector<int64_t>>& host_i64() const { return p_->host_i64; }
@@ -106,6 +117,7 @@ T pad(const T& a, const Shape& lo, const Shape& hi);
 T ewise1(int op, const T& a);
 T ewise2(int op, const T& a, const T& b);
 T lazy_mul(const T& a, const T& b);                                // a * b, not yet written to memory
+T lazy_contract(const T& a, const T& b, int n_keep);               // sum of a * b over the trailing dims, pending
 T compare(int cmp, const T& a, const T& b);
 bool compare_all(int cmp, const T& a, const T& b);
 T select(const T& c, const T& a, const T& b);

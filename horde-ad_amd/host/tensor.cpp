@@ -14,6 +14,10 @@ void Backend::check(int rc) const {
 }
 
 Shape T::shape() const {
+  if (pending_contraction()) {   // the kept dims of the first factor
+    Shape f = T(p_->fa).shape();
+    return Shape(f.begin(), f.begin() + p_->keep);
+  }
   Shape s((size_t)rank());
   if (!s.empty()) be()->api->shape(meta_h(), s.data());
   return s;
@@ -104,13 +108,25 @@ T iota(Backend* be, int64_t n, int dtype) {
   be__->check(be__->api->call);           \
   return T(be__, o__)
 
+static T contract_now(const T& a, const T* b, int n_keep);
+
 void ArrHolder::force() {
   if (h || !fa) return;
-  T p = ewise2(HGPU_MUL, T(fa), T(fb));
+  T fbt(fb);
+  T p = keep >= 0 ? contract_now(T(fa), &fbt, keep) : ewise2(HGPU_MUL, T(fa), fbt);
   be->check(be->api->retain(p.h()));
   h = p.h();
   fa.reset();
   fb.reset();
+  keep = -1;
+}
+
+T lazy_contract(const T& a, const T& b, int n_keep) {
+  auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
+  p->fa = a.holder();
+  p->fb = b.holder();
+  p->keep = n_keep;
+  return T(p);
 }
 
 T lazy_mul(const T& a, const T& b) {
@@ -126,6 +142,8 @@ T lazy_mul(const T& a, const T& b) {
 
 T transpose(const T& a, const std::vector<int>& perm) {
   HD_VIEW_OF_PRODUCT(transpose(a0, perm), transpose(b0, perm))
+  if (a.pending_contraction() && (int)perm.size() <= a.pending_keep())   // permutes kept dims only
+    return lazy_contract(transpose(a.factor_a(), perm), transpose(a.factor_b(), perm), a.pending_keep());
   static const int dummy = 0;
   HD_OUT(transpose(be__->ctx, a.h(), (int)perm.size(), perm.empty() ? &dummy : perm.data(), &o__));
 }
@@ -167,10 +185,11 @@ T convert(const T& a, int dtype, int mode) {
   HD_OUT(convert(be__->ctx, a.h(), dtype, mode, &o__));
 }
 T contract(const T& a, const T* b, int n_keep) {
-  if (!b && a.pending_product()) {  // sum (u * v) = the contraction of u and v
-    T fa = a.factor_a(), fb = a.factor_b();
-    return contract(fa, &fb, n_keep);
-  }
+  if (!b && a.pending_product())   // sum (u * v) = the contraction of u and v; stays pending
+    return lazy_contract(a.factor_a(), a.factor_b(), n_keep);
+  return contract_now(a, b, n_keep);
+}
+static T contract_now(const T& a, const T* b, int n_keep) {
   HD_OUT(contract(be__->ctx, a.h(), b ? b->h() : nullptr, n_keep, &o__));
 }
 T argminmax_last(const T& a, bool want_max) { HD_OUT(argminmax_last(be__->ctx, a.h(), want_max ? 1 : 0, &o__)); }
@@ -485,9 +504,9 @@ T tsgather(const T& src, const Shape& shm, const std::vector<Ix>& ix) {
 // component, read as a mixed-radix number in the variables it uses, determines
 // those variables, and together the components use every variable.
 static bool provably_injective(const Shape& shm, const std::vector<Ix>& ix) {
-  if (!all_affine(ix)) return false;
   std::vector<bool> covered(shm.size(), false);
   for (auto& x : ix) {
+    if (!x.affine) continue;   // the affine components alone may already separate all positions
     std::vector<std::pair<int64_t, size_t>> terms;
     for (size_t d = 0; d < shm.size(); ++d)
       if (x.coef[d] != 0 && shm[d] > 1) terms.push_back({std::llabs(x.coef[d]), d});
@@ -506,6 +525,120 @@ static bool provably_injective(const Shape& shm, const std::vector<Ix>& ix) {
   return true;
 }
 
+// A view of f with the dims listed in `dims` zero-extended by lo / hi; dims f
+// is merely replicated along (stride 0) and that get no padding stay replicated.
+static T pad_dims(const T& f, const Shape& lo, const Shape& hi) {
+  Shape sh = f.shape(), st = f.strides();
+  bool any = false;
+  for (size_t d = 0; d < sh.size(); ++d) any = any || lo[d] > 0 || hi[d] > 0;
+  if (!any) return f;
+  Shape sh1 = sh, st1 = st;
+  for (size_t d = 0; d < sh.size(); ++d)
+    if (st[d] == 0 && lo[d] == 0 && hi[d] == 0) sh1[d] = 1;
+  T small = as_strided(f, sh1, st1, 0);
+  T padded = pad(small, lo, hi);
+  Shape psh = padded.shape(), pst = padded.strides();
+  for (size_t d = 0; d < sh.size(); ++d)
+    if (sh1[d] == 1 && sh[d] != 1) { psh[d] = sh[d]; pst[d] = 0; }
+  return as_strided(padded, psh, pst, 0);
+}
+
+// tsscatter with an affine, overlapping index function as a contraction:
+//   out[P.., n..] = sum over the positions m with ix(m) = P of src[m.., n..].
+// Every component P_j = c_j + m_v + sum_u a_ju m_u must have a "pivot" variable
+// m_v (coefficient 1, used by no other component); substituting
+// m_v = P_j - c_j - sum_u a_ju m_u turns src into a skewed view over
+// (P.., n.., u..) of its zero-extended self, summed over the remaining
+// variables u: col2im without atomics, in a fixed summation order.  When src is
+// itself a pending contraction the skew is applied to its factors and the
+// whole is ONE contraction (the transposed convolution).
+static T scatter_as_contraction(const T& src, int rank_m, const Shape& shp, const std::vector<Ix>& ix) {
+  Shape ssh = src.shape();
+  size_t rm = (size_t)rank_m, n_ix = ix.size(), rank_n = ssh.size() - rm;
+  std::vector<int> pivot(n_ix, -1);
+  std::vector<bool> is_pivot(rm, false);
+  for (size_t j = 0; j < n_ix; ++j) {
+    for (size_t d = 0; d < rm && pivot[j] < 0; ++d) {
+      if (ix[j].coef[d] != 1 || ssh[d] <= 1 || is_pivot[d]) continue;
+      bool elsewhere = false;
+      for (size_t j2 = 0; j2 < n_ix; ++j2)
+        if (j2 != j && ix[j2].coef[d] != 0) elsewhere = true;
+      if (!elsewhere) { pivot[j] = (int)d; is_pivot[d] = true; }
+    }
+    if (pivot[j] < 0) return T();
+  }
+  std::vector<size_t> summed;   // position variables that are not pivots
+  for (size_t d = 0; d < rm; ++d)
+    if (!is_pivot[d]) summed.push_back(d);
+
+  std::vector<T> factors;
+  int keep0;   // kept dims of the factors = rank_m + rank_n
+  if (src.pending_contraction()) {
+    factors = {src.factor_a(), src.factor_b()};
+    keep0 = src.pending_keep();
+  } else {
+    factors = {src};
+    keep0 = (int)ssh.size();
+  }
+  // every pivot must be felt by at least one factor, or out-of-range positions would not vanish
+  for (size_t j = 0; j < n_ix; ++j) {
+    bool felt = false;
+    for (auto& f : factors)
+      if (f.strides()[(size_t)pivot[j]] != 0) felt = true;
+    if (!felt) return T();
+  }
+  std::vector<T> views;
+  for (auto& f0 : factors) {
+    Shape fsh = f0.shape(), fst0 = f0.strides();
+    Shape lo(fsh.size(), 0), hi(fsh.size(), 0);
+    for (size_t j = 0; j < n_ix; ++j) {
+      size_t v = (size_t)pivot[j];
+      if (fst0[v] == 0) continue;
+      int64_t smin = 0, smax = 0;   // range of sum_u a_ju m_u
+      for (size_t d = 0; d < rm; ++d) {
+        if (d == v) continue;
+        int64_t span = ix[j].coef[d] * (ssh[d] - 1);
+        if (span > 0) smax += span; else smin += span;
+      }
+      int64_t c = ix[j].c0;
+      lo[v] = std::max<int64_t>(0, c + smax);
+      hi[v] = std::max<int64_t>(0, (shp[j] - 1 - c - smin) - (ssh[v] - 1));
+    }
+    int64_t grown = 1, plain = 1;
+    for (size_t d = 0; d < fsh.size(); ++d)
+      if (fst0[d] != 0) { plain *= fsh[d]; grown *= fsh[d] + lo[d] + hi[d]; }
+    if (grown > 4 * plain + 4096) return T();
+    T f = pad_dims(f0, lo, hi);
+    Shape fst = f.strides();
+    Shape nsh, nst;
+    int64_t offset = 0;
+    for (size_t j = 0; j < n_ix; ++j) {            // P dims
+      size_t v = (size_t)pivot[j];
+      nsh.push_back(shp[j]);
+      nst.push_back(fst[v]);
+      offset += (lo[v] - ix[j].c0) * fst[v];
+    }
+    for (size_t i = 0; i < rank_n; ++i) {          // n dims
+      nsh.push_back(fsh[rm + i]);
+      nst.push_back(fst[rm + i]);
+    }
+    for (size_t u : summed) {                      // summed position variables, skewed
+      int64_t s = fst[u];
+      for (size_t j = 0; j < n_ix; ++j) s -= ix[j].coef[u] * fst[(size_t)pivot[j]];
+      nsh.push_back(ssh[u]);
+      nst.push_back(s);
+    }
+    for (size_t i = (size_t)keep0; i < fsh.size(); ++i) {   // the factors' own reduced dims
+      nsh.push_back(fsh[i]);
+      nst.push_back(fst[i]);
+    }
+    views.push_back(as_strided(f, nsh, nst, offset));
+  }
+  int n_keep = (int)(n_ix + rank_n);
+  if (views.size() == 2) return contract_now(views[0], &views[1], n_keep);
+  return contract_now(views[0], nullptr, n_keep);
+}
+
 // Ops.hs:689-693; OpsConcrete.hs:1581-1619
 T tsscatter(const T& src, int rank_m, const Shape& shp, const std::vector<Ix>& ix) {
   if (rank_m > src.rank() || ix.size() != shp.size()) throw HostError(HGPU_ERR_INVALID, "tsscatter: ranks do not agree");
@@ -513,9 +646,14 @@ T tsscatter(const T& src, int rank_m, const Shape& shp, const std::vector<Ix>& i
   Shape shm(ssh.begin(), ssh.begin() + rank_m);
   check_ix(shm, ix);
   Backend* be = src.be();
+  bool injective = provably_injective(shm, ix);
+  if (!injective && all_affine(ix) && src.size() > 0) {
+    T r = scatter_as_contraction(src, rank_m, shp, ix);
+    if (r.valid()) return r;
+  }
   std::vector<T> arrs;
   for (auto& x : ix) arrs.push_back(ix_array(be, x));
-  return scatter_raw(src, arrs, rank_m, shp, provably_injective(shm, ix) ? 1 : 0);
+  return scatter_raw(src, arrs, rank_m, shp, injective ? 1 : 0);
 }
 
 // tsindex0 at lane-batched indices (AstIndexK, AstInterpret.hs:181-185)

@@ -1,0 +1,178 @@
+"""Index functions through the host layer: gather / scatter with lane-batched
+scalars against a per-position brute force (the reference's own algorithm,
+src/HordeAd/Core/OpsConcrete.hs:1581-1665: call the index function for every
+position, check bounds, copy or accumulate).  CPU half runs on the checker; the
+GPU half repeats the cases on the device and compares bit for bit (gather) or
+to 1e-10 (scatter sums).
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from conftest import capi, entry, pkg
+
+H = pkg.hostapi
+RNG = np.random.default_rng(7)
+
+
+@pytest.fixture(scope="module")
+def host_cpu():
+    return H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+
+
+@pytest.fixture(scope="module")
+def host_gpu():
+    return H.Host()
+
+
+def quot(a, b):
+    return a if b == 0 else int(abs(a) // abs(b)) * (1 if (a >= 0) == (b >= 0) else -1)
+
+
+def rem(a, b):
+    return a if b == 0 else a - quot(a, b) * b
+
+
+# (source shape, position space shm, index function on IxV, the same on ints, affine?)
+CASES = [
+    ((9, 3), (5, 4), lambda i, k: [i + k], lambda i, k: [i + k], True),                       # conv window, runs out of bounds
+    ((9, 3), (5, 4), lambda i, k: [i + k, k], lambda i, k: [i + k, k], True),
+    ((8, 6, 2), (4, 2, 3, 2), lambda i, p, j, q: [2 * i + p, 2 * j + q], lambda i, p, j, q: [2 * i + p, 2 * j + q], True),  # pooling windows
+    ((7, 5), (3, 6), lambda i, k: [6 - 2 * i, k - 1], lambda i, k: [6 - 2 * i, k - 1], True),  # negative coefficient, offset
+    ((7,), (4, 3), lambda i, k: [i * k], lambda i, k: [i * k], False),
+    ((7, 4), (5, 2), lambda i, k: [(i + 1).quotH(k), (2 * i).remH(3)], lambda i, k: [quot(i + 1, k), rem(2 * i, 3)], False),
+    ((6, 4), (6,), lambda i: [i.minH(3), (5 - i).maxH(1)], lambda i: [min(i, 3), max(5 - i, 1)], False),
+    ((5, 3), (), lambda: [2], lambda: [2], True),
+    ((5, 3), (4,), lambda i: [7, i], lambda i: [7, i], True),                                  # always out of bounds
+]
+
+
+def brute_gather(src, shm, f):
+    probe = f(*[0] * len(shm))
+    n_ix = len(probe)
+    out = np.zeros(tuple(shm) + src.shape[n_ix:], src.dtype)
+    for m in itertools.product(*[range(s) for s in shm]):
+        p = tuple(f(*m))
+        if all(0 <= p[k] < src.shape[k] for k in range(n_ix)):
+            out[m] = src[p]
+    return out
+
+
+def brute_scatter(src, rank_m, shp, f):
+    out = np.zeros(tuple(shp) + src.shape[rank_m:], src.dtype)
+    for m in itertools.product(*[range(s) for s in src.shape[:rank_m]]):
+        p = tuple(f(*m))
+        if all(0 <= p[k] < shp[k] for k in range(len(shp))):
+            out[p] += src[m]
+    return out
+
+
+def run_cases(host, exact_scatter):
+    for ssh, shm, f, fi, affine in CASES:
+        src = RNG.uniform(-1, 1, ssh)
+        v = host.concrete(src)
+        g = v.sgather(shm, f)
+        want = brute_gather(src, shm, fi)
+        assert np.array_equal(g.numpy(), want), (ssh, shm)
+        n_ix = len(fi(*[0] * len(shm)))
+        data = RNG.uniform(-1, 1, tuple(shm) + ssh[n_ix:])
+        s = host.concrete(data).sscatter(len(shm), ssh[:n_ix], f)
+        wants = brute_scatter(data, len(shm), ssh[:n_ix], fi)
+        assert s.shape == wants.shape
+        assert np.allclose(s.numpy(), wants, rtol=1e-12, atol=1e-13), (ssh, shm)
+        ix = f(*host.ix_space(shm)) if shm else f()
+        assert all((not isinstance(x, H.IxV)) or x.is_affine == affine or x.is_affine for x in ix)
+        # integer data: scatter sums are exact
+        idata = RNG.integers(-9, 9, tuple(shm) + ssh[n_ix:])
+        si = host.concrete(idata).sscatter(len(shm), ssh[:n_ix], f)
+        assert np.array_equal(si.numpy(), brute_scatter(idata, len(shm), ssh[:n_ix], fi))
+
+
+def test_gather_scatter_index_functions_cpu(host_cpu):
+    run_cases(host_cpu, True)
+
+
+def test_affine_gather_is_a_view(host_cpu):
+    """A gather with an affine, in-bounds index function moves no data: the
+    result is a strided view of the source (here checked through its values and
+    through the index function's classification)."""
+    src = np.arange(60.0).reshape(10, 6)
+    v = host_cpu.concrete(src)
+    i, k = host_cpu.ix_space((6, 4))
+    assert (i + k).is_affine and (2 * i + 3).is_affine and not (i * k).is_affine
+    g = v.sgather((6, 4), lambda i, k: [i + k])
+    assert np.array_equal(g.numpy(), np.lib.stride_tricks.sliding_window_view(src, 4, axis=0)[:6].transpose(0, 2, 1))
+    # a lookup in a constant table that is affine in its indices folds to an affine form
+    tbl = host_cpu.concrete(np.arange(14, dtype=np.int64).reshape(7, 2))
+    i, k = host_cpu.ix_space((7, 2))
+    assert tbl.sindex0([i, k]).is_affine
+    other = host_cpu.concrete(np.array([[0, 1], [2, 3], [4, 6]], np.int64))
+    i, k = host_cpu.ix_space((3, 2))
+    assert not other.sindex0([i, k]).is_affine
+
+
+def test_data_dependent_indices_cpu(host_cpu):
+    """relu mask and max-pool as the reference's simplified programs express them
+    (test/simplified/TestMnistPP.hs:735): gather from [0, 1] by
+    ifH (0 <=. negate x) 0 1, and gather at kargMax of a partial index."""
+    x = RNG.uniform(-1, 1, (4, 5))
+    t = host_cpu.concrete(x)
+    table = host_cpu.concrete(np.array([0.0, 1.0]))
+    zero = lambda: H.IxV.const(host_cpu, (4, 5), 0.0, capi.F64)  # noqa: E731
+    mask = table.sgather((4, 5), lambda i, j: [H.ifH(zero().leq(-t.sindex0([i, j]), capi.F64), 0, 1)])
+    assert np.array_equal(mask.numpy(), np.where(0.0 <= -x, 0.0, 1.0))
+    u = RNG.uniform(-1, 1, (3, 4, 6))
+    tu = host_cpu.concrete(u)
+    mx = tu.sgather((3, 4), lambda i, j: [i, j, tu.kargMax([i, j])])
+    assert np.array_equal(mx.numpy(), u.max(axis=-1))
+    mn = tu.sgather((3, 4), lambda i, j: [i, j, tu.kargMin([i, j])])
+    assert np.array_equal(mn.numpy(), u.min(axis=-1))
+
+
+def test_adjoint_law_cpu(host_cpu):
+    """sdot0 (sgather x f) y == sdot0 x (sscatter y f) (bench/ConvVjpBench.hs:564-584)."""
+    x = host_cpu.concrete(RNG.uniform(-1, 1, (12, 12, 3)))
+    f = lambda i, p, j, q: [i + p, j + q]  # noqa: E731
+    g = x.sgather((12, 3, 12, 3), f)
+    y = host_cpu.concrete(RNG.uniform(-1, 1, g.shape))
+    s = y.sscatter(4, (12, 12), f)
+    assert np.isclose(float(g.sdot0(y).numpy()), float(x.sdot0(s).numpy()), rtol=1e-12)
+
+
+def test_gradient_through_gather_matches_reference_kat(host_cpu):
+    """gatherNested1-style known answer: the gradient of a sum of gathered rows
+    counts how often each source element is read (cf. the expected arrays of
+    test/simplified/TestGatherSimplified.hs:154-159, which are such counts)."""
+    t = host_cpu.param(RNG.uniform(-1, 1, (7, 2)))
+    g = t.sgather((4, 2), lambda i, k: [i + k])          # rows 0..4, overlapping
+    grad = host_cpu.grad(g.ssum0(), [t])[0].numpy()
+    want = np.zeros((7, 2))
+    for i in range(4):
+        for k in range(2):
+            want[i + k] += 1
+    assert np.array_equal(grad, want)
+
+
+@pytest.mark.gpu
+def test_gather_scatter_index_functions_gpu(host_gpu):
+    run_cases(host_gpu, False)
+
+
+@pytest.mark.gpu
+def test_conv_vjp_chain_gpu_matches_cpu(host_gpu, host_cpu):
+    """Window gather -> contraction -> gradient: on the device the input gradient
+    is ONE contraction over skewed views (no patch gradient in memory, no
+    atomics); it must agree with the checker's literal scatter."""
+    a = RNG.uniform(-1, 1, (3, 2, 9, 8))
+    k = RNG.uniform(-1, 1, (4, 2, 3, 3))
+    res = []
+    for host in (host_gpu, host_cpu):
+        W = pkg.workloads
+        arr, ker = host.param(a), host.param(k)
+        out = W.conv2dPreservingS(ker, arr)
+        loss = (out * out).ssum0()
+        ga, gk = host.grad(loss, [arr, ker])
+        res.append((out.numpy(), ga.numpy(), gk.numpy()))
+    for g, c in zip(*res):
+        assert np.allclose(g, c, rtol=1e-10, atol=1e-12)
