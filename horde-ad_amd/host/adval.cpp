@@ -48,6 +48,8 @@ std::vector<T> Tape::backward(const D& out, const T& dt, const std::vector<D>& i
     if (i.node >= 0 && slots[(size_t)i.node].valid()) res.push_back(slots[(size_t)i.node]);
     else res.push_back(zeros(be, i.primal.dtype(), i.primal.shape()));   // tdefTarget
   }
+  // The gradient leaves are what the caller asked for: nothing stays pending.
+  for (auto& r : res) (void)r.h();
   return res;
 }
 
