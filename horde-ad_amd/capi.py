@@ -53,6 +53,7 @@ SIGNATURES = {
 GPU_ONLY = {
     "mem_stats": (I, [P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "stream": (P, [P]), "inject_alloc_failure": (I, [P, L]),
+    "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
     "profile_enable": (I, [P, I]), "profile_report": (I, [P, C.c_char_p, C.c_size_t]),
 }
 
@@ -125,6 +126,15 @@ class Ctx:
             name, cnt, ms, by, fl = line.split()
             out[name] = (int(cnt), float(ms), float(by), float(fl))
         return out
+
+    def fused_map(self, inputs, prog, out_slots):
+        """prog: list of (kind, op, dtype, a, b, c) over slots; returns the output arrays."""
+        ins = (C.c_void_p * len(inputs))(*[p.h for p in inputs])
+        flat = (C.c_int32 * (6 * len(prog)))(*[int(x) for q in prog for x in q])
+        slots = (C.c_int * len(out_slots))(*out_slots)
+        outs = (C.c_void_p * len(out_slots))()
+        self.check(self.lib.fused_map(self.h, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs))
+        return [Array(self, C.c_void_p(o)) for o in outs]
 
     def _wrap(self, h):
         return Array(self, h)

@@ -1,0 +1,403 @@
+// Fused elementwise maps: a chain of Num / Floating / comparison / conditional
+// / conversion operations over same-shaped views evaluated in ONE pass.
+//
+// horde-ad's interpreter calls `+`, `*`, `sin` ... one at a time
+// (src/HordeAd/Core/AstInterpret.hs:187-194) and the `Concrete` backend runs a
+// full pass over memory for each.  The host layer instead collects such calls
+// into a small straight-line program (inputs = views, one instruction per
+// call) and hands it over here; the program is turned into HIP source, compiled
+// once with hiprtc for gfx950 (cached by source text) and launched as one
+// kernel with any number of outputs, so every input element is read once and
+// every output element written once -- the traffic the HBM roofline is
+// computed from.
+//
+// Kernel shape: grid-stride loop, 256 lanes per block; when every non-scalar
+// input is dense each lane moves 16-byte vectors, otherwise each lane walks the
+// merged index space of the inputs (same decomposition as the eager kernels).
+#include <hip/hiprtc.h>
+
+#include <sstream>
+
+#include "common.hpp"
+
+using namespace hg;
+
+namespace {
+
+const char* ctype(int dt) {
+  switch (dt) {
+    case HGPU_F64: return "double";
+    case HGPU_F32: return "float";
+    case HGPU_I64: return "long long";
+    case HGPU_I32: return "int";
+    case HGPU_I16: return "short";
+    case HGPU_I8: return "signed char";
+    case HGPU_BOOL: return "unsigned char";
+  }
+  return "void";
+}
+
+// The device-side semantics of the opcodes: the same rules as the eager
+// kernels (signum of floats keeps zeros, quotH / remH divisor-0 rules, floor).
+const char* kPrelude = R"HG(
+typedef long long i64;
+template <typename T> struct is_fp { static constexpr bool value = false; };
+template <> struct is_fp<double> { static constexpr bool value = true; };
+template <> struct is_fp<float> { static constexpr bool value = true; };
+template <int OP, typename T> __device__ __forceinline__ T op1(T x) {
+  if constexpr (is_fp<T>::value) {
+    if constexpr (OP == 0) return -x;
+    else if constexpr (OP == 1) return fabs(x);
+    else if constexpr (OP == 2) return x > T(0) ? T(1) : (x < T(0) ? T(-1) : x);
+    else if constexpr (OP == 3) return T(1) / x;
+    else if constexpr (OP == 4) return exp(x);
+    else if constexpr (OP == 5) return log(x);
+    else if constexpr (OP == 6) return sqrt(x);
+    else if constexpr (OP == 7) return sin(x);
+    else if constexpr (OP == 8) return cos(x);
+    else if constexpr (OP == 9) return tan(x);
+    else if constexpr (OP == 10) return asin(x);
+    else if constexpr (OP == 11) return acos(x);
+    else if constexpr (OP == 12) return atan(x);
+    else if constexpr (OP == 13) return sinh(x);
+    else if constexpr (OP == 14) return cosh(x);
+    else if constexpr (OP == 15) return tanh(x);
+    else if constexpr (OP == 16) return asinh(x);
+    else if constexpr (OP == 17) return acosh(x);
+    else if constexpr (OP == 18) return atanh(x);
+    else return x;
+  } else {
+    if constexpr (OP == 0) return (T)(-x);
+    else if constexpr (OP == 1) return x < 0 ? (T)(-x) : x;
+    else if constexpr (OP == 2) return x > 0 ? T(1) : (x < 0 ? T(-1) : T(0));
+    else if constexpr (OP == 19) return (T)(x == 0 ? 1 : 0);
+    else return x;
+  }
+}
+template <int OP, typename T> __device__ __forceinline__ T op2(T x, T y) {
+  if constexpr (is_fp<T>::value) {
+    if constexpr (OP == 0) return x + y;
+    else if constexpr (OP == 1) return x * y;
+    else if constexpr (OP == 2) return x - y;
+    else if constexpr (OP == 3) return x / y;
+    else if constexpr (OP == 4) return pow(x, y);
+    else if constexpr (OP == 5) return log(y) / log(x);
+    else if constexpr (OP == 6) return atan2(x, y);
+    else if constexpr (OP == 10) return x <= y ? x : y;
+    else if constexpr (OP == 11) return x >= y ? x : y;
+    else return x;
+  } else {
+    if constexpr (OP == 0) return (T)(x + y);
+    else if constexpr (OP == 1) return (T)(x * y);
+    else if constexpr (OP == 2) return (T)(x - y);
+    else if constexpr (OP == 7) return y == 0 ? x : (T)(x / y);
+    else if constexpr (OP == 8) return y == 0 ? T(0) : (T)(x % y);
+    else if constexpr (OP == 9) return y == 0 ? x : (T)(x % y);
+    else if constexpr (OP == 10) return x <= y ? x : y;
+    else if constexpr (OP == 11) return x >= y ? x : y;
+    else if constexpr (OP == 12) return (T)((x != 0 && y != 0) ? 1 : 0);
+    else return x;
+  }
+}
+template <int OP, typename T> __device__ __forceinline__ unsigned char cmp2(T x, T y) {
+  if constexpr (OP == 0) return x <= y;
+  else if constexpr (OP == 1) return x == y;
+  else return x < y;
+}
+template <int MODE, typename D, typename S> __device__ __forceinline__ D conv(S x) {
+  if constexpr (is_fp<S>::value && !is_fp<D>::value) {
+    if constexpr (MODE == 1) return (D)(i64)floor((double)x);
+    else return (D)(i64)x;
+  } else {
+    return (D)x;
+  }
+}
+)HG";
+
+struct Compiled {
+  hipModule_t mod;
+  hipFunction_t fn;
+};
+
+std::map<std::string, Compiled>& cache_of(hgpu_ctx* ctx) {
+  // one cache per context, kept in the context's generic pointer map
+  auto it = ctx->jit_cache.find("__fused__");
+  if (it == ctx->jit_cache.end()) it = ctx->jit_cache.emplace("__fused__", new std::map<std::string, Compiled>()).first;
+  return *static_cast<std::map<std::string, Compiled>*>(it->second);
+}
+
+int compile(hgpu_ctx* ctx, const std::string& src, Compiled* out) {
+  hiprtcProgram prog;
+  if (hiprtcCreateProgram(&prog, src.c_str(), "fused_map.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+    return fail(ctx, HGPU_ERR_DEVICE, "hiprtcCreateProgram failed");
+  // packed FP32 instructions stay off, as in the ahead-of-time build; a hiprtc
+  // that does not take the feature switch compiles without it
+  const char* opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  hiprtcResult r = hiprtcCompileProgram(prog, 7, opts);
+  if (r != HIPRTC_SUCCESS) r = hiprtcCompileProgram(prog, 3, opts);
+  if (r != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, &log[0]);
+    hiprtcDestroyProgram(&prog);
+    return fail(ctx, HGPU_ERR_DEVICE, "hiprtc: %s: %.400s", hiprtcGetErrorString(r), log.c_str());
+  }
+  size_t n = 0;
+  hiprtcGetCodeSize(prog, &n);
+  std::vector<char> code(n);
+  hiprtcGetCode(prog, code.data());
+  hiprtcDestroyProgram(&prog);
+  hipError_t e = hipModuleLoadData(&out->mod, code.data());
+  if (e != hipSuccess) return check_hip(ctx, e, "hipModuleLoadData");
+  e = hipModuleGetFunction(&out->fn, out->mod, "fused_map");
+  if (e != hipSuccess) return check_hip(ctx, e, "hipModuleGetFunction");
+  return HGPU_OK;
+}
+
+constexpr int kMaxIn = 12, kMaxOut = 6, kMaxInstr = 96;
+
+struct FDims {
+  int nd;
+  int64_t shape[HG_KDIMS];
+  int64_t st[kMaxIn][HG_KDIMS];
+};
+
+}  // namespace
+
+extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
+                              int n_out, const int* out_slots, hgpu_array** outs) {
+  if (!ctx || !in || !prog || !out_slots || !outs) return HGPU_ERR_INVALID;
+  if (n_in < 1 || n_in > kMaxIn || n_out < 1 || n_out > kMaxOut || n_instr < 1 || n_instr > kMaxInstr)
+    return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map: %d inputs, %d instructions, %d outputs", n_in, n_instr, n_out);
+  const hgpu_array* a0 = in[0];
+  for (int i = 0; i < n_in; ++i) {
+    if (!in[i]) return HGPU_ERR_INVALID;
+    if (!same_shape(in[i], a0)) return fail(ctx, HGPU_ERR_INVALID, "fused_map: input %d has another shape", i);
+  }
+  // slot types, with the same checks the eager entry points make
+  std::vector<int> dt((size_t)(n_in + n_instr));
+  for (int i = 0; i < n_in; ++i) dt[(size_t)i] = in[i]->dtype;
+  for (int k = 0; k < n_instr; ++k) {
+    const hgpu_fused_instr& q = prog[k];
+    int self = n_in + k;
+    auto ok = [&](int s) { return s >= 0 && s < self; };
+    switch (q.kind) {
+      case HGPU_FUSED_OP1:
+        if (!ok(q.a) || q.op < 0 || q.op >= HGPU_OP1_COUNT) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad unary instruction %d", k);
+        if (q.op >= HGPU_RECIP && q.op <= HGPU_ATANH && !dtype_is_float(dt[(size_t)q.a])) return fail(ctx, HGPU_ERR_INVALID, "fused_map: floating opcode on a non-floating operand");
+        if ((q.op == HGPU_NOT) != (dt[(size_t)q.a] == HGPU_BOOL)) return fail(ctx, HGPU_ERR_INVALID, "fused_map: Bool mismatch");
+        dt[(size_t)self] = dt[(size_t)q.a];
+        break;
+      case HGPU_FUSED_OP2:
+        if (!ok(q.a) || !ok(q.b) || q.op < 0 || q.op >= HGPU_OP2_COUNT || dt[(size_t)q.a] != dt[(size_t)q.b]) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad binary instruction %d", k);
+        if (q.op >= HGPU_DIV && q.op <= HGPU_ATAN2 && !dtype_is_float(dt[(size_t)q.a])) return fail(ctx, HGPU_ERR_INVALID, "fused_map: floating opcode on a non-floating operand");
+        if (q.op >= HGPU_QUOT && q.op <= HGPU_REM_SCALAR && !dtype_is_int(dt[(size_t)q.a])) return fail(ctx, HGPU_ERR_INVALID, "fused_map: integral opcode on a non-integral operand");
+        if ((q.op == HGPU_AND) != (dt[(size_t)q.a] == HGPU_BOOL)) return fail(ctx, HGPU_ERR_INVALID, "fused_map: Bool mismatch");
+        dt[(size_t)self] = dt[(size_t)q.a];
+        break;
+      case HGPU_FUSED_CMP:
+        if (!ok(q.a) || !ok(q.b) || q.op < HGPU_LEQ || q.op > HGPU_LT || dt[(size_t)q.a] != dt[(size_t)q.b]) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad comparison %d", k);
+        dt[(size_t)self] = HGPU_BOOL;
+        break;
+      case HGPU_FUSED_SELECT:
+        if (!ok(q.a) || !ok(q.b) || !ok(q.c) || dt[(size_t)q.a] != HGPU_BOOL || dt[(size_t)q.b] != dt[(size_t)q.c]) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad select %d", k);
+        dt[(size_t)self] = dt[(size_t)q.b];
+        break;
+      case HGPU_FUSED_CONVERT:
+        if (!ok(q.a) || dtype_size(q.dtype) == 0) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad conversion %d", k);
+        if (q.op == HGPU_CONV_FLOOR && !(dtype_is_float(dt[(size_t)q.a]) && dtype_is_int(q.dtype))) return fail(ctx, HGPU_ERR_INVALID, "fused_map: floor needs float -> int");
+        dt[(size_t)self] = q.dtype;
+        break;
+      default:
+        return fail(ctx, HGPU_ERR_INVALID, "fused_map: unknown instruction kind %d", q.kind);
+    }
+  }
+  for (int o = 0; o < n_out; ++o)
+    if (out_slots[o] < 0 || out_slots[o] >= n_in + n_instr) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad output slot");
+
+  int64_t n = nelem(a0);
+  std::vector<hgpu_array*> res((size_t)n_out, nullptr);
+  auto release_all = [&] { for (auto* r : res) if (r) hgpu_release(r); };
+  for (int o = 0; o < n_out; ++o) {
+    int rc = new_dense(ctx, dt[(size_t)out_slots[o]], a0->rank, a0->shape, &res[(size_t)o]);
+    if (rc) { release_all(); return rc; }
+  }
+  if (n == 0) {
+    for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
+    return HGPU_OK;
+  }
+
+  // layout class of every input: 'd' dense, 's' one element broadcast, 'g' general
+  std::string layout((size_t)n_in, 'g');
+  bool all_simple = true;
+  int vec = 16;
+  for (int i = 0; i < n_in; ++i) {
+    bool all0 = true;
+    for (int d = 0; d < in[i]->rank; ++d)
+      if (in[i]->shape[d] != 1 && in[i]->strides[d] != 0) all0 = false;
+    if (all0) layout[(size_t)i] = 's';
+    else if (is_dense(in[i]) && ((uintptr_t)data_ptr(in[i]) & 15) == 0) layout[(size_t)i] = 'd';
+    else all_simple = false;
+  }
+  // vector width: 16 bytes of the widest type involved
+  size_t widest = 1;
+  for (int i = 0; i < n_in; ++i) widest = std::max(widest, dtype_size(in[i]->dtype));
+  for (int o = 0; o < n_out; ++o) widest = std::max(widest, dtype_size(res[(size_t)o]->dtype));
+  vec = (int)(16 / widest);
+  if (!all_simple) vec = 1;
+
+  // ---- source
+  std::ostringstream s;
+  s << kPrelude;
+  if (!all_simple) s << "struct FDims { int nd; i64 shape[" << HG_KDIMS << "]; i64 st[" << kMaxIn << "][" << HG_KDIMS << "]; };\n";
+  s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
+  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_map(i64 n";
+  if (!all_simple) s << ", FDims d";
+  for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
+  for (int o = 0; o < n_out; ++o) s << ", " << ctype(res[(size_t)o]->dtype) << "* __restrict__ o" << o;
+  s << ") {\n";
+  s << "  const i64 step = (i64)gridDim.x * 256;\n";
+  for (int i = 0; i < n_in; ++i)
+    if (layout[(size_t)i] == 's') s << "  const " << ctype(in[i]->dtype) << " s" << i << " = i" << i << "[0];\n";
+  auto emit_program = [&](const char* ind, const std::string& lane_suffix) {
+    for (int k = 0; k < n_instr; ++k) {
+      const hgpu_fused_instr& q = prog[k];
+      int self = n_in + k;
+      auto v = [&](int slot) { return "v" + std::to_string(slot) + lane_suffix; };
+      s << ind << "const " << ctype(dt[(size_t)self]) << " " << v(self) << " = ";
+      switch (q.kind) {
+        case HGPU_FUSED_OP1: s << "op1<" << q.op << ">(" << v(q.a) << ")"; break;
+        case HGPU_FUSED_OP2: s << "op2<" << q.op << ">(" << v(q.a) << ", " << v(q.b) << ")"; break;
+        case HGPU_FUSED_CMP: s << "cmp2<" << q.op << ">(" << v(q.a) << ", " << v(q.b) << ")"; break;
+        case HGPU_FUSED_SELECT: s << "(" << v(q.a) << " ? " << v(q.b) << " : " << v(q.c) << ")"; break;
+        default: s << "conv<" << q.op << ", " << ctype(q.dtype) << ">(" << v(q.a) << ")"; break;
+      }
+      s << ";\n";
+    }
+  };
+  if (all_simple) {
+    s << "  const i64 nv = n / " << vec << ";\n";
+    s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < nv; i += step) {\n";
+    for (int i = 0; i < n_in; ++i)
+      if (layout[(size_t)i] == 'd') s << "    const Vec<" << ctype(in[i]->dtype) << ", " << vec << "> l" << i << " = reinterpret_cast<const Vec<" << ctype(in[i]->dtype) << ", " << vec << ">*>(i" << i << ")[i];\n";
+    for (int o = 0; o < n_out; ++o) s << "    Vec<" << ctype(res[(size_t)o]->dtype) << ", " << vec << "> r" << o << ";\n";
+    for (int e = 0; e < vec; ++e) {
+      std::string suf = "_" + std::to_string(e);
+      s << "    {\n";
+      for (int i = 0; i < n_in; ++i) {
+        s << "      const " << ctype(in[i]->dtype) << " v" << i << suf << " = ";
+        if (layout[(size_t)i] == 's') s << "s" << i; else s << "l" << i << ".v[" << e << "]";
+        s << ";\n";
+      }
+      emit_program("      ", suf);
+      for (int o = 0; o < n_out; ++o) s << "      r" << o << ".v[" << e << "] = v" << out_slots[o] << suf << ";\n";
+      s << "    }\n";
+    }
+    for (int o = 0; o < n_out; ++o) s << "    reinterpret_cast<Vec<" << ctype(res[(size_t)o]->dtype) << ", " << vec << ">*>(o" << o << ")[i] = r" << o << ";\n";
+    s << "  }\n";
+    // tail
+    s << "  const i64 t = nv * " << vec << " + (i64)blockIdx.x * 256 + threadIdx.x;\n";
+    s << "  if (t < n) {\n";
+    for (int i = 0; i < n_in; ++i) {
+      s << "    const " << ctype(in[i]->dtype) << " v" << i << "_t = ";
+      if (layout[(size_t)i] == 's') s << "s" << i; else s << "i" << i << "[t]";
+      s << ";\n";
+    }
+    emit_program("    ", "_t");
+    for (int o = 0; o < n_out; ++o) s << "    o" << o << "[t] = v" << out_slots[o] << "_t;\n";
+    s << "  }\n";
+  } else {
+    s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {\n";
+    s << "    i64 off[" << n_in << "];\n";
+    s << "    for (int k = 0; k < " << n_in << "; ++k) off[k] = 0;\n";
+    s << "    i64 r = i;\n";
+    s << "    for (int q = d.nd - 1; q >= 0; --q) {\n";
+    s << "      i64 c = r;\n";
+    s << "      if (q > 0) { i64 w = r / d.shape[q]; c = r - w * d.shape[q]; r = w; }\n";
+    s << "      for (int k = 0; k < " << n_in << "; ++k) off[k] += c * d.st[k][q];\n";
+    s << "    }\n";
+    for (int i = 0; i < n_in; ++i) {
+      s << "    const " << ctype(in[i]->dtype) << " v" << i << "_g = ";
+      if (layout[(size_t)i] == 's') s << "s" << i; else s << "i" << i << "[off[" << i << "]]";
+      s << ";\n";
+    }
+    emit_program("    ", "_g");
+    for (int o = 0; o < n_out; ++o) s << "    o" << o << "[i] = v" << out_slots[o] << "_g;\n";
+    s << "  }\n";
+  }
+  s << "}\n";
+  std::string src = s.str();
+
+  LaunchGuard lg(ctx, "fused_map", 0, 0);
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c;
+    int rc = compile(ctx, src, &c);
+    if (rc) { release_all(); return rc; }
+    it = cache.emplace(src, c).first;
+  }
+  // algorithmic traffic: every distinct non-broadcast input once, every output once
+  double bytes = 0;
+  for (int i = 0; i < n_in; ++i) {
+    if (layout[(size_t)i] == 's') continue;
+    bool dup = false;
+    for (int j = 0; j < i; ++j)
+      if (data_ptr(in[j]) == data_ptr(in[i]) && layout[(size_t)j] != 's') dup = true;
+    int64_t distinct = 1;
+    for (int d = 0; d < in[i]->rank; ++d)
+      if (in[i]->strides[d] != 0) distinct *= in[i]->shape[d];
+    if (!dup) bytes += (double)distinct * dtype_size(in[i]->dtype);
+  }
+  for (int o = 0; o < n_out; ++o) bytes += (double)n * dtype_size(res[(size_t)o]->dtype);
+  if (lg.timed) { ctx->prof.back().bytes = bytes; ctx->prof.back().flops = (double)n * n_instr; }
+
+  FDims fd;
+  std::vector<void*> args;
+  int64_t nn = n;
+  args.push_back(&nn);
+  std::vector<const void*> ptrs((size_t)n_in);
+  std::vector<void*> optrs((size_t)n_out);
+  if (!all_simple) {
+    const int64_t* sts[kMaxIn];
+    for (int i = 0; i < n_in; ++i) sts[i] = in[i]->strides;
+    // merge dims jointly over all inputs
+    fd.nd = 0;
+    for (int d = 0; d < a0->rank; ++d) {
+      if (a0->shape[d] == 1) continue;
+      bool merged = false;
+      if (fd.nd > 0) {
+        int p = fd.nd - 1;
+        bool ok = true;
+        for (int k = 0; k < n_in; ++k)
+          if (fd.st[k][p] != sts[k][d] * a0->shape[d]) { ok = false; break; }
+        if (ok) {
+          fd.shape[p] *= a0->shape[d];
+          for (int k = 0; k < n_in; ++k) fd.st[k][p] = sts[k][d];
+          merged = true;
+        }
+      }
+      if (!merged) {
+        if (fd.nd == HG_KDIMS) { release_all(); return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map: more than %d merged dims", HG_KDIMS); }
+        fd.shape[fd.nd] = a0->shape[d];
+        for (int k = 0; k < n_in; ++k) fd.st[k][fd.nd] = sts[k][d];
+        fd.nd++;
+      }
+    }
+    if (fd.nd == 0) {
+      fd.nd = 1;
+      fd.shape[0] = 1;
+      for (int k = 0; k < n_in; ++k) fd.st[k][0] = 0;
+    }
+    args.push_back(&fd);
+  }
+  for (int i = 0; i < n_in; ++i) { ptrs[(size_t)i] = data_ptr(in[i]); args.push_back(&ptrs[(size_t)i]); }
+  for (int o = 0; o < n_out; ++o) { optrs[(size_t)o] = data_ptr(res[(size_t)o]); args.push_back(&optrs[(size_t)o]); }
+  int64_t work = all_simple ? (n + vec - 1) / vec : n;
+  unsigned grid = grid_for(work, 256, ctx->num_cu * 16);
+  hipError_t e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e != hipSuccess) { release_all(); return check_hip(ctx, e, "fused_map launch"); }
+  for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
+  return HGPU_OK;
+}

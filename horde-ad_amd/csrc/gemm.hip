@@ -232,14 +232,27 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__
   }
 }
 
-// Sums the split-K partials: out[i] = sum_s part[s * stride + i] for every element of the dense output.
+// Sums the split-K partials: out[i] = sum_s part[s * stride + i].  A block owns
+// 32 consecutive outputs; its 8 groups of 32 lanes each take every 8th partial
+// (coalesced rows of 32 elements) and combine through LDS in a fixed order.
 template <typename T>
 __global__ void __launch_bounds__(256) k_sum_partials(int64_t n, int S, int64_t stride, const T* __restrict__ part, T* __restrict__ out) {
-  int64_t step = (int64_t)gridDim.x * 256;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
-    T acc = part[i];
-    for (int s = 1; s < S; ++s) acc += part[(int64_t)s * stride + i];
-    out[i] = acc;
+  __shared__ T red[8][33];
+  const int ol = threadIdx.x & 31, g = threadIdx.x >> 5;
+  for (int64_t base = (int64_t)blockIdx.x * 32; base < n; base += (int64_t)gridDim.x * 32) {
+    int64_t i = base + ol;
+    T acc = T(0);
+    if (i < n)
+      for (int s = g; s < S; s += 8) acc += part[(int64_t)s * stride + i];
+    red[g][ol] = acc;
+    __syncthreads();
+    if (g == 0 && i < n) {
+      T t = red[0][ol];
+#pragma unroll
+      for (int k = 1; k < 8; ++k) t += red[k][ol];
+      out[i] = t;
+    }
+    __syncthreads();
   }
 }
 
@@ -436,12 +449,12 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
       double* cdst = split > 1 ? (double*)part->ptr : (double*)data_ptr(out);
       launch<double>(ctx, cfg, p, akc, bkc, grid, (const double*)data_ptr(a), (const double*)data_ptr(b), cdst, ka, kb);
       if (split > 1)
-        hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 256, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
+        hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
     } else {
       float* cdst = split > 1 ? (float*)part->ptr : (float*)data_ptr(out);
       launch<float>(ctx, cfg, p, akc, bkc, grid, (const float*)data_ptr(a), (const float*)data_ptr(b), cdst, ka, kb);
       if (split > 1)
-        hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 256, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
+        hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
     }
   }
   hipError_t e = hipGetLastError();

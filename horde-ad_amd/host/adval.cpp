@@ -48,8 +48,9 @@ std::vector<T> Tape::backward(const D& out, const T& dt, const std::vector<D>& i
     if (i.node >= 0 && slots[(size_t)i.node].valid()) res.push_back(slots[(size_t)i.node]);
     else res.push_back(zeros(be, i.primal.dtype(), i.primal.shape()));   // tdefTarget
   }
-  // The gradient leaves are what the caller asked for: nothing stays pending.
-  for (auto& r : res) (void)r.h();
+  // The gradient leaves are what the caller asked for: nothing stays pending,
+  // and leaves of one shape that are still elementwise programs share a pass.
+  force_many(res);
   return res;
 }
 

@@ -2,6 +2,11 @@
 // status codes out; C++ exceptions stop here.
 #include "hordead_host.h"
 
+#include <execinfo.h>
+#include <signal.h>
+#include <unistd.h>
+
+#include <cstdlib>
 #include <cstring>
 
 #include "host.hpp"
@@ -45,10 +50,20 @@ std::vector<Ix> ixs(int n, hh_ix* const* p) {
 
 }  // namespace
 
+// With HORDEAD_SEGV_TRACE set, a crash in native code prints its call stack.
+static void segv_trace(int sig) {
+  void* frames[64];
+  int n = backtrace(frames, 64);
+  backtrace_symbols_fd(frames, n, STDERR_FILENO);
+  signal(sig, SIG_DFL);
+  raise(sig);
+}
+
 extern "C" {
 
 int hh_create(const hgpu_api* api, int device, hh_ctx** out) {
   if (!api || !out) return HGPU_ERR_INVALID;
+  if (getenv("HORDEAD_SEGV_TRACE")) signal(SIGSEGV, segv_trace);
   hh_ctx* c = new hh_ctx;
   c->be.api = api;
   c->be.ctx = nullptr;
@@ -73,6 +88,7 @@ int hh_destroy(hh_ctx* c) {
 const char* hh_last_error(hh_ctx* c) { return c ? c->err.c_str() : "no context"; }
 int hh_sync(hh_ctx* c) { return guarded(c, [&] { c->be.check(c->be.api->sync(c->be.ctx)); }); }
 hgpu_ctx* hh_array_ctx(hh_ctx* c) { return c ? c->be.ctx : nullptr; }
+int hh_set_fusion(hh_ctx* c, int on) { c->be.fuse = on != 0; return HGPU_OK; }
 int hh_tape_reset(hh_ctx* c) { c->tape.recs.clear(); return HGPU_OK; }
 
 int hh_upload(hh_ctx* c, int dtype, int rank, const int64_t* shape, const void* host, int rg, hh_val** out) {

@@ -35,6 +35,7 @@ struct Backend {
   hgpu_ctx* ctx;
   std::map<std::pair<int, int64_t>, std::shared_ptr<ArrHolder>> iota_cache;   // (dtype, n)
   std::map<std::pair<int, uint64_t>, std::shared_ptr<ArrHolder>> const_cache; // (dtype, value bits)
+  bool fuse = true;   // defer elementwise operations into fused programs (when the provider has fused_map)
   void check(int rc) const;
 };
 
@@ -53,6 +54,14 @@ struct ArrHolder {
   // convolution never writes its patch gradient to memory).
   std::shared_ptr<ArrHolder> fa, fb;
   int keep = -1;
+  // A pending ELEMENTWISE operation (h == nullptr): kind/op as in
+  // hgpu_fused_instr, operands fa, fb, fc.  Chains of them are handed to the
+  // provider's fused_map as one program when the value is first needed as an
+  // array, so that `x * sin y + z` is one pass over memory, not three.
+  int ekind = -1, eop = 0, edtype = 0;
+  std::shared_ptr<ArrHolder> fc;
+  int esize = 0;          // pending nodes beneath, to bound program size
+  Shape eshape;
   ArrHolder(Backend* b, hgpu_array* a) : be(b), h(a) {}
   ~ArrHolder() { if (h) be->api->release(h); }
   ArrHolder(const ArrHolder&) = delete;
@@ -73,8 +82,9 @@ class T {
     if (!p_->h) p_->force();
     return p_->h;
   }
-  bool pending_product() const { return p_ && !p_->h && p_->fa && p_->keep < 0; }
-  bool pending_contraction() const { return p_ && !p_->h && p_->fa && p_->keep >= 0; }
+  bool pending_expr() const { return p_ && !p_->h && p_->ekind >= 0; }
+  bool pending_product() const { return pending_expr() && p_->ekind == HGPU_FUSED_OP2 && p_->eop == HGPU_MUL; }
+  bool pending_contraction() const { return p_ && !p_->h && p_->ekind < 0 && p_->fa && p_->keep >= 0; }
   int pending_keep() const { return p_->keep; }
   T factor_a() const { return T(p_->fa); }
   T factor_b() const { return T(p_->fb); }
@@ -84,8 +94,12 @@ class T {
     while (!q->h && q->fa) q = q->fa.get();
     return q->h;
   }
-  int rank() const { return pending_contraction() ? p_->keep : be()->api->rank(meta_h()); }
-  int dtype() const { return be()->api->dtype_of(meta_h()); }
+  int rank() const {
+    if (pending_expr()) return (int)p_->eshape.size();
+    return pending_contraction() ? p_->keep : be()->api->rank(meta_h());
+  }
+  int dtype() const { return pending_expr() ? p_->edtype : T(p_->fa ? p_->fa : p_).dtype_of_holder(); }
+  int dtype_of_holder() const { return p_->h ? be()->api->dtype_of(p_->h) : dtype(); }
   int64_t size() const {
     int64_t n = 1;
     for (auto e : shape()) n *= e;
@@ -117,6 +131,7 @@ T pad(const T& a, const Shape& lo, const Shape& hi);
 T ewise1(int op, const T& a);
 T ewise2(int op, const T& a, const T& b);
 T lazy_mul(const T& a, const T& b);                                // a * b, not yet written to memory
+void force_many(const std::vector<T>& ts);                         // pending values of one shape share a pass
 T lazy_contract(const T& a, const T& b, int n_keep);               // sum of a * b over the trailing dims, pending
 T compare(int cmp, const T& a, const T& b);
 bool compare_all(int cmp, const T& a, const T& b);

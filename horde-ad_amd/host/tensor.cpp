@@ -2,6 +2,7 @@
 // BaseTensor-named methods built from them, and the lane-batched evaluation of
 // index functions that turns gathers with affine indices into strided views.
 #include <algorithm>
+#include <cstddef>
 #include <cstring>
 #include <numeric>
 
@@ -14,6 +15,7 @@ void Backend::check(int rc) const {
 }
 
 Shape T::shape() const {
+  if (pending_expr()) return p_->eshape;
   if (pending_contraction()) {   // the kept dims of the first factor
     Shape f = T(p_->fa).shape();
     return Shape(f.begin(), f.begin() + p_->keep);
@@ -109,11 +111,175 @@ T iota(Backend* be, int64_t n, int dtype) {
   return T(be__, o__)
 
 static T contract_now(const T& a, const T* b, int n_keep);
+static T ewise1_now(int op, const T& a);
+static T ewise2_now(int op, const T& a, const T& b);
+static T compare_now(int cmp, const T& a, const T& b);
+static T select_now(const T& c, const T& a, const T& b);
+static T convert_now(const T& a, int dtype, int mode);
+
+// ------------------------------------------- pending elementwise expressions
+
+static bool fuses(Backend* be) {
+  return be->fuse && be->api->struct_size >= offsetof(hgpu_api, fused_map) + sizeof(be->api->fused_map) && be->api->fused_map != nullptr;
+}
+static int pending_size(const std::shared_ptr<ArrHolder>& p) { return (p && !p->h && p->ekind >= 0) ? p->esize : 0; }
+
+static T make_expr(int kind, int op, int dtype, const T& a, const T* b, const T* c) {
+  auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
+  p->ekind = kind;
+  p->eop = op;
+  p->edtype = dtype;
+  p->eshape = a.shape();
+  p->fa = a.holder();
+  if (b) p->fb = b->holder();
+  if (c) p->fc = c->holder();
+  // keep programs small: a large operand is written out first
+  int sz = 1 + pending_size(p->fa) + pending_size(p->fb) + pending_size(p->fc);
+  if (sz > 40) {
+    std::shared_ptr<ArrHolder>* big = &p->fa;
+    if (pending_size(p->fb) > pending_size(*big)) big = &p->fb;
+    if (pending_size(p->fc) > pending_size(*big)) big = &p->fc;
+    (*big)->force();
+    sz = 1 + pending_size(p->fa) + pending_size(p->fb) + pending_size(p->fc);
+  }
+  p->esize = sz;
+  return T(p);
+}
+
+namespace {
+struct Program {
+  std::vector<const ArrHolder*> inputs;
+  std::vector<std::pair<const ArrHolder*, hgpu_fused_instr>> instrs;   // operands hold holder slots until numbered
+  std::map<const ArrHolder*, int> in_slot, instr_slot;
+};
+
+// Post-order walk: materialised values (and pending contractions, which are
+// forced here) become inputs, pending elementwise nodes become instructions.
+int visit(Program& pg, ArrHolder* p) {
+  if (!p->h && p->ekind < 0 && p->fa) p->force();   // a pending contraction
+  if (p->h) {
+    auto it = pg.in_slot.find(p);
+    if (it != pg.in_slot.end()) return -1 - it->second;
+    int k = (int)pg.inputs.size();
+    pg.inputs.push_back(p);
+    pg.in_slot[p] = k;
+    return -1 - k;          // inputs are numbered after the walk: encode as negative
+  }
+  auto it = pg.instr_slot.find(p);
+  if (it != pg.instr_slot.end()) return it->second;
+  hgpu_fused_instr q;
+  q.kind = p->ekind;
+  q.op = p->eop;
+  q.dtype = p->edtype;
+  q.a = visit(pg, p->fa.get());
+  q.b = p->fb ? visit(pg, p->fb.get()) : 0;
+  q.c = p->fc ? visit(pg, p->fc.get()) : 0;
+  int k = (int)pg.instrs.size();
+  pg.instrs.push_back({p, q});
+  pg.instr_slot[p] = k;
+  return k;
+}
+}  // namespace
+
+static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
+  Program pg;
+  std::vector<int> root_slot;
+  for (auto* r : roots) root_slot.push_back(visit(pg, r));
+  int n_in = (int)pg.inputs.size(), n_instr = (int)pg.instrs.size();
+  auto slot = [&](int v) { return v < 0 ? -1 - v : n_in + v; };
+  std::vector<hgpu_fused_instr> prog;
+  for (auto& pi : pg.instrs) {
+    hgpu_fused_instr q = pi.second;
+    q.a = slot(q.a);
+    q.b = pi.first->fb ? slot(q.b) : 0;
+    q.c = pi.first->fc ? slot(q.c) : 0;
+    prog.push_back(q);
+  }
+  std::vector<const hgpu_array*> ins;
+  for (auto* p : pg.inputs) ins.push_back(p->h);
+  std::vector<int> outs_slot;
+  for (int v : root_slot) outs_slot.push_back(slot(v));
+  std::vector<hgpu_array*> outs(roots.size(), nullptr);
+  be->check(be->api->fused_map(be->ctx, n_in, ins.data(), n_instr, prog.data(), (int)roots.size(), outs_slot.data(), outs.data()));
+  for (size_t i = 0; i < roots.size(); ++i) {
+    ArrHolder* r = roots[i];
+    r->h = outs[i];
+    r->fa.reset();
+    r->fb.reset();
+    r->fc.reset();
+    r->ekind = -1;
+  }
+}
+
+// Counts the inputs and instructions a set of roots would need.
+static void measure(const std::vector<ArrHolder*>& roots, int* n_in, int* n_instr) {
+  std::map<const ArrHolder*, int> seen;
+  std::vector<const ArrHolder*> stack(roots.begin(), roots.end());
+  *n_in = *n_instr = 0;
+  while (!stack.empty()) {
+    const ArrHolder* p = stack.back();
+    stack.pop_back();
+    if (seen.count(p)) continue;
+    seen[p] = 1;
+    if (p->h || p->ekind < 0) { ++*n_in; continue; }
+    ++*n_instr;
+    if (p->fa) stack.push_back(p->fa.get());
+    if (p->fb) stack.push_back(p->fb.get());
+    if (p->fc) stack.push_back(p->fc.get());
+  }
+}
+
+static void force_roots(Backend* be, std::vector<ArrHolder*> roots) {
+  // drop roots that are already arrays, or that appear twice
+  std::vector<ArrHolder*> rs;
+  for (auto* r : roots)
+    if (!r->h && r->ekind >= 0 && std::find(rs.begin(), rs.end(), r) == rs.end()) rs.push_back(r);
+  if (rs.empty()) return;
+  int n_in, n_instr;
+  measure(rs, &n_in, &n_instr);
+  const int kIn = 12, kInstr = 96, kOut = 6;
+  if (rs.size() > 1 && ((int)rs.size() > kOut || n_in > kIn || n_instr > kInstr)) {
+    // too much for one pass: halve the set
+    std::vector<ArrHolder*> lo(rs.begin(), rs.begin() + (long)rs.size() / 2), hi(rs.begin() + (long)rs.size() / 2, rs.end());
+    force_roots(be, lo);
+    force_roots(be, hi);
+    return;
+  }
+  if (n_in > kIn || n_instr > kInstr) {
+    // one root with too many leaves: write its largest pending operand out first
+    ArrHolder* r = rs[0];
+    std::shared_ptr<ArrHolder> big = r->fa;
+    if (pending_size(r->fb) > pending_size(big)) big = r->fb;
+    if (pending_size(r->fc) > pending_size(big)) big = r->fc;
+    if (pending_size(big) == 0) {   // only arrays beneath: cannot shrink further
+      run_program(be, rs);
+      return;
+    }
+    force_roots(be, {big.get()});
+    force_roots(be, rs);
+    return;
+  }
+  run_program(be, rs);
+}
+
+void force_many(const std::vector<T>& ts) {
+  std::map<std::pair<Backend*, Shape>, std::vector<ArrHolder*>> groups;
+  for (auto& t : ts)
+    if (t.valid() && t.pending_expr()) groups[{t.be(), t.shape()}].push_back(t.holder().get());
+  for (auto& g : groups) force_roots(g.first.first, g.second);
+  for (auto& t : ts)
+    if (t.valid()) (void)t.h();
+}
 
 void ArrHolder::force() {
-  if (h || !fa) return;
+  if (h) return;
+  if (ekind >= 0) {
+    force_roots(be, {this});
+    return;
+  }
+  if (!fa) return;
   T fbt(fb);
-  T p = keep >= 0 ? contract_now(T(fa), &fbt, keep) : ewise2(HGPU_MUL, T(fa), fbt);
+  T p = contract_now(T(fa), &fbt, keep);
   be->check(be->api->retain(p.h()));
   h = p.h();
   fa.reset();
@@ -121,19 +287,13 @@ void ArrHolder::force() {
   keep = -1;
 }
 
+T lazy_mul(const T& a, const T& b) { return ewise2(HGPU_MUL, a, b); }
+
 T lazy_contract(const T& a, const T& b, int n_keep) {
   auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
   p->fa = a.holder();
   p->fb = b.holder();
   p->keep = n_keep;
-  return T(p);
-}
-
-T lazy_mul(const T& a, const T& b) {
-  if (a.dtype() != b.dtype() || a.shape() != b.shape()) return ewise2(HGPU_MUL, a, b);  // reports the mismatch
-  auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
-  p->fa = a.holder();
-  p->fb = b.holder();
   return T(p);
 }
 
@@ -171,18 +331,54 @@ T as_strided(const T& a, const Shape& shape, const Shape& strides, int64_t offse
 }
 T materialize(const T& a) { HD_OUT(materialize(be__->ctx, a.h(), &o__)); }
 T pad(const T& a, const Shape& lo, const Shape& hi) { HD_OUT(pad(be__->ctx, a.h(), ptr_or_dummy(lo), ptr_or_dummy(hi), &o__)); }
-T ewise1(int op, const T& a) { HD_OUT(ewise1(be__->ctx, op, a.h(), &o__)); }
-T ewise2(int op, const T& a, const T& b) { HD_OUT(ewise2(be__->ctx, op, a.h(), b.h(), &o__)); }
-T compare(int cmp, const T& a, const T& b) { HD_OUT(compare(be__->ctx, cmp, a.h(), b.h(), &o__)); }
+static T ewise1_now(int op, const T& a) { HD_OUT(ewise1(be__->ctx, op, a.h(), &o__)); }
+static T ewise2_now(int op, const T& a, const T& b) { HD_OUT(ewise2(be__->ctx, op, a.h(), b.h(), &o__)); }
+static T compare_now(int cmp, const T& a, const T& b) { HD_OUT(compare(be__->ctx, cmp, a.h(), b.h(), &o__)); }
+
+// The elementwise methods defer when the provider can run fused programs and
+// the operands agree (a mismatch goes to the eager entry point, which reports it).
+static bool agree(const T& a, const T& b) { return a.dtype() == b.dtype() && a.shape() == b.shape(); }
+static bool is_fp_dt(int dt) { return dt == HGPU_F64 || dt == HGPU_F32; }
+static bool is_int_dt(int dt) { return dt >= HGPU_I64 && dt <= HGPU_I8; }
+static bool op1_ok(int op, int dt) {
+  if (op < 0 || op >= HGPU_OP1_COUNT) return false;
+  if (op >= HGPU_RECIP && op <= HGPU_ATANH) return is_fp_dt(dt);
+  return (op == HGPU_NOT) == (dt == HGPU_BOOL);
+}
+static bool op2_ok(int op, int dt) {
+  if (op < 0 || op >= HGPU_OP2_COUNT) return false;
+  if (op >= HGPU_DIV && op <= HGPU_ATAN2) return is_fp_dt(dt);
+  if (op >= HGPU_QUOT && op <= HGPU_REM_SCALAR) return is_int_dt(dt);
+  return (op == HGPU_AND) == (dt == HGPU_BOOL);
+}
+T ewise1(int op, const T& a) {
+  if (!fuses(a.be()) || !op1_ok(op, a.dtype()) || a.size() == 0) return ewise1_now(op, a);
+  return make_expr(HGPU_FUSED_OP1, op, a.dtype(), a, nullptr, nullptr);
+}
+T ewise2(int op, const T& a, const T& b) {
+  if (!fuses(a.be()) || !agree(a, b) || !op2_ok(op, a.dtype()) || a.size() == 0) return ewise2_now(op, a, b);
+  return make_expr(HGPU_FUSED_OP2, op, a.dtype(), a, &b, nullptr);
+}
+T compare(int cmp, const T& a, const T& b) {
+  if (!fuses(a.be()) || !agree(a, b) || cmp < HGPU_LEQ || cmp > HGPU_LT || a.size() == 0) return compare_now(cmp, a, b);
+  return make_expr(HGPU_FUSED_CMP, cmp, HGPU_BOOL, a, &b, nullptr);
+}
 bool compare_all(int cmp, const T& a, const T& b) {
   int r = 0;
   a.be()->check(a.be()->api->compare_all(a.be()->ctx, cmp, a.h(), b.h(), &r));
   return r != 0;
 }
-T select(const T& c, const T& a, const T& b) { HD_OUT(select(be__->ctx, c.h(), a.h(), b.h(), &o__)); }
+static T select_now(const T& c, const T& a, const T& b) { HD_OUT(select(be__->ctx, c.h(), a.h(), b.h(), &o__)); }
+static T convert_now(const T& a, int dtype, int mode) { HD_OUT(convert(be__->ctx, a.h(), dtype, mode, &o__)); }
+T select(const T& c, const T& a, const T& b) {
+  if (!fuses(a.be()) || !agree(a, b) || c.dtype() != HGPU_BOOL || c.shape() != a.shape() || a.size() == 0) return select_now(c, a, b);
+  return make_expr(HGPU_FUSED_SELECT, 0, a.dtype(), c, &a, &b);
+}
 T convert(const T& a, int dtype, int mode) {
   if (a.dtype() == dtype && mode == HGPU_CONV_CAST) return a;
-  HD_OUT(convert(be__->ctx, a.h(), dtype, mode, &o__));
+  bool ok = dtype >= HGPU_F64 && dtype <= HGPU_BOOL && (mode == HGPU_CONV_CAST || (mode == HGPU_CONV_FLOOR && is_fp_dt(a.dtype()) && is_int_dt(dtype)));
+  if (!fuses(a.be()) || !ok || a.size() == 0) return convert_now(a, dtype, mode);
+  return make_expr(HGPU_FUSED_CONVERT, mode, dtype, a, nullptr, nullptr);
 }
 T contract(const T& a, const T* b, int n_keep) {
   if (!b && a.pending_product())   // sum (u * v) = the contraction of u and v; stays pending

@@ -19,7 +19,7 @@ LP, IP = C.POINTER(C.c_int64), C.POINTER(C.c_int)
 D = C.c_double
 SIG = {
     "create_gpu": (I, [I, PP]), "create": (I, [P, I, PP]), "destroy": (I, [P]),
-    "last_error": (C.c_char_p, [P]), "sync": (I, [P]), "array_ctx": (P, [P]), "tape_reset": (I, [P]),
+    "last_error": (C.c_char_p, [P]), "sync": (I, [P]), "array_ctx": (P, [P]), "tape_reset": (I, [P]), "set_fusion": (I, [P, I]),
     "upload": (I, [P, I, I, LP, P, I, PP]), "from_array": (I, [P, P, I, PP]),
     "constant": (I, [P, I, D, I, LP, PP]), "array": (I, [P, PP]), "download": (I, [P, P, P]),
     "val_rank": (I, [P]), "val_dtype": (I, [P]), "val_shape": (I, [P, LP]), "free": (I, [P]),
@@ -83,6 +83,9 @@ class Host:
 
     def sync(self):
         self.check(self.dll.hh_sync(self.h))
+
+    def set_fusion(self, on):
+        self.check(self.dll.hh_set_fusion(self.h, int(on)))
 
     def tape_reset(self):
         self.check(self.dll.hh_tape_reset(self.h))

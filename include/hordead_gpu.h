@@ -204,6 +204,21 @@ int hgpu_select(hgpu_ctx* ctx, const hgpu_array* cond, const hgpu_array* a, cons
 /* tsfloor / tsfromIntegral / tscast / tkcast (OpsConcrete.hs:352-368,455-532). */
 int hgpu_convert(hgpu_ctx* ctx, const hgpu_array* a, int dtype, int mode, hgpu_array** out);
 
+/* A chain of the elementwise operations above in one pass.  The program is
+ * straight-line code over numbered slots: slots 0 .. n_in-1 are the inputs
+ * (views of one shape), slot n_in + k is the result of instruction k, whose
+ * operands a, b, c name earlier slots.  `kind` selects the family: OP1 (op =
+ * hgpu_op1), OP2 (op = hgpu_op2), CMP (op = hgpu_cmp, result BOOL), SELECT
+ * (a = BOOL condition, b, c), CONVERT (op = hgpu_conv mode, dtype = target).
+ * outs[i] receives slot out_slots[i] as a dense array.  This is what the
+ * interpreter's one-call-per-node stream of `+`, `*`, `sin`, ...
+ * (AstInterpret.hs:187-194) becomes when the host layer defers it; results
+ * equal those of the single entry points applied in program order. */
+enum hgpu_fused_kind { HGPU_FUSED_OP1 = 0, HGPU_FUSED_OP2 = 1, HGPU_FUSED_CMP = 2, HGPU_FUSED_SELECT = 3, HGPU_FUSED_CONVERT = 4 };
+typedef struct hgpu_fused_instr { int32_t kind, op, dtype, a, b, c; } hgpu_fused_instr;
+int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
+                   int n_out, const int* out_slots, hgpu_array** outs);
+
 /* out[o] = sum_r a[o,r] * b[o,r]  (b == NULL: b = 1), o ranging over the first
  * n_keep dims and r over the rest.  With the free views above this one entry
  * point is tssum / tssumN / tssum0 (OpsConcrete.hs:215-230, b NULL, summed dims
@@ -251,6 +266,7 @@ int hgpu_onehot(hgpu_ctx* ctx, const hgpu_array* v, int n, const int64_t* ix, co
  * written against the table can be pointed at another provider of this ABI
  * (the test suite points it at a CPU checker). */
 typedef struct hgpu_api {
+  size_t struct_size;   /* sizeof(hgpu_api) of the provider's build: members beyond it are absent */
   int (*init)(int, hgpu_ctx**);
   int (*shutdown)(hgpu_ctx*);
   int (*sync)(hgpu_ctx*);
@@ -288,6 +304,8 @@ typedef struct hgpu_api {
   int (*gather)(hgpu_ctx*, const hgpu_array*, int, const hgpu_array* const*, int, const int64_t*, hgpu_array**);
   int (*scatter_add)(hgpu_ctx*, const hgpu_array*, int, const hgpu_array* const*, int, const int64_t*, int, hgpu_array**);
   int (*onehot)(hgpu_ctx*, const hgpu_array*, int, const int64_t*, const int64_t*, hgpu_array**);
+  /* optional (may be NULL): a provider without it gets the operations one by one */
+  int (*fused_map)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, const int*, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

@@ -38,6 +38,9 @@ int hh_destroy(hh_ctx* ctx);
 const char* hh_last_error(hh_ctx* ctx);
 int hh_sync(hh_ctx* ctx);
 hgpu_ctx* hh_array_ctx(hh_ctx* ctx);
+/* Elementwise operations are deferred and handed to the provider as fused
+ * programs (default, when the provider has fused_map); 0 runs them one by one. */
+int hh_set_fusion(hh_ctx* ctx, int on);
 /* Forgets the recorded operations; values made before stay usable as constants. */
 int hh_tape_reset(hh_ctx* ctx);
 

@@ -624,15 +624,54 @@ int horc_onehot(hgpu_ctx* c, const hgpu_array* v, int n, const int64_t* ix, cons
   return HGPU_OK;
 }
 
+// The meaning of a fused program: the single operations applied in program order.
+int horc_fused_map(hgpu_ctx* c, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
+                   int n_out, const int* out_slots, hgpu_array** outs) {
+  std::vector<hgpu_array*> slots;
+  std::vector<hgpu_array*> made;
+  for (int i = 0; i < n_in; ++i) slots.push_back(const_cast<hgpu_array*>(in[i]));
+  int rc = HGPU_OK;
+  for (int k = 0; k < n_instr && rc == HGPU_OK; ++k) {
+    const hgpu_fused_instr& q = prog[k];
+    int self = n_in + k;
+    auto ok = [&](int s) { return s >= 0 && s < self; };
+    hgpu_array* o = nullptr;
+    if (!ok(q.a) || (q.kind != HGPU_FUSED_OP1 && q.kind != HGPU_FUSED_CONVERT && !ok(q.b)) || (q.kind == HGPU_FUSED_SELECT && !ok(q.c))) {
+      rc = fail(c, HGPU_ERR_INVALID, "fused_map: bad operand slot");
+      break;
+    }
+    switch (q.kind) {
+      case HGPU_FUSED_OP1: rc = horc_ewise1(c, q.op, slots[q.a], &o); break;
+      case HGPU_FUSED_OP2: rc = horc_ewise2(c, q.op, slots[q.a], slots[q.b], &o); break;
+      case HGPU_FUSED_CMP: rc = horc_compare(c, q.op, slots[q.a], slots[q.b], &o); break;
+      case HGPU_FUSED_SELECT: rc = horc_select(c, slots[q.a], slots[q.b], slots[q.c], &o); break;
+      case HGPU_FUSED_CONVERT: rc = horc_convert(c, slots[q.a], q.dtype, q.op, &o); break;
+      default: rc = fail(c, HGPU_ERR_INVALID, "fused_map: unknown instruction kind");
+    }
+    if (rc == HGPU_OK) { slots.push_back(o); made.push_back(o); }
+  }
+  if (rc == HGPU_OK) {
+    for (int i = 0; i < n_out; ++i) {
+      int s = out_slots[i];
+      if (s < 0 || s >= (int)slots.size()) { rc = fail(c, HGPU_ERR_INVALID, "fused_map: bad output slot"); break; }
+      if (s < n_in) rc = horc_materialize(c, slots[s], &outs[i]);
+      else { outs[i] = slots[s]; horc_retain(slots[s]); }
+    }
+  }
+  for (auto* m : made) horc_release(m);
+  return rc;
+}
+
 const hgpu_api* horc_get_api(void) {
   static const hgpu_api api = {
+      sizeof(hgpu_api),
       horc_init,        horc_shutdown,  horc_sync,         horc_last_error, horc_upload,      horc_download,
       horc_read_scalar, horc_retain,    horc_release,      horc_rank,       horc_dtype_of,    horc_size,
       horc_shape,       horc_strides,   horc_is_dense,     horc_transpose,  horc_reshape,     horc_slice,
       horc_reverse,     horc_replicate, horc_index_prefix, horc_as_strided, horc_materialize, horc_pad,
       horc_ewise1,      horc_ewise2,    horc_compare,      horc_compare_all, horc_select,     horc_convert,
       horc_contract,    horc_argminmax_last, horc_iota,    horc_concat,     horc_gather,      horc_scatter_add,
-      horc_onehot,
+      horc_onehot,      horc_fused_map,
   };
   return &api;
 }

@@ -399,3 +399,81 @@ def test_contract_on_the_matrix_cores(both, gpu, dt):
     rep = gpu.profile_report()
     gpu.profile(False)
     assert any(k.startswith("gemm") for k in rep), rep
+
+
+def eval_program_eagerly(ctx, inputs, prog, out_slots):
+    """The meaning of a fused program: the single entry points applied in order."""
+    inv1 = {v: k for k, v in capi.OP1.items()}
+    inv2 = {v: k for k, v in capi.OP2.items()}
+    invc = {v: k for k, v in capi.CMP.items()}
+    slots = list(inputs)
+    for kind, op, dtype, a, b, c in prog:
+        if kind == 0:
+            slots.append(slots[a].ewise1(inv1[op]))
+        elif kind == 1:
+            slots.append(slots[a].ewise2(inv2[op], slots[b]))
+        elif kind == 2:
+            slots.append(slots[a].compare(invc[op], slots[b]))
+        elif kind == 3:
+            slots.append(slots[a].select(slots[b], slots[c]))
+        else:
+            slots.append(slots[a].convert(dtype, op))
+    return [slots[s] for s in out_slots]
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_fused_map_equals_the_single_operations(gpu, oracle, dt):
+    tol = TOL[np.dtype(dt)]
+    O1, O2 = capi.OP1, capi.OP2
+    # foo's gradient program: inputs x, y, z, dret (a broadcast scalar)
+    prog = [
+        (0, O1["sin"], 0, 1, 0, 0),      # 4: sin y
+        (1, O2["mul"], 0, 0, 4, 0),      # 5: w = x * sin y
+        (1, O2["mul"], 0, 2, 2, 0),      # 6: z*z
+        (1, O2["mul"], 0, 5, 5, 0),      # 7: w*w
+        (1, O2["add"], 0, 6, 7, 0),      # 8
+        (0, O1["recip"], 0, 8, 0, 0),    # 9: t
+        (0, O1["neg"], 0, 2, 0, 0),      # 10: -z
+        (1, O2["mul"], 0, 10, 9, 0),     # 11: -z t
+        (1, O2["add"], 0, 11, 2, 0),     # 12: dw = -z t + z
+        (1, O2["mul"], 0, 12, 3, 0),     # 13: dw * dret
+        (1, O2["mul"], 0, 13, 4, 0),     # 14: dx
+        (0, O1["cos"], 0, 1, 0, 0),      # 15
+        (1, O2["mul"], 0, 13, 0, 0),     # 16
+        (1, O2["mul"], 0, 16, 15, 0),    # 17: dy
+        (1, O2["mul"], 0, 5, 9, 0),      # 18: w t
+        (1, O2["add"], 0, 18, 5, 0),     # 19
+        (1, O2["mul"], 0, 19, 3, 0),     # 20: dz
+        (2, capi.CMP["leq"], 0, 0, 1, 0),            # 21: x <= y (Bool)
+        (3, 0, 0, 21, 14, 17),                        # 22: select
+        (4, 1, capi.I64, 22, 0, 0),                   # 23: floor -> Int
+        (4, 0, capi.F32 if dt == np.float64 else capi.F64, 20, 0, 0),   # 24: cast
+    ]
+    outs = [14, 17, 20, 21, 22, 23, 24][:6]
+    for shape, views in [((1031,), False), ((37, 29), False), ((6, 5, 7), True)]:
+        data = [rnd(shape, dt) + dt(2.5) for _ in range(3)]
+        res = []
+        for ctx in (gpu, oracle):
+            ins = [ctx.upload(d) for d in data] + [ctx.upload(dt(1.25)).replicate(list(shape))]
+            if views:
+                ins[0] = ctx.upload(np.ascontiguousarray(np.transpose(data[0], (2, 0, 1)))).transpose([1, 2, 0])
+                ins[1] = ins[1].reverse(1).reverse(1)
+            if ctx is gpu:
+                res.append([o.numpy() for o in ctx.fused_map(ins, prog, outs)])
+            else:
+                res.append([o.numpy() for o in eval_program_eagerly(ctx, ins, prog, outs)])
+        for g, o in zip(*res):
+            assert g.dtype == o.dtype and g.shape == o.shape
+            if g.dtype.kind == "f":
+                assert np.max(np.abs(g - o)) <= tol * max(np.max(np.abs(o)), 1e-300)
+            else:
+                assert np.array_equal(g, o)
+    # integer programs are exact, including the divisor-0 rules
+    x, y = rnd((500,), np.int32), rnd((500,), np.int32)
+    prog = [(1, O2["quot"], 0, 0, 1, 0), (1, O2["rem"], 0, 0, 1, 0), (1, O2["rem_scalar"], 0, 0, 1, 0), (1, O2["add"], 0, 2, 3, 0), (0, O1["signum"], 0, 5, 0, 0)]
+    g = [o.numpy() for o in gpu.fused_map([gpu.upload(x), gpu.upload(y)], prog, [2, 3, 4, 6])]
+    o = [o.numpy() for o in eval_program_eagerly(oracle, [oracle.upload(x), oracle.upload(y)], prog, [2, 3, 4, 6])]
+    for a, b in zip(g, o):
+        assert np.array_equal(a, b)
+    with pytest.raises(capi.HgpuError):
+        gpu.fused_map([gpu.upload(x)], [(0, O1["exp"], 0, 0, 0, 0)], [1])
