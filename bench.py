@@ -116,6 +116,8 @@ def main():
     ap.add_argument("--workload", default="c3", help="headline config: c0..c4")
     ap.add_argument("--only", action="store_true", help="measure the headline config only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run plain dense copies of 1 GiB (for scaling hardware traffic counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus,
@@ -124,6 +126,16 @@ def main():
 
     pkg = entry.load_package()
     capi, H, W = pkg.capi, pkg.hostapi, pkg.workloads
+    if args.calibrate_copy:
+        import numpy as np
+        ctx = capi.Lib().context(0)
+        src = ctx.upload(np.zeros(1 << 27, np.float64))       # 1 GiB
+        for _ in range(5):
+            dst = src.materialize()                            # k_copy: reads 1 GiB, writes 1 GiB
+            del dst
+        ctx.sync()
+        print(json.dumps({"calibration": "5 dense copies", "bytes_read_per_copy": 1 << 30, "bytes_written_per_copy": 1 << 30}))
+        return
     host = H.Host()      # raises when the HIP library is missing or no device is usable
 
     keys = [args.workload] if args.only else [args.workload] + [k for k in W.CONFIGS if k != args.workload]
