@@ -204,6 +204,43 @@ __global__ void __launch_bounds__(kBlock) k_argminmax_wave(Dims keep, int64_t n_
   }
 }
 
+// One block of 1024 lanes per row, for a few very long rows (the minimum of a
+// whole tensor): lanes scan strided subsequences, then combine through LDS with
+// the same "smaller index wins ties" rule.
+template <typename T>
+__global__ void __launch_bounds__(1024) k_argminmax_block(Dims keep, int64_t L, int64_t sl, int want_max, const T* __restrict__ a, int64_t* __restrict__ out) {
+  __shared__ T sbest[1024];
+  __shared__ int64_t sidx[1024];
+  int64_t ko[1];
+  decompose<1>(keep, blockIdx.x, ko);
+  const T* p = a + ko[0];
+  const int t = threadIdx.x;
+  bool have = t < L;
+  T best = have ? p[(int64_t)t * sl] : T(0);
+  int64_t bi = t;
+  for (int64_t j = t + 1024; j < L; j += 1024) {
+    T x = p[j * sl];
+    bool better = want_max ? (x > best) : (x < best);
+    if (better) { best = x; bi = j; }
+  }
+  sbest[t] = best;
+  sidx[t] = have ? bi : INT64_MAX;
+  __syncthreads();
+  for (int off = 512; off > 0; off >>= 1) {
+    if (t < off) {
+      T ob = sbest[t + off];
+      int64_t oi = sidx[t + off];
+      if (oi != INT64_MAX) {
+        bool mine = sidx[t] != INT64_MAX;
+        bool better = !mine || (want_max ? (ob > sbest[t]) : (ob < sbest[t])) || (ob == sbest[t] && oi < sidx[t]);
+        if (better) { sbest[t] = ob; sidx[t] = oi; }
+      }
+    }
+    __syncthreads();
+  }
+  if (t == 0) out[blockIdx.x] = sidx[0];
+}
+
 template <typename TI, typename TO>
 int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red_full, int64_t n_out, int64_t R, int S, const void* a, const void* b, void* out) {
   LaunchGuard lg(ctx, b ? (use_wave ? "contract_dot_wave" : "contract_dot_lane") : (use_wave ? "contract_sum_wave" : "contract_sum_lane"),
@@ -345,7 +382,10 @@ int hgpu_argminmax_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_a
     Dims keep;
     if (!collapse(a->rank - 1, a->shape, 1, ks, &keep)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "argminmax: too many dims"); }
     LaunchGuard lg(ctx, "argminmax", (double)n_out * (L * dtype_size(a->dtype) + 8), (double)n_out * L);
-    if (L >= 256 && n_out < (int64_t)ctx->num_cu * 64) {
+    if (L >= 8192 && n_out <= 64) {
+      // few long rows: a whole block per row
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_block<T>, dim3((unsigned)n_out), dim3(1024), 0, ctx->stream, keep, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
+    } else if (L >= 256 && n_out < (int64_t)ctx->num_cu * 64) {
       unsigned g = grid_for(n_out * 64, kBlock, ctx->num_cu * 8);
       HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_wave<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
     } else {

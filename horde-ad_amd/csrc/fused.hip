@@ -329,7 +329,15 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   s << "}\n";
   std::string src = s.str();
 
-  LaunchGuard lg(ctx, "fused_map", 0, 0);
+  const char* label = "fused_map";
+  if (ctx->profiling && ctx->profile_shapes) {
+    std::string sh;
+    for (int d = 0; d < a0->rank; ++d) sh += (d ? "x" : "") + std::to_string(a0->shape[d]);
+    char buf[160];
+    snprintf(buf, sizeof buf, "fused_map[%s,in%d(%s),instr%d(k%d.op%d..),out%d,vec%d,dt%d]", sh.c_str(), n_in, layout.c_str(), n_instr, prog[0].kind, prog[0].op, n_out, vec, a0->dtype);
+    label = ctx->label_pool.insert(buf).first->c_str();
+  }
+  LaunchGuard lg(ctx, label, 0, 0);
   auto& cache = cache_of(ctx);
   auto it = cache.find(src);
   if (it == cache.end()) {

@@ -25,6 +25,8 @@
 // so that each XCD (blockIdx mod 8) works on a contiguous run of tiles and its
 // L2 sees neighbouring rows of A.  Small outputs with long K are split along K
 // into partial products summed by a second launch (fixed order: reproducible).
+#include <algorithm>
+
 #include "common.hpp"
 
 using namespace hg;
@@ -43,6 +45,7 @@ struct Group {
 struct GemmParams {
   Group m, n, k, bt;
   int64_t M, N, K, BT;
+  int a_kc, b_kc;     // lanes staging A (B) run along k (1) or along m (n) (0)
   int split;          // K chunks
   int64_t kchunk;     // K elements per chunk (multiple of BK)
   int64_t c_split_stride;  // elements between partial outputs
@@ -93,16 +96,25 @@ template <> struct Mfma<float> {
   static __device__ __forceinline__ int row(int lane, int r) { return 4 * (lane >> 4) + r; }
 };
 
+template <typename T, int V> struct VecOf;
+template <> struct VecOf<double, 1> { using type = double; };
+template <> struct VecOf<float, 1> { using type = float; };
+template <> struct VecOf<double, 2> { using type = __attribute__((ext_vector_type(2))) double; };
+template <> struct VecOf<float, 4> { using type = __attribute__((ext_vector_type(4))) float; };
+
 // Block tile BM x BN = (WGM * TM * 16) x (WGN * TN * 16): the 4 wavefronts form a
-// WGM x WGN grid and each owns TM x TN MFMA tiles.  A_KC / B_KC: the operand's
-// innermost K dim has unit stride (lanes run along k); otherwise lanes run
-// along m (resp. n).
-template <typename T, int WGM, int WGN, int TM, int TN, bool A_KC, bool B_KC>
+// WGM x WGN grid and each owns TM x TN MFMA tiles.  p.a_kc / p.b_kc: the lanes
+// that stage an operand tile run along k (the operand's innermost K dim is the
+// contiguous one) or along m / n.  VA / VB: elements per global load (16-byte
+// vectors when the host has checked contiguity and alignment, else 1).
+template <typename T, int WGM, int WGN, int TM, int TN, int VA, int VB>
 __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                              const int64_t* __restrict__ koffA, const int64_t* __restrict__ koffB) {
   using V4 = typename Mfma<T>::V4;
+  using VecA = typename VecOf<T, VA>::type;
+  using VecB = typename VecOf<T, VB>::type;
   constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
-  constexpr int NA = BM * BK / NT, NB = BN * BK / NT;   // operand elements each thread stages per K-step
+  constexpr int NA = BM * BK / NT / VA, NB = BN * BK / NT / VB;   // loads each thread issues per K-step
   static_assert(WGM * WGN == 4 && NA >= 1 && NB >= 1, "tile shape");
   __shared__ T As[BK][BM + 1];
   __shared__ T Bs[BK][BN + 1];
@@ -127,17 +139,19 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__
   int64_t kend = kbeg + p.kchunk;
   if (kend > p.K) kend = p.K;
 
-  // this thread's (row, k) slots of each operand tile
+  // this thread's (row, k) slots of each operand tile; a slot covers VA (VB)
+  // consecutive elements along the direction the lanes run
   int aml[NA], akl[NA], bnl[NB], bkl[NB];
   int64_t aoff[NA], boff[NB];
   bool aok[NA], bok[NB];
+  const int adk = p.a_kc ? 1 : 0, adm = 1 - adk, bdk = p.b_kc ? 1 : 0, bdn = 1 - bdk;
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
-    if (A_KC) { aml[i] = (t >> 4) + 16 * i; akl[i] = t & 15; }
-    else { aml[i] = t % BM; akl[i] = t / BM + (NT / BM) * i; }
+    if (p.a_kc) { constexpr int KL = BK / VA; aml[i] = t / KL + (NT / KL) * i; akl[i] = (t % KL) * VA; }
+    else { constexpr int ML = BM / VA; aml[i] = (t % ML) * VA; akl[i] = t / ML + (NT / ML) * i; }
     int64_t m = m0 + aml[i];
     aok[i] = m < p.M;
-    if (A_KC || i == 0) {
+    if (p.a_kc || i == 0) {
       int64_t oa = 0, ob = 0, oc = 0;
       if (aok[i]) group_off(p.m, m, &oa, &ob, &oc);
       aoff[i] = oa + bta;
@@ -147,11 +161,11 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__
   }
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    if (B_KC) { bnl[i] = (t >> 4) + 16 * i; bkl[i] = t & 15; }
-    else { bnl[i] = t % BN; bkl[i] = t / BN + (NT / BN) * i; }
+    if (p.b_kc) { constexpr int KL = BK / VB; bnl[i] = t / KL + (NT / KL) * i; bkl[i] = (t % KL) * VB; }
+    else { constexpr int NL = BN / VB; bnl[i] = (t % NL) * VB; bkl[i] = t / NL + (NT / NL) * i; }
     int64_t n = n0 + bnl[i];
     bok[i] = n < p.N;
-    if (B_KC || i == 0) {
+    if (p.b_kc || i == 0) {
       int64_t oa = 0, ob = 0, oc = 0;
       if (bok[i]) group_off(p.n, n, &oa, &ob, &oc);
       boff[i] = ob + btb;
@@ -166,26 +180,41 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = V4{0, 0, 0, 0};
 
-  T ra[NA], rb[NB];
+  VecA ra[NA];
+  VecB rb[NB];
   auto load_tile = [&](int64_t k0) {
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
       int64_t ka = k0 + akl[i];
-      ra[i] = (aok[i] && ka < kend) ? A[aoff[i] + koffA[ka]] : T(0);
+      if (aok[i] && ka < kend) ra[i] = *reinterpret_cast<const VecA*>(A + aoff[i] + koffA[ka]);
+      else ra[i] = VecA{};
     }
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       int64_t kb = k0 + bkl[i];
-      rb[i] = (bok[i] && kb < kend) ? B[boff[i] + koffB[kb]] : T(0);
+      if (bok[i] && kb < kend) rb[i] = *reinterpret_cast<const VecB*>(B + boff[i] + koffB[kb]);
+      else rb[i] = VecB{};
     }
   };
 
   if (kbeg < kend) load_tile(kbeg);
   for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
 #pragma unroll
-    for (int i = 0; i < NA; ++i) As[akl[i]][aml[i]] = ra[i];
+    for (int i = 0; i < NA; ++i) {
+      if constexpr (VA == 1) As[akl[i]][aml[i]] = ra[i];
+      else {
 #pragma unroll
-    for (int i = 0; i < NB; ++i) Bs[bkl[i]][bnl[i]] = rb[i];
+        for (int j = 0; j < VA; ++j) As[akl[i] + j * adk][aml[i] + j * adm] = ra[i][j];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      if constexpr (VB == 1) Bs[bkl[i]][bnl[i]] = rb[i];
+      else {
+#pragma unroll
+        for (int j = 0; j < VB; ++j) Bs[bkl[i] + j * bdk][bnl[i] + j * bdn] = rb[i][j];
+      }
+    }
     __syncthreads();
     if (k0 + BK < kend) load_tile(k0 + BK);
 #pragma unroll
@@ -314,28 +343,49 @@ const TileCfg kTiles[] = {
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 template <typename T, int WGM, int WGN, int TM, int TN>
-void launch_cfg(hgpu_ctx* ctx, const GemmParams& p, bool akc, bool bkc, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
-  if (akc && bkc) hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, true, true>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
-  else if (akc) hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, true, false>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
-  else if (bkc) hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, false, true>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
-  else hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, false, false>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
+void launch_cfg(hgpu_ctx* ctx, const GemmParams& p, bool va, bool vb, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
+  constexpr int V = 16 / sizeof(T);
+  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
+  // 16-byte loads only for tiles whose rows are long enough to share a load's lanes sensibly
+  if constexpr (BM >= 64 && BN >= 64) {
+    if (va && vb) { hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, V, V>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb); return; }
+    if (va) { hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, V, 1>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb); return; }
+    if (vb) { hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, 1, V>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb); return; }
+  }
+  hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, 1, 1>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
 }
 
 template <typename T>
-void launch(hgpu_ctx* ctx, int cfg, const GemmParams& p, bool akc, bool bkc, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
+void launch(hgpu_ctx* ctx, int cfg, const GemmParams& p, bool va, bool vb, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
   switch (cfg) {
-    case 0: launch_cfg<T, 2, 2, 4, 4>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    case 1: launch_cfg<T, 2, 2, 4, 2>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    case 2: launch_cfg<T, 2, 2, 2, 4>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    case 3: launch_cfg<T, 4, 1, 4, 2>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    case 4: launch_cfg<T, 1, 4, 2, 4>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    case 5: launch_cfg<T, 4, 1, 4, 1>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    case 6: launch_cfg<T, 1, 4, 1, 4>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    case 7: launch_cfg<T, 2, 2, 2, 2>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    case 8: launch_cfg<T, 2, 2, 1, 1>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    case 9: launch_cfg<T, 4, 1, 1, 1>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
-    default: launch_cfg<T, 1, 4, 1, 1>(ctx, p, akc, bkc, grid, A, B, C, ka, kb); break;
+    case 0: launch_cfg<T, 2, 2, 4, 4>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    case 1: launch_cfg<T, 2, 2, 4, 2>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    case 2: launch_cfg<T, 2, 2, 2, 4>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    case 3: launch_cfg<T, 4, 1, 4, 2>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    case 4: launch_cfg<T, 1, 4, 2, 4>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    case 5: launch_cfg<T, 4, 1, 4, 1>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    case 6: launch_cfg<T, 1, 4, 1, 4>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    case 7: launch_cfg<T, 2, 2, 2, 2>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    case 8: launch_cfg<T, 2, 2, 1, 1>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    case 9: launch_cfg<T, 4, 1, 1, 1>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
+    default: launch_cfg<T, 1, 4, 1, 1>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
   }
+}
+
+// True when 16-byte loads along the direction the staging lanes run are safe
+// for one operand: unit stride and an extent that is a multiple of the vector
+// there, every other stride and the base address a multiple of the vector.
+bool vector_ok(const void* base, size_t es, const Group& run, int run_dim, const int64_t* run_st,
+               const Group* others[3], const int64_t* const other_st[3]) {
+  const int64_t v = (int64_t)(16 / es);
+  if (((uintptr_t)base & 15) != 0) return false;
+  if (run_st[run_dim] != 1 || run.shape[run_dim] % v != 0) return false;
+  for (int i = 0; i < run.nd; ++i)
+    if (i != run_dim && run_st[i] % v != 0) return false;
+  for (int g = 0; g < 3; ++g)
+    for (int i = 0; i < others[g]->nd; ++i)
+      if (other_st[g][i] % v != 0) return false;
+  return true;
 }
 
 }  // namespace
@@ -348,23 +398,44 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   if (a->dtype != HGPU_F64 && a->dtype != HGPU_F32) return HGPU_OK;
   GemmParams p;
   p.m.nd = p.n.nd = p.k.nd = p.bt.nd = 0;
-  // classify the kept dims (output strides are the dense ones of `out`)
+  // Classify the dims.  The dims of a group are an index SET: any order works
+  // as long as A, B and C agree, so each group is sorted with the dim that is
+  // most contiguous in memory last (innermost) -- that is the dim the lanes of
+  // a load run along -- and only then merged.
+  struct DimRec { int64_t e, sa, sb, sc; };
+  std::vector<DimRec> gm, gn, gk, gb;
   for (int i = 0; i < n_keep; ++i) {
     int64_t e = a->shape[i], sa = a->strides[i], sb = b->strides[i], sc = out->strides[i];
     if (e == 1) continue;
-    bool ok;
-    if (sa != 0 && sb == 0) ok = push_dim(p.m, e, sa, 0, sc);
-    else if (sa == 0 && sb != 0) ok = push_dim(p.n, e, 0, sb, sc);
-    else if (sa != 0 && sb != 0) ok = push_dim(p.bt, e, sa, sb, sc);
+    if (sa != 0 && sb == 0) gm.push_back({e, sa, 0, sc});
+    else if (sa == 0 && sb != 0) gn.push_back({e, 0, sb, sc});
+    else if (sa != 0 && sb != 0) gb.push_back({e, sa, sb, sc});
     else return HGPU_OK;  // an output dim neither operand depends on
-    if (!ok) return HGPU_OK;
   }
   for (int i = n_keep; i < a->rank; ++i) {
     int64_t e = a->shape[i], sa = a->strides[i], sb = b->strides[i];
     if (e == 1) continue;
     if (sa == 0 || sb == 0) return HGPU_OK;  // a plain sum hidden in the contraction
-    if (!push_dim(p.k, e, sa, sb, 0)) return HGPU_OK;
+    gk.push_back({e, sa, sb, 0});
   }
+  auto mag = [](int64_t v) { return v < 0 ? -v : v; };
+  std::stable_sort(gm.begin(), gm.end(), [&](const DimRec& x, const DimRec& y) { return mag(x.sa) > mag(y.sa); });
+  std::stable_sort(gn.begin(), gn.end(), [&](const DimRec& x, const DimRec& y) { return mag(x.sb) > mag(y.sb); });
+  {
+    // K: follow the operand that has a unit-stride K dim; when both or neither
+    // do, the one that is larger (more rows to stream)
+    int64_t rows_a = 1, rows_b = 1;
+    for (auto& d : gm) rows_a *= d.e;
+    for (auto& d : gn) rows_b *= d.e;
+    bool a_unit = false, b_unit = false;
+    for (auto& d : gk) { a_unit = a_unit || mag(d.sa) == 1; b_unit = b_unit || mag(d.sb) == 1; }
+    bool by_a = (a_unit != b_unit) ? a_unit : rows_a >= rows_b;
+    std::stable_sort(gk.begin(), gk.end(), [&](const DimRec& x, const DimRec& y) { return by_a ? mag(x.sa) > mag(y.sa) : mag(x.sb) > mag(y.sb); });
+  }
+  for (auto& d : gm) if (!push_dim(p.m, d.e, d.sa, d.sb, d.sc)) return HGPU_OK;
+  for (auto& d : gn) if (!push_dim(p.n, d.e, d.sa, d.sb, d.sc)) return HGPU_OK;
+  for (auto& d : gk) if (!push_dim(p.k, d.e, d.sa, d.sb, d.sc)) return HGPU_OK;
+  for (auto& d : gb) if (!push_dim(p.bt, d.e, d.sa, d.sb, d.sc)) return HGPU_OK;
   finish(p.m);
   finish(p.n);
   finish(p.k);
@@ -431,8 +502,27 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   p.c_split_stride = split > 1 ? out_n : 0;
   int64_t* ka = (int64_t*)koff->ptr;
   int64_t* kb = ka + p.K;
-  bool akc = p.k.sa[p.k.nd - 1] == 1;
-  bool bkc = p.k.sb[p.k.nd - 1] == 1;
+  // lanes run along k when the innermost K dim is contiguous and long enough to
+  // fill a 16-lane group, or when running along m / n would be no better
+  auto along_k = [](int64_t sk, int64_t ek, int64_t srow) {
+    if (sk < 0) sk = -sk;
+    if (srow < 0) srow = -srow;
+    if (sk == 1 && (ek >= 16 || srow != 1)) return true;
+    return srow != 1 && sk < srow;
+  };
+  bool akc = along_k(p.k.sa[p.k.nd - 1], p.k.shape[p.k.nd - 1], p.m.sa[p.m.nd - 1]);
+  bool bkc = along_k(p.k.sb[p.k.nd - 1], p.k.shape[p.k.nd - 1], p.n.sb[p.n.nd - 1]);
+  p.a_kc = akc ? 1 : 0;
+  p.b_kc = bkc ? 1 : 0;
+  bool va, vb;
+  {
+    const Group* oa[3] = {akc ? &p.m : &p.k, &p.bt, &p.bt};
+    const int64_t* const osa[3] = {akc ? p.m.sa : p.k.sa, p.bt.sa, p.bt.sa};
+    va = vector_ok(data_ptr(a), dtype_size(a->dtype), akc ? p.k : p.m, (akc ? p.k.nd : p.m.nd) - 1, akc ? p.k.sa : p.m.sa, oa, osa);
+    const Group* ob[3] = {bkc ? &p.n : &p.k, &p.bt, &p.bt};
+    const int64_t* const osb[3] = {bkc ? p.n.sb : p.k.sb, p.bt.sb, p.bt.sb};
+    vb = vector_ok(data_ptr(b), dtype_size(b->dtype), bkc ? p.k : p.n, (bkc ? p.k.nd : p.n.nd) - 1, bkc ? p.k.sb : p.n.sb, ob, osb);
+  }
   dim3 grid((unsigned)tiles, (unsigned)split, (unsigned)p.BT);
   {
     double flops = 2.0 * p.M * p.N * p.K * p.BT;
@@ -440,19 +530,19 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     const char* label = a->dtype == HGPU_F64 ? "gemm_f64" : "gemm_f32";
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[128];
-      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,%s%s,t%lldx%lld]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, split, akc ? "k" : "m", bkc ? "k" : "n", (long long)BM, (long long)BN);
+      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,%s%s,t%lldx%lld]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, split, akc ? (va ? "K" : "k") : (va ? "M" : "m"), bkc ? (vb ? "K" : "k") : (vb ? "N" : "n"), (long long)BM, (long long)BN);
       label = ctx->label_pool.insert(buf).first->c_str();
     }
     LaunchGuard lg(ctx, label, bytes, flops);
     hipLaunchKernelGGL(k_koff, dim3((unsigned)((p.K + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, ka, kb);
     if (a->dtype == HGPU_F64) {
       double* cdst = split > 1 ? (double*)part->ptr : (double*)data_ptr(out);
-      launch<double>(ctx, cfg, p, akc, bkc, grid, (const double*)data_ptr(a), (const double*)data_ptr(b), cdst, ka, kb);
+      launch<double>(ctx, cfg, p, va, vb, grid, (const double*)data_ptr(a), (const double*)data_ptr(b), cdst, ka, kb);
       if (split > 1)
         hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
     } else {
       float* cdst = split > 1 ? (float*)part->ptr : (float*)data_ptr(out);
-      launch<float>(ctx, cfg, p, akc, bkc, grid, (const float*)data_ptr(a), (const float*)data_ptr(b), cdst, ka, kb);
+      launch<float>(ctx, cfg, p, va, vb, grid, (const float*)data_ptr(a), (const float*)data_ptr(b), cdst, ka, kb);
       if (split > 1)
         hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
     }

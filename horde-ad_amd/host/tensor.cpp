@@ -831,8 +831,43 @@ static T scatter_as_contraction(const T& src, int rank_m, const Shape& shp, cons
     views.push_back(as_strided(f, nsh, nst, offset));
   }
   int n_keep = (int)(n_ix + rank_n);
-  if (views.size() == 2) return contract_now(views[0], &views[1], n_keep);
-  return contract_now(views[0], nullptr, n_keep);
+  // The result may be laid out in any order of its dims: take the memory order
+  // of the larger factor (most distinct elements), so the contraction streams
+  // it and writes the result in the same order, and hand back a transposed view.
+  size_t main_f = 0;
+  if (views.size() == 2) {
+    auto distinct = [](const T& v) {
+      Shape sh = v.shape(), st = v.strides();
+      int64_t n = 1;
+      for (size_t d = 0; d < sh.size(); ++d)
+        if (st[d] != 0) n *= sh[d];
+      return n;
+    };
+    if (distinct(views[1]) > distinct(views[0])) main_f = 1;
+  }
+  Shape mst = views[main_f].strides();
+  std::vector<int> order((size_t)n_keep);
+  for (int i = 0; i < n_keep; ++i) order[(size_t)i] = i;
+  std::stable_sort(order.begin(), order.end(), [&](int x, int y) {
+    int64_t sx = std::llabs(mst[(size_t)x]), sy = std::llabs(mst[(size_t)y]);
+    if (sx == 0) sx = INT64_MAX;   // dims the main factor is replicated along go outermost
+    if (sy == 0) sy = INT64_MAX;
+    return sx > sy;
+  });
+  bool identity = true;
+  for (int i = 0; i < n_keep; ++i) identity = identity && order[(size_t)i] == i;
+  if (identity) {
+    if (views.size() == 2) return contract_now(views[0], &views[1], n_keep);
+    return contract_now(views[0], nullptr, n_keep);
+  }
+  std::vector<int> inv((size_t)n_keep);
+  for (int i = 0; i < n_keep; ++i) inv[(size_t)order[(size_t)i]] = i;
+  T va = transpose(views[0], order);
+  if (views.size() == 2) {
+    T vb = transpose(views[1], order);
+    return transpose(contract_now(va, &vb, n_keep), inv);
+  }
+  return transpose(contract_now(va, nullptr, n_keep), inv);
 }
 
 // Ops.hs:689-693; OpsConcrete.hs:1581-1619
