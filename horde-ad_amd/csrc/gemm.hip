@@ -27,50 +27,12 @@
 // into partial products summed by a second launch (fixed order: reproducible).
 #include <algorithm>
 
-#include "common.hpp"
+#include "gemm_kernel.hpp"
 
 using namespace hg;
+using namespace hg::gemm;
 
 namespace {
-
-constexpr int BK = 16, NT = 256;
-constexpr int GD = 5;  // dims per index group after merging
-
-struct Group {
-  int nd;
-  int64_t shape[GD];
-  int64_t sa[GD], sb[GD], sc[GD];
-};
-
-struct GemmParams {
-  Group m, n, k, bt;
-  int64_t M, N, K, BT;
-  int a_kc, b_kc;     // lanes staging A (B) run along k (1) or along m (n) (0)
-  int split;          // K chunks
-  int64_t kchunk;     // K elements per chunk (multiple of BK)
-  int64_t c_split_stride;  // elements between partial outputs
-};
-
-__device__ __forceinline__ void group_off(const Group& g, int64_t lin, int64_t* oa, int64_t* ob, int64_t* oc) {
-  int64_t a = 0, b = 0, c = 0;
-  int64_t r = lin;
-  for (int i = g.nd - 1; i >= 0; --i) {
-    int64_t idx;
-    if (i > 0) {
-      int64_t q = r / g.shape[i];
-      idx = r - q * g.shape[i];
-      r = q;
-    } else {
-      idx = r;
-    }
-    a += idx * g.sa[i];
-    b += idx * g.sb[i];
-    c += idx * g.sc[i];
-  }
-  *oa = a;
-  *ob = b;
-  *oc = c;
-}
 
 __global__ void k_koff(Group k, int64_t K, int64_t* __restrict__ ka, int64_t* __restrict__ kb) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -79,185 +41,6 @@ __global__ void k_koff(Group k, int64_t K, int64_t* __restrict__ ka, int64_t* __
     group_off(k, i, &a, &b, &c);
     ka[i] = a;
     kb[i] = b;
-  }
-}
-
-template <typename T> struct Mfma;
-template <> struct Mfma<double> {
-  using V4 = __attribute__((ext_vector_type(4))) double;
-  static __device__ __forceinline__ V4 run(double a, double b, V4 c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
-  // accumulator register r of a lane holds D[4 r + lane / 16][lane % 16]
-  static __device__ __forceinline__ int row(int lane, int r) { return 4 * r + (lane >> 4); }
-};
-template <> struct Mfma<float> {
-  using V4 = __attribute__((ext_vector_type(4))) float;
-  static __device__ __forceinline__ V4 run(float a, float b, V4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
-  // accumulator register r of a lane holds D[4 (lane / 16) + r][lane % 16]
-  static __device__ __forceinline__ int row(int lane, int r) { return 4 * (lane >> 4) + r; }
-};
-
-template <typename T, int V> struct VecOf;
-template <> struct VecOf<double, 1> { using type = double; };
-template <> struct VecOf<float, 1> { using type = float; };
-template <> struct VecOf<double, 2> { using type = __attribute__((ext_vector_type(2))) double; };
-template <> struct VecOf<float, 4> { using type = __attribute__((ext_vector_type(4))) float; };
-
-// Block tile BM x BN = (WGM * TM * 16) x (WGN * TN * 16): the 4 wavefronts form a
-// WGM x WGN grid and each owns TM x TN MFMA tiles.  p.a_kc / p.b_kc: the lanes
-// that stage an operand tile run along k (the operand's innermost K dim is the
-// contiguous one) or along m / n.  VA / VB: elements per global load (16-byte
-// vectors when the host has checked contiguity and alignment, else 1).
-template <typename T, int WGM, int WGN, int TM, int TN, int VA, int VB>
-__global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
-                                             const int64_t* __restrict__ koffA, const int64_t* __restrict__ koffB) {
-  using V4 = typename Mfma<T>::V4;
-  using VecA = typename VecOf<T, VA>::type;
-  using VecB = typename VecOf<T, VB>::type;
-  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
-  constexpr int NA = BM * BK / NT / VA, NB = BN * BK / NT / VB;   // loads each thread issues per K-step
-  static_assert(WGM * WGN == 4 && NA >= 1 && NB >= 1, "tile shape");
-  __shared__ T As[BK][BM + 1];
-  __shared__ T Bs[BK][BN + 1];
-
-  const int t = threadIdx.x;
-  const int lane = t & 63, wave = t >> 6;
-  const int wm = wave / WGN, wn = wave % WGN;
-
-  // XCD-aware tile numbering: blocks b, b+8, b+16, ... share an XCD; give each
-  // XCD a contiguous range of tiles.
-  const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-  const int64_t ntiles = tiles_m * tiles_n;
-  int64_t bid = blockIdx.x;
-  if (ntiles >= 64 && (ntiles & 7) == 0) bid = (bid & 7) * (ntiles >> 3) + (bid >> 3);
-  const int64_t tile_m = bid / tiles_n, tile_n = bid - tile_m * tiles_n;
-  const int64_t m0 = tile_m * BM, n0 = tile_n * BN;
-
-  int64_t bta, btb, btc;
-  group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
-  const int s = blockIdx.y;
-  const int64_t kbeg = (int64_t)s * p.kchunk;
-  int64_t kend = kbeg + p.kchunk;
-  if (kend > p.K) kend = p.K;
-
-  // this thread's (row, k) slots of each operand tile; a slot covers VA (VB)
-  // consecutive elements along the direction the lanes run
-  int aml[NA], akl[NA], bnl[NB], bkl[NB];
-  int64_t aoff[NA], boff[NB];
-  bool aok[NA], bok[NB];
-  const int adk = p.a_kc ? 1 : 0, adm = 1 - adk, bdk = p.b_kc ? 1 : 0, bdn = 1 - bdk;
-#pragma unroll
-  for (int i = 0; i < NA; ++i) {
-    if (p.a_kc) { constexpr int KL = BK / VA; aml[i] = t / KL + (NT / KL) * i; akl[i] = (t % KL) * VA; }
-    else { constexpr int ML = BM / VA; aml[i] = (t % ML) * VA; akl[i] = t / ML + (NT / ML) * i; }
-    int64_t m = m0 + aml[i];
-    aok[i] = m < p.M;
-    if (p.a_kc || i == 0) {
-      int64_t oa = 0, ob = 0, oc = 0;
-      if (aok[i]) group_off(p.m, m, &oa, &ob, &oc);
-      aoff[i] = oa + bta;
-    } else {
-      aoff[i] = aoff[0];
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < NB; ++i) {
-    if (p.b_kc) { constexpr int KL = BK / VB; bnl[i] = t / KL + (NT / KL) * i; bkl[i] = (t % KL) * VB; }
-    else { constexpr int NL = BN / VB; bnl[i] = (t % NL) * VB; bkl[i] = t / NL + (NT / NL) * i; }
-    int64_t n = n0 + bnl[i];
-    bok[i] = n < p.N;
-    if (p.b_kc || i == 0) {
-      int64_t oa = 0, ob = 0, oc = 0;
-      if (bok[i]) group_off(p.n, n, &oa, &ob, &oc);
-      boff[i] = ob + btb;
-    } else {
-      boff[i] = boff[0];
-    }
-  }
-
-  V4 acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = V4{0, 0, 0, 0};
-
-  VecA ra[NA];
-  VecB rb[NB];
-  auto load_tile = [&](int64_t k0) {
-#pragma unroll
-    for (int i = 0; i < NA; ++i) {
-      int64_t ka = k0 + akl[i];
-      if (aok[i] && ka < kend) ra[i] = *reinterpret_cast<const VecA*>(A + aoff[i] + koffA[ka]);
-      else ra[i] = VecA{};
-    }
-#pragma unroll
-    for (int i = 0; i < NB; ++i) {
-      int64_t kb = k0 + bkl[i];
-      if (bok[i] && kb < kend) rb[i] = *reinterpret_cast<const VecB*>(B + boff[i] + koffB[kb]);
-      else rb[i] = VecB{};
-    }
-  };
-
-  if (kbeg < kend) load_tile(kbeg);
-  for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
-#pragma unroll
-    for (int i = 0; i < NA; ++i) {
-      if constexpr (VA == 1) As[akl[i]][aml[i]] = ra[i];
-      else {
-#pragma unroll
-        for (int j = 0; j < VA; ++j) As[akl[i] + j * adk][aml[i] + j * adm] = ra[i][j];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < NB; ++i) {
-      if constexpr (VB == 1) Bs[bkl[i]][bnl[i]] = rb[i];
-      else {
-#pragma unroll
-        for (int j = 0; j < VB; ++j) Bs[bkl[i] + j * bdk][bnl[i] + j * bdn] = rb[i][j];
-      }
-    }
-    __syncthreads();
-    if (k0 + BK < kend) load_tile(k0 + BK);
-#pragma unroll
-    for (int kk = 0; kk < BK; kk += 4) {
-      const int kr = kk + (lane >> 4);
-      T fa[TM], fb[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) fa[i] = As[kr][(wm * TM + i) * 16 + (lane & 15)];
-#pragma unroll
-      for (int j = 0; j < TN; ++j) fb[j] = Bs[kr][(wn * TN + j) * 16 + (lane & 15)];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
-    }
-    __syncthreads();
-  }
-
-  // each lane holds 4 rows of one column of every 16x16 tile (Mfma<T>::row)
-  T* Cout = C + btc + (int64_t)s * p.c_split_stride;
-  int64_t coln[TN];
-  bool colok[TN];
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    int64_t n = n0 + (wn * TN + j) * 16 + (lane & 15);
-    colok[j] = n < p.N;
-    int64_t oa = 0, ob = 0, oc = 0;
-    if (colok[j]) group_off(p.n, n, &oa, &ob, &oc);
-    coln[j] = oc;
-  }
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      int64_t m = m0 + (wm * TM + i) * 16 + Mfma<T>::row(lane, r);
-      if (m < p.M) {
-        int64_t oa, ob, oc;
-        group_off(p.m, m, &oa, &ob, &oc);
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          if (colok[j]) Cout[oc + coln[j]] = acc[i][j][r];
-      }
-    }
   }
 }
 
@@ -325,53 +108,6 @@ int64_t total(const Group& g) {
   return n;
 }
 
-struct TileCfg { int wgm, wgn, tm, tn; double eff; };
-// Candidate tiles, with a rough relative efficiency (operand reuse from LDS).
-const TileCfg kTiles[] = {
-    {2, 2, 4, 4, 1.00},  // 128 x 128
-    {2, 2, 4, 2, 0.85},  // 128 x 64
-    {2, 2, 2, 4, 0.85},  // 64 x 128
-    {4, 1, 4, 2, 0.70},  // 256 x 32
-    {1, 4, 2, 4, 0.70},  // 32 x 256
-    {4, 1, 4, 1, 0.50},  // 256 x 16
-    {1, 4, 1, 4, 0.50},  // 16 x 256
-    {2, 2, 2, 2, 0.65},  // 64 x 64
-    {2, 2, 1, 1, 0.35},  // 32 x 32
-    {4, 1, 1, 1, 0.30},  // 64 x 16
-    {1, 4, 1, 1, 0.30},  // 16 x 64
-};
-constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
-
-template <typename T, int WGM, int WGN, int TM, int TN>
-void launch_cfg(hgpu_ctx* ctx, const GemmParams& p, bool va, bool vb, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
-  constexpr int V = 16 / sizeof(T);
-  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
-  // 16-byte loads only for tiles whose rows are long enough to share a load's lanes sensibly
-  if constexpr (BM >= 64 && BN >= 64) {
-    if (va && vb) { hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, V, V>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb); return; }
-    if (va) { hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, V, 1>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb); return; }
-    if (vb) { hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, 1, V>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb); return; }
-  }
-  hipLaunchKernelGGL((k_gemm<T, WGM, WGN, TM, TN, 1, 1>), grid, dim3(NT), 0, ctx->stream, p, A, B, C, ka, kb);
-}
-
-template <typename T>
-void launch(hgpu_ctx* ctx, int cfg, const GemmParams& p, bool va, bool vb, dim3 grid, const T* A, const T* B, T* C, const int64_t* ka, const int64_t* kb) {
-  switch (cfg) {
-    case 0: launch_cfg<T, 2, 2, 4, 4>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    case 1: launch_cfg<T, 2, 2, 4, 2>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    case 2: launch_cfg<T, 2, 2, 2, 4>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    case 3: launch_cfg<T, 4, 1, 4, 2>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    case 4: launch_cfg<T, 1, 4, 2, 4>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    case 5: launch_cfg<T, 4, 1, 4, 1>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    case 6: launch_cfg<T, 1, 4, 1, 4>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    case 7: launch_cfg<T, 2, 2, 2, 2>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    case 8: launch_cfg<T, 2, 2, 1, 1>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    case 9: launch_cfg<T, 4, 1, 1, 1>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-    default: launch_cfg<T, 1, 4, 1, 1>(ctx, p, va, vb, grid, A, B, C, ka, kb); break;
-  }
-}
-
 // True when 16-byte loads along the direction the staging lanes run are safe
 // for one operand: unit stride and an extent that is a multiple of the vector
 // there, every other stride and the base address a multiple of the vector.
@@ -387,7 +123,6 @@ bool vector_ok(const void* base, size_t es, const Group& run, int run_dim, const
       if (other_st[g][i] % v != 0) return false;
   return true;
 }
-
 }  // namespace
 
 namespace hg {
@@ -534,15 +269,18 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
       label = ctx->label_pool.insert(buf).first->c_str();
     }
     LaunchGuard lg(ctx, label, bytes, flops);
-    hipLaunchKernelGGL(k_koff, dim3((unsigned)((p.K + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, ka, kb);
+    if (p.k.nd > 1) hipLaunchKernelGGL(k_koff, dim3((unsigned)((p.K + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, ka, kb);
+    else ka = kb = nullptr;    // single K dim: offsets are k * stride
     if (a->dtype == HGPU_F64) {
       double* cdst = split > 1 ? (double*)part->ptr : (double*)data_ptr(out);
-      launch<double>(ctx, cfg, p, va, vb, grid, (const double*)data_ptr(a), (const double*)data_ptr(b), cdst, ka, kb);
+      LaunchArgs la{ctx->stream, cfg, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
+      launch_f64(p, la);
       if (split > 1)
         hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
     } else {
       float* cdst = split > 1 ? (float*)part->ptr : (float*)data_ptr(out);
-      launch<float>(ctx, cfg, p, va, vb, grid, (const float*)data_ptr(a), (const float*)data_ptr(b), cdst, ka, kb);
+      LaunchArgs la{ctx->stream, cfg, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
+      launch_f32(p, la);
       if (split > 1)
         hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
     }

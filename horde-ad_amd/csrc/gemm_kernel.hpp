@@ -1,0 +1,369 @@
+// The MFMA kernel behind hgpu_contract's matrix-product path, shared by the
+// per-precision translation units (gemm_f32.hip, gemm_f64.hip).
+//
+// Operands are addressed through separable offset maps,
+//     A[m, k] = A0 + offAm(m) + offAk(k),   B[n, k] = B0 + offBn(n) + offBk(k),
+//     C[m, n] = C0 + offCm(m) + offCn(n),
+// with m, n, k linear indices into merged dim groups (Group).  The K offsets
+// come from two tables written by k_koff (or, for a single K dim, from a
+// multiplication); row offsets are decomposed once per thread.
+//
+// 256 threads = 4 wavefronts in a WGM x WGN grid; block tile BM x BN with
+// K-step 16.  Operand tiles go global -> registers -> LDS ([k][row] order, one
+// element of padding per k-row); the global loads of step t+1 are in flight
+// while the MFMAs of step t run, and with two LDS buffers a step needs a single
+// barrier.  Lanes staging an operand run along whichever of row / k is
+// contiguous in memory (run-time choice per operand), with 16-byte loads when
+// the host has checked contiguity and alignment.
+#pragma once
+#include "common.hpp"
+
+namespace hg {
+namespace gemm {
+
+constexpr int BK = 16, NT = 256;
+constexpr int GD = 5;  // dims per index group after merging
+
+struct Group {
+  int nd;
+  int64_t shape[GD];
+  int64_t sa[GD], sb[GD], sc[GD];
+};
+
+struct GemmParams {
+  Group m, n, k, bt;
+  int64_t M, N, K, BT;
+  int a_kc, b_kc;     // lanes staging A (B) run along k (1) or along m (n) (0)
+  int split;          // K chunks
+  int64_t kchunk;     // K elements per chunk (multiple of BK)
+  int64_t c_split_stride;  // elements between partial outputs
+};
+
+__device__ __forceinline__ void group_off(const Group& g, int64_t lin, int64_t* oa, int64_t* ob, int64_t* oc) {
+  int64_t a = 0, b = 0, c = 0;
+  int64_t r = lin;
+  for (int i = g.nd - 1; i >= 0; --i) {
+    int64_t idx;
+    if (i > 0) {
+      int64_t q = r / g.shape[i];
+      idx = r - q * g.shape[i];
+      r = q;
+    } else {
+      idx = r;
+    }
+    a += idx * g.sa[i];
+    b += idx * g.sb[i];
+    c += idx * g.sc[i];
+  }
+  *oa = a;
+  *ob = b;
+  *oc = c;
+}
+
+// MFMA flavours.  A fragment: lane l supplies A[row = l % 16][k = l / 16].
+// B fragment: lane l supplies B[k = l / 16][col = bcol(l)].  Accumulator
+// register r of lane l holds D[row(l, r)][col(l)] of an (16 x NBW) block.
+struct MfmaF32 {
+  using T = float;
+  using Acc = __attribute__((ext_vector_type(4))) float;
+  static constexpr int NBW = 16, NR = 4;
+  static __device__ __forceinline__ Acc zero() { return Acc{0, 0, 0, 0}; }
+  static __device__ __forceinline__ Acc run(T a, T b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int bcol(int l) { return l & 15; }
+  static __device__ __forceinline__ int row(int l, int r) { return 4 * (l >> 4) + r; }
+  static __device__ __forceinline__ int col(int l) { return l & 15; }
+  static __device__ __forceinline__ T get(const Acc& c, int r) { return c[r]; }
+};
+struct MfmaF64 {
+  using T = double;
+  using Acc = __attribute__((ext_vector_type(4))) double;
+  static constexpr int NBW = 16, NR = 4;
+  static __device__ __forceinline__ Acc zero() { return Acc{0, 0, 0, 0}; }
+  static __device__ __forceinline__ Acc run(T a, T b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int bcol(int l) { return l & 15; }
+  static __device__ __forceinline__ int row(int l, int r) { return 4 * r + (l >> 4); }
+  static __device__ __forceinline__ int col(int l) { return l & 15; }
+  static __device__ __forceinline__ T get(const Acc& c, int r) { return c[r]; }
+};
+template <typename T, int V> struct VecOf;
+template <> struct VecOf<double, 1> { using type = double; };
+template <> struct VecOf<float, 1> { using type = float; };
+template <> struct VecOf<double, 2> { using type = __attribute__((ext_vector_type(2))) double; };
+template <> struct VecOf<float, 4> { using type = __attribute__((ext_vector_type(4))) float; };
+
+// K offset of linear index k for one operand: a product when the K group is a
+// single dim, else a table lookup.
+struct KOff {
+  const int64_t* __restrict__ tab;
+  int64_t stride;   // used when tab == nullptr
+  __device__ __forceinline__ int64_t at(int64_t k) const { return tab ? tab[k] : k * stride; }
+};
+
+// Stages one operand tile (R rows x BK) from global memory into LDS.  A slot is
+// V consecutive elements along the direction the lanes run.  K offsets that
+// have to be fetched per lane are fetched one K-step ahead of their use, so a
+// tile's loads never wait on a table lookup.
+template <typename T, int R, int V>
+struct Stager {
+  static constexpr int NL = R * BK / NT / V;
+  static_assert(NL >= 1, "tile too small for 256 threads");
+  using Vec = typename VecOf<T, V>::type;
+  static constexpr int ML = R / V;        // lanes per k-row when running along rows
+  static constexpr int KL = BK / V;       // lanes per row when running along k
+  static constexpr bool kUniformK = (ML % 64 == 0);   // along rows: a wavefront shares one k
+  static constexpr int NKV = kUniformK ? 1 : NL;
+
+  int rl[NL], kl[NL];
+  const T* rowp[NL];
+  Vec reg[NL];
+  int kc;
+  int64_t kv[NKV];    // per-lane K offsets of the next tile to load
+
+  __device__ __forceinline__ void fetch_kv(const KOff& ko, int64_t k0, int64_t K) {
+    if (kc) {
+      int64_t k = k0 + kl[0];
+      kv[0] = ko.at(k < K ? k : K - 1);
+    } else if constexpr (!kUniformK) {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        int64_t k = k0 + kl[i];
+        kv[i] = ko.at(k < K ? k : K - 1);
+      }
+    }
+  }
+
+  // which: 0 = operand A (offsets sa), 1 = operand B (offsets sb)
+  __device__ __forceinline__ void init(int t, int kc_, int which, const T* base, const Group& g, int64_t r0, int64_t rows,
+                                       const KOff& ko, int64_t kbeg, int64_t K) {
+    kc = kc_;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      if (kc) { rl[i] = t / KL + (NT / KL) * i; kl[i] = (t % KL) * V; }
+      else { rl[i] = (t % ML) * V; kl[i] = t / ML + (NT / ML) * i; }
+      if (kc || i == 0) {
+        int64_t r = r0 + rl[i];
+        if (r >= rows) r = rows - (kc ? 1 : V);   // clamp: the values are never stored
+        int64_t oa, ob, oc;
+        group_off(g, r, &oa, &ob, &oc);
+        rowp[i] = base + (which == 0 ? oa : ob);
+      } else {
+        rowp[i] = rowp[0];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NKV; ++i) kv[i] = 0;
+    fetch_kv(ko, kbeg, K);
+  }
+
+  __device__ __forceinline__ void load(int64_t k0, int64_t kend, const KOff& ko, int64_t K) {
+    if (kc) {
+      const bool ok = k0 + kl[0] < kend;
+#pragma unroll
+      for (int i = 0; i < NL; ++i) reg[i] = ok ? *reinterpret_cast<const Vec*>(rowp[i] + kv[0]) : Vec{};
+    } else {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        if constexpr (kUniformK) {
+          int64_t k = k0 + __builtin_amdgcn_readfirstlane(kl[i]);
+          if (k < kend) reg[i] = *reinterpret_cast<const Vec*>(rowp[0] + ko.at(k));
+          else reg[i] = Vec{};
+        } else {
+          reg[i] = (k0 + kl[i] < kend) ? *reinterpret_cast<const Vec*>(rowp[0] + kv[i]) : Vec{};
+        }
+      }
+    }
+    fetch_kv(ko, k0 + BK, K);
+  }
+
+  __device__ __forceinline__ void store(T (*S)[R + 1]) const {
+    const int dk = kc ? 1 : 0, dr = 1 - dk;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      if constexpr (V == 1) S[kl[i]][rl[i]] = reg[i];
+      else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) S[kl[i] + j * dk][rl[i] + j * dr] = reg[i][j];
+      }
+    }
+  }
+};
+
+// Block tile BM x BN = (WGM * TM * 16) x (WGN * TN * 16).  NBUF LDS buffers.
+template <typename X, int WGM, int WGN, int TM, int TN, int VA, int VB, int NBUF>
+__global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const typename X::T* __restrict__ A, const typename X::T* __restrict__ B,
+                                             typename X::T* __restrict__ C, const int64_t* __restrict__ koffA,
+                                             const int64_t* __restrict__ koffB) {
+  using T = typename X::T;
+  using Acc = typename X::Acc;
+  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
+  constexpr int TNB = TN * 16 / X::NBW;     // MFMA blocks per wavefront along n
+  static_assert(WGM * WGN == 4, "four wavefronts");
+  __shared__ T As[NBUF][BK][BM + 1];
+  __shared__ T Bs[NBUF][BK][BN + 1];
+
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  // XCD-aware tile numbering: blocks b, b+8, b+16, ... share an XCD; give each
+  // XCD a contiguous range of tiles.
+  const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int64_t ntiles = tiles_m * tiles_n;
+  int64_t bid = blockIdx.x;
+  if (ntiles >= 64 && (ntiles & 7) == 0) bid = (bid & 7) * (ntiles >> 3) + (bid >> 3);
+  const int64_t tile_m = bid / tiles_n, tile_n = bid - tile_m * tiles_n;
+  const int64_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+  int64_t bta, btb, btc;
+  group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
+  const int s = blockIdx.y;
+  const int64_t kbeg = (int64_t)s * p.kchunk;
+  int64_t kend = kbeg + p.kchunk;
+  if (kend > p.K) kend = p.K;
+
+  Stager<T, BM, VA> sa;
+  Stager<T, BN, VB> sb;
+  const KOff koa{koffA, p.k.sa[0]}, kob{koffB, p.k.sb[0]};
+  sa.init(t, p.a_kc, 0, A + bta, p.m, m0, p.M, koa, kbeg, p.K);
+  sb.init(t, p.b_kc, 1, B + btb, p.n, n0, p.N, kob, kbeg, p.K);
+
+  Acc acc[TM][TNB];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TNB; ++j) acc[i][j] = X::zero();
+
+  if (kbeg < kend) {
+    sa.load(kbeg, kend, koa, p.K);
+    sb.load(kbeg, kend, kob, p.K);
+    sa.store(As[0]);
+    sb.store(Bs[0]);
+  }
+  __syncthreads();
+  int cur = 0;
+  for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
+    const bool more = k0 + BK < kend;
+    if (more) {
+      sa.load(k0 + BK, kend, koa, p.K);
+      sb.load(k0 + BK, kend, kob, p.K);
+    }
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 4) {
+      const int kr = kk + (lane >> 4);
+      T fa[TM], fb[TNB];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[i] = As[cur][kr][(wm * TM + i) * 16 + (lane & 15)];
+#pragma unroll
+      for (int j = 0; j < TNB; ++j) fb[j] = Bs[cur][kr][wn * TN * 16 + j * X::NBW + X::bcol(lane)];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TNB; ++j) acc[i][j] = X::run(fa[i], fb[j], acc[i][j]);
+    }
+    if constexpr (NBUF == 1) __syncthreads();   // every wavefront is done reading the tile
+    const int nxt = NBUF == 2 ? cur ^ 1 : 0;
+    if (more) {
+      sa.store(As[nxt]);
+      sb.store(Bs[nxt]);
+    }
+    __syncthreads();
+    cur = nxt;
+  }
+
+  T* Cout = C + btc + (int64_t)s * p.c_split_stride;
+  int64_t coln[TNB];
+  bool colok[TNB];
+#pragma unroll
+  for (int j = 0; j < TNB; ++j) {
+    int64_t n = n0 + wn * TN * 16 + j * X::NBW + X::col(lane);
+    colok[j] = n < p.N;
+    int64_t oa = 0, ob = 0, oc = 0;
+    if (colok[j]) group_off(p.n, n, &oa, &ob, &oc);
+    coln[j] = oc;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int r = 0; r < X::NR; ++r) {
+      int64_t m = m0 + (wm * TM + i) * 16 + X::row(lane, r);
+      if (m < p.M) {
+        int64_t oa, ob, oc;
+        group_off(p.m, m, &oa, &ob, &oc);
+#pragma unroll
+        for (int j = 0; j < TNB; ++j)
+          if (colok[j]) Cout[oc + coln[j]] = X::get(acc[i][j], r);
+      }
+    }
+  }
+}
+
+struct TileCfg { int wgm, wgn, tm, tn; double eff; };
+// Candidate tiles, with a rough relative efficiency (operand reuse from LDS).
+constexpr TileCfg kTiles[] = {
+    {2, 2, 4, 4, 1.00},  // 128 x 128
+    {2, 2, 4, 2, 0.85},  // 128 x 64
+    {2, 2, 2, 4, 0.85},  // 64 x 128
+    {4, 1, 4, 2, 0.70},  // 256 x 32
+    {1, 4, 2, 4, 0.70},  // 32 x 256
+    {4, 1, 4, 1, 0.50},  // 256 x 16
+    {1, 4, 1, 4, 0.50},  // 16 x 256
+    {2, 2, 2, 2, 0.65},  // 64 x 64
+    {2, 2, 1, 1, 0.35},  // 32 x 32
+    {4, 1, 1, 1, 0.30},  // 64 x 16
+    {1, 4, 1, 1, 0.30},  // 16 x 64
+};
+constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
+
+struct LaunchArgs {
+  hipStream_t stream;
+  int cfg;
+  bool va, vb;
+  dim3 grid;
+  const void *A, *B;
+  void* C;
+  const int64_t *ka, *kb;
+};
+
+template <typename X, int WGM, int WGN, int TM, int TN>
+void launch_cfg(const GemmParams& p, const LaunchArgs& a) {
+  using T = typename X::T;
+  constexpr int V = 16 / sizeof(T);
+  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
+  // two LDS buffers where they still leave room for two blocks per CU next to
+  // the accumulators' registers; skinny tiles keep one buffer and more blocks
+  constexpr int NBUF = (BM >= 64 && BN >= 64 && BM + BN >= 192) ? 2 : 1;
+  const T* A = (const T*)a.A;
+  const T* B = (const T*)a.B;
+  T* C = (T*)a.C;
+  // 16-byte loads only for tiles whose rows are long enough to share a load's lanes sensibly
+  if constexpr (BM >= 64 && BN >= 64) {
+    if (a.va && a.vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, V, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+    if (a.va) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, 1, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+    if (a.vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, V, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+  }
+  hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, 1, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+}
+
+template <typename X>
+void launch(const GemmParams& p, const LaunchArgs& a) {
+  switch (a.cfg) {
+    case 0: launch_cfg<X, 2, 2, 4, 4>(p, a); break;
+    case 1: launch_cfg<X, 2, 2, 4, 2>(p, a); break;
+    case 2: launch_cfg<X, 2, 2, 2, 4>(p, a); break;
+    case 3: launch_cfg<X, 4, 1, 4, 2>(p, a); break;
+    case 4: launch_cfg<X, 1, 4, 2, 4>(p, a); break;
+    case 5: launch_cfg<X, 4, 1, 4, 1>(p, a); break;
+    case 6: launch_cfg<X, 1, 4, 1, 4>(p, a); break;
+    case 7: launch_cfg<X, 2, 2, 2, 2>(p, a); break;
+    case 8: launch_cfg<X, 2, 2, 1, 1>(p, a); break;
+    case 9: launch_cfg<X, 4, 1, 1, 1>(p, a); break;
+    default: launch_cfg<X, 1, 4, 1, 1>(p, a); break;
+  }
+}
+
+// defined in gemm_f32.hip / gemm_f64.hip
+void launch_f32(const GemmParams& p, const LaunchArgs& a);
+void launch_f64(const GemmParams& p, const LaunchArgs& a);
+
+}  // namespace gemm
+}  // namespace hg
