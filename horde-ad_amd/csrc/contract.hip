@@ -243,7 +243,19 @@ __global__ void __launch_bounds__(1024) k_argminmax_block(Dims keep, int64_t L, 
 
 template <typename TI, typename TO>
 int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red_full, int64_t n_out, int64_t R, int S, const void* a, const void* b, void* out) {
-  LaunchGuard lg(ctx, b ? (use_wave ? "contract_dot_wave" : "contract_dot_lane") : (use_wave ? "contract_sum_wave" : "contract_sum_lane"),
+  const char* label = b ? (use_wave ? "contract_dot_wave" : "contract_dot_lane") : (use_wave ? "contract_sum_wave" : "contract_sum_lane");
+  if (ctx->profiling && ctx->profile_shapes) {
+    char buf[160];
+    int n = snprintf(buf, sizeof buf, "%s[out%lld,R%lld,S%d,red", label, (long long)n_out, (long long)R, S);
+    for (int i = 0; i < red_full.nd && n < (int)sizeof buf - 40; ++i)
+      n += snprintf(buf + n, sizeof buf - n, "_%lld:%lld/%lld", (long long)red_full.shape[i], (long long)red_full.st[0][i], (long long)red_full.st[1][i]);
+    n += snprintf(buf + n, sizeof buf - n, ",keep");
+    for (int i = 0; i < keep.nd && n < (int)sizeof buf - 40; ++i)
+      n += snprintf(buf + n, sizeof buf - n, "_%lld:%lld/%lld", (long long)keep.shape[i], (long long)keep.st[0][i], (long long)keep.st[1][i]);
+    snprintf(buf + n, sizeof buf - n, "]");
+    label = ctx->label_pool.insert(buf).first->c_str();
+  }
+  LaunchGuard lg(ctx, label,
                  (double)n_out * R * sizeof(TI) * (b ? 2 : 1) + (double)n_out * S * sizeof(TO), (double)n_out * R * (b ? 2 : 1));
   int maxb = ctx->num_cu * 8;
   if (use_wave) {

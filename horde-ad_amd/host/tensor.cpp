@@ -297,11 +297,40 @@ T lazy_contract(const T& a, const T& b, int n_keep) {
   return T(p);
 }
 
-#define HD_VIEW_OF_PRODUCT(expr_a, expr_b) \
-  if (a.pending_product()) { T a0 = a.factor_a(), b0 = a.factor_b(); return lazy_mul(expr_a, expr_b); }
+// A view of a pending elementwise expression is the expression of the views
+// of its leaves (every operand of an expression has the expression's shape), so
+// transposes, slices and windows between two elementwise stages cost no pass
+// over memory.  Shared sub-expressions stay shared.
+static T map_leaves(const T& a, const std::function<T(const T&)>& view) {
+  std::map<const ArrHolder*, std::shared_ptr<ArrHolder>> memo;
+  std::function<std::shared_ptr<ArrHolder>(const std::shared_ptr<ArrHolder>&)> go =
+      [&](const std::shared_ptr<ArrHolder>& p) -> std::shared_ptr<ArrHolder> {
+    auto it = memo.find(p.get());
+    if (it != memo.end()) return it->second;
+    std::shared_ptr<ArrHolder> r;
+    if (p->h || p->ekind < 0) {
+      r = view(T(p)).holder();
+    } else {
+      r = std::make_shared<ArrHolder>(p->be, nullptr);
+      r->ekind = p->ekind;
+      r->eop = p->eop;
+      r->edtype = p->edtype;
+      r->esize = p->esize;
+      r->fa = go(p->fa);
+      if (p->fb) r->fb = go(p->fb);
+      if (p->fc) r->fc = go(p->fc);
+      r->eshape = T(r->fa).shape();
+    }
+    memo[p.get()] = r;
+    return r;
+  };
+  return T(go(a.holder()));
+}
+#define HD_VIEW_OF_EXPR(call) \
+  if (a.pending_expr()) return map_leaves(a, [&](const T& x) { return call; });
 
 T transpose(const T& a, const std::vector<int>& perm) {
-  HD_VIEW_OF_PRODUCT(transpose(a0, perm), transpose(b0, perm))
+  HD_VIEW_OF_EXPR(transpose(x, perm))
   if (a.pending_contraction() && (int)perm.size() <= a.pending_keep())   // permutes kept dims only
     return lazy_contract(transpose(a.factor_a(), perm), transpose(a.factor_b(), perm), a.pending_keep());
   static const int dummy = 0;
@@ -309,21 +338,21 @@ T transpose(const T& a, const std::vector<int>& perm) {
 }
 T reshape(const T& a, const Shape& s) { HD_OUT(reshape(be__->ctx, a.h(), (int)s.size(), ptr_or_dummy(s), &o__)); }
 T slice(const T& a, int dim, int64_t start, int64_t len) {
-  HD_VIEW_OF_PRODUCT(slice(a0, dim, start, len), slice(b0, dim, start, len))
+  HD_VIEW_OF_EXPR(slice(x, dim, start, len))
   HD_OUT(slice(be__->ctx, a.h(), dim, start, len, &o__));
 }
 T reverse(const T& a, int dim) {
-  HD_VIEW_OF_PRODUCT(reverse(a0, dim), reverse(b0, dim))
+  HD_VIEW_OF_EXPR(reverse(x, dim))
   HD_OUT(reverse(be__->ctx, a.h(), dim, &o__));
 }
 T replicate(const T& a, const Shape& pre) {
   if (pre.empty()) return a;
-  // a pending product is written out before it is replicated: only shrinking
+  // a pending expression is written out before it is replicated: only shrinking
   // or permuting views of it are worth keeping pending
   HD_OUT(replicate(be__->ctx, a.h(), (int)pre.size(), pre.data(), &o__));
 }
 T index_prefix(const T& a, const Shape& ix) {
-  HD_VIEW_OF_PRODUCT(index_prefix(a0, ix), index_prefix(b0, ix))
+  HD_VIEW_OF_EXPR(index_prefix(x, ix))
   HD_OUT(index_prefix(be__->ctx, a.h(), (int)ix.size(), ptr_or_dummy(ix), &o__));
 }
 T as_strided(const T& a, const Shape& shape, const Shape& strides, int64_t offset) {
@@ -688,6 +717,19 @@ T tsgather(const T& src, const Shape& shm, const std::vector<Ix>& ix) {
   check_ix(shm, ix);
   Backend* be = src.be();
   if (all_affine(ix)) {
+    // windows of a pending expression that stay in bounds and do not multiply
+    // its elements are taken of its leaves instead
+    if (src.pending_expr()) {
+      Shape ssh = src.shape();
+      int64_t n_out = prod(shm) * prod(ssh, ix.size());
+      bool inside = n_out <= src.size();
+      for (size_t j = 0; j < ix.size() && inside; ++j) {
+        int64_t lo, hi;
+        affine_range(ix[j], &lo, &hi);
+        inside = lo >= 0 && hi <= ssh[j] - 1;
+      }
+      if (inside && n_out > 0) return map_leaves(src, [&](const T& x) { return affine_view(x, shm, ix); });
+    }
     T v = affine_view(src, shm, ix);
     if (v.valid()) return v;
   }
