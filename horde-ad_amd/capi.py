@@ -48,6 +48,7 @@ SIGNATURES = {
     "iota": (I, [P, L, I, PP]), "concat": (I, [P, I, PP, PP]),
     "gather": (I, [P, P, I, PP, I, LP, PP]), "scatter_add": (I, [P, P, I, PP, I, LP, I, PP]),
     "onehot": (I, [P, P, I, LP, LP, PP]), "get_api": (P, []),
+    "scatter_affine": (I, [P, P, I, I, LP, LP, LP, PP]),
 }
 # exported by the GPU library only
 GPU_ONLY = {
@@ -162,6 +163,11 @@ class Ctx:
     def gather(self, src, ix, shm):
         arr = (C.c_void_p * max(len(ix), 1))(*[p.h for p in ix])
         return self._out(self.lib.gather, src.h, len(ix), arr, len(shm), _larr(shm))
+
+    def scatter_affine(self, src, rank_m, c0, coef, shp):
+        """coef[d][j]: coefficient of position variable d in index component j."""
+        flat = [int(v) for row in coef for v in row]
+        return self._out(self.lib.scatter_affine, src.h, rank_m, len(shp), _larr(c0), _larr(flat), _larr(shp))
 
     def scatter_add(self, src, ix, rank_m, shp, flags=0):
         arr = (C.c_void_p * max(len(ix), 1))(*[p.h for p in ix])

@@ -10,7 +10,7 @@ extern "C" const hgpu_api* hgpu_get_api(void) {
       hgpu_reverse,     hgpu_replicate, hgpu_index_prefix, hgpu_as_strided, hgpu_materialize, hgpu_pad,
       hgpu_ewise1,      hgpu_ewise2,    hgpu_compare,     hgpu_compare_all, hgpu_select,     hgpu_convert,
       hgpu_contract,    hgpu_argminmax_last, hgpu_iota,   hgpu_concat,     hgpu_gather,      hgpu_scatter_add,
-      hgpu_onehot,      hgpu_fused_map,
+      hgpu_onehot,      hgpu_fused_map, hgpu_scatter_affine,
   };
   return &api;
 }

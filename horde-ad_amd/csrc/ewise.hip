@@ -327,6 +327,71 @@ int hgpu_pad(hgpu_ctx* ctx, const hgpu_array* a, const int64_t* lo, const int64_
   return HGPU_OK;
 }
 
+int hgpu_scatter_affine(hgpu_ctx* ctx, const hgpu_array* src, int rank_m, int n_ix, const int64_t* c0, const int64_t* coef,
+                        const int64_t* shp, hgpu_array** out) {
+  if (!ctx || !src || !out || (n_ix > 0 && (!c0 || !shp)) || (n_ix > 0 && rank_m > 0 && !coef)) return HGPU_ERR_INVALID;
+  if (rank_m < 0 || rank_m > src->rank || n_ix < 0) return fail(ctx, HGPU_ERR_INVALID, "scatter_affine: bad ranks");
+  const int rank_n = src->rank - rank_m, rank_o = n_ix + rank_n;
+  if (rank_o > HGPU_MAX_RANK) return fail(ctx, HGPU_ERR_INVALID, "scatter_affine: result rank too large");
+  int64_t osh[HGPU_MAX_RANK];
+  for (int j = 0; j < n_ix; ++j) osh[j] = shp[j];
+  for (int i = 0; i < rank_n; ++i) osh[n_ix + i] = src->shape[rank_m + i];
+  const int64_t n_src = nelem(src);
+  int64_t n_out = 1;
+  for (int i = 0; i < rank_o; ++i) n_out *= osh[i];
+  if (n_src > 0) {
+    for (int j = 0; j < n_ix; ++j) {   // range of every component over the box of positions
+      int64_t lo = c0[j], hi = c0[j];
+      for (int d = 0; d < rank_m; ++d) {
+        int64_t span = coef[d * n_ix + j] * (src->shape[d] - 1);
+        if (span > 0) hi += span; else lo += span;
+      }
+      if (lo < 0 || hi > shp[j] - 1) return fail(ctx, HGPU_ERR_INVALID, "scatter_affine: a position leaves the bounds");
+    }
+  }
+  // The result keeps src's order of dims in memory: an output dim is as
+  // contiguous as the most contiguous source dim that moves it.
+  int64_t key[HGPU_MAX_RANK];
+  auto mag = [](int64_t v) { return v < 0 ? -v : v; };
+  for (int j = 0; j < n_ix; ++j) {
+    key[j] = INT64_MAX;
+    for (int d = 0; d < rank_m; ++d)
+      if (coef[d * n_ix + j] != 0 && src->shape[d] > 1 && src->strides[d] != 0 && mag(src->strides[d]) < key[j]) key[j] = mag(src->strides[d]);
+  }
+  for (int i = 0; i < rank_n; ++i) {
+    int d = rank_m + i;
+    key[n_ix + i] = (src->shape[d] > 1 && src->strides[d] != 0) ? mag(src->strides[d]) : INT64_MAX;
+  }
+  int order[HGPU_MAX_RANK];
+  for (int i = 0; i < rank_o; ++i) order[i] = i;
+  for (int i = 1; i < rank_o; ++i)   // stable insertion sort, largest key first
+    for (int j = i; j > 0 && key[order[j]] > key[order[j - 1]]; --j) { int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t; }
+  int64_t psh[HGPU_MAX_RANK];
+  for (int i = 0; i < rank_o; ++i) psh[i] = osh[order[i]];
+  hgpu_array* phys = nullptr;
+  // distinct positions fill distinct places: with as many positions as places nothing stays zero
+  int rc = (n_src == n_out) ? new_dense(ctx, src->dtype, rank_o, psh, &phys) : new_zeros(ctx, src->dtype, rank_o, psh, &phys);
+  if (rc) return rc;
+  int64_t st[HGPU_MAX_RANK];
+  for (int i = 0; i < rank_o; ++i) st[order[i]] = phys->strides[i];
+  hgpu_array* o = new_view(ctx, phys->buf, src->dtype, rank_o, osh, st, 0);
+  hgpu_release(phys);
+  if (n_src > 0) {
+    int64_t off = 0, ds[HGPU_MAX_RANK];
+    for (int j = 0; j < n_ix; ++j) off += c0[j] * st[j];
+    for (int d = 0; d < rank_m; ++d) {
+      ds[d] = 0;
+      for (int j = 0; j < n_ix; ++j) ds[d] += coef[d * n_ix + j] * st[j];
+    }
+    for (int i = 0; i < rank_n; ++i) ds[rank_m + i] = st[n_ix + i];
+    rc = copy_view(ctx, src->dtype, src->rank, src->shape, data_ptr(src), src->strides,
+                   (char*)data_ptr(o) + off * (int64_t)dtype_size(src->dtype), ds);
+    if (rc) { hgpu_release(o); return rc; }
+  }
+  *out = o;
+  return HGPU_OK;
+}
+
 int hgpu_ewise1(hgpu_ctx* ctx, int op, const hgpu_array* a, hgpu_array** out) {
   if (!ctx || !a || !out) return HGPU_ERR_INVALID;
   if (op < 0 || op >= HGPU_OP1_COUNT) return fail(ctx, HGPU_ERR_INVALID, "ewise1: unknown opcode %d", op);

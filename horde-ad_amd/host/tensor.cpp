@@ -924,6 +924,26 @@ T tsscatter(const T& src, int rank_m, const Shape& shp, const std::vector<Ix>& i
     T r = scatter_as_contraction(src, rank_m, shp, ix);
     if (r.valid()) return r;
   }
+  if (injective && all_affine(ix) && src.size() > 0 &&
+      be->api->struct_size >= offsetof(hgpu_api, scatter_affine) + sizeof(be->api->scatter_affine) && be->api->scatter_affine) {
+    // no index arrays: the places are computed from the positions
+    bool inside = true;
+    for (size_t j = 0; j < ix.size() && inside; ++j) {
+      int64_t lo, hi;
+      affine_range(ix[j], &lo, &hi);
+      inside = lo >= 0 && hi <= shp[j] - 1;
+    }
+    if (inside) {
+      std::vector<int64_t> c0(ix.size() + 1, 0), coef((size_t)rank_m * ix.size() + 1, 0);
+      for (size_t j = 0; j < ix.size(); ++j) {
+        c0[j] = ix[j].c0;
+        for (size_t d = 0; d < (size_t)rank_m; ++d) coef[d * ix.size() + j] = ix[j].coef[d];
+      }
+      hgpu_array* o = nullptr;
+      be->check(be->api->scatter_affine(be->ctx, src.h(), rank_m, (int)ix.size(), c0.data(), coef.data(), ptr_or_dummy(shp), &o));
+      return T(be, o);
+    }
+  }
   std::vector<T> arrs;
   for (auto& x : ix) arrs.push_back(ix_array(be, x));
   return scatter_raw(src, arrs, rank_m, shp, injective ? 1 : 0);

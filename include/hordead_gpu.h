@@ -256,6 +256,18 @@ int hgpu_gather(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array
  * positions map to distinct destinations (plain stores suffice). */
 int hgpu_scatter_add(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array* const* ix,
                      int rank_m, const int64_t* shp, int flags, hgpu_array** out);
+/* tsscatter (OpsConcrete.hs:1581-1619) for an index function that is AFFINE in
+ * the positions and sends distinct positions to distinct places (the caller's
+ * promise; a violation leaves one of the colliding values, it corrupts
+ * nothing):
+ *   out = 0;  out[c0[0] + sum_d coef[d*n_ix+0]*m_d, ..., n..] = src[m.., n..]
+ * for all positions m of src's first rank_m dims; out has shape shp ++ shn.
+ * Every position must land inside shp (else HGPU_ERR_INVALID: use
+ * hgpu_scatter_add, which skips them).  No index arrays are read; the result
+ * keeps src's order of dims in memory and may be a transposed view.  Pure data
+ * movement: bit-exact. */
+int hgpu_scatter_affine(hgpu_ctx* ctx, const hgpu_array* src, int rank_m, int n_ix, const int64_t* c0,
+                        const int64_t* coef, const int64_t* shp, hgpu_array** out);
 /* tsoneHot / toneHotS (OpsConcrete.hs:1516-1525): zeros of shape shp ++ shape(v)
  * with v written at prefix index ix; all zeros when ix is out of bounds. */
 int hgpu_onehot(hgpu_ctx* ctx, const hgpu_array* v, int n, const int64_t* ix, const int64_t* shp, hgpu_array** out);
@@ -306,6 +318,7 @@ typedef struct hgpu_api {
   int (*onehot)(hgpu_ctx*, const hgpu_array*, int, const int64_t*, const int64_t*, hgpu_array**);
   /* optional (may be NULL): a provider without it gets the operations one by one */
   int (*fused_map)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, const int*, hgpu_array**);
+  int (*scatter_affine)(hgpu_ctx*, const hgpu_array*, int, int, const int64_t*, const int64_t*, const int64_t*, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

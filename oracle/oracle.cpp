@@ -607,6 +607,42 @@ int horc_scatter_add(hgpu_ctx* c, const hgpu_array* src, int n_ix, const hgpu_ar
   return HGPU_OK;
 }
 
+// tscatterZSScalar (OpsConcrete.hs:1581-1619) with the index function given as
+// an affine form: the same loop, the index computed instead of read.
+int horc_scatter_affine(hgpu_ctx* c, const hgpu_array* src, int rank_m, int n_ix, const int64_t* c0, const int64_t* coef,
+                        const int64_t* shp, hgpu_array** out) {
+  int rank = (int)src->shape.size();
+  if (rank_m < 0 || rank_m > rank || n_ix < 0) return fail(c, HGPU_ERR_INVALID, "scatter_affine: bad ranks");
+  std::vector<int64_t> shm(src->shape.begin(), src->shape.begin() + rank_m);
+  std::vector<int64_t> osh(shp, shp + n_ix);
+  osh.insert(osh.end(), src->shape.begin() + rank_m, src->shape.end());
+  if ((int)osh.size() > HGPU_MAX_RANK) return fail(c, HGPU_ERR_INVALID, "scatter_affine: result rank too large");
+  int64_t M = prod(shm), N = prod(src->shape, rank_m);
+  std::vector<int64_t> lins((size_t)M);
+  std::vector<int64_t> idx((size_t)rank_m, 0);
+  for (int64_t m = 0; m < M; ++m) {
+    int64_t lin = 0;
+    for (int k = 0; k < n_ix; ++k) {
+      int64_t i = c0[k];
+      for (int d = 0; d < rank_m; ++d) i += coef[d * n_ix + k] * idx[(size_t)d];
+      if (!(0 <= i && i < shp[k])) return fail(c, HGPU_ERR_INVALID, "scatter_affine: a position leaves the bounds");
+      lin = lin * shp[k] + i;
+    }
+    lins[(size_t)m] = lin;
+    for (int d = rank_m - 1; d >= 0; --d) {
+      if (++idx[(size_t)d] < shm[(size_t)d]) break;
+      idx[(size_t)d] = 0;
+    }
+  }
+  hgpu_array* o = make(c, src->dtype, osh);
+  DISPATCH(src->dtype, T, {
+    for (int64_t m = 0; m < M; ++m)
+      for (int64_t n = 0; n < N; ++n) ptr<T>(o)[lins[(size_t)m] * N + n] = ptr<T>(src)[m * N + n];
+  });
+  *out = o;
+  return HGPU_OK;
+}
+
 // toneHotS (OpsConcrete.hs:1516-1525)
 int horc_onehot(hgpu_ctx* c, const hgpu_array* v, int n, const int64_t* ix, const int64_t* shp, hgpu_array** out) {
   if (n < 0 || n + (int)v->shape.size() > HGPU_MAX_RANK) return fail(c, HGPU_ERR_INVALID, "onehot: rank too large");
@@ -671,7 +707,7 @@ const hgpu_api* horc_get_api(void) {
       horc_reverse,     horc_replicate, horc_index_prefix, horc_as_strided, horc_materialize, horc_pad,
       horc_ewise1,      horc_ewise2,    horc_compare,      horc_compare_all, horc_select,     horc_convert,
       horc_contract,    horc_argminmax_last, horc_iota,    horc_concat,     horc_gather,      horc_scatter_add,
-      horc_onehot,      horc_fused_map,
+      horc_onehot,      horc_fused_map, horc_scatter_affine,
   };
   return &api;
 }

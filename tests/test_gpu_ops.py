@@ -293,6 +293,24 @@ def test_scatter(both, dt):
     assert_same(both.scatter_add(src, [perm], 1, [500], flags=1))
 
 
+@pytest.mark.parametrize("dt", [np.float64, np.float32, np.int64, np.int8, np.bool_])
+def test_scatter_affine(both, dt):
+    # pooling windows over a transposed source: a bijection, nothing stays zero
+    src = both.upload(rnd((5, 3, 4, 2, 6, 2), dt)).transpose([2, 3, 4, 5, 0, 1])
+    assert_same(both.scatter_affine(src, 4, [0, 0], [[2, 0], [1, 0], [0, 2], [0, 1]], [8, 12]))
+    # offsets, negative and skewed coefficients, zeros left in place
+    src = random_view(both, dt, rank=3)
+    s = src.shape
+    c0 = [3 * (s[0] - 1) + 1, 2]
+    coef = [[-3, 0], [0, s[2] + 1], [0, 1]]
+    shp = [c0[0] + 2, 2 + (s[1] - 1) * (s[2] + 1) + s[2] + 1]
+    assert_same(both.scatter_affine(src, 3, c0, coef, shp), 0.0, (s, c0, coef, shp))
+    # trailing dims carried along, rank-0 position space
+    src = both.upload(rnd((4, 7), dt))
+    assert_same(both.scatter_affine(src, 1, [1], [[2]], [9]))
+    assert_same(both.scatter_affine(src, 0, [2], [], [5]))
+
+
 def test_scatter_small_ints(both, gpu):
     perm = both.upload(RNG.permutation(64).astype(np.int64))
     for dt in (np.int16, np.int8):

@@ -241,6 +241,28 @@ def test_gather_scatter_bruteforce(oracle):
     assert np.array_equal(s, want)
 
 
+def test_scatter_affine_bruteforce(oracle):
+    """The affine form agrees with the brute-force scatter fed the same indices as arrays."""
+    # pooling windows: (i, p, j, q, n) -> (2 i + p, 2 j + q), a bijection
+    src = rnd((3, 2, 4, 2, 5), np.float64)
+    c0, coef, shp = [0, 0], [[2, 0], [1, 0], [0, 2], [0, 1]], (6, 8)
+    got = oracle.scatter_affine(oracle.upload(src), 4, c0, coef, shp).numpy()
+    grid = np.indices(src.shape[:4])
+    ix = [c0[j] + sum(coef[d][j] * grid[d] for d in range(4)) for j in range(2)]
+    assert np.array_equal(got, brute_scatter(src, ix, 4, shp))
+    # offsets, a negative coefficient, and places that stay zero
+    src = rnd((4, 3), np.int32)
+    c0, coef, shp = [9, 1], [[-2, 0], [0, 3]], (11, 9)
+    got = oracle.scatter_affine(oracle.upload(src), 2, c0, coef, shp).numpy()
+    grid = np.indices(src.shape)
+    ix = [c0[j] + sum(coef[d][j] * grid[d] for d in range(2)) for j in range(2)]
+    assert np.array_equal(got, brute_scatter(src, ix, 2, shp))
+    assert np.count_nonzero(got) <= src.size
+    # a position outside the bounds is an error, not a skipped position
+    with pytest.raises(capi.HgpuError):
+        oracle.scatter_affine(oracle.upload(src), 2, [9, 1], coef, (9, 9))
+
+
 def test_gather_scatter_adjoint(oracle):
     """<gather x f, y> == <x, scatter y f> (bench/ConvVjpBench.hs:564-584)."""
     x, shm = rnd((7, 6, 2), np.float64), (5, 3)
