@@ -58,6 +58,7 @@ struct hgpu_ctx {
   bool profile_shapes = false;           // hgpu_profile_enable(ctx, 2): labels carry the problem shape
   std::set<std::string> label_pool;
   std::vector<ProfRec> prof;
+  hgpu_buffer* zero_block = nullptr;     // 256 zero bytes, for kernels that want a dummy table
 };
 
 namespace hg {
@@ -79,6 +80,7 @@ int check_hip(hgpu_ctx* ctx, hipError_t e, const char* what);
 
 // Allocator (runtime.hip).
 int buffer_alloc(hgpu_ctx* ctx, size_t bytes, hgpu_buffer** out);
+int zero_block(hgpu_ctx* ctx, const void** out);   // a context-lifetime block of 256 zero bytes
 void buffer_retain(hgpu_buffer* b);
 void buffer_release(hgpu_buffer* b);
 

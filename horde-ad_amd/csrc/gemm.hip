@@ -34,11 +34,19 @@ using namespace hg::gemm;
 
 namespace {
 
-__global__ void k_koff(Group k, int64_t K, int64_t* __restrict__ ka, int64_t* __restrict__ kb) {
+// K offset tables of both operands, Kp >= K entries: entries past K repeat the
+// last four valid k (so that a 4-element vector load at a padded entry stays
+// inside the operand).
+__global__ void k_koff(Group k, int64_t K, int64_t Kp, int64_t* __restrict__ ka, int64_t* __restrict__ kb) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < K) {
+  if (i < Kp) {
+    int64_t idx = i;
+    if (i >= K) {
+      idx = K >= 4 ? K - 4 + (i & 3) : K - 1;
+      if (idx > K - 1) idx = K - 1;
+    }
     int64_t a, b, c;
-    group_off(k, i, &a, &b, &c);
+    group_off(k, idx, &a, &b, &c);
     ka[i] = a;
     kb[i] = b;
   }
@@ -123,6 +131,104 @@ bool vector_ok(const void* base, size_t es, const Group& run, int run_dim, const
       if (other_st[g][i] % v != 0) return false;
   return true;
 }
+// Products with at most 32 rows or columns: the LDS-free kernel, the small side as N.
+int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled) {
+  if (p.N > 32) {   // swap the roles of the operands: C^T = B A^T
+    std::swap(p.m, p.n);
+    std::swap(p.M, p.N);
+    std::swap(pa, pb);
+    for (Group* g : {&p.m, &p.n, &p.k, &p.bt})
+      for (int i = 0; i < GD; ++i) std::swap(g->sa[i], g->sb[i]);
+  }
+  const int tn = p.N <= 16 ? 1 : 2, tm = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
+  const int64_t tiles = ((p.M + 16 * tm - 1) / (16 * tm)) * ((p.N + 16 * tn - 1) / (16 * tn));
+  if (tiles > 0x3fffffff) return HGPU_OK;
+  // one wavefront per (tile, K chunk): aim at four per SIMD, chunks of at least 64
+  const int64_t want = (int64_t)ctx->num_cu * 16;
+  const int64_t out_elems = p.M * p.N * p.BT;
+  int64_t split = 1;
+  if (tiles * p.BT * 2 <= want && p.K >= 128) {
+    split = (want + tiles * p.BT - 1) / (tiles * p.BT);
+    int64_t cap = (int64_t)((double)(p.M + p.N) * p.K * p.BT / (2.0 * out_elems));   // partials stay small next to the operands
+    if (cap > 4096) cap = 4096;
+    if (split > cap) split = cap;
+    if (split > p.K / 64) split = p.K / 64;
+    if (split < 1) split = 1;
+  }
+  p.kchunk = ((p.K + split - 1) / split + 15) / 16 * 16;
+  p.split = (int)((p.K + p.kchunk - 1) / p.kchunk);
+  split = p.split;
+  p.a_kc = p.b_kc = 0;
+
+  const size_t es = dtype_size(dtype);
+  const int64_t out_n = nelem(out);
+  const void* zero_tab = nullptr;
+  int rc = zero_block(ctx, &zero_tab);
+  if (rc) return rc;
+  hgpu_buffer* koff = nullptr;
+  const int64_t Kp = (p.K + 15) / 16 * 16 + 32;   // padded tables (see k_gemm_direct)
+  rc = buffer_alloc(ctx, (size_t)Kp * 16, &koff);
+  if (rc) return rc;
+  hgpu_buffer* part = nullptr;
+  if (split > 1) {
+    rc = buffer_alloc(ctx, (size_t)out_n * split * es, &part);
+    if (rc) { buffer_release(koff); return rc; }
+  }
+  p.c_split_stride = split > 1 ? out_n : 0;
+  int64_t* ka = (int64_t*)koff->ptr;
+  int64_t* kb = ka + Kp;
+  dim3 grid((unsigned)((tiles * split + 3) / 4), 1, (unsigned)p.BT);
+  {
+    double flops = 2.0 * p.M * p.N * p.K * p.BT;
+    double bytes = ((double)p.M * p.K + (double)p.N * p.K + (double)p.M * p.N) * p.BT * es;
+    const char* label = dtype == HGPU_F64 ? "gemm_f64" : "gemm_f32";
+    if (ctx->profiling && ctx->profile_shapes) {
+      char buf[128];
+      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,direct,t%dx%d,k%lld:%lld/%lld]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, (int)split, 16 * tm, 16 * tn, (long long)p.k.shape[p.k.nd - 1], (long long)p.k.sa[p.k.nd - 1], (long long)p.k.sb[p.k.nd - 1]);
+      label = ctx->label_pool.insert(buf).first->c_str();
+    }
+    LaunchGuard lg(ctx, label, bytes, flops);
+    if (p.k.nd > 1) {
+      hipLaunchKernelGGL(k_koff, dim3((unsigned)((Kp + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, Kp, ka, kb);
+      p.kmask = -1;
+      p.ksa = p.ksb = 0;
+    } else {   // single K dim: offsets are k * stride, the table a block of zeros
+      ka = kb = (int64_t*)zero_tab;
+      p.kmask = 0;
+      p.ksa = p.k.sa[0];
+      p.ksb = p.k.sb[0];
+    }
+    void* cdst = split > 1 ? part->ptr : data_ptr(out);
+    // an operand contiguous along K is read four elements at a time
+    auto k_vector = [&](const void* base, const int64_t* ks, const int64_t* rs, const Group& rows, const int64_t* bs) {
+      const int64_t v = (int64_t)(16 / es);
+      const int kd = p.k.nd - 1;
+      if (((uintptr_t)base & 15) != 0 || p.K < 16 || ks[kd] != 1 || p.k.shape[kd] % 4 != 0) return false;
+      for (int i = 0; i < kd; ++i) if (ks[i] % v != 0) return false;
+      for (int i = 0; i < rows.nd; ++i) if (rs[i] % v != 0) return false;
+      for (int i = 0; i < p.bt.nd; ++i) if (bs[i] % v != 0) return false;
+      return true;
+    };
+    const bool va = k_vector(pa, p.k.sa, p.m.sa, p.m, p.bt.sa), vb = k_vector(pb, p.k.sb, p.n.sb, p.n, p.bt.sb);
+    LaunchArgs la{ctx->stream, -1, tm, tn, va, vb, grid, pa, pb, cdst, ka, kb};
+    if (dtype == HGPU_F64) {
+      launch_f64(p, la);
+      if (split > 1)
+        hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, (int)split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
+    } else {
+      launch_f32(p, la);
+      if (split > 1)
+        hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, (int)split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
+    }
+  }
+  hipError_t e = hipGetLastError();
+  buffer_release(koff);
+  if (part) buffer_release(part);
+  if (e != hipSuccess) return check_hip(ctx, e, "gemm");
+  *handled = true;
+  return HGPU_OK;
+}
+
 }  // namespace
 
 namespace hg {
@@ -184,6 +290,10 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   if (p.BT > 65535) return HGPU_OK;
   if ((double)p.M * p.N * p.K * p.BT < 2.0e6) return HGPU_OK;
 
+  const void* pa = data_ptr(a);
+  const void* pb = data_ptr(b);
+  if (p.M <= 32 || p.N <= 32) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled);
+
   // tile shape: least padded work per unit of efficiency
   int cfg = 0;
   double best = 1e300;
@@ -226,8 +336,12 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
 
   size_t es = dtype_size(a->dtype);
   int64_t out_n = nelem(out);
+  const void* zero_tab = nullptr;
+  int rc = zero_block(ctx, &zero_tab);
+  if (rc) return rc;
   hgpu_buffer* koff = nullptr;
-  int rc = buffer_alloc(ctx, (size_t)p.K * 16, &koff);
+  const int64_t Kp = p.K;
+  rc = buffer_alloc(ctx, (size_t)Kp * 16, &koff);
   if (rc) return rc;
   hgpu_buffer* part = nullptr;
   if (split > 1) {
@@ -269,17 +383,25 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
       label = ctx->label_pool.insert(buf).first->c_str();
     }
     LaunchGuard lg(ctx, label, bytes, flops);
-    if (p.k.nd > 1) hipLaunchKernelGGL(k_koff, dim3((unsigned)((p.K + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, ka, kb);
-    else ka = kb = nullptr;    // single K dim: offsets are k * stride
+    if (p.k.nd > 1) {
+      hipLaunchKernelGGL(k_koff, dim3((unsigned)((Kp + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, Kp, ka, kb);
+      p.kmask = -1;
+      p.ksa = p.ksb = 0;
+    } else {   // single K dim: offsets are k * stride, the table a block of zeros
+      ka = kb = (int64_t*)zero_tab;
+      p.kmask = 0;
+      p.ksa = p.k.sa[0];
+      p.ksb = p.k.sb[0];
+    }
     if (a->dtype == HGPU_F64) {
       double* cdst = split > 1 ? (double*)part->ptr : (double*)data_ptr(out);
-      LaunchArgs la{ctx->stream, cfg, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
+      LaunchArgs la{ctx->stream, cfg, 0, 0, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
       launch_f64(p, la);
       if (split > 1)
         hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
     } else {
       float* cdst = split > 1 ? (float*)part->ptr : (float*)data_ptr(out);
-      LaunchArgs la{ctx->stream, cfg, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
+      LaunchArgs la{ctx->stream, cfg, 0, 0, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
       launch_f32(p, la);
       if (split > 1)
         hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const float*)part->ptr, (float*)data_ptr(out));

@@ -6,7 +6,7 @@
 //     C[m, n] = C0 + offCm(m) + offCn(n),
 // with m, n, k linear indices into merged dim groups (Group).  The K offsets
 // come from two tables written by k_koff (or, for a single K dim, from a
-// multiplication); row offsets are decomposed once per thread.
+// multiplication: see KOff); row offsets are decomposed once per thread.
 //
 // 256 threads = 4 wavefronts in a WGM x WGN grid; block tile BM x BN with
 // K-step 16.  Operand tiles go global -> registers -> LDS ([k][row] order, one
@@ -37,6 +37,7 @@ struct GemmParams {
   int split;          // K chunks
   int64_t kchunk;     // K elements per chunk (multiple of BK)
   int64_t c_split_stride;  // elements between partial outputs
+  int64_t kmask, ksa, ksb; // K offsets: table[k & kmask] + k * ks; kmask 0 = no table (see KOff)
 };
 
 __device__ __forceinline__ void group_off(const Group& g, int64_t lin, int64_t* oa, int64_t* ob, int64_t* oc) {
@@ -91,8 +92,11 @@ template <> struct VecOf<float, 1> { using type = float; };
 template <> struct VecOf<double, 2> { using type = __attribute__((ext_vector_type(2))) double; };
 template <> struct VecOf<float, 4> { using type = __attribute__((ext_vector_type(4))) float; };
 
-// K offset of linear index k for one operand: a product when the K group is a
-// single dim, else a table lookup.
+// K offset of linear index k for one operand.  Several K dims: a table written
+// by k_koff.  A single K dim: a multiplication.
+//   KOff  (staged kernel): tab == nullptr selects the multiplication;
+//   direct kernel: branch-free tab[k & kmask] + k * stride, with kmask 0 on a
+//   table of zeros when the stride does the work.
 struct KOff {
   const int64_t* __restrict__ tab;
   int64_t stride;   // used when tab == nullptr
@@ -223,7 +227,7 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const typename X::T* 
 
   Stager<T, BM, VA> sa;
   Stager<T, BN, VB> sb;
-  const KOff koa{koffA, p.k.sa[0]}, kob{koffB, p.k.sb[0]};
+  const KOff koa{p.kmask ? koffA : nullptr, p.ksa}, kob{p.kmask ? koffB : nullptr, p.ksb};
   sa.init(t, p.a_kc, 0, A + bta, p.m, m0, p.M, koa, kbeg, p.K);
   sb.init(t, p.b_kc, 1, B + btb, p.n, n0, p.N, kob, kbeg, p.K);
 
@@ -297,6 +301,170 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const typename X::T* 
   }
 }
 
+// Skinny products (N <= 32): one wavefront owns a (16 TM) x (16 TN) block of the
+// output over one K chunk and loads its MFMA operand fragments straight from
+// global memory.  With so few columns no operand element is shared between
+// wavefronts, so staging through LDS (and its barriers) would buy nothing; the
+// wavefronts run independently, each with the loads of the next 16 K elements
+// in flight while the MFMAs of the current 16 run.
+//
+// K is walked in groups of 16.  Within a group lane (r, q) -- r = lane % 16 the
+// row, q = lane / 16 -- owns k = k0 + 4 q + j at MFMA step j (any assignment of
+// k to steps is a valid summation order as long as A and B agree).  The four k
+// of a lane are consecutive, so an operand that is contiguous along K is read
+// with one 4-element vector load per row block (VA / VB); otherwise with four
+// loads at offsets taken from the K table (itself read as one vector).
+// The K tables are padded: entries up to K + 32 exist and repeat the last four
+// valid k (see k_koff).
+// grid.x * 4 wavefronts cover (split, tile_m, tile_n); grid.z is the batch.
+template <typename T> struct Vec4Of { using type = T __attribute__((ext_vector_type(4), aligned(16))); };
+using Off4 = int64_t __attribute__((ext_vector_type(4), aligned(16)));
+
+template <typename X, int TM, int TN, bool VA, bool VB>
+__global__ void __launch_bounds__(NT) k_gemm_direct(GemmParams p, const typename X::T* __restrict__ A, const typename X::T* __restrict__ B,
+                                                    typename X::T* __restrict__ C, const int64_t* __restrict__ koffA,
+                                                    const int64_t* __restrict__ koffB) {
+  using T = typename X::T;
+  using Acc = typename X::Acc;
+  using V4 = typename Vec4Of<T>::type;
+  static_assert(X::NBW == 16, "16-column MFMA blocks");
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 15, q = lane >> 4;
+  const int64_t tiles_m = (p.M + 16 * TM - 1) / (16 * TM), tiles_n = (p.N + 16 * TN - 1) / (16 * TN);
+  const int64_t per_split = tiles_m * tiles_n;
+  const int64_t item = (int64_t)blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
+  if (item >= per_split * p.split) return;
+  const int64_t s = item / per_split, tile = item - s * per_split;
+  const int64_t tile_m = tile / tiles_n, tile_n = tile - tile_m * tiles_n;
+  const int64_t m0 = tile_m * 16 * TM, n0 = tile_n * 16 * TN;
+
+  int64_t bta, btb, btc;
+  group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
+  const int64_t kbeg = s * p.kchunk;
+  int64_t kend = kbeg + p.kchunk;
+  if (kend > p.K) kend = p.K;
+
+  const T* ra[TM];
+  const T* rb[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    int64_t m = m0 + 16 * i + r;
+    if (m >= p.M) m = p.M - 1;              // clamp: the values are never stored
+    int64_t oa, ob, oc;
+    group_off(p.m, m, &oa, &ob, &oc);
+    ra[i] = A + bta + oa;
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int64_t n = n0 + 16 * j + r;
+    if (n >= p.N) n = p.N - 1;
+    int64_t oa, ob, oc;
+    group_off(p.n, n, &oa, &ob, &oc);
+    rb[j] = B + btb + ob;
+  }
+
+  Acc acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = X::zero();
+
+  // offsets of this lane's four k of the next group to load (vector operands
+  // need only the first), and two buffers of operand values
+  Off4 oa4, ob4;
+  V4 va[2][TM], vb[2][TN];
+  // first k of the lane in the group at k0; past the end the group is masked and
+  // any valid position will do
+  const int64_t klast = ((p.K + 15) / 16) * 16;       // the tables reach klast + 16
+  auto fetch_off = [&](int64_t k0) {
+    const int64_t k = (k0 < klast ? k0 : klast) + 4 * q;
+    const int64_t kt = k & p.kmask;
+    oa4 = *reinterpret_cast<const Off4*>(koffA + kt);
+    ob4 = *reinterpret_cast<const Off4*>(koffB + kt);
+    // past K: the last four valid k, so that a vector load there stays inside
+    const int64_t base = k < p.K ? k : (p.K >= 4 ? p.K - 4 : 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int64_t kj = base + j < p.K ? base + j : p.K - 1;
+      oa4[j] += kj * p.ksa;
+      ob4[j] += kj * p.ksb;
+    }
+  };
+  auto fetch = [&](int buf, int64_t k0) {
+    const int64_t k = k0 + 4 * q;
+    bool ok[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ok[j] = k + j < kend;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      V4 x;
+      if constexpr (VA) x = *reinterpret_cast<const V4*>(ra[i] + oa4[0]);
+      else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[j] = ra[i][oa4[j]];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) va[buf][i][j] = ok[j] ? x[j] : T(0);
+    }
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      V4 x;
+      if constexpr (VB) x = *reinterpret_cast<const V4*>(rb[i] + ob4[0]);
+      else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[j] = rb[i][ob4[j]];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) vb[buf][i][j] = ok[j] ? x[j] : T(0);
+    }
+  };
+  auto compute = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = X::run(va[buf][i][u], vb[buf][j][u], acc[i][j]);
+  };
+  fetch_off(kbeg);
+  fetch(0, kbeg);
+  fetch_off(kbeg + 16);
+  for (int64_t k0 = kbeg; k0 < kend; k0 += 32) {
+    fetch(1, k0 + 16);
+    fetch_off(k0 + 32);
+    compute(0);
+    fetch(0, k0 + 32);
+    fetch_off(k0 + 48);
+    compute(1);
+  }
+
+  T* Cout = C + btc + s * p.c_split_stride;
+  int64_t coln[TN];
+  bool colok[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int64_t n = n0 + 16 * j + X::col(lane);
+    colok[j] = n < p.N;
+    int64_t oa = 0, ob = 0, oc = 0;
+    if (colok[j]) group_off(p.n, n, &oa, &ob, &oc);
+    coln[j] = oc;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int w = 0; w < X::NR; ++w) {
+      int64_t m = m0 + 16 * i + X::row(lane, w);
+      if (m < p.M) {
+        int64_t oa, ob, oc;
+        group_off(p.m, m, &oa, &ob, &oc);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          if (colok[j]) Cout[oc + coln[j]] = X::get(acc[i][j], w);
+      }
+    }
+  }
+}
+
 struct TileCfg { int wgm, wgn, tm, tn; double eff; };
 // Candidate tiles, with a rough relative efficiency (operand reuse from LDS).
 constexpr TileCfg kTiles[] = {
@@ -316,7 +484,8 @@ constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 struct LaunchArgs {
   hipStream_t stream;
-  int cfg;
+  int cfg;            // index into kTiles, or -1: the direct kernel with direct_tm x direct_tn blocks per wavefront
+  int direct_tm, direct_tn;
   bool va, vb;
   dim3 grid;
   const void *A, *B;
@@ -344,8 +513,32 @@ void launch_cfg(const GemmParams& p, const LaunchArgs& a) {
   hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, 1, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
 }
 
+template <typename X, int TM, int TN>
+void launch_direct_cfg(const GemmParams& p, const LaunchArgs& a) {
+  using T = typename X::T;
+  const T* A = (const T*)a.A;
+  const T* B = (const T*)a.B;
+  T* C = (T*)a.C;
+  if (a.va && a.vb) hipLaunchKernelGGL((k_gemm_direct<X, TM, TN, true, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+  else if (a.va) hipLaunchKernelGGL((k_gemm_direct<X, TM, TN, true, false>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+  else if (a.vb) hipLaunchKernelGGL((k_gemm_direct<X, TM, TN, false, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+  else hipLaunchKernelGGL((k_gemm_direct<X, TM, TN, false, false>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+}
+
 template <typename X>
 void launch(const GemmParams& p, const LaunchArgs& a) {
+  if (a.cfg < 0) {
+    if (a.direct_tn == 2) {
+      if (a.direct_tm == 1) launch_direct_cfg<X, 1, 2>(p, a);
+      else if (a.direct_tm == 2) launch_direct_cfg<X, 2, 2>(p, a);
+      else launch_direct_cfg<X, 4, 2>(p, a);
+    } else {
+      if (a.direct_tm == 1) launch_direct_cfg<X, 1, 1>(p, a);
+      else if (a.direct_tm == 2) launch_direct_cfg<X, 2, 1>(p, a);
+      else launch_direct_cfg<X, 4, 1>(p, a);
+    }
+    return;
+  }
   switch (a.cfg) {
     case 0: launch_cfg<X, 2, 2, 4, 4>(p, a); break;
     case 1: launch_cfg<X, 2, 2, 4, 2>(p, a); break;

@@ -230,6 +230,21 @@ static int ensure_staging(hgpu_ctx* ctx, size_t bytes) {
 
 using namespace hg;
 
+namespace hg {
+int zero_block(hgpu_ctx* ctx, const void** out) {
+  if (!ctx->zero_block) {
+    hgpu_buffer* b = nullptr;
+    int rc = buffer_alloc(ctx, 256, &b);
+    if (rc) return rc;
+    rc = zero_fill(ctx, b->ptr, 256);
+    if (rc) { buffer_release(b); return rc; }
+    ctx->zero_block = b;
+  }
+  *out = ctx->zero_block->ptr;
+  return HGPU_OK;
+}
+}  // namespace hg
+
 extern "C" {
 
 int hgpu_init(int device, hgpu_ctx** out) {
@@ -257,6 +272,7 @@ int hgpu_shutdown(hgpu_ctx* ctx) {
   if (!ctx) return HGPU_ERR_INVALID;
   (void)hipSetDevice(ctx->device);
   (void)hipStreamSynchronize(ctx->stream);
+  if (ctx->zero_block) { buffer_release(ctx->zero_block); ctx->zero_block = nullptr; }
   {
     std::lock_guard<std::mutex> g(ctx->mu);
     drop_cache_locked(ctx);
