@@ -143,8 +143,9 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
   const int tn = p.N <= 16 ? 1 : 2, tm = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
   const int64_t tiles = ((p.M + 16 * tm - 1) / (16 * tm)) * ((p.N + 16 * tn - 1) / (16 * tn));
   if (tiles > 0x3fffffff) return HGPU_OK;
-  // one wavefront per (tile, K chunk): aim at four per SIMD, chunks of at least 64
-  const int64_t want = (int64_t)ctx->num_cu * 16;
+  // one wavefront per (tile, K chunk): aim at one per SIMD (more, shorter chunks
+  // measured slower: set-up and partial sums per wavefront), chunks of at least 64
+  const int64_t want = (int64_t)ctx->num_cu * 4;
   const int64_t out_elems = p.M * p.N * p.BT;
   int64_t split = 1;
   if (tiles * p.BT * 2 <= want && p.K >= 128) {
@@ -292,7 +293,9 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
 
   const void* pa = data_ptr(a);
   const void* pb = data_ptr(b);
-  if (p.M <= 32 || p.N <= 32) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled);
+  // A small output under a long K (weight gradients, the last layer of a
+  // classifier) is better served by independent wavefronts than by staged tiles.
+  if ((p.M <= 32 || p.N <= 32) && p.M <= 1024 && p.N <= 1024) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled);
 
   // tile shape: least padded work per unit of efficiency
   int cfg = 0;
