@@ -117,19 +117,12 @@ int64_t total(const Group& g) {
 }
 
 // True when 16-byte loads along the direction the staging lanes run are safe
-// for one operand: unit stride and an extent that is a multiple of the vector
-// there, every other stride and the base address a multiple of the vector.
-bool vector_ok(const void* base, size_t es, const Group& run, int run_dim, const int64_t* run_st,
-               const Group* others[3], const int64_t* const other_st[3]) {
+// for one operand: unit stride there and an extent that is a multiple of the
+// vector, so that the elements of a vector are neighbours in memory.  The
+// vectors need element alignment only.
+bool vector_ok(size_t es, const Group& run, int run_dim, const int64_t* run_st) {
   const int64_t v = (int64_t)(16 / es);
-  if (((uintptr_t)base & 15) != 0) return false;
-  if (run_st[run_dim] != 1 || run.shape[run_dim] % v != 0) return false;
-  for (int i = 0; i < run.nd; ++i)
-    if (i != run_dim && run_st[i] % v != 0) return false;
-  for (int g = 0; g < 3; ++g)
-    for (int i = 0; i < others[g]->nd; ++i)
-      if (other_st[g][i] % v != 0) return false;
-  return true;
+  return run_st[run_dim] == 1 && run.shape[run_dim] % v == 0;
 }
 // Products with at most 32 rows or columns: the LDS-free kernel, the small side as N.
 int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled) {
@@ -368,12 +361,8 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   p.b_kc = bkc ? 1 : 0;
   bool va, vb;
   {
-    const Group* oa[3] = {akc ? &p.m : &p.k, &p.bt, &p.bt};
-    const int64_t* const osa[3] = {akc ? p.m.sa : p.k.sa, p.bt.sa, p.bt.sa};
-    va = vector_ok(data_ptr(a), dtype_size(a->dtype), akc ? p.k : p.m, (akc ? p.k.nd : p.m.nd) - 1, akc ? p.k.sa : p.m.sa, oa, osa);
-    const Group* ob[3] = {bkc ? &p.n : &p.k, &p.bt, &p.bt};
-    const int64_t* const osb[3] = {bkc ? p.n.sb : p.k.sb, p.bt.sb, p.bt.sb};
-    vb = vector_ok(data_ptr(b), dtype_size(b->dtype), bkc ? p.k : p.n, (bkc ? p.k.nd : p.n.nd) - 1, bkc ? p.k.sb : p.n.sb, ob, osb);
+    va = vector_ok(es, akc ? p.k : p.m, (akc ? p.k.nd : p.m.nd) - 1, akc ? p.k.sa : p.m.sa);
+    vb = vector_ok(es, bkc ? p.k : p.n, (bkc ? p.k.nd : p.n.nd) - 1, bkc ? p.k.sb : p.n.sb);
   }
   dim3 grid((unsigned)tiles, (unsigned)split, (unsigned)p.BT);
   {

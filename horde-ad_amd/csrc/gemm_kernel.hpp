@@ -89,8 +89,9 @@ struct MfmaF64 {
 template <typename T, int V> struct VecOf;
 template <> struct VecOf<double, 1> { using type = double; };
 template <> struct VecOf<float, 1> { using type = float; };
-template <> struct VecOf<double, 2> { using type = __attribute__((ext_vector_type(2))) double; };
-template <> struct VecOf<float, 4> { using type = __attribute__((ext_vector_type(4))) float; };
+// element-aligned vectors: multi-dword global loads need dword alignment only
+template <> struct VecOf<double, 2> { using type = double __attribute__((ext_vector_type(2), aligned(8))); };
+template <> struct VecOf<float, 4> { using type = float __attribute__((ext_vector_type(4), aligned(4))); };
 
 // K offset of linear index k for one operand.  Several K dims: a table written
 // by k_koff.  A single K dim: a multiplication.
@@ -504,11 +505,17 @@ void launch_cfg(const GemmParams& p, const LaunchArgs& a) {
   const T* A = (const T*)a.A;
   const T* B = (const T*)a.B;
   T* C = (T*)a.C;
-  // 16-byte loads only for tiles whose rows are long enough to share a load's lanes sensibly
-  if constexpr (BM >= 64 && BN >= 64) {
-    if (a.va && a.vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, V, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
-    if (a.va) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, 1, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
-    if (a.vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, V, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+  // 16-byte loads only on a side of the tile long enough to share a load's lanes sensibly
+  constexpr bool CA = BM >= 64, CB = BN >= 64;
+  const bool va = CA && a.va, vb = CB && a.vb;
+  if constexpr (CA && CB) {
+    if (va && vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, V, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+  }
+  if constexpr (CA) {
+    if (va) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, 1, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+  }
+  if constexpr (CB) {
+    if (vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, V, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
   }
   hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, 1, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
 }
