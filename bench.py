@@ -4,7 +4,11 @@
 One "step" = one full forward + reverse gradient of a config's objective on one
 batch of synthetic input that is already resident in HBM (uploads happen before
 the timed region; every step ends with a stream sync, the equivalent of the
-reference forcing every gradient leaf, bench/ConvVjpBench.hs:174-175).
+reference forcing every gradient leaf, bench/ConvVjpBench.hs:174-175).  As the
+reference builds its gradient artifact once and times its evaluation
+(bench/ConvVjpBench.hs:254-257), the gradient program is recorded once into a
+device graph and a step launches that graph; `ms_per_step_eager` is the same
+program submitted operation by operation from Python, and --eager times that.
 
 Prints ONE JSON line.  `value` is gradient samples/s of the headline config
 (the CNN); the other configs ride along under "configs".  "roofline" prices the
@@ -54,6 +58,26 @@ def time_steps(host, wl, ps, ds, steps, warmup):
     host.sync()
     dt = time.perf_counter() - t0
     return dt / steps, float(loss.numpy())
+
+
+def time_graph(host, wl, ps, ds, steps, warmup):
+    """The same gradient recorded once (the reference builds its gradient
+    artifact once, outside the timed region) and launched per step."""
+    graph, (loss, grads) = host.capture(lambda: wl.gradient(host, ps, ds))
+    try:
+        for _ in range(warmup):
+            graph.launch()
+            host.sync()
+        host.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.launch()
+            host.sync()
+        host.sync()
+        dt = time.perf_counter() - t0
+        return dt / steps, float(loss.numpy())
+    finally:
+        graph.free()
 
 
 def profile(capi, host, wl, ps, ds, reps=2):
@@ -116,6 +140,7 @@ def main():
     ap.add_argument("--workload", default="c3", help="headline config: c0..c4")
     ap.add_argument("--only", action="store_true", help="measure the headline config only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--eager", action="store_true", help="time op-by-op submission instead of the recorded graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run plain dense copies of 1 GiB (for scaling hardware traffic counters) and exit")
     args = ap.parse_args()
@@ -144,13 +169,17 @@ def main():
         wl = W.CONFIGS[key]()
         ps, ds = wl.upload(host)
         host.sync()
-        sec, loss = time_steps(host, wl, ps, ds, args.steps, args.warmup)
+        eager_sec, loss = time_steps(host, wl, ps, ds, args.steps, args.warmup)
+        sec, graph_loss = (eager_sec, loss) if args.eager else time_graph(host, wl, ps, ds, args.steps, args.warmup)
+        if graph_loss != loss:
+            raise SystemExit(f"bench.py: {key}: the recorded program computed {graph_loss!r}, the eager one {loss!r}")
         rep = profile(capi, host, wl, ps, ds)
         dn = DTYPE_NAME[wl.dtype]
         roof, shares = roofline_of(rep, dn)
         dev_ms = sum(v[1] for v in rep.values())
         results[key] = {"workload": wl.name, "dtype": dn, "batch": wl.batch, "ms_per_step": sec * 1e3,
                         "samples_per_s": wl.batch / sec, "gradients_per_s": 1.0 / sec, "loss": loss,
+                        "ms_per_step_eager": eager_sec * 1e3, "execution": "eager" if args.eager else "recorded graph, one launch per step",
                         "device_ms_per_step": dev_ms, "algorithmic_gflop": wl.flops / 1e9,
                         "achieved_tflops": wl.flops / sec / 1e12, "roofline": roof, "kernel_ms": shares}
         if wl.bytes:

@@ -44,6 +44,7 @@ extern "C" int hgpu_compare_all(hgpu_ctx* ctx, int cmp, const hgpu_array* a, con
   if (cmp < HGPU_LEQ || cmp > HGPU_LT) return fail(ctx, HGPU_ERR_INVALID, "compare_all: unknown opcode %d", cmp);
   if (a->dtype != b->dtype) return fail(ctx, HGPU_ERR_INVALID, "compare_all: dtypes differ");
   if (!same_shape(a, b)) return fail(ctx, HGPU_ERR_INVALID, "compare_all: shapes differ");
+  if (int rc = no_capture(ctx, "compare_all")) return rc;
   int64_t n = nelem(a);
   if (n == 0) {
     *result = cmp == HGPU_LT ? 0 : 1;

@@ -20,11 +20,21 @@
 // are contiguous in every operand have been merged.
 #define HG_KDIMS 10
 
+// Blocks handed out while a graph is being captured belong to the capture's
+// pool: replays of the graph write them again, so they may be reused by the
+// capture itself but never by other work while the graph lives.
+struct hgpu_cap_pool {
+  std::multimap<size_t, void*> cache;   // guarded by the context's allocator mutex
+  bool alive = true;                    // false once the graph is destroyed: blocks return to the context's cache
+  int refs = 1;                         // the graph (or the open capture) + every live buffer
+};
+
 struct hgpu_buffer {
   hgpu_ctx* ctx;
   void* ptr;
   size_t bytes;      // size of the block handed out by the allocator
   std::atomic<int> refs;
+  hgpu_cap_pool* pool = nullptr;
 };
 
 struct hgpu_array {
@@ -59,6 +69,14 @@ struct hgpu_ctx {
   std::set<std::string> label_pool;
   std::vector<ProfRec> prof;
   hgpu_buffer* zero_block = nullptr;     // 256 zero bytes, for kernels that want a dummy table
+  hgpu_cap_pool* cap = nullptr;          // non-null while the stream is capturing into a graph
+};
+
+struct hgpu_graph {
+  hgpu_ctx* ctx;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  hgpu_cap_pool* pool = nullptr;
 };
 
 namespace hg {
@@ -81,6 +99,8 @@ int check_hip(hgpu_ctx* ctx, hipError_t e, const char* what);
 // Allocator (runtime.hip).
 int buffer_alloc(hgpu_ctx* ctx, size_t bytes, hgpu_buffer** out);
 int zero_block(hgpu_ctx* ctx, const void** out);   // a context-lifetime block of 256 zero bytes
+// Fails (HGPU_ERR_UNSUPPORTED) when the stream is capturing: for entry points that must talk to the host.
+int no_capture(hgpu_ctx* ctx, const char* what);
 void buffer_retain(hgpu_buffer* b);
 void buffer_release(hgpu_buffer* b);
 
@@ -141,7 +161,7 @@ struct LaunchGuard {
   explicit LaunchGuard(hgpu_ctx* c, const char* name = nullptr, double bytes = 0, double flops = 0) : ctx(c) {
     c->launch_mu.lock();
     (void)hipSetDevice(c->device);
-    if (c->profiling && name) {
+    if (c->profiling && name && !c->cap) {
       hgpu_ctx::ProfRec r{name, nullptr, nullptr, bytes, flops};
       if (hipEventCreate(&r.a) == hipSuccess && hipEventCreate(&r.b) == hipSuccess) {
         (void)hipEventRecord(r.a, c->stream);

@@ -49,10 +49,11 @@ int buffer_alloc(hgpu_ctx* ctx, size_t bytes, hgpu_buffer** out) {
   void* p = nullptr;
   {
     std::lock_guard<std::mutex> g(ctx->mu);
-    auto it = ctx->cache.find(blk);
-    if (it != ctx->cache.end()) {
+    std::multimap<size_t, void*>& cache = ctx->cap ? ctx->cap->cache : ctx->cache;
+    auto it = cache.find(blk);
+    if (it != cache.end()) {
       p = it->second;
-      ctx->cache.erase(it);
+      cache.erase(it);
     } else {
       if (ctx->fail_after >= 0 && (int64_t)ctx->n_device_allocs >= ctx->fail_after) {
         ctx->err = "device allocation failed (injected)";
@@ -60,7 +61,7 @@ int buffer_alloc(hgpu_ctx* ctx, size_t bytes, hgpu_buffer** out) {
       }
       (void)hipSetDevice(ctx->device);
       hipError_t e = hipMalloc(&p, blk);
-      if (e != hipSuccess) {
+      if (e != hipSuccess && !ctx->cap) {
         (void)hipGetLastError();
         // Cached blocks may still be read by enqueued kernels: drain first.
         (void)hipStreamSynchronize(ctx->stream);
@@ -84,6 +85,11 @@ int buffer_alloc(hgpu_ctx* ctx, size_t bytes, hgpu_buffer** out) {
   b->ptr = p;
   b->bytes = blk;
   b->refs.store(1);
+  {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    b->pool = ctx->cap;
+    if (b->pool) b->pool->refs++;
+  }
   *out = b;
   return HGPU_OK;
 }
@@ -101,7 +107,10 @@ void buffer_release(hgpu_buffer* b) {
       // already enqueued on the in-order stream, and whatever reuses it is
       // enqueued behind that work.
       std::lock_guard<std::mutex> g(ctx->mu);
-      ctx->cache.emplace(b->bytes, b->ptr);
+      hgpu_cap_pool* pool = b->pool;
+      if (pool && pool->alive) pool->cache.emplace(b->bytes, b->ptr);
+      else ctx->cache.emplace(b->bytes, b->ptr);
+      if (pool && --pool->refs == 0) delete pool;
       ctx->in_use -= b->bytes;
     }
     delete b;
@@ -231,6 +240,11 @@ static int ensure_staging(hgpu_ctx* ctx, size_t bytes) {
 using namespace hg;
 
 namespace hg {
+int no_capture(hgpu_ctx* ctx, const char* what) {
+  if (ctx->cap) return fail(ctx, HGPU_ERR_UNSUPPORTED, "%s: not while a graph is being captured (it needs the host)", what);
+  return HGPU_OK;
+}
+
 int zero_block(hgpu_ctx* ctx, const void** out) {
   if (!ctx->zero_block) {
     hgpu_buffer* b = nullptr;
@@ -264,7 +278,91 @@ int hgpu_init(int device, hgpu_ctx** out) {
   }
   hipDeviceProp_t prop;
   if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->num_cu = prop.multiProcessorCount;
+  const void* z = nullptr;
+  (void)zero_block(ctx, &z);     // made now, so that no capture ever owns it
   *out = ctx;
+  return HGPU_OK;
+}
+
+// ---- graphs: one captured sequence of launches, replayed as a unit ---------
+
+int hgpu_capture_begin(hgpu_ctx* ctx) {
+  if (!ctx) return HGPU_ERR_INVALID;
+  if (ctx->cap) return fail(ctx, HGPU_ERR_INVALID, "capture_begin: a capture is already open");
+  (void)hipSetDevice(ctx->device);
+  hipError_t e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) return check_hip(ctx, e, "capture_begin");
+  hgpu_cap_pool* pool = new hgpu_cap_pool;
+  {
+    // The warm blocks of the context move into the capture's pool: a capture
+    // after a warm-up run allocates nothing.
+    std::lock_guard<std::mutex> g(ctx->mu);
+    pool->cache.swap(ctx->cache);
+  }
+  e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed);
+  if (e != hipSuccess) {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    ctx->cache.swap(pool->cache);
+    delete pool;
+    return check_hip(ctx, e, "hipStreamBeginCapture");
+  }
+  std::lock_guard<std::mutex> g(ctx->mu);
+  ctx->cap = pool;
+  return HGPU_OK;
+}
+
+static void retire_pool(hgpu_ctx* ctx, hgpu_cap_pool* pool) {
+  std::lock_guard<std::mutex> g(ctx->mu);
+  pool->alive = false;
+  for (auto& kv : pool->cache) ctx->cache.emplace(kv.first, kv.second);
+  pool->cache.clear();
+  if (--pool->refs == 0) delete pool;
+}
+
+int hgpu_capture_end(hgpu_ctx* ctx, hgpu_graph** out) {
+  if (!ctx || !out) return HGPU_ERR_INVALID;
+  if (!ctx->cap) return fail(ctx, HGPU_ERR_INVALID, "capture_end: no capture is open");
+  (void)hipSetDevice(ctx->device);
+  hgpu_cap_pool* pool;
+  {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    pool = ctx->cap;
+    ctx->cap = nullptr;
+  }
+  hgpu_graph* gr = new hgpu_graph;
+  gr->ctx = ctx;
+  gr->pool = pool;
+  hipError_t e = hipStreamEndCapture(ctx->stream, &gr->graph);
+  if (e == hipSuccess) e = hipGraphInstantiate(&gr->exec, gr->graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    if (gr->graph) (void)hipGraphDestroy(gr->graph);
+    retire_pool(ctx, pool);
+    delete gr;
+    return check_hip(ctx, e, "capture_end");
+  }
+  *out = gr;
+  return HGPU_OK;
+}
+
+int hgpu_graph_launch(hgpu_graph* gr) {
+  if (!gr) return HGPU_ERR_INVALID;
+  hgpu_ctx* ctx = gr->ctx;
+  if (ctx->cap) return fail(ctx, HGPU_ERR_INVALID, "graph_launch: not inside a capture");
+  std::lock_guard<std::mutex> lk(ctx->launch_mu);
+  (void)hipSetDevice(ctx->device);
+  return check_hip(ctx, hipGraphLaunch(gr->exec, ctx->stream), "hipGraphLaunch");
+}
+
+int hgpu_graph_destroy(hgpu_graph* gr) {
+  if (!gr) return HGPU_ERR_INVALID;
+  hgpu_ctx* ctx = gr->ctx;
+  (void)hipSetDevice(ctx->device);
+  (void)hipStreamSynchronize(ctx->stream);     // a replay may still be running on the blocks
+  if (gr->exec) (void)hipGraphExecDestroy(gr->exec);
+  if (gr->graph) (void)hipGraphDestroy(gr->graph);
+  retire_pool(ctx, gr->pool);
+  delete gr;
   return HGPU_OK;
 }
 
@@ -287,6 +385,7 @@ int hgpu_shutdown(hgpu_ctx* ctx) {
 
 int hgpu_sync(hgpu_ctx* ctx) {
   if (!ctx) return HGPU_ERR_INVALID;
+  if (int rc = no_capture(ctx, "sync")) return rc;
   (void)hipSetDevice(ctx->device);
   return check_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
 }
@@ -364,6 +463,7 @@ int hgpu_upload(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const 
   if (!ctx || !out) return HGPU_ERR_INVALID;
   *out = nullptr;
   if (dtype_size(dtype) == 0) return fail(ctx, HGPU_ERR_INVALID, "unknown dtype %d", dtype);
+  if (int rc0 = no_capture(ctx, "upload")) return rc0;
   hgpu_array* a = nullptr;
   int rc = new_dense(ctx, dtype, rank, shape, &a);
   if (rc) return rc;
@@ -387,8 +487,22 @@ int hgpu_upload(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const 
   return HGPU_OK;
 }
 
+int hgpu_overwrite(hgpu_ctx* ctx, hgpu_array* a, const void* host) {
+  if (!ctx || !a) return HGPU_ERR_INVALID;
+  if (int rc = no_capture(ctx, "overwrite")) return rc;
+  if (!is_dense(a)) return fail(ctx, HGPU_ERR_INVALID, "overwrite: the array is a strided view");
+  size_t bytes = (size_t)nelem(a) * dtype_size(a->dtype);
+  if (bytes == 0) return HGPU_OK;
+  if (!host) return fail(ctx, HGPU_ERR_INVALID, "null host pointer");
+  LaunchGuard lg(ctx);
+  hipError_t e = hipMemcpyAsync(data_ptr(a), host, bytes, hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  return check_hip(ctx, e, "overwrite");
+}
+
 int hgpu_download(hgpu_ctx* ctx, const hgpu_array* a, void* host) {
   if (!ctx || !a) return HGPU_ERR_INVALID;
+  if (int rc = no_capture(ctx, "download")) return rc;
   int64_t n = nelem(a);
   if (n == 0) return HGPU_OK;
   if (!host) return fail(ctx, HGPU_ERR_INVALID, "null host pointer");
@@ -413,6 +527,7 @@ int hgpu_download(hgpu_ctx* ctx, const hgpu_array* a, void* host) {
 int hgpu_read_scalar(hgpu_ctx* ctx, const hgpu_array* a, void* host) {
   if (!ctx || !a || !host) return HGPU_ERR_INVALID;
   if (nelem(a) != 1) return fail(ctx, HGPU_ERR_INVALID, "read_scalar of an array with %lld elements", (long long)nelem(a));
+  if (int rc = no_capture(ctx, "read_scalar")) return rc;
   LaunchGuard lg(ctx);
   hipError_t e = hipMemcpyAsync(host, data_ptr(a), dtype_size(a->dtype), hipMemcpyDeviceToHost, ctx->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);

@@ -6,6 +6,7 @@
 #include <signal.h>
 #include <unistd.h>
 
+#include <cstddef>
 #include <cstdlib>
 #include <cstring>
 
@@ -119,6 +120,43 @@ int hh_array(hh_val* v, hgpu_array** out) {
 
 int hh_download(hh_ctx* c, hh_val* v, void* host) {
   return guarded(c, [&] { c->be.check(c->be.api->download(c->be.ctx, v->d.primal.h(), host)); });
+}
+struct hh_graph { hgpu_graph* g; };
+static bool has_graphs(const hgpu_api* api) {
+  return api->struct_size >= offsetof(hgpu_api, overwrite) + sizeof(api->overwrite) && api->capture_begin && api->capture_end &&
+         api->graph_launch && api->graph_destroy && api->overwrite;
+}
+int hh_capture_begin(hh_ctx* c) {
+  return guarded(c, [&] {
+    if (!has_graphs(c->be.api)) throw HostError(HGPU_ERR_UNSUPPORTED, "this provider records no graphs");
+    c->be.check(c->be.api->capture_begin(c->be.ctx));
+  });
+}
+int hh_capture_end(hh_ctx* c, hh_graph** out) {
+  return guarded(c, [&] {
+    if (!has_graphs(c->be.api)) throw HostError(HGPU_ERR_UNSUPPORTED, "this provider records no graphs");
+    hgpu_graph* g = nullptr;
+    c->be.check(c->be.api->capture_end(c->be.ctx, &g));
+    *out = new hh_graph{g};
+  });
+}
+int hh_graph_launch(hh_ctx* c, hh_graph* g) {
+  return guarded(c, [&] { c->be.check(c->be.api->graph_launch(g->g)); });
+}
+int hh_graph_free(hh_ctx* c, hh_graph* g) {
+  if (!g) return HGPU_OK;
+  int rc = guarded(c, [&] { c->be.check(c->be.api->graph_destroy(g->g)); });
+  delete g;
+  return rc;
+}
+int hh_force(hh_ctx* c, hh_val* v) {
+  return guarded(c, [&] { (void)v->d.primal.h(); });
+}
+int hh_overwrite(hh_ctx* c, hh_val* v, const void* host) {
+  return guarded(c, [&] {
+    if (!has_graphs(c->be.api)) throw HostError(HGPU_ERR_UNSUPPORTED, "this provider has no overwrite");
+    c->be.check(c->be.api->overwrite(c->be.ctx, v->d.primal.h(), host));
+  });
 }
 int hh_val_rank(hh_val* v) { return v->d.primal.rank(); }
 int hh_val_dtype(hh_val* v) { return v->d.primal.dtype(); }

@@ -37,6 +37,8 @@ SIG = {
     "ix_index0": (I, [P, P, I, PP, PP]), "ix_argminmax": (I, [P, P, I, PP, I, PP]), "ix_free": (I, [P]),
     "ix_is_affine": (I, [P]),
     "tsgather": (I, [P, P, I, LP, I, PP, PP]), "tsscatter": (I, [P, P, I, I, LP, PP, PP]),
+    "capture_begin": (I, [P]), "capture_end": (I, [P, PP]), "graph_launch": (I, [P, P]), "graph_free": (I, [P, P]),
+    "force": (I, [P, P]), "overwrite": (I, [P, P, P]),
 }
 
 _dll = None
@@ -54,6 +56,27 @@ def _lib():
             fn.restype, fn.argtypes = res, args
         _dll = dll
     return _dll
+
+
+def _values(x):
+    if isinstance(x, V):
+        yield x
+    elif isinstance(x, (list, tuple)):
+        for y in x:
+            yield from _values(y)
+
+
+class Graph:
+    def __init__(self, host, h):
+        self.host, self.h = host, h
+
+    def launch(self):
+        self.host.check(self.host.dll.hh_graph_launch(self.host.h, self.h))
+
+    def free(self):
+        if self.h:
+            self.host.check(self.host.dll.hh_graph_free(self.host.h, self.h))
+            self.h = None
 
 
 class Host:
@@ -92,6 +115,26 @@ class Host:
 
     def destroy(self):
         self.dll.hh_destroy(self.h)
+
+    # -- one recorded program, launched many times
+    def capture(self, program):
+        """Records the device work of `program()` (run it once without capture
+        first) and returns (graph, what program returned); every value made
+        inside is refreshed by graph.launch()."""
+        self.check(self.dll.hh_capture_begin(self.h))
+        try:
+            result = program()
+            for v in _values(result):
+                self.check(self.dll.hh_force(self.h, v.h))
+        except BaseException:
+            g = C.c_void_p()
+            self.dll.hh_capture_end(self.h, C.byref(g))
+            if g:
+                self.dll.hh_graph_free(self.h, g)
+            raise
+        g = C.c_void_p()
+        self.check(self.dll.hh_capture_end(self.h, C.byref(g)))
+        return Graph(self, g), result
 
     # -- values
     def concrete(self, x, requires_grad=False):
@@ -232,6 +275,12 @@ class V:
         out = np.empty(self.shape, dtype=_DT2NP[self.dtype])
         self.host.check(self.host.dll.hh_download(self.host.h, self.h, out.ctypes.data_as(C.c_void_p)))
         return out
+
+    def overwrite(self, x):
+        """New contents for an input of a recorded program (same shape and dtype)."""
+        x = np.ascontiguousarray(x, dtype=_DT2NP[self.dtype])
+        assert tuple(x.shape) == tuple(self.shape)
+        self.host.check(self.host.dll.hh_overwrite(self.host.h, self.h, x.ctypes.data_as(C.c_void_p)))
 
     def _o(self, fn, *args):
         return self.host._out(fn, *args)

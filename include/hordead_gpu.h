@@ -272,6 +272,32 @@ int hgpu_scatter_affine(hgpu_ctx* ctx, const hgpu_array* src, int rank_m, int n_
  * with v written at prefix index ix; all zeros when ix is out of bounds. */
 int hgpu_onehot(hgpu_ctx* ctx, const hgpu_array* v, int n, const int64_t* ix, const int64_t* shp, hgpu_array** out);
 
+/* ------------------------------------------------------------- graphs */
+
+/* A gradient program is evaluated again and again on arrays of the same
+ * shapes (ADEngine.hs:266-288, revInterpretArtifact: the artifact is built
+ * once, interpreted per batch).  Between hgpu_capture_begin and
+ * hgpu_capture_end every compute call of this header is RECORDED instead of
+ * executed: the arrays it returns have the right shapes but no contents yet.
+ * hgpu_graph_launch then runs the whole recorded sequence as one submission
+ * (a HIP graph) and refreshes those arrays in place; it may be called any
+ * number of times.  Arrays that existed before the capture are read at every
+ * launch (refresh them with hgpu_overwrite to feed a new batch).
+ * Entry points that need the host -- upload, download, read_scalar,
+ * compare_all, sync -- fail with HGPU_ERR_UNSUPPORTED during a capture: make
+ * constants beforehand.  Memory handed out during a capture stays reserved for
+ * the graph until hgpu_graph_destroy.  One capture at a time per context; the
+ * capturing thread is the only one that may use the context meanwhile. */
+typedef struct hgpu_graph hgpu_graph;
+int hgpu_capture_begin(hgpu_ctx* ctx);
+int hgpu_capture_end(hgpu_ctx* ctx, hgpu_graph** out);
+int hgpu_graph_launch(hgpu_graph* g);
+int hgpu_graph_destroy(hgpu_graph* g);
+/* Replaces the contents of a dense array with host data (same shape and
+ * dtype).  The one exception to "arrays are immutable": meant for the input
+ * arrays of a captured graph, between launches. */
+int hgpu_overwrite(hgpu_ctx* ctx, hgpu_array* a, const void* host);
+
 /* ------------------------------------------------------------- api table */
 
 /* The same entry points as a table of function pointers, so that host code
@@ -319,6 +345,11 @@ typedef struct hgpu_api {
   /* optional (may be NULL): a provider without it gets the operations one by one */
   int (*fused_map)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, const int*, hgpu_array**);
   int (*scatter_affine)(hgpu_ctx*, const hgpu_array*, int, int, const int64_t*, const int64_t*, const int64_t*, hgpu_array**);
+  int (*capture_begin)(hgpu_ctx*);
+  int (*capture_end)(hgpu_ctx*, hgpu_graph**);
+  int (*graph_launch)(hgpu_graph*);
+  int (*graph_destroy)(hgpu_graph*);
+  int (*overwrite)(hgpu_ctx*, hgpu_array*, const void*);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

@@ -55,6 +55,24 @@ int hh_constant(hh_ctx* ctx, int dtype, double value, int rank, const int64_t* s
 /* The primal array of a value (a new reference the caller releases). */
 int hh_array(hh_val* v, hgpu_array** out);
 int hh_download(hh_ctx* ctx, hh_val* v, void* host);
+/* ---- evaluating one gradient program many times (ADEngine.hs:266-288) ----
+ * revInterpretArtifact interprets a gradient artifact that was built once.
+ * Here the operations issued between hh_capture_begin and hh_capture_end are
+ * recorded into a device graph instead of being executed; hh_graph_launch runs
+ * the recording as one submission and refreshes, in place, every value made
+ * inside the capture (results included).  Values that existed before the
+ * capture are the program's inputs: they are read at every launch, and
+ * hh_overwrite replaces their contents between launches.  Run the same
+ * program once without capture first, so that constants and generated kernels
+ * exist (nothing may be uploaded or read back during a capture).
+ * hh_force writes a deferred value out (inside a capture: records that). */
+typedef struct hh_graph hh_graph;
+int hh_capture_begin(hh_ctx* ctx);
+int hh_capture_end(hh_ctx* ctx, hh_graph** out);
+int hh_graph_launch(hh_ctx* ctx, hh_graph* g);
+int hh_graph_free(hh_ctx* ctx, hh_graph* g);
+int hh_force(hh_ctx* ctx, hh_val* v);
+int hh_overwrite(hh_ctx* ctx, hh_val* v, const void* host);
 int hh_val_rank(hh_val* v);
 int hh_val_dtype(hh_val* v);
 int hh_val_shape(hh_val* v, int64_t* shape);

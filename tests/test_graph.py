@@ -1,0 +1,82 @@
+"""A gradient program recorded once and launched many times (GPU only).
+
+Every replay must reproduce the eager result bit for bit: it launches the very
+same kernels on the very same arrays.  Eager work runs between the replays, so
+a block of memory that leaked out of the recording's pool would show up as a
+changed result.
+"""
+import numpy as np
+import pytest
+
+from conftest import capi, pkg
+from test_workloads import MEDIUM, SMALL
+
+H, W = pkg.hostapi, pkg.workloads
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def host():
+    return H.Host()
+
+
+def eager(host, wl, ps, ds):
+    loss, grads = wl.gradient(host, ps, ds)
+    return loss.numpy(), [g.numpy() for g in grads]
+
+
+@pytest.mark.parametrize("name,table", [("c0", SMALL), ("c1", MEDIUM), ("c3", SMALL), ("c3", MEDIUM), ("c4", SMALL), ("c2", MEDIUM)])
+def test_replays_match_eager(host, name, table):
+    mk, kw = table[name]
+    wl = mk(**kw)
+    ps, ds = wl.upload(host)
+    want_loss, want_grads = eager(host, wl, ps, ds)          # also the warm-up run
+    graph, (loss, grads) = host.capture(lambda: wl.gradient(host, ps, ds))
+    other = mk(**kw)
+    ops, ods = other.upload(host)
+    try:
+        for replay in range(3):
+            graph.launch()
+            host.sync()
+            assert np.array_equal(loss.numpy(), want_loss), (name, replay)
+            for g, w in zip(grads, want_grads):
+                assert np.array_equal(g.numpy(), w), (name, replay)
+            eager(host, other, ops, ods)                      # unrelated eager work between replays
+        # new contents for the inputs: the replay follows them
+        new_params = [np.ascontiguousarray(p * 0.5) for p in wl.params]
+        for p, x in zip(ps, new_params):
+            p.overwrite(x)
+        graph.launch()
+        host.sync()
+        got_loss, got_grads = loss.numpy(), [g.numpy() for g in grads]
+        fresh = [host.param(x) for x in new_params]
+        ref_loss, ref_grads = eager(host, wl, fresh, ds)
+        assert np.array_equal(got_loss, ref_loss)
+        for g, w in zip(got_grads, ref_grads):
+            assert np.array_equal(g, w)
+    finally:
+        graph.free()
+
+
+def test_host_calls_refused_while_recording(host):
+    x = host.concrete(np.arange(6.0).reshape(2, 3))
+    y = (x * x).ssum0()
+    y.numpy()
+
+    def program():
+        z = (x * x).ssum0()
+        with pytest.raises(capi.HgpuError) as e:
+            z.numpy()                     # a read-back needs the host
+        assert e.value.code == 4
+        with pytest.raises(capi.HgpuError):
+            host.concrete(np.ones(3))     # so does an upload
+        return z
+
+    graph, z = host.capture(program)
+    graph.launch()
+    host.sync()
+    assert float(z.numpy()) == 55.0
+    graph.free()
+    # the context works as before
+    assert float((x * x).ssum0().numpy()) == 55.0
