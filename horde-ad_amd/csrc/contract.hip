@@ -102,6 +102,33 @@ __global__ void __launch_bounds__(kBlock) k_contract_lane(Dims keep, Dims red, i
   }
 }
 
+// Sum over j = j_first, j_first + 64, ... < j_end of a[j * sa] (* b[j * sb]): four
+// independent accumulators keep four loads per operand in flight.
+template <typename TI, typename A, bool HASB>
+__device__ __forceinline__ A lane_strided_sum(const TI* __restrict__ pa, const TI* __restrict__ pb, int64_t sa, int64_t sb, int64_t j_first, int64_t j_end) {
+  A acc0 = 0, acc1 = 0, acc2 = 0, acc3 = 0;
+  int64_t j = j_first;
+  for (; j + 192 < j_end; j += 256) {
+    A x0 = (A)pa[j * sa], x1 = (A)pa[(j + 64) * sa], x2 = (A)pa[(j + 128) * sa], x3 = (A)pa[(j + 192) * sa];
+    if (HASB) {
+      x0 *= (A)pb[j * sb];
+      x1 *= (A)pb[(j + 64) * sb];
+      x2 *= (A)pb[(j + 128) * sb];
+      x3 *= (A)pb[(j + 192) * sb];
+    }
+    acc0 += x0;
+    acc1 += x1;
+    acc2 += x2;
+    acc3 += x3;
+  }
+  for (; j < j_end; j += 64) {
+    A x = (A)pa[j * sa];
+    if (HASB) x *= (A)pb[j * sb];
+    acc0 += x;
+  }
+  return (acc0 + acc1) + (acc2 + acc3);
+}
+
 // One wavefront per work item.  `red` has its innermost dim split off:
 // Lin = extent, (sa_in, sb_in) = strides; `red` keeps the outer reduced dims
 // with Q = their product.  Chunks split Q when Q > 1, else Lin.
@@ -127,14 +154,50 @@ __global__ void __launch_bounds__(kBlock) k_contract_wave(Dims keep, Dims red, i
       decompose<2>(red, q, ro);
       const TI* pa = a + ko[0] + ro[0];
       const TI* pb = HASB ? b + ko[1] + ro[1] : nullptr;
-      for (int64_t j = j0 + lane; j < j1; j += 64) {
-        A x = (A)pa[j * sa_in];
-        if (HASB) x *= (A)pb[j * sb_in];
-        acc += x;
-      }
+      acc += lane_strided_sum<TI, A, HASB>(pa, pb, sa_in, sb_in, j0 + lane, j1);
     }
     acc = wave_sum<A>(acc);
     if (lane == 0) out[item] = (TO)acc;
+  }
+}
+
+// One block of four wavefronts per output: for a few hundred outputs with a few
+// thousand reduced elements each, where one wavefront per output leaves most of
+// the device idle and splitting into chunks would cost a second launch.  The
+// wavefronts take every fourth outer reduced index (or a quarter of the inner
+// dim when there is no outer one) and combine through LDS in a fixed order.
+template <typename TI, typename TO, bool HASB>
+__global__ void __launch_bounds__(kBlock) k_contract_block(Dims keep, Dims red, int64_t n_out, int64_t Q, int64_t Lin, int64_t sa_in, int64_t sb_in,
+                                                            const TI* __restrict__ a, const TI* __restrict__ b, TO* __restrict__ out) {
+  using A = typename acc_of<TI>::type;
+  __shared__ A part[kBlock / 64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  constexpr int NW = kBlock / 64;
+  for (int64_t o = blockIdx.x; o < n_out; o += gridDim.x) {
+    int64_t ko[2];
+    decompose<2>(keep, o, ko);
+    A acc = 0;
+    if (Q > 1) {
+      for (int64_t q = w; q < Q; q += NW) {
+        int64_t ro[2];
+        decompose<2>(red, q, ro);
+        acc += lane_strided_sum<TI, A, HASB>(a + ko[0] + ro[0], HASB ? b + ko[1] + ro[1] : nullptr, sa_in, sb_in, lane, Lin);
+      }
+    } else {
+      const int64_t quarter = (Lin + NW - 1) / NW;
+      const int64_t j0 = w * quarter, j1 = j0 + quarter < Lin ? j0 + quarter : Lin;
+      acc = lane_strided_sum<TI, A, HASB>(a + ko[0], HASB ? b + ko[1] : nullptr, sa_in, sb_in, j0 + lane, j1);
+    }
+    acc = wave_sum<A>(acc);
+    if (lane == 0) part[w] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      A t = part[0];
+#pragma unroll
+      for (int k = 1; k < NW; ++k) t += part[k];
+      out[o] = (TO)t;
+    }
+    __syncthreads();
   }
 }
 
@@ -258,7 +321,16 @@ int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red
   LaunchGuard lg(ctx, label,
                  (double)n_out * R * sizeof(TI) * (b ? 2 : 1) + (double)n_out * S * sizeof(TO), (double)n_out * R * (b ? 2 : 1));
   int maxb = ctx->num_cu * 8;
-  if (use_wave) {
+  if (use_wave && S == 0) {       // one block per output, no partials
+    Dims red = red_full;
+    int last = red.nd - 1;
+    int64_t Lin = red.shape[last], sa = red.st[0][last], sb = red.st[1][last];
+    int64_t Q = R / Lin;
+    if (red.nd > 1) { red.nd -= 1; } else { red.shape[0] = 1; red.st[0][0] = red.st[1][0] = 0; }
+    unsigned g = (unsigned)(n_out < (int64_t)maxb ? n_out : maxb);
+    if (b) hipLaunchKernelGGL((k_contract_block<TI, TO, true>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red, n_out, Q, Lin, sa, sb, (const TI*)a, (const TI*)b, (TO*)out);
+    else hipLaunchKernelGGL((k_contract_block<TI, TO, false>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red, n_out, Q, Lin, sa, sb, (const TI*)a, (const TI*)nullptr, (TO*)out);
+  } else if (use_wave) {
     Dims red = red_full;
     int last = red.nd - 1;
     int64_t Lin = red.shape[last], sa = red.st[0][last], sb = red.st[1][last];
@@ -302,6 +374,32 @@ int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n
     if (!same_shape(a, b)) return fail(ctx, HGPU_ERR_INVALID, "contract: shapes differ");
   }
   if (a->dtype == HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "contract: Bool arrays have no sum");
+  // A kept dim along which neither operand moves (both replicated) repeats the
+  // same values: compute once without it, replicate the result as a view.
+  {
+    bool repeats = false;
+    int64_t sh1[HGPU_MAX_RANK];
+    for (int i = 0; i < a->rank; ++i) {
+      sh1[i] = a->shape[i];
+      if (i < n_keep && a->shape[i] > 1 && a->strides[i] == 0 && (!b || b->strides[i] == 0)) { sh1[i] = 1; repeats = true; }
+    }
+    bool empty = false;
+    for (int i = 0; i < a->rank; ++i) empty = empty || a->shape[i] == 0;
+    if (repeats && !empty) {
+      hgpu_array* a1 = new_view(ctx, a->buf, a->dtype, a->rank, sh1, a->strides, a->offset);
+      hgpu_array* b1 = b ? new_view(ctx, b->buf, b->dtype, b->rank, sh1, b->strides, b->offset) : nullptr;
+      hgpu_array* small = nullptr;
+      int rc1 = hgpu_contract(ctx, a1, b1, n_keep, &small);
+      hgpu_release(a1);
+      if (b1) hgpu_release(b1);
+      if (rc1) return rc1;
+      int64_t st[HGPU_MAX_RANK];
+      for (int i = 0; i < n_keep; ++i) st[i] = sh1[i] != a->shape[i] ? 0 : small->strides[i];
+      *out = new_view(ctx, small->buf, small->dtype, n_keep, a->shape, st, small->offset);
+      hgpu_release(small);
+      return HGPU_OK;
+    }
+  }
   hgpu_array* o = nullptr;
   int64_t n_out = 1, R = 1;
   for (int i = 0; i < n_keep; ++i) n_out *= a->shape[i];
@@ -344,7 +442,7 @@ int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n
   if (n_out < want_items) {
     S = (want_items + n_out - 1) / n_out;
     int64_t span = use_wave ? ((R / Lin) > 1 ? (R / Lin) : Lin) : R;
-    int64_t per = use_wave ? ((R / Lin) > 1 ? 2048 / (Lin < 2048 ? Lin : 2048) : 2048) : 256;
+    int64_t per = use_wave ? ((R / Lin) > 1 ? 2048 / (Lin < 2048 ? Lin : 2048) : 1024) : 256;
     if (per < 1) per = 1;
     int64_t maxS = span / per;
     if (maxS < 1) maxS = 1;
@@ -353,7 +451,10 @@ int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n
   }
   const void* pa = data_ptr(a);
   const void* pb = b ? data_ptr(b) : nullptr;
-  if (S == 1) {
+  if (use_wave && n_out >= 64 && n_out <= 1024 && R >= 1024 && R <= 65536) {
+    // a few hundred outputs of a few thousand elements: a block per output, one launch
+    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, true, keep, red, n_out, R, 0, pa, pb, data_ptr(o))));
+  } else if (S == 1) {
     HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, use_wave, keep, red, n_out, R, 1, pa, pb, data_ptr(o))));
   } else {
     // stage 1: partials [n_out, S] in the accumulator type; stage 2 sums them.
