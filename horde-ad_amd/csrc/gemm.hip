@@ -153,6 +153,7 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
   p.split = (int)((p.K + p.kchunk - 1) / p.kchunk);
   split = p.split;
   p.a_kc = p.b_kc = 0;
+  p.c_rows_contig = 0;
 
   const size_t es = dtype_size(dtype);
   const int64_t out_n = nelem(out);
@@ -359,6 +360,7 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   bool bkc = along_k(p.k.sb[p.k.nd - 1], p.k.shape[p.k.nd - 1], p.n.sb[p.n.nd - 1]);
   p.a_kc = akc ? 1 : 0;
   p.b_kc = bkc ? 1 : 0;
+  p.c_rows_contig = (p.m.sc[p.m.nd - 1] == 1 && p.n.sc[p.n.nd - 1] != 1 && p.M >= 64) ? 1 : 0;
   bool va, vb;
   {
     va = vector_ok(es, akc ? p.k : p.m, (akc ? p.k.nd : p.m.nd) - 1, akc ? p.k.sa : p.m.sa);

@@ -37,6 +37,7 @@ struct GemmParams {
   int split;          // K chunks
   int64_t kchunk;     // K elements per chunk (multiple of BK)
   int64_t c_split_stride;  // elements between partial outputs
+  int c_rows_contig;       // staged kernel: the output is contiguous along m (and not along n)
   int64_t kmask, ksa, ksb; // K offsets: table[k & kmask] + k * ks; kmask 0 = no table (see KOff)
 };
 
@@ -194,8 +195,12 @@ struct Stager {
 };
 
 // Block tile BM x BN = (WGM * TM * 16) x (WGN * TN * 16).  NBUF LDS buffers.
+// Skinny tiles keep few accumulators: ask for three wavefronts per SIMD there
+// (the loads of one tile are only hidden by the MFMAs of other blocks).
+constexpr int waves_wanted(int tm, int tn, int esize) { return tm * tn * esize <= 32 ? 3 : 1; }
+
 template <typename X, int WGM, int WGN, int TM, int TN, int VA, int VB, int NBUF>
-__global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const typename X::T* __restrict__ A, const typename X::T* __restrict__ B,
+__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_wanted(TM, TN, (int)sizeof(typename X::T)), 8))) k_gemm(GemmParams p, const typename X::T* __restrict__ A, const typename X::T* __restrict__ B,
                                              typename X::T* __restrict__ C, const int64_t* __restrict__ koffA,
                                              const int64_t* __restrict__ koffB) {
   using T = typename X::T;
@@ -276,6 +281,39 @@ __global__ void __launch_bounds__(NT) k_gemm(GemmParams p, const typename X::T* 
   }
 
   T* Cout = C + btc + (int64_t)s * p.c_split_stride;
+  if constexpr (BN == 16 && BM >= 64) {
+    if (p.c_rows_contig) {
+      // A 16-column output that is contiguous along m, not n (a convolution
+      // writing [image, channel, h, w]): the accumulators, whose lanes run
+      // along n, go through LDS once and are stored with lanes along m.
+      T (*Cs)[BM + 1] = As[0];
+      __shared__ int64_t ccol[16];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int r = 0; r < X::NR; ++r) Cs[X::col(lane)][(wm * TM + i) * 16 + X::row(lane, r)] = X::get(acc[i][0], r);
+      if (t < 16) {
+        int64_t n = n0 + t;
+        int64_t oa = 0, ob = 0, oc = 0;
+        if (n < p.N) group_off(p.n, n, &oa, &ob, &oc);
+        ccol[t] = oc;
+      }
+      __syncthreads();
+      constexpr int MG = NT / BM;                           // column groups stored per pass
+      const int ml = t % BM, ng = t / BM;
+      const int64_t m = m0 + ml;
+      if (m < p.M) {
+        int64_t oa, ob, oc;
+        group_off(p.m, m, &oa, &ob, &oc);
+#pragma unroll
+        for (int e = 0; e < 16 / MG; ++e) {
+          const int nl = ng + MG * e;
+          if (n0 + nl < p.N) Cout[oc + ccol[nl]] = Cs[nl][ml];
+        }
+      }
+      return;
+    }
+  }
   int64_t coln[TNB];
   bool colok[TNB];
 #pragma unroll
