@@ -163,6 +163,29 @@ class Host:
         self.check(self.dll.hh_backward(self.h, out.h, dt.h, len(inputs), arr, outs))
         return [V(self, C.c_void_p(o)) for o in outs]
 
+    # -- host loops of the tensor class (the reference's `Concrete` instance runs
+    #    these closures once per index on the host as well)
+    def sfromVector(self, vs):
+        """tsfromVector (OpsConcrete.hs:144-151): stacks values of one shape along a new outermost dim."""
+        out = None
+        for v in vs:
+            row = v.sreshape([1] + list(v.shape))
+            out = row if out is None else out.sappend(row)
+        return out
+
+    def sbuild1(self, k, f):
+        """tsbuild1 (OpsConcrete.hs:1761-1774): [f 0, ..., f (k-1)] stacked; f gets a concrete index."""
+        return self.sfromVector([f(i) for i in range(k)])
+
+    def smapAccumL(self, f, acc0, xs):
+        """tmapAccumL (OpsConcrete.hs:990-1019): threads `acc` through the outermost
+        dim of xs; f(acc, x) -> (acc', y).  Returns (final acc, stacked ys)."""
+        acc, ys = acc0, []
+        for t in range(xs.shape[0]):
+            acc, y = f(acc, xs.sindex([t]))
+            ys.append(y)
+        return acc, self.sfromVector(ys)
+
     # -- index functions
     def ix_space(self, shm):
         return [IxV(self, self._ixo(self.dll.hh_ix_var, len(shm), _larr(shm), d), tuple(shm)) for d in range(len(shm))]

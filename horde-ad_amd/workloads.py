@@ -242,9 +242,27 @@ def c4_rnn(batch=5000, dtype=F32, steps=28, n_in=28, width=128, n_classes=10):
         loss = lossSoftMaxCrossEntropyS(lab, result)
         return host.srepl((), 1.0 / batch, dtype) * loss
 
+    def objective_mapaccum(ps, ds):
+        """The same network as a tmapAccumL over the sequence (the fold form of
+        the reference's recurrent example) instead of an unrolled loop."""
+        xs_, lab = ds
+        wx, ws, b, wx2, ws2, b2, w3, b3 = ps
+        host = wx.host
+
+        def step(s, x):
+            v1 = layer(s.sslice(0, width), x, wx, ws, b)
+            v2 = layer(s.sslice(width, width), v1, wx2, ws2, b2)
+            return v1.sappend(v2), v2
+
+        _, outs = host.smapAccumL(step, host.srepl((2 * width, batch), 0.0, dtype), xs_)
+        result = w3.smatmul2(outs.sindex([steps - 1])) + b3.sreplicate(batch).str_()
+        return host.srepl((), 1.0 / batch, dtype) * lossSoftMaxCrossEntropyS(lab, result)
+
     per_step = 2.0 * batch * (width * n_in + 3 * width * width)
     flops = 3 * steps * per_step + 3 * 2.0 * batch * width * n_classes
-    return Workload("c4_rnn", dtype, batch, params, [xs, labels], objective, flops=flops, bytes_=None)
+    wl = Workload("c4_rnn", dtype, batch, params, [xs, labels], objective, flops=flops, bytes_=None)
+    wl.objective_mapaccum = objective_mapaccum
+    return wl
 
 
 CONFIGS = {"c0": c0_elementwise, "c1": c1_fcnn, "c2": c2_wide, "c3": c3_cnn, "c4": c4_rnn}

@@ -1,0 +1,120 @@
+"""Known answers held by the reference's own tests, for gather / scatter and
+their transposes (test/simplified/TestGatherSimplified.hs).  The programs below
+restate that file's definitions one to one; the expected gradients live in
+tests/golden/gather_scatter_kats.json with the line ranges they were copied
+from.  CPU: host layer on the checker.  GPU: the same on the device.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from conftest import capi, entry, pkg
+
+H = pkg.hostapi
+KATS = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "gather_scatter_kats.json")))
+
+
+# --- the reference's definitions (rgather shm t f: out[m] = t[f m]) ---------
+
+def gatherNested1(t):
+    inner = t.sgather((4,), lambda k3: [k3])
+    return inner.sgather((2,), lambda i2: [i2 + i2, i2])
+
+
+def gather1(t):
+    return t.sslice(0, 4).sgather((2,), lambda i2: [i2 + i2, i2])
+
+
+def gatherNested02(t):
+    inner = t.sgather((2,), lambda k3: [k3 + k3])
+    return inner.sgather((1,), lambda i1: [i1 + i1 + i1])
+
+
+def gatherNested2(t):
+    inner = t.sgather((2, 3, 4), lambda k1, k2, k3: [k1 + k2 + k3])
+    return inner.sgather((2, 3), lambda i1, i2: [i1, i2, i1 + i2, i1])
+
+
+def gather2(t):
+    return t.sgather((2, 3), lambda i1, i2: [i1 + i2 + i1 + i2, i1])
+
+
+def gatherNested12(t):
+    inner = t.sgather((2, 3, 4), lambda k1, k2, k3: [k1 + k2 + k3, k1])
+    return inner.sgather((2,), lambda i1: [i1, i1 + i1])
+
+
+def gather12(t):
+    return t.sgather((2, 4), lambda i1, k3: [i1 + i1 + i1 + k3, i1])
+
+
+def gatherReshape22(t):
+    return t.sreshape([2, 2, 3]).sreshape([3, 1, 1, 4]).sreshape([1, 12, 1]).sreshape([3, 1, 2, 1, 1, 2]).sreshape([2, 6])
+
+
+def scatterNested1(t):
+    inner = t.sscatter(1, (7,), lambda k3: [k3])
+    return inner.sscatter(2, (2,), lambda i1, i2: [i2.quotH(1 + i1)])
+
+
+def scatter1(t):
+    return t.sscatter(2, (2,), lambda i1, i2: [(i2 + 2 * i1).minH(1)])
+
+
+def build_if(host, f, k=5):
+    """rbuild1 k (\\i -> ifH (i >. 2) (f t) (t ! [i]))"""
+    return lambda t: host.sbuild1(k, lambda i: f(t) if i > 2 else t.sindex([i]))
+
+
+def build_scaled(host, f, shape, k=4):
+    """rbuild1 k (\\i -> f (t * rreplicate0N shape (fromIndex i)))"""
+    return lambda t: host.sbuild1(k, lambda i: f(t * host.srepl(shape, float(i))))
+
+
+def build12(host, f):
+    """rindex (rbuild1 5 (\\i -> ifH (i >. 2) (f t) (rtranspose [1,0] $ rreplicate 4 $ t ! [i]))) [1]"""
+    return lambda t: host.sbuild1(5, lambda i: f(t) if i > 2 else t.sindex([i]).sreplicate(4).str_()).sindex([1])
+
+
+def programs(host):
+    return {
+        "gatherNested1": gatherNested1, "gather1": gather1, "gatherNested02": gatherNested02,
+        "gatherNested2": gatherNested2, "gather2": gather2, "gatherNested12": gatherNested12, "gather12": gather12,
+        "gatherReshape22": gatherReshape22, "scatterNested1": scatterNested1, "scatter1": scatter1,
+        "gatherNestedBuild1": build_if(host, gatherNested1), "gatherBuild1": build_if(host, gather1),
+        "scatterNestedBuild1": build_if(host, scatterNested1), "scatterBuild1": build_if(host, scatter1),
+        "gatherNestedBuild2": build_scaled(host, gatherNested2, [7, 2]),
+        "gatherReshapeBuild22": build_scaled(host, gatherReshape22, [6, 2]),
+        "gatherBuild12": build12(host, gather12),
+    }
+
+
+def check_all(host):
+    progs = programs(host)
+    for name, f in progs.items():
+        kat = KATS[name]
+        x = np.array(kat["input"], dtype=np.float64)
+        t = host.param(x)
+        host.tape_reset()
+        t = t.as_input()
+        grad = host.grad(f(t).ssum0(), [t])[0].numpy()
+        want = np.array(kat["expected"]).reshape(x.shape)
+        assert np.allclose(grad, want, rtol=0, atol=1e-10), (name, grad.ravel().tolist())
+    # value equalities of testGatherSimp1/2/12 on the explicit input
+    vals = np.array(KATS["value_chain_input"], dtype=np.float64).reshape(7, 2)
+    v = host.concrete(vals)
+    assert np.array_equal(gatherNested1(v).numpy(), gather1(v).numpy())
+    assert np.array_equal(gatherNested2(v).numpy(), gather2(v).numpy())
+    assert np.array_equal(gatherNested12(v).numpy(), gather12(v).numpy())
+    assert np.array_equal(gatherNested1(v).numpy(), np.array([vals[0, 0], vals[2, 1]]))
+
+
+def test_reference_kats_on_checker():
+    check_all(H.Host(capi.Lib(entry.ORACLE_LIB, "horc_")))
+
+
+@pytest.mark.gpu
+def test_reference_kats_on_device():
+    check_all(H.Host())

@@ -100,6 +100,19 @@ def test_foo_known_answers(host_cpu):
         assert np.allclose(g.numpy(), wv, rtol=1e-13)
 
 
+def test_rnn_as_mapaccum_matches_unrolled(host_cpu):
+    """tmapAccumL (OpsConcrete.hs:990-1019) is a host loop: the fold form of the
+    recurrent objective gives the gradient of the unrolled one."""
+    mk, kw = SMALL["c4"]
+    wl = mk(**kw)
+    loss, grads = run(host_cpu, wl)
+    wl.objective = wl.objective_mapaccum
+    loss2, grads2 = run(host_cpu, wl)
+    assert abs(loss - loss2) <= 1e-6 * abs(loss)
+    for g, g2 in zip(grads, grads2):
+        assert close(g2, g, 1e-5)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("size", ["small", "medium"])
 @pytest.mark.parametrize("name", list(SMALL))
