@@ -118,3 +118,36 @@ def test_reference_kats_on_checker():
 @pytest.mark.gpu
 def test_reference_kats_on_device():
     check_all(H.Host())
+
+
+def conv_vjp_constants(host):
+    """test_conv2dPreservingVjp_dInp / _dKrn (test/simplified/TestConvQuickCheck.hs:351-387):
+    constant arrays A = 1.1 [5,2,4,8], K = -2.2 / 2.2 [7,2,1,3], cotangent B = -3.3
+    [5,7,4,8]; the reference compares against its handwritten derivatives
+    (ibid. :290-349), which on constants are counts of in-bounds window
+    positions: the window extends FORWARD from each output position, so the
+    input's cotangent at column w collects min(w + 1, 3) kernel taps and the
+    kernel's cotangent at tap q collects 8 - q columns."""
+    W = pkg.workloads
+    A = np.full((5, 2, 4, 8), 1.1)
+    B = host.concrete(np.full((5, 7, 4, 8), -3.3))
+    for kval in (-2.2, 2.2):
+        K = np.full((7, 2, 1, 3), kval)
+        host.tape_reset()
+        a, k = host.param(A).as_input(), host.param(K).as_input()
+        y = W.conv2dPreservingS(k, a)
+        assert np.allclose(y.numpy()[0, 0, 0], 2 * 1.1 * kval * np.minimum(8 - np.arange(8), 3), atol=1e-12)
+        d_inp, d_krn = [g.numpy() for g in host.grad(y.sdot0(B), [a, k])]
+        want_inp = np.broadcast_to(-3.3 * kval * 7 * np.minimum(np.arange(8) + 1, 3), (5, 2, 4, 8))
+        want_krn = np.broadcast_to(-3.3 * 1.1 * 5 * 4 * (8 - np.arange(3)), (7, 2, 1, 3))
+        assert np.allclose(d_inp, want_inp, rtol=0, atol=1e-7)
+        assert np.allclose(d_krn, want_krn, rtol=0, atol=1e-7)
+
+
+def test_conv_vjp_constants_on_checker():
+    conv_vjp_constants(H.Host(capi.Lib(entry.ORACLE_LIB, "horc_")))
+
+
+@pytest.mark.gpu
+def test_conv_vjp_constants_on_device():
+    conv_vjp_constants(H.Host())
