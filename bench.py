@@ -31,7 +31,7 @@ import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3}
-MFMA_KERNELS = ("gemm",)          # kernel families priced against the matrix-core peak
+MFMA_KERNELS = ("gemm_f64", "gemm_f32")   # kernel families priced against the matrix-core peak
 DTYPE_NAME = {0: "f64", 1: "f32"}
 # CPU-baseline sample sizes (batch) chosen so the checker runs ~10-30 s in total
 CPU_SAMPLE = {"c0": dict(n=1024, m=1024), "c1": dict(batch=250), "c2": dict(batch=64),
@@ -81,18 +81,39 @@ def time_graph(host, wl, ps, ds, steps, warmup):
 
 
 def profile(capi, host, wl, ps, ds, reps=2):
+    """Per-launch HIP-event timing by the library, one label per kernel and
+    problem shape: {label: (launches, ms, bytes, flops)} per gradient."""
     actx = array_ctx(capi, host)
-    actx.profile(True)
+    actx.check(actx.lib.profile_enable(actx.h, 2))
     for _ in range(reps):
         wl.gradient(host, ps, ds)
         host.sync()
     rep = actx.profile_report()
-    actx.profile(False)
+    actx.check(actx.lib.profile_enable(actx.h, 0))
     return {k: (v[0] / reps, v[1] / reps, v[2] / reps, v[3] / reps) for k, v in rep.items()}
 
 
+def family(label):
+    return label.split("[", 1)[0]
+
+
+def measured_traffic(label):
+    """HBM bytes per launch of a kernel, where a counter run has measured them
+    (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy; the
+    figures and the commands are in profiles/)."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if not os.path.exists(path):
+        return None
+    table = json.load(open(path))
+    for prefix, val in table.items():
+        if not prefix.startswith("_") and label.startswith(prefix):
+            return val
+    return None
+
+
 def roofline_of(rep, dtype_name):
-    """Prices the kernel family with the largest share of device time."""
+    """Prices the kernel (one label = one kernel at one problem shape) with the
+    largest share of device time."""
     if not rep:
         return None, {}
     name = max(rep, key=lambda k: rep[k][1])
@@ -100,16 +121,21 @@ def roofline_of(rep, dtype_name):
     if launches == 0 or ms <= 0:
         return None, {}
     avg_ms = ms / launches
-    if name.startswith(MFMA_KERNELS):
+    if family(name) in MFMA_KERNELS:
         ach = fl / launches / (avg_ms * 1e-3) / 1e12
         peak = MFMA_PEAK_TFLOPS[dtype_name]
-        roof = {"bound": "mfma", "achieved": ach, "peak": peak, "unit": "TFLOP/s", "frac": ach / peak}
+        roof = {"bound": "mfma", "achieved": ach, "peak": peak, "unit": "TFLOP/s", "frac": ach / peak,
+                "algorithmic_gflop_per_launch": fl / launches / 1e9}
     else:
         ach = by / launches / (avg_ms * 1e-3) / 1e9
-        roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS}
+        roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS,
+                "algorithmic_mb_per_launch": by / launches / 1e6}
     roof.update({"kernel": name, "launches_per_step": launches, "avg_launch_ms": avg_ms,
-                 "share_of_device_time": ms / sum(v[1] for v in rep.values()), "traffic": None})
-    shares = {k: round(v[1], 4) for k, v in sorted(rep.items(), key=lambda kv: -kv[1][1])}
+                 "share_of_device_time": ms / sum(v[1] for v in rep.values()), "traffic": measured_traffic(name)})
+    fams = {}
+    for k, v in rep.items():
+        fams[family(k)] = fams.get(family(k), 0.0) + v[1]
+    shares = {k: round(v, 4) for k, v in sorted(fams.items(), key=lambda kv: -kv[1])}
     return roof, shares
 
 
@@ -177,11 +203,15 @@ def main():
         dn = DTYPE_NAME[wl.dtype]
         roof, shares = roofline_of(rep, dn)
         dev_ms = sum(v[1] for v in rep.values())
+        gemm_ms = sum(v[1] for k, v in rep.items() if family(k) in MFMA_KERNELS)
+        gemm_fl = sum(v[3] for k, v in rep.items() if family(k) in MFMA_KERNELS)
         results[key] = {"workload": wl.name, "dtype": dn, "batch": wl.batch, "ms_per_step": sec * 1e3,
                         "samples_per_s": wl.batch / sec, "gradients_per_s": 1.0 / sec, "loss": loss,
                         "ms_per_step_eager": eager_sec * 1e3, "execution": "eager" if args.eager else "recorded graph, one launch per step",
                         "device_ms_per_step": dev_ms, "algorithmic_gflop": wl.flops / 1e9,
-                        "achieved_tflops": wl.flops / sec / 1e12, "roofline": roof, "kernel_ms": shares}
+                        "achieved_tflops": wl.flops / sec / 1e12, "roofline": roof, "kernel_ms": shares,
+                        "all_matrix_products": {"ms": gemm_ms, "tflops": gemm_fl / gemm_ms / 1e9 if gemm_ms > 0 else None,
+                                                "frac_of_peak": gemm_fl / gemm_ms / 1e9 / MFMA_PEAK_TFLOPS[dn] if gemm_ms > 0 else None}}
         if wl.bytes:
             results[key]["algorithmic_gb"] = wl.bytes / 1e9
             results[key]["achieved_gbs_whole_step"] = wl.bytes / sec / 1e9

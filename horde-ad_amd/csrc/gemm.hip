@@ -182,8 +182,9 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
       snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,direct,t%dx%d,k%lld:%lld/%lld]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, (int)split, 16 * tm, 16 * tn, (long long)p.k.shape[p.k.nd - 1], (long long)p.k.sa[p.k.nd - 1], (long long)p.k.sb[p.k.nd - 1]);
       label = ctx->label_pool.insert(buf).first->c_str();
     }
-    LaunchGuard lg(ctx, label, bytes, flops);
+    // the helper launches are timed under their own names, the label times the MFMA kernel alone
     if (p.k.nd > 1) {
+      LaunchGuard lk(ctx, "gemm_k_offsets", (double)Kp * 16, 0);
       hipLaunchKernelGGL(k_koff, dim3((unsigned)((Kp + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, Kp, ka, kb);
       p.kmask = -1;
       p.ksa = p.ksb = 0;
@@ -206,13 +207,16 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
     };
     const bool va = k_vector(pa, p.k.sa, p.m.sa, p.m, p.bt.sa), vb = k_vector(pb, p.k.sb, p.n.sb, p.n, p.bt.sb);
     LaunchArgs la{ctx->stream, -1, tm, tn, va, vb, grid, pa, pb, cdst, ka, kb};
-    if (dtype == HGPU_F64) {
-      launch_f64(p, la);
-      if (split > 1)
+    {
+      LaunchGuard lg(ctx, label, bytes, flops);
+      if (dtype == HGPU_F64) launch_f64(p, la);
+      else launch_f32(p, la);
+    }
+    if (split > 1) {
+      LaunchGuard ls(ctx, "gemm_sum_partials", (double)out_n * (split + 1) * es, (double)out_n * split);
+      if (dtype == HGPU_F64)
         hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, (int)split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
-    } else {
-      launch_f32(p, la);
-      if (split > 1)
+      else
         hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, (int)split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
     }
   }
@@ -376,8 +380,9 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
       snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,%s%s,t%lldx%lld]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, split, akc ? (va ? "K" : "k") : (va ? "M" : "m"), bkc ? (vb ? "K" : "k") : (vb ? "N" : "n"), (long long)BM, (long long)BN);
       label = ctx->label_pool.insert(buf).first->c_str();
     }
-    LaunchGuard lg(ctx, label, bytes, flops);
+    // the helper launches are timed under their own names, the label times the MFMA kernel alone
     if (p.k.nd > 1) {
+      LaunchGuard lk(ctx, "gemm_k_offsets", (double)Kp * 16, 0);
       hipLaunchKernelGGL(k_koff, dim3((unsigned)((Kp + 255) / 256)), dim3(256), 0, ctx->stream, p.k, p.K, Kp, ka, kb);
       p.kmask = -1;
       p.ksa = p.ksb = 0;
@@ -387,17 +392,18 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
       p.ksa = p.k.sa[0];
       p.ksb = p.k.sb[0];
     }
-    if (a->dtype == HGPU_F64) {
-      double* cdst = split > 1 ? (double*)part->ptr : (double*)data_ptr(out);
-      LaunchArgs la{ctx->stream, cfg, 0, 0, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
-      launch_f64(p, la);
-      if (split > 1)
+    void* cdst = split > 1 ? part->ptr : data_ptr(out);
+    LaunchArgs la{ctx->stream, cfg, 0, 0, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
+    {
+      LaunchGuard lg(ctx, label, bytes, flops);
+      if (a->dtype == HGPU_F64) launch_f64(p, la);
+      else launch_f32(p, la);
+    }
+    if (split > 1) {
+      LaunchGuard ls(ctx, "gemm_sum_partials", (double)out_n * (split + 1) * es, (double)out_n * split);
+      if (a->dtype == HGPU_F64)
         hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
-    } else {
-      float* cdst = split > 1 ? (float*)part->ptr : (float*)data_ptr(out);
-      LaunchArgs la{ctx->stream, cfg, 0, 0, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
-      launch_f32(p, la);
-      if (split > 1)
+      else
         hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
     }
   }
