@@ -247,13 +247,53 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   vec = (int)(16 / widest);
   if (!all_simple) vec = 1;
 
+  // general views: the dims merged jointly over all inputs.  For large arrays
+  // the merged shape and strides are compiled into the kernel (a division by a
+  // constant is a multiplication; 32-bit index arithmetic), one kernel per
+  // layout; small ones share a kernel that takes them as an argument.
+  FDims fd;
+  fd.nd = 0;
+  if (!all_simple) {
+    const int64_t* sts[kMaxIn];
+    for (int i = 0; i < n_in; ++i) sts[i] = in[i]->strides;
+    // merge dims jointly over all inputs
+    fd.nd = 0;
+    for (int d = 0; d < a0->rank; ++d) {
+      if (a0->shape[d] == 1) continue;
+      bool merged = false;
+      if (fd.nd > 0) {
+        int p = fd.nd - 1;
+        bool ok = true;
+        for (int k = 0; k < n_in; ++k)
+          if (fd.st[k][p] != sts[k][d] * a0->shape[d]) { ok = false; break; }
+        if (ok) {
+          fd.shape[p] *= a0->shape[d];
+          for (int k = 0; k < n_in; ++k) fd.st[k][p] = sts[k][d];
+          merged = true;
+        }
+      }
+      if (!merged) {
+        if (fd.nd == HG_KDIMS) { release_all(); return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map: more than %d merged dims", HG_KDIMS); }
+        fd.shape[fd.nd] = a0->shape[d];
+        for (int k = 0; k < n_in; ++k) fd.st[k][fd.nd] = sts[k][d];
+        fd.nd++;
+      }
+    }
+    if (fd.nd == 0) {
+      fd.nd = 1;
+      fd.shape[0] = 1;
+      for (int k = 0; k < n_in; ++k) fd.st[k][0] = 0;
+    }
+  }
+  const bool bake = !all_simple && n >= (1 << 18) && n < (1LL << 31);
+
   // ---- source
   std::ostringstream s;
   s << kPrelude;
   if (!all_simple) s << "struct FDims { int nd; i64 shape[" << HG_KDIMS << "]; i64 st[" << kMaxIn << "][" << HG_KDIMS << "]; };\n";
   s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
   s << "extern \"C\" __global__ void __launch_bounds__(256) fused_map(i64 n";
-  if (!all_simple) s << ", FDims d";
+  if (!all_simple && !bake) s << ", FDims d";
   for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
   for (int o = 0; o < n_out; ++o) s << ", " << ctype(res[(size_t)o]->dtype) << "* __restrict__ o" << o;
   s << ") {\n";
@@ -306,6 +346,28 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     }
     emit_program("    ", "_t");
     for (int o = 0; o < n_out; ++o) s << "    o" << o << "[t] = v" << out_slots[o] << "_t;\n";
+    s << "  }\n";
+  } else if (bake) {
+    s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {\n";
+    s << "    unsigned r = (unsigned)i;\n";
+    for (int q = fd.nd - 1; q >= 0; --q) {
+      if (q > 0) s << "    const unsigned c" << q << " = r % " << fd.shape[q] << "u; r /= " << fd.shape[q] << "u;\n";
+      else s << "    const unsigned c0 = r;\n";
+    }
+    for (int i = 0; i < n_in; ++i) {
+      if (layout[(size_t)i] == 's') continue;
+      s << "    const i64 off" << i << " = 0";
+      for (int q = 0; q < fd.nd; ++q)
+        if (fd.st[i][q] != 0) s << " + (i64)c" << q << " * " << fd.st[i][q] << "ll";
+      s << ";\n";
+    }
+    for (int i = 0; i < n_in; ++i) {
+      s << "    const " << ctype(in[i]->dtype) << " v" << i << "_g = ";
+      if (layout[(size_t)i] == 's') s << "s" << i; else s << "i" << i << "[off" << i << "]";
+      s << ";\n";
+    }
+    emit_program("    ", "_g");
+    for (int o = 0; o < n_out; ++o) s << "    o" << o << "[i] = v" << out_slots[o] << "_g;\n";
     s << "  }\n";
   } else {
     s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {\n";
@@ -361,45 +423,12 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   for (int o = 0; o < n_out; ++o) bytes += (double)n * dtype_size(res[(size_t)o]->dtype);
   if (lg.timed) { ctx->prof.back().bytes = bytes; ctx->prof.back().flops = (double)n * n_instr; }
 
-  FDims fd;
   std::vector<void*> args;
   int64_t nn = n;
   args.push_back(&nn);
   std::vector<const void*> ptrs((size_t)n_in);
   std::vector<void*> optrs((size_t)n_out);
-  if (!all_simple) {
-    const int64_t* sts[kMaxIn];
-    for (int i = 0; i < n_in; ++i) sts[i] = in[i]->strides;
-    // merge dims jointly over all inputs
-    fd.nd = 0;
-    for (int d = 0; d < a0->rank; ++d) {
-      if (a0->shape[d] == 1) continue;
-      bool merged = false;
-      if (fd.nd > 0) {
-        int p = fd.nd - 1;
-        bool ok = true;
-        for (int k = 0; k < n_in; ++k)
-          if (fd.st[k][p] != sts[k][d] * a0->shape[d]) { ok = false; break; }
-        if (ok) {
-          fd.shape[p] *= a0->shape[d];
-          for (int k = 0; k < n_in; ++k) fd.st[k][p] = sts[k][d];
-          merged = true;
-        }
-      }
-      if (!merged) {
-        if (fd.nd == HG_KDIMS) { release_all(); return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map: more than %d merged dims", HG_KDIMS); }
-        fd.shape[fd.nd] = a0->shape[d];
-        for (int k = 0; k < n_in; ++k) fd.st[k][fd.nd] = sts[k][d];
-        fd.nd++;
-      }
-    }
-    if (fd.nd == 0) {
-      fd.nd = 1;
-      fd.shape[0] = 1;
-      for (int k = 0; k < n_in; ++k) fd.st[k][0] = 0;
-    }
-    args.push_back(&fd);
-  }
+  if (!all_simple && !bake) args.push_back(&fd);
   for (int i = 0; i < n_in; ++i) { ptrs[(size_t)i] = data_ptr(in[i]); args.push_back(&ptrs[(size_t)i]); }
   for (int o = 0; o < n_out; ++o) { optrs[(size_t)o] = data_ptr(res[(size_t)o]); args.push_back(&optrs[(size_t)o]); }
   int64_t work = all_simple ? (n + vec - 1) / vec : n;
