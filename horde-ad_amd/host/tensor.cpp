@@ -919,6 +919,49 @@ T tsscatter(const T& src, int rank_m, const Shape& shp, const std::vector<Ix>& i
   Shape shm(ssh.begin(), ssh.begin() + rank_m);
   check_ix(shm, ix);
   Backend* be = src.be();
+  // "Write each position's value at a data-dependent place of a new small dim"
+  // (the adjoint of taking the maximum of a window): every component but the
+  // last is the position variable of its own dim.  Then
+  //   out[m.., e, n..] = (last(m) == e) ? src[m.., n..] : 0,
+  // an elementwise expression: no zero fill, no index traffic, and it fuses
+  // with whatever consumes it.  Out-of-bounds places match no e, as they must.
+  if (fuses(be) && (size_t)rank_m + 1 == ix.size() && rank_m > 0 && src.size() > 0 && !ix.back().affine && shp.back() > 0) {
+    bool identity = true;
+    for (size_t j = 0; j + 1 < ix.size() && identity; ++j) {
+      const Ix& x = ix[j];
+      identity = x.affine && x.c0 == 0 && shp[j] == shm[j];
+      for (size_t d = 0; d < x.coef.size() && identity; ++d) identity = x.coef[d] == (d == j ? 1 : 0);
+    }
+    if (identity) {
+      const int64_t E = shp.back();
+      const size_t rm = (size_t)rank_m, rank_n = ssh.size() - rm;
+      Shape osh(shm);
+      osh.push_back(E);
+      osh.insert(osh.end(), ssh.begin() + rank_m, ssh.end());
+      auto spread = [&](const T& a, size_t lead, bool has_e) {     // a: [lead dims of osh] (+ [E]) -> shape osh, missing dims replicated
+        Shape ast = a.strides(), st(osh.size(), 0);
+        for (size_t d = 0; d < lead; ++d) st[d] = ast[d];
+        if (has_e) st[rm] = ast[lead];
+        return as_strided(a, osh, st, 0);
+      };
+      T srcv;
+      {
+        Shape ast = src.strides(), st(osh.size(), 0);
+        for (size_t d = 0; d < rm; ++d) st[d] = ast[d];
+        for (size_t d = 0; d < rank_n; ++d) st[rm + 1 + d] = ast[rm + d];
+        srcv = as_strided(src, osh, st, 0);
+      }
+      T where = spread(ix_array(be, ix.back()), rm, false);
+      T which;
+      {
+        T io = iota(be, E, HGPU_I64);
+        Shape st(osh.size(), 0);
+        st[rm] = 1;
+        which = as_strided(io, osh, st, 0);
+      }
+      return select(compare(HGPU_EQ, which, where), srcv, zeros(be, src.dtype(), osh));
+    }
+  }
   bool injective = provably_injective(shm, ix);
   if (!injective && all_affine(ix) && src.size() > 0) {
     T r = scatter_as_contraction(src, rank_m, shp, ix);
