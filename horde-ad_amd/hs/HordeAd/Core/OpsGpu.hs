@@ -11,7 +11,7 @@
 -- methods are the same calls with shapes taken from 'gpuShape' at run time and
 -- are omitted from this excerpt.  Not compiled in this repository's build
 -- environment (no GHC there).
-module HordeAd.Core.OpsGpu (revInterpretArtifactGpu) where
+module HordeAd.Core.OpsGpu (revInterpretArtifactGpu, recordArtifactGpu) where
 
 import Data.Int (Int64)
 import Foreign
@@ -154,3 +154,20 @@ revInterpretArtifactGpu AstArtifactRev{..} parameters mdt =
         Nothing -> extendEnv artVarDtRev (treplTarget 1 azftk) env
         Just dt -> extendEnv artVarDtRev dt env
   in (interpretAstFull envDt artDerivativeRev, interpretAstFull env artPrimalRev)
+
+
+-- | The same artifact recorded once as a device graph: returns an action that
+-- re-runs the whole gradient in one submission, refreshing (in place) the
+-- arrays behind the returned values.  Call 'revInterpretArtifactGpu' once
+-- beforehand so that constants and generated kernels exist; feed new inputs
+-- with @hh_overwrite@ on the arrays of @parameters@.
+recordArtifactGpu
+  :: AstArtifactRev x z -> Gpu x -> Maybe (Gpu (ADTensorKind z))
+  -> IO ((Gpu (ADTensorKind x), Gpu z), IO ())
+recordArtifactGpu art parameters mdt = do
+  ctx <- theCtx
+  c_hh_capture_begin ctx >>= check ctx
+  let r@(g, v) = revInterpretArtifactGpu art parameters mdt
+  forceGpu ctx g >> forceGpu ctx v          -- hh_force on every array of the results
+  gr <- alloca $ \o -> c_hh_capture_end ctx o >>= check ctx >> peek o
+  pure (r, c_hh_graph_launch ctx gr >>= check ctx)

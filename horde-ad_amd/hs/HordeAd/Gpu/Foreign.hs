@@ -10,6 +10,7 @@
 module HordeAd.Gpu.Foreign
   ( Ctx, Val, Ix, ValPtr, IxPtr
   , withGpu, theCtx, check
+  , Graph, c_hh_capture_begin, c_hh_capture_end, c_hh_graph_launch, c_hh_graph_free, c_hh_force, c_hh_overwrite
   , c_hh_upload, c_hh_download, c_hh_constant, c_hh_val_rank, c_hh_val_shape
   , c_hh_ewise1, c_hh_ewise2, c_hh_compare, c_hh_compare_all, c_hh_select
   , c_hh_convert, c_hh_tssumN, c_hh_tssum0, c_hh_tsdot0, c_hh_tsdot1In
@@ -42,6 +43,16 @@ foreign import ccall unsafe "hh_last_error" c_hh_last_error :: Ptr Ctx -> IO CSt
 foreign import ccall safe "hh_upload" c_hh_upload
   :: Ptr Ctx -> CInt -> CInt -> Ptr Int64 -> Ptr () -> CInt -> Ptr (Ptr Val) -> IO CInt
 foreign import ccall safe "hh_download" c_hh_download :: Ptr Ctx -> Ptr Val -> Ptr () -> IO CInt
+
+-- One gradient program recorded as a device graph and launched per batch
+-- (include/hordead_host.h, "evaluating one gradient program many times").
+data Graph
+foreign import ccall safe "hh_capture_begin" c_hh_capture_begin :: Ptr Ctx -> IO CInt
+foreign import ccall safe "hh_capture_end" c_hh_capture_end :: Ptr Ctx -> Ptr (Ptr Graph) -> IO CInt
+foreign import ccall safe "hh_graph_launch" c_hh_graph_launch :: Ptr Ctx -> Ptr Graph -> IO CInt
+foreign import ccall safe "hh_graph_free" c_hh_graph_free :: Ptr Ctx -> Ptr Graph -> IO CInt
+foreign import ccall safe "hh_force" c_hh_force :: Ptr Ctx -> Ptr Val -> IO CInt
+foreign import ccall safe "hh_overwrite" c_hh_overwrite :: Ptr Ctx -> Ptr Val -> Ptr () -> IO CInt
 foreign import ccall safe "hh_constant" c_hh_constant
   :: Ptr Ctx -> CInt -> CDouble -> CInt -> Ptr Int64 -> Ptr (Ptr Val) -> IO CInt
 foreign import ccall unsafe "hh_val_rank" c_hh_val_rank :: Ptr Val -> IO CInt
