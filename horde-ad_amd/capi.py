@@ -49,6 +49,7 @@ SIGNATURES = {
     "gather": (I, [P, P, I, PP, I, LP, PP]), "scatter_add": (I, [P, P, I, PP, I, LP, I, PP]),
     "onehot": (I, [P, P, I, LP, LP, PP]), "get_api": (P, []),
     "scatter_affine": (I, [P, P, I, I, LP, LP, LP, PP]),
+    "contract_sum": (I, [P, I, PP, PP, I, PP]),
 }
 # exported by the GPU library only
 GPU_ONLY = {
@@ -163,6 +164,11 @@ class Ctx:
     def gather(self, src, ix, shm):
         arr = (C.c_void_p * max(len(ix), 1))(*[p.h for p in ix])
         return self._out(self.lib.gather, src.h, len(ix), arr, len(shm), _larr(shm))
+
+    def contract_sum(self, pairs, n_keep):
+        a = (C.c_void_p * len(pairs))(*[x.h for x, _ in pairs])
+        b = (C.c_void_p * len(pairs))(*[y.h for _, y in pairs])
+        return self._out(self.lib.contract_sum, len(pairs), a, b, n_keep)
 
     def scatter_affine(self, src, rank_m, c0, coef, shp):
         """coef[d][j]: coefficient of position variable d in index component j."""

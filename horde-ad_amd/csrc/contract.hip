@@ -21,7 +21,9 @@ using namespace hg;
 namespace hg {
 // gemm.hip: returns HGPU_OK and sets *handled when the contraction was
 // recognised as a matrix product and executed on the matrix cores.
-int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled);
+int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled,
+             int n_terms = 0, const hgpu_array* const* as = nullptr, const hgpu_array* const* bs = nullptr);
+constexpr int kGemmMaxTerms = 32;   // products one launch of try_gemm sums (kMaxTerms of the kernels)
 }
 
 namespace {
@@ -362,9 +364,70 @@ int64_t min_abs_nonzero(const Dims& d, int dim) {
   return m;
 }
 
+// *acc += x, taking over x (the first term becomes the accumulator).
+int add_into(hgpu_ctx* ctx, hgpu_array** acc, hgpu_array* x) {
+  if (!*acc) { *acc = x; return HGPU_OK; }
+  hgpu_array* sum = nullptr;
+  int rc = hgpu_ewise2(ctx, HGPU_ADD, *acc, x, &sum);
+  hgpu_release(*acc);
+  hgpu_release(x);
+  *acc = rc ? nullptr : sum;
+  return rc;
+}
+
 }  // namespace
 
 extern "C" {
+
+int hgpu_contract_sum(hgpu_ctx* ctx, int n, const hgpu_array* const* as, const hgpu_array* const* bs, int n_keep, hgpu_array** out) {
+  if (!ctx || !as || !bs || !out || n < 1) return HGPU_ERR_INVALID;
+  for (int t = 0; t < n; ++t) {
+    if (!as[t] || !bs[t]) return HGPU_ERR_INVALID;
+    if (as[t]->dtype != as[0]->dtype || bs[t]->dtype != as[0]->dtype) return fail(ctx, HGPU_ERR_INVALID, "contract_sum: dtypes differ");
+    if (!same_shape(as[t], as[0]) || !same_shape(bs[t], as[0])) return fail(ctx, HGPU_ERR_INVALID, "contract_sum: shapes differ");
+  }
+  const hgpu_array* a = as[0];
+  if (n_keep < 0 || n_keep > a->rank) return fail(ctx, HGPU_ERR_INVALID, "contract_sum: n_keep %d of rank %d", n_keep, a->rank);
+  if (n == 1) return hgpu_contract(ctx, as[0], bs[0], n_keep, out);
+  // Terms of one layout go out together, 32 to a launch: when such a group is a
+  // matrix product the K chunks of all its terms are summed in one fixed order
+  // by one kernel.  Groups are formed in order of first appearance and their
+  // results added in that order.
+  const bool groupable = nelem(a) > 0 && (a->dtype == HGPU_F64 || a->dtype == HGPU_F32);
+  auto same_layout = [&](int s, int t) {
+    for (int d = 0; d < a->rank; ++d)
+      if (as[s]->strides[d] != as[t]->strides[d] || bs[s]->strides[d] != bs[t]->strides[d]) return false;
+    return true;
+  };
+  std::vector<char> taken((size_t)n, 0);
+  hgpu_array* acc = nullptr;
+  for (int t0 = 0; t0 < n; ++t0) {
+    if (taken[(size_t)t0]) continue;
+    std::vector<const hgpu_array*> ga{as[t0]}, gb{bs[t0]};
+    taken[(size_t)t0] = 1;
+    for (int t = t0 + 1; t < n && groupable && ga.size() < (size_t)kGemmMaxTerms; ++t)
+      if (!taken[(size_t)t] && same_layout(t0, t)) { ga.push_back(as[t]); gb.push_back(bs[t]); taken[(size_t)t] = 1; }
+    hgpu_array* part = nullptr;
+    int rc = HGPU_OK;
+    size_t done = 0;
+    if (ga.size() > 1) {
+      rc = new_dense(ctx, a->dtype, n_keep, a->shape, &part);
+      bool handled = false;
+      if (!rc) rc = try_gemm(ctx, ga[0], gb[0], n_keep, part, &handled, (int)ga.size(), ga.data(), gb.data());
+      if (rc || !handled) { if (part) hgpu_release(part); part = nullptr; }
+      else done = ga.size();
+    }
+    for (size_t t = done; t < ga.size() && !rc; ++t) {   // not a matrix product (or a single term): one by one
+      hgpu_array* one = nullptr;
+      rc = hgpu_contract(ctx, ga[t], gb[t], n_keep, &one);
+      if (!rc) rc = add_into(ctx, &part, one);
+    }
+    if (!rc) rc = add_into(ctx, &acc, part), part = nullptr;
+    if (rc) { if (part) hgpu_release(part); if (acc) hgpu_release(acc); return rc; }
+  }
+  *out = acc;
+  return HGPU_OK;
+}
 
 int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array** out) {
   if (!ctx || !a || !out) return HGPU_ERR_INVALID;

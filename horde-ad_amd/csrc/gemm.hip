@@ -125,11 +125,12 @@ bool vector_ok(size_t es, const Group& run, int run_dim, const int64_t* run_st) 
   return run_st[run_dim] == 1 && run.shape[run_dim] % v == 0;
 }
 // Products with at most 32 rows or columns: the LDS-free kernel, the small side as N.
-int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled) {
+int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled, int n_terms) {
   if (p.N > 32) {   // swap the roles of the operands: C^T = B A^T
     std::swap(p.m, p.n);
     std::swap(p.M, p.N);
     std::swap(pa, pb);
+    for (int t = 0; t < n_terms; ++t) std::swap(p.a_term[t], p.b_term[t]);
     for (Group* g : {&p.m, &p.n, &p.k, &p.bt})
       for (int i = 0; i < GD; ++i) std::swap(g->sa[i], g->sb[i]);
   }
@@ -140,9 +141,10 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
   // measured slower: set-up and partial sums per wavefront), chunks of at least 64
   const int64_t want = (int64_t)ctx->num_cu * 4;
   const int64_t out_elems = p.M * p.N * p.BT;
+  const int64_t nt = n_terms > 0 ? n_terms : 1;      // products summed by this launch
   int64_t split = 1;
-  if (tiles * p.BT * 2 <= want && p.K >= 128) {
-    split = (want + tiles * p.BT - 1) / (tiles * p.BT);
+  if (tiles * p.BT * nt * 2 <= want && p.K >= 128) {
+    split = (want + tiles * p.BT * nt - 1) / (tiles * p.BT * nt);
     int64_t cap = (int64_t)((double)(p.M + p.N) * p.K * p.BT / (2.0 * out_elems));   // partials stay small next to the operands
     if (cap > 4096) cap = 4096;
     if (split > cap) split = cap;
@@ -150,7 +152,9 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
     if (split < 1) split = 1;
   }
   p.kchunk = ((p.K + split - 1) / split + 15) / 16 * 16;
-  p.split = (int)((p.K + p.kchunk - 1) / p.kchunk);
+  p.term_split = (int)((p.K + p.kchunk - 1) / p.kchunk);
+  p.n_terms = n_terms;
+  p.split = (int)(p.term_split * nt);                // K chunks of all terms
   split = p.split;
   p.a_kc = p.b_kc = 0;
   p.c_rows_contig = 0;
@@ -174,8 +178,8 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
   int64_t* kb = ka + Kp;
   dim3 grid((unsigned)((tiles * split + 3) / 4), 1, (unsigned)p.BT);
   {
-    double flops = 2.0 * p.M * p.N * p.K * p.BT;
-    double bytes = ((double)p.M * p.K + (double)p.N * p.K + (double)p.M * p.N) * p.BT * es;
+    double flops = 2.0 * p.M * p.N * p.K * p.BT * nt;
+    double bytes = (((double)p.M * p.K + (double)p.N * p.K) * nt + (double)p.M * p.N) * p.BT * es;
     const char* label = dtype == HGPU_F64 ? "gemm_f64" : "gemm_f32";
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[128];
@@ -232,7 +236,10 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
 
 namespace hg {
 
-int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled) {
+int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled,
+             int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs) {
+  // n_terms > 0: out = sum_t contract(as[t], bs[t]); all terms have the shapes,
+  // strides and dtype of a = as[0], b = bs[0] (the caller has checked).
   *handled = false;
   if (!b) return HGPU_OK;
   if (a->dtype != HGPU_F64 && a->dtype != HGPU_F32) return HGPU_OK;
@@ -293,7 +300,11 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   const void* pb = data_ptr(b);
   // A small output under a long K (weight gradients, the last layer of a
   // classifier) is better served by independent wavefronts than by staged tiles.
-  if ((p.M <= 32 || p.N <= 32) && p.M <= 1024 && p.N <= 1024) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled);
+  static_assert(kMaxTerms == 32, "hgpu_contract_sum groups 32 terms to a launch");
+  if (n_terms > kMaxTerms) return HGPU_OK;
+  p.n_terms = n_terms;
+  for (int t = 0; t < n_terms; ++t) { p.a_term[t] = data_ptr(as[t]); p.b_term[t] = data_ptr(bs[t]); }
+  if ((p.M <= 32 || p.N <= 32) && p.M <= 1024 && p.N <= 1024) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled, n_terms);
 
   // tile shape: least padded work per unit of efficiency
   int cfg = 0;
@@ -319,8 +330,9 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   int split = 1;
   int64_t want = (int64_t)ctx->num_cu * 2;
   int64_t out_elems = p.M * p.N * p.BT;
-  if (tiles * p.BT < want && p.K >= 8 * BK) {
-    split = (int)((want + tiles * p.BT - 1) / (tiles * p.BT));
+  const int64_t nt = n_terms > 0 ? n_terms : 1;      // products summed by this launch
+  if (tiles * p.BT * nt < want && p.K >= 8 * BK) {
+    split = (int)((want + tiles * p.BT * nt - 1) / (tiles * p.BT * nt));
     int64_t max_split = p.K / (4 * BK);
     if (split > max_split) split = (int)max_split;
     // the partial products must stay small next to the operands
@@ -330,10 +342,11 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     if (split > cap) split = (int)cap;
     if (split < 1) split = 1;
   }
-  p.split = split;
   p.kchunk = ((p.K + split - 1) / split + BK - 1) / BK * BK;
-  p.split = (int)((p.K + p.kchunk - 1) / p.kchunk);
+  p.term_split = (int)((p.K + p.kchunk - 1) / p.kchunk);
+  p.split = (int)(p.term_split * nt);                // K chunks of all terms
   split = p.split;
+  if (split > 65535) return HGPU_OK;
 
   size_t es = dtype_size(a->dtype);
   int64_t out_n = nelem(out);
@@ -372,8 +385,8 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   }
   dim3 grid((unsigned)tiles, (unsigned)split, (unsigned)p.BT);
   {
-    double flops = 2.0 * p.M * p.N * p.K * p.BT;
-    double bytes = ((double)p.M * p.K + (double)p.N * p.K + (double)p.M * p.N) * p.BT * es;
+    double flops = 2.0 * p.M * p.N * p.K * p.BT * nt;
+    double bytes = (((double)p.M * p.K + (double)p.N * p.K) * nt + (double)p.M * p.N) * p.BT * es;
     const char* label = a->dtype == HGPU_F64 ? "gemm_f64" : "gemm_f32";
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[128];

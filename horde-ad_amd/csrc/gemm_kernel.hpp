@@ -23,6 +23,7 @@ namespace gemm {
 
 constexpr int BK = 16, NT = 256;
 constexpr int GD = 5;  // dims per index group after merging
+constexpr int kMaxTerms = 32;   // products summed by one launch (hgpu_contract_sum)
 
 struct Group {
   int nd;
@@ -37,6 +38,13 @@ struct GemmParams {
   int split;          // K chunks
   int64_t kchunk;     // K elements per chunk (multiple of BK)
   int64_t c_split_stride;  // elements between partial outputs
+  // A sum of products of one shape and layout (hgpu_contract_sum): the K chunks
+  // of all terms are enumerated together, chunk index = term * term_split + chunk
+  // within the term, and term t reads a_term[t] / b_term[t].  n_terms == 0: one
+  // product, the operands are the kernel's pointer arguments.
+  int n_terms, term_split;
+  const void* a_term[kMaxTerms];
+  const void* b_term[kMaxTerms];
   int c_rows_contig;       // staged kernel: the output is contiguous along m (and not along n)
   int64_t kmask, ksa, ksb; // K offsets: table[k & kmask] + k * ks; kmask 0 = no table (see KOff)
 };
@@ -227,7 +235,14 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
   int64_t bta, btb, btc;
   group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
   const int s = blockIdx.y;
-  const int64_t kbeg = (int64_t)s * p.kchunk;
+  int sk = s;                              // chunk within its term
+  if (p.n_terms > 0) {
+    const int term = s / p.term_split;
+    sk = s - term * p.term_split;
+    A = (const T*)p.a_term[term];
+    B = (const T*)p.b_term[term];
+  }
+  const int64_t kbeg = (int64_t)sk * p.kchunk;
   int64_t kend = kbeg + p.kchunk;
   if (kend > p.K) kend = p.K;
 
@@ -379,7 +394,14 @@ __global__ void __launch_bounds__(NT) k_gemm_direct(GemmParams p, const typename
 
   int64_t bta, btb, btc;
   group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
-  const int64_t kbeg = s * p.kchunk;
+  int64_t sk = s;                          // chunk within its term
+  if (p.n_terms > 0) {
+    const int64_t term = s / p.term_split;
+    sk = s - term * p.term_split;
+    A = (const T*)p.a_term[term];
+    B = (const T*)p.b_term[term];
+  }
+  const int64_t kbeg = sk * p.kchunk;
   int64_t kend = kbeg + p.kchunk;
   if (kend > p.K) kend = p.K;
 

@@ -26,7 +26,7 @@ int Tape::push(std::function<void(const T&, std::vector<T>&)> f) {
 static void accum(std::vector<T>& slots, int node, const T& cot) {
   if (node < 0) return;
   T& s = slots[(size_t)node];
-  s = s.valid() ? ewise2(HGPU_ADD, s, cot) : cot;
+  s = s.valid() ? add_cotangents(s, cot) : cot;
 }
 
 std::vector<T> Tape::backward(const D& out, const T& dt, const std::vector<D>& inputs) {

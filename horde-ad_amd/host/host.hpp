@@ -54,6 +54,15 @@ struct ArrHolder {
   // convolution never writes its patch gradient to memory).
   std::shared_ptr<ArrHolder> fa, fb;
   int keep = -1;
+  // Further (fa, fb) pairs of a pending SUM of contractions of one shape (the
+  // cotangent of a parameter used once per step of an unrolled recurrence):
+  // written out by one grouped launch when the provider has contract_sum.
+  std::vector<std::pair<std::shared_ptr<ArrHolder>, std::shared_ptr<ArrHolder>>> more;
+  // A pending contraction that is a transpose of another pending contraction
+  // remembers it: if anyone else still wants the original, the original is
+  // computed once and this one becomes a view of it.
+  std::shared_ptr<ArrHolder> origin;
+  std::vector<int> origin_perm;
   // A pending ELEMENTWISE operation (h == nullptr): kind/op as in
   // hgpu_fused_instr, operands fa, fb, fc.  Chains of them are handed to the
   // provider's fused_map as one program when the value is first needed as an
@@ -84,7 +93,8 @@ class T {
   }
   bool pending_expr() const { return p_ && !p_->h && p_->ekind >= 0; }
   bool pending_product() const { return pending_expr() && p_->ekind == HGPU_FUSED_OP2 && p_->eop == HGPU_MUL; }
-  bool pending_contraction() const { return p_ && !p_->h && p_->ekind < 0 && p_->fa && p_->keep >= 0; }
+  bool contraction_like() const { return p_ && !p_->h && p_->ekind < 0 && p_->fa && p_->keep >= 0; }
+  bool pending_contraction() const { return contraction_like() && p_->more.empty(); }   // a single one: open to rewrites
   int pending_keep() const { return p_->keep; }
   T factor_a() const { return T(p_->fa); }
   T factor_b() const { return T(p_->fb); }
@@ -96,7 +106,7 @@ class T {
   }
   int rank() const {
     if (pending_expr()) return (int)p_->eshape.size();
-    return pending_contraction() ? p_->keep : be()->api->rank(meta_h());
+    return contraction_like() ? p_->keep : be()->api->rank(meta_h());
   }
   int dtype() const { return pending_expr() ? p_->edtype : T(p_->fa ? p_->fa : p_).dtype_of_holder(); }
   int dtype_of_holder() const { return p_->h ? be()->api->dtype_of(p_->h) : dtype(); }
@@ -133,6 +143,7 @@ T ewise2(int op, const T& a, const T& b);
 T lazy_mul(const T& a, const T& b);                                // a * b, not yet written to memory
 void force_many(const std::vector<T>& ts);                         // pending values of one shape share a pass
 T lazy_contract(const T& a, const T& b, int n_keep);               // sum of a * b over the trailing dims, pending
+T add_cotangents(const T& a, const T& b);                          // a + b; pending contractions of one shape stay a pending sum
 T compare(int cmp, const T& a, const T& b);
 bool compare_all(int cmp, const T& a, const T& b);
 T select(const T& c, const T& a, const T& b);

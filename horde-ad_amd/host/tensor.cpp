@@ -16,7 +16,7 @@ void Backend::check(int rc) const {
 
 Shape T::shape() const {
   if (pending_expr()) return p_->eshape;
-  if (pending_contraction()) {   // the kept dims of the first factor
+  if (contraction_like()) {   // the kept dims of the first factor
     Shape f = T(p_->fa).shape();
     return Shape(f.begin(), f.begin() + p_->keep);
   }
@@ -278,13 +278,60 @@ void ArrHolder::force() {
     return;
   }
   if (!fa) return;
-  T fbt(fb);
-  T p = contract_now(T(fa), &fbt, keep);
+  if (!more.empty()) {   // a sum of contractions: one grouped call when the provider has it
+    std::vector<T> as{T(fa)}, bs{T(fb)};
+    for (auto& m : more) { as.push_back(T(m.first)); bs.push_back(T(m.second)); }
+    const hgpu_api* api = be->api;
+    hgpu_array* o = nullptr;
+    if (api->struct_size >= offsetof(hgpu_api, contract_sum) + sizeof(api->contract_sum) && api->contract_sum) {
+      std::vector<const hgpu_array*> ah, bh;
+      for (size_t i = 0; i < as.size(); ++i) { ah.push_back(as[i].h()); bh.push_back(bs[i].h()); }
+      be->check(api->contract_sum(be->ctx, (int)ah.size(), ah.data(), bh.data(), keep, &o));
+    } else {
+      T acc = contract_now(as[0], &bs[0], keep);
+      for (size_t i = 1; i < as.size(); ++i) acc = ewise2_now(HGPU_ADD, acc, contract_now(as[i], &bs[i], keep));
+      be->check(api->retain(acc.h()));
+      o = acc.h();
+    }
+    h = o;
+    fa.reset();
+    fb.reset();
+    more.clear();
+    origin.reset();
+    keep = -1;
+    return;
+  }
+  T p;
+  if (origin && (origin->h || origin.use_count() > 1)) {
+    origin->force();   // once for all its users
+    p = transpose(T(origin), origin_perm);
+  } else {
+    T fbt(fb);
+    p = contract_now(T(fa), &fbt, keep);
+  }
   be->check(be->api->retain(p.h()));
   h = p.h();
   fa.reset();
   fb.reset();
+  origin.reset();
   keep = -1;
+}
+
+T add_cotangents(const T& a, const T& b) {
+  if (a.contraction_like() && b.contraction_like() && a.be() == b.be() && a.holder()->keep == b.holder()->keep &&
+      a.dtype() == b.dtype() && T(a.holder()->fa).shape() == T(b.holder()->fa).shape()) {
+    auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
+    const ArrHolder* x = a.holder().get();
+    const ArrHolder* y = b.holder().get();
+    p->fa = x->fa;
+    p->fb = x->fb;
+    p->keep = x->keep;
+    p->more = x->more;
+    p->more.push_back({y->fa, y->fb});
+    p->more.insert(p->more.end(), y->more.begin(), y->more.end());
+    return T(p);
+  }
+  return ewise2(HGPU_ADD, a, b);
 }
 
 T lazy_mul(const T& a, const T& b) { return ewise2(HGPU_MUL, a, b); }
@@ -309,6 +356,7 @@ static T map_leaves(const T& a, const std::function<T(const T&)>& view) {
     if (it != memo.end()) return it->second;
     std::shared_ptr<ArrHolder> r;
     if (p->h || p->ekind < 0) {
+      if (!p->h) p->force();   // a pending contraction among the leaves is computed once, for every view of it
       r = view(T(p)).holder();
     } else {
       r = std::make_shared<ArrHolder>(p->be, nullptr);
@@ -332,7 +380,12 @@ static T map_leaves(const T& a, const std::function<T(const T&)>& view) {
 T transpose(const T& a, const std::vector<int>& perm) {
   HD_VIEW_OF_EXPR(transpose(x, perm))
   if (a.pending_contraction() && (int)perm.size() <= a.pending_keep())   // permutes kept dims only
-    return lazy_contract(transpose(a.factor_a(), perm), transpose(a.factor_b(), perm), a.pending_keep());
+  {
+    T r = lazy_contract(transpose(a.factor_a(), perm), transpose(a.factor_b(), perm), a.pending_keep());
+    r.holder()->origin = a.holder();
+    r.holder()->origin_perm = perm;
+    return r;
+  }
   static const int dummy = 0;
   HD_OUT(transpose(be__->ctx, a.h(), (int)perm.size(), perm.empty() ? &dummy : perm.data(), &o__));
 }
@@ -412,6 +465,11 @@ T convert(const T& a, int dtype, int mode) {
 T contract(const T& a, const T* b, int n_keep) {
   if (!b && a.pending_product())   // sum (u * v) = the contraction of u and v; stays pending
     return lazy_contract(a.factor_a(), a.factor_b(), n_keep);
+  // a contraction of two arrays of one shape and dtype stays pending too: sums of
+  // such (add_cotangents) are then written out by one grouped launch
+  if (b && a.be()->fuse && a.dtype() == b->dtype() && a.shape() == b->shape() && n_keep >= 0 && n_keep <= a.rank() && a.size() > 0 &&
+      (a.dtype() == HGPU_F64 || a.dtype() == HGPU_F32))
+    return lazy_contract(a, *b, n_keep);
   return contract_now(a, b, n_keep);
 }
 static T contract_now(const T& a, const T* b, int n_keep) {

@@ -228,6 +228,13 @@ int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_i
  * order is unspecified (as it is in ox-arrays); integers are exact. */
 int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array** out);
 
+/* out = sum_t contract(a[t], b[t], n_keep): the same contraction of n pairs of
+ * one shape and dtype, summed.  This is what the cotangent of a parameter
+ * that is used once per step of an unrolled recurrence amounts to
+ * (DeltaEval.hs:391-595 adds the per-use contributions one by one); when all
+ * pairs share one layout and the whole is a matrix product it is one launch
+ * whose K chunks run over all pairs.  Summation order is fixed by the shapes. */
+int hgpu_contract_sum(hgpu_ctx* ctx, int n, const hgpu_array* const* a, const hgpu_array* const* b, int n_keep, hgpu_array** out);
 /* tsargMin / tsargMax (OpsConcrete.hs:533-534, targMinS :1712-1746): index of
  * the first minimal / maximal element along the LAST dim; result I64 of shape
  * init(shape). */
@@ -350,6 +357,7 @@ typedef struct hgpu_api {
   int (*graph_launch)(hgpu_graph*);
   int (*graph_destroy)(hgpu_graph*);
   int (*overwrite)(hgpu_ctx*, hgpu_array*, const void*);
+  int (*contract_sum)(hgpu_ctx*, int, const hgpu_array* const*, const hgpu_array* const*, int, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

@@ -643,6 +643,26 @@ int horc_scatter_affine(hgpu_ctx* c, const hgpu_array* src, int rank_m, int n_ix
   return HGPU_OK;
 }
 
+// Sum of n contractions of one shape, term by term in order.
+int horc_contract_sum(hgpu_ctx* c, int n, const hgpu_array* const* as, const hgpu_array* const* bs, int n_keep, hgpu_array** out) {
+  if (n < 1) return fail(c, HGPU_ERR_INVALID, "contract_sum: no terms");
+  hgpu_array* acc = nullptr;
+  for (int t = 0; t < n; ++t) {
+    hgpu_array* part = nullptr;
+    int rc = horc_contract(c, as[t], bs[t], n_keep, &part);
+    if (rc) return rc;
+    if (!acc) { acc = part; continue; }
+    hgpu_array* sum = nullptr;
+    rc = horc_ewise2(c, HGPU_ADD, acc, part, &sum);
+    horc_release(acc);
+    horc_release(part);
+    if (rc) return rc;
+    acc = sum;
+  }
+  *out = acc;
+  return HGPU_OK;
+}
+
 // toneHotS (OpsConcrete.hs:1516-1525)
 int horc_onehot(hgpu_ctx* c, const hgpu_array* v, int n, const int64_t* ix, const int64_t* shp, hgpu_array** out) {
   if (n < 0 || n + (int)v->shape.size() > HGPU_MAX_RANK) return fail(c, HGPU_ERR_INVALID, "onehot: rank too large");
@@ -709,6 +729,7 @@ const hgpu_api* horc_get_api(void) {
       horc_contract,    horc_argminmax_last, horc_iota,    horc_concat,     horc_gather,      horc_scatter_add,
       horc_onehot,      horc_fused_map, horc_scatter_affine,
       nullptr, nullptr, nullptr, nullptr, nullptr,   // no graphs: the checker executes eagerly
+      horc_contract_sum,
   };
   return &api;
 }

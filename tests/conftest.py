@@ -76,6 +76,9 @@ class Both:
     def scatter_add(self, src, ix, rank_m, shp, flags=0):
         return Pair([c.scatter_add(src.arrays[i], [p.arrays[i] for p in ix], rank_m, shp, flags) for i, c in enumerate(self.ctxs)])
 
+    def contract_sum(self, pairs, n_keep):
+        return Pair([c.contract_sum([(a.arrays[i], b.arrays[i]) for a, b in pairs], n_keep) for i, c in enumerate(self.ctxs)])
+
     def scatter_affine(self, src, rank_m, c0, coef, shp):
         return Pair([c.scatter_affine(src.arrays[i], rank_m, c0, coef, shp) for i, c in enumerate(self.ctxs)])
 

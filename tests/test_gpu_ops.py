@@ -311,6 +311,38 @@ def test_scatter_affine(both, dt):
     assert_same(both.scatter_affine(src, 0, [2], [], [5]))
 
 
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_contract_sum(both, dt):
+    """Sums of products of one shape: one launch over all terms (weight gradients
+    of an unrolled recurrence), small outputs, many terms, mixed layouts."""
+    tol = TOL[np.dtype(dt)]
+    for m, n, k, terms in [(128, 128, 600, 5), (128, 28, 900, 7), (64, 200, 512, 40), (10, 16, 3000, 3)]:
+        pairs = []
+        for _ in range(terms):
+            a = both.upload(rnd((m, k), dt)).replicate([n]).transpose([1, 0, 2])      # [m, n, k]
+            b = both.upload(rnd((k, n), dt)).transpose([1, 0]).replicate([m])          # [m, n, k], K strided
+            pairs.append((a, b))
+        assert_same(both.contract_sum(pairs, 2), tol * 4, (m, n, k, terms))
+    # terms of different layouts: term by term
+    a1 = both.upload(rnd((40, 30, 50), dt))
+    b1 = both.upload(rnd((40, 30, 50), dt))
+    a2 = both.upload(rnd((30, 40, 50), dt)).transpose([1, 0, 2])
+    b2 = both.upload(rnd((40, 30, 50), dt))
+    assert_same(both.contract_sum([(a1, b1), (a2, b2)], 2), tol * 4)
+    assert_same(both.contract_sum([(a1, b1)], 1), tol * 4)
+    # two layouts interleaved, one of them with a replicated (stride 0) operand:
+    # each layout is one grouped launch
+    pairs = []
+    for t in range(9):
+        a = both.upload(rnd((128, 700), dt)).replicate([96]).transpose([1, 0, 2])
+        if t % 3 == 0:
+            b = both.upload(rnd((700,), dt)).replicate([128, 96])
+        else:
+            b = both.upload(rnd((700, 96), dt)).transpose([1, 0]).replicate([128])
+        pairs.append((a, b))
+    assert_same(both.contract_sum(pairs, 2), tol * 4)
+
+
 def test_scatter_small_ints(both, gpu):
     perm = both.upload(RNG.permutation(64).astype(np.int64))
     for dt in (np.int16, np.int8):
