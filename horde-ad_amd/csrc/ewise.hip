@@ -263,7 +263,16 @@ int copy_view(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const vo
   const int64_t* sts[2] = {pss, pds};
   Dims d;
   if (!collapse(rank, psh, 2, sts, &d)) return fail(ctx, HGPU_ERR_UNSUPPORTED, "copy: more than %d merged dims", HG_KDIMS);
-  LaunchGuard lg(ctx, "copy_view", 2.0 * n * dtype_size(dtype), 0);
+  const char* label = "copy_view";
+  if (ctx->profiling && ctx->profile_shapes) {
+    char buf[200];
+    int w = snprintf(buf, sizeof buf, "copy_view[es%d", (int)dtype_size(dtype));
+    for (int i = 0; i < d.nd && w < (int)sizeof buf - 60; ++i)
+      w += snprintf(buf + w, sizeof buf - w, ",%lld:%lld>%lld", (long long)d.shape[i], (long long)d.st[0][i], (long long)d.st[1][i]);
+    snprintf(buf + w, sizeof buf - w, "]");
+    label = ctx->label_pool.insert(buf).first->c_str();
+  }
+  LaunchGuard lg(ctx, label, 2.0 * n * dtype_size(dtype), 0);
   unsigned g = grid_for(n, kBlock, max_blocks(ctx));
   switch (dtype_size(dtype)) {
     case 8: hipLaunchKernelGGL(k_copy<uint64_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint64_t*)src, (uint64_t*)dst); break;

@@ -236,6 +236,19 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
 
 namespace hg {
 
+int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled);
+
+int sum_partials(hgpu_ctx* ctx, int dtype, int64_t n, int parts, const void* part, void* out) {
+  size_t es = dtype_size(dtype);
+  LaunchGuard ls(ctx, "gemm_sum_partials", (double)n * (parts + 1) * es, (double)n * parts);
+  if (dtype == HGPU_F64)
+    hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, parts, n, (const double*)part, (double*)out);
+  else
+    hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, parts, n, (const float*)part, (float*)out);
+  HG_CHECK_LAUNCH(ctx, "gemm_sum_partials");
+  return HGPU_OK;
+}
+
 int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled,
              int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs) {
   // n_terms > 0: out = sum_t contract(as[t], bs[t]); all terms have the shapes,
@@ -304,6 +317,10 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   if (n_terms > kMaxTerms) return HGPU_OK;
   p.n_terms = n_terms;
   for (int t = 0; t < n_terms; ++t) { p.a_term[t] = data_ptr(as[t]); p.b_term[t] = data_ptr(bs[t]); }
+  if (n_terms == 0) {   // windows into small footprints: operands from LDS
+    int rc = try_footprint(ctx, p, a->dtype, pa, pb, out, handled);
+    if (rc || *handled) return rc;
+  }
   if ((p.M <= 32 || p.N <= 32) && p.M <= 1024 && p.N <= 1024) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled, n_terms);
 
   // tile shape: least padded work per unit of efficiency

@@ -214,7 +214,13 @@ int hgpu_gather(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array
   Dims inner;
   if (!collapse(rank_n, src->shape + n_ix, 1, is, &inner)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "gather: too many inner dims"); }
   {
-    LaunchGuard lg(ctx, "gather", 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, 0);
+    const char* label = "gather";
+    if (ctx->profiling && ctx->profile_shapes) {
+      char buf[120];
+      snprintf(buf, sizeof buf, "gather[es%d,M%lld,N%lld,ix%d]", (int)dtype_size(src->dtype), (long long)M, (long long)N, n_ix);
+      label = ctx->label_pool.insert(buf).first->c_str();
+    }
+    LaunchGuard lg(ctx, label, 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, 0);
     unsigned g = grid_for(M * N, kBlock, ctx->num_cu * 8);
     switch (dtype_size(src->dtype)) {
       case 8: hipLaunchKernelGGL(k_gather<uint64_t>, dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, (const uint64_t*)data_ptr(src), (uint64_t*)data_ptr(o)); break;

@@ -451,6 +451,57 @@ def test_contract_on_the_matrix_cores(both, gpu, dt):
     assert any(k.startswith("gemm") for k in rep), rep
 
 
+def conv_views(both, dt, b, ci, h, w, co, kh, kw):
+    """The window views of a 'same' convolution: input windows [b, h, w, ci, kh, kw]
+    of the zero-extended image, the kernel, and a cotangent of the output."""
+    img, ker = both.upload(rnd((b, ci, h, w), dt)), both.upload(rnd((co, ci, kh, kw), dt))
+    padded = img.pad([0, 0, 0, 0], [0, 0, kh - 1, kw - 1])
+    st = padded.arrays[0].strides
+    win = padded.as_strided([b, h, w, ci, kh, kw], [st[0], st[2], st[3], st[1], st[2], st[3]], 0)
+    dout = both.upload(rnd((b, co, h, w), dt))
+    return win, ker, dout
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+@pytest.mark.parametrize("shape", [
+    (160, 8, 12, 12, 16, 3, 3),     # row blocks dealt evenly and split along K
+    (200, 16, 14, 14, 16, 5, 5),    # the CNN's second layer at a fifth of its batch
+    (512, 3, 9, 11, 12, 3, 2),      # fewer than 16 output channels, K not a multiple of 4
+    (192, 1, 20, 20, 8, 5, 5),      # one input channel
+])
+def test_conv_contractions_from_lds_footprints(both, gpu, dt, shape):
+    """Forward convolution, kernel gradient and input gradient as contractions
+    over window views, at batch sizes where a block keeps one image's footprint
+    of each operand in LDS."""
+    b, ci, h, w, co, kh, kw = shape
+    tol = TOL[np.dtype(dt)] * 20
+    win, ker, dout = conv_views(both, dt, b, ci, h, w, co, kh, kw)
+    gpu.check(gpu.lib.profile_enable(gpu.h, 2))     # kernel names with shapes
+    gpu.profile_report()
+    # forward: out[b, co, h, w]
+    lhs = win.replicate([co]).transpose([1, 0, 2, 3])             # [b, co, h, w, ci, kh, kw]
+    rhs = ker.replicate([b, h, w]).transpose([0, 3, 1, 2])        # [b, co, h, w, ci, kh, kw]
+    assert_same(lhs.contract(rhs, 4), tol, ("conv", shape))
+    # kernel gradient: dK[co, ci, kh, kw], K = (b, h, w) on both operands
+    lhs = win.replicate([co]).transpose([0, 4, 5, 6, 1, 2, 3])            # [co, ci, kh, kw, b, h, w]
+    rhs = dout.replicate([ci, kh, kw]).transpose([4, 0, 1, 2, 3, 5, 6])   # [co, ci, kh, kw, b, h, w]
+    assert_same(lhs.contract(rhs, 4), tol, ("conv dK", shape))
+    # input gradient as a convolution of the zero-extended cotangent with the
+    # reversed kernel: dX[b, ci, y, x] = sum dout_pad[b, co, y + p, x + q] * ker[co, ci, kh-1-p, kw-1-q]
+    dpad = dout.pad([0, 0, kh - 1, kw - 1], [0, 0, 0, 0])
+    st = dpad.arrays[0].strides
+    dwin = dpad.as_strided([b, h, w, co, kh, kw], [st[0], st[2], st[3], st[1], st[2], st[3]], 0)
+    lhs = dwin.replicate([ci]).transpose([1, 0, 2, 3])                     # [b, ci, y, x, co, kh, kw]
+    rker = ker.reverse(2).reverse(3).transpose([1, 0, 2, 3])               # [ci, co, kh, kw]
+    rhs = rker.replicate([b, h, w]).transpose([0, 3, 1, 2])                # [b, ci, y, x, co, kh, kw]
+    assert_same(lhs.contract(rhs, 4), tol, ("conv dX", shape))
+    rep = gpu.profile_report()
+    gpu.profile(False)
+    # at least the kernel gradient and the forward product of the larger shapes run from LDS footprints
+    if ci * kh * kw >= 16:
+        assert any("footprint" in k for k in rep), list(rep)
+
+
 def eval_program_eagerly(ctx, inputs, prog, out_slots):
     """The meaning of a fused program: the single entry points applied in order."""
     inv1 = {v: k for k, v in capi.OP1.items()}
