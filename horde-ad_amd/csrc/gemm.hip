@@ -345,15 +345,19 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   if (tiles > 0x7fffffff) return HGPU_OK;
   // split K when the tiles alone cannot fill the device
   int split = 1;
-  int64_t want = (int64_t)ctx->num_cu * 2;
+  // small tiles do little work per K step and hide the latency of a step only
+  // behind other blocks on the CU: ask for more of them
+  const int64_t per_cu = BM * BN >= 128 * 64 ? 2 : (BM * BN >= 64 * 64 ? 4 : 8);
+  int64_t want = (int64_t)ctx->num_cu * per_cu;
   int64_t out_elems = p.M * p.N * p.BT;
   const int64_t nt = n_terms > 0 ? n_terms : 1;      // products summed by this launch
   if (tiles * p.BT * nt < want && p.K >= 8 * BK) {
     split = (int)((want + tiles * p.BT * nt - 1) / (tiles * p.BT * nt));
     int64_t max_split = p.K / (4 * BK);
     if (split > max_split) split = (int)max_split;
-    // the partial products must stay small next to the operands
+    // the partial products must stay small next to the operands, or small outright
     int64_t cap = out_elems > 0 ? (int64_t)((double)(p.M + p.N) * p.K * p.BT / (2.0 * out_elems)) : 1;
+    if (out_elems * (int64_t)dtype_size(a->dtype) <= (1 << 20) && cap < 16) cap = 16;
     if (cap > 512) cap = 512;
     if (cap < 1) cap = 1;
     if (split > cap) split = (int)cap;
