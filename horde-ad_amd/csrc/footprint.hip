@@ -95,6 +95,9 @@ struct Plan {
   // the 16 columns of a B fragment fall into different banks (ypad 0: a plain copy)
   int64_t ys;
   int ypad;
+  int addr_regs;   // per-lane address registers of the kernel
+  int nbufs;   // LDS chunk buffers: 2, or 1 when two do not fit (the prefetch then waits in registers)
+  bool cvec;   // groups of four rows are adjacent in C and 16-byte aligned: vector stores
 };
 
 int64_t prod(const std::vector<Dim>& d) {
@@ -199,7 +202,8 @@ bool make_plan(bool f64, std::vector<Dim> rows, std::vector<Dim> cols, std::vect
   const int MB = (int)((R + 15) / 16), NBF = MB / 4, REM = MB % 4, NG = (int)ng, NSLOT = (NG + 3) / 4;
   if (NBF * NG + REM * NSLOT > kMaxMfma) return false;
   if (NBF + REM > 20) return false;                       // accumulators
-  if (NBF * (int)pl->px.size() + REM * NSLOT * 2 > 160) return false;   // address registers
+  pl->addr_regs = NBF * (int)pl->px.size() + REM * NSLOT * 2 + 8 * (NBF + REM);
+  if (pl->addr_regs > 300) return false;   // address registers and accumulators
   return true;
 }
 
@@ -219,12 +223,15 @@ template <int I> struct IC { static constexpr int v = I; };
 typedef double T;
 typedef __attribute__((ext_vector_type(4))) double Acc;
 #define MFMA(a, b, c) __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0)
-#define ACC_ROW(q4, j) (4 * (j) + (q4))
+// Register j of a lane holds row 4 j + lane / 16 of the block's A fragment.  A
+// lane r of the A fragment reads matrix row ROW_OF(r) of the block, chosen so
+// that the four registers of a lane are four consecutive matrix rows.
+#define ROW_OF(r) (4 * ((r) & 3) + ((r) >> 2))
 #else
 typedef float T;
 typedef __attribute__((ext_vector_type(4))) float Acc;
 #define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0)
-#define ACC_ROW(q4, j) (4 * (q4) + (j))
+#define ROW_OF(r) (r)   // register j of a lane holds row 4 (lane / 16) + j already
 #endif
 template <int N> struct VT { typedef T type __attribute__((ext_vector_type(N))); };
 template <> struct VT<1> { typedef T type; };
@@ -242,8 +249,30 @@ constexpr int NLD = MODE == 0 ? NLX + NLY : NLX;        // loads per thread and 
 constexpr int PH = NG >= 12 ? 3 : 1;                    // prefetch phases
 constexpr int LPP = (NLD + PH - 1) / PH;
 constexpr int BUF = MODE == 0 ? LX + LY : LX;           // elements per chunk buffer
-constexpr int RED0 = 2 * BUF + (MODE == 0 ? 0 : LY);    // scratch for adding up split row blocks
+constexpr int RED0 = NBUFS * BUF + (MODE == 0 ? 0 : LY);    // scratch for adding up split row blocks
 constexpr int LDS_ELEMS = RED0 + (REM > 0 ? REM * 4 * 256 : 0);
+
+// The four registers of a lane are rows m0 .. m0 + 3 of column col.
+__device__ __forceinline__ void store_rows(T* __restrict__ out, int m0, int col, T v0, T v1, T v2, T v3) {
+  if (col >= NIN) return;
+  if (CVEC) {      // the four rows are adjacent in memory and 16-byte aligned
+    if (m0 < MIN) {
+      T* dst = out + kRowC[m0] + kColC[col];
+#if F64
+      reinterpret_cast<Vec<2>*>(dst)[0] = Vec<2>{v0, v1};
+      reinterpret_cast<Vec<2>*>(dst)[1] = Vec<2>{v2, v3};
+#else
+      reinterpret_cast<Vec<4>*>(dst)[0] = Vec<4>{v0, v1, v2, v3};
+#endif
+    }
+  } else {
+    const int cc = kColC[col];
+    if (m0 < MIN) out[kRowC[m0] + cc] = v0;
+    if (m0 + 1 < MIN) out[kRowC[m0 + 1] + cc] = v1;
+    if (m0 + 2 < MIN) out[kRowC[m0 + 2] + cc] = v2;
+    if (m0 + 3 < MIN) out[kRowC[m0 + 3] + cc] = v3;
+  }
+}
 
 extern "C" __global__ void __launch_bounds__(256, 1)
 footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 nch, i64 chx, i64 chy, i64 chc, i64 part_stride) {
@@ -255,7 +284,7 @@ footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__
   int ax[NBF > 0 ? NBF : 1][NPAT];
 #pragma unroll
   for (int t = 0; t < NBF; ++t) {
-    int m = (wave + 4 * t) * 16 + r;
+    int m = (wave + 4 * t) * 16 + ROW_OF(r);
     int ro = kRowX[m < MIN ? m : MIN - 1];
 #pragma unroll
     for (int p = 0; p < NPAT; ++p) ax[t][p] = ro + kPatX[p * 4 + q4];
@@ -268,7 +297,7 @@ footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__
   int remx[REM > 0 ? REM * NSLOT : 1], remy[REM > 0 ? REM * NSLOT : 1];
 #pragma unroll
   for (int rb = 0; rb < REM; ++rb) {
-    int m = (4 * NBF + rb) * 16 + r;
+    int m = (4 * NBF + rb) * 16 + ROW_OF(r);
     int ro = kRowX[m < MIN ? m : MIN - 1];
 #pragma clang loop unroll(full)
     for (int s = 0; s < NSLOT; ++s) {
@@ -299,14 +328,19 @@ footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__
   }
   if (MODE == 1) {   // the columns operand does not change with the chunk
     for (int v = tid; v < YV; v += 256)
-      reinterpret_cast<Vec<VY>*>(lds + 2 * BUF)[ypos(v)] = reinterpret_cast<const Vec<VY>*>(Y)[v];
+      reinterpret_cast<Vec<VY>*>(lds + NBUFS * BUF)[ypos(v)] = reinterpret_cast<const Vec<VY>*>(Y)[v];
   }
   int cur = 0;
   for (; ch < nch; ch += gridDim.x) {
     __syncthreads();
     const T* L = lds + cur * BUF;
-    T* Ln = lds + (cur ^ 1) * BUF;
-    const T* LYp = MODE == 0 ? L : lds + 2 * BUF - LX;   // so that YOFF = LX addresses Y in both modes
+    T* Ln = lds + (NBUFS == 2 ? cur ^ 1 : 0) * BUF;
+    const T* LYp = MODE == 0 ? L : lds + NBUFS * BUF - LX;   // so that YOFF = LX addresses Y in both modes
+    // the next chunk's footprint on its way from memory: with two buffers a
+    // phase's share goes to LDS when the phase ends, with one buffer everything
+    // waits in registers until this chunk has been multiplied
+    Vec<VX> prex[PH * LPP];
+    Vec<VY> prey[PH * LPP];
     i64 chn = ch + gridDim.x;
     if (chn >= nch) chn = nch - 1;    // the last prefetch is not used
     if (MODE == 1) {
@@ -316,14 +350,12 @@ footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__
     auto phase = [&](auto PHI) {
       constexpr int ph = decltype(PHI)::v;
       constexpr int g0 = ph < PH ? NG * ph / PH : NG, g1 = ph < PH ? NG * (ph + 1) / PH : NG;
-      Vec<VX> prex[LPP];
-      Vec<VY> prey[LPP];
 #pragma unroll
       for (int j = 0; j < LPP; ++j) {
         int jj = ph * LPP + j;
         if (jj < NLD) {
-          if (jj < NLX) prex[j] = reinterpret_cast<const Vec<VX>*>(X + chn * chx)[vidx(jj)];
-          else prey[j] = reinterpret_cast<const Vec<VY>*>(Y + chn * chy)[vidx(jj)];
+          if (jj < NLX) prex[jj] = reinterpret_cast<const Vec<VX>*>(X + chn * chx)[vidx(jj)];
+          else prey[jj] = reinterpret_cast<const Vec<VY>*>(Y + chn * chy)[vidx(jj)];
         }
       }
       auto groups = [&](auto self, auto GI) -> void {
@@ -355,29 +387,34 @@ footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__
         }
       };
       groups(groups, IC<g0>{});
+      if (NBUFS == 2) {
 #pragma unroll
-      for (int j = 0; j < LPP; ++j) {
-        int jj = ph * LPP + j;
-        if (jj < NLD) {
-          if (jj < NLX) reinterpret_cast<Vec<VX>*>(Ln)[vidx(jj)] = prex[j];
-          else reinterpret_cast<Vec<VY>*>(Ln + LX)[ypos(vidx(jj))] = prey[j];
+        for (int j = 0; j < LPP; ++j) {
+          int jj = ph * LPP + j;
+          if (jj < NLD) {
+            if (jj < NLX) reinterpret_cast<Vec<VX>*>(Ln)[vidx(jj)] = prex[jj];
+            else reinterpret_cast<Vec<VY>*>(Ln + LX)[ypos(vidx(jj))] = prey[jj];
+          }
         }
       }
     };
     phase(IC<0>{});
     if constexpr (PH > 1) phase(IC<1>{});
     if constexpr (PH > 2) phase(IC<2>{});
-    cur ^= 1;
+    if (NBUFS == 2) {
+      cur ^= 1;
+    } else {
+      __syncthreads();    // everyone has finished reading this chunk
+#pragma unroll
+      for (int jj = 0; jj < NLD; ++jj) {
+        if (jj < NLX) reinterpret_cast<Vec<VX>*>(Ln)[vidx(jj)] = prex[jj];
+        else reinterpret_cast<Vec<VY>*>(Ln + LX)[ypos(vidx(jj))] = prey[jj];
+      }
+    }
     if (MODE == 1) {
       T* out = C + ch * chc;
 #pragma unroll
-      for (int t = 0; t < NBF; ++t) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          int m = (wave + 4 * t) * 16 + ACC_ROW(q4, j);
-          if (m < MIN && r < NIN) out[kRowC[m] + kColC[r]] = acc[t][j];
-        }
-      }
+      for (int t = 0; t < NBF; ++t) store_rows(out, (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
       if (REM > 0) {
         T* red = lds + RED0;
 #pragma unroll
@@ -387,14 +424,14 @@ footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__
         __syncthreads();
         if (wave < REM) {
           const int rb = wave;
+          T s[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            T s = T(0);
+            s[j] = T(0);
 #pragma unroll
-            for (int w = 0; w < 4; ++w) s += red[((rb * 4 + w) * 4 + j) * 64 + lane];
-            int m = (4 * NBF + rb) * 16 + ACC_ROW(q4, j);
-            if (m < MIN && r < NIN) out[kRowC[m] + kColC[r]] = s;
+            for (int w = 0; w < 4; ++w) s[j] += red[((rb * 4 + w) * 4 + j) * 64 + lane];
           }
+          store_rows(out, (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
         }
       }
     }
@@ -402,13 +439,7 @@ footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__
   if (MODE == 0) {
     T* out = C + (i64)blockIdx.x * part_stride;
 #pragma unroll
-    for (int t = 0; t < NBF; ++t) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int m = (wave + 4 * t) * 16 + ACC_ROW(q4, j);
-        if (m < MIN && r < NIN) out[kRowC[m] + kColC[r]] = acc[t][j];
-      }
-    }
+    for (int t = 0; t < NBF; ++t) store_rows(out, (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
     if (REM > 0) {
       T* red = lds + RED0;
       __syncthreads();
@@ -419,14 +450,14 @@ footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__
       __syncthreads();
       if (wave < REM) {
         const int rb = wave;
+        T s[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          T s = T(0);
+          s[j] = T(0);
 #pragma unroll
-          for (int w = 0; w < 4; ++w) s += red[((rb * 4 + w) * 4 + j) * 64 + lane];
-          int m = (4 * NBF + rb) * 16 + ACC_ROW(q4, j);
-          if (m < MIN && r < NIN) out[kRowC[m] + kColC[r]] = s;
+          for (int w = 0; w < 4; ++w) s[j] += red[((rb * 4 + w) * 4 + j) * 64 + lane];
         }
+        store_rows(out, (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
       }
     }
   }
@@ -442,6 +473,8 @@ std::string generate(const Plan& pl) {
   s << "#define NPAT " << pl.px.size() << "\n#define KVALID " << pl.kvalid << "\n";
   s << "#define SPANX " << pl.span_x << "\n#define SPANY " << pl.span_y << "\n";
   s << "#define VX " << pl.vx << "\n#define VY " << pl.vy << "\n";
+  s << "#define NBUFS " << pl.nbufs << "\n";
+  s << "#define CVEC " << (pl.cvec ? 1 : 0) << "\n";
   s << "#define YS " << (pl.ypad ? pl.ys : 1) << "\n#define YPAD " << pl.ypad << "\n";
   // Y sits behind X in a chunk buffer
   int64_t xv = (pl.span_x + pl.vx - 1) / pl.vx;
@@ -468,7 +501,7 @@ int lds_bytes(const Plan& pl) {
   if (pl.ypad) ly += (ly / pl.ys) * pl.ypad;
   int64_t buf = pl.mode == 0 ? lx + ly : lx;
   int MB = (pl.min_rows + 15) / 16, REM = MB % 4;
-  int64_t total = 2 * buf + (pl.mode == 0 ? 0 : ly) + (REM > 0 ? REM * 4 * 256 : 0);
+  int64_t total = pl.nbufs * buf + (pl.mode == 0 ? 0 : ly) + (REM > 0 ? REM * 4 * 256 : 0);
   total *= es;
   return total > INT32_MAX ? INT32_MAX : (int)total;
 }
@@ -536,10 +569,24 @@ int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa,
             }
           }
         }
+        {
+          const int V16 = 16 / es;
+          const char* cp = (const char*)data_ptr(out);
+          bool ok = pl.min_rows % 4 == 0 && ((uintptr_t)cp & 15) == 0 && pl.chc % V16 == 0;
+          for (size_t m = 0; m < pl.row_c.size() && ok; m += 4)
+            ok = pl.row_c[m] % V16 == 0 && pl.row_c[m + 1] == pl.row_c[m] + 1 && pl.row_c[m + 2] == pl.row_c[m] + 2 && pl.row_c[m + 3] == pl.row_c[m] + 3;
+          for (size_t c = 0; c < pl.col_c.size() && ok; ++c) ok = pl.col_c[c] % V16 == 0;
+          if (pl.mode == 0) ok = ok && nelem(out) % V16 == 0;   // partial outputs lie nelem(out) apart
+          pl.cvec = ok;
+        }
         // scalar staging of a large footprint would need too many loads in flight
         int64_t loads = (pl.span_x / pl.vx + 255) / 256 + (pl.mode == 0 ? (pl.span_y / pl.vy + 255) / 256 : 0);
         if (loads > 48) continue;
-        if (lds_bytes(pl) > kLdsBudget) continue;
+        pl.nbufs = 2;
+        if (lds_bytes(pl) > kLdsBudget) {
+          pl.nbufs = 1;
+          if (lds_bytes(pl) > kLdsBudget || loads * 4 + pl.addr_regs > 330) continue;   // the prefetch must fit the register file
+        }
         best = pl;
         best_swapped = swapped != 0;
         found = true;
