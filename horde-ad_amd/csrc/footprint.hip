@@ -50,7 +50,7 @@ std::map<std::string, Compiled>& cache_of(hgpu_ctx* ctx) {
   return *static_cast<std::map<std::string, Compiled>*>(it->second);
 }
 
-int compile(hgpu_ctx* ctx, const std::string& src, Compiled* out) {
+int compile(hgpu_ctx* ctx, const std::string& src, const std::string& kname, Compiled* out) {
   hiprtcProgram prog;
   if (hiprtcCreateProgram(&prog, src.c_str(), "footprint_gemm.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
     return fail(ctx, HGPU_ERR_DEVICE, "hiprtcCreateProgram failed");
@@ -72,7 +72,7 @@ int compile(hgpu_ctx* ctx, const std::string& src, Compiled* out) {
   hiprtcDestroyProgram(&prog);
   hipError_t e = hipModuleLoadData(&out->mod, code.data());
   if (e != hipSuccess) return check_hip(ctx, e, "hipModuleLoadData");
-  e = hipModuleGetFunction(&out->fn, out->mod, "footprint_gemm");
+  e = hipModuleGetFunction(&out->fn, out->mod, kname.c_str());
   if (e != hipSuccess) return check_hip(ctx, e, "hipModuleGetFunction");
   return HGPU_OK;
 }
@@ -275,7 +275,7 @@ __device__ __forceinline__ void store_rows(T* __restrict__ out, int m0, int col,
 }
 
 extern "C" __global__ void __launch_bounds__(256, 1)
-footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 nch, i64 chx, i64 chy, i64 chc, i64 part_stride) {
+KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 nch, i64 chx, i64 chy, i64 chc, i64 part_stride) {
   __shared__ T lds[LDS_ELEMS];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -464,8 +464,9 @@ footprint_gemm(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__
 }
 )HG";
 
-std::string generate(const Plan& pl) {
+std::string generate(const Plan& pl, const std::string& kname) {
   std::ostringstream s;
+  s << "#define KNAME " << kname << "\n";
   const int es = pl.f64 ? 8 : 4;
   s << "#define F64 " << (pl.f64 ? 1 : 0) << "\n";
   s << "#define MODE " << pl.mode << "\n";
@@ -595,12 +596,16 @@ int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa,
   }
   if (!found) return HGPU_OK;
   const Plan& pl = best;
-  std::string src = generate(pl);
+  // the kernel's name tells a profiler which product it is
+  char kname[128];
+  snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_%s%s", f64 ? "f64" : "f32", (long long)p.M, (long long)p.N, (long long)p.K,
+           pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? "_swapped" : "");
+  std::string src = generate(pl, kname);
   auto& cache = cache_of(ctx);
   auto it = cache.find(src);
   if (it == cache.end()) {
     Compiled c;
-    int rc = compile(ctx, src, &c);
+    int rc = compile(ctx, src, kname, &c);
     if (rc) return rc;
     it = cache.emplace(src, c).first;
   }
