@@ -604,11 +604,12 @@ int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa,
   auto& cache = cache_of(ctx);
   auto it = cache.find(src);
   if (it == cache.end()) {
-    Compiled c;
-    int rc = compile(ctx, src, kname, &c);
-    if (rc) return rc;
+    Compiled c{nullptr, nullptr};
+    // a shape the compiler rejects is remembered and left to the other kernels
+    if (compile(ctx, src, kname, &c) != HGPU_OK) c = Compiled{nullptr, nullptr};
     it = cache.emplace(src, c).first;
   }
+  if (!it->second.fn) return HGPU_OK;
   const char* xp = (const char*)(best_swapped ? pb : pa) + pl.shift_x * es;
   const char* yp = (const char*)(best_swapped ? pa : pb) + pl.shift_y * es;
   int64_t out_n = nelem(out);

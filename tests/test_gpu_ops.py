@@ -468,6 +468,10 @@ def conv_views(both, dt, b, ci, h, w, co, kh, kw):
     (200, 16, 14, 14, 16, 5, 5),    # the CNN's second layer at a fifth of its batch
     (512, 3, 9, 11, 12, 3, 2),      # fewer than 16 output channels, K not a multiple of 4
     (192, 1, 20, 20, 8, 5, 5),      # one input channel
+    (300, 5, 7, 9, 16, 2, 4),       # odd extents everywhere, K tails
+    (600, 2, 16, 16, 4, 3, 3),      # four output channels
+    (128, 32, 8, 8, 16, 3, 3),      # 18 row blocks in the kernel gradient: dealt and split
+    (150, 7, 10, 10, 16, 3, 3),     # 63 rows
 ])
 def test_conv_contractions_from_lds_footprints(both, gpu, dt, shape):
     """Forward convolution, kernel gradient and input gradient as contractions
