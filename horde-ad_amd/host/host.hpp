@@ -63,6 +63,16 @@ struct ArrHolder {
   // computed once and this one becomes a view of it.
   std::shared_ptr<ArrHolder> origin;
   std::vector<int> origin_perm;
+  // A pending CONCATENATION along the first dim (h == nullptr, pieces not
+  // empty): `tsappend`, and the zero-extension that is the adjoint of a slice
+  // (a piece without an array is zeros).  Slicing it hands back the pieces, and
+  // adding two of them piece by piece adds only where both have data -- the
+  // stacked state of an unrolled recurrence and its cotangent are then never
+  // copied, cleared or added as a whole.
+  struct Piece { int64_t len; std::shared_ptr<ArrHolder> v; };
+  std::vector<Piece> pieces;
+  Shape pshape;
+  int pdtype = 0;
   // A pending ELEMENTWISE operation (h == nullptr): kind/op as in
   // hgpu_fused_instr, operands fa, fb, fc.  Chains of them are handed to the
   // provider's fused_map as one program when the value is first needed as an
@@ -93,6 +103,7 @@ class T {
   }
   bool pending_expr() const { return p_ && !p_->h && p_->ekind >= 0; }
   bool pending_product() const { return pending_expr() && p_->ekind == HGPU_FUSED_OP2 && p_->eop == HGPU_MUL; }
+  bool pending_pieces() const { return p_ && !p_->h && !p_->pieces.empty(); }
   bool contraction_like() const { return p_ && !p_->h && p_->ekind < 0 && p_->fa && p_->keep >= 0; }
   bool pending_contraction() const { return contraction_like() && p_->more.empty(); }   // a single one: open to rewrites
   int pending_keep() const { return p_->keep; }
@@ -105,10 +116,14 @@ class T {
     return q->h;
   }
   int rank() const {
+    if (pending_pieces()) return (int)p_->pshape.size();
     if (pending_expr()) return (int)p_->eshape.size();
     return contraction_like() ? p_->keep : be()->api->rank(meta_h());
   }
-  int dtype() const { return pending_expr() ? p_->edtype : T(p_->fa ? p_->fa : p_).dtype_of_holder(); }
+  int dtype() const {
+    if (pending_pieces()) return p_->pdtype;
+    return pending_expr() ? p_->edtype : T(p_->fa ? p_->fa : p_).dtype_of_holder();
+  }
   int dtype_of_holder() const { return p_->h ? be()->api->dtype_of(p_->h) : dtype(); }
   int64_t size() const {
     int64_t n = 1;

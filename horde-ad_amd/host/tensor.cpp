@@ -15,6 +15,7 @@ void Backend::check(int rc) const {
 }
 
 Shape T::shape() const {
+  if (pending_pieces()) return p_->pshape;
   if (pending_expr()) return p_->eshape;
   if (contraction_like()) {   // the kept dims of the first factor
     Shape f = T(p_->fa).shape();
@@ -111,6 +112,9 @@ T iota(Backend* be, int64_t n, int dtype) {
   return T(be__, o__)
 
 static T contract_now(const T& a, const T* b, int n_keep);
+static void pieces_of(const T& t, std::vector<ArrHolder::Piece>* out);
+static T from_pieces(Backend* be, std::vector<ArrHolder::Piece> pcs, const Shape& shape, int dtype);
+static T slice_pieces(const T& a, int64_t start, int64_t len);
 static T ewise1_now(int op, const T& a);
 static T ewise2_now(int op, const T& a, const T& b);
 static T compare_now(int cmp, const T& a, const T& b);
@@ -273,6 +277,21 @@ void force_many(const std::vector<T>& ts) {
 
 void ArrHolder::force() {
   if (h) return;
+  if (!pieces.empty()) {   // write the concatenation out: one allocation, one copy (or fill) per piece
+    std::vector<T> parts;
+    for (auto& pc : pieces) {
+      Shape sh = pshape;
+      sh[0] = pc.len;
+      parts.push_back(pc.v ? T(pc.v) : zeros(be, pdtype, sh));
+    }
+    std::vector<const hgpu_array*> hs;
+    for (auto& t : parts) hs.push_back(t.h());
+    hgpu_array* o = nullptr;
+    be->check(be->api->concat(be->ctx, (int)hs.size(), hs.data(), &o));
+    h = o;
+    pieces.clear();
+    return;
+  }
   if (ekind >= 0) {
     force_roots(be, {this});
     return;
@@ -330,6 +349,31 @@ T add_cotangents(const T& a, const T& b) {
     p->more.push_back({y->fa, y->fb});
     p->more.insert(p->more.end(), y->more.begin(), y->more.end());
     return T(p);
+  }
+  if ((a.pending_pieces() || b.pending_pieces()) && a.be() == b.be() && a.dtype() == b.dtype() && a.shape() == b.shape()) {
+    // piece by piece over the common segmentation: data is added only where both have some
+    std::vector<ArrHolder::Piece> pa, pb, out;
+    pieces_of(a, &pa);
+    pieces_of(b, &pb);
+    size_t i = 0, j = 0;
+    int64_t ua = 0, ub = 0;   // rows of pa[i] / pb[j] already consumed
+    while (i < pa.size() && j < pb.size()) {
+      int64_t n = std::min(pa[i].len - ua, pb[j].len - ub);
+      auto part = [&](const ArrHolder::Piece& pc, int64_t used) -> T {
+        if (!pc.v) return T();
+        return (used == 0 && n == pc.len) ? T(pc.v) : slice(T(pc.v), 0, used, n);
+      };
+      T x = part(pa[i], ua), y = part(pb[j], ub);
+      if (x.valid() && y.valid()) out.push_back({n, add_cotangents(x, y).holder()});
+      else if (x.valid()) out.push_back({n, x.holder()});
+      else if (y.valid()) out.push_back({n, y.holder()});
+      else out.push_back({n, nullptr});
+      ua += n;
+      ub += n;
+      if (ua == pa[i].len) { ++i; ua = 0; }
+      if (ub == pb[j].len) { ++j; ub = 0; }
+    }
+    return from_pieces(a.be(), std::move(out), a.shape(), a.dtype());
   }
   return ewise2(HGPU_ADD, a, b);
 }
@@ -391,6 +435,7 @@ T transpose(const T& a, const std::vector<int>& perm) {
 }
 T reshape(const T& a, const Shape& s) { HD_OUT(reshape(be__->ctx, a.h(), (int)s.size(), ptr_or_dummy(s), &o__)); }
 T slice(const T& a, int dim, int64_t start, int64_t len) {
+  if (dim == 0 && a.pending_pieces() && start >= 0 && len >= 0 && start + len <= a.shape().at(0)) return slice_pieces(a, start, len);
   HD_VIEW_OF_EXPR(slice(x, dim, start, len))
   HD_OUT(slice(be__->ctx, a.h(), dim, start, len, &o__));
 }
@@ -412,7 +457,21 @@ T as_strided(const T& a, const Shape& shape, const Shape& strides, int64_t offse
   HD_OUT(as_strided(be__->ctx, a.h(), (int)shape.size(), ptr_or_dummy(shape), ptr_or_dummy(strides), offset, &o__));
 }
 T materialize(const T& a) { HD_OUT(materialize(be__->ctx, a.h(), &o__)); }
-T pad(const T& a, const Shape& lo, const Shape& hi) { HD_OUT(pad(be__->ctx, a.h(), ptr_or_dummy(lo), ptr_or_dummy(hi), &o__)); }
+T pad(const T& a, const Shape& lo, const Shape& hi) {
+  // zeros before and after along the first dim only: a pending concatenation
+  bool first_only = a.be()->fuse && a.rank() >= 1 && (int)lo.size() == a.rank() && (int)hi.size() == a.rank() && lo[0] >= 0 && hi[0] >= 0 && lo[0] + hi[0] > 0;
+  for (size_t i = 1; i < lo.size() && first_only; ++i) first_only = lo[i] == 0 && hi[i] == 0;
+  if (first_only) {
+    std::vector<ArrHolder::Piece> pcs;
+    pcs.push_back({lo[0], nullptr});
+    pieces_of(a, &pcs);
+    pcs.push_back({hi[0], nullptr});
+    Shape sh = a.shape();
+    sh[0] += lo[0] + hi[0];
+    return from_pieces(a.be(), std::move(pcs), sh, a.dtype());
+  }
+  HD_OUT(pad(be__->ctx, a.h(), ptr_or_dummy(lo), ptr_or_dummy(hi), &o__));
+}
 static T ewise1_now(int op, const T& a) { HD_OUT(ewise1(be__->ctx, op, a.h(), &o__)); }
 static T ewise2_now(int op, const T& a, const T& b) { HD_OUT(ewise2(be__->ctx, op, a.h(), b.h(), &o__)); }
 static T compare_now(int cmp, const T& a, const T& b) { HD_OUT(compare(be__->ctx, cmp, a.h(), b.h(), &o__)); }
@@ -476,8 +535,67 @@ static T contract_now(const T& a, const T* b, int n_keep) {
   HD_OUT(contract(be__->ctx, a.h(), b ? b->h() : nullptr, n_keep, &o__));
 }
 T argminmax_last(const T& a, bool want_max) { HD_OUT(argminmax_last(be__->ctx, a.h(), want_max ? 1 : 0, &o__)); }
+// The pieces of t along its first dim (t itself when it is not a pending concatenation).
+static void pieces_of(const T& t, std::vector<ArrHolder::Piece>* out) {
+  if (t.pending_pieces()) {
+    for (auto& pc : t.holder()->pieces) out->push_back(pc);
+  } else {
+    out->push_back({t.shape().at(0), t.holder()});
+  }
+}
+static T from_pieces(Backend* be, std::vector<ArrHolder::Piece> pcs, const Shape& shape, int dtype) {
+  // neighbours without data merge; a single piece with data is that array
+  std::vector<ArrHolder::Piece> m;
+  for (auto& pc : pcs) {
+    if (pc.len == 0) continue;
+    if (!pc.v && !m.empty() && !m.back().v) m.back().len += pc.len;
+    else m.push_back(pc);
+  }
+  if (m.size() == 1 && m[0].v) return T(m[0].v);
+  if (m.empty()) return zeros(be, dtype, shape);
+  auto p = std::make_shared<ArrHolder>(be, nullptr);
+  p->pieces = std::move(m);
+  p->pshape = shape;
+  p->pdtype = dtype;
+  return T(p);
+}
+// rows [start, start + len) of a pending concatenation: the pieces that overlap them
+static T slice_pieces(const T& a, int64_t start, int64_t len) {
+  std::vector<ArrHolder::Piece> out;
+  int64_t at = 0;
+  for (auto& pc : a.holder()->pieces) {
+    int64_t lo = std::max(start, at), hi = std::min(start + len, at + pc.len);
+    if (lo < hi) {
+      if (!pc.v) out.push_back({hi - lo, nullptr});
+      else if (lo == at && hi == at + pc.len) out.push_back(pc);
+      else out.push_back({hi - lo, slice(T(pc.v), 0, lo - at, hi - lo).holder()});
+    }
+    at += pc.len;
+  }
+  Shape sh = a.shape();
+  sh[0] = len;
+  return from_pieces(a.be(), std::move(out), sh, a.dtype());
+}
+
 T concat(const std::vector<T>& parts) {
   if (parts.empty()) throw HostError(HGPU_ERR_INVALID, "concat of nothing");
+  {
+    const T& a0 = parts[0];
+    bool lazy = a0.be()->fuse && a0.rank() >= 1;
+    Shape sh = a0.shape();
+    int64_t total = 0;
+    for (auto& p : parts) {
+      Shape s = p.shape();
+      lazy = lazy && p.dtype() == a0.dtype() && s.size() == sh.size() && std::equal(s.begin() + 1, s.end(), sh.begin() + 1);
+      if (lazy) total += s[0];
+    }
+    if (lazy) {   // shapes agree: stays a list of pieces until someone needs the whole
+      std::vector<ArrHolder::Piece> pcs;
+      for (auto& p : parts) pieces_of(p, &pcs);
+      sh[0] = total;
+      return from_pieces(a0.be(), std::move(pcs), sh, a0.dtype());
+    }
+  }
   std::vector<const hgpu_array*> hs;
   for (auto& p : parts) hs.push_back(p.h());
   const T& a = parts[0];

@@ -176,3 +176,65 @@ def test_conv_vjp_chain_gpu_matches_cpu(host_gpu, host_cpu):
         res.append((out.numpy(), ga.numpy(), gk.numpy()))
     for g, c in zip(*res):
         assert np.allclose(g, c, rtol=1e-10, atol=1e-12)
+
+
+def append_slice_program(host, a, b, c):
+    """Stacked state of an unrolled recurrence in miniature: appends, slices that
+    hit piece boundaries and slices that straddle them, a slice used twice."""
+    pa, pb, pc = host.param(a), host.param(b), host.param(c)
+    s = pa.sappend(pb).sappend(pc)                     # [3+4+2, 5]
+    top, mid, low = s.sslice(0, 3), s.sslice(3, 4), s.sslice(7, 2)
+    straddle = s.sslice(2, 4)                          # rows of a and b
+    inner = s.sslice(4, 2)                             # inside b
+    t = top.op1("sin").sappend(mid * mid)              # [7, 5]
+    loss = (t.sslice(1, 5) * straddle.sappend(inner).sslice(0, 5)).ssum0() + (low * low).ssum0() + (s * s).ssum0() * host.srepl((), 0.5, pa.dtype)
+    grads = host.grad(loss, [pa, pb, pc])
+    return s.numpy(), loss.numpy(), [g.numpy() for g in grads]
+
+
+def append_slice_numpy(a, b, c):
+    s = np.concatenate([a, b, c])
+    t = np.concatenate([np.sin(a), b * b])
+    u = np.concatenate([s[2:6], s[4:6]])[0:5]
+    loss = (t[1:6] * u).sum() + (c * c).sum() + 0.5 * (s * s).sum()
+    # gradient by hand
+    gs = s.copy()                                      # from 0.5 * sum s^2
+    gt = np.zeros_like(t)
+    gt[1:6] = u
+    gu = np.zeros((6, 5))
+    gu[0:5] = t[1:6]
+    gs[2:6] += gu[0:4]
+    gs[4:6] += gu[4:6]
+    ga = gs[0:3] + gt[0:3] * np.cos(a)
+    gb = gs[3:7] + gt[3:7] * 2 * b
+    gc = gs[7:9] + 2 * c
+    return s, loss, [ga, gb, gc]
+
+
+def check_append_slice(host):
+    a, b, c = RNG.uniform(-1, 1, (3, 5)), RNG.uniform(-1, 1, (4, 5)), RNG.uniform(-1, 1, (2, 5))
+    s, loss, grads = append_slice_program(host, a, b, c)
+    ws, wl, wg = append_slice_numpy(a, b, c)
+    assert np.array_equal(s, ws)
+    assert np.isclose(float(loss), wl, rtol=1e-12)
+    for g, w in zip(grads, wg):
+        assert np.allclose(g, w, rtol=1e-12, atol=1e-14)
+    # the same with deferred evaluation off: every append and zero-extension is written out
+    host.set_fusion(False)
+    try:
+        s2, loss2, grads2 = append_slice_program(host, a, b, c)
+    finally:
+        host.set_fusion(True)
+    assert np.array_equal(s2, s)
+    assert np.isclose(float(loss2), float(loss), rtol=1e-12)
+    for g, w in zip(grads2, grads):
+        assert np.allclose(g, w, rtol=1e-12, atol=1e-14)
+
+
+def test_append_slice_pieces_cpu(host_cpu):
+    check_append_slice(host_cpu)
+
+
+@pytest.mark.gpu
+def test_append_slice_pieces_gpu(host_gpu):
+    check_append_slice(host_gpu)
