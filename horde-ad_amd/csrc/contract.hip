@@ -34,6 +34,16 @@ template <typename T> struct acc_of { using type = int64_t; };
 template <> struct acc_of<double> { using type = double; };
 template <> struct acc_of<float> { using type = double; };
 
+// Several products of one layout reduced by one launch (hgpu_contract_sum):
+// the chunk index s of a work item also selects the term, s = term * s_per +
+// chunk within the term, and the term's operands replace the kernel's pointer
+// arguments.  n == 0: one product.
+struct TermPtrs {
+  int n, s_per;
+  const void* a[hg::kGemmMaxTerms];
+  const void* b[hg::kGemmMaxTerms];
+};
+
 template <typename A>
 __device__ __forceinline__ A wave_sum(A v) {
 #pragma unroll
@@ -55,12 +65,21 @@ __device__ __forceinline__ A wave_sum(A v) {
 // [s*chunk, min(R, (s+1)*chunk)).  out is dense [n_out, S].
 template <typename TI, typename TO, bool HASB>
 __global__ void __launch_bounds__(kBlock) k_contract_lane(Dims keep, Dims red, int64_t n_out, int64_t R, int S, int64_t chunk,
-                                                           const TI* __restrict__ a, const TI* __restrict__ b, TO* __restrict__ out) {
+                                                           const TI* __restrict__ a0, const TI* __restrict__ b0, TO* __restrict__ out, TermPtrs tp) {
   using A = typename acc_of<TI>::type;
   int64_t items = n_out * S;
   int64_t step = (int64_t)gridDim.x * kBlock;
   for (int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x; item < items; item += step) {
     int64_t o = item % n_out, s = item / n_out;
+    const int64_t s_all = s;
+    const TI* a = a0;
+    const TI* b = b0;
+    if (tp.n) {
+      int term = (int)(s / tp.s_per);
+      s -= (int64_t)term * tp.s_per;
+      a = (const TI*)tp.a[term];
+      b = (const TI*)tp.b[term];
+    }
     int64_t ko[2];
     decompose<2>(keep, o, ko);
     int64_t r0 = s * chunk, r1 = r0 + chunk;
@@ -100,7 +119,7 @@ __global__ void __launch_bounds__(kBlock) k_contract_lane(Dims keep, Dims red, i
         ob += red.st[1][i];
       }
     }
-    out[o * S + s] = (TO)acc;
+    out[o * S + s_all] = (TO)acc;
   }
 }
 
@@ -136,7 +155,7 @@ __device__ __forceinline__ A lane_strided_sum(const TI* __restrict__ pa, const T
 // with Q = their product.  Chunks split Q when Q > 1, else Lin.
 template <typename TI, typename TO, bool HASB>
 __global__ void __launch_bounds__(kBlock) k_contract_wave(Dims keep, Dims red, int64_t n_out, int64_t Q, int64_t Lin, int64_t sa_in, int64_t sb_in,
-                                                           int S, int64_t chunk, const TI* __restrict__ a, const TI* __restrict__ b, TO* __restrict__ out) {
+                                                           int S, int64_t chunk, const TI* __restrict__ a0, const TI* __restrict__ b0, TO* __restrict__ out, TermPtrs tp) {
   using A = typename acc_of<TI>::type;
   const int lane = threadIdx.x & 63;
   int64_t wave = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
@@ -145,6 +164,14 @@ __global__ void __launch_bounds__(kBlock) k_contract_wave(Dims keep, Dims red, i
   for (int64_t item = wave; item < items; item += nwaves) {
     int64_t o = item / S;
     int s = (int)(item - o * S);
+    const TI* a = a0;
+    const TI* b = b0;
+    if (tp.n) {
+      int term = s / tp.s_per;
+      s -= term * tp.s_per;
+      a = (const TI*)tp.a[term];
+      b = (const TI*)tp.b[term];
+    }
     int64_t ko[2];
     decompose<2>(keep, o, ko);
     int64_t q0 = 0, q1 = Q, j0 = 0, j1 = Lin;
@@ -307,7 +334,14 @@ __global__ void __launch_bounds__(1024) k_argminmax_block(Dims keep, int64_t L, 
 }
 
 template <typename TI, typename TO>
-int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red_full, int64_t n_out, int64_t R, int S, const void* a, const void* b, void* out) {
+int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red_full, int64_t n_out, int64_t R, int S, const void* a, const void* b, void* out,
+                 const TermPtrs* terms = nullptr) {
+  // with terms, S counts the chunks of all of them; each term is cut into s_per
+  TermPtrs tp;
+  tp.n = 0;
+  tp.s_per = S;
+  if (terms) tp = *terms;
+  const int S_per = tp.n ? tp.s_per : S;
   const char* label = b ? (use_wave ? "contract_dot_wave" : "contract_dot_lane") : (use_wave ? "contract_sum_wave" : "contract_sum_lane");
   if (ctx->profiling && ctx->profile_shapes) {
     char buf[160];
@@ -339,16 +373,16 @@ int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red
     int64_t Q = R / Lin;
     if (red.nd > 1) { red.nd -= 1; } else { red.shape[0] = 1; red.st[0][0] = red.st[1][0] = 0; }
     int64_t span = Q > 1 ? Q : Lin;
-    int64_t chunk = (span + S - 1) / S;
+    int64_t chunk = (span + S_per - 1) / S_per;
     int64_t items = n_out * S;
     unsigned g = grid_for(items * 64, kBlock, maxb);
-    if (b) hipLaunchKernelGGL((k_contract_wave<TI, TO, true>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red, n_out, Q, Lin, sa, sb, S, chunk, (const TI*)a, (const TI*)b, (TO*)out);
-    else hipLaunchKernelGGL((k_contract_wave<TI, TO, false>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red, n_out, Q, Lin, sa, sb, S, chunk, (const TI*)a, (const TI*)nullptr, (TO*)out);
+    if (b) hipLaunchKernelGGL((k_contract_wave<TI, TO, true>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red, n_out, Q, Lin, sa, sb, S, chunk, (const TI*)a, (const TI*)b, (TO*)out, tp);
+    else hipLaunchKernelGGL((k_contract_wave<TI, TO, false>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red, n_out, Q, Lin, sa, sb, S, chunk, (const TI*)a, (const TI*)nullptr, (TO*)out, tp);
   } else {
-    int64_t chunk = (R + S - 1) / S;
+    int64_t chunk = (R + S_per - 1) / S_per;
     unsigned g = grid_for(n_out * S, kBlock, maxb);
-    if (b) hipLaunchKernelGGL((k_contract_lane<TI, TO, true>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red_full, n_out, R, S, chunk, (const TI*)a, (const TI*)b, (TO*)out);
-    else hipLaunchKernelGGL((k_contract_lane<TI, TO, false>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red_full, n_out, R, S, chunk, (const TI*)a, (const TI*)nullptr, (TO*)out);
+    if (b) hipLaunchKernelGGL((k_contract_lane<TI, TO, true>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red_full, n_out, R, S, chunk, (const TI*)a, (const TI*)b, (TO*)out, tp);
+    else hipLaunchKernelGGL((k_contract_lane<TI, TO, false>), dim3(g), dim3(kBlock), 0, ctx->stream, keep, red_full, n_out, R, S, chunk, (const TI*)a, (const TI*)nullptr, (TO*)out, tp);
   }
   HG_CHECK_LAUNCH(ctx, "contract");
   return HGPU_OK;
@@ -372,6 +406,59 @@ int add_into(hgpu_ctx* ctx, hgpu_array** acc, hgpu_array* x) {
   hgpu_release(*acc);
   hgpu_release(x);
   *acc = rc ? nullptr : sum;
+  return rc;
+}
+
+// out = sum_t contract(as[t], bs[t]) for terms of one layout that are not a
+// matrix product: the terms' chunks are reduced by one launch into partials
+// [n_out, n * S], a second launch adds the partials up.
+int contract_terms(hgpu_ctx* ctx, int n, const hgpu_array* const* as, const hgpu_array* const* bs, int n_keep, hgpu_array* o) {
+  const hgpu_array* a = as[0];
+  const hgpu_array* b = bs[0];
+  int64_t n_out = nelem(o), R = 1;
+  for (int i = n_keep; i < a->rank; ++i) R *= a->shape[i];
+  const int64_t* ks[2] = {a->strides, b->strides};
+  const int64_t* rs[2] = {a->strides + n_keep, b->strides + n_keep};
+  Dims keep, red;
+  if (!collapse(n_keep, a->shape, 2, ks, &keep) || !collapse(a->rank - n_keep, a->shape + n_keep, 2, rs, &red))
+    return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract_sum: more than %d merged dims", HG_KDIMS);
+  int64_t sr = min_abs_nonzero(red, red.nd - 1), sk = min_abs_nonzero(keep, keep.nd - 1);
+  int64_t Lin = red.shape[red.nd - 1];
+  bool use_wave = n_out < 2048 || (sr <= sk && Lin >= 16);
+  int64_t want_items = (int64_t)ctx->num_cu * (use_wave ? 16 : 1024);
+  int64_t S = 1;
+  if (n_out * n < want_items) {
+    S = (want_items + n_out * n - 1) / (n_out * n);
+    int64_t span = use_wave ? ((R / Lin) > 1 ? (R / Lin) : Lin) : R;
+    int64_t per = use_wave ? ((R / Lin) > 1 ? 2048 / (Lin < 2048 ? Lin : 2048) : 1024) : 256;
+    if (per < 1) per = 1;
+    int64_t maxS = span / per;
+    if (maxS < 1) maxS = 1;
+    if (S > maxS) S = maxS;
+    if (S > 128) S = 128;
+  }
+  TermPtrs tp;
+  tp.n = n;
+  tp.s_per = (int)S;
+  for (int t = 0; t < n; ++t) { tp.a[t] = data_ptr(as[t]); tp.b[t] = data_ptr(bs[t]); }
+  const int64_t S_all = S * n;
+  int accdt = dtype_is_float(a->dtype) ? HGPU_F64 : HGPU_I64;
+  int64_t psh[2] = {n_out, S_all};
+  hgpu_array* part = nullptr;
+  int rc = new_dense(ctx, accdt, 2, psh, &part);
+  if (rc) return rc;
+  HG_DISPATCH_DTYPE(a->dtype, T, { using A = typename acc_of<T>::type; rc = (launch_stage<T, A>(ctx, use_wave, keep, red, n_out, R, (int)S_all, tp.a[0], tp.b[0], data_ptr(part), &tp)); });
+  if (!rc) {
+    Dims k2, r2;
+    int64_t z1[1] = {0};
+    const int64_t* ks2[2] = {part->strides, z1};
+    const int64_t* rs2[2] = {part->strides + 1, z1};
+    collapse(1, psh, 2, ks2, &k2);
+    collapse(1, psh + 1, 2, rs2, &r2);
+    bool wave2 = n_out < 65536;
+    HG_DISPATCH_DTYPE(a->dtype, T, { using A = typename acc_of<T>::type; rc = (launch_stage<A, T>(ctx, wave2, k2, r2, n_out, S_all, 1, data_ptr(part), nullptr, data_ptr(o))); });
+  }
+  hgpu_release(part);
   return rc;
 }
 
@@ -414,6 +501,10 @@ int hgpu_contract_sum(hgpu_ctx* ctx, int n, const hgpu_array* const* as, const h
       rc = new_dense(ctx, a->dtype, n_keep, a->shape, &part);
       bool handled = false;
       if (!rc) rc = try_gemm(ctx, ga[0], gb[0], n_keep, part, &handled, (int)ga.size(), ga.data(), gb.data());
+      if (!rc && !handled && nelem(part) > 0) {   // not a matrix product: the grouped reduction
+        rc = contract_terms(ctx, (int)ga.size(), ga.data(), gb.data(), n_keep, part);
+        handled = !rc;
+      }
       if (rc || !handled) { if (part) hgpu_release(part); part = nullptr; }
       else done = ga.size();
     }

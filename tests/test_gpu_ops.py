@@ -330,6 +330,16 @@ def test_contract_sum(both, dt):
     b2 = both.upload(rnd((40, 30, 50), dt))
     assert_same(both.contract_sum([(a1, b1), (a2, b2)], 2), tol * 4)
     assert_same(both.contract_sum([(a1, b1)], 1), tol * 4)
+    # terms of one layout that are no matrix product (row-wise dots: bias gradients
+    # of an unrolled recurrence): one grouped reduction
+    for shape, keep, perm in [((128, 700), 1, None), ((128, 700), 0, None), ((300, 40), 1, [1, 0]), ((6, 5, 64), 2, None), ((3000, 8), 1, None)]:
+        pairs = []
+        for _ in range(7):
+            a, b = both.upload(rnd(shape, dt)), both.upload(rnd(shape, dt))
+            if perm:
+                a, b = a.transpose(perm), b.transpose(perm)
+            pairs.append((a, b))
+        assert_same(both.contract_sum(pairs, keep), tol * 4, (shape, keep, perm))
     # two layouts interleaved, one of them with a replicated (stride 0) operand:
     # each layout is one grouped launch
     pairs = []
