@@ -80,6 +80,47 @@ def time_graph(host, wl, ps, ds, steps, warmup):
         graph.free()
 
 
+def time_train_graph(pkg, host, wl, steps, warmup):
+    """One training step -- gradient, Adam update of every parameter array, new
+    parameters and moments written back where the next launch reads them --
+    recorded once and launched per step: the parameters never leave the device."""
+    import numpy as np
+    OPT = pkg.optimizer
+    ps, ds = wl.upload(host)
+    args = OPT.defaultArgsAdam
+    ms = [host.concrete(np.zeros_like(x)) for x in wl.params]
+    vs = [host.concrete(np.zeros_like(x)) for x in wl.params]
+    alphat = OPT.adamStepSize(host, ps[0].dtype, args, 1)
+
+    def step():
+        loss, grads = wl.gradient(host, ps, ds)
+        mn, vn, pn = OPT.adamApply(args, alphat, ms, vs, ps, grads)
+        for dst, src in zip(ms + vs + ps, mn + vn + pn):
+            dst.assign(src)
+        return loss
+
+    step()
+    host.sync()
+    graph, loss = host.capture(step)
+    try:
+        t = 1
+        for _ in range(warmup):
+            t += 1
+            alphat.overwrite(OPT.adamStepSize(host, ps[0].dtype, args, t).numpy())
+            graph.launch()
+            host.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            t += 1
+            alphat.overwrite(OPT.adamStepSize(host, ps[0].dtype, args, t).numpy())
+            graph.launch()
+            host.sync()
+        dt = time.perf_counter() - t0
+        return dt / steps
+    finally:
+        graph.free()
+
+
 def profile(capi, host, wl, ps, ds, reps=2):
     """Per-launch HIP-event timing by the library, one label per kernel and
     problem shape: {label: (launches, ms, bytes, flops)} per gradient."""
@@ -167,6 +208,8 @@ def main():
     ap.add_argument("--only", action="store_true", help="measure the headline config only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--eager", action="store_true", help="time op-by-op submission instead of the recorded graph")
+    ap.add_argument("--train", action="store_true",
+                    help="also time a recorded training step (gradient + Adam + write-back) of the headline config")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run plain dense copies of 1 GiB (for scaling hardware traffic counters) and exit")
     args = ap.parse_args()
@@ -218,6 +261,12 @@ def main():
         del ps, ds
 
     head = results[args.workload]
+    train = None
+    if args.train:
+        wl = W.CONFIGS[args.workload]()
+        sec = time_train_graph(pkg, host, wl, args.steps, args.warmup)
+        train = {"ms_per_step": sec * 1e3, "samples_per_s": wl.batch / sec, "optimizer": "Adam, reference defaults",
+                 "execution": "recorded graph: gradient, update and write-back in one launch"}
     cpu = None if args.no_cpu else cpu_baseline(pkg, args.workload, W.CONFIGS[args.workload])
     line = {
         "metric": "gradient samples/sec at 1 GPU", "value": head["samples_per_s"], "unit": "samples/s",
@@ -229,6 +278,8 @@ def main():
         "configs": {k: v for k, v in results.items() if k != args.workload},
         "headline_detail": {k: v for k, v in head.items() if k != "roofline"},
     }
+    if train:
+        line["training_step"] = train
     print(json.dumps(line))
 
 

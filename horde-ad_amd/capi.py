@@ -50,6 +50,7 @@ SIGNATURES = {
     "onehot": (I, [P, P, I, LP, LP, PP]), "get_api": (P, []),
     "scatter_affine": (I, [P, P, I, I, LP, LP, LP, PP]),
     "contract_sum": (I, [P, I, PP, PP, I, PP]),
+    "assign": (I, [P, P, P]),
 }
 # exported by the GPU library only
 GPU_ONLY = {

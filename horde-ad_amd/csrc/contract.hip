@@ -354,8 +354,9 @@ int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red
     snprintf(buf + n, sizeof buf - n, "]");
     label = ctx->label_pool.insert(buf).first->c_str();
   }
+  const double nterms = tp.n ? tp.n : 1;
   LaunchGuard lg(ctx, label,
-                 (double)n_out * R * sizeof(TI) * (b ? 2 : 1) + (double)n_out * S * sizeof(TO), (double)n_out * R * (b ? 2 : 1));
+                 (double)n_out * R * sizeof(TI) * (b ? 2 : 1) * nterms + (double)n_out * S * sizeof(TO), (double)n_out * R * (b ? 2 : 1) * nterms);
   int maxb = ctx->num_cu * 8;
   if (use_wave && S == 0) {       // one block per output, no partials
     Dims red = red_full;

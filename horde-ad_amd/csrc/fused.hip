@@ -395,8 +395,13 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   if (ctx->profiling && ctx->profile_shapes) {
     std::string sh;
     for (int d = 0; d < a0->rank; ++d) sh += (d ? "x" : "") + std::to_string(a0->shape[d]);
-    char buf[160];
-    snprintf(buf, sizeof buf, "fused_map[%s,in%d(%s),instr%d(k%d.op%d..),out%d,vec%d,dt%d]", sh.c_str(), n_in, layout.c_str(), n_instr, prog[0].kind, prog[0].op, n_out, vec, a0->dtype);
+    // strides of the first input that is a general view
+    std::string gst;
+    for (int i = 0; i < n_in && gst.empty(); ++i)
+      if (layout[(size_t)i] == 'g')
+        for (int d = 0; d < in[i]->rank; ++d) gst += (d ? ":" : ",g") + std::to_string(in[i]->strides[d]);
+    char buf[200];
+    snprintf(buf, sizeof buf, "fused_map[%s,in%d(%s),instr%d(k%d.op%d..),out%d,vec%d,dt%d%s]", sh.c_str(), n_in, layout.c_str(), n_instr, prog[0].kind, prog[0].op, n_out, vec, a0->dtype, gst.c_str());
     label = ctx->label_pool.insert(buf).first->c_str();
   }
   LaunchGuard lg(ctx, label, 0, 0);

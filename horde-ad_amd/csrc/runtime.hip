@@ -500,6 +500,15 @@ int hgpu_overwrite(hgpu_ctx* ctx, hgpu_array* a, const void* host) {
   return check_hip(ctx, e, "overwrite");
 }
 
+int hgpu_assign(hgpu_ctx* ctx, hgpu_array* dst, const hgpu_array* src) {
+  if (!ctx || !dst || !src) return HGPU_ERR_INVALID;
+  if (dst->dtype != src->dtype || !same_shape(dst, src)) return fail(ctx, HGPU_ERR_INVALID, "assign: shapes or dtypes differ");
+  if (!is_dense(dst)) return fail(ctx, HGPU_ERR_INVALID, "assign: the destination is a strided view");
+  if (nelem(dst) == 0) return HGPU_OK;
+  if (dst->buf == src->buf) return fail(ctx, HGPU_ERR_INVALID, "assign: source and destination share memory");
+  return copy_view(ctx, dst->dtype, dst->rank, dst->shape, data_ptr(src), src->strides, data_ptr(dst), dst->strides);
+}
+
 int hgpu_download(hgpu_ctx* ctx, const hgpu_array* a, void* host) {
   if (!ctx || !a) return HGPU_ERR_INVALID;
   if (int rc = no_capture(ctx, "download")) return rc;

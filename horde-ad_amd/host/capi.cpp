@@ -158,6 +158,43 @@ int hh_overwrite(hh_ctx* c, hh_val* v, const void* host) {
     c->be.check(c->be.api->overwrite(c->be.ctx, v->d.primal.h(), host));
   });
 }
+int hh_assign(hh_ctx* c, hh_val* dst, hh_val* src) {
+  return guarded(c, [&] { assign(dst->d.primal, src->d.primal); });
+}
+static hh_val* box_plain(const T& t) {
+  D d;
+  d.primal = t;
+  return box(d);
+}
+int hh_update_with_gradient(hh_ctx* c, double gamma, hh_val* p, hh_val* g, hh_val** out) {
+  return guarded(c, [&] { *out = box_plain(update_with_gradient(gamma, p->d.primal, g->d.primal)); });
+}
+int hh_adam_step_size(hh_ctx* c, int dtype, double alpha, double beta1, double beta2, int t_new, hh_val** out) {
+  return guarded(c, [&] { *out = box_plain(adam_step_size(&c->be, dtype, alpha, beta1, beta2, t_new)); });
+}
+int hh_adam_apply(hh_ctx* c, hh_val* alphat, double beta1, double beta2, double epsilon, hh_val* m, hh_val* v, hh_val* p, hh_val* g, hh_val** m_new,
+                  hh_val** v_new, hh_val** p_new) {
+  return guarded(c, [&] {
+    T mn, vn, pn;
+    adam_update(alphat->d.primal, beta1, beta2, epsilon, m->d.primal, v->d.primal, p->d.primal, g->d.primal, &mn, &vn, &pn);
+    *m_new = box_plain(mn);
+    *v_new = box_plain(vn);
+    *p_new = box_plain(pn);
+  });
+}
+int hh_update_with_gradient_adam(hh_ctx* c, double alpha, double beta1, double beta2, double epsilon, int t_new, hh_val* m, hh_val* v, hh_val* p,
+                                 hh_val* g, hh_val** m_new, hh_val** v_new, hh_val** p_new) {
+  return guarded(c, [&] {
+    T mn, vn, pn;
+    const T& pp = p->d.primal;
+    T at = (pp.dtype() == HGPU_F64 || pp.dtype() == HGPU_F32) ? adam_step_size(&c->be, pp.dtype(), alpha, beta1, beta2, t_new) : T();
+    if (!at.valid()) { mn = m->d.primal; vn = v->d.primal; pn = pp; }
+    else adam_update(at, beta1, beta2, epsilon, m->d.primal, v->d.primal, pp, g->d.primal, &mn, &vn, &pn);
+    *m_new = box_plain(mn);
+    *v_new = box_plain(vn);
+    *p_new = box_plain(pn);
+  });
+}
 int hh_val_rank(hh_val* v) { return v->d.primal.rank(); }
 int hh_val_dtype(hh_val* v) { return v->d.primal.dtype(); }
 int hh_val_shape(hh_val* v, int64_t* s) {

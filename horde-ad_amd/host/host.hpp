@@ -170,6 +170,11 @@ T gather_raw(const T& src, const std::vector<T>& ix, const Shape& shm);
 T scatter_raw(const T& src, const std::vector<T>& ix, int rank_m, const Shape& shp, int flags);
 T onehot(const T& v, const Shape& ix, const Shape& shp);
 T zeros(Backend* be, int dtype, const Shape& shape);               // stride-0 view of a cached 0
+// optimizer.cpp (External/OptimizerTools.hs)
+T update_with_gradient(double gamma, const T& p, const T& g);
+void adam_update(const T& alphat, double beta1, double beta2, double epsilon, const T& m, const T& v, const T& p, const T& g, T* m_new, T* v_new, T* p_new);
+T adam_step_size(Backend* be, int dtype, double alpha, double beta1, double beta2, int t_new);
+void assign(const T& dst, const T& src);                           // dst's memory takes src's elements
 T broadcast_scalar(const T& s, const Shape& shape);                // tsreplicate0N
 
 // ---- BaseTensor-named operations (Ops.hs line of each method in the .cpp) --

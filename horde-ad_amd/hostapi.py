@@ -38,7 +38,11 @@ SIG = {
     "ix_is_affine": (I, [P]),
     "tsgather": (I, [P, P, I, LP, I, PP, PP]), "tsscatter": (I, [P, P, I, I, LP, PP, PP]),
     "capture_begin": (I, [P]), "capture_end": (I, [P, PP]), "graph_launch": (I, [P, P]), "graph_free": (I, [P, P]),
-    "force": (I, [P, P]), "overwrite": (I, [P, P, P]),
+    "force": (I, [P, P]), "overwrite": (I, [P, P, P]), "assign": (I, [P, P, P]),
+    "update_with_gradient": (I, [P, D, P, P, PP]),
+    "update_with_gradient_adam": (I, [P, D, D, D, D, I, P, P, P, P, PP, PP, PP]),
+    "adam_step_size": (I, [P, I, D, D, D, I, PP]),
+    "adam_apply": (I, [P, P, D, D, D, P, P, P, P, PP, PP, PP]),
 }
 
 _dll = None
@@ -301,9 +305,16 @@ class V:
 
     def overwrite(self, x):
         """New contents for an input of a recorded program (same shape and dtype)."""
-        x = np.ascontiguousarray(x, dtype=_DT2NP[self.dtype])
+        x = np.asarray(x, dtype=_DT2NP[self.dtype])
+        if not x.flags.c_contiguous:
+            x = x.copy(order="C")
         assert tuple(x.shape) == tuple(self.shape)
         self.host.check(self.host.dll.hh_overwrite(self.host.h, self.h, x.ctypes.data_as(C.c_void_p)))
+
+    def assign(self, src):
+        """This array's memory takes src's elements (how a recorded training step
+        hands updated parameters to its next launch)."""
+        self.host.check(self.host.dll.hh_assign(self.host.h, self.h, src.h))
 
     def _o(self, fn, *args):
         return self.host._out(fn, *args)

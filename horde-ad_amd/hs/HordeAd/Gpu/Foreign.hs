@@ -97,6 +97,19 @@ foreign import ccall safe "hh_tsgather" c_hh_tsgather
 foreign import ccall safe "hh_tsscatter" c_hh_tsscatter
   :: Ptr Ctx -> Ptr Val -> CInt -> CInt -> Ptr Int64 -> Ptr (Ptr Ix) -> Ptr (Ptr Val) -> IO CInt
 
+-- Gradient descent on device arrays (External/OptimizerTools.hs:20-47, 137-225)
+foreign import ccall safe "hh_update_with_gradient" c_hh_update_with_gradient
+  :: Ptr Ctx -> CDouble -> Ptr Val -> Ptr Val -> Ptr (Ptr Val) -> IO CInt
+foreign import ccall safe "hh_update_with_gradient_adam" c_hh_update_with_gradient_adam
+  :: Ptr Ctx -> CDouble -> CDouble -> CDouble -> CDouble -> CInt -> Ptr Val -> Ptr Val -> Ptr Val -> Ptr Val
+  -> Ptr (Ptr Val) -> Ptr (Ptr Val) -> Ptr (Ptr Val) -> IO CInt
+foreign import ccall safe "hh_adam_step_size" c_hh_adam_step_size
+  :: Ptr Ctx -> CInt -> CDouble -> CDouble -> CDouble -> CInt -> Ptr (Ptr Val) -> IO CInt
+foreign import ccall safe "hh_adam_apply" c_hh_adam_apply
+  :: Ptr Ctx -> Ptr Val -> CDouble -> CDouble -> CDouble -> Ptr Val -> Ptr Val -> Ptr Val -> Ptr Val
+  -> Ptr (Ptr Val) -> Ptr (Ptr Val) -> Ptr (Ptr Val) -> IO CInt
+foreign import ccall safe "hh_assign" c_hh_assign :: Ptr Ctx -> Ptr Val -> Ptr Val -> IO CInt
+
 -- | The process-wide context (the tensor classes are pure, so there is no
 -- place to thread a handle through; the reference has the same kind of global
 -- in its AST variable counter, src/HordeAd/Core/AstFreshId.hs:35-48).

@@ -304,6 +304,13 @@ int hgpu_graph_destroy(hgpu_graph* g);
  * dtype).  The one exception to "arrays are immutable": meant for the input
  * arrays of a captured graph, between launches. */
 int hgpu_overwrite(hgpu_ctx* ctx, hgpu_array* a, const void* host);
+/* Replaces the contents of the dense array dst with the elements of src (same
+ * shape and dtype, any view, not of dst's own memory), on the device.  The
+ * second exception to "arrays are immutable": the parameter update of a
+ * training step (External/OptimizerTools.hs:20-47, 137-225 return new arrays;
+ * a recorded step must put them where its next launch reads its parameters).
+ * May be recorded into a graph. */
+int hgpu_assign(hgpu_ctx* ctx, hgpu_array* dst, const hgpu_array* src);
 
 /* ------------------------------------------------------------- api table */
 
@@ -358,6 +365,7 @@ typedef struct hgpu_api {
   int (*graph_destroy)(hgpu_graph*);
   int (*overwrite)(hgpu_ctx*, hgpu_array*, const void*);
   int (*contract_sum)(hgpu_ctx*, int, const hgpu_array* const*, const hgpu_array* const*, int, hgpu_array**);
+  int (*assign)(hgpu_ctx*, hgpu_array*, const hgpu_array*);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

@@ -73,10 +73,31 @@ int hh_graph_launch(hh_ctx* ctx, hh_graph* g);
 int hh_graph_free(hh_ctx* ctx, hh_graph* g);
 int hh_force(hh_ctx* ctx, hh_val* v);
 int hh_overwrite(hh_ctx* ctx, hh_val* v, const void* host);
+/* dst's memory takes src's elements (same shape and type; dst an array made by
+ * upload, src not a view of it): how a recorded training step hands the
+ * updated parameters to its next launch. */
+int hh_assign(hh_ctx* ctx, hh_val* dst, hh_val* src);
 int hh_val_rank(hh_val* v);
 int hh_val_dtype(hh_val* v);
 int hh_val_shape(hh_val* v, int64_t* shape);
 int hh_free(hh_val* v);
+
+/* Gradient descent on device arrays (External/OptimizerTools.hs).
+ * hh_update_with_gradient: updateWithGradient (:20-47), params - gamma * gradient
+ * for one array; arrays of a non-differentiable type come back unchanged.
+ * hh_update_with_gradient_adam: updateWithGradientAdam (:137-225) for one array;
+ * t_new is the iteration count AFTER this step (tAdam + 1), from which the
+ * step size alphat = alpha * sqrt (1 - beta2^t) / (1 - beta1^t) is computed on
+ * the host as the reference does.  hh_adam_apply is the same update with
+ * alphat given as a rank-0 array (hh_adam_step_size makes one), for a recorded
+ * step whose step size changes between launches (hh_overwrite it).
+ * defaultArgsAdam (:82-88): alpha 0.001, beta1 0.9, beta2 0.999, epsilon 1e-7. */
+int hh_update_with_gradient(hh_ctx* ctx, double gamma, hh_val* params, hh_val* gradient, hh_val** out);
+int hh_update_with_gradient_adam(hh_ctx* ctx, double alpha, double beta1, double beta2, double epsilon, int t_new, hh_val* m, hh_val* v,
+                                 hh_val* params, hh_val* gradient, hh_val** m_new, hh_val** v_new, hh_val** params_new);
+int hh_adam_step_size(hh_ctx* ctx, int dtype, double alpha, double beta1, double beta2, int t_new, hh_val** out);
+int hh_adam_apply(hh_ctx* ctx, hh_val* alphat, double beta1, double beta2, double epsilon, hh_val* m, hh_val* v, hh_val* params, hh_val* gradient,
+                  hh_val** m_new, hh_val** v_new, hh_val** params_new);
 
 /* gradientFromDelta (DeltaEval.hs:64-78): cotangents of `inputs` for d(out)=dt. */
 int hh_backward(hh_ctx* ctx, hh_val* out, hh_val* dt, int n, hh_val* const* inputs, hh_val** grads);

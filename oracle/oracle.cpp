@@ -663,6 +663,14 @@ int horc_contract_sum(hgpu_ctx* c, int n, const hgpu_array* const* as, const hgp
   return HGPU_OK;
 }
 
+// Every array of the checker owns dense data, so assigning is copying the data.
+int horc_assign(hgpu_ctx* c, hgpu_array* dst, const hgpu_array* src) {
+  if (dst->dtype != src->dtype || dst->shape != src->shape) return fail(c, HGPU_ERR_INVALID, "assign: shapes or dtypes differ");
+  if (dst == src) return fail(c, HGPU_ERR_INVALID, "assign: source and destination share memory");
+  dst->data = src->data;
+  return HGPU_OK;
+}
+
 // toneHotS (OpsConcrete.hs:1516-1525)
 int horc_onehot(hgpu_ctx* c, const hgpu_array* v, int n, const int64_t* ix, const int64_t* shp, hgpu_array** out) {
   if (n < 0 || n + (int)v->shape.size() > HGPU_MAX_RANK) return fail(c, HGPU_ERR_INVALID, "onehot: rank too large");
@@ -729,7 +737,7 @@ const hgpu_api* horc_get_api(void) {
       horc_contract,    horc_argminmax_last, horc_iota,    horc_concat,     horc_gather,      horc_scatter_add,
       horc_onehot,      horc_fused_map, horc_scatter_affine,
       nullptr, nullptr, nullptr, nullptr, nullptr,   // no graphs: the checker executes eagerly
-      horc_contract_sum,
+      horc_contract_sum, horc_assign,
   };
   return &api;
 }
