@@ -54,6 +54,7 @@ SIGNATURES = {
 }
 # exported by the GPU library only
 GPU_ONLY = {
+    "extremum_last": (I, [P, P, I, PP, PP]),
     "mem_stats": (I, [P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "stream": (P, [P]), "inject_alloc_failure": (I, [P, L]),
     "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
@@ -287,6 +288,12 @@ class Array:
 
     def argminmax_last(self, want_max):
         return self._o(self.ctx.lib.argminmax_last, int(want_max))
+
+    def extremum_last(self, want_max):
+        """(values, indices) of the first extremum along the last dim (gfx950 library only)."""
+        v, i = C.c_void_p(), C.c_void_p()
+        self.ctx.check(self.ctx.lib.extremum_last(self.ctx.h, self.h, int(want_max), C.byref(v), C.byref(i)))
+        return Array(self.ctx, v), Array(self.ctx, i)
 
     def onehot(self, ix, shp):
         return self._o(self.ctx.lib.onehot, len(ix), _larr(ix), _larr(shp))

@@ -232,7 +232,7 @@ __global__ void __launch_bounds__(kBlock) k_contract_block(Dims keep, Dims red, 
 
 // First (want_max = 0: minimal, 1: maximal) element along the last dim.
 template <typename T>
-__global__ void __launch_bounds__(kBlock) k_argminmax(Dims keep, int64_t n_out, int64_t L, int64_t sl, int want_max, const T* __restrict__ a, int64_t* __restrict__ out) {
+__global__ void __launch_bounds__(kBlock) k_argminmax(Dims keep, int64_t n_out, int64_t L, int64_t sl, int want_max, const T* __restrict__ a, int64_t* __restrict__ out, T* __restrict__ vals) {
   int64_t step = (int64_t)gridDim.x * kBlock;
   for (int64_t o = (int64_t)blockIdx.x * kBlock + threadIdx.x; o < n_out; o += step) {
     int64_t ko[1];
@@ -246,6 +246,7 @@ __global__ void __launch_bounds__(kBlock) k_argminmax(Dims keep, int64_t n_out, 
       if (better) { best = x; bi = j; }
     }
     out[o] = bi;
+    if (vals) vals[o] = best;
   }
 }
 
@@ -253,7 +254,7 @@ __global__ void __launch_bounds__(kBlock) k_argminmax(Dims keep, int64_t n_out, 
 // strided subsequence keeping its first extremum, then lanes combine; on equal
 // values the smaller index wins, which keeps "first occurrence".
 template <typename T>
-__global__ void __launch_bounds__(kBlock) k_argminmax_wave(Dims keep, int64_t n_out, int64_t L, int64_t sl, int want_max, const T* __restrict__ a, int64_t* __restrict__ out) {
+__global__ void __launch_bounds__(kBlock) k_argminmax_wave(Dims keep, int64_t n_out, int64_t L, int64_t sl, int want_max, const T* __restrict__ a, int64_t* __restrict__ out, T* __restrict__ vals) {
   const int lane = threadIdx.x & 63;
   int64_t wave = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
   int64_t nwaves = ((int64_t)gridDim.x * kBlock) >> 6;
@@ -292,7 +293,10 @@ __global__ void __launch_bounds__(kBlock) k_argminmax_wave(Dims keep, int64_t n_
         if (better) { best = o_best; bi = o_bi; have = true; }
       }
     }
-    if (lane == 0) out[o] = bi;
+    if (lane == 0) {
+      out[o] = bi;
+      if (vals) vals[o] = best;
+    }
   }
 }
 
@@ -300,7 +304,7 @@ __global__ void __launch_bounds__(kBlock) k_argminmax_wave(Dims keep, int64_t n_
 // whole tensor): lanes scan strided subsequences, then combine through LDS with
 // the same "smaller index wins ties" rule.
 template <typename T>
-__global__ void __launch_bounds__(1024) k_argminmax_block(Dims keep, int64_t L, int64_t sl, int want_max, const T* __restrict__ a, int64_t* __restrict__ out) {
+__global__ void __launch_bounds__(1024) k_argminmax_block(Dims keep, int64_t L, int64_t sl, int want_max, const T* __restrict__ a, int64_t* __restrict__ out, T* __restrict__ vals) {
   __shared__ T sbest[1024];
   __shared__ int64_t sidx[1024];
   int64_t ko[1];
@@ -330,7 +334,10 @@ __global__ void __launch_bounds__(1024) k_argminmax_block(Dims keep, int64_t L, 
     }
     __syncthreads();
   }
-  if (t == 0) out[blockIdx.x] = sidx[0];
+  if (t == 0) {
+    out[blockIdx.x] = sidx[0];
+    if (vals) vals[blockIdx.x] = sbest[0];
+  }
 }
 
 template <typename TI, typename TO>
@@ -636,7 +643,7 @@ int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n
   return HGPU_OK;
 }
 
-int hgpu_argminmax_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_array** out) {
+int hgpu_extremum_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_array** values, hgpu_array** out) {
   if (!ctx || !a || !out) return HGPU_ERR_INVALID;
   if (a->rank < 1) return fail(ctx, HGPU_ERR_INVALID, "argminmax: rank 0");
   int64_t L = a->shape[a->rank - 1];
@@ -644,27 +651,38 @@ int hgpu_argminmax_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_a
   hgpu_array* o = nullptr;
   int rc = new_dense(ctx, HGPU_I64, a->rank - 1, a->shape, &o);
   if (rc) return rc;
+  hgpu_array* v = nullptr;
+  if (values) {
+    rc = new_dense(ctx, a->dtype, a->rank - 1, a->shape, &v);
+    if (rc) { hgpu_release(o); return rc; }
+  }
   int64_t n_out = nelem(o);
   if (n_out > 0) {
     const int64_t* ks[1] = {a->strides};
     Dims keep;
-    if (!collapse(a->rank - 1, a->shape, 1, ks, &keep)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "argminmax: too many dims"); }
-    LaunchGuard lg(ctx, "argminmax", (double)n_out * (L * dtype_size(a->dtype) + 8), (double)n_out * L);
+    if (!collapse(a->rank - 1, a->shape, 1, ks, &keep)) { hgpu_release(o); if (v) hgpu_release(v); return fail(ctx, HGPU_ERR_UNSUPPORTED, "argminmax: too many dims"); }
+    LaunchGuard lg(ctx, "argminmax", (double)n_out * (L * dtype_size(a->dtype) + 8 + (v ? dtype_size(a->dtype) : 0)), (double)n_out * L);
+    void* vp = v ? data_ptr(v) : nullptr;
     if (L >= 8192 && n_out <= 64) {
       // few long rows: a whole block per row
-      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_block<T>, dim3((unsigned)n_out), dim3(1024), 0, ctx->stream, keep, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_block<T>, dim3((unsigned)n_out), dim3(1024), 0, ctx->stream, keep, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o), (T*)vp));
     } else if (L >= 256 && n_out < (int64_t)ctx->num_cu * 64) {
       unsigned g = grid_for(n_out * 64, kBlock, ctx->num_cu * 8);
-      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_wave<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_wave<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o), (T*)vp));
     } else {
       unsigned g = grid_for(n_out, kBlock, ctx->num_cu * 8);
-      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o)));
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax<T>, dim3(g), dim3(kBlock), 0, ctx->stream, keep, n_out, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o), (T*)vp));
     }
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "argminmax"); }
+    if (e != hipSuccess) { hgpu_release(o); if (v) hgpu_release(v); return check_hip(ctx, e, "argminmax"); }
   }
   *out = o;
+  if (values) *values = v;
   return HGPU_OK;
+}
+
+int hgpu_argminmax_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_array** out) {
+  return hgpu_extremum_last(ctx, a, want_max, nullptr, out);
 }
 
 }  // extern "C"

@@ -219,6 +219,11 @@ struct Ix {
   std::vector<int64_t> coef;
   T arr;                       // otherwise: array of shape shm (any dtype, any strides)
   int dtype = HGPU_I64;
+  // kargMin / kargMax of `arg_of !$ [m_0, ..]` at the position itself: the
+  // extremal values came out of the same pass (arg_vals), so a gather of
+  // arg_of at [m_0, .., this] is arg_vals.
+  std::shared_ptr<ArrHolder> arg_of;
+  T arg_vals;
 };
 
 Ix ix_var(Backend* be, const Shape& shm, int d);

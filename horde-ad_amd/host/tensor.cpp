@@ -892,6 +892,17 @@ T tsgather(const T& src, const Shape& shm, const std::vector<Ix>& ix) {
   if ((int)ix.size() > src.rank()) throw HostError(HGPU_ERR_INVALID, "tsgather: more indices than dims");
   check_ix(shm, ix);
   Backend* be = src.be();
+  // src at [m_0, .., kargMax (src !$ [m_0, ..])]: the values the arg pass produced
+  if (!ix.empty() && (int)ix.size() == src.rank() && ix.back().arg_of && ix.back().arg_of == src.holder() && shm.size() + 1 == ix.size()) {
+    bool identity = true;
+    Shape ssh = src.shape();
+    for (size_t d = 0; d + 1 < ix.size() && identity; ++d) {
+      const Ix& x = ix[d];
+      identity = x.affine && x.c0 == 0 && shm[d] == ssh[d];
+      for (size_t e = 0; e < x.coef.size() && identity; ++e) identity = x.coef[e] == (e == d ? 1 : 0);
+    }
+    if (identity) return ix.back().arg_vals;
+  }
   if (all_affine(ix)) {
     // windows of a pending expression that stay in bounds and do not multiply
     // its elements are taken of its leaves instead
@@ -1230,10 +1241,28 @@ Ix ix_index0(Backend* be, const T& t, const std::vector<Ix>& ix) {
   return from_array(shm, gather_raw(t, arrs, shm));
 }
 
-Ix ix_argminmax(Backend*, const T& t, const std::vector<Ix>& ix, bool want_max) {
+Ix ix_argminmax(Backend* be, const T& t, const std::vector<Ix>& ix, bool want_max) {
   if ((int)ix.size() + 1 != t.rank()) throw HostError(HGPU_ERR_INVALID, "ix_argminmax: the partial index must leave one dim");
   if (ix.empty()) throw HostError(HGPU_ERR_INVALID, "ix_argminmax: no position space");
   const Shape& shm = ix[0].shm;
+  // the index is the position itself (kargMax (t !$ [i, j, ..]) over t's own
+  // leading dims): one pass yields the arguments and the extremal values
+  bool identity = shm.size() == ix.size();
+  Shape tsh = t.shape();
+  for (size_t d = 0; d < ix.size() && identity; ++d) {
+    const Ix& x = ix[d];
+    identity = x.affine && x.c0 == 0 && shm[d] == tsh[d];
+    for (size_t e = 0; e < x.coef.size() && identity; ++e) identity = x.coef[e] == (e == d ? 1 : 0);
+  }
+  const hgpu_api* api = be->api;
+  if (identity && be->fuse && api->struct_size >= offsetof(hgpu_api, extremum_last) + sizeof(api->extremum_last) && api->extremum_last) {
+    hgpu_array *vals = nullptr, *idx = nullptr;
+    be->check(api->extremum_last(be->ctx, t.h(), want_max ? 1 : 0, &vals, &idx));
+    Ix r = from_array(shm, T(be, idx));
+    r.arg_of = t.holder();
+    r.arg_vals = T(be, vals);
+    return r;
+  }
   T part = tsgather(t, shm, ix);  // shm ++ [n]
   return from_array(shm, argminmax_last(part, want_max));
 }

@@ -239,6 +239,10 @@ int hgpu_contract_sum(hgpu_ctx* ctx, int n, const hgpu_array* const* a, const hg
  * the first minimal / maximal element along the LAST dim; result I64 of shape
  * init(shape). */
 int hgpu_argminmax_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_array** out);
+/* The same pass also hands out the extremal VALUES (values may be NULL):
+ * `sgather t (\ix -> ix ++ [kargMax (t !$ ix)])`, the maximum of every pooling
+ * window (External/CommonShapedOps.hs:241-260), is then no gather at all. */
+int hgpu_extremum_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_array** values, hgpu_array** indices);
 /* tsiota (OpsConcrete.hs:535-536): [0, 1, ..., n-1] of the given dtype. */
 int hgpu_iota(hgpu_ctx* ctx, int64_t n, int dtype, hgpu_array** out);
 /* tsappend / trconcat (OpsConcrete.hs:623-625,638-640): concatenation along
@@ -366,6 +370,7 @@ typedef struct hgpu_api {
   int (*overwrite)(hgpu_ctx*, hgpu_array*, const void*);
   int (*contract_sum)(hgpu_ctx*, int, const hgpu_array* const*, const hgpu_array* const*, int, hgpu_array**);
   int (*assign)(hgpu_ctx*, hgpu_array*, const hgpu_array*);
+  int (*extremum_last)(hgpu_ctx*, const hgpu_array*, int, hgpu_array**, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

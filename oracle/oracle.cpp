@@ -738,6 +738,7 @@ const hgpu_api* horc_get_api(void) {
       horc_onehot,      horc_fused_map, horc_scatter_affine,
       nullptr, nullptr, nullptr, nullptr, nullptr,   // no graphs: the checker executes eagerly
       horc_contract_sum, horc_assign,
+      nullptr,   // no extremum_last: the checker gathers at the arg-extremum as the reference does
   };
   return &api;
 }

@@ -251,6 +251,23 @@ def test_argminmax_iota_concat(both):
     assert_same(both.concat(parts))
 
 
+def test_extremum_values_with_indices(gpu):
+    """One pass yields the arg-extremum and the extremal value: the same indices
+    as argminmax_last, and the value found there."""
+    for dt in ALL:
+        for shape, perm in [((6, 5, 4), None), ((3, 700), None), ((2, 9000), None), ((40, 30, 8), [1, 0, 2]), ((5, 7), [1, 0])]:
+            x = rnd(shape, dt)
+            a = gpu.upload(x)
+            if perm:
+                a, x = a.transpose(perm), x.transpose(perm)
+            for want_max in (True, False):
+                vals, idx = a.extremum_last(want_max)
+                want_idx = (np.argmax if want_max else np.argmin)(x, axis=-1)
+                assert np.array_equal(idx.numpy(), want_idx)
+                assert np.array_equal(idx.numpy(), a.argminmax_last(want_max).numpy())
+                assert np.array_equal(vals.numpy(), np.take_along_axis(x, want_idx[..., None], axis=-1)[..., 0])
+
+
 def ix_arrays(both, shm, extents, oob=True, view=False):
     out = []
     for e in extents:
