@@ -326,7 +326,7 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   // tile shape: least padded work per unit of efficiency
   int cfg = 0;
   double best = 1e300;
-  for (int c = 0; c < kNumTiles; ++c) {
+  for (int c = 0; c < (a->dtype == HGPU_F32 ? kNumTiles : kFirstF32OnlyTile); ++c) {
     int64_t bm = kTiles[c].wgm * kTiles[c].tm * 16, bn = kTiles[c].wgn * kTiles[c].tn * 16;
     double padded = (double)((p.M + bm - 1) / bm * bm) * (double)((p.N + bn - 1) / bn * bn);
     double cost = padded / kTiles[c].eff;

@@ -540,7 +540,10 @@ constexpr TileCfg kTiles[] = {
     {2, 2, 1, 1, 0.35},  // 32 x 32
     {4, 1, 1, 1, 0.30},  // 64 x 16
     {1, 4, 1, 1, 0.30},  // 16 x 64
+    {2, 2, 8, 4, 1.15},  // 256 x 128, fp32 only (the accumulators of an fp64 tile this size do not fit)
+    {2, 2, 4, 8, 1.15},  // 128 x 256, fp32 only
 };
+constexpr int kFirstF32OnlyTile = 11;
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 struct LaunchArgs {
@@ -617,7 +620,13 @@ void launch(const GemmParams& p, const LaunchArgs& a) {
     case 7: launch_cfg<X, 2, 2, 2, 2>(p, a); break;
     case 8: launch_cfg<X, 2, 2, 1, 1>(p, a); break;
     case 9: launch_cfg<X, 4, 1, 1, 1>(p, a); break;
-    default: launch_cfg<X, 1, 4, 1, 1>(p, a); break;
+    case 10: launch_cfg<X, 1, 4, 1, 1>(p, a); break;
+    case 11:
+      if constexpr (sizeof(typename X::T) == 4) launch_cfg<X, 2, 2, 8, 4>(p, a);
+      break;
+    default:
+      if constexpr (sizeof(typename X::T) == 4) launch_cfg<X, 2, 2, 4, 8>(p, a);
+      break;
   }
 }
 
