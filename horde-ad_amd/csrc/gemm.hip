@@ -362,6 +362,9 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     if (cap < 1) cap = 1;
     if (split > cap) split = (int)cap;
     if (split < 1) split = 1;
+    // fewer tiles than CUs: two K halves per tile keep every CU busy, and the
+    // second pass over the output costs less than the idle quarter of the device
+    if (split == 1 && tiles * p.BT * nt < ctx->num_cu && p.K >= 16 * BK) split = 2;
   }
   p.kchunk = ((p.K + split - 1) / split + BK - 1) / BK * BK;
   p.term_split = (int)((p.K + p.kchunk - 1) / p.kchunk);
