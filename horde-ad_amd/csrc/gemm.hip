@@ -316,6 +316,7 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   static_assert(kMaxTerms == 32, "hgpu_contract_sum groups 32 terms to a launch");
   if (n_terms > kMaxTerms) return HGPU_OK;
   p.n_terms = n_terms;
+  p.term_loop = 0;
   for (int t = 0; t < n_terms; ++t) { p.a_term[t] = data_ptr(as[t]); p.b_term[t] = data_ptr(bs[t]); }
   if (n_terms == 0) {   // windows into small footprints: operands from LDS
     int rc = try_footprint(ctx, p, a->dtype, pa, pb, out, handled);
@@ -369,6 +370,11 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   p.kchunk = ((p.K + split - 1) / split + BK - 1) / BK * BK;
   p.term_split = (int)((p.K + p.kchunk - 1) / p.kchunk);
   p.split = (int)(p.term_split * nt);                // K chunks of all terms
+  // terms that are one chunk each, under tiles that fill the device by
+  // themselves: every block adds the terms up in its registers, no partials
+  p.term_loop = (nt > 1 && p.term_split == 1 && tiles * p.BT >= ctx->num_cu / 2 &&
+                 term_loop_tile(kTiles[cfg].wgm, kTiles[cfg].wgn, kTiles[cfg].tm, kTiles[cfg].tn)) ? 1 : 0;
+  if (p.term_loop) p.split = 1;
   split = p.split;
   if (split > 65535) return HGPU_OK;
 
@@ -414,7 +420,9 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     const char* label = a->dtype == HGPU_F64 ? "gemm_f64" : "gemm_f32";
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[128];
-      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,%s%s,t%lldx%lld]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, split, akc ? (va ? "K" : "k") : (va ? "M" : "m"), bkc ? (vb ? "K" : "k") : (vb ? "N" : "n"), (long long)BM, (long long)BN);
+      char terms[24] = "";
+      if (nt > 1) snprintf(terms, sizeof terms, ",terms%lld%s", (long long)nt, p.term_loop ? "loop" : "");
+      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,%s%s,t%lldx%lld%s]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, split, akc ? (va ? "K" : "k") : (va ? "M" : "m"), bkc ? (vb ? "K" : "k") : (vb ? "N" : "n"), (long long)BM, (long long)BN, terms);
       label = ctx->label_pool.insert(buf).first->c_str();
     }
     // the helper launches are timed under their own names, the label times the MFMA kernel alone

@@ -43,6 +43,7 @@ struct GemmParams {
   // within the term, and term t reads a_term[t] / b_term[t].  n_terms == 0: one
   // product, the operands are the kernel's pointer arguments.
   int n_terms, term_split;
+  int term_loop;           // staged kernel: every block walks all terms itself (k_gemm_terms)
   const void* a_term[kMaxTerms];
   const void* b_term[kMaxTerms];
   int c_rows_contig;       // staged kernel: the output is contiguous along m (and not along n)
@@ -355,6 +356,123 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
   }
 }
 
+// The staged kernel for a SUM of products of one layout whose tiles fill the
+// device by themselves: every block walks all terms (GemmParams::a_term /
+// b_term) and adds them up in its accumulators, so there are no partial
+// outputs.  blockIdx.y counts K chunks only.
+template <typename X, int WGM, int WGN, int TM, int TN, int VA, int VB, int NBUF>
+__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_wanted(TM, TN, (int)sizeof(typename X::T)), 8))) k_gemm_terms(GemmParams p, const typename X::T* __restrict__ A, const typename X::T* __restrict__ B,
+                                             typename X::T* __restrict__ C, const int64_t* __restrict__ koffA,
+                                             const int64_t* __restrict__ koffB) {
+  using T = typename X::T;
+  using Acc = typename X::Acc;
+  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
+  constexpr int TNB = TN * 16 / X::NBW;     // MFMA blocks per wavefront along n
+  static_assert(WGM * WGN == 4, "four wavefronts");
+  __shared__ T As[NBUF][BK][BM + 1];
+  __shared__ T Bs[NBUF][BK][BN + 1];
+
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  // XCD-aware tile numbering: blocks b, b+8, b+16, ... share an XCD; give each
+  // XCD a contiguous range of tiles.
+  const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int64_t ntiles = tiles_m * tiles_n;
+  int64_t bid = blockIdx.x;
+  if (ntiles >= 64 && (ntiles & 7) == 0) bid = (bid & 7) * (ntiles >> 3) + (bid >> 3);
+  const int64_t tile_m = bid / tiles_n, tile_n = bid - tile_m * tiles_n;
+  const int64_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+  int64_t bta, btb, btc;
+  group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
+  const int s = blockIdx.y;
+  int sk = s;                              // chunk within its term
+  const int term0 = 0, nterm = p.n_terms;
+  const int64_t kbeg = (int64_t)sk * p.kchunk;
+  int64_t kend = kbeg + p.kchunk;
+  if (kend > p.K) kend = p.K;
+
+  Acc acc[TM][TNB];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TNB; ++j) acc[i][j] = X::zero();
+
+  const KOff koa{p.kmask ? koffA : nullptr, p.ksa}, kob{p.kmask ? koffB : nullptr, p.ksb};
+  for (int term = term0; term < term0 + nterm; ++term) {
+    A = (const T*)p.a_term[term];
+    B = (const T*)p.b_term[term];
+    Stager<T, BM, VA> sa;
+    Stager<T, BN, VB> sb;
+    sa.init(t, p.a_kc, 0, A + bta, p.m, m0, p.M, koa, kbeg, p.K);
+    sb.init(t, p.b_kc, 1, B + btb, p.n, n0, p.N, kob, kbeg, p.K);
+    if (kbeg < kend) {
+      sa.load(kbeg, kend, koa, p.K);
+      sb.load(kbeg, kend, kob, p.K);
+      sa.store(As[0]);
+      sb.store(Bs[0]);
+    }
+    __syncthreads();
+    int cur = 0;
+    for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
+      const bool more = k0 + BK < kend;
+      if (more) {
+        sa.load(k0 + BK, kend, koa, p.K);
+        sb.load(k0 + BK, kend, kob, p.K);
+      }
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 4) {
+        const int kr = kk + (lane >> 4);
+        T fa[TM], fb[TNB];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = As[cur][kr][(wm * TM + i) * 16 + (lane & 15)];
+#pragma unroll
+        for (int j = 0; j < TNB; ++j) fb[j] = Bs[cur][kr][wn * TN * 16 + j * X::NBW + X::bcol(lane)];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TNB; ++j) acc[i][j] = X::run(fa[i], fb[j], acc[i][j]);
+      }
+      if constexpr (NBUF == 1) __syncthreads();   // every wavefront is done reading the tile
+      const int nxt = NBUF == 2 ? cur ^ 1 : 0;
+      if (more) {
+        sa.store(As[nxt]);
+        sb.store(Bs[nxt]);
+      }
+      __syncthreads();
+      cur = nxt;
+    }
+  }
+
+  T* Cout = C + btc + (int64_t)s * p.c_split_stride;
+  int64_t coln[TNB];
+  bool colok[TNB];
+#pragma unroll
+  for (int j = 0; j < TNB; ++j) {
+    int64_t n = n0 + wn * TN * 16 + j * X::NBW + X::col(lane);
+    colok[j] = n < p.N;
+    int64_t oa = 0, ob = 0, oc = 0;
+    if (colok[j]) group_off(p.n, n, &oa, &ob, &oc);
+    coln[j] = oc;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int r = 0; r < X::NR; ++r) {
+      int64_t m = m0 + (wm * TM + i) * 16 + X::row(lane, r);
+      if (m < p.M) {
+        int64_t oa, ob, oc;
+        group_off(p.m, m, &oa, &ob, &oc);
+#pragma unroll
+        for (int j = 0; j < TNB; ++j)
+          if (colok[j]) Cout[oc + coln[j]] = X::get(acc[i][j], r);
+      }
+    }
+  }
+}
+
 // Skinny products (N <= 32): one wavefront owns a (16 TM) x (16 TN) block of the
 // output over one K chunk and loads its MFMA operand fragments straight from
 // global memory.  With so few columns no operand element is shared between
@@ -557,6 +675,10 @@ struct LaunchArgs {
   const int64_t *ka, *kb;
 };
 
+// Blocks that walk the terms of a sum themselves exist for tiles up to 64 x 64
+// (small products whose tiles fill the device).
+constexpr bool term_loop_tile(int wgm, int wgn, int tm, int tn) { return wgm * tm * 16 * wgn * tn * 16 <= 64 * 64; }
+
 template <typename X, int WGM, int WGN, int TM, int TN>
 void launch_cfg(const GemmParams& p, const LaunchArgs& a) {
   using T = typename X::T;
@@ -565,6 +687,26 @@ void launch_cfg(const GemmParams& p, const LaunchArgs& a) {
   // two LDS buffers where they still leave room for two blocks per CU next to
   // the accumulators' registers; skinny tiles keep one buffer and more blocks
   constexpr int NBUF = (BM >= 64 && BN >= 64 && BM + BN >= 192) ? 2 : 1;
+  if constexpr (term_loop_tile(WGM, WGN, TM, TN)) {
+    if (p.term_loop) {
+      const T* A = (const T*)a.A;
+      const T* B = (const T*)a.B;
+      T* C = (T*)a.C;
+      constexpr bool CA = BM >= 64, CB = BN >= 64;
+      const bool va = CA && a.va, vb = CB && a.vb;
+      if constexpr (CA && CB) {
+        if (va && vb) { hipLaunchKernelGGL((k_gemm_terms<X, WGM, WGN, TM, TN, V, V, 1>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+      }
+      if constexpr (CA) {
+        if (va) { hipLaunchKernelGGL((k_gemm_terms<X, WGM, WGN, TM, TN, V, 1, 1>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+      }
+      if constexpr (CB) {
+        if (vb) { hipLaunchKernelGGL((k_gemm_terms<X, WGM, WGN, TM, TN, 1, V, 1>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+      }
+      hipLaunchKernelGGL((k_gemm_terms<X, WGM, WGN, TM, TN, 1, 1, 1>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+      return;
+    }
+  }
   const T* A = (const T*)a.A;
   const T* B = (const T*)a.B;
   T* C = (T*)a.C;

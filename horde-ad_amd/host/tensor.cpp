@@ -497,6 +497,10 @@ T ewise1(int op, const T& a) {
   return make_expr(HGPU_FUSED_OP1, op, a.dtype(), a, nullptr, nullptr);
 }
 T ewise2(int op, const T& a, const T& b) {
+  // W x + V s, both products still pending and of one shape: a pending sum of contractions
+  if (op == HGPU_ADD && a.contraction_like() && b.contraction_like() && a.be() == b.be() && a.be()->fuse && a.holder()->keep == b.holder()->keep &&
+      a.dtype() == b.dtype() && T(a.holder()->fa).shape() == T(b.holder()->fa).shape())
+    return add_cotangents(a, b);
   if (!fuses(a.be()) || !agree(a, b) || !op2_ok(op, a.dtype()) || a.size() == 0) return ewise2_now(op, a, b);
   return make_expr(HGPU_FUSED_OP2, op, a.dtype(), a, &b, nullptr);
 }
