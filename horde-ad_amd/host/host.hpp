@@ -69,6 +69,16 @@ struct ArrHolder {
   // adding two of them piece by piece adds only where both have data -- the
   // stacked state of an unrolled recurrence and its cotangent are then never
   // copied, cleared or added as a whole.
+  // A pending expression over a REFINED index space (h == nullptr, mv_inner
+  // set): mv_inner has the shape of this value with some dims split in two or
+  // more (mv_groups[d] adjacent dims of it make dim d of mv_shape).  Written out
+  // densely, the inner array IS this value (merging dims of a dense array is
+  // free), so elementwise consumers are evaluated over the refined space and
+  // `out[2 i + p, 2 j + q] = src[i, j, p, q]` -- the adjoint of taking pooling
+  // windows -- costs no pass of its own.
+  std::shared_ptr<ArrHolder> mv_inner;
+  Shape mv_shape;
+  std::vector<int> mv_groups;
   struct Piece { int64_t len; std::shared_ptr<ArrHolder> v; };
   std::vector<Piece> pieces;
   Shape pshape;
@@ -104,6 +114,7 @@ class T {
   bool pending_expr() const { return p_ && !p_->h && p_->ekind >= 0; }
   bool pending_product() const { return pending_expr() && p_->ekind == HGPU_FUSED_OP2 && p_->eop == HGPU_MUL; }
   bool pending_pieces() const { return p_ && !p_->h && !p_->pieces.empty(); }
+  bool pending_merged() const { return p_ && !p_->h && p_->mv_inner; }
   bool contraction_like() const { return p_ && !p_->h && p_->ekind < 0 && p_->fa && p_->keep >= 0; }
   bool pending_contraction() const { return contraction_like() && p_->more.empty(); }   // a single one: open to rewrites
   int pending_keep() const { return p_->keep; }
@@ -117,11 +128,13 @@ class T {
   }
   int rank() const {
     if (pending_pieces()) return (int)p_->pshape.size();
+    if (pending_merged()) return (int)p_->mv_shape.size();
     if (pending_expr()) return (int)p_->eshape.size();
     return contraction_like() ? p_->keep : be()->api->rank(meta_h());
   }
   int dtype() const {
     if (pending_pieces()) return p_->pdtype;
+    if (pending_merged()) return T(p_->mv_inner).dtype();
     return pending_expr() ? p_->edtype : T(p_->fa ? p_->fa : p_).dtype_of_holder();
   }
   int dtype_of_holder() const { return p_->h ? be()->api->dtype_of(p_->h) : dtype(); }

@@ -16,6 +16,7 @@ void Backend::check(int rc) const {
 
 Shape T::shape() const {
   if (pending_pieces()) return p_->pshape;
+  if (pending_merged()) return p_->mv_shape;
   if (pending_expr()) return p_->eshape;
   if (contraction_like()) {   // the kept dims of the first factor
     Shape f = T(p_->fa).shape();
@@ -113,6 +114,9 @@ T iota(Backend* be, int64_t n, int dtype) {
 
 static T contract_now(const T& a, const T* b, int n_keep);
 static void pieces_of(const T& t, std::vector<ArrHolder::Piece>* out);
+static T make_merged(const T& inner, const Shape& shape, const std::vector<int>& groups);
+static T split_view(const T& y, const Shape& fine);
+static T lift_merged(const std::vector<const T*>& ops, const std::function<T(const std::vector<T>&)>& apply);
 static T from_pieces(Backend* be, std::vector<ArrHolder::Piece> pcs, const Shape& shape, int dtype);
 static T slice_pieces(const T& a, int64_t start, int64_t len);
 static T ewise1_now(int op, const T& a);
@@ -277,6 +281,14 @@ void force_many(const std::vector<T>& ts) {
 
 void ArrHolder::force() {
   if (h) return;
+  if (mv_inner) {   // the refined expression written out densely, its dims merged (a view)
+    T in(mv_inner);
+    hgpu_array* o = nullptr;
+    be->check(be->api->reshape(be->ctx, in.h(), (int)mv_shape.size(), ptr_or_dummy(mv_shape), &o));
+    h = o;
+    mv_inner.reset();
+    return;
+  }
   if (!pieces.empty()) {   // write the concatenation out: one allocation, one copy (or fill) per piece
     std::vector<T> parts;
     for (auto& pc : pieces) {
@@ -421,7 +433,86 @@ static T map_leaves(const T& a, const std::function<T(const T&)>& view) {
 #define HD_VIEW_OF_EXPR(call) \
   if (a.pending_expr()) return map_leaves(a, [&](const T& x) { return call; });
 
+// ---- pending expressions over a refined index space (ArrHolder::mv_inner) ----
+
+// fine splits dims of coarse: groups[d] adjacent dims of fine multiply to coarse[d].
+static bool refines(const Shape& fine, const Shape& coarse, std::vector<int>* groups) {
+  groups->clear();
+  size_t f = 0;
+  for (size_t d = 0; d < coarse.size(); ++d) {
+    int64_t n = 1;
+    int cnt = 0;
+    if (coarse[d] == 1 && (f >= fine.size() || fine[f] != 1)) { groups->push_back(0); continue; }
+    while (f < fine.size() && (cnt == 0 || n < coarse[d])) { n *= fine[f++]; ++cnt; }
+    if (n != coarse[d]) return false;
+    groups->push_back(cnt);
+  }
+  return f == fine.size();
+}
+
+static T make_merged(const T& inner, const Shape& shape, const std::vector<int>& groups) {
+  if (!inner.pending_expr()) return reshape(inner, shape);   // already an array: merge its dims now
+  auto p = std::make_shared<ArrHolder>(inner.be(), nullptr);
+  p->mv_inner = inner.holder();
+  p->mv_shape = shape;
+  p->mv_groups = groups;
+  return T(p);
+}
+
+// y, whose shape `fine` refines, seen over the refined space (a view for arrays
+// and for the leaves of a pending expression: splitting a dim never copies).
+static T split_view(const T& y, const Shape& fine) {
+  if (y.pending_merged()) {
+    T in(y.holder()->mv_inner);
+    if (in.shape() == fine) return in;
+    return reshape(y, fine);     // writes y out first
+  }
+  if (y.shape() == fine) return y;
+  if (y.pending_expr()) return map_leaves(y, [&](const T& x) { return reshape(x, fine); });
+  return reshape(y, fine);
+}
+
+// An elementwise operation with a refined operand is applied over the refined
+// space; the result is again a refined expression of the same logical shape.
+static T lift_merged(const std::vector<const T*>& ops, const std::function<T(const std::vector<T>&)>& apply) {
+  const T* m = nullptr;
+  for (const T* o : ops)
+    if (o->pending_merged()) { m = o; break; }
+  const Shape fine = T(m->holder()->mv_inner).shape();
+  std::vector<T> split;
+  for (const T* o : ops) split.push_back(split_view(*o, fine));
+  return make_merged(apply(split), m->holder()->mv_shape, m->holder()->mv_groups);
+}
+static bool any_merged_same_shape(const std::vector<const T*>& ops) {
+  bool any = false;
+  for (const T* o : ops) any = any || o->pending_merged();
+  if (!any) return false;
+  for (const T* o : ops)
+    if (o->shape() != ops[0]->shape()) return false;
+  return true;
+}
+
 T transpose(const T& a, const std::vector<int>& perm) {
+  // A refined expression that others hold too (a cotangent fanning out to several
+  // consumers) is written out once, below, and viewed; one of our own is permuted
+  // group by group and stays pending.
+  if (a.pending_merged() && a.holder().use_count() <= 1) {
+    const ArrHolder* h = a.holder().get();
+    const int rank = (int)h->mv_shape.size();
+    std::vector<int> full(perm);
+    for (int d = (int)perm.size(); d < rank; ++d) full.push_back(d);
+    std::vector<int> first((size_t)rank, 0);
+    for (int d = 1; d < rank; ++d) first[(size_t)d] = first[(size_t)d - 1] + h->mv_groups[(size_t)d - 1];
+    std::vector<int> fine_perm, groups;
+    Shape shape;
+    for (int d : full) {
+      if (d < 0 || d >= rank) throw HostError(HGPU_ERR_INVALID, "transpose: bad permutation");
+      for (int k = 0; k < h->mv_groups[(size_t)d]; ++k) fine_perm.push_back(first[(size_t)d] + k);
+      groups.push_back(h->mv_groups[(size_t)d]);
+      shape.push_back(h->mv_shape[(size_t)d]);
+    }
+    return make_merged(transpose(T(h->mv_inner), fine_perm), shape, groups);
+  }
   HD_VIEW_OF_EXPR(transpose(x, perm))
   if (a.pending_contraction() && (int)perm.size() <= a.pending_keep())   // permutes kept dims only
   {
@@ -433,7 +524,13 @@ T transpose(const T& a, const std::vector<int>& perm) {
   static const int dummy = 0;
   HD_OUT(transpose(be__->ctx, a.h(), (int)perm.size(), perm.empty() ? &dummy : perm.data(), &o__));
 }
-T reshape(const T& a, const Shape& s) { HD_OUT(reshape(be__->ctx, a.h(), (int)s.size(), ptr_or_dummy(s), &o__)); }
+T reshape(const T& a, const Shape& s) {
+  if (a.pending_expr() && s != a.shape()) {   // only splits dims: a view of every leaf
+    std::vector<int> g;
+    if (refines(s, a.shape(), &g)) return map_leaves(a, [&](const T& x) { return reshape(x, s); });
+  }
+  HD_OUT(reshape(be__->ctx, a.h(), (int)s.size(), ptr_or_dummy(s), &o__));
+}
 T slice(const T& a, int dim, int64_t start, int64_t len) {
   if (dim == 0 && a.pending_pieces() && start >= 0 && len >= 0 && start + len <= a.shape().at(0)) return slice_pieces(a, start, len);
   HD_VIEW_OF_EXPR(slice(x, dim, start, len))
@@ -493,10 +590,12 @@ static bool op2_ok(int op, int dt) {
   return (op == HGPU_AND) == (dt == HGPU_BOOL);
 }
 T ewise1(int op, const T& a) {
+  if (a.pending_merged()) return lift_merged({&a}, [&](const std::vector<T>& v) { return ewise1(op, v[0]); });
   if (!fuses(a.be()) || !op1_ok(op, a.dtype()) || a.size() == 0) return ewise1_now(op, a);
   return make_expr(HGPU_FUSED_OP1, op, a.dtype(), a, nullptr, nullptr);
 }
 T ewise2(int op, const T& a, const T& b) {
+  if (any_merged_same_shape({&a, &b})) return lift_merged({&a, &b}, [&](const std::vector<T>& v) { return ewise2(op, v[0], v[1]); });
   // W x + V s, both products still pending and of one shape: a pending sum of contractions
   if (op == HGPU_ADD && a.contraction_like() && b.contraction_like() && a.be() == b.be() && a.be()->fuse && a.holder()->keep == b.holder()->keep &&
       a.dtype() == b.dtype() && T(a.holder()->fa).shape() == T(b.holder()->fa).shape())
@@ -505,6 +604,7 @@ T ewise2(int op, const T& a, const T& b) {
   return make_expr(HGPU_FUSED_OP2, op, a.dtype(), a, &b, nullptr);
 }
 T compare(int cmp, const T& a, const T& b) {
+  if (any_merged_same_shape({&a, &b})) return lift_merged({&a, &b}, [&](const std::vector<T>& v) { return compare(cmp, v[0], v[1]); });
   if (!fuses(a.be()) || !agree(a, b) || cmp < HGPU_LEQ || cmp > HGPU_LT || a.size() == 0) return compare_now(cmp, a, b);
   return make_expr(HGPU_FUSED_CMP, cmp, HGPU_BOOL, a, &b, nullptr);
 }
@@ -516,11 +616,13 @@ bool compare_all(int cmp, const T& a, const T& b) {
 static T select_now(const T& c, const T& a, const T& b) { HD_OUT(select(be__->ctx, c.h(), a.h(), b.h(), &o__)); }
 static T convert_now(const T& a, int dtype, int mode) { HD_OUT(convert(be__->ctx, a.h(), dtype, mode, &o__)); }
 T select(const T& c, const T& a, const T& b) {
+  if (any_merged_same_shape({&c, &a, &b})) return lift_merged({&c, &a, &b}, [&](const std::vector<T>& v) { return select(v[0], v[1], v[2]); });
   if (!fuses(a.be()) || !agree(a, b) || c.dtype() != HGPU_BOOL || c.shape() != a.shape() || a.size() == 0) return select_now(c, a, b);
   return make_expr(HGPU_FUSED_SELECT, 0, a.dtype(), c, &a, &b);
 }
 T convert(const T& a, int dtype, int mode) {
   if (a.dtype() == dtype && mode == HGPU_CONV_CAST) return a;
+  if (a.pending_merged()) return lift_merged({&a}, [&](const std::vector<T>& v) { return convert(v[0], dtype, mode); });
   bool ok = dtype >= HGPU_F64 && dtype <= HGPU_BOOL && (mode == HGPU_CONV_CAST || (mode == HGPU_CONV_FLOOR && is_fp_dt(a.dtype()) && is_int_dt(dtype)));
   if (!fuses(a.be()) || !ok || a.size() == 0) return convert_now(a, dtype, mode);
   return make_expr(HGPU_FUSED_CONVERT, mode, dtype, a, nullptr, nullptr);
@@ -1157,6 +1259,40 @@ T tsscatter(const T& src, int rank_m, const Shape& shp, const std::vector<Ix>& i
   if (!injective && all_affine(ix) && src.size() > 0) {
     T r = scatter_as_contraction(src, rank_m, shp, ix);
     if (r.valid()) return r;
+  }
+  // Every destination index is a mixed-radix number whose digits are position
+  // variables (out[2 i + p, 2 j + q] = src[i, j, p, q], the adjoint of taking
+  // pooling windows) and all of the destination is written exactly once: the
+  // scatter is a transposition followed by a merge of the digits.  Of a
+  // pending expression that costs nothing: it stays pending over the refined
+  // space and is written out, dims merged, by whoever consumes it.
+  if (injective && all_affine(ix) && src.size() > 0 && src.pending_expr()) {
+    std::vector<int> perm, groups;
+    std::vector<bool> used((size_t)rank_m, false);
+    bool ok = true;
+    for (size_t j = 0; j < ix.size() && ok; ++j) {
+      std::vector<std::pair<int64_t, int>> digits;   // (coefficient, position dim)
+      for (int d = 0; d < rank_m; ++d)
+        if (ix[j].coef[(size_t)d] != 0) digits.push_back({ix[j].coef[(size_t)d], d});
+      std::sort(digits.begin(), digits.end(), [](const std::pair<int64_t, int>& x, const std::pair<int64_t, int>& y) { return x.first > y.first; });
+      ok = ix[j].c0 == 0 && !digits.empty() && digits.back().first == 1;
+      for (size_t k = 0; k < digits.size() && ok; ++k) {
+        int d = digits[k].second;
+        ok = !used[(size_t)d];
+        used[(size_t)d] = true;
+        int64_t above = k == 0 ? shp[j] : digits[k - 1].first;      // the next digit up counts in units of this one's range
+        ok = ok && digits[k].first * shm[(size_t)d] == above && shm[(size_t)d] > 1;
+        perm.push_back(d);
+      }
+      groups.push_back((int)digits.size());
+    }
+    for (int d = 0; d < rank_m && ok; ++d) ok = used[(size_t)d];
+    if (ok) {
+      for (int d = rank_m; d < (int)ssh.size(); ++d) { perm.push_back(d); groups.push_back(1); }
+      Shape osh(shp);
+      osh.insert(osh.end(), ssh.begin() + rank_m, ssh.end());
+      return make_merged(transpose(src, perm), osh, groups);
+    }
   }
   if (injective && all_affine(ix) && src.size() > 0 &&
       be->api->struct_size >= offsetof(hgpu_api, scatter_affine) + sizeof(be->api->scatter_affine) && be->api->scatter_affine) {

@@ -238,3 +238,28 @@ def test_append_slice_pieces_cpu(host_cpu):
 @pytest.mark.gpu
 def test_append_slice_pieces_gpu(host_gpu):
     check_append_slice(host_gpu)
+
+
+@pytest.mark.gpu
+def test_pooling_adjoint_stays_pending_gpu(host_gpu, host_cpu):
+    """relu -> 2x2 max pooling -> a cotangent that fans out: on the device the
+    adjoint of taking the windows (out[2i+p, 2j+q] = src[i, j, p, q]) is no pass
+    of its own, the expression stays pending over the refined index space and is
+    written out once; the checker scatters literally.  Shapes with odd channel
+    counts and a second use of the pooled cotangent."""
+    W = pkg.workloads
+    x = RNG.uniform(-1, 1, (5, 3, 8, 12))
+    b = RNG.uniform(-0.5, 0.5, (3,))
+    w = RNG.uniform(-1, 1, (5, 3, 4, 6))
+    res = []
+    for host in (host_gpu, host_cpu):
+        px, pb = host.param(x), host.param(b)
+        y = px + pb.sreplicateN([5, 8, 12]).stranspose([0, 3, 1, 2])
+        r = W.reluS(y)
+        pooled = W.maxPool2dUnpaddedS(r)                          # [5, 3, 4, 6]
+        loss = (pooled * host.concrete(w)).ssum0() + (pooled * pooled).ssum0() + (r.stranspose([1, 0, 2, 3]) * r.stranspose([1, 0, 2, 3])).ssum0()
+        gx, gb = host.grad(loss, [px, pb])
+        res.append((loss.numpy(), gx.numpy(), gb.numpy()))
+        host.tape_reset()
+    for got, want in zip(res[0], res[1]):
+        assert np.allclose(got, want, rtol=1e-12, atol=1e-13)
