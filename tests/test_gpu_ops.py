@@ -499,6 +499,7 @@ def conv_views(both, dt, b, ci, h, w, co, kh, kw):
     (600, 2, 16, 16, 4, 3, 3),      # four output channels
     (128, 32, 8, 8, 16, 3, 3),      # 18 row blocks in the kernel gradient: dealt and split
     (150, 7, 10, 10, 16, 3, 3),     # 63 rows
+    (130, 1, 28, 28, 16, 5, 5),     # the CNN's first layer: the kernel gradient's footprints fit LDS once, not twice
 ])
 def test_conv_contractions_from_lds_footprints(both, gpu, dt, shape):
     """Forward convolution, kernel gradient and input gradient as contractions
