@@ -55,6 +55,7 @@ SIGNATURES = {
 # exported by the GPU library only
 GPU_ONLY = {
     "extremum_last": (I, [P, P, I, PP, PP]),
+    "fused_extremum": (I, [P, I, PP, I, P, I, I, I, PP, PP]),
     "mem_stats": (I, [P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "stream": (P, [P]), "inject_alloc_failure": (I, [P, L]),
     "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
@@ -139,6 +140,14 @@ class Ctx:
         outs = (C.c_void_p * len(out_slots))()
         self.check(self.lib.fused_map(self.h, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs))
         return [Array(self, C.c_void_p(o)) for o in outs]
+
+    def fused_extremum(self, inputs, prog, slot, n_reduce, want_max):
+        """(values, indices) of the first extremum of slot's values over the trailing n_reduce dims."""
+        ins = (C.c_void_p * len(inputs))(*[p.h for p in inputs])
+        flat = (C.c_int32 * max(6 * len(prog), 1))(*[int(x) for q in prog for x in q])
+        v, i = C.c_void_p(), C.c_void_p()
+        self.check(self.lib.fused_extremum(self.h, len(inputs), ins, len(prog), flat, slot, n_reduce, int(want_max), C.byref(v), C.byref(i)))
+        return Array(self, v), Array(self, i)
 
     def _wrap(self, h):
         return Array(self, h)

@@ -126,7 +126,7 @@ std::map<std::string, Compiled>& cache_of(hgpu_ctx* ctx) {
   return *static_cast<std::map<std::string, Compiled>*>(it->second);
 }
 
-int compile(hgpu_ctx* ctx, const std::string& src, Compiled* out) {
+int compile(hgpu_ctx* ctx, const std::string& src, Compiled* out, const char* kname = "fused_map") {
   hiprtcProgram prog;
   if (hiprtcCreateProgram(&prog, src.c_str(), "fused_map.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
     return fail(ctx, HGPU_ERR_DEVICE, "hiprtcCreateProgram failed");
@@ -150,7 +150,7 @@ int compile(hgpu_ctx* ctx, const std::string& src, Compiled* out) {
   hiprtcDestroyProgram(&prog);
   hipError_t e = hipModuleLoadData(&out->mod, code.data());
   if (e != hipSuccess) return check_hip(ctx, e, "hipModuleLoadData");
-  e = hipModuleGetFunction(&out->fn, out->mod, "fused_map");
+  e = hipModuleGetFunction(&out->fn, out->mod, kname);
   if (e != hipSuccess) return check_hip(ctx, e, "hipModuleGetFunction");
   return HGPU_OK;
 }
@@ -163,20 +163,10 @@ struct FDims {
   int64_t st[kMaxIn][HG_KDIMS];
 };
 
-}  // namespace
-
-extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
-                              int n_out, const int* out_slots, hgpu_array** outs) {
-  if (!ctx || !in || !prog || !out_slots || !outs) return HGPU_ERR_INVALID;
-  if (n_in < 1 || n_in > kMaxIn || n_out < 1 || n_out > kMaxOut || n_instr < 1 || n_instr > kMaxInstr)
-    return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map: %d inputs, %d instructions, %d outputs", n_in, n_instr, n_out);
-  const hgpu_array* a0 = in[0];
-  for (int i = 0; i < n_in; ++i) {
-    if (!in[i]) return HGPU_ERR_INVALID;
-    if (!same_shape(in[i], a0)) return fail(ctx, HGPU_ERR_INVALID, "fused_map: input %d has another shape", i);
-  }
-  // slot types, with the same checks the eager entry points make
-  std::vector<int> dt((size_t)(n_in + n_instr));
+// Slot types of a program, with the same checks the eager entry points make.
+int check_program(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, std::vector<int>* dtp) {
+  std::vector<int>& dt = *dtp;
+  dt.assign((size_t)(n_in + n_instr), 0);
   for (int i = 0; i < n_in; ++i) dt[(size_t)i] = in[i]->dtype;
   for (int k = 0; k < n_instr; ++k) {
     const hgpu_fused_instr& q = prog[k];
@@ -213,6 +203,41 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
         return fail(ctx, HGPU_ERR_INVALID, "fused_map: unknown instruction kind %d", q.kind);
     }
   }
+  return HGPU_OK;
+}
+
+// One instruction per line: `const T v<slot><suffix> = ...;`
+void emit_program(std::ostringstream& s, int n_in, int n_instr, const hgpu_fused_instr* prog, const std::vector<int>& dt, const char* ind, const std::string& lane_suffix) {
+  for (int k = 0; k < n_instr; ++k) {
+    const hgpu_fused_instr& q = prog[k];
+    int self = n_in + k;
+    auto v = [&](int slot) { return "v" + std::to_string(slot) + lane_suffix; };
+    s << ind << "const " << ctype(dt[(size_t)self]) << " " << v(self) << " = ";
+    switch (q.kind) {
+      case HGPU_FUSED_OP1: s << "op1<" << q.op << ">(" << v(q.a) << ")"; break;
+      case HGPU_FUSED_OP2: s << "op2<" << q.op << ">(" << v(q.a) << ", " << v(q.b) << ")"; break;
+      case HGPU_FUSED_CMP: s << "cmp2<" << q.op << ">(" << v(q.a) << ", " << v(q.b) << ")"; break;
+      case HGPU_FUSED_SELECT: s << "(" << v(q.a) << " ? " << v(q.b) << " : " << v(q.c) << ")"; break;
+      default: s << "conv<" << q.op << ", " << ctype(q.dtype) << ">(" << v(q.a) << ")"; break;
+    }
+    s << ";\n";
+  }
+}
+
+}  // namespace
+
+extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
+                              int n_out, const int* out_slots, hgpu_array** outs) {
+  if (!ctx || !in || !prog || !out_slots || !outs) return HGPU_ERR_INVALID;
+  if (n_in < 1 || n_in > kMaxIn || n_out < 1 || n_out > kMaxOut || n_instr < 1 || n_instr > kMaxInstr)
+    return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map: %d inputs, %d instructions, %d outputs", n_in, n_instr, n_out);
+  const hgpu_array* a0 = in[0];
+  for (int i = 0; i < n_in; ++i) {
+    if (!in[i]) return HGPU_ERR_INVALID;
+    if (!same_shape(in[i], a0)) return fail(ctx, HGPU_ERR_INVALID, "fused_map: input %d has another shape", i);
+  }
+  std::vector<int> dt;
+  if (int rc = check_program(ctx, n_in, in, n_instr, prog, &dt)) return rc;
   for (int o = 0; o < n_out; ++o)
     if (out_slots[o] < 0 || out_slots[o] >= n_in + n_instr) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad output slot");
 
@@ -441,5 +466,153 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   hipError_t e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
   if (e != hipSuccess) { release_all(); return check_hip(ctx, e, "fused_map launch"); }
   for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
+  return HGPU_OK;
+}
+
+// The first extremum of an elementwise program's result along its trailing
+// `n_reduce` dims (taken together, row-major), evaluated on the fly: the
+// program's result is never written.  values / indices have the leading dims'
+// shape; the index counts positions within the reduced dims.
+extern "C" int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot,
+                                   int n_reduce, int want_max, hgpu_array** values, hgpu_array** indices) {
+  if (!ctx || !in || (!prog && n_instr > 0) || !values || !indices) return HGPU_ERR_INVALID;
+  if (n_in < 1 || n_in > kMaxIn || n_instr < 0 || n_instr > kMaxInstr) return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_extremum: %d inputs, %d instructions", n_in, n_instr);
+  const hgpu_array* a0 = in[0];
+  for (int i = 0; i < n_in; ++i) {
+    if (!in[i]) return HGPU_ERR_INVALID;
+    if (!same_shape(in[i], a0)) return fail(ctx, HGPU_ERR_INVALID, "fused_extremum: input %d has another shape", i);
+  }
+  if (n_reduce < 1 || n_reduce > a0->rank) return fail(ctx, HGPU_ERR_INVALID, "fused_extremum: %d reduced dims of rank %d", n_reduce, a0->rank);
+  std::vector<int> dt;
+  if (int rc = check_program(ctx, n_in, in, n_instr, prog, &dt)) return rc;
+  if (slot < 0 || slot >= n_in + n_instr) return fail(ctx, HGPU_ERR_INVALID, "fused_extremum: bad slot");
+  const int rank_o = a0->rank - n_reduce;
+  int64_t L = 1, n_out = 1;
+  for (int d = rank_o; d < a0->rank; ++d) L *= a0->shape[d];
+  for (int d = 0; d < rank_o; ++d) n_out *= a0->shape[d];
+  if (L < 1) return fail(ctx, HGPU_ERR_INVALID, "fused_extremum: empty reduced dims");
+  if (L > 64 || n_out >= (1LL << 31)) return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_extremum: %lld reduced elements per result", (long long)L);
+  hgpu_array *v = nullptr, *ix = nullptr;
+  int rc = new_dense(ctx, dt[(size_t)slot], rank_o, a0->shape, &v);
+  if (rc) return rc;
+  rc = new_dense(ctx, HGPU_I64, rank_o, a0->shape, &ix);
+  if (rc) { hgpu_release(v); return rc; }
+  if (n_out == 0) { *values = v; *indices = ix; return HGPU_OK; }
+
+  std::string layout((size_t)n_in, 'g');
+  for (int i = 0; i < n_in; ++i) {
+    bool all0 = true;
+    for (int d = 0; d < in[i]->rank; ++d)
+      if (in[i]->shape[d] != 1 && in[i]->strides[d] != 0) all0 = false;
+    if (all0) layout[(size_t)i] = 's';
+  }
+  // leading dims merged jointly over all inputs
+  FDims fd;
+  fd.nd = 0;
+  for (int d = 0; d < rank_o; ++d) {
+    if (a0->shape[d] == 1) continue;
+    bool merged = false;
+    if (fd.nd > 0) {
+      int p = fd.nd - 1;
+      bool ok = true;
+      for (int k = 0; k < n_in; ++k)
+        if (fd.st[k][p] != in[k]->strides[d] * a0->shape[d]) { ok = false; break; }
+      if (ok) {
+        fd.shape[p] *= a0->shape[d];
+        for (int k = 0; k < n_in; ++k) fd.st[k][p] = in[k]->strides[d];
+        merged = true;
+      }
+    }
+    if (!merged) {
+      if (fd.nd == HG_KDIMS) { hgpu_release(v); hgpu_release(ix); return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_extremum: more than %d merged dims", HG_KDIMS); }
+      fd.shape[fd.nd] = a0->shape[d];
+      for (int k = 0; k < n_in; ++k) fd.st[k][fd.nd] = in[k]->strides[d];
+      fd.nd++;
+    }
+  }
+  // ---- source: shapes and strides are constants of the kernel
+  std::ostringstream s;
+  s << kPrelude;
+  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_extremum(i64 n";
+  for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
+  s << ", " << ctype(dt[(size_t)slot]) << "* __restrict__ ov, i64* __restrict__ oi) {\n";
+  s << "  const i64 step = (i64)gridDim.x * 256;\n";
+  for (int i = 0; i < n_in; ++i)
+    if (layout[(size_t)i] == 's') s << "  const " << ctype(in[i]->dtype) << " s" << i << " = i" << i << "[0];\n";
+  s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {\n";
+  s << "    unsigned r = (unsigned)i;\n";
+  for (int q = fd.nd - 1; q >= 0; --q) {
+    if (q > 0) s << "    const unsigned c" << q << " = r % " << fd.shape[q] << "u; r /= " << fd.shape[q] << "u;\n";
+    else s << "    const unsigned c0 = r;\n";
+  }
+  for (int i = 0; i < n_in; ++i) {
+    if (layout[(size_t)i] == 's') continue;
+    s << "    const " << ctype(in[i]->dtype) << "* p" << i << " = i" << i;
+    for (int q = 0; q < fd.nd; ++q)
+      if (fd.st[i][q] != 0) s << " + (i64)c" << q << " * " << fd.st[i][q] << "ll";
+    s << ";\n";
+  }
+  s << "    " << ctype(dt[(size_t)slot]) << " best;\n    i64 bi = 0;\n";
+  for (int64_t e = 0; e < L; ++e) {
+    // offsets of reduced position e
+    std::string suf = "_" + std::to_string(e);
+    s << "    {\n";
+    for (int i = 0; i < n_in; ++i) {
+      s << "      const " << ctype(in[i]->dtype) << " v" << i << suf << " = ";
+      if (layout[(size_t)i] == 's') { s << "s" << i << ";\n"; continue; }
+      int64_t off = 0, rr = e;
+      for (int d = a0->rank - 1; d >= rank_o; --d) {
+        off += (rr % a0->shape[d]) * in[i]->strides[d];
+        rr /= a0->shape[d];
+      }
+      s << "p" << i << "[" << off << "ll];\n";
+    }
+    emit_program(s, n_in, n_instr, prog, dt, "      ", suf);
+    if (e == 0) s << "      best = v" << slot << suf << ";\n";
+    else s << "      if (v" << slot << suf << (want_max ? " > " : " < ") << "best) { best = v" << slot << suf << "; bi = " << e << "; }\n";
+    s << "    }\n";
+  }
+  s << "    ov[i] = best;\n    oi[i] = bi;\n  }\n}\n";
+  std::string src = s.str();
+
+  const char* label = "fused_extremum";
+  if (ctx->profiling && ctx->profile_shapes) {
+    std::string sh;
+    for (int d = 0; d < a0->rank; ++d) sh += (d ? "x" : "") + std::to_string(a0->shape[d]);
+    char buf[160];
+    snprintf(buf, sizeof buf, "fused_extremum[%s,reduce%d,in%d(%s),instr%d]", sh.c_str(), n_reduce, n_in, layout.c_str(), n_instr);
+    label = ctx->label_pool.insert(buf).first->c_str();
+  }
+  double bytes = (double)n_out * (dtype_size(dt[(size_t)slot]) + 8);
+  for (int i = 0; i < n_in; ++i) {
+    if (layout[(size_t)i] == 's') continue;
+    int64_t distinct = 1;
+    for (int d = 0; d < in[i]->rank; ++d)
+      if (in[i]->strides[d] != 0) distinct *= in[i]->shape[d];
+    bytes += (double)distinct * dtype_size(in[i]->dtype);
+  }
+  LaunchGuard lg(ctx, label, bytes, (double)n_out * L * (n_instr + 1));
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c;
+    rc = compile(ctx, src, &c, "fused_extremum");
+    if (rc) { hgpu_release(v); hgpu_release(ix); return rc; }
+    it = cache.emplace(src, c).first;
+  }
+  std::vector<void*> args;
+  int64_t nn = n_out;
+  args.push_back(&nn);
+  std::vector<const void*> ptrs((size_t)n_in);
+  for (int i = 0; i < n_in; ++i) { ptrs[(size_t)i] = data_ptr(in[i]); args.push_back(&ptrs[(size_t)i]); }
+  void* pv = data_ptr(v);
+  void* pi = data_ptr(ix);
+  args.push_back(&pv);
+  args.push_back(&pi);
+  unsigned grid = grid_for(n_out, 256, ctx->num_cu * 16);
+  hipError_t e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e != hipSuccess) { hgpu_release(v); hgpu_release(ix); return check_hip(ctx, e, "fused_extremum launch"); }
+  *values = v;
+  *indices = ix;
   return HGPU_OK;
 }

@@ -164,7 +164,7 @@ struct Program {
 // Post-order walk: materialised values (and pending contractions, which are
 // forced here) become inputs, pending elementwise nodes become instructions.
 int visit(Program& pg, ArrHolder* p) {
-  if (!p->h && p->ekind < 0 && p->fa) p->force();   // a pending contraction
+  if (!p->h && p->ekind < 0) p->force();   // a pending contraction, concatenation or refined expression
   if (p->h) {
     auto it = pg.in_slot.find(p);
     if (it != pg.in_slot.end()) return -1 - it->second;
@@ -189,24 +189,31 @@ int visit(Program& pg, ArrHolder* p) {
 }
 }  // namespace
 
-static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
+// The roots' expressions as one numbered program: inputs, instructions, and the slot of every root.
+static void number_program(const std::vector<ArrHolder*>& roots, std::vector<const hgpu_array*>* ins, std::vector<hgpu_fused_instr>* prog,
+                           std::vector<int>* outs_slot) {
   Program pg;
   std::vector<int> root_slot;
   for (auto* r : roots) root_slot.push_back(visit(pg, r));
-  int n_in = (int)pg.inputs.size(), n_instr = (int)pg.instrs.size();
+  int n_in = (int)pg.inputs.size();
   auto slot = [&](int v) { return v < 0 ? -1 - v : n_in + v; };
-  std::vector<hgpu_fused_instr> prog;
   for (auto& pi : pg.instrs) {
     hgpu_fused_instr q = pi.second;
     q.a = slot(q.a);
     q.b = pi.first->fb ? slot(q.b) : 0;
     q.c = pi.first->fc ? slot(q.c) : 0;
-    prog.push_back(q);
+    prog->push_back(q);
   }
+  for (auto* p : pg.inputs) ins->push_back(p->h);
+  for (int v : root_slot) outs_slot->push_back(slot(v));
+}
+
+static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
   std::vector<const hgpu_array*> ins;
-  for (auto* p : pg.inputs) ins.push_back(p->h);
+  std::vector<hgpu_fused_instr> prog;
   std::vector<int> outs_slot;
-  for (int v : root_slot) outs_slot.push_back(slot(v));
+  number_program(roots, &ins, &prog, &outs_slot);
+  int n_in = (int)ins.size(), n_instr = (int)prog.size();
   std::vector<hgpu_array*> outs(roots.size(), nullptr);
   be->check(be->api->fused_map(be->ctx, n_in, ins.data(), n_instr, prog.data(), (int)roots.size(), outs_slot.data(), outs.data()));
   for (size_t i = 0; i < roots.size(); ++i) {
@@ -528,6 +535,8 @@ T reshape(const T& a, const Shape& s) {
   if (a.pending_expr() && s != a.shape()) {   // only splits dims: a view of every leaf
     std::vector<int> g;
     if (refines(s, a.shape(), &g)) return map_leaves(a, [&](const T& x) { return reshape(x, s); });
+    // only merges dims: the expression stays pending over its own, finer space
+    if (refines(a.shape(), s, &g)) return make_merged(a, s, g);
   }
   HD_OUT(reshape(be__->ctx, a.h(), (int)s.size(), ptr_or_dummy(s), &o__));
 }
@@ -1395,6 +1404,34 @@ Ix ix_argminmax(Backend* be, const T& t, const std::vector<Ix>& ix, bool want_ma
     for (size_t e = 0; e < x.coef.size() && identity; ++e) identity = x.coef[e] == (e == d ? 1 : 0);
   }
   const hgpu_api* api = be->api;
+  // t is a pending expression whose last dim merges trailing dims of its own
+  // space (pooling windows [.., 2, 2] seen as [.., 4]): the extremum is taken
+  // while the expression is evaluated, which is then never written out
+  if (identity && be->fuse && t.pending_merged() && api->struct_size >= offsetof(hgpu_api, fused_extremum) + sizeof(api->fused_extremum) &&
+      api->fused_extremum) {
+    const ArrHolder* mh = t.holder().get();
+    int n_reduce = mh->mv_groups.back();
+    T inner(mh->mv_inner);
+    if (n_reduce >= 1 && inner.pending_expr() && tsh.back() <= 64 && inner.size() / tsh.back() < (int64_t(1) << 31) &&
+        pending_size(inner.holder()) <= 40) {
+      bool leading_whole = true;    // the leading logical dims may be merged too; only their product matters here
+      (void)leading_whole;
+      std::vector<const hgpu_array*> ins;
+      std::vector<hgpu_fused_instr> prog;
+      std::vector<int> slots;
+      number_program({inner.holder().get()}, &ins, &prog, &slots);
+      if ((int)ins.size() <= 12 && (int)prog.size() <= 96) {
+        hgpu_array *vals = nullptr, *idx = nullptr;
+        be->check(api->fused_extremum(be->ctx, (int)ins.size(), ins.data(), (int)prog.size(), prog.data(), slots[0], n_reduce, want_max ? 1 : 0, &vals, &idx));
+        // results have the inner space's leading dims: merge them to the logical ones
+        Shape lead(tsh.begin(), tsh.end() - 1);
+        Ix r = from_array(shm, reshape(T(be, idx), lead));
+        r.arg_of = t.holder();
+        r.arg_vals = reshape(T(be, vals), lead);
+        return r;
+      }
+    }
+  }
   if (identity && be->fuse && api->struct_size >= offsetof(hgpu_api, extremum_last) + sizeof(api->extremum_last) && api->extremum_last) {
     hgpu_array *vals = nullptr, *idx = nullptr;
     be->check(api->extremum_last(be->ctx, t.h(), want_max ? 1 : 0, &vals, &idx));

@@ -218,6 +218,15 @@ enum hgpu_fused_kind { HGPU_FUSED_OP1 = 0, HGPU_FUSED_OP2 = 1, HGPU_FUSED_CMP = 
 typedef struct hgpu_fused_instr { int32_t kind, op, dtype, a, b, c; } hgpu_fused_instr;
 int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
                    int n_out, const int* out_slots, hgpu_array** outs);
+/* The first extremum of such a program's result along its trailing n_reduce
+ * dims (taken together, row-major), evaluated on the fly: the result itself is
+ * never written.  values / indices get the leading dims' shape; an index
+ * counts positions within the reduced dims (at most 64 of them).  With this,
+ * `maxPool2dUnpaddedS (reluS (conv + bias))` (External/CommonShapedOps.hs:
+ * 241-260) reads the convolution once and writes only the pooled maxima and
+ * their arguments. */
+int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot, int n_reduce,
+                        int want_max, hgpu_array** values, hgpu_array** indices);
 
 /* out[o] = sum_r a[o,r] * b[o,r]  (b == NULL: b = 1), o ranging over the first
  * n_keep dims and r over the rest.  With the free views above this one entry
@@ -371,6 +380,7 @@ typedef struct hgpu_api {
   int (*contract_sum)(hgpu_ctx*, int, const hgpu_array* const*, const hgpu_array* const*, int, hgpu_array**);
   int (*assign)(hgpu_ctx*, hgpu_array*, const hgpu_array*);
   int (*extremum_last)(hgpu_ctx*, const hgpu_array*, int, hgpu_array**, hgpu_array**);
+  int (*fused_extremum)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, int, int, hgpu_array**, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

@@ -739,6 +739,7 @@ const hgpu_api* horc_get_api(void) {
       nullptr, nullptr, nullptr, nullptr, nullptr,   // no graphs: the checker executes eagerly
       horc_contract_sum, horc_assign,
       nullptr,   // no extremum_last: the checker gathers at the arg-extremum as the reference does
+      nullptr,   // no fused_extremum
   };
   return &api;
 }

@@ -251,6 +251,30 @@ def test_argminmax_iota_concat(both):
     assert_same(both.concat(parts))
 
 
+@pytest.mark.parametrize("dt", [np.float64, np.float32, np.int32])
+def test_fused_extremum_equals_program_then_extremum(gpu, dt):
+    """The extremum of a program's result over its trailing dims, taken on the
+    fly, against the program written out (fused_map) and reduced (extremum_last)."""
+    O2 = capi.OP2
+    prog = [(1, O2["mul"], 0, 0, 1, 0), (1, O2["add"], 0, 3, 2, 0), (1, O2["max"], 0, 4, 0, 0)]   # max (a * b + c) a
+    for shape, n_reduce in [((6, 5, 2, 2), 2), ((4, 3, 7), 1), ((9, 64), 1), ((3, 2, 2, 2, 2), 3), ((5,), 1)]:
+        a = gpu.upload(rnd(shape, dt))
+        b = gpu.upload(rnd(shape[-1:], dt)).replicate(list(shape[:-1]))                # broadcast view
+        c = gpu.upload(np.ascontiguousarray(np.moveaxis(rnd(shape, dt), -1, 0))).transpose(list(range(1, len(shape))) + [0]) if len(shape) > 1 else gpu.upload(rnd(shape, dt))
+        ins = [a, b, c]
+        for slot in (5, 3, 0):
+            full = gpu.fused_map(ins, prog, [slot])[0] if slot >= 3 else a
+            lead = list(shape[:len(shape) - n_reduce])
+            flat = full.reshape(lead + [int(np.prod(shape[len(shape) - n_reduce:]))])
+            for want_max in (True, False):
+                wv, wi = flat.extremum_last(want_max)
+                gv, gi = gpu.fused_extremum(ins, prog, slot, n_reduce, want_max)
+                assert np.array_equal(gi.numpy(), wi.numpy()), (shape, slot, want_max)
+                assert np.array_equal(gv.numpy(), wv.numpy())
+    with pytest.raises(capi.HgpuError):
+        gpu.fused_extremum([gpu.upload(rnd((3, 100), dt))], [], 0, 1, True)      # more than 64 reduced elements
+
+
 def test_extremum_values_with_indices(gpu):
     """One pass yields the arg-extremum and the extremal value: the same indices
     as argminmax_last, and the value found there."""
