@@ -1414,8 +1414,6 @@ Ix ix_argminmax(Backend* be, const T& t, const std::vector<Ix>& ix, bool want_ma
     T inner(mh->mv_inner);
     if (n_reduce >= 1 && inner.pending_expr() && tsh.back() <= 64 && inner.size() / tsh.back() < (int64_t(1) << 31) &&
         pending_size(inner.holder()) <= 40) {
-      bool leading_whole = true;    // the leading logical dims may be merged too; only their product matters here
-      (void)leading_whole;
       std::vector<const hgpu_array*> ins;
       std::vector<hgpu_fused_instr> prog;
       std::vector<int> slots;
