@@ -56,6 +56,7 @@ SIGNATURES = {
 GPU_ONLY = {
     "extremum_last": (I, [P, P, I, PP, PP]),
     "fused_extremum": (I, [P, I, PP, I, P, I, I, I, PP, PP]),
+    "fused_sum": (I, [P, I, PP, I, P, I, PP]),
     "mem_stats": (I, [P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "stream": (P, [P]), "inject_alloc_failure": (I, [P, L]),
     "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
@@ -140,6 +141,12 @@ class Ctx:
         outs = (C.c_void_p * len(out_slots))()
         self.check(self.lib.fused_map(self.h, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs))
         return [Array(self, C.c_void_p(o)) for o in outs]
+
+    def fused_sum(self, inputs, prog, slot):
+        """The sum of slot's values over all elements, a rank-0 array."""
+        ins = (C.c_void_p * len(inputs))(*[p.h for p in inputs])
+        flat = (C.c_int32 * max(6 * len(prog), 1))(*[int(x) for q in prog for x in q])
+        return self._out(self.lib.fused_sum, len(inputs), ins, len(prog), flat, slot)
 
     def fused_extremum(self, inputs, prog, slot, n_reduce, want_max):
         """(values, indices) of the first extremum of slot's values over the trailing n_reduce dims."""

@@ -616,3 +616,155 @@ extern "C" int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   *indices = ix;
   return HGPU_OK;
 }
+
+// The sum of all elements of an elementwise program's result, evaluated on the
+// fly (the result is never written): per-block partial sums in double / int64,
+// added up in a fixed order by a second, one-block launch.  Inputs must be dense
+// (16-byte aligned) or one broadcast element; anything else is left to the
+// caller (HGPU_ERR_UNSUPPORTED), who writes the result out and sums that.
+extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot,
+                              hgpu_array** out) {
+  if (!ctx || !in || (!prog && n_instr > 0) || !out) return HGPU_ERR_INVALID;
+  if (n_in < 1 || n_in > kMaxIn || n_instr < 0 || n_instr > kMaxInstr) return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_sum: %d inputs, %d instructions", n_in, n_instr);
+  const hgpu_array* a0 = in[0];
+  for (int i = 0; i < n_in; ++i) {
+    if (!in[i]) return HGPU_ERR_INVALID;
+    if (!same_shape(in[i], a0)) return fail(ctx, HGPU_ERR_INVALID, "fused_sum: input %d has another shape", i);
+  }
+  std::vector<int> dt;
+  if (int rc = check_program(ctx, n_in, in, n_instr, prog, &dt)) return rc;
+  if (slot < 0 || slot >= n_in + n_instr) return fail(ctx, HGPU_ERR_INVALID, "fused_sum: bad slot");
+  const int odt = dt[(size_t)slot];
+  if (odt == HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "fused_sum: Bool values have no sum");
+  std::string layout((size_t)n_in, 'g');
+  size_t widest = dtype_size(odt);
+  for (int i = 0; i < n_in; ++i) {
+    bool all0 = true;
+    for (int d = 0; d < in[i]->rank; ++d)
+      if (in[i]->shape[d] != 1 && in[i]->strides[d] != 0) all0 = false;
+    if (all0) layout[(size_t)i] = 's';
+    else if (is_dense(in[i]) && ((uintptr_t)data_ptr(in[i]) & 15) == 0) layout[(size_t)i] = 'd';
+    else return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_sum: input %d is a strided view", i);
+    widest = std::max(widest, dtype_size(in[i]->dtype));
+  }
+  const int vec = (int)(16 / widest);
+  const int64_t n = nelem(a0);
+  hgpu_array* o = nullptr;
+  int rc = new_zeros(ctx, odt, 0, nullptr, &o);
+  if (rc) return rc;
+  if (n == 0) { *out = o; return HGPU_OK; }
+  const bool fp = dtype_is_float(odt);
+  const char* acc = fp ? "double" : "i64";
+  const unsigned grid = grid_for((n + vec - 1) / vec, 256, ctx->num_cu * 8);
+  hgpu_buffer* part = nullptr;
+  rc = buffer_alloc(ctx, (size_t)grid * 8, &part);
+  if (rc) { hgpu_release(o); return rc; }
+
+  std::ostringstream s;
+  s << kPrelude;
+  s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
+  s << "typedef " << acc << " ACC;\n";
+  s << "__device__ __forceinline__ ACC wave_sum(ACC v) {\n"
+       "  for (int off = 32; off > 0; off >>= 1) {\n"
+       "    unsigned long long u = *reinterpret_cast<unsigned long long*>(&v);\n"
+       "    unsigned lo = __shfl_down((unsigned)(u & 0xffffffffu), off, 64), hi = __shfl_down((unsigned)(u >> 32), off, 64);\n"
+       "    unsigned long long w = ((unsigned long long)hi << 32) | lo;\n"
+       "    v += *reinterpret_cast<ACC*>(&w);\n"
+       "  }\n  return v;\n}\n";
+  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_sum(i64 n";
+  for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
+  s << ", ACC* __restrict__ part) {\n";
+  s << "  __shared__ ACC red[4];\n";
+  s << "  const i64 step = (i64)gridDim.x * 256;\n";
+  for (int i = 0; i < n_in; ++i)
+    if (layout[(size_t)i] == 's') s << "  const " << ctype(in[i]->dtype) << " s" << i << " = i" << i << "[0];\n";
+  s << "  ACC acc = 0;\n";
+  s << "  const i64 nv = n / " << vec << ";\n";
+  s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < nv; i += step) {\n";
+  for (int i = 0; i < n_in; ++i)
+    if (layout[(size_t)i] == 'd') s << "    const Vec<" << ctype(in[i]->dtype) << ", " << vec << "> l" << i << " = reinterpret_cast<const Vec<" << ctype(in[i]->dtype) << ", " << vec << ">*>(i" << i << ")[i];\n";
+  for (int e = 0; e < vec; ++e) {
+    std::string suf = "_" + std::to_string(e);
+    s << "    {\n";
+    for (int i = 0; i < n_in; ++i) {
+      s << "      const " << ctype(in[i]->dtype) << " v" << i << suf << " = ";
+      if (layout[(size_t)i] == 's') s << "s" << i; else s << "l" << i << ".v[" << e << "]";
+      s << ";\n";
+    }
+    emit_program(s, n_in, n_instr, prog, dt, "      ", suf);
+    s << "      acc += (ACC)v" << slot << suf << ";\n    }\n";
+  }
+  s << "  }\n";
+  s << "  const i64 t = nv * " << vec << " + (i64)blockIdx.x * 256 + threadIdx.x;\n";
+  s << "  if (t < n) {\n";
+  for (int i = 0; i < n_in; ++i) {
+    s << "    const " << ctype(in[i]->dtype) << " v" << i << "_t = ";
+    if (layout[(size_t)i] == 's') s << "s" << i; else s << "i" << i << "[t]";
+    s << ";\n";
+  }
+  emit_program(s, n_in, n_instr, prog, dt, "    ", "_t");
+  s << "    acc += (ACC)v" << slot << "_t;\n  }\n";
+  s << "  acc = wave_sum(acc);\n";
+  s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n";
+  s << "  __syncthreads();\n";
+  s << "  if (threadIdx.x == 0) part[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);\n";
+  s << "}\n";
+  // second launch: one block adds the partial sums up, always in the same order
+  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_sum_final(int g, const ACC* __restrict__ part, " << ctype(odt) << "* __restrict__ out) {\n";
+  s << "  __shared__ ACC red[4];\n";
+  s << "  ACC acc = 0;\n";
+  s << "  for (int i = threadIdx.x; i < g; i += 256) acc += part[i];\n";
+  s << "  acc = wave_sum(acc);\n";
+  s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n";
+  s << "  __syncthreads();\n";
+  s << "  if (threadIdx.x == 0) out[0] = (" << ctype(odt) << ")((red[0] + red[1]) + (red[2] + red[3]));\n";
+  s << "}\n";
+  std::string src = s.str();
+
+  const char* label = "fused_sum";
+  if (ctx->profiling && ctx->profile_shapes) {
+    std::string sh;
+    for (int d = 0; d < a0->rank; ++d) sh += (d ? "x" : "") + std::to_string(a0->shape[d]);
+    char buf[160];
+    snprintf(buf, sizeof buf, "fused_sum[%s,in%d(%s),instr%d,vec%d]", sh.c_str(), n_in, layout.c_str(), n_instr, vec);
+    label = ctx->label_pool.insert(buf).first->c_str();
+  }
+  double bytes = 0;
+  for (int i = 0; i < n_in; ++i) {
+    if (layout[(size_t)i] == 's') continue;
+    bool dup = false;
+    for (int j = 0; j < i; ++j)
+      if (data_ptr(in[j]) == data_ptr(in[i]) && layout[(size_t)j] != 's') dup = true;
+    if (!dup) bytes += (double)n * dtype_size(in[i]->dtype);
+  }
+  LaunchGuard lg(ctx, label, bytes, (double)n * (n_instr + 1));
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c;
+    rc = compile(ctx, src, &c, "fused_sum");
+    if (rc) { buffer_release(part); hgpu_release(o); return rc; }
+    it = cache.emplace(src, c).first;
+  }
+  hipFunction_t fin = nullptr;
+  hipError_t e = hipModuleGetFunction(&fin, it->second.mod, "fused_sum_final");
+  if (e != hipSuccess) { buffer_release(part); hgpu_release(o); return check_hip(ctx, e, "hipModuleGetFunction"); }
+  std::vector<void*> args;
+  int64_t nn = n;
+  args.push_back(&nn);
+  std::vector<const void*> ptrs((size_t)n_in);
+  for (int i = 0; i < n_in; ++i) { ptrs[(size_t)i] = data_ptr(in[i]); args.push_back(&ptrs[(size_t)i]); }
+  void* pp = part->ptr;
+  args.push_back(&pp);
+  e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e == hipSuccess) {
+    int g = (int)grid;
+    void* po = data_ptr(o);
+    void* fargs[] = {&g, &pp, &po};
+    e = hipModuleLaunchKernel(fin, 1, 1, 1, 256, 1, 1, 0, ctx->stream, fargs, nullptr);
+  }
+  buffer_release(part);
+  if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "fused_sum launch"); }
+  *out = o;
+  return HGPU_OK;
+}

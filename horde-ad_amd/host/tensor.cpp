@@ -639,6 +639,23 @@ T convert(const T& a, int dtype, int mode) {
 T contract(const T& a, const T* b, int n_keep) {
   if (!b && a.pending_product())   // sum (u * v) = the contraction of u and v; stays pending
     return lazy_contract(a.factor_a(), a.factor_b(), n_keep);
+  // ssum0 of a pending expression: summed while it is evaluated, never written
+  if (!b && n_keep == 0 && a.pending_expr() && a.size() > 0 && (a.dtype() == HGPU_F64 || a.dtype() == HGPU_F32)) {
+    Backend* be = a.be();
+    const hgpu_api* api = be->api;
+    if (api->struct_size >= offsetof(hgpu_api, fused_sum) + sizeof(api->fused_sum) && api->fused_sum && pending_size(a.holder()) <= 96) {
+      std::vector<const hgpu_array*> ins;
+      std::vector<hgpu_fused_instr> prog;
+      std::vector<int> slots;
+      number_program({a.holder().get()}, &ins, &prog, &slots);
+      if ((int)ins.size() <= 12 && (int)prog.size() <= 96) {
+        hgpu_array* o = nullptr;
+        int rc = api->fused_sum(be->ctx, (int)ins.size(), ins.data(), (int)prog.size(), prog.data(), slots[0], &o);
+        if (rc == HGPU_OK) return T(be, o);
+        if (rc != HGPU_ERR_UNSUPPORTED) be->check(rc);
+      }
+    }
+  }
   // a contraction of two arrays of one shape and dtype stays pending too: sums of
   // such (add_cotangents) are then written out by one grouped launch
   if (b && a.be()->fuse && a.dtype() == b->dtype() && a.shape() == b->shape() && n_keep >= 0 && n_keep <= a.rank() && a.size() > 0 &&

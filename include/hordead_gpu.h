@@ -225,6 +225,11 @@ int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_i
  * `maxPool2dUnpaddedS (reluS (conv + bias))` (External/CommonShapedOps.hs:
  * 241-260) reads the convolution once and writes only the pooled maxima and
  * their arguments. */
+/* tssum0 of such a program's result (OpsConcrete.hs:229-230), evaluated on the
+ * fly: the result itself is never written.  Inputs must be dense or one
+ * broadcast element (else HGPU_ERR_UNSUPPORTED: write the result out and sum
+ * that).  Accumulates in double / int64 in an order fixed by the size. */
+int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot, hgpu_array** out);
 int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot, int n_reduce,
                         int want_max, hgpu_array** values, hgpu_array** indices);
 
@@ -381,6 +386,7 @@ typedef struct hgpu_api {
   int (*assign)(hgpu_ctx*, hgpu_array*, const hgpu_array*);
   int (*extremum_last)(hgpu_ctx*, const hgpu_array*, int, hgpu_array**, hgpu_array**);
   int (*fused_extremum)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, int, int, hgpu_array**, hgpu_array**);
+  int (*fused_sum)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

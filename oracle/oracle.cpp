@@ -740,6 +740,7 @@ const hgpu_api* horc_get_api(void) {
       horc_contract_sum, horc_assign,
       nullptr,   // no extremum_last: the checker gathers at the arg-extremum as the reference does
       nullptr,   // no fused_extremum
+      nullptr,   // no fused_sum
   };
   return &api;
 }

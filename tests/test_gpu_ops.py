@@ -251,6 +251,30 @@ def test_argminmax_iota_concat(both):
     assert_same(both.concat(parts))
 
 
+@pytest.mark.parametrize("dt", [np.float64, np.float32, np.int64])
+def test_fused_sum_equals_program_then_sum(gpu, dt):
+    """The sum of a program's result taken on the fly against numpy on the same program."""
+    O1, O2 = capi.OP1, capi.OP2
+    fp = np.dtype(dt).kind == "f"
+    prog = [(1, O2["mul"], 0, 0, 1, 0), (1, O2["add"], 0, 3, 2, 0)] + ([(0, O1["sin"], 0, 4, 0, 0)] if fp else [(0, O1["abs"], 0, 4, 0, 0)])
+    for shape in [(1031,), (37, 29), (4096, 33), ()]:
+        a, b = rnd(shape, dt), rnd(shape, dt)
+        c = dt(3) if fp else dt(3)
+        ins = [gpu.upload(a), gpu.upload(b), gpu.upload(c).replicate(list(shape))]
+        got = gpu.fused_sum(ins, prog, 5).numpy()
+        acc = np.float64 if fp else np.int64
+        want = (np.sin(a.astype(acc) * b + c) if fp else np.abs(a.astype(acc) * b + c)).sum()
+        assert got.dtype == np.dtype(dt) and got.shape == ()
+        if fp:
+            assert np.isclose(got, want, rtol=TOL[np.dtype(dt)] * 10, atol=TOL[np.dtype(dt)] * max(1, a.size))
+        else:
+            assert got == want
+        assert np.isclose(float(gpu.fused_sum(ins, prog, 0).numpy()), float(a.astype(acc).sum()), rtol=1e-5)
+    with pytest.raises(capi.HgpuError) as e:
+        gpu.fused_sum([gpu.upload(rnd((8, 6), dt)).transpose([1, 0])], [], 0)        # a strided view: left to the caller
+    assert e.value.code == 4
+
+
 @pytest.mark.parametrize("dt", [np.float64, np.float32, np.int32])
 def test_fused_extremum_equals_program_then_extremum(gpu, dt):
     """The extremum of a program's result over its trailing dims, taken on the
