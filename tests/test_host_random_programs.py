@@ -1,0 +1,139 @@
+"""Differential test of the host layer's deferred evaluation: random programs
+of structural and elementwise operations, their values and gradients on the
+device (where elementwise work, contractions, concatenations, zero-extensions
+and merged reshapes stay pending and fuse) against the checker (where every
+operation is executed at once, as the reference's `Concrete` instance does).
+The programs are drawn from a fixed seed."""
+import numpy as np
+import pytest
+
+from conftest import capi, entry, pkg
+
+H = pkg.hostapi
+
+pytestmark = pytest.mark.gpu
+
+
+def factorizations(n):
+    return [(a, n // a) for a in range(2, n) if n % a == 0]
+
+
+def random_program(seed):
+    """A list of steps (name, args) over a stack of values; generated once, replayed on both hosts."""
+    rng = np.random.default_rng(seed)
+    shapes = [tuple(int(x) for x in rng.integers(2, 7, int(rng.integers(2, 4))))]
+    steps = []
+    stack = [shapes[0]]                        # shapes of the values made so far (value 0 is the input)
+    for _ in range(int(rng.integers(6, 14))):
+        i = int(rng.integers(0, len(stack)))
+        sh = stack[i]
+        kind = rng.choice(["unary", "binary", "transpose", "split", "merge", "slice", "append", "sum", "scale", "bias", "pool"])
+        if kind == "unary":
+            steps.append(("unary", i, str(rng.choice(["sin", "tanh", "cos"]))))
+            stack.append(sh)
+        elif kind == "binary":
+            same = [j for j, s in enumerate(stack) if s == sh]
+            j = int(rng.choice(same))
+            steps.append(("binary", i, j, str(rng.choice(["add", "mul", "sub"]))))
+            stack.append(sh)
+        elif kind == "transpose" and len(sh) >= 2:
+            perm = [int(p) for p in rng.permutation(len(sh))]
+            steps.append(("transpose", i, perm))
+            stack.append(tuple(sh[p] for p in perm))
+        elif kind == "split":
+            d = int(rng.integers(0, len(sh)))
+            f = factorizations(sh[d])
+            if f and len(sh) < 6:
+                a, b = f[int(rng.integers(0, len(f)))]
+                new = sh[:d] + (a, b) + sh[d + 1:]
+                steps.append(("reshape", i, list(new)))
+                stack.append(new)
+        elif kind == "merge" and len(sh) >= 2:
+            d = int(rng.integers(0, len(sh) - 1))
+            new = sh[:d] + (sh[d] * sh[d + 1],) + sh[d + 2:]
+            steps.append(("reshape", i, list(new)))
+            stack.append(new)
+        elif kind == "slice" and sh[0] >= 2:
+            start = int(rng.integers(0, sh[0] - 1))
+            ln = int(rng.integers(1, sh[0] - start + 1))
+            steps.append(("slice", i, start, ln))
+            stack.append((ln,) + sh[1:])
+        elif kind == "append":
+            same = [j for j, s in enumerate(stack) if s[1:] == sh[1:]]
+            j = int(rng.choice(same))
+            steps.append(("append", i, j))
+            stack.append((sh[0] + stack[j][0],) + sh[1:])
+        elif kind == "sum" and len(sh) >= 2:
+            k = int(rng.integers(1, len(sh)))
+            steps.append(("sum", i, k))
+            stack.append(sh[k:])
+        elif kind == "scale":
+            steps.append(("scale", i, float(rng.uniform(-2, 2))))
+            stack.append(sh)
+        elif kind == "bias" and len(sh) >= 2:
+            steps.append(("bias", i, int(rng.integers(0, 1000))))
+            stack.append(sh)
+        elif kind == "pool" and len(sh) >= 2 and sh[-1] % 2 == 0 and sh[-2] % 2 == 0:
+            steps.append(("pool", i))
+            stack.append(sh[:-2] + (sh[-2] // 2, sh[-1] // 2))
+    return shapes[0], steps, stack
+
+
+def run(host, x0, steps):
+    vals = [host.param(x0)]
+    for st in steps:
+        v = vals[st[1]]
+        if st[0] == "unary":
+            vals.append(v.op1(st[2]))
+        elif st[0] == "binary":
+            vals.append(v.op2(st[3], vals[st[2]]))
+        elif st[0] == "transpose":
+            vals.append(v.stranspose(st[2]))
+        elif st[0] == "reshape":
+            vals.append(v.sreshape(st[2]))
+        elif st[0] == "slice":
+            vals.append(v.sslice(st[2], st[3]))
+        elif st[0] == "append":
+            vals.append(v.sappend(vals[st[2]]))
+        elif st[0] == "sum":
+            vals.append(v.ssumN(st[2]))
+        elif st[0] == "scale":
+            vals.append(v * host.srepl(v.shape, st[2], v.dtype))
+        elif st[0] == "bias":
+            sh = v.shape
+            b = np.random.default_rng(st[2]).uniform(-1, 1, sh[-1])
+            vals.append(v + host.concrete(b).sreplicateN(list(sh[:-1])))
+        elif st[0] == "pool":      # 2x2 max over the last two dims: window gather, merged reshape, kargMax, gather
+            sh = v.shape
+            lead, h2, w2 = list(sh[:-2]), sh[-2] // 2, sh[-1] // 2
+            r = len(lead)
+            t = v.stranspose([r, r + 1] + list(range(r)))
+            win = t.sgather((h2, 2, w2, 2), lambda i, p, j, q: [2 * i + p, 2 * j + q])
+            win = win.stranspose(list(range(4, 4 + r)) + [0, 2, 1, 3]).sreshape(lead + [h2, w2, 4])
+            wp = win.sprimalPart()
+            shm = tuple(lead + [h2, w2])
+            vals.append(win.sgather(shm, lambda *ix: list(ix) + [wp.kargMax(list(ix))]))
+    # an objective that uses every value made
+    loss = None
+    for k, v in enumerate(vals[1:], 1):
+        term = (v * v).ssum0() * host.srepl((), 0.5 + 0.1 * k, v.dtype)
+        loss = term if loss is None else loss + term
+    if loss is None:
+        loss = (vals[0] * vals[0]).ssum0()
+    (g,) = host.grad(loss, [vals[0]])
+    out = [v.numpy() for v in vals], loss.numpy(), g.numpy()
+    host.tape_reset()
+    return out
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_program_matches_the_checker(seed):
+    shape, steps, _ = random_program(seed)
+    x0 = np.random.default_rng(1000 + seed).uniform(-1, 1, shape)
+    cpu = run(H.Host(capi.Lib(entry.ORACLE_LIB, "horc_")), x0, steps)
+    gpu = run(H.Host(), x0, steps)
+    for a, b in zip(gpu[0], cpu[0]):
+        assert a.shape == b.shape
+        assert np.allclose(a, b, rtol=1e-11, atol=1e-12), steps
+    assert np.isclose(gpu[1], cpu[1], rtol=1e-11), steps
+    assert np.allclose(gpu[2], cpu[2], rtol=1e-10, atol=1e-11), steps
