@@ -631,7 +631,8 @@ def test_fused_map_equals_the_single_operations(gpu, oracle, dt):
         (4, 0, capi.F32 if dt == np.float64 else capi.F64, 20, 0, 0),   # 24: cast
     ]
     outs = [14, 17, 20, 21, 22, 23, 24][:6]
-    for shape, views in [((1031,), False), ((37, 29), False), ((6, 5, 7), True)]:
+    # the last two are large enough for the kernels compiled with their shapes and strides
+    for shape, views in [((1031,), False), ((37, 29), False), ((6, 5, 7), True), ((601, 701), False), ((96, 81, 70), True)]:
         data = [rnd(shape, dt) + dt(2.5) for _ in range(3)]
         res = []
         for ctx in (gpu, oracle):
