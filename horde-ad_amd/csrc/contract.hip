@@ -438,7 +438,7 @@ int contract_terms(hgpu_ctx* ctx, int n, const hgpu_array* const* as, const hgpu
   if (n_out * n < want_items) {
     S = (want_items + n_out * n - 1) / (n_out * n);
     int64_t span = use_wave ? ((R / Lin) > 1 ? (R / Lin) : Lin) : R;
-    int64_t per = use_wave ? ((R / Lin) > 1 ? 2048 / (Lin < 2048 ? Lin : 2048) : 1024) : 256;
+    int64_t per = use_wave ? ((R / Lin) > 1 ? 512 / (Lin < 512 ? Lin : 512) : 1024) : 256;
     if (per < 1) per = 1;
     int64_t maxS = span / per;
     if (maxS < 1) maxS = 1;
@@ -598,13 +598,13 @@ int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n
   if (n_out < 2048) use_wave = true;
   else if (sr <= sk && Lin >= 16) use_wave = true;
   else use_wave = false;
-  // Enough work items to fill the device, chunks of at least 2048 elements.
+  // Enough work items to fill the device, chunks of at least 512 elements.
   int64_t want_items = (int64_t)ctx->num_cu * (use_wave ? 16 : 1024);
   int64_t S = 1;
   if (n_out < want_items) {
     S = (want_items + n_out - 1) / n_out;
     int64_t span = use_wave ? ((R / Lin) > 1 ? (R / Lin) : Lin) : R;
-    int64_t per = use_wave ? ((R / Lin) > 1 ? 2048 / (Lin < 2048 ? Lin : 2048) : 1024) : 256;
+    int64_t per = use_wave ? ((R / Lin) > 1 ? 512 / (Lin < 512 ? Lin : 512) : 1024) : 256;
     if (per < 1) per = 1;
     int64_t maxS = span / per;
     if (maxS < 1) maxS = 1;

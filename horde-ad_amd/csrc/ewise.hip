@@ -170,6 +170,46 @@ __global__ void __launch_bounds__(kBlock) k_copy(Dims d, int64_t n, const T* __r
   }
 }
 
+// Zero padding in one pass over the result: the dims of the (dense) result in
+// memory order, for each the padding in front, the source's extent and stride.
+struct PadDims {
+  int nd;
+  int64_t shape[HG_KDIMS], lo[HG_KDIMS], ext[HG_KDIMS], sst[HG_KDIMS];
+};
+
+struct alignas(16) Bytes16 { uint64_t lo, hi; };
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_pad(PadDims d, int64_t n, const T* __restrict__ a, T* __restrict__ o) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) {
+    int64_t off = 0;
+    bool inside = true;
+    if (n <= (int64_t)0x7fffffff) {
+      uint32_t r = (uint32_t)i;
+      for (int k = d.nd - 1; k >= 0; --k) {
+        uint32_t s = (uint32_t)d.shape[k];
+        uint32_t q = k > 0 ? r / s : 0;
+        int64_t c = (int64_t)(r - q * s) - d.lo[k];
+        r = q;
+        inside = inside && (uint64_t)c < (uint64_t)d.ext[k];
+        off += c * d.sst[k];
+      }
+    } else {
+      int64_t r = i;
+      for (int k = d.nd - 1; k >= 0; --k) {
+        int64_t s = d.shape[k];
+        int64_t q = k > 0 ? r / s : 0;
+        int64_t c = r - q * s - d.lo[k];
+        r = q;
+        inside = inside && (uint64_t)c < (uint64_t)d.ext[k];
+        off += c * d.sst[k];
+      }
+    }
+    o[i] = inside ? a[off] : T{};
+  }
+}
+
 // ---- dense fast paths: 16-byte vectors, flags say which operands broadcast --
 
 template <typename T> struct Vec16 { static constexpr int N = 16 / sizeof(T); T v[N]; };
@@ -319,19 +359,75 @@ int hgpu_pad(hgpu_ctx* ctx, const hgpu_array* a, const int64_t* lo, const int64_
     for (int j = i; j > 0 && key(order[j]) > key(order[j - 1]); --j) { int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t; }
   int64_t psh[HGPU_MAX_RANK];
   for (int i = 0; i < a->rank; ++i) psh[i] = sh[order[i]];
+  // dims of the result in memory order; neighbours without padding whose source
+  // strides nest become one dim, dims of extent 1 vanish
+  PadDims d;
+  d.nd = 0;
+  int64_t n = 1;
+  for (int i = 0; i < a->rank; ++i) {
+    const int dim = order[i];
+    n *= psh[i];
+    if (psh[i] == 1 && a->shape[dim] == 1) continue;
+    const bool plain = lo[dim] == 0 && hi[dim] == 0;
+    if (d.nd > 0 && plain && d.lo[d.nd - 1] == 0 && d.ext[d.nd - 1] == d.shape[d.nd - 1] && d.sst[d.nd - 1] == a->strides[dim] * a->shape[dim]) {
+      d.shape[d.nd - 1] *= psh[i];
+      d.ext[d.nd - 1] *= psh[i];
+      d.sst[d.nd - 1] = a->strides[dim];
+      continue;
+    }
+    if (d.nd == HG_KDIMS) return fail(ctx, HGPU_ERR_UNSUPPORTED, "pad: more than %d merged dims", HG_KDIMS);
+    d.shape[d.nd] = psh[i];
+    d.lo[d.nd] = lo[dim];
+    d.ext[d.nd] = a->shape[dim];
+    d.sst[d.nd] = a->strides[dim];
+    ++d.nd;
+  }
+  if (d.nd == 0) { d.nd = 1; d.shape[0] = 1; d.lo[0] = 0; d.ext[0] = 1; d.sst[0] = 0; }
   hgpu_array* phys = nullptr;
-  int rc = new_zeros(ctx, a->dtype, a->rank, psh, &phys);
+  int rc = new_dense(ctx, a->dtype, a->rank, psh, &phys);
   if (rc) return rc;
   int64_t st[HGPU_MAX_RANK];
   for (int i = 0; i < a->rank; ++i) st[order[i]] = phys->strides[i];
   hgpu_array* o = new_view(ctx, phys->buf, a->dtype, a->rank, sh, st, 0);
   hgpu_release(phys);
-  int64_t off = 0;
-  for (int i = 0; i < a->rank; ++i) off += lo[i] * o->strides[i];
-  if (nelem(a) > 0)
-    rc = copy_view(ctx, a->dtype, a->rank, a->shape, data_ptr(a), a->strides,
-                   (char*)data_ptr(o) + off * (int64_t)dtype_size(a->dtype), o->strides);
-  if (rc) { hgpu_release(o); return rc; }
+  if (n > 0) {
+    const char* label = "pad";
+    if (ctx->profiling && ctx->profile_shapes) {
+      char buf[200];
+      int w = snprintf(buf, sizeof buf, "pad[es%d", (int)dtype_size(a->dtype));
+      for (int i = 0; i < d.nd && w < (int)sizeof buf - 80; ++i)
+        w += snprintf(buf + w, sizeof buf - w, ",%lld+%lld/%lld:%lld", (long long)d.lo[i], (long long)d.ext[i], (long long)d.shape[i], (long long)d.sst[i]);
+      snprintf(buf + w, sizeof buf - w, "]");
+      label = ctx->label_pool.insert(buf).first->c_str();
+    }
+    LaunchGuard lg(ctx, label, (double)(n + nelem(a)) * dtype_size(a->dtype), 0);
+    const void* src = data_ptr(a);
+    void* dst = data_ptr(o);
+    // rows whose extents, paddings and addresses are all multiples of 16 bytes move as 16-byte elements
+    size_t es = dtype_size(a->dtype);
+    const int64_t f = 16 / (int64_t)es;
+    const int in = d.nd - 1;
+    bool wide = es < 16 && d.sst[in] == 1 && d.shape[in] % f == 0 && d.lo[in] % f == 0 && d.ext[in] % f == 0 && ((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0;
+    for (int i = 0; i < in && wide; ++i) wide = d.sst[i] % f == 0;
+    if (wide) {
+      d.shape[in] /= f;
+      d.lo[in] /= f;
+      d.ext[in] /= f;
+      for (int i = 0; i < in; ++i) d.sst[i] /= f;
+      n /= f;
+      es = 16;
+    }
+    unsigned g = grid_for(n, kBlock, max_blocks(ctx));
+    switch (es) {
+      case 16: hipLaunchKernelGGL(k_pad<Bytes16>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const Bytes16*)src, (Bytes16*)dst); break;
+      case 8: hipLaunchKernelGGL(k_pad<uint64_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint64_t*)src, (uint64_t*)dst); break;
+      case 4: hipLaunchKernelGGL(k_pad<uint32_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint32_t*)src, (uint32_t*)dst); break;
+      case 2: hipLaunchKernelGGL(k_pad<uint16_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint16_t*)src, (uint16_t*)dst); break;
+      default: hipLaunchKernelGGL(k_pad<uint8_t>, dim3(g), dim3(kBlock), 0, ctx->stream, d, n, (const uint8_t*)src, (uint8_t*)dst); break;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "pad"); }
+  }
   *out = o;
   return HGPU_OK;
 }

@@ -252,12 +252,23 @@ constexpr int BUF = MODE == 0 ? LX + LY : LX;           // elements per chunk bu
 constexpr int RED0 = NBUFS * BUF + (MODE == 0 ? 0 : LY);    // scratch for adding up split row blocks
 constexpr int LDS_ELEMS = RED0 + (REM > 0 ? REM * 4 * 256 : 0);
 
-// The four registers of a lane are rows m0 .. m0 + 3 of column col.
-__device__ __forceinline__ void store_rows(T* __restrict__ out, int m0, int col, T v0, T v1, T v2, T v3) {
+// The four registers of a lane are rows m0 .. m0 + 3 of column col.  Where
+// they go inside a chunk's output comes from two tables in memory; a kernel that
+// stores once per chunk looks them up before its loop over the chunks, because a
+// wait for such a lookup is also a wait for every store issued before it.
+struct OutPos { int o[CVEC ? 1 : 4]; };
+__device__ __forceinline__ OutPos out_pos(int m0, int col) {
+  OutPos p;
+  const int cc = kColC[col < NIN ? col : NIN - 1];
+#pragma unroll
+  for (int j = 0; j < (CVEC ? 1 : 4); ++j) p.o[j] = kRowC[m0 + j < MIN ? m0 + j : MIN - 1] + cc;
+  return p;
+}
+__device__ __forceinline__ void store_rows(T* __restrict__ out, const OutPos& p, int m0, int col, T v0, T v1, T v2, T v3) {
   if (col >= NIN) return;
   if (CVEC) {      // the four rows are adjacent in memory and 16-byte aligned
     if (m0 < MIN) {
-      T* dst = out + kRowC[m0] + kColC[col];
+      T* dst = out + p.o[0];
 #if F64
       reinterpret_cast<Vec<2>*>(dst)[0] = Vec<2>{v0, v1};
       reinterpret_cast<Vec<2>*>(dst)[1] = Vec<2>{v2, v3};
@@ -266,11 +277,10 @@ __device__ __forceinline__ void store_rows(T* __restrict__ out, int m0, int col,
 #endif
     }
   } else {
-    const int cc = kColC[col];
-    if (m0 < MIN) out[kRowC[m0] + cc] = v0;
-    if (m0 + 1 < MIN) out[kRowC[m0 + 1] + cc] = v1;
-    if (m0 + 2 < MIN) out[kRowC[m0 + 2] + cc] = v2;
-    if (m0 + 3 < MIN) out[kRowC[m0 + 3] + cc] = v3;
+    if (m0 < MIN) out[p.o[0]] = v0;
+    if (m0 + 1 < MIN) out[p.o[CVEC ? 0 : 1]] = v1;
+    if (m0 + 2 < MIN) out[p.o[CVEC ? 0 : 2]] = v2;
+    if (m0 + 3 < MIN) out[p.o[CVEC ? 0 : 3]] = v3;
   }
 }
 
@@ -310,6 +320,12 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   }
   // lanes past the end of K in the last group contribute zero
   const bool tail_lane = q4 >= KVALID;
+  OutPos pos[MODE == 1 ? NACC : 1];
+  if (MODE == 1) {
+#pragma unroll
+    for (int t = 0; t < NBF; ++t) pos[t] = out_pos((wave + 4 * t) * 16 + 4 * q4, r);
+    if (REM > 0) pos[NBF] = out_pos((4 * NBF + (wave < REM ? wave : 0)) * 16 + 4 * q4, r);
+  }
   Acc acc[NACC];
 #pragma unroll
   for (int t = 0; t < NACC; ++t) acc[t] = Acc{0, 0, 0, 0};
@@ -414,7 +430,7 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
     if (MODE == 1) {
       T* out = C + ch * chc;
 #pragma unroll
-      for (int t = 0; t < NBF; ++t) store_rows(out, (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      for (int t = 0; t < NBF; ++t) store_rows(out, pos[t], (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
       if (REM > 0) {
         T* red = lds + RED0;
 #pragma unroll
@@ -431,7 +447,7 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
 #pragma unroll
             for (int w = 0; w < 4; ++w) s[j] += red[((rb * 4 + w) * 4 + j) * 64 + lane];
           }
-          store_rows(out, (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
+          store_rows(out, pos[MODE == 1 ? NBF : 0], (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
         }
       }
     }
@@ -439,7 +455,7 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   if (MODE == 0) {
     T* out = C + (i64)blockIdx.x * part_stride;
 #pragma unroll
-    for (int t = 0; t < NBF; ++t) store_rows(out, (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+    for (int t = 0; t < NBF; ++t) store_rows(out, out_pos((wave + 4 * t) * 16 + 4 * q4, r), (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
     if (REM > 0) {
       T* red = lds + RED0;
       __syncthreads();
@@ -457,7 +473,7 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
 #pragma unroll
           for (int w = 0; w < 4; ++w) s[j] += red[((rb * 4 + w) * 4 + j) * 64 + lane];
         }
-        store_rows(out, (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
+        store_rows(out, out_pos((4 * NBF + rb) * 16 + 4 * q4, r), (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
       }
     }
   }

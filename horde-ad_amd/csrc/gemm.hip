@@ -53,27 +53,40 @@ __global__ void k_koff(Group k, int64_t K, int64_t Kp, int64_t* __restrict__ ka,
 }
 
 // Sums the split-K partials: out[i] = sum_s part[s * stride + i].  A block owns
-// 32 consecutive outputs; its 8 groups of 32 lanes each take every 8th partial
-// (coalesced rows of 32 elements) and combine through LDS in a fixed order.
-template <typename T>
+// OPB consecutive outputs; its 256 / OPB groups of lanes each take every
+// (256 / OPB)-th partial (coalesced rows of OPB elements), several loads in
+// flight at a time, and combine through LDS in a fixed order.  Few outputs get
+// the narrow blocks: more of them, and fewer partials for a lane to walk through.
+template <typename T, int OPB>
 __global__ void __launch_bounds__(256) k_sum_partials(int64_t n, int S, int64_t stride, const T* __restrict__ part, T* __restrict__ out) {
-  __shared__ T red[8][33];
-  const int ol = threadIdx.x & 31, g = threadIdx.x >> 5;
-  for (int64_t base = (int64_t)blockIdx.x * 32; base < n; base += (int64_t)gridDim.x * 32) {
+  constexpr int G = 256 / OPB;
+  __shared__ T red[G][OPB + 1];
+  const int ol = threadIdx.x % OPB, g = threadIdx.x / OPB;
+  for (int64_t base = (int64_t)blockIdx.x * OPB; base < n; base += (int64_t)gridDim.x * OPB) {
     int64_t i = base + ol;
     T acc = T(0);
-    if (i < n)
-      for (int s = g; s < S; s += 8) acc += part[(int64_t)s * stride + i];
+    if (i < n) {
+#pragma unroll 8
+      for (int s = g; s < S; s += G) acc += part[(int64_t)s * stride + i];
+    }
     red[g][ol] = acc;
     __syncthreads();
     if (g == 0 && i < n) {
       T t = red[0][ol];
 #pragma unroll
-      for (int k = 1; k < 8; ++k) t += red[k][ol];
+      for (int k = 1; k < G; ++k) t += red[k][ol];
       out[i] = t;
     }
     __syncthreads();
   }
+}
+
+template <typename T>
+void launch_sum_partials(hgpu_ctx* ctx, int64_t n, int S, const T* part, T* out) {
+  if (n <= 32768 && S >= 32)
+    hipLaunchKernelGGL((k_sum_partials<T, 8>), dim3(grid_for(n, 8, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out);
+  else
+    hipLaunchKernelGGL((k_sum_partials<T, 32>), dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out);
 }
 
 // Appends dim (extent e, strides a, b, c) to a group, merging with the previous dim when all strides allow.
@@ -218,10 +231,8 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
     }
     if (split > 1) {
       LaunchGuard ls(ctx, "gemm_sum_partials", (double)out_n * (split + 1) * es, (double)out_n * split);
-      if (dtype == HGPU_F64)
-        hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, (int)split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
-      else
-        hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, (int)split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
+      if (dtype == HGPU_F64) launch_sum_partials<double>(ctx, out_n, (int)split, (const double*)part->ptr, (double*)data_ptr(out));
+      else launch_sum_partials<float>(ctx, out_n, (int)split, (const float*)part->ptr, (float*)data_ptr(out));
     }
   }
   hipError_t e = hipGetLastError();
@@ -241,10 +252,8 @@ int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa,
 int sum_partials(hgpu_ctx* ctx, int dtype, int64_t n, int parts, const void* part, void* out) {
   size_t es = dtype_size(dtype);
   LaunchGuard ls(ctx, "gemm_sum_partials", (double)n * (parts + 1) * es, (double)n * parts);
-  if (dtype == HGPU_F64)
-    hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, parts, n, (const double*)part, (double*)out);
-  else
-    hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, parts, n, (const float*)part, (float*)out);
+  if (dtype == HGPU_F64) launch_sum_partials<double>(ctx, n, parts, (const double*)part, (double*)out);
+  else launch_sum_partials<float>(ctx, n, parts, (const float*)part, (float*)out);
   HG_CHECK_LAUNCH(ctx, "gemm_sum_partials");
   return HGPU_OK;
 }
@@ -446,10 +455,8 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     }
     if (split > 1) {
       LaunchGuard ls(ctx, "gemm_sum_partials", (double)out_n * (split + 1) * es, (double)out_n * split);
-      if (a->dtype == HGPU_F64)
-        hipLaunchKernelGGL(k_sum_partials<double>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const double*)part->ptr, (double*)data_ptr(out));
-      else
-        hipLaunchKernelGGL(k_sum_partials<float>, dim3(grid_for(out_n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, out_n, split, out_n, (const float*)part->ptr, (float*)data_ptr(out));
+      if (a->dtype == HGPU_F64) launch_sum_partials<double>(ctx, out_n, (int)split, (const double*)part->ptr, (double*)data_ptr(out));
+      else launch_sum_partials<float>(ctx, out_n, (int)split, (const float*)part->ptr, (float*)data_ptr(out));
     }
   }
   hipError_t e = hipGetLastError();

@@ -88,6 +88,35 @@ def test_reshape_view_or_copy(both, gpu):
     assert_same(p.reverse(2).reshape([4, 30]))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [np.float64, np.float32, np.int64, np.int32, np.int16, np.int8, np.bool_])
+def test_pad_against_numpy(gpu, dt):
+    """Zero padding (the out-of-bounds rows of an affine gather, OpsConcrete.hs:1654-1665)
+    of dense, transposed, reversed, replicated, sliced and empty sources: bit-exact."""
+    x = rnd((5, 4, 6, 7), dt)
+    a = gpu.upload(x)
+    cases = [
+        (a, x, [0, 0, 2, 2], [0, 0, 2, 2]),
+        (a, x, [1, 0, 0, 3], [0, 2, 1, 0]),
+        (a, x, [0, 0, 0, 0], [0, 0, 0, 0]),
+        (a.transpose([2, 0, 3, 1]), np.transpose(x, (2, 0, 3, 1)), [1, 0, 2, 0], [0, 1, 0, 2]),
+        (a.reverse(2), x[:, :, ::-1], [0, 1, 1, 0], [2, 0, 0, 1]),
+        (a.slice(3, 2, 4), x[..., 2:6], [0, 0, 0, 1], [0, 0, 0, 1]),
+        (a.slice(0, 1, 0), x[1:1], [2, 0, 0, 0], [1, 0, 1, 0]),
+    ]
+    v = rnd((6,), dt)
+    cases.append((gpu.upload(v).replicate([3]), np.broadcast_to(v, (3, 6)), [1, 2], [0, 1]))
+    cases.append((gpu.upload(v).reshape([6, 1]), v.reshape(6, 1), [0, 1], [1, 1]))
+    for arr, ref, lo, hi in cases:
+        got = arr.pad(lo, hi).numpy()
+        want = np.pad(ref, list(zip(lo, hi)))
+        assert got.dtype == want.dtype and got.shape == want.shape
+        assert np.array_equal(got, want), (lo, hi)
+    big = rnd((300, 16, 14, 14), dt)   # the second convolution's input at a size that fills the device
+    got = gpu.upload(big).pad([0, 0, 2, 2], [0, 0, 2, 2]).numpy()
+    assert np.array_equal(got, np.pad(big, [(0, 0), (0, 0), (2, 2), (2, 2)]))
+
+
 def test_index_pad_onehot_as_strided(both):
     p = random_view(both, np.float64, rank=4, steps=3)
     sh = p.shape
