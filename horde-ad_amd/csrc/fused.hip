@@ -311,6 +311,27 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     }
   }
   const bool bake = !all_simple && n >= (1 << 18) && n < (1LL << 31);
+  // A compiled-in layout whose innermost dim holds whole 16-byte groups of the
+  // widest type: a lane takes one group.  An input that does not move along that
+  // dim is loaded once for the group, one that runs along it (and whose other
+  // strides and address keep the groups aligned) with one vector load.
+  int gvec = 1;
+  std::string inner((size_t)n_in, 'x');   // per input: '0' broadcast, 'v' vector load, 'x' one load per element
+  if (bake) {
+    const int W = (int)(16 / widest);
+    const int in_d = fd.nd - 1;
+    if (W > 1 && fd.shape[in_d] % W == 0) {
+      gvec = W;
+      for (int i = 0; i < n_in; ++i) {
+        if (layout[(size_t)i] == 's') continue;
+        if (fd.st[i][in_d] == 0) { inner[(size_t)i] = '0'; continue; }
+        if (fd.st[i][in_d] != 1) continue;
+        bool ok = ((uintptr_t)data_ptr(in[i]) % (dtype_size(in[i]->dtype) * W)) == 0;
+        for (int q = 0; q < in_d && ok; ++q) ok = fd.st[i][q] % W == 0;
+        if (ok) inner[(size_t)i] = 'v';
+      }
+    }
+  }
 
   // ---- source
   std::ostringstream s;
@@ -372,6 +393,43 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     emit_program("    ", "_t");
     for (int o = 0; o < n_out; ++o) s << "    o" << o << "[t] = v" << out_slots[o] << "_t;\n";
     s << "  }\n";
+  } else if (bake && gvec > 1) {
+    const int W = gvec, in_d = fd.nd - 1;
+    s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n / " << W << "; i += step) {\n";
+    s << "    unsigned r = (unsigned)i;\n";
+    for (int q = in_d; q >= 0; --q) {
+      const long long ext = q == in_d ? fd.shape[q] / W : fd.shape[q];
+      if (q > 0) s << "    const unsigned c" << q << " = (r % " << ext << "u)" << (q == in_d ? " * " + std::to_string(W) + "u" : std::string()) << "; r /= " << ext << "u;\n";
+      else s << "    const unsigned c0 = r" << (q == in_d ? " * " + std::to_string(W) + "u" : std::string()) << ";\n";
+    }
+    for (int i = 0; i < n_in; ++i) {
+      if (layout[(size_t)i] == 's') continue;
+      s << "    const i64 off" << i << " = 0";
+      for (int q = 0; q < fd.nd; ++q)
+        if (fd.st[i][q] != 0) s << " + (i64)c" << q << " * " << fd.st[i][q] << "ll";
+      s << ";\n";
+      const char* ct = ctype(in[i]->dtype);
+      if (inner[(size_t)i] == 'v') s << "    const Vec<" << ct << ", " << W << "> l" << i << " = *reinterpret_cast<const Vec<" << ct << ", " << W << ">*>(i" << i << " + off" << i << ");\n";
+      else if (inner[(size_t)i] == '0') s << "    const " << ct << " b" << i << " = i" << i << "[off" << i << "];\n";
+    }
+    for (int o = 0; o < n_out; ++o) s << "    Vec<" << ctype(res[(size_t)o]->dtype) << ", " << W << "> r" << o << ";\n";
+    for (int e = 0; e < W; ++e) {
+      std::string suf = "_" + std::to_string(e);
+      s << "    {\n";
+      for (int i = 0; i < n_in; ++i) {
+        s << "      const " << ctype(in[i]->dtype) << " v" << i << suf << " = ";
+        if (layout[(size_t)i] == 's') s << "s" << i;
+        else if (inner[(size_t)i] == 'v') s << "l" << i << ".v[" << e << "]";
+        else if (inner[(size_t)i] == '0') s << "b" << i;
+        else s << "i" << i << "[off" << i << " + " << (long long)e * fd.st[i][in_d] << "ll]";
+        s << ";\n";
+      }
+      emit_program("      ", suf);
+      for (int o = 0; o < n_out; ++o) s << "      r" << o << ".v[" << e << "] = v" << out_slots[o] << suf << ";\n";
+      s << "    }\n";
+    }
+    for (int o = 0; o < n_out; ++o) s << "    reinterpret_cast<Vec<" << ctype(res[(size_t)o]->dtype) << ", " << W << ">*>(o" << o << ")[i] = r" << o << ";\n";
+    s << "  }\n";
   } else if (bake) {
     s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {\n";
     s << "    unsigned r = (unsigned)i;\n";
@@ -426,7 +484,7 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
       if (layout[(size_t)i] == 'g')
         for (int d = 0; d < in[i]->rank; ++d) gst += (d ? ":" : ",g") + std::to_string(in[i]->strides[d]);
     char buf[200];
-    snprintf(buf, sizeof buf, "fused_map[%s,in%d(%s),instr%d(k%d.op%d..),out%d,vec%d,dt%d%s]", sh.c_str(), n_in, layout.c_str(), n_instr, prog[0].kind, prog[0].op, n_out, vec, a0->dtype, gst.c_str());
+    snprintf(buf, sizeof buf, "fused_map[%s,in%d(%s),instr%d(k%d.op%d..),out%d,vec%d,dt%d%s]", sh.c_str(), n_in, layout.c_str(), n_instr, prog[0].kind, prog[0].op, n_out, all_simple ? vec : gvec, a0->dtype, gst.c_str());
     label = ctx->label_pool.insert(buf).first->c_str();
   }
   LaunchGuard lg(ctx, label, 0, 0);
@@ -461,7 +519,7 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   if (!all_simple && !bake) args.push_back(&fd);
   for (int i = 0; i < n_in; ++i) { ptrs[(size_t)i] = data_ptr(in[i]); args.push_back(&ptrs[(size_t)i]); }
   for (int o = 0; o < n_out; ++o) { optrs[(size_t)o] = data_ptr(res[(size_t)o]); args.push_back(&optrs[(size_t)o]); }
-  int64_t work = all_simple ? (n + vec - 1) / vec : n;
+  int64_t work = all_simple ? (n + vec - 1) / vec : n / gvec;
   unsigned grid = grid_for(work, 256, ctx->num_cu * 16);
   hipError_t e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
   if (e != hipSuccess) { release_all(); return check_hip(ctx, e, "fused_map launch"); }

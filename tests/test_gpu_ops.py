@@ -631,6 +631,43 @@ def eval_program_eagerly(ctx, inputs, prog, out_slots):
     return [slots[s] for s in out_slots]
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_fused_map_groups_of_the_innermost_dim(gpu, dt):
+    """Large strided programs take 16 bytes of the innermost dim per lane; inputs that
+    run along it (aligned or not), stand still along it, or cross it are all read
+    correctly: against numpy, to the tolerance of the dtype."""
+    O2 = capi.OP2
+    sh = (96, 81, 72)
+    a = rnd(sh, dt)
+    b = rnd(sh[:2], dt)
+    c = rnd((sh[2], sh[0], sh[1]), dt)
+    d = rnd((sh[0], sh[1], sh[2] + 2), dt)
+    m = rnd(sh, np.int32)
+    ins = [gpu.upload(a),
+           gpu.upload(b).replicate([sh[2]]).transpose([1, 2, 0]),
+           gpu.upload(c).transpose([1, 2, 0]),
+           gpu.upload(d).slice(2, 1, sh[2]),
+           gpu.upload(m).reverse(2)]
+    prog = [(1, O2["mul"], 0, 0, 1, 0),            # 5: a * b
+            (1, O2["add"], 0, 5, 2, 0),            # 6: + c
+            (1, O2["sub"], 0, 6, 3, 0),            # 7: - d
+            (4, 0, capi.F64 if dt == np.float64 else capi.F32, 4, 0, 0),   # 8: m as a float
+            (2, capi.CMP["leq"], 0, 8, 7, 0),      # 9: m <= (..)
+            (3, 0, 0, 9, 7, 1)]                    # 10: select
+    got = [o.numpy() for o in gpu.fused_map(ins, prog, [7, 9, 10])]
+    t = a * b[:, :, None] + np.transpose(c, (1, 2, 0)) - d[:, :, 1:-1]
+    mf = m[:, :, ::-1].astype(dt)
+    want = [t, mf <= t, np.where(mf <= t, t, np.broadcast_to(b[:, :, None], sh))]
+    tol = TOL[np.dtype(dt)]
+    assert np.max(np.abs(got[0] - want[0])) <= tol * np.max(np.abs(want[0]))
+    # comparisons may differ where rounding moves the value across m
+    close_call = np.abs(mf - t) <= 4 * tol * np.abs(t)
+    assert np.array_equal(got[1] | close_call, want[1] | close_call)
+    sel = np.where(got[1], got[0], np.broadcast_to(b[:, :, None], sh))
+    assert np.array_equal(got[2], sel)
+
+
 @pytest.mark.parametrize("dt", [np.float64, np.float32])
 def test_fused_map_equals_the_single_operations(gpu, oracle, dt):
     tol = TOL[np.dtype(dt)]
@@ -661,7 +698,7 @@ def test_fused_map_equals_the_single_operations(gpu, oracle, dt):
     ]
     outs = [14, 17, 20, 21, 22, 23, 24][:6]
     # the last two are large enough for the kernels compiled with their shapes and strides
-    for shape, views in [((1031,), False), ((37, 29), False), ((6, 5, 7), True), ((601, 701), False), ((96, 81, 70), True)]:
+    for shape, views in [((1031,), False), ((37, 29), False), ((6, 5, 7), True), ((601, 701), False), ((96, 81, 72), True)]:
         data = [rnd(shape, dt) + dt(2.5) for _ in range(3)]
         res = []
         for ctx in (gpu, oracle):
