@@ -63,6 +63,24 @@ def scatter1(t):
     return t.sscatter(2, (2,), lambda i1, i2: [(i2 + 2 * i1).minH(1)])
 
 
+def scatterNested2(t):
+    inner = t.sscatter(1, (2, 3, 4), lambda k1: [k1.minH(1), k1.minH(2), k1.minH(3)])
+    return inner.sscatter(4, (2, 3), lambda i1, i2, _i3, i4: [(i1 + i2).minH(1), (i4 + i1).minH(2)])
+
+
+def scatter2(t):
+    return t.sscatter(2, (2, 3), lambda i1, i2: [(i1 + i2 + i1 + i2).minH(1), i1.minH(2)])
+
+
+def scatterNested12(t):
+    inner = t.sscatter(2, (2, 3, 4), lambda k1, k2: [k1.minH(1), (k2 + k1).minH(2), k1.minH(3)])
+    return inner.sscatter(2, (2,), lambda i1, _i2: [(i1 + i1).minH(1)])
+
+
+def scatter12(t):
+    return t.sscatter(2, (2, 4), lambda i1, k3: [(i1 + i1 + i1 + k3).minH(1), i1.minH(3)])
+
+
 def build_if(host, f, k=5):
     """rbuild1 k (\\i -> ifH (i >. 2) (f t) (t ! [i]))"""
     return lambda t: host.sbuild1(k, lambda i: f(t) if i > 2 else t.sindex([i]))
@@ -88,6 +106,9 @@ def programs(host):
         "gatherNestedBuild2": build_scaled(host, gatherNested2, [7, 2]),
         "gatherReshapeBuild22": build_scaled(host, gatherReshape22, [6, 2]),
         "gatherBuild12": build12(host, gather12),
+        "scatterNested2": scatterNested2, "scatter2": scatter2, "scatterNested12": scatterNested12, "scatter12": scatter12,
+        "scatterNestedBuild2": build_scaled(host, scatterNested2, [7, 2]), "scatterBuild2": build_scaled(host, scatter2, [7, 2]),
+        "scatterNestedBuild12": build12(host, scatterNested12), "scatterBuild12": build12(host, scatter12),
     }
 
 
