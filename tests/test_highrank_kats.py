@@ -62,6 +62,29 @@ def check_all(host):
     assert np.allclose(g.ravel(), KATS["testFooBuildOut"]["expected"], rtol=0, atol=1e-10)
 
 
+RELU_INPUT = [1.1, -2.2, 0, 4.4, 5.5, 6.6, 7.7, 8.8, -9.9, -10, 11, 12]          # [3, 4]
+RELU_MASK = [1.0, 0.0, 0.0, 1.0, 1.0, 1.0, 1.0, 1.0, 0.0, 0.0, 1.0, 1.0]
+
+
+def relu_kats(host):
+    """test/simplified/TestAdaptorSimplified.hs: testReluSimpler (:1247-1251), testReluMax
+    (:1408-1412) -- the derivative at 0 is 0 for both forms -- and testReluSimpler3 /
+    testReluMax3 (:1300-1308, :1451-1459): relu (t * replicate r) at r = 7."""
+    W = pkg.workloads
+    x = np.array(RELU_INPUT).reshape(3, 4)
+    relu_max = lambda v: host.srepl(v.shape, 0.0).op2("max", v)         # rmap0N (maxH 0)
+    for relu in (W.reluS, relu_max):
+        host.tape_reset()
+        t = host.param(x).as_input()
+        g = host.grad(relu(t).ssum0(), [t])[0].numpy()
+        assert np.allclose(g.ravel(), RELU_MASK, rtol=0, atol=1e-10)
+        host.tape_reset()
+        t, r = host.param(x).as_input(), host.param(np.array(7.0)).as_input()
+        gt, gr = [a.numpy() for a in host.grad(relu(t * r.sreplicate(4).sreplicate(3)).ssum0(), [t, r])]
+        assert np.allclose(gt.ravel(), 7.0 * np.array(RELU_MASK), rtol=0, atol=1e-10)
+        assert abs(float(gr) - 57.1) <= 1e-10
+
+
 def conv_kats(host):
     W = pkg.workloads
     t128 = np.array(KATS["t128"]["values"])
@@ -88,6 +111,7 @@ def test_highrank_kats_on_checker():
     host = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
     check_all(host)
     conv_kats(host)
+    relu_kats(host)
 
 
 @pytest.mark.gpu
@@ -95,3 +119,4 @@ def test_highrank_kats_on_device():
     host = H.Host()
     check_all(host)
     conv_kats(host)
+    relu_kats(host)
