@@ -132,13 +132,37 @@ def check_all(host):
     assert np.array_equal(gatherNested1(v).numpy(), np.array([vals[0, 0], vals[2, 1]]))
 
 
+def overleaf_and_piecewise(host):
+    """test/simplified/TestAdaptorSimplified.hs: overleaf v = rsum (rbuild [50] (\\[i] -> v ! [i `remH` width v]))
+    (:503-517: positions 0..21 are read twice, 22..27 once; one position read 50 times) and the
+    piecewise linear functions through ifH on the argument (:462-468, :482-488)."""
+    def overleaf(v):
+        return v.sgather((50,), lambda i: [i.remH(v.shape[0])]).ssum0()
+    for x, want in [(np.arange(28.0), [2.0] * 22 + [1.0] * 6), (np.array([27.0]), [50.0])]:
+        host.tape_reset()
+        t = host.param(x).as_input()
+        g = host.grad(overleaf(t), [t])[0].numpy()
+        assert np.allclose(g, want, rtol=0, atol=1e-10)
+    two, five = host.srepl([], 2.0), host.srepl([], 5.0)
+    for x0, f, want in [(42.0, lambda x: (x * 0.0).lt(x).select(two * x, five * x), 2.0),
+                        (-42.0, lambda x: (x * 0.0).lt(x).select(two, five) * x, 5.0)]:
+        host.tape_reset()
+        t = host.param(np.array(x0)).as_input()
+        g = host.grad(f(t), [t])[0].numpy()
+        assert abs(float(g) - want) <= 1e-10
+
+
 def test_reference_kats_on_checker():
-    check_all(H.Host(capi.Lib(entry.ORACLE_LIB, "horc_")))
+    host = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    check_all(host)
+    overleaf_and_piecewise(host)
 
 
 @pytest.mark.gpu
 def test_reference_kats_on_device():
-    check_all(H.Host())
+    host = H.Host()
+    check_all(host)
+    overleaf_and_piecewise(host)
 
 
 def conv_vjp_constants(host):
