@@ -708,7 +708,7 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   const int vec = (int)(16 / widest);
   const int64_t n = nelem(a0);
   hgpu_array* o = nullptr;
-  int rc = new_zeros(ctx, odt, 0, nullptr, &o);
+  int rc = n == 0 ? new_zeros(ctx, odt, 0, nullptr, &o) : new_dense(ctx, odt, 0, nullptr, &o);   // the last launch writes it
   if (rc) return rc;
   if (n == 0) { *out = o; return HGPU_OK; }
   const bool fp = dtype_is_float(odt);

@@ -244,7 +244,7 @@ int hh_tstranspose(hh_ctx* c, hh_val* t, int n, const int* perm, hh_val** out) {
 }
 int hh_tsreshape(hh_ctx* c, hh_val* t, int rank, const int64_t* shape, hh_val** out) { HH_OP(d_tsreshape(c->tape, t->d, mk(rank, shape))); }
 int hh_tsindex(hh_ctx* c, hh_val* t, int n, const int64_t* ix, hh_val** out) { HH_OP(d_tsindex(c->tape, t->d, mk(n, ix))); }
-int hh_tsargminmax(hh_ctx* c, hh_val* t, int want_max, hh_val** out) { HH_OP(d_const(argminmax_last(t->d.primal, want_max != 0))); }
+int hh_tsargminmax(hh_ctx* c, hh_val* t, int want_max, hh_val** out) { HH_OP(d_const(want_max ? tsargMax(t->d.primal) : tsargMin(t->d.primal))); }
 int hh_tsiota(hh_ctx* c, int64_t n, int dtype, hh_val** out) { HH_OP(d_const(tsiota(&c->be, n, dtype))); }
 
 #define HH_IX(body) return guarded(c, [&] { *out = boxi(body); })

@@ -91,6 +91,10 @@ struct ArrHolder {
   std::shared_ptr<ArrHolder> fc;
   int esize = 0;          // pending nodes beneath, to bound program size
   Shape eshape;
+  // The result of tsargMin / tsargMax over the last dim remembers its source and
+  // the extremal values the same pass produced: `sindex0 t [kargMin t]` (the
+  // minimum of the reference's soft-max loss) is then those values, not a gather.
+  std::shared_ptr<ArrHolder> arg_src, arg_values;
   ArrHolder(Backend* b, hgpu_array* a) : be(b), h(a) {}
   ~ArrHolder() { if (h) be->api->release(h); }
   ArrHolder(const ArrHolder&) = delete;

@@ -810,8 +810,21 @@ T tsoneHot(const T& v, const Shape& ix, const Shape& shp) { return onehot(v, ix,
 T tsfloor(const T& t, int dtype) { return convert(t, dtype, HGPU_CONV_FLOOR); }            // OpsConcrete.hs:455
 T tsfromIntegral(const T& t, int dtype) { return convert(t, dtype, HGPU_CONV_CAST); }      // OpsConcrete.hs:456
 T tscast(const T& t, int dtype) { return convert(t, dtype, HGPU_CONV_CAST); }              // OpsConcrete.hs:518
-T tsargMin(const T& t) { return argminmax_last(t, false); }                    // OpsConcrete.hs:533
-T tsargMax(const T& t) { return argminmax_last(t, true); }                     // OpsConcrete.hs:534
+static T arg_with_values(const T& t, bool want_max) {
+  Backend* be = t.be();
+  const hgpu_api* api = be->api;
+  if (be->fuse && t.rank() >= 1 && api->struct_size >= offsetof(hgpu_api, extremum_last) + sizeof(api->extremum_last) && api->extremum_last) {
+    hgpu_array *vals = nullptr, *idx = nullptr;
+    be->check(api->extremum_last(be->ctx, t.h(), want_max ? 1 : 0, &vals, &idx));
+    T r(be, idx);
+    r.holder()->arg_src = t.holder();
+    r.holder()->arg_values = T(be, vals).holder();
+    return r;
+  }
+  return argminmax_last(t, want_max);
+}
+T tsargMin(const T& t) { return arg_with_values(t, false); }                   // OpsConcrete.hs:533
+T tsargMax(const T& t) { return arg_with_values(t, true); }                    // OpsConcrete.hs:534
 T tsiota(Backend* be, int64_t n, int dtype) { return iota(be, n, dtype); }     // OpsConcrete.hs:535
 
 // ----------------------------------------------------- lane-batched scalars
@@ -845,6 +858,10 @@ Ix ix_lift(const Shape& shm, const T& scalar) {
   x.shm = shm;
   x.dtype = scalar.dtype();
   x.arr = broadcast_scalar(scalar, shm);
+  if (shm.empty() && scalar.rank() == 0 && scalar.holder()->arg_src) {   // kargMin t of a rank-1 t, used once
+    x.arg_of = scalar.holder()->arg_src;
+    x.arg_vals = T(scalar.holder()->arg_values);
+  }
   return x;
 }
 

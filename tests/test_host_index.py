@@ -263,3 +263,28 @@ def test_pooling_adjoint_stays_pending_gpu(host_gpu, host_cpu):
         host.tape_reset()
     for got, want in zip(res[0], res[1]):
         assert np.allclose(got, want, rtol=1e-12, atol=1e-13)
+
+
+def value_at_own_extremum(host):
+    """`sindex0 t [kargMin t]` on a flat tensor (sminimum of the reference's soft-max loss,
+    CommonShapedOps.hs:33-44) equals the minimum, with ties and with the index reused on
+    another tensor (where it has to be a real gather)."""
+    for dt in (np.float64, np.float32):
+        v = RNG.uniform(-3, 3, 1000).astype(dt)
+        v[[17, 400]] = v.min() - 1          # a tie: the first position counts
+        w = RNG.uniform(-3, 3, 1000).astype(dt)
+        t, o = host.concrete(v), host.concrete(w)
+        for arg_of, pick in ((lambda x: x.sargMin(), np.argmin), (lambda x: x.sargMax(), np.argmax)):
+            arg = arg_of(t)
+            assert int(arg.numpy()) == int(pick(v))
+            assert t.sgather((), lambda: [arg.lift(())]).numpy() == v[pick(v)]
+            assert o.sgather((), lambda: [arg.lift(())]).numpy() == w[pick(v)]
+
+
+def test_value_at_own_extremum_cpu(host_cpu):
+    value_at_own_extremum(host_cpu)
+
+
+@pytest.mark.gpu
+def test_value_at_own_extremum_gpu(host_gpu):
+    value_at_own_extremum(host_gpu)
