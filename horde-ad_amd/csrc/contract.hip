@@ -314,7 +314,19 @@ __global__ void __launch_bounds__(1024) k_argminmax_block(Dims keep, int64_t L, 
   bool have = t < L;
   T best = have ? p[(int64_t)t * sl] : T(0);
   int64_t bi = t;
-  for (int64_t j = t + 1024; j < L; j += 1024) {
+  // eight loads in flight; the comparisons keep the order of the positions
+  int64_t j = (int64_t)t + 1024;
+  for (; j + 7 * 1024 < L; j += 8 * 1024) {
+    T x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) x[u] = p[(j + u * 1024) * sl];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      bool better = want_max ? (x[u] > best) : (x[u] < best);
+      if (better) { best = x[u]; bi = j + u * 1024; }
+    }
+  }
+  for (; j < L; j += 1024) {
     T x = p[j * sl];
     bool better = want_max ? (x > best) : (x < best);
     if (better) { best = x; bi = j; }
