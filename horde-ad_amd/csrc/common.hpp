@@ -146,6 +146,15 @@ inline unsigned grid_for(int64_t n, int block, int max_blocks) {
   return (unsigned)g;
 }
 
+// Compiles `src` for gfx950 at run time (runtime.hip) and hands back the code
+// object.  Code objects are kept on disk between processes, keyed by the
+// source, the options and the compiler's version: a kernel that was compiled
+// once (a second or so for the larger ones) is read back in under a
+// millisecond.  The directory is $HORDEAD_GPU_CACHE, else
+// $XDG_CACHE_HOME/hordead_gpu, else $HOME/.cache/hordead_gpu; HORDEAD_GPU_CACHE=off
+// (or an unwritable directory) means no files.  `what` names the caller in errors.
+int rtc_compile(hgpu_ctx* ctx, const std::string& src, const char* what, std::vector<char>* code);
+
 // Zeroes `bytes` bytes (rounded up to 16) with a fill kernel (ewise.hip).
 int zero_fill(hgpu_ctx* ctx, void* p, size_t bytes);
 // Strided copy between two views of equal shape (ewise.hip).

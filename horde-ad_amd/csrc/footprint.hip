@@ -51,25 +51,9 @@ std::map<std::string, Compiled>& cache_of(hgpu_ctx* ctx) {
 }
 
 int compile(hgpu_ctx* ctx, const std::string& src, const std::string& kname, Compiled* out) {
-  hiprtcProgram prog;
-  if (hiprtcCreateProgram(&prog, src.c_str(), "footprint_gemm.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
-    return fail(ctx, HGPU_ERR_DEVICE, "hiprtcCreateProgram failed");
-  const char* opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-  hiprtcResult r = hiprtcCompileProgram(prog, 7, opts);
-  if (r != HIPRTC_SUCCESS) r = hiprtcCompileProgram(prog, 3, opts);
-  if (r != HIPRTC_SUCCESS) {
-    size_t n = 0;
-    hiprtcGetProgramLogSize(prog, &n);
-    std::string log(n, '\0');
-    if (n) hiprtcGetProgramLog(prog, &log[0]);
-    hiprtcDestroyProgram(&prog);
-    return fail(ctx, HGPU_ERR_DEVICE, "hiprtc (footprint gemm): %s: %.600s", hiprtcGetErrorString(r), log.c_str());
-  }
-  size_t n = 0;
-  hiprtcGetCodeSize(prog, &n);
-  std::vector<char> code(n);
-  hiprtcGetCode(prog, code.data());
-  hiprtcDestroyProgram(&prog);
+  std::vector<char> code;
+  int rc = rtc_compile(ctx, src, "footprint gemm", &code);
+  if (rc) return rc;
   hipError_t e = hipModuleLoadData(&out->mod, code.data());
   if (e != hipSuccess) return check_hip(ctx, e, "hipModuleLoadData");
   e = hipModuleGetFunction(&out->fn, out->mod, kname.c_str());

@@ -4,6 +4,16 @@
 // (src/HordeAd/Core/OpsConcrete.hs:243-246,641-652): no element is touched.
 #include "common.hpp"
 
+#include <hip/hiprtc.h>
+
+#include <sys/stat.h>
+#include <sys/types.h>
+#include <unistd.h>
+
+#include <cerrno>
+#include <cstdlib>
+#include <fstream>
+
 namespace hg {
 
 int fail(hgpu_ctx* ctx, int code, const char* fmt, ...) {
@@ -738,3 +748,94 @@ int hgpu_as_strided(hgpu_ctx* ctx, const hgpu_array* a, int rank, const int64_t*
 }
 
 }  // extern "C"
+
+// ---- run-time compilation with a cache on disk -----------------------------
+
+namespace hg {
+namespace {
+
+uint64_t fnv1a(const std::string& s, uint64_t h) {
+  for (unsigned char c : s) { h ^= c; h *= 1099511628211ull; }
+  return h;
+}
+
+// "" when there is to be no cache
+std::string rtc_cache_dir() {
+  std::string dir;
+  if (const char* e = getenv("HORDEAD_GPU_CACHE")) {
+    dir = e;
+    if (dir.empty() || dir == "off" || dir == "0") return "";
+  } else if (const char* x = getenv("XDG_CACHE_HOME")) {
+    if (*x) dir = std::string(x) + "/hordead_gpu";
+  }
+  if (dir.empty()) {
+    const char* home = getenv("HOME");
+    if (!home || !*home) return "";
+    dir = std::string(home) + "/.cache";
+    mkdir(dir.c_str(), 0700);
+    dir += "/hordead_gpu";
+  }
+  if (mkdir(dir.c_str(), 0700) != 0 && errno != EEXIST) return "";
+  return dir;
+}
+
+const char* kRtcOpts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+
+}  // namespace
+
+int rtc_compile(hgpu_ctx* ctx, const std::string& src, const char* what, std::vector<char>* code) {
+  // the key: everything the code object depends on
+  int major = 0, minor = 0;
+  hiprtcVersion(&major, &minor);
+  std::string stamp = "hiprtc " + std::to_string(major) + "." + std::to_string(minor);
+  for (const char* o : kRtcOpts) { stamp += " "; stamp += o; }
+  const uint64_t h1 = fnv1a(src, fnv1a(stamp, 14695981039346656037ull)), h2 = fnv1a(stamp, fnv1a(src, 1469598103934665603ull));
+  char name[64];
+  snprintf(name, sizeof name, "%016llx%016llx.co", (unsigned long long)h1, (unsigned long long)h2);
+  const std::string dir = rtc_cache_dir();
+  const std::string path = dir.empty() ? "" : dir + "/" + name;
+  const std::string header = stamp + "\n" + std::to_string(src.size()) + "\n";
+  if (!path.empty()) {
+    std::ifstream f(path, std::ios::binary);
+    if (f) {
+      std::string all((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+      if (all.size() > header.size() && all.compare(0, header.size(), header) == 0) {
+        code->assign(all.begin() + (long)header.size(), all.end());
+        return HGPU_OK;
+      }
+    }
+  }
+  hiprtcProgram prog;
+  if (hiprtcCreateProgram(&prog, src.c_str(), "hordead_gpu_rtc.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+    return fail(ctx, HGPU_ERR_DEVICE, "hiprtcCreateProgram failed");
+  // packed FP32 instructions stay off, as in the ahead-of-time build; a hiprtc
+  // that does not take the feature switch compiles without it
+  hiprtcResult r = hiprtcCompileProgram(prog, 7, kRtcOpts);
+  if (r != HIPRTC_SUCCESS) r = hiprtcCompileProgram(prog, 3, kRtcOpts);
+  if (r != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, &log[0]);
+    hiprtcDestroyProgram(&prog);
+    return fail(ctx, HGPU_ERR_DEVICE, "hiprtc (%s): %s: %.600s", what, hiprtcGetErrorString(r), log.c_str());
+  }
+  size_t n = 0;
+  hiprtcGetCodeSize(prog, &n);
+  code->resize(n);
+  hiprtcGetCode(prog, code->data());
+  hiprtcDestroyProgram(&prog);
+  if (!path.empty()) {   // written under another name first: a reader never sees half a file
+    const std::string tmp = path + "." + std::to_string((long)getpid()) + ".tmp";
+    std::ofstream f(tmp, std::ios::binary | std::ios::trunc);
+    if (f) {
+      f.write(header.data(), (std::streamsize)header.size());
+      f.write(code->data(), (std::streamsize)code->size());
+      f.close();
+      if (!f || rename(tmp.c_str(), path.c_str()) != 0) unlink(tmp.c_str());
+    }
+  }
+  return HGPU_OK;
+}
+
+}  // namespace hg
