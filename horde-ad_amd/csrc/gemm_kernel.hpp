@@ -103,110 +103,182 @@ template <> struct VecOf<float, 1> { using type = float; };
 template <> struct VecOf<double, 2> { using type = double __attribute__((ext_vector_type(2), aligned(8))); };
 template <> struct VecOf<float, 4> { using type = float __attribute__((ext_vector_type(4), aligned(4))); };
 
-// K offset of linear index k for one operand.  Several K dims: a table written
-// by k_koff.  A single K dim: a multiplication.
-//   KOff  (staged kernel): tab == nullptr selects the multiplication;
-//   direct kernel: branch-free tab[k & kmask] + k * stride, with kmask 0 on a
-//   table of zeros when the stride does the work.
+// K offset of linear index k for one operand: tab[k & kmask] + k * stride.
+// Several K dims: a table written by k_koff, kmask all ones, stride 0.  A single
+// K dim: kmask 0 on a table of zeros and the dim's stride.
 struct KOff {
   const int64_t* __restrict__ tab;
-  int64_t stride;   // used when tab == nullptr
-  __device__ __forceinline__ int64_t at(int64_t k) const { return tab ? tab[k] : k * stride; }
+  int64_t stride;
 };
 
 // Stages one operand tile (R rows x BK) from global memory into LDS.  A slot is
-// V consecutive elements along the direction the lanes run.  K offsets that
-// have to be fetched per lane are fetched one K-step ahead of their use, so a
-// tile's loads never wait on a table lookup.
-template <typename T, int R, int V>
+// V consecutive elements along the direction the lanes run (along k when kc,
+// else along the rows); a lane owns NL slots.
+//
+// The loads of a tile are issued together, unconditionally (rows and k past the
+// end are clamped to the last valid slot and zeroed when the tile is stored),
+// and nothing between issuing them and storing them to LDS waits on memory: the
+// MFMAs of the current tile run under the whole latency.  A load that sits in a
+// branch, or whose value is consumed before the MFMAs, makes the compiler wait
+// for every load in flight at that point, which serialises the tile's loads.
+// For the same reason the K table (TAB) is read one tile ahead and its entries
+// are first used when the next tile's addresses are formed; the kernels choose
+// TAB once, outside the K loop, so that the loop itself has no table branch.
+template <typename T, int R, int V, bool TAB>
 struct Stager {
   static constexpr int NL = R * BK / NT / V;
   static_assert(NL >= 1, "tile too small for 256 threads");
   using Vec = typename VecOf<T, V>::type;
   static constexpr int ML = R / V;        // lanes per k-row when running along rows
   static constexpr int KL = BK / V;       // lanes per row when running along k
-  static constexpr bool kUniformK = (ML % 64 == 0);   // along rows: a wavefront shares one k
-  static constexpr int NKV = kUniformK ? 1 : NL;
 
-  int rl[NL], kl[NL];
-  const T* rowp[NL];
-  Vec reg[NL];
-  int kc;
-  int64_t kv[NKV];    // per-lane K offsets of the next tile to load
+  // slot i sits at row rl0 + i * drl, k kl0 + i * dkl of the tile
+  int rl0, kl0, drl, dkl;
+  int dk;
+  int64_t klast;                  // last k a slot may start at
+  // Where slot i of the next tile to issue starts.  Without a table: the
+  // address itself, moved on by one K-step at a time.  With a table: the row's
+  // address and, apart, the table entry of the slot's k.
+  const T* ptr[NL];
+  int64_t tv[TAB ? NL : 1];
+  int64_t kstep;                  // BK * stride
 
-  __device__ __forceinline__ void fetch_kv(const KOff& ko, int64_t k0, int64_t K) {
-    if (kc) {
-      int64_t k = k0 + kl[0];
-      kv[0] = ko.at(k < K ? k : K - 1);
-    } else if constexpr (!kUniformK) {
-#pragma unroll
-      for (int i = 0; i < NL; ++i) {
-        int64_t k = k0 + kl[i];
-        kv[i] = ko.at(k < K ? k : K - 1);
-      }
-    }
+  __device__ __forceinline__ int rl(int i) const { return rl0 + i * drl; }
+  __device__ __forceinline__ int kl(int i) const { return kl0 + i * dkl; }
+  __device__ __forceinline__ int64_t clamp_k(int64_t k) const {
+    k = k < klast ? k : klast;
+    return k > 0 ? k : 0;
   }
 
   // which: 0 = operand A (offsets sa), 1 = operand B (offsets sb)
-  __device__ __forceinline__ void init(int t, int kc_, int which, const T* base, const Group& g, int64_t r0, int64_t rows,
+  __device__ __forceinline__ void init(int t, int kc, int which, const T* base, const Group& g, int64_t r0, int64_t rows,
                                        const KOff& ko, int64_t kbeg, int64_t K) {
-    kc = kc_;
+    dk = kc ? 1 : 0;
+    klast = K - (kc ? V : 1);
+    kstep = (int64_t)BK * ko.stride;
+    if (kc) { rl0 = t / KL; drl = NT / KL; kl0 = (t % KL) * V; dkl = 0; }
+    else { rl0 = (t % ML) * V; drl = 0; kl0 = t / ML; dkl = NT / ML; }
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      if (kc) { rl[i] = t / KL + (NT / KL) * i; kl[i] = (t % KL) * V; }
-      else { rl[i] = (t % ML) * V; kl[i] = t / ML + (NT / ML) * i; }
       if (kc || i == 0) {
-        int64_t r = r0 + rl[i];
+        int64_t r = r0 + rl(i);
         if (r >= rows) r = rows - (kc ? 1 : V);   // clamp: the values are never stored
         int64_t oa, ob, oc;
         group_off(g, r, &oa, &ob, &oc);
-        rowp[i] = base + (which == 0 ? oa : ob);
+        ptr[i] = base + (which == 0 ? oa : ob);
       } else {
-        rowp[i] = rowp[0];
+        ptr[i] = ptr[0];
       }
     }
-#pragma unroll
-    for (int i = 0; i < NKV; ++i) kv[i] = 0;
-    fetch_kv(ko, kbeg, K);
-  }
-
-  __device__ __forceinline__ void load(int64_t k0, int64_t kend, const KOff& ko, int64_t K) {
-    if (kc) {
-      const bool ok = k0 + kl[0] < kend;
-#pragma unroll
-      for (int i = 0; i < NL; ++i) reg[i] = ok ? *reinterpret_cast<const Vec*>(rowp[i] + kv[0]) : Vec{};
-    } else {
-#pragma unroll
-      for (int i = 0; i < NL; ++i) {
-        if constexpr (kUniformK) {
-          int64_t k = k0 + __builtin_amdgcn_readfirstlane(kl[i]);
-          if (k < kend) reg[i] = *reinterpret_cast<const Vec*>(rowp[0] + ko.at(k));
-          else reg[i] = Vec{};
-        } else {
-          reg[i] = (k0 + kl[i] < kend) ? *reinterpret_cast<const Vec*>(rowp[0] + kv[i]) : Vec{};
-        }
-      }
-    }
-    fetch_kv(ko, k0 + BK, K);
-  }
-
-  __device__ __forceinline__ void store(T (*S)[R + 1]) const {
-    const int dk = kc ? 1 : 0, dr = 1 - dk;
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      if constexpr (V == 1) S[kl[i]][rl[i]] = reg[i];
+      const int64_t k = clamp_k(kbeg + kl(i));
+      if constexpr (TAB) tv[i] = ko.tab[k];
+      else ptr[i] += k * ko.stride;
+    }
+  }
+
+  // the slots move on to the tile that starts at k0
+  __device__ __forceinline__ void advance(const KOff& ko, int64_t k0) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int64_t k = k0 + kl(i);
+      if constexpr (TAB) tv[i] = ko.tab[clamp_k(k)];
+      else ptr[i] += k <= klast ? kstep : 0;      // a slot past the end stays where it is: still readable, never stored
+    }
+  }
+
+  __device__ __forceinline__ void issue(Vec* __restrict__ r) const {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      if constexpr (TAB) r[i] = *reinterpret_cast<const Vec*>(ptr[i] + tv[i]);
+      else r[i] = *reinterpret_cast<const Vec*>(ptr[i]);
+    }
+  }
+
+  // r holds the tile that starts at k0
+  __device__ __forceinline__ void store(const Vec* __restrict__ r, int64_t k0, int64_t kend, T (*S)[R + 1]) const {
+    const int dr = 1 - dk;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const bool ok = k0 + kl(i) < kend;
+      if constexpr (V == 1) S[kl(i)][rl(i)] = ok ? r[i] : T(0);
       else {
 #pragma unroll
-        for (int j = 0; j < V; ++j) S[kl[i] + j * dk][rl[i] + j * dr] = reg[i][j];
+        for (int j = 0; j < V; ++j) S[kl(i) + j * dk][rl(i) + j * dr] = ok ? r[i][j] : T(0);
       }
     }
   }
 };
 
+// One block's K loop over [kbeg, kend) of one product: accumulates into acc.
+// Ends with a barrier, so the LDS tiles are free when it returns.
+template <typename X, int WGM, int WGN, int TM, int TN, int VA, int VB, int NBUF, bool TAB>
+__device__ __forceinline__ void k_loop(const GemmParams& p, const typename X::T* A, const typename X::T* B, const int64_t* koffA,
+                                       const int64_t* koffB, int64_t m0, int64_t n0, int64_t kbeg, int64_t kend,
+                                       typename X::T (*As)[BK][WGM * TM * 16 + 1], typename X::T (*Bs)[BK][WGN * TN * 16 + 1],
+                                       typename X::Acc (*acc)[TN * 16 / X::NBW]) {
+  using T = typename X::T;
+  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
+  constexpr int TNB = TN * 16 / X::NBW;
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+  using SA = Stager<T, BM, VA, TAB>;
+  using SB = Stager<T, BN, VB, TAB>;
+  SA sa;
+  SB sb;
+  typename SA::Vec ra[SA::NL];
+  typename SB::Vec rb[SB::NL];
+  const KOff koa{koffA, p.ksa}, kob{koffB, p.ksb};
+  sa.init(t, p.a_kc, 0, A, p.m, m0, p.M, koa, kbeg, p.K);
+  sb.init(t, p.b_kc, 1, B, p.n, n0, p.N, kob, kbeg, p.K);
+  if (kbeg < kend) {
+    sa.issue(ra);
+    sb.issue(rb);
+    sa.advance(koa, kbeg + BK);
+    sb.advance(kob, kbeg + BK);
+    sa.store(ra, kbeg, kend, As[0]);
+    sb.store(rb, kbeg, kend, Bs[0]);
+  }
+  __syncthreads();
+  int cur = 0;
+  for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
+    const bool more = k0 + BK < kend;
+    if (more) {
+      sa.issue(ra);
+      sb.issue(rb);
+      sa.advance(koa, k0 + 2 * BK);
+      sb.advance(kob, k0 + 2 * BK);
+    }
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 4) {
+      const int kr = kk + (lane >> 4);
+      T fa[TM], fb[TNB];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[i] = As[cur][kr][(wm * TM + i) * 16 + (lane & 15)];
+#pragma unroll
+      for (int j = 0; j < TNB; ++j) fb[j] = Bs[cur][kr][wn * TN * 16 + j * X::NBW + X::bcol(lane)];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TNB; ++j) acc[i][j] = X::run(fa[i], fb[j], acc[i][j]);
+    }
+    if constexpr (NBUF == 1) __syncthreads();   // every wavefront is done reading the tile
+    const int nxt = NBUF == 2 ? cur ^ 1 : 0;
+    if (more) {
+      sa.store(ra, k0 + BK, kend, As[nxt]);
+      sb.store(rb, k0 + BK, kend, Bs[nxt]);
+    }
+    __syncthreads();
+    cur = nxt;
+  }
+}
+
 // Block tile BM x BN = (WGM * TM * 16) x (WGN * TN * 16).  NBUF LDS buffers.
 // Skinny tiles keep few accumulators: ask for three wavefronts per SIMD there
 // (the loads of one tile are only hidden by the MFMAs of other blocks).
-constexpr int waves_wanted(int tm, int tn, int esize) { return tm * tn * esize <= 32 ? 3 : 1; }
+constexpr int waves_wanted(int tm, int tn, int esize) { return tm * tn * esize <= 32 ? 2 : 1; }
 
 template <typename X, int WGM, int WGN, int TM, int TN, int VA, int VB, int NBUF>
 __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_wanted(TM, TN, (int)sizeof(typename X::T)), 8))) k_gemm(GemmParams p, const typename X::T* __restrict__ A, const typename X::T* __restrict__ B,
@@ -247,54 +319,14 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
   int64_t kend = kbeg + p.kchunk;
   if (kend > p.K) kend = p.K;
 
-  Stager<T, BM, VA> sa;
-  Stager<T, BN, VB> sb;
-  const KOff koa{p.kmask ? koffA : nullptr, p.ksa}, kob{p.kmask ? koffB : nullptr, p.ksb};
-  sa.init(t, p.a_kc, 0, A + bta, p.m, m0, p.M, koa, kbeg, p.K);
-  sb.init(t, p.b_kc, 1, B + btb, p.n, n0, p.N, kob, kbeg, p.K);
-
   Acc acc[TM][TNB];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TNB; ++j) acc[i][j] = X::zero();
 
-  if (kbeg < kend) {
-    sa.load(kbeg, kend, koa, p.K);
-    sb.load(kbeg, kend, kob, p.K);
-    sa.store(As[0]);
-    sb.store(Bs[0]);
-  }
-  __syncthreads();
-  int cur = 0;
-  for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
-    const bool more = k0 + BK < kend;
-    if (more) {
-      sa.load(k0 + BK, kend, koa, p.K);
-      sb.load(k0 + BK, kend, kob, p.K);
-    }
-#pragma unroll
-    for (int kk = 0; kk < BK; kk += 4) {
-      const int kr = kk + (lane >> 4);
-      T fa[TM], fb[TNB];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) fa[i] = As[cur][kr][(wm * TM + i) * 16 + (lane & 15)];
-#pragma unroll
-      for (int j = 0; j < TNB; ++j) fb[j] = Bs[cur][kr][wn * TN * 16 + j * X::NBW + X::bcol(lane)];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TNB; ++j) acc[i][j] = X::run(fa[i], fb[j], acc[i][j]);
-    }
-    if constexpr (NBUF == 1) __syncthreads();   // every wavefront is done reading the tile
-    const int nxt = NBUF == 2 ? cur ^ 1 : 0;
-    if (more) {
-      sa.store(As[nxt]);
-      sb.store(Bs[nxt]);
-    }
-    __syncthreads();
-    cur = nxt;
-  }
+  if (p.kmask) k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, true>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
+  else k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, false>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
 
   T* Cout = C + btc + (int64_t)s * p.c_split_stride;
   if constexpr (BN == 16 && BM >= 64) {
@@ -400,50 +432,11 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
 #pragma unroll
     for (int j = 0; j < TNB; ++j) acc[i][j] = X::zero();
 
-  const KOff koa{p.kmask ? koffA : nullptr, p.ksa}, kob{p.kmask ? koffB : nullptr, p.ksb};
   for (int term = term0; term < term0 + nterm; ++term) {
     A = (const T*)p.a_term[term];
     B = (const T*)p.b_term[term];
-    Stager<T, BM, VA> sa;
-    Stager<T, BN, VB> sb;
-    sa.init(t, p.a_kc, 0, A + bta, p.m, m0, p.M, koa, kbeg, p.K);
-    sb.init(t, p.b_kc, 1, B + btb, p.n, n0, p.N, kob, kbeg, p.K);
-    if (kbeg < kend) {
-      sa.load(kbeg, kend, koa, p.K);
-      sb.load(kbeg, kend, kob, p.K);
-      sa.store(As[0]);
-      sb.store(Bs[0]);
-    }
-    __syncthreads();
-    int cur = 0;
-    for (int64_t k0 = kbeg; k0 < kend; k0 += BK) {
-      const bool more = k0 + BK < kend;
-      if (more) {
-        sa.load(k0 + BK, kend, koa, p.K);
-        sb.load(k0 + BK, kend, kob, p.K);
-      }
-#pragma unroll
-      for (int kk = 0; kk < BK; kk += 4) {
-        const int kr = kk + (lane >> 4);
-        T fa[TM], fb[TNB];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = As[cur][kr][(wm * TM + i) * 16 + (lane & 15)];
-#pragma unroll
-        for (int j = 0; j < TNB; ++j) fb[j] = Bs[cur][kr][wn * TN * 16 + j * X::NBW + X::bcol(lane)];
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TNB; ++j) acc[i][j] = X::run(fa[i], fb[j], acc[i][j]);
-      }
-      if constexpr (NBUF == 1) __syncthreads();   // every wavefront is done reading the tile
-      const int nxt = NBUF == 2 ? cur ^ 1 : 0;
-      if (more) {
-        sa.store(As[nxt]);
-        sb.store(Bs[nxt]);
-      }
-      __syncthreads();
-      cur = nxt;
-    }
+    if (p.kmask) k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, true>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
+    else k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, false>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
   }
 
   T* Cout = C + btc + (int64_t)s * p.c_split_stride;
