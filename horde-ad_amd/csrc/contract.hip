@@ -178,7 +178,36 @@ __global__ void __launch_bounds__(kBlock) k_contract_wave(Dims keep, Dims red, i
     if (Q > 1) { q0 = s * chunk; q1 = q0 + chunk; if (q1 > Q) q1 = Q; }
     else { j0 = s * chunk; j1 = j0 + chunk; if (j1 > Lin) j1 = Lin; }
     A acc = 0;
-    for (int64_t q = q0; q < q1; ++q) {
+    int64_t q = q0;
+    if (Lin <= 1024) {
+      // short inner rows: four outer indices at a time, so that a lane has four
+      // loads per operand in flight although a row gives it only a few elements
+      for (; q + 3 < q1; q += 4) {
+        const TI* pa[4];
+        const TI* pb[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          int64_t ro[2];
+          decompose<2>(red, q + u, ro);
+          pa[u] = a + ko[0] + ro[0];
+          pb[u] = HASB ? b + ko[1] + ro[1] : nullptr;
+        }
+        A c[4] = {0, 0, 0, 0};
+        for (int64_t j = j0 + lane; j < j1; j += 64) {
+          A x[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) x[u] = (A)pa[u][j * sa_in];
+          if (HASB) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] *= (A)pb[u][j * sb_in];
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) c[u] += x[u];
+        }
+        acc += (c[0] + c[1]) + (c[2] + c[3]);
+      }
+    }
+    for (; q < q1; ++q) {
       int64_t ro[2];
       decompose<2>(red, q, ro);
       const TI* pa = a + ko[0] + ro[0];

@@ -316,19 +316,42 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
 
   // j-th staging vector of this thread; the tail repeats the last vector
   auto vidx = [&](int j) -> int { int v = tid + 256 * (j < NLX ? j : j - NLX); int lim = (j < NLX ? XV : YV) - 1; return v < lim ? v : lim; };
-  auto stage = [&](T* dst, i64 ch, int j) {
-    if (j < NLX) reinterpret_cast<Vec<VX>*>(dst)[vidx(j)] = reinterpret_cast<const Vec<VX>*>(X + ch * chx)[vidx(j)];
-    else reinterpret_cast<Vec<VY>*>(dst + LX)[ypos(vidx(j))] = reinterpret_cast<const Vec<VY>*>(Y + ch * chy)[vidx(j)];
-  };
-
+  // The first chunk, and the columns operand of mode 1, go to LDS eight vectors
+  // at a time: eight loads in flight, then eight stores.  Copied one by one,
+  // every vector would wait out its own trip to memory.
+  constexpr int kFill = 8;
   i64 ch = blockIdx.x;
   if (ch < nch) {
 #pragma unroll
-    for (int j = 0; j < NLD; ++j) stage(lds, ch, j);
+    for (int j0 = 0; j0 < NLD; j0 += kFill) {
+      Vec<VX> fx[kFill];
+      Vec<VY> fy[kFill];
+#pragma unroll
+      for (int j = j0; j < j0 + kFill && j < NLD; ++j) {
+        if (j < NLX) fx[j - j0] = reinterpret_cast<const Vec<VX>*>(X + ch * chx)[vidx(j)];
+        else fy[j - j0] = reinterpret_cast<const Vec<VY>*>(Y + ch * chy)[vidx(j)];
+      }
+#pragma unroll
+      for (int j = j0; j < j0 + kFill && j < NLD; ++j) {
+        if (j < NLX) reinterpret_cast<Vec<VX>*>(lds)[vidx(j)] = fx[j - j0];
+        else reinterpret_cast<Vec<VY>*>(lds + LX)[ypos(vidx(j))] = fy[j - j0];
+      }
+    }
   }
   if (MODE == 1) {   // the columns operand does not change with the chunk
-    for (int v = tid; v < YV; v += 256)
-      reinterpret_cast<Vec<VY>*>(lds + NBUFS * BUF)[ypos(v)] = reinterpret_cast<const Vec<VY>*>(Y)[v];
+    for (int v0 = tid; v0 < YV; v0 += 256 * kFill) {
+      Vec<VY> fy[kFill];
+#pragma unroll
+      for (int u = 0; u < kFill; ++u) {
+        const int v = v0 + 256 * u;
+        fy[u] = reinterpret_cast<const Vec<VY>*>(Y)[v < YV ? v : YV - 1];
+      }
+#pragma unroll
+      for (int u = 0; u < kFill; ++u) {
+        const int v = v0 + 256 * u;
+        if (v < YV) reinterpret_cast<Vec<VY>*>(lds + NBUFS * BUF)[ypos(v)] = fy[u];
+      }
+    }
   }
   int cur = 0;
   for (; ch < nch; ch += gridDim.x) {

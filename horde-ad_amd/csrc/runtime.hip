@@ -795,6 +795,16 @@ int rtc_compile(hgpu_ctx* ctx, const std::string& src, const char* what, std::ve
   const std::string dir = rtc_cache_dir();
   const std::string path = dir.empty() ? "" : dir + "/" + name;
   const std::string header = stamp + "\n" + std::to_string(src.size()) + "\n";
+  // HORDEAD_GPU_KEEP_SOURCES=<dir>: the generated sources are written there,
+  // under the names of their code objects, for reading or compiling by hand
+  if (const char* keep = getenv("HORDEAD_GPU_KEEP_SOURCES")) {
+    if (*keep) {
+      std::string sp = std::string(keep) + "/" + name;
+      sp.replace(sp.size() - 3, 3, ".hip");
+      std::ofstream f(sp, std::ios::trunc);
+      if (f) f << "// " << what << "\n" << src;
+    }
+  }
   if (!path.empty()) {
     std::ifstream f(path, std::ios::binary);
     if (f) {
