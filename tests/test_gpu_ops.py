@@ -555,6 +555,41 @@ def test_contract_on_the_matrix_cores(both, gpu, dt):
     assert any(k.startswith("gemm") for k in rep), rep
 
 
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_staged_products_at_the_edges_of_their_tiles(both, dt):
+    """The staged kernel reads whole tiles with clamped addresses and zeroes what
+    lies past the end when it stores to LDS: K and rows that are no multiples
+    of the K step, of the vector width or of the tile, K tables (two K dims that
+    do not merge) with lanes along K, K chunks that end inside a step."""
+    tol = TOL[np.dtype(dt)]
+
+    def nt_views(a, b):      # a [m, ...k], b [n, ...k] -> operands [m, n, ...k]
+        m, n = a.shape[0], b.shape[0]
+        r = len(a.shape) - 1
+        lhs = a.replicate([n]).transpose([1, 0] + list(range(2, 2 + r)))
+        rhs = b.replicate([m])
+        return lhs, rhs
+
+    for (m, n, k) in [(70, 50, 18), (70, 50, 20), (66, 129, 130), (64, 64, 16), (65, 35, 1030), (33, 40, 7), (200, 36, 36)]:
+        a, b = both.upload(rnd((m, k), dt)), both.upload(rnd((n, k), dt))      # lanes along K on both
+        lhs, rhs = nt_views(a, b)
+        assert_same(lhs.contract(rhs, 2), tol, ("NT", m, n, k))
+        at, bt = both.upload(rnd((k, m), dt)).transpose([1, 0]), both.upload(rnd((k, n), dt)).transpose([1, 0])   # lanes along the rows
+        lhs, rhs = nt_views(at, bt)
+        assert_same(lhs.contract(rhs, 2), tol, ("TN", m, n, k))
+    # two K dims that do not merge (the inner one is a window of a longer row): K table, vectors along K
+    for (m, n, k1, k2, k2p) in [(70, 50, 5, 8, 12), (64, 48, 3, 20, 21), (40, 130, 7, 6, 16)]:
+        af, bf = both.upload(rnd((m, k1, k2p), dt)), both.upload(rnd((n, k1, k2p), dt))
+        a = af.as_strided([m, k1, k2], [k1 * k2p, k2p, 1], 0)
+        b = bf.as_strided([n, k1, k2], [k1 * k2p, k2p, 1], k2p - k2)     # ends with the allocation
+        lhs, rhs = nt_views(a, b)
+        assert_same(lhs.contract(rhs, 2), tol, ("table", m, n, k1, k2))
+    # K chunks that end inside a K step, partial sums
+    a, b = both.upload(rnd((64, 20008), dt)), both.upload(rnd((48, 20008), dt))
+    lhs, rhs = nt_views(a, b)
+    assert_same(lhs.contract(rhs, 2), 10 * tol, "split-K, ragged chunks")
+
+
 def conv_views(both, dt, b, ci, h, w, co, kh, kw):
     """The window views of a 'same' convolution: input windows [b, h, w, ci, kh, kw]
     of the zero-extended image, the kernel, and a cotangent of the output."""
