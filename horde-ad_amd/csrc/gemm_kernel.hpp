@@ -142,6 +142,10 @@ struct Stager {
   const T* ptr[NL];
   int64_t tv[TAB ? NL : 1];
   int64_t kstep;                  // BK * stride
+  int64_t kfull;                  // K: a tile that ends at or before it needs no clamping
+  // LDS element offset of slot i's first element in a [BK][R + 1] tile, and the
+  // step from one element of a slot to the next: fixed for the whole K loop
+  int so0, dso, dj;
 
   __device__ __forceinline__ int rl(int i) const { return rl0 + i * drl; }
   __device__ __forceinline__ int kl(int i) const { return kl0 + i * dkl; }
@@ -156,8 +160,12 @@ struct Stager {
     dk = kc ? 1 : 0;
     klast = K - (kc ? V : 1);
     kstep = (int64_t)BK * ko.stride;
+    kfull = K;
     if (kc) { rl0 = t / KL; drl = NT / KL; kl0 = (t % KL) * V; dkl = 0; }
     else { rl0 = (t % ML) * V; drl = 0; kl0 = t / ML; dkl = NT / ML; }
+    so0 = kl0 * (R + 1) + rl0;
+    dso = dkl * (R + 1) + drl;
+    dj = kc ? R + 1 : 1;
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
       if (kc || i == 0) {
@@ -180,11 +188,19 @@ struct Stager {
 
   // the slots move on to the tile that starts at k0
   __device__ __forceinline__ void advance(const KOff& ko, int64_t k0) {
+    if (k0 + BK <= kfull) {       // the whole tile lies inside K (uniform): no clamping
 #pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      const int64_t k = k0 + kl(i);
-      if constexpr (TAB) tv[i] = ko.tab[clamp_k(k)];
-      else ptr[i] += k <= klast ? kstep : 0;      // a slot past the end stays where it is: still readable, never stored
+      for (int i = 0; i < NL; ++i) {
+        if constexpr (TAB) tv[i] = ko.tab[k0 + kl(i)];
+        else ptr[i] += kstep;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        const int64_t k = k0 + kl(i);
+        if constexpr (TAB) tv[i] = ko.tab[clamp_k(k)];
+        else ptr[i] += k <= klast ? kstep : 0;      // a slot past the end stays where it is: still readable, never stored
+      }
     }
   }
 
@@ -198,14 +214,25 @@ struct Stager {
 
   // r holds the tile that starts at k0
   __device__ __forceinline__ void store(const Vec* __restrict__ r, int64_t k0, int64_t kend, T (*S)[R + 1]) const {
-    const int dr = 1 - dk;
+    T* S0 = &S[0][0];
+    if (k0 + BK <= kend) {        // a whole tile (uniform): nothing to zero
 #pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      const bool ok = k0 + kl(i) < kend;
-      if constexpr (V == 1) S[kl(i)][rl(i)] = ok ? r[i] : T(0);
-      else {
+      for (int i = 0; i < NL; ++i) {
+        if constexpr (V == 1) S0[so0 + i * dso] = r[i];
+        else {
 #pragma unroll
-        for (int j = 0; j < V; ++j) S[kl(i) + j * dk][rl(i) + j * dr] = ok ? r[i][j] : T(0);
+          for (int j = 0; j < V; ++j) S0[so0 + i * dso + j * dj] = r[i][j];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        const bool ok = k0 + kl(i) < kend;
+        if constexpr (V == 1) S0[so0 + i * dso] = ok ? r[i] : T(0);
+        else {
+#pragma unroll
+          for (int j = 0; j < V; ++j) S0[so0 + i * dso + j * dj] = ok ? r[i][j] : T(0);
+        }
       }
     }
   }
@@ -296,18 +323,25 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
   const int lane = t & 63, wave = t >> 6;
   const int wm = wave / WGN, wn = wave % WGN;
 
-  // XCD-aware tile numbering: blocks b, b+8, b+16, ... share an XCD; give each
-  // XCD a contiguous range of tiles.
+  // XCD-aware numbering of (K chunk, tile): blocks b, b+8, b+16, ... of the
+  // grid's x-then-y order share an XCD and its L2.  Each XCD gets a contiguous
+  // range of the chunk-major order, so the tiles that read the same rows of A
+  // or B over the same K chunk run on one XCD and share those rows in its L2.
   const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int64_t ntiles = tiles_m * tiles_n;
-  int64_t bid = blockIdx.x;
-  if (ntiles >= 64 && (ntiles & 7) == 0) bid = (bid & 7) * (ntiles >> 3) + (bid >> 3);
+  const int64_t nblocks = ntiles * gridDim.y;
+  int64_t lin = blockIdx.x + ntiles * (int64_t)blockIdx.y;
+  if (nblocks >= 64) {
+    const int64_t x = lin & 7, per = nblocks >> 3, rem = nblocks & 7;
+    lin = x * per + (x < rem ? x : rem) + (lin >> 3);
+  }
+  const int s = (int)(lin / ntiles);
+  const int64_t bid = lin - s * ntiles;
   const int64_t tile_m = bid / tiles_n, tile_n = bid - tile_m * tiles_n;
   const int64_t m0 = tile_m * BM, n0 = tile_n * BN;
 
   int64_t bta, btb, btc;
   group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
-  const int s = blockIdx.y;
   int sk = s;                              // chunk within its term
   if (p.n_terms > 0) {
     const int term = s / p.term_split;
@@ -408,18 +442,25 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
   const int lane = t & 63, wave = t >> 6;
   const int wm = wave / WGN, wn = wave % WGN;
 
-  // XCD-aware tile numbering: blocks b, b+8, b+16, ... share an XCD; give each
-  // XCD a contiguous range of tiles.
+  // XCD-aware numbering of (K chunk, tile): blocks b, b+8, b+16, ... of the
+  // grid's x-then-y order share an XCD and its L2.  Each XCD gets a contiguous
+  // range of the chunk-major order, so the tiles that read the same rows of A
+  // or B over the same K chunk run on one XCD and share those rows in its L2.
   const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int64_t ntiles = tiles_m * tiles_n;
-  int64_t bid = blockIdx.x;
-  if (ntiles >= 64 && (ntiles & 7) == 0) bid = (bid & 7) * (ntiles >> 3) + (bid >> 3);
+  const int64_t nblocks = ntiles * gridDim.y;
+  int64_t lin = blockIdx.x + ntiles * (int64_t)blockIdx.y;
+  if (nblocks >= 64) {
+    const int64_t x = lin & 7, per = nblocks >> 3, rem = nblocks & 7;
+    lin = x * per + (x < rem ? x : rem) + (lin >> 3);
+  }
+  const int s = (int)(lin / ntiles);
+  const int64_t bid = lin - s * ntiles;
   const int64_t tile_m = bid / tiles_n, tile_n = bid - tile_m * tiles_n;
   const int64_t m0 = tile_m * BM, n0 = tile_n * BN;
 
   int64_t bta, btb, btc;
   group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
-  const int s = blockIdx.y;
   int sk = s;                              // chunk within its term
   const int term0 = 0, nterm = p.n_terms;
   const int64_t kbeg = (int64_t)sk * p.kchunk;
