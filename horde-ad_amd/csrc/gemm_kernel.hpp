@@ -303,8 +303,10 @@ __device__ __forceinline__ void k_loop(const GemmParams& p, const typename X::T*
 }
 
 // Block tile BM x BN = (WGM * TM * 16) x (WGN * TN * 16).  NBUF LDS buffers.
-// Skinny tiles keep few accumulators: ask for three wavefronts per SIMD there
-// (the loads of one tile are only hidden by the MFMAs of other blocks).
+// Skinny tiles keep few accumulators: ask for two wavefronts per SIMD there, so
+// that a second block on the CU runs through the first one's barriers and LDS
+// stores (three would leave the staging registers of the 256-row tiles too few
+// VGPRs: they spill).
 constexpr int waves_wanted(int tm, int tn, int esize) { return tm * tn * esize <= 32 ? 2 : 1; }
 
 template <typename X, int WGM, int WGN, int TM, int TN, int VA, int VB, int NBUF>
