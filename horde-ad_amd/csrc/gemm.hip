@@ -81,9 +81,39 @@ __global__ void __launch_bounds__(256) k_sum_partials(int64_t n, int S, int64_t 
   }
 }
 
+// The same sum for a handful of partials (S <= 8), where the blocks above would
+// leave most of their lane groups without a partial: one output per lane, the
+// partials added in the same order (0 + p0 + p1 + ...), four loads in flight.
+template <typename T>
+__global__ void __launch_bounds__(256) k_sum_partials_few(int64_t n, int S, int64_t stride, const T* __restrict__ part, T* __restrict__ out) {
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
+    const T* p = part + i;
+    T acc = T(0);
+    int s = 0;
+    for (; s + 3 < S; s += 4) {
+      const T a = p[(int64_t)s * stride], b = p[(int64_t)(s + 1) * stride], c = p[(int64_t)(s + 2) * stride], d = p[(int64_t)(s + 3) * stride];
+      acc += a;
+      acc += b;
+      acc += c;
+      acc += d;
+    }
+    if (s + 1 < S) {
+      const T a = p[(int64_t)s * stride], b = p[(int64_t)(s + 1) * stride];
+      acc += a;
+      acc += b;
+      s += 2;
+    }
+    if (s < S) acc += p[(int64_t)s * stride];
+    out[i] = acc;
+  }
+}
+
 template <typename T>
 void launch_sum_partials(hgpu_ctx* ctx, int64_t n, int S, const T* part, T* out) {
-  if (n <= 32768 && S >= 32)
+  if (S <= 8)
+    hipLaunchKernelGGL((k_sum_partials_few<T>), dim3(grid_for(n, 256, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out);
+  else if (n <= 32768 && S >= 32)
     hipLaunchKernelGGL((k_sum_partials<T, 8>), dim3(grid_for(n, 8, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out);
   else
     hipLaunchKernelGGL((k_sum_partials<T, 32>), dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out);
