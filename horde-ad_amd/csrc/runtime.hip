@@ -818,10 +818,10 @@ int rtc_compile(hgpu_ctx* ctx, const std::string& src, const char* what, std::ve
   hiprtcProgram prog;
   if (hiprtcCreateProgram(&prog, src.c_str(), "hordead_gpu_rtc.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
     return fail(ctx, HGPU_ERR_DEVICE, "hiprtcCreateProgram failed");
-  // packed FP32 instructions stay off, as in the ahead-of-time build; a hiprtc
-  // that does not take the feature switch compiles without it
-  hiprtcResult r = hiprtcCompileProgram(prog, 7, kRtcOpts);
-  if (r != HIPRTC_SUCCESS) r = hiprtcCompileProgram(prog, 3, kRtcOpts);
+  // packed FP32 instructions stay off, as in the ahead-of-time build.  There is
+  // no retry without the switch: a compiler that rejects it fails here, with its
+  // log, rather than handing back code built under other options than the key says.
+  hiprtcResult r = hiprtcCompileProgram(prog, (int)(sizeof kRtcOpts / sizeof kRtcOpts[0]), kRtcOpts);
   if (r != HIPRTC_SUCCESS) {
     size_t n = 0;
     hiprtcGetProgramLogSize(prog, &n);
