@@ -61,6 +61,7 @@ GPU_ONLY = {
     "stream": (P, [P]), "inject_alloc_failure": (I, [P, L]),
     "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
     "profile_enable": (I, [P, I]), "profile_report": (I, [P, C.c_char_p, C.c_size_t]),
+    "contract_noalloc": (I, [P, P, P, I, P]),
 }
 
 
@@ -301,6 +302,11 @@ class Array:
 
     def contract(self, other, n_keep):
         return self.ctx._out(self.ctx.lib.contract, self.h, other.h if other is not None else None, n_keep)
+
+    def contract_noalloc(self, other, n_keep, out):
+        """hgpu_contract into the caller's array `out`, without device allocation (gfx950 library only)."""
+        self.ctx.check(self.ctx.lib.contract_noalloc(self.ctx.h, self.h, other.h if other is not None else None, n_keep, out.h))
+        return out
 
     def argminmax_last(self, want_max):
         return self._o(self.ctx.lib.argminmax_last, int(want_max))

@@ -447,6 +447,106 @@ int64_t min_abs_nonzero(const Dims& d, int dim) {
   return m;
 }
 
+// The HBM-bound path of hgpu_contract: out[o] = sum_r a[o,r] * b[o,r] (b may be
+// null) written densely at `out`.  Long reductions with few outputs are split
+// into S chunks whose partial sums a second launch adds up.  The partial sums
+// live in `scratch` when the caller brings one (then nothing is allocated here,
+// and a request whose partial sums exceed scratch_bytes is refused), else in a
+// block from the context's allocator.
+int reduce_views(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, void* out, void* scratch, size_t scratch_bytes) {
+  int64_t n_out = 1, R = 1;
+  for (int i = 0; i < n_keep; ++i) n_out *= a->shape[i];
+  for (int i = n_keep; i < a->rank; ++i) R *= a->shape[i];
+  int64_t zero[HGPU_MAX_RANK] = {0};
+  const int64_t* bst = b ? b->strides : zero;
+  const int64_t* ks[2] = {a->strides, bst};
+  const int64_t* rs[2] = {a->strides + n_keep, bst + n_keep};
+  Dims keep, red;
+  if (!collapse(n_keep, a->shape, 2, ks, &keep) || !collapse(a->rank - n_keep, a->shape + n_keep, 2, rs, &red))
+    return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract: more than %d merged dims", HG_KDIMS);
+  // Which way is memory contiguous: along the kept or along the reduced index?
+  int64_t sr = min_abs_nonzero(red, red.nd - 1);
+  int64_t sk = min_abs_nonzero(keep, keep.nd - 1);
+  int64_t Lin = red.shape[red.nd - 1];
+  bool use_wave;
+  if (n_out < 2048) use_wave = true;
+  else if (sr <= sk && Lin >= 16) use_wave = true;
+  else use_wave = false;
+  // Enough work items to fill the device, chunks of at least 512 elements.
+  int64_t want_items = (int64_t)ctx->num_cu * (use_wave ? 16 : 1024);
+  int64_t S = 1;
+  if (n_out < want_items) {
+    S = (want_items + n_out - 1) / n_out;
+    int64_t span = use_wave ? ((R / Lin) > 1 ? (R / Lin) : Lin) : R;
+    int64_t per = use_wave ? ((R / Lin) > 1 ? 512 / (Lin < 512 ? Lin : 512) : 1024) : 256;
+    if (per < 1) per = 1;
+    int64_t maxS = span / per;
+    if (maxS < 1) maxS = 1;
+    if (S > maxS) S = maxS;
+    if (S > 4096) S = 4096;
+  }
+  const void* pa = data_ptr(a);
+  const void* pb = b ? data_ptr(b) : nullptr;
+  int rc = HGPU_OK;
+  if (use_wave && n_out >= 64 && n_out <= 1024 && R >= 1024 && R <= 65536) {
+    // a few hundred outputs of a few thousand elements: a block per output, one launch
+    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, true, keep, red, n_out, R, 0, pa, pb, out)));
+  } else if (S == 1) {
+    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, use_wave, keep, red, n_out, R, 1, pa, pb, out)));
+  } else {
+    // stage 1: partials [n_out, S] in the accumulator type; stage 2 sums them.
+    const size_t need = (size_t)n_out * (size_t)S * 8;
+    hgpu_buffer* part = nullptr;
+    void* pp = scratch;
+    if (scratch) {
+      if (need > scratch_bytes)
+        return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract: %lld outputs in %lld chunks need %zu bytes of partial sums, the fixed scratch holds %zu",
+                    (long long)n_out, (long long)S, need, scratch_bytes);
+    } else {
+      rc = buffer_alloc(ctx, need, &part);
+      if (rc) return rc;
+      pp = part->ptr;
+    }
+    int64_t psh[2] = {n_out, S}, pst[2] = {S, 1};
+    HG_DISPATCH_DTYPE(a->dtype, T, { using A = typename acc_of<T>::type; rc = (launch_stage<T, A>(ctx, use_wave, keep, red, n_out, R, (int)S, pa, pb, pp)); });
+    if (!rc) {
+      Dims k2, r2;
+      int64_t z1[1] = {0};
+      const int64_t* ks2[2] = {pst, z1};
+      const int64_t* rs2[2] = {pst + 1, z1};
+      collapse(1, psh, 2, ks2, &k2);
+      collapse(1, psh + 1, 2, rs2, &r2);
+      bool wave2 = n_out < 65536;
+      HG_DISPATCH_DTYPE(a->dtype, T, { using A = typename acc_of<T>::type; rc = (launch_stage<A, T>(ctx, wave2, k2, r2, n_out, S, 1, pp, nullptr, out)); });
+    }
+    if (part) buffer_release(part);
+  }
+  return rc;
+}
+
+// Partial sums of hgpu_contract_noalloc: one array per device, held until the
+// process ends.  In host code the name below is only a stand-in for the symbol:
+// the device address comes from hipGetSymbolAddress, once per device.
+constexpr size_t kScratchBytes = 1u << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mu;
+
+int scratch_of(hgpu_ctx* ctx, void** out) {
+  if (ctx->device < 0 || ctx->device >= kMaxDevices) return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract_noalloc: device %d", ctx->device);
+  std::lock_guard<std::mutex> g(g_scratch_mu);
+  if (!g_scratch_ptr[ctx->device]) {
+    hipError_t e = hipSetDevice(ctx->device);
+    void* p = nullptr;
+    if (e == hipSuccess) e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return check_hip(ctx, e == hipSuccess ? hipErrorInvalidSymbol : e, "hipGetSymbolAddress(scratch)");
+    g_scratch_ptr[ctx->device] = p;
+  }
+  *out = g_scratch_ptr[ctx->device];
+  return HGPU_OK;
+}
+
 // *acc += x, taking over x (the first term becomes the accumulator).
 int add_into(hgpu_ctx* ctx, hgpu_array** acc, hgpu_array* x) {
   if (!*acc) { *acc = x; return HGPU_OK; }
@@ -622,66 +722,34 @@ int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n
   if (rc) { hgpu_release(o); return rc; }
   if (handled) { *out = o; return HGPU_OK; }
 
-  int64_t zero[HGPU_MAX_RANK] = {0};
-  const int64_t* bst = b ? b->strides : zero;
-  const int64_t* ks[2] = {a->strides, bst};
-  const int64_t* rs[2] = {a->strides + n_keep, bst + n_keep};
-  Dims keep, red;
-  if (!collapse(n_keep, a->shape, 2, ks, &keep) || !collapse(a->rank - n_keep, a->shape + n_keep, 2, rs, &red)) {
-    hgpu_release(o);
-    return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract: more than %d merged dims", HG_KDIMS);
-  }
-  // Which way is memory contiguous: along the kept or along the reduced index?
-  int64_t sr = min_abs_nonzero(red, red.nd - 1);
-  int64_t sk = min_abs_nonzero(keep, keep.nd - 1);
-  int64_t Lin = red.shape[red.nd - 1];
-  bool use_wave;
-  if (n_out < 2048) use_wave = true;
-  else if (sr <= sk && Lin >= 16) use_wave = true;
-  else use_wave = false;
-  // Enough work items to fill the device, chunks of at least 512 elements.
-  int64_t want_items = (int64_t)ctx->num_cu * (use_wave ? 16 : 1024);
-  int64_t S = 1;
-  if (n_out < want_items) {
-    S = (want_items + n_out - 1) / n_out;
-    int64_t span = use_wave ? ((R / Lin) > 1 ? (R / Lin) : Lin) : R;
-    int64_t per = use_wave ? ((R / Lin) > 1 ? 512 / (Lin < 512 ? Lin : 512) : 1024) : 256;
-    if (per < 1) per = 1;
-    int64_t maxS = span / per;
-    if (maxS < 1) maxS = 1;
-    if (S > maxS) S = maxS;
-    if (S > 4096) S = 4096;
-  }
-  const void* pa = data_ptr(a);
-  const void* pb = b ? data_ptr(b) : nullptr;
-  if (use_wave && n_out >= 64 && n_out <= 1024 && R >= 1024 && R <= 65536) {
-    // a few hundred outputs of a few thousand elements: a block per output, one launch
-    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, true, keep, red, n_out, R, 0, pa, pb, data_ptr(o))));
-  } else if (S == 1) {
-    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, use_wave, keep, red, n_out, R, 1, pa, pb, data_ptr(o))));
-  } else {
-    // stage 1: partials [n_out, S] in the accumulator type; stage 2 sums them.
-    int accdt = dtype_is_float(a->dtype) ? HGPU_F64 : HGPU_I64;
-    int64_t psh[2] = {n_out, S};
-    hgpu_array* part = nullptr;
-    rc = new_dense(ctx, accdt, 2, psh, &part);
-    if (rc) { hgpu_release(o); return rc; }
-    HG_DISPATCH_DTYPE(a->dtype, T, { using A = typename acc_of<T>::type; rc = (launch_stage<T, A>(ctx, use_wave, keep, red, n_out, R, (int)S, pa, pb, data_ptr(part))); });
-    if (!rc) {
-      Dims k2, r2;
-      int64_t z1[1] = {0};
-      const int64_t* ks2[2] = {part->strides, z1};
-      const int64_t* rs2[2] = {part->strides + 1, z1};
-      collapse(1, psh, 2, ks2, &k2);
-      collapse(1, psh + 1, 2, rs2, &r2);
-      bool wave2 = n_out < 65536;
-      HG_DISPATCH_DTYPE(a->dtype, T, { using A = typename acc_of<T>::type; rc = (launch_stage<A, T>(ctx, wave2, k2, r2, n_out, S, 1, data_ptr(part), nullptr, data_ptr(o))); });
-    }
-    hgpu_release(part);
-  }
+  rc = reduce_views(ctx, a, b, n_keep, data_ptr(o), nullptr, 0);
   if (rc) { hgpu_release(o); return rc; }
   *out = o;
   return HGPU_OK;
+}
+
+int hgpu_contract_noalloc(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (n_keep < 0 || n_keep > a->rank) return fail(ctx, HGPU_ERR_INVALID, "contract_noalloc: n_keep %d of rank %d", n_keep, a->rank);
+  if (b) {
+    if (b->dtype != a->dtype) return fail(ctx, HGPU_ERR_INVALID, "contract_noalloc: dtypes differ");
+    if (!same_shape(a, b)) return fail(ctx, HGPU_ERR_INVALID, "contract_noalloc: shapes differ");
+  }
+  if (a->dtype == HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "contract_noalloc: Bool arrays have no sum");
+  if (out->dtype != a->dtype || out->rank != n_keep || !is_dense(out)) return fail(ctx, HGPU_ERR_INVALID, "contract_noalloc: the result array must be dense, of the operands' dtype and of the kept shape");
+  for (int i = 0; i < n_keep; ++i)
+    if (out->shape[i] != a->shape[i]) return fail(ctx, HGPU_ERR_INVALID, "contract_noalloc: the result array must have the kept shape");
+  if (out->buf && (out->buf == a->buf || (b && out->buf == b->buf))) return fail(ctx, HGPU_ERR_INVALID, "contract_noalloc: the result shares memory with an operand");
+  int64_t n_out = nelem(out), R = 1;
+  for (int i = n_keep; i < a->rank; ++i) R *= a->shape[i];
+  if (n_out == 0) return HGPU_OK;
+  if (R == 0) {   // an empty sum: zeros (the fill rounds up to 16 bytes, which stays inside a block only from its start)
+    if (out->offset != 0) return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract_noalloc: an empty sum into a view that does not start its block");
+    return zero_fill(ctx, data_ptr(out), (size_t)n_out * dtype_size(out->dtype));
+  }
+  void* sp = nullptr;
+  if (int rc = scratch_of(ctx, &sp)) return rc;
+  return reduce_views(ctx, a, b, n_keep, data_ptr(out), sp, kScratchBytes);
 }
 
 int hgpu_extremum_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_array** values, hgpu_array** out) {

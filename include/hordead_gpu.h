@@ -249,6 +249,21 @@ int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n
  * pairs share one layout and the whole is a matrix product it is one launch
  * whose K chunks run over all pairs.  Summation order is fixed by the shapes. */
 int hgpu_contract_sum(hgpu_ctx* ctx, int n, const hgpu_array* const* a, const hgpu_array* const* b, int n_keep, hgpu_array** out);
+/* hgpu_contract for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  The caller brings the result array `out`
+ * (dense, of the operands' dtype, of the kept shape, not sharing memory with an
+ * operand); this call makes no device allocation and frees none.  It always
+ * takes the HBM-bound reduction kernels (never the matrix-product path, which
+ * needs tables and partial products of its own), so floating-point sums may be
+ * associated differently from hgpu_contract's when that runs a matrix product;
+ * for plain sums and dot products the two agree bit for bit.  The partial sums
+ * of a split reduction live in one fixed array of 1 MiB per device, held until
+ * the process ends: a request that needs more (outputs x chunks x 8 bytes) fails
+ * with HGPU_ERR_UNSUPPORTED and a message naming the size.  Every call on a
+ * device uses that device's one array: calls that overlap on one device (two
+ * contexts, two streams) race; calls on one context are ordered by its stream. */
+int hgpu_contract_noalloc(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out);
 /* tsargMin / tsargMax (OpsConcrete.hs:533-534, targMinS :1712-1746): index of
  * the first minimal / maximal element along the LAST dim; result I64 of shape
  * init(shape). */
