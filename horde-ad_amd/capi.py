@@ -62,6 +62,7 @@ GPU_ONLY = {
     "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
     "profile_enable": (I, [P, I]), "profile_report": (I, [P, C.c_char_p, C.c_size_t]),
     "contract_noalloc": (I, [P, P, P, I, P]),
+    "contract_map": (I, [P, P, P, I, I, PP, I, P, I, IP, PP, I, I, LP, LP, I, I, PP, PP]),
 }
 
 
@@ -79,7 +80,7 @@ def _larr(xs):
 class Lib:
     """One provider of the ABI: a shared library plus the symbol prefix."""
 
-    def __init__(self, path=GPU_LIB, prefix="hgpu_"):
+    def __init__(self, path=GPU_LIB, prefix="hgpu_", api_table="get_api"):
         if not os.path.exists(path):
             raise FileNotFoundError(
                 f"{path} is not built; run `python -c 'import __graft_entry__ as g; g.build()'`")
@@ -92,6 +93,10 @@ class Lib:
             fn = getattr(self.dll, prefix + name)
             fn.restype, fn.argtypes = res, args
             setattr(self, name, fn)
+        if api_table != "get_api":   # another table of the same provider (the checker's one with the fused entry points)
+            fn = getattr(self.dll, prefix + api_table)
+            fn.restype, fn.argtypes = P, []
+            self.get_api = fn
 
     def context(self, device=0):
         return Ctx(self, device)
@@ -142,6 +147,24 @@ class Ctx:
         outs = (C.c_void_p * len(out_slots))()
         self.check(self.lib.fused_map(self.h, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs))
         return [Array(self, C.c_void_p(o)) for o in outs]
+
+    def contract_map(self, a, b, n_keep, inputs, prog, out_slots, ext=None):
+        """hgpu_contract_map: `inputs` holds None where the contraction of a and b stands;
+        ext = (slot, view_shape, view_strides, n_reduce, want_max) asks for the extremum over
+        windows.  Returns (outs, values, indices); the last two None without ext."""
+        ins = (C.c_void_p * len(inputs))(*[None if p is None else p.h for p in inputs])
+        flat = (C.c_int32 * max(6 * len(prog), 1))(*[int(x) for q in prog for x in q])
+        slots = (C.c_int * max(len(out_slots), 1))(*out_slots)
+        outs = (C.c_void_p * max(len(out_slots), 1))()
+        v, i = C.c_void_p(), C.c_void_p()
+        if ext is None:
+            self.check(self.lib.contract_map(self.h, a.h, b.h, n_keep, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs,
+                                             0, 0, None, None, 0, 0, None, None))
+            return [Array(self, C.c_void_p(o)) for o in outs[:len(out_slots)]], None, None
+        slot, vshape, vstrides, n_reduce, want_max = ext
+        self.check(self.lib.contract_map(self.h, a.h, b.h, n_keep, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs,
+                                         slot, len(vshape), _larr(vshape), _larr(vstrides), n_reduce, int(want_max), C.byref(v), C.byref(i)))
+        return [Array(self, C.c_void_p(o)) for o in outs[:len(out_slots)]], Array(self, v), Array(self, i)
 
     def fused_sum(self, inputs, prog, slot):
         """The sum of slot's values over all elements, a rank-0 array."""

@@ -19,6 +19,7 @@
 // product over its chunks, summed afterwards in a fixed order.  Chunk index in
 // the rows: each chunk writes its own rows of C.
 #include "common.hpp"
+#include "fused_gen.hpp"
 #include "gemm_kernel.hpp"
 
 #include <hip/hiprtc.h>
@@ -53,6 +54,8 @@ std::map<std::string, Compiled>& cache_of(hgpu_ctx* ctx) {
 int compile(hgpu_ctx* ctx, const std::string& src, const std::string& kname, Compiled* out) {
   std::vector<char> code;
   int rc = rtc_compile(ctx, src, "footprint gemm", &code);
+  // callers leave a shape the compiler rejects to the other kernels: say so when asked
+  if (rc && getenv("HORDEAD_GPU_DEBUG")) fprintf(stderr, "hordead_gpu: %s rejected: %s\n", kname.c_str(), hgpu_last_error(ctx));
   if (rc) return rc;
   hipError_t e = hipModuleLoadData(&out->mod, code.data());
   if (e != hipSuccess) return check_hip(ctx, e, "hipModuleLoadData");
@@ -268,9 +271,20 @@ __device__ __forceinline__ void store_rows(T* __restrict__ out, const OutPos& p,
   }
 }
 
+//@EPILOGUE@
 extern "C" __global__ void __launch_bounds__(256, 1)
-KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 nch, i64 chx, i64 chy, i64 chc, i64 part_stride) {
+KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 nch, i64 chx, i64 chy, i64 chc, i64 part_stride
+#if EPI
+      , EpiArgs ea
+#endif
+      ) {
   __shared__ T lds[LDS_ELEMS];
+#if EPI_STAGE
+  // the chunk's results in the layout they have in memory, written out with whole vectors once the chunk is done
+  __shared__ __attribute__((aligned(16))) unsigned char stage[EPI_STAGE];
+#else
+  unsigned char* const stage = nullptr;
+#endif
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, q4 = lane >> 4;
@@ -304,12 +318,21 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   }
   // lanes past the end of K in the last group contribute zero
   const bool tail_lane = q4 >= KVALID;
+#if EPI
+  // where a lane's rows and windows go, and the program inputs that do not change with the row
+  EPos epos[NACC];
+#pragma unroll
+  for (int t = 0; t < NBF; ++t) epos[t] = epi_pos((wave + 4 * t) * 16 + 4 * q4, r);
+  if (REM > 0) epos[NBF] = epi_pos((4 * NBF + (wave < REM ? wave : 0)) * 16 + 4 * q4, r);
+  const Hoist hz = epi_hoist(ea, r < NIN ? r : NIN - 1);
+#else
   OutPos pos[MODE == 1 ? NACC : 1];
   if (MODE == 1) {
 #pragma unroll
     for (int t = 0; t < NBF; ++t) pos[t] = out_pos((wave + 4 * t) * 16 + 4 * q4, r);
     if (REM > 0) pos[NBF] = out_pos((4 * NBF + (wave < REM ? wave : 0)) * 16 + 4 * q4, r);
   }
+#endif
   Acc acc[NACC];
 #pragma unroll
   for (int t = 0; t < NACC; ++t) acc[t] = Acc{0, 0, 0, 0};
@@ -435,9 +458,14 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
       }
     }
     if (MODE == 1) {
+#if EPI
+#pragma unroll
+      for (int t = 0; t < NBF; ++t) epi_tile(ea, hz, epos[t], stage, ch, (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+#else
       T* out = C + ch * chc;
 #pragma unroll
       for (int t = 0; t < NBF; ++t) store_rows(out, pos[t], (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+#endif
       if (REM > 0) {
         T* red = lds + RED0;
 #pragma unroll
@@ -454,11 +482,20 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
 #pragma unroll
             for (int w = 0; w < 4; ++w) s[j] += red[((rb * 4 + w) * 4 + j) * 64 + lane];
           }
+#if EPI
+          epi_tile(ea, hz, epos[NBF], stage, ch, (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
+#else
           store_rows(out, pos[MODE == 1 ? NBF : 0], (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
+#endif
         }
       }
+#if EPI_STAGE
+      __syncthreads();
+      epi_flush(ea, stage, ch, tid);
+#endif
     }
   }
+#if !EPI
   if (MODE == 0) {
     T* out = C + (i64)blockIdx.x * part_stride;
 #pragma unroll
@@ -484,12 +521,25 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
       }
     }
   }
+#endif
 }
 )HG";
 
-std::string generate(const Plan& pl, const std::string& kname) {
+int lds_bytes(const Plan& pl) {
+  const int es = pl.f64 ? 8 : 4;
+  int64_t lx = (pl.span_x + pl.vx - 1) / pl.vx * pl.vx, ly = (pl.span_y + pl.vy - 1) / pl.vy * pl.vy;
+  if (pl.ypad) ly += (ly / pl.ys) * pl.ypad;
+  int64_t buf = pl.mode == 0 ? lx + ly : lx;
+  int MB = (pl.min_rows + 15) / 16, REM = MB % 4;
+  int64_t total = pl.nbufs * buf + (pl.mode == 0 ? 0 : ly) + (REM > 0 ? REM * 4 * 256 : 0);
+  total *= es;
+  return total > INT32_MAX ? INT32_MAX : (int)total;
+}
+
+std::string generate(const Plan& pl, const std::string& kname, const std::string& epilogue = std::string(), int stage_bytes = 0) {
   std::ostringstream s;
   s << "#define KNAME " << kname << "\n";
+  s << "#define EPI " << (epilogue.empty() ? 0 : 1) << "\n#define EPI_STAGE " << stage_bytes << "\n";
   const int es = pl.f64 ? 8 : 4;
   s << "#define F64 " << (pl.f64 ? 1 : 0) << "\n";
   s << "#define MODE " << pl.mode << "\n";
@@ -515,19 +565,56 @@ std::string generate(const Plan& pl, const std::string& kname) {
   if (pl.ypad)
     for (auto& c : col_y) c += (int)(c / pl.ys) * pl.ypad;
   s << table("__device__ const", "kColY", col_y) << table("__device__ const", "kColC", pl.col_c);
-  s << kBody;
+  std::string body = kBody;
+  const std::string mark = "//@EPILOGUE@";
+  body.replace(body.find(mark), mark.size(), epilogue);
+  s << body;
   return s.str();
 }
 
-int lds_bytes(const Plan& pl) {
+// Staging vectors, LDS padding of the columns operand, output vectors and the
+// number of chunk buffers of a plan whose operands sit at xp / yp; false when
+// the plan does not fit the CU.
+bool finish_plan(Plan& pl, const char* xp, const char* yp, const char* cp, int64_t out_n, int extra_lds_bytes) {
   const int es = pl.f64 ? 8 : 4;
-  int64_t lx = (pl.span_x + pl.vx - 1) / pl.vx * pl.vx, ly = (pl.span_y + pl.vy - 1) / pl.vy * pl.vy;
-  if (pl.ypad) ly += (ly / pl.ys) * pl.ypad;
-  int64_t buf = pl.mode == 0 ? lx + ly : lx;
-  int MB = (pl.min_rows + 15) / 16, REM = MB % 4;
-  int64_t total = pl.nbufs * buf + (pl.mode == 0 ? 0 : ly) + (REM > 0 ? REM * 4 * 256 : 0);
-  total *= es;
-  return total > INT32_MAX ? INT32_MAX : (int)total;
+  const int V = 16 / es;
+  pl.vx = (((uintptr_t)xp & 15) == 0 && (pl.chx * es) % 16 == 0) ? V : 1;
+  pl.vy = (((uintptr_t)yp & 15) == 0 && (pl.chy * es) % 16 == 0) ? V : 1;
+  // columns a constant stride apart, each with its K offsets inside the
+  // stride: pad the stride in LDS until 16 columns hit 16 different banks
+  pl.ys = 1;
+  pl.ypad = 0;
+  if (pl.col_y.size() >= 2 && pl.col_y[1] > 0) {
+    const int64_t S = pl.col_y[1];
+    bool regular = S % pl.vy == 0 && pl.span_y <= S * (int64_t)pl.col_y.size();
+    for (size_t c = 0; c < pl.col_y.size() && regular; ++c) regular = pl.col_y[c] == (int64_t)c * S;
+    int64_t inner = pl.span_y - S * ((int64_t)pl.col_y.size() - 1);
+    if (regular && inner <= S) {
+      const int dw = es / 4;
+      // a column stride of 4 (or 2) dwords modulo 8 (4) walks 16 lanes over all 64 banks
+      for (int pad = 0; pad <= 16; pad += pl.vy) {
+        int64_t sdw = (S + pad) * dw;
+        if (sdw % 8 == 4 || sdw % 4 == 2) { pl.ys = S; pl.ypad = pad; break; }
+      }
+    }
+  }
+  {
+    bool ok = cp != nullptr && pl.min_rows % 4 == 0 && ((uintptr_t)cp & 15) == 0 && pl.chc % V == 0;
+    for (size_t m = 0; m < pl.row_c.size() && ok; m += 4)
+      ok = pl.row_c[m] % V == 0 && pl.row_c[m + 1] == pl.row_c[m] + 1 && pl.row_c[m + 2] == pl.row_c[m] + 2 && pl.row_c[m + 3] == pl.row_c[m] + 3;
+    for (size_t c = 0; c < pl.col_c.size() && ok; ++c) ok = pl.col_c[c] % V == 0;
+    if (pl.mode == 0) ok = ok && out_n % V == 0;   // partial outputs lie out_n apart
+    pl.cvec = ok;
+  }
+  // scalar staging of a large footprint would need too many loads in flight
+  int64_t loads = (pl.span_x / pl.vx + 255) / 256 + (pl.mode == 0 ? (pl.span_y / pl.vy + 255) / 256 : 0);
+  if (loads > 48) return false;
+  pl.nbufs = 2;
+  if (lds_bytes(pl) + extra_lds_bytes > kLdsBudget) {
+    pl.nbufs = 1;
+    if (lds_bytes(pl) + extra_lds_bytes > kLdsBudget || loads * 4 + pl.addr_regs > 330) return false;   // the prefetch must fit the register file
+  }
+  return true;
 }
 
 }  // namespace
@@ -569,48 +656,9 @@ int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa,
         if (cand[ci].e < 64) continue;
         Plan pl;
         if (!make_plan(f64, rows, colsd, kd, in_k != 0, ci, ctx->num_cu, &pl)) continue;
-        // staging vectors: 16 bytes when bases, chunk strides and buffers allow
         const char* xp = (const char*)(swapped ? pb : pa) + pl.shift_x * es;
         const char* yp = (const char*)(swapped ? pa : pb) + pl.shift_y * es;
-        const int V = 16 / es;
-        pl.vx = (((uintptr_t)xp & 15) == 0 && (pl.chx * es) % 16 == 0) ? V : 1;
-        pl.vy = (((uintptr_t)yp & 15) == 0 && (pl.chy * es) % 16 == 0) ? V : 1;
-        // columns a constant stride apart, each with its K offsets inside the
-        // stride: pad the stride in LDS until 16 columns hit 16 different banks
-        pl.ys = 1;
-        pl.ypad = 0;
-        if (pl.col_y.size() >= 2 && pl.col_y[1] > 0) {
-          const int64_t S = pl.col_y[1];
-          bool regular = S % pl.vy == 0 && pl.span_y <= S * (int64_t)pl.col_y.size();
-          for (size_t c = 0; c < pl.col_y.size() && regular; ++c) regular = pl.col_y[c] == (int64_t)c * S;
-          int64_t inner = pl.span_y - S * ((int64_t)pl.col_y.size() - 1);
-          if (regular && inner <= S) {
-            const int dw = es / 4;
-            // a column stride of 4 (or 2) dwords modulo 8 (4) walks 16 lanes over all 64 banks
-            for (int pad = 0; pad <= 16; pad += pl.vy) {
-              int64_t sdw = (S + pad) * dw;
-              if (sdw % 8 == 4 || sdw % 4 == 2) { pl.ys = S; pl.ypad = pad; break; }
-            }
-          }
-        }
-        {
-          const int V16 = 16 / es;
-          const char* cp = (const char*)data_ptr(out);
-          bool ok = pl.min_rows % 4 == 0 && ((uintptr_t)cp & 15) == 0 && pl.chc % V16 == 0;
-          for (size_t m = 0; m < pl.row_c.size() && ok; m += 4)
-            ok = pl.row_c[m] % V16 == 0 && pl.row_c[m + 1] == pl.row_c[m] + 1 && pl.row_c[m + 2] == pl.row_c[m] + 2 && pl.row_c[m + 3] == pl.row_c[m] + 3;
-          for (size_t c = 0; c < pl.col_c.size() && ok; ++c) ok = pl.col_c[c] % V16 == 0;
-          if (pl.mode == 0) ok = ok && nelem(out) % V16 == 0;   // partial outputs lie nelem(out) apart
-          pl.cvec = ok;
-        }
-        // scalar staging of a large footprint would need too many loads in flight
-        int64_t loads = (pl.span_x / pl.vx + 255) / 256 + (pl.mode == 0 ? (pl.span_y / pl.vy + 255) / 256 : 0);
-        if (loads > 48) continue;
-        pl.nbufs = 2;
-        if (lds_bytes(pl) > kLdsBudget) {
-          pl.nbufs = 1;
-          if (lds_bytes(pl) > kLdsBudget || loads * 4 + pl.addr_regs > 330) continue;   // the prefetch must fit the register file
-        }
+        if (!finish_plan(pl, xp, yp, (const char*)data_ptr(out), nelem(out), 0)) continue;
         best = pl;
         best_swapped = swapped != 0;
         found = true;
@@ -674,3 +722,537 @@ int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa,
 }
 
 }  // namespace hg
+
+// ---------------------------------------------------------------------------
+// hgpu_contract_map: a contraction, an elementwise program over its result and
+// an extremum over windows of that, as one footprint kernel.
+//
+// The view (the windows) refines the kept dims: every view dim walks ONE kept
+// dim with a constant step, and together the view dims of a kept dim count
+// through it exactly once (h = 2 h2 + p).  The product's rows are then
+// enumerated over the view dims, the reduced ones innermost, so that the four
+// accumulator registers of a lane -- four consecutive rows of one column -- hold
+// whole windows: the program and the extremum need no data from another lane.
+namespace {
+
+using namespace hg::fusedgen;
+
+struct EpiSpec {
+  int n_in = 0, c_slot = -1, n_instr = 0;
+  const hgpu_fused_instr* prog = nullptr;
+  std::vector<int> dt;                 // type of every slot
+  std::vector<char> cls;               // per input: 'C' the contraction, 's' one element, 'c' moves with the column only, 'g' general
+  std::vector<std::vector<int>> in_row, in_col;   // per input: offsets of every inner row / column
+  std::vector<int64_t> in_chs;         // per input: chunk stride
+  std::vector<int> out_slots;
+  bool has_ext = false, want_max = true;
+  int ext_slot = 0, L = 1;             // window = L consecutive rows
+  std::vector<int> win_row, win_col;   // offsets of every window / column in values and indices
+  int64_t win_chs = 0, out_chs = 0;
+  // Staged: a chunk's part of every result is one dense block of memory; the
+  // block is put together in LDS and written with 16-byte vectors.
+  bool staged = false;
+  std::vector<int> out_off;            // per output: byte offset of its block in the stage buffer
+  int val_off = 0, idx_off = 0, stage_bytes = 0;
+};
+
+std::string epilogue_source(const Plan& pl, const EpiSpec& e) {
+  std::ostringstream s;
+  s << kPrelude;
+  const int WPL = 4 / e.L;
+  for (int i = 0; i < e.n_in; ++i) {
+    if (e.cls[(size_t)i] == 'g') s << table("__device__ const", ("kRowI" + std::to_string(i)).c_str(), e.in_row[(size_t)i]);
+    if (e.cls[(size_t)i] == 'g' || e.cls[(size_t)i] == 'c') s << table("__device__ const", ("kColI" + std::to_string(i)).c_str(), e.in_col[(size_t)i]);
+  }
+  if (e.has_ext) s << table("__device__ const", "kWinO", e.win_row) << table("__device__ const", "kColO", e.win_col);
+  s << "struct EpiArgs {\n";
+  for (int i = 0; i < e.n_in; ++i)
+    if (i != e.c_slot) s << "  const " << ctype(e.dt[(size_t)i]) << "* i" << i << ";\n";
+  for (size_t o = 0; o < e.out_slots.size(); ++o) s << "  " << ctype(e.dt[(size_t)e.out_slots[o]]) << "* o" << o << ";\n";
+  if (e.has_ext) s << "  " << ctype(e.dt[(size_t)e.ext_slot]) << "* ov;\n  i64* oi;\n";
+  s << "  int unused;\n};\n";
+  s << "struct Hoist {\n";
+  for (int i = 0; i < e.n_in; ++i)
+    if (e.cls[(size_t)i] == 's' || e.cls[(size_t)i] == 'c') s << "  " << ctype(e.dt[(size_t)i]) << " h" << i << ";\n";
+  s << "  int unused;\n};\n";
+  s << "__device__ __forceinline__ Hoist epi_hoist(const EpiArgs& ea, int col) {\n  Hoist z;\n  z.unused = 0;\n";
+  for (int i = 0; i < e.n_in; ++i) {
+    if (e.cls[(size_t)i] == 's') s << "  z.h" << i << " = ea.i" << i << "[0];\n";
+    if (e.cls[(size_t)i] == 'c') s << "  z.h" << i << " = ea.i" << i << "[kColI" << i << "[col]];\n";
+  }
+  s << "  return z;\n}\n";
+  // positions of a lane's four rows (outputs of the kept shape, general inputs) and of its windows
+  s << "struct EPos {\n  int o[4];\n  int w[" << WPL << "];\n";
+  for (int i = 0; i < e.n_in; ++i)
+    if (e.cls[(size_t)i] == 'g') s << "  int g" << i << "[4];\n";
+  s << "};\n";
+  s << "__device__ __forceinline__ EPos epi_pos(int m0, int col) {\n  EPos p;\n";
+  s << "  const int cc = col < NIN ? col : NIN - 1;\n";
+  s << "#pragma unroll\n  for (int j = 0; j < 4; ++j) {\n    const int m = m0 + j < MIN ? m0 + j : MIN - 1;\n";
+  s << "    p.o[j] = kRowC[m] + kColC[cc];\n";
+  for (int i = 0; i < e.n_in; ++i)
+    if (e.cls[(size_t)i] == 'g') s << "    p.g" << i << "[j] = kRowI" << i << "[m] + kColI" << i << "[cc];\n";
+  s << "  }\n";
+  s << "#pragma unroll\n  for (int w = 0; w < " << WPL << "; ++w) {\n";
+  if (e.has_ext) s << "    const int wi = m0 / " << e.L << " + w;\n    p.w[w] = kWinO[wi < MIN / " << e.L << " ? wi : MIN / " << e.L << " - 1] + kColO[cc];\n";
+  else s << "    p.w[w] = 0;\n";
+  s << "  }\n  return p;\n}\n";
+  s << "__device__ __forceinline__ void epi_tile(const EpiArgs& ea, const Hoist& hz, const EPos& ep, unsigned char* stage, i64 ch, int m0, int col, T c0, T c1, T c2, T c3) {\n";
+  s << "  if (col >= NIN || m0 >= MIN) return;\n";
+  s << "  const T cv[4] = {c0, c1, c2, c3};\n";
+  if (e.has_ext) s << "  " << ctype(e.dt[(size_t)e.ext_slot]) << " ev[4];\n";
+  for (int j = 0; j < 4; ++j) {
+    std::string suf = "_" + std::to_string(j);
+    s << "  {\n";
+    for (int i = 0; i < e.n_in; ++i) {
+      s << "    const " << ctype(e.dt[(size_t)i]) << " v" << i << suf << " = ";
+      switch (e.cls[(size_t)i]) {
+        case 'C': s << "cv[" << j << "]"; break;
+        case 's': case 'c': s << "hz.h" << i; break;
+        default: s << "ea.i" << i << "[ch * " << e.in_chs[(size_t)i] << "ll + ep.g" << i << "[" << j << "]]"; break;
+      }
+      s << ";\n";
+    }
+    emit_program(s, e.n_in, e.n_instr, e.prog, e.dt, "    ", suf);
+    for (size_t o = 0; o < e.out_slots.size(); ++o) {
+      if (e.staged) s << "    reinterpret_cast<" << ctype(e.dt[(size_t)e.out_slots[o]]) << "*>(stage + " << e.out_off[o] << ")[ep.o[" << j << "]] = v" << e.out_slots[o] << suf << ";\n";
+      else s << "    ea.o" << o << "[ch * " << e.out_chs << "ll + ep.o[" << j << "]] = v" << e.out_slots[o] << suf << ";\n";
+    }
+    if (e.has_ext) s << "    ev[" << j << "] = v" << e.ext_slot << suf << ";\n";
+    s << "  }\n";
+  }
+  if (e.has_ext) {
+    for (int w = 0; w < WPL; ++w) {
+      s << "  {\n    " << ctype(e.dt[(size_t)e.ext_slot]) << " best = ev[" << w * e.L << "];\n    i64 bi = 0;\n";
+      for (int u = 1; u < e.L; ++u)
+        s << "    if (ev[" << w * e.L + u << "] " << (e.want_max ? ">" : "<") << " best) { best = ev[" << w * e.L + u << "]; bi = " << u << "; }\n";
+      if (e.staged) {
+        s << "    reinterpret_cast<" << ctype(e.dt[(size_t)e.ext_slot]) << "*>(stage + " << e.val_off << ")[ep.w[" << w << "]] = best;\n";
+        s << "    reinterpret_cast<i64*>(stage + " << e.idx_off << ")[ep.w[" << w << "]] = bi;\n  }\n";
+      } else {
+        s << "    const i64 at = ch * " << e.win_chs << "ll + ep.w[" << w << "];\n    ea.ov[at] = best;\n    ea.oi[at] = bi;\n  }\n";
+      }
+    }
+  }
+  s << "}\n";
+  if (e.staged) {
+    // every block of the stage buffer to its place in memory, 16 bytes per lane and step
+    s << "struct alignas(16) V16 { unsigned int w[4]; };\n";
+    s << "__device__ __forceinline__ void epi_flush(const EpiArgs& ea, const unsigned char* stage, i64 ch, int tid) {\n";
+    auto block = [&](const std::string& ptr, const char* ct, int64_t chs, int off, int64_t elems, size_t es) {
+      const int64_t nv = elems * (int64_t)es / 16;
+      s << "  {\n    V16* dst = reinterpret_cast<V16*>(" << ptr << " + ch * " << chs << "ll);\n";
+      s << "    const V16* src = reinterpret_cast<const V16*>(stage + " << off << ");\n";
+      s << "#pragma unroll 4\n    for (int v = tid; v < " << nv << "; v += 256) dst[v] = src[v];\n  }\n";
+      (void)ct;
+    };
+    const int64_t n_el = (int64_t)pl.min_rows * pl.nin;
+    for (size_t o = 0; o < e.out_slots.size(); ++o) block("ea.o" + std::to_string(o), ctype(e.dt[(size_t)e.out_slots[o]]), e.out_chs, e.out_off[o], n_el, dtype_size(e.dt[(size_t)e.out_slots[o]]));
+    if (e.has_ext) {
+      block("ea.ov", ctype(e.dt[(size_t)e.ext_slot]), e.win_chs, e.val_off, n_el / e.L, dtype_size(e.dt[(size_t)e.ext_slot]));
+      block("ea.oi", "i64", e.win_chs, e.idx_off, n_el / e.L, 8);
+    }
+    s << "}\n";
+  }
+  (void)pl;
+  return s.str();
+}
+
+// offsets of every flat index over dims with the given strides (row-major, last dim fastest)
+std::vector<int> offsets_of(const std::vector<int64_t>& ext, const std::vector<int64_t>& st, bool* fits) {
+  int64_t n = 1;
+  for (auto e : ext) n *= e;
+  std::vector<int> out((size_t)n, 0);
+  for (int64_t i = 0; i < n; ++i) {
+    int64_t r = i, o = 0;
+    for (int k = (int)ext.size() - 1; k >= 0; --k) { o += (r % ext[(size_t)k]) * st[(size_t)k]; r /= ext[(size_t)k]; }
+    if (o < 0 || o > INT32_MAX) *fits = false;
+    out[(size_t)i] = (int)o;
+  }
+  return out;
+}
+
+struct ViewDim { int64_t e; int kd; int64_t coef; };
+
+// Every view dim as a constant step along one kept dim; the view dims of a kept
+// dim must count through it exactly once.
+bool refine_view(int n_keep, const int64_t* kshape, int view_rank, const int64_t* vshape, const int64_t* vstrides, std::vector<ViewDim>* out) {
+  int64_t D[HGPU_MAX_RANK];
+  dense_strides(n_keep, kshape, D);
+  int64_t nk = 1, nv = 1;
+  for (int k = 0; k < n_keep; ++k) nk *= kshape[k];
+  for (int j = 0; j < view_rank; ++j) nv *= vshape[j];
+  if (nk != nv || nk == 0) return false;
+  out->clear();
+  for (int j = 0; j < view_rank; ++j) {
+    ViewDim v{vshape[j], -1, 0};
+    if (v.e > 1) {
+      if (vstrides[j] <= 0) return false;
+      for (int k = 0; k < n_keep; ++k)
+        if (kshape[k] > 1 && D[k] <= vstrides[j] && (v.kd < 0 || D[k] > D[v.kd])) v.kd = k;
+      if (v.kd < 0 || vstrides[j] % D[v.kd] != 0) return false;
+      v.coef = vstrides[j] / D[v.kd];
+    }
+    out->push_back(v);
+  }
+  for (int k = 0; k < n_keep; ++k) {
+    if (kshape[k] <= 1) continue;
+    std::vector<std::pair<int64_t, int64_t>> digits;   // (step, extent)
+    for (auto& v : *out)
+      if (v.kd == k) digits.push_back({v.coef, v.e});
+    std::sort(digits.begin(), digits.end());
+    int64_t reach = 1;
+    for (auto& d : digits) {
+      if (d.first != reach) return false;
+      reach *= d.second;
+    }
+    if (reach != kshape[k]) return false;
+  }
+  return true;
+}
+
+int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, int n_in, const hgpu_array* const* in, int c_slot, int n_instr,
+                     const hgpu_fused_instr* prog, const std::vector<int>& dt, int n_out, const int* out_slots, hgpu_array** outs, int ext_slot, int view_rank,
+                     const int64_t* view_shape, const int64_t* view_strides, int n_reduce, int want_max, hgpu_array** values, hgpu_array** indices, bool* handled) {
+  *handled = false;
+  if (a->dtype != HGPU_F64 && a->dtype != HGPU_F32) return HGPU_OK;
+  const bool f64 = a->dtype == HGPU_F64;
+  const int es = f64 ? 8 : 4;
+  const bool has_ext = values != nullptr;
+  // without windows the "view" is the kept shape itself
+  int64_t dshape[HGPU_MAX_RANK], dstrides[HGPU_MAX_RANK];
+  if (!has_ext) {
+    view_rank = n_keep;
+    for (int k = 0; k < n_keep; ++k) dshape[k] = a->shape[k];
+    dense_strides(n_keep, dshape, dstrides);
+    view_shape = dshape;
+    view_strides = dstrides;
+    n_reduce = 0;
+  }
+  std::vector<ViewDim> vd;
+  if (!refine_view(n_keep, a->shape, view_rank, view_shape, view_strides, &vd)) return HGPU_OK;
+  int64_t L = 1;
+  for (int j = view_rank - n_reduce; j < view_rank; ++j) L *= view_shape[j];
+  if (L != 1 && L != 2 && L != 4) return HGPU_OK;
+  // strides of the operands and outputs along every view dim
+  struct VS { int64_t e, sa, sb, sc, so; bool red; std::vector<int64_t> sin; };
+  std::vector<VS> dims;
+  {
+    int64_t lead[HGPU_MAX_RANK], lst[HGPU_MAX_RANK];
+    const int rl = view_rank - n_reduce;
+    for (int j = 0; j < rl; ++j) lead[j] = view_shape[j];
+    dense_strides(rl, lead, lst);
+    for (int j = 0; j < view_rank; ++j) {
+      if (vd[(size_t)j].e <= 1) continue;
+      const int k = vd[(size_t)j].kd;
+      const int64_t c = vd[(size_t)j].coef;
+      VS v{vd[(size_t)j].e, c * a->strides[k], c * b->strides[k], view_strides[j], j < rl ? lst[j] : 0, j >= rl, {}};
+      for (int i = 0; i < n_in; ++i) v.sin.push_back(i == c_slot ? 0 : c * in[i]->strides[k]);
+      dims.push_back(v);
+    }
+  }
+  // rows: the side the reduced dims are on (else the larger side); columns: the other one, at most 16
+  int side_of_red = -1;   // 0: a, 1: b
+  int64_t Ma = 1, Nb = 1;
+  for (auto& v : dims) {
+    const bool ma = v.sa != 0 && v.sb == 0, nb = v.sa == 0 && v.sb != 0;
+    if (!ma && !nb) return HGPU_OK;   // a batch dim, or a dim neither operand moves along
+    if (ma) Ma *= v.e; else Nb *= v.e;
+    if (v.red) {
+      int sd = ma ? 0 : 1;
+      if (side_of_red >= 0 && side_of_red != sd) return HGPU_OK;
+      side_of_red = sd;
+    }
+  }
+  const bool swapped = side_of_red >= 0 ? side_of_red == 1 : Nb > Ma;   // rows operand is b
+  if ((swapped ? Ma : Nb) > 16) return HGPU_OK;
+  std::vector<Dim> rows, cols, kd;
+  std::vector<size_t> row_ix, col_ix;   // indices into dims, in the order of rows / cols
+  {
+    std::vector<size_t> plain, red;
+    for (size_t i = 0; i < dims.size(); ++i) {
+      const bool on_a = dims[i].sa != 0;
+      if (on_a == !swapped) (dims[i].red ? red : plain).push_back(i);
+      else col_ix.push_back(i);
+    }
+    auto mag = [](int64_t v) { return v < 0 ? -v : v; };
+    std::stable_sort(plain.begin(), plain.end(), [&](size_t x, size_t y) { return mag(swapped ? dims[x].sb : dims[x].sa) > mag(swapped ? dims[y].sb : dims[y].sa); });
+    row_ix = plain;
+    row_ix.insert(row_ix.end(), red.begin(), red.end());
+    for (size_t i : row_ix) rows.push_back(Dim{dims[i].e, swapped ? dims[i].sb : dims[i].sa, 0, dims[i].sc});
+    for (size_t i : col_ix) cols.push_back(Dim{dims[i].e, 0, swapped ? dims[i].sa : dims[i].sb, dims[i].sc});
+  }
+  double K = 1;
+  for (int i = n_keep; i < a->rank; ++i) {
+    if (a->shape[i] == 1) continue;
+    if (a->strides[i] == 0 || b->strides[i] == 0) return HGPU_OK;
+    kd.push_back(Dim{a->shape[i], swapped ? b->strides[i] : a->strides[i], swapped ? a->strides[i] : b->strides[i], 0});
+    K *= (double)a->shape[i];
+  }
+  if (kd.empty() || cols.empty() || rows.empty()) return HGPU_OK;
+  if ((double)Ma * (double)Nb * K < 1.0e7) return HGPU_OK;
+  const char* pa = (const char*)data_ptr(a);
+  const char* pb = (const char*)data_ptr(b);
+  Plan pl;
+  size_t chunk = 0;
+  bool found = false;
+  for (size_t ci = 0; ci < rows.size() && !found; ++ci) {
+    if (rows[ci].e < 64 || dims[row_ix[ci]].red) continue;
+    Plan p2;
+    if (!make_plan(f64, rows, cols, kd, false, ci, ctx->num_cu, &p2)) continue;
+    if (p2.min_rows % 4 != 0) continue;
+    const char* xp = (swapped ? pb : pa) + p2.shift_x * es;
+    const char* yp = (swapped ? pa : pb) + p2.shift_y * es;
+    if (!finish_plan(p2, xp, yp, nullptr, 0, 0)) continue;
+    pl = p2;
+    chunk = ci;
+    found = true;
+  }
+  if (!found) return HGPU_OK;
+
+  // ---- the epilogue's tables
+  EpiSpec e;
+  e.n_in = n_in;
+  e.c_slot = c_slot;
+  e.n_instr = n_instr;
+  e.prog = prog;
+  e.dt = dt;
+  e.out_slots.assign(out_slots, out_slots + n_out);
+  e.has_ext = has_ext;
+  e.want_max = want_max != 0;
+  e.ext_slot = ext_slot;
+  e.L = (int)L;
+  bool fits = true;
+  std::vector<int64_t> rext, cext;
+  for (size_t i = 0; i < row_ix.size(); ++i)
+    if (i != chunk) rext.push_back(dims[row_ix[i]].e);
+  for (size_t i : col_ix) cext.push_back(dims[i].e);
+  auto row_strides = [&](auto get) { std::vector<int64_t> st; for (size_t i = 0; i < row_ix.size(); ++i) if (i != chunk) st.push_back(get(dims[row_ix[i]])); return st; };
+  auto col_strides = [&](auto get) { std::vector<int64_t> st; for (size_t i : col_ix) st.push_back(get(dims[i])); return st; };
+  e.out_chs = dims[row_ix[chunk]].sc;
+  e.win_chs = dims[row_ix[chunk]].so;
+  e.cls.assign((size_t)n_in, 'g');
+  e.in_row.resize((size_t)n_in);
+  e.in_col.resize((size_t)n_in);
+  e.in_chs.assign((size_t)n_in, 0);
+  for (int i = 0; i < n_in; ++i) {
+    if (i == c_slot) { e.cls[(size_t)i] = 'C'; continue; }
+    bool any = false, any_row = false;
+    for (size_t d = 0; d < dims.size(); ++d) any = any || dims[d].sin[(size_t)i] != 0;
+    for (size_t q = 0; q < row_ix.size(); ++q) any_row = any_row || dims[row_ix[q]].sin[(size_t)i] != 0;
+    if (!any) { e.cls[(size_t)i] = 's'; continue; }
+    e.in_col[(size_t)i] = offsets_of(cext, col_strides([&](const VS& v) { return v.sin[(size_t)i]; }), &fits);
+    if (!any_row) { e.cls[(size_t)i] = 'c'; continue; }
+    e.in_row[(size_t)i] = offsets_of(rext, row_strides([&](const VS& v) { return v.sin[(size_t)i]; }), &fits);
+    e.in_chs[(size_t)i] = dims[row_ix[chunk]].sin[(size_t)i];
+  }
+  if (has_ext) {
+    // windows: the rows without the reduced dims
+    std::vector<int64_t> wext, wst;
+    for (size_t i = 0; i < row_ix.size(); ++i)
+      if (i != chunk && !dims[row_ix[i]].red) { wext.push_back(dims[row_ix[i]].e); wst.push_back(dims[row_ix[i]].so); }
+    e.win_row = offsets_of(wext, wst, &fits);
+    e.win_col = offsets_of(cext, col_strides([&](const VS& v) { return v.so; }), &fits);
+    if ((int64_t)e.win_row.size() * L != pl.min_rows) return HGPU_OK;
+  }
+  if (!fits) return HGPU_OK;
+  // A chunk's share of every result one dense block (the offsets of its rows
+  // and columns count through 0 .. n-1), blocks and chunk strides whole 16-byte
+  // vectors: the blocks are put together in LDS.
+  {
+    auto dense_block = [](const std::vector<int>& rowo, const std::vector<int>& colo) {
+      const size_t n = rowo.size() * colo.size();
+      std::vector<char> hit(n, 0);
+      for (int r0 : rowo)
+        for (int c0 : colo) {
+          const int64_t o = (int64_t)r0 + c0;
+          if (o < 0 || o >= (int64_t)n || hit[(size_t)o]) return false;
+          hit[(size_t)o] = 1;
+        }
+      return true;
+    };
+    bool ok = n_out == 0 || dense_block(pl.row_c, pl.col_c);
+    if (has_ext) ok = ok && dense_block(e.win_row, e.win_col);
+    const int64_t n_el = (int64_t)pl.min_rows * pl.nin;
+    int off = 0;
+    auto place = [&](int64_t elems, size_t esz, int64_t chs) {
+      if ((elems * (int64_t)esz) % 16 != 0 || (chs * (int64_t)esz) % 16 != 0) ok = false;
+      int at = off;
+      off += (int)((elems * (int64_t)esz + 15) / 16 * 16);
+      return at;
+    };
+    for (int o = 0; o < n_out; ++o) e.out_off.push_back(place(n_el, dtype_size(dt[(size_t)out_slots[o]]), e.out_chs));
+    if (has_ext) {
+      e.val_off = place(n_el / L, dtype_size(dt[(size_t)ext_slot]), e.win_chs);
+      e.idx_off = place(n_el / L, 8, e.win_chs);
+    }
+    e.stage_bytes = off;
+    Plan p3 = pl;
+    const char* xp3 = (swapped ? pb : pa) + pl.shift_x * es;
+    const char* yp3 = (swapped ? pa : pb) + pl.shift_y * es;
+    if (ok && off > 0 && finish_plan(p3, xp3, yp3, nullptr, 0, off) && p3.nbufs == pl.nbufs) { e.staged = true; pl = p3; }
+    else e.stage_bytes = 0;
+  }
+
+  // ---- results
+  std::vector<hgpu_array*> res((size_t)n_out, nullptr);
+  hgpu_array *v = nullptr, *ix = nullptr;
+  auto release_all = [&] { for (auto* r : res) if (r) hgpu_release(r); if (v) hgpu_release(v); if (ix) hgpu_release(ix); };
+  for (int o = 0; o < n_out; ++o) {
+    int rc = new_dense(ctx, dt[(size_t)out_slots[o]], n_keep, a->shape, &res[(size_t)o]);
+    if (rc) { release_all(); return rc; }
+  }
+  if (has_ext) {
+    int rc = new_dense(ctx, dt[(size_t)ext_slot], view_rank - n_reduce, view_shape, &v);
+    if (!rc) rc = new_dense(ctx, HGPU_I64, view_rank - n_reduce, view_shape, &ix);
+    if (rc) { release_all(); return rc; }
+  }
+
+  char kname[160];
+  snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_chunkM%s_map%d%s", f64 ? "f64" : "f32", (long long)(swapped ? Nb : Ma), (long long)(swapped ? Ma : Nb),
+           (long long)K, swapped ? "_swapped" : "", n_instr, has_ext ? (want_max ? "_max" : "_min") : "");
+  std::string src = generate(pl, kname, epilogue_source(pl, e), e.staged ? e.stage_bytes : 0);
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c{nullptr, nullptr};
+    if (compile(ctx, src, kname, &c) != HGPU_OK) c = Compiled{nullptr, nullptr};
+    it = cache.emplace(src, c).first;
+  }
+  if (!it->second.fn) { release_all(); return HGPU_OK; }
+
+  // kernel arguments: the footprint kernel's own, then the EpiArgs struct (pointers in declaration order)
+  const char* xp = (swapped ? pb : pa) + pl.shift_x * es;
+  const char* yp = (swapped ? pa : pb) + pl.shift_y * es;
+  void* cnull = nullptr;
+  int64_t nch = pl.nch, chx = pl.chx, chy = pl.chy, chc = 0, part_stride = 0;
+  std::vector<const void*> ea;
+  for (int i = 0; i < n_in; ++i)
+    if (i != c_slot) ea.push_back(data_ptr(in[i]));
+  for (int o = 0; o < n_out; ++o) ea.push_back(data_ptr(res[(size_t)o]));
+  if (has_ext) { ea.push_back(data_ptr(v)); ea.push_back(data_ptr(ix)); }
+  ea.push_back(nullptr);   // the int at the end, padded to a pointer
+  void* args[] = {(void*)&xp, (void*)&yp, (void*)&cnull, (void*)&nch, (void*)&chx, (void*)&chy, (void*)&chc, (void*)&part_stride, (void*)ea.data()};
+  int64_t grid = pl.nch < ctx->num_cu ? pl.nch : ctx->num_cu;
+  {
+    const double M = (double)(swapped ? Nb : Ma), N = (double)(swapped ? Ma : Nb);
+    double flops = 2.0 * M * N * K;
+    double bytes = (M * K + N * K) * es;   // as for the plain product: operands once ...
+    for (int o = 0; o < n_out; ++o) bytes += M * N * (double)dtype_size(res[(size_t)o]->dtype);   // ... and what is written
+    if (has_ext) bytes += M * N / (double)L * (dtype_size(v->dtype) + 8.0);
+    const char* label = f64 ? "gemm_f64" : "gemm_f32";
+    if (ctx->profiling && ctx->profile_shapes) {
+      char buf[200];
+      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB1,footprint,chunkM%s,chunks%lld,rows%d,kgroups%d,lds%dK,map(instr%d,out%d%s)]", label, (long long)M, (long long)N,
+               (long long)K, swapped ? ",swapped" : "", (long long)pl.nch, pl.min_rows, (int)pl.gx.size(), lds_bytes(pl) / 1024, n_instr, n_out,
+               has_ext ? (L == 4 ? ",ext4" : (L == 2 ? ",ext2" : ",ext1")) : "");
+      label = ctx->label_pool.insert(buf).first->c_str();
+    }
+    LaunchGuard lg(ctx, label, bytes, flops);
+    hipError_t err = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+    if (err != hipSuccess) { release_all(); return check_hip(ctx, err, "contract_map launch"); }
+  }
+  for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
+  if (has_ext) { *values = v; *indices = ix; }
+  *handled = true;
+  return HGPU_OK;
+}
+
+}  // namespace
+
+extern "C" int hgpu_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, int n_in, const hgpu_array* const* in, int n_instr,
+                                 const hgpu_fused_instr* prog, int n_out, const int* out_slots, hgpu_array** outs, int ext_slot, int view_rank,
+                                 const int64_t* view_shape, const int64_t* view_strides, int n_reduce, int want_max, hgpu_array** values, hgpu_array** indices) {
+  if (!ctx || !a || !b || !in || (n_instr > 0 && !prog) || (n_out > 0 && (!out_slots || !outs))) return HGPU_ERR_INVALID;
+  if ((values == nullptr) != (indices == nullptr)) return HGPU_ERR_INVALID;
+  if (n_keep < 1 || n_keep > a->rank) return fail(ctx, HGPU_ERR_INVALID, "contract_map: n_keep %d of rank %d", n_keep, a->rank);
+  if (b->dtype != a->dtype || !same_shape(a, b)) return fail(ctx, HGPU_ERR_INVALID, "contract_map: operands differ in dtype or shape");
+  if (n_in < 1 || n_in > 12 || n_instr < 0 || n_instr > 96 || n_out < 0 || n_out > 6) return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract_map: %d inputs, %d instructions, %d outputs", n_in, n_instr, n_out);
+  int c_slot = -1;
+  for (int i = 0; i < n_in; ++i) {
+    if (!in[i]) {
+      if (c_slot >= 0) return fail(ctx, HGPU_ERR_INVALID, "contract_map: more than one input stands for the contraction");
+      c_slot = i;
+      continue;
+    }
+    bool ok = in[i]->rank == n_keep;
+    for (int d = 0; d < n_keep && ok; ++d) ok = in[i]->shape[d] == a->shape[d];
+    if (!ok) return fail(ctx, HGPU_ERR_INVALID, "contract_map: input %d does not have the kept shape", i);
+  }
+  if (c_slot < 0) return fail(ctx, HGPU_ERR_INVALID, "contract_map: no input stands for the contraction");
+  // slot types: the contraction's slot has the operands' dtype
+  std::vector<int> dt;
+  {
+    std::vector<const hgpu_array*> tin(in, in + n_in);
+    tin[(size_t)c_slot] = a;   // only the dtype is read
+    if (int rc = check_program(ctx, n_in, tin.data(), n_instr, prog, &dt)) return rc;
+  }
+  for (int o = 0; o < n_out; ++o)
+    if (out_slots[o] < 0 || out_slots[o] >= n_in + n_instr) return fail(ctx, HGPU_ERR_INVALID, "contract_map: bad output slot");
+  int64_t n_kept = 1;
+  for (int d = 0; d < n_keep; ++d) n_kept *= a->shape[d];
+  if (values) {
+    if (ext_slot < 0 || ext_slot >= n_in + n_instr) return fail(ctx, HGPU_ERR_INVALID, "contract_map: bad extremum slot");
+    if (view_rank < 1 || view_rank > HGPU_MAX_RANK || !view_shape || !view_strides || n_reduce < 1 || n_reduce > view_rank)
+      return fail(ctx, HGPU_ERR_INVALID, "contract_map: bad view");
+    int64_t hi = 0;
+    for (int j = 0; j < view_rank; ++j) {
+      if (view_shape[j] < 1 || view_strides[j] < 0) return fail(ctx, HGPU_ERR_INVALID, "contract_map: the view must have positive extents and no negative strides");
+      hi += (view_shape[j] - 1) * view_strides[j];
+    }
+    if (hi >= n_kept) return fail(ctx, HGPU_ERR_INVALID, "contract_map: the view leaves the result");
+  }
+  if (n_kept > 0) {
+    bool handled = false;
+    int rc = try_contract_map(ctx, a, b, n_keep, n_in, in, c_slot, n_instr, prog, dt, n_out, out_slots, outs, ext_slot, view_rank, view_shape, view_strides, n_reduce,
+                              want_max, values, indices, &handled);
+    if (rc || handled) return rc;
+  }
+  // one entry point after another
+  hgpu_array* c = nullptr;
+  int rc = hgpu_contract(ctx, a, b, n_keep, &c);
+  if (rc) return rc;
+  std::vector<const hgpu_array*> ins(in, in + n_in);
+  ins[(size_t)c_slot] = c;
+  std::vector<int> slots(out_slots, out_slots + n_out);
+  if (values) slots.push_back(ext_slot);
+  std::vector<hgpu_array*> res(slots.size(), nullptr);
+  auto release_res = [&] { for (auto*& r : res) if (r) { hgpu_release(r); r = nullptr; } };
+  // slots that are inputs are copied, the others come out of one fused pass
+  std::vector<int> fslots;
+  std::vector<size_t> fpos;
+  for (size_t i = 0; i < slots.size() && !rc; ++i) {
+    if (slots[i] < n_in) rc = hgpu_materialize(ctx, ins[(size_t)slots[i]], &res[i]);
+    else { fslots.push_back(slots[i]); fpos.push_back(i); }
+  }
+  if (!rc && !fslots.empty()) {
+    std::vector<hgpu_array*> fres(fslots.size(), nullptr);
+    rc = hgpu_fused_map(ctx, n_in, ins.data(), n_instr, prog, (int)fslots.size(), fslots.data(), fres.data());
+    if (!rc) for (size_t i = 0; i < fpos.size(); ++i) res[fpos[i]] = fres[i];
+  }
+  hgpu_release(c);
+  if (rc) { release_res(); return rc; }
+  if (values) {
+    hgpu_array *vw = nullptr, *flat = nullptr;
+    rc = hgpu_as_strided(ctx, res.back(), view_rank, view_shape, view_strides, 0, &vw);
+    if (!rc) {
+      int64_t sh[HGPU_MAX_RANK];
+      const int rl = view_rank - n_reduce;
+      int64_t L = 1;
+      for (int j = 0; j < rl; ++j) sh[j] = view_shape[j];
+      for (int j = rl; j < view_rank; ++j) L *= view_shape[j];
+      sh[rl] = L;
+      rc = hgpu_reshape(ctx, vw, rl + 1, sh, &flat);
+      hgpu_release(vw);
+    }
+    if (!rc) {
+      rc = hgpu_extremum_last(ctx, flat, want_max, values, indices);
+      hgpu_release(flat);
+    }
+    hgpu_release(res.back());
+    res.back() = nullptr;
+    if (rc) { release_res(); return rc; }
+  }
+  for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
+  return HGPU_OK;
+}

@@ -19,100 +19,13 @@
 #include <sstream>
 
 #include "common.hpp"
+#include "fused_gen.hpp"
 
 using namespace hg;
 
 namespace {
 
-const char* ctype(int dt) {
-  switch (dt) {
-    case HGPU_F64: return "double";
-    case HGPU_F32: return "float";
-    case HGPU_I64: return "long long";
-    case HGPU_I32: return "int";
-    case HGPU_I16: return "short";
-    case HGPU_I8: return "signed char";
-    case HGPU_BOOL: return "unsigned char";
-  }
-  return "void";
-}
-
-// The device-side semantics of the opcodes: the same rules as the eager
-// kernels (signum of floats keeps zeros, quotH / remH divisor-0 rules, floor).
-const char* kPrelude = R"HG(
-typedef long long i64;
-template <typename T> struct is_fp { static constexpr bool value = false; };
-template <> struct is_fp<double> { static constexpr bool value = true; };
-template <> struct is_fp<float> { static constexpr bool value = true; };
-template <int OP, typename T> __device__ __forceinline__ T op1(T x) {
-  if constexpr (is_fp<T>::value) {
-    if constexpr (OP == 0) return -x;
-    else if constexpr (OP == 1) return fabs(x);
-    else if constexpr (OP == 2) return x > T(0) ? T(1) : (x < T(0) ? T(-1) : x);
-    else if constexpr (OP == 3) return T(1) / x;
-    else if constexpr (OP == 4) return exp(x);
-    else if constexpr (OP == 5) return log(x);
-    else if constexpr (OP == 6) return sqrt(x);
-    else if constexpr (OP == 7) return sin(x);
-    else if constexpr (OP == 8) return cos(x);
-    else if constexpr (OP == 9) return tan(x);
-    else if constexpr (OP == 10) return asin(x);
-    else if constexpr (OP == 11) return acos(x);
-    else if constexpr (OP == 12) return atan(x);
-    else if constexpr (OP == 13) return sinh(x);
-    else if constexpr (OP == 14) return cosh(x);
-    else if constexpr (OP == 15) return tanh(x);
-    else if constexpr (OP == 16) return asinh(x);
-    else if constexpr (OP == 17) return acosh(x);
-    else if constexpr (OP == 18) return atanh(x);
-    else return x;
-  } else {
-    if constexpr (OP == 0) return (T)(-x);
-    else if constexpr (OP == 1) return x < 0 ? (T)(-x) : x;
-    else if constexpr (OP == 2) return x > 0 ? T(1) : (x < 0 ? T(-1) : T(0));
-    else if constexpr (OP == 19) return (T)(x == 0 ? 1 : 0);
-    else return x;
-  }
-}
-template <int OP, typename T> __device__ __forceinline__ T op2(T x, T y) {
-  if constexpr (is_fp<T>::value) {
-    if constexpr (OP == 0) return x + y;
-    else if constexpr (OP == 1) return x * y;
-    else if constexpr (OP == 2) return x - y;
-    else if constexpr (OP == 3) return x / y;
-    else if constexpr (OP == 4) return pow(x, y);
-    else if constexpr (OP == 5) return log(y) / log(x);
-    else if constexpr (OP == 6) return atan2(x, y);
-    else if constexpr (OP == 10) return x <= y ? x : y;
-    else if constexpr (OP == 11) return x >= y ? x : y;
-    else return x;
-  } else {
-    if constexpr (OP == 0) return (T)(x + y);
-    else if constexpr (OP == 1) return (T)(x * y);
-    else if constexpr (OP == 2) return (T)(x - y);
-    else if constexpr (OP == 7) return y == 0 ? x : (T)(x / y);
-    else if constexpr (OP == 8) return y == 0 ? T(0) : (T)(x % y);
-    else if constexpr (OP == 9) return y == 0 ? x : (T)(x % y);
-    else if constexpr (OP == 10) return x <= y ? x : y;
-    else if constexpr (OP == 11) return x >= y ? x : y;
-    else if constexpr (OP == 12) return (T)((x != 0 && y != 0) ? 1 : 0);
-    else return x;
-  }
-}
-template <int OP, typename T> __device__ __forceinline__ unsigned char cmp2(T x, T y) {
-  if constexpr (OP == 0) return x <= y;
-  else if constexpr (OP == 1) return x == y;
-  else return x < y;
-}
-template <int MODE, typename D, typename S> __device__ __forceinline__ D conv(S x) {
-  if constexpr (is_fp<S>::value && !is_fp<D>::value) {
-    if constexpr (MODE == 1) return (D)(i64)floor((double)x);
-    else return (D)(i64)x;
-  } else {
-    return (D)x;
-  }
-}
-)HG";
+using namespace hg::fusedgen;
 
 struct Compiled {
   hipModule_t mod;
@@ -144,67 +57,6 @@ struct FDims {
   int64_t shape[HG_KDIMS];
   int64_t st[kMaxIn][HG_KDIMS];
 };
-
-// Slot types of a program, with the same checks the eager entry points make.
-int check_program(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, std::vector<int>* dtp) {
-  std::vector<int>& dt = *dtp;
-  dt.assign((size_t)(n_in + n_instr), 0);
-  for (int i = 0; i < n_in; ++i) dt[(size_t)i] = in[i]->dtype;
-  for (int k = 0; k < n_instr; ++k) {
-    const hgpu_fused_instr& q = prog[k];
-    int self = n_in + k;
-    auto ok = [&](int s) { return s >= 0 && s < self; };
-    switch (q.kind) {
-      case HGPU_FUSED_OP1:
-        if (!ok(q.a) || q.op < 0 || q.op >= HGPU_OP1_COUNT) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad unary instruction %d", k);
-        if (q.op >= HGPU_RECIP && q.op <= HGPU_ATANH && !dtype_is_float(dt[(size_t)q.a])) return fail(ctx, HGPU_ERR_INVALID, "fused_map: floating opcode on a non-floating operand");
-        if ((q.op == HGPU_NOT) != (dt[(size_t)q.a] == HGPU_BOOL)) return fail(ctx, HGPU_ERR_INVALID, "fused_map: Bool mismatch");
-        dt[(size_t)self] = dt[(size_t)q.a];
-        break;
-      case HGPU_FUSED_OP2:
-        if (!ok(q.a) || !ok(q.b) || q.op < 0 || q.op >= HGPU_OP2_COUNT || dt[(size_t)q.a] != dt[(size_t)q.b]) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad binary instruction %d", k);
-        if (q.op >= HGPU_DIV && q.op <= HGPU_ATAN2 && !dtype_is_float(dt[(size_t)q.a])) return fail(ctx, HGPU_ERR_INVALID, "fused_map: floating opcode on a non-floating operand");
-        if (q.op >= HGPU_QUOT && q.op <= HGPU_REM_SCALAR && !dtype_is_int(dt[(size_t)q.a])) return fail(ctx, HGPU_ERR_INVALID, "fused_map: integral opcode on a non-integral operand");
-        if ((q.op == HGPU_AND) != (dt[(size_t)q.a] == HGPU_BOOL)) return fail(ctx, HGPU_ERR_INVALID, "fused_map: Bool mismatch");
-        dt[(size_t)self] = dt[(size_t)q.a];
-        break;
-      case HGPU_FUSED_CMP:
-        if (!ok(q.a) || !ok(q.b) || q.op < HGPU_LEQ || q.op > HGPU_LT || dt[(size_t)q.a] != dt[(size_t)q.b]) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad comparison %d", k);
-        dt[(size_t)self] = HGPU_BOOL;
-        break;
-      case HGPU_FUSED_SELECT:
-        if (!ok(q.a) || !ok(q.b) || !ok(q.c) || dt[(size_t)q.a] != HGPU_BOOL || dt[(size_t)q.b] != dt[(size_t)q.c]) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad select %d", k);
-        dt[(size_t)self] = dt[(size_t)q.b];
-        break;
-      case HGPU_FUSED_CONVERT:
-        if (!ok(q.a) || dtype_size(q.dtype) == 0) return fail(ctx, HGPU_ERR_INVALID, "fused_map: bad conversion %d", k);
-        if (q.op == HGPU_CONV_FLOOR && !(dtype_is_float(dt[(size_t)q.a]) && dtype_is_int(q.dtype))) return fail(ctx, HGPU_ERR_INVALID, "fused_map: floor needs float -> int");
-        dt[(size_t)self] = q.dtype;
-        break;
-      default:
-        return fail(ctx, HGPU_ERR_INVALID, "fused_map: unknown instruction kind %d", q.kind);
-    }
-  }
-  return HGPU_OK;
-}
-
-// One instruction per line: `const T v<slot><suffix> = ...;`
-void emit_program(std::ostringstream& s, int n_in, int n_instr, const hgpu_fused_instr* prog, const std::vector<int>& dt, const char* ind, const std::string& lane_suffix) {
-  for (int k = 0; k < n_instr; ++k) {
-    const hgpu_fused_instr& q = prog[k];
-    int self = n_in + k;
-    auto v = [&](int slot) { return "v" + std::to_string(slot) + lane_suffix; };
-    s << ind << "const " << ctype(dt[(size_t)self]) << " " << v(self) << " = ";
-    switch (q.kind) {
-      case HGPU_FUSED_OP1: s << "op1<" << q.op << ">(" << v(q.a) << ")"; break;
-      case HGPU_FUSED_OP2: s << "op2<" << q.op << ">(" << v(q.a) << ", " << v(q.b) << ")"; break;
-      case HGPU_FUSED_CMP: s << "cmp2<" << q.op << ">(" << v(q.a) << ", " << v(q.b) << ")"; break;
-      case HGPU_FUSED_SELECT: s << "(" << v(q.a) << " ? " << v(q.b) << " : " << v(q.c) << ")"; break;
-      default: s << "conv<" << q.op << ", " << ctype(q.dtype) << ">(" << v(q.a) << ")"; break;
-    }
-    s << ";\n";
-  }
-}
 
 }  // namespace
 

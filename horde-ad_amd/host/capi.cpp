@@ -263,6 +263,11 @@ int hh_ix_argminmax(hh_ctx* c, hh_val* t, int n, hh_ix* const* ix, int want_max,
 }
 int hh_ix_free(hh_ix* x) { delete x; return HGPU_OK; }
 int hh_ix_is_affine(hh_ix* x) { return x && x->x.affine ? 1 : 0; }
+int64_t hh_counter(hh_ctx* c, const char* name) {
+  if (!c || !name) return -1;
+  auto it = c->be.counters.find(name);
+  return it == c->be.counters.end() ? 0 : it->second;
+}
 
 int hh_tsgather(hh_ctx* c, hh_val* src, int rank_m, const int64_t* shm, int n_ix, hh_ix* const* ix, hh_val** out) {
   HH_OP(d_tsgather(c->tape, src->d, mk(rank_m, shm), ixs(n_ix, ix)));

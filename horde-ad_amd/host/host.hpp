@@ -36,7 +36,15 @@ struct Backend {
   std::map<std::pair<int, int64_t>, std::shared_ptr<ArrHolder>> iota_cache;   // (dtype, n)
   std::map<std::pair<int, uint64_t>, std::shared_ptr<ArrHolder>> const_cache; // (dtype, value bits)
   bool fuse = true;   // defer elementwise operations into fused programs (when the provider has fused_map)
+  std::map<std::string, int64_t> counters;   // how often each rewrite onto a fused entry point was taken (diagnostic)
   void check(int rc) const;
+};
+
+// Shape, element strides and offset of a strided view over the dense row-major
+// layout of some value.
+struct Meta {
+  Shape shape, strides;
+  int64_t offset = 0;
 };
 
 struct ArrHolder {
@@ -95,6 +103,18 @@ struct ArrHolder {
   // the extremal values the same pass produced: `sindex0 t [kargMin t]` (the
   // minimum of the reference's soft-max loss) is then those values, not a gather.
   std::shared_ptr<ArrHolder> arg_src, arg_values;
+  // A pending VIEW (h == nullptr, ekind < 0, vsrc set): the strided view vmeta
+  // over the dense row-major result of vsrc, a value that is itself still
+  // pending (a contraction, an elementwise expression).  Views of it compose
+  // on the host; it is computed by computing vsrc once and viewing that.  An
+  // elementwise expression made by viewing the leaves of another one (ekind >= 0)
+  // carries the same two fields as a note: it equals that view of vsrc's result.
+  std::shared_ptr<ArrHolder> vsrc;
+  Meta vmeta;
+  // A stand-in without data that view operations are tried on to learn the
+  // strides they produce (vmeta holds its shape and strides).
+  bool probe = false;
+  int probe_dtype = 0;
   ArrHolder(Backend* b, hgpu_array* a) : be(b), h(a) {}
   ~ArrHolder() { if (h) be->api->release(h); }
   ArrHolder(const ArrHolder&) = delete;
@@ -116,6 +136,9 @@ class T {
     return p_->h;
   }
   bool pending_expr() const { return p_ && !p_->h && p_->ekind >= 0; }
+  bool is_probe() const { return p_ && p_->probe; }
+  bool pending_view() const { return p_ && !p_->h && p_->ekind < 0 && p_->vsrc && !p_->probe; }
+  bool meta_only() const { return is_probe() || pending_view(); }   // shape and strides known on the host, no array yet
   bool pending_product() const { return pending_expr() && p_->ekind == HGPU_FUSED_OP2 && p_->eop == HGPU_MUL; }
   bool pending_pieces() const { return p_ && !p_->h && !p_->pieces.empty(); }
   bool pending_merged() const { return p_ && !p_->h && p_->mv_inner; }
@@ -131,12 +154,15 @@ class T {
     return q->h;
   }
   int rank() const {
+    if (meta_only()) return (int)p_->vmeta.shape.size();
     if (pending_pieces()) return (int)p_->pshape.size();
     if (pending_merged()) return (int)p_->mv_shape.size();
     if (pending_expr()) return (int)p_->eshape.size();
     return contraction_like() ? p_->keep : be()->api->rank(meta_h());
   }
   int dtype() const {
+    if (is_probe()) return p_->probe_dtype;
+    if (pending_view()) return T(p_->vsrc).dtype();
     if (pending_pieces()) return p_->pdtype;
     if (pending_merged()) return T(p_->mv_inner).dtype();
     return pending_expr() ? p_->edtype : T(p_->fa ? p_->fa : p_).dtype_of_holder();

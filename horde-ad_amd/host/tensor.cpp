@@ -15,6 +15,7 @@ void Backend::check(int rc) const {
 }
 
 Shape T::shape() const {
+  if (meta_only()) return p_->vmeta.shape;
   if (pending_pieces()) return p_->pshape;
   if (pending_merged()) return p_->mv_shape;
   if (pending_expr()) return p_->eshape;
@@ -27,6 +28,7 @@ Shape T::shape() const {
   return s;
 }
 Shape T::strides() const {
+  if (meta_only()) return p_->vmeta.strides;   // over the dense result of the source: what its array will have
   Shape s((size_t)rank());
   if (!s.empty()) be()->api->strides(h(), s.data());
   return s;
@@ -106,6 +108,155 @@ T iota(Backend* be, int64_t n, int dtype) {
   return t;
 }
 
+// ---- views known on the host only: probes and pending views -----------------
+
+namespace {
+struct ProbeFail {};   // a view operation that cannot be expressed by strides alone was tried on a probe
+
+Meta dense_meta(const Shape& sh) {
+  Meta m;
+  m.shape = sh;
+  m.strides.assign(sh.size(), 0);
+  int64_t s = 1;
+  for (size_t i = sh.size(); i-- > 0;) { m.strides[i] = s; s *= sh[i]; }
+  return m;
+}
+
+bool meta_transpose(const Meta& a, const std::vector<int>& perm, Meta* o) {
+  const size_t rank = a.shape.size();
+  if (perm.size() > rank) return false;
+  std::vector<bool> seen(perm.size(), false);
+  *o = a;
+  for (size_t i = 0; i < perm.size(); ++i) {
+    int sdim = perm[i];
+    if (sdim < 0 || sdim >= (int)perm.size() || seen[(size_t)sdim]) return false;
+    seen[(size_t)sdim] = true;
+    o->shape[i] = a.shape[(size_t)sdim];
+    o->strides[i] = a.strides[(size_t)sdim];
+  }
+  return true;
+}
+
+// `shape` as a view of a (the rule of hgpu_reshape: runs of dims that are contiguous among themselves may be split and merged)
+bool meta_reshape(const Meta& a, const Shape& shape, Meta* o) {
+  int64_t na = 1, nn = 1;
+  for (auto e : a.shape) na *= e;
+  for (auto e : shape) nn *= e;
+  if (na != nn || na == 0) return false;
+  Shape rsh, rst;
+  for (size_t i = 0; i < a.shape.size(); ++i) {
+    if (a.shape[i] == 1) continue;
+    if (!rsh.empty() && rst.back() == a.strides[i] * a.shape[i]) { rsh.back() *= a.shape[i]; rst.back() = a.strides[i]; }
+    else { rsh.push_back(a.shape[i]); rst.push_back(a.strides[i]); }
+  }
+  o->shape = shape;
+  o->strides.assign(shape.size(), 0);
+  o->offset = a.offset;
+  size_t r = 0;
+  int64_t rem = rsh.empty() ? 1 : rsh[0];
+  for (size_t i = 0; i < shape.size(); ++i) {
+    int64_t e = shape[i];
+    if (e == 1) continue;
+    if (r >= rsh.size() || rem % e != 0) return false;
+    rem /= e;
+    o->strides[i] = rst[r] * rem;
+    if (rem == 1) { ++r; rem = r < rsh.size() ? rsh[r] : 1; }
+  }
+  return r == rsh.size();
+}
+
+bool meta_slice(const Meta& a, int dim, int64_t start, int64_t len, Meta* o) {
+  if (dim < 0 || dim >= (int)a.shape.size() || start < 0 || len < 0 || start + len > a.shape[(size_t)dim]) return false;
+  *o = a;
+  o->shape[(size_t)dim] = len;
+  o->offset += start * a.strides[(size_t)dim];
+  return true;
+}
+
+bool meta_reverse(const Meta& a, int dim, Meta* o) {
+  if (dim < 0 || dim >= (int)a.shape.size()) return false;
+  *o = a;
+  if (a.shape[(size_t)dim] > 0) o->offset += (a.shape[(size_t)dim] - 1) * a.strides[(size_t)dim];
+  o->strides[(size_t)dim] = -a.strides[(size_t)dim];
+  return true;
+}
+
+bool meta_replicate(const Meta& a, const Shape& pre, Meta* o) {
+  for (auto e : pre)
+    if (e <= 0) return false;
+  o->shape = pre;
+  o->shape.insert(o->shape.end(), a.shape.begin(), a.shape.end());
+  o->strides.assign(pre.size(), 0);
+  o->strides.insert(o->strides.end(), a.strides.begin(), a.strides.end());
+  o->offset = a.offset;
+  return true;
+}
+
+bool meta_index_prefix(const Meta& a, const Shape& ix, Meta* o) {
+  if (ix.size() > a.shape.size()) return false;
+  o->offset = a.offset;
+  for (size_t i = 0; i < ix.size(); ++i) {
+    if (ix[i] < 0 || ix[i] >= a.shape[i]) return false;   // out of bounds means zeros: not a view
+    o->offset += ix[i] * a.strides[i];
+  }
+  o->shape.assign(a.shape.begin() + (long)ix.size(), a.shape.end());
+  o->strides.assign(a.strides.begin() + (long)ix.size(), a.strides.end());
+  return true;
+}
+
+// the elements a view addresses, relative to the start of its source's layout
+void meta_range(const Meta& a, int64_t* lo, int64_t* hi, bool* empty) {
+  *lo = *hi = a.offset;
+  *empty = false;
+  for (size_t i = 0; i < a.shape.size(); ++i) {
+    if (a.shape[i] == 0) { *empty = true; continue; }
+    int64_t span = (a.shape[i] - 1) * a.strides[i];
+    if (span > 0) *hi += span; else *lo += span;
+  }
+}
+
+bool meta_as_strided(const Meta& a, const Shape& shape, const Shape& strides, int64_t offset, Meta* o) {
+  if (shape.size() != strides.size()) return false;
+  o->shape = shape;
+  o->strides = strides;
+  o->offset = a.offset + offset;
+  int64_t lo, hi, alo, ahi;
+  bool e1, e2;
+  meta_range(*o, &lo, &hi, &e1);
+  meta_range(a, &alo, &ahi, &e2);
+  return !e1 && !e2 && lo >= alo && hi <= ahi;   // as hgpu_as_strided: inside what the source view addresses
+}
+}  // namespace
+
+static T make_probe(Backend* be, const Meta& m, int dtype) {
+  auto p = std::make_shared<ArrHolder>(be, nullptr);
+  p->probe = true;
+  p->probe_dtype = dtype;
+  p->vmeta = m;
+  return T(p);
+}
+// The view m over the dense result of the pending value src.
+static T make_view(const std::shared_ptr<ArrHolder>& src, const Meta& m) {
+  auto p = std::make_shared<ArrHolder>(src->be, nullptr);
+  p->vsrc = src;
+  p->vmeta = m;
+  return T(p);
+}
+// a with the strides of m: a probe stays a probe, a pending view stays one of the same source
+static T with_meta(const T& a, const Meta& m) {
+  if (a.is_probe()) return make_probe(a.be(), m, a.dtype());
+  return make_view(a.holder()->vsrc, m);
+}
+// Tries a view operation on strides alone.  A probe that cannot take it gives
+// up (ProbeFail); a pending view falls through to the array path, which
+// computes its source first.
+#define HD_META_VIEW(call)                          \
+  if (a.meta_only()) {                              \
+    Meta m__;                                       \
+    if (call) return with_meta(a, m__);             \
+    if (a.is_probe()) throw ProbeFail{};            \
+  }
+
 #define HD_OUT(call)                      \
   hgpu_array* o__ = nullptr;              \
   Backend* be__ = a.be();                 \
@@ -157,13 +308,31 @@ static T make_expr(int kind, int op, int dtype, const T& a, const T* b, const T*
 namespace {
 struct Program {
   std::vector<const ArrHolder*> inputs;
-  std::vector<std::pair<const ArrHolder*, hgpu_fused_instr>> instrs;   // operands hold holder slots until numbered
+  std::vector<std::pair<ArrHolder*, hgpu_fused_instr>> instrs;   // operands hold holder slots until numbered
   std::map<const ArrHolder*, int> in_slot, instr_slot;
+  // keep_contraction: one pending contraction of two arrays among the leaves
+  // stays as it is (an input without an array), for a kernel that computes it
+  // and runs the program over its result in one pass
+  bool keep_contraction = false;
+  ArrHolder* kept = nullptr;
 };
+
+bool single_contraction(const ArrHolder* p) {
+  return !p->h && p->ekind < 0 && p->fa && p->fb && p->keep >= 1 && p->more.empty() && !p->origin && !p->vsrc && p->pieces.empty() && !p->mv_inner;
+}
 
 // Post-order walk: materialised values (and pending contractions, which are
 // forced here) become inputs, pending elementwise nodes become instructions.
 int visit(Program& pg, ArrHolder* p) {
+  if (pg.keep_contraction && single_contraction(p) && (!pg.kept || pg.kept == p)) {
+    pg.kept = p;
+    auto it = pg.in_slot.find(p);
+    if (it != pg.in_slot.end()) return -1 - it->second;
+    int k = (int)pg.inputs.size();
+    pg.inputs.push_back(p);
+    pg.in_slot[p] = k;
+    return -1 - k;
+  }
   if (!p->h && p->ekind < 0) p->force();   // a pending contraction, concatenation or refined expression
   if (p->h) {
     auto it = pg.in_slot.find(p);
@@ -190,9 +359,12 @@ int visit(Program& pg, ArrHolder* p) {
 }  // namespace
 
 // The roots' expressions as one numbered program: inputs, instructions, and the slot of every root.
+// With `kept`: one pending contraction among the leaves stays pending (*kept; its
+// entry of ins is null), and nodes receives the holder of every instruction.
 static void number_program(const std::vector<ArrHolder*>& roots, std::vector<const hgpu_array*>* ins, std::vector<hgpu_fused_instr>* prog,
-                           std::vector<int>* outs_slot) {
+                           std::vector<int>* outs_slot, ArrHolder** kept = nullptr, std::vector<ArrHolder*>* nodes = nullptr) {
   Program pg;
+  pg.keep_contraction = kept != nullptr;
   std::vector<int> root_slot;
   for (auto* r : roots) root_slot.push_back(visit(pg, r));
   int n_in = (int)pg.inputs.size();
@@ -206,6 +378,9 @@ static void number_program(const std::vector<ArrHolder*>& roots, std::vector<con
   }
   for (auto* p : pg.inputs) ins->push_back(p->h);
   for (int v : root_slot) outs_slot->push_back(slot(v));
+  if (kept) *kept = pg.kept;
+  if (nodes)
+    for (auto& pi : pg.instrs) nodes->push_back(pi.first);
 }
 
 static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
@@ -222,6 +397,7 @@ static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
     r->fa.reset();
     r->fb.reset();
     r->fc.reset();
+    r->vsrc.reset();
     r->ekind = -1;
   }
 }
@@ -288,6 +464,26 @@ void force_many(const std::vector<T>& ts) {
 
 void ArrHolder::force() {
   if (h) return;
+  if (probe) throw ProbeFail{};
+  if (vsrc && ekind < 0) {   // a pending view: its source once, for every view of it, then the strides
+    T s(vsrc);
+    hgpu_array* base = s.h();
+    be->check(be->api->retain(base));
+    if (!be->api->is_dense(base)) {   // vmeta counts in the dense row-major layout of the source
+      hgpu_array* d = nullptr;
+      int rc = be->api->materialize(be->ctx, base, &d);
+      be->api->release(base);
+      be->check(rc);
+      base = d;
+    }
+    hgpu_array* o = nullptr;
+    int rc = be->api->as_strided(be->ctx, base, (int)vmeta.shape.size(), ptr_or_dummy(vmeta.shape), ptr_or_dummy(vmeta.strides), vmeta.offset, &o);
+    be->api->release(base);
+    be->check(rc);
+    h = o;
+    vsrc.reset();
+    return;
+  }
   if (mv_inner) {   // the refined expression written out densely, its dims merged (a view)
     T in(mv_inner);
     hgpu_array* o = nullptr;
@@ -419,8 +615,14 @@ static T map_leaves(const T& a, const std::function<T(const T&)>& view) {
     if (it != memo.end()) return it->second;
     std::shared_ptr<ArrHolder> r;
     if (p->h || p->ekind < 0) {
-      if (!p->h) p->force();   // a pending contraction among the leaves is computed once, for every view of it
-      r = view(T(p)).holder();
+      // A pending contraction among the leaves is computed once, for every view
+      // of it -- but not yet: the view stays pending (strides over its dense
+      // result), so that whoever consumes the viewed expression may still take
+      // the contraction in with it.
+      T leaf(p);
+      if (!p->h && p->ekind < 0 && p->fa && p->keep >= 0 && T(p).size() > 0) leaf = make_view(p, dense_meta(T(p).shape()));
+      else if (!p->h && !leaf.pending_view()) p->force();
+      r = view(leaf).holder();
     } else {
       r = std::make_shared<ArrHolder>(p->be, nullptr);
       r->ekind = p->ekind;
@@ -435,7 +637,20 @@ static T map_leaves(const T& a, const std::function<T(const T&)>& view) {
     memo[p.get()] = r;
     return r;
   };
-  return T(go(a.holder()));
+  T res(go(a.holder()));
+  // the note: res equals this view of the dense result of the expression it was made from
+  if (res.pending_expr() && !a.is_probe()) {
+    const ArrHolder* ah = a.holder().get();
+    try {
+      T pr = view(make_probe(a.be(), ah->vsrc ? ah->vmeta : dense_meta(a.shape()), a.dtype()));
+      if (pr.is_probe() && pr.shape() == res.shape()) {
+        res.holder()->vsrc = ah->vsrc ? ah->vsrc : a.holder();
+        res.holder()->vmeta = pr.holder()->vmeta;
+      }
+    } catch (ProbeFail&) {
+    }
+  }
+  return res;
 }
 #define HD_VIEW_OF_EXPR(call) \
   if (a.pending_expr()) return map_leaves(a, [&](const T& x) { return call; });
@@ -520,6 +735,7 @@ T transpose(const T& a, const std::vector<int>& perm) {
     }
     return make_merged(transpose(T(h->mv_inner), fine_perm), shape, groups);
   }
+  HD_META_VIEW(meta_transpose(a.holder()->vmeta, perm, &m__))
   HD_VIEW_OF_EXPR(transpose(x, perm))
   if (a.pending_contraction() && (int)perm.size() <= a.pending_keep())   // permutes kept dims only
   {
@@ -532,6 +748,7 @@ T transpose(const T& a, const std::vector<int>& perm) {
   HD_OUT(transpose(be__->ctx, a.h(), (int)perm.size(), perm.empty() ? &dummy : perm.data(), &o__));
 }
 T reshape(const T& a, const Shape& s) {
+  HD_META_VIEW(meta_reshape(a.holder()->vmeta, s, &m__))
   if (a.pending_expr() && s != a.shape()) {   // only splits dims: a view of every leaf
     std::vector<int> g;
     if (refines(s, a.shape(), &g)) return map_leaves(a, [&](const T& x) { return reshape(x, s); });
@@ -542,28 +759,37 @@ T reshape(const T& a, const Shape& s) {
 }
 T slice(const T& a, int dim, int64_t start, int64_t len) {
   if (dim == 0 && a.pending_pieces() && start >= 0 && len >= 0 && start + len <= a.shape().at(0)) return slice_pieces(a, start, len);
+  HD_META_VIEW(meta_slice(a.holder()->vmeta, dim, start, len, &m__))
   HD_VIEW_OF_EXPR(slice(x, dim, start, len))
   HD_OUT(slice(be__->ctx, a.h(), dim, start, len, &o__));
 }
 T reverse(const T& a, int dim) {
+  HD_META_VIEW(meta_reverse(a.holder()->vmeta, dim, &m__))
   HD_VIEW_OF_EXPR(reverse(x, dim))
   HD_OUT(reverse(be__->ctx, a.h(), dim, &o__));
 }
 T replicate(const T& a, const Shape& pre) {
   if (pre.empty()) return a;
+  HD_META_VIEW(meta_replicate(a.holder()->vmeta, pre, &m__))
   // a pending expression is written out before it is replicated: only shrinking
   // or permuting views of it are worth keeping pending
   HD_OUT(replicate(be__->ctx, a.h(), (int)pre.size(), pre.data(), &o__));
 }
 T index_prefix(const T& a, const Shape& ix) {
+  HD_META_VIEW(meta_index_prefix(a.holder()->vmeta, ix, &m__))
   HD_VIEW_OF_EXPR(index_prefix(x, ix))
   HD_OUT(index_prefix(be__->ctx, a.h(), (int)ix.size(), ptr_or_dummy(ix), &o__));
 }
 T as_strided(const T& a, const Shape& shape, const Shape& strides, int64_t offset) {
+  HD_META_VIEW(meta_as_strided(a.holder()->vmeta, shape, strides, offset, &m__))
   HD_OUT(as_strided(be__->ctx, a.h(), (int)shape.size(), ptr_or_dummy(shape), ptr_or_dummy(strides), offset, &o__));
 }
-T materialize(const T& a) { HD_OUT(materialize(be__->ctx, a.h(), &o__)); }
+T materialize(const T& a) {
+  if (a.is_probe()) throw ProbeFail{};
+  HD_OUT(materialize(be__->ctx, a.h(), &o__));
+}
 T pad(const T& a, const Shape& lo, const Shape& hi) {
+  if (a.is_probe()) throw ProbeFail{};
   // zeros before and after along the first dim only: a pending concatenation
   bool first_only = a.be()->fuse && a.rank() >= 1 && (int)lo.size() == a.rank() && (int)hi.size() == a.rank() && lo[0] >= 0 && hi[0] >= 0 && lo[0] + hi[0] > 0;
   for (size_t i = 1; i < lo.size() && first_only; ++i) first_only = lo[i] == 0 && hi[i] == 0;
@@ -1424,6 +1650,90 @@ Ix ix_index0(Backend* be, const T& t, const std::vector<Ix>& ix) {
   return from_array(shm, gather_raw(t, arrs, shm));
 }
 
+// `inner` (a pending expression over [lead.., reduced..]) is noted to be a view
+// of an expression whose leaves are arrays and ONE pending contraction of the
+// expression's own shape.  Then hgpu_contract_map computes the contraction, the
+// expression over it and the first extremum over the view's trailing n_reduce
+// dims as one kernel.  Returns false when the pattern or the provider does not fit.
+static bool contract_map_extremum(Backend* be, const T& inner, int n_reduce, bool want_max, const Shape& shm, const Shape& lead, Ix* out) {
+  const hgpu_api* api = be->api;
+  if (!(api->struct_size >= offsetof(hgpu_api, contract_map) + sizeof(api->contract_map) && api->contract_map)) return false;
+  const ArrHolder* ih = inner.holder().get();
+  if (!ih->vsrc || ih->vmeta.offset != 0 || ih->vmeta.shape != inner.shape()) return false;
+  T origin(ih->vsrc);
+  if (!origin.pending_expr() || pending_size(origin.holder()) > 40) return false;
+  // is there exactly one pending contraction among the leaves?  (look before anything is forced)
+  {
+    std::map<const ArrHolder*, int> seen;
+    std::vector<const ArrHolder*> stack{origin.holder().get()};
+    int n_contr = 0;
+    while (!stack.empty()) {
+      const ArrHolder* p = stack.back();
+      stack.pop_back();
+      if (seen.count(p)) continue;
+      seen[p] = 1;
+      if (single_contraction(p)) { ++n_contr; continue; }
+      if (p->h || p->ekind < 0) continue;
+      if (p->fa) stack.push_back(p->fa.get());
+      if (p->fb) stack.push_back(p->fb.get());
+      if (p->fc) stack.push_back(p->fc.get());
+    }
+    if (n_contr != 1) return false;
+  }
+  std::vector<const hgpu_array*> ins;
+  std::vector<hgpu_fused_instr> prog;
+  std::vector<int> slots;
+  std::vector<ArrHolder*> nodes;
+  ArrHolder* kept = nullptr;
+  number_program({origin.holder().get()}, &ins, &prog, &slots, &kept, &nodes);
+  if (!kept || (int)ins.size() > 12 || (int)prog.size() > 96) {
+    if (kept) kept->force();
+    return false;
+  }
+  T fa(kept->fa), fb(kept->fb);
+  if (fa.shape() != fb.shape() || fa.dtype() != fb.dtype() || (fa.dtype() != HGPU_F64 && fa.dtype() != HGPU_F32)) return false;
+  // Bool results that depend on the contraction are written out as well
+  const int n_in = (int)ins.size();
+  int c_slot = -1;
+  for (int i = 0; i < n_in; ++i)
+    if (!ins[(size_t)i]) c_slot = i;
+  std::vector<char> dep((size_t)n_in + prog.size(), 0);
+  dep[(size_t)c_slot] = 1;
+  std::vector<int> out_slots;
+  std::vector<ArrHolder*> out_nodes;
+  for (size_t k = 0; k < prog.size(); ++k) {
+    const hgpu_fused_instr& q = prog[k];
+    bool d = dep[(size_t)q.a] != 0;
+    if (q.kind == HGPU_FUSED_OP2 || q.kind == HGPU_FUSED_CMP) d = d || dep[(size_t)q.b];
+    if (q.kind == HGPU_FUSED_SELECT) d = d || dep[(size_t)q.b] || dep[(size_t)q.c];
+    dep[(size_t)n_in + k] = d;
+    const bool is_bool = q.kind == HGPU_FUSED_CMP || nodes[k]->edtype == HGPU_BOOL;
+    if (d && is_bool && (int)out_slots.size() < 4 && n_in + (int)k != slots[0]) { out_slots.push_back(n_in + (int)k); out_nodes.push_back(nodes[k]); }
+  }
+  std::vector<hgpu_array*> outs(out_slots.size() + 1, nullptr);
+  hgpu_array *vals = nullptr, *idx = nullptr;
+  int rc = api->contract_map(be->ctx, fa.h(), fb.h(), kept->keep, n_in, ins.data(), (int)prog.size(), prog.data(), (int)out_slots.size(), out_slots.data(),
+                             outs.data(), slots[0], (int)ih->vmeta.shape.size(), ptr_or_dummy(ih->vmeta.shape), ptr_or_dummy(ih->vmeta.strides), n_reduce,
+                             want_max ? 1 : 0, &vals, &idx);
+  be->check(rc);
+  be->counters["contract_map"]++;
+  for (size_t i = 0; i < out_nodes.size(); ++i) {
+    ArrHolder* r = out_nodes[i];
+    r->h = outs[i];
+    r->fa.reset();
+    r->fb.reset();
+    r->fc.reset();
+    r->vsrc.reset();
+    r->ekind = -1;
+  }
+  *out = Ix();
+  out->shm = shm;
+  out->arr = reshape(T(be, idx), lead);
+  out->dtype = HGPU_I64;
+  out->arg_vals = reshape(T(be, vals), lead);
+  return true;
+}
+
 Ix ix_argminmax(Backend* be, const T& t, const std::vector<Ix>& ix, bool want_max) {
   if ((int)ix.size() + 1 != t.rank()) throw HostError(HGPU_ERR_INVALID, "ix_argminmax: the partial index must leave one dim");
   if (ix.empty()) throw HostError(HGPU_ERR_INVALID, "ix_argminmax: no position space");
@@ -1448,6 +1758,18 @@ Ix ix_argminmax(Backend* be, const T& t, const std::vector<Ix>& ix, bool want_ma
     T inner(mh->mv_inner);
     if (n_reduce >= 1 && inner.pending_expr() && tsh.back() <= 64 && inner.size() / tsh.back() < (int64_t(1) << 31) &&
         pending_size(inner.holder()) <= 40) {
+      // The expression is a view of another one that sits right on a pending
+      // contraction (windows of relu (conv + bias)): the contraction, the
+      // expression and the extremum in one pass.  The convolution's own result is
+      // never written; the Bool values computed on the way (the relu mask) are, for
+      // whoever differentiates the expression later.
+      {
+        Ix r;
+        if (contract_map_extremum(be, inner, n_reduce, want_max, shm, Shape(tsh.begin(), tsh.end() - 1), &r)) {
+          r.arg_of = t.holder();
+          return r;
+        }
+      }
       std::vector<const hgpu_array*> ins;
       std::vector<hgpu_fused_instr> prog;
       std::vector<int> slots;

@@ -35,7 +35,7 @@ SIG = {
     "ix_op1": (I, [P, I, P, PP]), "ix_op2": (I, [P, I, P, P, PP]), "ix_compare": (I, [P, I, P, P, PP]),
     "ix_select": (I, [P, P, P, P, PP]), "ix_convert": (I, [P, P, I, I, PP]),
     "ix_index0": (I, [P, P, I, PP, PP]), "ix_argminmax": (I, [P, P, I, PP, I, PP]), "ix_free": (I, [P]),
-    "ix_is_affine": (I, [P]),
+    "ix_is_affine": (I, [P]), "counter": (L, [P, C.c_char_p]),
     "tsgather": (I, [P, P, I, LP, I, PP, PP]), "tsscatter": (I, [P, P, I, I, LP, PP, PP]),
     "capture_begin": (I, [P]), "capture_end": (I, [P, PP]), "graph_launch": (I, [P, P]), "graph_free": (I, [P, P]),
     "force": (I, [P, P]), "overwrite": (I, [P, P, P]), "assign": (I, [P, P, P]),
@@ -113,6 +113,10 @@ class Host:
 
     def set_fusion(self, on):
         self.check(self.dll.hh_set_fusion(self.h, int(on)))
+
+    def counter(self, name):
+        """How often the named rewrite onto a fused entry point was taken (diagnostic)."""
+        return int(self.dll.hh_counter(self.h, name.encode()))
 
     def tape_reset(self):
         self.check(self.dll.hh_tape_reset(self.h))

@@ -249,6 +249,27 @@ int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n
  * pairs share one layout and the whole is a matrix product it is one launch
  * whose K chunks run over all pairs.  Summation order is fixed by the shapes. */
 int hgpu_contract_sum(hgpu_ctx* ctx, int n, const hgpu_array* const* a, const hgpu_array* const* b, int n_keep, hgpu_array** out);
+/* A contraction followed, in the same pass, by an elementwise program over its
+ * result -- `maxPool2dUnpaddedS (reluS (conv2dPreservingS ker x + bias))`
+ * (example/MnistCnnShaped2.hs:45-64, External/CommonShapedOps.hs:33-44,241-260)
+ * reaches the backend as a contraction, `+`, a comparison, a conditional, `*`
+ * and an arg-maximum over windows; this entry point runs them as one kernel
+ * when the shapes allow and never writes the convolution's own result.
+ *   C = hgpu_contract(a, b, n_keep)                       (shape: the kept dims)
+ *   program: as for hgpu_fused_map; exactly one entry of `in` is NULL and
+ *   stands for C, the others are views of the kept shape;
+ *   outs[i] = slot out_slots[i], dense, of the kept shape (n_out may be 0);
+ *   when `values` is not NULL: V = the view (view_rank, view_shape,
+ *   view_strides in elements, offset 0) of the dense row-major result of slot
+ *   ext_slot, and values / indices are the first extremum of V over its
+ *   trailing n_reduce dims, as for hgpu_fused_extremum.
+ * Results equal those of the single entry points applied one after another. */
+int hgpu_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep,
+                      int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
+                      int n_out, const int* out_slots, hgpu_array** outs,
+                      int ext_slot, int view_rank, const int64_t* view_shape, const int64_t* view_strides,
+                      int n_reduce, int want_max, hgpu_array** values, hgpu_array** indices);
+
 /* hgpu_contract for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
  * no counterpart in the reference.  The caller brings the result array `out`
@@ -402,6 +423,8 @@ typedef struct hgpu_api {
   int (*extremum_last)(hgpu_ctx*, const hgpu_array*, int, hgpu_array**, hgpu_array**);
   int (*fused_extremum)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, int, int, hgpu_array**, hgpu_array**);
   int (*fused_sum)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, hgpu_array**);
+  int (*contract_map)(hgpu_ctx*, const hgpu_array*, const hgpu_array*, int, int, const hgpu_array* const*, int, const hgpu_fused_instr*,
+                      int, const int*, hgpu_array**, int, int, const int64_t*, const int64_t*, int, int, hgpu_array**, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

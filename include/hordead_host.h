@@ -159,6 +159,9 @@ int hh_ix_argminmax(hh_ctx* ctx, hh_val* t, int n, hh_ix* const* ix, int want_ma
 int hh_ix_free(hh_ix* x);
 /* 1 when the value is an affine form of the position variables (diagnostic). */
 int hh_ix_is_affine(hh_ix* x);
+/* How many times this context has taken the named rewrite onto a fused entry
+ * point of the provider (diagnostic; "contract_map", "contract_operands"). */
+int64_t hh_counter(hh_ctx* ctx, const char* name);
 
 /* tsgather (Ops.hs:701-705): out[m.., n..] = src[ix(m).., n..], zeros out of bounds. */
 int hh_tsgather(hh_ctx* ctx, hh_val* src, int rank_m, const int64_t* shm, int n_ix, hh_ix* const* ix, hh_val** out);

@@ -726,6 +726,95 @@ int horc_fused_map(hgpu_ctx* c, int n_in, const hgpu_array* const* in, int n_ins
   return rc;
 }
 
+// ---- definitions by composition of the optional fused entry points ----------
+// The checker's own table (horc_get_api) leaves them out, so a host program
+// run on it takes the reference's route (a gather at the arg-extremum, one pass
+// per operation).  horc_get_api_fused offers them, each DEFINED as the single
+// entry points applied one after another, so that the host layer's rewrites
+// onto them can be exercised without a device and compared with the plain table.
+
+int horc_extremum_last(hgpu_ctx* c, const hgpu_array* a, int want_max, hgpu_array** values, hgpu_array** indices) {
+  hgpu_array* ix = nullptr;
+  int rc = horc_argminmax_last(c, a, want_max, &ix);
+  if (rc) return rc;
+  if (values) {
+    std::vector<int64_t> osh(a->shape.begin(), a->shape.end() - 1);
+    hgpu_array* v = make(c, a->dtype, osh);
+    int64_t no = prod(osh), L = a->shape.back();
+    size_t es = dsize(a->dtype);
+    for (int64_t i = 0; i < no; ++i)
+      std::memcpy(v->data.data() + (size_t)i * es, a->data.data() + (size_t)(i * L + ptr<int64_t>(ix)[i]) * es, es);
+    *values = v;
+  }
+  *indices = ix;
+  return HGPU_OK;
+}
+
+// first extremum of `r` over its trailing n_reduce dims taken together
+static int extremum_trailing(hgpu_ctx* c, const hgpu_array* r, int n_reduce, int want_max, hgpu_array** values, hgpu_array** indices) {
+  int rank = (int)r->shape.size();
+  if (n_reduce < 1 || n_reduce > rank) return fail(c, HGPU_ERR_INVALID, "extremum: bad n_reduce");
+  std::vector<int64_t> sh(r->shape.begin(), r->shape.end() - n_reduce);
+  sh.push_back(prod(r->shape, (size_t)(rank - n_reduce)));
+  hgpu_array* flat = nullptr;
+  int rc = horc_reshape(c, r, (int)sh.size(), sh.data(), &flat);
+  if (rc) return rc;
+  rc = horc_extremum_last(c, flat, want_max, values, indices);
+  horc_release(flat);
+  return rc;
+}
+
+int horc_fused_extremum(hgpu_ctx* c, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot, int n_reduce,
+                        int want_max, hgpu_array** values, hgpu_array** indices) {
+  hgpu_array* r = nullptr;
+  int rc = horc_fused_map(c, n_in, in, n_instr, prog, 1, &slot, &r);
+  if (rc) return rc;
+  rc = extremum_trailing(c, r, n_reduce, want_max, values, indices);
+  horc_release(r);
+  return rc;
+}
+
+int horc_fused_sum(hgpu_ctx* c, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot, hgpu_array** out) {
+  hgpu_array* r = nullptr;
+  int rc = horc_fused_map(c, n_in, in, n_instr, prog, 1, &slot, &r);
+  if (rc) return rc;
+  rc = horc_contract(c, r, nullptr, 0, out);
+  horc_release(r);
+  return rc;
+}
+
+int horc_contract_map(hgpu_ctx* c, const hgpu_array* a, const hgpu_array* b, int n_keep, int n_in, const hgpu_array* const* in, int n_instr,
+                      const hgpu_fused_instr* prog, int n_out, const int* out_slots, hgpu_array** outs, int ext_slot, int view_rank,
+                      const int64_t* view_shape, const int64_t* view_strides, int n_reduce, int want_max, hgpu_array** values, hgpu_array** indices) {
+  hgpu_array* cr = nullptr;
+  int rc = horc_contract(c, a, b, n_keep, &cr);
+  if (rc) return rc;
+  std::vector<const hgpu_array*> ins(in, in + n_in);
+  int n_null = 0;
+  for (auto& p : ins)
+    if (!p) { p = cr; ++n_null; }
+  if (n_null != 1) { horc_release(cr); return fail(c, HGPU_ERR_INVALID, "contract_map: exactly one input must stand for the contraction"); }
+  std::vector<int> slots(out_slots, out_slots + n_out);
+  if (values) slots.push_back(ext_slot);
+  std::vector<hgpu_array*> res(slots.size(), nullptr);
+  if (!slots.empty()) rc = horc_fused_map(c, n_in, ins.data(), n_instr, prog, (int)slots.size(), slots.data(), res.data());
+  horc_release(cr);
+  if (rc) return rc;
+  for (int i = 0; i < n_out; ++i) outs[i] = res[(size_t)i];
+  if (values) {
+    hgpu_array* v = nullptr;
+    rc = horc_as_strided(c, res.back(), view_rank, view_shape, view_strides, 0, &v);
+    horc_release(res.back());
+    if (!rc) {
+      rc = extremum_trailing(c, v, n_reduce, want_max, values, indices);
+      horc_release(v);
+    }
+    if (rc)
+      for (int i = 0; i < n_out; ++i) { horc_release(outs[i]); outs[i] = nullptr; }
+  }
+  return rc;
+}
+
 const hgpu_api* horc_get_api(void) {
   static const hgpu_api api = {
       sizeof(hgpu_api),
@@ -741,7 +830,17 @@ const hgpu_api* horc_get_api(void) {
       nullptr,   // no extremum_last: the checker gathers at the arg-extremum as the reference does
       nullptr,   // no fused_extremum
       nullptr,   // no fused_sum
+      nullptr,   // no contract_map
   };
+  return &api;
+}
+
+const hgpu_api* horc_get_api_fused(void) {
+  static hgpu_api api = *horc_get_api();
+  api.extremum_last = horc_extremum_last;
+  api.fused_extremum = horc_fused_extremum;
+  api.fused_sum = horc_fused_sum;
+  api.contract_map = horc_contract_map;
   return &api;
 }
 

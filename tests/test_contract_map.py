@@ -1,0 +1,141 @@
+"""hgpu_contract_map: a contraction, an elementwise program over its result and
+the first extremum over windows of that, in one pass -- the form
+`maxPool2dUnpaddedS (reluS (conv2dPreservingS ker x + bias))` takes
+(example/MnistCnnShaped2.hs:45-64, External/CommonShapedOps.hs:33-44,241-260).
+
+The device results are checked against numpy's convolution, relu and window
+maximum; the host layer's rewrite onto the entry point is checked without a
+device, on the CPU checker's table of fused entry points (each defined there as
+the single entry points applied one after another) against its plain table."""
+import numpy as np
+import pytest
+
+from conftest import capi, entry, pkg
+
+O2, CMP = capi.OP2, capi.CMP
+# slots: 0 = the convolution, 1 = bias, 2 = zeros, 3 = ones; 4 = conv + bias; 5 = (4 <= 0); 6 = 5 ? 0 : 1; 7 = 6 * 4
+RELU = [(1, O2["add"], 0, 0, 1, 0), (2, CMP["leq"], 0, 4, 2, 0), (3, 0, 0, 5, 2, 3), (1, O2["mul"], 0, 6, 4, 0)]
+
+
+def conv_layer(ctx, x, ker, bias, pool=True):
+    """(mask, values, indices, kernel labels) of relu (conv + bias) pooled 2x2, through hgpu_contract_map."""
+    B, Ci, Hp, Wp = x.shape
+    Co, _, kh, kw = ker.shape
+    H, Wd = Hp - kh + 1, Wp - kw + 1
+    dtype = x.dtype
+    gx, gk, gb = ctx.upload(x), ctx.upload(ker), ctx.upload(bias)
+    sh = [B, Co, H, Wd, Ci, kh, kw]
+    a = gx.as_strided(sh, [Ci * Hp * Wp, 0, Wp, 1, Hp * Wp, Wp, 1], 0)      # windows of the zero-extended input
+    b = gk.as_strided(sh, [0, Ci * kh * kw, 0, 0, kh * kw, kw, 1], 0)
+    kept = [B, Co, H, Wd]
+    bias_v = gb.as_strided(kept, [0, 1, 0, 0], 0)
+    zero = ctx.upload(np.zeros((), dtype)).as_strided(kept, [0, 0, 0, 0], 0)
+    one = ctx.upload(np.ones((), dtype)).as_strided(kept, [0, 0, 0, 0], 0)
+    ext = None
+    if pool:
+        ext = (7, [B, Co, H // 2, Wd // 2, 2, 2], [Co * H * Wd, H * Wd, 2 * Wd, 2, Wd, 1], 2, True)
+    ctx.profile(2)
+    outs, vals, idx = ctx.contract_map(a, b, 4, [None, bias_v, zero, one], RELU, [5] if pool else [5, 7], ext)
+    labels = list(ctx.profile_report())
+    ctx.profile(0)
+    return outs, vals, idx, labels
+
+
+def reference(x, ker, bias):
+    kh, kw = ker.shape[2:]
+    win = np.lib.stride_tricks.sliding_window_view(x, (kh, kw), axis=(2, 3))
+    z = np.einsum("bihwpq,oipq->bohw", win.astype(np.float64), ker.astype(np.float64)).astype(x.dtype) + bias[None, :, None, None]
+    r = np.where(z <= 0, 0, 1).astype(x.dtype) * z
+    B, Co, H, Wd = r.shape
+    wv = r.reshape(B, Co, H // 2, 2, Wd // 2, 2).transpose(0, 1, 2, 4, 3, 5).reshape(B, Co, H // 2, Wd // 2, 4)
+    return z, r, wv
+
+
+CASES = [  # B, Ci, Co, H, W, k, dtype, fused kernel expected
+    (300, 1, 16, 28, 28, 5, np.float64, True),
+    (300, 16, 16, 14, 14, 5, np.float64, True),
+    (300, 1, 16, 28, 28, 5, np.float32, True),
+    (130, 3, 8, 12, 20, 3, np.float64, False),     # 8 output channels, short K: composition of the single kernels
+    (7, 2, 4, 8, 8, 3, np.float64, False),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,Ci,Co,H,Wd,k,dtype,fused", CASES)
+def test_conv_relu_pool_in_one_pass(gpu, B, Ci, Co, H, Wd, k, dtype, fused):
+    rng = np.random.default_rng(5)
+    x = np.zeros((B, Ci, H + k - 1, Wd + k - 1), dtype)
+    x[:, :, :H, :Wd] = rng.uniform(-1, 1, (B, Ci, H, Wd))
+    x[0, :, :H, :Wd] = 0.75                      # a constant image: whole windows of equal, positive values (ties)
+    ker = rng.uniform(-0.4, 0.4, (Co, Ci, k, k)).astype(dtype)
+    ker[1] = np.abs(ker[1])                      # ... in channel 1
+    bias = rng.uniform(-0.4, 0.4, (Co,)).astype(dtype)
+    bias[0] = -100.0                             # channel 0: every window all-negative before the relu
+    bias[1] = 0.25
+    outs, vals, idx, labels = conv_layer(gpu, x, ker, bias)
+    assert any("map(" in l for l in labels) == fused, labels
+    z, r, wv = reference(x, ker, bias)
+    tol = 1e-10 if dtype == np.float64 else 1e-5
+    gv, gi, gm = vals.numpy(), idx.numpy(), outs[0].numpy()
+    assert gi.dtype == np.int64 and gm.dtype == np.bool_ and gv.dtype == dtype
+    scale = float(np.max(np.abs(wv)))
+    assert np.max(np.abs(gv - wv.max(-1))) <= tol * scale
+    # all-negative windows: zeros, first position
+    assert np.all(gv[:, 0] == 0) and np.all(gi[:, 0] == 0) and np.all(gm[:, 0])
+    # ties of positive values (the interior of the constant image, channel 1): first position, as the reference's maxIndex
+    inner = slice(0, (H - k + 1) // 2)
+    assert np.all(gv[0, 1, inner, : (Wd - k + 1) // 2] > 0) and np.all(gi[0, 1, inner, : (Wd - k + 1) // 2] == 0)
+    # elsewhere arguments and masks may differ from numpy's only where values are within rounding of each other / of zero
+    srt = np.sort(wv, -1)
+    clear = (srt[..., -1] - srt[..., -2]) > 4 * tol * scale
+    assert np.array_equal(gi[clear], wv.argmax(-1)[clear])
+    sure = np.abs(z) > 4 * tol * float(np.max(np.abs(z)))
+    assert np.array_equal(gm[sure], (z <= 0)[sure])
+
+
+@pytest.mark.gpu
+def test_contract_map_without_windows(gpu):
+    """Only the program: relu (conv + bias) and its mask written at full size."""
+    rng = np.random.default_rng(6)
+    B, Ci, Co, H, Wd, k = 260, 2, 16, 12, 12, 3
+    x = rng.uniform(-1, 1, (B, Ci, H + k - 1, Wd + k - 1))
+    ker = rng.uniform(-0.4, 0.4, (Co, Ci, k, k))
+    bias = rng.uniform(-0.4, 0.4, (Co,))
+    outs, vals, idx, labels = conv_layer(gpu, x, ker, bias, pool=False)
+    assert vals is None and idx is None
+    z, r, _ = reference(x, ker, bias)
+    assert np.max(np.abs(outs[1].numpy() - r)) <= 1e-10 * np.max(np.abs(r))
+    sure = np.abs(z) > 1e-9
+    assert np.array_equal(outs[0].numpy()[sure], (z <= 0)[sure])
+
+
+@pytest.mark.gpu
+def test_contract_map_argument_errors(gpu):
+    a = gpu.upload(np.ones((4, 3, 5)))
+    k = gpu.upload(np.ones((4, 3)))
+    with pytest.raises(capi.HgpuError) as e:       # no input stands for the contraction
+        gpu.contract_map(a, a, 2, [k], [(0, capi.OP1["neg"], 0, 0, 0, 0)], [1])
+    assert e.value.code == 1
+    with pytest.raises(capi.HgpuError) as e:       # a view that leaves the result
+        gpu.contract_map(a, a, 2, [None], [(0, capi.OP1["neg"], 0, 0, 0, 0)], [], (1, [4, 4], [3, 1], 1, True))
+    assert e.value.code == 1
+    outs, v, i = gpu.contract_map(a, a, 2, [None], [(0, capi.OP1["neg"], 0, 0, 0, 0)], [1], (1, [4, 3], [3, 1], 1, False))
+    assert np.array_equal(outs[0].numpy(), np.full((4, 3), -5.0)) and np.array_equal(v.numpy(), np.full(4, -5.0)) and np.array_equal(i.numpy(), np.zeros(4, np.int64))
+
+
+def test_host_rewrites_pooling_layers_onto_contract_map():
+    """The CNN objective on the checker's fused table takes the rewrite for both
+    convolution layers and computes what the plain table computes."""
+    H, W = pkg.hostapi, pkg.workloads
+    plain = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    fused = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_", api_table="get_api_fused"))
+    wl = W.c3_cnn(batch=5)
+    res = []
+    for host in (plain, fused):
+        ps, ds = wl.upload(host)
+        loss, grads = wl.gradient(host, ps, ds)
+        res.append((float(loss.numpy()), [g.numpy() for g in grads]))
+    assert plain.counter("contract_map") == 0 and fused.counter("contract_map") == 2
+    assert res[0][0] == res[1][0]
+    for g0, g1 in zip(res[0][1], res[1][1]):
+        assert np.array_equal(g0, g1)
