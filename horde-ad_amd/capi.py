@@ -63,7 +63,16 @@ GPU_ONLY = {
     "profile_enable": (I, [P, I]), "profile_report": (I, [P, C.c_char_p, C.c_size_t]),
     "contract_noalloc": (I, [P, P, P, I, P]),
     "contract_map": (I, [P, P, P, I, I, PP, I, P, I, IP, PP, I, I, LP, LP, I, I, PP, PP]),
+    "contract_operands": (I, [P, P, P, I, I, PP]),
 }
+
+
+class Operand(C.Structure):
+    """hgpu_operand: a plain array, or an elementwise program's result seen through a view."""
+    _fields_ = [("array", C.c_void_p), ("n_in", C.c_int), ("inputs", C.POINTER(C.c_void_p)), ("n_instr", C.c_int),
+                ("prog", C.c_void_p), ("slot", C.c_int), ("rank_m", C.c_int), ("mshape", C.POINTER(C.c_int64)),
+                ("lo", C.POINTER(C.c_int64)), ("hi", C.POINTER(C.c_int64)), ("rank", C.c_int),
+                ("shape", C.POINTER(C.c_int64)), ("strides", C.POINTER(C.c_int64)), ("offset", C.c_int64)]
 
 
 class HgpuError(RuntimeError):
@@ -165,6 +174,36 @@ class Ctx:
         self.check(self.lib.contract_map(self.h, a.h, b.h, n_keep, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs,
                                          slot, len(vshape), _larr(vshape), _larr(vstrides), n_reduce, int(want_max), C.byref(v), C.byref(i)))
         return [Array(self, C.c_void_p(o)) for o in outs[:len(out_slots)]], Array(self, v), Array(self, i)
+
+    def operand(self, inputs, prog, slot, mshape, view, pad=None):
+        """An expression operand for contract_operands: view = (shape, strides, offset) over the
+        dense layout of the program's result with dims merged to mshape and zero-extended by pad = (lo, hi)."""
+        keep = []
+        o = Operand()
+        ins = (C.c_void_p * len(inputs))(*[p.h for p in inputs])
+        flat = (C.c_int32 * max(6 * len(prog), 1))(*[int(x) for q in prog for x in q])
+        ms, sh, st = _larr(mshape), _larr(view[0]), _larr(view[1])
+        keep += [ins, flat, ms, sh, st, list(inputs)]
+        o.array, o.n_in, o.inputs, o.n_instr, o.prog, o.slot = None, len(inputs), ins, len(prog), C.cast(flat, C.c_void_p), slot
+        o.rank_m, o.mshape, o.rank, o.shape, o.strides, o.offset = len(mshape), ms, len(view[0]), sh, st, view[2]
+        if pad is not None:
+            lo, hi = _larr(pad[0]), _larr(pad[1])
+            keep += [lo, hi]
+            o.lo, o.hi = lo, hi
+        o._keep = keep
+        return o
+
+    def contract_operands(self, a, b, n_keep, fused_only=False):
+        """hgpu_contract_operands; a, b: Array or the result of operand()."""
+        def conv(x):
+            if x is None or isinstance(x, Operand):
+                return x
+            o = Operand()
+            o.array = x.h
+            o._keep = [x]
+            return o
+        oa, ob = conv(a), conv(b)
+        return self._out(self.lib.contract_operands, C.byref(oa), C.byref(ob) if ob is not None else None, n_keep, int(fused_only))
 
     def fused_sum(self, inputs, prog, slot):
         """The sum of slot's values over all elements, a rank-0 array."""

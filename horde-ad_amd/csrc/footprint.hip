@@ -272,12 +272,47 @@ __device__ __forceinline__ void store_rows(T* __restrict__ out, const OutPos& p,
 }
 
 //@EPILOGUE@
+// An operand that is an unevaluated expression is computed where a stored one
+// is loaded, in three steps: the element's place in the expression's inputs
+// (once per lane and staging slot, before the loop over the chunks), the loads
+// (issued like a stored operand's, ahead of the multiplications), and the
+// program on the loaded values (when the vector goes to LDS).
+#if VIRT_X
+typedef VRaw_x RawX;
+#define LOAD_X(ch_, j_) vfetch_x(vax, vpx[j_], ch_)
+#define FIN_X(j_, r_) vfinish_x(hsx, vpx[j_], r_)
+#else
+typedef Vec<VX> RawX;
+#define LOAD_X(ch_, j_) reinterpret_cast<const Vec<VX>*>(X + (ch_) * chx)[vidx(j_)]
+#define FIN_X(j_, r_) (r_)
+#endif
+#if VIRT_Y
+typedef VRaw_y RawY;
+#define LOAD_Y(ch_, j_) vfetch_y(vay, vpy[(j_) - NLX], ch_)
+#define FIN_Y(j_, r_) vfinish_y(hsy, vpy[(j_) - NLX], r_)
+#else
+typedef Vec<VY> RawY;
+#define LOAD_Y(ch_, j_) reinterpret_cast<const Vec<VY>*>(Y + (ch_) * chy)[vidx(j_)]
+#define FIN_Y(j_, r_) (r_)
+#endif
 extern "C" __global__ void __launch_bounds__(256, 1)
 KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 nch, i64 chx, i64 chy, i64 chc, i64 part_stride
 #if EPI
       , EpiArgs ea
 #endif
+#if VIRT_X
+      , VArgs_x vax
+#endif
+#if VIRT_Y
+      , VArgs_y vay
+#endif
       ) {
+#if VIRT_X
+  const VHoist_x hsx = vhoist_x(vax);
+#endif
+#if VIRT_Y
+  const VHoist_y hsy = vhoist_y(vay);
+#endif
   __shared__ T lds[LDS_ELEMS];
 #if EPI_STAGE
   // the chunk's results in the layout they have in memory, written out with whole vectors once the chunk is done
@@ -343,21 +378,31 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   // at a time: eight loads in flight, then eight stores.  Copied one by one,
   // every vector would wait out its own trip to memory.
   constexpr int kFill = 8;
+#if VIRT_X
+  VPre_x vpx[NLX];
+#pragma unroll
+  for (int j = 0; j < NLX; ++j) vpx[j] = vpre_x(XBASE + (i64)vidx(j) * VX);
+#endif
+#if VIRT_Y
+  VPre_y vpy[NLY];
+#pragma unroll
+  for (int j = 0; j < NLY; ++j) vpy[j] = vpre_y(YBASE + (i64)vidx(NLX + j) * VY);
+#endif
   i64 ch = blockIdx.x;
   if (ch < nch) {
 #pragma unroll
     for (int j0 = 0; j0 < NLD; j0 += kFill) {
-      Vec<VX> fx[kFill];
-      Vec<VY> fy[kFill];
+      RawX fx[kFill];
+      RawY fy[kFill];
 #pragma unroll
       for (int j = j0; j < j0 + kFill && j < NLD; ++j) {
-        if (j < NLX) fx[j - j0] = reinterpret_cast<const Vec<VX>*>(X + ch * chx)[vidx(j)];
-        else fy[j - j0] = reinterpret_cast<const Vec<VY>*>(Y + ch * chy)[vidx(j)];
+        if (j < NLX) fx[j - j0] = LOAD_X(ch, j);
+        else fy[j - j0] = LOAD_Y(ch, j);
       }
 #pragma unroll
       for (int j = j0; j < j0 + kFill && j < NLD; ++j) {
-        if (j < NLX) reinterpret_cast<Vec<VX>*>(lds)[vidx(j)] = fx[j - j0];
-        else reinterpret_cast<Vec<VY>*>(lds + LX)[ypos(vidx(j))] = fy[j - j0];
+        if (j < NLX) reinterpret_cast<Vec<VX>*>(lds)[vidx(j)] = FIN_X(j, fx[j - j0]);
+        else reinterpret_cast<Vec<VY>*>(lds + LX)[ypos(vidx(j))] = FIN_Y(j, fy[j - j0]);
       }
     }
   }
@@ -385,8 +430,12 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
     // the next chunk's footprint on its way from memory: with two buffers a
     // phase's share goes to LDS when the phase ends, with one buffer everything
     // waits in registers until this chunk has been multiplied
-    Vec<VX> prex[PH * LPP];
-    Vec<VY> prey[PH * LPP];
+    RawX prex[PH * LPP];
+    RawY prey[PH * LPP];
+    // one buffer and an expression operand: a phase's loads are turned into values
+    // when the phase ends, so that only one phase's raw loads are alive at a time
+    Vec<VX> finx[(NBUFS == 1 && VIRT_X) ? PH * LPP : 1];
+    Vec<VY> finy[(NBUFS == 1 && VIRT_Y) ? PH * LPP : 1];
     i64 chn = ch + gridDim.x;
     if (chn >= nch) chn = nch - 1;    // the last prefetch is not used
     if (MODE == 1) {
@@ -400,8 +449,8 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
       for (int j = 0; j < LPP; ++j) {
         int jj = ph * LPP + j;
         if (jj < NLD) {
-          if (jj < NLX) prex[jj] = reinterpret_cast<const Vec<VX>*>(X + chn * chx)[vidx(jj)];
-          else prey[jj] = reinterpret_cast<const Vec<VY>*>(Y + chn * chy)[vidx(jj)];
+          if (jj < NLX) prex[jj] = LOAD_X(chn, jj);
+          else prey[jj] = LOAD_Y(chn, jj);
         }
       }
       auto groups = [&](auto self, auto GI) -> void {
@@ -438,8 +487,17 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
         for (int j = 0; j < LPP; ++j) {
           int jj = ph * LPP + j;
           if (jj < NLD) {
-            if (jj < NLX) reinterpret_cast<Vec<VX>*>(Ln)[vidx(jj)] = prex[jj];
-            else reinterpret_cast<Vec<VY>*>(Ln + LX)[ypos(vidx(jj))] = prey[jj];
+            if (jj < NLX) reinterpret_cast<Vec<VX>*>(Ln)[vidx(jj)] = FIN_X(jj, prex[jj]);
+            else reinterpret_cast<Vec<VY>*>(Ln + LX)[ypos(vidx(jj))] = FIN_Y(jj, prey[jj]);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < LPP; ++j) {
+          int jj = ph * LPP + j;
+          if (jj < NLD) {
+            if (VIRT_X && jj < NLX) finx[VIRT_X ? jj : 0] = FIN_X(jj, prex[jj]);
+            if (VIRT_Y && jj >= NLX) finy[VIRT_Y ? jj : 0] = FIN_Y(jj, prey[jj]);
           }
         }
       }
@@ -453,8 +511,16 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
       __syncthreads();    // everyone has finished reading this chunk
 #pragma unroll
       for (int jj = 0; jj < NLD; ++jj) {
+#if VIRT_X
+        if (jj < NLX) reinterpret_cast<Vec<VX>*>(Ln)[vidx(jj)] = finx[jj];
+#else
         if (jj < NLX) reinterpret_cast<Vec<VX>*>(Ln)[vidx(jj)] = prex[jj];
-        else reinterpret_cast<Vec<VY>*>(Ln + LX)[ypos(vidx(jj))] = prey[jj];
+#endif
+#if VIRT_Y
+        if (jj >= NLX) reinterpret_cast<Vec<VY>*>(Ln + LX)[ypos(vidx(jj))] = finy[jj];
+#else
+        if (jj >= NLX) reinterpret_cast<Vec<VY>*>(Ln + LX)[ypos(vidx(jj))] = prey[jj];
+#endif
       }
     }
     if (MODE == 1) {
@@ -536,9 +602,12 @@ int lds_bytes(const Plan& pl) {
   return total > INT32_MAX ? INT32_MAX : (int)total;
 }
 
-std::string generate(const Plan& pl, const std::string& kname, const std::string& epilogue = std::string(), int stage_bytes = 0) {
+std::string generate(const Plan& pl, const std::string& kname, const std::string& epilogue = std::string(), int stage_bytes = 0,
+                     const std::string& virt_x = std::string(), int64_t xbase = 0, const std::string& virt_y = std::string(), int64_t ybase = 0) {
   std::ostringstream s;
   s << "#define KNAME " << kname << "\n";
+  s << "#define VIRT_X " << (virt_x.empty() ? 0 : 1) << "\n#define XBASE " << xbase << "ll\n";
+  s << "#define VIRT_Y " << (virt_y.empty() ? 0 : 1) << "\n#define YBASE " << ybase << "ll\n";
   s << "#define EPI " << (epilogue.empty() ? 0 : 1) << "\n#define EPI_STAGE " << stage_bytes << "\n";
   const int es = pl.f64 ? 8 : 4;
   s << "#define F64 " << (pl.f64 ? 1 : 0) << "\n";
@@ -567,19 +636,235 @@ std::string generate(const Plan& pl, const std::string& kname, const std::string
   s << table("__device__ const", "kColY", col_y) << table("__device__ const", "kColC", pl.col_c);
   std::string body = kBody;
   const std::string mark = "//@EPILOGUE@";
-  body.replace(body.find(mark), mark.size(), epilogue);
+  std::string pre = epilogue;
+  if (epilogue.empty() && (!virt_x.empty() || !virt_y.empty())) pre = fusedgen::kPrelude;
+  body.replace(body.find(mark), mark.size(), pre + virt_x + virt_y);
   s << body;
+  return s.str();
+}
+
+// An operand that is an elementwise program's result, its dims merged to M,
+// zero-extended to P = M + lo + hi, seen through a strided view of P's dense
+// row-major layout.  The kernels address it by element offsets in that layout.
+struct VirtualOp {
+  int n_in = 0, n_instr = 0, slot = 0, dtype = 0;
+  const hgpu_array* const* in = nullptr;
+  const hgpu_fused_instr* prog = nullptr;
+  std::vector<int> dt;                       // type of every slot
+  std::vector<int64_t> E, M, lo, hi, P;      // shape of the inputs; merged; extension; extended
+  int64_t total = 0;                         // elements of P
+  bool padded = false;
+};
+
+// true when V consecutive elements of the layout, starting at a multiple of V,
+// are V consecutive elements of the innermost dim of the inputs (all valid or all padding)
+bool vector_ok(const VirtualOp& v, int V) {
+  if (V == 1) return true;
+  if (v.E.empty() || v.M.empty()) return false;
+  return v.E.back() % V == 0 && v.P.back() % V == 0 && v.lo.back() % V == 0 && v.total % V == 0;
+}
+
+// Source of the three steps that stand in for the load of V consecutive
+// elements of an expression operand (tag "x" or "y"):
+//   VPre  vpre(w)                the place of element offset w (the chunk's own
+//                                offset left out) in the inputs of the expression;
+//   VRaw  vfetch(args, pre, ch)  the loads for chunk ch;
+//   Vec   vfinish(hoisted, pre, raw)   the program on the loaded values; elements
+//                                in the zero-extension, or past the end, are zero.
+// chunk_stride: elements of the layout between chunks.  When a chunk is a step
+// along the outermost dim of the layout, and that dim is one of the inputs' own
+// (not merged, not extended), the place is decoded once, before the loop over
+// the chunks, and a chunk only adds a constant to every input offset; else the
+// offset is decoded for every chunk.  Divisors are constants of the kernel.
+std::string vops_source(const VirtualOp& v, const char* tag_, int V, int64_t chunk_stride, int64_t max_elem = INT64_MAX) {
+  using namespace hg::fusedgen;
+  std::ostringstream s;
+  const std::string tag = tag_;
+  const std::string T_ = ctype(v.dtype);
+  const size_t rm = v.M.size(), re = v.E.size();
+  // per input: one broadcast element; no move along the innermost dim (one load
+  // serves a vector); V neighbours there that one aligned load fetches
+  std::vector<char> scalar((size_t)v.n_in, 0), shared((size_t)v.n_in, 0), vecload((size_t)v.n_in, 0), wide((size_t)v.n_in, 0);
+  std::vector<int> rep((size_t)v.n_in, -1);   // the first input with the same strides: they share their offsets
+  for (int i = 0; i < v.n_in; ++i) {
+    const hgpu_array* a = v.in[i];
+    bool all0 = true;
+    int64_t reach = 0;
+    for (int d = 0; d < a->rank; ++d) {
+      if (a->shape[d] != 1 && a->strides[d] != 0) all0 = false;
+      reach += (a->shape[d] - 1) * (a->strides[d] < 0 ? -a->strides[d] : a->strides[d]);
+    }
+    scalar[(size_t)i] = all0;
+    wide[(size_t)i] = reach >= (1LL << 31);
+    shared[(size_t)i] = !all0 && V > 1 && (v.E[re - 1] == 1 || a->strides[re - 1] == 0);
+    if (!all0 && V > 1 && !shared[(size_t)i] && a->strides[re - 1] == 1) {
+      bool ok = ((uintptr_t)data_ptr(a) % (dtype_size(a->dtype) * (size_t)V)) == 0;
+      for (size_t j = 0; j + 1 < re && ok; ++j) ok = v.E[j] == 1 || a->strides[j] % V == 0;
+      vecload[(size_t)i] = ok;
+    }
+    rep[(size_t)i] = i;
+    for (int k = 0; k < i && !all0; ++k) {
+      if (scalar[(size_t)k]) continue;
+      bool same = true;
+      for (size_t j = 0; j < re && same; ++j) same = v.E[j] == 1 || v.in[k]->strides[j] == a->strides[j];
+      if (same) { rep[(size_t)i] = rep[(size_t)k]; break; }
+    }
+  }
+  auto own = [&](int i) { return !scalar[(size_t)i] && rep[(size_t)i] == i; };   // carries offsets of its own
+  auto oty = [&](int i) { return wide[(size_t)i] ? "i64" : "int"; };
+  std::vector<int64_t> PS(rm), MS(rm), ES(re);
+  { int64_t a = 1, b = 1; for (size_t k = rm; k-- > 0;) { PS[k] = a; a *= v.P[k]; MS[k] = b; b *= v.M[k]; } }
+  { int64_t a = 1; for (size_t j = re; j-- > 0;) { ES[j] = a; a *= v.E[j]; } }
+  // first dims with more than one element
+  size_t k0 = 0, j0 = 0;
+  while (k0 < rm && v.P[k0] == 1) ++k0;
+  while (j0 < re && v.E[j0] == 1) ++j0;
+  const bool separable = chunk_stride != 0 && k0 < rm && j0 < re && chunk_stride % PS[k0] == 0 && v.lo[k0] == 0 && v.hi[k0] == 0 && v.E[j0] == v.M[k0] &&
+                         ES[j0] == MS[k0] && !(V > 1 && j0 == re - 1);
+  const int64_t chunk_step = separable ? chunk_stride / PS[k0] : 0;   // coordinates along the outermost dim per chunk
+  const bool range_check = max_elem > v.total;        // some lane of some chunk may address past the layout's end
+  const bool has_ok = range_check || v.padded;
+  auto gp = [&](int i, const std::string& ty) { return std::string("const __attribute__((address_space(1))) ") + ty + "*"; };
+
+  s << "struct VArgs_" << tag << " {\n";
+  for (int i = 0; i < v.n_in; ++i) s << "  const " << ctype(v.dt[(size_t)i]) << "* i" << i << ";\n";
+  s << "};\nstruct VHoist_" << tag << " {\n";
+  for (int i = 0; i < v.n_in; ++i)
+    if (scalar[(size_t)i]) s << "  " << ctype(v.dt[(size_t)i]) << " s" << i << ";\n";
+  s << "  int unused;\n};\n";
+  s << "__device__ __forceinline__ VHoist_" << tag << " vhoist_" << tag << "(const VArgs_" << tag << "& va) {\n  VHoist_" << tag << " h;\n  h.unused = 0;\n";
+  for (int i = 0; i < v.n_in; ++i)
+    if (scalar[(size_t)i]) s << "  h.s" << i << " = va.i" << i << "[0];\n";
+  s << "  return h;\n}\n";
+  for (int i = 0; i < v.n_in; ++i)
+    if (vecload[(size_t)i]) s << "struct alignas(" << dtype_size(v.dt[(size_t)i]) * (size_t)V << ") VPack_" << tag << i << " { " << ctype(v.dt[(size_t)i]) << " v[" << V << "]; };\n";
+
+  // decode: element offset `e` (unsigned, in range) -> ok, input offsets o<i>
+  auto emit_decode = [&](const char* ind) {
+    if (v.padded) {
+      s << ind << "unsigned flat = 0;\n";
+      for (size_t k = 0; k < rm; ++k) {
+        if (v.P[k] == 1) continue;
+        s << ind << "{\n" << ind << "  const unsigned c = " << (k == k0 ? "e / " + std::to_string(PS[k]) + "u" : "(e / " + std::to_string(PS[k]) + "u) % " + std::to_string(v.P[k]) + "u") << ";\n";
+        if (v.lo[k] != 0 || v.hi[k] != 0) s << ind << "  ok = ok && c >= " << v.lo[k] << "u && c < " << v.lo[k] + v.M[k] << "u;\n";
+        s << ind << "  flat += (c - " << v.lo[k] << "u) * " << MS[k] << "u;\n" << ind << "}\n";
+      }
+      s << ind << "if (!ok) flat = 0;\n";
+    } else {
+      s << ind << "const unsigned flat = e;\n";
+    }
+    for (size_t j = 0; j < re; ++j) {
+      bool used = false;
+      for (int i = 0; i < v.n_in; ++i) used = used || (!scalar[(size_t)i] && v.in[i]->strides[j] != 0);
+      if (!used || v.E[j] == 1) continue;
+      if (V > 1 && j == re - 1) s << ind << "const unsigned x" << j << " = flat % " << v.E[j] << "u;\n";
+      else s << ind << "const unsigned x" << j << " = " << (j == j0 ? "flat / " + std::to_string(ES[j]) + "u" : "(flat / " + std::to_string(ES[j]) + "u) % " + std::to_string(v.E[j]) + "u") << ";\n";
+    }
+    for (int i = 0; i < v.n_in; ++i) {
+      if (!own(i)) continue;
+      s << ind << "const " << oty(i) << " o" << i << " = 0";
+      for (size_t j = 0; j < re; ++j)
+        if (v.E[j] != 1 && v.in[i]->strides[j] != 0) s << " + (" << oty(i) << ")x" << j << " * " << v.in[i]->strides[j] << (wide[(size_t)i] ? "ll" : "");
+      s << ";\n";
+    }
+  };
+
+  s << "struct VPre_" << tag << " {\n";
+  if (separable) {
+    for (int i = 0; i < v.n_in; ++i)
+      if (own(i)) s << "  " << oty(i) << " o" << i << ";\n";
+    if (v.padded) s << "  bool ok;\n";
+  }
+  if (!separable || range_check) s << "  i64 w;\n";
+  s << "  int unused[0];\n};\n";
+  s << "__device__ __forceinline__ VPre_" << tag << " vpre_" << tag << "(i64 w) {\n  VPre_" << tag << " p;\n";
+  if (separable) {
+    s << "  bool ok = w >= 0 && w < " << v.total << "ll;\n";
+    s << "  const unsigned e = ok ? (unsigned)w : 0u;\n";
+    emit_decode("  ");
+    for (int i = 0; i < v.n_in; ++i)
+      if (own(i)) s << "  p.o" << i << " = o" << i << ";\n";
+    if (v.padded) s << "  p.ok = ok;\n";
+  }
+  if (!separable || range_check) s << "  p.w = w;\n";
+  s << "  return p;\n}\n";
+
+  s << "struct VRaw_" << tag << " {\n";
+  for (int i = 0; i < v.n_in; ++i) {
+    if (scalar[(size_t)i]) continue;
+    if (vecload[(size_t)i]) s << "  VPack_" << tag << i << " r" << i << ";\n";
+    else s << "  " << ctype(v.dt[(size_t)i]) << " r" << i << (shared[(size_t)i] ? "" : "[" + std::to_string(V) + "]") << ";\n";
+  }
+  if (has_ok) s << "  bool ok;\n";
+  s << "  int unused[0];\n};\n";
+  s << "__device__ __forceinline__ VRaw_" << tag << " vfetch_" << tag << "(const VArgs_" << tag << "& va, const VPre_" << tag << "& p, i64 ch) {\n  VRaw_" << tag << " r;\n";
+  if (separable) {
+    // the chunk moves every input by a constant; an element past the layout's end reads the first one's place (its value is dropped)
+    if (has_ok) {
+      s << "  bool ok = " << (v.padded ? "p.ok" : "true") << (range_check ? " && p.w + ch * " + std::to_string(chunk_stride) + "ll < " + std::to_string(v.total) + "ll" : "") << ";\n";
+      s << "  const i64 cq = ok ? ch * " << chunk_step << "ll : 0;\n";
+    } else {
+      s << "  const i64 cq = ch * " << chunk_step << "ll;\n";
+    }
+    for (int i = 0; i < v.n_in; ++i)
+      if (own(i)) s << "  const i64 o" << i << " = (i64)" << (has_ok ? "(ok ? p.o" + std::to_string(i) + " : 0)" : "p.o" + std::to_string(i)) << " + cq * " << v.in[i]->strides[j0] << "ll;\n";
+  } else {
+    s << "  const i64 e0 = p.w + ch * " << chunk_stride << "ll;\n";
+    s << "  bool ok = e0 >= 0 && e0 < " << v.total << "ll;\n";
+    s << "  const unsigned e = ok ? (unsigned)e0 : 0u;\n";
+    emit_decode("  ");
+  }
+  for (int i = 0; i < v.n_in; ++i) {
+    if (scalar[(size_t)i]) continue;
+    const std::string ct = ctype(v.dt[(size_t)i]);
+    const std::string off = "o" + std::to_string(rep[(size_t)i]);
+    if (vecload[(size_t)i]) {
+      const std::string pk = "VPack_" + tag + std::to_string(i);
+      s << "  r.r" << i << " = *(" << gp(i, pk) << ")((" << gp(i, ct) << ")va.i" << i << " + " << off << ");\n";
+    } else {
+      s << "  {\n    " << gp(i, ct) << " g = (" << gp(i, ct) << ")va.i" << i << ";\n";
+      if (shared[(size_t)i]) s << "    r.r" << i << " = g[" << off << "];\n";
+      else for (int el = 0; el < V; ++el) s << "    r.r" << i << "[" << el << "] = g[" << off << " + " << (int64_t)el * (re > 0 ? v.in[i]->strides[re - 1] : 0) << "ll];\n";
+      s << "  }\n";
+    }
+  }
+  if (has_ok) s << "  r.ok = ok;\n";
+  s << "  return r;\n}\n";
+
+  s << "__device__ __forceinline__ Vec<" << V << "> vfinish_" << tag << "(const VHoist_" << tag << "& hs, const VPre_" << tag << "&, const VRaw_" << tag << "& raw) {\n";
+  s << "  Vec<" << V << "> r;\n";
+  for (int el = 0; el < V; ++el) {
+    std::string suf = "_" + std::to_string(el);
+    s << "  {\n";
+    for (int i = 0; i < v.n_in; ++i) {
+      s << "    const " << ctype(v.dt[(size_t)i]) << " v" << i << suf << " = ";
+      if (scalar[(size_t)i]) s << "hs.s" << i;
+      else if (vecload[(size_t)i]) s << "raw.r" << i << ".v[" << el << "]";
+      else if (shared[(size_t)i]) s << "raw.r" << i;
+      else s << "raw.r" << i << "[" << el << "]";
+      s << ";\n";
+    }
+    emit_program(s, v.n_in, v.n_instr, v.prog, v.dt, "    ", suf);
+    const std::string val = has_ok ? "raw.ok ? v" + std::to_string(v.slot) + suf + " : " + T_ + "(0)" : "v" + std::to_string(v.slot) + suf;
+    if (V > 1) s << "    r[" << el << "] = " << val << ";\n";
+    else s << "    r = " << val << ";\n";
+    s << "  }\n";
+  }
+  s << "  return r;\n}\n";
   return s.str();
 }
 
 // Staging vectors, LDS padding of the columns operand, output vectors and the
 // number of chunk buffers of a plan whose operands sit at xp / yp; false when
 // the plan does not fit the CU.
-bool finish_plan(Plan& pl, const char* xp, const char* yp, const char* cp, int64_t out_n, int extra_lds_bytes) {
+bool finish_plan(Plan& pl, const char* xp, const char* yp, const char* cp, int64_t out_n, int extra_lds_bytes, const VirtualOp* virt_x = nullptr,
+                 const VirtualOp* virt_y = nullptr) {
   const int es = pl.f64 ? 8 : 4;
   const int V = 16 / es;
   pl.vx = (((uintptr_t)xp & 15) == 0 && (pl.chx * es) % 16 == 0) ? V : 1;
   pl.vy = (((uintptr_t)yp & 15) == 0 && (pl.chy * es) % 16 == 0) ? V : 1;
+  if (virt_x && !vector_ok(*virt_x, pl.vx)) pl.vx = 1;
+  if (virt_y && !vector_ok(*virt_y, pl.vy)) pl.vy = 1;
   // columns a constant stride apart, each with its K offsets inside the
   // stride: pad the stride in LDS until 16 columns hit 16 different banks
   pl.ys = 1;
@@ -606,8 +891,22 @@ bool finish_plan(Plan& pl, const char* xp, const char* yp, const char* cp, int64
     if (pl.mode == 0) ok = ok && out_n % V == 0;   // partial outputs lie out_n apart
     pl.cvec = ok;
   }
-  // scalar staging of a large footprint would need too many loads in flight
-  int64_t loads = (pl.span_x / pl.vx + 255) / 256 + (pl.mode == 0 ? (pl.span_y / pl.vy + 255) / 256 : 0);
+  // scalar staging of a large footprint would need too many loads in flight; a
+  // staging slot of an expression operand costs one load per input that is not a
+  // single broadcast element (the kernel is bound by the number of loads a
+  // wavefront can have in flight, not by their size)
+  auto per_slot = [](const VirtualOp* v) {
+    if (!v) return (int64_t)1;
+    int64_t n = 0;
+    for (int i = 0; i < v->n_in; ++i) {
+      bool all0 = true;
+      for (int d = 0; d < v->in[i]->rank; ++d)
+        if (v->in[i]->shape[d] != 1 && v->in[i]->strides[d] != 0) all0 = false;
+      if (!all0) ++n;
+    }
+    return n > 0 ? n : (int64_t)1;
+  };
+  int64_t loads = (pl.span_x / pl.vx + 255) / 256 * per_slot(virt_x) + (pl.mode == 0 ? (pl.span_y / pl.vy + 255) / 256 * per_slot(virt_y) : 0);
   if (loads > 48) return false;
   pl.nbufs = 2;
   if (lds_bytes(pl) + extra_lds_bytes > kLdsBudget) {
@@ -624,9 +923,22 @@ namespace hg {
 // gemm.hip: out[i] = sum over the `parts` partial outputs of part[s * n + i], in a fixed order.
 int sum_partials(hgpu_ctx* ctx, int dtype, int64_t n, int parts, const void* part, void* out);
 
+int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled,
+                          const void* va_, const void* vb_);
+
 // Runs the contraction described by p with the footprint kernel when its shape
 // suits it (*handled), else leaves it to the caller's other kernels.
 int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled) {
+  return try_footprint_virtual(ctx, p, dtype, pa, pb, out, handled, nullptr, nullptr);
+}
+
+// The same with operands that may be unevaluated expressions (va / vb not null:
+// pa / pb are then the element offset of the operand's view in the layout of
+// its expression, times the element size, as a pointer from address 0).
+int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled,
+                          const void* va_, const void* vb_) {
+  const VirtualOp* va = static_cast<const VirtualOp*>(va_);
+  const VirtualOp* vb = static_cast<const VirtualOp*>(vb_);
   *handled = false;
   if (p.BT != 1 || p.n_terms > 0) return HGPU_OK;
   if (dtype != HGPU_F64 && dtype != HGPU_F32) return HGPU_OK;
@@ -658,7 +970,8 @@ int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa,
         if (!make_plan(f64, rows, colsd, kd, in_k != 0, ci, ctx->num_cu, &pl)) continue;
         const char* xp = (const char*)(swapped ? pb : pa) + pl.shift_x * es;
         const char* yp = (const char*)(swapped ? pa : pb) + pl.shift_y * es;
-        if (!finish_plan(pl, xp, yp, (const char*)data_ptr(out), nelem(out), 0)) continue;
+        if (!finish_plan(pl, xp, yp, (const char*)data_ptr(out), nelem(out), 0, swapped ? vb : va, swapped ? va : vb)) continue;
+        if (pl.mode == 1 && (swapped ? va : vb)) continue;   // the columns operand of this mode is staged once, from memory
         best = pl;
         best_swapped = swapped != 0;
         found = true;
@@ -669,9 +982,17 @@ int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa,
   const Plan& pl = best;
   // the kernel's name tells a profiler which product it is
   char kname[128];
-  snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_%s%s", f64 ? "f64" : "f32", (long long)p.M, (long long)p.N, (long long)p.K,
-           pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? "_swapped" : "");
-  std::string src = generate(pl, kname);
+  const VirtualOp* vx = best_swapped ? vb : va;
+  const VirtualOp* vy = best_swapped ? va : vb;
+  snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_%s%s%s%s", f64 ? "f64" : "f32", (long long)p.M, (long long)p.N, (long long)p.K,
+           pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? "_swapped" : "", vx ? "_xmap" : "", vy ? "_ymap" : "");
+  const int64_t xbase = (int64_t)((uintptr_t)((const char*)(best_swapped ? pb : pa) + pl.shift_x * es) / (uintptr_t)es);
+  const int64_t ybase = (int64_t)((uintptr_t)((const char*)(best_swapped ? pa : pb) + pl.shift_y * es) / (uintptr_t)es);
+  // the last staging vector of the last chunk may reach past its footprint: how far at most
+  const int64_t xmax = xbase + (pl.nch - 1) * pl.chx + (pl.span_x + pl.vx - 1) / pl.vx * pl.vx;
+  const int64_t ymax = ybase + (pl.nch - 1) * pl.chy + (pl.span_y + pl.vy - 1) / pl.vy * pl.vy;
+  std::string src = generate(pl, kname, std::string(), 0, vx ? vops_source(*vx, "x", pl.vx, pl.chx, xmax) : std::string(), vx ? xbase : 0,
+                             vy ? vops_source(*vy, "y", pl.vy, pl.chy, ymax) : std::string(), vy ? ybase : 0);
   auto& cache = cache_of(ctx);
   auto it = cache.find(src);
   if (it == cache.end()) {
@@ -695,20 +1016,27 @@ int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa,
     part_stride = out_n;
   }
   int64_t nch = pl.nch, chx = pl.chx, chy = pl.chy, chc = pl.chc;
-  void* args[] = {(void*)&xp, (void*)&yp, (void*)&cdst, (void*)&nch, (void*)&chx, (void*)&chy, (void*)&chc, (void*)&part_stride};
+  // the inputs of an expression operand follow as one struct of pointers each
+  std::vector<const void*> vxa, vya;
+  if (vx) { xp = nullptr; for (int i = 0; i < vx->n_in; ++i) vxa.push_back(data_ptr(vx->in[i])); }
+  if (vy) { yp = nullptr; for (int i = 0; i < vy->n_in; ++i) vya.push_back(data_ptr(vy->in[i])); }
+  std::vector<void*> args = {(void*)&xp, (void*)&yp, (void*)&cdst, (void*)&nch, (void*)&chx, (void*)&chy, (void*)&chc, (void*)&part_stride};
+  if (vx) args.push_back((void*)vxa.data());
+  if (vy) args.push_back((void*)vya.data());
   {
     double flops = 2.0 * p.M * p.N * p.K;
     double bytes = ((double)p.M * p.K + (double)p.N * p.K + (double)p.M * p.N) * es;
     const char* label = f64 ? "gemm_f64" : "gemm_f32";
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[160];
-      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB1,footprint,%s%s,chunks%lld,rows%d,kgroups%d,lds%dK]", label, (long long)p.M, (long long)p.N,
-               (long long)p.K, pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? ",swapped" : "", (long long)pl.nch, pl.min_rows, (int)pl.gx.size(), lds_bytes(pl) / 1024);
+      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB1,footprint,%s%s,chunks%lld,rows%d,kgroups%d,lds%dK%s%s]", label, (long long)p.M, (long long)p.N,
+               (long long)p.K, pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? ",swapped" : "", (long long)pl.nch, pl.min_rows, (int)pl.gx.size(), lds_bytes(pl) / 1024,
+               vx ? ",xmap" : "", vy ? ",ymap" : "");
       label = ctx->label_pool.insert(buf).first->c_str();
     }
     {
       LaunchGuard lg(ctx, label, bytes, flops);
-      hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+      hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
       if (e != hipSuccess) { if (part) buffer_release(part); return check_hip(ctx, e, "footprint gemm launch"); }
     }
     if (pl.mode == 0) {
@@ -1255,4 +1583,263 @@ extern "C" int hgpu_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_
   }
   for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
   return HGPU_OK;
+}
+
+// ---------------------------------------------------------------------------
+// hgpu_contract_operands: contractions whose operands may be unevaluated
+// elementwise expressions (see VirtualOp).
+namespace {
+
+// Checks the description of an expression operand and fills in v.
+int virtual_from_operand(hgpu_ctx* ctx, const hgpu_operand* o, VirtualOp* v) {
+  if (o->n_in < 1 || o->n_in > 12 || o->n_instr < 0 || o->n_instr > 96 || !o->in || (o->n_instr > 0 && !o->prog))
+    return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract_operands: %d inputs, %d instructions", o->n_in, o->n_instr);
+  for (int i = 0; i < o->n_in; ++i) {
+    if (!o->in[i]) return HGPU_ERR_INVALID;
+    if (!same_shape(o->in[i], o->in[0])) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: input %d has another shape", i);
+  }
+  if (int rc = hg::fusedgen::check_program(ctx, o->n_in, o->in, o->n_instr, o->prog, &v->dt)) return rc;
+  if (o->slot < 0 || o->slot >= o->n_in + o->n_instr) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: bad slot");
+  if (o->rank_m < 0 || o->rank_m > HGPU_MAX_RANK || o->rank < 0 || o->rank > HGPU_MAX_RANK || (o->rank_m > 0 && !o->mshape) || (o->rank > 0 && (!o->shape || !o->strides)))
+    return fail(ctx, HGPU_ERR_INVALID, "contract_operands: bad ranks");
+  if ((o->lo == nullptr) != (o->hi == nullptr)) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: lo and hi go together");
+  v->n_in = o->n_in;
+  v->in = o->in;
+  v->n_instr = o->n_instr;
+  v->prog = o->prog;
+  v->slot = o->slot;
+  v->dtype = v->dt[(size_t)o->slot];
+  v->E.assign(o->in[0]->shape, o->in[0]->shape + o->in[0]->rank);
+  int64_t ne = 1, nm = 1;
+  for (auto e : v->E) ne *= e;
+  v->total = 1;
+  v->padded = false;
+  for (int k = 0; k < o->rank_m; ++k) {
+    const int64_t lo = o->lo ? o->lo[k] : 0, hi = o->hi ? o->hi[k] : 0;
+    if (o->mshape[k] < 0 || lo < 0 || hi < 0) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: negative extent");
+    v->M.push_back(o->mshape[k]);
+    v->lo.push_back(lo);
+    v->hi.push_back(hi);
+    v->P.push_back(o->mshape[k] + lo + hi);
+    nm *= o->mshape[k];
+    v->total *= v->P.back();
+    v->padded = v->padded || lo != 0 || hi != 0;
+  }
+  if (ne != nm) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: %lld elements seen as %lld", (long long)ne, (long long)nm);
+  // the view must stay inside the extended layout
+  int64_t lo = o->offset, hi = o->offset;
+  bool empty = false;
+  for (int d = 0; d < o->rank; ++d) {
+    if (o->shape[d] < 0) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: negative extent");
+    if (o->shape[d] == 0) { empty = true; continue; }
+    const int64_t span = (o->shape[d] - 1) * o->strides[d];
+    if (span > 0) hi += span; else lo += span;
+  }
+  if (!empty && (lo < 0 || hi >= v->total)) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: the view leaves the layout");
+  return HGPU_OK;
+}
+
+// The operand as an array: program, merged dims, zero-extension, view.
+int write_out(hgpu_ctx* ctx, const hgpu_operand* o, hgpu_array** out) {
+  if (o->array) { hgpu_retain(const_cast<hgpu_array*>(o->array)); *out = const_cast<hgpu_array*>(o->array); return HGPU_OK; }
+  hgpu_array *e = nullptr, *m = nullptr, *p = nullptr;
+  int rc;
+  if (o->slot < o->n_in) rc = hgpu_materialize(ctx, o->in[o->slot], &e);
+  else rc = hgpu_fused_map(ctx, o->n_in, o->in, o->n_instr, o->prog, 1, &o->slot, &e);
+  if (rc) return rc;
+  rc = hgpu_reshape(ctx, e, o->rank_m, o->mshape, &m);
+  hgpu_release(e);
+  if (rc) return rc;
+  if (o->lo) {
+    rc = hgpu_pad(ctx, m, o->lo, o->hi, &p);
+    hgpu_release(m);
+    if (rc) return rc;
+  } else {
+    p = m;
+  }
+  rc = hgpu_as_strided(ctx, p, o->rank, o->shape, o->strides, o->offset, out);
+  hgpu_release(p);
+  return rc;
+}
+
+// out[o] = sum over the dims behind the first n_keep of the view of an
+// expression: blocks take (output, chunk of the summed index range), lanes
+// evaluate the expression at their elements, partial sums are added up in a
+// fixed order by a second launch.
+int try_mapped_sum(hgpu_ctx* ctx, const VirtualOp& v, const hgpu_operand* o, int n_keep, hgpu_array* out, bool* handled) {
+  *handled = false;
+  if (v.dtype != HGPU_F64 && v.dtype != HGPU_F32) return HGPU_OK;
+  if (v.total >= (1LL << 31)) return HGPU_OK;
+  const int es = v.dtype == HGPU_F64 ? 8 : 4;
+  // dims of the view, each group merged where contiguous
+  struct D2 { int64_t e, s; };
+  auto merged = [&](int from, int to) {
+    std::vector<D2> g;
+    for (int d = from; d < to; ++d) {
+      if (o->shape[d] == 1) continue;
+      if (!g.empty() && g.back().s == o->strides[d] * o->shape[d]) { g.back().e *= o->shape[d]; g.back().s = o->strides[d]; }
+      else g.push_back({o->shape[d], o->strides[d]});
+    }
+    return g;
+  };
+  std::vector<D2> kd = merged(0, n_keep), rd = merged(n_keep, o->rank);
+  int64_t n_out = 1, R = 1;
+  for (auto& d : kd) n_out *= d.e;
+  for (auto& d : rd) R *= d.e;
+  if (n_out > 4096 || R < 16384 || rd.empty()) return HGPU_OK;   // few outputs under long sums: what this kernel is for
+  int W = 16 / es;
+  {
+    bool ok = rd.back().s == 1 && rd.back().e % W == 0 && o->offset % W == 0 && vector_ok(v, W);
+    for (size_t i = 0; i + 1 < rd.size(); ++i) ok = ok && rd[i].s % W == 0;
+    for (auto& d : kd) ok = ok && d.s % W == 0;
+    if (!ok) W = 1;
+  }
+  int64_t S = ((int64_t)ctx->num_cu * 8 + n_out - 1) / n_out;
+  if (S > R / 4096) S = R / 4096;
+  if (S < 1) S = 1;
+  int64_t CH = ((R + S - 1) / S + W - 1) / W * W;
+  S = (R + CH - 1) / CH;
+  std::ostringstream s;
+  s << "typedef long long i64;\n";
+  s << "typedef " << (es == 8 ? "double" : "float") << " T;\n";
+  s << "template <int N> struct VT { typedef T type __attribute__((ext_vector_type(N))); };\ntemplate <> struct VT<1> { typedef T type; };\ntemplate <int N> using Vec = typename VT<N>::type;\n";
+  s << hg::fusedgen::kPrelude;
+  s << vops_source(v, "x", W, 0);
+  s << "extern \"C\" __global__ void __launch_bounds__(256) mapped_sum(VArgs_x vax, T* __restrict__ part) {\n";
+  s << "  __shared__ double red[4];\n";
+  s << "  const VHoist_x hsx = vhoist_x(vax);\n";
+  s << "  const unsigned o = blockIdx.x % " << n_out << "u, sc = blockIdx.x / " << n_out << "u;\n";
+  s << "  i64 base = " << o->offset << "ll;\n  {\n    unsigned r = o;\n";
+  for (size_t i = kd.size(); i-- > 0;) {
+    if (i > 0) s << "    base += (i64)(r % " << kd[i].e << "u) * " << kd[i].s << "ll; r /= " << kd[i].e << "u;\n";
+    else s << "    base += (i64)r * " << kd[i].s << "ll;\n";
+  }
+  s << "  }\n";
+  s << "  const i64 r0 = (i64)sc * " << CH << "ll, r1 = r0 + " << CH << "ll < " << R << "ll ? r0 + " << CH << "ll : " << R << "ll;\n";
+  s << "  double acc = 0;\n";
+  s << "  for (i64 rr = r0 + (i64)threadIdx.x * " << W << "; rr < r1; rr += 256 * " << W << ") {\n";
+  s << "    unsigned r = (unsigned)rr;\n    i64 e = base;\n";
+  for (size_t i = rd.size(); i-- > 0;) {
+    if (i > 0) s << "    e += (i64)(r % " << rd[i].e << "u) * " << rd[i].s << "ll; r /= " << rd[i].e << "u;\n";
+    else s << "    e += (i64)r * " << rd[i].s << "ll;\n";
+  }
+  s << "    const VPre_x pre = vpre_x(e);\n    const Vec<" << W << "> x = vfinish_x(hsx, pre, vfetch_x(vax, pre, 0));\n";
+  if (W == 1) s << "    acc += (double)x;\n";
+  else for (int k = 0; k < W; ++k) s << "    acc += (double)x[" << k << "];\n";
+  s << "  }\n";
+  s << "  for (int off = 32; off > 0; off >>= 1) {\n"
+       "    unsigned long long u = *reinterpret_cast<unsigned long long*>(&acc);\n"
+       "    unsigned lo = __shfl_down((unsigned)(u & 0xffffffffu), off, 64), hi = __shfl_down((unsigned)(u >> 32), off, 64);\n"
+       "    unsigned long long w = ((unsigned long long)hi << 32) | lo;\n"
+       "    acc += *reinterpret_cast<double*>(&w);\n  }\n";
+  s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n  __syncthreads();\n";
+  s << "  if (threadIdx.x == 0) part[(i64)sc * " << n_out << "ll + o] = (T)((red[0] + red[1]) + (red[2] + red[3]));\n}\n";
+  std::string src = s.str();
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c{nullptr, nullptr};
+    if (compile(ctx, src, "mapped_sum", &c) != HGPU_OK) c = Compiled{nullptr, nullptr};
+    it = cache.emplace(src, c).first;
+  }
+  if (!it->second.fn) return HGPU_OK;
+  hgpu_buffer* part = nullptr;
+  void* dst = data_ptr(out);
+  if (S > 1) {
+    int rc = buffer_alloc(ctx, (size_t)(n_out * S) * es, &part);
+    if (rc) return rc;
+    dst = part->ptr;
+  }
+  std::vector<const void*> vxa;
+  for (int i = 0; i < v.n_in; ++i) vxa.push_back(data_ptr(v.in[i]));
+  void* args[] = {(void*)vxa.data(), (void*)&dst};
+  {
+    double bytes = 0;
+    for (int i = 0; i < v.n_in; ++i) {
+      int64_t distinct = 1;
+      for (int d = 0; d < v.in[i]->rank; ++d)
+        if (v.in[i]->strides[d] != 0) distinct *= v.in[i]->shape[d];
+      if (distinct > 1) bytes += (double)distinct * dtype_size(v.in[i]->dtype);
+    }
+    const char* label = "mapped_sum";
+    if (ctx->profiling && ctx->profile_shapes) {
+      char buf[160];
+      snprintf(buf, sizeof buf, "mapped_sum[out%lld,R%lld,S%lld,in%d,instr%d,vec%d%s]", (long long)n_out, (long long)R, (long long)S, v.n_in, v.n_instr, W, v.padded ? ",padded" : "");
+      label = ctx->label_pool.insert(buf).first->c_str();
+    }
+    LaunchGuard lg(ctx, label, bytes, (double)n_out * R * (v.n_instr + 1));
+    hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)(n_out * S), 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+    if (e != hipSuccess) { if (part) buffer_release(part); return check_hip(ctx, e, "mapped_sum launch"); }
+  }
+  if (part) {
+    int rc = hg::sum_partials(ctx, v.dtype, n_out, (int)S, part->ptr, data_ptr(out));
+    buffer_release(part);
+    if (rc) return rc;
+  }
+  *handled = true;
+  return HGPU_OK;
+}
+
+}  // namespace
+
+namespace hg {
+bool classify_contraction(int rank, const int64_t* shape, const int64_t* st_a, const int64_t* st_b, const int64_t* st_c, int n_keep, gemm::GemmParams* p);
+}
+
+extern "C" int hgpu_contract_operands(hgpu_ctx* ctx, const hgpu_operand* a, const hgpu_operand* b, int n_keep, int flags, hgpu_array** out) {
+  if (!ctx || !a || !out) return HGPU_ERR_INVALID;
+  if (a->array && (!b || b->array)) {   // nothing to evaluate on the way: the plain contraction
+    return hgpu_contract(ctx, a->array, b ? b->array : nullptr, n_keep, out);
+  }
+  VirtualOp va, vb;
+  if (!a->array) if (int rc = virtual_from_operand(ctx, a, &va)) return rc;
+  if (b && !b->array) if (int rc = virtual_from_operand(ctx, b, &vb)) return rc;
+  // shape, strides and dtype of both operands
+  auto rank_of = [](const hgpu_operand* o) { return o->array ? o->array->rank : o->rank; };
+  auto shape_of = [](const hgpu_operand* o) { return o->array ? o->array->shape : o->shape; };
+  auto strides_of = [](const hgpu_operand* o) { return o->array ? o->array->strides : o->strides; };
+  const int rank = rank_of(a);
+  const int dtype = a->array ? a->array->dtype : va.dtype;
+  if (n_keep < 0 || n_keep > rank) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: n_keep %d of rank %d", n_keep, rank);
+  if (b) {
+    if (rank_of(b) != rank) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: ranks differ");
+    for (int d = 0; d < rank; ++d)
+      if (shape_of(b)[d] != shape_of(a)[d]) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: shapes differ");
+    if ((b->array ? b->array->dtype : vb.dtype) != dtype) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: dtypes differ");
+  }
+  if (dtype == HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "contract_operands: Bool values have no sum");
+  int64_t n_all = 1;
+  for (int d = 0; d < rank; ++d) n_all *= shape_of(a)[d];
+  if (n_all > 0 && (dtype == HGPU_F64 || dtype == HGPU_F32)) {
+    hgpu_array* o = nullptr;
+    int rc = new_dense(ctx, dtype, n_keep, shape_of(a), &o);
+    if (rc) return rc;
+    bool handled = false;
+    if (!b) {
+      rc = try_mapped_sum(ctx, va, a, n_keep, o, &handled);
+    } else if ((a->array || va.total < (1LL << 31)) && (b->array || vb.total < (1LL << 31))) {
+      GemmParams p;
+      if (hg::classify_contraction(rank, shape_of(a), strides_of(a), strides_of(b), o->strides, n_keep, &p)) {
+        p.n_terms = 0;
+        p.term_loop = 0;
+        const size_t es = dtype_size(dtype);
+        const void* pa = a->array ? data_ptr(a->array) : (const void*)(uintptr_t)(a->offset * (int64_t)es);
+        const void* pb = b->array ? data_ptr(b->array) : (const void*)(uintptr_t)(b->offset * (int64_t)es);
+        rc = hg::try_footprint_virtual(ctx, p, dtype, pa, pb, o, &handled, a->array ? nullptr : &va, b->array ? nullptr : &vb);
+      }
+    }
+    if (rc || handled) {
+      if (rc) hgpu_release(o); else *out = o;
+      return rc;
+    }
+    hgpu_release(o);
+  }
+  if (flags & 1) return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract_operands: no kernel takes these operands unevaluated");
+  hgpu_array *aa = nullptr, *bb = nullptr;
+  int rc = write_out(ctx, a, &aa);
+  if (!rc && b) rc = write_out(ctx, b, &bb);
+  if (!rc) rc = hgpu_contract(ctx, aa, bb, n_keep, out);
+  if (aa) hgpu_release(aa);
+  if (bb) hgpu_release(bb);
+  return rc;
 }

@@ -279,6 +279,60 @@ namespace hg {
 
 int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled);
 
+// The dims of a contraction out[kept] = sum a[kept, red] * b[kept, red] sorted
+// into row (M), column (N), reduced (K) and batch groups by which operand moves
+// along them; false when the strides do not make it a matrix product.
+bool classify_contraction(int rank, const int64_t* shape, const int64_t* st_a, const int64_t* st_b, const int64_t* st_c, int n_keep, GemmParams* p) {
+  p->m.nd = p->n.nd = p->k.nd = p->bt.nd = 0;
+  // Classify the dims.  The dims of a group are an index SET: any order works
+  // as long as A, B and C agree, so each group is sorted with the dim that is
+  // most contiguous in memory last (innermost) -- that is the dim the lanes of
+  // a load run along -- and only then merged.
+  struct DimRec { int64_t e, sa, sb, sc; };
+  std::vector<DimRec> gm, gn, gk, gb;
+  for (int i = 0; i < n_keep; ++i) {
+    int64_t e = shape[i], sa = st_a[i], sb = st_b[i], sc = st_c[i];
+    if (e == 1) continue;
+    if (sa != 0 && sb == 0) gm.push_back({e, sa, 0, sc});
+    else if (sa == 0 && sb != 0) gn.push_back({e, 0, sb, sc});
+    else if (sa != 0 && sb != 0) gb.push_back({e, sa, sb, sc});
+    else return false;  // an output dim neither operand depends on
+  }
+  for (int i = n_keep; i < rank; ++i) {
+    int64_t e = shape[i], sa = st_a[i], sb = st_b[i];
+    if (e == 1) continue;
+    if (sa == 0 || sb == 0) return false;  // a plain sum hidden in the contraction
+    gk.push_back({e, sa, sb, 0});
+  }
+  auto mag = [](int64_t v) { return v < 0 ? -v : v; };
+  std::stable_sort(gm.begin(), gm.end(), [&](const DimRec& x, const DimRec& y) { return mag(x.sa) > mag(y.sa); });
+  std::stable_sort(gn.begin(), gn.end(), [&](const DimRec& x, const DimRec& y) { return mag(x.sb) > mag(y.sb); });
+  {
+    // K: follow the operand that has a unit-stride K dim; when both or neither
+    // do, the one that is larger (more rows to stream)
+    int64_t rows_a = 1, rows_b = 1;
+    for (auto& d : gm) rows_a *= d.e;
+    for (auto& d : gn) rows_b *= d.e;
+    bool a_unit = false, b_unit = false;
+    for (auto& d : gk) { a_unit = a_unit || mag(d.sa) == 1; b_unit = b_unit || mag(d.sb) == 1; }
+    bool by_a = (a_unit != b_unit) ? a_unit : rows_a >= rows_b;
+    std::stable_sort(gk.begin(), gk.end(), [&](const DimRec& x, const DimRec& y) { return by_a ? mag(x.sa) > mag(y.sa) : mag(x.sb) > mag(y.sb); });
+  }
+  for (auto& d : gm) if (!push_dim(p->m, d.e, d.sa, d.sb, d.sc)) return false;
+  for (auto& d : gn) if (!push_dim(p->n, d.e, d.sa, d.sb, d.sc)) return false;
+  for (auto& d : gk) if (!push_dim(p->k, d.e, d.sa, d.sb, d.sc)) return false;
+  for (auto& d : gb) if (!push_dim(p->bt, d.e, d.sa, d.sb, d.sc)) return false;
+  finish(p->m);
+  finish(p->n);
+  finish(p->k);
+  finish(p->bt);
+  p->M = total(p->m);
+  p->N = total(p->n);
+  p->K = total(p->k);
+  p->BT = total(p->bt);
+  return true;
+}
+
 int sum_partials(hgpu_ctx* ctx, int dtype, int64_t n, int parts, const void* part, void* out) {
   size_t es = dtype_size(dtype);
   LaunchGuard ls(ctx, "gemm_sum_partials", (double)n * (parts + 1) * es, (double)n * parts);
@@ -296,53 +350,7 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   if (!b) return HGPU_OK;
   if (a->dtype != HGPU_F64 && a->dtype != HGPU_F32) return HGPU_OK;
   GemmParams p;
-  p.m.nd = p.n.nd = p.k.nd = p.bt.nd = 0;
-  // Classify the dims.  The dims of a group are an index SET: any order works
-  // as long as A, B and C agree, so each group is sorted with the dim that is
-  // most contiguous in memory last (innermost) -- that is the dim the lanes of
-  // a load run along -- and only then merged.
-  struct DimRec { int64_t e, sa, sb, sc; };
-  std::vector<DimRec> gm, gn, gk, gb;
-  for (int i = 0; i < n_keep; ++i) {
-    int64_t e = a->shape[i], sa = a->strides[i], sb = b->strides[i], sc = out->strides[i];
-    if (e == 1) continue;
-    if (sa != 0 && sb == 0) gm.push_back({e, sa, 0, sc});
-    else if (sa == 0 && sb != 0) gn.push_back({e, 0, sb, sc});
-    else if (sa != 0 && sb != 0) gb.push_back({e, sa, sb, sc});
-    else return HGPU_OK;  // an output dim neither operand depends on
-  }
-  for (int i = n_keep; i < a->rank; ++i) {
-    int64_t e = a->shape[i], sa = a->strides[i], sb = b->strides[i];
-    if (e == 1) continue;
-    if (sa == 0 || sb == 0) return HGPU_OK;  // a plain sum hidden in the contraction
-    gk.push_back({e, sa, sb, 0});
-  }
-  auto mag = [](int64_t v) { return v < 0 ? -v : v; };
-  std::stable_sort(gm.begin(), gm.end(), [&](const DimRec& x, const DimRec& y) { return mag(x.sa) > mag(y.sa); });
-  std::stable_sort(gn.begin(), gn.end(), [&](const DimRec& x, const DimRec& y) { return mag(x.sb) > mag(y.sb); });
-  {
-    // K: follow the operand that has a unit-stride K dim; when both or neither
-    // do, the one that is larger (more rows to stream)
-    int64_t rows_a = 1, rows_b = 1;
-    for (auto& d : gm) rows_a *= d.e;
-    for (auto& d : gn) rows_b *= d.e;
-    bool a_unit = false, b_unit = false;
-    for (auto& d : gk) { a_unit = a_unit || mag(d.sa) == 1; b_unit = b_unit || mag(d.sb) == 1; }
-    bool by_a = (a_unit != b_unit) ? a_unit : rows_a >= rows_b;
-    std::stable_sort(gk.begin(), gk.end(), [&](const DimRec& x, const DimRec& y) { return by_a ? mag(x.sa) > mag(y.sa) : mag(x.sb) > mag(y.sb); });
-  }
-  for (auto& d : gm) if (!push_dim(p.m, d.e, d.sa, d.sb, d.sc)) return HGPU_OK;
-  for (auto& d : gn) if (!push_dim(p.n, d.e, d.sa, d.sb, d.sc)) return HGPU_OK;
-  for (auto& d : gk) if (!push_dim(p.k, d.e, d.sa, d.sb, d.sc)) return HGPU_OK;
-  for (auto& d : gb) if (!push_dim(p.bt, d.e, d.sa, d.sb, d.sc)) return HGPU_OK;
-  finish(p.m);
-  finish(p.n);
-  finish(p.k);
-  finish(p.bt);
-  p.M = total(p.m);
-  p.N = total(p.n);
-  p.K = total(p.k);
-  p.BT = total(p.bt);
+  if (!classify_contraction(a->rank, a->shape, a->strides, b->strides, out->strides, n_keep, &p)) return HGPU_OK;
   // Worth the matrix cores only when there is reuse on both sides.
   if (p.K < 4 || p.M * p.N < 256) return HGPU_OK;
   if (p.BT > 65535) return HGPU_OK;

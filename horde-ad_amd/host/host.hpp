@@ -104,13 +104,15 @@ struct ArrHolder {
   // minimum of the reference's soft-max loss) is then those values, not a gather.
   std::shared_ptr<ArrHolder> arg_src, arg_values;
   // A pending VIEW (h == nullptr, ekind < 0, vsrc set): the strided view vmeta
-  // over the dense row-major result of vsrc, a value that is itself still
+  // over the dense row-major (and possibly zero-extended, vlo / vhi) result of vsrc, a value that is itself still
   // pending (a contraction, an elementwise expression).  Views of it compose
   // on the host; it is computed by computing vsrc once and viewing that.  An
   // elementwise expression made by viewing the leaves of another one (ekind >= 0)
   // carries the same two fields as a note: it equals that view of vsrc's result.
   std::shared_ptr<ArrHolder> vsrc;
   Meta vmeta;
+  // ... of vsrc's result zero-extended by vlo / vhi per dim (empty: not extended)
+  Shape vlo, vhi;
   // A stand-in without data that view operations are tried on to learn the
   // strides they produce (vmeta holds its shape and strides).
   bool probe = false;

@@ -245,7 +245,57 @@ static T make_view(const std::shared_ptr<ArrHolder>& src, const Meta& m) {
 // a with the strides of m: a probe stays a probe, a pending view stays one of the same source
 static T with_meta(const T& a, const Meta& m) {
   if (a.is_probe()) return make_probe(a.be(), m, a.dtype());
-  return make_view(a.holder()->vsrc, m);
+  T v = make_view(a.holder()->vsrc, m);
+  v.holder()->vlo = a.holder()->vlo;
+  v.holder()->vhi = a.holder()->vhi;
+  return v;
+}
+// an elementwise expression (also one over a refined index space) that is not yet written out
+static bool expression_like(const T& t) {
+  return t.valid() && (t.pending_expr() || (t.pending_merged() && T(t.holder()->mv_inner).pending_expr()));
+}
+// The zero-extension of a pending view, when the view merely permutes and
+// replicates the dims of its source's (zero-extended) result: the extension is
+// then one of the source's dims, and the view one of the larger layout.
+static bool pad_view(const T& a, const Shape& lo, const Shape& hi, T* out) {
+  const ArrHolder* h = a.holder().get();
+  T src(h->vsrc);
+  Shape M = src.shape();
+  Shape slo = h->vlo.empty() ? Shape(M.size(), 0) : h->vlo, shi = h->vhi.empty() ? Shape(M.size(), 0) : h->vhi;
+  Shape P(M.size());
+  for (size_t k = 0; k < M.size(); ++k) P[k] = M[k] + slo[k] + shi[k];
+  const Meta pd = dense_meta(P);
+  const Meta& vm = h->vmeta;
+  if (vm.offset != 0 || lo.size() != vm.shape.size() || hi.size() != vm.shape.size()) return false;
+  std::vector<int> dim_of(vm.shape.size(), -1);
+  std::vector<bool> used(M.size(), false);
+  for (size_t d = 0; d < vm.shape.size(); ++d) {
+    if (vm.shape[d] == 1 || vm.strides[d] == 0) {
+      if (lo[d] != 0 || hi[d] != 0) return false;   // a replicated dim cannot be extended by zeros here
+      continue;
+    }
+    for (size_t k = 0; k < M.size(); ++k)
+      if (!used[k] && P[k] == vm.shape[d] && pd.strides[k] == vm.strides[d] && P[k] > 1) { dim_of[d] = (int)k; break; }
+    if (dim_of[d] < 0) return false;
+    used[(size_t)dim_of[d]] = true;
+  }
+  for (size_t d = 0; d < vm.shape.size(); ++d) {
+    if (lo[d] < 0 || hi[d] < 0) return false;
+    if (dim_of[d] >= 0) { slo[(size_t)dim_of[d]] += lo[d]; shi[(size_t)dim_of[d]] += hi[d]; }
+  }
+  Shape P2(M.size());
+  for (size_t k = 0; k < M.size(); ++k) P2[k] = M[k] + slo[k] + shi[k];
+  const Meta pd2 = dense_meta(P2);
+  Meta m2;
+  m2.shape = vm.shape;
+  m2.strides.assign(vm.shape.size(), 0);
+  for (size_t d = 0; d < vm.shape.size(); ++d)
+    if (dim_of[d] >= 0) { m2.shape[d] = P2[(size_t)dim_of[d]]; m2.strides[d] = pd2.strides[(size_t)dim_of[d]]; }
+  T v = make_view(h->vsrc, m2);
+  v.holder()->vlo = slo;
+  v.holder()->vhi = shi;
+  *out = v;
+  return true;
 }
 // Tries a view operation on strides alone.  A probe that cannot take it gives
 // up (ProbeFail); a pending view falls through to the array path, which
@@ -472,6 +522,13 @@ void ArrHolder::force() {
     if (!be->api->is_dense(base)) {   // vmeta counts in the dense row-major layout of the source
       hgpu_array* d = nullptr;
       int rc = be->api->materialize(be->ctx, base, &d);
+      be->api->release(base);
+      be->check(rc);
+      base = d;
+    }
+    if (!vlo.empty()) {
+      hgpu_array* d = nullptr;
+      int rc = be->api->pad(be->ctx, base, ptr_or_dummy(vlo), ptr_or_dummy(vhi), &d);
       be->api->release(base);
       be->check(rc);
       base = d;
@@ -736,6 +793,7 @@ T transpose(const T& a, const std::vector<int>& perm) {
     return make_merged(transpose(T(h->mv_inner), fine_perm), shape, groups);
   }
   HD_META_VIEW(meta_transpose(a.holder()->vmeta, perm, &m__))
+  if (a.pending_merged() && expression_like(a) && a.size() > 0) return transpose(make_view(a.holder(), dense_meta(a.shape())), perm);
   HD_VIEW_OF_EXPR(transpose(x, perm))
   if (a.pending_contraction() && (int)perm.size() <= a.pending_keep())   // permutes kept dims only
   {
@@ -771,6 +829,14 @@ T reverse(const T& a, int dim) {
 T replicate(const T& a, const Shape& pre) {
   if (pre.empty()) return a;
   HD_META_VIEW(meta_replicate(a.holder()->vmeta, pre, &m__))
+  // An expression that is replicated stays unevaluated behind a pending view:
+  // a contraction may take it in as it is, anything else computes it once, for
+  // every view of it.
+  if (expression_like(a) && a.size() > 0 && a.be()->fuse) {
+    bool pos = true;
+    for (auto e : pre) pos = pos && e > 0;
+    if (pos) return replicate(make_view(a.holder(), dense_meta(a.shape())), pre);
+  }
   // a pending expression is written out before it is replicated: only shrinking
   // or permuting views of it are worth keeping pending
   HD_OUT(replicate(be__->ctx, a.h(), (int)pre.size(), pre.data(), &o__));
@@ -790,6 +856,10 @@ T materialize(const T& a) {
 }
 T pad(const T& a, const Shape& lo, const Shape& hi) {
   if (a.is_probe()) throw ProbeFail{};
+  if (a.pending_view() && expression_like(T(a.holder()->vsrc))) {
+    T v;
+    if (pad_view(a, lo, hi, &v)) return v;
+  }
   // zeros before and after along the first dim only: a pending concatenation
   bool first_only = a.be()->fuse && a.rank() >= 1 && (int)lo.size() == a.rank() && (int)hi.size() == a.rank() && lo[0] >= 0 && hi[0] >= 0 && lo[0] + hi[0] > 0;
   for (size_t i = 1; i < lo.size() && first_only; ++i) first_only = lo[i] == 0 && hi[i] == 0;
@@ -889,7 +959,66 @@ T contract(const T& a, const T* b, int n_keep) {
     return lazy_contract(a, *b, n_keep);
   return contract_now(a, b, n_keep);
 }
+namespace {
+// One operand of hgpu_contract_operands and the storage its pointers point into.
+struct OperandBuf {
+  hgpu_operand op;
+  std::vector<const hgpu_array*> ins;
+  std::vector<hgpu_fused_instr> prog;
+  std::vector<int> slots;
+  Shape mshape, lo, hi, shape, strides;
+};
+bool virtual_operand(const T& t) { return t.valid() && t.pending_view() && expression_like(T(t.holder()->vsrc)); }
+void fill_operand(const T& t, OperandBuf* ob) {
+  std::memset(&ob->op, 0, sizeof ob->op);
+  if (!virtual_operand(t)) { ob->op.array = t.h(); return; }
+  const ArrHolder* h = t.holder().get();
+  T src(h->vsrc);
+  T e = src.pending_merged() ? T(src.holder()->mv_inner) : src;
+  number_program({e.holder().get()}, &ob->ins, &ob->prog, &ob->slots);
+  ob->mshape = src.shape();
+  ob->lo = h->vlo;
+  ob->hi = h->vhi;
+  ob->shape = h->vmeta.shape;
+  ob->strides = h->vmeta.strides;
+  ob->op.n_in = (int)ob->ins.size();
+  ob->op.in = ob->ins.data();
+  ob->op.n_instr = (int)ob->prog.size();
+  ob->op.prog = ob->prog.data();
+  ob->op.slot = ob->slots[0];
+  ob->op.rank_m = (int)ob->mshape.size();
+  ob->op.mshape = ptr_or_dummy(ob->mshape);
+  ob->op.lo = ob->lo.empty() ? nullptr : ob->lo.data();
+  ob->op.hi = ob->hi.empty() ? nullptr : ob->hi.data();
+  ob->op.rank = (int)ob->shape.size();
+  ob->op.shape = ptr_or_dummy(ob->shape);
+  ob->op.strides = ptr_or_dummy(ob->strides);
+  ob->op.offset = h->vmeta.offset;
+}
+}  // namespace
+
 static T contract_now(const T& a, const T* b, int n_keep) {
+  // An operand that is a view of an unevaluated expression goes to the provider
+  // as the expression: a kernel that evaluates it while staging never writes it
+  // out.  Where there is no such kernel the expression is computed once (for
+  // all its views) and the plain contraction runs on the views.
+  Backend* be = a.be();
+  const hgpu_api* api = be->api;
+  if ((virtual_operand(a) || (b && virtual_operand(*b))) && api->struct_size >= offsetof(hgpu_api, contract_operands) + sizeof(api->contract_operands) &&
+      api->contract_operands && a.size() > 0) {
+    OperandBuf oa, ob;
+    fill_operand(a, &oa);
+    if (b) fill_operand(*b, &ob);
+    if ((int)oa.ins.size() <= 12 && (int)oa.prog.size() <= 96 && (int)ob.ins.size() <= 12 && (int)ob.prog.size() <= 96) {
+      hgpu_array* o = nullptr;
+      int rc = api->contract_operands(be->ctx, &oa.op, b ? &ob.op : nullptr, n_keep, 1, &o);
+      if (rc == HGPU_OK) {
+        be->counters["contract_operands"]++;
+        return T(be, o);
+      }
+      if (rc != HGPU_ERR_UNSUPPORTED) be->check(rc);
+    }
+  }
   HD_OUT(contract(be__->ctx, a.h(), b ? b->h() : nullptr, n_keep, &o__));
 }
 T argminmax_last(const T& a, bool want_max) { HD_OUT(argminmax_last(be__->ctx, a.h(), want_max ? 1 : 0, &o__)); }

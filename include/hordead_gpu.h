@@ -270,6 +270,38 @@ int hgpu_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, i
                       int ext_slot, int view_rank, const int64_t* view_shape, const int64_t* view_strides,
                       int n_reduce, int want_max, hgpu_array** values, hgpu_array** indices);
 
+/* hgpu_contract whose operands need not exist in memory.  The cotangent of a
+ * pooled, rectified convolution -- `sscatter` at the arg-maxima, times the relu
+ * mask (test/simplified/TestMnistPP.hs:734-735) -- is an elementwise expression
+ * of small arrays, four times their size, that three contractions consume (the
+ * bias, kernel and input gradients).  An operand is either a plain array or
+ *   E = slot `slot` of an elementwise program over `in` (views of one shape),
+ *   P = E, its dims merged to `mshape` (same element count; row-major, so
+ *       merging is free), zero-extended by lo / hi per dim (NULL: none),
+ *   operand = the view (rank, shape, strides, offset) of P's dense row-major layout,
+ * evaluated while the kernel stages it.  b == NULL is a plain sum of a over the
+ * dims behind the first n_keep.  flags bit 0: fail with HGPU_ERR_UNSUPPORTED when
+ * no kernel takes the operands in this form, instead of writing them out first
+ * (what the call otherwise does: results equal hgpu_fused_map, hgpu_reshape,
+ * hgpu_pad, hgpu_as_strided and hgpu_contract applied one after another). */
+typedef struct hgpu_operand {
+  const hgpu_array* array;              /* not NULL: the operand is this array, the rest is ignored */
+  int n_in;
+  const hgpu_array* const* in;
+  int n_instr;
+  const hgpu_fused_instr* prog;
+  int slot;
+  int rank_m;
+  const int64_t* mshape;
+  const int64_t* lo;
+  const int64_t* hi;
+  int rank;
+  const int64_t* shape;
+  const int64_t* strides;
+  int64_t offset;
+} hgpu_operand;
+int hgpu_contract_operands(hgpu_ctx* ctx, const hgpu_operand* a, const hgpu_operand* b, int n_keep, int flags, hgpu_array** out);
+
 /* hgpu_contract for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
  * no counterpart in the reference.  The caller brings the result array `out`
@@ -425,6 +457,7 @@ typedef struct hgpu_api {
   int (*fused_sum)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, hgpu_array**);
   int (*contract_map)(hgpu_ctx*, const hgpu_array*, const hgpu_array*, int, int, const hgpu_array* const*, int, const hgpu_fused_instr*,
                       int, const int*, hgpu_array**, int, int, const int64_t*, const int64_t*, int, int, hgpu_array**, hgpu_array**);
+  int (*contract_operands)(hgpu_ctx*, const hgpu_operand*, const hgpu_operand*, int, int, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

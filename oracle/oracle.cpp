@@ -37,6 +37,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -815,6 +816,52 @@ int horc_contract_map(hgpu_ctx* c, const hgpu_array* a, const hgpu_array* b, int
   return rc;
 }
 
+// an operand of horc_contract_operands written out: program, merged dims, zero-extension, view
+static int operand_array(hgpu_ctx* c, const hgpu_operand* o, hgpu_array** out) {
+  if (o->array) { horc_retain(const_cast<hgpu_array*>(o->array)); *out = const_cast<hgpu_array*>(o->array); return HGPU_OK; }
+  hgpu_array *e = nullptr, *m = nullptr, *p = nullptr;
+  int rc = horc_fused_map(c, o->n_in, o->in, o->n_instr, o->prog, 1, &o->slot, &e);
+  if (rc) return rc;
+  rc = horc_reshape(c, e, o->rank_m, o->mshape, &m);
+  horc_release(e);
+  if (rc) return rc;
+  if (o->lo && o->hi) {
+    rc = horc_pad(c, m, o->lo, o->hi, &p);
+    horc_release(m);
+    if (rc) return rc;
+  } else {
+    p = m;
+  }
+  rc = horc_as_strided(c, p, o->rank, o->shape, o->strides, o->offset, out);
+  horc_release(p);
+  return rc;
+}
+
+int horc_contract_operands(hgpu_ctx* c, const hgpu_operand* a, const hgpu_operand* b, int n_keep, int, hgpu_array** out) {
+  if (getenv("HORC_TRACE")) {
+    auto show = [](const char* name, const hgpu_operand* o) {
+      if (!o) { fprintf(stderr, "  %s: none\n", name); return; }
+      if (o->array) { fprintf(stderr, "  %s: array rank %d\n", name, (int)o->array->shape.size()); return; }
+      fprintf(stderr, "  %s: program in%d instr%d, mshape", name, o->n_in, o->n_instr);
+      for (int i = 0; i < o->rank_m; ++i) fprintf(stderr, " %lld", (long long)o->mshape[i]);
+      if (o->lo) { fprintf(stderr, " lo"); for (int i = 0; i < o->rank_m; ++i) fprintf(stderr, " %lld", (long long)o->lo[i]); fprintf(stderr, " hi"); for (int i = 0; i < o->rank_m; ++i) fprintf(stderr, " %lld", (long long)o->hi[i]); }
+      fprintf(stderr, "; view");
+      for (int i = 0; i < o->rank; ++i) fprintf(stderr, " %lld:%lld", (long long)o->shape[i], (long long)o->strides[i]);
+      fprintf(stderr, " +%lld\n", (long long)o->offset);
+    };
+    fprintf(stderr, "contract_operands n_keep %d\n", n_keep);
+    show("a", a);
+    show("b", b);
+  }
+  hgpu_array *aa = nullptr, *bb = nullptr;
+  int rc = operand_array(c, a, &aa);
+  if (!rc && b) rc = operand_array(c, b, &bb);
+  if (!rc) rc = horc_contract(c, aa, bb, n_keep, out);
+  if (aa) horc_release(aa);
+  if (bb) horc_release(bb);
+  return rc;
+}
+
 const hgpu_api* horc_get_api(void) {
   static const hgpu_api api = {
       sizeof(hgpu_api),
@@ -831,6 +878,7 @@ const hgpu_api* horc_get_api(void) {
       nullptr,   // no fused_extremum
       nullptr,   // no fused_sum
       nullptr,   // no contract_map
+      nullptr,   // no contract_operands
   };
   return &api;
 }
@@ -841,6 +889,7 @@ const hgpu_api* horc_get_api_fused(void) {
   api.fused_extremum = horc_fused_extremum;
   api.fused_sum = horc_fused_sum;
   api.contract_map = horc_contract_map;
+  api.contract_operands = horc_contract_operands;
   return &api;
 }
 

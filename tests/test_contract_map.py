@@ -139,3 +139,102 @@ def test_host_rewrites_pooling_layers_onto_contract_map():
     assert res[0][0] == res[1][0]
     for g0, g1 in zip(res[0][1], res[1][1]):
         assert np.array_equal(g0, g1)
+
+
+# ---- hgpu_contract_operands: operands that are unevaluated expressions ------
+
+def pooled_cotangent(ctx, rng, B, Co, H, Wd, dtype):
+    """The cotangent of relu + 2x2 max-pooling as an expression over the refined space
+    [B, Co, H/2, 2, W/2, 2]: (which == arg ? dpool : 0) * (mask ? 0 : 1).  Returns
+    (inputs, program, slot, merged shape, the same as a numpy array)."""
+    O2, CMP = capi.OP2, capi.CMP
+    H2, W2 = H // 2, Wd // 2
+    dpool = rng.uniform(-1, 1, (B, Co, H2, W2)).astype(dtype)
+    arg = rng.integers(0, 4, (B, Co, H2, W2)).astype(np.int64)
+    mask = rng.integers(0, 2, (B, Co, H, Wd)).astype(bool)
+    cz = np.zeros((B, Co, H2, 2, W2, 2), dtype)
+    for p in range(2):
+        for q in range(2):
+            cz[:, :, :, p, :, q] = np.where(arg == 2 * p + q, dpool, 0)
+    cz = cz.reshape(B, Co, H, Wd) * np.where(mask, 0, 1)
+    E = [B, Co, H2, 2, W2, 2]
+    small = [Co * H2 * W2, H2 * W2, W2, 0, 1, 0]
+    ins = [ctx.upload(dpool).as_strided(E, small, 0), ctx.upload(arg).as_strided(E, small, 0), ctx.upload(mask).reshape(E),
+           ctx.iota(4).as_strided(E, [0, 0, 0, 2, 0, 1], 0), ctx.upload(np.zeros((), dtype)).as_strided(E, [0] * 6, 0),
+           ctx.upload(np.ones((), dtype)).as_strided(E, [0] * 6, 0)]
+    # 6 = (which == arg); 7 = 6 ? dpool : 0; 8 = mask ? 0 : 1; 9 = 8 * 7
+    prog = [(2, CMP["eq"], 0, 3, 1, 0), (3, 0, 0, 6, 0, 4), (3, 0, 0, 2, 4, 5), (1, O2["mul"], 0, 8, 7, 0)]
+    return ins, prog, 9, [B, Co, H, Wd], cz
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,Ci,Co,H,Wd,k,dtype,fused", [(300, 16, 16, 14, 14, 5, np.float64, True), (300, 16, 16, 14, 14, 5, np.float32, None),
+                                                        (280, 1, 16, 28, 28, 5, np.float64, False), (5, 2, 4, 8, 8, 3, np.float64, False)])
+def test_gradients_of_a_convolution_from_an_unevaluated_cotangent(gpu, B, Ci, Co, H, Wd, k, dtype, fused):
+    """Bias, kernel and input gradient of a convolution layer read the pooled
+    cotangent through arg-maxima and relu mask while staging (`fused`: a kernel
+    takes it so; False: the call writes it out first; None: either) -- against numpy."""
+    rng = np.random.default_rng(8)
+    ins, prog, slot, M, cz = pooled_cotangent(gpu, rng, B, Co, H, Wd, dtype)
+    x = rng.uniform(-1, 1, (B, Ci, H + k - 1, Wd + k - 1)).astype(dtype)
+    ker = rng.uniform(-0.4, 0.4, (Co, Ci, k, k)).astype(dtype)
+    tol = 1e-10 if dtype == np.float64 else 1e-5
+    Hp, Wp, pad = H + k - 1, Wd + k - 1, k - 1
+
+    def close(got, want):
+        return np.max(np.abs(got - want)) <= tol * np.max(np.abs(want))
+
+    def call(a, b, n_keep):
+        gpu.profile(2)
+        try:
+            out = gpu.contract_operands(a, b, n_keep, fused_only=True).numpy()
+            took = True
+        except capi.HgpuError as e:
+            assert e.code == 4
+            out = gpu.contract_operands(a, b, n_keep).numpy()
+            took = False
+        labels = list(gpu.profile_report())
+        gpu.profile(0)
+        return out, took, labels
+
+    # the bias gradient: a sum over image, row and column
+    op = gpu.operand(ins, prog, slot, M, ([Co, B, H, Wd], [H * Wd, Co * H * Wd, Wd, 1], 0))
+    got, took, labels = call(op, None, 1)
+    assert close(got, cz.sum(axis=(0, 2, 3)).astype(dtype)) and took == (B * H * Wd >= 16384), labels
+    # the kernel gradient: dK[co, ci, p, q] = sum_{b, h, w} cz[b, co, h, w] * x[b, ci, h + p, w + q]
+    sh = [Co, Ci, k, k, B, H, Wd]
+    a_op = gpu.operand(ins, prog, slot, M, (sh, [H * Wd, 0, 0, 0, Co * H * Wd, Wd, 1], 0))
+    gx = gpu.upload(x).as_strided(sh, [0, Hp * Wp, Wp, 1, Ci * Hp * Wp, Wp, 1], 0)
+    got, took, labels = call(a_op, gx, 4)
+    win = np.lib.stride_tricks.sliding_window_view(x, (k, k), axis=(2, 3))[:, :, :H, :Wd]
+    assert close(got, np.einsum("bohw,bihwpq->oipq", cz.astype(np.float64), win.astype(np.float64))) and (fused is None or took == fused), labels
+    # the input gradient over the zero-extended cotangent, the kernel flipped
+    sh = [B, Ci, Hp, Wp, Co, k, k]
+    Pl = [B, Co, H + 2 * pad, Wd + 2 * pad]
+    ps = [Co * Pl[2] * Pl[3], Pl[2] * Pl[3], Pl[3], 1]
+    b_op = gpu.operand(ins, prog, slot, M, (sh, [ps[0], 0, ps[2], ps[3], ps[1], -ps[2], -ps[3]], pad * ps[2] + pad * ps[3]),
+                       pad=([0, 0, pad, pad], [0, 0, pad, pad]))
+    gk = gpu.upload(ker).as_strided(sh, [0, k * k, 0, 0, Ci * k * k, k, 1], 0)
+    got, took, labels = call(gk, b_op, 4)
+    czp = np.pad(cz, ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+    wz = np.lib.stride_tricks.sliding_window_view(czp, (k, k), axis=(2, 3))
+    # (whether a kernel takes this one unevaluated depends on how many loads a staging pass of the extended footprint needs)
+    assert close(got, np.einsum("bcyxuv,ciuv->biyx", wz.astype(np.float64), ker[:, :, ::-1, ::-1].astype(np.float64))), labels
+
+
+def test_host_rewrites_gradients_onto_contract_operands():
+    """On the checker's fused table the cotangents of the CNN's pooled layers reach
+    the contractions unevaluated, and the gradients equal the plain table's."""
+    H, W = pkg.hostapi, pkg.workloads
+    plain = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    fused = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_", api_table="get_api_fused"))
+    for wl in (W.c3_cnn(batch=4), W.c1_fcnn(batch=7), W.c4_rnn(batch=3, steps=4)):
+        res = []
+        for host in (plain, fused):
+            ps, ds = wl.upload(host)
+            loss, grads = wl.gradient(host, ps, ds)
+            res.append((float(loss.numpy()), [g.numpy() for g in grads]))
+        assert res[0][0] == res[1][0], wl.name
+        for g0, g1 in zip(res[0][1], res[1][1]):
+            assert np.array_equal(g0, g1), wl.name
+    assert plain.counter("contract_operands") == 0 and fused.counter("contract_operands") >= 5
