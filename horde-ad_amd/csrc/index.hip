@@ -9,7 +9,16 @@
 //
 // Out-of-bounds rule (OpsConcrete.hs:923-950): a position with any index
 // outside [0, extent) reads zeros in gather and is skipped in scatter.
+//
+// Scatter-add adds colliding positions in ascending row-major order of the
+// positions, the reference's own order (tscatterZSScalar walks `shsEnum shm`,
+// OpsConcrete.hs:1581-1619), and without atomics: the positions are sorted by
+// destination with a stable radix sort, and every destination's run is summed
+// front to back by one lane per element.  Results do not depend on the run and,
+// for floating point, carry the rounding of that very order.
 #include "common.hpp"
+
+#include <rocprim/rocprim.hpp>
 
 using namespace hg;
 
@@ -84,26 +93,10 @@ __global__ void __launch_bounds__(kBlock) k_gather(IxSpace sp, Dims inner, int64
   }
 }
 
-template <typename T> struct atomic_ok { static constexpr bool value = false; };
-template <> struct atomic_ok<double> { static constexpr bool value = true; };
-template <> struct atomic_ok<float> { static constexpr bool value = true; };
-template <> struct atomic_ok<int32_t> { static constexpr bool value = true; };
-template <> struct atomic_ok<int64_t> { static constexpr bool value = true; };
-
-template <typename T>
-__device__ __forceinline__ void atomic_add(T* p, T v) {
-  if constexpr (sizeof(T) == 8 && !std::is_floating_point<T>::value) {
-    atomicAdd(reinterpret_cast<unsigned long long*>(p), (unsigned long long)v);
-  } else if constexpr (std::is_floating_point<T>::value) {
-    unsafeAtomicAdd(p, v);
-  } else {
-    atomicAdd(p, v);
-  }
-}
-
 // src is a view [M (position dims), N (inner dims)]; out dense [P, N], zeroed.
-template <typename T, bool INJECTIVE>
-__global__ void __launch_bounds__(kBlock) k_scatter(IxSpace sp, Dims inner, int64_t M, int64_t N, const T* __restrict__ src, T* __restrict__ out) {
+// Distinct positions go to distinct places (the caller's promise): plain stores.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_scatter_store(IxSpace sp, Dims inner, int64_t M, int64_t N, const T* __restrict__ src, T* __restrict__ out) {
   int64_t total = M * N;
   int64_t step = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += step) {
@@ -114,10 +107,52 @@ __global__ void __launch_bounds__(kBlock) k_scatter(IxSpace sp, Dims inner, int6
     if (ok) {
       int64_t io[1];
       decompose<1>(inner, n, io);
-      T v = src[doff + io[0]];
-      if constexpr (INJECTIVE) out[toff + n] = v;
-      else atomic_add<T>(&out[toff + n], v);
+      out[toff + n] = src[doff + io[0]];
     }
+  }
+}
+
+// key[m] = where position m's slice starts in out (the same for colliding
+// positions), or `skip` when an index is out of bounds; val[m] = m.
+__global__ void __launch_bounds__(kBlock) k_scatter_keys(IxSpace sp, int64_t M, uint64_t skip, uint64_t* __restrict__ key, uint32_t* __restrict__ val) {
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t m = (int64_t)blockIdx.x * kBlock + threadIdx.x; m < M; m += step) {
+    int64_t toff, doff;
+    bool ok = resolve(sp, m, &toff, &doff);
+    key[m] = ok ? (uint64_t)toff : skip;
+    val[m] = (uint32_t)m;
+  }
+}
+
+// the data operand's offset of position m (resolve() without the index arrays)
+__device__ __forceinline__ int64_t data_offset(const IxSpace& sp, int64_t m) {
+  int64_t doff = 0, r = m;
+  for (int i = sp.nd - 1; i >= 0; --i) {
+    int64_t c = r;
+    if (i > 0) { int64_t q = r / sp.shape[i]; c = r - q * sp.shape[i]; r = q; }
+    doff += c * sp.data_st[i];
+  }
+  return doff;
+}
+
+// key / val sorted by key, equal keys in ascending position order.  One lane per
+// (run, inner element): the lane at a run's first entry adds the run's slices
+// front to back, starting from zero, and writes the sum; the others have nothing to do.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_scatter_runs(IxSpace sp, Dims inner, int64_t M, int64_t N, uint64_t skip, const uint64_t* __restrict__ key,
+                                                         const uint32_t* __restrict__ val, const T* __restrict__ src, T* __restrict__ out) {
+  int64_t total = M * N;
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += step) {
+    int64_t at = N == 1 ? i : i / N;
+    int64_t n = N == 1 ? 0 : i - at * N;
+    const uint64_t k = key[at];
+    if (k == skip || (at > 0 && key[at - 1] == k)) continue;
+    int64_t io[1];
+    decompose<1>(inner, n, io);
+    T acc = T(0);
+    for (int64_t j = at; j < M && key[j] == k; ++j) acc = (T)(acc + src[data_offset(sp, (int64_t)val[j]) + io[0]]);
+    out[(int64_t)k + n] = acc;
   }
 }
 
@@ -261,23 +296,45 @@ int hgpu_scatter_add(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_
   Dims inner;
   if (!collapse(rank_n, src->shape + rank_m, 1, is, &inner)) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "scatter: too many inner dims"); }
   bool inj = (flags & 1) != 0;
-  bool launched = false;
-  {
-    LaunchGuard lg(ctx, inj ? "scatter_store" : "scatter_atomic", 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, (double)M * N);
+  if (inj) {
+    LaunchGuard lg(ctx, "scatter_store", 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, 0);
     unsigned g = grid_for(M * N, kBlock, ctx->num_cu * 8);
-    HG_DISPATCH_DTYPE(src->dtype, T, {
-      if constexpr (atomic_ok<T>::value) {
-        if (inj) hipLaunchKernelGGL((k_scatter<T, true>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, (const T*)data_ptr(src), (T*)data_ptr(o));
-        else hipLaunchKernelGGL((k_scatter<T, false>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, (const T*)data_ptr(src), (T*)data_ptr(o));
-        launched = true;
-      } else {
-        if (inj) { hipLaunchKernelGGL((k_scatter<T, true>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, (const T*)data_ptr(src), (T*)data_ptr(o)); launched = true; }
-      }
-    });
+    HG_DISPATCH_DTYPE(src->dtype, T, hipLaunchKernelGGL((k_scatter_store<T>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, (const T*)data_ptr(src), (T*)data_ptr(o)));
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "scatter"); }
+    *out = o;
+    return HGPU_OK;
   }
-  if (!launched) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "scatter: no accumulating kernel for dtype %d", src->dtype); }
+  // sort the positions by destination (stable: colliding positions stay in ascending order), then sum every run in that order
+  if (M >= (int64_t)1 << 32) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "scatter: %lld positions", (long long)M); }
+  const uint64_t skip = (uint64_t)nelem(o);   // larger than every slice start
+  int end_bit = 1;
+  while (end_bit < 64 && (skip >> end_bit) != 0) ++end_bit;
+  hgpu_buffer *kb = nullptr, *vb = nullptr, *tb = nullptr;
+  auto drop = [&] { if (kb) buffer_release(kb); if (vb) buffer_release(vb); if (tb) buffer_release(tb); };
+  rc = buffer_alloc(ctx, (size_t)M * 16, &kb);          // keys in, keys out
+  if (!rc) rc = buffer_alloc(ctx, (size_t)M * 8, &vb);  // positions in, positions out
+  if (rc) { drop(); hgpu_release(o); return rc; }
+  uint64_t* key_in = (uint64_t*)kb->ptr;
+  uint64_t* key_out = key_in + M;
+  uint32_t* val_in = (uint32_t*)vb->ptr;
+  uint32_t* val_out = val_in + M;
+  size_t temp_bytes = 0;
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp_bytes, key_in, key_out, val_in, val_out, (size_t)M, 0, (unsigned)end_bit, ctx->stream);
+  if (e == hipSuccess) {
+    rc = buffer_alloc(ctx, temp_bytes > 0 ? temp_bytes : 1, &tb);
+    if (rc) { drop(); hgpu_release(o); return rc; }
+    LaunchGuard lg(ctx, "scatter_sorted", 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, (double)M * N);
+    hipLaunchKernelGGL(k_scatter_keys, dim3(grid_for(M, kBlock, ctx->num_cu * 8)), dim3(kBlock), 0, ctx->stream, sp, M, skip, key_in, val_in);
+    e = rocprim::radix_sort_pairs(tb->ptr, temp_bytes, key_in, key_out, val_in, val_out, (size_t)M, 0, (unsigned)end_bit, ctx->stream);
+    if (e == hipSuccess) {
+      unsigned g = grid_for(M * N, kBlock, ctx->num_cu * 8);
+      HG_DISPATCH_DTYPE(src->dtype, T, hipLaunchKernelGGL((k_scatter_runs<T>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, skip, key_out, val_out, (const T*)data_ptr(src), (T*)data_ptr(o)));
+      e = hipGetLastError();
+    }
+  }
+  drop();
+  if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "scatter"); }
   *out = o;
   return HGPU_OK;
 }

@@ -343,10 +343,14 @@ int hgpu_gather(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array
  *   out = 0;  out[ix[0][m..], ..., ix[n_ix-1][m..], n..] += src[m.., n..]
  * src has shape shm ++ shn (rank_m leading dims are shm), out has shape
  * shp ++ shn with shp given (n_ix dims).  Positions with an index out of
- * bounds are skipped (OpsConcrete.hs:944-950).  Integers exact; floating
- * point sums may be associated differently from the reference's ascending
- * row-major order.  `flags`: bit 0 = the caller guarantees distinct
- * positions map to distinct destinations (plain stores suffice). */
+ * bounds are skipped (OpsConcrete.hs:944-950).  Positions that land on one
+ * place are added in ascending row-major order of the positions, starting
+ * from zero -- the reference's order (`shsEnum`, OpsConcrete.hs:1594,1613) --
+ * without atomics (a stable sort by destination, then every run summed front
+ * to back): results are the same from run to run, for every element type of
+ * the whitelist, and floating-point sums carry the rounding of that order.
+ * `flags`: bit 0 = the caller guarantees distinct positions map to distinct
+ * destinations (plain stores, no sort). */
 int hgpu_scatter_add(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array* const* ix,
                      int rank_m, const int64_t* shp, int flags, hgpu_array** out);
 /* tsscatter (OpsConcrete.hs:1581-1619) for an index function that is AFFINE in
