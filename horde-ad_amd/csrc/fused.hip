@@ -660,3 +660,182 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   *out = o;
   return HGPU_OK;
 }
+
+// hgpu_fused_map with sums: the map's outputs and the sums of some slots from
+// one pass over dense inputs.  Per-block partial sums (double / int64), added
+// up in a fixed order by a second, one-block launch.
+extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int n_out,
+                                   const int* out_slots, hgpu_array** outs, int n_sum, const int* sum_slots, hgpu_array** sums) {
+  if (!ctx || !in || !prog || (n_out > 0 && (!out_slots || !outs)) || (n_sum > 0 && (!sum_slots || !sums))) return HGPU_ERR_INVALID;
+  if (n_in < 1 || n_in > kMaxIn || n_out < 0 || n_out > kMaxOut || n_sum < 1 || n_sum > 4 || n_instr < 1 || n_instr > kMaxInstr)
+    return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map_sums: %d inputs, %d instructions, %d outputs, %d sums", n_in, n_instr, n_out, n_sum);
+  const hgpu_array* a0 = in[0];
+  for (int i = 0; i < n_in; ++i) {
+    if (!in[i]) return HGPU_ERR_INVALID;
+    if (!same_shape(in[i], a0)) return fail(ctx, HGPU_ERR_INVALID, "fused_map_sums: input %d has another shape", i);
+  }
+  std::vector<int> dt;
+  if (int rc = check_program(ctx, n_in, in, n_instr, prog, &dt)) return rc;
+  for (int o = 0; o < n_out; ++o)
+    if (out_slots[o] < 0 || out_slots[o] >= n_in + n_instr) return fail(ctx, HGPU_ERR_INVALID, "fused_map_sums: bad output slot");
+  for (int j = 0; j < n_sum; ++j) {
+    if (sum_slots[j] < 0 || sum_slots[j] >= n_in + n_instr) return fail(ctx, HGPU_ERR_INVALID, "fused_map_sums: bad sum slot");
+    if (dt[(size_t)sum_slots[j]] == HGPU_BOOL) return fail(ctx, HGPU_ERR_INVALID, "fused_map_sums: Bool values have no sum");
+  }
+  const int64_t n = nelem(a0);
+  if (n == 0) return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map_sums: empty arrays");
+  std::string layout((size_t)n_in, 'g');
+  size_t widest = 1;
+  for (int i = 0; i < n_in; ++i) {
+    bool all0 = true;
+    for (int d = 0; d < in[i]->rank; ++d)
+      if (in[i]->shape[d] != 1 && in[i]->strides[d] != 0) all0 = false;
+    if (all0) layout[(size_t)i] = 's';
+    else if (is_dense(in[i]) && ((uintptr_t)data_ptr(in[i]) & 15) == 0) layout[(size_t)i] = 'd';
+    else return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map_sums: input %d is a strided view", i);
+    widest = std::max(widest, dtype_size(in[i]->dtype));
+  }
+  std::vector<hgpu_array*> res((size_t)n_out, nullptr), sres((size_t)n_sum, nullptr);
+  auto release_all = [&] { for (auto* r : res) if (r) hgpu_release(r); for (auto* r : sres) if (r) hgpu_release(r); };
+  for (int o = 0; o < n_out; ++o) {
+    int rc = new_dense(ctx, dt[(size_t)out_slots[o]], a0->rank, a0->shape, &res[(size_t)o]);
+    if (rc) { release_all(); return rc; }
+    widest = std::max(widest, dtype_size(res[(size_t)o]->dtype));
+  }
+  for (int j = 0; j < n_sum; ++j) {
+    int rc = new_dense(ctx, dt[(size_t)sum_slots[j]], 0, nullptr, &sres[(size_t)j]);
+    if (rc) { release_all(); return rc; }
+    widest = std::max(widest, dtype_size(dt[(size_t)sum_slots[j]]));
+  }
+  const int vec = (int)(16 / widest);
+  const unsigned grid = grid_for((n + vec - 1) / vec, 256, ctx->num_cu * 16);
+  hgpu_buffer* part = nullptr;
+  int rc = buffer_alloc(ctx, (size_t)grid * 8 * (size_t)n_sum, &part);
+  if (rc) { release_all(); return rc; }
+
+  std::ostringstream s;
+  s << kPrelude;
+  s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
+  s << "template <typename A> __device__ __forceinline__ A wave_sum(A v) {\n"
+       "  for (int off = 32; off > 0; off >>= 1) {\n"
+       "    unsigned long long u = *reinterpret_cast<unsigned long long*>(&v);\n"
+       "    unsigned lo = __shfl_down((unsigned)(u & 0xffffffffu), off, 64), hi = __shfl_down((unsigned)(u >> 32), off, 64);\n"
+       "    unsigned long long w = ((unsigned long long)hi << 32) | lo;\n"
+       "    v += *reinterpret_cast<A*>(&w);\n"
+       "  }\n  return v;\n}\n";
+  auto acc_t = [&](int j) { return dtype_is_float(dt[(size_t)sum_slots[j]]) ? "double" : "i64"; };
+  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_map_sums(i64 n";
+  for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
+  for (int o = 0; o < n_out; ++o) s << ", " << ctype(res[(size_t)o]->dtype) << "* __restrict__ o" << o;
+  s << ", unsigned long long* __restrict__ part) {\n";
+  s << "  __shared__ unsigned long long red[4];\n";
+  s << "  const i64 step = (i64)gridDim.x * 256;\n";
+  for (int i = 0; i < n_in; ++i)
+    if (layout[(size_t)i] == 's') s << "  const " << ctype(in[i]->dtype) << " s" << i << " = i" << i << "[0];\n";
+  for (int j = 0; j < n_sum; ++j) s << "  " << acc_t(j) << " acc" << j << " = 0;\n";
+  s << "  const i64 nv = n / " << vec << ";\n";
+  s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < nv; i += step) {\n";
+  for (int i = 0; i < n_in; ++i)
+    if (layout[(size_t)i] == 'd') s << "    const Vec<" << ctype(in[i]->dtype) << ", " << vec << "> l" << i << " = reinterpret_cast<const Vec<" << ctype(in[i]->dtype) << ", " << vec << ">*>(i" << i << ")[i];\n";
+  for (int o = 0; o < n_out; ++o) s << "    Vec<" << ctype(res[(size_t)o]->dtype) << ", " << vec << "> r" << o << ";\n";
+  for (int e = 0; e < vec; ++e) {
+    std::string suf = "_" + std::to_string(e);
+    s << "    {\n";
+    for (int i = 0; i < n_in; ++i) {
+      s << "      const " << ctype(in[i]->dtype) << " v" << i << suf << " = ";
+      if (layout[(size_t)i] == 's') s << "s" << i; else s << "l" << i << ".v[" << e << "]";
+      s << ";\n";
+    }
+    emit_program(s, n_in, n_instr, prog, dt, "      ", suf);
+    for (int o = 0; o < n_out; ++o) s << "      r" << o << ".v[" << e << "] = v" << out_slots[o] << suf << ";\n";
+    for (int j = 0; j < n_sum; ++j) s << "      acc" << j << " += (" << acc_t(j) << ")v" << sum_slots[j] << suf << ";\n";
+    s << "    }\n";
+  }
+  for (int o = 0; o < n_out; ++o) s << "    reinterpret_cast<Vec<" << ctype(res[(size_t)o]->dtype) << ", " << vec << ">*>(o" << o << ")[i] = r" << o << ";\n";
+  s << "  }\n";
+  s << "  const i64 t = nv * " << vec << " + (i64)blockIdx.x * 256 + threadIdx.x;\n";
+  s << "  if (t < n) {\n";
+  for (int i = 0; i < n_in; ++i) {
+    s << "    const " << ctype(in[i]->dtype) << " v" << i << "_t = ";
+    if (layout[(size_t)i] == 's') s << "s" << i; else s << "i" << i << "[t]";
+    s << ";\n";
+  }
+  emit_program(s, n_in, n_instr, prog, dt, "    ", "_t");
+  for (int o = 0; o < n_out; ++o) s << "    o" << o << "[t] = v" << out_slots[o] << "_t;\n";
+  for (int j = 0; j < n_sum; ++j) s << "    acc" << j << " += (" << acc_t(j) << ")v" << sum_slots[j] << "_t;\n";
+  s << "  }\n";
+  for (int j = 0; j < n_sum; ++j) {
+    s << "  acc" << j << " = wave_sum(acc" << j << ");\n";
+    s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = *reinterpret_cast<unsigned long long*>(&acc" << j << ");\n";
+    s << "  __syncthreads();\n";
+    s << "  if (threadIdx.x == 0) {\n    " << acc_t(j) << " t4[4];\n    for (int k = 0; k < 4; ++k) t4[k] = *reinterpret_cast<" << acc_t(j) << "*>(&red[k]);\n";
+    s << "    " << acc_t(j) << " tot = (t4[0] + t4[1]) + (t4[2] + t4[3]);\n";
+    s << "    part[(i64)" << j << " * gridDim.x + blockIdx.x] = *reinterpret_cast<unsigned long long*>(&tot);\n  }\n";
+    s << "  __syncthreads();\n";
+  }
+  s << "}\n";
+  // second launch: block j adds the partial sums of sum j, always in the same order
+  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_map_sums_final(int g, const unsigned long long* __restrict__ part";
+  for (int j = 0; j < n_sum; ++j) s << ", " << ctype(dt[(size_t)sum_slots[j]]) << "* __restrict__ out" << j;
+  s << ") {\n  __shared__ unsigned long long red[4];\n";
+  for (int j = 0; j < n_sum; ++j) {
+    s << "  if (blockIdx.x == " << j << ") {\n    " << acc_t(j) << " acc = 0;\n";
+    s << "    for (int i = threadIdx.x; i < g; i += 256) acc += *reinterpret_cast<const " << acc_t(j) << "*>(&part[(i64)" << j << " * g + i]);\n";
+    s << "    acc = wave_sum(acc);\n    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = *reinterpret_cast<unsigned long long*>(&acc);\n    __syncthreads();\n";
+    s << "    if (threadIdx.x == 0) {\n      " << acc_t(j) << " t4[4];\n      for (int k = 0; k < 4; ++k) t4[k] = *reinterpret_cast<" << acc_t(j) << "*>(&red[k]);\n";
+    s << "      out" << j << "[0] = (" << ctype(dt[(size_t)sum_slots[j]]) << ")((t4[0] + t4[1]) + (t4[2] + t4[3]));\n    }\n  }\n";
+  }
+  s << "}\n";
+  std::string src = s.str();
+
+  const char* label = "fused_map_sums";
+  if (ctx->profiling && ctx->profile_shapes) {
+    std::string sh;
+    for (int d = 0; d < a0->rank; ++d) sh += (d ? "x" : "") + std::to_string(a0->shape[d]);
+    char buf[160];
+    snprintf(buf, sizeof buf, "fused_map_sums[%s,in%d(%s),instr%d,out%d,sums%d,vec%d]", sh.c_str(), n_in, layout.c_str(), n_instr, n_out, n_sum, vec);
+    label = ctx->label_pool.insert(buf).first->c_str();
+  }
+  double bytes = 0;
+  for (int i = 0; i < n_in; ++i) {
+    if (layout[(size_t)i] == 's') continue;
+    bool dup = false;
+    for (int k = 0; k < i; ++k)
+      if (data_ptr(in[k]) == data_ptr(in[i]) && layout[(size_t)k] != 's') dup = true;
+    if (!dup) bytes += (double)n * dtype_size(in[i]->dtype);
+  }
+  for (int o = 0; o < n_out; ++o) bytes += (double)n * dtype_size(res[(size_t)o]->dtype);
+  LaunchGuard lg(ctx, label, bytes, (double)n * n_instr);
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c;
+    rc = compile(ctx, src, &c, "fused_map_sums");
+    if (rc) { buffer_release(part); release_all(); return rc; }
+    it = cache.emplace(src, c).first;
+  }
+  hipFunction_t fin = nullptr;
+  hipError_t e = hipModuleGetFunction(&fin, it->second.mod, "fused_map_sums_final");
+  if (e != hipSuccess) { buffer_release(part); release_all(); return check_hip(ctx, e, "hipModuleGetFunction"); }
+  std::vector<void*> args;
+  int64_t nn = n;
+  args.push_back(&nn);
+  std::vector<const void*> ptrs((size_t)n_in);
+  std::vector<void*> optrs((size_t)n_out), sptrs((size_t)n_sum);
+  for (int i = 0; i < n_in; ++i) { ptrs[(size_t)i] = data_ptr(in[i]); args.push_back(&ptrs[(size_t)i]); }
+  for (int o = 0; o < n_out; ++o) { optrs[(size_t)o] = data_ptr(res[(size_t)o]); args.push_back(&optrs[(size_t)o]); }
+  void* pp = part->ptr;
+  args.push_back(&pp);
+  e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e == hipSuccess) {
+    int g = (int)grid;
+    std::vector<void*> fargs = {&g, &pp};
+    for (int j = 0; j < n_sum; ++j) { sptrs[(size_t)j] = data_ptr(sres[(size_t)j]); fargs.push_back(&sptrs[(size_t)j]); }
+    e = hipModuleLaunchKernel(fin, (unsigned)n_sum, 1, 1, 256, 1, 1, 0, ctx->stream, fargs.data(), nullptr);
+  }
+  buffer_release(part);
+  if (e != hipSuccess) { release_all(); return check_hip(ctx, e, "fused_map_sums launch"); }
+  for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
+  for (int j = 0; j < n_sum; ++j) sums[j] = sres[(size_t)j];
+  return HGPU_OK;
+}

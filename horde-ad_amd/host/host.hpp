@@ -36,6 +36,7 @@ struct Backend {
   std::map<std::pair<int, int64_t>, std::shared_ptr<ArrHolder>> iota_cache;   // (dtype, n)
   std::map<std::pair<int, uint64_t>, std::shared_ptr<ArrHolder>> const_cache; // (dtype, value bits)
   bool fuse = true;   // defer elementwise operations into fused programs (when the provider has fused_map)
+  std::vector<std::weak_ptr<ArrHolder>> pending_sums;   // sums of all elements of an expression, not yet taken (ArrHolder::ssrc)
   std::map<std::string, int64_t> counters;   // how often each rewrite onto a fused entry point was taken (diagnostic)
   void check(int rc) const;
 };
@@ -113,6 +114,11 @@ struct ArrHolder {
   Meta vmeta;
   // ... of vsrc's result zero-extended by vlo / vhi per dim (empty: not extended)
   Shape vlo, vhi;
+  // A pending SUM (h == nullptr, ssrc set): the sum of all elements of the
+  // pending expression ssrc.  It is taken in the pass that writes other
+  // expressions of the same shape out (an objective's value in the pass of its
+  // gradient), or by a pass of its own when somebody needs it first.
+  std::shared_ptr<ArrHolder> ssrc;
   // A stand-in without data that view operations are tried on to learn the
   // strides they produce (vmeta holds its shape and strides).
   bool probe = false;
@@ -139,6 +145,7 @@ class T {
   }
   bool pending_expr() const { return p_ && !p_->h && p_->ekind >= 0; }
   bool is_probe() const { return p_ && p_->probe; }
+  bool pending_sum() const { return p_ && !p_->h && p_->ssrc; }
   bool pending_view() const { return p_ && !p_->h && p_->ekind < 0 && p_->vsrc && !p_->probe; }
   bool meta_only() const { return is_probe() || pending_view(); }   // shape and strides known on the host, no array yet
   bool pending_product() const { return pending_expr() && p_->ekind == HGPU_FUSED_OP2 && p_->eop == HGPU_MUL; }
@@ -156,6 +163,7 @@ class T {
     return q->h;
   }
   int rank() const {
+    if (pending_sum()) return 0;
     if (meta_only()) return (int)p_->vmeta.shape.size();
     if (pending_pieces()) return (int)p_->pshape.size();
     if (pending_merged()) return (int)p_->mv_shape.size();
@@ -163,6 +171,7 @@ class T {
     return contraction_like() ? p_->keep : be()->api->rank(meta_h());
   }
   int dtype() const {
+    if (pending_sum()) return T(p_->ssrc).dtype();
     if (is_probe()) return p_->probe_dtype;
     if (pending_view()) return T(p_->vsrc).dtype();
     if (pending_pieces()) return p_->pdtype;

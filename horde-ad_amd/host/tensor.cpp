@@ -15,6 +15,7 @@ void Backend::check(int rc) const {
 }
 
 Shape T::shape() const {
+  if (pending_sum()) return {};
   if (meta_only()) return p_->vmeta.shape;
   if (pending_pieces()) return p_->pshape;
   if (pending_merged()) return p_->mv_shape;
@@ -433,14 +434,56 @@ static void number_program(const std::vector<ArrHolder*>& roots, std::vector<con
     for (auto& pi : pg.instrs) nodes->push_back(pi.first);
 }
 
+static void measure(const std::vector<ArrHolder*>& roots, int* n_in, int* n_instr);
+
 static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
   std::vector<const hgpu_array*> ins;
   std::vector<hgpu_fused_instr> prog;
   std::vector<int> outs_slot;
-  number_program(roots, &ins, &prog, &outs_slot);
-  int n_in = (int)ins.size(), n_instr = (int)prog.size();
   std::vector<hgpu_array*> outs(roots.size(), nullptr);
-  be->check(be->api->fused_map(be->ctx, n_in, ins.data(), n_instr, prog.data(), (int)roots.size(), outs_slot.data(), outs.data()));
+  // Pending sums over expressions of this shape ride along: one pass for the
+  // values written out and the sums.
+  std::vector<std::shared_ptr<ArrHolder>> sums;
+  const hgpu_api* api = be->api;
+  if (api->struct_size >= offsetof(hgpu_api, fused_map_sums) + sizeof(api->fused_map_sums) && api->fused_map_sums) {
+    for (auto& w : be->pending_sums) {
+      auto q = w.lock();
+      if (!q || q->h || !q->ssrc || sums.size() >= 4) continue;
+      T e(q->ssrc);
+      if (e.pending_expr() && e.shape() == roots[0]->eshape && e.be() == be) sums.push_back(q);
+    }
+  }
+  if (!sums.empty()) {
+    std::vector<ArrHolder*> all(roots);
+    for (auto& q : sums) all.push_back(q->ssrc.get());
+    int n_in_all, n_instr_all;
+    measure(all, &n_in_all, &n_instr_all);
+    if (n_in_all <= 12 && n_instr_all <= 96 && roots.size() <= 6) {
+      std::vector<int> slots;
+      number_program(all, &ins, &prog, &slots);
+      std::vector<int> sum_slots(slots.begin() + (long)roots.size(), slots.end());
+      std::vector<hgpu_array*> souts(sums.size(), nullptr);
+      int rc = api->fused_map_sums(be->ctx, (int)ins.size(), ins.data(), (int)prog.size(), prog.data(), (int)roots.size(), slots.data(), outs.data(),
+                                   (int)sums.size(), sum_slots.data(), souts.data());
+      if (rc == HGPU_OK) {
+        be->counters["fused_map_sums"]++;
+        for (size_t j = 0; j < sums.size(); ++j) { sums[j]->h = souts[j]; sums[j]->ssrc.reset(); }
+        outs_slot.assign(slots.begin(), slots.begin() + (long)roots.size());
+      } else {
+        if (rc != HGPU_ERR_UNSUPPORTED) be->check(rc);
+        ins.clear();
+        prog.clear();
+        sums.clear();
+      }
+    } else {
+      sums.clear();
+    }
+  }
+  if (sums.empty()) {
+    number_program(roots, &ins, &prog, &outs_slot);
+    int n_in = (int)ins.size(), n_instr = (int)prog.size();
+    be->check(be->api->fused_map(be->ctx, n_in, ins.data(), n_instr, prog.data(), (int)roots.size(), outs_slot.data(), outs.data()));
+  }
   for (size_t i = 0; i < roots.size(); ++i) {
     ArrHolder* r = roots[i];
     r->h = outs[i];
@@ -515,6 +558,28 @@ void force_many(const std::vector<T>& ts) {
 void ArrHolder::force() {
   if (h) return;
   if (probe) throw ProbeFail{};
+  if (ssrc) {   // a sum nobody's pass has taken along: a pass of its own
+    T e(ssrc);
+    ssrc.reset();
+    T r;
+    const hgpu_api* api = be->api;
+    if (e.pending_expr() && api->struct_size >= offsetof(hgpu_api, fused_sum) + sizeof(api->fused_sum) && api->fused_sum) {
+      std::vector<const hgpu_array*> ins;
+      std::vector<hgpu_fused_instr> prog;
+      std::vector<int> slots;
+      number_program({e.holder().get()}, &ins, &prog, &slots);
+      if ((int)ins.size() <= 12 && (int)prog.size() <= 96) {
+        hgpu_array* o = nullptr;
+        int rc = api->fused_sum(be->ctx, (int)ins.size(), ins.data(), (int)prog.size(), prog.data(), slots[0], &o);
+        if (rc == HGPU_OK) r = T(be, o);
+        else if (rc != HGPU_ERR_UNSUPPORTED) be->check(rc);
+      }
+    }
+    if (!r.valid()) r = contract_now(e, nullptr, 0);
+    be->check(be->api->retain(r.h()));
+    h = r.h();
+    return;
+  }
   if (vsrc && ekind < 0) {   // a pending view: its source once, for every view of it, then the strides
     T s(vsrc);
     hgpu_array* base = s.h();
@@ -939,6 +1004,17 @@ T contract(const T& a, const T* b, int n_keep) {
   if (!b && n_keep == 0 && a.pending_expr() && a.size() > 0 && (a.dtype() == HGPU_F64 || a.dtype() == HGPU_F32)) {
     Backend* be = a.be();
     const hgpu_api* api = be->api;
+    // ... and when the provider can sum in the pass that writes other expressions
+    // of this shape, the sum waits for such a pass (the gradient's)
+    if (be->fuse && api->struct_size >= offsetof(hgpu_api, fused_map_sums) + sizeof(api->fused_map_sums) && api->fused_map_sums && pending_size(a.holder()) <= 40 &&
+        a.size() >= 4096) {
+      auto p = std::make_shared<ArrHolder>(be, nullptr);
+      p->ssrc = a.holder();
+      auto& ps = be->pending_sums;
+      ps.erase(std::remove_if(ps.begin(), ps.end(), [](const std::weak_ptr<ArrHolder>& w) { auto q = w.lock(); return !q || q->h || !q->ssrc; }), ps.end());
+      ps.push_back(p);
+      return T(p);
+    }
     if (api->struct_size >= offsetof(hgpu_api, fused_sum) + sizeof(api->fused_sum) && api->fused_sum && pending_size(a.holder()) <= 96) {
       std::vector<const hgpu_array*> ins;
       std::vector<hgpu_fused_instr> prog;

@@ -218,6 +218,16 @@ enum hgpu_fused_kind { HGPU_FUSED_OP1 = 0, HGPU_FUSED_OP2 = 1, HGPU_FUSED_CMP = 
 typedef struct hgpu_fused_instr { int32_t kind, op, dtype, a, b, c; } hgpu_fused_instr;
 int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
                    int n_out, const int* out_slots, hgpu_array** outs);
+/* hgpu_fused_map that also sums: outs[i] = slot out_slots[i] as for
+ * hgpu_fused_map, and sums[j] = the sum of all elements of slot sum_slots[j]
+ * (a rank-0 array of the slot's type, accumulated in double / int64 in an order
+ * fixed by the size), all from ONE pass over the inputs.  An objective
+ * `ssum0 (f x y z)` and its gradient (test/simplified/TestAdaptorSimplified.hs:
+ * 610-624,682) share most of their program: evaluated together they read x, y, z
+ * once.  Inputs must be dense or one broadcast element (else
+ * HGPU_ERR_UNSUPPORTED: run hgpu_fused_map and hgpu_fused_sum). */
+int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
+                        int n_out, const int* out_slots, hgpu_array** outs, int n_sum, const int* sum_slots, hgpu_array** sums);
 /* The first extremum of such a program's result along its trailing n_reduce
  * dims (taken together, row-major), evaluated on the fly: the result itself is
  * never written.  values / indices get the leading dims' shape; an index
@@ -462,6 +472,7 @@ typedef struct hgpu_api {
   int (*contract_map)(hgpu_ctx*, const hgpu_array*, const hgpu_array*, int, int, const hgpu_array* const*, int, const hgpu_fused_instr*,
                       int, const int*, hgpu_array**, int, int, const int64_t*, const int64_t*, int, int, hgpu_array**, hgpu_array**);
   int (*contract_operands)(hgpu_ctx*, const hgpu_operand*, const hgpu_operand*, int, int, hgpu_array**);
+  int (*fused_map_sums)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, const int*, hgpu_array**, int, const int*, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

@@ -862,6 +862,14 @@ int horc_contract_operands(hgpu_ctx* c, const hgpu_operand* a, const hgpu_operan
   return rc;
 }
 
+int horc_fused_map_sums(hgpu_ctx* c, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int n_out, const int* out_slots,
+                        hgpu_array** outs, int n_sum, const int* sum_slots, hgpu_array** sums) {
+  int rc = HGPU_OK;
+  if (n_out > 0) rc = horc_fused_map(c, n_in, in, n_instr, prog, n_out, out_slots, outs);
+  for (int j = 0; j < n_sum && !rc; ++j) rc = horc_fused_sum(c, n_in, in, n_instr, prog, sum_slots[j], &sums[j]);
+  return rc;
+}
+
 const hgpu_api* horc_get_api(void) {
   static const hgpu_api api = {
       sizeof(hgpu_api),
@@ -879,6 +887,7 @@ const hgpu_api* horc_get_api(void) {
       nullptr,   // no fused_sum
       nullptr,   // no contract_map
       nullptr,   // no contract_operands
+      nullptr,   // no fused_map_sums
   };
   return &api;
 }
@@ -890,6 +899,7 @@ const hgpu_api* horc_get_api_fused(void) {
   api.fused_sum = horc_fused_sum;
   api.contract_map = horc_contract_map;
   api.contract_operands = horc_contract_operands;
+  api.fused_map_sums = horc_fused_map_sums;
   return &api;
 }
 
