@@ -12,8 +12,10 @@ import os
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-GPU_LIB = os.path.join(HERE, "lib", "libhordead_gpu.so")
-HOST_LIB = os.path.join(HERE, "lib", "libhordead_host.so")
+# HORDEAD_LIB_DIR points at another build of the libraries (the sanitizer build of the host layer)
+LIB_DIR = os.environ.get("HORDEAD_LIB_DIR") or os.path.join(HERE, "lib")
+GPU_LIB = os.path.join(LIB_DIR, "libhordead_gpu.so")
+HOST_LIB = os.path.join(LIB_DIR, "libhordead_host.so")
 
 F64, F32, I64, I32, I16, I8, BOOL = range(7)
 _NP2DT = {np.dtype(np.float64): F64, np.dtype(np.float32): F32, np.dtype(np.int64): I64,
@@ -51,6 +53,7 @@ SIGNATURES = {
     "scatter_affine": (I, [P, P, I, I, LP, LP, LP, PP]),
     "contract_sum": (I, [P, I, PP, PP, I, PP]),
     "assign": (I, [P, P, P]),
+    "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
 }
 # exported by the GPU library only
 GPU_ONLY = {
@@ -59,7 +62,6 @@ GPU_ONLY = {
     "fused_sum": (I, [P, I, PP, I, P, I, PP]),
     "mem_stats": (I, [P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "stream": (P, [P]), "inject_alloc_failure": (I, [P, L]),
-    "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
     "profile_enable": (I, [P, I]), "profile_report": (I, [P, C.c_char_p, C.c_size_t]),
     "contract_noalloc": (I, [P, P, P, I, P]),
     "contract_map": (I, [P, P, P, I, I, PP, I, P, I, IP, PP, I, I, LP, LP, I, I, PP, PP]),
@@ -364,6 +366,11 @@ class Array:
 
     def contract(self, other, n_keep):
         return self.ctx._out(self.ctx.lib.contract, self.h, other.h if other is not None else None, n_keep)
+
+    def assign(self, src):
+        """hgpu_assign: this array's memory takes src's elements."""
+        self.ctx.check(self.ctx.lib.assign(self.ctx.h, self.h, src.h))
+        return self
 
     def contract_noalloc(self, other, n_keep, out):
         """hgpu_contract into the caller's array `out`, without device allocation (gfx950 library only)."""

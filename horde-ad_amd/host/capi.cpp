@@ -231,6 +231,32 @@ int hh_tsdotNIn(hh_ctx* c, hh_val* a, hh_val* b, int n, hh_val** out) { HH_OP(d_
 int hh_as_input(hh_ctx* c, hh_val* v, hh_val** out) { HH_OP(c->tape.input(v->d.primal)); }
 int hh_tprimalPart(hh_ctx* c, hh_val* v, hh_val** out) { HH_OP(d_const(v->d.primal)); }
 int hh_tD(hh_ctx* c, hh_val* primal, hh_val* dual, hh_val** out) { HH_OP(d_tD(primal->d, dual->d)); }
+// ConvertTensor (ConvertTensor.hs:25-236, OpsConcrete.hs:777-904): on a carrier whose
+// arrays hold their shape at run time every conversion is the identity on the
+// data and on the dual part; what is left of it is the reference's check.
+int hh_tconvert(hh_ctx* c, int conv, hh_val* v, int rank, const int64_t* shape, hh_val** out) {
+  if (!c || !v || !out || rank < 0 || (rank > 0 && !shape)) return HGPU_ERR_INVALID;
+  return guarded(c, [&] {
+    const Shape have = v->d.primal.shape();
+    const Shape want = mk(rank, shape);
+    switch (conv) {
+      case HH_CONV_K_FROM_S: case HH_CONV_S_FROM_K:
+        if (!have.empty()) throw HostError(HGPU_ERR_INVALID, "tconvert: a scalar conversion of an array of rank " + std::to_string(have.size()));
+        break;
+      case HH_CONV_S_FROM_R: case HH_CONV_S_FROM_X:
+        if (have != want) throw HostError(HGPU_ERR_INVALID, "tconvert: the array does not have the shape the shaped type names");
+        break;
+      case HH_CONV_R_FROM_S: case HH_CONV_X_FROM_S:
+        break;
+      case HH_CONV_NEST: case HH_CONV_UNNEST:   // rank = dims of the outer array; shape, when given, names them
+        if ((size_t)rank > have.size() || (shape && !std::equal(want.begin(), want.end(), have.begin())))
+          throw HostError(HGPU_ERR_INVALID, "tconvert: the outer dims do not lead the array's shape");
+        break;
+      default: throw HostError(HGPU_ERR_INVALID, "tconvert: unknown conversion");
+    }
+    *out = box(v->d);
+  });
+}
 int hh_tsmatvecmul(hh_ctx* c, hh_val* m, hh_val* v, hh_val** out) {
   HH_OP(d_tsdot1In(c->tape, m->d, d_tsreplicateN(c->tape, v->d, {m->d.primal.shape().at(0)})));
 }

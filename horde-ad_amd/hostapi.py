@@ -36,6 +36,7 @@ SIG = {
     "ix_select": (I, [P, P, P, P, PP]), "ix_convert": (I, [P, P, I, I, PP]),
     "ix_index0": (I, [P, P, I, PP, PP]), "ix_argminmax": (I, [P, P, I, PP, I, PP]), "ix_free": (I, [P]),
     "ix_is_affine": (I, [P]), "counter": (L, [P, C.c_char_p]),
+    "tconvert": (I, [P, I, P, I, LP, PP]),
     "tsgather": (I, [P, P, I, LP, I, PP, PP]), "tsscatter": (I, [P, P, I, I, LP, PP, PP]),
     "capture_begin": (I, [P]), "capture_end": (I, [P, PP]), "graph_launch": (I, [P, P]), "graph_free": (I, [P, P]),
     "force": (I, [P, P]), "overwrite": (I, [P, P, P]), "assign": (I, [P, P, P]),
@@ -379,6 +380,13 @@ class V:
     def as_input(self): return self._o(self.host.dll.hh_as_input, self.h)
     def sprimalPart(self): return self._o(self.host.dll.hh_tprimalPart, self.h)
     def tD(self, dual): return self._o(self.host.dll.hh_tD, self.h, dual.h)
+    def tconvert(self, conv, shape=None):
+        """ConvertTensor: "kfromS", "sfromK", "sfromR", "rfromS", "sfromX", "xfromS", "nest", "unnest";
+        shape = the shape the shaped type names (sfromR / sfromX) or the outer dims (nest / unnest)."""
+        kinds = ["kfromS", "sfromK", "sfromR", "rfromS", "sfromX", "xfromS", "nest", "unnest"]
+        sh = list(shape) if shape is not None else []
+        return self._o(self.host.dll.hh_tconvert, kinds.index(conv), self.h, len(sh), _larr(sh))
+
     def smatvecmul(self, v): return self._o(self.host.dll.hh_tsmatvecmul, self.h, v.h)
     def smatmul2(self, o): return self._o(self.host.dll.hh_tsmatmul2, self.h, o.h)
     def sargMax(self): return self._o(self.host.dll.hh_tsargminmax, self.h, 1)

@@ -128,6 +128,22 @@ int hh_tprimalPart(hh_ctx* ctx, hh_val* v, hh_val** out);
 /* tD: the primal part of `primal` with the dual part (tape node) of `dual`
  * (lossSoftMaxCrossEntropyS, External/CommonShapedOps.hs:89-111). */
 int hh_tD(hh_ctx* ctx, hh_val* primal, hh_val* dual, hh_val** out);
+/* ConvertTensor (src/HordeAd/Core/ConvertTensor.hs:25-236; Concrete instance
+ * OpsConcrete.hs:777-876, interpretTKConversion :878-904).  The carrier's arrays
+ * know their shape at run time and a product is a pair of handles on the host,
+ * so kfromS / sfromK / sfromR / rfromS / sfromX / xfromS and nest / unnest are
+ * the identity on data and dual part (zip / unzip never reach this layer: the
+ * host keeps the two handles).  What remains is the reference's check:
+ * K_FROM_S / S_FROM_K need a rank-0 array; S_FROM_R / S_FROM_X need the array's
+ * shape to equal (rank, shape), the shape the shaped type names; NEST / UNNEST
+ * take in `rank` the number of outer dims (<= the array's rank; `shape`, when
+ * not NULL, must equal the leading dims).  A failed check is HGPU_ERR_INVALID
+ * (the reference calls `error`). */
+enum hh_conversion {
+  HH_CONV_K_FROM_S = 0, HH_CONV_S_FROM_K, HH_CONV_S_FROM_R, HH_CONV_R_FROM_S, HH_CONV_S_FROM_X, HH_CONV_X_FROM_S,
+  HH_CONV_NEST, HH_CONV_UNNEST
+};
+int hh_tconvert(hh_ctx* ctx, int conv, hh_val* v, int rank, const int64_t* shape, hh_val** out);
 int hh_tsmatvecmul(hh_ctx* ctx, hh_val* m, hh_val* v, hh_val** out);     /* Ops.hs:538 */
 int hh_tsmatmul2(hh_ctx* ctx, hh_val* a, hh_val* b, hh_val** out);       /* Ops.hs:543 */
 int hh_tsreplicateN(hh_ctx* ctx, hh_val* t, int n, const int64_t* shm, hh_val** out);   /* Ops.hs:552; also tsreplicate0N */

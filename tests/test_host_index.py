@@ -112,22 +112,71 @@ def test_affine_gather_is_a_view(host_cpu):
     assert not other.sindex0([i, k]).is_affine
 
 
-def test_data_dependent_indices_cpu(host_cpu):
+def data_dependent_indices(host):
     """relu mask and max-pool as the reference's simplified programs express them
     (test/simplified/TestMnistPP.hs:735): gather from [0, 1] by
     ifH (0 <=. negate x) 0 1, and gather at kargMax of a partial index."""
     x = RNG.uniform(-1, 1, (4, 5))
-    t = host_cpu.concrete(x)
-    table = host_cpu.concrete(np.array([0.0, 1.0]))
-    zero = lambda: H.IxV.const(host_cpu, (4, 5), 0.0, capi.F64)  # noqa: E731
+    x[1, 2] = 0.0                                            # 0 <=. negate 0: the mask is 0 at zero
+    t = host.concrete(x)
+    table = host.concrete(np.array([0.0, 1.0]))
+    zero = lambda: H.IxV.const(host, (4, 5), 0.0, capi.F64)  # noqa: E731
     mask = table.sgather((4, 5), lambda i, j: [H.ifH(zero().leq(-t.sindex0([i, j]), capi.F64), 0, 1)])
     assert np.array_equal(mask.numpy(), np.where(0.0 <= -x, 0.0, 1.0))
     u = RNG.uniform(-1, 1, (3, 4, 6))
-    tu = host_cpu.concrete(u)
+    u[2, 1, 3] = u[2, 1, 5] = 2.0                            # a tie: the first of the equal maxima is taken
+    tu = host.concrete(u)
     mx = tu.sgather((3, 4), lambda i, j: [i, j, tu.kargMax([i, j])])
     assert np.array_equal(mx.numpy(), u.max(axis=-1))
     mn = tu.sgather((3, 4), lambda i, j: [i, j, tu.kargMin([i, j])])
     assert np.array_equal(mn.numpy(), u.min(axis=-1))
+    # the VJP of the mask gather is a scatter with the same index function (DeltaEval.hs:556-562)
+    cot = RNG.uniform(-1, 1, (4, 5))
+    back = host.concrete(cot).sscatter(2, [2], lambda i, j: [H.ifH(zero().leq(-t.sindex0([i, j]), capi.F64), 0, 1)])
+    want = np.array([cot[0.0 <= -x].sum(), cot[~(0.0 <= -x)].sum()])
+    assert np.allclose(back.numpy(), want, rtol=1e-12, atol=1e-13)
+
+
+def test_data_dependent_indices_cpu(host_cpu):
+    data_dependent_indices(host_cpu)
+
+
+@pytest.mark.gpu
+def test_data_dependent_indices_gpu(host_gpu):
+    data_dependent_indices(host_gpu)
+
+
+def test_convert_tensor_is_a_checked_identity(host_cpu):
+    """ConvertTensor on this carrier (ConvertTensor.hs:25-236, OpsConcrete.hs:777-904):
+    arrays carry their shape at run time, so kfromS / sfromK / sfromR / rfromS / sfromX /
+    xfromS / nest / unnest hand back the same data and the same dual part; the shape
+    the shaped type names is checked as the reference checks it."""
+    x = RNG.uniform(-1, 1, (3, 4, 5))
+    p = host_cpu.param(x)
+    r = p.tconvert("rfromS")                                 # forget the static shape ...
+    s = r.tconvert("sfromR", (3, 4, 5))                      # ... and name it again
+    assert np.array_equal(s.numpy(), x) and s.shape == (3, 4, 5)
+    with pytest.raises(capi.HgpuError) as e:
+        r.tconvert("sfromR", (3, 5, 4))
+    assert e.value.code == 1
+    assert np.array_equal(p.tconvert("xfromS").tconvert("sfromX", (3, 4, 5)).numpy(), x)
+    # scalars: a rank-0 array either way
+    k = (s * s).ssum0().tconvert("kfromS")
+    assert k.shape == () and abs(float(k.numpy()) - float((x * x).sum())) <= 1e-12
+    with pytest.raises(capi.HgpuError):
+        s.tconvert("kfromS")
+    # nest / unnest: the outer dims lead the shape; the data does not move
+    n = s.tconvert("nest", (3, 4))
+    assert np.array_equal(n.tconvert("unnest", (3,)).numpy(), x)
+    with pytest.raises(capi.HgpuError):
+        s.tconvert("nest", (4,))
+    # the dual part flows through: d/dx sum (sfromR (rfromS x))^2 = 2 x
+    host_cpu.tape_reset()
+    q = host_cpu.param(x).as_input()
+    y = q.tconvert("rfromS").tconvert("sfromR", (3, 4, 5))
+    loss = (y * y).ssum0().tconvert("kfromS").tconvert("sfromK")
+    (g,) = host_cpu.grad(loss, [q])
+    assert np.allclose(g.numpy(), 2 * x, rtol=1e-13, atol=0)
 
 
 def test_adjoint_law_cpu(host_cpu):

@@ -272,3 +272,82 @@ def test_gather_scatter_adjoint(oracle):
     g = oracle.gather(oracle.upload(x), aix, shm).numpy()
     s = oracle.scatter_add(oracle.upload(y), aix, 2, (7, 6)).numpy()
     assert np.isclose((g * y).sum(), (x * s).sum(), rtol=1e-12)
+
+
+def test_materialize_assign_contract_sum_fused_map(oracle):
+    """The entry points that are compositions of the ones above, each against its own numpy statement."""
+    x = rnd((4, 6, 5), np.float64)
+    a = oracle.upload(x)
+    # materialize: the logical contents of a view, densely
+    v = a.transpose([2, 0, 1]).slice(1, 1, 3).reverse(0)
+    assert np.array_equal(v.materialize().numpy(), np.transpose(x, (2, 0, 1))[:, 1:4][::-1])
+    # assign: dst's memory takes src's elements
+    dst = oracle.upload(np.zeros((5, 3, 6)))
+    dst.assign(v)
+    assert np.array_equal(dst.numpy(), np.transpose(x, (2, 0, 1))[:, 1:4][::-1])
+    with pytest.raises(capi.HgpuError):
+        dst.assign(a)                                       # another shape
+    # contract_sum: the sum over the pairs of the pairwise contractions
+    for dt, tol in ((np.float64, 1e-12), (np.float32, 1e-5), (np.int64, 0)):
+        pairs = [(rnd((3, 4, 7), dt), rnd((3, 4, 7), dt)) for _ in range(5)]
+        for keep, spec in ((2, "ijk,ijk->ij"), (1, "ijk,ijk->i"), (0, "ijk,ijk->"), (3, "ijk,ijk->ijk")):
+            want = sum(np.einsum(spec, p.astype(np.float64) if tol else p, q.astype(np.float64) if tol else q) for p, q in pairs)
+            got = oracle.contract_sum([(oracle.upload(p), oracle.upload(q)) for p, q in pairs], keep).numpy()
+            assert got.dtype == np.dtype(dt)
+            if tol == 0:
+                assert np.array_equal(got, want)
+            else:
+                assert np.max(np.abs(got - want)) <= tol * max(1.0, float(np.max(np.abs(want))))
+    # fused_map: the single operations in program order; slots: 0 x, 1 y, 2 = x * y, 3 = sin 2, 4 = (3 <= x), 5 = 4 ? y : 3, 6 = floor 5 as Int
+    O1, O2, CMP = capi.OP1, capi.OP2, capi.CMP
+    xx, yy = rnd((6, 7), np.float64), rnd((6, 7), np.float64)
+    prog = [(1, O2["mul"], 0, 0, 1, 0), (0, O1["sin"], 0, 2, 0, 0), (2, CMP["leq"], 0, 3, 0, 0), (3, 0, 0, 4, 1, 3), (4, 1, capi.I64, 5, 0, 0)]
+    outs = oracle.fused_map([oracle.upload(xx), oracle.upload(yy)], prog, [3, 4, 5, 6, 0])
+    s = np.sin(xx * yy)
+    assert np.array_equal(outs[0].numpy(), s) and np.array_equal(outs[1].numpy(), s <= xx)
+    sel = np.where(s <= xx, yy, s)
+    assert np.array_equal(outs[2].numpy(), sel) and np.array_equal(outs[3].numpy(), np.floor(sel).astype(np.int64))
+    assert np.array_equal(outs[4].numpy(), xx)
+
+
+def test_fused_table_definitions(oracle):
+    """The checker's second table defines the optional fused entry points by
+    composition; each is pinned here against numpy, as the plain ones are above."""
+    lib = capi.Lib(oracle.lib.path, "horc_")
+    dll = lib.dll
+    import ctypes as C
+    O1, O2, CMP = capi.OP1, capi.OP2, capi.CMP
+    P, PP, I, LP, IP = C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int)
+    x = rnd((3, 4, 2, 3), np.float64)
+    x[1, 2] = x[1, 2, 0, 0]                                  # a window of equal values: the first one wins
+    a = oracle.upload(x)
+    # extremum_last / fused_extremum: first extremum over the trailing dims taken together
+    fe = dll.horc_fused_extremum
+    fe.restype, fe.argtypes = I, [P, I, PP, I, P, I, I, I, PP, PP]
+    ins = (C.c_void_p * 1)(a.h)
+    prog = [(0, O1["neg"], 0, 0, 0, 0)]
+    flat = (C.c_int32 * 6)(*[int(v) for q in prog for v in q])
+    for want_max in (1, 0):
+        v, i = C.c_void_p(), C.c_void_p()
+        assert fe(oracle.h, 1, ins, 1, flat, 1, 2, want_max, C.byref(v), C.byref(i)) == 0
+        gv, gi = capi.Array(oracle, v).numpy(), capi.Array(oracle, i).numpy()
+        w = (-x).reshape(3, 4, 6)
+        assert np.array_equal(gi, w.argmax(-1) if want_max else w.argmin(-1))
+        assert np.array_equal(gv, w.max(-1) if want_max else w.min(-1))
+    assert gi[1, 2] == 0
+    # fused_sum and fused_map_sums: sums of a slot's values
+    fs = dll.horc_fused_sum
+    fs.restype, fs.argtypes = I, [P, I, PP, I, P, I, PP]
+    o = C.c_void_p()
+    assert fs(oracle.h, 1, ins, 1, flat, 1, C.byref(o)) == 0
+    assert abs(capi.Array(oracle, o).numpy() - (-x).sum()) <= 1e-12
+    # contract_operands: program, merged dims, zero-extension, view, contraction
+    y = rnd((2, 3, 4), np.float64)
+    z = rnd((2, 3, 4), np.float64)
+    op = oracle.operand([oracle.upload(y), oracle.upload(z)], [(1, O2["mul"], 0, 0, 1, 0)], 2, [2, 12], ([14, 2], [1, 14], 0), pad=([0, 1], [0, 1]))
+    co = dll.horc_contract_operands
+    co.restype, co.argtypes = I, [P, P, P, I, I, PP]
+    o = C.c_void_p()
+    assert co(oracle.h, C.byref(op), None, 1, 0, C.byref(o)) == 0
+    padded = np.pad((y * z).reshape(2, 12), [(0, 0), (1, 1)])
+    assert np.allclose(capi.Array(oracle, o).numpy(), padded.T.sum(axis=1), rtol=1e-13, atol=1e-13)
