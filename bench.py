@@ -210,6 +210,8 @@ def main():
     ap.add_argument("--eager", action="store_true", help="time op-by-op submission instead of the recorded graph")
     ap.add_argument("--train", action="store_true",
                     help="also time a recorded training step (gradient + Adam + write-back) of the headline config")
+    ap.add_argument("--calibrate-mfma", action="store_true",
+                    help="time loops of single matrix-core instructions (the ceiling of the product kernels) and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run plain dense copies of 1 GiB (for scaling hardware traffic counters) and exit")
     args = ap.parse_args()
@@ -220,6 +222,20 @@ def main():
 
     pkg = entry.load_package()
     capi, H, W = pkg.capi, pkg.hostapi, pkg.workloads
+    if args.calibrate_mfma:
+        ctx = capi.Lib().context(0)
+        out = {}
+        names = ["v_mfma_f64_16x16x4_f64", "v_mfma_f64_4x4x4_4b_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"]
+        for variant, name in enumerate(names):
+            best = 0.0
+            for _ in range(3):
+                t = C.c_double()
+                ctx.check(ctx.lib.mfma_probe(ctx.h, variant, 20000, C.byref(t)))
+                best = max(best, t.value)
+            out[name] = {"sustained_tflops": best, "nominal_peak_tflops": MFMA_PEAK_TFLOPS["f64" if "f64_" in name[:12] else "f32"],
+                         "fraction_of_nominal": best / MFMA_PEAK_TFLOPS["f64" if "f64_" in name[:12] else "f32"]}
+        print(json.dumps({"calibration": "loops of one MFMA instruction, 16 wavefronts per CU, 20000 iterations of 4 (8, 2) independent accumulators", "instructions": out}))
+        return
     if args.calibrate_copy:
         import numpy as np
         ctx = capi.Lib().context(0)

@@ -66,6 +66,7 @@ GPU_ONLY = {
     "contract_noalloc": (I, [P, P, P, I, P]),
     "contract_map": (I, [P, P, P, I, I, PP, I, P, I, IP, PP, I, I, LP, LP, I, I, PP, PP]),
     "contract_operands": (I, [P, P, P, I, I, PP]),
+    "mfma_probe": (I, [P, I, I, C.POINTER(C.c_double)]),
 }
 
 

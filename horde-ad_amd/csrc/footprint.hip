@@ -372,7 +372,8 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
 #pragma unroll
   for (int t = 0; t < NACC; ++t) acc[t] = Acc{0, 0, 0, 0};
 
-  // j-th staging vector of this thread; the tail repeats the last vector
+  // j-th staging vector of this thread; the tail repeats the last vector.  The last vector of a footprint may reach up to
+  // VX - 1 elements past it: still inside the operand's block, which the allocator ends with 16 spare bytes.
   auto vidx = [&](int j) -> int { int v = tid + 256 * (j < NLX ? j : j - NLX); int lim = (j < NLX ? XV : YV) - 1; return v < lim ? v : lim; };
   // The first chunk, and the columns operand of mode 1, go to LDS eight vectors
   // at a time: eight loads in flight, then eight stores.  Copied one by one,

@@ -506,3 +506,102 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
 }
 
 }  // namespace hg
+
+// ---- the matrix cores' ceiling, measured -----------------------------------
+// Loops of nothing but one MFMA instruction on independent accumulators: what
+// a product kernel built on that instruction cannot exceed on this part.
+namespace {
+typedef __attribute__((ext_vector_type(4))) double probe_d4;
+typedef __attribute__((ext_vector_type(4))) float probe_f4;
+typedef __attribute__((ext_vector_type(16))) float probe_f16;
+
+__global__ void __launch_bounds__(256) mfma_probe_f64_16x16x4(double* out, int iters) {
+  probe_d4 acc[4];
+  for (int i = 0; i < 4; ++i) acc[i] = probe_d4{0, 0, 0, 0};
+  const double a = threadIdx.x * 0.001, b = threadIdx.x * 0.002;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, acc[i], 0, 0, 0);
+  }
+  double s = 0;
+  for (int i = 0; i < 4; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+__global__ void __launch_bounds__(256) mfma_probe_f64_4x4x4(double* out, int iters) {
+  double acc[8];
+  for (int i = 0; i < 8; ++i) acc[i] = 0;
+  const double a = threadIdx.x * 0.001, b = threadIdx.x * 0.002;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f64_4x4x4f64(a, b, acc[i], 0, 0, 0);
+  }
+  double s = 0;
+  for (int i = 0; i < 8; ++i) s += acc[i];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+__global__ void __launch_bounds__(256) mfma_probe_f32_16x16x4(float* out, int iters) {
+  probe_f4 acc[4];
+  for (int i = 0; i < 4; ++i) acc[i] = probe_f4{0, 0, 0, 0};
+  const float a = threadIdx.x * 0.001f, b = threadIdx.x * 0.002f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[i], 0, 0, 0);
+  }
+  float s = 0;
+  for (int i = 0; i < 4; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+__global__ void __launch_bounds__(256) mfma_probe_f32_32x32x2(float* out, int iters) {
+  probe_f16 acc[2];
+  for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < 16; ++j) acc[i][j] = 0;
+  const float a = threadIdx.x * 0.001f, b = threadIdx.x * 0.002f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
+  }
+  float s = 0;
+  for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < 16; ++j) s += acc[i][j];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+}  // namespace
+
+extern "C" int hgpu_mfma_probe(hgpu_ctx* ctx, int variant, int iters, double* tflops) {
+  if (!ctx || !tflops || iters < 1) return HGPU_ERR_INVALID;
+  if (int rc = no_capture(ctx, "mfma_probe")) return rc;
+  const int blocks = ctx->num_cu * 4;      // 16 wavefronts per CU: every SIMD has four to pick from
+  hgpu_buffer* buf = nullptr;
+  int rc = buffer_alloc(ctx, (size_t)blocks * 256 * 8, &buf);
+  if (rc) return rc;
+  double flops_per_wave_iter = 0;
+  auto launch = [&]() {
+    switch (variant) {
+      case 0: hipLaunchKernelGGL(mfma_probe_f64_16x16x4, dim3(blocks), dim3(256), 0, ctx->stream, (double*)buf->ptr, iters); flops_per_wave_iter = 4 * 2.0 * 16 * 16 * 4; break;
+      case 1: hipLaunchKernelGGL(mfma_probe_f64_4x4x4, dim3(blocks), dim3(256), 0, ctx->stream, (double*)buf->ptr, iters); flops_per_wave_iter = 8 * 2.0 * 4 * 4 * 4 * 4; break;
+      case 2: hipLaunchKernelGGL(mfma_probe_f32_16x16x4, dim3(blocks), dim3(256), 0, ctx->stream, (float*)buf->ptr, iters); flops_per_wave_iter = 4 * 2.0 * 16 * 16 * 4; break;
+      case 3: hipLaunchKernelGGL(mfma_probe_f32_32x32x2, dim3(blocks), dim3(256), 0, ctx->stream, (float*)buf->ptr, iters); flops_per_wave_iter = 2 * 2.0 * 32 * 32 * 2; break;
+      default: break;
+    }
+  };
+  if (variant < 0 || variant > 3) { buffer_release(buf); return fail(ctx, HGPU_ERR_INVALID, "mfma_probe: variant %d", variant); }
+  hipEvent_t e0, e1;
+  LaunchGuard lg(ctx);
+  launch();   // warm-up
+  hipError_t e = hipEventCreate(&e0);
+  if (e == hipSuccess) e = hipEventCreate(&e1);
+  if (e == hipSuccess) {
+    (void)hipEventRecord(e0, ctx->stream);
+    launch();
+    (void)hipEventRecord(e1, ctx->stream);
+    e = hipEventSynchronize(e1);
+  }
+  float ms = 0;
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  buffer_release(buf);
+  if (e != hipSuccess || ms <= 0) return check_hip(ctx, e == hipSuccess ? hipErrorUnknown : e, "mfma_probe");
+  *tflops = flops_per_wave_iter * (double)iters * (double)blocks * 4.0 / ((double)ms * 1e-3) / 1e12;
+  return HGPU_OK;
+}

@@ -54,8 +54,13 @@ static void drop_cache_locked(hgpu_ctx* ctx) {
   ctx->cache.clear();
 }
 
+// Every block has at least kSlack bytes behind the bytes asked for: kernels that
+// move whole 16-byte vectors may read (never write) up to one vector past the
+// last element of an array without leaving the block.
+constexpr size_t kSlack = 16;
+
 int buffer_alloc(hgpu_ctx* ctx, size_t bytes, hgpu_buffer** out) {
-  size_t blk = round_block(bytes);
+  size_t blk = round_block(bytes + kSlack);
   void* p = nullptr;
   {
     std::lock_guard<std::mutex> g(ctx->mu);

@@ -130,12 +130,14 @@ int hh_capture_begin(hh_ctx* c) {
   return guarded(c, [&] {
     if (!has_graphs(c->be.api)) throw HostError(HGPU_ERR_UNSUPPORTED, "this provider records no graphs");
     c->be.check(c->be.api->capture_begin(c->be.ctx));
+    c->be.capturing = true;
   });
 }
 int hh_capture_end(hh_ctx* c, hh_graph** out) {
   return guarded(c, [&] {
     if (!has_graphs(c->be.api)) throw HostError(HGPU_ERR_UNSUPPORTED, "this provider records no graphs");
     hgpu_graph* g = nullptr;
+    c->be.capturing = false;
     c->be.check(c->be.api->capture_end(c->be.ctx, &g));
     *out = new hh_graph{g};
   });

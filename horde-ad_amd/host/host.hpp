@@ -35,6 +35,7 @@ struct Backend {
   hgpu_ctx* ctx;
   std::map<std::pair<int, int64_t>, std::shared_ptr<ArrHolder>> iota_cache;   // (dtype, n)
   std::map<std::pair<int, uint64_t>, std::shared_ptr<ArrHolder>> const_cache; // (dtype, value bits)
+  bool capturing = false;   // between hh_capture_begin and hh_capture_end
   bool fuse = true;   // defer elementwise operations into fused programs (when the provider has fused_map)
   std::vector<std::weak_ptr<ArrHolder>> pending_sums;   // sums of all elements of an expression, not yet taken (ArrHolder::ssrc)
   std::map<std::string, int64_t> counters;   // how often each rewrite onto a fused entry point was taken (diagnostic)

@@ -102,6 +102,11 @@ T iota(Backend* be, int64_t n, int dtype) {
   auto key = std::make_pair(dtype, n);
   auto it = be->iota_cache.find(key);
   if (it != be->iota_cache.end()) return T(it->second);
+  // Made inside a recording, the array would only be filled when the graph is
+  // launched, yet the cache would hand it to eager code before (or after an
+  // aborted recording, never filled): refused, as an upload is -- run the
+  // program once before recording it.
+  if (be->capturing) throw HostError(HGPU_ERR_UNSUPPORTED, "iota of a length first asked for during a recording: run the program once before recording it");
   hgpu_array* o = nullptr;
   be->check(be->api->iota(be->ctx, n, dtype, &o));
   T t(be, o);

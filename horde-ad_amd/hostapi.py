@@ -82,6 +82,7 @@ class Graph:
         if self.h:
             self.host.check(self.host.dll.hh_graph_free(self.host.h, self.h))
             self.h = None
+            self.keeps = None
 
 
 class Host:
@@ -143,7 +144,11 @@ class Host:
             raise
         g = C.c_void_p()
         self.check(self.dll.hh_capture_end(self.h, C.byref(g)))
-        return Graph(self, g), result
+        graph = Graph(self, g)
+        # The recording reads, at every launch, the arrays that existed before it:
+        # they must outlive it.  The recorded function holds them (its closure), so the graph holds the function.
+        graph.keeps = program
+        return graph, result
 
     # -- values
     def concrete(self, x, requires_grad=False):

@@ -122,6 +122,14 @@ int hgpu_inject_alloc_failure(hgpu_ctx* ctx, int64_t limit);
 int hgpu_profile_enable(hgpu_ctx* ctx, int on);
 int hgpu_profile_report(hgpu_ctx* ctx, char* buf, size_t n);
 
+/* Calibration for benchmarks (no reference counterpart): a loop of nothing but
+ * one matrix-core instruction on independent accumulators, 16 wavefronts per
+ * CU, timed with events on the context's stream.  variant 0: v_mfma_f64_16x16x4,
+ * 1: v_mfma_f64_4x4x4 (four blocks), 2: v_mfma_f32_16x16x4, 3: v_mfma_f32_32x32x2.
+ * *tflops is what the instruction sustains on this device: the ceiling of any
+ * product kernel built on it.  Waits for the stream. */
+int hgpu_mfma_probe(hgpu_ctx* ctx, int variant, int iters, double* tflops);
+
 /* ----------------------------------------------------------------- memory */
 
 /* tkconcrete/tsconcrete/tconcrete (OpsConcrete.hs:120-124): identity on the
@@ -389,7 +397,10 @@ int hgpu_onehot(hgpu_ctx* ctx, const hgpu_array* v, int n, const int64_t* ix, co
  * hgpu_graph_launch then runs the whole recorded sequence as one submission
  * (a HIP graph) and refreshes those arrays in place; it may be called any
  * number of times.  Arrays that existed before the capture are read at every
- * launch (refresh them with hgpu_overwrite to feed a new batch).
+ * launch (refresh them with hgpu_overwrite to feed a new batch).  The graph
+ * does NOT retain them: the caller keeps every array the recording read alive
+ * until hgpu_graph_destroy -- a released array's block returns to the
+ * allocator, and later launches would read whatever was allocated there next.
  * Entry points that need the host -- upload, download, read_scalar,
  * compare_all, sync -- fail with HGPU_ERR_UNSUPPORTED during a capture: make
  * constants beforehand.  Memory handed out during a capture stays reserved for

@@ -62,7 +62,8 @@ int hh_download(hh_ctx* ctx, hh_val* v, void* host);
  * the recording as one submission and refreshes, in place, every value made
  * inside the capture (results included).  Values that existed before the
  * capture are the program's inputs: they are read at every launch, and
- * hh_overwrite replaces their contents between launches.  Run the same
+ * hh_overwrite replaces their contents between launches; the caller keeps them
+ * alive (not hh_free'd) until hh_graph_free, the graph holds no reference.  Run the same
  * program once without capture first, so that constants and generated kernels
  * exist (nothing may be uploaded or read back during a capture).
  * hh_force writes a deferred value out (inside a capture: records that). */

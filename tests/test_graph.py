@@ -80,3 +80,29 @@ def test_host_calls_refused_while_recording(host):
     graph.free()
     # the context works as before
     assert float((x * x).ssum0().numpy()) == 55.0
+
+
+def test_first_iota_of_a_length_is_refused_while_recording(host):
+    """An index vector is written once and kept for later calls.  Written only
+    by a recorded launch it would be read unwritten by eager code, so a length
+    never asked for before is refused during a recording; after one eager run
+    the recording just reads the kept vector."""
+    n = 1237                                   # a length no other test asks for
+    x = host.concrete(np.arange(float(n)))
+
+    def program():
+        return (x * host.siota(n, capi.F64)).ssum0()
+
+    with pytest.raises(capi.HgpuError) as e:
+        host.capture(program)
+    assert e.value.code == 4
+    want = program().numpy()                   # eager: the vector now exists
+    graph, z = host.capture(program)
+    try:
+        for _ in range(2):
+            graph.launch()
+            host.sync()
+            assert np.array_equal(z.numpy(), want)
+            assert np.array_equal(host.siota(n, capi.F64).numpy(), np.arange(float(n)))
+    finally:
+        graph.free()
