@@ -54,6 +54,7 @@ SIGNATURES = {
     "contract_sum": (I, [P, I, PP, PP, I, PP]),
     "assign": (I, [P, P, P]),
     "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
+    "contract_sum_map": (I, [P, I, PP, PP, I, I, PP, I, P, I, IP, PP]),
 }
 # exported by the GPU library only
 GPU_ONLY = {
@@ -177,6 +178,18 @@ class Ctx:
         self.check(self.lib.contract_map(self.h, a.h, b.h, n_keep, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs,
                                          slot, len(vshape), _larr(vshape), _larr(vstrides), n_reduce, int(want_max), C.byref(v), C.byref(i)))
         return [Array(self, C.c_void_p(o)) for o in outs[:len(out_slots)]], Array(self, v), Array(self, i)
+
+    def contract_sum_map(self, terms, n_keep, inputs, prog, out_slots):
+        """hgpu_contract_sum_map: terms = [(a, b), ...]; `inputs` holds None where the sum of the
+        contractions stands.  Returns the arrays of out_slots."""
+        as_ = (C.c_void_p * len(terms))(*[a.h for a, _ in terms])
+        bs_ = (C.c_void_p * len(terms))(*[b.h for _, b in terms])
+        ins = (C.c_void_p * len(inputs))(*[None if p is None else p.h for p in inputs])
+        flat = (C.c_int32 * max(6 * len(prog), 1))(*[int(x) for q in prog for x in q])
+        slots = (C.c_int * max(len(out_slots), 1))(*out_slots)
+        outs = (C.c_void_p * max(len(out_slots), 1))()
+        self.check(self.lib.contract_sum_map(self.h, len(terms), as_, bs_, n_keep, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs))
+        return [Array(self, C.c_void_p(o)) for o in outs[:len(out_slots)]]
 
     def operand(self, inputs, prog, slot, mshape, view, pad=None):
         """An expression operand for contract_operands: view = (shape, strides, offset) over the

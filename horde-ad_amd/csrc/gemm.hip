@@ -278,6 +278,8 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
 namespace hg {
 
 int try_footprint(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled);
+int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs, int n_keep, int n_in, const hgpu_array* const* in, int c_slot,
+               int n_instr, const hgpu_fused_instr* prog, const std::vector<int>& dt, int n_out, const int* out_slots, hgpu_array* const* outs, bool* handled);
 
 // The dims of a contraction out[kept] = sum a[kept, red] * b[kept, red] sorted
 // into row (M), column (N), reduced (K) and batch groups by which operand moves
@@ -367,6 +369,14 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   for (int t = 0; t < n_terms; ++t) { p.a_term[t] = data_ptr(as[t]); p.b_term[t] = data_ptr(bs[t]); }
   if (n_terms == 0) {   // windows into small footprints: operands from LDS
     int rc = try_footprint(ctx, p, a->dtype, pa, pb, out, handled);
+    if (rc || *handled) return rc;
+  }
+  if (p.K <= 512 && p.BT == 1) {   // the whole contracted dim in LDS: no K loop, no K table
+    const hgpu_array* const* ta = n_terms > 0 ? as : &a;
+    const hgpu_array* const* tb = n_terms > 0 ? bs : &b;
+    const hgpu_array* none = nullptr;
+    const int slot = 0;
+    int rc = try_smallk(ctx, n_terms > 0 ? n_terms : 1, ta, tb, n_keep, 1, &none, 0, 0, nullptr, std::vector<int>{a->dtype}, 1, &slot, &out, handled);
     if (rc || *handled) return rc;
   }
   if ((p.M <= 32 || p.N <= 32) && p.M <= 1024 && p.N <= 1024) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled, n_terms);

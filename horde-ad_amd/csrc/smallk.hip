@@ -1,0 +1,651 @@
+// hgpu_contract_sum_map: a sum of matrix products with short contracted dims and
+// an elementwise program over the sum, as ONE kernel compiled for the shapes.
+//
+//     outs = program( sum_t  X_t[p, k] * Y_t[q, k]  , other inputs at [q, p] )
+//
+// This is the layer of the reference's recurrent example,
+// `tanh (wX `rmatmul2` x + wS `rmatmul2` s + rtr (rreplicate batch_size b))`
+// (example/MnistRnnRanked2.hs:62-75), and the head of its cotangent,
+// `(wX2^T dz2 + wS^T dz1) * (1 - h * h)`: products whose whole contracted dim
+// (28 or 128 elements) fits into LDS next to a tile of the result, so that a
+// kernel with a K loop, a K table and a separate pass for `+ b`, `tanh` spends
+// most of its time on fixed costs.
+//
+// The kernel (256 threads = 4 wavefronts, tile BP x BQ of the result):
+//   * P is the kept dim that is contiguous in the results, Q the other one; X_t
+//     is whichever factor of term t moves along P, Y_t the one along Q.
+//   * The contracted dims of all terms are cut into chunks of at most 128 (fp32)
+//     or 64 (fp64) elements.  A chunk's two operand tiles are loaded with
+//     16-byte loads into registers, stored to LDS, and the loads of the NEXT
+//     chunk are issued before the MFMAs of this one start, so a chunk's memory
+//     latency hides behind the previous chunk's arithmetic; a single chunk (one
+//     product with K <= 128) has no loop at all.  Extents, strides and chunk
+//     bounds are compile-time constants: addresses are immediates.
+//   * LDS layouts are chosen per operand by which of (row, k) is contiguous in
+//     memory, with row pitches that make the 64 lanes of a fragment read hit 64
+//     different banks.
+//   * fp32: v_mfma_f32_16x16x4 with X as the A operand, so the four accumulator
+//     registers of a lane are four CONSECUTIVE p of one q: inputs of the
+//     program and its results move as 16-byte vectors.  fp64: X as the B
+//     operand, so the 16 lanes of an accumulator row are 16 consecutive p.
+//   * The program runs on the accumulators in registers; only its results are
+//     written.
+//
+// Shapes the kernel does not cover (long K, batched or higher-rank products,
+// too many terms) are computed by the other entry points one after another.
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <map>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+#include "fused_gen.hpp"
+
+using namespace hg;
+using namespace hg::fusedgen;
+
+namespace hg {
+int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled,
+             int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs);
+}
+
+namespace {
+
+constexpr int kMaxTermsSmallK = 4;
+constexpr int64_t kMaxKTotal = 512;
+
+struct Compiled {
+  hipModule_t mod;
+  hipFunction_t fn;
+};
+
+std::map<std::string, Compiled>& cache_of(hgpu_ctx* ctx) {
+  auto it = ctx->jit_cache.find("__smallk__");
+  if (it == ctx->jit_cache.end()) it = ctx->jit_cache.emplace("__smallk__", new std::map<std::string, Compiled>()).first;
+  return *static_cast<std::map<std::string, Compiled>*>(it->second);
+}
+
+struct Term {
+  const void *x, *y;
+  int64_t K, sxp, sxk, syq, syk;
+};
+
+struct Operand {       // one operand tile of one chunk
+  int rows;            // BP or BQ
+  int layout;          // 0: LDS [k][row], 1: LDS [row][k]
+  int V;               // elements per load
+  int pitch;           // LDS elements between k rows (layout 0) or rows (layout 1)
+  int64_t sr, sk;      // element strides in memory
+  int64_t extent;      // rows of the whole operand (P or Q)
+};
+
+struct Chunk {
+  int term, k0, kc, kcp;   // valid k, rounded up to 4
+  Operand x, y;
+};
+
+struct Spec {
+  bool f64;
+  int64_t P, Q;
+  int BP, BQ, WP, WQ;
+  std::vector<Term> terms;
+  std::vector<Chunk> chunks;
+  int n_in, c_slot, n_instr;
+  const hgpu_fused_instr* prog;
+  std::vector<int> dt;
+  std::vector<int64_t> in_sp, in_sq;
+  std::vector<int> out_slots;
+  int x_elems, y_elems;    // LDS elements of the largest X / Y tile
+};
+
+// LDS pitch of a tile: the fragment reads of 16 rows x 4 k must not collide.
+int pitch_for(int layout, int rows, int kcp, bool f64) {
+  if (layout == 0) {           // [k][row]: lanes of one k are adjacent, the four k of a fragment sit `pitch` apart
+    int p = rows;
+    while (p % 32 != 16) p += 4;
+    return p;
+  }
+  int p = kcp;                 // [row][k]: the 16 rows of a fragment sit `pitch` apart
+  if (f64) { while (p % 4 != 2) p += 2; }
+  else { while (p % 8 != 4) p += 4; }
+  return p;
+}
+
+Operand make_operand(bool f64, int rows, int64_t extent, int64_t sr, int64_t sk, int kc, int kcp) {
+  Operand o;
+  o.rows = rows;
+  o.extent = extent;
+  o.sr = sr;
+  o.sk = sk;
+  const int vmax = f64 ? 2 : 4;
+  if (sk == 1 && kc % vmax == 0 && kc >= vmax) {          // k contiguous
+    o.layout = 1;
+    o.V = vmax;
+  } else if (sr == 1 && extent % vmax == 0 && extent >= vmax) {   // rows contiguous
+    o.layout = 0;
+    o.V = vmax;
+  } else {
+    o.layout = 0;
+    o.V = 1;
+  }
+  o.pitch = pitch_for(o.layout, rows, kcp, f64);
+  return o;
+}
+
+int tile_elems(const Operand& o, int kcp) { return o.layout == 0 ? kcp * o.pitch : o.rows * o.pitch; }
+
+void emit_stage_fn(std::ostringstream& s, const char* name, const Operand& o, const Chunk& c, const char* ptr, const char* r0) {
+  // registers of the next chunk's tile: load_<name>() issues the loads, store_<name>() puts them into LDS
+  const int slots = o.rows * c.kcp / o.V;
+  const int ns = (slots + 255) / 256;
+  const bool ragged = slots % 256 != 0;
+  const char* vec = o.V == 1 ? "T" : (o.V == 2 ? "V2" : "V4");
+  const char* veca = o.V == 1 ? "T" : (o.V == 2 ? "A2" : "A4");
+  auto decode = [&](const char* ind) {
+    s << ind << "int s = tid + 256 * i;\n";
+    if (ragged) s << ind << "const bool live = s < " << slots << ";\n" << ind << "s = live ? s : " << slots - 1 << ";\n";
+    if (o.layout == 0) s << ind << "const int k = s / " << o.rows / o.V << ", r = (s % " << o.rows / o.V << ") * " << o.V << ";\n";
+    else s << ind << "const int r = s / " << c.kcp / o.V << ", k = (s % " << c.kcp / o.V << ") * " << o.V << ";\n";
+  };
+  s << "struct Regs_" << name << " { " << vec << " v[" << ns << "]; };\n";
+  s << "__device__ __forceinline__ void load_" << name << "(Regs_" << name << "& rg, const T* __restrict__ base, i64 r0, int tid) {\n";
+  s << "#pragma unroll\n  for (int i = 0; i < " << ns << "; ++i) {\n";
+  decode("    ");
+  // rows past the end read the last valid vector (never stored to a result); k past the end reads a valid k (zeroed in LDS)
+  s << "    i64 rr = r0 + r;\n    rr = rr > " << o.extent - (o.layout == 0 ? o.V : 1) << "LL ? " << o.extent - (o.layout == 0 ? o.V : 1) << "LL : rr;\n";
+  s << "    int kk = k > " << c.kc - (o.layout == 1 ? o.V : 1) << " ? " << c.kc - (o.layout == 1 ? o.V : 1) << " : k;\n";
+  s << "    rg.v[i] = *reinterpret_cast<const " << vec << "*>(base + rr * " << o.sr << "LL + (i64)(" << c.k0 << " + kk) * " << o.sk << "LL);\n";
+  s << "  }\n}\n";
+  s << "__device__ __forceinline__ void store_" << name << "(const Regs_" << name << "& rg, T* lds, int tid) {\n";
+  s << "#pragma unroll\n  for (int i = 0; i < " << ns << "; ++i) {\n";
+  decode("    ");
+  if (ragged) s << "    if (!live) continue;\n";
+  s << "    " << vec << " v = rg.v[i];\n";
+  if (c.kcp != c.kc) {
+    if (o.V == 1) s << "    if (k >= " << c.kc << ") v = T(0);\n";
+    else {
+      s << "    if (k >= " << c.kc << ") {";
+      for (int e = 0; e < o.V; ++e) s << " v[" << e << "] = T(0);";
+      s << " }\n";
+    }
+  }
+  if (o.layout == 0) s << "    *reinterpret_cast<" << veca << "*>(lds + k * " << o.pitch << " + r) = v;\n";
+  else s << "    *reinterpret_cast<" << veca << "*>(lds + r * " << o.pitch << " + k) = v;\n";
+  s << "  }\n}\n";
+  (void)ptr;
+  (void)r0;
+}
+
+std::string generate(const Spec& sp, const std::string& kname) {
+  std::ostringstream s;
+  const int TP = sp.BP / (16 * sp.WP), TQ = sp.BQ / (16 * sp.WQ);
+  const int64_t nbp = (sp.P + sp.BP - 1) / sp.BP, nbq = (sp.Q + sp.BQ - 1) / sp.BQ;
+  const int64_t nblk = nbp * nbq, per_xcd = (nblk + 7) / 8;
+  const bool vec_epi = !sp.f64 && sp.P % 4 == 0;
+  s << kPrelude;
+  s << "typedef " << (sp.f64 ? "double" : "float") << " T;\n";
+  s << "typedef T V2 __attribute__((ext_vector_type(2), aligned(" << (sp.f64 ? 8 : 4) << ")));\n";
+  s << "typedef T V4 __attribute__((ext_vector_type(4), aligned(" << (sp.f64 ? 8 : 4) << ")));\n";
+  s << "typedef T A2 __attribute__((ext_vector_type(2)));\ntypedef T A4 __attribute__((ext_vector_type(4)));\n";
+  s << "typedef T Acc __attribute__((ext_vector_type(4)));\n";
+  // vectors of four for every type the program reads or writes
+  s << "template <typename E> struct Vec4 { typedef E type __attribute__((ext_vector_type(4), aligned(sizeof(E)))); };\n";
+  s << "struct Args {\n";
+  for (size_t t = 0; t < sp.terms.size(); ++t) s << "  const T* x" << t << ";\n  const T* y" << t << ";\n";
+  for (int i = 0; i < sp.n_in; ++i)
+    if (i != sp.c_slot) s << "  const " << ctype(sp.dt[(size_t)i]) << "* i" << i << ";\n";
+  for (size_t o = 0; o < sp.out_slots.size(); ++o) s << "  " << ctype(sp.dt[(size_t)sp.out_slots[o]]) << "* o" << o << ";\n";
+  s << "};\n";
+  for (size_t c = 0; c < sp.chunks.size(); ++c) {
+    emit_stage_fn(s, ("x" + std::to_string(c)).c_str(), sp.chunks[c].x, sp.chunks[c], "", "");
+    emit_stage_fn(s, ("y" + std::to_string(c)).c_str(), sp.chunks[c].y, sp.chunks[c], "", "");
+  }
+  // the MFMAs of one chunk
+  s << "template <int KCP, int LX, int PX, int LY, int PY>\n";
+  s << "__device__ __forceinline__ void compute(const T* __restrict__ xs, const T* __restrict__ ys, Acc (&acc)[" << TP << "][" << TQ << "], int r, int g, int wp, int wq) {\n";
+  s << "#pragma unroll\n  for (int j = 0; j < KCP / 4; ++j) {\n";
+  s << "    T xf[" << TP << "], yf[" << TQ << "];\n";
+  s << "#pragma unroll\n    for (int a = 0; a < " << TP << "; ++a) xf[a] = LX == 0 ? xs[(4 * j + g) * PX + (wp * " << TP << " + a) * 16 + r] : xs[((wp * " << TP
+    << " + a) * 16 + r) * PX + 4 * j + g];\n";
+  s << "#pragma unroll\n    for (int b = 0; b < " << TQ << "; ++b) yf[b] = LY == 0 ? ys[(4 * j + g) * PY + (wq * " << TQ << " + b) * 16 + r] : ys[((wq * " << TQ
+    << " + b) * 16 + r) * PY + 4 * j + g];\n";
+  s << "#pragma unroll\n    for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n      for (int b = 0; b < " << TQ << "; ++b)\n";
+  if (sp.f64) s << "        acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(yf[b], xf[a], acc[a][b], 0, 0, 0);\n";
+  else s << "        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xf[a], yf[b], acc[a][b], 0, 0, 0);\n";
+  s << "  }\n}\n";
+  // The program over one accumulator block.  What it reads besides the
+  // accumulators is loaded by epi_load (rows past the end read a valid place
+  // and are never written), which the kernel calls before the first chunk's
+  // MFMAs when the registers allow: the loads then wait behind the arithmetic.
+  s << "struct EpiIn {\n";
+  for (int i = 0; i < sp.n_in; ++i) {
+    if (i == sp.c_slot) continue;
+    const char* ct = ctype(sp.dt[(size_t)i]);
+    if (vec_epi && sp.in_sp[(size_t)i] == 1) s << "  Vec4<" << ct << ">::type w" << i << ";\n";
+    else if (sp.in_sp[(size_t)i] == 0 && !sp.f64) s << "  " << ct << " w" << i << ";\n";      // one q per lane
+    else if (sp.in_sp[(size_t)i] == 0) s << "  " << ct << " w" << i << "x[4];\n";                  // fp64: a lane's four values are four q
+    else s << "  " << ct << " w" << i << "[4];\n";
+  }
+  s << "  int unused;\n};\n";
+  s << "__device__ __forceinline__ EpiIn epi_load(const Args& ar, i64 pb, i64 qb, int r, int g) {\n  EpiIn z;\n  z.unused = 0;\n";
+  if (vec_epi) {
+    s << "  i64 p = pb + 4 * g, q = qb + r;\n  p = p > " << sp.P - 4 << "LL ? " << sp.P - 4 << "LL : p;\n  q = q > " << sp.Q - 1 << "LL ? " << sp.Q - 1 << "LL : q;\n";
+    for (int i = 0; i < sp.n_in; ++i) {
+      if (i == sp.c_slot) continue;
+      const char* ct = ctype(sp.dt[(size_t)i]);
+      if (sp.in_sp[(size_t)i] == 1) s << "  z.w" << i << " = *reinterpret_cast<const Vec4<" << ct << ">::type*>(ar.i" << i << " + q * " << sp.in_sq[(size_t)i] << "LL + p);\n";
+      else if (sp.in_sp[(size_t)i] == 0) s << "  z.w" << i << " = ar.i" << i << "[q * " << sp.in_sq[(size_t)i] << "LL];\n";
+      else
+        for (int e = 0; e < 4; ++e) s << "  z.w" << i << "[" << e << "] = ar.i" << i << "[q * " << sp.in_sq[(size_t)i] << "LL + (p + " << e << ") * " << sp.in_sp[(size_t)i] << "LL];\n";
+    }
+  } else {
+    bool any_q = false;
+    for (int i = 0; i < sp.n_in; ++i) any_q = any_q || (i != sp.c_slot);
+    if (any_q) {
+      s << "#pragma unroll\n  for (int e = 0; e < 4; ++e) {\n";
+      if (sp.f64) s << "    i64 p = pb + r, q = qb + 4 * e + g;\n";
+      else s << "    i64 p = pb + 4 * g + e, q = qb + r;\n";
+      s << "    p = p > " << sp.P - 1 << "LL ? " << sp.P - 1 << "LL : p;\n    q = q > " << sp.Q - 1 << "LL ? " << sp.Q - 1 << "LL : q;\n";
+      for (int i = 0; i < sp.n_in; ++i) {
+        if (i == sp.c_slot) continue;
+        if (sp.in_sp[(size_t)i] == 0 && !sp.f64) s << "    if (e == 0) z.w" << i << " = ar.i" << i << "[q * " << sp.in_sq[(size_t)i] << "LL];\n";
+        else if (sp.in_sp[(size_t)i] == 0) s << "    z.w" << i << "x[e] = ar.i" << i << "[q * " << sp.in_sq[(size_t)i] << "LL];\n";
+        else s << "    z.w" << i << "[e] = ar.i" << i << "[q * " << sp.in_sq[(size_t)i] << "LL + p * " << sp.in_sp[(size_t)i] << "LL];\n";
+      }
+      s << "  }\n";
+    }
+  }
+  s << "  return z;\n}\n";
+  s << "__device__ __forceinline__ void epilogue(const Args& ar, i64 pb, i64 qb, int r, int g, const Acc& c, const EpiIn& z) {\n";
+  if (vec_epi) {
+    // four consecutive p of one q
+    s << "  const i64 p = pb + 4 * g, q = qb + r;\n  if (p >= " << sp.P << "LL || q >= " << sp.Q << "LL) return;\n";
+    for (int i = 0; i < sp.n_in; ++i) {
+      const char* ct = ctype(sp.dt[(size_t)i]);
+      for (int e = 0; e < 4; ++e) {
+        s << "  const " << ct << " v" << i << "_" << e << " = ";
+        if (i == sp.c_slot) s << "c[" << e << "];\n";
+        else if (sp.in_sp[(size_t)i] == 0) s << "z.w" << i << ";\n";
+        else s << "z.w" << i << "[" << e << "];\n";
+      }
+    }
+    for (int e = 0; e < 4; ++e) emit_program(s, sp.n_in, sp.n_instr, sp.prog, sp.dt, "  ", "_" + std::to_string(e));
+    for (size_t o = 0; o < sp.out_slots.size(); ++o) {
+      const char* ct = ctype(sp.dt[(size_t)sp.out_slots[o]]);
+      s << "  {\n    Vec4<" << ct << ">::type w;\n";
+      for (int e = 0; e < 4; ++e) s << "    w[" << e << "] = v" << sp.out_slots[o] << "_" << e << ";\n";
+      s << "    *reinterpret_cast<Vec4<" << ct << ">::type*>(ar.o" << o << " + q * " << sp.P << "LL + p) = w;\n  }\n";
+    }
+  } else {
+    s << "#pragma unroll\n  for (int e = 0; e < 4; ++e) {\n";
+    if (sp.f64) s << "    const i64 p = pb + r, q = qb + 4 * e + g;\n";
+    else s << "    const i64 p = pb + 4 * g + e, q = qb + r;\n";
+    s << "    if (p >= " << sp.P << "LL || q >= " << sp.Q << "LL) continue;\n";
+    for (int i = 0; i < sp.n_in; ++i) {
+      const char* ct = ctype(sp.dt[(size_t)i]);
+      if (i == sp.c_slot) s << "    const T v" << i << " = c[e];\n";
+      else if (sp.in_sp[(size_t)i] == 0 && !sp.f64) s << "    const " << ct << " v" << i << " = z.w" << i << ";\n";
+      else if (sp.in_sp[(size_t)i] == 0) s << "    const " << ct << " v" << i << " = z.w" << i << "x[e];\n";
+      else s << "    const " << ct << " v" << i << " = z.w" << i << "[e];\n";
+    }
+    emit_program(s, sp.n_in, sp.n_instr, sp.prog, sp.dt, "    ", "");
+    for (size_t o = 0; o < sp.out_slots.size(); ++o) s << "    ar.o" << o << "[q * " << sp.P << "LL + p] = v" << sp.out_slots[o] << ";\n";
+    s << "  }\n";
+  }
+  s << "}\n";
+  s << "extern \"C\" __global__ void __launch_bounds__(256) " << kname << "(Args ar) {\n";
+  s << "  __shared__ __attribute__((aligned(16))) T lds[" << sp.x_elems + sp.y_elems << "];\n";
+  s << "  T* const xs = lds;\n  T* const ys = lds + " << sp.x_elems << ";\n";
+  // consecutive block ids go round the eight XCDs: blocks that share operand tiles get ids of one XCD
+  s << "  const i64 blk = (i64)(blockIdx.x % 8) * " << per_xcd << "LL + blockIdx.x / 8;\n";
+  s << "  if (blk >= " << nblk << "LL) return;\n";
+  s << "  const i64 q0 = (blk % " << nbq << "LL) * " << sp.BQ << ", p0 = (blk / " << nbq << "LL) * " << sp.BP << ";\n";
+  s << "  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r = lane & 15, g = lane >> 4;\n";
+  s << "  const int wp = w % " << sp.WP << ", wq = w / " << sp.WP << ";\n";
+  s << "  Acc acc[" << TP << "][" << TQ << "];\n";
+  s << "#pragma unroll\n  for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n    for (int b = 0; b < " << TQ << "; ++b) acc[a][b] = Acc{0, 0, 0, 0};\n";
+  const size_t nc = sp.chunks.size();
+  for (size_t c = 0; c < nc; ++c) s << "  Regs_x" << c << " rx" << c << ";\n  Regs_y" << c << " ry" << c << ";\n";
+  auto load = [&](size_t c) {
+    int t = sp.chunks[c].term;
+    s << "  load_x" << c << "(rx" << c << ", ar.x" << t << ", p0, tid);\n  load_y" << c << "(ry" << c << ", ar.y" << t << ", q0, tid);\n";
+  };
+  load(0);
+  int n_read = 0;
+  for (int i = 0; i < sp.n_in; ++i) n_read += i != sp.c_slot;
+  const bool prefetch = n_read > 0 && n_read * TP * TQ <= 16;
+  if (n_read > 0) s << "  EpiIn ei[" << TP << "][" << TQ << "];\n";
+  auto epi_loads = [&]() {
+    s << "#pragma unroll\n  for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n    for (int b = 0; b < " << TQ << "; ++b)\n";
+    s << "      ei[a][b] = epi_load(ar, p0 + (wp * " << TP << " + a) * 16, q0 + (wq * " << TQ << " + b) * 16, r, g);\n";
+  };
+  if (prefetch) epi_loads();
+  for (size_t c = 0; c < nc; ++c) {
+    const Chunk& ch = sp.chunks[c];
+    s << "  store_x" << c << "(rx" << c << ", xs, tid);\n  store_y" << c << "(ry" << c << ", ys, tid);\n  __syncthreads();\n";
+    if (c + 1 < nc) load(c + 1);
+    s << "  compute<" << ch.kcp << ", " << ch.x.layout << ", " << ch.x.pitch << ", " << ch.y.layout << ", " << ch.y.pitch << ">(xs, ys, acc, r, g, wp, wq);\n";
+    if (c + 1 < nc) s << "  __syncthreads();\n";
+  }
+  if (n_read > 0 && !prefetch) epi_loads();
+  s << "#pragma unroll\n  for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n    for (int b = 0; b < " << TQ << "; ++b)\n";
+  if (n_read > 0) s << "      epilogue(ar, p0 + (wp * " << TP << " + a) * 16, q0 + (wq * " << TQ << " + b) * 16, r, g, acc[a][b], ei[a][b]);\n";
+  else s << "      epilogue(ar, p0 + (wp * " << TP << " + a) * 16, q0 + (wq * " << TQ << " + b) * 16, r, g, acc[a][b], EpiIn{0});\n";
+  s << "}\n";
+  return s.str();
+}
+
+// Tile shape by a small model of the busiest CU: its blocks are resident
+// together (as far as LDS allows), so after the first block's loads have
+// arrived the loads of one block hide behind the MFMAs of another; a CU with a
+// single block pays load latency, loads and arithmetic one after the other.
+// Measured on the recurrent layer (128 x 5000, K 128, fp32): 16 x 64 tiles
+// 4.9 us per launch, 64 x 64 5.5, 64 x 128 7.8 -- the model's order.
+void choose_tile(hgpu_ctx* ctx, Spec& sp, int64_t ktot) {
+  static const int cand[][4] = {{16, 64, 1, 4}, {64, 16, 4, 1}, {32, 32, 2, 2}, {32, 64, 2, 2}, {64, 32, 2, 2}, {16, 128, 1, 4},
+                                {64, 64, 2, 2}, {32, 128, 2, 2}, {128, 32, 2, 2}, {64, 128, 2, 2}, {128, 64, 2, 2}};
+  const double es = sp.f64 ? 8 : 4;
+  const double cu_flops = (sp.f64 ? 78.6e12 : 157.3e12) / ctx->num_cu;
+  const double cu_load = 150e9, latency = 1.0e-6;
+  const int kc = (int)std::min<int64_t>(ktot, sp.f64 ? 64 : 128);
+  double best = 1e300;
+  for (auto& c : cand) {
+    double blocks = (double)((sp.P + c[0] - 1) / c[0]) * (double)((sp.Q + c[1] - 1) / c[1]);
+    double n = std::ceil(blocks / ctx->num_cu);
+    double comp = 2.0 * c[0] * c[1] * (double)ktot / cu_flops, load = (c[0] + c[1]) * (double)ktot * es / cu_load;
+    double lds = (c[0] + c[1] + 20) * (double)kc * es;
+    double resident = std::max(1.0, std::min(n, std::floor(160.0 * 1024 / lds)));
+    double t = std::ceil(n / resident) * (latency + load + comp + (resident - 1) * std::max(load, comp));
+    if (t < best) { best = t; sp.BP = c[0]; sp.BQ = c[1]; sp.WP = c[2]; sp.WQ = c[3]; }
+  }
+  if (const char* e = getenv("HORDEAD_SMALLK_TILE")) {   // for measurements: BPxBQxWPxWQ
+    int bp, bq, wp, wq;
+    if (sscanf(e, "%dx%dx%dx%d", &bp, &bq, &wp, &wq) == 4 && wp * wq == 4 && bp % (16 * wp) == 0 && bq % (16 * wq) == 0 && bp >= 16 && bq >= 16 &&
+        bp / (16 * wp) * (bq / (16 * wq)) <= 16) {
+      sp.BP = bp; sp.BQ = bq; sp.WP = wp; sp.WQ = wq;
+    }
+  }
+}
+
+// Cuts the contracted dims of the terms into chunks and lays their tiles out in LDS.
+bool plan_chunks(Spec& sp) {
+  const int kcmax = sp.f64 ? 64 : 128;
+  sp.x_elems = sp.y_elems = 0;
+  sp.chunks.clear();
+  for (int t = 0; t < (int)sp.terms.size(); ++t) {
+    const Term& tm = sp.terms[(size_t)t];
+    int n = (int)((tm.K + kcmax - 1) / kcmax);
+    int per = (int)((tm.K + n - 1) / n);
+    per = (per + 3) / 4 * 4;
+    for (int k0 = 0; k0 < tm.K; k0 += per) {
+      Chunk c;
+      c.term = t;
+      c.k0 = k0;
+      c.kc = (int)std::min<int64_t>(per, tm.K - k0);
+      c.kcp = (c.kc + 3) / 4 * 4;
+      c.x = make_operand(sp.f64, sp.BP, sp.P, tm.sxp, tm.sxk, c.kc, c.kcp);
+      c.y = make_operand(sp.f64, sp.BQ, sp.Q, tm.syq, tm.syk, c.kc, c.kcp);
+      sp.x_elems = std::max(sp.x_elems, tile_elems(c.x, c.kcp));
+      sp.y_elems = std::max(sp.y_elems, tile_elems(c.y, c.kcp));
+      sp.chunks.push_back(c);
+    }
+  }
+  sp.x_elems = (sp.x_elems + 3) / 4 * 4;
+  if (sp.chunks.size() > 8) return false;
+  return (size_t)(sp.x_elems + sp.y_elems) * (sp.f64 ? 8 : 4) <= 150 * 1024;
+}
+
+// The non-unit kept dims of the terms must be two: P (contiguous in a dense
+// result: the later one) and Q.
+struct KeptDims { int dp, dq; int64_t P, Q; };
+
+bool kept_dims(int n_keep, const int64_t* shape, KeptDims* kd) {
+  int found[2], n = 0;
+  for (int d = 0; d < n_keep; ++d) {
+    if (shape[d] == 1) continue;
+    if (n == 2) return false;
+    found[n++] = d;
+  }
+  if (n != 2) return false;
+  kd->dq = found[0];
+  kd->dp = found[1];
+  kd->Q = shape[found[0]];
+  kd->P = shape[found[1]];
+  return true;
+}
+
+// One term: which factor moves along P, and the single contracted dim.
+bool term_of(const hgpu_array* a, const hgpu_array* b, int n_keep, const KeptDims& kd, Term* t) {
+  const hgpu_array *x = nullptr, *y = nullptr;
+  if (a->strides[kd.dp] != 0 && a->strides[kd.dq] == 0 && b->strides[kd.dp] == 0 && b->strides[kd.dq] != 0) { x = a; y = b; }
+  else if (b->strides[kd.dp] != 0 && b->strides[kd.dq] == 0 && a->strides[kd.dp] == 0 && a->strides[kd.dq] != 0) { x = b; y = a; }
+  else return false;
+  // contracted dims: merge what merges in both factors; one dim must remain
+  int64_t K = 1, sxk = 0, syk = 0;
+  bool have = false;
+  for (int d = a->rank - 1; d >= n_keep; --d) {
+    int64_t e = a->shape[d];
+    if (e == 1) continue;
+    if (x->strides[d] == 0 || y->strides[d] == 0) return false;
+    if (!have) { K = e; sxk = x->strides[d]; syk = y->strides[d]; have = true; continue; }
+    if (x->strides[d] == sxk * K && y->strides[d] == syk * K) { K *= e; continue; }
+    return false;
+  }
+  if (!have) return false;
+  t->x = data_ptr(x);
+  t->y = data_ptr(y);
+  t->K = K;
+  t->sxp = x->strides[kd.dp];
+  t->sxk = sxk;
+  t->syq = y->strides[kd.dq];
+  t->syk = syk;
+  return true;
+}
+
+bool fits_int(int64_t v) { return v > -(1LL << 40) && v < (1LL << 40); }
+
+}  // namespace
+
+namespace hg {
+
+// outs[i] (dense, of the kept shape, allocated by the caller) = slot
+// out_slots[i] of the program over sum_t contract(as[t], bs[t]).  *handled says
+// whether the kernel took the case.
+int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs, int n_keep, int n_in, const hgpu_array* const* in, int c_slot,
+               int n_instr, const hgpu_fused_instr* prog, const std::vector<int>& dt, int n_out, const int* out_slots, hgpu_array* const* outs, bool* handled) {
+  *handled = false;
+  const hgpu_array* a0 = as[0];
+  if (a0->dtype != HGPU_F64 && a0->dtype != HGPU_F32) return HGPU_OK;
+  if (n_terms < 1 || n_terms > kMaxTermsSmallK || n_out < 1) return HGPU_OK;
+  if (getenv("HORDEAD_NO_SMALLK")) return HGPU_OK;
+  KeptDims kd;
+  if (!kept_dims(n_keep, a0->shape, &kd)) return HGPU_OK;
+  Spec sp;
+  sp.f64 = a0->dtype == HGPU_F64;
+  sp.P = kd.P;
+  sp.Q = kd.Q;
+  int64_t ktot = 0;
+  for (int t = 0; t < n_terms; ++t) {
+    Term tm;
+    if (!as[t]->buf || !bs[t]->buf) return HGPU_OK;
+    if (!term_of(as[t], bs[t], n_keep, kd, &tm)) return HGPU_OK;
+    if (!fits_int(tm.sxp * sp.P) || !fits_int(tm.syq * sp.Q) || !fits_int(tm.sxk * tm.K) || !fits_int(tm.syk * tm.K)) return HGPU_OK;
+    ktot += tm.K;
+    sp.terms.push_back(tm);
+  }
+  if (ktot < 4 || ktot > kMaxKTotal) return HGPU_OK;
+  if (sp.P < 16 || sp.Q < 4 || (double)sp.P * sp.Q * ktot < 2.0e6) return HGPU_OK;
+  for (int o = 0; o < n_out; ++o) {
+    if (out_slots[o] < n_in && out_slots[o] != c_slot) return HGPU_OK;   // a copy of an input: not this kernel's business
+    if (!outs[o]->buf) return HGPU_OK;
+  }
+  sp.n_in = n_in;
+  sp.c_slot = c_slot;
+  sp.n_instr = n_instr;
+  sp.prog = prog;
+  sp.dt = dt;
+  sp.in_sp.assign((size_t)n_in, 0);
+  sp.in_sq.assign((size_t)n_in, 0);
+  for (int i = 0; i < n_in; ++i) {
+    if (i == c_slot) continue;
+    if (!in[i]->buf) return HGPU_OK;
+    sp.in_sp[(size_t)i] = in[i]->strides[kd.dp];
+    sp.in_sq[(size_t)i] = in[i]->strides[kd.dq];
+    if (!fits_int(sp.in_sp[(size_t)i] * sp.P) || !fits_int(sp.in_sq[(size_t)i] * sp.Q)) return HGPU_OK;
+  }
+  sp.out_slots.assign(out_slots, out_slots + n_out);
+  choose_tile(ctx, sp, ktot);
+  if (!plan_chunks(sp)) return HGPU_OK;
+
+  char kname[96];
+  snprintf(kname, sizeof kname, "smallk_%s_p%lld_q%lld_k%lld_t%d", sp.f64 ? "f64" : "f32", (long long)sp.P, (long long)sp.Q, (long long)ktot, n_terms);
+  std::string src = generate(sp, kname);
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c{nullptr, nullptr};
+    std::vector<char> code;
+    int rc = rtc_compile(ctx, src, "small-K product", &code);
+    if (rc && getenv("HORDEAD_GPU_DEBUG")) fprintf(stderr, "hordead_gpu: %s rejected: %s\n", kname, hgpu_last_error(ctx));
+    if (!rc) {
+      hipError_t e = hipModuleLoadData(&c.mod, code.data());
+      if (e == hipSuccess) e = hipModuleGetFunction(&c.fn, c.mod, kname);
+      if (e != hipSuccess) c = Compiled{nullptr, nullptr};
+    }
+    it = cache.emplace(src, c).first;
+  }
+  if (!it->second.fn) return HGPU_OK;
+
+  std::vector<const void*> ar;
+  for (auto& tm : sp.terms) { ar.push_back(tm.x); ar.push_back(tm.y); }
+  for (int i = 0; i < n_in; ++i)
+    if (i != c_slot) ar.push_back(data_ptr(in[i]));
+  for (int o = 0; o < n_out; ++o) ar.push_back(data_ptr(outs[o]));
+  void* args[] = {(void*)ar.data()};
+  const int64_t nblk = ((sp.P + sp.BP - 1) / sp.BP) * ((sp.Q + sp.BQ - 1) / sp.BQ);
+  const int64_t grid = (nblk + 7) / 8 * 8;
+  if (grid > 0x7fffffff) return HGPU_OK;
+  const double es = sp.f64 ? 8 : 4;
+  double flops = 2.0 * (double)sp.P * sp.Q * ktot;
+  double bytes = ((double)sp.P + sp.Q) * ktot * es;
+  for (int i = 0; i < n_in; ++i)
+    if (i != c_slot) bytes += (sp.in_sp[(size_t)i] ? (double)sp.P : 1.0) * (sp.in_sq[(size_t)i] ? (double)sp.Q : 1.0) * (double)dtype_size(in[i]->dtype);
+  for (int o = 0; o < n_out; ++o) bytes += (double)sp.P * sp.Q * (double)dtype_size(outs[o]->dtype);
+  const char* label = sp.f64 ? "gemm_f64" : "gemm_f32";
+  if (ctx->profiling && ctx->profile_shapes) {
+    char buf[200];
+    std::string ks;
+    for (auto& tm : sp.terms) ks += (ks.empty() ? "" : "+") + std::to_string(tm.K);
+    snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%sxB1,wholeK,t%dx%d,chunks%d,lds%dK,map(in%d,instr%d,out%d)]", label, (long long)sp.Q, (long long)sp.P, ks.c_str(), sp.BQ,
+             sp.BP, (int)sp.chunks.size(), (int)((sp.x_elems + sp.y_elems) * (int)es / 1024), n_in - 1, n_instr, n_out);
+    label = ctx->label_pool.insert(buf).first->c_str();
+  }
+  LaunchGuard lg(ctx, label, bytes, flops);
+  hipError_t err = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+  if (err != hipSuccess) return check_hip(ctx, err, "small-K product launch");
+  *handled = true;
+  return HGPU_OK;
+}
+
+}  // namespace hg
+
+extern "C" int hgpu_contract_sum_map(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs, int n_keep, int n_in,
+                                     const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int n_out, const int* out_slots, hgpu_array** outs) {
+  if (!ctx || !as || !bs || !in || n_terms < 1 || (n_instr > 0 && !prog) || n_out < 1 || !out_slots || !outs) return HGPU_ERR_INVALID;
+  for (int t = 0; t < n_terms; ++t)
+    if (!as[t] || !bs[t]) return HGPU_ERR_INVALID;
+  const hgpu_array* a0 = as[0];
+  if (n_keep < 1 || n_keep > a0->rank) return fail(ctx, HGPU_ERR_INVALID, "contract_sum_map: n_keep %d of rank %d", n_keep, a0->rank);
+  for (int t = 0; t < n_terms; ++t) {
+    if (as[t]->dtype != a0->dtype || bs[t]->dtype != a0->dtype || !same_shape(as[t], bs[t])) return fail(ctx, HGPU_ERR_INVALID, "contract_sum_map: factors differ in dtype or shape");
+    bool ok = as[t]->rank >= n_keep;
+    for (int d = 0; d < n_keep && ok; ++d) ok = as[t]->shape[d] == a0->shape[d];
+    if (!ok) return fail(ctx, HGPU_ERR_INVALID, "contract_sum_map: term %d does not have the kept shape", t);
+  }
+  if (n_in < 1 || n_in > 12 || n_instr < 0 || n_instr > 96 || n_out > 6) return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract_sum_map: %d inputs, %d instructions, %d outputs", n_in, n_instr, n_out);
+  int c_slot = -1;
+  for (int i = 0; i < n_in; ++i) {
+    if (!in[i]) {
+      if (c_slot >= 0) return fail(ctx, HGPU_ERR_INVALID, "contract_sum_map: more than one input stands for the sum");
+      c_slot = i;
+      continue;
+    }
+    bool ok = in[i]->rank == n_keep;
+    for (int d = 0; d < n_keep && ok; ++d) ok = in[i]->shape[d] == a0->shape[d];
+    if (!ok) return fail(ctx, HGPU_ERR_INVALID, "contract_sum_map: input %d does not have the kept shape", i);
+  }
+  if (c_slot < 0) return fail(ctx, HGPU_ERR_INVALID, "contract_sum_map: no input stands for the sum");
+  std::vector<int> dt;
+  {
+    std::vector<const hgpu_array*> tin(in, in + n_in);
+    tin[(size_t)c_slot] = a0;   // only the dtype is read
+    if (int rc = check_program(ctx, n_in, tin.data(), n_instr, prog, &dt)) return rc;
+  }
+  for (int o = 0; o < n_out; ++o)
+    if (out_slots[o] < 0 || out_slots[o] >= n_in + n_instr) return fail(ctx, HGPU_ERR_INVALID, "contract_sum_map: bad output slot");
+  int64_t n_kept = 1;
+  for (int d = 0; d < n_keep; ++d) n_kept *= a0->shape[d];
+  if (n_kept > 0) {
+    std::vector<hgpu_array*> res((size_t)n_out, nullptr);
+    auto release_res = [&] { for (auto*& r : res) if (r) { hgpu_release(r); r = nullptr; } };
+    int rc = HGPU_OK;
+    for (int o = 0; o < n_out && !rc; ++o) rc = new_dense(ctx, dt[(size_t)out_slots[o]], n_keep, a0->shape, &res[(size_t)o]);
+    bool handled = false;
+    if (!rc) rc = try_smallk(ctx, n_terms, as, bs, n_keep, n_in, in, c_slot, n_instr, prog, dt, n_out, out_slots, res.data(), &handled);
+    if (rc || !handled) release_res();
+    if (rc) return rc;
+    if (handled) {
+      for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
+      return HGPU_OK;
+    }
+  }
+  // one entry point after another: the products (terms of one shape together), their sum, the program
+  hgpu_array* c = nullptr;
+  {
+    std::vector<char> taken((size_t)n_terms, 0);
+    for (int t0 = 0; t0 < n_terms; ++t0) {
+      if (taken[(size_t)t0]) continue;
+      std::vector<const hgpu_array*> ga, gb;
+      for (int t = t0; t < n_terms; ++t)
+        if (!taken[(size_t)t] && same_shape(as[t], as[t0])) { ga.push_back(as[t]); gb.push_back(bs[t]); taken[(size_t)t] = 1; }
+      hgpu_array* part = nullptr;
+      int rc = hgpu_contract_sum(ctx, (int)ga.size(), ga.data(), gb.data(), n_keep, &part);
+      if (!rc && c) {
+        hgpu_array* sum = nullptr;
+        rc = hgpu_ewise2(ctx, HGPU_ADD, c, part, &sum);
+        hgpu_release(part);
+        hgpu_release(c);
+        c = sum;
+      } else if (!rc) {
+        c = part;
+      }
+      if (rc) { if (c) hgpu_release(c); return rc; }
+    }
+  }
+  std::vector<const hgpu_array*> ins(in, in + n_in);
+  ins[(size_t)c_slot] = c;
+  std::vector<hgpu_array*> res((size_t)n_out, nullptr);
+  int rc = HGPU_OK;
+  std::vector<int> fslots;
+  std::vector<size_t> fpos;
+  for (int o = 0; o < n_out && !rc; ++o) {
+    if (out_slots[o] == c_slot) { hgpu_retain(c); res[(size_t)o] = c; }
+    else if (out_slots[o] < n_in) rc = hgpu_materialize(ctx, ins[(size_t)out_slots[o]], &res[(size_t)o]);
+    else { fslots.push_back(out_slots[o]); fpos.push_back((size_t)o); }
+  }
+  if (!rc && !fslots.empty()) {
+    std::vector<hgpu_array*> fres(fslots.size(), nullptr);
+    rc = hgpu_fused_map(ctx, n_in, ins.data(), n_instr, prog, (int)fslots.size(), fslots.data(), fres.data());
+    if (!rc) for (size_t i = 0; i < fpos.size(); ++i) res[fpos[i]] = fres[i];
+  }
+  hgpu_release(c);
+  if (rc) {
+    for (auto* r : res) if (r) hgpu_release(r);
+    return rc;
+  }
+  for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
+  return HGPU_OK;
+}

@@ -320,6 +320,7 @@ static bool pad_view(const T& a, const Shape& lo, const Shape& hi, T* out) {
   return T(be__, o__)
 
 static T contract_now(const T& a, const T* b, int n_keep);
+static bool holds_pending_contraction(const ArrHolder* root);
 static void pieces_of(const T& t, std::vector<ArrHolder::Piece>* out);
 static T make_merged(const T& inner, const Shape& shape, const std::vector<int>& groups);
 static T split_view(const T& y, const Shape& fine);
@@ -370,6 +371,7 @@ struct Program {
   // stays as it is (an input without an array), for a kernel that computes it
   // and runs the program over its result in one pass
   bool keep_contraction = false;
+  bool keep_sums = false;     // ... or one pending SUM of contractions (for a kernel that adds the products too)
   ArrHolder* kept = nullptr;
 };
 
@@ -379,8 +381,13 @@ bool single_contraction(const ArrHolder* p) {
 
 // Post-order walk: materialised values (and pending contractions, which are
 // forced here) become inputs, pending elementwise nodes become instructions.
+// a pending contraction of two arrays, or a pending sum of such
+bool contraction_or_sum(const ArrHolder* p) {
+  return !p->h && p->ekind < 0 && p->fa && p->fb && p->keep >= 1 && !p->origin && !p->vsrc && p->pieces.empty() && !p->mv_inner && !p->ssrc && !p->probe;
+}
+
 int visit(Program& pg, ArrHolder* p) {
-  if (pg.keep_contraction && single_contraction(p) && (!pg.kept || pg.kept == p)) {
+  if (pg.keep_contraction && (pg.keep_sums ? contraction_or_sum(p) : single_contraction(p)) && (!pg.kept || pg.kept == p)) {
     pg.kept = p;
     auto it = pg.in_slot.find(p);
     if (it != pg.in_slot.end()) return -1 - it->second;
@@ -418,9 +425,10 @@ int visit(Program& pg, ArrHolder* p) {
 // With `kept`: one pending contraction among the leaves stays pending (*kept; its
 // entry of ins is null), and nodes receives the holder of every instruction.
 static void number_program(const std::vector<ArrHolder*>& roots, std::vector<const hgpu_array*>* ins, std::vector<hgpu_fused_instr>* prog,
-                           std::vector<int>* outs_slot, ArrHolder** kept = nullptr, std::vector<ArrHolder*>* nodes = nullptr) {
+                           std::vector<int>* outs_slot, ArrHolder** kept = nullptr, std::vector<ArrHolder*>* nodes = nullptr, bool keep_sums = false) {
   Program pg;
   pg.keep_contraction = kept != nullptr;
+  pg.keep_sums = keep_sums;
   std::vector<int> root_slot;
   for (auto* r : roots) root_slot.push_back(visit(pg, r));
   int n_in = (int)pg.inputs.size();
@@ -440,6 +448,77 @@ static void number_program(const std::vector<ArrHolder*>& roots, std::vector<con
 }
 
 static void measure(const std::vector<ArrHolder*>& roots, int* n_in, int* n_instr);
+
+// `tanh (W x + V s + b)`: when one leaf of the roots' expressions is a pending
+// contraction (or sum of contractions) and the provider has
+// hgpu_contract_sum_map, the products, their sum and the program go out as one
+// call and the sum is never written -- unless someone outside the program still
+// holds it, in which case it is one more result of the same call.
+static bool products_then_program(Backend* be, const std::vector<ArrHolder*>& roots, std::vector<hgpu_array*>* outs) {
+  const hgpu_api* api = be->api;
+  if (!be->fuse || !(api->struct_size >= offsetof(hgpu_api, contract_sum_map) + sizeof(api->contract_sum_map) && api->contract_sum_map)) return false;
+  if (roots.size() > 5) return false;
+  // is there such a leaf at all?  (walk without forcing anything)
+  {
+    std::map<const ArrHolder*, int> seen;
+    std::vector<const ArrHolder*> stack(roots.begin(), roots.end());
+    bool found = false;
+    while (!stack.empty() && !found) {
+      const ArrHolder* p = stack.back();
+      stack.pop_back();
+      if (seen.count(p)) continue;
+      seen[p] = 1;
+      if (contraction_or_sum(p)) { found = true; break; }
+      if (p->h || p->ekind < 0) continue;
+      if (p->fa) stack.push_back(p->fa.get());
+      if (p->fb) stack.push_back(p->fb.get());
+      if (p->fc) stack.push_back(p->fc.get());
+    }
+    if (!found) return false;
+  }
+  std::vector<const hgpu_array*> ins;
+  std::vector<hgpu_fused_instr> prog;
+  std::vector<int> slots;
+  std::vector<ArrHolder*> nodes;
+  ArrHolder* kept = nullptr;
+  number_program(roots, &ins, &prog, &slots, &kept, &nodes, true);
+  if (!kept) return false;
+  if (T(kept->fa).dtype() != HGPU_F64 && T(kept->fa).dtype() != HGPU_F32) { kept->force(); return false; }
+  int c_slot = -1;
+  for (size_t i = 0; i < ins.size(); ++i)
+    if (!ins[i]) c_slot = (int)i;
+  // who else holds the sum?
+  std::shared_ptr<ArrHolder> ks;
+  long inside = 0;
+  for (auto* nd : nodes)
+    for (auto* f : {&nd->fa, &nd->fb, &nd->fc})
+      if (f->get() == kept) { ks = *f; ++inside; }
+  for (auto* r : roots)
+    if (r == kept) return false;   // cannot be: roots are expressions
+  const bool shared = !ks || ks.use_count() - 1 > inside;
+  if (c_slot < 0 || (int)ins.size() > 12 || (int)prog.size() > 96) { kept->force(); return false; }
+  std::vector<T> fas{T(kept->fa)}, fbs{T(kept->fb)};
+  for (auto& m : kept->more) { fas.push_back(T(m.first)); fbs.push_back(T(m.second)); }
+  std::vector<const hgpu_array*> ah, bh;
+  for (size_t t = 0; t < fas.size(); ++t) { ah.push_back(fas[t].h()); bh.push_back(fbs[t].h()); }
+  std::vector<int> out_slots(slots);
+  if (shared) out_slots.push_back(c_slot);
+  std::vector<hgpu_array*> res(out_slots.size(), nullptr);
+  int rc = api->contract_sum_map(be->ctx, (int)ah.size(), ah.data(), bh.data(), kept->keep, (int)ins.size(), ins.data(), (int)prog.size(), prog.data(), (int)out_slots.size(),
+                                 out_slots.data(), res.data());
+  if (rc == HGPU_ERR_UNSUPPORTED) { kept->force(); return false; }
+  be->check(rc);
+  be->counters["contract_sum_map"]++;
+  for (size_t i = 0; i < roots.size(); ++i) (*outs)[i] = res[i];
+  if (shared) {
+    kept->h = res.back();
+    kept->fa.reset();
+    kept->fb.reset();
+    kept->more.clear();
+    kept->keep = -1;
+  }
+  return true;
+}
 
 static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
   std::vector<const hgpu_array*> ins;
@@ -484,7 +563,9 @@ static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
       sums.clear();
     }
   }
-  if (sums.empty()) {
+  if (sums.empty() && products_then_program(be, roots, &outs)) {
+    // done by one kernel: products, their sum and the program
+  } else if (sums.empty()) {
     number_program(roots, &ins, &prog, &outs_slot);
     int n_in = (int)ins.size(), n_instr = (int)prog.size();
     be->check(be->api->fused_map(be->ctx, n_in, ins.data(), n_instr, prog.data(), (int)roots.size(), outs_slot.data(), outs.data()));
@@ -644,7 +725,16 @@ void ArrHolder::force() {
     for (auto& m : more) { as.push_back(T(m.first)); bs.push_back(T(m.second)); }
     const hgpu_api* api = be->api;
     hgpu_array* o = nullptr;
-    if (api->struct_size >= offsetof(hgpu_api, contract_sum) + sizeof(api->contract_sum) && api->contract_sum) {
+    bool one_shape = true;
+    for (size_t i = 1; i < as.size(); ++i) one_shape = one_shape && as[i].shape() == as[0].shape();
+    if (!one_shape && api->struct_size >= offsetof(hgpu_api, contract_sum_map) + sizeof(api->contract_sum_map) && api->contract_sum_map) {
+      // products over contracted dims of different lengths (W x + V s): the sum alone, by the kernel that would also run a program over it
+      std::vector<const hgpu_array*> ah, bh;
+      for (size_t i = 0; i < as.size(); ++i) { ah.push_back(as[i].h()); bh.push_back(bs[i].h()); }
+      const hgpu_array* none = nullptr;
+      const int slot = 0;
+      be->check(api->contract_sum_map(be->ctx, (int)ah.size(), ah.data(), bh.data(), keep, 1, &none, 0, nullptr, 1, &slot, &o));
+    } else if (one_shape && api->struct_size >= offsetof(hgpu_api, contract_sum) + sizeof(api->contract_sum) && api->contract_sum) {
       std::vector<const hgpu_array*> ah, bh;
       for (size_t i = 0; i < as.size(); ++i) { ah.push_back(as[i].h()); bh.push_back(bs[i].h()); }
       be->check(api->contract_sum(be->ctx, (int)ah.size(), ah.data(), bh.data(), keep, &o));
@@ -678,9 +768,19 @@ void ArrHolder::force() {
   keep = -1;
 }
 
+// Two pending contractions can wait as one pending sum when their factors have
+// one shape, or -- with a provider that sums products of different contracted
+// lengths in one kernel (hgpu_contract_sum_map) -- when they keep the same dims.
+static bool sums_with(const T& a, const T& b) {
+  if (T(a.holder()->fa).shape() == T(b.holder()->fa).shape()) return true;
+  const hgpu_api* api = a.be()->api;
+  if (!(api->struct_size >= offsetof(hgpu_api, contract_sum_map) + sizeof(api->contract_sum_map) && api->contract_sum_map)) return false;
+  return a.holder()->keep >= 1 && a.shape() == b.shape();
+}
+
 T add_cotangents(const T& a, const T& b) {
   if (a.contraction_like() && b.contraction_like() && a.be() == b.be() && a.holder()->keep == b.holder()->keep &&
-      a.dtype() == b.dtype() && T(a.holder()->fa).shape() == T(b.holder()->fa).shape()) {
+      a.dtype() == b.dtype() && sums_with(a, b)) {
     auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
     const ArrHolder* x = a.holder().get();
     const ArrHolder* y = b.holder().get();
@@ -864,6 +964,11 @@ T transpose(const T& a, const std::vector<int>& perm) {
   }
   HD_META_VIEW(meta_transpose(a.holder()->vmeta, perm, &m__))
   if (a.pending_merged() && expression_like(a) && a.size() > 0) return transpose(make_view(a.holder(), dense_meta(a.shape())), perm);
+  // A product that others hold too and that has an uncomputed contraction beneath
+  // it (a cotangent `(W^T dz) * (1 - h * h)` on its way to the bias and to the
+  // next products): one kernel will write it out for all of them; this is a view of that.
+  if (a.pending_product() && a.holder().use_count() > 1 && a.size() > 0 && holds_pending_contraction(a.holder().get()))
+    return transpose(make_view(a.holder(), dense_meta(a.shape())), perm);
   HD_VIEW_OF_EXPR(transpose(x, perm))
   if (a.pending_contraction() && (int)perm.size() <= a.pending_keep())   // permutes kept dims only
   {
@@ -973,7 +1078,7 @@ T ewise2(int op, const T& a, const T& b) {
   if (any_merged_same_shape({&a, &b})) return lift_merged({&a, &b}, [&](const std::vector<T>& v) { return ewise2(op, v[0], v[1]); });
   // W x + V s, both products still pending and of one shape: a pending sum of contractions
   if (op == HGPU_ADD && a.contraction_like() && b.contraction_like() && a.be() == b.be() && a.be()->fuse && a.holder()->keep == b.holder()->keep &&
-      a.dtype() == b.dtype() && T(a.holder()->fa).shape() == T(b.holder()->fa).shape())
+      a.dtype() == b.dtype() && sums_with(a, b))
     return add_cotangents(a, b);
   if (!fuses(a.be()) || !agree(a, b) || !op2_ok(op, a.dtype()) || a.size() == 0) return ewise2_now(op, a, b);
   return make_expr(HGPU_FUSED_OP2, op, a.dtype(), a, &b, nullptr);
@@ -1002,9 +1107,40 @@ T convert(const T& a, int dtype, int mode) {
   if (!fuses(a.be()) || !ok || a.size() == 0) return convert_now(a, dtype, mode);
   return make_expr(HGPU_FUSED_CONVERT, mode, dtype, a, nullptr, nullptr);
 }
+// Does the expression beneath p have a leaf that is a contraction (or a sum of contractions) not yet computed?
+static bool holds_pending_contraction(const ArrHolder* root) {
+  std::map<const ArrHolder*, int> seen;
+  std::vector<const ArrHolder*> stack{root};
+  while (!stack.empty()) {
+    const ArrHolder* p = stack.back();
+    stack.pop_back();
+    if (seen.count(p)) continue;
+    seen[p] = 1;
+    if (contraction_or_sum(p)) return true;
+    if (!p->h && p->vsrc) { stack.push_back(p->vsrc.get()); continue; }
+    if (p->h || p->ekind < 0) continue;
+    if (p->fa) stack.push_back(p->fa.get());
+    if (p->fb) stack.push_back(p->fb.get());
+    if (p->fc) stack.push_back(p->fc.get());
+  }
+  return false;
+}
+
 T contract(const T& a, const T* b, int n_keep) {
-  if (!b && a.pending_product())   // sum (u * v) = the contraction of u and v; stays pending
+  if (!b && a.pending_product()) {   // sum (u * v) = the contraction of u and v; stays pending
+    // ... unless a factor still holds an uncomputed contraction (the cotangent
+    // W^T dz under `* (1 - h * h)`): taken apart, the factors would be written
+    // out one by one; whole, the product is one kernel's result, which the
+    // other consumers of the product need anyway.  Its sum is then its
+    // contraction with ones.
+    if (n_keep >= 1 && fuses(a.be()) && holds_pending_contraction(a.holder().get()))
+      return lazy_contract(a, broadcast_scalar(constant(a.be(), a.dtype(), 1.0), a.shape()), n_keep);
     return lazy_contract(a.factor_a(), a.factor_b(), n_keep);
+  }
+  // the sum of a view of such a product likewise waits (sums of one shape then go out together)
+  if (!b && n_keep >= 1 && n_keep < a.rank() && a.pending_view() && fuses(a.be()) && a.holder()->vlo.empty() && T(a.holder()->vsrc).pending_product() &&
+      (a.dtype() == HGPU_F64 || a.dtype() == HGPU_F32) && holds_pending_contraction(a.holder()->vsrc.get()))
+    return lazy_contract(a, broadcast_scalar(constant(a.be(), a.dtype(), 1.0), a.shape()), n_keep);
   // ssum0 of a pending expression: summed while it is evaluated, never written
   if (!b && n_keep == 0 && a.pending_expr() && a.size() > 0 && (a.dtype() == HGPU_F64 || a.dtype() == HGPU_F32)) {
     Backend* be = a.be();

@@ -288,6 +288,26 @@ int hgpu_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, i
                       int ext_slot, int view_rank, const int64_t* view_shape, const int64_t* view_strides,
                       int n_reduce, int want_max, hgpu_array** values, hgpu_array** indices);
 
+/* A SUM of contractions followed, in the same pass, by an elementwise program
+ * over the sum: a layer of the reference's recurrent network,
+ * `tanh (wX `rmatmul2` x + wS `rmatmul2` s + rtr (rreplicate batch_size b))`
+ * (example/MnistRnnRanked2.hs:62-75), reaches the backend as two matrix
+ * products, two `+` and a `tanh`, and the head of its cotangent as two
+ * products, a `+` and `* (1 - h * h)` (DeltaEval.hs:391-595 adds the two uses
+ * of a layer's output).  Neither the products nor their sum are written.
+ *   C = sum_t hgpu_contract(a[t], b[t], n_keep); the terms agree in dtype and
+ *   in their first n_keep dims, the contracted dims may differ from term to term;
+ *   program, in, out_slots, outs: as for hgpu_contract_map (exactly one entry
+ *   of `in` is NULL and stands for C; n_out >= 1).
+ * When the contracted dims are short (together at most 512 elements) and the
+ * kept shape has two non-unit dims this is one kernel compiled for the shapes,
+ * with the whole contracted dim of a term in LDS; otherwise the single entry
+ * points run one after another.  Results equal theirs up to the order of the
+ * floating-point sums. */
+int hgpu_contract_sum_map(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* a, const hgpu_array* const* b, int n_keep,
+                          int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
+                          int n_out, const int* out_slots, hgpu_array** outs);
+
 /* hgpu_contract whose operands need not exist in memory.  The cotangent of a
  * pooled, rectified convolution -- `sscatter` at the arg-maxima, times the relu
  * mask (test/simplified/TestMnistPP.hs:734-735) -- is an elementwise expression
@@ -484,6 +504,8 @@ typedef struct hgpu_api {
                       int, const int*, hgpu_array**, int, int, const int64_t*, const int64_t*, int, int, hgpu_array**, hgpu_array**);
   int (*contract_operands)(hgpu_ctx*, const hgpu_operand*, const hgpu_operand*, int, int, hgpu_array**);
   int (*fused_map_sums)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, const int*, hgpu_array**, int, const int*, hgpu_array**);
+  int (*contract_sum_map)(hgpu_ctx*, int, const hgpu_array* const*, const hgpu_array* const*, int, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int,
+                         const int*, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

@@ -870,6 +870,36 @@ int horc_fused_map_sums(hgpu_ctx* c, int n_in, const hgpu_array* const* in, int 
   return rc;
 }
 
+// sum of contractions (terms may differ in their contracted dims), then the program: each term by
+// horc_contract, the terms added in order, the program by horc_fused_map
+int horc_contract_sum_map(hgpu_ctx* c, int n_terms, const hgpu_array* const* a, const hgpu_array* const* b, int n_keep, int n_in, const hgpu_array* const* in,
+                          int n_instr, const hgpu_fused_instr* prog, int n_out, const int* out_slots, hgpu_array** outs) {
+  if (n_terms < 1 || n_out < 1) return fail(c, HGPU_ERR_INVALID, "contract_sum_map: needs a term and an output");
+  hgpu_array* acc = nullptr;
+  for (int t = 0; t < n_terms; ++t) {
+    hgpu_array* part = nullptr;
+    int rc = horc_contract(c, a[t], b[t], n_keep, &part);
+    if (!rc && acc) {
+      hgpu_array* sum = nullptr;
+      rc = horc_ewise2(c, HGPU_ADD, acc, part, &sum);
+      horc_release(part);
+      horc_release(acc);
+      acc = sum;
+    } else if (!rc) {
+      acc = part;
+    }
+    if (rc) { if (acc) horc_release(acc); return rc; }
+  }
+  std::vector<const hgpu_array*> ins(in, in + n_in);
+  int n_null = 0;
+  for (auto& p : ins)
+    if (!p) { p = acc; ++n_null; }
+  int rc = n_null == 1 ? HGPU_OK : fail(c, HGPU_ERR_INVALID, "contract_sum_map: exactly one input must stand for the sum");
+  if (!rc) rc = horc_fused_map(c, n_in, ins.data(), n_instr, prog, n_out, out_slots, outs);
+  horc_release(acc);
+  return rc;
+}
+
 const hgpu_api* horc_get_api(void) {
   static const hgpu_api api = {
       sizeof(hgpu_api),
@@ -888,6 +918,7 @@ const hgpu_api* horc_get_api(void) {
       nullptr,   // no contract_map
       nullptr,   // no contract_operands
       nullptr,   // no fused_map_sums
+      nullptr,   // no contract_sum_map
   };
   return &api;
 }
@@ -900,6 +931,7 @@ const hgpu_api* horc_get_api_fused(void) {
   api.contract_map = horc_contract_map;
   api.contract_operands = horc_contract_operands;
   api.fused_map_sums = horc_fused_map_sums;
+  api.contract_sum_map = horc_contract_sum_map;
   return &api;
 }
 

@@ -1,0 +1,186 @@
+"""hgpu_contract_sum_map: a sum of matrix products with short contracted dims and
+an elementwise program over the sum -- the layer of the reference's recurrent
+network, `tanh (wX `rmatmul2` x + wS `rmatmul2` s + rtr (rreplicate batch_size b))`
+(example/MnistRnnRanked2.hs:62-75), and the head of its cotangent.
+
+Device against the checker through the C ABI; the checker DEFINES the entry
+point as hgpu_contract per term, `+` in order, hgpu_fused_map.  fp64 within
+1e-10, fp32 within 1e-5 normwise; Bool results of comparisons are compared
+away from the ties that rounding can flip.
+"""
+import numpy as np
+import pytest
+
+from conftest import capi
+
+O1, O2 = capi.OP1, capi.OP2      # instruction kinds: 0 unary, 1 binary, 2 comparison
+RNG = np.random.default_rng(2024)
+TOL = {np.dtype(np.float64): 1e-10, np.dtype(np.float32): 1e-5}
+
+
+def matmul_views(w, x):
+    """w [m, k], x [k, n] as the two factors of tsmatmul2: both of shape [m, n, k]."""
+    m, n = w.shape[0], x.shape[1]
+    return w.replicate([n]).transpose([1, 0]), x.replicate([m]).transpose([0, 2, 1])
+
+
+def rel(got, want):
+    scale = max(float(np.max(np.abs(want))), 1e-300)
+    return float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+
+
+def layer_case(ctx, dt, m, n, ks, layouts, bias=True):
+    """sum_t w_t . x_t (+ bias) -> tanh; layouts[t] = 'mk' (w stored [m, k]) or 'km' (stored [k, m], used transposed)."""
+    terms, want = [], np.zeros((m, n), np.float64)
+    for k, lay in zip(ks, layouts):
+        w = RNG.uniform(-0.3, 0.3, (m, k)).astype(dt)
+        x = RNG.uniform(-1, 1, (k, n)).astype(dt)
+        wa = ctx.upload(w) if lay == "mk" else ctx.upload(np.ascontiguousarray(w.T)).transpose([1, 0])
+        terms.append(matmul_views(wa, ctx.upload(x)))
+        want += w.astype(np.float64) @ x.astype(np.float64)
+    b = RNG.uniform(-0.5, 0.5, (m,)).astype(dt)
+    if bias:
+        ins = [None, ctx.upload(b).replicate([n]).transpose([1, 0])]
+        prog = [(1, O2["add"], 0, 0, 1, 0), (0, O1["tanh"], 0, 2, 0, 0)]
+        want = np.tanh(want + b.astype(np.float64)[:, None])
+        slots = [3]
+    else:
+        ins, prog, slots = [None], [], [0]
+    return terms, ins, prog, slots, want
+
+
+SHAPES = [
+    # dtype, m, n, ks, layouts
+    (np.float32, 128, 1000, [28, 128], ["mk", "mk"]),       # the first layer of the recurrent network
+    (np.float32, 128, 1000, [128, 128], ["km", "km"]),      # the cotangent's two products (weights transposed)
+    (np.float32, 128, 1000, [128], ["mk"]),
+    (np.float64, 300, 1000, [100], ["km"]),                 # a dense layer's cotangent
+    (np.float64, 100, 1000, [300], ["mk"]),                 # five chunks
+    (np.float64, 10, 999, [30], ["mk"]),                    # odd extent: no vectors along n, k padded to 32
+    (np.float32, 10, 998, [27], ["mk"]),                    # k neither a multiple of 4 nor contiguous vectors
+    (np.float32, 40, 1004, [8, 12, 16, 20], ["mk", "km", "mk", "km"]),
+    (np.float32, 128, 1000, [600], ["mk"]),                 # too long for the kernel: the entry points one after another
+    (np.float32, 6, 20, [5], ["mk"]),                       # too small for it
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,m,n,ks,layouts", SHAPES)
+def test_layer_matches_checker_and_numpy(gpu, oracle, dt, m, n, ks, layouts):
+    one_kernel = sum(ks) <= 512 and m * n * sum(ks) >= 2e6      # what the compiled kernel covers
+    for bias in (True, False):
+        gpu.check(gpu.lib.profile_enable(gpu.h, 2))
+        state = RNG.bit_generator.state
+        res = []
+        for ctx in (gpu, oracle):
+            RNG.bit_generator.state = state
+            terms, ins, prog, slots, want = layer_case(ctx, dt, m, n, ks, layouts, bias)
+            res.append(ctx.contract_sum_map(terms, 2, ins, prog, slots)[0].numpy())
+        labels = list(gpu.profile_report())
+        gpu.check(gpu.lib.profile_enable(gpu.h, 0))
+        assert any("wholeK" in k for k in labels) == one_kernel, labels
+        if one_kernel:
+            assert len(labels) == 1, labels
+        assert res[0].shape == (m, n) and res[0].dtype == np.dtype(dt)
+        tol = TOL[np.dtype(dt)]
+        assert rel(res[0], res[1]) <= tol, (dt, m, n, ks, rel(res[0], res[1]))
+        assert rel(res[0], want) <= 4 * tol and rel(res[1], want) <= 4 * tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_cotangent_head_with_several_results(gpu, oracle, dt):
+    """(w2^T dz2 + w1^T dz1) * (1 - h * h), the sum itself, and a comparison, from one call;
+    the program reads h (dense), and the sum stands at slot 1."""
+    m, n, k = 128, 1000, 128
+    w2 = RNG.uniform(-0.3, 0.3, (k, m)).astype(dt)
+    w1 = RNG.uniform(-0.3, 0.3, (k, m)).astype(dt)
+    dz2 = RNG.uniform(-1, 1, (k, n)).astype(dt)
+    dz1 = RNG.uniform(-1, 1, (k, n)).astype(dt)
+    h = np.tanh(RNG.uniform(-2, 2, (m, n))).astype(dt)
+    one = np.asarray(1.0, dt)
+    prog = [(1, O2["mul"], 0, 0, 0, 0),        # 3: h * h
+            (1, O2["sub"], 0, 2, 3, 0),        # 4: 1 - h * h
+            (1, O2["mul"], 0, 1, 4, 0),        # 5: C * (1 - h * h)
+            (2, capi.CMP["lt"], 0, 1, 0, 0)]   # 6: C < h
+    res = []
+    for ctx in (gpu, oracle):
+        terms = [matmul_views(ctx.upload(w2).transpose([1, 0]), ctx.upload(dz2)), matmul_views(ctx.upload(w1).transpose([1, 0]), ctx.upload(dz1))]
+        ins = [ctx.upload(h), None, ctx.upload(one).replicate([m, n])]
+        res.append([a.numpy() for a in ctx.contract_sum_map(terms, 2, ins, prog, [5, 1, 6])])
+    c = w2.T.astype(np.float64) @ dz2.astype(np.float64) + w1.T.astype(np.float64) @ dz1.astype(np.float64)
+    want = c * (1 - h.astype(np.float64) ** 2)
+    tol = TOL[np.dtype(dt)]
+    assert rel(res[0][0], res[1][0]) <= tol and rel(res[0][0], want) <= 4 * tol
+    assert rel(res[0][1], res[1][1]) <= tol and rel(res[0][1], c) <= 4 * tol
+    assert res[0][2].dtype == np.bool_ and res[0][2].shape == (m, n)
+    clear = np.abs(c - h) > 1e-3 * np.max(np.abs(c))     # away from ties
+    assert np.array_equal(res[0][2][clear], (c < h)[clear]) and np.array_equal(res[1][2][clear], (c < h)[clear])
+
+
+@pytest.mark.gpu
+def test_plain_contractions_with_short_k_take_the_same_kernel(gpu, oracle):
+    """hgpu_contract and hgpu_contract_sum of such shapes (no program) agree with the checker too."""
+    for dt, m, n, k in [(np.float32, 128, 5000, 128), (np.float64, 300, 5000, 100), (np.float32, 128, 5000, 28)]:
+        w = RNG.uniform(-0.3, 0.3, (m, k)).astype(dt)
+        x = RNG.uniform(-1, 1, (k, n)).astype(dt)
+        got = []
+        for ctx in (gpu, oracle):
+            a, b = matmul_views(ctx.upload(w), ctx.upload(x))
+            got.append(a.contract(b, 2).numpy())
+        want = w.astype(np.float64) @ x.astype(np.float64)
+        assert rel(got[0], got[1]) <= TOL[np.dtype(dt)] and rel(got[0], want) <= 4 * TOL[np.dtype(dt)]
+
+
+@pytest.mark.gpu
+def test_argument_errors(gpu):
+    w, x = gpu.upload(np.ones((8, 4), np.float32)), gpu.upload(np.ones((4, 6), np.float32))
+    a, b = matmul_views(w, x)
+    with pytest.raises(capi.HgpuError) as e:
+        gpu.contract_sum_map([(a, b)], 2, [gpu.upload(np.ones((8, 6), np.float32))], [], [0])     # nothing stands for the sum
+    assert e.value.code == 1
+    with pytest.raises(capi.HgpuError):
+        gpu.contract_sum_map([(a, b)], 2, [None, gpu.upload(np.ones((8, 5), np.float32))], [], [0])   # an input of another shape
+    w2, x2 = gpu.upload(np.ones((7, 4), np.float32)), gpu.upload(np.ones((4, 6), np.float32))
+    with pytest.raises(capi.HgpuError):
+        gpu.contract_sum_map([(a, b), matmul_views(w2, x2)], 2, [None], [], [0])                  # terms of different kept shapes
+    with pytest.raises(capi.HgpuError):
+        gpu.contract_sum_map([(a, b)], 2, [None], [], [3])                                        # a slot that does not exist
+
+
+def test_checker_definition_against_numpy(oracle):
+    """The checker's composition itself, pinned by numpy on a case small enough to read."""
+    w1 = np.arange(6.0).reshape(2, 3)
+    x1 = np.arange(12.0).reshape(3, 4) - 5
+    w2 = np.array([[1.0, -1.0], [0.5, 2.0]])
+    x2 = np.arange(8.0).reshape(2, 4)
+    b = np.array([0.25, -0.75])
+    terms = [matmul_views(oracle.upload(w1), oracle.upload(x1)), matmul_views(oracle.upload(w2), oracle.upload(x2))]
+    ins = [None, oracle.upload(b).replicate([4]).transpose([1, 0])]
+    prog = [(1, O2["add"], 0, 0, 1, 0), (0, O1["tanh"], 0, 2, 0, 0)]
+    got, raw = oracle.contract_sum_map(terms, 2, ins, prog, [3, 0])
+    c = w1 @ x1 + w2 @ x2
+    assert np.allclose(raw.numpy(), c, rtol=0, atol=1e-12)
+    assert np.allclose(got.numpy(), np.tanh(c + b[:, None]), rtol=0, atol=1e-12)
+
+
+def test_host_rewrites_layers_onto_contract_sum_map():
+    """On a table that has the entry point, the recurrent network's layers (two
+    products of different contracted lengths, `+ b`, tanh) and the heads of their
+    cotangents go out as one call each, and the gradient equals the plain table's."""
+    from conftest import entry, pkg
+    H, W = pkg.hostapi, pkg.workloads
+    plain = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    fused = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_", api_table="get_api_fused"))
+    steps = 4
+    wl = W.c4_rnn(batch=3, steps=steps)
+    res = []
+    for host in (plain, fused):
+        ps, ds = wl.upload(host)
+        loss, grads = wl.gradient(host, ps, ds)
+        res.append((float(loss.numpy()), [g.numpy() for g in grads]))
+    assert res[0][0] == res[1][0]
+    for g0, g1 in zip(res[0][1], res[1][1]):
+        assert np.array_equal(g0, g1)
+    # two layers per step forward; backward one call per layer and step but the very first layer's input needs no cotangent
+    assert plain.counter("contract_sum_map") == 0 and fused.counter("contract_sum_map") >= 4 * steps
