@@ -203,19 +203,29 @@ std::string generate(const Spec& sp, const std::string& kname) {
     emit_stage_fn(s, ("x" + std::to_string(c)).c_str(), sp.chunks[c].x, sp.chunks[c], "", "");
     emit_stage_fn(s, ("y" + std::to_string(c)).c_str(), sp.chunks[c].y, sp.chunks[c], "", "");
   }
-  // the MFMAs of one chunk
+  // The MFMAs of one chunk.  Fragments are read from LDS a group of four k-steps
+  // ahead of the MFMAs that use them (two register sets, alternating): left to
+  // itself the compiler reads a step's fragments right before its MFMAs and
+  // waits out the whole LDS latency at every step.
   s << "template <int KCP, int LX, int PX, int LY, int PY>\n";
   s << "__device__ __forceinline__ void compute(const T* __restrict__ xs, const T* __restrict__ ys, Acc (&acc)[" << TP << "][" << TQ << "], int r, int g, int wp, int wq) {\n";
-  s << "#pragma unroll\n  for (int j = 0; j < KCP / 4; ++j) {\n";
-  s << "    T xf[" << TP << "], yf[" << TQ << "];\n";
-  s << "#pragma unroll\n    for (int a = 0; a < " << TP << "; ++a) xf[a] = LX == 0 ? xs[(4 * j + g) * PX + (wp * " << TP << " + a) * 16 + r] : xs[((wp * " << TP
+  s << "  constexpr int NS = KCP / 4, G = 4;\n";
+  s << "  T xf[2][G][" << TP << "], yf[2][G][" << TQ << "];\n";
+  s << "  auto rd = [&](int buf, int j0) {\n";
+  s << "#pragma unroll\n    for (int u = 0; u < G; ++u) {\n      const int j = j0 + u;\n      if (j >= NS) break;\n";
+  s << "#pragma unroll\n      for (int a = 0; a < " << TP << "; ++a) xf[buf][u][a] = LX == 0 ? xs[(4 * j + g) * PX + (wp * " << TP << " + a) * 16 + r] : xs[((wp * " << TP
     << " + a) * 16 + r) * PX + 4 * j + g];\n";
-  s << "#pragma unroll\n    for (int b = 0; b < " << TQ << "; ++b) yf[b] = LY == 0 ? ys[(4 * j + g) * PY + (wq * " << TQ << " + b) * 16 + r] : ys[((wq * " << TQ
+  s << "#pragma unroll\n      for (int b = 0; b < " << TQ << "; ++b) yf[buf][u][b] = LY == 0 ? ys[(4 * j + g) * PY + (wq * " << TQ << " + b) * 16 + r] : ys[((wq * " << TQ
     << " + b) * 16 + r) * PY + 4 * j + g];\n";
-  s << "#pragma unroll\n    for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n      for (int b = 0; b < " << TQ << "; ++b)\n";
-  if (sp.f64) s << "        acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(yf[b], xf[a], acc[a][b], 0, 0, 0);\n";
-  else s << "        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xf[a], yf[b], acc[a][b], 0, 0, 0);\n";
-  s << "  }\n}\n";
+  s << "    }\n  };\n";
+  s << "  rd(0, 0);\n";
+  // (the scheduling barriers keep the compiler from moving the reads back down to their uses)
+  s << "#pragma unroll\n  for (int j0 = 0; j0 < NS; j0 += G) {\n    const int cur = (j0 / G) & 1;\n    if (j0 + G < NS) rd(cur ^ 1, j0 + G);\n    __builtin_amdgcn_sched_barrier(0);\n";
+  s << "#pragma unroll\n    for (int u = 0; u < G; ++u) {\n      if (j0 + u >= NS) break;\n";
+  s << "#pragma unroll\n      for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n        for (int b = 0; b < " << TQ << "; ++b)\n";
+  if (sp.f64) s << "          acc[a][b] = __builtin_amdgcn_mfma_f64_16x16x4f64(yf[cur][u][b], xf[cur][u][a], acc[a][b], 0, 0, 0);\n";
+  else s << "          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xf[cur][u][a], yf[cur][u][b], acc[a][b], 0, 0, 0);\n";
+  s << "    }\n    __builtin_amdgcn_sched_barrier(0);\n  }\n}\n";
   // The program over one accumulator block.  What it reads besides the
   // accumulators is loaded by epi_load (rows past the end read a valid place
   // and are never written), which the kernel calls before the first chunk's
@@ -372,7 +382,11 @@ void choose_tile(hgpu_ctx* ctx, Spec& sp, int64_t ktot) {
 
 // Cuts the contracted dims of the terms into chunks and lays their tiles out in LDS.
 bool plan_chunks(Spec& sp) {
-  const int kcmax = sp.f64 ? 64 : 128;
+  int kcmax = sp.f64 ? 64 : 128;
+  if (const char* e = getenv("HORDEAD_SMALLK_KC")) {   // for measurements
+    int v = atoi(e);
+    if (v >= 8 && v <= 256 && v % 4 == 0) kcmax = v;
+  }
   sp.x_elems = sp.y_elems = 0;
   sp.chunks.clear();
   for (int t = 0; t < (int)sp.terms.size(); ++t) {
@@ -394,7 +408,7 @@ bool plan_chunks(Spec& sp) {
     }
   }
   sp.x_elems = (sp.x_elems + 3) / 4 * 4;
-  if (sp.chunks.size() > 8) return false;
+  if (sp.chunks.size() > 16) return false;
   return (size_t)(sp.x_elems + sp.y_elems) * (sp.f64 ? 8 : 4) <= 150 * 1024;
 }
 
