@@ -276,6 +276,23 @@ def main():
             results[key]["achieved_gbs_whole_step"] = wl.bytes / sec / 1e9
         del ps, ds
 
+    # the same work written another way (the reference's derived form of relu and pooling): timed beside the configs
+    riders = {}
+    if not args.only:
+        for key, make in getattr(W, "RIDERS", {}).items():
+            wl = make()
+            ps, ds = wl.upload(host)
+            host.sync()
+            eager_sec, loss = time_steps(host, wl, ps, ds, args.steps, args.warmup)
+            sec, graph_loss = (eager_sec, loss) if args.eager else time_graph(host, wl, ps, ds, args.steps, args.warmup)
+            if graph_loss != loss:
+                raise SystemExit(f"bench.py: {key}: the recorded program computed {graph_loss!r}, the eager one {loss!r}")
+            riders[key] = {"workload": wl.name, "batch": wl.batch, "ms_per_step": sec * 1e3, "loss": loss}
+            if "c3" in results and key.startswith("c3"):
+                riders[key]["ms_per_step_over_c3"] = sec * 1e3 / results["c3"]["ms_per_step"]
+                riders[key]["loss_equals_c3"] = loss == results["c3"]["loss"]
+            del ps, ds
+
     head = results[args.workload]
     train = None
     if args.train:
@@ -294,6 +311,8 @@ def main():
         "configs": {k: v for k, v in results.items() if k != args.workload},
         "headline_detail": {k: v for k, v in head.items() if k != "roofline"},
     }
+    if riders:
+        line["riders"] = riders
     if train:
         line["training_step"] = train
     print(json.dumps(line))

@@ -515,7 +515,8 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
   if (!plan_chunks(sp)) return HGPU_OK;
 
   char kname[96];
-  snprintf(kname, sizeof kname, "smallk_%s_p%lld_q%lld_k%lld_t%d", sp.f64 ? "f64" : "f32", (long long)sp.P, (long long)sp.Q, (long long)ktot, n_terms);
+  snprintf(kname, sizeof kname, "smallk_%s_p%lld_q%lld_k%lld_t%d_in%d_instr%d_out%d", sp.f64 ? "f64" : "f32", (long long)sp.P, (long long)sp.Q, (long long)ktot, n_terms, n_in - 1,
+           n_instr, n_out);
   std::string src = generate(sp, kname);
   auto& cache = cache_of(ctx);
   auto it = cache.find(src);

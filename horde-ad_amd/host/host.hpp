@@ -55,6 +55,8 @@ struct ArrHolder {
   // Small integer arrays that came from the host keep their values: index
   // functions that look constants up in them can then be folded on the host.
   std::shared_ptr<std::vector<int64_t>> host_i64;
+  // The one-element array this array repeats at every position (set by broadcast_scalar).
+  std::shared_ptr<ArrHolder> scalar_src;
   // A pending elementwise product fa * fb (h == nullptr until it is needed as
   // an array).  Views of it stay pending, and summing it is a contraction of
   // the two factors, so `tssumN (u * v)` never writes the product to memory.
@@ -128,6 +130,7 @@ struct ArrHolder {
   ~ArrHolder() { if (h) be->api->release(h); }
   ArrHolder(const ArrHolder&) = delete;
   void force();
+  bool view_of_written_source();
 };
 
 // `Gpu (TKS sh r)`: an immutable strided view on the device.  Scalars
@@ -279,6 +282,11 @@ struct Ix {
   // arg_of at [m_0, .., this] is arg_vals.
   std::shared_ptr<ArrHolder> arg_of;
   T arg_vals;
+  // ifH cond a b with constant a, b: a gather from a table by this index alone is
+  // a choice between two of the table's elements (`sgather [0.0, 1.0] (\.. -> [ifH c 0 1])`,
+  // the mask of relu in the reference's simplified programs, test/simplified/TestMnistPP.hs:735).
+  T sel_cond;
+  int64_t sel_a = 0, sel_b = 0;
 };
 
 Ix ix_var(Backend* be, const Shape& shm, int d);

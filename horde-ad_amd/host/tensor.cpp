@@ -340,6 +340,48 @@ static bool fuses(Backend* be) {
 }
 static int pending_size(const std::shared_ptr<ArrHolder>& p) { return (p && !p->h && p->ekind >= 0) ? p->esize : 0; }
 
+static T make_expr(int kind, int op, int dtype, const T& a, const T* b, const T* c);
+
+// f (view A) (view B) = view (f A B): when every operand of a new elementwise
+// node is the SAME view of some expression's dense result (or one broadcast
+// element), the node is that view of the node over the sources.  The note
+// (vsrc, vmeta -- as map_leaves leaves it) lets a consumer that knows how to
+// evaluate the source expression inside another kernel (a window extremum in a
+// convolution's epilogue) recognise `mask (windows t) * windows t`, the way the
+// reference's derived programs write relu under pooling, as windows of
+// `mask t * t`.
+static bool one_element(const T& t) { return (bool)t.holder()->scalar_src; }
+static void note_common_view(ArrHolder* p, int kind, int op, int dtype, const T& a, const T* b, const T* c) {
+  const T* ops[3] = {&a, b, c};
+  const ArrHolder* first = nullptr;
+  for (auto* o : ops) {
+    if (!o) continue;
+    const ArrHolder* h = o->holder().get();
+    const bool noted = !h->h && h->vsrc && h->vlo.empty() && !h->probe && (h->ekind >= 0 || o->pending_view());
+    if (noted) {
+      if (first && (h->vmeta.shape != first->vmeta.shape || h->vmeta.strides != first->vmeta.strides || h->vmeta.offset != first->vmeta.offset ||
+                    T(h->vsrc).shape() != T(first->vsrc).shape())) {
+        return;
+      }
+      if (!first) first = h;
+    } else if (!one_element(*o)) {
+      return;
+    }
+  }
+  if (!first) return;
+  const Shape src_shape = T(first->vsrc).shape();
+  T src[3];
+  for (int i = 0; i < 3; ++i) {
+    if (!ops[i]) continue;
+    const ArrHolder* h = ops[i]->holder().get();
+    if (!h->h && h->vsrc) src[i] = T(h->vsrc);
+    else src[i] = broadcast_scalar(T(h->scalar_src), src_shape);
+  }
+  T whole = make_expr(kind, op, dtype, src[0], b ? &src[1] : nullptr, c ? &src[2] : nullptr);
+  p->vsrc = whole.holder();
+  p->vmeta = first->vmeta;
+}
+
 static T make_expr(int kind, int op, int dtype, const T& a, const T* b, const T* c) {
   auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
   p->ekind = kind;
@@ -359,6 +401,7 @@ static T make_expr(int kind, int op, int dtype, const T& a, const T* b, const T*
     sz = 1 + pending_size(p->fa) + pending_size(p->fb) + pending_size(p->fc);
   }
   p->esize = sz;
+  note_common_view(p.get(), kind, op, dtype, a, b, c);
   return T(p);
 }
 
@@ -397,6 +440,7 @@ int visit(Program& pg, ArrHolder* p) {
     return -1 - k;
   }
   if (!p->h && p->ekind < 0) p->force();   // a pending contraction, concatenation or refined expression
+  if (!p->h && p->vsrc && p->vsrc->h) p->view_of_written_source();
   if (p->h) {
     auto it = pg.in_slot.find(p);
     if (it != pg.in_slot.end()) return -1 - it->second;
@@ -641,6 +685,26 @@ void force_many(const std::vector<T>& ts) {
     if (t.valid()) (void)t.h();
 }
 
+// An expression noted to be a view of another expression's dense result, when
+// that result has been written out in the meantime (as a side result of the
+// kernel that consumed it): the view of that array, nothing to compute.
+bool ArrHolder::view_of_written_source() {
+  if (h || ekind < 0 || !vsrc || !vsrc->h || !vlo.empty()) return false;
+  hgpu_array* base = vsrc->h;
+  if (!be->api->is_dense(base)) return false;
+  hgpu_array* o = nullptr;
+  if (be->api->as_strided(be->ctx, base, (int)vmeta.shape.size(), vmeta.shape.empty() ? nullptr : vmeta.shape.data(),
+                          vmeta.strides.empty() ? nullptr : vmeta.strides.data(), vmeta.offset, &o) != HGPU_OK)
+    return false;
+  h = o;
+  fa.reset();
+  fb.reset();
+  fc.reset();
+  vsrc.reset();
+  ekind = -1;
+  return true;
+}
+
 void ArrHolder::force() {
   if (h) return;
   if (probe) throw ProbeFail{};
@@ -716,6 +780,7 @@ void ArrHolder::force() {
     return;
   }
   if (ekind >= 0) {
+    if (view_of_written_source()) return;
     force_roots(be, {this});
     return;
   }
@@ -841,6 +906,7 @@ static T map_leaves(const T& a, const std::function<T(const T&)>& view) {
     auto it = memo.find(p.get());
     if (it != memo.end()) return it->second;
     std::shared_ptr<ArrHolder> r;
+    if (!p->h && p->ekind >= 0 && p->vsrc && p->vsrc->h) p->view_of_written_source();   // its source has been written since: a leaf
     if (p->h || p->ekind < 0) {
       // A pending contraction among the leaves is computed once, for every view
       // of it -- but not yet: the view stays pending (strides over its dense
@@ -1326,7 +1392,9 @@ T broadcast_scalar(const T& s, const Shape& shape) {
   Shape st(shape.size(), 0);
   for (auto e : shape)
     if (e == 0) return replicate(reshape(s, {}), shape);
-  return as_strided(s, shape, st, 0);
+  T r = as_strided(s, shape, st, 0);
+  if (r.holder() != s.holder()) r.holder()->scalar_src = s.holder();
+  return r;
 }
 
 T zeros(Backend* be, int dtype, const Shape& shape) { return broadcast_scalar(constant_i(be, dtype, 0), shape); }
@@ -1535,7 +1603,14 @@ Ix ix_compare(Backend* be, int cmp, const Ix& a, const Ix& b) {
 Ix ix_select(Backend* be, const Ix& c, const Ix& a, const Ix& b) {
   same_space(a, b);
   if (c.shm != a.shm || c.dtype != HGPU_BOOL) throw HostError(HGPU_ERR_INVALID, "ix_select: condition is not a Bool of the same space");
-  return from_array(a.shm, select(ix_array(be, c), ix_array(be, a), ix_array(be, b)));
+  T cond = ix_array(be, c);
+  Ix r = from_array(a.shm, select(cond, ix_array(be, a), ix_array(be, b)));
+  if (is_const(a) && is_const(b) && a.dtype == HGPU_I64) {
+    r.sel_cond = cond;
+    r.sel_a = a.c0;
+    r.sel_b = b.c0;
+  }
+  return r;
 }
 
 Ix ix_convert(Backend* be, const Ix& a, int dtype, int mode) {
@@ -1623,6 +1698,16 @@ T tsgather(const T& src, const Shape& shm, const std::vector<Ix>& ix) {
       for (size_t e = 0; e < x.coef.size() && identity; ++e) identity = x.coef[e] == (e == d ? 1 : 0);
     }
     if (identity) return ix.back().arg_vals;
+  }
+  // A rank-1 table at `ifH c a b` with constant a, b: c ? table[a] : table[b],
+  // an elementwise choice (positions outside the table read zero, as any gather).
+  if (ix.size() == 1 && src.rank() == 1 && ix[0].sel_cond.valid() && prod(shm) > 0) {
+    const int64_t n = src.shape()[0];
+    auto element = [&](int64_t k) {
+      if (k < 0 || k >= n) return zeros(be, src.dtype(), shm);
+      return broadcast_scalar(index_prefix(src, {k}), shm);
+    };
+    return select(ix[0].sel_cond, element(ix[0].sel_a), element(ix[0].sel_b));
   }
   if (all_affine(ix)) {
     // windows of a pending expression that stay in bounds and do not multiply
@@ -1988,6 +2073,8 @@ Ix ix_index0(Backend* be, const T& t, const std::vector<Ix>& ix) {
         }
       }
     }
+    // (through tsgather: windows of a pending expression are taken of its leaves, and the result remembers which view of it they are)
+    if (t.pending_expr()) return from_array(shm, tsgather(t, shm, ix));
     T v = affine_view(t, shm, ix);
     if (v.valid()) return from_array(shm, v);
   }
@@ -2005,8 +2092,11 @@ static bool contract_map_extremum(Backend* be, const T& inner, int n_reduce, boo
   const hgpu_api* api = be->api;
   if (!(api->struct_size >= offsetof(hgpu_api, contract_map) + sizeof(api->contract_map) && api->contract_map)) return false;
   const ArrHolder* ih = inner.holder().get();
+  static const bool dbg = getenv("HORDEAD_HOST_DEBUG") != nullptr;
+  if (dbg) fprintf(stderr, "contract_map_extremum: vsrc %d offset %lld shape_eq %d\n", (int)(bool)ih->vsrc, (long long)ih->vmeta.offset, (int)(ih->vmeta.shape == inner.shape()));
   if (!ih->vsrc || ih->vmeta.offset != 0 || ih->vmeta.shape != inner.shape()) return false;
   T origin(ih->vsrc);
+  if (dbg) fprintf(stderr, "  origin pending_expr %d size %d\n", (int)origin.pending_expr(), pending_size(origin.holder()));
   if (!origin.pending_expr() || pending_size(origin.holder()) > 40) return false;
   // is there exactly one pending contraction among the leaves?  (look before anything is forced)
   {
@@ -2024,6 +2114,7 @@ static bool contract_map_extremum(Backend* be, const T& inner, int n_reduce, boo
       if (p->fb) stack.push_back(p->fb.get());
       if (p->fc) stack.push_back(p->fc.get());
     }
+    if (dbg) fprintf(stderr, "  contractions among the leaves: %d\n", n_contr);
     if (n_contr != 1) return false;
   }
   std::vector<const hgpu_array*> ins;

@@ -161,6 +161,19 @@ class Host:
     def param(self, x):
         return self.concrete(x, requires_grad=True)
 
+    def sconcrete(self, x):
+        """A small constant of the program (`sconcrete (sfromListLinear ..)`: an index table,
+        the [0.0, 1.0] of a mask): uploaded the first time its value is asked for and kept, so
+        a program that names constants can be recorded after one eager run."""
+        x = np.ascontiguousarray(x)
+        key = (x.dtype.str, x.shape, x.tobytes())
+        cache = self.__dict__.setdefault("_constants", {})
+        if key not in cache:
+            if x.nbytes > 1 << 16:
+                return self.concrete(x)
+            cache[key] = self.concrete(x)
+        return cache[key]
+
     def srepl(self, shape, value, dtype=capi.F64):
         """sconcrete (sreplicate shape value)"""
         return self._out(self.dll.hh_constant, dtype, float(value), len(shape), _larr(shape))

@@ -104,11 +104,50 @@ def convMnistLayerS(ker, inp, bias):
     return maxPool2dUnpaddedS(reluS(y + bias_stretched))
 
 
-def convMnistTwoS(inp, params):
+def reluMaxPoolArtifactS(t):
+    """relu and 2x2 max-pooling of t [b, c, h, w] written as the reference's derived
+    (simplified) programs express them (test/simplified/TestMnistPP.hs:734-735):
+      w248 = sgather table (\\ix -> [ifH (0.0 <=. negate (splainPart t `sindex0` [.., m_h `sindex0` [j, p], m_w `sindex0` [k, q]])) 0 1])
+      w249 = sgather t (\\[j, k, p, q] -> [m_h `sindex0` [j, p], m_w `sindex0` [k, q]])
+      u    = sreshape (w248 * w249)               -- the windows, relu applied
+      sgather u (\\[i, j, k, l] -> [i, j, k, l, kargMax (splainPart u !$ [i, j, k, l])])
+    with table = [0.0, 1.0] and the constant index tables m = [[0, 1], [2, 3], ..]."""
+    from .hostapi import IxV, ifH
+    host = t.host
+    b, c, h, w = t.shape
+    h2, w2 = h // 2, w // 2
+    table = host.sconcrete(np.array([0.0, 1.0], NP[t.dtype]))
+    m_h = host.sconcrete(np.arange(2 * h2, dtype=np.int64).reshape(h2, 2))
+    m_w = host.sconcrete(np.arange(2 * w2, dtype=np.int64).reshape(w2, 2))
+    tp = t.sprimalPart()
+    shm = (b, c, h2, w2, 2, 2)
+
+    def mask_index(n, i, j, k, p, q):
+        zero = IxV.const(host, shm, 0.0, t.dtype)
+        x = tp.sindex0([n, i, m_h.sindex0([j, p]), m_w.sindex0([k, q])])
+        return [ifH(zero.leq(-x, t.dtype), 0, 1)]
+
+    w248 = table.sgather(shm, mask_index)
+    w249 = t.stranspose([2, 3, 0, 1]).sgather((h2, w2, 2, 2), lambda j, k, p, q: [m_h.sindex0([j, p]), m_w.sindex0([k, q])])
+    w249 = w249.stranspose([4, 5, 0, 1, 2, 3])                          # [b, c, h2, w2, 2, 2]
+    u = (w248 * w249).sreshape([b, c, h2, w2, 4])
+    up = u.sprimalPart()
+    return u.sgather((b, c, h2, w2), lambda i, j, k, l: [i, j, k, l, up.kargMax([i, j, k, l])])
+
+
+def convMnistLayerArtifactS(ker, inp, bias):
+    b, _, h, w = inp.shape
+    y = conv2dPreservingS(ker, inp)
+    bias_stretched = bias.sreplicateN([b, h, w]).stranspose([0, 3, 1, 2])
+    return reluMaxPoolArtifactS(y + bias_stretched)
+
+
+def convMnistTwoS(inp, params, layer=None):
     (k1, b1), (k2, b2), (wd, bd), (wr, br) = params
+    layer = layer or convMnistLayerS
     b = inp.shape[0]
-    t1 = convMnistLayerS(k1, inp, b1)
-    t2 = convMnistLayerS(k2, t1, b2)
+    t1 = layer(k1, inp, b1)
+    t2 = layer(k2, t1, b2)
     m1 = t2.sreshape([b, int(np.prod(t2.shape[1:]))])
     dense = wd.smatmul2(m1.str_()) + bd.sreplicate(b).str_()
     return wr.smatmul2(reluS(dense)) + br.sreplicate(b).str_()
@@ -199,9 +238,9 @@ def c3_cnn(batch=1000, dtype=F64, h=28, w=28, ksize=5, c_out=16, n_hidden=128, n
               (n_hidden, flat), (n_hidden,), (n_classes, n_hidden), (n_classes,)]
     params = [rng.uniform(-0.4, 0.4, s).astype(NP[dtype]) for s in shapes]
 
-    def objective(ps, ds):
+    def objective(ps, ds, layer=None):
         x, lab = ds
-        result = convMnistTwoS(x, list(zip(ps[0::2], ps[1::2])))
+        result = convMnistTwoS(x, list(zip(ps[0::2], ps[1::2])), layer)
         loss = lossSoftMaxCrossEntropyS(lab, result)
         return loss.host.srepl((), 1.0 / batch, dtype) * loss
 
@@ -211,7 +250,18 @@ def c3_cnn(batch=1000, dtype=F64, h=28, w=28, ksize=5, c_out=16, n_hidden=128, n
     dense = 2.0 * batch * flat * n_hidden
     ro = 2.0 * batch * n_hidden * n_classes
     flops = 2 * conv1 + 3 * conv2 + 3 * dense + 3 * ro
-    return Workload("c3_cnn", dtype, batch, params, [inp, labels], objective, flops=flops, bytes_=None)
+    wl = Workload("c3_cnn", dtype, batch, params, [inp, labels], objective, flops=flops, bytes_=None)
+    wl.objective_artifact = lambda ps, ds: objective(ps, ds, convMnistLayerArtifactS)
+    return wl
+
+
+def c3_cnn_artifact(**kw):
+    """The same network with relu and pooling written as the reference's derived programs
+    print them (gathers from [0.0, 1.0] by an `ifH` index, constant index tables)."""
+    wl = c3_cnn(**kw)
+    wl.name = "c3_cnn_artifact_form"
+    wl.objective = wl.objective_artifact
+    return wl
 
 
 def c4_rnn(batch=5000, dtype=F32, steps=28, n_in=28, width=128, n_classes=10):
@@ -266,3 +316,5 @@ def c4_rnn(batch=5000, dtype=F32, steps=28, n_in=28, width=128, n_classes=10):
 
 
 CONFIGS = {"c0": c0_elementwise, "c1": c1_fcnn, "c2": c2_wide, "c3": c3_cnn, "c4": c4_rnn}
+# the same work written another way: timed beside the configs, never the headline
+RIDERS = {"c3_artifact_form": c3_cnn_artifact}

@@ -113,6 +113,54 @@ def test_rnn_as_mapaccum_matches_unrolled(host_cpu):
         assert close(g2, g, 1e-5)
 
 
+def artifact_form(size):
+    mk, kw = (SMALL if size == "small" else MEDIUM)["c3"]
+    return W.c3_cnn_artifact(**kw)
+
+
+@pytest.mark.parametrize("table", ["get_api", "get_api_fused"])
+def test_cnn_in_the_reference_derived_form_matches(table):
+    """relu as a gather from [0.0, 1.0] by an `ifH` index over constant index tables and
+    pooling as a gather at kargMax (the form the reference's derived programs print,
+    test/simplified/TestMnistPP.hs:734-735): the value and gradient of the form written
+    with comparisons and conditionals, bit for bit, and numpy's.  On a table with the
+    composed entry points both convolution layers still go out as one call each."""
+    host = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_", api_table=table))
+    mk, kw = SMALL["c3"]
+    loss, grads = run(host, mk(**kw))
+    before = host.counter("contract_map")
+    wl = artifact_form("small")
+    aloss, agrads = run(host, wl)
+    assert aloss == loss
+    for g, a in zip(grads, agrads):
+        assert np.array_equal(g, a)
+    rloss, rgrads = ref.cnn(wl.params, *wl.data)
+    assert abs(aloss - rloss) <= 1e-11 * abs(rloss)
+    for a, r in zip(agrads, rgrads):
+        assert close(a, r, 1e-11)
+    assert host.counter("contract_map") - before == (2 if table == "get_api_fused" else 0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("size", ["small", "medium"])
+def test_gpu_cnn_in_the_reference_derived_form(host_gpu, host_cpu, size):
+    """The derived form on the device: equal to the checker within the fp64 tolerance, and
+    taking the same kernels as the other form (both convolution layers fused with relu and pooling)."""
+    wl = artifact_form(size)
+    before = host_gpu.counter("contract_map")
+    gl, gg = run(host_gpu, wl)
+    assert host_gpu.counter("contract_map") - before == 2
+    cl, cg = run(host_cpu, wl)
+    assert abs(gl - cl) <= 1e-10 * abs(cl)
+    for i, (g, c) in enumerate(zip(gg, cg)):
+        assert g.shape == c.shape and close(g, c, 1e-10), (size, i)
+    mk, kw = (SMALL if size == "small" else MEDIUM)["c3"]
+    pl, pg = run(host_gpu, mk(**kw))
+    assert pl == gl                       # the same kernels in the same order: the same bits
+    for g, p in zip(gg, pg):
+        assert np.array_equal(g, p)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("size", ["small", "medium"])
 @pytest.mark.parametrize("name", list(SMALL))
