@@ -54,7 +54,6 @@ def time_steps(host, wl, ps, ds, steps, warmup):
     t0 = time.perf_counter()
     for _ in range(steps):
         loss, grads = wl.gradient(host, ps, ds)
-        host.sync()
     host.sync()
     dt = time.perf_counter() - t0
     return dt / steps, float(loss.numpy())
@@ -70,9 +69,8 @@ def time_graph(host, wl, ps, ds, steps, warmup):
             host.sync()
         host.sync()
         t0 = time.perf_counter()
-        for _ in range(steps):
+        for _ in range(steps):       # the steps queue up on the one stream; the host waits once, after the last
             graph.launch()
-            host.sync()
         host.sync()
         dt = time.perf_counter() - t0
         return dt / steps, float(loss.numpy())
@@ -287,7 +285,12 @@ def main():
             sec, graph_loss = (eager_sec, loss) if args.eager else time_graph(host, wl, ps, ds, args.steps, args.warmup)
             if graph_loss != loss:
                 raise SystemExit(f"bench.py: {key}: the recorded program computed {graph_loss!r}, the eager one {loss!r}")
-            riders[key] = {"workload": wl.name, "batch": wl.batch, "ms_per_step": sec * 1e3, "loss": loss}
+            riders[key] = {"workload": wl.name, "batch": wl.batch, "ms_per_step": sec * 1e3, "ms_per_step_eager": eager_sec * 1e3, "loss": loss}
+            if wl.bytes:      # a chain of a few microseconds, timed by itself: launching a recorded graph costs more than its one or two kernels
+                best = min(sec, eager_sec)
+                riders[key]["us_per_call"] = best * 1e6
+                riders[key]["algorithmic_mb"] = wl.bytes / 1e6
+                riders[key]["achieved_gbs"] = wl.bytes / best / 1e9
             if "c3" in results and key.startswith("c3"):
                 riders[key]["ms_per_step_over_c3"] = sec * 1e3 / results["c3"]["ms_per_step"]
                 riders[key]["loss_equals_c3"] = loss == results["c3"]["loss"]

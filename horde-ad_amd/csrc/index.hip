@@ -93,6 +93,37 @@ __global__ void __launch_bounds__(kBlock) k_gather(IxSpace sp, Dims inner, int64
   }
 }
 
+// Slices that are contiguous in the table and a whole number of V-sized units
+// (16 bytes when sizes and strides allow): a lane moves one unit, so the lanes
+// of a slice read consecutive units of one place in the table, and the position
+// of a slice is resolved by each of its lanes from the same few index entries
+// (one cache line).  `units` = units per slice; tbl_unit = table element size /
+// sizeof(V) as a fraction num/den folded into the offsets by the caller:
+// table offsets arrive in elements and are scaled by es_over_v (elements per unit
+// inverted: unit offset = element offset / elems_per_unit, exact by the caller's checks).
+template <typename V>
+__global__ void __launch_bounds__(kBlock) k_gather_units(IxSpace sp, int64_t M, int64_t units, int64_t elems_per_unit, const V* __restrict__ src, V* __restrict__ out) {
+  const int64_t total = M * units;
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  const bool small = total < (int64_t)0x7fffffff;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += step) {
+    int64_t m, u;
+    if (small) {
+      const uint32_t q = (uint32_t)i / (uint32_t)units;
+      m = q;
+      u = (uint32_t)i - q * (uint32_t)units;
+    } else {
+      m = i / units;
+      u = i - m * units;
+    }
+    int64_t toff, doff;
+    const bool ok = resolve(sp, m, &toff, &doff);
+    V v{};
+    if (ok) v = src[toff / elems_per_unit + u];
+    out[i] = v;
+  }
+}
+
 // src is a view [M (position dims), N (inner dims)]; out dense [P, N], zeroed.
 // Distinct positions go to distinct places (the caller's promise): plain stores.
 template <typename T>
@@ -256,6 +287,27 @@ int hgpu_gather(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array
       label = ctx->label_pool.insert(buf).first->c_str();
     }
     LaunchGuard lg(ctx, label, 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, 0);
+    // contiguous slices of whole 16-byte (or 8-byte) units: one unit per lane
+    const int64_t es = (int64_t)dtype_size(src->dtype);
+    int unit = 0;
+    if (N > 1 && inner.nd == 1 && inner.st[0][0] == 1) {
+      for (int cand : {16, 8}) {
+        if (cand <= es || (N * es) % cand != 0 || ((uintptr_t)data_ptr(src)) % (uintptr_t)cand != 0) continue;
+        bool ok = true;
+        for (int k = 0; k < n_ix && ok; ++k) ok = (src->strides[k] * es) % cand == 0;
+        if (ok) { unit = cand; break; }
+      }
+    }
+    if (unit) {
+      const int64_t units = N * es / unit, epu = unit / es;
+      unsigned g = grid_for(M * units, kBlock, ctx->num_cu * 16);
+      if (unit == 16) hipLaunchKernelGGL(k_gather_units<uint4>, dim3(g), dim3(kBlock), 0, ctx->stream, sp, M, units, epu, (const uint4*)data_ptr(src), (uint4*)data_ptr(o));
+      else hipLaunchKernelGGL(k_gather_units<uint64_t>, dim3(g), dim3(kBlock), 0, ctx->stream, sp, M, units, epu, (const uint64_t*)data_ptr(src), (uint64_t*)data_ptr(o));
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "gather"); }
+      *out = o;
+      return HGPU_OK;
+    }
     unsigned g = grid_for(M * N, kBlock, ctx->num_cu * 8);
     switch (dtype_size(src->dtype)) {
       case 8: hipLaunchKernelGGL(k_gather<uint64_t>, dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, (const uint64_t*)data_ptr(src), (uint64_t*)data_ptr(o)); break;

@@ -154,6 +154,17 @@ int hh_graph_free(hh_ctx* c, hh_graph* g) {
 int hh_force(hh_ctx* c, hh_val* v) {
   return guarded(c, [&] { (void)v->d.primal.h(); });
 }
+int hh_dense(hh_ctx* c, hh_val* v, hh_val** out) {
+  if (!c || !v || !out) return HGPU_ERR_INVALID;
+  return guarded(c, [&] {
+    Backend* be = &c->be;
+    hgpu_array* a = v->d.primal.h();
+    if (be->api->is_dense(a)) { *out = box(d_const(v->d.primal)); return; }
+    hgpu_array* o = nullptr;
+    be->check(be->api->materialize(be->ctx, a, &o));
+    *out = box(d_const(T(be, o)));
+  });
+}
 int hh_overwrite(hh_ctx* c, hh_val* v, const void* host) {
   return guarded(c, [&] {
     if (!has_graphs(c->be.api)) throw HostError(HGPU_ERR_UNSUPPORTED, "this provider has no overwrite");

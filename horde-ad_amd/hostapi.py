@@ -36,7 +36,7 @@ SIG = {
     "ix_select": (I, [P, P, P, P, PP]), "ix_convert": (I, [P, P, I, I, PP]),
     "ix_index0": (I, [P, P, I, PP, PP]), "ix_argminmax": (I, [P, P, I, PP, I, PP]), "ix_free": (I, [P]),
     "ix_is_affine": (I, [P]), "counter": (L, [P, C.c_char_p]),
-    "tconvert": (I, [P, I, P, I, LP, PP]),
+    "tconvert": (I, [P, I, P, I, LP, PP]), "dense": (I, [P, P, PP]),
     "tsgather": (I, [P, P, I, LP, I, PP, PP]), "tsscatter": (I, [P, P, I, I, LP, PP, PP]),
     "capture_begin": (I, [P]), "capture_end": (I, [P, PP]), "graph_launch": (I, [P, P]), "graph_free": (I, [P, P]),
     "force": (I, [P, P]), "overwrite": (I, [P, P, P]), "assign": (I, [P, P, P]),
@@ -423,6 +423,10 @@ class V:
     def sindex(self, ix): return self._o(self.host.dll.hh_tsindex, self.h, len(ix), _larr(ix))   # `!$` with concrete indices
 
     # -- indexing with index functions
+    def dense(self):
+        """The primal part as a dense row-major array (a copy when the value is a strided view)."""
+        return self._o(self.host.dll.hh_dense, self.h)
+
     def sgather(self, shm, f):
         """sgather @shm self (\\[i...] -> [ix...])"""
         shm, ix = self.host._apply_index_fn(shm, f)

@@ -315,6 +315,46 @@ def c4_rnn(batch=5000, dtype=F32, steps=28, n_in=28, width=128, n_classes=10):
     return wl
 
 
+class Micro(Workload):
+    """A chain of operations timed by itself (the reference's bench/ConvVjpBench.hs groups
+    gather48 / scatter48): `gradient` evaluates the chain into a dense array and hands back
+    (one element of it, [the array]) in the places of the loss and the gradients."""
+
+    def __init__(self, name, dtype, data, chain, bytes_):
+        super().__init__(name, dtype, 1, [], data, None, flops=0.0, bytes_=bytes_)
+        self.chain = chain
+
+    def gradient(self, host, ps, ds):
+        out = self.chain(*ds).dense()
+        return out.sindex([0] * len(out.shape)), [out]
+
+
+def gather48(dtype=F64):
+    """twoAd of bench/ConvVjpBench.hs:429-439: the two-gather chain of a 48x48 im2col,
+    [50, 3, 3, 50] -> [48, 3, 3, 48, 3, 3] (186624 elements), big position dim first."""
+    x = uniform(42, (50, 3, 3, 50), -0.5, 0.5, dtype)
+
+    def chain(src):
+        g1 = src.sgather((48, 3), lambda a, b: [a + b])                                   # [48, 3, 3, 3, 50]
+        return g1.stranspose([4, 2, 0, 3, 1]).sgather((48, 3), lambda c, d: [c + d])       # [48, 3, 3, 48, 3, 3]
+
+    es = np.dtype(NP[dtype]).itemsize
+    return Micro("gather48_two_gather_chain", dtype, [x], chain, bytes_=(50 * 3 * 3 * 50 + 48 * 3 * 3 * 48 * 3 * 3) * es)
+
+
+def scatter48(dtype=F64):
+    """The adjoint of that chain (bench/ConvVjpBench.hs:586-700, checked there by checkAdjoint):
+    [48, 3, 3, 48, 3, 3] -> [50, 3, 3, 50] through two scatters with the gathers' index functions."""
+    y = uniform(43, (48, 3, 3, 48, 3, 3), -0.5, 0.5, dtype)
+
+    def chain(cot):
+        s2 = cot.sscatter(2, [50], lambda c, d: [c + d])                                    # [50, 3, 48, 3, 3]
+        return s2.stranspose([2, 4, 1, 3, 0]).sscatter(2, [50], lambda a, b: [a + b])       # [50, 3, 3, 50]
+
+    es = np.dtype(NP[dtype]).itemsize
+    return Micro("scatter48_two_scatter_chain", dtype, [y], chain, bytes_=(50 * 3 * 3 * 50 + 48 * 3 * 3 * 48 * 3 * 3) * es)
+
+
 CONFIGS = {"c0": c0_elementwise, "c1": c1_fcnn, "c2": c2_wide, "c3": c3_cnn, "c4": c4_rnn}
 # the same work written another way: timed beside the configs, never the headline
-RIDERS = {"c3_artifact_form": c3_cnn_artifact}
+RIDERS = {"c3_artifact_form": c3_cnn_artifact, "gather48": gather48, "scatter48": scatter48}

@@ -74,6 +74,12 @@ int hh_graph_launch(hh_ctx* ctx, hh_graph* g);
 int hh_graph_free(hh_ctx* ctx, hh_graph* g);
 int hh_force(hh_ctx* ctx, hh_val* v);
 int hh_overwrite(hh_ctx* ctx, hh_val* v, const void* host);
+/* The primal part of v as a dense row-major array: a copy when the value is a
+ * strided view (an affine gather, a transpose), v's own array otherwise.  The
+ * reference's Concrete backend copies in every gather (OpsConcrete.hs:1621-1665);
+ * here affine gathers are views, and this is where such a chain is written out
+ * when a caller wants the array itself (bench/ConvVjpBench.hs times exactly that). */
+int hh_dense(hh_ctx* ctx, hh_val* v, hh_val** out);
 /* dst's memory takes src's elements (same shape and type; dst an array made by
  * upload, src not a view of it): how a recorded training step hands the
  * updated parameters to its next launch. */

@@ -368,6 +368,31 @@ def test_gather_exact(both, dt):
     assert_same(both.gather(src, ix_arrays(both, [0, 3], [4]), [0, 3]))
 
 
+@pytest.mark.parametrize("dt", [np.float64, np.float32, np.int16, np.int8])
+def test_gather_of_wide_slices(both, dt):
+    """Slices that are contiguous in the table and whole 16-byte (or 8-byte) units go
+    out one unit per lane; indices outside the table read zeros; tables whose rows do
+    not start on a unit boundary (a sliced view, an odd row length) take the element
+    kernel.  Bit-exact against the checker and numpy either way."""
+    es = np.dtype(dt).itemsize
+    for rows, n, m in [(300, 256 // es, 5000), (300, 1024 // es, 700), (50, 24 // es, 999), (64, 40 // es + 1, 300)]:
+        t = rnd((rows, n), dt)
+        idx = RNG.integers(-3, rows + 3, m).astype(np.int64)        # some outside
+        got = both.gather(both.upload(t), [both.upload(idx)], [m])
+        assert_same(got, 0.0, (dt, rows, n, m))
+        ok = (idx >= 0) & (idx < rows)
+        want = np.where(ok[:, None], t[np.clip(idx, 0, rows - 1)], 0).astype(dt)
+        assert np.array_equal(got.numpy()[0], want)
+    # two indexed dims, slices of the last one; and a table that is a view with an offset
+    t = both.upload(rnd((12, 9, 32), dt))
+    i0, i1 = both.upload(RNG.integers(0, 12, (40, 3)).astype(np.int64)), both.upload(RNG.integers(0, 9, (40, 3)).astype(np.int64))
+    assert_same(both.gather(t, [i0, i1], [40, 3]), 0.0)
+    v = both.upload(rnd((20, 33), dt)).slice(1, 1, 32)                  # rows start 1 element in
+    assert_same(both.gather(v, [both.upload(RNG.integers(0, 20, 77).astype(np.int64))], [77]), 0.0)
+    w = both.upload(rnd((16, 30), dt)).transpose([1, 0])                # slices strided in memory
+    assert_same(both.gather(w, [both.upload(RNG.integers(0, 30, 50).astype(np.int64))], [50]), 0.0)
+
+
 @pytest.mark.parametrize("dt", [np.float64, np.float32, np.int64, np.int32])
 def test_scatter(both, dt):
     tol = TOL.get(np.dtype(dt), 0.0)

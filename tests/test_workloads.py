@@ -113,6 +113,39 @@ def test_rnn_as_mapaccum_matches_unrolled(host_cpu):
         assert close(g2, g, 1e-5)
 
 
+def im2col_chain_numpy(x):
+    """twoAd of bench/ConvVjpBench.hs:429-439 in numpy: [50, 3, 3, 50] -> [48, 3, 3, 48, 3, 3]."""
+    g1 = np.stack([np.stack([x[a + b] for b in range(3)]) for a in range(48)])           # [48, 3, 3, 3, 50]
+    t = g1.transpose(4, 2, 0, 3, 1)
+    return np.stack([np.stack([t[c + d] for d in range(3)]) for c in range(48)])          # [48, 3, 3, 48, 3, 3]
+
+
+def test_gather48_scatter48_chains(host_cpu):
+    """The reference's gather48 / scatter48 micro-benchmarks: the two-gather chain against
+    numpy, and the two-scatter chain as its adjoint, <gather x, y> = <x, scatter y>
+    (the check the reference makes at start-up, bench/ConvVjpBench.hs checkAdjoint)."""
+    g, s = W.gather48(), W.scatter48()
+    _, [out] = g.gradient(host_cpu, *g.upload(host_cpu))
+    x, y = g.data[0], s.data[0]
+    want = im2col_chain_numpy(x)
+    assert np.array_equal(out.numpy(), want)
+    _, [back] = s.gradient(host_cpu, *s.upload(host_cpu))
+    assert back.shape == x.shape
+    lhs, rhs = float(np.sum(want * y)), float(np.sum(x * back.numpy()))
+    assert abs(lhs - rhs) <= 1e-12 * abs(lhs)
+
+
+@pytest.mark.gpu
+def test_gpu_gather48_scatter48_chains(host_gpu, host_cpu):
+    for wl in (W.gather48(), W.scatter48()):
+        _, [got] = wl.gradient(host_gpu, *wl.upload(host_gpu))
+        _, [want] = wl.gradient(host_cpu, *wl.upload(host_cpu))
+        if wl.name.startswith("gather"):
+            assert np.array_equal(got.numpy(), want.numpy())
+        else:
+            assert close(got.numpy(), want.numpy(), 1e-12)
+
+
 def artifact_form(size):
     mk, kw = (SMALL if size == "small" else MEDIUM)["c3"]
     return W.c3_cnn_artifact(**kw)
