@@ -43,7 +43,7 @@ struct GemmParams {
   // within the term, and term t reads a_term[t] / b_term[t].  n_terms == 0: one
   // product, the operands are the kernel's pointer arguments.
   int n_terms, term_split;
-  int term_loop;           // staged kernel: every block walks all terms itself (k_gemm_terms)
+  int term_loop;           // staged kernel: every block walks all terms itself (k_gemm with LOOP)
   const void* a_term[kMaxTerms];
   const void* b_term[kMaxTerms];
   int c_rows_contig;       // staged kernel: the output is contiguous along m (and not along n)
@@ -309,7 +309,13 @@ __device__ __forceinline__ void k_loop(const GemmParams& p, const typename X::T*
 // VGPRs: they spill).
 constexpr int waves_wanted(int tm, int tn, int esize) { return tm * tn * esize <= 32 ? 2 : 1; }
 
-template <typename X, int WGM, int WGN, int TM, int TN, int VA, int VB, int NBUF>
+//
+// LOOP: a SUM of products of one layout whose tiles fill the device by
+// themselves -- every block walks all terms (GemmParams::a_term / b_term) and
+// adds them up in its accumulators, so there are no partial outputs and
+// blockIdx.y counts K chunks only.  Otherwise a block works on one term, which
+// its chunk index selects.
+template <typename X, int WGM, int WGN, int TM, int TN, int VA, int VB, int NBUF, bool LOOP = false>
 __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_wanted(TM, TN, (int)sizeof(typename X::T)), 8))) k_gemm(GemmParams p, const typename X::T* __restrict__ A, const typename X::T* __restrict__ B,
                                              typename X::T* __restrict__ C, const int64_t* __restrict__ koffA,
                                              const int64_t* __restrict__ koffB) {
@@ -345,11 +351,13 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
   int64_t bta, btb, btc;
   group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
   int sk = s;                              // chunk within its term
-  if (p.n_terms > 0) {
-    const int term = s / p.term_split;
-    sk = s - term * p.term_split;
-    A = (const T*)p.a_term[term];
-    B = (const T*)p.b_term[term];
+  if constexpr (!LOOP) {
+    if (p.n_terms > 0) {
+      const int term = s / p.term_split;
+      sk = s - term * p.term_split;
+      A = (const T*)p.a_term[term];
+      B = (const T*)p.b_term[term];
+    }
   }
   const int64_t kbeg = (int64_t)sk * p.kchunk;
   int64_t kend = kbeg + p.kchunk;
@@ -361,8 +369,15 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
 #pragma unroll
     for (int j = 0; j < TNB; ++j) acc[i][j] = X::zero();
 
-  if (p.kmask) k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, true>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
-  else k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, false>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
+  const int nterm = LOOP ? p.n_terms : 1;
+  for (int term = 0; term < nterm; ++term) {
+    if constexpr (LOOP) {
+      A = (const T*)p.a_term[term];
+      B = (const T*)p.b_term[term];
+    }
+    if (p.kmask) k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, true>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
+    else k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, false>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
+  }
 
   T* Cout = C + btc + (int64_t)s * p.c_split_stride;
   if constexpr (BN == 16 && BM >= 64) {
@@ -398,91 +413,6 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
       return;
     }
   }
-  int64_t coln[TNB];
-  bool colok[TNB];
-#pragma unroll
-  for (int j = 0; j < TNB; ++j) {
-    int64_t n = n0 + wn * TN * 16 + j * X::NBW + X::col(lane);
-    colok[j] = n < p.N;
-    int64_t oa = 0, ob = 0, oc = 0;
-    if (colok[j]) group_off(p.n, n, &oa, &ob, &oc);
-    coln[j] = oc;
-  }
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int r = 0; r < X::NR; ++r) {
-      int64_t m = m0 + (wm * TM + i) * 16 + X::row(lane, r);
-      if (m < p.M) {
-        int64_t oa, ob, oc;
-        group_off(p.m, m, &oa, &ob, &oc);
-#pragma unroll
-        for (int j = 0; j < TNB; ++j)
-          if (colok[j]) Cout[oc + coln[j]] = X::get(acc[i][j], r);
-      }
-    }
-  }
-}
-
-// The staged kernel for a SUM of products of one layout whose tiles fill the
-// device by themselves: every block walks all terms (GemmParams::a_term /
-// b_term) and adds them up in its accumulators, so there are no partial
-// outputs.  blockIdx.y counts K chunks only.
-template <typename X, int WGM, int WGN, int TM, int TN, int VA, int VB, int NBUF>
-__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_wanted(TM, TN, (int)sizeof(typename X::T)), 8))) k_gemm_terms(GemmParams p, const typename X::T* __restrict__ A, const typename X::T* __restrict__ B,
-                                             typename X::T* __restrict__ C, const int64_t* __restrict__ koffA,
-                                             const int64_t* __restrict__ koffB) {
-  using T = typename X::T;
-  using Acc = typename X::Acc;
-  constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
-  constexpr int TNB = TN * 16 / X::NBW;     // MFMA blocks per wavefront along n
-  static_assert(WGM * WGN == 4, "four wavefronts");
-  __shared__ T As[NBUF][BK][BM + 1];
-  __shared__ T Bs[NBUF][BK][BN + 1];
-
-  const int t = threadIdx.x;
-  const int lane = t & 63, wave = t >> 6;
-  const int wm = wave / WGN, wn = wave % WGN;
-
-  // XCD-aware numbering of (K chunk, tile): blocks b, b+8, b+16, ... of the
-  // grid's x-then-y order share an XCD and its L2.  Each XCD gets a contiguous
-  // range of the chunk-major order, so the tiles that read the same rows of A
-  // or B over the same K chunk run on one XCD and share those rows in its L2.
-  const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-  const int64_t ntiles = tiles_m * tiles_n;
-  const int64_t nblocks = ntiles * gridDim.y;
-  int64_t lin = blockIdx.x + ntiles * (int64_t)blockIdx.y;
-  if (nblocks >= 64) {
-    const int64_t x = lin & 7, per = nblocks >> 3, rem = nblocks & 7;
-    lin = x * per + (x < rem ? x : rem) + (lin >> 3);
-  }
-  const int s = (int)(lin / ntiles);
-  const int64_t bid = lin - s * ntiles;
-  const int64_t tile_m = bid / tiles_n, tile_n = bid - tile_m * tiles_n;
-  const int64_t m0 = tile_m * BM, n0 = tile_n * BN;
-
-  int64_t bta, btb, btc;
-  group_off(p.bt, blockIdx.z, &bta, &btb, &btc);
-  int sk = s;                              // chunk within its term
-  const int term0 = 0, nterm = p.n_terms;
-  const int64_t kbeg = (int64_t)sk * p.kchunk;
-  int64_t kend = kbeg + p.kchunk;
-  if (kend > p.K) kend = p.K;
-
-  Acc acc[TM][TNB];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TNB; ++j) acc[i][j] = X::zero();
-
-  for (int term = term0; term < term0 + nterm; ++term) {
-    A = (const T*)p.a_term[term];
-    B = (const T*)p.b_term[term];
-    if (p.kmask) k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, true>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
-    else k_loop<X, WGM, WGN, TM, TN, VA, VB, NBUF, false>(p, A + bta, B + btb, koffA, koffB, m0, n0, kbeg, kend, As, Bs, acc);
-  }
-
-  T* Cout = C + btc + (int64_t)s * p.c_split_stride;
   int64_t coln[TNB];
   bool colok[TNB];
 #pragma unroll
@@ -731,15 +661,15 @@ void launch_cfg(const GemmParams& p, const LaunchArgs& a) {
       constexpr bool CA = BM >= 64, CB = BN >= 64;
       const bool va = CA && a.va, vb = CB && a.vb;
       if constexpr (CA && CB) {
-        if (va && vb) { hipLaunchKernelGGL((k_gemm_terms<X, WGM, WGN, TM, TN, V, V, 1>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+        if (va && vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, V, 1, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
       }
       if constexpr (CA) {
-        if (va) { hipLaunchKernelGGL((k_gemm_terms<X, WGM, WGN, TM, TN, V, 1, 1>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+        if (va) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, 1, 1, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
       }
       if constexpr (CB) {
-        if (vb) { hipLaunchKernelGGL((k_gemm_terms<X, WGM, WGN, TM, TN, 1, V, 1>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+        if (vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, V, 1, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
       }
-      hipLaunchKernelGGL((k_gemm_terms<X, WGM, WGN, TM, TN, 1, 1, 1>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+      hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, 1, 1, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
       return;
     }
   }
