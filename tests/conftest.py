@@ -92,7 +92,19 @@ def assert_same(pair, rtol=0.0, what=""):
     else:
         scale = max(float(np.max(np.abs(o))) if o.size else 0.0, 1e-300)
         err = float(np.max(np.abs(g - o))) if o.size else 0.0
+        record_error(what, err / scale, rtol)
         assert err <= rtol * scale, (what, err / scale)
+
+
+def record_error(what, err, tol):
+    """With HORDEAD_TEST_ERRORS=<file>, every floating-point comparison appends the error it
+    measured and the bound it was held to (how the tolerances written in the tests were set)."""
+    path = os.environ.get("HORDEAD_TEST_ERRORS")
+    if path:
+        import inspect
+        fr = inspect.stack()[2]
+        with open(path, "a") as f:
+            f.write("%s:%d\t%s\t%.3e\t%.1e\n" % (os.path.basename(fr.filename), fr.lineno, str(what)[:60], err, tol))
 
 
 @pytest.fixture(scope="session")

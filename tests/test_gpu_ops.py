@@ -168,7 +168,7 @@ def test_binary_float(both, dt):
     x = rnd((4, 9), dt)
     px, py = both.upload(np.abs(x) + dt(0.5)), both.upload(np.abs(x[::-1]) + dt(0.5))
     assert_same(px.ewise2("pow", both.upload(x)), tol, "pow")
-    assert_same(px.ewise2("logbase", py), 100 * tol, "logbase")
+    assert_same(px.ewise2("logbase", py), tol, "logbase")
     # dense paths: dense*dense, dense*broadcast scalar, odd length
     a, b = both.upload(rnd((3001,), dt)), both.upload(rnd((3001,), dt))
     s = both.upload(dt(1.5)).replicate([3001])
@@ -292,10 +292,11 @@ def test_fused_sum_equals_program_then_sum(gpu, dt):
         ins = [gpu.upload(a), gpu.upload(b), gpu.upload(c).replicate(list(shape))]
         got = gpu.fused_sum(ins, prog, 5).numpy()
         acc = np.float64 if fp else np.int64
-        want = (np.sin(a.astype(acc) * b + c) if fp else np.abs(a.astype(acc) * b + c)).sum()
+        terms = np.sin(a.astype(acc) * b + c) if fp else np.abs(a.astype(acc) * b + c)
+        want = terms.sum()
         assert got.dtype == np.dtype(dt) and got.shape == ()
-        if fp:
-            assert np.isclose(got, want, rtol=TOL[np.dtype(dt)] * 10, atol=TOL[np.dtype(dt)] * max(1, a.size))
+        if fp:   # a sum is held to the tolerance relative to the sum of the magnitudes of its terms
+            assert abs(float(got) - float(want)) <= TOL[np.dtype(dt)] * float(np.abs(terms).sum())
         else:
             assert got == want
         assert np.isclose(float(gpu.fused_sum(ins, prog, 0).numpy()), float(a.astype(acc).sum()), rtol=1e-5)
@@ -450,14 +451,14 @@ def test_contract_sum(both, dt):
             a = both.upload(rnd((m, k), dt)).replicate([n]).transpose([1, 0, 2])      # [m, n, k]
             b = both.upload(rnd((k, n), dt)).transpose([1, 0]).replicate([m])          # [m, n, k], K strided
             pairs.append((a, b))
-        assert_same(both.contract_sum(pairs, 2), tol * 4, (m, n, k, terms))
+        assert_same(both.contract_sum(pairs, 2), tol, (m, n, k, terms))
     # terms of different layouts: term by term
     a1 = both.upload(rnd((40, 30, 50), dt))
     b1 = both.upload(rnd((40, 30, 50), dt))
     a2 = both.upload(rnd((30, 40, 50), dt)).transpose([1, 0, 2])
     b2 = both.upload(rnd((40, 30, 50), dt))
-    assert_same(both.contract_sum([(a1, b1), (a2, b2)], 2), tol * 4)
-    assert_same(both.contract_sum([(a1, b1)], 1), tol * 4)
+    assert_same(both.contract_sum([(a1, b1), (a2, b2)], 2), tol)
+    assert_same(both.contract_sum([(a1, b1)], 1), tol)
     # terms of one layout that are no matrix product (row-wise dots: bias gradients
     # of an unrolled recurrence): one grouped reduction
     for shape, keep, perm in [((128, 700), 1, None), ((128, 700), 0, None), ((300, 40), 1, [1, 0]), ((6, 5, 64), 2, None), ((3000, 8), 1, None)]:
@@ -467,7 +468,7 @@ def test_contract_sum(both, dt):
             if perm:
                 a, b = a.transpose(perm), b.transpose(perm)
             pairs.append((a, b))
-        assert_same(both.contract_sum(pairs, keep), tol * 4, (shape, keep, perm))
+        assert_same(both.contract_sum(pairs, keep), tol, (shape, keep, perm))
     # two layouts interleaved, one of them with a replicated (stride 0) operand:
     # each layout is one grouped launch
     pairs = []
@@ -478,7 +479,7 @@ def test_contract_sum(both, dt):
         else:
             b = both.upload(rnd((700, 96), dt)).transpose([1, 0]).replicate([128])
         pairs.append((a, b))
-    assert_same(both.contract_sum(pairs, 2), tol * 4)
+    assert_same(both.contract_sum(pairs, 2), tol)
 
 
 def test_scatter_small_ints(both, gpu):
@@ -563,7 +564,7 @@ def test_contract_on_the_matrix_cores(both, gpu, dt):
     # long K with a small output: split along K
     a, b = both.upload(rnd((24, 40000), dt)), both.upload(rnd((40000, 20), dt))
     lhs, rhs = matmul_views(a, b)
-    assert_same(lhs.contract(rhs, 2), 10 * tol, "split-K")
+    assert_same(lhs.contract(rhs, 2), tol, "split-K")
     # a batch dim on both operands
     x, y = both.upload(rnd((5, 40, 30), dt)), both.upload(rnd((5, 30, 50), dt))
     lhs = x.replicate([50]).transpose([1, 2, 0])            # [5, 40, 50, 30]
@@ -623,7 +624,7 @@ def test_staged_products_at_the_edges_of_their_tiles(both, dt):
     # K chunks that end inside a K step, partial sums
     a, b = both.upload(rnd((64, 20008), dt)), both.upload(rnd((48, 20008), dt))
     lhs, rhs = nt_views(a, b)
-    assert_same(lhs.contract(rhs, 2), 10 * tol, "split-K, ragged chunks")
+    assert_same(lhs.contract(rhs, 2), tol, "split-K, ragged chunks")
 
 
 def conv_views(both, dt, b, ci, h, w, co, kh, kw):
@@ -654,7 +655,7 @@ def test_conv_contractions_from_lds_footprints(both, gpu, dt, shape):
     over window views, at batch sizes where a block keeps one image's footprint
     of each operand in LDS."""
     b, ci, h, w, co, kh, kw = shape
-    tol = TOL[np.dtype(dt)] * 20
+    tol = TOL[np.dtype(dt)]
     win, ker, dout = conv_views(both, dt, b, ci, h, w, co, kh, kw)
     gpu.check(gpu.lib.profile_enable(gpu.h, 2))     # kernel names with shapes
     gpu.profile_report()

@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 
 import ref_numpy as ref
-from conftest import capi, entry, pkg
+from conftest import capi, entry, pkg, record_error
 
 H, W = pkg.hostapi, pkg.workloads
 
@@ -206,6 +206,7 @@ def test_gpu_matches_checker(host_gpu, host_cpu, name, size):
     assert abs(gl - cl) <= tol * abs(cl), (gl, cl)
     for i, (g, c) in enumerate(zip(gg, cg)):
         assert g.shape == c.shape and g.dtype == c.dtype
+        record_error("%s %s gradient %d" % (name, size, i), float(np.max(np.abs(g - c))) / max(float(np.max(np.abs(c))), 1e-300), tol)
         assert close(g, c, tol), (name, size, i, float(np.max(np.abs(g - c))) / max(float(np.max(np.abs(c))), 1e-300))
 
 
@@ -249,12 +250,15 @@ def test_gpu_full_size_matches_numpy(host_gpu, name):
     if wl.dtype == capi.F32:
         # A relu whose argument rounds to the other side of zero changes a whole
         # gradient term, so at these sizes single precision itself sits further than
-        # 1e-5 from the double-precision gradients: numpy's own fp32 evaluation of
-        # the same formulas measures that distance, and the device may be at most
-        # twice as far.
+        # 1e-5 from the double-precision gradients (the wide relu network: 5.5e-4,
+        # 2.8e-4, 1.7e-4, 1.4e-4 for its four big arrays; the tanh recurrence stays
+        # within 4e-7).  numpy's own fp32 evaluation of the same formulas measures
+        # that distance, and the device may be at most a quarter further away
+        # (measured: 0.99, 1.03, 0.98, 0.89 of numpy's distance).
         _, sgrads = reference(wl.params, wl.data)
-        tols = [max(tol, 2 * err(s.astype(np.float64), r)) for s, r in zip(sgrads, rgrads)]
+        tols = [max(tol, 1.25 * err(s.astype(np.float64), r)) for s, r in zip(sgrads, rgrads)]
     assert abs(loss - rloss) <= tol * abs(rloss), (loss, rloss)
     for i, (g, r) in enumerate(zip(grads, rgrads)):
         assert g.shape == r.shape
+        record_error("full size %s gradient %d" % (name, i), err(g.astype(np.float64), r), tols[i])
         assert err(g.astype(np.float64), r) <= tols[i], (name, i, err(g.astype(np.float64), r), tols[i])
