@@ -26,6 +26,7 @@
 // L2 sees neighbouring rows of A.  Small outputs with long K are split along K
 // into partial products summed by a second launch (fixed order: reproducible).
 #include <algorithm>
+#include <cmath>
 
 #include "gemm_kernel.hpp"
 
@@ -423,6 +424,28 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     // fewer tiles than CUs: two K halves per tile keep every CU busy, and the
     // second pass over the output costs less than the idle quarter of the device
     if (split == 1 && tiles * p.BT * nt < ctx->num_cu && p.K >= 16 * BK) split = 2;
+    // A few more chunks when they fill the last round of blocks: with `per_cu`
+    // blocks resident on a CU, blocks run in rounds of num_cu * per_cu, and a
+    // round that is three quarters empty costs as much as a full one.  (300 x 784
+    // over K 5000 in 64 x 128 tiles: 11 chunks = 385 blocks take 82 us, 14 chunks
+    // = 490 blocks 70 us, 15 chunks = 525 blocks 94 us.)
+    if (split > 1) {
+      const double slots = (double)ctx->num_cu * per_cu;
+      auto fill = [&](int cand) {
+        const double blocks = (double)tiles * p.BT * nt * cand;
+        return blocks / (std::ceil(blocks / slots) * slots);
+      };
+      int best_s = split;
+      double best_fill = fill(split);
+      const int hi = (int)std::min<int64_t>(max_split, split + (split * 3 + 9) / 10);
+      for (int cand = split + 1; cand <= hi; ++cand)
+        if (fill(cand) > best_fill + 0.1) { best_fill = fill(cand); best_s = cand; }
+      split = best_s;
+    }
+  }
+  if (const char* e = getenv("HORDEAD_GEMM_SPLIT")) {   // for measurements
+    int v = atoi(e);
+    if (v >= 1 && v <= p.K / BK) split = v;
   }
   p.kchunk = ((p.K + split - 1) / split + BK - 1) / BK * BK;
   p.term_split = (int)((p.K + p.kchunk - 1) / p.kchunk);
