@@ -17,6 +17,7 @@
 // the host has checked contiguity and alignment.
 #pragma once
 #include "common.hpp"
+#include <type_traits>
 
 namespace hg {
 namespace gemm {
@@ -71,13 +72,14 @@ __device__ __forceinline__ void group_off(const Group& g, int64_t lin, int64_t* 
   *oc = c;
 }
 
-// MFMA flavours.  A fragment: lane l supplies A[row = l % 16][k = l / 16].
-// B fragment: lane l supplies B[k = l / 16][col = bcol(l)].  Accumulator
-// register r of lane l holds D[row(l, r)][col(l)] of an (16 x NBW) block.
+// MFMA flavours.  One instruction multiplies a BMR x KI block of A by a KI x NBW
+// block of B.  A fragment: lane l supplies A[row = l % BMR][k = l / BMR].
+// B fragment: lane l supplies B[k = l / NBW][col = bcol(l)].  Accumulator
+// register r of lane l holds D[row(l, r)][col(l)] of a (BMR x NBW) block.
 struct MfmaF32 {
   using T = float;
   using Acc = __attribute__((ext_vector_type(4))) float;
-  static constexpr int NBW = 16, NR = 4;
+  static constexpr int NBW = 16, NR = 4, BMR = 16, KI = 4;
   static __device__ __forceinline__ Acc zero() { return Acc{0, 0, 0, 0}; }
   static __device__ __forceinline__ Acc run(T a, T b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
   static __device__ __forceinline__ int bcol(int l) { return l & 15; }
@@ -85,10 +87,24 @@ struct MfmaF32 {
   static __device__ __forceinline__ int col(int l) { return l & 15; }
   static __device__ __forceinline__ T get(const Acc& c, int r) { return c[r]; }
 };
+// v_mfma_f32_32x32x2_f32: the instruction stream of 32 x 32 blocks sustains
+// nearly the published fp32 rate where that of 16 x 16 x 4 blocks stays near
+// 0.8 of it (hgpu_mfma_probe measures both); same LDS reads per flop.
+struct MfmaF32W {
+  using T = float;
+  using Acc = __attribute__((ext_vector_type(16))) float;
+  static constexpr int NBW = 32, NR = 16, BMR = 32, KI = 2;
+  static __device__ __forceinline__ Acc zero() { return Acc{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}; }
+  static __device__ __forceinline__ Acc run(T a, T b, Acc c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int bcol(int l) { return l & 31; }
+  static __device__ __forceinline__ int row(int l, int r) { return 8 * (r >> 2) + 4 * (l >> 5) + (r & 3); }
+  static __device__ __forceinline__ int col(int l) { return l & 31; }
+  static __device__ __forceinline__ T get(const Acc& c, int r) { return c[r]; }
+};
 struct MfmaF64 {
   using T = double;
   using Acc = __attribute__((ext_vector_type(4))) double;
-  static constexpr int NBW = 16, NR = 4;
+  static constexpr int NBW = 16, NR = 4, BMR = 16, KI = 4;
   static __device__ __forceinline__ Acc zero() { return Acc{0, 0, 0, 0}; }
   static __device__ __forceinline__ Acc run(T a, T b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
   static __device__ __forceinline__ int bcol(int l) { return l & 15; }
@@ -247,7 +263,7 @@ __device__ __forceinline__ void k_loop(const GemmParams& p, const typename X::T*
                                        typename X::Acc (*acc)[TN * 16 / X::NBW]) {
   using T = typename X::T;
   constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
-  constexpr int TNB = TN * 16 / X::NBW;
+  constexpr int TNB = TN * 16 / X::NBW, TMB = TM * 16 / X::BMR;
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;
   const int wm = wave / WGN, wn = wave % WGN;
@@ -279,15 +295,15 @@ __device__ __forceinline__ void k_loop(const GemmParams& p, const typename X::T*
       sb.advance(kob, k0 + 2 * BK);
     }
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 4) {
-      const int kr = kk + (lane >> 4);
-      T fa[TM], fb[TNB];
+    for (int kk = 0; kk < BK; kk += X::KI) {
+      const int kr = kk + lane / X::BMR;
+      T fa[TMB], fb[TNB];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) fa[i] = As[cur][kr][(wm * TM + i) * 16 + (lane & 15)];
+      for (int i = 0; i < TMB; ++i) fa[i] = As[cur][kr][wm * TM * 16 + i * X::BMR + (lane & (X::BMR - 1))];
 #pragma unroll
       for (int j = 0; j < TNB; ++j) fb[j] = Bs[cur][kr][wn * TN * 16 + j * X::NBW + X::bcol(lane)];
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TMB; ++i)
 #pragma unroll
         for (int j = 0; j < TNB; ++j) acc[i][j] = X::run(fa[i], fb[j], acc[i][j]);
     }
@@ -323,6 +339,8 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
   using Acc = typename X::Acc;
   constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
   constexpr int TNB = TN * 16 / X::NBW;     // MFMA blocks per wavefront along n
+  constexpr int TMB = TM * 16 / X::BMR;     // and along m
+  static_assert(TMB * X::BMR == TM * 16 && TNB * X::NBW == TN * 16, "whole MFMA blocks per wavefront");
   static_assert(WGM * WGN == 4, "four wavefronts");
   __shared__ T As[NBUF][BK][BM + 1];
   __shared__ T Bs[NBUF][BK][BN + 1];
@@ -363,9 +381,9 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
   int64_t kend = kbeg + p.kchunk;
   if (kend > p.K) kend = p.K;
 
-  Acc acc[TM][TNB];
+  Acc acc[TMB][TNB];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TMB; ++i)
 #pragma unroll
     for (int j = 0; j < TNB; ++j) acc[i][j] = X::zero();
 
@@ -388,9 +406,9 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
       T (*Cs)[BM + 1] = As[0];
       __shared__ int64_t ccol[16];
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TMB; ++i)
 #pragma unroll
-        for (int r = 0; r < X::NR; ++r) Cs[X::col(lane)][(wm * TM + i) * 16 + X::row(lane, r)] = X::get(acc[i][0], r);
+        for (int r = 0; r < X::NR; ++r) Cs[X::col(lane)][wm * TM * 16 + i * X::BMR + X::row(lane, r)] = X::get(acc[i][0], r);
       if (t < 16) {
         int64_t n = n0 + t;
         int64_t oa = 0, ob = 0, oc = 0;
@@ -424,10 +442,10 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
     coln[j] = oc;
   }
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  for (int i = 0; i < TMB; ++i) {
 #pragma unroll
     for (int r = 0; r < X::NR; ++r) {
-      int64_t m = m0 + (wm * TM + i) * 16 + X::row(lane, r);
+      int64_t m = m0 + wm * TM * 16 + i * X::BMR + X::row(lane, r);
       if (m < p.M) {
         int64_t oa, ob, oc;
         group_off(p.m, m, &oa, &ob, &oc);
@@ -645,8 +663,16 @@ struct LaunchArgs {
 // (small products whose tiles fill the device).
 constexpr bool term_loop_tile(int wgm, int wgn, int tm, int tn) { return wgm * tm * 16 * wgn * tn * 16 <= 64 * 64; }
 
-template <typename X, int WGM, int WGN, int TM, int TN>
+// The MFMA flavour a tile runs on: fp32 tiles whose wavefronts hold whole
+// 32 x 32 blocks take the 32x32x2 instruction.
+template <typename X0, int TM, int TN> struct FlavourOf { using type = X0; };
+template <int TM, int TN> struct FlavourOf<MfmaF32, TM, TN> {
+  using type = typename std::conditional<TM % 2 == 0 && TN % 2 == 0, MfmaF32W, MfmaF32>::type;
+};
+
+template <typename X0, int WGM, int WGN, int TM, int TN>
 void launch_cfg(const GemmParams& p, const LaunchArgs& a) {
+  using X = typename FlavourOf<X0, TM, TN>::type;
   using T = typename X::T;
   constexpr int V = 16 / sizeof(T);
   constexpr int BM = WGM * TM * 16, BN = WGN * TN * 16;
