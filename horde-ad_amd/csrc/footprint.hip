@@ -236,6 +236,14 @@ constexpr int NLD = MODE == 0 ? NLX + NLY : NLX;        // loads per thread and 
 constexpr int PH = NG >= 12 ? 3 : 1;                    // prefetch phases
 constexpr int LPP = (NLD + PH - 1) / PH;
 constexpr int BUF = MODE == 0 ? LX + LY : LX;           // elements per chunk buffer
+// split row blocks: slots whose turn comes before K group g (slot s runs after group min(4 s + 3, NG - 1))
+constexpr int rem_slots_before(int g) {
+  int c = 0;
+  for (int sl = 0; sl < NSLOT; ++sl) c += (sl == NSLOT - 1 ? NG - 1 : 4 * sl + 3) < g ? 1 : 0;
+  return c;
+}
+constexpr int RGB = REM > 0 ? (4 / REM > 1 ? 4 / REM : 1) : 1;     // slots per batch of LDS reads
+struct RemOps { T a[RGB][REM > 0 ? REM : 1], b[RGB][REM > 0 ? REM : 1]; };
 constexpr int RED0 = NBUFS * BUF + (MODE == 0 ? 0 : LY);    // scratch for adding up split row blocks
 constexpr int LDS_ELEMS = RED0 + (REM > 0 ? REM * 4 * 256 : 0);
 
@@ -375,10 +383,10 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   // j-th staging vector of this thread; the tail repeats the last vector.  The last vector of a footprint may reach up to
   // VX - 1 elements past it: still inside the operand's block, which the allocator ends with 16 spare bytes.
   auto vidx = [&](int j) -> int { int v = tid + 256 * (j < NLX ? j : j - NLX); int lim = (j < NLX ? XV : YV) - 1; return v < lim ? v : lim; };
-  // The first chunk, and the columns operand of mode 1, go to LDS eight vectors
-  // at a time: eight loads in flight, then eight stores.  Copied one by one,
-  // every vector would wait out its own trip to memory.
-  constexpr int kFill = 8;
+  // The first chunk, and the columns operand of mode 1, go to LDS up to 32
+  // vectors at a time: the loads in flight together, then the stores.  Copied
+  // one by one, every vector would wait out its own trip to memory.
+  constexpr int kFill = NLD < 32 ? (NLD > 0 ? NLD : 1) : 32;
 #if VIRT_X
   VPre_x vpx[NLX];
 #pragma unroll
@@ -482,7 +490,55 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
           self(self, IC<gi + 1>{});
         }
       };
-      groups(groups, IC<g0>{});
+      if constexpr (NBF == 0 && REM > 0) {
+        // Nothing but split row blocks: every multiplication has LDS operands of
+        // its own.  They are read a batch of slots ahead of the batch being
+        // multiplied (the fences keep the compiler from sinking each read to
+        // its use, where every MFMA would wait out a trip to LDS).
+        constexpr int S0 = rem_slots_before(g0), S1 = rem_slots_before(g1);
+        auto rem_load = [&](auto SI) {
+          constexpr int sb = decltype(SI)::v;
+          RemOps o;
+#pragma unroll
+          for (int u = 0; u < RGB; ++u)
+#pragma unroll
+            for (int rb = 0; rb < REM; ++rb) {
+              const int sl = sb + u < S1 ? sb + u : S1 - 1;
+              o.a[u][rb] = L[remx[rb * NSLOT + sl]];
+              o.b[u][rb] = LYp[remy[rb * NSLOT + sl]];
+            }
+          return o;
+        };
+        auto rem_run = [&](auto self, auto SI, const RemOps& cur) -> void {
+          constexpr int sb = decltype(SI)::v;
+          if constexpr (sb < S1) {
+            constexpr int sn = sb + RGB;
+            RemOps nxt;
+            if constexpr (sn < S1) nxt = rem_load(IC<sn>{});
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < RGB; ++u) {
+              if (sb + u < S1) {
+#pragma unroll
+                for (int rb = 0; rb < REM; ++rb) {
+                  const int sl = sb + u;
+                  const int g2 = 4 * sl + ((wave + rb) & 3);
+                  if (sl < NSLOT - 1 || g2 < NG) {
+                    T a2 = cur.a[u][rb], b2 = cur.b[u][rb];
+                    if (KVALID < 4 && g2 == NG - 1 && tail_lane) { a2 = T(0); b2 = T(0); }
+                    acc[NBF + rb] = MFMA(a2, b2, acc[NBF + rb]);
+                  }
+                }
+              }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (sn < S1) self(self, IC<sn>{}, nxt);
+          }
+        };
+        if constexpr (S0 < S1) rem_run(rem_run, IC<S0>{}, rem_load(IC<S0>{}));
+      } else {
+        groups(groups, IC<g0>{});
+      }
       if (NBUFS == 2) {
 #pragma unroll
         for (int j = 0; j < LPP; ++j) {

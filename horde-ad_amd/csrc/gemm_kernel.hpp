@@ -408,7 +408,9 @@ __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(waves_w
 #pragma unroll
       for (int i = 0; i < TMB; ++i)
 #pragma unroll
-        for (int r = 0; r < X::NR; ++r) Cs[X::col(lane)][wm * TM * 16 + i * X::BMR + X::row(lane, r)] = X::get(acc[i][0], r);
+        for (int j = 0; j < TNB; ++j)
+#pragma unroll
+          for (int r = 0; r < X::NR; ++r) Cs[j * X::NBW + X::col(lane)][wm * TM * 16 + i * X::BMR + X::row(lane, r)] = X::get(acc[i][j], r);
       if (t < 16) {
         int64_t n = n0 + t;
         int64_t oa = 0, ob = 0, oc = 0;

@@ -2092,11 +2092,8 @@ static bool contract_map_extremum(Backend* be, const T& inner, int n_reduce, boo
   const hgpu_api* api = be->api;
   if (!(api->struct_size >= offsetof(hgpu_api, contract_map) + sizeof(api->contract_map) && api->contract_map)) return false;
   const ArrHolder* ih = inner.holder().get();
-  static const bool dbg = getenv("HORDEAD_HOST_DEBUG") != nullptr;
-  if (dbg) fprintf(stderr, "contract_map_extremum: vsrc %d offset %lld shape_eq %d\n", (int)(bool)ih->vsrc, (long long)ih->vmeta.offset, (int)(ih->vmeta.shape == inner.shape()));
   if (!ih->vsrc || ih->vmeta.offset != 0 || ih->vmeta.shape != inner.shape()) return false;
   T origin(ih->vsrc);
-  if (dbg) fprintf(stderr, "  origin pending_expr %d size %d\n", (int)origin.pending_expr(), pending_size(origin.holder()));
   if (!origin.pending_expr() || pending_size(origin.holder()) > 40) return false;
   // is there exactly one pending contraction among the leaves?  (look before anything is forced)
   {
@@ -2114,7 +2111,6 @@ static bool contract_map_extremum(Backend* be, const T& inner, int n_reduce, boo
       if (p->fb) stack.push_back(p->fb.get());
       if (p->fc) stack.push_back(p->fc.get());
     }
-    if (dbg) fprintf(stderr, "  contractions among the leaves: %d\n", n_contr);
     if (n_contr != 1) return false;
   }
   std::vector<const hgpu_array*> ins;
