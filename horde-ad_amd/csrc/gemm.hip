@@ -374,7 +374,7 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     int rc = try_footprint(ctx, p, a->dtype, pa, pb, out, handled);
     if (rc || *handled) return rc;
   }
-  if (p.K <= 512 && p.BT == 1) {   // the whole contracted dim in LDS: no K loop, no K table
+  if ((p.K <= 512 || (p.K <= 1024 && p.M * p.N <= 160000)) && p.BT == 1) {   // the whole contracted dim in LDS: no K loop, no K table
     const hgpu_array* const* ta = n_terms > 0 ? as : &a;
     const hgpu_array* const* tb = n_terms > 0 ? bs : &b;
     const hgpu_array* none = nullptr;

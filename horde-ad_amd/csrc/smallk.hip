@@ -55,7 +55,9 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
 namespace {
 
 constexpr int kMaxTermsSmallK = 4;
-constexpr int64_t kMaxKTotal = 512;
+constexpr int64_t kMaxKTotal = 512;        // contracted elements of all terms together ...
+constexpr int64_t kMaxKSmallOut = 1024;    // ... and when the result is small (a staged product would split K to fill the device and add partial results)
+constexpr int64_t kSmallOut = 160000;
 
 struct Compiled {
   hipModule_t mod;
@@ -490,7 +492,7 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
     ktot += tm.K;
     sp.terms.push_back(tm);
   }
-  if (ktot < 4 || ktot > kMaxKTotal) return HGPU_OK;
+  if (ktot < 4 || ktot > (sp.P * sp.Q <= kSmallOut ? kMaxKSmallOut : kMaxKTotal)) return HGPU_OK;
   if (sp.P < 16 || sp.Q < 4 || (double)sp.P * sp.Q * ktot < 2.0e6) return HGPU_OK;
   for (int o = 0; o < n_out; ++o) {
     if (out_slots[o] < n_in && out_slots[o] != c_slot) return HGPU_OK;   // a copy of an input: not this kernel's business

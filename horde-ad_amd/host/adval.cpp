@@ -116,12 +116,15 @@ D d_ewise2(Tape& tp, int op, const D& a, const D& b) {
     case HGPU_SUB:
       r.node = tp.push([an, bn](const T& c, std::vector<T>& s) { accum(s, an, c); if (bn >= 0) accum(s, bn, neg(c)); });
       break;
-    case HGPU_MUL:
-      r.node = tp.push([an, bn, u, v](const T& c, std::vector<T>& s) {
-        if (an >= 0) accum(s, an, mul(v, c));
-        if (bn >= 0) accum(s, bn, mul(u, c));
+    case HGPU_MUL: {
+      // a factor is kept only for the other side's cotangent
+      const T ku = bn >= 0 ? u : T(), kv = an >= 0 ? v : T();
+      r.node = tp.push([an, bn, ku, kv](const T& c, std::vector<T>& s) {
+        if (an >= 0) accum(s, an, mul(kv, c));
+        if (bn >= 0) accum(s, bn, mul(ku, c));
       });
       break;
+    }
     case HGPU_DIV:  // dAdd (dScale (recip v) u') (dScale ((-u) / (v*v)) v')
       r.node = tp.push([an, bn, u, v](const T& c, std::vector<T>& s) {
         if (an >= 0) accum(s, an, mul(recip(v), c));

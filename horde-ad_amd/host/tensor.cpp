@@ -545,7 +545,34 @@ static bool products_then_program(Backend* be, const std::vector<ArrHolder*>& ro
   for (auto& m : kept->more) { fas.push_back(T(m.first)); fbs.push_back(T(m.second)); }
   std::vector<const hgpu_array*> ah, bh;
   for (size_t t = 0; t < fas.size(); ++t) { ah.push_back(fas[t].h()); bh.push_back(fbs[t].h()); }
+  // An inner node of the program that contains the products and that someone
+  // outside still holds (the condition of a select, kept for the reverse pass)
+  // would later be computed again, products and all: it is one more result of
+  // the same call.  (Inner nodes without the products are cheap to redo.)
+  std::vector<std::pair<ArrHolder*, int>> promoted;   // node, its slot
+  {
+    std::map<const ArrHolder*, bool> has_products;     // instructions come children first
+    has_products[kept] = true;
+    for (size_t i = 0; i < nodes.size(); ++i) {
+      ArrHolder* nd = nodes[i];
+      bool hp = false;
+      for (auto* f : {&nd->fa, &nd->fb, &nd->fc})
+        if (*f) { auto it = has_products.find(f->get()); hp = hp || (it != has_products.end() && it->second); }
+      has_products[nd] = hp;
+      if (!hp || std::find(roots.begin(), roots.end(), nd) != roots.end()) continue;
+      std::shared_ptr<ArrHolder> sp;
+      long in = 0;
+      for (auto* q : nodes)
+        for (auto* f : {&q->fa, &q->fb, &q->fc})
+          if (f->get() == nd) { sp = *f; ++in; }
+      if (sp && sp.use_count() - 1 > in && roots.size() + promoted.size() < 6) {
+        promoted.push_back({nd, (int)ins.size() + (int)i});
+        has_products[nd] = false;     // written: what is built on it can be redone from the array
+      }
+    }
+  }
   std::vector<int> out_slots(slots);
+  for (auto& pr : promoted) out_slots.push_back(pr.second);
   if (shared) out_slots.push_back(c_slot);
   std::vector<hgpu_array*> res(out_slots.size(), nullptr);
   int rc = api->contract_sum_map(be->ctx, (int)ah.size(), ah.data(), bh.data(), kept->keep, (int)ins.size(), ins.data(), (int)prog.size(), prog.data(), (int)out_slots.size(),
@@ -554,6 +581,16 @@ static bool products_then_program(Backend* be, const std::vector<ArrHolder*>& ro
   be->check(rc);
   be->counters["contract_sum_map"]++;
   for (size_t i = 0; i < roots.size(); ++i) (*outs)[i] = res[i];
+  for (size_t j = 0; j < promoted.size(); ++j) {
+    ArrHolder* nd = promoted[j].first;
+    nd->h = res[roots.size() + j];
+    nd->fa.reset();
+    nd->fb.reset();
+    nd->fc.reset();
+    nd->vsrc.reset();
+    nd->ekind = -1;
+    be->counters["contract_sum_map_kept_nodes"]++;
+  }
   if (shared) {
     kept->h = res.back();
     kept->fa.reset();

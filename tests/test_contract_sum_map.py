@@ -59,7 +59,11 @@ SHAPES = [
     (np.float64, 10, 999, [30], ["mk"]),                    # odd extent: no vectors along n, k padded to 32
     (np.float32, 10, 998, [27], ["mk"]),                    # k neither a multiple of 4 nor contiguous vectors
     (np.float32, 40, 1004, [8, 12, 16, 20], ["mk", "km", "mk", "km"]),
-    (np.float32, 128, 1000, [600], ["mk"]),                 # too long for the kernel: the entry points one after another
+    (np.float32, 128, 1000, [600], ["mk"]),                 # up to 1024 contracted elements when the result is small ...
+    (np.float64, 128, 1000, [784], ["mk"]),                 # ... (a dense layer over a flattened image: 13 chunks)
+    (np.float64, 128, 784, [1000], ["km"]),                 # its weight gradient: 16 chunks
+    (np.float32, 128, 1000, [1100], ["mk"]),                # too long for the kernel: the entry points one after another
+    (np.float32, 300, 1000, [600], ["mk"]),                 # too long for a result of this size
     (np.float32, 6, 20, [5], ["mk"]),                       # too small for it
 ]
 
@@ -67,7 +71,7 @@ SHAPES = [
 @pytest.mark.gpu
 @pytest.mark.parametrize("dt,m,n,ks,layouts", SHAPES)
 def test_layer_matches_checker_and_numpy(gpu, oracle, dt, m, n, ks, layouts):
-    one_kernel = sum(ks) <= 512 and m * n * sum(ks) >= 2e6      # what the compiled kernel covers
+    one_kernel = sum(ks) <= (1024 if m * n <= 160000 else 512) and m * n * sum(ks) >= 2e6      # what the compiled kernel covers
     for bias in (True, False):
         gpu.check(gpu.lib.profile_enable(gpu.h, 2))
         state = RNG.bit_generator.state
@@ -184,3 +188,26 @@ def test_host_rewrites_layers_onto_contract_sum_map():
         assert np.array_equal(g0, g1)
     # two layers per step forward; backward one call per layer and step but the very first layer's input needs no cotangent
     assert plain.counter("contract_sum_map") == 0 and fused.counter("contract_sum_map") >= 4 * steps
+
+
+def test_condition_of_relu_is_a_result_of_the_layer_call():
+    """relu (W x + b) keeps `0 < W x + b` for the reverse pass.  On a table with
+    the entry point the condition leaves the layer's call as one more result, so
+    the reverse pass does not multiply W x a second time; values and gradients
+    equal the plain table's."""
+    from conftest import entry, pkg
+    H, W = pkg.hostapi, pkg.workloads
+    plain = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    fused = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_", api_table="get_api_fused"))
+    wl = W.c2_wide(batch=7, widths=(12, 9, 8, 5))
+    res = []
+    for host in (plain, fused):
+        ps, ds = wl.upload(host)
+        loss, grads = wl.gradient(host, ps, ds)
+        res.append((float(loss.numpy()), [g.numpy() for g in grads]))
+    assert res[0][0] == res[1][0]
+    for g0, g1 in zip(res[0][1], res[1][1]):
+        assert np.array_equal(g0, g1)
+    assert fused.counter("contract_sum_map_kept_nodes") == 2        # the two hidden layers
+    # products per gradient: 3 forward, 2 input cotangents, 3 weight gradients; none twice
+    assert fused.counter("contract_sum_map") + fused.counter("contract") + fused.counter("contract_sum") <= 8
