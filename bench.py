@@ -223,7 +223,9 @@ def main():
     if args.calibrate_mfma:
         ctx = capi.Lib().context(0)
         out = {}
-        names = ["v_mfma_f64_16x16x4_f64", "v_mfma_f64_4x4x4_4b_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32"]
+        names = ["v_mfma_f64_16x16x4_f64", "v_mfma_f64_4x4x4_4b_f64", "v_mfma_f32_16x16x4_f32", "v_mfma_f32_32x32x2_f32",
+                 "v_mfma_f64_16x16x4_f64 fed from LDS, 1 wavefront per SIMD", "v_mfma_f64_16x16x4_f64 fed from LDS, 2 wavefronts per SIMD",
+                 "v_mfma_f64_16x16x4_f64 fed from LDS, 4 wavefronts per SIMD"]
         for variant, name in enumerate(names):
             best = 0.0
             for _ in range(3):
@@ -232,7 +234,7 @@ def main():
                 best = max(best, t.value)
             out[name] = {"sustained_tflops": best, "nominal_peak_tflops": MFMA_PEAK_TFLOPS["f64" if "f64_" in name[:12] else "f32"],
                          "fraction_of_nominal": best / MFMA_PEAK_TFLOPS["f64" if "f64_" in name[:12] else "f32"]}
-        print(json.dumps({"calibration": "loops of one MFMA instruction, 16 wavefronts per CU, 20000 iterations of 4 (8, 2) independent accumulators", "instructions": out}))
+        print(json.dumps({"calibration": "loops of one MFMA instruction, 20000 iterations: operands in registers, 16 wavefronts per CU, 4 (8, 2) independent accumulators; and fed from LDS as a 64 x 64 tile of four wavefronts (2 x 2 blocks each, a barrier per 16 k)", "instructions": out}))
         return
     if args.calibrate_copy:
         import numpy as np

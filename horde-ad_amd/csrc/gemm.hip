@@ -600,12 +600,44 @@ __global__ void __launch_bounds__(256) mfma_probe_f32_32x32x2(float* out, int it
     for (int j = 0; j < 16; ++j) s += acc[i][j];
   out[blockIdx.x * 256 + threadIdx.x] = s;
 }
+// The same instruction fed the way a product kernel feeds it: four wavefronts
+// hold a 64 x 64 tile (2 x 2 blocks each), every K step of 16 reads its
+// fragments from LDS and ends with a barrier; nothing is loaded from memory.
+__global__ void __launch_bounds__(256) mfma_probe_f64_16x16x4_lds(double* out, int iters) {
+  __shared__ double As[16][65], Bs[16][65];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
+  for (int i = t; i < 16 * 65; i += 256) { (&As[0][0])[i] = i * 1e-3; (&Bs[0][0])[i] = i * 2e-3; }
+  __syncthreads();
+  probe_d4 acc[2][2];
+  for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < 2; ++j) acc[i][j] = probe_d4{0, 0, 0, 0};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int kk = 0; kk < 16; kk += 4) {
+      double fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[i] = As[kk + (lane >> 4)][wm * 32 + i * 16 + (lane & 15)];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fb[j] = Bs[kk + (lane >> 4)][wn * 32 + j * 16 + (lane & 15)];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  double s = 0;
+  for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < 2; ++j) s += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+  out[blockIdx.x * 256 + t] = s;
+}
 }  // namespace
 
 extern "C" int hgpu_mfma_probe(hgpu_ctx* ctx, int variant, int iters, double* tflops) {
   if (!ctx || !tflops || iters < 1) return HGPU_ERR_INVALID;
   if (int rc = no_capture(ctx, "mfma_probe")) return rc;
-  const int blocks = ctx->num_cu * 4;      // 16 wavefronts per CU: every SIMD has four to pick from
+  // 16 wavefronts per CU: every SIMD has four to pick from; the LDS-fed variants 4, 5, 6 run one, two, four per SIMD
+  const int blocks = ctx->num_cu * (variant == 4 ? 1 : variant == 5 ? 2 : 4);
   hgpu_buffer* buf = nullptr;
   int rc = buffer_alloc(ctx, (size_t)blocks * 256 * 8, &buf);
   if (rc) return rc;
@@ -616,10 +648,14 @@ extern "C" int hgpu_mfma_probe(hgpu_ctx* ctx, int variant, int iters, double* tf
       case 1: hipLaunchKernelGGL(mfma_probe_f64_4x4x4, dim3(blocks), dim3(256), 0, ctx->stream, (double*)buf->ptr, iters); flops_per_wave_iter = 8 * 2.0 * 4 * 4 * 4 * 4; break;
       case 2: hipLaunchKernelGGL(mfma_probe_f32_16x16x4, dim3(blocks), dim3(256), 0, ctx->stream, (float*)buf->ptr, iters); flops_per_wave_iter = 4 * 2.0 * 16 * 16 * 4; break;
       case 3: hipLaunchKernelGGL(mfma_probe_f32_32x32x2, dim3(blocks), dim3(256), 0, ctx->stream, (float*)buf->ptr, iters); flops_per_wave_iter = 2 * 2.0 * 32 * 32 * 2; break;
+      case 4: case 5: case 6:
+        hipLaunchKernelGGL(mfma_probe_f64_16x16x4_lds, dim3(blocks), dim3(256), 0, ctx->stream, (double*)buf->ptr, iters);
+        flops_per_wave_iter = 16 * 2.0 * 16 * 16 * 4;
+        break;
       default: break;
     }
   };
-  if (variant < 0 || variant > 3) { buffer_release(buf); return fail(ctx, HGPU_ERR_INVALID, "mfma_probe: variant %d", variant); }
+  if (variant < 0 || variant > 6) { buffer_release(buf); return fail(ctx, HGPU_ERR_INVALID, "mfma_probe: variant %d", variant); }
   hipEvent_t e0, e1;
   LaunchGuard lg(ctx);
   launch();   // warm-up

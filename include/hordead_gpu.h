@@ -126,8 +126,12 @@ int hgpu_profile_report(hgpu_ctx* ctx, char* buf, size_t n);
  * one matrix-core instruction on independent accumulators, 16 wavefronts per
  * CU, timed with events on the context's stream.  variant 0: v_mfma_f64_16x16x4,
  * 1: v_mfma_f64_4x4x4 (four blocks), 2: v_mfma_f32_16x16x4, 3: v_mfma_f32_32x32x2.
- * *tflops is what the instruction sustains on this device: the ceiling of any
- * product kernel built on it.  Waits for the stream. */
+ * Variants 4, 5, 6: v_mfma_f64_16x16x4 fed as a product kernel feeds it (four
+ * wavefronts hold a 64 x 64 tile, fragments read from LDS, a barrier per 16 k,
+ * nothing loaded from memory) at one, two and four wavefronts per SIMD.
+ * *tflops is what the loop sustains on this device: with its way of feeding
+ * the instruction, the ceiling of a product kernel built on it.  Waits for
+ * the stream. */
 int hgpu_mfma_probe(hgpu_ctx* ctx, int variant, int iters, double* tflops);
 
 /* ----------------------------------------------------------------- memory */
@@ -299,7 +303,9 @@ int hgpu_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, i
  *   in their first n_keep dims, the contracted dims may differ from term to term;
  *   program, in, out_slots, outs: as for hgpu_contract_map (exactly one entry
  *   of `in` is NULL and stands for C; n_out >= 1).
- * When the contracted dims are short (together at most 512 elements) and the
+ * When the contracted dims are short (together at most 512 elements, 1024 when
+ * the result has at most 160,000 elements -- where a product with a K loop
+ * would split K to fill the device and add partial results) and the
  * kept shape has two non-unit dims this is one kernel compiled for the shapes,
  * with the whole contracted dim of a term in LDS; otherwise the single entry
  * points run one after another.  Results equal theirs up to the order of the
