@@ -458,3 +458,25 @@ class V:
     def lift(self, shm):
         """A rank-0 tensor as a scalar of the position space shm."""
         return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_lift, len(shm), _larr(shm), self.h), tuple(shm))
+
+
+# Ranked (`tr*`, user-facing `r*`) and mixed (`tx*` / `x*`) methods of the tensor
+# class (Ops.hs:297-1255): the ABI takes shapes at run time, so a ranked or
+# mixed method is its shaped twin under another name -- the same entry point,
+# the same kernel.  `rtr` = `str_`, `rmaxIndex` / `rminIndex` = `sargMax` /
+# `sargMin` as in the reference's naming.
+_TWINS = ["cast", "fromIntegral", "floor", "sum", "sumN", "sum0", "dot0", "dot1In", "dotNIn", "matvecmul", "matmul2",
+          "replicate", "replicateN", "append", "slice", "reverse", "transpose", "reshape", "index", "gather", "scatter", "index0"]
+for _n in _TWINS:
+    for _p in ("r", "x"):
+        setattr(V, _p + _n, getattr(V, "s" + _n))
+for _p in ("r", "x"):
+    setattr(V, _p + "tr", V.str_)
+    setattr(V, _p + "maxIndex", V.sargMax)
+    setattr(V, _p + "minIndex", V.sargMin)
+    setattr(Host, _p + "concrete", Host.sconcrete)
+    setattr(Host, _p + "repl", Host.srepl)
+    setattr(Host, _p + "iota", Host.siota)
+    setattr(Host, _p + "fromVector", Host.sfromVector)
+    setattr(Host, _p + "build1", Host.sbuild1)
+    setattr(Host, _p + "mapAccumL", Host.smapAccumL)

@@ -272,23 +272,25 @@ def c4_rnn(batch=5000, dtype=F32, steps=28, n_in=28, width=128, n_classes=10):
               (n_classes, width), (n_classes,)]
     params = [rng.uniform(-0.1, 0.1, s).astype(NP[dtype]) for s in shapes]
 
+    # the reference writes this network with the ranked methods (rmatmul2, rtr,
+    # rreplicate, rslice, rappend): here they are the shaped ones by another name
     def layer(s, x, wx, ws, b):
-        return (wx.smatmul2(x) + ws.smatmul2(s) + b.sreplicate(batch).str_()).op1("tanh")
+        return (wx.rmatmul2(x) + ws.rmatmul2(s) + b.rreplicate(batch).rtr()).op1("tanh")
 
     def objective(ps, ds):
         xs_, lab = ds
         wx, ws, b, wx2, ws2, b2, w3, b3 = ps
         host = wx.host
-        s = host.srepl((2 * width, batch), 0.0, dtype)           # zeroStateR
+        s = host.rrepl((2 * width, batch), 0.0, dtype)           # zeroStateR
         out = None
         for t in range(steps):                                    # unrollLastR: foldl' over runravelToList
-            x = xs_.sindex([t])
-            s1, s2 = s.sslice(0, width), s.sslice(width, width)
+            x = xs_.rindex([t])
+            s1, s2 = s.rslice(0, width), s.rslice(width, width)
             v1 = layer(s1, x, wx, ws, b)
             v2 = layer(s2, v1, wx2, ws2, b2)
-            s = v1.sappend(v2)
-            out = s.sslice(width, width)
-        result = w3.smatmul2(out) + b3.sreplicate(batch).str_()
+            s = v1.rappend(v2)
+            out = s.rslice(width, width)
+        result = w3.rmatmul2(out) + b3.rreplicate(batch).rtr()
         loss = lossSoftMaxCrossEntropyS(lab, result)
         return host.srepl((), 1.0 / batch, dtype) * loss
 

@@ -337,3 +337,27 @@ def test_value_at_own_extremum_cpu(host_cpu):
 @pytest.mark.gpu
 def test_value_at_own_extremum_gpu(host_gpu):
     value_at_own_extremum(host_gpu)
+
+
+def test_ranked_and_mixed_methods_are_the_shaped_ones(host_cpu):
+    host = host_cpu
+    """Ops.hs:297-1255 gives every operation a ranked (tr*), a shaped (ts*) and a
+    mixed (tx*) method; the ABI takes shapes at run time, so all three bind to
+    one entry point.  The twins give the same arrays, through a gather with an
+    index function and a scatter too."""
+    rng = np.random.default_rng(5)
+    a, b = rng.standard_normal((4, 6)), rng.standard_normal((6, 3))
+    A, B = host.concrete(a), host.concrete(b)
+    want = a @ b
+    for pre in ("s", "r", "x"):
+        mm = getattr(A, pre + "matmul2")(B)
+        assert np.allclose(mm.numpy(), want, rtol=0, atol=1e-12)
+        assert np.array_equal(getattr(A, pre + "slice")(1, 2).numpy(), a[1:3])
+        assert np.array_equal(getattr(getattr(A, pre + "replicate")(2), pre + "sum")().numpy(), 2 * a)
+        assert np.array_equal(getattr(A, pre + "reshape")([6, 4]).numpy(), a.reshape(6, 4))
+        g = getattr(A, pre + "gather")((3,), lambda i: [i + 1, i * 2])
+        assert np.array_equal(g.numpy(), np.array([a[1, 0], a[2, 2], a[3, 4]]))
+        sc = getattr(g, pre + "scatter")(1, (5,), lambda i: [i * 2])
+        assert np.array_equal(sc.numpy(), np.array([a[1, 0], 0, a[2, 2], 0, a[3, 4]]))
+    assert np.array_equal(A.rtr().numpy(), a.T) and np.array_equal(A.rmaxIndex().numpy(), a.argmax(-1))
+    assert np.array_equal(host.rrepl((2, 2), 1.5).numpy(), np.full((2, 2), 1.5))
