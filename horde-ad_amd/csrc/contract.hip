@@ -381,6 +381,82 @@ __global__ void __launch_bounds__(1024) k_argminmax_block(Dims keep, int64_t L, 
   }
 }
 
+// A few very long rows whose data one CU cannot fetch fast enough (a block
+// draws some tens of GB/s): G blocks per row scan consecutive pieces, then one
+// wavefront per row picks among the G candidates, the earlier piece winning ties.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_argminmax_pieces(Dims keep, int64_t L, int64_t sl, int want_max, int G, int64_t piece, const T* __restrict__ a,
+                                                              T* __restrict__ pbest, int64_t* __restrict__ pidx) {
+  __shared__ T sbest[kBlock];
+  __shared__ int64_t sidx[kBlock];
+  const int row = blockIdx.x / G, g = blockIdx.x % G;
+  int64_t ko[1];
+  decompose<1>(keep, row, ko);
+  const T* p = a + ko[0];
+  const int t = threadIdx.x;
+  const int64_t j0 = (int64_t)g * piece, j1 = j0 + piece < L ? j0 + piece : L;
+  T best = T(0);
+  int64_t bi = INT64_MAX;
+  int64_t j = j0 + t;
+  for (; j + 3 * kBlock < j1; j += 4 * kBlock) {
+    T x[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) x[u] = p[(j + u * kBlock) * sl];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      bool better = bi == INT64_MAX || (want_max ? (x[u] > best) : (x[u] < best));
+      if (better) { best = x[u]; bi = j + u * kBlock; }
+    }
+  }
+  for (; j < j1; j += kBlock) {
+    T x = p[j * sl];
+    bool better = bi == INT64_MAX || (want_max ? (x > best) : (x < best));
+    if (better) { best = x; bi = j; }
+  }
+  sbest[t] = best;
+  sidx[t] = bi;
+  __syncthreads();
+  for (int off = kBlock / 2; off > 0; off >>= 1) {
+    if (t < off) {
+      T ob = sbest[t + off];
+      int64_t oi = sidx[t + off];
+      if (oi != INT64_MAX) {
+        bool mine = sidx[t] != INT64_MAX;
+        bool better = !mine || (want_max ? (ob > sbest[t]) : (ob < sbest[t])) || (ob == sbest[t] && oi < sidx[t]);
+        if (better) { sbest[t] = ob; sidx[t] = oi; }
+      }
+    }
+    __syncthreads();
+  }
+  if (t == 0) { pbest[blockIdx.x] = sbest[0]; pidx[blockIdx.x] = sidx[0]; }
+}
+template <typename T>
+__global__ void __launch_bounds__(64) k_argminmax_pick(int G, int want_max, const T* __restrict__ pbest, const int64_t* __restrict__ pidx, int64_t* __restrict__ out,
+                                                        T* __restrict__ vals) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  T best = T(0);
+  int64_t bi = INT64_MAX;
+  for (int g = lane; g < G; g += 64) {
+    T x = pbest[row * G + g];
+    int64_t xi = pidx[row * G + g];
+    if (xi == INT64_MAX) continue;
+    bool better = bi == INT64_MAX || (want_max ? (x > best) : (x < best));    // pieces of a lane come in ascending order
+    if (better) { best = x; bi = xi; }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    T ob = __shfl_down(best, off);
+    int64_t oi = __shfl_down(bi, off);
+    if (oi != INT64_MAX) {
+      bool better = bi == INT64_MAX || (want_max ? (ob > best) : (ob < best)) || (ob == best && oi < bi);
+      if (better) { best = ob; bi = oi; }
+    }
+  }
+  if (lane == 0) {
+    out[row] = bi;
+    if (vals) vals[row] = best;
+  }
+}
+
 template <typename TI, typename TO>
 int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red_full, int64_t n_out, int64_t R, int S, const void* a, const void* b, void* out,
                  const TermPtrs* terms = nullptr) {
@@ -772,7 +848,20 @@ int hgpu_extremum_last(hgpu_ctx* ctx, const hgpu_array* a, int want_max, hgpu_ar
     if (!collapse(a->rank - 1, a->shape, 1, ks, &keep)) { hgpu_release(o); if (v) hgpu_release(v); return fail(ctx, HGPU_ERR_UNSUPPORTED, "argminmax: too many dims"); }
     LaunchGuard lg(ctx, "argminmax", (double)n_out * (L * dtype_size(a->dtype) + 8 + (v ? dtype_size(a->dtype) : 0)), (double)n_out * L);
     void* vp = v ? data_ptr(v) : nullptr;
-    if (L >= 8192 && n_out <= 64) {
+    if (L >= 16384 && n_out <= 16) {
+      // very few, very long rows: pieces of a row to many blocks, then one pick per row
+      const int G = (int)std::min<int64_t>(128, L / 2048);
+      const int64_t piece = (L + G - 1) / G;
+      hgpu_buffer* scratch = nullptr;
+      const size_t vb = ((size_t)n_out * G * dtype_size(a->dtype) + 15) / 16 * 16;
+      rc = buffer_alloc(ctx, vb + (size_t)n_out * G * 8, &scratch);
+      if (rc) { hgpu_release(o); if (v) hgpu_release(v); return rc; }
+      void* pb = scratch->ptr;
+      int64_t* pi = (int64_t*)((char*)scratch->ptr + vb);
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_pieces<T>, dim3((unsigned)(n_out * G)), dim3(kBlock), 0, ctx->stream, keep, L, a->strides[a->rank - 1], want_max, G, piece, (const T*)data_ptr(a), (T*)pb, pi));
+      HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_pick<T>, dim3((unsigned)n_out), dim3(64), 0, ctx->stream, G, want_max, (const T*)pb, (const int64_t*)pi, (int64_t*)data_ptr(o), (T*)vp));
+      buffer_release(scratch);
+    } else if (L >= 8192 && n_out <= 64) {
       // few long rows: a whole block per row
       HG_DISPATCH_DTYPE(a->dtype, T, hipLaunchKernelGGL(k_argminmax_block<T>, dim3((unsigned)n_out), dim3(1024), 0, ctx->stream, keep, L, a->strides[a->rank - 1], want_max, (const T*)data_ptr(a), (int64_t*)data_ptr(o), (T*)vp));
     } else if (L >= 256 && n_out < (int64_t)ctx->num_cu * 64) {

@@ -346,6 +346,30 @@ def test_extremum_values_with_indices(gpu):
                 assert np.array_equal(vals.numpy(), np.take_along_axis(x, want_idx[..., None], axis=-1)[..., 0])
 
 
+def test_extremum_of_very_long_rows(gpu):
+    """A few rows of tens of thousands of elements (the minimum of a whole tensor)
+    are scanned in pieces by many blocks: first occurrence wins also when the tie
+    lies in another piece, rows may be strided, and the last piece may be ragged."""
+    for dt in (np.float64, np.float32, np.int32):
+        for shape in [(50000,), (3, 81920), (2, 16385)]:
+            x = rnd(shape, dt)
+            flat = x.reshape(-1, shape[-1])
+            for r in range(flat.shape[0]):                       # the extremes several times, far apart
+                hi, lo = flat[r].max() + 1, flat[r].min() - 1
+                flat[r, [shape[-1] - 7, 9000, 40000 % shape[-1]]] = hi
+                flat[r, [shape[-1] - 1, 12001, 5]] = lo
+            a = gpu.upload(x)
+            for want_max in (True, False):
+                vals, idx = a.extremum_last(want_max)
+                want_idx = (np.argmax if want_max else np.argmin)(x, axis=-1)
+                assert np.array_equal(idx.numpy(), want_idx)
+                assert np.array_equal(vals.numpy(), np.take_along_axis(x, np.asarray(want_idx)[..., None], axis=-1)[..., 0])
+    x = rnd((20000, 4), np.float64)                              # rows of a transposed view: stride 4
+    a = gpu.upload(x).transpose([1, 0])
+    assert np.array_equal(a.argminmax_last(True).numpy(), np.argmax(x.T, axis=-1))
+    assert np.array_equal(a.argminmax_last(False).numpy(), np.argmin(x.T, axis=-1))
+
+
 def ix_arrays(both, shm, extents, oob=True, view=False):
     out = []
     for e in extents:
