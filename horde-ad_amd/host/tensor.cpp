@@ -566,8 +566,19 @@ static bool products_then_program(Backend* be, const std::vector<ArrHolder*>& ro
         for (auto* f : {&q->fa, &q->fb, &q->fc})
           if (f->get() == nd) { sp = *f; ++in; }
       if (sp && sp.use_count() - 1 > in && roots.size() + promoted.size() < 6) {
-        promoted.push_back({nd, (int)ins.size() + (int)i});
-        has_products[nd] = false;     // written: what is built on it can be redone from the array
+        // `ifH c 0 1` between constants: its condition says as much in a byte per element
+        ArrHolder* w = nd;
+        size_t wi = i;
+        if (nd->ekind == HGPU_FUSED_SELECT && nd->fa && !nd->fa->h && nd->fa->ekind >= 0 && has_products[nd->fa.get()] && !has_products[nd->fb.get()] &&
+            !has_products[nd->fc.get()] && std::find(roots.begin(), roots.end(), nd->fa.get()) == roots.end()) {
+          auto at = std::find(nodes.begin(), nodes.end(), nd->fa.get());
+          if (at != nodes.end() && T(nd->fa).dtype() == HGPU_BOOL) { w = *at; wi = (size_t)(at - nodes.begin()); }
+        }
+        bool have = false;
+        for (auto& pr : promoted) have = have || pr.first == w;
+        if (!have) promoted.push_back({w, (int)ins.size() + (int)wi});
+        has_products[w] = false;      // written: what is built on it can be redone from the array
+        has_products[nd] = false;
       }
     }
   }
