@@ -360,6 +360,10 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   if (p.K < 4 || p.M * p.N < 256) return HGPU_OK;
   if (p.BT > 65535) return HGPU_OK;
   if ((double)p.M * p.N * p.K * p.BT < 2.0e6) return HGPU_OK;
+  // a thousand outputs under a long K (the last layer's weight gradient: 100 x 10
+  // over 5000): the split-K kernels have a handful of wavefronts to work with,
+  // a wavefront per output in the reduction kernels has a thousand
+  if ((p.M <= 16 || p.N <= 16) && p.K > 1024 && (double)p.M * p.N * p.K * p.BT < 2.0e7) return HGPU_OK;
 
   const void* pa = data_ptr(a);
   const void* pb = data_ptr(b);
