@@ -446,6 +446,11 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
       const int hi = (int)std::min<int64_t>(max_split, split + (split * 3 + 9) / 10);
       for (int cand = split + 1; cand <= hi; ++cand)
         if (fill(cand) > best_fill + 0.1) { best_fill = fill(cand); best_s = cand; }
+      // ... or a few less, when that makes whole rounds (28 products of 128 x 128 over
+      // K 5000 in 64 x 64 tiles: 12 chunks each = 1344 blocks on 1024 places, 9 = 1008)
+      const int lo = std::max(2, split - (split * 3 + 9) / 10);
+      for (int cand = split - 1; cand >= lo; --cand)
+        if (fill(cand) > best_fill + 0.1) { best_fill = fill(cand); best_s = cand; }
       split = best_s;
     }
   }
