@@ -388,13 +388,72 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   }
   if ((p.M <= 32 || p.N <= 32) && p.M <= 1024 && p.N <= 1024) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled, n_terms);
 
-  // tile shape: least padded work per unit of efficiency
+  const int64_t nt = n_terms > 0 ? n_terms : 1;      // products summed by this launch
+  const int64_t out_elems = p.M * p.N * p.BT;
+  // K chunks for a tile shape, and how well the blocks then fill the device
+  // (blocks / places of the rounds they take)
+  auto plan_split = [&](int c, double* fill_out) {
+    const int64_t bm = kTiles[c].wgm * kTiles[c].tm * 16, bn = kTiles[c].wgn * kTiles[c].tn * 16;
+    const int64_t tl = ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
+    // small tiles do little work per K step and hide the latency of a step only
+    // behind other blocks on the CU: ask for more of them
+    const int64_t per_cu = bm * bn >= 128 * 64 ? 2 : (bm * bn >= 64 * 64 ? 4 : 8);
+    const double slots = (double)ctx->num_cu * per_cu;
+    auto fill = [&](int cand) {
+      const double blocks = (double)tl * p.BT * nt * cand;
+      return blocks / (std::ceil(blocks / slots) * slots);
+    };
+    int split = 1;
+    const int64_t want = (int64_t)ctx->num_cu * per_cu;
+    if (tl * p.BT * nt < want && p.K >= 8 * BK) {
+      split = (int)((want + tl * p.BT * nt - 1) / (tl * p.BT * nt));
+      int64_t max_split = p.K / (4 * BK);
+      if (split > max_split) split = (int)max_split;
+      // the partial products must stay small next to the operands, or small outright
+      int64_t cap = out_elems > 0 ? (int64_t)((double)(p.M + p.N) * p.K * p.BT / (2.0 * out_elems)) : 1;
+      if (out_elems * (int64_t)dtype_size(a->dtype) <= (1 << 20) && cap < 16) cap = 16;
+      if (cap > 512) cap = 512;
+      if (cap < 1) cap = 1;
+      if (split > cap) split = (int)cap;
+      if (split < 1) split = 1;
+      // fewer tiles than CUs: two K halves per tile keep every CU busy, and the
+      // second pass over the output costs less than the idle quarter of the device
+      if (split == 1 && tl * p.BT * nt < ctx->num_cu && p.K >= 16 * BK) split = 2;
+      // A few more chunks when they fill the last round of blocks: with `per_cu`
+      // blocks resident on a CU, blocks run in rounds of num_cu * per_cu, and a
+      // round that is three quarters empty costs as much as a full one.  (300 x 784
+      // over K 5000 in 64 x 128 tiles: 11 chunks = 385 blocks take 82 us, 14 chunks
+      // = 490 blocks 70 us, 15 chunks = 525 blocks 94 us.)
+      if (split > 1) {
+        int best_s = split;
+        double best_fill = fill(split);
+        const int hi = (int)std::min<int64_t>(max_split, split + (split * 3 + 9) / 10);
+        for (int cand = split + 1; cand <= hi; ++cand)
+          if (fill(cand) > best_fill + 0.1) { best_fill = fill(cand); best_s = cand; }
+        // ... or a few less, when that makes whole rounds (28 products of 128 x 128 over
+        // K 5000 in 64 x 64 tiles: 12 chunks each = 1344 blocks on 1024 places, 9 = 1008)
+        const int lo = std::max(2, split - (split * 3 + 9) / 10);
+        for (int cand = split - 1; cand >= lo; --cand)
+          if (fill(cand) > best_fill + 0.1) { best_fill = fill(cand); best_s = cand; }
+        split = best_s;
+      }
+    }
+    if (fill_out) *fill_out = fill(split);
+    return split;
+  };
+  // tile shape: least padded work per unit of efficiency and of device filled
+  const bool f64 = a->dtype == HGPU_F64;
   int cfg = 0;
   double best = 1e300;
+  double costs[kNumTiles];
   for (int c = 0; c < (a->dtype == HGPU_F32 ? kNumTiles : kFirstF32OnlyTile); ++c) {
     int64_t bm = kTiles[c].wgm * kTiles[c].tm * 16, bn = kTiles[c].wgn * kTiles[c].tn * 16;
     double padded = (double)((p.M + bm - 1) / bm * bm) * (double)((p.N + bn - 1) / bn * bn);
-    double cost = padded / kTiles[c].eff;
+    // fp64: the instruction is slow next to LDS, so the operand reuse of a larger
+    // tile buys little and three 64 x 64 blocks on a CU run it as well as two of
+    // 64 x 128 (300 x 784 over K 5000: 64 against 74 us)
+    const double eff = (f64 && bm == 64 && bn == 64) ? 0.85 : kTiles[c].eff;
+    double cost = padded / eff;
     // a tile shape that cannot occupy the device even with K split pays for the idle CUs
     double blocks = (double)((p.M + bm - 1) / bm) * (double)((p.N + bn - 1) / bn) * (double)p.BT;
     double can_split = (double)(p.K / (4 * BK));
@@ -403,57 +462,25 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     if (can_split > 512) can_split = 512;
     if (can_split < 1) can_split = 1;
     if (blocks * can_split < ctx->num_cu) cost *= ctx->num_cu / (blocks * can_split);
+    costs[c] = cost;
     if (cost < best * 0.999) { best = cost; cfg = c; }
+  }
+  if (f64) {
+    // among shapes within 15 % of the least, the one whose blocks fill their rounds
+    // best (the fp32 choices were tuned without this step)
+    double best2 = 1e300;
+    for (int c = 0; c < kFirstF32OnlyTile; ++c) {
+      if (costs[c] > best * 1.15) continue;
+      double fl = 1;
+      (void)plan_split(c, &fl);
+      const double c2 = costs[c] / std::max(fl, 0.25);
+      if (c2 < best2 * 0.999) { best2 = c2; cfg = c; }
+    }
   }
   const int64_t BM = kTiles[cfg].wgm * kTiles[cfg].tm * 16, BN = kTiles[cfg].wgn * kTiles[cfg].tn * 16;
   int64_t tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   if (tiles > 0x7fffffff) return HGPU_OK;
-  // split K when the tiles alone cannot fill the device
-  int split = 1;
-  // small tiles do little work per K step and hide the latency of a step only
-  // behind other blocks on the CU: ask for more of them
-  const int64_t per_cu = BM * BN >= 128 * 64 ? 2 : (BM * BN >= 64 * 64 ? 4 : 8);
-  int64_t want = (int64_t)ctx->num_cu * per_cu;
-  int64_t out_elems = p.M * p.N * p.BT;
-  const int64_t nt = n_terms > 0 ? n_terms : 1;      // products summed by this launch
-  if (tiles * p.BT * nt < want && p.K >= 8 * BK) {
-    split = (int)((want + tiles * p.BT * nt - 1) / (tiles * p.BT * nt));
-    int64_t max_split = p.K / (4 * BK);
-    if (split > max_split) split = (int)max_split;
-    // the partial products must stay small next to the operands, or small outright
-    int64_t cap = out_elems > 0 ? (int64_t)((double)(p.M + p.N) * p.K * p.BT / (2.0 * out_elems)) : 1;
-    if (out_elems * (int64_t)dtype_size(a->dtype) <= (1 << 20) && cap < 16) cap = 16;
-    if (cap > 512) cap = 512;
-    if (cap < 1) cap = 1;
-    if (split > cap) split = (int)cap;
-    if (split < 1) split = 1;
-    // fewer tiles than CUs: two K halves per tile keep every CU busy, and the
-    // second pass over the output costs less than the idle quarter of the device
-    if (split == 1 && tiles * p.BT * nt < ctx->num_cu && p.K >= 16 * BK) split = 2;
-    // A few more chunks when they fill the last round of blocks: with `per_cu`
-    // blocks resident on a CU, blocks run in rounds of num_cu * per_cu, and a
-    // round that is three quarters empty costs as much as a full one.  (300 x 784
-    // over K 5000 in 64 x 128 tiles: 11 chunks = 385 blocks take 82 us, 14 chunks
-    // = 490 blocks 70 us, 15 chunks = 525 blocks 94 us.)
-    if (split > 1) {
-      const double slots = (double)ctx->num_cu * per_cu;
-      auto fill = [&](int cand) {
-        const double blocks = (double)tiles * p.BT * nt * cand;
-        return blocks / (std::ceil(blocks / slots) * slots);
-      };
-      int best_s = split;
-      double best_fill = fill(split);
-      const int hi = (int)std::min<int64_t>(max_split, split + (split * 3 + 9) / 10);
-      for (int cand = split + 1; cand <= hi; ++cand)
-        if (fill(cand) > best_fill + 0.1) { best_fill = fill(cand); best_s = cand; }
-      // ... or a few less, when that makes whole rounds (28 products of 128 x 128 over
-      // K 5000 in 64 x 64 tiles: 12 chunks each = 1344 blocks on 1024 places, 9 = 1008)
-      const int lo = std::max(2, split - (split * 3 + 9) / 10);
-      for (int cand = split - 1; cand >= lo; --cand)
-        if (fill(cand) > best_fill + 0.1) { best_fill = fill(cand); best_s = cand; }
-      split = best_s;
-    }
-  }
+  int split = plan_split(cfg, nullptr);
   if (const char* e = getenv("HORDEAD_GEMM_SPLIT")) {   // for measurements
     int v = atoi(e);
     if (v >= 1 && v <= p.K / BK) split = v;
