@@ -170,7 +170,8 @@ def roofline_of(rep, dtype_name):
         roof = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS,
                 "algorithmic_mb_per_launch": by / launches / 1e6}
     roof.update({"kernel": name, "launches_per_step": launches, "avg_launch_ms": avg_ms,
-                 "share_of_device_time": ms / sum(v[1] for v in rep.values()), "traffic": measured_traffic(name)})
+                 "share_of_device_time": ms / sum(v[1] for v in rep.values()), "traffic": measured_traffic(name),
+                 "traffic_source": "profiles/hbm_traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel, committed with the build (not measured in this run)"})
     fams = {}
     for k, v in rep.items():
         fams[family(k)] = fams.get(family(k), 0.0) + v[1]
