@@ -48,6 +48,12 @@ struct hgpu_array {
   int64_t offset;                  // in elements, from buf->ptr
 };
 
+namespace hg {
+struct DeferredQueue;                         // launches held back to be grouped (smallk.hip)
+void flush_deferred_locked(hgpu_ctx* ctx);    // the caller holds launch_mu
+void flush_deferred(hgpu_ctx* ctx);
+}  // namespace hg
+
 struct hgpu_ctx {
   int device;
   hipStream_t stream;
@@ -70,6 +76,11 @@ struct hgpu_ctx {
   std::vector<ProfRec> prof;
   hgpu_buffer* zero_block = nullptr;     // 256 zero bytes, for kernels that want a dummy table
   hgpu_cap_pool* cap = nullptr;          // non-null while the stream is capturing into a graph
+  // Small products whose launch is held back until something else needs the
+  // stream: those that do not depend on one another then go out as one kernel.
+  hg::DeferredQueue* dq = nullptr;
+  bool dq_pending = false;
+  int deferred_rc = 0;                   // first error of a held-back launch, reported by hgpu_sync
 };
 
 struct hgpu_graph {
@@ -170,6 +181,7 @@ struct LaunchGuard {
   explicit LaunchGuard(hgpu_ctx* c, const char* name = nullptr, double bytes = 0, double flops = 0) : ctx(c) {
     c->launch_mu.lock();
     (void)hipSetDevice(c->device);
+    if (c->dq_pending) flush_deferred_locked(c);   // what was held back goes first: stream order is program order
     if (c->profiling && name && !c->cap) {
       hgpu_ctx::ProfRec r{name, nullptr, nullptr, bytes, flops};
       if (hipEventCreate(&r.a) == hipSuccess && hipEventCreate(&r.b) == hipSuccess) {

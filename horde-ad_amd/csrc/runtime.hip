@@ -305,6 +305,7 @@ int hgpu_capture_begin(hgpu_ctx* ctx) {
   if (!ctx) return HGPU_ERR_INVALID;
   if (ctx->cap) return fail(ctx, HGPU_ERR_INVALID, "capture_begin: a capture is already open");
   (void)hipSetDevice(ctx->device);
+  flush_deferred(ctx);
   hipError_t e = hipStreamSynchronize(ctx->stream);
   if (e != hipSuccess) return check_hip(ctx, e, "capture_begin");
   hgpu_cap_pool* pool = new hgpu_cap_pool;
@@ -338,6 +339,7 @@ int hgpu_capture_end(hgpu_ctx* ctx, hgpu_graph** out) {
   if (!ctx || !out) return HGPU_ERR_INVALID;
   if (!ctx->cap) return fail(ctx, HGPU_ERR_INVALID, "capture_end: no capture is open");
   (void)hipSetDevice(ctx->device);
+  flush_deferred(ctx);          // launches still held back belong to the graph
   hgpu_cap_pool* pool;
   {
     std::lock_guard<std::mutex> g(ctx->mu);
@@ -366,6 +368,7 @@ int hgpu_graph_launch(hgpu_graph* gr) {
   if (ctx->cap) return fail(ctx, HGPU_ERR_INVALID, "graph_launch: not inside a capture");
   std::lock_guard<std::mutex> lk(ctx->launch_mu);
   (void)hipSetDevice(ctx->device);
+  if (ctx->dq_pending) flush_deferred_locked(ctx);
   return check_hip(ctx, hipGraphLaunch(gr->exec, ctx->stream), "hipGraphLaunch");
 }
 
@@ -373,6 +376,7 @@ int hgpu_graph_destroy(hgpu_graph* gr) {
   if (!gr) return HGPU_ERR_INVALID;
   hgpu_ctx* ctx = gr->ctx;
   (void)hipSetDevice(ctx->device);
+  flush_deferred(ctx);
   (void)hipStreamSynchronize(ctx->stream);     // a replay may still be running on the blocks
   if (gr->exec) (void)hipGraphExecDestroy(gr->exec);
   if (gr->graph) (void)hipGraphDestroy(gr->graph);
@@ -384,6 +388,7 @@ int hgpu_graph_destroy(hgpu_graph* gr) {
 int hgpu_shutdown(hgpu_ctx* ctx) {
   if (!ctx) return HGPU_ERR_INVALID;
   (void)hipSetDevice(ctx->device);
+  flush_deferred(ctx);
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->zero_block) { buffer_release(ctx->zero_block); ctx->zero_block = nullptr; }
   {
@@ -402,7 +407,13 @@ int hgpu_sync(hgpu_ctx* ctx) {
   if (!ctx) return HGPU_ERR_INVALID;
   if (int rc = no_capture(ctx, "sync")) return rc;
   (void)hipSetDevice(ctx->device);
-  return check_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+  flush_deferred(ctx);
+  int rc = check_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+  if (ctx->deferred_rc) {      // a launch that was held back failed after its call had returned
+    rc = ctx->deferred_rc;
+    ctx->deferred_rc = 0;
+  }
+  return rc;
 }
 
 const char* hgpu_last_error(hgpu_ctx* ctx) {
@@ -422,10 +433,15 @@ int hgpu_mem_stats(hgpu_ctx* ctx, uint64_t* in_use, uint64_t* reserved, uint64_t
   return HGPU_OK;
 }
 
-void* hgpu_stream(hgpu_ctx* ctx) { return ctx ? (void*)ctx->stream : nullptr; }
+void* hgpu_stream(hgpu_ctx* ctx) {
+  if (!ctx) return nullptr;
+  flush_deferred(ctx);      // whoever enqueues on the stream next comes after everything issued so far
+  return (void*)ctx->stream;
+}
 
 int hgpu_inject_alloc_failure(hgpu_ctx* ctx, int64_t limit) {
   if (!ctx) return HGPU_ERR_INVALID;
+  flush_deferred(ctx);
   std::lock_guard<std::mutex> g(ctx->mu);
   if (limit < 0) {
     ctx->fail_after = -1;
@@ -441,6 +457,7 @@ int hgpu_inject_alloc_failure(hgpu_ctx* ctx, int64_t limit) {
 int hgpu_profile_enable(hgpu_ctx* ctx, int on) {
   if (!ctx) return HGPU_ERR_INVALID;
   std::lock_guard<std::mutex> g(ctx->launch_mu);
+  if (ctx->dq_pending) flush_deferred_locked(ctx);
   (void)hipStreamSynchronize(ctx->stream);
   for (auto& r : ctx->prof) { (void)hipEventDestroy(r.a); (void)hipEventDestroy(r.b); }
   ctx->prof.clear();
@@ -452,6 +469,7 @@ int hgpu_profile_enable(hgpu_ctx* ctx, int on) {
 int hgpu_profile_report(hgpu_ctx* ctx, char* buf, size_t n) {
   if (!ctx || !buf || n == 0) return HGPU_ERR_INVALID;
   std::lock_guard<std::mutex> g(ctx->launch_mu);
+  if (ctx->dq_pending) flush_deferred_locked(ctx);
   (void)hipStreamSynchronize(ctx->stream);
   struct Agg { long count = 0; double ms = 0, bytes = 0, flops = 0; };
   std::map<std::string, Agg> agg;

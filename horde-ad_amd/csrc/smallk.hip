@@ -181,13 +181,16 @@ void emit_stage_fn(std::ostringstream& s, const char* name, const Operand& o, co
   (void)r0;
 }
 
-std::string generate(const Spec& sp, const std::string& kname) {
+// The device code of one problem, ending in
+// `body(const Args&, unsigned block, T* lds)`: what one block of 256 threads
+// does.  It names nothing outside itself but the prelude, so several problems'
+// code can sit in one source file, each in a namespace of its own.
+std::string generate_body(const Spec& sp) {
   std::ostringstream s;
   const int TP = sp.BP / (16 * sp.WP), TQ = sp.BQ / (16 * sp.WQ);
   const int64_t nbp = (sp.P + sp.BP - 1) / sp.BP, nbq = (sp.Q + sp.BQ - 1) / sp.BQ;
   const int64_t nblk = nbp * nbq, per_xcd = (nblk + 7) / 8;
   const bool vec_epi = !sp.f64 && sp.P % 4 == 0;
-  s << kPrelude;
   s << "typedef " << (sp.f64 ? "double" : "float") << " T;\n";
   s << "typedef T V2 __attribute__((ext_vector_type(2), aligned(" << (sp.f64 ? 8 : 4) << ")));\n";
   s << "typedef T V4 __attribute__((ext_vector_type(4), aligned(" << (sp.f64 ? 8 : 4) << ")));\n";
@@ -308,11 +311,10 @@ std::string generate(const Spec& sp, const std::string& kname) {
     s << "  }\n";
   }
   s << "}\n";
-  s << "extern \"C\" __global__ void __launch_bounds__(256) " << kname << "(Args ar) {\n";
-  s << "  __shared__ __attribute__((aligned(16))) T lds[" << sp.x_elems + sp.y_elems << "];\n";
+  s << "__device__ __forceinline__ void body(const Args& ar, unsigned bid, T* __restrict__ lds) {\n";
   s << "  T* const xs = lds;\n  T* const ys = lds + " << sp.x_elems << ";\n";
   // consecutive block ids go round the eight XCDs: blocks that share operand tiles get ids of one XCD
-  s << "  const i64 blk = (i64)(blockIdx.x % 8) * " << per_xcd << "LL + blockIdx.x / 8;\n";
+  s << "  const i64 blk = (i64)(bid % 8) * " << per_xcd << "LL + bid / 8;\n";
   s << "  if (blk >= " << nblk << "LL) return;\n";
   s << "  const i64 q0 = (blk % " << nbq << "LL) * " << sp.BQ << ", p0 = (blk / " << nbq << "LL) * " << sp.BP << ";\n";
   s << "  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r = lane & 15, g = lane >> 4;\n";
@@ -346,6 +348,34 @@ std::string generate(const Spec& sp, const std::string& kname) {
   s << "#pragma unroll\n  for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n    for (int b = 0; b < " << TQ << "; ++b)\n";
   if (n_read > 0) s << "      epilogue(ar, p0 + (wp * " << TP << " + a) * 16, q0 + (wq * " << TQ << " + b) * 16, r, g, acc[a][b], ei[a][b]);\n";
   else s << "      epilogue(ar, p0 + (wp * " << TP << " + a) * 16, q0 + (wq * " << TQ << " + b) * 16, r, g, acc[a][b], EpiIn{0});\n";
+  s << "}\n";
+  return s.str();
+}
+
+// One kernel over several problems that do not depend on one another: the
+// first blocks run problem 0, the next ones problem 1, ...  (`grids[k]` blocks
+// each, multiples of 8 so that every problem's block ids keep their place in
+// the round of the XCDs).  A single problem gives the kernel of that problem.
+std::string kernel_source(const std::vector<const std::string*>& bodies, const std::vector<unsigned>& grids, const std::vector<int>& lds_bytes, const std::string& kname) {
+  std::ostringstream s;
+  s << kPrelude;
+  int lds = 16;
+  for (size_t k = 0; k < bodies.size(); ++k) {
+    s << "namespace g" << k << " {\n" << *bodies[k] << "}\n";
+    lds = std::max(lds, lds_bytes[k]);
+  }
+  s << "struct GroupArgs {\n";
+  for (size_t k = 0; k < bodies.size(); ++k) s << "  g" << k << "::Args a" << k << ";\n";
+  s << "};\n";
+  s << "extern \"C\" __global__ void __launch_bounds__(256) " << kname << "(GroupArgs ar) {\n";
+  s << "  __shared__ __attribute__((aligned(16))) double lds[" << (lds + 7) / 8 << "];\n";
+  unsigned first = 0;
+  for (size_t k = 0; k < bodies.size(); ++k) {
+    s << "  ";
+    if (k + 1 < bodies.size()) s << "if (blockIdx.x < " << first + grids[k] << "u) ";
+    s << "{ g" << k << "::body(ar.a" << k << ", blockIdx.x - " << first << "u, reinterpret_cast<g" << k << "::T*>(lds)); return; }\n";
+    first += grids[k];
+  }
   s << "}\n";
   return s.str();
 }
@@ -436,8 +466,9 @@ bool kept_dims(int n_keep, const int64_t* shape, KeptDims* kd) {
 // One term: which factor moves along P, and the single contracted dim.
 bool term_of(const hgpu_array* a, const hgpu_array* b, int n_keep, const KeptDims& kd, Term* t) {
   const hgpu_array *x = nullptr, *y = nullptr;
-  if (a->strides[kd.dp] != 0 && a->strides[kd.dq] == 0 && b->strides[kd.dp] == 0 && b->strides[kd.dq] != 0) { x = a; y = b; }
-  else if (b->strides[kd.dp] != 0 && b->strides[kd.dq] == 0 && a->strides[kd.dp] == 0 && a->strides[kd.dq] != 0) { x = b; y = a; }
+  // (a factor that moves along neither -- the broadcast zero a recurrence starts from -- fits both places)
+  if (a->strides[kd.dq] == 0 && b->strides[kd.dp] == 0 && (a->strides[kd.dp] != 0 || b->strides[kd.dq] != 0)) { x = a; y = b; }
+  else if (b->strides[kd.dq] == 0 && a->strides[kd.dp] == 0 && (b->strides[kd.dp] != 0 || a->strides[kd.dq] != 0)) { x = b; y = a; }
   else return false;
   // contracted dims: merge what merges in both factors; one dim must remain
   int64_t K = 1, sxk = 0, syk = 0;
@@ -445,7 +476,6 @@ bool term_of(const hgpu_array* a, const hgpu_array* b, int n_keep, const KeptDim
   for (int d = a->rank - 1; d >= n_keep; --d) {
     int64_t e = a->shape[d];
     if (e == 1) continue;
-    if (x->strides[d] == 0 || y->strides[d] == 0) return false;
     if (!have) { K = e; sxk = x->strides[d]; syk = y->strides[d]; have = true; continue; }
     if (x->strides[d] == sxk * K && y->strides[d] == syk * K) { K *= e; continue; }
     return false;
@@ -463,7 +493,54 @@ bool term_of(const hgpu_array* a, const hgpu_array* b, int n_keep, const KeptDim
 
 bool fits_int(int64_t v) { return v > -(1LL << 40) && v < (1LL << 40); }
 
+// The kernel over the given problems, compiled once per source text; nullptr when the compiler refuses it.
+hipFunction_t compiled_kernel(hgpu_ctx* ctx, const std::vector<const std::string*>& bodies, const std::vector<unsigned>& grids, const std::vector<int>& lds_bytes,
+                              const std::string& kname) {
+  std::string src = kernel_source(bodies, grids, lds_bytes, kname);
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c{nullptr, nullptr};
+    std::vector<char> code;
+    int rc = rtc_compile(ctx, src, "small-K product", &code);
+    if (rc && getenv("HORDEAD_GPU_DEBUG")) fprintf(stderr, "hordead_gpu: %s rejected: %s\n", kname.c_str(), hgpu_last_error(ctx));
+    if (!rc) {
+      hipError_t e = hipModuleLoadData(&c.mod, code.data());
+      if (e == hipSuccess) e = hipModuleGetFunction(&c.fn, c.mod, kname.c_str());
+      if (e != hipSuccess) c = Compiled{nullptr, nullptr};
+    }
+    it = cache.emplace(src, c).first;
+  }
+  return it->second.fn;
+}
+
+constexpr size_t kMaxHeld = 256;          // launches held back at most
+constexpr size_t kMaxGroup = 4;           // problems in one kernel at most
+constexpr int64_t kGroupBlocksPerCu = 4;  // a problem with more blocks than this per CU fills the device alone
+
 }  // namespace
+
+namespace hg {
+// A launch that is held back: everything the kernel needs, and the buffers it
+// reads and writes (retained, so that none is handed out again before the launch).
+struct Deferred {
+  std::string body, kname;
+  hipFunction_t fn = nullptr;
+  unsigned grid = 0;
+  int lds_bytes = 0;
+  std::vector<const void*> args;
+  std::vector<hgpu_buffer*> reads, writes;
+  const char* label = nullptr;
+  double bytes = 0, flops = 0;
+  int level = 0;
+};
+
+struct DeferredQueue {
+  std::vector<Deferred> items;
+  std::map<std::string, int> seen;   // how often a set of problems came up together
+  long n_launches = 0, n_grouped = 0;
+};
+}  // namespace hg
 
 namespace hg {
 
@@ -519,52 +596,156 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
   char kname[96];
   snprintf(kname, sizeof kname, "smallk_%s_p%lld_q%lld_k%lld_t%d_in%d_instr%d_out%d", sp.f64 ? "f64" : "f32", (long long)sp.P, (long long)sp.Q, (long long)ktot, n_terms, n_in - 1,
            n_instr, n_out);
-  std::string src = generate(sp, kname);
-  auto& cache = cache_of(ctx);
-  auto it = cache.find(src);
-  if (it == cache.end()) {
-    Compiled c{nullptr, nullptr};
-    std::vector<char> code;
-    int rc = rtc_compile(ctx, src, "small-K product", &code);
-    if (rc && getenv("HORDEAD_GPU_DEBUG")) fprintf(stderr, "hordead_gpu: %s rejected: %s\n", kname, hgpu_last_error(ctx));
-    if (!rc) {
-      hipError_t e = hipModuleLoadData(&c.mod, code.data());
-      if (e == hipSuccess) e = hipModuleGetFunction(&c.fn, c.mod, kname);
-      if (e != hipSuccess) c = Compiled{nullptr, nullptr};
-    }
-    it = cache.emplace(src, c).first;
-  }
-  if (!it->second.fn) return HGPU_OK;
-
-  std::vector<const void*> ar;
-  for (auto& tm : sp.terms) { ar.push_back(tm.x); ar.push_back(tm.y); }
-  for (int i = 0; i < n_in; ++i)
-    if (i != c_slot) ar.push_back(data_ptr(in[i]));
-  for (int o = 0; o < n_out; ++o) ar.push_back(data_ptr(outs[o]));
-  void* args[] = {(void*)ar.data()};
+  Deferred d;
+  d.body = generate_body(sp);
+  d.kname = kname;
   const int64_t nblk = ((sp.P + sp.BP - 1) / sp.BP) * ((sp.Q + sp.BQ - 1) / sp.BQ);
   const int64_t grid = (nblk + 7) / 8 * 8;
   if (grid > 0x7fffffff) return HGPU_OK;
-  const double es = sp.f64 ? 8 : 4;
-  double flops = 2.0 * (double)sp.P * sp.Q * ktot;
-  double bytes = ((double)sp.P + sp.Q) * ktot * es;
+  d.grid = (unsigned)grid;
+  d.lds_bytes = (sp.x_elems + sp.y_elems) * (sp.f64 ? 8 : 4);
+  d.fn = compiled_kernel(ctx, {&d.body}, {d.grid}, {d.lds_bytes}, d.kname);
+  if (!d.fn) return HGPU_OK;
+
+  for (auto& tm : sp.terms) { d.args.push_back(tm.x); d.args.push_back(tm.y); }
   for (int i = 0; i < n_in; ++i)
-    if (i != c_slot) bytes += (sp.in_sp[(size_t)i] ? (double)sp.P : 1.0) * (sp.in_sq[(size_t)i] ? (double)sp.Q : 1.0) * (double)dtype_size(in[i]->dtype);
-  for (int o = 0; o < n_out; ++o) bytes += (double)sp.P * sp.Q * (double)dtype_size(outs[o]->dtype);
-  const char* label = sp.f64 ? "gemm_f64" : "gemm_f32";
+    if (i != c_slot) d.args.push_back(data_ptr(in[i]));
+  for (int o = 0; o < n_out; ++o) d.args.push_back(data_ptr(outs[o]));
+  const double es = sp.f64 ? 8 : 4;
+  d.flops = 2.0 * (double)sp.P * sp.Q * ktot;
+  d.bytes = ((double)sp.P + sp.Q) * ktot * es;
+  for (int i = 0; i < n_in; ++i)
+    if (i != c_slot) d.bytes += (sp.in_sp[(size_t)i] ? (double)sp.P : 1.0) * (sp.in_sq[(size_t)i] ? (double)sp.Q : 1.0) * (double)dtype_size(in[i]->dtype);
+  for (int o = 0; o < n_out; ++o) d.bytes += (double)sp.P * sp.Q * (double)dtype_size(outs[o]->dtype);
+  d.label = sp.f64 ? "gemm_f64" : "gemm_f32";
   if (ctx->profiling && ctx->profile_shapes) {
     char buf[200];
     std::string ks;
     for (auto& tm : sp.terms) ks += (ks.empty() ? "" : "+") + std::to_string(tm.K);
-    snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%sxB1,wholeK,t%dx%d,chunks%d,lds%dK,map(in%d,instr%d,out%d)]", label, (long long)sp.Q, (long long)sp.P, ks.c_str(), sp.BQ,
+    snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%sxB1,wholeK,t%dx%d,chunks%d,lds%dK,map(in%d,instr%d,out%d)]", d.label, (long long)sp.Q, (long long)sp.P, ks.c_str(), sp.BQ,
              sp.BP, (int)sp.chunks.size(), (int)((sp.x_elems + sp.y_elems) * (int)es / 1024), n_in - 1, n_instr, n_out);
-    label = ctx->label_pool.insert(buf).first->c_str();
+    d.label = ctx->label_pool.insert(buf).first->c_str();
   }
-  LaunchGuard lg(ctx, label, bytes, flops);
-  hipError_t err = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+  static const bool hold = getenv("HORDEAD_NO_GROUPED_LAUNCH") == nullptr;
+  if (hold && nblk <= kGroupBlocksPerCu * ctx->num_cu) {
+    // held back: the next small products may be independent of this one
+    for (int t = 0; t < n_terms; ++t) { d.reads.push_back(as[t]->buf); d.reads.push_back(bs[t]->buf); }
+    for (int i = 0; i < n_in; ++i)
+      if (i != c_slot) d.reads.push_back(in[i]->buf);
+    for (int o = 0; o < n_out; ++o) d.writes.push_back(outs[o]->buf);
+    for (auto* b : d.reads) buffer_retain(b);
+    for (auto* b : d.writes) buffer_retain(b);
+    std::lock_guard<std::mutex> lk(ctx->launch_mu);
+    if (!ctx->dq) ctx->dq = new DeferredQueue;
+    if (ctx->dq->items.size() >= kMaxHeld) flush_deferred_locked(ctx);
+    ctx->dq->items.push_back(std::move(d));
+    ctx->dq_pending = true;
+    *handled = true;
+    return HGPU_OK;
+  }
+  LaunchGuard lg(ctx, d.label, d.bytes, d.flops);
+  void* args[] = {(void*)d.args.data()};
+  hipError_t err = hipModuleLaunchKernel(d.fn, d.grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
   if (err != hipSuccess) return check_hip(ctx, err, "small-K product launch");
   *handled = true;
   return HGPU_OK;
+}
+
+// Launches what was held back.  Products are levelled by who reads whose
+// results (arrays are never written twice, so reads-after-writes are the only
+// order there is); the members of one level are independent and go out
+// together, the levels one after another.  For an unrolled recurrence of two
+// layers, issued layer by layer, level k holds step k + 1 of the first layer
+// and step k of the second: the diagonal of the time x layer grid.
+void flush_deferred_locked(hgpu_ctx* ctx) {
+  ctx->dq_pending = false;
+  if (!ctx->dq || ctx->dq->items.empty()) return;
+  std::vector<Deferred> items;
+  items.swap(ctx->dq->items);
+  (void)hipSetDevice(ctx->device);
+  std::map<const hgpu_buffer*, int> written_at;
+  int top = 0;
+  for (auto& d : items) {
+    d.level = 0;
+    for (auto* b : d.reads) {
+      auto it = written_at.find(b);
+      if (it != written_at.end()) d.level = std::max(d.level, it->second + 1);
+    }
+    for (auto* b : d.writes) written_at[b] = d.level;
+    top = std::max(top, d.level);
+  }
+  auto timed_launch = [&](hipFunction_t fn, unsigned grid, const std::vector<const void*>& ar, const char* label, double bytes, double flops) {
+    bool timed = false;
+    if (ctx->profiling && !ctx->cap) {
+      hgpu_ctx::ProfRec r{label, nullptr, nullptr, bytes, flops};
+      if (hipEventCreate(&r.a) == hipSuccess && hipEventCreate(&r.b) == hipSuccess) {
+        (void)hipEventRecord(r.a, ctx->stream);
+        ctx->prof.push_back(r);
+        timed = true;
+      }
+    }
+    void* args[] = {(void*)ar.data()};
+    hipError_t err = hipModuleLaunchKernel(fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+    if (timed) (void)hipEventRecord(ctx->prof.back().b, ctx->stream);
+    if (err != hipSuccess) {
+      int rc = check_hip(ctx, err, "small-K product launch");
+      if (!ctx->deferred_rc) ctx->deferred_rc = rc;
+    }
+  };
+  for (int lv = 0; lv <= top; ++lv) {
+    std::vector<Deferred*> here;
+    for (auto& d : items)
+      if (d.level == lv) here.push_back(&d);
+    for (size_t g0 = 0; g0 < here.size(); g0 += kMaxGroup) {
+      std::vector<Deferred*> grp(here.begin() + (long)g0, here.begin() + (long)std::min(here.size(), g0 + kMaxGroup));
+      hipFunction_t fn = nullptr;
+      std::string gname;
+      if (grp.size() > 1) {
+        // one order for a set of problems, whichever way round they were issued
+        std::stable_sort(grp.begin(), grp.end(), [](const Deferred* a, const Deferred* b) { return a->kname != b->kname ? a->kname < b->kname : a->body < b->body; });
+        gname = "smallk_x" + std::to_string(grp.size());
+        std::string key;
+        for (auto* d : grp) { gname += "__" + d->kname.substr(7); key += d->body + "\x1f"; }
+        // a set seen once may never come again (a second or so of compilation): the second time pays
+        if (++ctx->dq->seen[key] >= 2) {
+          std::vector<const std::string*> bodies;
+          std::vector<unsigned> grids;
+          std::vector<int> lds;
+          for (auto* d : grp) { bodies.push_back(&d->body); grids.push_back(d->grid); lds.push_back(d->lds_bytes); }
+          fn = compiled_kernel(ctx, bodies, grids, lds, gname);
+        }
+      }
+      if (fn) {
+        std::vector<const void*> ar;
+        unsigned grid = 0;
+        double bytes = 0, flops = 0;
+        std::string lab = "group[";
+        for (auto* d : grp) {
+          ar.insert(ar.end(), d->args.begin(), d->args.end());
+          grid += d->grid;
+          bytes += d->bytes;
+          flops += d->flops;
+          lab += (d == grp[0] ? "" : "|") + std::string(d->label);
+        }
+        const char* label = grp[0]->label;
+        if (ctx->profiling && ctx->profile_shapes) label = ctx->label_pool.insert(lab + "]").first->c_str();
+        timed_launch(fn, grid, ar, label, bytes, flops);
+        ctx->dq->n_grouped += (long)grp.size();
+      } else {
+        for (auto* d : grp) timed_launch(d->fn, d->grid, d->args, d->label, d->bytes, d->flops);
+      }
+      ctx->dq->n_launches += fn ? 1 : (long)grp.size();
+    }
+  }
+  for (auto& d : items) {
+    for (auto* b : d.reads) buffer_release(b);
+    for (auto* b : d.writes) buffer_release(b);
+  }
+}
+
+void flush_deferred(hgpu_ctx* ctx) {
+  std::lock_guard<std::mutex> lk(ctx->launch_mu);
+  if (ctx->dq_pending) flush_deferred_locked(ctx);
 }
 
 }  // namespace hg

@@ -211,3 +211,77 @@ def test_condition_of_relu_is_a_result_of_the_layer_call():
     assert fused.counter("contract_sum_map_kept_nodes") == 2        # the two hidden layers
     # products per gradient: 3 forward, 2 input cotangents, 3 weight gradients; none twice
     assert fused.counter("contract_sum_map") + fused.counter("contract") + fused.counter("contract_sum") <= 8
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_two_layer_recurrence_issued_layer_by_layer(gpu, oracle, dt):
+    """h1_t = tanh (wX x_t + wS h1_(t-1) + b1), h2_t = tanh (wX2 h1_t + wS2 h2_(t-1) + b2)
+    (example/MnistRnnRanked2.hs:62-110), all steps of the first layer issued before the
+    second layer's: on the device the launches wait until something reads a result, and
+    step t + 1 of the first layer then shares a kernel with step t of the second, which
+    does not depend on it.  Results against the checker (one call after another) and numpy."""
+    width, batch, k_in, steps = 128, 1000, 28, 6
+    ws = [RNG.uniform(-0.3, 0.3, s).astype(dt) for s in ((width, k_in), (width, width), (width, width), (width, width))]
+    bs = [RNG.uniform(-0.5, 0.5, (width,)).astype(dt) for _ in range(2)]
+    xs = [RNG.uniform(-1, 1, (k_in, batch)).astype(dt) for _ in range(steps)]
+    prog = [(1, O2["add"], 0, 0, 1, 0), (0, O1["tanh"], 0, 2, 0, 0)]
+    want1, want2 = [], []
+    s1 = s2 = np.zeros((width, batch), np.float64)
+    for t in range(steps):
+        s1 = np.tanh(ws[0].astype(np.float64) @ xs[t] + ws[1].astype(np.float64) @ s1 + bs[0].astype(np.float64)[:, None])
+        s2 = np.tanh(ws[2].astype(np.float64) @ s1 + ws[3].astype(np.float64) @ s2 + bs[1].astype(np.float64)[:, None])
+        want1.append(s1)
+        want2.append(s2)
+
+    def run(ctx):
+        w = [ctx.upload(a) for a in ws]
+        b = [ctx.upload(a).replicate([batch]).transpose([1, 0]) for a in bs]
+        zero = ctx.upload(np.zeros((), dt)).replicate([batch]).replicate([width])     # one element for the whole state, as `rrepl sh 0`
+        xa = [ctx.upload(a) for a in xs]
+        h1, h2 = [], []
+        for t in range(steps):
+            terms = [matmul_views(w[0], xa[t]), matmul_views(w[1], h1[-1] if h1 else zero)]
+            h1.append(ctx.contract_sum_map(terms, 2, [None, b[0]], prog, [3])[0])
+        for t in range(steps):
+            terms = [matmul_views(w[2], h1[t]), matmul_views(w[3], h2[-1] if h2 else zero)]
+            h2.append(ctx.contract_sum_map(terms, 2, [None, b[1]], prog, [3])[0])
+        return h1, h2
+
+    tol = TOL[np.dtype(dt)]
+    for attempt in range(2):     # a set of problems is compiled into one kernel the second time it comes up
+        gpu.check(gpu.lib.profile_enable(gpu.h, 2))
+        g1, g2 = run(gpu)
+        got = [a.numpy() for a in g1 + g2]
+        labels = gpu.profile_report()
+        gpu.check(gpu.lib.profile_enable(gpu.h, 0))
+        launches = sum(v[0] for k, v in labels.items() if "wholeK" in k)
+        if attempt == 1:
+            # 6 + 6 problems on 7 diagonals: the two ends alone, five pairs
+            assert launches == steps + 1, labels
+            assert sum(v[0] for k, v in labels.items() if k.startswith("group[")) == steps - 1, labels
+    c1, c2 = run(oracle)
+    chk = [a.numpy() for a in c1 + c2]
+    for g, c, w in zip(got, chk, want1 + want2):
+        assert g.dtype == np.dtype(dt) and rel(g, c) <= tol * steps and rel(g, w) <= 4 * tol * steps
+
+
+@pytest.mark.gpu
+def test_held_back_products_come_before_whatever_reads_them(gpu, oracle):
+    """A held-back product followed by other work on its result (an elementwise call, a
+    product too long for the compiled kernel, a download), and by a release of its inputs
+    before anything has run."""
+    m, n, k = 64, 1000, 64
+    w = RNG.uniform(-0.3, 0.3, (m, k)).astype(np.float32)
+    x = RNG.uniform(-1, 1, (k, n)).astype(np.float32)
+    res = []
+    for ctx in (gpu, oracle):
+        wa, xa = ctx.upload(w), ctx.upload(x)
+        c = ctx.contract_sum_map([matmul_views(wa, xa)], 2, [None], [], [0])[0]
+        del wa, xa                                             # the queue holds what the launch reads
+        e = ctx.fused_map([c], [(0, O1["tanh"], 0, 0, 0, 0)], [1])[0]
+        d = ctx.contract_sum_map([matmul_views(ctx.upload(w.T.copy()), c)], 2, [None], [], [0])[0]   # reads c, still held back
+        res.append((c.numpy(), e.numpy(), d.numpy()))
+    want_c = w.astype(np.float64) @ x
+    for g, c, want in zip(res[0], res[1], (want_c, np.tanh(want_c), w.T.astype(np.float64) @ want_c)):
+        assert rel(g, c) <= 1e-5 and rel(g, want) <= 4e-5
