@@ -33,6 +33,13 @@
 //
 // Shapes the kernel does not cover (long K, batched or higher-rank products,
 // too many terms) are computed by the other entry points one after another.
+//
+// A problem of this size cannot fill the device and pays a launch and a round
+// of memory latency for a few microseconds of arithmetic, so launches are held
+// back (DeferredQueue) until something else needs the stream, and held-back
+// problems that do not read one another's results run as one kernel: each
+// problem's code in a namespace of its own, the first blocks of the grid for
+// problem 0, the next for problem 1, ...
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
@@ -719,13 +726,16 @@ void flush_deferred_locked(hgpu_ctx* ctx) {
         std::vector<const void*> ar;
         unsigned grid = 0;
         double bytes = 0, flops = 0;
-        std::string lab = "group[";
+        std::string lab = std::string(grp[0]->label).substr(0, std::string(grp[0]->label).find('[')) + "[group:";   // same family as its members
         for (auto* d : grp) {
           ar.insert(ar.end(), d->args.begin(), d->args.end());
           grid += d->grid;
           bytes += d->bytes;
           flops += d->flops;
-          lab += (d == grp[0] ? "" : "|") + std::string(d->label);
+          std::string in(d->label);
+          size_t at = in.find('[');
+          if (at != std::string::npos && in.back() == ']') in = in.substr(at + 1, in.size() - at - 2);
+          lab += (d == grp[0] ? "" : "|") + in;
         }
         const char* label = grp[0]->label;
         if (ctx->profiling && ctx->profile_shapes) label = ctx->label_pool.insert(lab + "]").first->c_str();

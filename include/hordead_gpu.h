@@ -309,7 +309,14 @@ int hgpu_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, i
  * kept shape has two non-unit dims this is one kernel compiled for the shapes,
  * with the whole contracted dim of a term in LDS; otherwise the single entry
  * points run one after another.  Results equal theirs up to the order of the
- * floating-point sums. */
+ * floating-point sums.
+ * The compiled kernel's launch may be held back until the next call that
+ * needs the stream (any other launch, copy, synchronisation, hgpu_stream, the
+ * ends of a graph capture): held-back products that do not read one another's
+ * results then go out as one kernel -- step t + 1 of the first layer of an
+ * unrolled recurrence with step t of the second.  The order of results as the
+ * stream sees it is the order of the calls; a launch error that shows up late
+ * is returned by hgpu_sync. */
 int hgpu_contract_sum_map(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* a, const hgpu_array* const* b, int n_keep,
                           int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
                           int n_out, const int* out_slots, hgpu_array** outs);
