@@ -55,6 +55,7 @@ SIGNATURES = {
     "assign": (I, [P, P, P]),
     "fused_map": (I, [P, I, PP, I, P, I, IP, PP]),
     "contract_sum_map": (I, [P, I, PP, PP, I, I, PP, I, P, I, IP, PP]),
+    "fused_map_dimsum": (I, [P, I, PP, I, P, I, IP, PP, I, I, PP]),
 }
 # exported by the GPU library only
 GPU_ONLY = {
@@ -160,6 +161,16 @@ class Ctx:
         outs = (C.c_void_p * len(out_slots))()
         self.check(self.lib.fused_map(self.h, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs))
         return [Array(self, C.c_void_p(o)) for o in outs]
+
+    def fused_map_dimsum(self, inputs, prog, out_slots, sum_slot, keep_dim):
+        """hgpu_fused_map_dimsum: (outs, sum of slot sum_slot over every dim but keep_dim)."""
+        ins = (C.c_void_p * len(inputs))(*[p.h for p in inputs])
+        flat = (C.c_int32 * (6 * len(prog)))(*[int(x) for q in prog for x in q])
+        slots = (C.c_int * len(out_slots))(*out_slots)
+        outs = (C.c_void_p * len(out_slots))()
+        sm = C.c_void_p()
+        self.check(self.lib.fused_map_dimsum(self.h, len(inputs), ins, len(prog), flat, len(out_slots), slots, outs, sum_slot, keep_dim, C.byref(sm)))
+        return [Array(self, C.c_void_p(o)) for o in outs], Array(self, sm)
 
     def contract_map(self, a, b, n_keep, inputs, prog, out_slots, ext=None):
         """hgpu_contract_map: `inputs` holds None where the contraction of a and b stands;

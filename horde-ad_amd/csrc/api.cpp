@@ -12,7 +12,7 @@ extern "C" const hgpu_api* hgpu_get_api(void) {
       hgpu_contract,    hgpu_argminmax_last, hgpu_iota,   hgpu_concat,     hgpu_gather,      hgpu_scatter_add,
       hgpu_onehot,      hgpu_fused_map, hgpu_scatter_affine,
       hgpu_capture_begin, hgpu_capture_end, hgpu_graph_launch, hgpu_graph_destroy, hgpu_overwrite, hgpu_contract_sum, hgpu_assign, hgpu_extremum_last, hgpu_fused_extremum, hgpu_fused_sum,
-      hgpu_contract_map, hgpu_contract_operands, hgpu_fused_map_sums, hgpu_contract_sum_map,
+      hgpu_contract_map, hgpu_contract_operands, hgpu_fused_map_sums, hgpu_contract_sum_map, hgpu_fused_map_dimsum,
   };
   return &api;
 }

@@ -16,6 +16,7 @@
 // merged index space of the inputs (same decomposition as the eager kernels).
 #include <hip/hiprtc.h>
 
+#include <memory>
 #include <sstream>
 
 #include "common.hpp"
@@ -60,8 +61,14 @@ struct FDims {
 
 }  // namespace
 
-extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
-                              int n_out, const int* out_slots, hgpu_array** outs) {
+namespace hg {
+int sum_partials(hgpu_ctx* ctx, int dtype, int64_t n, int parts, const void* part, void* out);
+}
+
+// hgpu_fused_map, and with sum_slot >= 0 hgpu_fused_map_dimsum: the same pass
+// also adds up slot sum_slot over every dim but keep_dim.
+static int fused_map_impl(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int n_out, const int* out_slots,
+                          hgpu_array** outs, int sum_slot, int keep_dim, hgpu_array** sum) {
   if (!ctx || !in || !prog || !out_slots || !outs) return HGPU_ERR_INVALID;
   if (n_in < 1 || n_in > kMaxIn || n_out < 1 || n_out > kMaxOut || n_instr < 1 || n_instr > kMaxInstr)
     return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map: %d inputs, %d instructions, %d outputs", n_in, n_instr, n_out);
@@ -87,6 +94,16 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     return HGPU_OK;
   }
 
+  // the sum over all dims but keep_dim: blocks take (element of keep_dim, chunk of the rest)
+  int64_t dsO = 1, dsC = 1, dsI = 1;
+  if (sum_slot >= 0) {
+    if (sum_slot >= n_in + n_instr || keep_dim < 0 || keep_dim >= a0->rank || !sum) { release_all(); return fail(ctx, HGPU_ERR_INVALID, "fused_map_dimsum: bad sum slot or dim"); }
+    if (dt[(size_t)sum_slot] != HGPU_F64 && dt[(size_t)sum_slot] != HGPU_F32) { release_all(); return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map_dimsum: sums of floating-point values only"); }
+    for (int d = 0; d < keep_dim; ++d) dsO *= a0->shape[d];
+    dsC = a0->shape[keep_dim];
+    for (int d = keep_dim + 1; d < a0->rank; ++d) dsI *= a0->shape[d];
+  }
+
   // layout class of every input: 'd' dense, 's' one element broadcast, 'g' general
   std::string layout((size_t)n_in, 'g');
   bool all_simple = true;
@@ -104,6 +121,7 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   for (int i = 0; i < n_in; ++i) widest = std::max(widest, dtype_size(in[i]->dtype));
   for (int o = 0; o < n_out; ++o) widest = std::max(widest, dtype_size(res[(size_t)o]->dtype));
   vec = (int)(16 / widest);
+  if (sum_slot >= 0) all_simple = false;     // the summing kernel wants coordinates
   if (!all_simple) vec = 1;
 
   // general views: the dims merged jointly over all inputs.  For large arrays
@@ -167,15 +185,32 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     }
   }
 
+  const int dsum_es = sum_slot >= 0 ? (int)dtype_size(dt[(size_t)sum_slot]) : 0;
+  int64_t ds_chunks = 1, ds_ch = 0;     // chunks of the summed index range per kept element, vector groups per chunk
+  if (sum_slot >= 0) {
+    if (!bake || dsC > 65536) { release_all(); return fail(ctx, HGPU_ERR_UNSUPPORTED, "fused_map_dimsum: array too small, too large or too many sums"); }
+    if (dsI % gvec != 0) {
+      gvec = 1;
+      std::fill(inner.begin(), inner.end(), 'x');
+    }
+    const int64_t groups = dsO * (dsI / gvec);      // per kept element
+    // 32 blocks per CU: measured on the first convolution layer's cotangent (16 x 784,000 fp64), 8 / 16 / 32 / 64 per CU: 42 / 39 / 36 / 38 us
+    ds_chunks = std::max<int64_t>(1, std::min<int64_t>(((int64_t)ctx->num_cu * 32 + dsC - 1) / dsC, groups / 512));
+    ds_ch = (groups + ds_chunks - 1) / ds_chunks;
+    ds_chunks = (groups + ds_ch - 1) / ds_ch;
+  }
+
   // ---- source
   std::ostringstream s;
   s << kPrelude;
   if (!all_simple) s << "struct FDims { int nd; i64 shape[" << HG_KDIMS << "]; i64 st[" << kMaxIn << "][" << HG_KDIMS << "]; };\n";
   s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
-  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_map(i64 n";
+  const char* kernel_name = sum_slot >= 0 ? "fused_map_dimsum" : "fused_map";
+  s << "extern \"C\" __global__ void __launch_bounds__(256) " << kernel_name << "(i64 n";
   if (!all_simple && !bake) s << ", FDims d";
   for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
   for (int o = 0; o < n_out; ++o) s << ", " << ctype(res[(size_t)o]->dtype) << "* __restrict__ o" << o;
+  if (sum_slot >= 0) s << ", " << ctype(dt[(size_t)sum_slot]) << "* __restrict__ part";
   s << ") {\n";
   s << "  const i64 step = (i64)gridDim.x * 256;\n";
   for (int i = 0; i < n_in; ++i)
@@ -227,9 +262,21 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     emit_program("    ", "_t");
     for (int o = 0; o < n_out; ++o) s << "    o" << o << "[t] = v" << out_slots[o] << "_t;\n";
     s << "  }\n";
-  } else if (bake && gvec > 1) {
+  } else if (bake && (gvec > 1 || sum_slot >= 0)) {
     const int W = gvec, in_d = fd.nd - 1;
-    s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n / " << W << "; i += step) {\n";
+    if (sum_slot >= 0) {
+      // a block adds up one chunk of one kept element; a lane's groups lie 256 apart in the chunk
+      const long long IV = dsI / W, groups = dsO * IV;
+      s << "  __shared__ double red[4];\n";
+      s << "  const unsigned ck = blockIdx.x % " << dsC << "u, chunk = blockIdx.x / " << dsC << "u;\n";
+      s << "  const unsigned j1 = (chunk + 1u) * " << ds_ch << "u < " << groups << "u ? (chunk + 1u) * " << ds_ch << "u : " << groups << "u;\n";
+      s << "  double acc = 0;\n";
+      s << "  for (unsigned j = chunk * " << ds_ch << "u + threadIdx.x; j < j1; j += 256u) {\n";
+      s << "    const unsigned jo = j / " << IV << "u;\n";
+      s << "    const i64 i = ((i64)jo * " << dsC << " + ck) * " << IV << " + (j - jo * " << IV << "u);\n";
+    } else {
+      s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n / " << W << "; i += step) {\n";
+    }
     s << "    unsigned r = (unsigned)i;\n";
     for (int q = in_d; q >= 0; --q) {
       const long long ext = q == in_d ? fd.shape[q] / W : fd.shape[q];
@@ -260,10 +307,20 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
       }
       emit_program("      ", suf);
       for (int o = 0; o < n_out; ++o) s << "      r" << o << ".v[" << e << "] = v" << out_slots[o] << suf << ";\n";
+      if (sum_slot >= 0) s << "      acc += (double)v" << sum_slot << suf << ";\n";
       s << "    }\n";
     }
     for (int o = 0; o < n_out; ++o) s << "    reinterpret_cast<Vec<" << ctype(res[(size_t)o]->dtype) << ", " << W << ">*>(o" << o << ")[i] = r" << o << ";\n";
     s << "  }\n";
+    if (sum_slot >= 0) {
+      s << "  for (int off = 32; off > 0; off >>= 1) {\n"
+           "    unsigned long long u = *reinterpret_cast<unsigned long long*>(&acc);\n"
+           "    unsigned lo = __shfl_down((unsigned)(u & 0xffffffffu), off, 64), hi = __shfl_down((unsigned)(u >> 32), off, 64);\n"
+           "    unsigned long long w = ((unsigned long long)hi << 32) | lo;\n"
+           "    acc += *reinterpret_cast<double*>(&w);\n  }\n";
+      s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n  __syncthreads();\n";
+      s << "  if (threadIdx.x == 0) part[(i64)chunk * " << dsC << " + ck] = (" << ctype(dt[(size_t)sum_slot]) << ")((red[0] + red[1]) + (red[2] + red[3]));\n";
+    }
   } else if (bake) {
     s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {\n";
     s << "    unsigned r = (unsigned)i;\n";
@@ -308,7 +365,7 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   s << "}\n";
   std::string src = s.str();
 
-  const char* label = "fused_map";
+  const char* label = kernel_name;
   if (ctx->profiling && ctx->profile_shapes) {
     std::string sh;
     for (int d = 0; d < a0->rank; ++d) sh += (d ? "x" : "") + std::to_string(a0->shape[d]);
@@ -318,15 +375,16 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
       if (layout[(size_t)i] == 'g')
         for (int d = 0; d < in[i]->rank; ++d) gst += (d ? ":" : ",g") + std::to_string(in[i]->strides[d]);
     char buf[200];
-    snprintf(buf, sizeof buf, "fused_map[%s,in%d(%s),instr%d(k%d.op%d..),out%d,vec%d,dt%d%s]", sh.c_str(), n_in, layout.c_str(), n_instr, prog[0].kind, prog[0].op, n_out, all_simple ? vec : gvec, a0->dtype, gst.c_str());
+    snprintf(buf, sizeof buf, "%s[%s,in%d(%s),instr%d(k%d.op%d..),out%d,vec%d,dt%d%s]", kernel_name, sh.c_str(), n_in, layout.c_str(), n_instr, prog[0].kind, prog[0].op, n_out, all_simple ? vec : gvec, a0->dtype, gst.c_str());
     label = ctx->label_pool.insert(buf).first->c_str();
   }
-  LaunchGuard lg(ctx, label, 0, 0);
+  std::unique_ptr<LaunchGuard> guard(new LaunchGuard(ctx, label, 0, 0));   // ends before the partial sums' own launch
+  LaunchGuard& lg = *guard;
   auto& cache = cache_of(ctx);
   auto it = cache.find(src);
   if (it == cache.end()) {
     Compiled c;
-    int rc = compile(ctx, src, &c);
+    int rc = compile(ctx, src, &c, kernel_name);
     if (rc) { release_all(); return rc; }
     it = cache.emplace(src, c).first;
   }
@@ -355,10 +413,39 @@ extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   for (int o = 0; o < n_out; ++o) { optrs[(size_t)o] = data_ptr(res[(size_t)o]); args.push_back(&optrs[(size_t)o]); }
   int64_t work = all_simple ? (n + vec - 1) / vec : n / gvec;
   unsigned grid = grid_for(work, 256, ctx->num_cu * 16);
+  hgpu_array* sums = nullptr;
+  hgpu_buffer* part = nullptr;
+  void* part_ptr = nullptr;
+  if (sum_slot >= 0) {
+    int rc = new_dense(ctx, dt[(size_t)sum_slot], 1, &dsC, &sums);
+    if (!rc && ds_chunks > 1) rc = buffer_alloc(ctx, (size_t)(dsC * ds_chunks) * (size_t)dsum_es, &part);
+    if (rc) { if (sums) hgpu_release(sums); release_all(); return rc; }
+    part_ptr = part ? part->ptr : data_ptr(sums);
+    args.push_back(&part_ptr);
+    grid = (unsigned)(dsC * ds_chunks);
+  }
   hipError_t e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
-  if (e != hipSuccess) { release_all(); return check_hip(ctx, e, "fused_map launch"); }
+  if (e != hipSuccess) { if (part) buffer_release(part); if (sums) hgpu_release(sums); release_all(); return check_hip(ctx, e, "fused_map launch"); }
+  guard.reset();
+  if (part) {
+    int rc = hg::sum_partials(ctx, dt[(size_t)sum_slot], dsC, (int)ds_chunks, part->ptr, data_ptr(sums));
+    buffer_release(part);
+    if (rc) { hgpu_release(sums); release_all(); return rc; }
+  }
   for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
+  if (sum_slot >= 0) *sum = sums;
   return HGPU_OK;
+}
+
+extern "C" int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
+                              int n_out, const int* out_slots, hgpu_array** outs) {
+  return fused_map_impl(ctx, n_in, in, n_instr, prog, n_out, out_slots, outs, -1, 0, nullptr);
+}
+
+extern "C" int hgpu_fused_map_dimsum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int n_out, const int* out_slots,
+                                     hgpu_array** outs, int sum_slot, int keep_dim, hgpu_array** sum) {
+  if (!sum || sum_slot < 0) return HGPU_ERR_INVALID;
+  return fused_map_impl(ctx, n_in, in, n_instr, prog, n_out, out_slots, outs, sum_slot, keep_dim, sum);
 }
 
 // The first extremum of an elementwise program's result along its trailing

@@ -37,6 +37,7 @@ struct Backend {
   std::map<std::pair<int, uint64_t>, std::shared_ptr<ArrHolder>> const_cache; // (dtype, value bits)
   bool capturing = false;   // between hh_capture_begin and hh_capture_end
   bool fuse = true;   // defer elementwise operations into fused programs (when the provider has fused_map)
+  std::vector<std::weak_ptr<ArrHolder>> pending_dimsums;   // sums over all dims but one of an expression, not yet taken (ArrHolder::ones_b)
   std::vector<std::weak_ptr<ArrHolder>> pending_sums;   // sums of all elements of an expression, not yet taken (ArrHolder::ssrc)
   std::map<std::string, int64_t> counters;   // how often each rewrite onto a fused entry point was taken (diagnostic)
   void check(int rc) const;
@@ -70,6 +71,12 @@ struct ArrHolder {
   // cotangent of a parameter used once per step of an unrolled recurrence):
   // written out by one grouped launch when the provider has contract_sum.
   std::vector<std::pair<std::shared_ptr<ArrHolder>, std::shared_ptr<ArrHolder>>> more;
+  // fb is all ones: the value is the SUM of fa over its trailing dims.  When fa
+  // is a transposed view of an expression (a bias's cotangent: the layer's
+  // cotangent summed over batch, height and width) the sum waits for the pass
+  // that writes the expression out and is taken in that pass
+  // (Backend::pending_dimsums, hgpu_fused_map_dimsum).
+  bool ones_b = false;
   // A pending contraction that is a transpose of another pending contraction
   // remembers it: if anyone else still wants the original, the original is
   // computed once and this one becomes a view of it.

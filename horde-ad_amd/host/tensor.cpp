@@ -419,14 +419,14 @@ struct Program {
 };
 
 bool single_contraction(const ArrHolder* p) {
-  return !p->h && p->ekind < 0 && p->fa && p->fb && p->keep >= 1 && p->more.empty() && !p->origin && !p->vsrc && p->pieces.empty() && !p->mv_inner;
+  return !p->h && p->ekind < 0 && p->fa && p->fb && p->keep >= 1 && p->more.empty() && !p->origin && !p->vsrc && p->pieces.empty() && !p->mv_inner && !p->ones_b;
 }
 
 // Post-order walk: materialised values (and pending contractions, which are
 // forced here) become inputs, pending elementwise nodes become instructions.
 // a pending contraction of two arrays, or a pending sum of such
 bool contraction_or_sum(const ArrHolder* p) {
-  return !p->h && p->ekind < 0 && p->fa && p->fb && p->keep >= 1 && !p->origin && !p->vsrc && p->pieces.empty() && !p->mv_inner && !p->ssrc && !p->probe;
+  return !p->h && p->ekind < 0 && p->fa && p->fb && p->keep >= 1 && !p->origin && !p->vsrc && p->pieces.empty() && !p->mv_inner && !p->ssrc && !p->probe && !p->ones_b;
 }
 
 int visit(Program& pg, ArrHolder* p) {
@@ -612,6 +612,38 @@ static bool products_then_program(Backend* be, const std::vector<ArrHolder*>& ro
   return true;
 }
 
+// A view that brings ONE dim of its source to the front and leaves the others
+// in order (offset 0, nothing repeated or left out): that dim, counted in the
+// dims of the expression that computes the source; else -1.
+static int front_dim_of_view(const ArrHolder* v) {
+  if (!v || v->h || !v->vsrc || !v->vlo.empty() || v->vmeta.offset != 0 || v->probe) return -1;   // (an expression over viewed leaves carries the view as a note)
+  T src(v->vsrc);
+  const Shape M = src.shape();
+  const Shape& vs = v->vmeta.shape;
+  const Shape& vt = v->vmeta.strides;
+  if (M.empty() || vs.size() != M.size()) return -1;
+  Shape ds(M.size());
+  int64_t acc = 1;
+  for (size_t i = M.size(); i-- > 0;) { ds[i] = acc; acc *= M[i]; }
+  int d = -1;
+  for (size_t i = 0; i < M.size(); ++i)
+    if (vs[0] == M[i] && vt[0] == ds[i] && M[i] > 1) { d = (int)i; break; }
+  if (d < 0) return -1;
+  size_t k = 1;
+  for (size_t i = 0; i < M.size(); ++i) {
+    if ((int)i == d) continue;
+    if (vs[k] != M[i] || (M[i] > 1 && vt[k] != ds[i])) return -1;
+    ++k;
+  }
+  if (!src.pending_merged()) return d;
+  // the source is an expression over a refined index space: its dim d must be one dim there too
+  const auto& g = src.holder()->mv_groups;
+  if ((size_t)d >= g.size() || g[(size_t)d] != 1) return -1;
+  int rd = 0;
+  for (int i = 0; i < d; ++i) rd += g[(size_t)i];
+  return rd;
+}
+
 static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
   std::vector<const hgpu_array*> ins;
   std::vector<hgpu_fused_instr> prog;
@@ -660,7 +692,41 @@ static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
   } else if (sums.empty()) {
     number_program(roots, &ins, &prog, &outs_slot);
     int n_in = (int)ins.size(), n_instr = (int)prog.size();
-    be->check(be->api->fused_map(be->ctx, n_in, ins.data(), n_instr, prog.data(), (int)roots.size(), outs_slot.data(), outs.data()));
+    // A pending sum over all dims but one of what is being written out (a
+    // bias's cotangent) is taken in the same pass.
+    bool done = false;
+    if (api->struct_size >= offsetof(hgpu_api, fused_map_dimsum) + sizeof(api->fused_map_dimsum) && api->fused_map_dimsum && n_instr >= 1) {
+      auto& pd = be->pending_dimsums;
+      pd.erase(std::remove_if(pd.begin(), pd.end(), [](const std::weak_ptr<ArrHolder>& w) { auto q = w.lock(); return !q || q->h || !q->ones_b; }), pd.end());
+      for (auto& w : pd) {
+        auto q = w.lock();
+        if (!q || !q->fa || !q->more.empty() || q->keep != 1) continue;
+        const ArrHolder* v = q->fa.get();
+        if (v->h || !v->vsrc) continue;
+        const ArrHolder* src = v->vsrc.get();
+        const ArrHolder* e = src->mv_inner ? src->mv_inner.get() : src;
+        size_t ri = 0;
+        while (ri < roots.size() && roots[ri] != e) ++ri;
+        if (ri == roots.size()) continue;
+        const int d = front_dim_of_view(v);
+        if (d < 0) continue;
+        hgpu_array* so = nullptr;
+        int rc = api->fused_map_dimsum(be->ctx, n_in, ins.data(), n_instr, prog.data(), (int)roots.size(), outs_slot.data(), outs.data(), outs_slot[ri], d, &so);
+        if (rc == HGPU_OK) {
+          be->counters["fused_map_dimsum"]++;
+          q->h = so;
+          q->fa.reset();
+          q->fb.reset();
+          q->keep = -1;
+          q->ones_b = false;
+          done = true;
+        } else if (rc != HGPU_ERR_UNSUPPORTED) {
+          be->check(rc);
+        }
+        break;
+      }
+    }
+    if (!done) be->check(be->api->fused_map(be->ctx, n_in, ins.data(), n_instr, prog.data(), (int)roots.size(), outs_slot.data(), outs.data()));
   }
   for (size_t i = 0; i < roots.size(); ++i) {
     ArrHolder* r = roots[i];
@@ -871,7 +937,7 @@ void ArrHolder::force() {
     p = transpose(T(origin), origin_perm);
   } else {
     T fbt(fb);
-    p = contract_now(T(fa), &fbt, keep);
+    p = ones_b ? contract_now(T(fa), nullptr, keep) : contract_now(T(fa), &fbt, keep);   // a sum nobody's pass has taken along
   }
   be->check(be->api->retain(p.h()));
   h = p.h();
@@ -879,6 +945,7 @@ void ArrHolder::force() {
   fb.reset();
   origin.reset();
   keep = -1;
+  ones_b = false;
 }
 
 // Two pending contractions can wait as one pending sum when their factors have
@@ -1255,6 +1322,20 @@ T contract(const T& a, const T* b, int n_keep) {
   if (!b && n_keep >= 1 && n_keep < a.rank() && a.pending_view() && fuses(a.be()) && a.holder()->vlo.empty() && T(a.holder()->vsrc).pending_product() &&
       (a.dtype() == HGPU_F64 || a.dtype() == HGPU_F32) && holds_pending_contraction(a.holder()->vsrc.get()))
     return lazy_contract(a, broadcast_scalar(constant(a.be(), a.dtype(), 1.0), a.shape()), n_keep);
+  // The sum over all dims but one of an expression seen through a transpose (the
+  // cotangent of a bias that was replicated and transposed into a layer's
+  // shape): when somebody writes the expression out, the sum is taken in that
+  // pass; it waits for that (forced on its own it is what it would be now).
+  if (!b && n_keep == 1 && (a.pending_view() || (a.pending_expr() && a.holder()->vsrc)) && fuses(a.be()) && (a.dtype() == HGPU_F64 || a.dtype() == HGPU_F32) && a.size() > 0 &&
+      expression_like(T(a.holder()->vsrc)) && front_dim_of_view(a.holder().get()) >= 0) {
+    const hgpu_api* api = a.be()->api;
+    if (api->struct_size >= offsetof(hgpu_api, fused_map_dimsum) + sizeof(api->fused_map_dimsum) && api->fused_map_dimsum) {
+      T r = lazy_contract(a, broadcast_scalar(constant(a.be(), a.dtype(), 1.0), a.shape()), 1);
+      r.holder()->ones_b = true;
+      a.be()->pending_dimsums.push_back(r.holder());
+      return r;
+    }
+  }
   // ssum0 of a pending expression: summed while it is evaluated, never written
   if (!b && n_keep == 0 && a.pending_expr() && a.size() > 0 && (a.dtype() == HGPU_F64 || a.dtype() == HGPU_F32)) {
     Backend* be = a.be();

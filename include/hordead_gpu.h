@@ -240,6 +240,20 @@ int hgpu_fused_map(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_i
  * HGPU_ERR_UNSUPPORTED: run hgpu_fused_map and hgpu_fused_sum). */
 int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
                         int n_out, const int* out_slots, hgpu_array** outs, int n_sum, const int* sum_slots, hgpu_array** sums);
+
+/* hgpu_fused_map that also sums one slot over every dim but one:
+ * sum[c] = the sum of slot sum_slot over all elements whose index along dim
+ * keep_dim is c (a rank-1 array of the slot's floating-point type, accumulated
+ * in double in an order fixed by the shape), from the pass that writes outs.
+ * The convolution layers add their bias as
+ * `stranspose @'[0, 3, 1, 2] $ sreplicate $ sreplicate $ sreplicate bias`
+ * (example/MnistCnnShaped2.hs:57-63): the bias's cotangent is the layer's
+ * cotangent summed over batch, height and width, and that cotangent is written
+ * out anyway for the kernel's gradient.  HGPU_ERR_UNSUPPORTED for arrays of
+ * fewer than 2^18 or more than 2^31 elements (run hgpu_fused_map and
+ * hgpu_contract). */
+int hgpu_fused_map_dimsum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
+                          int n_out, const int* out_slots, hgpu_array** outs, int sum_slot, int keep_dim, hgpu_array** sum);
 /* The first extremum of such a program's result along its trailing n_reduce
  * dims (taken together, row-major), evaluated on the fly: the result itself is
  * never written.  values / indices get the leading dims' shape; an index
@@ -519,6 +533,7 @@ typedef struct hgpu_api {
   int (*fused_map_sums)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, const int*, hgpu_array**, int, const int*, hgpu_array**);
   int (*contract_sum_map)(hgpu_ctx*, int, const hgpu_array* const*, const hgpu_array* const*, int, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int,
                          const int*, hgpu_array**);
+  int (*fused_map_dimsum)(hgpu_ctx*, int, const hgpu_array* const*, int, const hgpu_fused_instr*, int, const int*, hgpu_array**, int, int, hgpu_array**);
 } hgpu_api;
 
 /* The table of this library's own entry points. */

@@ -870,6 +870,34 @@ int horc_fused_map_sums(hgpu_ctx* c, int n_in, const hgpu_array* const* in, int 
   return rc;
 }
 
+// the program by horc_fused_map; the sum of one slot over all dims but keep_dim: that slot written
+// out, keep_dim brought to the front (horc_transpose), every other dim summed (horc_contract)
+int horc_fused_map_dimsum(hgpu_ctx* c, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int n_out, const int* out_slots,
+                          hgpu_array** outs, int sum_slot, int keep_dim, hgpu_array** sum) {
+  if (!sum || sum_slot < 0 || sum_slot >= n_in + n_instr) return fail(c, HGPU_ERR_INVALID, "fused_map_dimsum: bad sum slot");
+  int rc = horc_fused_map(c, n_in, in, n_instr, prog, n_out, out_slots, outs);
+  if (rc) return rc;
+  hgpu_array *v = nullptr, *t = nullptr;
+  if (sum_slot < n_in) { v = const_cast<hgpu_array*>(in[sum_slot]); horc_retain(v); }
+  else rc = horc_fused_map(c, n_in, in, n_instr, prog, 1, &sum_slot, &v);
+  if (!rc) {
+    const int rank = horc_rank(v);
+    if (keep_dim < 0 || keep_dim >= rank) rc = fail(c, HGPU_ERR_INVALID, "fused_map_dimsum: bad dim");
+    if (!rc) {
+      std::vector<int> perm{keep_dim};
+      for (int d = 0; d < rank; ++d)
+        if (d != keep_dim) perm.push_back(d);
+      rc = horc_transpose(c, v, (int)perm.size(), perm.data(), &t);
+    }
+    if (!rc) rc = horc_contract(c, t, nullptr, 1, sum);
+  }
+  if (t) horc_release(t);
+  if (v) horc_release(v);
+  if (rc)
+    for (int o = 0; o < n_out; ++o) { horc_release(outs[o]); outs[o] = nullptr; }
+  return rc;
+}
+
 // sum of contractions (terms may differ in their contracted dims), then the program: each term by
 // horc_contract, the terms added in order, the program by horc_fused_map
 int horc_contract_sum_map(hgpu_ctx* c, int n_terms, const hgpu_array* const* a, const hgpu_array* const* b, int n_keep, int n_in, const hgpu_array* const* in,
@@ -919,6 +947,7 @@ const hgpu_api* horc_get_api(void) {
       nullptr,   // no contract_operands
       nullptr,   // no fused_map_sums
       nullptr,   // no contract_sum_map
+      nullptr,   // no fused_map_dimsum
   };
   return &api;
 }
@@ -932,6 +961,7 @@ const hgpu_api* horc_get_api_fused(void) {
   api.contract_operands = horc_contract_operands;
   api.fused_map_sums = horc_fused_map_sums;
   api.contract_sum_map = horc_contract_sum_map;
+  api.fused_map_dimsum = horc_fused_map_dimsum;
   return &api;
 }
 

@@ -238,3 +238,35 @@ def test_host_rewrites_gradients_onto_contract_operands():
         for g0, g1 in zip(res[0][1], res[1][1]):
             assert np.array_equal(g0, g1), wl.name
     assert plain.counter("contract_operands") == 0 and fused.counter("contract_operands") >= 5
+
+
+def test_host_takes_a_bias_cotangent_in_the_pass_that_writes_the_layer_cotangent():
+    """`stranspose @'[0, 3, 1, 2] $ sreplicate $ sreplicate $ sreplicate bias`
+    (example/MnistCnnShaped2.hs:57-63) has the layer's cotangent, transposed
+    back and summed over batch, height and width, as the bias's cotangent.  The
+    sum waits: when the cotangent expression is written out first (the kernel
+    gradient needs it as an array) the sum comes from that pass
+    (hgpu_fused_map_dimsum, on the checker's fused table defined as program,
+    transpose, sum); asked for first, or without that entry point, it is a pass
+    of its own.  All against numpy."""
+    H = pkg.hostapi
+    rng = np.random.default_rng(3)
+    x, y = rng.standard_normal((5, 4, 6, 7)), rng.standard_normal((5, 4, 6, 7))
+    want = x * y + x
+    for table, order, rides in [("get_api", "expression first", 0), ("get_api_fused", "expression first", 1), ("get_api_fused", "sum first", 0)]:
+        host = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_", api_table=table))
+        e = host.sconcrete(x) * host.sconcrete(y) + host.sconcrete(x)
+        s = e.stranspose([0, 2, 3, 1]).ssumN(3)
+        assert s.shape == (4,)
+        if order == "expression first":
+            ev, sv = e.numpy(), s.numpy()
+        else:
+            sv, ev = s.numpy(), e.numpy()
+        assert host.counter("fused_map_dimsum") == rides, (table, order)
+        assert np.array_equal(ev, want)
+        assert np.max(np.abs(sv - want.sum(axis=(0, 2, 3)))) <= 1e-12 * np.abs(want).sum(axis=(0, 2, 3)).max()
+    # a dim that is not brought to the front alone (two kept dims) is summed at once, as before
+    host = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_", api_table="get_api_fused"))
+    e = host.sconcrete(x) * host.sconcrete(y) + host.sconcrete(x)
+    s2 = e.stranspose([0, 2, 3, 1]).ssumN(2)
+    assert np.allclose(s2.numpy(), want.transpose(0, 2, 3, 1).sum(axis=(0, 1)), rtol=1e-12, atol=1e-12) and host.counter("fused_map_dimsum") == 0

@@ -821,3 +821,47 @@ def test_fused_map_equals_the_single_operations(gpu, oracle, dt):
         assert np.array_equal(a, b)
     with pytest.raises(capi.HgpuError):
         gpu.fused_map([gpu.upload(x)], [(0, O1["exp"], 0, 0, 0, 0)], [1])
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_fused_map_dimsum_against_checker_and_numpy(gpu, oracle, dt):
+    """hgpu_fused_map_dimsum: the cotangent of a convolution layer written out
+    (example/MnistCnnShaped2.hs:57-63: the cotangent of the pooled, rectified
+    output spread over the pooling windows under a mask) and, from the same
+    pass, its sum over batch, height and width -- the bias's cotangent.  Dense
+    inputs and broadcast views over a refined index space; every kept dim."""
+    O2 = capi.OP2
+    rng = np.random.default_rng(77)
+    b, c, h, w = 24, 16, 14, 14
+    pooled = rng.standard_normal((b, c, h, w)).astype(dt)
+    mask = (rng.random((b, c, h, 2, w, 2)) < 0.3).astype(dt)
+    scale = np.asarray(0.5, dt)
+    prog = [(1, O2["mul"], 0, 0, 1, 0), (1, O2["mul"], 0, 3, 2, 0)]     # 3: pooled * mask, 4: ... * scale
+    want_map = pooled[:, :, :, None, :, None].astype(np.float64) * mask * 0.5
+    tol = TOL[np.dtype(dt)]
+    for keep in (1, 0, 5, 2):
+        res = []
+        for ctx in (gpu, oracle):
+            pv = ctx.upload(pooled).reshape([b, c, h, 1, w, 1]).as_strided([b, c, h, 2, w, 2], [c * h * w, h * w, w, 0, 1, 0], 0)
+            ins = [pv, ctx.upload(mask), ctx.upload(scale).replicate([b, c, h, 2, w, 2])]
+            outs, sm = ctx.fused_map_dimsum(ins, prog, [4], 4, keep)
+            res.append((outs[0].numpy(), sm.numpy()))
+        other = tuple(d for d in range(6) if d != keep)
+        want_sum = want_map.sum(axis=other)
+        scale_sum = np.abs(want_map).sum(axis=other).max()
+        for got_map, got_sum in res:
+            assert got_map.dtype == np.dtype(dt) and np.allclose(got_map, want_map, rtol=tol, atol=0)
+            assert got_sum.shape == want_sum.shape and got_sum.dtype == np.dtype(dt)
+            assert np.max(np.abs(got_sum - want_sum)) <= tol * scale_sum
+        assert np.array_equal(res[0][0], res[1][0])
+    # all inputs dense, the kept dim last (its elements are neighbours in memory: no vectors across it)
+    x = rng.standard_normal((700, 500)).astype(dt)
+    y = rng.standard_normal((700, 500)).astype(dt)
+    for keep in (0, 1):
+        outs, sm = gpu.fused_map_dimsum([gpu.upload(x), gpu.upload(y)], [(1, O2["mul"], 0, 0, 1, 0)], [2], 2, keep)
+        prod = x.astype(np.float64) * y
+        assert np.allclose(outs[0].numpy(), prod, rtol=tol, atol=0)
+        assert np.max(np.abs(sm.numpy() - prod.sum(axis=1 - keep))) <= tol * np.abs(prod).sum(axis=1 - keep).max()
+    # too small for the compiled kernel: refused, the caller runs the two steps
+    with pytest.raises(capi.HgpuError):
+        gpu.fused_map_dimsum([gpu.upload(x[:10]), gpu.upload(y[:10])], [(1, O2["mul"], 0, 0, 1, 0)], [2], 2, 0)

@@ -341,6 +341,18 @@ def test_fused_table_definitions(oracle):
     o = C.c_void_p()
     assert fs(oracle.h, 1, ins, 1, flat, 1, C.byref(o)) == 0
     assert abs(capi.Array(oracle, o).numpy() - (-x).sum()) <= 1e-12
+    # fused_map_dimsum: the program's results, and one slot summed over every dim but one
+    fd = dll.horc_fused_map_dimsum
+    fd.restype, fd.argtypes = I, [P, I, PP, I, P, I, C.POINTER(C.c_int), PP, I, I, PP]
+    x3 = x.reshape(3, 4, 6)
+    a3 = oracle.upload(x3)
+    ins3 = (C.c_void_p * 1)(a3.h)
+    for keep in range(3):
+        outs, sm = (C.c_void_p * 1)(), C.c_void_p()
+        assert fd(oracle.h, 1, ins3, 1, flat, 1, (C.c_int * 1)(1), outs, 1, keep, C.byref(sm)) == 0
+        assert np.array_equal(capi.Array(oracle, C.c_void_p(outs[0])).numpy(), -x3)
+        other = tuple(d for d in range(3) if d != keep)
+        assert np.allclose(capi.Array(oracle, sm).numpy(), (-x3).sum(axis=other), rtol=1e-13, atol=1e-13)
     # contract_operands: program, merged dims, zero-extension, view, contraction
     y = rnd((2, 3, 4), np.float64)
     z = rnd((2, 3, 4), np.float64)
