@@ -426,6 +426,7 @@ const char* hgpu_last_error(hgpu_ctx* ctx) {
 
 int hgpu_mem_stats(hgpu_ctx* ctx, uint64_t* in_use, uint64_t* reserved, uint64_t* n_allocs) {
   if (!ctx) return HGPU_ERR_INVALID;
+  flush_deferred(ctx);      // launches that are held back hold their buffers
   std::lock_guard<std::mutex> g(ctx->mu);
   if (in_use) *in_use = ctx->in_use;
   if (reserved) *reserved = ctx->reserved;

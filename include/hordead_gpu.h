@@ -107,7 +107,10 @@ const char* hgpu_last_error(hgpu_ctx* ctx);
 /* Allocator statistics: bytes held by live arrays, bytes reserved from the
  * device (live + cached), number of device allocations made so far. */
 int hgpu_mem_stats(hgpu_ctx* ctx, uint64_t* in_use, uint64_t* reserved, uint64_t* n_device_allocs);
-/* The stream all work is enqueued on, as a `hipStream_t` cast to void*. */
+/* The stream all work is enqueued on, as a `hipStream_t` cast to void*.  The
+ * call first enqueues whatever launches the library is holding back (see
+ * hgpu_contract_sum_map): a caller that puts work of its own on the stream
+ * asks for the stream each time, right before it does. */
 void* hgpu_stream(hgpu_ctx* ctx);
 /* When `limit` >= 0, the next `limit`-th device allocation and all later ones
  * fail with HGPU_ERR_OOM (host-forced fault injection for tests of the error
