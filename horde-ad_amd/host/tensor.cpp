@@ -1289,6 +1289,46 @@ T convert(const T& a, int dtype, int mode) {
   return make_expr(HGPU_FUSED_CONVERT, mode, dtype, a, nullptr, nullptr);
 }
 // Does the expression beneath p have a leaf that is a contraction (or a sum of contractions) not yet computed?
+// The pending contraction (or sum of contractions) among the leaves of an expression, if there is one.
+static const ArrHolder* pending_contraction_in(const ArrHolder* root) {
+  std::map<const ArrHolder*, int> seen;
+  std::vector<const ArrHolder*> stack{root};
+  while (!stack.empty()) {
+    const ArrHolder* p = stack.back();
+    stack.pop_back();
+    if (seen.count(p)) continue;
+    seen[p] = 1;
+    if (contraction_or_sum(p)) return p;
+    if (!p->h && p->vsrc) { stack.push_back(p->vsrc.get()); continue; }
+    if (p->h || p->ekind < 0) continue;
+    if (p->fa) stack.push_back(p->fa.get());
+    if (p->fb) stack.push_back(p->fb.get());
+    if (p->fc) stack.push_back(p->fc.get());
+  }
+  return nullptr;
+}
+
+// A matrix product with a short contracted dim (two kept dims that are not 1,
+// at most 1024 contracted elements over all terms): what the provider's
+// hgpu_contract_sum_map computes together with a program over it.
+static bool short_matrix_product(const ArrHolder* c) {
+  if (!c || c->keep < 1) return false;
+  const Shape kept = T(std::const_pointer_cast<ArrHolder>(c->fa)).shape();
+  int wide = 0;
+  for (int d = 0; d < c->keep; ++d) wide += kept[(size_t)d] != 1;
+  if (wide != 2) return false;
+  int64_t k = 0;
+  auto contracted = [&](const std::shared_ptr<ArrHolder>& f) {
+    const Shape sh = T(f).shape();
+    int64_t n = 1;
+    for (size_t d = (size_t)c->keep; d < sh.size(); ++d) n *= sh[d];
+    return n;
+  };
+  k += contracted(c->fa);
+  for (auto& m : c->more) k += contracted(m.first);
+  return k <= 1024;
+}
+
 static bool holds_pending_contraction(const ArrHolder* root) {
   std::map<const ArrHolder*, int> seen;
   std::vector<const ArrHolder*> stack{root};
@@ -1416,6 +1456,17 @@ static T contract_now(const T& a, const T* b, int n_keep) {
   // all its views) and the plain contraction runs on the views.
   Backend* be = a.be();
   const hgpu_api* api = be->api;
+  // ... unless the expression stands on a short matrix product that is still
+  // pending (the cotangent `W^T dz` under `* (1 - h * h)`): product and program
+  // are one kernel of their own, and numbering the expression as an operand
+  // would write the product out alone first.
+  if (api->struct_size >= offsetof(hgpu_api, contract_sum_map) + sizeof(api->contract_sum_map) && api->contract_sum_map && be->fuse) {
+    for (const T* t : {&a, b}) {
+      if (!t || !virtual_operand(*t)) continue;
+      const ArrHolder* src = t->holder()->vsrc.get();
+      if (short_matrix_product(pending_contraction_in(src->mv_inner ? src->mv_inner.get() : src))) (void)T(t->holder()->vsrc).h();
+    }
+  }
   if ((virtual_operand(a) || (b && virtual_operand(*b))) && api->struct_size >= offsetof(hgpu_api, contract_operands) + sizeof(api->contract_operands) &&
       api->contract_operands && a.size() > 0) {
     OperandBuf oa, ob;
