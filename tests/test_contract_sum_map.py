@@ -285,3 +285,32 @@ def test_held_back_products_come_before_whatever_reads_them(gpu, oracle):
     want_c = w.astype(np.float64) @ x
     for g, c, want in zip(res[0], res[1], (want_c, np.tanh(want_c), w.T.astype(np.float64) @ want_c)):
         assert rel(g, c) <= 1e-5 and rel(g, want) <= 4e-5
+
+
+def test_cotangent_of_a_dense_layer_is_one_call():
+    """`(W^T dz) * (1 - h * h)`, the cotangent that a dense tanh layer hands down
+    (the reference's dense layers: example/MnistFcnnRanked2.hs, `tanh` hidden
+    activations), reaches the weight gradient below it as an operand seen through
+    views.  The product under it is short (the layer above is 8 or 5 wide): it goes
+    out with its program as one call, not alone and then the program.  Gradient
+    against the plain table's bit for bit and numpy's within 1e-12."""
+    from conftest import entry, pkg
+    import ref_numpy as ref
+    H, W = pkg.hostapi, pkg.workloads
+    plain = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    fused = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_", api_table="get_api_fused"))
+    wl = W.c1_fcnn(batch=9, widths=(12, 8, 5, 4))
+    res = []
+    for host in (plain, fused):
+        ps, ds = wl.upload(host)
+        loss, grads = wl.gradient(host, ps, ds)
+        res.append((float(loss.numpy()), [g.numpy() for g in grads]))
+    assert res[0][0] == res[1][0]
+    for g0, g1 in zip(res[0][1], res[1][1]):
+        assert np.array_equal(g0, g1)
+    # three layers forward, two cotangents handed down
+    assert fused.counter("contract_sum_map") == 5
+    rloss, rgrads = ref.dense_net(wl.params, *wl.data, "tanh")
+    assert abs(res[1][0] - rloss) <= 1e-12 * abs(rloss)
+    for g, r in zip(res[1][1], rgrads):
+        assert np.max(np.abs(g - r)) <= 1e-12 * max(1.0, float(np.max(np.abs(r))))
