@@ -544,7 +544,7 @@ struct Deferred {
 
 struct DeferredQueue {
   std::vector<Deferred> items;
-  std::map<std::string, int> seen;   // how often a set of problems came up together
+  std::map<size_t, int> seen;        // how often a set of problems came up together, by the hash of their code
   long n_launches = 0, n_grouped = 0;
 };
 }  // namespace hg
@@ -611,7 +611,10 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
   if (grid > 0x7fffffff) return HGPU_OK;
   d.grid = (unsigned)grid;
   d.lds_bytes = (sp.x_elems + sp.y_elems) * (sp.f64 ? 8 : 4);
-  d.fn = compiled_kernel(ctx, {&d.body}, {d.grid}, {d.lds_bytes}, d.kname);
+  {
+    std::lock_guard<std::mutex> lk(ctx->launch_mu);   // the kernel cache is shared with the thread that launches what is held back
+    d.fn = compiled_kernel(ctx, {&d.body}, {d.grid}, {d.lds_bytes}, d.kname);
+  }
   if (!d.fn) return HGPU_OK;
 
   for (auto& tm : sp.terms) { d.args.push_back(tm.x); d.args.push_back(tm.y); }
@@ -714,7 +717,7 @@ void flush_deferred_locked(hgpu_ctx* ctx) {
         std::string key;
         for (auto* d : grp) { gname += "__" + d->kname.substr(7); key += d->body + "\x1f"; }
         // a set seen once may never come again (a second or so of compilation): the second time pays
-        if (++ctx->dq->seen[key] >= 2) {
+        if (++ctx->dq->seen[std::hash<std::string>()(key)] >= 2) {
           std::vector<const std::string*> bodies;
           std::vector<unsigned> grids;
           std::vector<int> lds;
