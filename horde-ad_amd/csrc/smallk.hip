@@ -577,7 +577,9 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
     sp.terms.push_back(tm);
   }
   if (ktot < 4 || ktot > (sp.P * sp.Q <= kSmallOut ? kMaxKSmallOut : kMaxKTotal)) return HGPU_OK;
-  if (sp.P < 16 || sp.Q < 4 || (double)sp.P * sp.Q * ktot < 2.0e6) return HGPU_OK;
+  // below about a million multiply-adds the wave-per-output kernels are as fast; from there on this kernel wins, the more so with a program to
+  // run over the result (the CNN's readout layer and its cotangent, 10 x 1000 x 128 each: the gradient 0.453 -> 0.430 ms with them in)
+  if (sp.P < 16 || sp.Q < 4 || (double)sp.P * sp.Q * ktot < 1.0e6) return HGPU_OK;
   for (int o = 0; o < n_out; ++o) {
     if (out_slots[o] < n_in && out_slots[o] != c_slot) return HGPU_OK;   // a copy of an input: not this kernel's business
     if (!outs[o]->buf) return HGPU_OK;
