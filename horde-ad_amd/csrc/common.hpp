@@ -52,6 +52,7 @@ namespace hg {
 struct DeferredQueue;                         // launches held back to be grouped (smallk.hip)
 void flush_deferred_locked(hgpu_ctx* ctx);    // the caller holds launch_mu
 void flush_deferred(hgpu_ctx* ctx);
+void drop_deferred(hgpu_ctx* ctx);            // flush, then free the queue
 }  // namespace hg
 
 struct hgpu_ctx {

@@ -22,7 +22,7 @@ namespace hg {
 // gemm.hip: returns HGPU_OK and sets *handled when the contraction was
 // recognised as a matrix product and executed on the matrix cores.
 int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled,
-             int n_terms = 0, const hgpu_array* const* as = nullptr, const hgpu_array* const* bs = nullptr);
+             int n_terms = 0, const hgpu_array* const* as = nullptr, const hgpu_array* const* bs = nullptr, hgpu_array** partials_out = nullptr);
 constexpr int kGemmMaxTerms = 32;   // products one launch of try_gemm sums (kMaxTerms of the kernels)
 }
 

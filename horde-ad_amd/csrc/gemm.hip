@@ -348,10 +348,15 @@ int sum_partials(hgpu_ctx* ctx, int dtype, int64_t n, int parts, const void* par
 }
 
 int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled,
-             int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs) {
+             int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs, hgpu_array** partials_out) {
   // n_terms > 0: out = sum_t contract(as[t], bs[t]); all terms have the shapes,
   // strides and dtype of a = as[0], b = bs[0] (the caller has checked).
+  // partials_out: a caller that runs an elementwise pass over the result anyway
+  // takes the two or three partial results of a product split along K instead
+  // (an array of shape [parts, kept dims...]; `out` is then left unwritten) and
+  // adds them in that pass.
   *handled = false;
+  if (partials_out) *partials_out = nullptr;
   if (!b) return HGPU_OK;
   if (a->dtype != HGPU_F64 && a->dtype != HGPU_F32) return HGPU_OK;
   GemmParams p;
@@ -562,7 +567,13 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
       if (a->dtype == HGPU_F64) launch_f64(p, la);
       else launch_f32(p, la);
     }
-    if (split > 1) {
+    if (split > 1 && partials_out && split <= 3 && is_dense(out)) {
+      int64_t sh[HGPU_MAX_RANK + 1], st[HGPU_MAX_RANK + 1];
+      sh[0] = split;
+      for (int d = 0; d < out->rank; ++d) sh[d + 1] = out->shape[d];
+      dense_strides(out->rank + 1, sh, st);
+      *partials_out = new_view(ctx, part, a->dtype, out->rank + 1, sh, st, 0);
+    } else if (split > 1) {
       LaunchGuard ls(ctx, "gemm_sum_partials", (double)out_n * (split + 1) * es, (double)out_n * split);
       if (a->dtype == HGPU_F64) launch_sum_partials<double>(ctx, out_n, (int)split, (const double*)part->ptr, (double*)data_ptr(out));
       else launch_sum_partials<float>(ctx, out_n, (int)split, (const float*)part->ptr, (float*)data_ptr(out));
@@ -571,7 +582,10 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
   hipError_t e = hipGetLastError();
   buffer_release(koff);
   if (part) buffer_release(part);
-  if (e != hipSuccess) return check_hip(ctx, e, "gemm");
+  if (e != hipSuccess) {
+    if (partials_out && *partials_out) { hgpu_release(*partials_out); *partials_out = nullptr; }
+    return check_hip(ctx, e, "gemm");
+  }
   *handled = true;
   return HGPU_OK;
 }

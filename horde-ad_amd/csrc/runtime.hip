@@ -388,7 +388,7 @@ int hgpu_graph_destroy(hgpu_graph* gr) {
 int hgpu_shutdown(hgpu_ctx* ctx) {
   if (!ctx) return HGPU_ERR_INVALID;
   (void)hipSetDevice(ctx->device);
-  flush_deferred(ctx);
+  drop_deferred(ctx);
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->zero_block) { buffer_release(ctx->zero_block); ctx->zero_block = nullptr; }
   {

@@ -56,7 +56,7 @@ using namespace hg::fusedgen;
 
 namespace hg {
 int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out, bool* handled,
-             int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs);
+             int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs, hgpu_array** partials_out = nullptr);
 }
 
 namespace {
@@ -763,6 +763,14 @@ void flush_deferred(hgpu_ctx* ctx) {
   if (ctx->dq_pending) flush_deferred_locked(ctx);
 }
 
+// Launches what is held back and gives the queue's own memory back (hgpu_shutdown).
+void drop_deferred(hgpu_ctx* ctx) {
+  std::lock_guard<std::mutex> lk(ctx->launch_mu);
+  if (ctx->dq_pending) flush_deferred_locked(ctx);
+  delete ctx->dq;
+  ctx->dq = nullptr;
+}
+
 }  // namespace hg
 
 extern "C" int hgpu_contract_sum_map(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hgpu_array* const* bs, int n_keep, int n_in,
@@ -817,7 +825,53 @@ extern "C" int hgpu_contract_sum_map(hgpu_ctx* ctx, int n_terms, const hgpu_arra
   }
   // one entry point after another: the products (terms of one shape together), their sum, the program
   hgpu_array* c = nullptr;
-  {
+  // A single product that the staged kernel splits in two or three along K
+  // leaves partial results to add: the pass that runs the program adds them.
+  bool sum_is_output = false;
+  for (int o = 0; o < n_out; ++o) sum_is_output = sum_is_output || out_slots[o] == c_slot;
+  if (n_terms == 1 && !sum_is_output && n_instr >= 1 && n_in + 2 <= 12 && n_instr + 2 <= 96 && n_kept > 0 && (a0->dtype == HGPU_F64 || a0->dtype == HGPU_F32)) {
+    hgpu_array *c0 = nullptr, *parts = nullptr;
+    int rc = new_dense(ctx, a0->dtype, n_keep, a0->shape, &c0);
+    bool handled = false;
+    if (!rc) rc = try_gemm(ctx, as[0], bs[0], n_keep, c0, &handled, 0, nullptr, nullptr, &parts);
+    if (rc) { if (c0) hgpu_release(c0); return rc; }
+    if (handled && parts) {
+      hgpu_release(c0);
+      const int S = (int)parts->shape[0], n_in2 = n_in + S - 1, shift = (S - 1) + (S - 1);
+      std::vector<hgpu_array*> slices((size_t)S, nullptr);
+      for (int s2 = 0; s2 < S && !rc; ++s2) {
+        const int64_t ix = s2;
+        rc = hgpu_index_prefix(ctx, parts, 1, &ix, &slices[(size_t)s2]);
+      }
+      std::vector<const hgpu_array*> ins2(in, in + n_in);
+      std::vector<hgpu_fused_instr> prog2;
+      if (!rc) {
+        ins2[(size_t)c_slot] = slices[0];
+        for (int s2 = 1; s2 < S; ++s2) ins2.push_back(slices[(size_t)s2]);
+        // the sum: (p0 + p1) + p2, then the caller's program with its slots moved
+        for (int s2 = 1; s2 < S; ++s2)
+          prog2.push_back(hgpu_fused_instr{HGPU_FUSED_OP2, HGPU_ADD, a0->dtype, s2 == 1 ? c_slot : n_in2 + s2 - 2, n_in + s2 - 1, 0});
+        const int sum_slot = n_in2 + S - 2;
+        auto moved = [&](int v) { return v == c_slot ? sum_slot : (v < n_in ? v : v + shift); };
+        for (int k = 0; k < n_instr; ++k) {
+          hgpu_fused_instr q = prog[k];
+          q.a = moved(q.a);
+          if (q.kind == HGPU_FUSED_OP2 || q.kind == HGPU_FUSED_CMP || q.kind == HGPU_FUSED_SELECT) q.b = moved(q.b);
+          if (q.kind == HGPU_FUSED_SELECT) q.c = moved(q.c);
+          prog2.push_back(q);
+        }
+        std::vector<int> slots2;
+        for (int o = 0; o < n_out; ++o) slots2.push_back(moved(out_slots[o]));
+        rc = hgpu_fused_map(ctx, n_in2, ins2.data(), (int)prog2.size(), prog2.data(), n_out, slots2.data(), outs);
+      }
+      for (auto* sl : slices) if (sl) hgpu_release(sl);
+      hgpu_release(parts);
+      return rc;
+    }
+    if (handled) c = c0;            // computed whole: the program below
+    else hgpu_release(c0);
+  }
+  if (!c) {
     std::vector<char> taken((size_t)n_terms, 0);
     for (int t0 = 0; t0 < n_terms; ++t0) {
       if (taken[(size_t)t0]) continue;

@@ -325,8 +325,9 @@ int hgpu_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, i
  * would split K to fill the device and add partial results) and the
  * kept shape has two non-unit dims this is one kernel compiled for the shapes,
  * with the whole contracted dim of a term in LDS; otherwise the single entry
- * points run one after another.  Results equal theirs up to the order of the
- * floating-point sums.
+ * points run one after another (a single product that is split in two or
+ * three along its contracted dim is added up by the pass that runs the
+ * program).  Results equal theirs up to the order of the floating-point sums.
  * The compiled kernel's launch may be held back until the next call that
  * needs the stream (any other launch, copy, synchronisation, hgpu_stream, the
  * ends of a graph capture): held-back products that do not read one another's

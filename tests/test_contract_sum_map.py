@@ -64,6 +64,7 @@ SHAPES = [
     (np.float64, 128, 784, [1000], ["km"]),                 # its weight gradient: 16 chunks
     (np.float32, 128, 1000, [1100], ["mk"]),                # too long for the kernel: the entry points one after another
     (np.float32, 300, 1000, [600], ["mk"]),                 # too long for a result of this size
+    (np.float64, 300, 5000, [784], ["mk"]),                 # ... a dense layer over a flattened image at batch 5000: split in two along K, the program adds the halves
     (np.float32, 6, 20, [5], ["mk"]),                       # too small for it
 ]
 
