@@ -391,7 +391,9 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     int rc = try_smallk(ctx, n_terms > 0 ? n_terms : 1, ta, tb, n_keep, 1, &none, 0, 0, nullptr, std::vector<int>{a->dtype}, 1, &slot, &out, handled);
     if (rc || *handled) return rc;
   }
-  if ((p.M <= 32 || p.N <= 32) && p.M <= 1024 && p.N <= 1024) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled, n_terms);
+  // (under a long K the staged kernel's coalesced tile loads win even with most of a 32-wide tile empty: the recurrent network's
+  // input weight gradient, 128 x 28 over 28 x 5000, 52 -> 45 us)
+  if ((p.M <= 32 || p.N <= 32) && p.M <= 1024 && p.N <= 1024 && p.K < 4096) return gemm_direct(ctx, p, a->dtype, pa, pb, out, handled, n_terms);
 
   const int64_t nt = n_terms > 0 ? n_terms : 1;      // products summed by this launch
   const int64_t out_elems = p.M * p.N * p.BT;
