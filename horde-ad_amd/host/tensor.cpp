@@ -527,6 +527,8 @@ static bool products_then_program(Backend* be, const std::vector<ArrHolder*>& ro
   ArrHolder* kept = nullptr;
   number_program(roots, &ins, &prog, &slots, &kept, &nodes, true);
   if (!kept) return false;
+  // Computed during the walk after all (a view of it among the later leaves needed it as an array): nothing is left to fuse.
+  if (kept->h || !kept->fa) return false;
   if (T(kept->fa).dtype() != HGPU_F64 && T(kept->fa).dtype() != HGPU_F32) { kept->force(); return false; }
   int c_slot = -1;
   for (size_t i = 0; i < ins.size(); ++i)

@@ -126,7 +126,7 @@ def run(host, x0, steps):
     return out
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", list(range(40)) + [683])     # 683: a pending product whose view among the later leaves of the same program computed it
 def test_random_program_matches_the_checker(seed):
     shape, steps, _ = random_program(seed)
     x0 = np.random.default_rng(1000 + seed).uniform(-1, 1, shape)
