@@ -5,6 +5,7 @@
 #include <cstddef>
 #include <cstring>
 #include <numeric>
+#include <set>
 
 #include "host.hpp"
 
@@ -468,8 +469,57 @@ int visit(Program& pg, ArrHolder* p) {
 // The roots' expressions as one numbered program: inputs, instructions, and the slot of every root.
 // With `kept`: one pending contraction among the leaves stays pending (*kept; its
 // entry of ins is null), and nodes receives the holder of every instruction.
+// Computing a leaf can run other programs, and those may write out (and take
+// apart) nodes of the very expression that is being numbered.  So everything
+// that has to be computed is computed first, one leaf at a time with a fresh
+// look at the expression after each; the numbering walk that follows computes
+// nothing and its raw pointers stay good.  In numbering order: the pending
+// contraction that stays pending (with keep_contraction) has its operands
+// written out, every other pending leaf is written out itself.
+static void settle_leaves(const std::vector<ArrHolder*>& roots, bool keep_contraction, bool keep_sums) {
+  std::set<const ArrHolder*> tried_view;
+  for (int round = 0; round < 100000; ++round) {
+    std::set<const ArrHolder*> seen;
+    const ArrHolder* kept = nullptr;
+    std::shared_ptr<ArrHolder> todo;      // shared: what it is computed from may let go of it meanwhile
+    ArrHolder* todo_root = nullptr;
+    bool todo_is_view = false;
+    std::function<bool(ArrHolder*, const std::shared_ptr<ArrHolder>*)> walk = [&](ArrHolder* p, const std::shared_ptr<ArrHolder>* owner) -> bool {
+      if (!seen.insert(p).second) return false;
+      auto take = [&](bool view) { if (owner) todo = *owner; else todo_root = p; todo_is_view = view; return true; };
+      if (keep_contraction && (keep_sums ? contraction_or_sum(p) : single_contraction(p)) && (!kept || kept == p)) {
+        kept = p;
+        for (auto* f : {&p->fa, &p->fb})
+          if (*f && !(*f)->h) { todo = *f; return true; }
+        for (auto& m : p->more)
+          for (auto* f : {&m.first, &m.second})
+            if (*f && !(*f)->h) { todo = *f; return true; }
+        return false;
+      }
+      if (!p->h && p->ekind < 0) return take(false);
+      if (!p->h && p->vsrc && p->vsrc->h && !tried_view.count(p)) return take(true);
+      if (p->h) return false;
+      for (auto* f : {&p->fa, &p->fb, &p->fc})
+        if (*f && walk(f->get(), f)) return true;
+      return false;
+    };
+    bool found = false;
+    for (auto* r : roots)
+      if (walk(r, nullptr)) { found = true; break; }
+    if (!found) return;
+    ArrHolder* q = todo ? todo.get() : todo_root;
+    if (todo_is_view) {
+      tried_view.insert(q);
+      q->view_of_written_source();
+    } else {
+      q->force();
+    }
+  }
+}
+
 static void number_program(const std::vector<ArrHolder*>& roots, std::vector<const hgpu_array*>* ins, std::vector<hgpu_fused_instr>* prog,
                            std::vector<int>* outs_slot, ArrHolder** kept = nullptr, std::vector<ArrHolder*>* nodes = nullptr, bool keep_sums = false) {
+  settle_leaves(roots, kept != nullptr, keep_sums);
   Program pg;
   pg.keep_contraction = kept != nullptr;
   pg.keep_sums = keep_sums;
@@ -646,7 +696,13 @@ static int front_dim_of_view(const ArrHolder* v) {
   return rd;
 }
 
-static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
+static void run_program(Backend* be, const std::vector<ArrHolder*>& all_roots) {
+  // computing the leaves may write a root out on the way (as a view of a source written meanwhile): those are done
+  settle_leaves(all_roots, true, true);
+  std::vector<ArrHolder*> roots;
+  for (auto* r : all_roots)
+    if (!r->h && r->ekind >= 0) roots.push_back(r);
+  if (roots.empty()) return;
   std::vector<const hgpu_array*> ins;
   std::vector<hgpu_fused_instr> prog;
   std::vector<int> outs_slot;
@@ -693,6 +749,16 @@ static void run_program(Backend* be, const std::vector<ArrHolder*>& roots) {
     // done by one kernel: products, their sum and the program
   } else if (sums.empty()) {
     number_program(roots, &ins, &prog, &outs_slot);
+    {
+      // the attempt above may have written the source a root is a view of: that root is done (the walk has made it the view)
+      std::vector<ArrHolder*> rest;
+      for (auto* r : roots)
+        if (!r->h && r->ekind >= 0) rest.push_back(r);
+      if (rest.size() != roots.size()) {
+        if (!rest.empty()) run_program(be, rest);
+        return;
+      }
+    }
     int n_in = (int)ins.size(), n_instr = (int)prog.size();
     // A pending sum over all dims but one of what is being written out (a
     // bias's cotangent) is taken in the same pass.
@@ -764,6 +830,10 @@ static void force_roots(Backend* be, std::vector<ArrHolder*> roots) {
   std::vector<ArrHolder*> rs;
   for (auto* r : roots)
     if (!r->h && r->ekind >= 0 && std::find(rs.begin(), rs.end(), r) == rs.end()) rs.push_back(r);
+  if (rs.empty()) return;
+  // the leaves first: what they turn into decides how many inputs and instructions there are to count
+  settle_leaves(rs, true, true);
+  rs.erase(std::remove_if(rs.begin(), rs.end(), [](ArrHolder* r) { return r->h || r->ekind < 0; }), rs.end());
   if (rs.empty()) return;
   int n_in, n_instr;
   measure(rs, &n_in, &n_instr);

@@ -692,6 +692,10 @@ int horc_onehot(hgpu_ctx* c, const hgpu_array* v, int n, const int64_t* ix, cons
 // The meaning of a fused program: the single operations applied in program order.
 int horc_fused_map(hgpu_ctx* c, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
                    int n_out, const int* out_slots, hgpu_array** outs) {
+  // the limits of the device library's kernel generator are part of the entry point's contract: a host layer that
+  // exceeds them is caught here, without a device
+  if (n_in < 1 || n_in > 12 || n_out < 1 || n_out > 6 || n_instr < 1 || n_instr > 96)
+    return fail(c, HGPU_ERR_UNSUPPORTED, "fused_map: " + std::to_string(n_in) + " inputs, " + std::to_string(n_instr) + " instructions, " + std::to_string(n_out) + " outputs");
   std::vector<hgpu_array*> slots;
   std::vector<hgpu_array*> made;
   for (int i = 0; i < n_in; ++i) slots.push_back(const_cast<hgpu_array*>(in[i]));
@@ -820,7 +824,7 @@ int horc_contract_map(hgpu_ctx* c, const hgpu_array* a, const hgpu_array* b, int
 static int operand_array(hgpu_ctx* c, const hgpu_operand* o, hgpu_array** out) {
   if (o->array) { horc_retain(const_cast<hgpu_array*>(o->array)); *out = const_cast<hgpu_array*>(o->array); return HGPU_OK; }
   hgpu_array *e = nullptr, *m = nullptr, *p = nullptr;
-  int rc = horc_fused_map(c, o->n_in, o->in, o->n_instr, o->prog, 1, &o->slot, &e);
+  int rc = o->slot < o->n_in ? horc_materialize(c, o->in[o->slot], &e) : horc_fused_map(c, o->n_in, o->in, o->n_instr, o->prog, 1, &o->slot, &e);
   if (rc) return rc;
   rc = horc_reshape(c, e, o->rank_m, o->mshape, &m);
   horc_release(e);
@@ -923,7 +927,14 @@ int horc_contract_sum_map(hgpu_ctx* c, int n_terms, const hgpu_array* const* a, 
   for (auto& p : ins)
     if (!p) { p = acc; ++n_null; }
   int rc = n_null == 1 ? HGPU_OK : fail(c, HGPU_ERR_INVALID, "contract_sum_map: exactly one input must stand for the sum");
-  if (!rc) rc = horc_fused_map(c, n_in, ins.data(), n_instr, prog, n_out, out_slots, outs);
+  if (!rc && n_instr == 0) {   // no program: the outputs are inputs, written out
+    for (int o = 0; o < n_out && !rc; ++o) {
+      if (out_slots[o] < 0 || out_slots[o] >= n_in) rc = fail(c, HGPU_ERR_INVALID, "contract_sum_map: bad output slot");
+      else rc = horc_materialize(c, ins[(size_t)out_slots[o]], &outs[o]);
+    }
+  } else if (!rc) {
+    rc = horc_fused_map(c, n_in, ins.data(), n_instr, prog, n_out, out_slots, outs);
+  }
   horc_release(acc);
   return rc;
 }

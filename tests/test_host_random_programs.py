@@ -18,8 +18,9 @@ def factorizations(n):
     return [(a, n // a) for a in range(2, n) if n % a == 0]
 
 
-def random_program(seed):
-    """A list of steps (name, args) over a stack of values; generated once, replayed on both hosts."""
+def random_program(seed, extended=False):
+    """A list of steps (name, args) over a stack of values; generated once, replayed on both hosts.
+    extended: also dense layers (one or two matrix products, bias, tanh) and sums over all dims but one."""
     rng = np.random.default_rng(seed)
     shapes = [tuple(int(x) for x in rng.integers(2, 7, int(rng.integers(2, 4))))]
     steps = []
@@ -27,7 +28,10 @@ def random_program(seed):
     for _ in range(int(rng.integers(6, 14))):
         i = int(rng.integers(0, len(stack)))
         sh = stack[i]
-        kind = rng.choice(["unary", "binary", "transpose", "split", "merge", "slice", "append", "sum", "scale", "bias", "pool"])
+        kinds = ["unary", "binary", "transpose", "split", "merge", "slice", "append", "sum", "scale", "bias", "pool"]
+        if extended:
+            kinds += ["layer", "layer", "keepdim"]
+        kind = rng.choice(kinds)
         if kind == "unary":
             steps.append(("unary", i, str(rng.choice(["sin", "tanh", "cos"]))))
             stack.append(sh)
@@ -76,6 +80,17 @@ def random_program(seed):
         elif kind == "pool" and len(sh) >= 2 and sh[-1] % 2 == 0 and sh[-2] % 2 == 0:
             steps.append(("pool", i))
             stack.append(sh[:-2] + (sh[-2] // 2, sh[-1] // 2))
+        elif kind == "layer" and len(sh) == 2:
+            # act (W v [+ U u] + b): u another value of the same batch (second dim)
+            width = int(rng.integers(2, 7))
+            others = [j for j, s2 in enumerate(stack) if len(s2) == 2 and s2[1] == sh[1]]
+            j = int(rng.choice(others)) if rng.random() < 0.5 else -1
+            steps.append(("layer", i, j, width, int(rng.integers(0, 1000)), str(rng.choice(["tanh", "none", "sin"]))))
+            stack.append((width, sh[1]))
+        elif kind == "keepdim" and len(sh) >= 2:
+            d = int(rng.integers(0, len(sh)))
+            steps.append(("keepdim", i, d))
+            stack.append((sh[d],))
     return shapes[0], steps, stack
 
 
@@ -103,6 +118,20 @@ def run(host, x0, steps):
             sh = v.shape
             b = np.random.default_rng(st[2]).uniform(-1, 1, sh[-1])
             vals.append(v + host.concrete(b).sreplicateN(list(sh[:-1])))
+        elif st[0] == "layer":
+            _, i, j, width, wseed, act = st
+            r = np.random.default_rng(wseed)
+            w = host.concrete(r.uniform(-1, 1, (width, v.shape[0])))
+            z = w.smatmul2(v)
+            if j >= 0:
+                u = vals[j]
+                z = z + host.concrete(r.uniform(-1, 1, (width, u.shape[0]))).smatmul2(u)
+            z = z + host.concrete(r.uniform(-1, 1, (width,))).sreplicate(v.shape[1]).str_()
+            vals.append(z if act == "none" else z.op1(act))
+        elif st[0] == "keepdim":   # the sum over every dim but one, as the cotangent of a replicated and transposed bias is taken
+            d, rk = st[2], len(v.shape)
+            perm = [q for q in range(rk) if q != d] + [d]
+            vals.append(v.stranspose(perm).ssumN(rk - 1) if rk > 1 else v)
         elif st[0] == "pool":      # 2x2 max over the last two dims: window gather, merged reshape, kargMax, gather
             sh = v.shape
             lead, h2, w2 = list(sh[:-2]), sh[-2] // 2, sh[-1] // 2
@@ -126,11 +155,33 @@ def run(host, x0, steps):
     return out
 
 
+def reference_host():
+    """The host layer on the checker with deferral switched off: every operation executed at once, as the
+    reference's `Concrete` instance does -- nothing of what is under test here takes part."""
+    h = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    h.set_fusion(0)
+    return h
+
+
 @pytest.mark.parametrize("seed", list(range(40)) + [683])     # 683: a pending product whose view among the later leaves of the same program computed it
 def test_random_program_matches_the_checker(seed):
     shape, steps, _ = random_program(seed)
     x0 = np.random.default_rng(1000 + seed).uniform(-1, 1, shape)
-    cpu = run(H.Host(capi.Lib(entry.ORACLE_LIB, "horc_")), x0, steps)
+    cpu = run(reference_host(), x0, steps)
+    gpu = run(H.Host(), x0, steps)
+    for a, b in zip(gpu[0], cpu[0]):
+        assert a.shape == b.shape
+        assert np.allclose(a, b, rtol=1e-11, atol=1e-12), steps
+    assert np.isclose(gpu[1], cpu[1], rtol=1e-11), steps
+    assert np.allclose(gpu[2], cpu[2], rtol=1e-10, atol=1e-11), steps
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_program_with_layers_matches_the_checker(seed):
+    """Programs that also hold dense layers (one or two matrix products, bias, tanh) and sums over all dims but one."""
+    shape, steps, _ = random_program(seed, extended=True)
+    x0 = np.random.default_rng(1000 + seed).uniform(-1, 1, shape)
+    cpu = run(reference_host(), x0, steps)
     gpu = run(H.Host(), x0, steps)
     for a, b in zip(gpu[0], cpu[0]):
         assert a.shape == b.shape

@@ -36,7 +36,10 @@ TOL = {capi.F64: 1e-10, capi.F32: 1e-5}
 
 @pytest.fixture(scope="module")
 def host_cpu():
-    return H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    """The checker with the host layer's deferral switched off: every operation at once."""
+    h = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    h.set_fusion(0)
+    return h
 
 
 @pytest.fixture(scope="module")
