@@ -18,7 +18,9 @@ RNG = np.random.default_rng(7)
 
 @pytest.fixture(scope="module")
 def host_cpu():
-    return H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    h = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    h.set_fusion(0)      # every operation at once: nothing of the deferral under test takes part in the reference
+    return h
 
 
 @pytest.fixture(scope="module")

@@ -16,7 +16,9 @@ RNG = np.random.default_rng(5)
 
 @pytest.fixture(scope="module")
 def host_cpu():
-    return H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    h = H.Host(capi.Lib(entry.ORACLE_LIB, "horc_"))
+    h.set_fusion(0)      # every operation at once: nothing of the deferral under test takes part in the reference
+    return h
 
 
 @pytest.fixture(scope="module")
