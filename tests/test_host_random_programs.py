@@ -18,11 +18,15 @@ def factorizations(n):
     return [(a, n // a) for a in range(2, n) if n % a == 0]
 
 
-def random_program(seed, extended=False):
+def random_program(seed, extended=False, big=False):
     """A list of steps (name, args) over a stack of values; generated once, replayed on both hosts.
-    extended: also dense layers (one or two matrix products, bias, tanh) and sums over all dims but one."""
+    extended: also dense layers (one or two matrix products, bias, tanh) and sums over all dims but one.
+    big: a [32..96, 256..768] matrix to start from and layers 16 to 64 wide, so that the device takes the kernels it
+    compiles for shapes (and holds their launches back) in the middle of other work."""
     rng = np.random.default_rng(seed)
     shapes = [tuple(int(x) for x in rng.integers(2, 7, int(rng.integers(2, 4))))]
+    if big:
+        shapes = [(int(rng.integers(32, 97)), int(rng.integers(256, 769)))]
     steps = []
     stack = [shapes[0]]                        # shapes of the values made so far (value 0 is the input)
     for _ in range(int(rng.integers(6, 14))):
@@ -82,7 +86,7 @@ def random_program(seed, extended=False):
             stack.append(sh[:-2] + (sh[-2] // 2, sh[-1] // 2))
         elif kind == "layer" and len(sh) == 2:
             # act (W v [+ U u] + b): u another value of the same batch (second dim)
-            width = int(rng.integers(2, 7))
+            width = int(rng.integers(16, 65)) if big else int(rng.integers(2, 7))
             others = [j for j, s2 in enumerate(stack) if len(s2) == 2 and s2[1] == sh[1]]
             j = int(rng.choice(others)) if rng.random() < 0.5 else -1
             steps.append(("layer", i, j, width, int(rng.integers(0, 1000)), str(rng.choice(["tanh", "none", "sin"]))))
@@ -188,3 +192,17 @@ def test_random_program_with_layers_matches_the_checker(seed):
         assert np.allclose(a, b, rtol=1e-11, atol=1e-12), steps
     assert np.isclose(gpu[1], cpu[1], rtol=1e-11), steps
     assert np.allclose(gpu[2], cpu[2], rtol=1e-10, atol=1e-11), steps
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_program_with_layers_at_kernel_sizes_matches_the_checker(seed):
+    """The same at sizes where the device runs its shape-compiled kernels and holds launches back."""
+    shape, steps, _ = random_program(seed, extended=True, big=True)
+    x0 = np.random.default_rng(1000 + seed).uniform(-1, 1, shape)
+    cpu = run(reference_host(), x0, steps)
+    gpu = run(H.Host(), x0, steps)
+    for a, b in zip(gpu[0], cpu[0]):
+        assert a.shape == b.shape
+        assert np.allclose(a, b, rtol=1e-10, atol=1e-10), steps
+    assert np.isclose(gpu[1], cpu[1], rtol=1e-10), steps
+    assert np.allclose(gpu[2], cpu[2], rtol=1e-9, atol=1e-9 * max(1.0, float(np.max(np.abs(cpu[2]))))), steps
