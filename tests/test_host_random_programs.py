@@ -120,17 +120,17 @@ def run(host, x0, steps):
             vals.append(v * host.srepl(v.shape, st[2], v.dtype))
         elif st[0] == "bias":
             sh = v.shape
-            b = np.random.default_rng(st[2]).uniform(-1, 1, sh[-1])
+            b = np.random.default_rng(st[2]).uniform(-1, 1, sh[-1]).astype(x0.dtype)
             vals.append(v + host.concrete(b).sreplicateN(list(sh[:-1])))
         elif st[0] == "layer":
             _, i, j, width, wseed, act = st
             r = np.random.default_rng(wseed)
-            w = host.concrete(r.uniform(-1, 1, (width, v.shape[0])))
+            w = host.concrete(r.uniform(-1, 1, (width, v.shape[0])).astype(x0.dtype))
             z = w.smatmul2(v)
             if j >= 0:
                 u = vals[j]
-                z = z + host.concrete(r.uniform(-1, 1, (width, u.shape[0]))).smatmul2(u)
-            z = z + host.concrete(r.uniform(-1, 1, (width,))).sreplicate(v.shape[1]).str_()
+                z = z + host.concrete(r.uniform(-1, 1, (width, u.shape[0])).astype(x0.dtype)).smatmul2(u)
+            z = z + host.concrete(r.uniform(-1, 1, (width,)).astype(x0.dtype)).sreplicate(v.shape[1]).str_()
             vals.append(z if act == "none" else z.op1(act))
         elif st[0] == "keepdim":   # the sum over every dim but one, as the cotangent of a replicated and transposed bias is taken
             d, rk = st[2], len(v.shape)
@@ -206,3 +206,18 @@ def test_random_program_with_layers_at_kernel_sizes_matches_the_checker(seed):
         assert np.allclose(a, b, rtol=1e-10, atol=1e-10), steps
     assert np.isclose(gpu[1], cpu[1], rtol=1e-10), steps
     assert np.allclose(gpu[2], cpu[2], rtol=1e-9, atol=1e-9 * max(1.0, float(np.max(np.abs(cpu[2]))))), steps
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_program_with_layers_single_precision(seed):
+    """The same in fp32 (tolerances relative to the largest magnitude of each result: the programs chain up to a
+    dozen steps and sum hundreds of terms)."""
+    shape, steps, _ = random_program(seed, extended=True, big=True)
+    x0 = np.random.default_rng(1000 + seed).uniform(-1, 1, shape).astype(np.float32)
+    cpu = run(reference_host(), x0, steps)
+    gpu = run(H.Host(), x0, steps)
+    for a, b in zip(gpu[0], cpu[0]):
+        assert a.shape == b.shape and a.dtype == b.dtype
+        assert np.allclose(a, b, rtol=2e-4, atol=2e-4 * max(1.0, float(np.max(np.abs(b))) if b.size else 1.0)), steps
+    assert np.isclose(gpu[1], cpu[1], rtol=1e-3), steps
+    assert np.allclose(gpu[2], cpu[2], rtol=1e-3, atol=1e-3 * max(1.0, float(np.max(np.abs(cpu[2]))))), steps
