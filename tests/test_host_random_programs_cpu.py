@@ -35,3 +35,16 @@ def test_random_program_matches_every_operation_at_once(seed):
 @pytest.mark.parametrize("seed", [1, 57, 251] + list(range(2, 40)))
 def test_random_program_with_layers_matches_every_operation_at_once(seed):
     check(seed, True)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_program_with_layers_single_precision(seed):
+    shape, steps, _ = tp.random_program(seed, extended=True)
+    x0 = np.random.default_rng(1000 + seed).uniform(-1, 1, shape).astype(np.float32)
+    want = tp.run(tp.reference_host(), x0, steps)
+    got = tp.run(tp.H.Host(capi.Lib(entry.ORACLE_LIB, "horc_", api_table="get_api_fused")), x0, steps)
+    for a, b in zip(got[0], want[0]):
+        assert a.shape == b.shape and a.dtype == b.dtype == np.float32
+        assert np.allclose(a, b, rtol=2e-4, atol=2e-4 * max(1.0, float(np.max(np.abs(b))) if b.size else 1.0)), steps
+    assert np.isclose(got[1], want[1], rtol=1e-3), steps
+    assert np.allclose(got[2], want[2], rtol=1e-3, atol=1e-3 * max(1.0, float(np.max(np.abs(want[2]))))), steps
