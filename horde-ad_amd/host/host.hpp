@@ -37,6 +37,7 @@ struct Backend {
   std::map<std::pair<int, uint64_t>, std::shared_ptr<ArrHolder>> const_cache; // (dtype, value bits)
   bool capturing = false;   // between hh_capture_begin and hh_capture_end
   bool fuse = true;   // defer elementwise operations into fused programs (when the provider has fused_map)
+  uint64_t walk_gen = 0;    // walks over pending expressions number themselves: a node seen carries the walk's number
   std::vector<std::weak_ptr<ArrHolder>> pending_dimsums;   // sums over all dims but one of an expression, not yet taken (ArrHolder::ones_b)
   std::vector<std::weak_ptr<ArrHolder>> pending_sums;   // sums of all elements of an expression, not yet taken (ArrHolder::ssrc)
   std::map<std::string, int64_t> counters;   // how often each rewrite onto a fused entry point was taken (diagnostic)
@@ -77,6 +78,7 @@ struct ArrHolder {
   // that writes the expression out and is taken in that pass
   // (Backend::pending_dimsums, hgpu_fused_map_dimsum).
   bool ones_b = false;
+  uint64_t walk_mark = 0;   // the last walk over pending expressions that has seen this node (Backend::walk_gen)
   // A pending contraction that is a transpose of another pending contraction
   // remembers it: if anyone else still wants the original, the original is
   // computed once and this one becomes a view of it.

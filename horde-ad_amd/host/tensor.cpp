@@ -476,39 +476,55 @@ int visit(Program& pg, ArrHolder* p) {
 // nothing and its raw pointers stay good.  In numbering order: the pending
 // contraction that stays pending (with keep_contraction) has its operands
 // written out, every other pending leaf is written out itself.
+namespace {
+// One look at the expression: the first thing that has to be computed, in numbering order.
+struct SettleWalk {
+  bool keep_contraction, keep_sums;
+  uint64_t gen;                          // nodes seen in this walk carry it (no allocation per walk)
+  const std::set<const ArrHolder*>* tried_view;
+  const ArrHolder* kept = nullptr;
+  std::shared_ptr<ArrHolder> todo;       // shared: what it is computed from may let go of it meanwhile
+  ArrHolder* todo_root = nullptr;
+  bool todo_is_view = false;
+  bool take(ArrHolder* p, const std::shared_ptr<ArrHolder>* owner, bool view) {
+    if (owner) todo = *owner; else todo_root = p;
+    todo_is_view = view;
+    return true;
+  }
+  bool walk(ArrHolder* p, const std::shared_ptr<ArrHolder>* owner) {
+    if (p->walk_mark == gen) return false;
+    p->walk_mark = gen;
+    if (keep_contraction && (keep_sums ? contraction_or_sum(p) : single_contraction(p)) && (!kept || kept == p)) {
+      kept = p;
+      for (auto* f : {&p->fa, &p->fb})
+        if (*f && !(*f)->h) { todo = *f; return true; }
+      for (auto& m : p->more)
+        for (auto* f : {&m.first, &m.second})
+          if (*f && !(*f)->h) { todo = *f; return true; }
+      return false;
+    }
+    if (!p->h && p->ekind < 0) return take(p, owner, false);
+    if (!p->h && p->vsrc && p->vsrc->h && !tried_view->count(p)) return take(p, owner, true);
+    if (p->h) return false;
+    for (auto* f : {&p->fa, &p->fb, &p->fc})
+      if (*f && walk(f->get(), f)) return true;
+    return false;
+  }
+};
+}  // namespace
+
 static void settle_leaves(const std::vector<ArrHolder*>& roots, bool keep_contraction, bool keep_sums) {
+  if (roots.empty()) return;
+  Backend* be = roots[0]->be;
   std::set<const ArrHolder*> tried_view;
   for (int round = 0; round < 100000; ++round) {
-    std::set<const ArrHolder*> seen;
-    const ArrHolder* kept = nullptr;
-    std::shared_ptr<ArrHolder> todo;      // shared: what it is computed from may let go of it meanwhile
-    ArrHolder* todo_root = nullptr;
-    bool todo_is_view = false;
-    std::function<bool(ArrHolder*, const std::shared_ptr<ArrHolder>*)> walk = [&](ArrHolder* p, const std::shared_ptr<ArrHolder>* owner) -> bool {
-      if (!seen.insert(p).second) return false;
-      auto take = [&](bool view) { if (owner) todo = *owner; else todo_root = p; todo_is_view = view; return true; };
-      if (keep_contraction && (keep_sums ? contraction_or_sum(p) : single_contraction(p)) && (!kept || kept == p)) {
-        kept = p;
-        for (auto* f : {&p->fa, &p->fb})
-          if (*f && !(*f)->h) { todo = *f; return true; }
-        for (auto& m : p->more)
-          for (auto* f : {&m.first, &m.second})
-            if (*f && !(*f)->h) { todo = *f; return true; }
-        return false;
-      }
-      if (!p->h && p->ekind < 0) return take(false);
-      if (!p->h && p->vsrc && p->vsrc->h && !tried_view.count(p)) return take(true);
-      if (p->h) return false;
-      for (auto* f : {&p->fa, &p->fb, &p->fc})
-        if (*f && walk(f->get(), f)) return true;
-      return false;
-    };
+    SettleWalk w{keep_contraction, keep_sums, ++be->walk_gen, &tried_view};
     bool found = false;
     for (auto* r : roots)
-      if (walk(r, nullptr)) { found = true; break; }
+      if (w.walk(r, nullptr)) { found = true; break; }
     if (!found) return;
-    ArrHolder* q = todo ? todo.get() : todo_root;
-    if (todo_is_view) {
+    ArrHolder* q = w.todo ? w.todo.get() : w.todo_root;
+    if (w.todo_is_view) {
       tried_view.insert(q);
       q->view_of_written_source();
     } else {
