@@ -58,10 +58,11 @@ extern "C" int hgpu_compare_all(hgpu_ctx* ctx, int cmp, const hgpu_array* a, con
   if (rc) return rc;
   unsigned long long* first = (unsigned long long*)scratch->ptr;
   int* flag = (int*)((char*)scratch->ptr + 64);
-  int host = 0;
+  int host = 0, held_rc;
   hipError_t e;
   {
     LaunchGuard lg(ctx, "compare_all", 2.0 * n * dtype_size(a->dtype), (double)n);
+    held_rc = take_deferred_rc(ctx);
     hipLaunchKernelGGL(k_set_u64, dim3(1), dim3(1), 0, ctx->stream, first, ~0ull);
     unsigned g = grid_for(n, kBlock, ctx->num_cu * 8);
     HG_DISPATCH_DTYPE(a->dtype, T, {
@@ -73,6 +74,7 @@ extern "C" int hgpu_compare_all(hgpu_ctx* ctx, int cmp, const hgpu_array* a, con
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   }
   buffer_release(scratch);
+  if (held_rc) return held_rc;
   if (e != hipSuccess) return check_hip(ctx, e, "compare_all");
   *result = host;
   return HGPU_OK;

@@ -74,6 +74,7 @@ struct hgpu_ctx {
   bool profiling = false;
   bool profile_shapes = false;           // hgpu_profile_enable(ctx, 2): labels carry the problem shape
   std::set<std::string> label_pool;
+  std::mutex label_mu;                    // guards label_pool: labels are made on any calling thread
   std::vector<ProfRec> prof;
   hgpu_buffer* zero_block = nullptr;     // 256 zero bytes, for kernels that want a dummy table
   hgpu_cap_pool* cap = nullptr;          // non-null while the stream is capturing into a graph
@@ -81,7 +82,7 @@ struct hgpu_ctx {
   // stream: those that do not depend on one another then go out as one kernel.
   hg::DeferredQueue* dq = nullptr;
   bool dq_pending = false;
-  int deferred_rc = 0;                   // first error of a held-back launch, reported by hgpu_sync
+  int deferred_rc = 0;                   // first error of a held-back launch, reported by the next call that hands results to the host
 };
 
 struct hgpu_graph {
@@ -197,6 +198,22 @@ struct LaunchGuard {
     ctx->launch_mu.unlock();
   }
 };
+
+// A label with the lifetime of the context (profiling records keep the pointer).
+inline const char* intern_label(hgpu_ctx* c, const std::string& s) {
+  std::lock_guard<std::mutex> g(c->label_mu);
+  return c->label_pool.insert(s).first->c_str();
+}
+
+// The first error of a launch that had been held back and failed after its own
+// call returned; cleared once handed out.  Every entry point that hands data or
+// a finished recording to the host reports it, since the caller would otherwise
+// read a result that was never written.  Call with launch_mu held.
+inline int take_deferred_rc(hgpu_ctx* c) {
+  const int rc = c->deferred_rc;
+  c->deferred_rc = 0;
+  return rc;
+}
 
 }  // namespace hg
 

@@ -476,7 +476,7 @@ int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red
     for (int i = 0; i < keep.nd && n < (int)sizeof buf - 40; ++i)
       n += snprintf(buf + n, sizeof buf - n, "_%lld:%lld/%lld", (long long)keep.shape[i], (long long)keep.st[0][i], (long long)keep.st[1][i]);
     snprintf(buf + n, sizeof buf - n, "]");
-    label = ctx->label_pool.insert(buf).first->c_str();
+    label = intern_label(ctx, buf);
   }
   const double nterms = tp.n ? tp.n : 1;
   LaunchGuard lg(ctx, label,

@@ -310,7 +310,7 @@ int copy_view(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const vo
     for (int i = 0; i < d.nd && w < (int)sizeof buf - 60; ++i)
       w += snprintf(buf + w, sizeof buf - w, ",%lld:%lld>%lld", (long long)d.shape[i], (long long)d.st[0][i], (long long)d.st[1][i]);
     snprintf(buf + w, sizeof buf - w, "]");
-    label = ctx->label_pool.insert(buf).first->c_str();
+    label = intern_label(ctx, buf);
   }
   LaunchGuard lg(ctx, label, 2.0 * n * dtype_size(dtype), 0);
   unsigned g = grid_for(n, kBlock, max_blocks(ctx));
@@ -398,7 +398,7 @@ int hgpu_pad(hgpu_ctx* ctx, const hgpu_array* a, const int64_t* lo, const int64_
       for (int i = 0; i < d.nd && w < (int)sizeof buf - 80; ++i)
         w += snprintf(buf + w, sizeof buf - w, ",%lld+%lld/%lld:%lld", (long long)d.lo[i], (long long)d.ext[i], (long long)d.shape[i], (long long)d.sst[i]);
       snprintf(buf + w, sizeof buf - w, "]");
-      label = ctx->label_pool.insert(buf).first->c_str();
+      label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, (double)(n + nelem(a)) * dtype_size(a->dtype), 0);
     const void* src = data_ptr(a);

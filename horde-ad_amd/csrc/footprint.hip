@@ -1089,7 +1089,7 @@ int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const v
       snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB1,footprint,%s%s,chunks%lld,rows%d,kgroups%d,lds%dK%s%s]", label, (long long)p.M, (long long)p.N,
                (long long)p.K, pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? ",swapped" : "", (long long)pl.nch, pl.min_rows, (int)pl.gx.size(), lds_bytes(pl) / 1024,
                vx ? ",xmap" : "", vy ? ",ymap" : "");
-      label = ctx->label_pool.insert(buf).first->c_str();
+      label = intern_label(ctx, buf);
     }
     {
       LaunchGuard lg(ctx, label, bytes, flops);
@@ -1531,7 +1531,7 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
       snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB1,footprint,chunkM%s,chunks%lld,rows%d,kgroups%d,lds%dK,map(instr%d,out%d%s)]", label, (long long)M, (long long)N,
                (long long)K, swapped ? ",swapped" : "", (long long)pl.nch, pl.min_rows, (int)pl.gx.size(), lds_bytes(pl) / 1024, n_instr, n_out,
                has_ext ? (L == 4 ? ",ext4" : (L == 2 ? ",ext2" : ",ext1")) : "");
-      label = ctx->label_pool.insert(buf).first->c_str();
+      label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, bytes, flops);
     hipError_t err = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
@@ -1822,7 +1822,7 @@ int try_mapped_sum(hgpu_ctx* ctx, const VirtualOp& v, const hgpu_operand* o, int
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[160];
       snprintf(buf, sizeof buf, "mapped_sum[out%lld,R%lld,S%lld,in%d,instr%d,vec%d%s]", (long long)n_out, (long long)R, (long long)S, v.n_in, v.n_instr, W, v.padded ? ",padded" : "");
-      label = ctx->label_pool.insert(buf).first->c_str();
+      label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, bytes, (double)n_out * R * (v.n_instr + 1));
     hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)(n_out * S), 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);

@@ -376,7 +376,7 @@ static int fused_map_impl(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, 
         for (int d = 0; d < in[i]->rank; ++d) gst += (d ? ":" : ",g") + std::to_string(in[i]->strides[d]);
     char buf[200];
     snprintf(buf, sizeof buf, "%s[%s,in%d(%s),instr%d(k%d.op%d..),out%d,vec%d,dt%d%s]", kernel_name, sh.c_str(), n_in, layout.c_str(), n_instr, prog[0].kind, prog[0].op, n_out, all_simple ? vec : gvec, a0->dtype, gst.c_str());
-    label = ctx->label_pool.insert(buf).first->c_str();
+    label = intern_label(ctx, buf);
   }
   std::unique_ptr<LaunchGuard> guard(new LaunchGuard(ctx, label, 0, 0));   // ends before the partial sums' own launch
   LaunchGuard& lg = *guard;
@@ -560,7 +560,7 @@ extern "C" int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     for (int d = 0; d < a0->rank; ++d) sh += (d ? "x" : "") + std::to_string(a0->shape[d]);
     char buf[160];
     snprintf(buf, sizeof buf, "fused_extremum[%s,reduce%d,in%d(%s),instr%d]", sh.c_str(), n_reduce, n_in, layout.c_str(), n_instr);
-    label = ctx->label_pool.insert(buf).first->c_str();
+    label = intern_label(ctx, buf);
   }
   double bytes = (double)n_out * (dtype_size(dt[(size_t)slot]) + 8);
   for (int i = 0; i < n_in; ++i) {
@@ -706,7 +706,7 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     for (int d = 0; d < a0->rank; ++d) sh += (d ? "x" : "") + std::to_string(a0->shape[d]);
     char buf[160];
     snprintf(buf, sizeof buf, "fused_sum[%s,in%d(%s),instr%d,vec%d]", sh.c_str(), n_in, layout.c_str(), n_instr, vec);
-    label = ctx->label_pool.insert(buf).first->c_str();
+    label = intern_label(ctx, buf);
   }
   double bytes = 0;
   for (int i = 0; i < n_in; ++i) {
@@ -881,7 +881,7 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     for (int d = 0; d < a0->rank; ++d) sh += (d ? "x" : "") + std::to_string(a0->shape[d]);
     char buf[160];
     snprintf(buf, sizeof buf, "fused_map_sums[%s,in%d(%s),instr%d,out%d,sums%d,vec%d]", sh.c_str(), n_in, layout.c_str(), n_instr, n_out, n_sum, vec);
-    label = ctx->label_pool.insert(buf).first->c_str();
+    label = intern_label(ctx, buf);
   }
   double bytes = 0;
   for (int i = 0; i < n_in; ++i) {

@@ -230,7 +230,7 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[128];
       snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,direct,t%dx%d,k%lld:%lld/%lld]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, (int)split, 16 * tm, 16 * tn, (long long)p.k.shape[p.k.nd - 1], (long long)p.k.sa[p.k.nd - 1], (long long)p.k.sb[p.k.nd - 1]);
-      label = ctx->label_pool.insert(buf).first->c_str();
+      label = intern_label(ctx, buf);
     }
     // the helper launches are timed under their own names, the label times the MFMA kernel alone
     if (p.k.nd > 1) {
@@ -548,7 +548,7 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
       char terms[24] = "";
       if (nt > 1) snprintf(terms, sizeof terms, ",terms%lld%s", (long long)nt, p.term_loop ? "loop" : "");
       snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB%lld,s%d,%s%s,t%lldx%lld%s]", label, (long long)p.M, (long long)p.N, (long long)p.K, (long long)p.BT, split, akc ? (va ? "K" : "k") : (va ? "M" : "m"), bkc ? (vb ? "K" : "k") : (vb ? "N" : "n"), (long long)BM, (long long)BN, terms);
-      label = ctx->label_pool.insert(buf).first->c_str();
+      label = intern_label(ctx, buf);
     }
     // the helper launches are timed under their own names, the label times the MFMA kernel alone
     if (p.k.nd > 1) {

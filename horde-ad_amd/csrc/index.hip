@@ -15,7 +15,10 @@
 // OpsConcrete.hs:1581-1619), and without atomics: the positions are sorted by
 // destination with a stable radix sort, and every destination's run is summed
 // front to back by one lane per element.  Results do not depend on the run and,
-// for floating point, carry the rounding of that very order.
+// for floating point, carry the rounding of that very order as long as no
+// destination is hit more than 256 times; a longer run is summed in segments
+// of 256 entries (each front to back) whose sums are added in ascending order,
+// so that the serial part of a scatter into a handful of cells stays bounded.
 #include "common.hpp"
 
 #include <rocprim/rocprim.hpp>
@@ -143,15 +146,25 @@ __global__ void __launch_bounds__(kBlock) k_scatter_store(IxSpace sp, Dims inner
   }
 }
 
+// Entries of one run that a lane adds front to back.  A destination hit by at most
+// kSeg positions is summed in exactly the reference's order; a longer run is cut,
+// from its first entry, into segments of kSeg entries that separate lanes add up,
+// and the segment sums are then added in ascending order (k_scatter_combine).
+constexpr int kSeg = 256;
+
 // key[m] = where position m's slice starts in out (the same for colliding
-// positions), or `skip` when an index is out of bounds; val[m] = m.
-__global__ void __launch_bounds__(kBlock) k_scatter_keys(IxSpace sp, int64_t M, uint64_t skip, uint64_t* __restrict__ key, uint32_t* __restrict__ val) {
+// positions), or `skip` when an index is out of bounds; val[m] = m.  Also clears
+// long_head, one entry per kSeg sorted entries (see k_scatter_runs).
+template <typename K>
+__global__ void __launch_bounds__(kBlock) k_scatter_keys(IxSpace sp, int64_t M, K skip, K* __restrict__ key, uint32_t* __restrict__ val,
+                                                         uint32_t* __restrict__ long_head, int64_t n_buckets) {
   int64_t step = (int64_t)gridDim.x * kBlock;
   for (int64_t m = (int64_t)blockIdx.x * kBlock + threadIdx.x; m < M; m += step) {
     int64_t toff, doff;
     bool ok = resolve(sp, m, &toff, &doff);
-    key[m] = ok ? (uint64_t)toff : skip;
+    key[m] = ok ? (K)toff : skip;
     val[m] = (uint32_t)m;
+    if (m < n_buckets) long_head[m] = 0;
   }
 }
 
@@ -167,24 +180,126 @@ __device__ __forceinline__ int64_t data_offset(const IxSpace& sp, int64_t m) {
 }
 
 // key / val sorted by key, equal keys in ascending position order.  One lane per
-// (run, inner element): the lane at a run's first entry adds the run's slices
-// front to back, starting from zero, and writes the sum; the others have nothing to do.
-template <typename T>
-__global__ void __launch_bounds__(kBlock) k_scatter_runs(IxSpace sp, Dims inner, int64_t M, int64_t N, uint64_t skip, const uint64_t* __restrict__ key,
-                                                         const uint32_t* __restrict__ val, const T* __restrict__ src, T* __restrict__ out) {
+// (sorted entry, inner element); a lane works when its entry starts a SEGMENT:
+// the first entry of a run, or an entry a multiple of kSeg entries after it.
+// It adds the segment's slices front to back, starting from zero.  A run of one
+// segment is written to `out` at once.  The segment sums of a longer run go to
+// `part`, two places per bucket of kSeg sorted entries -- a bucket holds at most
+// one first segment of a long run (place 1) and one later segment (place 0),
+// because segments of one run start kSeg entries apart and a long run is
+// longer than a bucket -- and long_head[bucket] remembers where the run starts.
+template <typename T, typename K>
+__global__ void __launch_bounds__(kBlock) k_scatter_runs(IxSpace sp, Dims inner, int64_t M, int64_t N, K skip, const K* __restrict__ key,
+                                                         const uint32_t* __restrict__ val, const T* __restrict__ src, T* __restrict__ out,
+                                                         T* __restrict__ part, uint32_t* __restrict__ long_head) {
   int64_t total = M * N;
   int64_t step = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += step) {
     int64_t at = N == 1 ? i : i / N;
     int64_t n = N == 1 ? 0 : i - at * N;
-    const uint64_t k = key[at];
-    if (k == skip || (at > 0 && key[at - 1] == k)) continue;
+    const K k = key[at];
+    if (k == skip) continue;
+    const bool head = at == 0 || key[at - 1] != k;
+    if (!head) {
+      if (at < kSeg || key[at - kSeg] != k) continue;   // fewer than kSeg entries of this run before this one
+      int64_t lo = 0, hi = at - kSeg;                   // the run's first entry: the first key that is not smaller
+      while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (key[mid] < k) lo = mid + 1; else hi = mid;
+      }
+      if ((at - lo) % kSeg != 0) continue;
+    }
     int64_t io[1];
     decompose<1>(inner, n, io);
+    const int64_t end = at + kSeg < M ? at + kSeg : M;
     T acc = T(0);
-    for (int64_t j = at; j < M && key[j] == k; ++j) acc = (T)(acc + src[data_offset(sp, (int64_t)val[j]) + io[0]]);
+    int64_t j = at;
+    for (; j + 4 <= end; j += 4) {                      // four loads in flight, added in order
+      const K k1 = key[j + 1], k2 = key[j + 2], k3 = key[j + 3];
+      if (k1 != k || k2 != k || k3 != k) break;
+      const T v0 = src[data_offset(sp, (int64_t)val[j]) + io[0]], v1 = src[data_offset(sp, (int64_t)val[j + 1]) + io[0]];
+      const T v2 = src[data_offset(sp, (int64_t)val[j + 2]) + io[0]], v3 = src[data_offset(sp, (int64_t)val[j + 3]) + io[0]];
+      acc = (T)(acc + v0);
+      acc = (T)(acc + v1);
+      acc = (T)(acc + v2);
+      acc = (T)(acc + v3);
+    }
+    for (; j < end && key[j] == k; ++j) acc = (T)(acc + src[data_offset(sp, (int64_t)val[j]) + io[0]]);
+    const bool more = j < M && key[j] == k;
+    if (head && !more) {
+      out[(int64_t)k + n] = acc;
+    } else {
+      const int64_t q = at / kSeg;
+      part[(q * 2 + (head ? 1 : 0)) * N + n] = acc;
+      if (head && n == 0) long_head[q] = (uint32_t)(at - q * kSeg) + 1;
+    }
+  }
+}
+
+// One lane per (bucket, inner element): where a long run starts in the bucket,
+// its segment sums are added in ascending order and written to `out`.
+template <typename T, typename K>
+__global__ void __launch_bounds__(kBlock) k_scatter_combine(int64_t M, int64_t N, int64_t n_buckets, const K* __restrict__ key, const T* __restrict__ part,
+                                                            const uint32_t* __restrict__ long_head, T* __restrict__ out) {
+  int64_t total = n_buckets * N;
+  int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += step) {
+    int64_t q = N == 1 ? i : i / N;
+    int64_t n = N == 1 ? 0 : i - q * N;
+    const uint32_t h = long_head[q];
+    if (!h) continue;
+    const int64_t at = q * kSeg + (int64_t)h - 1;
+    const K k = key[at];
+    T acc = part[(q * 2 + 1) * N + n];
+    for (int64_t a = at + kSeg; a < M && key[a] == k; a += kSeg) acc = (T)(acc + part[(a / kSeg) * 2 * N + n]);
     out[(int64_t)k + n] = acc;
   }
+}
+
+// k_scatter_keys -> stable radix sort by key -> k_scatter_runs -> k_scatter_combine.
+// bufs: keys (in, out), positions (in, out), sort workspace, segment sums, long_head.
+template <typename K>
+hipError_t scatter_sorted(hgpu_ctx* ctx, const IxSpace& sp, const Dims& inner, int64_t M, int64_t N, const hgpu_array* src, hgpu_array* o, int* rc_out) {
+  const K skip = (K)nelem(o);   // larger than every slice start
+  int end_bit = 1;
+  while (end_bit < (int)(8 * sizeof(K)) && ((uint64_t)skip >> end_bit) != 0) ++end_bit;
+  const int64_t n_buckets = (M + kSeg - 1) / kSeg;
+  const size_t es = dtype_size(src->dtype);
+  hgpu_buffer *kb = nullptr, *vb = nullptr, *tb = nullptr, *pb = nullptr, *hb = nullptr;
+  auto drop = [&] { for (hgpu_buffer* b : {kb, vb, tb, pb, hb}) if (b) buffer_release(b); };
+  int rc = buffer_alloc(ctx, (size_t)M * 2 * sizeof(K), &kb);
+  if (!rc) rc = buffer_alloc(ctx, (size_t)M * 8, &vb);
+  if (!rc) rc = buffer_alloc(ctx, (size_t)n_buckets * 2 * (size_t)N * es, &pb);
+  if (!rc) rc = buffer_alloc(ctx, (size_t)n_buckets * 4, &hb);
+  if (rc) { drop(); *rc_out = rc; return hipSuccess; }
+  K* key_in = (K*)kb->ptr;
+  K* key_out = key_in + M;
+  uint32_t* val_in = (uint32_t*)vb->ptr;
+  uint32_t* val_out = val_in + M;
+  uint32_t* long_head = (uint32_t*)hb->ptr;
+  size_t temp_bytes = 0;
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp_bytes, key_in, key_out, val_in, val_out, (size_t)M, 0, (unsigned)end_bit, ctx->stream);
+  if (e == hipSuccess) {
+    rc = buffer_alloc(ctx, temp_bytes > 0 ? temp_bytes : 1, &tb);
+    if (rc) { drop(); *rc_out = rc; return hipSuccess; }
+    hipLaunchKernelGGL(k_scatter_keys<K>, dim3(grid_for(M, kBlock, ctx->num_cu * 8)), dim3(kBlock), 0, ctx->stream, sp, M, skip, key_in, val_in, long_head, n_buckets);
+    e = rocprim::radix_sort_pairs(tb->ptr, temp_bytes, key_in, key_out, val_in, val_out, (size_t)M, 0, (unsigned)end_bit, ctx->stream);
+    if (e == hipSuccess) {
+      unsigned g = grid_for(M * N, kBlock, ctx->num_cu * 8);
+      HG_DISPATCH_DTYPE(src->dtype, T, hipLaunchKernelGGL((k_scatter_runs<T, K>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, skip, (const K*)key_out, (const uint32_t*)val_out,
+                                                          (const T*)data_ptr(src), (T*)data_ptr(o), (T*)pb->ptr, long_head));
+      e = hipGetLastError();
+    }
+    if (e == hipSuccess) {
+      unsigned g = grid_for(n_buckets * N, kBlock, ctx->num_cu * 8);
+      HG_DISPATCH_DTYPE(src->dtype, T, hipLaunchKernelGGL((k_scatter_combine<T, K>), dim3(g), dim3(kBlock), 0, ctx->stream, M, N, n_buckets, (const K*)key_out, (const T*)pb->ptr,
+                                                          (const uint32_t*)long_head, (T*)data_ptr(o)));
+      e = hipGetLastError();
+    }
+  }
+  drop();
+  *rc_out = HGPU_OK;
+  return e;
 }
 
 int build_space(hgpu_ctx* ctx, const char* who, int n_ix, const hgpu_array* const* ix, int rank_m, const int64_t* shm,
@@ -284,7 +399,7 @@ int hgpu_gather(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_array
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[120];
       snprintf(buf, sizeof buf, "gather[es%d,M%lld,N%lld,ix%d]", (int)dtype_size(src->dtype), (long long)M, (long long)N, n_ix);
-      label = ctx->label_pool.insert(buf).first->c_str();
+      label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, 0);
     // contiguous slices of whole 16-byte (or 8-byte) units: one unit per lane
@@ -359,33 +474,13 @@ int hgpu_scatter_add(hgpu_ctx* ctx, const hgpu_array* src, int n_ix, const hgpu_
   }
   // sort the positions by destination (stable: colliding positions stay in ascending order), then sum every run in that order
   if (M >= (int64_t)1 << 32) { hgpu_release(o); return fail(ctx, HGPU_ERR_UNSUPPORTED, "scatter: %lld positions", (long long)M); }
-  const uint64_t skip = (uint64_t)nelem(o);   // larger than every slice start
-  int end_bit = 1;
-  while (end_bit < 64 && (skip >> end_bit) != 0) ++end_bit;
-  hgpu_buffer *kb = nullptr, *vb = nullptr, *tb = nullptr;
-  auto drop = [&] { if (kb) buffer_release(kb); if (vb) buffer_release(vb); if (tb) buffer_release(tb); };
-  rc = buffer_alloc(ctx, (size_t)M * 16, &kb);          // keys in, keys out
-  if (!rc) rc = buffer_alloc(ctx, (size_t)M * 8, &vb);  // positions in, positions out
-  if (rc) { drop(); hgpu_release(o); return rc; }
-  uint64_t* key_in = (uint64_t*)kb->ptr;
-  uint64_t* key_out = key_in + M;
-  uint32_t* val_in = (uint32_t*)vb->ptr;
-  uint32_t* val_out = val_in + M;
-  size_t temp_bytes = 0;
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, temp_bytes, key_in, key_out, val_in, val_out, (size_t)M, 0, (unsigned)end_bit, ctx->stream);
-  if (e == hipSuccess) {
-    rc = buffer_alloc(ctx, temp_bytes > 0 ? temp_bytes : 1, &tb);
-    if (rc) { drop(); hgpu_release(o); return rc; }
+  hipError_t e;
+  {
     LaunchGuard lg(ctx, "scatter_sorted", 2.0 * M * N * dtype_size(src->dtype) + 8.0 * M * n_ix, (double)M * N);
-    hipLaunchKernelGGL(k_scatter_keys, dim3(grid_for(M, kBlock, ctx->num_cu * 8)), dim3(kBlock), 0, ctx->stream, sp, M, skip, key_in, val_in);
-    e = rocprim::radix_sort_pairs(tb->ptr, temp_bytes, key_in, key_out, val_in, val_out, (size_t)M, 0, (unsigned)end_bit, ctx->stream);
-    if (e == hipSuccess) {
-      unsigned g = grid_for(M * N, kBlock, ctx->num_cu * 8);
-      HG_DISPATCH_DTYPE(src->dtype, T, hipLaunchKernelGGL((k_scatter_runs<T>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, skip, key_out, val_out, (const T*)data_ptr(src), (T*)data_ptr(o)));
-      e = hipGetLastError();
-    }
+    // destinations that fit 32 bits sort as 32-bit keys: half the bytes per sorting pass
+    e = nelem(o) < (int64_t)0xffffffff ? scatter_sorted<uint32_t>(ctx, sp, inner, M, N, src, o, &rc) : scatter_sorted<uint64_t>(ctx, sp, inner, M, N, src, o, &rc);
   }
-  drop();
+  if (rc) { hgpu_release(o); return rc; }
   if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "scatter"); }
   *out = o;
   return HGPU_OK;

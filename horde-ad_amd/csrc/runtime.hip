@@ -340,6 +340,11 @@ int hgpu_capture_end(hgpu_ctx* ctx, hgpu_graph** out) {
   if (!ctx->cap) return fail(ctx, HGPU_ERR_INVALID, "capture_end: no capture is open");
   (void)hipSetDevice(ctx->device);
   flush_deferred(ctx);          // launches still held back belong to the graph
+  int held_rc;
+  {
+    std::lock_guard<std::mutex> lk(ctx->launch_mu);
+    held_rc = take_deferred_rc(ctx);
+  }
   hgpu_cap_pool* pool;
   {
     std::lock_guard<std::mutex> g(ctx->mu);
@@ -350,13 +355,13 @@ int hgpu_capture_end(hgpu_ctx* ctx, hgpu_graph** out) {
   gr->ctx = ctx;
   gr->pool = pool;
   hipError_t e = hipStreamEndCapture(ctx->stream, &gr->graph);
-  if (e == hipSuccess) e = hipGraphInstantiate(&gr->exec, gr->graph, nullptr, nullptr, 0);
-  if (e != hipSuccess) {
+  if (e == hipSuccess && !held_rc) e = hipGraphInstantiate(&gr->exec, gr->graph, nullptr, nullptr, 0);
+  if (e != hipSuccess || held_rc) {
     (void)hipGetLastError();
     if (gr->graph) (void)hipGraphDestroy(gr->graph);
     retire_pool(ctx, pool);
     delete gr;
-    return check_hip(ctx, e, "capture_end");
+    return held_rc ? held_rc : check_hip(ctx, e, "capture_end");   // a recording that lacks a launch is no recording
   }
   *out = gr;
   return HGPU_OK;
@@ -369,6 +374,7 @@ int hgpu_graph_launch(hgpu_graph* gr) {
   std::lock_guard<std::mutex> lk(ctx->launch_mu);
   (void)hipSetDevice(ctx->device);
   if (ctx->dq_pending) flush_deferred_locked(ctx);
+  if (int rc = take_deferred_rc(ctx)) return rc;
   return check_hip(ctx, hipGraphLaunch(gr->exec, ctx->stream), "hipGraphLaunch");
 }
 
@@ -409,10 +415,8 @@ int hgpu_sync(hgpu_ctx* ctx) {
   (void)hipSetDevice(ctx->device);
   flush_deferred(ctx);
   int rc = check_hip(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
-  if (ctx->deferred_rc) {      // a launch that was held back failed after its call had returned
-    rc = ctx->deferred_rc;
-    ctx->deferred_rc = 0;
-  }
+  std::lock_guard<std::mutex> lk(ctx->launch_mu);
+  if (int held_rc = take_deferred_rc(ctx)) rc = held_rc;      // a launch that was held back failed after its call had returned
   return rc;
 }
 
@@ -558,12 +562,15 @@ int hgpu_download(hgpu_ctx* ctx, const hgpu_array* a, void* host) {
     src = dense;
   }
   hipError_t e;
+  int held_rc;
   {
     LaunchGuard lg(ctx);
+    held_rc = take_deferred_rc(ctx);
     e = hipMemcpyAsync(host, data_ptr(src), bytes, hipMemcpyDeviceToHost, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   }
   if (dense) hgpu_release(dense);
+  if (held_rc) return held_rc;
   return check_hip(ctx, e, "download");
 }
 
@@ -572,8 +579,10 @@ int hgpu_read_scalar(hgpu_ctx* ctx, const hgpu_array* a, void* host) {
   if (nelem(a) != 1) return fail(ctx, HGPU_ERR_INVALID, "read_scalar of an array with %lld elements", (long long)nelem(a));
   if (int rc = no_capture(ctx, "read_scalar")) return rc;
   LaunchGuard lg(ctx);
+  const int held_rc = take_deferred_rc(ctx);
   hipError_t e = hipMemcpyAsync(host, data_ptr(a), dtype_size(a->dtype), hipMemcpyDeviceToHost, ctx->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  if (held_rc) return held_rc;
   return check_hip(ctx, e, "read_scalar");
 }
 

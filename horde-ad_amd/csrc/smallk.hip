@@ -560,7 +560,8 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
   const hgpu_array* a0 = as[0];
   if (a0->dtype != HGPU_F64 && a0->dtype != HGPU_F32) return HGPU_OK;
   if (n_terms < 1 || n_terms > kMaxTermsSmallK || n_out < 1) return HGPU_OK;
-  if (getenv("HORDEAD_NO_SMALLK")) return HGPU_OK;
+  static const bool disabled = getenv("HORDEAD_NO_SMALLK") != nullptr;
+  if (disabled) return HGPU_OK;
   KeptDims kd;
   if (!kept_dims(n_keep, a0->shape, &kd)) return HGPU_OK;
   Spec sp;
@@ -636,7 +637,7 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
     for (auto& tm : sp.terms) ks += (ks.empty() ? "" : "+") + std::to_string(tm.K);
     snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%sxB1,wholeK,t%dx%d,chunks%d,lds%dK,map(in%d,instr%d,out%d)]", d.label, (long long)sp.Q, (long long)sp.P, ks.c_str(), sp.BQ,
              sp.BP, (int)sp.chunks.size(), (int)((sp.x_elems + sp.y_elems) * (int)es / 1024), n_in - 1, n_instr, n_out);
-    d.label = ctx->label_pool.insert(buf).first->c_str();
+    d.label = intern_label(ctx, buf);
   }
   static const bool hold = getenv("HORDEAD_NO_GROUPED_LAUNCH") == nullptr;
   if (hold && nblk <= kGroupBlocksPerCu * ctx->num_cu) {
@@ -743,7 +744,7 @@ void flush_deferred_locked(hgpu_ctx* ctx) {
           lab += (d == grp[0] ? "" : "|") + in;
         }
         const char* label = grp[0]->label;
-        if (ctx->profiling && ctx->profile_shapes) label = ctx->label_pool.insert(lab + "]").first->c_str();
+        if (ctx->profiling && ctx->profile_shapes) label = intern_label(ctx, lab + "]");
         timed_launch(fn, grid, ar, label, bytes, flops);
         ctx->dq->n_grouped += (long)grp.size();
       } else {

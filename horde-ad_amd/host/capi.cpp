@@ -300,6 +300,21 @@ int hh_ix_index0(hh_ctx* c, hh_val* t, int n, hh_ix* const* ix, hh_ix** out) { H
 int hh_ix_argminmax(hh_ctx* c, hh_val* t, int n, hh_ix* const* ix, int want_max, hh_ix** out) {
   HH_IX(ix_argminmax(&c->be, t->d.primal, ixs(n, ix), want_max != 0));
 }
+int hh_ix_from_val(hh_ctx* c, hh_val* v, hh_ix** out) {
+  if (!c || !v || !out) return HGPU_ERR_INVALID;
+  return guarded(c, [&] {
+    Ix x;
+    x.shm = v->d.primal.shape();
+    x.arr = v->d.primal;
+    x.dtype = v->d.primal.dtype();
+    *out = boxi(x);
+  });
+}
+int hh_ix_to_val(hh_ctx* c, hh_ix* x, hh_val** out) {
+  if (!c || !x || !out) return HGPU_ERR_INVALID;
+  HH_OP(d_const(ix_array(&c->be, x->x)));
+}
+int hh_ix_dtype(hh_ix* x) { return x ? x->x.dtype : -1; }
 int hh_ix_free(hh_ix* x) { delete x; return HGPU_OK; }
 int hh_ix_is_affine(hh_ix* x) { return x && x->x.affine ? 1 : 0; }
 int64_t hh_counter(hh_ctx* c, const char* name) {

@@ -36,6 +36,7 @@ SIG = {
     "ix_select": (I, [P, P, P, P, PP]), "ix_convert": (I, [P, P, I, I, PP]),
     "ix_index0": (I, [P, P, I, PP, PP]), "ix_argminmax": (I, [P, P, I, PP, I, PP]), "ix_free": (I, [P]),
     "ix_is_affine": (I, [P]), "counter": (L, [P, C.c_char_p]),
+    "ix_from_val": (I, [P, P, PP]), "ix_to_val": (I, [P, P, PP]), "ix_dtype": (I, [P]),
     "tconvert": (I, [P, I, P, I, LP, PP]), "dense": (I, [P, P, PP]),
     "tsgather": (I, [P, P, I, LP, I, PP, PP]), "tsscatter": (I, [P, P, I, I, LP, PP, PP]),
     "capture_begin": (I, [P]), "capture_end": (I, [P, PP]), "graph_launch": (I, [P, P]), "graph_free": (I, [P, P]),
@@ -204,6 +205,34 @@ class Host:
         """tsbuild1 (OpsConcrete.hs:1761-1774): [f 0, ..., f (k-1)] stacked; f gets a concrete index."""
         return self.sfromVector([f(i) for i in range(k)])
 
+    def kbuild(self, shm, f, dtype=None):
+        """tkbuild @shm f (Ops.hs:863-880; Concrete: one vector generate, OpsConcrete.hs:1081-1087):
+        f gets the position variables as lane values and runs once; its result (a lane
+        value, or a Python number with `dtype`) is written out as an array of shape shm."""
+        shm = tuple(int(s) for s in shm)
+        r = f(*self.ix_space(shm))
+        if not isinstance(r, IxV):
+            r = IxV.const(self, shm, r, capi.I64 if dtype is None else dtype)
+        elif dtype is not None and r.dtype != dtype:
+            raise HgpuError(1, "kbuild: the closure's result is not of the element type asked for")
+        return r.to_val()
+
+    def kbuild1(self, k, f, dtype=None):
+        """tkbuild1 @k f (Ops.hs:860-862)."""
+        return self.kbuild((k,), f, dtype)
+
+    def sbuild(self, shm, f):
+        """tsbuild @shm f for a closure that yields arrays (Ops.hs:913-928, OpsConcrete.hs:1776-1789):
+        the reference's nest of tsbuild1 host loops, f gets concrete indices.  With scalar
+        elements (shn = []) the reference takes tbuildK instead: that is `kbuild`."""
+        shm = tuple(int(s) for s in shm)
+
+        def level(prefix, rest):
+            if not rest:
+                return f(*prefix)
+            return self.sbuild1(rest[0], lambda i: level(prefix + [i], rest[1:]))
+        return level([], list(shm))
+
     def smapAccumL(self, f, acc0, xs):
         """tmapAccumL (OpsConcrete.hs:990-1019): threads `acc` through the outermost
         dim of xs; f(acc, x) -> (acc', y).  Returns (final acc, stacked ys)."""
@@ -250,14 +279,29 @@ class IxV:
     def const(host, shm, value, dtype=capi.I64):
         return IxV(host, host._ixo(host.dll.hh_ix_const, len(shm), _larr(shm), dtype, float(value)), shm)
 
-    def _coerce(self, o, dtype=capi.I64):
-        return o if isinstance(o, IxV) else IxV.const(self.host, self.shm, o, dtype)
+    @staticmethod
+    def from_val(v):
+        """The elements of an array as a lane value over the array's own index space
+        (what the scalar closure of tsmap0N / tszipWith0N is applied to)."""
+        return IxV(v.host, v.host._ixo(v.host.dll.hh_ix_from_val, v.h), tuple(v.shape))
 
-    def _op2(self, op, o, dtype=capi.I64):
+    def to_val(self):
+        """This lane value as an array of shape shm."""
+        return self.host._out(self.host.dll.hh_ix_to_val, self.h)
+
+    @property
+    def dtype(self):
+        return int(self.host.dll.hh_ix_dtype(self.h))
+
+    def _coerce(self, o, dtype=None):
+        """A Python number beside a lane value is a literal of the lane value's element type."""
+        return o if isinstance(o, IxV) else IxV.const(self.host, self.shm, o, self.dtype if dtype is None else dtype)
+
+    def _op2(self, op, o, dtype=None):
         o = self._coerce(o, dtype)
         return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_op2, OP2[op], self.h, o.h), self.shm)
 
-    def _rop2(self, op, o, dtype=capi.I64):
+    def _rop2(self, op, o, dtype=None):
         return self._coerce(o, dtype)._op2(op, self)
 
     @property
@@ -270,6 +314,10 @@ class IxV:
     def __rsub__(self, o): return self._rop2("sub", o)
     def __mul__(self, o): return self._op2("mul", o)
     def __rmul__(self, o): return self._rop2("mul", o)
+    def __truediv__(self, o): return self._op2("div", o)
+    def __rtruediv__(self, o): return self._rop2("div", o)
+    def __pow__(self, o): return self._op2("pow", o)
+    def atan2H(self, o): return self._op2("atan2", o)
     def __neg__(self): return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_op1, OP1["neg"], self.h), self.shm)
     def quotH(self, o): return self._op2("quot", o)
     def remH(self, o): return self._op2("rem_scalar", o)      # scalar rule: remH a 0 = a (Types.hs:402-419)
@@ -281,18 +329,23 @@ class IxV:
         o = self._coerce(o, dtype)
         return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_compare, CMP[c], self.h, o.h), self.shm)
 
-    def leq(self, o, dtype=capi.I64): return self._cmp("leq", o, dtype)     # <=.
-    def lt(self, o, dtype=capi.I64): return self._cmp("lt", o, dtype)       # <.
-    def eq(self, o, dtype=capi.I64): return self._cmp("eq", o, dtype)       # ==.
+    def leq(self, o, dtype=None): return self._cmp("leq", o, dtype)     # <=.
+    def lt(self, o, dtype=None): return self._cmp("lt", o, dtype)       # <.
+    def eq(self, o, dtype=None): return self._cmp("eq", o, dtype)       # ==.
+    def notB(self): return self.op1("not")
+    def andB(self, o): return self._op2("and", o)                        # &&*
 
     def convert(self, dtype, mode=0):
         return IxV(self.host, self.host._ixo(self.host.dll.hh_ix_convert, self.h, dtype, mode), self.shm)
 
 
-def ifH(cond, a, b):
-    """ifH / kcond on lane-batched scalars."""
-    a = a if isinstance(a, IxV) else IxV.const(cond.host, cond.shm, a)
-    b = b if isinstance(b, IxV) else IxV.const(cond.host, cond.shm, b)
+def ifH(cond, a, b, dtype=None):
+    """ifH / kcond on lane-batched scalars.  Python numbers take the other branch's element
+    type, or `dtype`, or Int."""
+    if dtype is None:
+        dtype = a.dtype if isinstance(a, IxV) else b.dtype if isinstance(b, IxV) else capi.I64
+    a = a if isinstance(a, IxV) else IxV.const(cond.host, cond.shm, a, dtype)
+    b = b if isinstance(b, IxV) else IxV.const(cond.host, cond.shm, b, dtype)
     return IxV(cond.host, cond.host._ixo(cond.host.dll.hh_ix_select, cond.h, a.h, b.h), cond.shm)
 
 
@@ -388,6 +441,17 @@ class V:
     def sfromIntegral(self, dtype): return self._o(self.host.dll.hh_convert, self.h, dtype, 0)
     def sfloor(self, dtype=capi.I64): return self._o(self.host.dll.hh_convert, self.h, dtype, 1)
 
+    # -- maps of scalar closures (Ops.hs:929-941): the closure runs once, on lane values
+    def smap0N(self, f):
+        """tsmap0N f self"""
+        return f(IxV.from_val(self)).to_val()
+
+    def szipWith0N(self, f, o):
+        """tszipWith0N f self o"""
+        if tuple(self.shape) != tuple(o.shape):
+            raise HgpuError(1, "szipWith0N: the two arrays differ in shape")
+        return f(IxV.from_val(self), IxV.from_val(o)).to_val()
+
     # -- reductions and contractions
     def ssum(self): return self._o(self.host.dll.hh_tssumN, self.h, 1)
     def ssumN(self, k): return self._o(self.host.dll.hh_tssumN, self.h, k)
@@ -465,7 +529,7 @@ class V:
 # mixed method is its shaped twin under another name -- the same entry point,
 # the same kernel.  `rtr` = `str_`, `rmaxIndex` / `rminIndex` = `sargMax` /
 # `sargMin` as in the reference's naming.
-_TWINS = ["cast", "fromIntegral", "floor", "sum", "sumN", "sum0", "dot0", "dot1In", "dotNIn", "matvecmul", "matmul2",
+_TWINS = ["map0N", "zipWith0N", "cast", "fromIntegral", "floor", "sum", "sumN", "sum0", "dot0", "dot1In", "dotNIn", "matvecmul", "matmul2",
           "replicate", "replicateN", "append", "slice", "reverse", "transpose", "reshape", "index", "gather", "scatter", "index0"]
 for _n in _TWINS:
     for _p in ("r", "x"):
@@ -479,4 +543,5 @@ for _p in ("r", "x"):
     setattr(Host, _p + "iota", Host.siota)
     setattr(Host, _p + "fromVector", Host.sfromVector)
     setattr(Host, _p + "build1", Host.sbuild1)
+    setattr(Host, _p + "build", Host.sbuild)
     setattr(Host, _p + "mapAccumL", Host.smapAccumL)

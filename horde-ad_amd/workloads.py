@@ -49,7 +49,15 @@ def one_hot_labels(seed, n_classes, batch, dtype):
 # --------------------------------------------------------------- shared pieces
 
 def reluS(v):
-    """oneIfGtZero * v with oneIfGtZero = smap0N (\\x -> ifH (x <=. 0) 0 1) v."""
+    """oneIfGtZero * v with oneIfGtZero = smap0N (\\x -> ifH (x <=. 0) 0 1) (sprimalPart v),
+    the closure applied once to a lane value (External/CommonShapedOps.hs:42-44)."""
+    from .hostapi import ifH
+    one_if = v.sprimalPart().smap0N(lambda x: ifH(x.leq(0.0), 0.0, 1.0, v.dtype))
+    return one_if * v
+
+
+def reluS_select(v):
+    """The same with the mask written as an array comparison and an elementwise choice."""
     h = v.host
     mask = v.sprimalPart().leq(0.0)
     one_if = mask.select(h.srepl(v.shape, 0.0, v.dtype), h.srepl(v.shape, 1.0, v.dtype))

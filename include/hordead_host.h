@@ -179,6 +179,20 @@ int hh_ix_index0(hh_ctx* ctx, hh_val* t, int n, hh_ix* const* ix, hh_ix** out);
 /* AstArgMinK / AstArgMaxK of a partial index: kargMax (t !$ [ix...]); the
  * partial index must leave exactly the last dim of t. */
 int hh_ix_argminmax(hh_ctx* ctx, hh_val* t, int n, hh_ix* const* ix, int want_max, hh_ix** out);
+/* tkbuild / tsmap0N / tszipWith0N (Ops.hs:863-880, 929-941; Concrete runs them as one
+ * vector map over the elements, OpsConcrete.hs:671-714, 1081-1087, 1748-1759).
+ * hh_ix_from_val: the elements of an array (primal part) as a lane value over
+ * the position space shm = the array's own shape, so the scalar closure of a
+ * map runs once for all elements.  hh_ix_to_val: a lane value written out as
+ * an array of shape shm (no dual part).  The closure's arithmetic in between
+ * joins the deferred elementwise program like any other array arithmetic:
+ *   tsmap0N f v       = to_val (f (from_val v))
+ *   tszipWith0N f u v = to_val (f (from_val u) (from_val v))
+ *   tkbuild @sh f     = to_val (f [hh_ix_var 0, .., hh_ix_var (n-1)]) */
+int hh_ix_from_val(hh_ctx* ctx, hh_val* v, hh_ix** out);
+int hh_ix_to_val(hh_ctx* ctx, hh_ix* x, hh_val** out);
+/* The element type of a lane value (an hgpu dtype code). */
+int hh_ix_dtype(hh_ix* x);
 int hh_ix_free(hh_ix* x);
 /* 1 when the value is an affine form of the position variables (diagnostic). */
 int hh_ix_is_affine(hh_ix* x);

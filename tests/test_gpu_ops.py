@@ -427,13 +427,19 @@ def test_scatter(both, dt):
         shp = [int(RNG.integers(1, 6)) for _ in range(int(RNG.integers(0, 3)))]
         ix = ix_arrays(both, list(src.shape[:rank_m]), shp, view=True)
         assert_same(both.scatter_add(src, ix, rank_m, shp), 0.0, (src.shape, rank_m, shp))
-    # heavy collisions: 20000 positions into 7 cells.  Colliding positions are added in
-    # ascending order, as the reference and the checker do: bit-equal, also for floats,
-    # and the same from run to run
+    # collisions, at most 256 positions per cell: colliding positions are added in ascending
+    # order, as the reference and the checker do: bit-equal, also for floats
+    src = both.upload(rnd((1200, 2), dt))
+    ix = ix_arrays(both, [1200], [7])
+    assert np.bincount(ix[0].numpy()[0].ravel() + 1).max() <= 256
+    assert_same(both.scatter_add(src, ix, 1, [7]), 0.0)
+    # heavy collisions: 20000 positions into 7 cells.  A run longer than 256 is added in
+    # segments of 256 (each in ascending order) whose sums are added in ascending order:
+    # exact for integers, within the tolerance for floats, and the same from run to run
     src = both.upload(rnd((20000, 2), dt))
     ix = ix_arrays(both, [20000], [7])
     first = both.scatter_add(src, ix, 1, [7])
-    assert_same(first, 0.0)
+    assert_same(first, tol)
     again = both.scatter_add(src, ix, 1, [7])
     assert np.array_equal(first.numpy()[0], again.numpy()[0])
     # many destinations with a few positions each, some out of bounds, slices of 5
@@ -516,6 +522,32 @@ def test_scatter_small_ints(both, gpu):
         many = both.upload(rnd((5000, 3), dt))
         cells = [both.upload(RNG.integers(-1, 12, 5000).astype(np.int64))]
         assert_same(both.scatter_add(many, cells, 1, [11]))
+
+
+def test_scatter_into_a_handful_of_cells_is_bounded(both, gpu):
+    """A million positions into eight cells (a table's cotangent): runs of 125,000 are added
+    in segments of 256 by separate lanes, not by one lane front to back.  Exact for
+    integers; floats within the tolerance of a reordered sum; and the call, sort included,
+    takes milliseconds, not seconds."""
+    import time
+    M = 1 << 20
+    cells = RNG.integers(-1, 8, M).astype(np.int64)          # some out of bounds
+    for dt, n, tol in ((np.int64, 1, 0.0), (np.float64, 1, 1e-10), (np.float64, 24, 1e-10), (np.float32, 3, 1e-5)):
+        src = both.upload(rnd((M, n) if n > 1 else (M,), dt))
+        ix = [both.upload(cells)]
+        res = both.scatter_add(src, ix, 1, [8])
+        assert_same(res, tol, (dt, n))
+        got = res.numpy()[0]
+        want = np.zeros_like(got)
+        np.add.at(want, cells[(cells >= 0) & (cells < 8)], src.numpy()[1][(cells >= 0) & (cells < 8)])
+        np.testing.assert_allclose(got, want, rtol=max(tol, 1e-12) * 100, atol=1e-3 if dt == np.float32 else 1e-7)
+        dev = src.arrays[0]
+        gix = [ix[0].arrays[0]]
+        gpu.sync()
+        t0 = time.perf_counter()
+        gpu.scatter_add(dev, gix, 1, [8])
+        gpu.sync()
+        assert time.perf_counter() - t0 < 0.05, (dt, n, time.perf_counter() - t0)
 
 
 def test_gather_scatter_adjoint_large(both):
