@@ -3,8 +3,10 @@
 
 One "step" = one full forward + reverse gradient of a config's objective on one
 batch of synthetic input that is already resident in HBM (uploads happen before
-the timed region; every step ends with a stream sync, the equivalent of the
-reference forcing every gradient leaf, bench/ConvVjpBench.hs:174-175).  As the
+the timed region).  `ms_per_step` is throughput: the K timed steps are queued
+back to back and the host waits once after the last; `ms_per_step_synced` has
+the host wait for every step and read the loss back, the equivalent of the
+reference forcing every gradient leaf, bench/ConvVjpBench.hs:174-175.  As the
 reference builds its gradient artifact once and times its evaluation
 (bench/ConvVjpBench.hs:254-257), the gradient program is recorded once into a
 device graph and a step launches that graph; `ms_per_step_eager` is the same
@@ -73,7 +75,14 @@ def time_graph(host, wl, ps, ds, steps, warmup):
             graph.launch()
         host.sync()
         dt = time.perf_counter() - t0
-        return dt / steps, float(loss.numpy())
+        # the same with the host waiting for every step and reading the loss back, the way the reference's
+        # benchmark forces every gradient before the next one starts (bench/ConvVjpBench.hs:174-175)
+        t1 = time.perf_counter()
+        for _ in range(steps):
+            graph.launch()
+            last = float(loss.numpy())
+        dt_synced = time.perf_counter() - t1
+        return dt / steps, last, dt_synced / steps
     finally:
         graph.free()
 
@@ -144,10 +153,8 @@ def measured_traffic(label):
     if not os.path.exists(path):
         return None
     table = json.load(open(path))
-    for prefix, val in table.items():
-        if not prefix.startswith("_") and label.startswith(prefix):
-            return val
-    return None
+    val = table.get(label)      # the exact label only: a changed kernel or shape has no figure until it is measured again
+    return None if label.startswith("_") else val
 
 
 def roofline_of(rep, dtype_name):
@@ -194,7 +201,7 @@ def cpu_baseline(pkg, key, mk):
         if time.perf_counter() - t0 > 8.0 or n >= 3:
             break
     dt = (time.perf_counter() - t0) / n
-    return {"value": wl.batch / dt, "unit": "samples/s", "cores": 1, "kind": "port",
+    return {"value": wl.batch / dt, "unit": "samples/s", "cores": 1, "host_cores": os.cpu_count(), "kind": "port",
             "sample": f"{wl.name} at {CPU_SAMPLE[key]} ({wl.batch} samples per gradient, {n} gradients, {dt:.3f} s each)"}
 
 
@@ -256,7 +263,7 @@ def main():
         ps, ds = wl.upload(host)
         host.sync()
         eager_sec, loss = time_steps(host, wl, ps, ds, args.steps, args.warmup)
-        sec, graph_loss = (eager_sec, loss) if args.eager else time_graph(host, wl, ps, ds, args.steps, args.warmup)
+        sec, graph_loss, synced_sec = (eager_sec, loss, None) if args.eager else time_graph(host, wl, ps, ds, args.steps, args.warmup)
         if graph_loss != loss:
             raise SystemExit(f"bench.py: {key}: the recorded program computed {graph_loss!r}, the eager one {loss!r}")
         rep = profile(capi, host, wl, ps, ds)
@@ -267,7 +274,9 @@ def main():
         gemm_fl = sum(v[3] for k, v in rep.items() if family(k) in MFMA_KERNELS)
         results[key] = {"workload": wl.name, "dtype": dn, "batch": wl.batch, "ms_per_step": sec * 1e3,
                         "samples_per_s": wl.batch / sec, "gradients_per_s": 1.0 / sec, "loss": loss,
+                        "ms_per_step_synced": None if synced_sec is None else synced_sec * 1e3,
                         "ms_per_step_eager": eager_sec * 1e3, "execution": "eager" if args.eager else "recorded graph, one launch per step",
+                        "launches_per_step": sum(v[0] for v in rep.values()),
                         "device_ms_per_step": dev_ms, "algorithmic_gflop": wl.flops / 1e9,
                         "achieved_tflops": wl.flops / sec / 1e12, "roofline": roof, "kernel_ms": shares,
                         "all_matrix_products": {"ms": gemm_ms, "tflops": gemm_fl / gemm_ms / 1e9 if gemm_ms > 0 else None,
@@ -285,7 +294,7 @@ def main():
             ps, ds = wl.upload(host)
             host.sync()
             eager_sec, loss = time_steps(host, wl, ps, ds, args.steps, args.warmup)
-            sec, graph_loss = (eager_sec, loss) if args.eager else time_graph(host, wl, ps, ds, args.steps, args.warmup)
+            sec, graph_loss, _ = (eager_sec, loss, None) if args.eager else time_graph(host, wl, ps, ds, args.steps, args.warmup)
             if graph_loss != loss:
                 raise SystemExit(f"bench.py: {key}: the recorded program computed {graph_loss!r}, the eager one {loss!r}")
             riders[key] = {"workload": wl.name, "batch": wl.batch, "ms_per_step": sec * 1e3, "ms_per_step_eager": eager_sec * 1e3, "loss": loss}
@@ -310,6 +319,7 @@ def main():
     line = {
         "metric": "gradient samples/sec at 1 GPU", "value": head["samples_per_s"], "unit": "samples/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "ms_per_step_synced": head["ms_per_step_synced"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
         "data": "synthetic",
         "config": {"workload": f"{head['workload']}: forward + reverse gradient, batch {head['batch']}, {head['dtype']}"},

@@ -561,6 +561,12 @@ int reduce_views(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_
     if (S > maxS) S = maxS;
     if (S > 4096) S = 4096;
   }
+  // A caller's scratch bounds the partial sums: fewer chunks when they would not
+  // fit, none (one launch, every output summed whole) when not even two do.
+  if (scratch && S > 1 && (size_t)n_out * (size_t)S * 8 > scratch_bytes) {
+    S = (int64_t)(scratch_bytes / ((size_t)n_out * 8));
+    if (S < 2) S = 1;
+  }
   const void* pa = data_ptr(a);
   const void* pb = b ? data_ptr(b) : nullptr;
   int rc = HGPU_OK;
@@ -575,7 +581,7 @@ int reduce_views(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_
     hgpu_buffer* part = nullptr;
     void* pp = scratch;
     if (scratch) {
-      if (need > scratch_bytes)
+      if (need > scratch_bytes)   // cannot happen after the clamp above; kept as the guard of the fixed array
         return fail(ctx, HGPU_ERR_UNSUPPORTED, "contract: %lld outputs in %lld chunks need %zu bytes of partial sums, the fixed scratch holds %zu",
                     (long long)n_out, (long long)S, need, scratch_bytes);
     } else {

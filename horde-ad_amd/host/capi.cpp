@@ -168,6 +168,12 @@ int hh_dense(hh_ctx* c, hh_val* v, hh_val** out) {
 int hh_overwrite(hh_ctx* c, hh_val* v, const void* host) {
   return guarded(c, [&] {
     if (!has_graphs(c->be.api)) throw HostError(HGPU_ERR_UNSUPPORTED, "this provider has no overwrite");
+    const auto& holder = v->d.primal.holder();
+    if (holder->host_i64) {     // a small integer table is also kept on the host (index functions look constants up in it)
+      if (holder->host_i64_folded)
+        throw HostError(HGPU_ERR_INVALID, "overwrite: an index function has been simplified with this table's values; it is a constant of the program now");
+      std::memcpy(holder->host_i64->data(), host, holder->host_i64->size() * sizeof(int64_t));
+    }
     c->be.check(c->be.api->overwrite(c->be.ctx, v->d.primal.h(), host));
   });
 }

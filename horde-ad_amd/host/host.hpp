@@ -57,6 +57,7 @@ struct ArrHolder {
   // Small integer arrays that came from the host keep their values: index
   // functions that look constants up in them can then be folded on the host.
   std::shared_ptr<std::vector<int64_t>> host_i64;
+  bool host_i64_folded = false;   // some index function has been simplified with these values: they must not change any more
   // The one-element array this array repeats at every position (set by broadcast_scalar).
   std::shared_ptr<ArrHolder> scalar_src;
   // A pending elementwise product fa * fb (h == nullptr until it is needed as

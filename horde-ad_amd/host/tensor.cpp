@@ -2284,6 +2284,7 @@ T tsscatter(const T& src, int rank_m, const Shape& shp, const std::vector<Ix>& i
   }
   std::vector<T> arrs;
   for (auto& x : ix) arrs.push_back(ix_array(be, x));
+  be->counters[injective ? "scatter_stores" : "scatter_general"]++;
   return scatter_raw(src, arrs, rank_m, shp, injective ? 1 : 0);
 }
 
@@ -2328,6 +2329,7 @@ Ix ix_index0(Backend* be, const T& t, const std::vector<Ix>& ix) {
           }
         }
         if (affine_tab) {
+          t.holder()->host_i64_folded = true;
           Ix r;
           r.shm = shm;
           r.affine = true;

@@ -379,10 +379,15 @@ int hgpu_contract_operands(hgpu_ctx* ctx, const hgpu_operand* a, const hgpu_oper
  * takes the HBM-bound reduction kernels (never the matrix-product path, which
  * needs tables and partial products of its own), so floating-point sums may be
  * associated differently from hgpu_contract's when that runs a matrix product;
- * for plain sums and dot products the two agree bit for bit.  The partial sums
- * of a split reduction live in one fixed array of 1 MiB per device, held until
- * the process ends: a request that needs more (outputs x chunks x 8 bytes) fails
- * with HGPU_ERR_UNSUPPORTED and a message naming the size.  Every call on a
+ * for plain sums and dot products the two agree bit for bit as long as both
+ * cut the reduction into the same number of chunks.  The partial sums of a
+ * split reduction live in one fixed array of 1 MiB per device, held until the
+ * process ends: a request whose partial sums (outputs x chunks x 8 bytes) would
+ * exceed it runs with as many chunks as fit, or unsplit when not even two fit
+ * (then its sums are associated differently from hgpu_contract's: equal for
+ * integers, within rounding for floating point); no valid request is refused
+ * for its size.  A result array of the wrong shape, dtype or layout, or one
+ * that shares memory with an operand, is HGPU_ERR_INVALID.  Every call on a
  * device uses that device's one array: calls that overlap on one device (two
  * contexts, two streams) race; calls on one context are ordered by its stream. */
 int hgpu_contract_noalloc(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array* out);

@@ -59,6 +59,50 @@ def test_replays_match_eager(host, name, table):
         graph.free()
 
 
+def test_sorted_scatter_inside_a_recording(host):
+    """The general scatter-add (positions sorted by destination, runs added in order) recorded
+    into a graph: its sort is a library routine, so every replay is checked against the eager
+    result, with eager scatters of other sizes (which reuse the sort's workspace blocks) between
+    the replays, and again after the inputs changed."""
+    rng = np.random.default_rng(21)
+    m, cells_n = 50000, 301
+    cells = host.concrete(rng.integers(-3, cells_n + 3, m).astype(np.int64))
+    src = host.concrete(rng.standard_normal((m, 3)))
+    other_cells = host.concrete(rng.integers(0, 9, 7777).astype(np.int64))
+    other_src = host.concrete(rng.standard_normal(7777))
+
+    def program():
+        return src.sscatter(1, [cells_n], lambda i: [cells.sindex0([i])])
+
+    def numpy_scatter(c, x):
+        out = np.zeros((cells_n,) + x.shape[1:])
+        ok = (c >= 0) & (c < cells_n)
+        np.add.at(out, c[ok], x[ok])
+        return out
+
+    want = program().numpy()
+    np.testing.assert_allclose(want, numpy_scatter(cells.numpy(), src.numpy()), rtol=1e-10, atol=1e-12)
+    assert host.counter("scatter_general") > 0
+    graph, res = host.capture(program)
+    try:
+        for replay in range(3):
+            graph.launch()
+            host.sync()
+            assert np.array_equal(res.numpy(), want), replay
+            other_src.sscatter(1, [9], lambda i: [other_cells.sindex0([i])]).numpy()
+        new_cells = rng.integers(0, cells_n, m).astype(np.int64)
+        new_src = rng.standard_normal((m, 3))
+        cells.overwrite(new_cells)
+        src.overwrite(new_src)
+        graph.launch()
+        host.sync()
+        np.testing.assert_allclose(res.numpy(), numpy_scatter(new_cells, new_src), rtol=1e-10, atol=1e-12)
+        fresh = host.concrete(new_src).sscatter(1, [cells_n], lambda i: [host.concrete(new_cells).sindex0([i])])
+        assert np.array_equal(res.numpy(), fresh.numpy())
+    finally:
+        graph.free()
+
+
 def test_host_calls_refused_while_recording(host):
     x = host.concrete(np.arange(6.0).reshape(2, 3))
     y = (x * x).ssum0()

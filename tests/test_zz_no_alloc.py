@@ -1,7 +1,8 @@
 """hgpu_contract_noalloc: the contraction for callers that cannot allocate
 device memory.  Its partial sums live in one fixed array per device; every call
 is checked against hgpu_contract on the same operands, twice in a row, the
-second call on a smaller input (the array keeps the first call's contents)."""
+second call on a smaller input (the array keeps the first call's contents).
+Partial sums that would not fit the array run in fewer chunks."""
 import numpy as np
 import pytest
 
@@ -9,18 +10,26 @@ from conftest import capi
 
 
 def both_ways(gpu, a, b, n_keep):
-    """(hgpu_contract, hgpu_contract_noalloc) on the same uploaded operands; the
-    second must not change the number of device allocations."""
+    """(hgpu_contract, hgpu_contract_noalloc) on the same operands.  The entry point under
+    test runs FIRST and on a context of its own whose block cache is empty, so that any block
+    it asked the allocator for would be a counted device allocation (a cached block left by an
+    earlier hgpu_contract of the same size would hide it)."""
+    fresh = capi.Lib().context(0)
+    fa = fresh.upload(a)
+    fb = fresh.upload(b) if b is not None else None
+    out = fresh.upload(np.full(a.shape[:n_keep], 7, a.dtype))     # the caller's array, holding junk
+    fresh.sync()
+    before = fresh.mem_stats()
+    fa.contract_noalloc(fb, n_keep, out)
+    fresh.sync()
+    assert fresh.mem_stats()[2] == before[2], "hgpu_contract_noalloc allocated device memory"
+    got = out.numpy()
+    del fa, fb, out
+    fresh.shutdown()
     ga = gpu.upload(a)
     gb = gpu.upload(b) if b is not None else None
     want = ga.contract(gb, n_keep)
-    out = gpu.upload(np.full(a.shape[:n_keep], 7, a.dtype))       # the caller's array, holding junk
-    gpu.sync()
-    n_before = gpu.mem_stats()[2]
-    ga.contract_noalloc(gb, n_keep, out)
-    gpu.sync()
-    assert gpu.mem_stats()[2] == n_before, "hgpu_contract_noalloc allocated device memory"
-    return want.numpy(), out.numpy()
+    return want.numpy(), got
 
 
 @pytest.mark.gpu
@@ -52,14 +61,26 @@ def test_no_alloc_contract_matches_contract_twice_in_a_row(gpu):
 
 
 @pytest.mark.gpu
-def test_no_alloc_contract_refuses_what_does_not_fit(gpu):
-    # sums over the outer dim of [16384, 5000]: 5000 outputs in 53 chunks, 2.1 MB of partial sums, over the fixed 1 MiB
-    a = gpu.upload(np.ones((16384, 5000), np.int8)).transpose([1, 0])
+def test_no_alloc_contract_with_fewer_chunks_than_it_would_like(gpu):
+    # sums over the outer dim of [16384, 5000]: hgpu_contract cuts 5000 outputs into 53 chunks (2.1 MB of
+    # partial sums); the fixed 1 MiB holds 26, so the call runs with 26: integers exact, floats within rounding
+    a8 = np.ones((16384, 5000), np.int8)
+    a = gpu.upload(a8).transpose([1, 0])
     out = gpu.upload(np.zeros(5000, np.int8))
-    with pytest.raises(capi.HgpuError) as e:
-        a.contract_noalloc(None, 1, out)
-    assert e.value.code == 4 and "scratch" in str(e.value)
-    assert np.array_equal(a.contract(None, 1).numpy(), np.full(5000, 16384 % 256, np.int64).astype(np.int8))   # the allocating entry point takes it
+    a.contract_noalloc(None, 1, out)
+    assert np.array_equal(out.numpy(), np.full(5000, 16384 % 256, np.int64).astype(np.int8))
+    assert np.array_equal(a.contract(None, 1).numpy(), out.numpy())
+    x = np.random.default_rng(11).standard_normal((16384, 5000))
+    gx = gpu.upload(x).transpose([1, 0])
+    outx = gpu.upload(np.zeros(5000))
+    gx.contract_noalloc(None, 1, outx)
+    np.testing.assert_allclose(outx.numpy(), x.sum(axis=0), rtol=1e-10, atol=1e-9)
+    # so many outputs that not even two chunks fit: one unsplit launch, no scratch
+    y = np.random.default_rng(12).standard_normal((600, 70000))
+    gy = gpu.upload(y).transpose([1, 0])
+    outy = gpu.upload(np.zeros(70000))
+    gy.contract_noalloc(None, 1, outy)
+    np.testing.assert_allclose(outy.numpy(), y.sum(axis=0), rtol=1e-10, atol=1e-9)
     # a result array of the wrong shape is an argument error
     with pytest.raises(capi.HgpuError) as e2:
         a.contract_noalloc(None, 1, gpu.upload(np.zeros(3, np.int8)))
