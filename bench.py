@@ -186,6 +186,24 @@ def roofline_of(rep, dtype_name):
     return roof, shares
 
 
+def kernel_table(rep, dtype_name, top=14):
+    """The launches of one gradient by label (one label = one kernel at one problem shape), largest share first:
+    launches, average microseconds, and the rate on the label's own algorithmic flops / bytes."""
+    rows = []
+    for name, (launches, ms, by, fl) in sorted(rep.items(), key=lambda kv: -kv[1][1])[:top]:
+        if launches <= 0 or ms <= 0:
+            continue
+        row = {"kernel": name, "launches": launches, "avg_us": ms / launches * 1e3}
+        if family(name) in MFMA_KERNELS:
+            row["tflops"] = fl / ms / 1e9
+            row["frac_of_mfma_peak"] = row["tflops"] / MFMA_PEAK_TFLOPS[dtype_name]
+        elif by > 0:
+            row["gbs"] = by / ms / 1e6
+            row["frac_of_hbm_peak"] = row["gbs"] / HBM_PEAK_GBS
+        rows.append(row)
+    return rows
+
+
 def cpu_baseline(pkg, key, mk):
     capi, H = pkg.capi, pkg.hostapi
     if not os.path.exists(entry.ORACLE_LIB):
@@ -279,6 +297,7 @@ def main():
                         "launches_per_step": sum(v[0] for v in rep.values()),
                         "device_ms_per_step": dev_ms, "algorithmic_gflop": wl.flops / 1e9,
                         "achieved_tflops": wl.flops / sec / 1e12, "roofline": roof, "kernel_ms": shares,
+                        "kernels": kernel_table(rep, dn),
                         "all_matrix_products": {"ms": gemm_ms, "tflops": gemm_fl / gemm_ms / 1e9 if gemm_ms > 0 else None,
                                                 "frac_of_peak": gemm_fl / gemm_ms / 1e9 / MFMA_PEAK_TFLOPS[dn] if gemm_ms > 0 else None}}
         if wl.bytes:

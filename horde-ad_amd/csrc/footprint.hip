@@ -84,6 +84,7 @@ struct Plan {
   int ypad;
   int addr_regs;   // per-lane address registers of the kernel
   int nbufs;   // LDS chunk buffers: 2, or 1 when two do not fit (the prefetch then waits in registers)
+  int ks = 1;  // wavefronts per SIMD: the block's 4 ks wavefronts split the K groups of a chunk ks ways
   bool cvec;   // groups of four rows are adjacent in C and 16-byte aligned: vector stores
 };
 
@@ -224,16 +225,19 @@ template <int N> struct VT { typedef T type __attribute__((ext_vector_type(N)));
 template <> struct VT<1> { typedef T type; };
 template <int N> using Vec = typename VT<N>::type;
 
+// KS wavefronts per SIMD: the block has 4 KS wavefronts, wavefront 4 h + w takes the row blocks of w
+// and the h-th part of the K groups (half h); the parts' products are added through LDS.
+constexpr int NT = 256 * KS;
 constexpr int MB = (MIN + 15) / 16, NBF = MB / 4, REM = MB % 4, NSLOT = (NG + 3) / 4;
 constexpr int NACC = NBF + REM > 0 ? NBF + REM : 1;
 // staging: vectors per operand and loads per thread
 constexpr int XV = (SPANX + VX - 1) / VX, YV = (SPANY + VY - 1) / VY;
-constexpr int NLX = (XV + 255) / 256, NLY = (YV + 255) / 256;
+constexpr int NLX = (XV + NT - 1) / NT, NLY = (YV + NT - 1) / NT;
 constexpr int LX = XV * VX, LY = YV * VY + (YPAD ? (YV * VY / YS) * YPAD : 0);   // LDS elements per buffer
 // where vector v of the Y footprint sits in LDS (in vectors)
 __device__ __forceinline__ int ypos(int v) { return YPAD ? v + (v * VY / YS) * (YPAD / VY) : v; }
 constexpr int NLD = MODE == 0 ? NLX + NLY : NLX;        // loads per thread and chunk
-constexpr int PH = NG >= 12 ? 3 : 1;                    // prefetch phases
+constexpr int PH = (NG + KS - 1) / KS >= 12 ? 3 : 1;    // prefetch phases
 constexpr int LPP = (NLD + PH - 1) / PH;
 constexpr int BUF = MODE == 0 ? LX + LY : LX;           // elements per chunk buffer
 // split row blocks: slots whose turn comes before K group g (slot s runs after group min(4 s + 3, NG - 1))
@@ -245,7 +249,11 @@ constexpr int rem_slots_before(int g) {
 constexpr int RGB = REM > 0 ? (4 / REM > 1 ? 4 / REM : 1) : 1;     // slots per batch of LDS reads
 struct RemOps { T a[RGB][REM > 0 ? REM : 1], b[RGB][REM > 0 ? REM : 1]; };
 constexpr int RED0 = NBUFS * BUF + (MODE == 0 ? 0 : LY);    // scratch for adding up split row blocks
-constexpr int LDS_ELEMS = RED0 + (REM > 0 ? REM * 4 * 256 : 0);
+constexpr int LDS_ELEMS = RED0 + (REM > 0 && KS == 1 ? REM * 4 * 256 : 0);
+// where the parts' partial products meet (KS > 1): a chunk buffer that has been multiplied; the whole
+// row blocks first, the split ones behind them
+constexpr int XCH = 4 * NBF * (KS - 1) * 256;
+static_assert(KS == 1 || XCH + REM * 4 * KS * 256 <= (MODE == 0 ? RED0 : BUF), "the exchange area must fit a chunk buffer");
 
 // The four registers of a lane are rows m0 .. m0 + 3 of column col.  Where
 // they go inside a chunk's output comes from two tables in memory; a kernel that
@@ -303,7 +311,7 @@ typedef Vec<VY> RawY;
 #define LOAD_Y(ch_, j_) reinterpret_cast<const Vec<VY>*>(Y + (ch_) * chy)[vidx(j_)]
 #define FIN_Y(j_, r_) (r_)
 #endif
-extern "C" __global__ void __launch_bounds__(256, 1)
+extern "C" __global__ void __launch_bounds__(NT, 1)
 KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 nch, i64 chx, i64 chy, i64 chc, i64 part_stride
 #if EPI
       , EpiArgs ea
@@ -329,8 +337,15 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   unsigned char* const stage = nullptr;
 #endif
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = wave_all & 3;
   const int r = lane & 15, q4 = lane >> 4;
+  // everything below is compiled once per part of K (KH): its K groups, hence the LDS offsets of its loop, are constants
+  auto run = [&](auto KHI) {
+  constexpr int KH = decltype(KHI)::v;
+  if constexpr (KH < KS) {
+  constexpr int GA = NG * KH / KS, GB = NG * (KH + 1) / KS;        // this part's K groups
+  constexpr bool kRemOwner = KH == KS - 1;                          // its wavefronts 0 .. REM - 1 finish the split row blocks
   // per-lane addresses: row base + lane offset of each K pattern
   int ax[NBF > 0 ? NBF : 1][NPAT];
 #pragma unroll
@@ -352,6 +367,8 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
     int ro = kRowX[m < MIN ? m : MIN - 1];
 #pragma clang loop unroll(full)
     for (int s = 0; s < NSLOT; ++s) {
+      const int trig = s == NSLOT - 1 ? NG - 1 : 4 * s + 3;     // the slot runs after this K group: in the part that holds it
+      if (trig < GA || trig >= GB) continue;
       int gi = 4 * s + ((wave + rb) & 3);
       if (gi >= NG) gi = NG - 1;
       int p = kGrpPd[gi];
@@ -365,24 +382,70 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   // where a lane's rows and windows go, and the program inputs that do not change with the row
   EPos epos[NACC];
 #pragma unroll
-  for (int t = 0; t < NBF; ++t) epos[t] = epi_pos((wave + 4 * t) * 16 + 4 * q4, r);
-  if (REM > 0) epos[NBF] = epi_pos((4 * NBF + (wave < REM ? wave : 0)) * 16 + 4 * q4, r);
+  for (int t = 0; t < NBF; ++t)
+    if (t % KS == KH) epos[t] = epi_pos((wave + 4 * t) * 16 + 4 * q4, r);     // row block t is finished by part t % KS
+  if (REM > 0 && kRemOwner) epos[NBF] = epi_pos((4 * NBF + (wave < REM ? wave : 0)) * 16 + 4 * q4, r);
   const Hoist hz = epi_hoist(ea, r < NIN ? r : NIN - 1);
 #else
   OutPos pos[MODE == 1 ? NACC : 1];
   if (MODE == 1) {
 #pragma unroll
-    for (int t = 0; t < NBF; ++t) pos[t] = out_pos((wave + 4 * t) * 16 + 4 * q4, r);
-    if (REM > 0) pos[NBF] = out_pos((4 * NBF + (wave < REM ? wave : 0)) * 16 + 4 * q4, r);
+    for (int t = 0; t < NBF; ++t)
+      if (t % KS == KH) pos[t] = out_pos((wave + 4 * t) * 16 + 4 * q4, r);
+    if (REM > 0 && kRemOwner) pos[NBF] = out_pos((4 * NBF + (wave < REM ? wave : 0)) * 16 + 4 * q4, r);
   }
 #endif
   Acc acc[NACC];
 #pragma unroll
   for (int t = 0; t < NACC; ++t) acc[t] = Acc{0, 0, 0, 0};
+  // The parts' partial products of whole row block t go to the part t % KS, which adds them to its own
+  // (xch: an area of LDS nobody reads any more); the partial products of the split row blocks, of all
+  // 4 KS wavefronts, are added by wavefronts 0 .. REM - 1 of the last part into srem.
+  T srem[4] = {T(0), T(0), T(0), T(0)};
+  auto meet = [&](T* xch) {
+    if (KS > 1) {
+#pragma unroll
+      for (int t = 0; t < NBF; ++t) {
+        if (t % KS != KH) {
+          const int slot = KH < t % KS ? KH : KH - 1;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) xch[(((wave * NBF + t) * (KS - 1) + slot) * 4 + j) * 64 + lane] = acc[t][j];
+        }
+      }
+    }
+    T* red = KS > 1 ? xch + XCH : lds + RED0;
+    if (REM > 0) {
+#pragma unroll
+      for (int rb = 0; rb < REM; ++rb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) red[((rb * 4 * KS + wave_all) * 4 + j) * 64 + lane] = acc[NBF + rb][j];
+    }
+    if ((KS > 1 && NBF > 0) || REM > 0) __syncthreads();
+    if (KS > 1) {
+#pragma unroll
+      for (int t = 0; t < NBF; ++t) {
+        if (t % KS == KH) {
+#pragma unroll
+          for (int sl = 0; sl < KS - 1; ++sl)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[t][j] += xch[(((wave * NBF + t) * (KS - 1) + sl) * 4 + j) * 64 + lane];
+        }
+      }
+    }
+    if (REM > 0 && kRemOwner && wave < REM) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        T sum = T(0);
+#pragma unroll
+        for (int w = 0; w < 4 * KS; ++w) sum += red[((wave * 4 * KS + w) * 4 + j) * 64 + lane];
+        srem[j] = sum;
+      }
+    }
+  };
 
   // j-th staging vector of this thread; the tail repeats the last vector.  The last vector of a footprint may reach up to
   // VX - 1 elements past it: still inside the operand's block, which the allocator ends with 16 spare bytes.
-  auto vidx = [&](int j) -> int { int v = tid + 256 * (j < NLX ? j : j - NLX); int lim = (j < NLX ? XV : YV) - 1; return v < lim ? v : lim; };
+  auto vidx = [&](int j) -> int { int v = tid + NT * (j < NLX ? j : j - NLX); int lim = (j < NLX ? XV : YV) - 1; return v < lim ? v : lim; };
   // The first chunk, and the columns operand of mode 1, go to LDS up to 32
   // vectors at a time: the loads in flight together, then the stores.  Copied
   // one by one, every vector would wait out its own trip to memory.
@@ -416,16 +479,16 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
     }
   }
   if (MODE == 1) {   // the columns operand does not change with the chunk
-    for (int v0 = tid; v0 < YV; v0 += 256 * kFill) {
+    for (int v0 = tid; v0 < YV; v0 += NT * kFill) {
       Vec<VY> fy[kFill];
 #pragma unroll
       for (int u = 0; u < kFill; ++u) {
-        const int v = v0 + 256 * u;
+        const int v = v0 + NT * u;
         fy[u] = reinterpret_cast<const Vec<VY>*>(Y)[v < YV ? v : YV - 1];
       }
 #pragma unroll
       for (int u = 0; u < kFill; ++u) {
-        const int v = v0 + 256 * u;
+        const int v = v0 + NT * u;
         if (v < YV) reinterpret_cast<Vec<VY>*>(lds + NBUFS * BUF)[ypos(v)] = fy[u];
       }
     }
@@ -453,7 +516,7 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
     }
     auto phase = [&](auto PHI) {
       constexpr int ph = decltype(PHI)::v;
-      constexpr int g0 = ph < PH ? NG * ph / PH : NG, g1 = ph < PH ? NG * (ph + 1) / PH : NG;
+      constexpr int g0 = ph < PH ? GA + (GB - GA) * ph / PH : GB, g1 = ph < PH ? GA + (GB - GA) * (ph + 1) / PH : GB;
 #pragma unroll
       for (int j = 0; j < LPP; ++j) {
         int jj = ph * LPP + j;
@@ -562,6 +625,11 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
     phase(IC<0>{});
     if constexpr (PH > 1) phase(IC<1>{});
     if constexpr (PH > 2) phase(IC<2>{});
+    // ---- the parts' products meet (KS > 1), the split row blocks are added up
+    if (MODE == 1) {
+      if (KS > 1) __syncthreads();     // everyone has multiplied this chunk: its buffer becomes the exchange area
+      meet(const_cast<T*>(L));
+    }
     if (NBUFS == 2) {
       cur ^= 1;
     } else {
@@ -583,35 +651,16 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
     if (MODE == 1) {
 #if EPI
 #pragma unroll
-      for (int t = 0; t < NBF; ++t) epi_tile(ea, hz, epos[t], stage, ch, (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      for (int t = 0; t < NBF; ++t)
+        if (t % KS == KH) epi_tile(ea, hz, epos[t], stage, ch, (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      if (REM > 0 && kRemOwner && wave < REM) epi_tile(ea, hz, epos[NBF], stage, ch, (4 * NBF + wave) * 16 + 4 * q4, r, srem[0], srem[1], srem[2], srem[3]);
 #else
       T* out = C + ch * chc;
 #pragma unroll
-      for (int t = 0; t < NBF; ++t) store_rows(out, pos[t], (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      for (int t = 0; t < NBF; ++t)
+        if (t % KS == KH) store_rows(out, pos[t], (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      if (REM > 0 && kRemOwner && wave < REM) store_rows(out, pos[MODE == 1 ? NBF : 0], (4 * NBF + wave) * 16 + 4 * q4, r, srem[0], srem[1], srem[2], srem[3]);
 #endif
-      if (REM > 0) {
-        T* red = lds + RED0;
-#pragma unroll
-        for (int rb = 0; rb < REM; ++rb)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) red[((rb * 4 + wave) * 4 + j) * 64 + lane] = acc[NBF + rb][j];
-        __syncthreads();
-        if (wave < REM) {
-          const int rb = wave;
-          T s[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            s[j] = T(0);
-#pragma unroll
-            for (int w = 0; w < 4; ++w) s[j] += red[((rb * 4 + w) * 4 + j) * 64 + lane];
-          }
-#if EPI
-          epi_tile(ea, hz, epos[NBF], stage, ch, (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
-#else
-          store_rows(out, pos[MODE == 1 ? NBF : 0], (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
-#endif
-        }
-      }
 #if EPI_STAGE
       __syncthreads();
       epi_flush(ea, stage, ch, tid);
@@ -620,31 +669,29 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   }
 #if !EPI
   if (MODE == 0) {
+    if (KS > 1 || REM > 0) __syncthreads();      // all multiplications are done: the chunk buffers are free
+    meet(lds);
     T* out = C + (i64)blockIdx.x * part_stride;
 #pragma unroll
-    for (int t = 0; t < NBF; ++t) store_rows(out, out_pos((wave + 4 * t) * 16 + 4 * q4, r), (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
-    if (REM > 0) {
-      T* red = lds + RED0;
-      __syncthreads();
-#pragma unroll
-      for (int rb = 0; rb < REM; ++rb)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) red[((rb * 4 + wave) * 4 + j) * 64 + lane] = acc[NBF + rb][j];
-      __syncthreads();
-      if (wave < REM) {
-        const int rb = wave;
-        T s[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          s[j] = T(0);
-#pragma unroll
-          for (int w = 0; w < 4; ++w) s[j] += red[((rb * 4 + w) * 4 + j) * 64 + lane];
-        }
-        store_rows(out, out_pos((4 * NBF + rb) * 16 + 4 * q4, r), (4 * NBF + rb) * 16 + 4 * q4, r, s[0], s[1], s[2], s[3]);
-      }
-    }
+    for (int t = 0; t < NBF; ++t)
+      if (t % KS == KH) store_rows(out, out_pos((wave + 4 * t) * 16 + 4 * q4, r), (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+    if (REM > 0 && kRemOwner && wave < REM) store_rows(out, out_pos((4 * NBF + wave) * 16 + 4 * q4, r), (4 * NBF + wave) * 16 + 4 * q4, r, srem[0], srem[1], srem[2], srem[3]);
   }
 #endif
+  }
+  };   // run
+  if constexpr (KS == 1) {
+    run(IC<0>{});
+  } else if constexpr (KS == 2) {
+    if (wave_all < 4) run(IC<0>{}); else run(IC<1>{});
+  } else {
+    switch (wave_all >> 2) {
+      case 0: run(IC<0>{}); break;
+      case 1: run(IC<1>{}); break;
+      case 2: run(IC<2>{}); break;
+      default: run(IC<3>{}); break;
+    }
+  }
 }
 )HG";
 
@@ -654,7 +701,7 @@ int lds_bytes(const Plan& pl) {
   if (pl.ypad) ly += (ly / pl.ys) * pl.ypad;
   int64_t buf = pl.mode == 0 ? lx + ly : lx;
   int MB = (pl.min_rows + 15) / 16, REM = MB % 4;
-  int64_t total = pl.nbufs * buf + (pl.mode == 0 ? 0 : ly) + (REM > 0 ? REM * 4 * 256 : 0);
+  int64_t total = pl.nbufs * buf + (pl.mode == 0 ? 0 : ly) + (REM > 0 && pl.ks == 1 ? REM * 4 * 256 : 0);
   total *= es;
   return total > INT32_MAX ? INT32_MAX : (int)total;
 }
@@ -667,7 +714,7 @@ std::string generate(const Plan& pl, const std::string& kname, const std::string
   s << "#define VIRT_Y " << (virt_y.empty() ? 0 : 1) << "\n#define YBASE " << ybase << "ll\n";
   s << "#define EPI " << (epilogue.empty() ? 0 : 1) << "\n#define EPI_STAGE " << stage_bytes << "\n";
   const int es = pl.f64 ? 8 : 4;
-  s << "#define F64 " << (pl.f64 ? 1 : 0) << "\n";
+  s << "#define F64 " << (pl.f64 ? 1 : 0) << "\n#define KS " << pl.ks << "\n";
   s << "#define MODE " << pl.mode << "\n";
   s << "#define MIN " << pl.min_rows << "\n#define NIN " << pl.nin << "\n#define NG " << pl.gx.size() << "\n";
   s << "#define NPAT " << pl.px.size() << "\n#define KVALID " << pl.kvalid << "\n";
@@ -963,14 +1010,33 @@ bool finish_plan(Plan& pl, const char* xp, const char* yp, const char* cp, int64
     }
     return n > 0 ? n : (int64_t)1;
   };
-  int64_t loads = (pl.span_x / pl.vx + 255) / 256 * per_slot(virt_x) + (pl.mode == 0 ? (pl.span_y / pl.vy + 255) / 256 * per_slot(virt_y) : 0);
-  if (loads > 48) return false;
-  pl.nbufs = 2;
-  if (lds_bytes(pl) + extra_lds_bytes > kLdsBudget) {
-    pl.nbufs = 1;
-    if (lds_bytes(pl) + extra_lds_bytes > kLdsBudget || loads * 4 + pl.addr_regs > 330) return false;   // the prefetch must fit the register file
+  // Two wavefronts per SIMD, each multiplying half of a chunk's K groups, keep the matrix cores busier
+  // than one (a wavefront's LDS reads and waits hide behind the other's multiplications).  That needs K
+  // groups to share out and room for the halves' partial products in a chunk buffer.
+  static const int ks_env = getenv("HORDEAD_FOOTPRINT_KS") ? atoi(getenv("HORDEAD_FOOTPRINT_KS")) : 0;
+  const int MB = (pl.min_rows + 15) / 16, NBF = MB / 4, REM = MB % 4, NG = (int)pl.gx.size();
+  auto staged_loads = [&](int nt) {
+    return (pl.span_x / pl.vx + nt - 1) / nt * per_slot(virt_x) + (pl.mode == 0 ? (pl.span_y / pl.vy + nt - 1) / nt * per_slot(virt_y) : 0);
+  };
+  for (int ks : {ks_env == 1 ? 1 : 2, 1}) {
+    if (ks == 2 && NG < 16) continue;
+    pl.ks = ks;
+    const int64_t loads = staged_loads(256 * ks);
+    if (loads > 48) continue;
+    const int64_t lx = (pl.span_x + pl.vx - 1) / pl.vx * pl.vx;
+    int64_t ly = (pl.span_y + pl.vy - 1) / pl.vy * pl.vy;
+    if (pl.ypad) ly += (ly / pl.ys) * pl.ypad;
+    const int64_t exchange = (int64_t)4 * NBF * (ks - 1) * 256 + (int64_t)REM * 4 * ks * 256;
+    pl.nbufs = 2;
+    if (lds_bytes(pl) + extra_lds_bytes > kLdsBudget) {
+      pl.nbufs = 1;
+      // the prefetch must fit the register file (half of it with two wavefronts per SIMD)
+      if (lds_bytes(pl) + extra_lds_bytes > kLdsBudget || loads * 4 + pl.addr_regs > (ks == 1 ? 330 : 170)) continue;
+    }
+    if (ks > 1 && exchange > (pl.mode == 0 ? pl.nbufs * (lx + ly) : lx)) continue;
+    return true;
   }
-  return true;
+  return false;
 }
 
 }  // namespace
@@ -1041,8 +1107,8 @@ int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const v
   char kname[128];
   const VirtualOp* vx = best_swapped ? vb : va;
   const VirtualOp* vy = best_swapped ? va : vb;
-  snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_%s%s%s%s", f64 ? "f64" : "f32", (long long)p.M, (long long)p.N, (long long)p.K,
-           pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? "_swapped" : "", vx ? "_xmap" : "", vy ? "_ymap" : "");
+  snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_%s%s%s%s%s", f64 ? "f64" : "f32", (long long)p.M, (long long)p.N, (long long)p.K,
+           pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? "_swapped" : "", vx ? "_xmap" : "", vy ? "_ymap" : "", pl.ks == 2 ? "_w8" : "");
   const int64_t xbase = (int64_t)((uintptr_t)((const char*)(best_swapped ? pb : pa) + pl.shift_x * es) / (uintptr_t)es);
   const int64_t ybase = (int64_t)((uintptr_t)((const char*)(best_swapped ? pa : pb) + pl.shift_y * es) / (uintptr_t)es);
   // the last staging vector of the last chunk may reach past its footprint: how far at most
@@ -1086,14 +1152,14 @@ int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const v
     const char* label = f64 ? "gemm_f64" : "gemm_f32";
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[160];
-      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB1,footprint,%s%s,chunks%lld,rows%d,kgroups%d,lds%dK%s%s]", label, (long long)p.M, (long long)p.N,
+      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB1,footprint,%s%s,chunks%lld,rows%d,kgroups%d,lds%dK,waves%d%s%s]", label, (long long)p.M, (long long)p.N,
                (long long)p.K, pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? ",swapped" : "", (long long)pl.nch, pl.min_rows, (int)pl.gx.size(), lds_bytes(pl) / 1024,
-               vx ? ",xmap" : "", vy ? ",ymap" : "");
+               4 * pl.ks, vx ? ",xmap" : "", vy ? ",ymap" : "");
       label = intern_label(ctx, buf);
     }
     {
       LaunchGuard lg(ctx, label, bytes, flops);
-      hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
+      hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256u * (unsigned)pl.ks, 1, 1, 0, ctx->stream, args.data(), nullptr);
       if (e != hipSuccess) { if (part) buffer_release(part); return check_hip(ctx, e, "footprint gemm launch"); }
     }
     if (pl.mode == 0) {
@@ -1228,7 +1294,7 @@ std::string epilogue_source(const Plan& pl, const EpiSpec& e) {
       const int64_t nv = elems * (int64_t)es / 16;
       s << "  {\n    V16* dst = reinterpret_cast<V16*>(" << ptr << " + ch * " << chs << "ll);\n";
       s << "    const V16* src = reinterpret_cast<const V16*>(stage + " << off << ");\n";
-      s << "#pragma unroll 4\n    for (int v = tid; v < " << nv << "; v += 256) dst[v] = src[v];\n  }\n";
+      s << "#pragma unroll 4\n    for (int v = tid; v < " << nv << "; v += NT) dst[v] = src[v];\n  }\n";
       (void)ct;
     };
     const int64_t n_el = (int64_t)pl.min_rows * pl.nin;
@@ -1494,8 +1560,8 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
   }
 
   char kname[160];
-  snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_chunkM%s_map%d%s", f64 ? "f64" : "f32", (long long)(swapped ? Nb : Ma), (long long)(swapped ? Ma : Nb),
-           (long long)K, swapped ? "_swapped" : "", n_instr, has_ext ? (want_max ? "_max" : "_min") : "");
+  snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_chunkM%s_map%d%s%s", f64 ? "f64" : "f32", (long long)(swapped ? Nb : Ma), (long long)(swapped ? Ma : Nb),
+           (long long)K, swapped ? "_swapped" : "", n_instr, has_ext ? (want_max ? "_max" : "_min") : "", pl.ks == 2 ? "_w8" : "");
   std::string src = generate(pl, kname, epilogue_source(pl, e), e.staged ? e.stage_bytes : 0);
   auto& cache = cache_of(ctx);
   auto it = cache.find(src);
@@ -1528,13 +1594,13 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
     const char* label = f64 ? "gemm_f64" : "gemm_f32";
     if (ctx->profiling && ctx->profile_shapes) {
       char buf[200];
-      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB1,footprint,chunkM%s,chunks%lld,rows%d,kgroups%d,lds%dK,map(instr%d,out%d%s)]", label, (long long)M, (long long)N,
-               (long long)K, swapped ? ",swapped" : "", (long long)pl.nch, pl.min_rows, (int)pl.gx.size(), lds_bytes(pl) / 1024, n_instr, n_out,
+      snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%lldxB1,footprint,chunkM%s,chunks%lld,rows%d,kgroups%d,lds%dK,waves%d,map(instr%d,out%d%s)]", label, (long long)M, (long long)N,
+               (long long)K, swapped ? ",swapped" : "", (long long)pl.nch, pl.min_rows, (int)pl.gx.size(), lds_bytes(pl) / 1024, 4 * pl.ks, n_instr, n_out,
                has_ext ? (L == 4 ? ",ext4" : (L == 2 ? ",ext2" : ",ext1")) : "");
       label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, bytes, flops);
-    hipError_t err = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+    hipError_t err = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256u * (unsigned)pl.ks, 1, 1, 0, ctx->stream, args, nullptr);
     if (err != hipSuccess) { release_all(); return check_hip(ctx, err, "contract_map launch"); }
   }
   for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];

@@ -188,6 +188,54 @@ __device__ __forceinline__ int64_t data_offset(const IxSpace& sp, int64_t m) {
 // one first segment of a long run (place 1) and one later segment (place 0),
 // because segments of one run start kSeg entries apart and a long run is
 // longer than a bucket -- and long_head[bucket] remembers where the run starts.
+// Is sorted entry `at` (key k, not the first entry of its run) the start of a later segment of a long run?
+template <typename K>
+__device__ __forceinline__ bool later_segment_start(const K* __restrict__ key, int64_t at, K k) {
+  if (at < kSeg || key[at - kSeg] != k) return false;   // fewer than kSeg entries of this run before this one
+  int64_t lo = 0, hi = at - kSeg;                       // the run's first entry: the first key that is not smaller
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (key[mid] < k) lo = mid + 1; else hi = mid;
+  }
+  return (at - lo) % kSeg == 0;
+}
+
+// Adds entries j .. end - 1 of the run with key k to acc, front to back; stops at the first other key.
+// Keys, positions and values of four entries are in flight together.  Returns the first entry not added.
+template <typename T, typename K>
+__device__ __forceinline__ int64_t add_run(const IxSpace& sp, const K* __restrict__ key, const uint32_t* __restrict__ val, const T* __restrict__ src, int64_t io,
+                                           K k, int64_t j, int64_t end, int64_t M, T* acc) {
+  while (j < end) {
+    const int64_t j1 = j + 1 < M ? j + 1 : M - 1, j2 = j + 2 < M ? j + 2 : M - 1, j3 = j + 3 < M ? j + 3 : M - 1;
+    const K k0 = key[j], k1 = key[j1], k2 = key[j2], k3 = key[j3];
+    const uint32_t p0 = val[j], p1 = val[j1], p2 = val[j2], p3 = val[j3];
+    if (k0 != k) return j;
+    const bool m1 = j + 1 < end && k1 == k, m2 = m1 && j + 2 < end && k2 == k, m3 = m2 && j + 3 < end && k3 == k;
+    const T v0 = src[data_offset(sp, (int64_t)p0) + io];
+    const T v1 = src[data_offset(sp, (int64_t)(m1 ? p1 : p0)) + io];
+    const T v2 = src[data_offset(sp, (int64_t)(m2 ? p2 : p0)) + io];
+    const T v3 = src[data_offset(sp, (int64_t)(m3 ? p3 : p0)) + io];
+    *acc = (T)(*acc + v0);
+    if (!m1) return j + 1;
+    *acc = (T)(*acc + v1);
+    if (!m2) return j + 2;
+    *acc = (T)(*acc + v2);
+    if (!m3) return j + 3;
+    *acc = (T)(*acc + v3);
+    j += 4;
+  }
+  return j;
+}
+
+// key / val sorted by key, equal keys in ascending position order.  One lane per
+// (sorted entry, inner element); a lane works when its entry starts a SEGMENT:
+// the first entry of a run, or an entry a multiple of kSeg entries after it.
+// It adds the segment's slices front to back, starting from zero.  A run of one
+// segment is written to `out` at once.  The segment sums of a longer run go to
+// `part`, two places per bucket of kSeg sorted entries -- a bucket holds at most
+// one first segment of a long run (place 1) and one later segment (place 0),
+// because segments of one run start kSeg entries apart and a long run is
+// longer than a bucket -- and long_head[bucket] remembers where the run starts.
 template <typename T, typename K>
 __global__ void __launch_bounds__(kBlock) k_scatter_runs(IxSpace sp, Dims inner, int64_t M, int64_t N, K skip, const K* __restrict__ key,
                                                          const uint32_t* __restrict__ val, const T* __restrict__ src, T* __restrict__ out,
@@ -195,36 +243,17 @@ __global__ void __launch_bounds__(kBlock) k_scatter_runs(IxSpace sp, Dims inner,
   int64_t total = M * N;
   int64_t step = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += step) {
-    int64_t at = N == 1 ? i : i / N;
-    int64_t n = N == 1 ? 0 : i - at * N;
+    int64_t at = i / N;
+    int64_t n = i - at * N;
     const K k = key[at];
     if (k == skip) continue;
     const bool head = at == 0 || key[at - 1] != k;
-    if (!head) {
-      if (at < kSeg || key[at - kSeg] != k) continue;   // fewer than kSeg entries of this run before this one
-      int64_t lo = 0, hi = at - kSeg;                   // the run's first entry: the first key that is not smaller
-      while (lo < hi) {
-        const int64_t mid = (lo + hi) >> 1;
-        if (key[mid] < k) lo = mid + 1; else hi = mid;
-      }
-      if ((at - lo) % kSeg != 0) continue;
-    }
+    if (!head && !later_segment_start(key, at, k)) continue;
     int64_t io[1];
     decompose<1>(inner, n, io);
     const int64_t end = at + kSeg < M ? at + kSeg : M;
     T acc = T(0);
-    int64_t j = at;
-    for (; j + 4 <= end; j += 4) {                      // four loads in flight, added in order
-      const K k1 = key[j + 1], k2 = key[j + 2], k3 = key[j + 3];
-      if (k1 != k || k2 != k || k3 != k) break;
-      const T v0 = src[data_offset(sp, (int64_t)val[j]) + io[0]], v1 = src[data_offset(sp, (int64_t)val[j + 1]) + io[0]];
-      const T v2 = src[data_offset(sp, (int64_t)val[j + 2]) + io[0]], v3 = src[data_offset(sp, (int64_t)val[j + 3]) + io[0]];
-      acc = (T)(acc + v0);
-      acc = (T)(acc + v1);
-      acc = (T)(acc + v2);
-      acc = (T)(acc + v3);
-    }
-    for (; j < end && key[j] == k; ++j) acc = (T)(acc + src[data_offset(sp, (int64_t)val[j]) + io[0]]);
+    const int64_t j = add_run(sp, key, val, src, io[0], k, at, end, M, &acc);
     const bool more = j < M && key[j] == k;
     if (head && !more) {
       out[(int64_t)k + n] = acc;
@@ -232,6 +261,54 @@ __global__ void __launch_bounds__(kBlock) k_scatter_runs(IxSpace sp, Dims inner,
       const int64_t q = at / kSeg;
       part[(q * 2 + (head ? 1 : 0)) * N + n] = acc;
       if (head && n == 0) long_head[q] = (uint32_t)(at - q * kSeg) + 1;
+    }
+  }
+}
+
+// The same for single elements (N = 1), a wavefront per 64 sorted entries: EVERY
+// lane fetches its entry's value (coalesced keys and positions, one gather), and
+// the lane at a segment's start then collects the values of the lanes behind it
+// through the wavefront, nearest first -- the same order, without a chain of
+// dependent loads.  What lies beyond the wavefront's 64 entries it adds itself.
+template <typename T, typename K>
+__global__ void __launch_bounds__(kBlock) k_scatter_runs1(IxSpace sp, int64_t M, K skip, const K* __restrict__ key, const uint32_t* __restrict__ val,
+                                                          const T* __restrict__ src, T* __restrict__ out, T* __restrict__ part, uint32_t* __restrict__ long_head) {
+  const int lane = threadIdx.x & 63;
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t base = (int64_t)blockIdx.x * kBlock + (threadIdx.x & ~63); base < M; base += step) {   // the same trips for all lanes of a wavefront
+    const int64_t at = base + lane;
+    const bool valid = at < M;
+    const K k = valid ? key[at] : skip;
+    const bool live = valid && k != skip;
+    const T v = live ? src[data_offset(sp, (int64_t)val[at])] : T(0);
+    K before = (K)__shfl_up((unsigned long long)k, 1);
+    if (lane == 0) before = at > 0 && valid ? key[at - 1] : (K)~k;
+    const bool head = live && (at == 0 || before != k);
+    const bool start = head || (live && later_segment_start(key, at, k));
+    T acc = (T)(T(0) + v);
+    bool open = start;                      // still inside the run
+    int reach = 1;                          // entries of the segment this lane has added
+    for (int d = 1; d < 64; ++d) {
+      const K kd = (K)__shfl_down((unsigned long long)k, d);
+      const T vd = __shfl_down(v, d);
+      const bool take = open && lane + d < 64 && kd == k;      // (a segment is longer than a wavefront's share, so its end is not met here)
+      if (open && lane + d < 64 && !take) open = false;
+      if (take) { acc = (T)(acc + vd); reach = d + 1; }
+      if (!__any(take)) break;
+    }
+    if (!start) continue;
+    int64_t j = at + reach;
+    if (open && lane + reach >= 64) {       // the run goes on behind the wavefront's entries
+      const int64_t end = at + kSeg < M ? at + kSeg : M;
+      j = add_run(sp, key, val, src, (int64_t)0, k, j, end, M, &acc);
+    }
+    const bool more = j < M && key[j] == k && j - at >= kSeg;
+    if (head && !more) {
+      out[(int64_t)k] = acc;
+    } else {
+      const int64_t q = at / kSeg;
+      part[q * 2 + (head ? 1 : 0)] = acc;
+      if (head) long_head[q] = (uint32_t)(at - q * kSeg) + 1;
     }
   }
 }
@@ -286,8 +363,13 @@ hipError_t scatter_sorted(hgpu_ctx* ctx, const IxSpace& sp, const Dims& inner, i
     e = rocprim::radix_sort_pairs(tb->ptr, temp_bytes, key_in, key_out, val_in, val_out, (size_t)M, 0, (unsigned)end_bit, ctx->stream);
     if (e == hipSuccess) {
       unsigned g = grid_for(M * N, kBlock, ctx->num_cu * 8);
-      HG_DISPATCH_DTYPE(src->dtype, T, hipLaunchKernelGGL((k_scatter_runs<T, K>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, skip, (const K*)key_out, (const uint32_t*)val_out,
-                                                          (const T*)data_ptr(src), (T*)data_ptr(o), (T*)pb->ptr, long_head));
+      if (N == 1) {
+        HG_DISPATCH_DTYPE(src->dtype, T, hipLaunchKernelGGL((k_scatter_runs1<T, K>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, M, skip, (const K*)key_out, (const uint32_t*)val_out,
+                                                            (const T*)data_ptr(src), (T*)data_ptr(o), (T*)pb->ptr, long_head));
+      } else {
+        HG_DISPATCH_DTYPE(src->dtype, T, hipLaunchKernelGGL((k_scatter_runs<T, K>), dim3(g), dim3(kBlock), 0, ctx->stream, sp, inner, M, N, skip, (const K*)key_out, (const uint32_t*)val_out,
+                                                            (const T*)data_ptr(src), (T*)data_ptr(o), (T*)pb->ptr, long_head));
+      }
       e = hipGetLastError();
     }
     if (e == hipSuccess) {

@@ -442,6 +442,20 @@ def test_scatter(both, dt):
     assert_same(first, tol)
     again = both.scatter_add(src, ix, 1, [7])
     assert np.array_equal(first.numpy()[0], again.numpy()[0])
+    # single elements: runs of a few entries, runs that cross a wavefront's 64 sorted entries, runs just
+    # below and above the segment length, all still in the reference's order where they fit one segment
+    for m, cells in ((5000, 2000), (5000, 40), (7000, 30), (1000, 1), (300, 1), (64, 1), (65, 2)):
+        src = both.upload(rnd((m,), dt))
+        ix = [both.upload(RNG.integers(-1, cells + 1, m).astype(np.int64))]
+        longest = np.bincount(ix[0].numpy()[0] + 1).max()
+        res = both.scatter_add(src, ix, 1, [cells])
+        if longest <= 256 or tol == 0.0:
+            assert_same(res, 0.0, (m, cells))
+        else:   # a reordered sum: held against the sum of the magnitudes that went into a cell, not against what cancellation left of them
+            g, o = res.numpy()
+            mass = np.zeros(cells + 2)
+            np.add.at(mass, ix[0].numpy()[0] + 1, np.abs(src.numpy()[0]).astype(np.float64))
+            assert np.all(np.abs(g.astype(np.float64) - o) <= tol * mass[1:cells + 1]), (m, cells)
     # many destinations with a few positions each, some out of bounds, slices of 5
     src = both.upload(rnd((3000, 5), dt))
     ix = [both.upload(RNG.integers(-2, 700, 3000).astype(np.int64))]
@@ -538,9 +552,9 @@ def test_scatter_into_a_handful_of_cells_is_bounded(both, gpu):
         res = both.scatter_add(src, ix, 1, [8])
         assert_same(res, tol, (dt, n))
         got = res.numpy()[0]
-        want = np.zeros_like(got)
-        np.add.at(want, cells[(cells >= 0) & (cells < 8)], src.numpy()[1][(cells >= 0) & (cells < 8)])
-        np.testing.assert_allclose(got, want, rtol=max(tol, 1e-12) * 100, atol=1e-3 if dt == np.float32 else 1e-7)
+        want = np.zeros(got.shape, np.float64)      # the independent sum in double, whatever the element type
+        np.add.at(want, cells[(cells >= 0) & (cells < 8)], src.numpy()[1][(cells >= 0) & (cells < 8)].astype(np.float64))
+        np.testing.assert_allclose(got, want, rtol=max(tol, 1e-12) * 100, atol=0.5 if dt == np.float32 else 1e-7)   # 125,000 terms of size one per cell
         dev = src.arrays[0]
         gix = [ix[0].arrays[0]]
         gpu.sync()
