@@ -35,6 +35,13 @@ struct hgpu_buffer {
   size_t bytes;      // size of the block handed out by the allocator
   std::atomic<int> refs;
   hgpu_cap_pool* pool = nullptr;
+  // What the library knows about the block's contents without reading them (arrays are written
+  // once): element i is the I64 value i (hgpu_iota), or the block holds a single element of all
+  // zero bits.  A kernel chosen because of that knowledge marks the block, and the two entry points
+  // that write into existing arrays (hgpu_overwrite, hgpu_assign) refuse a marked block.
+  enum { kUnknown = 0, kIotaI64 = 1, kZeroScalar = 2 };
+  int known = kUnknown;
+  bool known_relied_on = false;
 };
 
 struct hgpu_array {
@@ -53,6 +60,7 @@ struct DeferredQueue;                         // launches held back to be groupe
 void flush_deferred_locked(hgpu_ctx* ctx);    // the caller holds launch_mu
 void flush_deferred(hgpu_ctx* ctx);
 void drop_deferred(hgpu_ctx* ctx);            // flush, then free the queue
+void forget_remembered_sums(hgpu_ctx* ctx);   // results kept for a later call, and the arrays held for them (footprint.hip)
 }  // namespace hg
 
 struct hgpu_ctx {
@@ -66,6 +74,7 @@ struct hgpu_ctx {
   void* staging = nullptr;       // pinned host staging block
   size_t staging_bytes = 0;
   std::mutex launch_mu;          // serialises enqueue order across host threads
+  uint64_t write_epoch = 0;      // counts the writes into existing arrays (hgpu_overwrite, hgpu_assign): results remembered for given inputs end with it
   int num_cu = 256;
   // JIT cache of fused elementwise kernels, keyed by generated source.
   std::map<std::string, void*> jit_cache;

@@ -659,6 +659,7 @@ int hgpu_iota(hgpu_ctx* ctx, int64_t n, int dtype, hgpu_array** out) {
     HG_DISPATCH_DTYPE(dtype, T, hipLaunchKernelGGL(k_iota<T>, dim3(g), dim3(kBlock), 0, ctx->stream, n, (T*)data_ptr(o)));
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "iota"); }
+    if (dtype == HGPU_I64 && o->buf && o->offset == 0) o->buf->known = hgpu_buffer::kIotaI64;
   }
   *out = o;
   return HGPU_OK;

@@ -1785,6 +1785,103 @@ int write_out(hgpu_ctx* ctx, const hgpu_operand* o, hgpu_array** out) {
   return rc;
 }
 
+// ---- sums that another kernel has made on its way ---------------------------
+// The sum of an expression over all merged dims but a few (a bias's cotangent:
+// the layer's cotangent summed over batch, height and width) costs nothing in
+// a kernel that evaluates the expression anyway (onehot_contract).  Such a sum
+// is remembered under the expression -- program, inputs (held, so that their
+// blocks stay theirs), merged shape, the dims kept -- for the caller that asks
+// for exactly it next.  Arrays are written once; the two entry points that
+// write into existing arrays end everything remembered (hgpu_ctx::write_epoch).
+struct MemoSum {
+  std::string key;
+  hgpu_array* sum;
+  std::vector<hgpu_buffer*> held;
+  uint64_t epoch;
+};
+struct MemoSums { std::vector<MemoSum> items; };
+
+MemoSums& memo_of(hgpu_ctx* ctx) {
+  auto it = ctx->jit_cache.find("__memo_sums__");
+  if (it == ctx->jit_cache.end()) it = ctx->jit_cache.emplace("__memo_sums__", new MemoSums()).first;
+  return *static_cast<MemoSums*>(it->second);
+}
+
+std::string expression_key(const VirtualOp& v, const std::vector<int>& kept) {
+  std::string k;
+  auto put = [&](const void* p, size_t n) { k.append((const char*)p, n); };
+  put(&v.n_in, sizeof v.n_in);
+  put(&v.n_instr, sizeof v.n_instr);
+  put(&v.slot, sizeof v.slot);
+  if (v.n_instr > 0) put(v.prog, sizeof(hgpu_fused_instr) * (size_t)v.n_instr);
+  for (int i = 0; i < v.n_in; ++i) {
+    const hgpu_array* a = v.in[i];
+    put(&a->buf, sizeof a->buf);
+    put(&a->dtype, sizeof a->dtype);
+    put(&a->rank, sizeof a->rank);
+    put(a->shape, sizeof(int64_t) * (size_t)a->rank);
+    put(a->strides, sizeof(int64_t) * (size_t)a->rank);
+    put(&a->offset, sizeof a->offset);
+  }
+  for (int64_t m : v.M) put(&m, sizeof m);
+  k += "|";
+  for (int d : kept) put(&d, sizeof d);
+  return k;
+}
+
+void forget(MemoSum& m) {
+  hgpu_release(m.sum);
+  for (auto* b : m.held) buffer_release(b);
+}
+
+// Takes over the caller's reference to `sum`.
+void remember_sum(hgpu_ctx* ctx, const VirtualOp& v, const std::vector<int>& kept, hgpu_array* sum) {
+  MemoSum m{expression_key(v, kept), sum, {}, 0};
+  for (int i = 0; i < v.n_in; ++i)
+    if (v.in[i]->buf) { buffer_retain(v.in[i]->buf); m.held.push_back(v.in[i]->buf); }
+  std::lock_guard<std::mutex> lk(ctx->launch_mu);
+  m.epoch = ctx->write_epoch;
+  MemoSums& ms = memo_of(ctx);
+  for (size_t i = 0; i < ms.items.size();)
+    if (ms.items[i].key == m.key || ms.items[i].epoch != m.epoch) { forget(ms.items[i]); ms.items.erase(ms.items.begin() + (long)i); } else ++i;
+  if (ms.items.size() >= 2) { forget(ms.items.front()); ms.items.erase(ms.items.begin()); }
+  ms.items.push_back(std::move(m));
+}
+
+// The remembered sum (a new reference), or nullptr.
+hgpu_array* recall_sum(hgpu_ctx* ctx, const VirtualOp& v, const std::vector<int>& kept) {
+  const std::string key = expression_key(v, kept);
+  std::lock_guard<std::mutex> lk(ctx->launch_mu);
+  MemoSums& ms = memo_of(ctx);
+  for (auto& m : ms.items)
+    if (m.epoch == ctx->write_epoch && m.key == key) { hgpu_retain(m.sum); return m.sum; }
+  return nullptr;
+}
+
+// The merged dims that the first n_keep dims of an operand's view walk whole, in order, when the view as
+// a whole walks every merged dim exactly once (no zero-extension, no offset): the sum over the other
+// dims of the view is then the sum over all other merged dims.  false: the view is something else.
+bool kept_merged_dims(const VirtualOp& v, const hgpu_operand* o, int n_keep, std::vector<int>* kept) {
+  if (v.padded || o->offset != 0) return false;
+  const size_t rm = v.M.size();
+  std::vector<int64_t> DM(rm, 1);
+  for (size_t k = rm; k-- > 1;) DM[k - 1] = DM[k] * v.M[k];
+  std::vector<char> covered(rm, 0);
+  kept->clear();
+  for (int d = 0; d < o->rank; ++d) {
+    if (o->shape[d] == 1) continue;
+    int found = -1;
+    for (size_t k = 0; k < rm; ++k)
+      if (v.M[k] > 1 && !covered[k] && DM[k] == o->strides[d] && v.M[k] == o->shape[d]) { found = (int)k; break; }
+    if (found < 0) return false;
+    covered[(size_t)found] = 1;
+    if (d < n_keep) kept->push_back(found);
+  }
+  for (size_t k = 0; k < rm; ++k)
+    if (v.M[k] > 1 && !covered[k]) return false;
+  return true;
+}
+
 // out[o] = sum over the dims behind the first n_keep of the view of an
 // expression: blocks take (output, chunk of the summed index range), lanes
 // evaluate the expression at their elements, partial sums are added up in a
@@ -1903,10 +2000,407 @@ int try_mapped_sum(hgpu_ctx* ctx, const VirtualOp& v, const hgpu_operand* o, int
   return HGPU_OK;
 }
 
+
+// ---------------------------------------------------------------------------
+// A contraction with an expression operand that is ONE-HOT along some of the
+// contracted dims: the expression is `select (which == where) u 0` (times other
+// factors) with `which` counting through those dims -- what the adjoint of
+// "gather at kargMax" (max-pooling, External/CommonShapedOps.hs:241-260) puts
+// into the cotangent of a convolution: one non-zero per pooling window, at the
+// window's argument.  Summing over the one-hot dims then takes ONE term per
+// position of the other dims: the expression is evaluated there only, its
+// values meet the other operand's rows (a few tens, read from LDS) in the
+// vector units, and the dense cotangent -- three quarters structural zeros
+// for 2 x 2 windows -- is neither written nor read.
+//
+// The structure is proved from the program and from what the library knows of
+// its input blocks without reading them (hgpu_buffer::known): `which` is a
+// view of an index vector, the else-branch a zero constant.
+
+// An instruction slot that can be non-zero only where input `which_in` (a view of an index vector)
+// equals input `where_in`.
+bool onehot_gate(const VirtualOp& v, int slot, int* which_in, int* where_in) {
+  if (slot < v.n_in) return false;
+  const hgpu_fused_instr& q = v.prog[slot - v.n_in];
+  auto zero_const = [&](int s0) {
+    if (s0 >= v.n_in) return false;
+    const hgpu_array* a = v.in[s0];
+    if (!a->buf || a->buf->known != hgpu_buffer::kZeroScalar) return false;
+    for (int d = 0; d < a->rank; ++d)
+      if (a->shape[d] != 1 && a->strides[d] != 0) return false;
+    return true;
+  };
+  auto index_vector = [&](int s0) {
+    return s0 < v.n_in && v.in[s0]->dtype == HGPU_I64 && v.in[s0]->buf && v.in[s0]->buf->known == hgpu_buffer::kIotaI64;
+  };
+  switch (q.kind) {
+    case HGPU_FUSED_OP2:
+      if (q.op == HGPU_MUL) return onehot_gate(v, q.a, which_in, where_in) || onehot_gate(v, q.b, which_in, where_in);
+      return false;
+    case HGPU_FUSED_OP1:
+      return q.op == HGPU_NEG && onehot_gate(v, q.a, which_in, where_in);
+    case HGPU_FUSED_SELECT: {
+      if (zero_const(q.b)) return onehot_gate(v, q.c, which_in, where_in);      // select c 0 u
+      if (!zero_const(q.c)) return false;
+      if (q.a >= v.n_in) {                                                       // select (x == y) u 0
+        const hgpu_fused_instr& c = v.prog[q.a - v.n_in];
+        if (c.kind == HGPU_FUSED_CMP && c.op == HGPU_EQ) {
+          for (int sw = 0; sw < 2; ++sw) {
+            const int x = sw ? c.b : c.a, y = sw ? c.a : c.b;
+            if (index_vector(x) && y < v.n_in && v.in[y]->dtype == HGPU_I64 && !index_vector(y)) { *which_in = x; *where_in = y; return true; }
+          }
+        }
+      }
+      return onehot_gate(v, q.b, which_in, where_in);
+    }
+    default:
+      return false;
+  }
+}
+
+// x: the operand that is an array; y: the expression operand.  Both seen through views of `rank` dims of one shape.
+int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, const hgpu_operand* yo, int n_keep, hgpu_array* out, bool* handled) {
+  *handled = false;
+  static const bool disabled = getenv("HORDEAD_NO_ONEHOT") != nullptr;
+  if (disabled) return HGPU_OK;
+  if (v.dtype != HGPU_F64 && v.dtype != HGPU_F32) return HGPU_OK;
+  if (v.padded || yo->offset != 0 || v.total >= (1LL << 31)) return HGPU_OK;
+  int which_in = -1, where_in = -1;
+  if (!onehot_gate(v, v.slot, &which_in, &where_in)) return HGPU_OK;
+  const int rank = yo->rank;
+  const size_t re = v.E.size(), rm = v.M.size();
+  // ---- the one-hot dims of the inputs' shape: where `which` moves; `where` must stand still there
+  const hgpu_array* wh = v.in[which_in];
+  const hgpu_array* wr = v.in[where_in];
+  std::vector<char> oh(re, 0);
+  std::vector<std::pair<int64_t, size_t>> digits;      // (stride of which, dim)
+  for (size_t j = 0; j < re; ++j) {
+    if (v.E[j] == 1 || wh->strides[j] == 0) continue;
+    if (wh->strides[j] < 0 || wr->strides[j] != 0) return HGPU_OK;
+    oh[j] = 1;
+    digits.push_back({wh->strides[j], j});
+  }
+  if (digits.empty()) return HGPU_OK;
+  std::sort(digits.begin(), digits.end());
+  int64_t EH = 1;                                        // values `which` takes: which.offset + 0 .. EH - 1, as a mixed-radix number of the one-hot dims
+  for (auto& d : digits) {
+    if (d.first != EH) return HGPU_OK;
+    EH *= v.E[d.second];
+  }
+  if (EH < 2 || EH > 64) return HGPU_OK;
+  // ---- the inputs' dims as parts of the merged dims; one-hot dims must be the innermost parts of theirs
+  std::vector<int> group_of(re, -1);
+  std::vector<int64_t> inner_oh(rm, 1);                  // product of the one-hot parts of merged dim k
+  std::vector<int64_t> unit(re, 1);                      // coordinate of merged dim k per step of input dim j
+  {
+    size_t j = 0;
+    for (size_t k = 0; k < rm; ++k) {
+      int64_t got = 1;
+      const size_t j_first = j;
+      while (j < re && (got < v.M[k] || (j < re && v.E[j] == 1))) { group_of[j] = (int)k; got *= v.E[j]; ++j; }
+      if (got != v.M[k]) return HGPU_OK;
+      int64_t u = 1;
+      bool below_all_onehot = true;
+      for (size_t q = j; q-- > j_first;) {
+        unit[q] = u;
+        u *= v.E[q];
+        if (v.E[q] == 1) continue;
+        if (oh[q]) { if (!below_all_onehot) return HGPU_OK; inner_oh[k] *= v.E[q]; }
+        else below_all_onehot = false;
+      }
+    }
+    for (; j < re; ++j) if (v.E[j] != 1) return HGPU_OK;
+  }
+  // ---- the view's dims: each walks one whole merged dim (or none: the operand stands still)
+  std::vector<int64_t> DM(rm, 1);
+  for (size_t k = rm; k-- > 1;) DM[k - 1] = DM[k] * v.M[k];
+  struct VD { int64_t e, sx, sy, so; int k; bool kept; };
+  std::vector<VD> vd;
+  std::vector<char> covered(rm, 0);
+  int64_t ostr[HGPU_MAX_RANK];
+  dense_strides(n_keep, yo->shape, ostr);
+  for (int d = 0; d < rank; ++d) {
+    if (yo->shape[d] == 1) continue;
+    VD q{yo->shape[d], x->strides[d], yo->strides[d], d < n_keep ? ostr[d] : 0, -1, d < n_keep};
+    if (q.sy != 0) {
+      for (size_t k = 0; k < rm; ++k)
+        if (v.M[k] > 1 && DM[k] == q.sy && v.M[k] == q.e && !covered[k]) { q.k = (int)k; covered[k] = 1; break; }
+      if (q.k < 0) return HGPU_OK;
+    }
+    vd.push_back(q);
+  }
+  for (size_t k = 0; k < rm; ++k) if (v.M[k] > 1 && !covered[k]) return HGPU_OK;
+  // ---- rows (the array's kept dims), columns (the expression's), contracted dims; the chunk dim
+  std::vector<int64_t> rx{0}, rco{0}, cy{0}, cco{0};
+  auto extend = [](std::vector<int64_t>& a, std::vector<int64_t>& b, int64_t e, int64_t sa, int64_t sb) {
+    std::vector<int64_t> a2, b2;
+    for (size_t i = 0; i < a.size(); ++i)
+      for (int64_t t = 0; t < e; ++t) { a2.push_back(a[i] + t * sa); b2.push_back(b[i] + t * sb); }
+    a.swap(a2); b.swap(b2);
+  };
+  int chunk = -1;
+  for (size_t i = 0; i < vd.size(); ++i) {
+    const VD& q = vd[i];
+    if (q.kept) {
+      if (q.sx != 0 && q.sy == 0) { if ((int64_t)rx.size() * q.e > 32) return HGPU_OK; extend(rx, rco, q.e, q.sx, q.so); }
+      else if (q.sx == 0 && q.sy != 0) { if (inner_oh[(size_t)q.k] != 1 || (int64_t)cy.size() * q.e > 64) return HGPU_OK; extend(cy, cco, q.e, q.sy, q.so); }
+      else return HGPU_OK;
+    } else {
+      if (q.sx == 0 || q.sy == 0) return HGPU_OK;
+      if (inner_oh[(size_t)q.k] == 1 && (chunk < 0 || q.e > vd[(size_t)chunk].e)) chunk = (int)i;
+    }
+  }
+  for (size_t k = 0; k < rm; ++k) {
+    if (inner_oh[k] == 1) continue;
+    bool contracted = false;
+    for (auto& q : vd) contracted = contracted || (q.k == (int)k && !q.kept);
+    if (!contracted) return HGPU_OK;                     // a one-hot dim that is kept: nothing to skip
+  }
+  if (chunk < 0 || vd[(size_t)chunk].e < 64) return HGPU_OK;
+  const int MR = (int)rx.size(), NC = (int)cy.size();
+  if (MR < 2) return HGPU_OK;
+  // ---- the other contracted positions of a chunk (one-hot parts left out), and where the one-hot parts lead
+  std::vector<int64_t> gx{0}, gy{0};
+  std::vector<int64_t> ohx((size_t)EH, 0), ohy((size_t)EH, 0);
+  for (size_t i = 0; i < vd.size(); ++i) {
+    const VD& q = vd[i];
+    if (q.kept || (int)i == chunk) continue;
+    const int64_t io = inner_oh[(size_t)q.k];
+    if (q.e / io > 1) {
+      if ((int64_t)gx.size() * (q.e / io) > 65536) return HGPU_OK;
+      extend(gx, gy, q.e / io, q.sx * io, q.sy * io);
+    }
+  }
+  for (int64_t e = 0; e < EH; ++e) {
+    int64_t r = e;
+    for (size_t t = digits.size(); t-- > 0;) {            // the largest stride is the first digit
+      const size_t j = digits[t].second;
+      const int64_t c = r / digits[t].first;
+      r -= c * digits[t].first;
+      for (auto& q : vd)
+        if (q.k == group_of[j]) { ohx[(size_t)e] += c * unit[j] * q.sx; ohy[(size_t)e] += c * unit[j] * q.sy; }
+    }
+  }
+  const int64_t G = (int64_t)gx.size();
+  if ((double)G * NC * (double)vd[(size_t)chunk].e * MR < 1.0e7) return HGPU_OK;     // too little work for a kernel of its own
+  int64_t lo = 0, hi = 0;
+  {
+    int64_t rlo = rx[0], rhi = rx[0], glo = gx[0], ghi = gx[0], olo = ohx[0], ohi = ohx[0];
+    for (int64_t a : rx) { rlo = std::min(rlo, a); rhi = std::max(rhi, a); }
+    for (int64_t a : gx) { glo = std::min(glo, a); ghi = std::max(ghi, a); }
+    for (int64_t a : ohx) { olo = std::min(olo, a); ohi = std::max(ohi, a); }
+    lo = rlo + glo + olo;
+    hi = rhi + ghi + ohi;
+  }
+  const int64_t span = hi - lo + 1;
+  const int es = v.dtype == HGPU_F64 ? 8 : 4;
+  if (span * es > 64 * 1024 || span < 1) return HGPU_OK;
+  for (int64_t a : gy) if (a < 0 || a > INT32_MAX) return HGPU_OK;
+  const VD& chd = vd[(size_t)chunk];
+  const int64_t nch = chd.e, chx = chd.sx, chy = chd.sy;
+  // threads per column, a power of two: 256 threads share the columns out
+  int TPC = 256;
+  while (TPC * NC > 256) TPC >>= 1;
+  if (TPC < 1) return HGPU_OK;
+  // ---- where every input of the expression is read: the offset of (chunk, column, position, one-hot place)
+  // is a sum of four parts, tabulated here from the inputs' strides; nothing is decoded in the kernel
+  std::vector<char> scalar((size_t)v.n_in, 0);
+  std::vector<int> rep((size_t)v.n_in, -1);
+  for (int i = 0; i < v.n_in; ++i) {
+    bool all0 = true;
+    for (size_t j = 0; j < re; ++j) all0 = all0 && (v.E[j] == 1 || v.in[i]->strides[j] == 0);
+    scalar[(size_t)i] = all0;
+    rep[(size_t)i] = i;
+    for (int k = 0; k < i && !all0; ++k) {
+      if (scalar[(size_t)k]) continue;
+      bool same = true;
+      for (size_t j = 0; j < re && same; ++j) same = v.E[j] == 1 || v.in[k]->strides[j] == v.in[i]->strides[j];
+      if (same) { rep[(size_t)i] = rep[(size_t)k]; break; }
+    }
+  }
+  auto in_off = [&](int i, int64_t yoff) {       // input i's offset at the element of the layout yoff elements in
+    int64_t o = 0;
+    size_t j = 0;
+    for (size_t k = 0; k < rm; ++k) {
+      const int64_t ck = (yoff / DM[k]) % v.M[k];
+      for (; j < re && group_of[j] == (int)k; ++j)
+        if (v.E[j] > 1) o += ((ck / unit[j]) % v.E[j]) * v.in[i]->strides[j];
+    }
+    return o;
+  };
+  std::vector<int64_t> chs((size_t)v.n_in, 0);
+  bool fits32 = true;
+  for (int i = 0; i < v.n_in; ++i) {
+    if (scalar[(size_t)i] || rep[(size_t)i] != i) continue;
+    chs[(size_t)i] = in_off(i, chy);
+    if (in_off(i, chy * (nch - 1)) != chs[(size_t)i] * (nch - 1)) return HGPU_OK;     // the chunk dim is one dim of the inputs
+    int64_t reach = 0;
+    for (size_t j = 0; j < re; ++j) reach += (v.E[j] - 1) * (v.in[i]->strides[j] < 0 ? -v.in[i]->strides[j] : v.in[i]->strides[j]);
+    fits32 = fits32 && reach < (1LL << 31);
+  }
+  if (!fits32) return HGPU_OK;
+  std::ostringstream s;
+  char kname[160];
+  snprintf(kname, sizeof kname, "onehot_contract_%s_m%d_n%d_k%lldx%lld_onehot%lld", es == 8 ? "f64" : "f32", MR, NC, (long long)nch, (long long)G, (long long)EH);
+  s << "typedef long long i64;\n";
+  s << "typedef " << (es == 8 ? "double" : "float") << " T;\n";
+  s << hg::fusedgen::kPrelude;
+  auto itab = [&](const std::string& name, const std::vector<int64_t>& t, int64_t shift) {
+    std::vector<int> t2;
+    for (int64_t a : t) t2.push_back((int)(a - shift));
+    return table("__device__ const", name.c_str(), t2);
+  };
+  int64_t rlo = rx[0], glo = gx[0], olo = ohx[0];
+  for (int64_t a : rx) rlo = std::min(rlo, a);
+  for (int64_t a : gx) glo = std::min(glo, a);
+  for (int64_t a : ohx) olo = std::min(olo, a);
+  s << itab("kGX", gx, glo) << itab("kOhX", ohx, olo) << itab("kColC", cco, 0) << itab("kRowC", rco, 0);
+  for (int i = 0; i < v.n_in; ++i) {
+    if (scalar[(size_t)i] || rep[(size_t)i] != i) continue;
+    std::vector<int64_t> tc, tg, to;
+    for (int64_t y : cy) tc.push_back(in_off(i, y));
+    for (int64_t y : gy) tg.push_back(in_off(i, y));
+    for (int64_t y : ohy) to.push_back(in_off(i, y));
+    const std::string n = std::to_string(i);
+    s << itab("kCol" + n, tc, 0) << itab("kG" + n, tg, 0) << itab("kOh" + n, to, 0);
+  }
+  s << "struct Ins {\n";
+  for (int i = 0; i < v.n_in; ++i) s << "  const " << ctype(v.dt[(size_t)i]) << "* i" << i << ";\n";
+  s << "};\n";
+  static const int knob_batch = getenv("HORDEAD_ONEHOT_BATCH") ? atoi(getenv("HORDEAD_ONEHOT_BATCH")) : 16;
+  const int RB = 4;       // rows of the result added up per round at the end
+  const int MA = MR + 1;  // the rows, and the plain sum of the expression's values per column
+  s << "extern \"C\" __global__ void __launch_bounds__(256) " << kname << "(const T* __restrict__ X, Ins ins, T* __restrict__ part, T* __restrict__ psum) {\n";
+  s << "  __shared__ T xs[" << span << "];\n  __shared__ T red[" << RB * 256 << "];\n";
+  s << "  const int tid = threadIdx.x, col = tid / " << TPC << ", li = tid % " << TPC << ";\n  const int cq = col < " << NC << " ? col : 0;\n";
+  for (int i = 0; i < v.n_in; ++i) {
+    if (scalar[(size_t)i]) s << "  const " << ctype(v.dt[(size_t)i]) << " h" << i << " = ins.i" << i << "[0];\n";
+    else if (rep[(size_t)i] == i) s << "  const int c" << i << " = kCol" << i << "[cq];\n";
+  }
+  s << "  T acc[" << MA << "];\n#pragma unroll\n  for (int m = 0; m < " << MA << "; ++m) acc[m] = T(0);\n";
+  s << "  for (i64 ch = blockIdx.x; ch < " << nch << "ll; ch += gridDim.x) {\n";
+  s << "    __syncthreads();\n";
+  s << "    for (int u = tid; u < " << span << "; u += 256) xs[u] = X[ch * " << chx << "ll + u];\n";
+  s << "    __syncthreads();\n";
+  // A thread's positions of a chunk are taken a batch at a time: all the loads of `where`, then all the loads
+  // of the expression's inputs at the places they name, then the multiplications -- each step's trips to memory overlap.
+  const int NI = (int)((G + TPC - 1) / TPC);
+  const int BATCH = NI < knob_batch ? NI : knob_batch;
+  const int rw = rep[(size_t)where_in];
+  s << "    if (col < " << NC << ") {\n";
+  s << "      for (int g0 = li; g0 < " << G << "; g0 += " << TPC * BATCH << ") {\n";
+  s << "        int gg[" << BATCH << "], ee[" << BATCH << "];\n        bool ok[" << BATCH << "];\n        i64 wv[" << BATCH << "];\n";
+  for (int i = 0; i < v.n_in; ++i)
+    if (!scalar[(size_t)i] && i != which_in && i != where_in) s << "        " << ctype(v.dt[(size_t)i]) << " r" << i << "[" << BATCH << "];\n";
+  s << "#pragma unroll\n        for (int it = 0; it < " << BATCH << "; ++it) {\n";
+  s << "          const int g = g0 + it * " << TPC << ";\n          ok[it] = g < " << G << ";\n          gg[it] = ok[it] ? g : 0;\n";
+  s << "          wv[it] = ins.i" << where_in << "[ch * " << chs[(size_t)rw] << "ll + (c" << rw << " + kG" << rw << "[gg[it]])];\n        }\n";
+  s << "#pragma unroll\n        for (int it = 0; it < " << BATCH << "; ++it) {\n";
+  s << "          const i64 e = wv[it] - " << wh->offset << "ll;\n";
+  s << "          ok[it] = ok[it] && e >= 0 && e < " << EH << ";\n          ee[it] = ok[it] ? (int)e : 0;\n";
+  for (int i = 0; i < v.n_in; ++i) {
+    if (scalar[(size_t)i] || i == which_in || i == where_in) continue;
+    const int r = rep[(size_t)i];
+    s << "          r" << i << "[it] = ins.i" << i << "[ch * " << chs[(size_t)r] << "ll + (c" << r << " + kG" << r << "[gg[it]] + kOh" << r << "[ee[it]])];\n";
+  }
+  s << "        }\n";
+  s << "#pragma unroll\n        for (int it = 0; it < " << BATCH << "; ++it) {\n";
+  for (int i = 0; i < v.n_in; ++i) {
+    s << "          const " << ctype(v.dt[(size_t)i]) << " v" << i << "_ = ";
+    if (scalar[(size_t)i]) s << "h" << i;
+    else if (i == which_in) s << "(i64)ee[it] + " << wh->offset << "ll";       // the index vector holds its own offsets
+    else if (i == where_in) s << "wv[it]";
+    else s << "r" << i << "[it]";
+    s << ";\n";
+  }
+  emit_program(s, v.n_in, v.n_instr, v.prog, v.dt, "          ", "_");
+  s << "          const T val = ok[it] ? v" << v.slot << "_ : T(0);\n";
+  s << "          const T* xp = xs + kGX[gg[it]] + kOhX[ee[it]];\n";
+  static const int knob_nofma = getenv("HORDEAD_ONEHOT_NOFMA") ? atoi(getenv("HORDEAD_ONEHOT_NOFMA")) : 0;
+  for (int m = 0; m < (knob_nofma ? 1 : MR); ++m) s << "          acc[" << m << "] += val * xp[" << rx[(size_t)m] - rlo << "];\n";
+  s << "          acc[" << MR << "] += val;\n";
+  s << "        }\n      }\n    }\n  }\n";
+  // the threads of a column add up, a few rows of the result per round; thread (row, column) writes the block's partial result
+  s << "#pragma unroll\n  for (int m0 = 0; m0 < " << MA << "; m0 += " << RB << ") {\n    __syncthreads();\n";
+  s << "#pragma unroll\n    for (int m = m0; m < m0 + " << RB << " && m < " << MA << "; ++m) red[(m - m0) * 256 + tid] = acc[m];\n    __syncthreads();\n";
+  s << "    for (int o = tid; o < " << RB * NC << "; o += 256) {\n      const int m = m0 + o / " << NC << ", c = o % " << NC << ";\n";
+  s << "      if (m < " << MA << ") {\n        T sum = T(0);\n";
+  s << "        for (int l = 0; l < " << TPC << "; ++l) sum += red[(m - m0) * 256 + c * " << TPC << " + l];\n";
+  s << "        if (m < " << MR << ") part[(i64)blockIdx.x * " << (int64_t)nelem(out) << "ll + kRowC[m] + kColC[c]] = sum;\n";
+  s << "        else psum[(i64)blockIdx.x * " << NC << " + c] = sum;\n      }\n    }\n  }\n}\n";
+  std::string src = s.str();
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c{nullptr, nullptr};
+    if (compile(ctx, src, kname, &c) != HGPU_OK) c = Compiled{nullptr, nullptr};
+    it = cache.emplace(src, c).first;
+  }
+  if (!it->second.fn) return HGPU_OK;
+  wh->buf->known_relied_on = true;
+  for (int i = 0; i < v.n_in; ++i)
+    if (v.in[i]->buf && v.in[i]->buf->known == hgpu_buffer::kZeroScalar) v.in[i]->buf->known_relied_on = true;
+  static const int knob_grid = getenv("HORDEAD_ONEHOT_GRID") ? atoi(getenv("HORDEAD_ONEHOT_GRID")) : 2;
+  const int64_t grid = std::min<int64_t>(nch, (int64_t)ctx->num_cu * knob_grid);
+  const int64_t out_n = nelem(out);
+  // the column sums: an array of the columns' shape, kept for a caller that asks for exactly that sum next
+  std::vector<int64_t> colshape;
+  std::vector<int> colk;
+  for (auto& q : vd)
+    if (q.kept && q.sx == 0) { colshape.push_back(q.e); colk.push_back(q.k); }
+  hgpu_array* colsum = nullptr;
+  int rc = new_dense(ctx, v.dtype, (int)colshape.size(), colshape.data(), &colsum);
+  if (rc) return rc;
+  hgpu_buffer* part = nullptr;
+  rc = buffer_alloc(ctx, (size_t)((out_n + NC) * grid) * es, &part);
+  if (rc) { hgpu_release(colsum); return rc; }
+  const char* xp = (const char*)data_ptr(x) + lo * es;
+  void* pdst = part->ptr;
+  void* sdst = (char*)part->ptr + (size_t)(out_n * grid) * es;
+  std::vector<const void*> ia;
+  for (int i = 0; i < v.n_in; ++i) ia.push_back(data_ptr(v.in[i]));
+  void* args[] = {(void*)&xp, (void*)ia.data(), (void*)&pdst, (void*)&sdst};
+  {
+    double bytes = (double)nch * span * es;
+    for (int i = 0; i < v.n_in; ++i) {
+      if (i == which_in) continue;
+      int64_t distinct = 1;
+      for (int d = 0; d < v.in[i]->rank; ++d)
+        if (v.in[i]->strides[d] != 0) distinct *= v.in[i]->shape[d];
+      if (distinct > 1) bytes += (double)distinct * dtype_size(v.in[i]->dtype);
+    }
+    const char* label = "onehot_contract";
+    if (ctx->profiling && ctx->profile_shapes) {
+      char buf[200];
+      snprintf(buf, sizeof buf, "onehot_contract[rows%d,cols%d,chunks%lld,positions%lld,onehot%lld,in%d,instr%d,es%d]", MR, NC, (long long)nch, (long long)G, (long long)EH, v.n_in, v.n_instr, es);
+      label = intern_label(ctx, buf);
+    }
+    LaunchGuard lg(ctx, label, bytes, 2.0 * MR * NC * (double)G * (double)nch);
+    hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+    if (e != hipSuccess) { buffer_release(part); hgpu_release(colsum); return check_hip(ctx, e, "onehot_contract launch"); }
+  }
+  rc = hg::sum_partials(ctx, v.dtype, out_n, (int)grid, part->ptr, data_ptr(out));
+  if (!rc) rc = hg::sum_partials(ctx, v.dtype, NC, (int)grid, sdst, data_ptr(colsum));
+  buffer_release(part);
+  if (rc) { hgpu_release(colsum); return rc; }
+  remember_sum(ctx, v, colk, colsum);
+  *handled = true;
+  return HGPU_OK;
+}
+
 }  // namespace
 
 namespace hg {
 bool classify_contraction(int rank, const int64_t* shape, const int64_t* st_a, const int64_t* st_b, const int64_t* st_c, int n_keep, gemm::GemmParams* p);
+
+void forget_remembered_sums(hgpu_ctx* ctx) {
+  std::vector<MemoSum> gone;
+  {
+    std::lock_guard<std::mutex> lk(ctx->launch_mu);
+    gone.swap(memo_of(ctx).items);
+  }
+  for (auto& m : gone) forget(m);
+}
 }
 
 extern "C" int hgpu_contract_operands(hgpu_ctx* ctx, const hgpu_operand* a, const hgpu_operand* b, int n_keep, int flags, hgpu_array** out) {
@@ -1939,8 +2433,24 @@ extern "C" int hgpu_contract_operands(hgpu_ctx* ctx, const hgpu_operand* a, cons
     if (rc) return rc;
     bool handled = false;
     if (!b) {
+      std::vector<int> kept;
+      if (kept_merged_dims(va, a, n_keep, &kept)) {
+        if (hgpu_array* known = recall_sum(ctx, va, kept)) {     // a kernel that evaluated the expression has left this sum behind
+          hgpu_release(o);
+          rc = hgpu_reshape(ctx, known, n_keep, shape_of(a), out);
+          hgpu_release(known);
+          return rc;
+        }
+      }
       rc = try_mapped_sum(ctx, va, a, n_keep, o, &handled);
     } else if ((a->array || va.total < (1LL << 31)) && (b->array || vb.total < (1LL << 31))) {
+      // one operand an array, the other an expression that is one-hot along contracted dims
+      if (a->array && !b->array) rc = try_onehot_contract(ctx, a->array, vb, b, n_keep, o, &handled);
+      else if (b->array && !a->array) rc = try_onehot_contract(ctx, b->array, va, a, n_keep, o, &handled);
+      if (rc || handled) {
+        if (rc) hgpu_release(o); else *out = o;
+        return rc;
+      }
       GemmParams p;
       if (hg::classify_contraction(rank, shape_of(a), strides_of(a), strides_of(b), o->strides, n_keep, &p)) {
         p.n_terms = 0;

@@ -396,6 +396,7 @@ int hgpu_shutdown(hgpu_ctx* ctx) {
   (void)hipSetDevice(ctx->device);
   drop_deferred(ctx);
   (void)hipStreamSynchronize(ctx->stream);
+  forget_remembered_sums(ctx);
   if (ctx->zero_block) { buffer_release(ctx->zero_block); ctx->zero_block = nullptr; }
   {
     std::lock_guard<std::mutex> g(ctx->mu);
@@ -520,6 +521,11 @@ int hgpu_upload(hgpu_ctx* ctx, int dtype, int rank, const int64_t* shape, const 
       hgpu_release(a);
       return check_hip(ctx, e, "upload");
     }
+    if (nelem(a) == 1 && a->buf && a->offset == 0) {      // a constant of a program: remember when it is zero
+      bool zero = true;
+      for (size_t i = 0; i < bytes; ++i) zero = zero && ((const unsigned char*)host)[i] == 0;
+      if (zero) a->buf->known = hgpu_buffer::kZeroScalar;
+    }
   }
   *out = a;
   return HGPU_OK;
@@ -532,7 +538,10 @@ int hgpu_overwrite(hgpu_ctx* ctx, hgpu_array* a, const void* host) {
   size_t bytes = (size_t)nelem(a) * dtype_size(a->dtype);
   if (bytes == 0) return HGPU_OK;
   if (!host) return fail(ctx, HGPU_ERR_INVALID, "null host pointer");
+  if (a->buf->known_relied_on) return fail(ctx, HGPU_ERR_INVALID, "overwrite: a kernel has been chosen for this array's contents (an index vector or a zero constant)");
+  a->buf->known = hgpu_buffer::kUnknown;
   LaunchGuard lg(ctx);
+  ctx->write_epoch++;
   hipError_t e = hipMemcpyAsync(data_ptr(a), host, bytes, hipMemcpyHostToDevice, ctx->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   return check_hip(ctx, e, "overwrite");
@@ -544,6 +553,12 @@ int hgpu_assign(hgpu_ctx* ctx, hgpu_array* dst, const hgpu_array* src) {
   if (!is_dense(dst)) return fail(ctx, HGPU_ERR_INVALID, "assign: the destination is a strided view");
   if (nelem(dst) == 0) return HGPU_OK;
   if (dst->buf == src->buf) return fail(ctx, HGPU_ERR_INVALID, "assign: source and destination share memory");
+  if (dst->buf->known_relied_on) return fail(ctx, HGPU_ERR_INVALID, "assign: a kernel has been chosen for the destination's contents (an index vector or a zero constant)");
+  dst->buf->known = hgpu_buffer::kUnknown;
+  {
+    std::lock_guard<std::mutex> lk(ctx->launch_mu);
+    ctx->write_epoch++;
+  }
   return copy_view(ctx, dst->dtype, dst->rank, dst->shape, data_ptr(src), src->strides, data_ptr(dst), dst->strides);
 }
 

@@ -7,9 +7,10 @@
 -- * Every array kind (@TKR@, @TKS@, @TKX@ of scalars) is a handle to a device
 --   value of the host layer (include/hordead_host.h); the shape lives with the
 --   value, so the three kinds share one representation and differ in what the
---   types promise.  Arrays of arrays and arrays of products are not
---   represented (the reference's examples and tests on the accelerated path
---   do not use them); the conversions that would make them raise @error@.
+--   types promise.  An array of pairs is a pair of arrays, and an array of
+--   arrays is one device array with the inner dims behind the outer ones
+--   ('ArrGpu') -- the layout ox-arrays gives them on the CPU -- so zip, unzip,
+--   nest and unnest (OpsConcrete.hs:821-876) move no data.
 -- * A scalar (@TKScalar r@) is a 'GpuIx': a literal known on the host, a
 --   rank-0 device value, or -- inside the closure of a gather, scatter or
 --   build -- a /lane/: one scalar per position of the index space, all
@@ -22,7 +23,8 @@
 -- written against horde-ad's modules as they are in the reference checkout.
 module HordeAd.Core.CarriersGpu
   ( -- * The carrier
-    Gpu (..), RepGpu, GpuFun (..), GpuIx (..)
+    Gpu (..), RepGpu, ArrGpu, GpuFun (..), GpuIx (..)
+  , arrMap, arrZip, arrZipN, arrLeaves
     -- * Calling the host layer
   , out1, un1, bin, withShape, withIxArray, outIx
   , gpuShape, dtypeOf, scalarVal, valScalar, laneOf, literal
@@ -33,6 +35,7 @@ module HordeAd.Core.CarriersGpu
 
 import Prelude
 
+import Control.DeepSeq (NFData (..))
 import Data.Boolean (Boolean (..))
 import Data.Int (Int16, Int32, Int64, Int8)
 import Data.Kind (Type)
@@ -50,13 +53,114 @@ import HordeAd.Gpu.Foreign
 
 type family RepGpu (y :: TK) :: Type where
   RepGpu (TKScalar r) = GpuIx
-  RepGpu (TKR2 n x) = ValPtr
-  RepGpu (TKS2 sh x) = ValPtr
-  RepGpu (TKX2 sh x) = ValPtr
+  RepGpu (TKR2 n x) = ArrGpu x
+  RepGpu (TKS2 sh x) = ArrGpu x
+  RepGpu (TKX2 sh x) = ArrGpu x
   RepGpu (TKProduct x z) = (RepGpu x, RepGpu z)
+
+-- | An array (of any shape) whose elements have kind @x@.  Scalars: one device
+-- array.  Pairs: a pair of arrays of one outer shape (struct of arrays, which is
+-- how @Nested.Mixed sh (a, b)@ is laid out too).  Arrays: the element's array
+-- with the inner dims trailing the outer ones, so that every operation on the
+-- outer dims (index, gather, transpose of a prefix, append, sum over the
+-- outermost dim) is the same call on the one flat array.
+type family ArrGpu (x :: TK) :: Type where
+  ArrGpu (TKScalar r) = ValPtr
+  ArrGpu (TKR2 n x) = ArrGpu x
+  ArrGpu (TKS2 sh x) = ArrGpu x
+  ArrGpu (TKX2 sh x) = ArrGpu x
+  ArrGpu (TKProduct x z) = (ArrGpu x, ArrGpu z)
+
+-- | One call per device array of an array value.
+arrMap :: SingletonTK x -> (ValPtr -> ValPtr) -> ArrGpu x -> ArrGpu x
+arrMap stk f a = case stk of
+  STKScalar -> f a
+  STKR _ x -> arrMap x f a
+  STKS _ x -> arrMap x f a
+  STKX _ x -> arrMap x f a
+  STKProduct s1 s2 -> (arrMap s1 f (fst a), arrMap s2 f (snd a))
+
+-- | The same for two array values of one element kind (append, select, addition of cotangents).
+arrZip :: SingletonTK x -> (ValPtr -> ValPtr -> ValPtr) -> ArrGpu x -> ArrGpu x -> ArrGpu x
+arrZip stk f a b = case stk of
+  STKScalar -> f a b
+  STKR _ x -> arrZip x f a b
+  STKS _ x -> arrZip x f a b
+  STKX _ x -> arrZip x f a b
+  STKProduct s1 s2 -> (arrZip s1 f (fst a) (fst b), arrZip s2 f (snd a) (snd b))
+
+-- | ... for a list of them (stacking).
+arrZipN :: SingletonTK x -> ([ValPtr] -> ValPtr) -> [ArrGpu x] -> ArrGpu x
+arrZipN stk f as = case stk of
+  STKScalar -> f as
+  STKR _ x -> arrZipN x f as
+  STKS _ x -> arrZipN x f as
+  STKX _ x -> arrZipN x f as
+  STKProduct s1 s2 -> (arrZipN s1 f (map fst as), arrZipN s2 f (map snd as))
+
+-- | Every device array of an array value, leftmost first (all share the outer dims).
+arrLeaves :: SingletonTK x -> ArrGpu x -> [ValPtr]
+arrLeaves stk a = case stk of
+  STKScalar -> [a]
+  STKR _ x -> arrLeaves x a
+  STKS _ x -> arrLeaves x a
+  STKX _ x -> arrLeaves x a
+  STKProduct s1 s2 -> arrLeaves s1 (fst a) ++ arrLeaves s2 (snd a)
 
 type role Gpu nominal
 newtype Gpu y = Gpu {unGpu :: RepGpu y}
+
+-- | As for @Concrete@ (CarriersConcrete.hs:295-298): 'AllTargetShow' asks for it
+-- (Ops.hs:1297-1313).  A device array shows as its element type, shape and elements
+-- (downloaded: showing is for tests and error messages).
+instance KnownSTK y => Show (Gpu y) where
+  showsPrec d (Gpu t) = showsRep (knownSTK @y) d t
+
+showsRep :: SingletonTK y -> Int -> RepGpu y -> ShowS
+showsRep stk d t = case stk of
+  STKScalar -> showsPrec d t
+  STKR _ x -> showsArr x t
+  STKS _ x -> showsArr x t
+  STKX _ x -> showsArr x t
+  STKProduct s1 s2 -> showParen (d > 10) $ showString "(" . showsRep s1 0 (fst t) . showString ", " . showsRep s2 0 (snd t) . showString ")"
+ where
+  showsArr :: SingletonTK x -> ArrGpu x -> ShowS
+  showsArr x a = showString "gpu" . showList (map showVal (arrLeaves x a))
+
+instance Show GpuIx where
+  showsPrec d (GpuIxLit x) = showsPrec d x
+  showsPrec _ (GpuIxVal v) = showString (showVal v)
+  showsPrec _ (GpuIxLane shm _) = showString "<lane over " . shows shm . showString ">"
+
+-- | dtype, shape and the elements of a device value as doubles (a synchronous read-back).
+showVal :: ValPtr -> String
+showVal v = unsafePerformIO $ do
+  ctx <- theCtx
+  let sh = gpuShape v
+      n = product sh
+  xs <- withForeignPtr (arr1AsDouble v) $ \p -> allocaArray (max 1 n) $ \buf -> do
+    c_hh_download ctx p (castPtr buf) >>= check ctx
+    peekArray n (buf :: Ptr Double)
+  pure (show sh ++ " " ++ show xs)
+ where
+  arr1AsDouble = un1 (\c p -> c_hh_convert c p 0 0)       -- tscast to Double (dtype code 0), the identity on Double arrays
+
+-- | Device values are evaluated when they are made: the calls are strict, the
+-- kernels run in stream order.  Forcing the handles is all @rnf@ has to do
+-- (CarriersConcrete.hs:297-298 forces the host arrays).
+instance KnownSTK y => NFData (Gpu y) where
+  rnf (Gpu t) = rnfRep (knownSTK @y) t
+
+rnfRep :: SingletonTK y -> RepGpu y -> ()
+rnfRep stk t = case stk of
+  STKScalar -> case t of
+    GpuIxLit x -> x `seq` ()
+    GpuIxVal v -> v `seq` ()
+    GpuIxLane _ x -> x `seq` ()
+  STKR _ x -> foldr seq () (arrLeaves x t)
+  STKS _ x -> foldr seq () (arrLeaves x t)
+  STKX _ x -> foldr seq () (arrLeaves x t)
+  STKProduct s1 s2 -> rnfRep s1 (fst t) `seq` rnfRep s2 (snd t)
 
 type role GpuFun nominal nominal
 newtype GpuFun x z = GpuFun (RepGpu x -> RepGpu z)
@@ -71,7 +175,9 @@ type instance ShareOf Gpu = Gpu
 
 -- | A scalar of the carrier.
 data GpuIx
-  = GpuIxLit Double          -- ^ a literal (@fromInteger@, @fromRational@, a host constant); exact for |n| < 2^53
+  = GpuIxLit Double          -- ^ a literal (@fromInteger@, @fromRational@, a host constant).  Integers are exact for
+                             --   |n| < 2^53 -- every index is -- so @tkconcrete \@Int64@ of a larger value takes the
+                             --   other road ('GpuIxVal', an uploaded rank-0 array: see @literal'@ in OpsGpu)
   | GpuIxVal ValPtr          -- ^ a rank-0 device value
   | GpuIxLane [Int] IxPtr    -- ^ one scalar per position of the space @shm@ (inside an index function)
 

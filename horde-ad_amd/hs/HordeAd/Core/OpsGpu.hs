@@ -10,7 +10,11 @@
 -- a host loop) through the C ABI of include/hordead_host.h.  The ranked,
 -- shaped and mixed methods of one operation are the same call: the shape
 -- lives with the device value, and what differs is how the static part of
--- the result's shape is put together for the type.
+-- the result's shape is put together for the type.  Methods that are
+-- polymorphic in the element kind @x@ (indexing, gather, scatter, the views,
+-- replicate, sum, stacking) make that call once per device array of the value
+-- ('arrMap': an array of pairs is a pair of arrays, an array of arrays one
+-- array with the inner dims behind the outer ones).
 --
 -- Not compiled in this repository's build environment (no GHC there); written
 -- against horde-ad's own modules as they are in the reference checkout.
@@ -62,6 +66,14 @@ import HordeAd.Gpu.Foreign
 
 dims :: RepGpu y ~ ValPtr => Gpu y -> [Int]
 dims (Gpu v) = gpuShape v
+
+-- | The outer dims of an array value of any element kind: the first @n@ dims of its first device array.
+outerDims :: SingletonTK x -> Int -> ArrGpu x -> [Int]
+outerDims stk n a = take n (gpuShape (head (arrLeaves stk a)))
+
+-- | Reshape of the outer dims (the first @nOld@ of them) with whatever inner dims there are kept behind.
+reshapeOuter :: Int -> [Int] -> ValPtr -> ValPtr
+reshapeOuter nOld new v = reshapeTo (new ++ drop nOld (gpuShape v)) v
 
 -- | rshape (OpsConcrete.hs:99): the rank in the type is the rank of the value.
 shrOf :: forall n. [Int] -> IShR n
@@ -175,14 +187,17 @@ instance ShareTensor Gpu where
 instance BaseTensor Gpu where
   isConcreteInstance = False
 
-  rshape = shrOf . dims
-  sshape = shsOf . dims
-  xshape @sh (Gpu v) = shxOf (mixedSkeleton @sh v) (gpuShape v)
+  rshape @n @x (Gpu v) = shrOf (outerDims (knownSTK @x) (valueOf @n) v)
+  sshape @sh @x (Gpu v) = shsOf (outerDims (knownSTK @x) (shsLength (knownShS @sh)) v)
+  xshape @sh @x (Gpu v) =
+    let v0 = head (arrLeaves (knownSTK @x) v)
+        n = ssxLength (mixedSkeleton @sh v0)
+    in shxOf (mixedSkeleton @sh v0) (take n (gpuShape v0))
   tftk stk (Gpu v) = case stk of             -- CarriersConcrete.hs:164 (tftkG)
     STKScalar -> FTKScalar
-    STKR _ x -> FTKR (shrOf (gpuShape v)) (scalarsOnly x)
-    STKS sh x -> FTKS sh (scalarsOnly x)
-    STKX ssx x -> FTKX (shxOf ssx (gpuShape v)) (scalarsOnly x)
+    STKR n x -> FTKR (shrOf (outerDims x (fromSNat' n) v)) (elemFTK x (fromSNat' n) v)
+    STKS sh x -> FTKS sh (elemFTK x (shsLength sh) v)
+    STKX ssx x -> FTKX (shxOf ssx (outerDims x (ssxLength ssx) v)) (elemFTK x (ssxLength ssx) v)
     STKProduct s1 s2 -> FTKProduct (tftk s1 (Gpu (fst v))) (tftk s2 (Gpu (snd v)))
 
   tpair (Gpu a) (Gpu b) = Gpu (a, b)                              -- :107
@@ -211,59 +226,64 @@ instance BaseTensor Gpu where
     FTKS _ FTKScalar -> tsconcrete a
     FTKX _ FTKScalar -> txconcrete a
     FTKProduct f1 f2 -> tpair (tconcrete f1 (Concrete (fst a))) (tconcrete f2 (Concrete (snd a)))
-    _ -> nestedArrays "tconcrete"
+    -- arrays of arrays and of pairs: unzipped and unnested on the host (both free in ox-arrays), then uploaded leaf by leaf
+    FTKR sh x -> Gpu (uploadNested (ftkToSTK x) (Foldable.toList sh) (Nested.rtoMixed a))
+    FTKS sh x -> Gpu (uploadNested (ftkToSTK x) (shsToList sh) (Nested.stoMixed a))
+    FTKX sh x -> Gpu (uploadNested (ftkToSTK x) (shxToList' sh) a)
 
   -- :125-214
-  trfromVectorN shm v = stackOf (Foldable.toList shm) (V.toList v)
+  trfromVectorN @_ @x shm v = stackOf (knownSTK @x) (Foldable.toList shm) (V.toList v)
   trfromVectorLinear @_ @r shm v = Gpu (stackVals (Foldable.toList shm) [] (map (scalarVal (dtypeOf @r) . unGpu) (V.toList v)))
-  tsfromVectorN shm v = stackOf (shsToList shm) (V.toList v)
+  tsfromVectorN @_ @_ @x shm v = stackOf (knownSTK @x) (shsToList shm) (V.toList v)
   tsfromVectorLinear @_ @r shm v = Gpu (stackVals (shsToList shm) [] (map (scalarVal (dtypeOf @r) . unGpu) (V.toList v)))
-  txfromVectorN shm v = stackOf (shxToList' shm) (V.toList v)
+  txfromVectorN @_ @_ @x shm v = stackOf (knownSTK @x) (shxToList' shm) (V.toList v)
   txfromVectorLinear @_ @r shm v = Gpu (stackVals (shxToList' shm) [] (map (scalarVal (dtypeOf @r) . unGpu) (V.toList v)))
 
-  trsumN @m (Gpu t) = Gpu (sumPrefix (valueOf @m) t)                                 -- :215-230
+  trsumN @m @_ @x (Gpu t) = Gpu (arrMap (knownSTK @x) (sumPrefix (valueOf @m)) t)      -- :215-230
   trsum0 (Gpu t) = Gpu (valScalar (un1 c_hh_tssum0 t))
   trdot0 (Gpu a) (Gpu b) = Gpu (valScalar (bin c_hh_tsdot0 a b))
   trdot1In (Gpu a) (Gpu b) = Gpu (bin c_hh_tsdot1In a b)
   trmatvecmul (Gpu m) (Gpu v) = Gpu (bin c_hh_tsmatvecmul m v)
   trmatmul2 (Gpu a) (Gpu b) = Gpu (bin c_hh_tsmatmul2 a b)
-  trreplicateN shm (Gpu t) = Gpu (replicatePrefix (Foldable.toList shm) t)
+  trreplicateN @_ @_ @x shm (Gpu t) = Gpu (arrMap (knownSTK @x) (replicatePrefix (Foldable.toList shm)) t)
   trreplicate0N @_ @r shm (Gpu s) = Gpu (replicatePrefix (Foldable.toList shm) (scalarVal (dtypeOf @r) s))
 
-  tssumN @shm (Gpu t) = Gpu (sumPrefix (shsLength (knownShS @shm)) t)
+  tssumN @shm @_ @x (Gpu t) = Gpu (arrMap (knownSTK @x) (sumPrefix (shsLength (knownShS @shm))) t)
   tssum0 (Gpu t) = Gpu (valScalar (un1 c_hh_tssum0 t))
   tsdot0 (Gpu a) (Gpu b) = Gpu (valScalar (bin c_hh_tsdot0 a b))                     -- :231
   tsdot1In _ (Gpu a) (Gpu b) = Gpu (bin c_hh_tsdot1In a b)                           -- :233
   tsmatvecmul (Gpu m) (Gpu v) = Gpu (bin c_hh_tsmatvecmul m v)                       -- :236
   tsmatmul2 (Gpu a) (Gpu b) = Gpu (bin c_hh_tsmatmul2 a b)                           -- :237
-  tsreplicateN shm (Gpu t) = Gpu (replicatePrefix (shsToList shm) t)                 -- :243
+  tsreplicateN @_ @_ @x shm (Gpu t) = Gpu (arrMap (knownSTK @x) (replicatePrefix (shsToList shm)) t)   -- :243
   tsreplicate0N @_ @r shm (Gpu s) = Gpu (replicatePrefix (shsToList shm) (scalarVal (dtypeOf @r) s))
 
-  txsumN @shm (Gpu t) = Gpu (sumPrefix (ssxLength (knownShX @shm)) t)
+  txsumN @shm @_ @x (Gpu t) = Gpu (arrMap (knownSTK @x) (sumPrefix (ssxLength (knownShX @shm))) t)
   txsum0 (Gpu t) = Gpu (valScalar (un1 c_hh_tssum0 t))
   txdot0 (Gpu a) (Gpu b) = Gpu (valScalar (bin c_hh_tsdot0 a b))
   txdot1In _ (Gpu a) (Gpu b) = Gpu (bin c_hh_tsdot1In a b)
   txmatvecmul _ _ (Gpu m) (Gpu v) = Gpu (bin c_hh_tsmatvecmul m v)
   txmatmul2 (Gpu a) (Gpu b) = Gpu (bin c_hh_tsmatmul2 a b)
-  txreplicateN shm (Gpu t) = Gpu (replicatePrefix (shxToList' shm) t)
+  txreplicateN @_ @_ @x shm (Gpu t) = Gpu (arrMap (knownSTK @x) (replicatePrefix (shxToList' shm)) t)
   txreplicate0N @_ @r shm (Gpu s) = Gpu (replicatePrefix (shxToList' shm) (scalarVal (dtypeOf @r) s))
 
   -- :246-360: indexing, gather, scatter
-  trindex (Gpu t) ix = Gpu (indexPrefix (ixList ix) t)
+  -- (the index function is applied once per device array of the value: it is pure, and the host layer
+  -- recognises equal index lanes)
+  trindex @_ @_ @x (Gpu t) ix = Gpu (arrMap (knownSTK @x) (indexPrefix (ixList ix)) t)
   trindex0 (Gpu t) ix = Gpu (valScalar (indexPrefix (ixList ix) t))
-  trscatter @m shp (Gpu t) f =
-    Gpu (scatterBy (take (valueOf @m) (gpuShape t)) (Foldable.toList shp) t (viaIxR f))
-  trgather shm (Gpu t) f = Gpu (gatherBy (Foldable.toList shm) t (viaIxR f))
-  tsindex (Gpu t) ix = Gpu (indexPrefix (ixList ix) t)
+  trscatter @m @_ @_ @x shp (Gpu t) f =
+    Gpu (arrMap (knownSTK @x) (\v -> scatterBy (take (valueOf @m) (gpuShape v)) (Foldable.toList shp) v (viaIxR f)) t)
+  trgather @_ @_ @_ @x shm (Gpu t) f = Gpu (arrMap (knownSTK @x) (\v -> gatherBy (Foldable.toList shm) v (viaIxR f)) t)
+  tsindex @_ @_ @x (Gpu t) ix = Gpu (arrMap (knownSTK @x) (indexPrefix (ixList ix)) t)
   tsindex0 (Gpu t) ix = Gpu (valScalar (indexPrefix (ixList ix) t))
-  tsscatter @shm @_ @shp (Gpu t) f =
-    Gpu (scatterBy (shsToList (knownShS @shm)) (shsToList (knownShS @shp)) t (viaIxS f))
-  tsgather @shm (Gpu t) f = Gpu (gatherBy (shsToList (knownShS @shm)) t (viaIxS f))
-  txindex (Gpu t) ix = Gpu (indexPrefix (ixList ix) t)
+  tsscatter @shm @_ @shp @x (Gpu t) f =
+    Gpu (arrMap (knownSTK @x) (\v -> scatterBy (shsToList (knownShS @shm)) (shsToList (knownShS @shp)) v (viaIxS f)) t)
+  tsgather @shm @_ @_ @x (Gpu t) f = Gpu (arrMap (knownSTK @x) (\v -> gatherBy (shsToList (knownShS @shm)) v (viaIxS f)) t)
+  txindex @_ @_ @x (Gpu t) ix = Gpu (arrMap (knownSTK @x) (indexPrefix (ixList ix)) t)
   txindex0 (Gpu t) ix = Gpu (valScalar (indexPrefix (ixList ix) t))
-  txscatter @shm shp (Gpu t) f =
-    Gpu (scatterBy (take (ssxLength (knownShX @shm)) (gpuShape t)) (shxToList' shp) t (viaIxX f))
-  txgather shm (Gpu t) f = Gpu (gatherBy (shxToList' shm) t (viaIxX f))
+  txscatter @shm @_ @_ @x shp (Gpu t) f =
+    Gpu (arrMap (knownSTK @x) (\v -> scatterBy (take (ssxLength (knownShX @shm)) (gpuShape v)) (shxToList' shp) v (viaIxX f)) t)
+  txgather @_ @_ @_ @x shm (Gpu t) f = Gpu (arrMap (knownSTK @x) (\v -> gatherBy (shxToList' shm) v (viaIxX f)) t)
 
   -- :361-560: conversions of the element type, arg-extrema, iota
   tkfloor @_ @r2 (Gpu a) = Gpu (scConvert (dtypeOf @r2) 1 a)
@@ -291,28 +311,41 @@ instance BaseTensor Gpu where
   txiota @n @r = Gpu (iotaArr (dtypeOf @r) (valueOf @n))
 
   -- :561-660: the views
-  trappend (Gpu a) (Gpu b) = Gpu (bin c_hh_tsappend a b)
-  trslice i n (Gpu t) = Gpu (sliceOuter i n t)
-  trreverse (Gpu t) = Gpu (un1 c_hh_tsreverse t)
-  trtranspose perm (Gpu t) = Gpu (transposeBy perm t)
-  trreshape sh (Gpu t) = Gpu (reshapeTo (Foldable.toList sh) t)
-  tsappend (Gpu a) (Gpu b) = Gpu (bin c_hh_tsappend a b)                             -- :638
-  tsslice i n _ (Gpu t) = Gpu (sliceOuter (fromSNat' i) (fromSNat' n) t)            -- :641
-  tsreverse (Gpu t) = Gpu (un1 c_hh_tsreverse t)                                     -- :644
-  tstranspose perm (Gpu t) = Gpu (transposeBy (Permutation.permToList' perm) t)      -- :647
-  tsreshape sh (Gpu t) = Gpu (reshapeTo (shsToList sh) t)                            -- :650
-  txappend (Gpu a) (Gpu b) = Gpu (bin c_hh_tsappend a b)
-  txslice i n _ (Gpu t) = Gpu (sliceOuter (fromSMayNat' i) (fromSMayNat' n) t)
-  txreverse (Gpu t) = Gpu (un1 c_hh_tsreverse t)
-  txtranspose perm (Gpu t) = Gpu (transposeBy (Permutation.permToList' perm) t)
-  txreshape sh (Gpu t) = Gpu (reshapeTo (shxToList' sh) t)
+  trappend @_ @x (Gpu a) (Gpu b) = Gpu (arrZip (knownSTK @x) (bin c_hh_tsappend) a b)
+  trslice @_ @x i n (Gpu t) = Gpu (arrMap (knownSTK @x) (sliceOuter i n) t)
+  trreverse @_ @x (Gpu t) = Gpu (arrMap (knownSTK @x) (un1 c_hh_tsreverse) t)
+  trtranspose @_ @x perm (Gpu t) = Gpu (arrMap (knownSTK @x) (transposeBy perm) t)
+  trreshape @n @_ @x sh (Gpu t) = Gpu (arrMap (knownSTK @x) (reshapeOuter (valueOf @n) (Foldable.toList sh)) t)
+  tsappend @_ @_ @_ @x (Gpu a) (Gpu b) = Gpu (arrZip (knownSTK @x) (bin c_hh_tsappend) a b)                      -- :638
+  tsslice @_ @_ @_ @_ @x i n _ (Gpu t) = Gpu (arrMap (knownSTK @x) (sliceOuter (fromSNat' i) (fromSNat' n)) t)   -- :641
+  tsreverse @_ @_ @x (Gpu t) = Gpu (arrMap (knownSTK @x) (un1 c_hh_tsreverse) t)                                  -- :644
+  tstranspose @_ @_ @x perm (Gpu t) = Gpu (arrMap (knownSTK @x) (transposeBy (Permutation.permToList' perm)) t)   -- :647
+  tsreshape @sh @_ @x sh2 (Gpu t) = Gpu (arrMap (knownSTK @x) (reshapeOuter (shsLength (knownShS @sh)) (shsToList sh2)) t)   -- :650
+  txappend @_ @_ @_ @x (Gpu a) (Gpu b) = Gpu (arrZip (knownSTK @x) (bin c_hh_tsappend) a b)
+  txslice @_ @_ @_ @_ @x i n _ (Gpu t) = Gpu (arrMap (knownSTK @x) (sliceOuter (fromSMayNat' i) (fromSMayNat' n)) t)
+  txreverse @_ @_ @x (Gpu t) = Gpu (arrMap (knownSTK @x) (un1 c_hh_tsreverse) t)
+  txtranspose @_ @_ @x perm (Gpu t) = Gpu (arrMap (knownSTK @x) (transposeBy (Permutation.permToList' perm)) t)
+  txreshape @sh @_ @x sh2 (Gpu t) = Gpu (arrMap (knownSTK @x) (reshapeOuter (ssxLength (knownShX @sh)) (shxToList' sh2)) t)
 
-  -- :661-740: build is the reference's host loop (tbuild1S, :1075-1100); the
-  -- closure may do anything a tensor program does, so it runs once per index
-  tkbuild1 @k @r f = Gpu (stackVals [valueOf @k] [] [scalarVal (dtypeOf @r) (unGpu (f (Gpu (literal i)))) | i <- [0 .. valueOf @k - 1 :: Int]])
-  trbuild1 k f = stackOfUnknown [k] [f (Gpu (literal i)) | i <- [0 .. k - 1]]
-  tsbuild1 @k f = stackOfUnknown [valueOf @k] [f (Gpu (literal i)) | i <- [0 .. valueOf @k - 1 :: Int]]
-  txbuild1 @k f = stackOfUnknown [valueOf @k] [f (Gpu (literal i)) | i <- [0 .. valueOf @k - 1 :: Int]]
+  -- :661-740.  A build or a map whose closure yields SCALARS runs the closure once,
+  -- on lanes (the position variables of the index space, or the array's own
+  -- elements: hh_ix_from_val), and writes the resulting lane out as an array
+  -- (hh_ix_to_val): one fused pass on the device, where Concrete runs one vector
+  -- generate / map (tbuildK :1081-1087, tmap0NS / tzipWith0NS :1748-1759).
+  tkbuild1 @k @r f = Gpu (laneToArr (dtypeOf @r) [valueOf @k] (unGpu (f (Gpu (head (laneVars [valueOf @k]))))))
+  tkbuild @sh @r f =
+    let shm = shsToList (knownShS @sh)
+    in Gpu (laneToArr (dtypeOf @r) shm (unGpu (f (fromList' (laneVars shm)))))
+  trmap0N @_ @_ @r f (Gpu v) = Gpu (laneToArr (dtypeOf @r) (gpuShape v) (unGpu (f (Gpu (arrToLane v)))))
+  trzipWith0N @_ @r f (Gpu u) (Gpu v) = Gpu (laneToArr (dtypeOf @r) (gpuShape u) (unGpu (f (Gpu (arrToLane u)) (Gpu (arrToLane v)))))
+  tsmap0N @_ @_ @r f (Gpu v) = Gpu (laneToArr (dtypeOf @r) (gpuShape v) (unGpu (f (Gpu (arrToLane v)))))      -- :708
+  tszipWith0N @_ @r f (Gpu u) (Gpu v) = Gpu (laneToArr (dtypeOf @r) (gpuShape u) (unGpu (f (Gpu (arrToLane u)) (Gpu (arrToLane v)))))   -- :710-714
+  -- A build whose closure yields ARRAYS is the reference's host loop (tbuild1S,
+  -- :1761-1774): the closure may do anything a tensor program does, so it runs
+  -- once per index, and the results are stacked.
+  trbuild1 @_ @x k f = stackOf (knownSTK @x) [k] [f (Gpu (literal i)) | i <- [0 .. k - 1]]
+  tsbuild1 @k @_ @x f = stackOf (knownSTK @x) [valueOf @k] [f (Gpu (literal i)) | i <- [0 .. valueOf @k - 1 :: Int]]
+  txbuild1 @k @_ @x f = stackOf (knownSTK @x) [valueOf @k] [f (Gpu (literal i)) | i <- [0 .. valueOf @k - 1 :: Int]]
 
   -- :736-760
   tmapAccumLDer _ k _ bftk eftk (GpuFun f) _df _rf acc0 es = mapAccumLGpu k bftk eftk f acc0 es
@@ -346,8 +379,8 @@ literal' :: forall r. GoodScalar r => r -> GpuIx
 literal' x
   | Just Refl <- testEquality (typeRep @r) (typeRep @Double) = GpuIxLit x
   | Just Refl <- testEquality (typeRep @r) (typeRep @Float) = GpuIxLit (realToFrac x)
-  | Just Refl <- testEquality (typeRep @r) (typeRep @Int) = GpuIxLit (fromIntegral x)
-  | Just Refl <- testEquality (typeRep @r) (typeRep @Int64) = GpuIxLit (fromIntegral x)
+  | Just Refl <- testEquality (typeRep @r) (typeRep @Int), abs x < 2 ^ (53 :: Int) = GpuIxLit (fromIntegral x)      -- exact as a Double
+  | Just Refl <- testEquality (typeRep @r) (typeRep @Int64), abs x < 2 ^ (53 :: Int) = GpuIxLit (fromIntegral x)
   | Just Refl <- testEquality (typeRep @r) (typeRep @Bool) = GpuIxLit (if x then 1 else 0)
   | otherwise = GpuIxVal (uploadArr @r [] (VS.singleton x))
 
@@ -363,13 +396,31 @@ mixedSkeleton :: forall sh. ValPtr -> StaticShX sh
 mixedSkeleton v = withShsFromShR (shrOf @(Rank sh) (gpuShape v)) $ \(sh' :: ShS sh') ->
   gcastWith (unsafeCoerceRefl :: MapJust sh' :~: sh) $ ssxFromShX (shxFromShS sh')
 
-scalarsOnly :: SingletonTK x -> FullShapeTK x
-scalarsOnly = \case
+-- | The shape of the elements of an array value: what lies behind the first @n@ (outer) dims of its device arrays.
+elemFTK :: SingletonTK x -> Int -> ArrGpu x -> FullShapeTK x
+elemFTK stk n a = case stk of
   STKScalar -> FTKScalar
-  _ -> nestedArrays "tftk"
+  STKR m x -> FTKR (shrOf (take (fromSNat' m) (drop n (gpuShape (head (arrLeaves x a)))))) (elemFTK x (n + fromSNat' m) a)
+  STKS sh x -> FTKS sh (elemFTK x (n + shsLength sh) a)
+  STKX ssx x -> FTKX (shxOf ssx (take (ssxLength ssx) (drop n (gpuShape (head (arrLeaves x a)))))) (elemFTK x (n + ssxLength ssx) a)
+  STKProduct s1 s2 -> FTKProduct (elemFTK s1 n (fst a)) (elemFTK s2 n (snd a))
 
-nestedArrays :: String -> a
-nestedArrays what = error (what ++ ": arrays of arrays and arrays of products are not represented on this carrier")
+-- | A host array of any element kind onto the device: pairs are unzipped, inner arrays unnested
+-- (their dims join the outer ones), scalars uploaded with the dims collected on the way.
+uploadNested :: SingletonTK x -> [Int] -> Nested.Mixed sh (RepConcrete x) -> ArrGpu x
+uploadNested stk outer a = case stk of
+  STKScalar -> uploadArr (outer ++ drop (length outer) (shxToList' (Nested.mshape a))) (Nested.mtoVector a)
+  STKProduct s1 s2 | Dict <- eltDictRep s1, Dict <- eltDictRep s2 ->
+    let (a1, a2) = Nested.munzip a in (uploadNested s1 outer a1, uploadNested s2 outer a2)
+  STKR _ x | Dict <- eltDictRep x ->
+    let flat = Nested.munNest (Nested.convert (Nested.ConvXX Nested.ConvRX) a)
+    in uploadNested x (shxToList' (Nested.mshape flat)) flat
+  STKS _ x | Dict <- eltDictRep x ->
+    let flat = Nested.munNest (Nested.convert (Nested.ConvXX Nested.ConvSX) a)
+    in uploadNested x (shxToList' (Nested.mshape flat)) flat
+  STKX _ x | Dict <- eltDictRep x ->
+    let flat = Nested.munNest a
+    in uploadNested x (shxToList' (Nested.mshape flat)) flat
 
 shxToList' :: IShX sh -> [Int]
 shxToList' = Foldable.toList
@@ -380,13 +431,19 @@ condArr b (Gpu u) (Gpu v) = Gpu $ out1 $ \ctx o ->
   let cond = replicatePrefix (gpuShape u) (scalarVal 6 b)
   in withForeignPtr cond $ \pc -> withForeignPtr u $ \pu -> withForeignPtr v $ \pv -> c_hh_select ctx pc pu pv o
 
-stackOf :: (RepGpu y ~ ValPtr, RepGpu z ~ ValPtr) => [Int] -> [Gpu y] -> Gpu z
-stackOf shm vs = case vs of
+-- | Array values of one element kind stacked along new outer dims @shm@, device array by device array.
+stackOf :: (RepGpu y ~ ArrGpu x, RepGpu z ~ ArrGpu x) => SingletonTK x -> [Int] -> [Gpu y] -> Gpu z
+stackOf stk shm vs = case vs of
   [] -> error "fromVector: an empty vector carries no element shape"
-  Gpu v0 : _ -> Gpu (stackVals shm (gpuShape v0) (map unGpu vs))
+  _ -> Gpu (arrZipN stk (\leaves -> stackVals shm (gpuShape (head leaves)) leaves) (map unGpu vs))
 
-stackOfUnknown :: (RepGpu y ~ ValPtr, RepGpu z ~ ValPtr) => [Int] -> [Gpu y] -> Gpu z
-stackOfUnknown = stackOf
+-- | A lane written out as an array of shape @shm@ (a literal or a rank-0 value is replicated).
+laneToArr :: CInt -> [Int] -> GpuIx -> ValPtr
+laneToArr dt shm s = out1 $ \ctx o -> withForeignPtr (laneOf dt shm s) $ \p -> c_hh_ix_to_val ctx p o
+
+-- | The elements of an array as a lane over the array's own index space.
+arrToLane :: ValPtr -> GpuIx
+arrToLane v = GpuIxLane (gpuShape v) (outIx $ \ctx o -> withForeignPtr v $ \p -> c_hh_ix_from_val ctx p o)
 
 viaIxR :: (IxROf Gpu m -> IxROf Gpu p) -> [GpuIx] -> [GpuIx]
 viaIxR f vars = ixList (f (fromList' vars))
@@ -419,16 +476,17 @@ mapAccumLGpu k bftk eftk f acc0 es =
 fromListGpu :: forall y k. SNat k -> SingletonTK y -> [Gpu y] -> Gpu (BuildTensorKind k y)
 fromListGpu snat@SNat stk l = case stk of
   STKScalar @r -> Gpu (stackVals [fromSNat' snat] [] (map (scalarVal (dtypeOf @r) . unGpu) l))
-  STKR{} -> stackOf [fromSNat' snat] l
-  STKS{} -> stackOf [fromSNat' snat] l
-  STKX{} -> stackOf [fromSNat' snat] l
+  STKR _ x -> stackOf x [fromSNat' snat] l
+  STKS _ x -> stackOf x [fromSNat' snat] l
+  STKX _ x -> stackOf x [fromSNat' snat] l
   STKProduct s1 s2 ->
     tpair (fromListGpu snat s1 (map tproject1 l)) (fromListGpu snat s2 (map tproject2 l))
 
 -- * ConvertTensor (ConvertTensor.hs:25-236, OpsConcrete.hs:777-904): arrays hold
 -- their shape at run time, so a conversion between array kinds is the identity
 -- on the device value, checked against the shape the target type names; a
--- scalar and a rank-0 array are the two forms of 'GpuIx'.
+-- scalar and a rank-0 array are the two forms of 'GpuIx'; zip / unzip / nest /
+-- unnest relate two types of one representation ('ArrGpu').
 
 instance ConvertTensor Gpu where
   tconvert c astk a = convertGpu c astk a
@@ -440,24 +498,26 @@ instance ConvertTensor Gpu where
   rfromS (Gpu v) = Gpu v
   rfromX (Gpu v) = Gpu v
   sfromK @r (Gpu s) = Gpu (scalarVal (dtypeOf @r) s)
-  sfromR @sh (Gpu v) = Gpu (checkedShape (shsToList (knownShS @sh)) v)
-  sfromX @sh (Gpu v) = Gpu (checkedShape (shsToList (knownShS @sh)) v)
+  sfromR @sh @x (Gpu v) = Gpu (arrMap (knownSTK @x) (checkedOuter (shsToList (knownShS @sh))) v)
+  sfromX @sh @_ @x (Gpu v) = Gpu (arrMap (knownSTK @x) (checkedOuter (shsToList (knownShS @sh))) v)
   xfromK @r (Gpu s) = Gpu (scalarVal (dtypeOf @r) s)
   xfromR (Gpu v) = Gpu v
   xfromS (Gpu v) = Gpu v
 
-  rzip _ = nestedArrays "rzip"
-  runzip _ = nestedArrays "runzip"
-  szip _ = nestedArrays "szip"
-  sunzip _ = nestedArrays "sunzip"
-  xzip _ = nestedArrays "xzip"
-  xunzip _ = nestedArrays "xunzip"
-  xnestR _ _ = nestedArrays "xnestR"
-  xnestS _ _ = nestedArrays "xnestS"
-  xnest _ _ = nestedArrays "xnest"
-  xunNestR _ = nestedArrays "xunNestR"
-  xunNestS _ = nestedArrays "xunNestS"
-  xunNest _ = nestedArrays "xunNest"
+  -- :821-876.  An array of pairs IS the pair of arrays, an array of arrays IS the flat array
+  -- ('ArrGpu'): the two sides of each of these have one representation, and no data moves.
+  rzip (Gpu p) = Gpu p
+  runzip (Gpu p) = Gpu p
+  szip (Gpu p) = Gpu p
+  sunzip (Gpu p) = Gpu p
+  xzip (Gpu p) = Gpu p
+  xunzip (Gpu p) = Gpu p
+  xnestR _ (Gpu a) = Gpu a
+  xnestS _ (Gpu a) = Gpu a
+  xnest _ (Gpu a) = Gpu a
+  xunNestR (Gpu a) = Gpu a
+  xunNestS (Gpu a) = Gpu a
+  xunNest (Gpu a) = Gpu a
 
   tpairConv = tpair
   tunpairConv = tunpair
@@ -466,6 +526,12 @@ checkedShape :: [Int] -> ValPtr -> ValPtr
 checkedShape want v
   | gpuShape v == want = v
   | otherwise = error ("the array has shape " ++ show (gpuShape v) ++ ", the shaped type names " ++ show want)
+
+-- | The same check on the outer dims of a device array that may carry inner dims behind them.
+checkedOuter :: [Int] -> ValPtr -> ValPtr
+checkedOuter want v
+  | take (length want) (gpuShape v) == want = v
+  | otherwise = error ("the array has outer shape " ++ show (take (length want) (gpuShape v)) ++ ", the shaped type names " ++ show want)
 
 -- | The universal conversion, by recursion on the recipe (Conversion.hs:37-73).
 convertGpu :: TKConversion a b -> SingletonTK a -> Gpu a -> Gpu b
@@ -478,18 +544,45 @@ convertGpu c0 astk a = case c0 of
   ConvXS -> Gpu (unGpu a)
   ConvXS' (FTKS sh _) -> Gpu (checkedShape (shsToList sh) (unGpu a))
   ConvXX' (FTKX sh _) -> Gpu (checkedShape (shxToList' sh) (unGpu a))
-  ConvRR c | Just Refl <- isIdentity c -> a
-  ConvSS c | Just Refl <- isIdentity c -> a
-  ConvXX c | Just Refl <- isIdentity c -> a
+  -- a conversion of the elements: arrays of arrays and of pairs share their elements' representation,
+  -- so only the shape checks inside the recipe are left of it
+  ConvRR c | STKR _ x <- astk -> convertElems c x a
+  ConvSS c | STKS _ x <- astk -> convertElems c x a
+  ConvXX c | STKX _ x <- astk -> convertElems c x a
+  ConvNest _ -> Gpu (unGpu a)
+  ConvUnnest -> Gpu (unGpu a)
+  ConvZip _ _ -> Gpu (unGpu a)
+  ConvUnzip _ _ -> Gpu (unGpu a)
   ConvT2 c1 c2 | STKProduct s1 s2 <- astk ->
     tpair (convertGpu c1 s1 (tproject1 a)) (convertGpu c2 s2 (tproject2 a))
   Conv0X STKScalar | STKScalar @r <- astk -> Gpu (scalarVal (dtypeOf @r) (unGpu a))
   ConvX0 | STKX _ STKScalar <- astk -> Gpu (valScalar (unGpu a))
-  _ -> nestedArrays "tconvert"
  where
-  isIdentity :: TKConversion x y -> Maybe (x :~: y)
-  isIdentity ConvId = Just Refl
-  isIdentity _ = Nothing
+  -- the element conversions that change the representation are the two between a scalar and a
+  -- rank-0 array (Conv0X / ConvX0): inside an array both are a device array already
+  convertElems :: forall x y f g. (RepGpu (f x) ~ ArrGpu x, RepGpu (g y) ~ ArrGpu y)
+               => TKConversion x y -> SingletonTK x -> Gpu (f x) -> Gpu (g y)
+  convertElems c x (Gpu v) = Gpu (elemsAs c x v)
+  elemsAs :: TKConversion x y -> SingletonTK x -> ArrGpu x -> ArrGpu y
+  elemsAs c x v = case c of
+    ConvId -> v
+    ConvCmp c2 c1 -> elemsAs c2 (convertSTK c1 x) (elemsAs c1 x v)
+    ConvRX -> v
+    ConvSX -> v
+    ConvXR _ -> v
+    ConvXS -> v
+    ConvXS' _ -> v
+    ConvXX' _ -> v
+    ConvRR c' | STKR _ x' <- x -> elemsAs c' x' v
+    ConvSS c' | STKS _ x' <- x -> elemsAs c' x' v
+    ConvXX c' | STKX _ x' <- x -> elemsAs c' x' v
+    ConvT2 c1 c2 | STKProduct s1 s2 <- x -> (elemsAs c1 s1 (fst v), elemsAs c2 s2 (snd v))
+    Conv0X _ -> v
+    ConvX0 -> v
+    ConvNest _ -> v
+    ConvUnnest -> v
+    ConvZip _ _ -> v
+    ConvUnzip _ _ -> v
 
 -- * Interpreting a gradient artifact at the carrier
 

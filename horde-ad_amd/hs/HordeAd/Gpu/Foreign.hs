@@ -20,6 +20,7 @@ module HordeAd.Gpu.Foreign
   , c_hh_ix_var, c_hh_ix_const, c_hh_ix_lift, c_hh_ix_op1, c_hh_ix_op2
   , c_hh_ix_compare, c_hh_ix_select, c_hh_ix_convert, c_hh_ix_index0
   , c_hh_ix_argminmax, c_hh_tsgather, c_hh_tsscatter
+  , c_hh_ix_from_val, c_hh_ix_to_val, c_hh_tconvert, c_hh_tprimalPart
   , p_hh_free, p_hh_ix_free
   ) where
 
@@ -92,6 +93,12 @@ foreign import ccall safe "hh_ix_select" c_hh_ix_select :: Ptr Ctx -> Ptr Ix -> 
 foreign import ccall safe "hh_ix_convert" c_hh_ix_convert :: Ptr Ctx -> Ptr Ix -> CInt -> CInt -> Ptr (Ptr Ix) -> IO CInt
 foreign import ccall safe "hh_ix_index0" c_hh_ix_index0 :: Ptr Ctx -> Ptr Val -> CInt -> Ptr (Ptr Ix) -> Ptr (Ptr Ix) -> IO CInt
 foreign import ccall safe "hh_ix_argminmax" c_hh_ix_argminmax :: Ptr Ctx -> Ptr Val -> CInt -> Ptr (Ptr Ix) -> CInt -> Ptr (Ptr Ix) -> IO CInt
+-- tsmap0N / tszipWith0N / tkbuild: an array as a lane over its own index space, and a lane written out as an array
+foreign import ccall safe "hh_ix_from_val" c_hh_ix_from_val :: Ptr Ctx -> Ptr Val -> Ptr (Ptr Ix) -> IO CInt
+foreign import ccall safe "hh_ix_to_val" c_hh_ix_to_val :: Ptr Ctx -> Ptr Ix -> Ptr (Ptr Val) -> IO CInt
+-- ConvertTensor: the checked identity (conversion code of enum hh_conversion, the shape the target type names)
+foreign import ccall safe "hh_tconvert" c_hh_tconvert :: Ptr Ctx -> CInt -> Ptr Val -> CInt -> Ptr Int64 -> Ptr (Ptr Val) -> IO CInt
+foreign import ccall safe "hh_tprimalPart" c_hh_tprimalPart :: Ptr Ctx -> Ptr Val -> Ptr (Ptr Val) -> IO CInt
 foreign import ccall safe "hh_tsgather" c_hh_tsgather
   :: Ptr Ctx -> Ptr Val -> CInt -> Ptr Int64 -> CInt -> Ptr (Ptr Ix) -> Ptr (Ptr Val) -> IO CInt
 foreign import ccall safe "hh_tsscatter" c_hh_tsscatter

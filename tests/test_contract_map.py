@@ -143,14 +143,14 @@ def test_host_rewrites_pooling_layers_onto_contract_map():
 
 # ---- hgpu_contract_operands: operands that are unevaluated expressions ------
 
-def pooled_cotangent(ctx, rng, B, Co, H, Wd, dtype):
+def pooled_cotangent(ctx, rng, B, Co, H, Wd, dtype, arg_range=(0, 4)):
     """The cotangent of relu + 2x2 max-pooling as an expression over the refined space
     [B, Co, H/2, 2, W/2, 2]: (which == arg ? dpool : 0) * (mask ? 0 : 1).  Returns
     (inputs, program, slot, merged shape, the same as a numpy array)."""
     O2, CMP = capi.OP2, capi.CMP
     H2, W2 = H // 2, Wd // 2
     dpool = rng.uniform(-1, 1, (B, Co, H2, W2)).astype(dtype)
-    arg = rng.integers(0, 4, (B, Co, H2, W2)).astype(np.int64)
+    arg = rng.integers(arg_range[0], arg_range[1], (B, Co, H2, W2)).astype(np.int64)
     mask = rng.integers(0, 2, (B, Co, H, Wd)).astype(bool)
     cz = np.zeros((B, Co, H2, 2, W2, 2), dtype)
     for p in range(2):
@@ -169,7 +169,7 @@ def pooled_cotangent(ctx, rng, B, Co, H, Wd, dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("B,Ci,Co,H,Wd,k,dtype,fused", [(300, 16, 16, 14, 14, 5, np.float64, True), (300, 16, 16, 14, 14, 5, np.float32, None),
-                                                        (280, 1, 16, 28, 28, 5, np.float64, False), (5, 2, 4, 8, 8, 3, np.float64, False)])
+                                                        (280, 1, 16, 28, 28, 5, np.float64, True), (5, 2, 4, 8, 8, 3, np.float64, False)])
 def test_gradients_of_a_convolution_from_an_unevaluated_cotangent(gpu, B, Ci, Co, H, Wd, k, dtype, fused):
     """Bias, kernel and input gradient of a convolution layer read the pooled
     cotangent through arg-maxima and relu mask while staging (`fused`: a kernel
@@ -220,6 +220,35 @@ def test_gradients_of_a_convolution_from_an_unevaluated_cotangent(gpu, B, Ci, Co
     wz = np.lib.stride_tricks.sliding_window_view(czp, (k, k), axis=(2, 3))
     # (whether a kernel takes this one unevaluated depends on how many loads a staging pass of the extended footprint needs)
     assert close(got, np.einsum("bcyxuv,ciuv->biyx", wz.astype(np.float64), ker[:, :, ::-1, ::-1].astype(np.float64))), labels
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,Ci,Co,H,Wd,k,dtype,arg_range", [(280, 1, 16, 28, 28, 5, np.float64, (0, 4)), (130, 1, 16, 28, 28, 5, np.float64, (-1, 6)),
+                                                            (2000, 1, 10, 12, 20, 3, np.float32, (0, 4)), (3000, 2, 7, 16, 8, 3, np.float64, (-2, 4))])
+def test_kernel_gradient_of_a_first_layer_from_one_term_per_window(gpu, B, Ci, Co, H, Wd, k, dtype, arg_range):
+    """The cotangent of relu + max-pooling has one non-zero per 2x2 window, at the window's
+    argument.  With a few rows on the other side (the kernel gradient of a layer of few input
+    channels) the contraction takes one term per window: the `onehot_contract` kernel.  Against
+    numpy; arguments outside 0 .. 3 (no term at all) included."""
+    rng = np.random.default_rng(18)
+    ins, prog, slot, M, cz = pooled_cotangent(gpu, rng, B, Co, H, Wd, dtype, arg_range)
+    x = rng.uniform(-1, 1, (B, Ci, H + k - 1, Wd + k - 1)).astype(dtype)
+    Hp, Wp = H + k - 1, Wd + k - 1
+    sh = [Co, Ci, k, k, B, H, Wd]
+    view = (sh, [H * Wd, 0, 0, 0, Co * H * Wd, Wd, 1], 0)
+    xst = [0, Hp * Wp, Wp, 1, Ci * Hp * Wp, Wp, 1]
+    win = np.lib.stride_tricks.sliding_window_view(x, (k, k), axis=(2, 3))[:, :, :H, :Wd]
+    want = np.einsum("bohw,bihwpq->oipq", cz.astype(np.float64), win.astype(np.float64))
+    tol = 1e-10 if dtype == np.float64 else 1e-5
+    for expression_first in (True, False):
+        a_op = gpu.operand(ins, prog, slot, M, view)
+        gx = gpu.upload(x).as_strided(sh, xst, 0)
+        gpu.profile(2)
+        got = (gpu.contract_operands(a_op, gx, 4, fused_only=True) if expression_first else gpu.contract_operands(gx, a_op, 4, fused_only=True)).numpy()
+        labels = list(gpu.profile_report())
+        gpu.profile(0)
+        assert any(l.startswith("onehot_contract") for l in labels), labels
+        assert got.shape == want.shape and np.max(np.abs(got - want)) <= tol * np.max(np.abs(want)), (expression_first, np.max(np.abs(got - want)))
 
 
 def test_host_rewrites_gradients_onto_contract_operands():

@@ -542,7 +542,8 @@ def test_scatter_into_a_handful_of_cells_is_bounded(both, gpu):
     """A million positions into eight cells (a table's cotangent): runs of 125,000 are added
     in segments of 256 by separate lanes, not by one lane front to back.  Exact for
     integers; floats within the tolerance of a reordered sum; and the call, sort included,
-    takes milliseconds, not seconds."""
+    takes milliseconds, not seconds.  (A sum of 125,000 terms added front to back in single precision,
+    which is what the reference's order gives, is itself some 1e-5 off: both are held to the sum in double.)"""
     import time
     M = 1 << 20
     cells = RNG.integers(-1, 8, M).astype(np.int64)          # some out of bounds
@@ -550,11 +551,20 @@ def test_scatter_into_a_handful_of_cells_is_bounded(both, gpu):
         src = both.upload(rnd((M, n) if n > 1 else (M,), dt))
         ix = [both.upload(cells)]
         res = both.scatter_add(src, ix, 1, [8])
-        assert_same(res, tol, (dt, n))
-        got = res.numpy()[0]
-        want = np.zeros(got.shape, np.float64)      # the independent sum in double, whatever the element type
-        np.add.at(want, cells[(cells >= 0) & (cells < 8)], src.numpy()[1][(cells >= 0) & (cells < 8)].astype(np.float64))
-        np.testing.assert_allclose(got, want, rtol=max(tol, 1e-12) * 100, atol=0.5 if dt == np.float32 else 1e-7)   # 125,000 terms of size one per cell
+        got, seq = res.numpy()                              # the device; the checker, which adds front to back in the element type
+        inb = (cells >= 0) & (cells < 8)
+        x64 = src.numpy()[1].astype(np.float64)
+        want = np.zeros(got.shape, np.float64)              # the independent sum, in double whatever the element type
+        mass = np.zeros(got.shape, np.float64)
+        np.add.at(want, cells[inb], x64[inb])
+        np.add.at(mass, cells[inb], np.abs(x64[inb]))
+        if tol == 0.0:
+            assert np.array_equal(got, seq) and np.array_equal(got, want.astype(dt)), (dt, n)
+        else:
+            # 125,000 terms per cell: both orders are held to the exact sum, by the magnitudes that went into a cell
+            eps = float(np.finfo(dt).eps)
+            assert np.all(np.abs(got - want) <= 8 * eps * mass), (dt, n, np.max(np.abs(got - want) / mass))
+            assert np.all(np.abs(seq - want) <= 600 * eps * mass), (dt, n)
         dev = src.arrays[0]
         gix = [ix[0].arrays[0]]
         gpu.sync()
