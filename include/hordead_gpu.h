@@ -257,6 +257,11 @@ int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, in
  * hgpu_contract). */
 int hgpu_fused_map_dimsum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog,
                           int n_out, const int* out_slots, hgpu_array** outs, int sum_slot, int keep_dim, hgpu_array** sum);
+/* tssum0 of such a program's result (OpsConcrete.hs:229-230), evaluated on the
+ * fly: the result itself is never written.  Inputs must be dense or one
+ * broadcast element (else HGPU_ERR_UNSUPPORTED: write the result out and sum
+ * that).  Accumulates in double / int64 in an order fixed by the size. */
+int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot, hgpu_array** out);
 /* The first extremum of such a program's result along its trailing n_reduce
  * dims (taken together, row-major), evaluated on the fly: the result itself is
  * never written.  values / indices get the leading dims' shape; an index
@@ -264,11 +269,6 @@ int hgpu_fused_map_dimsum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, 
  * `maxPool2dUnpaddedS (reluS (conv + bias))` (External/CommonShapedOps.hs:
  * 241-260) reads the convolution once and writes only the pooled maxima and
  * their arguments. */
-/* tssum0 of such a program's result (OpsConcrete.hs:229-230), evaluated on the
- * fly: the result itself is never written.  Inputs must be dense or one
- * broadcast element (else HGPU_ERR_UNSUPPORTED: write the result out and sum
- * that).  Accumulates in double / int64 in an order fixed by the size. */
-int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot, hgpu_array** out);
 int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int slot, int n_reduce,
                         int want_max, hgpu_array** values, hgpu_array** indices);
 

@@ -31,8 +31,10 @@
 //     once (ox-arrays' own blocking is not known here; the parity tolerance
 //     covers the difference).
 //
-// Parity status of each function against the reference's own tests is listed
-// in tests/test_oracle_golden.py.
+// What pins each function: numpy and brute force in tests/test_oracle_numpy.py,
+// the reference's own known answers in tests/test_reference_kats.py,
+// tests/test_highrank_kats.py and tests/test_fold_kats.py (vectors under
+// tests/golden/).
 #include <algorithm>
 #include <cmath>
 #include <cstdint>

@@ -148,7 +148,7 @@ def test_data_dependent_indices_gpu(host_gpu):
     data_dependent_indices(host_gpu)
 
 
-def test_convert_tensor_is_a_checked_identity(host_cpu):
+def convert_tensor_is_a_checked_identity(host_cpu):
     """ConvertTensor on this carrier (ConvertTensor.hs:25-236, OpsConcrete.hs:777-904):
     arrays carry their shape at run time, so kfromS / sfromK / sfromR / rfromS / sfromX /
     xfromS / nest / unnest hand back the same data and the same dual part; the shape
@@ -179,6 +179,15 @@ def test_convert_tensor_is_a_checked_identity(host_cpu):
     loss = (y * y).ssum0().tconvert("kfromS").tconvert("sfromK")
     (g,) = host_cpu.grad(loss, [q])
     assert np.allclose(g.numpy(), 2 * x, rtol=1e-13, atol=0)
+
+
+def test_convert_tensor_is_a_checked_identity(host_cpu):
+    convert_tensor_is_a_checked_identity(host_cpu)
+
+
+@pytest.mark.gpu
+def test_convert_tensor_is_a_checked_identity_gpu(host_gpu):
+    convert_tensor_is_a_checked_identity(host_gpu)
 
 
 def test_adjoint_law_cpu(host_cpu):
@@ -341,8 +350,7 @@ def test_value_at_own_extremum_gpu(host_gpu):
     value_at_own_extremum(host_gpu)
 
 
-def test_ranked_and_mixed_methods_are_the_shaped_ones(host_cpu):
-    host = host_cpu
+def ranked_and_mixed_methods_are_the_shaped_ones(host):
     """Ops.hs:297-1255 gives every operation a ranked (tr*), a shaped (ts*) and a
     mixed (tx*) method; the ABI takes shapes at run time, so all three bind to
     one entry point.  The twins give the same arrays, through a gather with an
@@ -363,3 +371,12 @@ def test_ranked_and_mixed_methods_are_the_shaped_ones(host_cpu):
         assert np.array_equal(sc.numpy(), np.array([a[1, 0], 0, a[2, 2], 0, a[3, 4]]))
     assert np.array_equal(A.rtr().numpy(), a.T) and np.array_equal(A.rmaxIndex().numpy(), a.argmax(-1))
     assert np.array_equal(host.rrepl((2, 2), 1.5).numpy(), np.full((2, 2), 1.5))
+
+
+def test_ranked_and_mixed_methods_are_the_shaped_ones(host_cpu):
+    ranked_and_mixed_methods_are_the_shaped_ones(host_cpu)
+
+
+@pytest.mark.gpu
+def test_ranked_and_mixed_methods_are_the_shaped_ones_gpu(host_gpu):
+    ranked_and_mixed_methods_are_the_shaped_ones(host_gpu)

@@ -7,7 +7,7 @@ The programs are drawn from a fixed seed."""
 import numpy as np
 import pytest
 
-from conftest import capi, entry, pkg
+from conftest import capi, entry, pkg, record_error
 
 H = pkg.hostapi
 
@@ -18,11 +18,13 @@ def factorizations(n):
     return [(a, n // a) for a in range(2, n) if n % a == 0]
 
 
-def random_program(seed, extended=False, big=False):
+def random_program(seed, extended=False, big=False, maps=False):
     """A list of steps (name, args) over a stack of values; generated once, replayed on both hosts.
     extended: also dense layers (one or two matrix products, bias, tanh) and sums over all dims but one.
     big: a [32..96, 256..768] matrix to start from and layers 16 to 64 wide, so that the device takes the kernels it
-    compiles for shapes (and holds their launches back) in the middle of other work."""
+    compiles for shapes (and holds their launches back) in the middle of other work.
+    maps: also maps and zips of scalar closures (tsmap0N / tszipWith0N: the closure runs once, on lane values) and a
+    build from the position variables (tkbuild).  (A flag of its own: the programs of the other seeds stay what they were.)"""
     rng = np.random.default_rng(seed)
     shapes = [tuple(int(x) for x in rng.integers(2, 7, int(rng.integers(2, 4))))]
     if big:
@@ -35,6 +37,8 @@ def random_program(seed, extended=False, big=False):
         kinds = ["unary", "binary", "transpose", "split", "merge", "slice", "append", "sum", "scale", "bias", "pool"]
         if extended:
             kinds += ["layer", "layer", "keepdim"]
+        if maps:
+            kinds += ["map0N", "map0N", "zip0N", "kbuild"]
         kind = rng.choice(kinds)
         if kind == "unary":
             steps.append(("unary", i, str(rng.choice(["sin", "tanh", "cos"]))))
@@ -95,6 +99,16 @@ def random_program(seed, extended=False, big=False):
             d = int(rng.integers(0, len(sh)))
             steps.append(("keepdim", i, d))
             stack.append((sh[d],))
+        elif kind == "map0N":
+            steps.append(("map0N", i, float(rng.uniform(-0.5, 0.5))))
+            stack.append(sh)
+        elif kind == "zip0N":
+            same = [j for j, s in enumerate(stack) if s == sh]
+            steps.append(("zip0N", i, int(rng.choice(same))))
+            stack.append(sh)
+        elif kind == "kbuild":
+            steps.append(("kbuild", i, float(rng.uniform(0.5, 2.0))))
+            stack.append(sh)
     return shapes[0], steps, stack
 
 
@@ -136,6 +150,15 @@ def run(host, x0, steps):
             d, rk = st[2], len(v.shape)
             perm = [q for q in range(rk) if q != d] + [d]
             vals.append(v.stranspose(perm).ssumN(rk - 1) if rk > 1 else v)
+        elif st[0] == "map0N":     # a leaky relu written as the scalar closure of a map: ifH (x <=. c) (x / 4) (sin x)
+            c = st[2]
+            vals.append(v.smap0N(lambda x: H.ifH(x.leq(c), x * 0.25, x.op1("sin"))) * v)
+        elif st[0] == "zip0N":     # zipWith (\p q -> p * q + ifH (p <. q) p q), times a differentiable factor
+            vals.append(v.szipWith0N(lambda a, b: a * b + H.ifH(a.lt(b), a, b), vals[st[2]]) + v)
+        elif st[0] == "kbuild":    # a build from the position variables: the sum of the indices, scaled, as the element type
+            scale, dt = st[2], v.dtype
+            ramp = host.kbuild(v.shape, lambda *ix: (sum(ix[1:], ix[0]) if len(ix) > 1 else ix[0]).convert(dt) * scale)
+            vals.append(ramp * v)
         elif st[0] == "pool":      # 2x2 max over the last two dims: window gather, merged reshape, kargMax, gather
             sh = v.shape
             lead, h2, w2 = list(sh[:-2]), sh[-2] // 2, sh[-1] // 2
@@ -208,6 +231,30 @@ def test_random_program_with_layers_at_kernel_sizes_matches_the_checker(seed):
     assert np.allclose(gpu[2], cpu[2], rtol=1e-9, atol=1e-9 * max(1.0, float(np.max(np.abs(cpu[2]))))), steps
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_program_with_maps_and_builds_matches_the_checker(seed):
+    """Programs that also map and zip scalar closures over arrays and build arrays from index closures."""
+    shape, steps, _ = random_program(seed, extended=True, maps=True, big=seed >= 16)
+    x0 = np.random.default_rng(2000 + seed).uniform(-1, 1, shape)
+    cpu = run(reference_host(), x0, steps)
+    gpu = run(H.Host(), x0, steps)
+    for a, b in zip(gpu[0], cpu[0]):
+        assert a.shape == b.shape
+        assert np.allclose(a, b, rtol=1e-10, atol=1e-10 * max(1.0, float(np.max(np.abs(b))) if b.size else 1.0)), steps
+    assert np.isclose(gpu[1], cpu[1], rtol=1e-10), steps
+    assert np.allclose(gpu[2], cpu[2], rtol=1e-9, atol=1e-9 * max(1.0, float(np.max(np.abs(cpu[2]))))), steps
+
+
+# Single precision, relative to the largest magnitude of each result.  Measured over the eight programs
+# (HORDEAD_TEST_ERRORS): values, loss and gradient; the bounds are those figures times a small factor.
+VALUE_TOL, LOSS_TOL, GRAD_TOL = 2e-4, 1e-3, 1e-3
+
+
+def worst(a, b):
+    """The largest difference of two results relative to the largest magnitude of the reference."""
+    return float(np.max(np.abs(a.astype(np.float64) - b))) / max(1.0, float(np.max(np.abs(b)))) if b.size else 0.0
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_random_program_with_layers_single_precision(seed):
     """The same in fp32 (tolerances relative to the largest magnitude of each result: the programs chain up to a
@@ -218,6 +265,9 @@ def test_random_program_with_layers_single_precision(seed):
     gpu = run(H.Host(), x0, steps)
     for a, b in zip(gpu[0], cpu[0]):
         assert a.shape == b.shape and a.dtype == b.dtype
-        assert np.allclose(a, b, rtol=2e-4, atol=2e-4 * max(1.0, float(np.max(np.abs(b))) if b.size else 1.0)), steps
-    assert np.isclose(gpu[1], cpu[1], rtol=1e-3), steps
-    assert np.allclose(gpu[2], cpu[2], rtol=1e-3, atol=1e-3 * max(1.0, float(np.max(np.abs(cpu[2]))))), steps
+        record_error(("value", seed), worst(a, b), VALUE_TOL)
+        assert worst(a, b) <= VALUE_TOL, steps
+    record_error(("loss", seed), abs(float(gpu[1]) - float(cpu[1])) / max(1.0, abs(float(cpu[1]))), LOSS_TOL)
+    assert abs(float(gpu[1]) - float(cpu[1])) <= LOSS_TOL * max(1.0, abs(float(cpu[1]))), steps
+    record_error(("gradient", seed), worst(gpu[2], cpu[2]), GRAD_TOL)
+    assert worst(gpu[2], cpu[2]) <= GRAD_TOL, steps

@@ -9,8 +9,8 @@ from conftest import capi, entry
 import test_host_random_programs as tp
 
 
-def check(seed, extended):
-    shape, steps, _ = tp.random_program(seed, extended=extended)
+def check(seed, extended, maps=False):
+    shape, steps, _ = tp.random_program(seed, extended=extended, maps=maps)
     x0 = np.random.default_rng(1000 + seed).uniform(-1, 1, shape)
     want = tp.run(tp.reference_host(), x0, steps)
     for table in ("get_api", "get_api_fused"):
@@ -35,6 +35,13 @@ def test_random_program_matches_every_operation_at_once(seed):
 @pytest.mark.parametrize("seed", [1, 57, 251] + list(range(2, 40)))
 def test_random_program_with_layers_matches_every_operation_at_once(seed):
     check(seed, True)
+
+
+# Programs that also map and zip scalar closures over arrays (the closure runs once, on lane values, and its
+# arithmetic joins the deferred elementwise program) and build arrays from the position variables.
+@pytest.mark.parametrize("seed", range(40))
+def test_random_program_with_maps_and_builds_matches_every_operation_at_once(seed):
+    check(seed, True, maps=True)
 
 
 @pytest.mark.parametrize("seed", range(12))
