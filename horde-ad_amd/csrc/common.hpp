@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -193,6 +194,8 @@ struct LaunchGuard {
     c->launch_mu.lock();
     (void)hipSetDevice(c->device);
     if (c->dq_pending) flush_deferred_locked(c);   // what was held back goes first: stream order is program order
+    static const bool trace = getenv("HORDEAD_GPU_TRACE_LAUNCHES") != nullptr;   // one line per launch, in program order
+    if (trace && name) fprintf(stderr, "hordead_gpu: launch %s\n", name);
     if (c->profiling && name && !c->cap) {
       hgpu_ctx::ProfRec r{name, nullptr, nullptr, bytes, flops};
       if (hipEventCreate(&r.a) == hipSuccess && hipEventCreate(&r.b) == hipSuccess) {

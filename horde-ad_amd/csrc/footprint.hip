@@ -1045,6 +1045,7 @@ namespace hg {
 
 // gemm.hip: out[i] = sum over the `parts` partial outputs of part[s * n + i], in a fixed order.
 int sum_partials(hgpu_ctx* ctx, int dtype, int64_t n, int parts, const void* part, void* out);
+int sum_partials_split(hgpu_ctx* ctx, int dtype, int64_t n1, int64_t n2, int parts, const void* part, void* out1, void* out2);
 
 int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const void* pa, const void* pb, hgpu_array* out, bool* handled,
                           const void* va_, const void* vb_);
@@ -2270,7 +2271,7 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   static const int knob_batch = getenv("HORDEAD_ONEHOT_BATCH") ? atoi(getenv("HORDEAD_ONEHOT_BATCH")) : 16;
   const int RB = 4;       // rows of the result added up per round at the end
   const int MA = MR + 1;  // the rows, and the plain sum of the expression's values per column
-  s << "extern \"C\" __global__ void __launch_bounds__(256) " << kname << "(const T* __restrict__ X, Ins ins, T* __restrict__ part, T* __restrict__ psum) {\n";
+  s << "extern \"C\" __global__ void __launch_bounds__(256) " << kname << "(const T* __restrict__ X, Ins ins, T* __restrict__ part) {\n";
   s << "  __shared__ T xs[" << span << "];\n  __shared__ T red[" << RB * 256 << "];\n";
   s << "  const int tid = threadIdx.x, col = tid / " << TPC << ", li = tid % " << TPC << ";\n  const int cq = col < " << NC << " ? col : 0;\n";
   for (int i = 0; i < v.n_in; ++i) {
@@ -2326,8 +2327,9 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   s << "    for (int o = tid; o < " << RB * NC << "; o += 256) {\n      const int m = m0 + o / " << NC << ", c = o % " << NC << ";\n";
   s << "      if (m < " << MA << ") {\n        T sum = T(0);\n";
   s << "        for (int l = 0; l < " << TPC << "; ++l) sum += red[(m - m0) * 256 + c * " << TPC << " + l];\n";
-  s << "        if (m < " << MR << ") part[(i64)blockIdx.x * " << (int64_t)nelem(out) << "ll + kRowC[m] + kColC[c]] = sum;\n";
-  s << "        else psum[(i64)blockIdx.x * " << NC << " + c] = sum;\n      }\n    }\n  }\n}\n";
+  // a block's partial result: the rows of the product, then the columns' plain sums
+  s << "        if (m < " << MR << ") part[(i64)blockIdx.x * " << (int64_t)nelem(out) + NC << "ll + kRowC[m] + kColC[c]] = sum;\n";
+  s << "        else part[(i64)blockIdx.x * " << (int64_t)nelem(out) + NC << "ll + " << (int64_t)nelem(out) << " + c] = sum;\n      }\n    }\n  }\n}\n";
   std::string src = s.str();
   auto& cache = cache_of(ctx);
   auto it = cache.find(src);
@@ -2356,10 +2358,9 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   if (rc) { hgpu_release(colsum); return rc; }
   const char* xp = (const char*)data_ptr(x) + lo * es;
   void* pdst = part->ptr;
-  void* sdst = (char*)part->ptr + (size_t)(out_n * grid) * es;
   std::vector<const void*> ia;
   for (int i = 0; i < v.n_in; ++i) ia.push_back(data_ptr(v.in[i]));
-  void* args[] = {(void*)&xp, (void*)ia.data(), (void*)&pdst, (void*)&sdst};
+  void* args[] = {(void*)&xp, (void*)ia.data(), (void*)&pdst};
   {
     double bytes = (double)nch * span * es;
     for (int i = 0; i < v.n_in; ++i) {
@@ -2379,8 +2380,7 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
     hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
     if (e != hipSuccess) { buffer_release(part); hgpu_release(colsum); return check_hip(ctx, e, "onehot_contract launch"); }
   }
-  rc = hg::sum_partials(ctx, v.dtype, out_n, (int)grid, part->ptr, data_ptr(out));
-  if (!rc) rc = hg::sum_partials(ctx, v.dtype, NC, (int)grid, sdst, data_ptr(colsum));
+  rc = hg::sum_partials_split(ctx, v.dtype, out_n, NC, (int)grid, part->ptr, data_ptr(out), data_ptr(colsum));
   buffer_release(part);
   if (rc) { hgpu_release(colsum); return rc; }
   remember_sum(ctx, v, colk, colsum);

@@ -634,10 +634,16 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   if (n == 0) { *out = o; return HGPU_OK; }
   const bool fp = dtype_is_float(odt);
   const char* acc = fp ? "double" : "i64";
-  const unsigned grid = grid_for((n + vec - 1) / vec, 256, ctx->num_cu * 8);
+  // Few elements: one block of 1024 threads sums them and writes the result, no second launch.
+  const bool single = (n + vec - 1) / vec <= 8192;
+  const int NT = single ? 1024 : 256;
+  const unsigned grid = single ? 1u : grid_for((n + vec - 1) / vec, 256, ctx->num_cu * 8);
   hgpu_buffer* part = nullptr;
-  rc = buffer_alloc(ctx, (size_t)grid * 8, &part);
-  if (rc) { hgpu_release(o); return rc; }
+  if (!single) {
+    rc = buffer_alloc(ctx, (size_t)grid * 8, &part);
+    if (rc) { hgpu_release(o); return rc; }
+  }
+  auto drop_part = [&] { if (part) buffer_release(part); };
 
   std::ostringstream s;
   s << kPrelude;
@@ -650,16 +656,17 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
        "    unsigned long long w = ((unsigned long long)hi << 32) | lo;\n"
        "    v += *reinterpret_cast<ACC*>(&w);\n"
        "  }\n  return v;\n}\n";
-  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_sum(i64 n";
+  s << "extern \"C\" __global__ void __launch_bounds__(" << NT << ") fused_sum(i64 n";
   for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
-  s << ", ACC* __restrict__ part) {\n";
-  s << "  __shared__ ACC red[4];\n";
-  s << "  const i64 step = (i64)gridDim.x * 256;\n";
+  if (single) s << ", " << ctype(odt) << "* __restrict__ out) {\n";
+  else s << ", ACC* __restrict__ part) {\n";
+  s << "  __shared__ ACC red[" << NT / 64 << "];\n";
+  s << "  const i64 step = (i64)gridDim.x * " << NT << ";\n";
   for (int i = 0; i < n_in; ++i)
     if (layout[(size_t)i] == 's') s << "  const " << ctype(in[i]->dtype) << " s" << i << " = i" << i << "[0];\n";
   s << "  ACC acc = 0;\n";
   s << "  const i64 nv = n / " << vec << ";\n";
-  s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < nv; i += step) {\n";
+  s << "  for (i64 i = (i64)blockIdx.x * " << NT << " + threadIdx.x; i < nv; i += step) {\n";
   for (int i = 0; i < n_in; ++i)
     if (layout[(size_t)i] == 'd') s << "    const Vec<" << ctype(in[i]->dtype) << ", " << vec << "> l" << i << " = reinterpret_cast<const Vec<" << ctype(in[i]->dtype) << ", " << vec << ">*>(i" << i << ")[i];\n";
   for (int e = 0; e < vec; ++e) {
@@ -674,7 +681,7 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     s << "      acc += (ACC)v" << slot << suf << ";\n    }\n";
   }
   s << "  }\n";
-  s << "  const i64 t = nv * " << vec << " + (i64)blockIdx.x * 256 + threadIdx.x;\n";
+  s << "  const i64 t = nv * " << vec << " + (i64)blockIdx.x * " << NT << " + threadIdx.x;\n";
   s << "  if (t < n) {\n";
   for (int i = 0; i < n_in; ++i) {
     s << "    const " << ctype(in[i]->dtype) << " v" << i << "_t = ";
@@ -686,7 +693,8 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   s << "  acc = wave_sum(acc);\n";
   s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n";
   s << "  __syncthreads();\n";
-  s << "  if (threadIdx.x == 0) part[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);\n";
+  if (single) s << "  if (threadIdx.x == 0) {\n    ACC tot = 0;\n    for (int k = 0; k < " << NT / 64 << "; ++k) tot += red[k];\n    out[0] = (" << ctype(odt) << ")tot;\n  }\n";
+  else s << "  if (threadIdx.x == 0) part[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);\n";
   s << "}\n";
   // second launch: one block adds the partial sums up, always in the same order
   s << "extern \"C\" __global__ void __launch_bounds__(256) fused_sum_final(int g, const ACC* __restrict__ part, " << ctype(odt) << "* __restrict__ out) {\n";
@@ -722,27 +730,27 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   if (it == cache.end()) {
     Compiled c;
     rc = compile(ctx, src, &c, "fused_sum");
-    if (rc) { buffer_release(part); hgpu_release(o); return rc; }
+    if (rc) { drop_part(); hgpu_release(o); return rc; }
     it = cache.emplace(src, c).first;
   }
   hipFunction_t fin = nullptr;
   hipError_t e = hipModuleGetFunction(&fin, it->second.mod, "fused_sum_final");
-  if (e != hipSuccess) { buffer_release(part); hgpu_release(o); return check_hip(ctx, e, "hipModuleGetFunction"); }
+  if (e != hipSuccess) { drop_part(); hgpu_release(o); return check_hip(ctx, e, "hipModuleGetFunction"); }
   std::vector<void*> args;
   int64_t nn = n;
   args.push_back(&nn);
   std::vector<const void*> ptrs((size_t)n_in);
   for (int i = 0; i < n_in; ++i) { ptrs[(size_t)i] = data_ptr(in[i]); args.push_back(&ptrs[(size_t)i]); }
-  void* pp = part->ptr;
+  void* pp = single ? data_ptr(o) : part->ptr;
   args.push_back(&pp);
-  e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
-  if (e == hipSuccess) {
+  e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e == hipSuccess && !single) {
     int g = (int)grid;
     void* po = data_ptr(o);
     void* fargs[] = {&g, &pp, &po};
     e = hipModuleLaunchKernel(fin, 1, 1, 1, 256, 1, 1, 0, ctx->stream, fargs, nullptr);
   }
-  buffer_release(part);
+  drop_part();
   if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "fused_sum launch"); }
   *out = o;
   return HGPU_OK;
@@ -795,10 +803,17 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     widest = std::max(widest, dtype_size(dt[(size_t)sum_slots[j]]));
   }
   const int vec = (int)(16 / widest);
-  const unsigned grid = grid_for((n + vec - 1) / vec, 256, ctx->num_cu * 16);
+  // Few elements: one block of 1024 threads writes the outputs and the finished sums, no second launch.
+  const bool single = (n + vec - 1) / vec <= 8192;
+  const int NT = single ? 1024 : 256;
+  const unsigned grid = single ? 1u : grid_for((n + vec - 1) / vec, 256, ctx->num_cu * 16);
   hgpu_buffer* part = nullptr;
-  int rc = buffer_alloc(ctx, (size_t)grid * 8 * (size_t)n_sum, &part);
-  if (rc) { release_all(); return rc; }
+  int rc = HGPU_OK;
+  if (!single) {
+    rc = buffer_alloc(ctx, (size_t)grid * 8 * (size_t)n_sum, &part);
+    if (rc) { release_all(); return rc; }
+  }
+  auto drop_part = [&] { if (part) buffer_release(part); };
 
   std::ostringstream s;
   s << kPrelude;
@@ -811,17 +826,19 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
        "    v += *reinterpret_cast<A*>(&w);\n"
        "  }\n  return v;\n}\n";
   auto acc_t = [&](int j) { return dtype_is_float(dt[(size_t)sum_slots[j]]) ? "double" : "i64"; };
-  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_map_sums(i64 n";
+  s << "extern \"C\" __global__ void __launch_bounds__(" << NT << ") fused_map_sums(i64 n";
   for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
   for (int o = 0; o < n_out; ++o) s << ", " << ctype(res[(size_t)o]->dtype) << "* __restrict__ o" << o;
-  s << ", unsigned long long* __restrict__ part) {\n";
-  s << "  __shared__ unsigned long long red[4];\n";
-  s << "  const i64 step = (i64)gridDim.x * 256;\n";
+  if (single) for (int j = 0; j < n_sum; ++j) s << ", " << ctype(dt[(size_t)sum_slots[j]]) << "* __restrict__ sum" << j;
+  else s << ", unsigned long long* __restrict__ part";
+  s << ") {\n";
+  s << "  __shared__ unsigned long long red[" << NT / 64 << "];\n";
+  s << "  const i64 step = (i64)gridDim.x * " << NT << ";\n";
   for (int i = 0; i < n_in; ++i)
     if (layout[(size_t)i] == 's') s << "  const " << ctype(in[i]->dtype) << " s" << i << " = i" << i << "[0];\n";
   for (int j = 0; j < n_sum; ++j) s << "  " << acc_t(j) << " acc" << j << " = 0;\n";
   s << "  const i64 nv = n / " << vec << ";\n";
-  s << "  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < nv; i += step) {\n";
+  s << "  for (i64 i = (i64)blockIdx.x * " << NT << " + threadIdx.x; i < nv; i += step) {\n";
   for (int i = 0; i < n_in; ++i)
     if (layout[(size_t)i] == 'd') s << "    const Vec<" << ctype(in[i]->dtype) << ", " << vec << "> l" << i << " = reinterpret_cast<const Vec<" << ctype(in[i]->dtype) << ", " << vec << ">*>(i" << i << ")[i];\n";
   for (int o = 0; o < n_out; ++o) s << "    Vec<" << ctype(res[(size_t)o]->dtype) << ", " << vec << "> r" << o << ";\n";
@@ -840,7 +857,7 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   }
   for (int o = 0; o < n_out; ++o) s << "    reinterpret_cast<Vec<" << ctype(res[(size_t)o]->dtype) << ", " << vec << ">*>(o" << o << ")[i] = r" << o << ";\n";
   s << "  }\n";
-  s << "  const i64 t = nv * " << vec << " + (i64)blockIdx.x * 256 + threadIdx.x;\n";
+  s << "  const i64 t = nv * " << vec << " + (i64)blockIdx.x * " << NT << " + threadIdx.x;\n";
   s << "  if (t < n) {\n";
   for (int i = 0; i < n_in; ++i) {
     s << "    const " << ctype(in[i]->dtype) << " v" << i << "_t = ";
@@ -855,9 +872,14 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     s << "  acc" << j << " = wave_sum(acc" << j << ");\n";
     s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = *reinterpret_cast<unsigned long long*>(&acc" << j << ");\n";
     s << "  __syncthreads();\n";
-    s << "  if (threadIdx.x == 0) {\n    " << acc_t(j) << " t4[4];\n    for (int k = 0; k < 4; ++k) t4[k] = *reinterpret_cast<" << acc_t(j) << "*>(&red[k]);\n";
-    s << "    " << acc_t(j) << " tot = (t4[0] + t4[1]) + (t4[2] + t4[3]);\n";
-    s << "    part[(i64)" << j << " * gridDim.x + blockIdx.x] = *reinterpret_cast<unsigned long long*>(&tot);\n  }\n";
+    if (single) {
+      s << "  if (threadIdx.x == 0) {\n    " << acc_t(j) << " tot = 0;\n    for (int k = 0; k < " << NT / 64 << "; ++k) tot += *reinterpret_cast<" << acc_t(j) << "*>(&red[k]);\n";
+      s << "    sum" << j << "[0] = (" << ctype(dt[(size_t)sum_slots[j]]) << ")tot;\n  }\n";
+    } else {
+      s << "  if (threadIdx.x == 0) {\n    " << acc_t(j) << " t4[4];\n    for (int k = 0; k < 4; ++k) t4[k] = *reinterpret_cast<" << acc_t(j) << "*>(&red[k]);\n";
+      s << "    " << acc_t(j) << " tot = (t4[0] + t4[1]) + (t4[2] + t4[3]);\n";
+      s << "    part[(i64)" << j << " * gridDim.x + blockIdx.x] = *reinterpret_cast<unsigned long long*>(&tot);\n  }\n";
+    }
     s << "  __syncthreads();\n";
   }
   s << "}\n";
@@ -898,12 +920,12 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   if (it == cache.end()) {
     Compiled c;
     rc = compile(ctx, src, &c, "fused_map_sums");
-    if (rc) { buffer_release(part); release_all(); return rc; }
+    if (rc) { drop_part(); release_all(); return rc; }
     it = cache.emplace(src, c).first;
   }
   hipFunction_t fin = nullptr;
   hipError_t e = hipModuleGetFunction(&fin, it->second.mod, "fused_map_sums_final");
-  if (e != hipSuccess) { buffer_release(part); release_all(); return check_hip(ctx, e, "hipModuleGetFunction"); }
+  if (e != hipSuccess) { drop_part(); release_all(); return check_hip(ctx, e, "hipModuleGetFunction"); }
   std::vector<void*> args;
   int64_t nn = n;
   args.push_back(&nn);
@@ -911,16 +933,18 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   std::vector<void*> optrs((size_t)n_out), sptrs((size_t)n_sum);
   for (int i = 0; i < n_in; ++i) { ptrs[(size_t)i] = data_ptr(in[i]); args.push_back(&ptrs[(size_t)i]); }
   for (int o = 0; o < n_out; ++o) { optrs[(size_t)o] = data_ptr(res[(size_t)o]); args.push_back(&optrs[(size_t)o]); }
-  void* pp = part->ptr;
-  args.push_back(&pp);
-  e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
-  if (e == hipSuccess) {
+  for (int j = 0; j < n_sum; ++j) sptrs[(size_t)j] = data_ptr(sres[(size_t)j]);
+  void* pp = part ? part->ptr : nullptr;
+  if (single) for (int j = 0; j < n_sum; ++j) args.push_back(&sptrs[(size_t)j]);
+  else args.push_back(&pp);
+  e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e == hipSuccess && !single) {
     int g = (int)grid;
     std::vector<void*> fargs = {&g, &pp};
-    for (int j = 0; j < n_sum; ++j) { sptrs[(size_t)j] = data_ptr(sres[(size_t)j]); fargs.push_back(&sptrs[(size_t)j]); }
+    for (int j = 0; j < n_sum; ++j) fargs.push_back(&sptrs[(size_t)j]);
     e = hipModuleLaunchKernel(fin, (unsigned)n_sum, 1, 1, 256, 1, 1, 0, ctx->stream, fargs.data(), nullptr);
   }
-  buffer_release(part);
+  drop_part();
   if (e != hipSuccess) { release_all(); return check_hip(ctx, e, "fused_map_sums launch"); }
   for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
   for (int j = 0; j < n_sum; ++j) sums[j] = sres[(size_t)j];

@@ -59,7 +59,7 @@ __global__ void k_koff(Group k, int64_t K, int64_t Kp, int64_t* __restrict__ ka,
 // flight at a time, and combine through LDS in a fixed order.  Few outputs get
 // the narrow blocks: more of them, and fewer partials for a lane to walk through.
 template <typename T, int OPB>
-__global__ void __launch_bounds__(256) k_sum_partials(int64_t n, int S, int64_t stride, const T* __restrict__ part, T* __restrict__ out) {
+__global__ void __launch_bounds__(256) k_sum_partials(int64_t n, int S, int64_t stride, const T* __restrict__ part, T* __restrict__ out, int64_t n1, T* __restrict__ out2) {
   constexpr int G = 256 / OPB;
   __shared__ T red[G][OPB + 1];
   const int ol = threadIdx.x % OPB, g = threadIdx.x / OPB;
@@ -76,7 +76,8 @@ __global__ void __launch_bounds__(256) k_sum_partials(int64_t n, int S, int64_t 
       T t = red[0][ol];
 #pragma unroll
       for (int k = 1; k < G; ++k) t += red[k][ol];
-      out[i] = t;
+      if (i < n1) out[i] = t;
+      else out2[i - n1] = t;
     }
     __syncthreads();
   }
@@ -86,7 +87,7 @@ __global__ void __launch_bounds__(256) k_sum_partials(int64_t n, int S, int64_t 
 // leave most of their lane groups without a partial: one output per lane, the
 // partials added in the same order (0 + p0 + p1 + ...), four loads in flight.
 template <typename T>
-__global__ void __launch_bounds__(256) k_sum_partials_few(int64_t n, int S, int64_t stride, const T* __restrict__ part, T* __restrict__ out) {
+__global__ void __launch_bounds__(256) k_sum_partials_few(int64_t n, int S, int64_t stride, const T* __restrict__ part, T* __restrict__ out, int64_t n1, T* __restrict__ out2) {
   const int64_t step = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
     const T* p = part + i;
@@ -106,20 +107,23 @@ __global__ void __launch_bounds__(256) k_sum_partials_few(int64_t n, int S, int6
       s += 2;
     }
     if (s < S) acc += p[(int64_t)s * stride];
-    out[i] = acc;
+    if (i < n1) out[i] = acc;
+    else out2[i - n1] = acc;
   }
 }
 
+// Outputs [0, n1) go to `out`, the rest to `out2` (two results whose partial sums one kernel wrote side by side).
 template <typename T>
-void launch_sum_partials(hgpu_ctx* ctx, int64_t n, int S, const T* part, T* out) {
+void launch_sum_partials(hgpu_ctx* ctx, int64_t n, int S, const T* part, T* out, int64_t n1 = -1, T* out2 = nullptr) {
+  if (n1 < 0) n1 = n;
   if (S <= 8)
-    hipLaunchKernelGGL((k_sum_partials_few<T>), dim3(grid_for(n, 256, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out);
+    hipLaunchKernelGGL((k_sum_partials_few<T>), dim3(grid_for(n, 256, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out, n1, out2);
   else if (sizeof(T) == 4)   // rows of 32 floats are whole 128-byte lines (16384 outputs x 270 partials: 12.9 us with rows of 8, 7.1 us with rows of 32)
-    hipLaunchKernelGGL((k_sum_partials<T, 32>), dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out);
+    hipLaunchKernelGGL((k_sum_partials<T, 32>), dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out, n1, out2);
   else if (n <= 32768 && S >= 32)
-    hipLaunchKernelGGL((k_sum_partials<T, 8>), dim3(grid_for(n, 8, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out);
+    hipLaunchKernelGGL((k_sum_partials<T, 8>), dim3(grid_for(n, 8, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out, n1, out2);
   else
-    hipLaunchKernelGGL((k_sum_partials<T, 32>), dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out);
+    hipLaunchKernelGGL((k_sum_partials<T, 32>), dim3(grid_for(n, 32, ctx->num_cu * 8)), dim3(256), 0, ctx->stream, n, S, n, part, out, n1, out2);
 }
 
 // Appends dim (extent e, strides a, b, c) to a group, merging with the previous dim when all strides allow.
@@ -343,6 +347,17 @@ int sum_partials(hgpu_ctx* ctx, int dtype, int64_t n, int parts, const void* par
   LaunchGuard ls(ctx, "gemm_sum_partials", (double)n * (parts + 1) * es, (double)n * parts);
   if (dtype == HGPU_F64) launch_sum_partials<double>(ctx, n, parts, (const double*)part, (double*)out);
   else launch_sum_partials<float>(ctx, n, parts, (const float*)part, (float*)out);
+  HG_CHECK_LAUNCH(ctx, "gemm_sum_partials");
+  return HGPU_OK;
+}
+
+// `parts` partial results of n1 + n2 elements each: the first n1 summed into out1, the other n2 into out2.
+int sum_partials_split(hgpu_ctx* ctx, int dtype, int64_t n1, int64_t n2, int parts, const void* part, void* out1, void* out2) {
+  const size_t es = dtype_size(dtype);
+  const int64_t n = n1 + n2;
+  LaunchGuard ls(ctx, "gemm_sum_partials", (double)n * (parts + 1) * es, (double)n * parts);
+  if (dtype == HGPU_F64) launch_sum_partials<double>(ctx, n, parts, (const double*)part, (double*)out1, n1, (double*)out2);
+  else launch_sum_partials<float>(ctx, n, parts, (const float*)part, (float*)out1, n1, (float*)out2);
   HG_CHECK_LAUNCH(ctx, "gemm_sum_partials");
   return HGPU_OK;
 }

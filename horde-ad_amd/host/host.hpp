@@ -69,6 +69,9 @@ struct ArrHolder {
   // convolution never writes its patch gradient to memory).
   std::shared_ptr<ArrHolder> fa, fb;
   int keep = -1;
+  // The product expression whose factors fa and fb are (tssumN (u * v) taken apart): when somebody has written
+  // the product out by the time the contraction is computed, the contraction is the sum of that array.
+  std::shared_ptr<ArrHolder> whole;
   // Further (fa, fb) pairs of a pending SUM of contractions of one shape (the
   // cotangent of a parameter used once per step of an unrolled recurrence):
   // written out by one grouped launch when the provider has contract_sum.

@@ -911,7 +911,7 @@ void ArrHolder::force() {
   if (h) return;
   if (probe) throw ProbeFail{};
   if (ssrc) {   // a sum nobody's pass has taken along: a pass of its own
-    T e(ssrc);
+      T e(ssrc);
     ssrc.reset();
     T r;
     const hgpu_api* api = be->api;
@@ -1024,13 +1024,16 @@ void ArrHolder::force() {
     origin->force();   // once for all its users
     p = transpose(T(origin), origin_perm);
   } else {
+    if (whole && !whole->h && whole->vsrc && whole->vsrc->h) whole->view_of_written_source();
     T fbt(fb);
-    p = ones_b ? contract_now(T(fa), nullptr, keep) : contract_now(T(fa), &fbt, keep);   // a sum nobody's pass has taken along
+    if (whole && whole->h && !ones_b) p = contract_now(T(whole), nullptr, keep);   // the product has been written out meanwhile
+    else p = ones_b ? contract_now(T(fa), nullptr, keep) : contract_now(T(fa), &fbt, keep);   // a sum nobody's pass has taken along
   }
   be->check(be->api->retain(p.h()));
   h = p.h();
   fa.reset();
   fb.reset();
+  whole.reset();
   origin.reset();
   keep = -1;
   ones_b = false;
@@ -1273,6 +1276,12 @@ T reverse(const T& a, int dim) {
 T replicate(const T& a, const Shape& pre) {
   if (pre.empty()) return a;
   HD_META_VIEW(meta_replicate(a.holder()->vmeta, pre, &m__))
+  // a one-element expression: evaluated by whoever consumes the copies (see broadcast_scalar)
+  if (a.pending_expr() && a.size() == 1 && fuses(a.be()) && pending_size(a.holder()) <= 8) {
+    Shape sh(pre);
+    for (auto e : a.shape()) sh.push_back(e);
+    if (prod(sh) > 1) return broadcast_scalar(a, sh);
+  }
   // An expression that is replicated stays unevaluated behind a pending view:
   // a contraction may take it in as it is, anything else computes it once, for
   // every view of it.
@@ -1444,7 +1453,9 @@ T contract(const T& a, const T* b, int n_keep) {
     // contraction with ones.
     if (n_keep >= 1 && fuses(a.be()) && holds_pending_contraction(a.holder().get()))
       return lazy_contract(a, broadcast_scalar(constant(a.be(), a.dtype(), 1.0), a.shape()), n_keep);
-    return lazy_contract(a.factor_a(), a.factor_b(), n_keep);
+    T r = lazy_contract(a.factor_a(), a.factor_b(), n_keep);
+    r.holder()->whole = a.holder();
+    return r;
   }
   // the sum of a view of such a product likewise waits (sums of one shape then go out together)
   if (!b && n_keep >= 1 && n_keep < a.rank() && a.pending_view() && fuses(a.be()) && a.holder()->vlo.empty() && T(a.holder()->vsrc).pending_product() &&
@@ -1490,6 +1501,21 @@ T contract(const T& a, const T* b, int n_keep) {
         if (rc == HGPU_OK) return T(be, o);
         if (rc != HGPU_ERR_UNSUPPORTED) be->check(rc);
       }
+    }
+  }
+  // sdot0 with an expression for an operand (`sdot0 (log soft) expected`, an objective's value): the sum
+  // of the product expression, which waits for a pass over arrays of this shape like any other such sum
+  if (b && n_keep == 0 && (a.pending_expr() || b->pending_expr()) && a.dtype() == b->dtype() && a.shape() == b->shape() && a.size() >= 4096 &&
+      (a.dtype() == HGPU_F64 || a.dtype() == HGPU_F32) && fuses(a.be()) && pending_size(a.holder()) + pending_size(b->holder()) < 40) {
+    const hgpu_api* api = a.be()->api;
+    if (api->struct_size >= offsetof(hgpu_api, fused_map_sums) + sizeof(api->fused_map_sums) && api->fused_map_sums) {
+      Backend* be = a.be();
+      auto p = std::make_shared<ArrHolder>(be, nullptr);
+      p->ssrc = make_expr(HGPU_FUSED_OP2, HGPU_MUL, a.dtype(), a, b, nullptr).holder();
+      auto& ps = be->pending_sums;
+      ps.erase(std::remove_if(ps.begin(), ps.end(), [](const std::weak_ptr<ArrHolder>& w) { auto q = w.lock(); return !q || q->h || !q->ssrc; }), ps.end());
+      ps.push_back(p);
+      return T(p);
     }
   }
   // a contraction of two arrays of one shape and dtype stays pending too: sums of
@@ -1660,6 +1686,11 @@ T broadcast_scalar(const T& s, const Shape& shape) {
   Shape st(shape.size(), 0);
   for (auto e : shape)
     if (e == 0) return replicate(reshape(s, {}), shape);
+  // A one-element EXPRESSION that is repeated stays an expression, over its leaves repeated: the
+  // consumer's pass evaluates it (`recip (ssum0 e)` under `sreplicate0N`, the negated cotangent
+  // of a negated objective), instead of a launch of its own for one element.
+  if (s.pending_expr() && prod(shape) > 1 && fuses(s.be()) && pending_size(s.holder()) <= 8)
+    return map_leaves(s, [&](const T& x) { return broadcast_scalar(x, shape); });
   T r = as_strided(s, shape, st, 0);
   if (r.holder() != s.holder()) r.holder()->scalar_src = s.holder();
   return r;
