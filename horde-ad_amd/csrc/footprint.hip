@@ -85,6 +85,7 @@ struct Plan {
   int addr_regs;   // per-lane address registers of the kernel
   int nbufs;   // LDS chunk buffers: 2, or 1 when two do not fit (the prefetch then waits in registers)
   int ks = 1;  // wavefronts per SIMD: the block's 4 ks wavefronts split the K groups of a chunk ks ways
+  int bpc = 1; // blocks that share a CU (their LDS fits together): one's loads and stores run under the other's multiplications
   bool cvec;   // groups of four rows are adjacent in C and 16-byte aligned: vector stores
 };
 
@@ -311,7 +312,7 @@ typedef Vec<VY> RawY;
 #define LOAD_Y(ch_, j_) reinterpret_cast<const Vec<VY>*>(Y + (ch_) * chy)[vidx(j_)]
 #define FIN_Y(j_, r_) (r_)
 #endif
-extern "C" __global__ void __launch_bounds__(NT, 1)
+extern "C" __global__ void __launch_bounds__(NT, BPC)
 KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 nch, i64 chx, i64 chy, i64 chc, i64 part_stride
 #if EPI
       , EpiArgs ea
@@ -712,7 +713,7 @@ std::string generate(const Plan& pl, const std::string& kname, const std::string
   s << "#define KNAME " << kname << "\n";
   s << "#define VIRT_X " << (virt_x.empty() ? 0 : 1) << "\n#define XBASE " << xbase << "ll\n";
   s << "#define VIRT_Y " << (virt_y.empty() ? 0 : 1) << "\n#define YBASE " << ybase << "ll\n";
-  s << "#define EPI " << (epilogue.empty() ? 0 : 1) << "\n#define EPI_STAGE " << stage_bytes << "\n";
+  s << "#define EPI " << (epilogue.empty() ? 0 : 1) << "\n#define EPI_STAGE " << stage_bytes << "\n#define BPC " << pl.bpc << "\n";
   const int es = pl.f64 ? 8 : 4;
   s << "#define F64 " << (pl.f64 ? 1 : 0) << "\n#define KS " << pl.ks << "\n";
   s << "#define MODE " << pl.mode << "\n";
@@ -1280,7 +1281,7 @@ std::string epilogue_source(const Plan& pl, const EpiSpec& e) {
         s << "    if (ev[" << w * e.L + u << "] " << (e.want_max ? ">" : "<") << " best) { best = ev[" << w * e.L + u << "]; bi = " << u << "; }\n";
       if (e.staged) {
         s << "    reinterpret_cast<" << ctype(e.dt[(size_t)e.ext_slot]) << "*>(stage + " << e.val_off << ")[ep.w[" << w << "]] = best;\n";
-        s << "    reinterpret_cast<i64*>(stage + " << e.idx_off << ")[ep.w[" << w << "]] = bi;\n  }\n";
+        s << "    (stage + " << e.idx_off << ")[ep.w[" << w << "]] = (unsigned char)bi;\n  }\n";
       } else {
         s << "    const i64 at = ch * " << e.win_chs << "ll + ep.w[" << w << "];\n    ea.ov[at] = best;\n    ea.oi[at] = bi;\n  }\n";
       }
@@ -1302,7 +1303,10 @@ std::string epilogue_source(const Plan& pl, const EpiSpec& e) {
     for (size_t o = 0; o < e.out_slots.size(); ++o) block("ea.o" + std::to_string(o), ctype(e.dt[(size_t)e.out_slots[o]]), e.out_chs, e.out_off[o], n_el, dtype_size(e.dt[(size_t)e.out_slots[o]]));
     if (e.has_ext) {
       block("ea.ov", ctype(e.dt[(size_t)e.ext_slot]), e.win_chs, e.val_off, n_el / e.L, dtype_size(e.dt[(size_t)e.ext_slot]));
-      block("ea.oi", "i64", e.win_chs, e.idx_off, n_el / e.L, 8);
+      // the places within the windows wait in LDS as bytes and are widened on their way out, two per lane and step
+      s << "  {\n    V16* dst = reinterpret_cast<V16*>(ea.oi + ch * " << e.win_chs << "ll);\n";
+      s << "    const unsigned char* src = stage + " << e.idx_off << ";\n";
+      s << "#pragma unroll 4\n    for (int v = tid; v < " << n_el / e.L / 2 << "; v += NT) dst[v] = V16{{src[2 * v], 0u, src[2 * v + 1], 0u}};\n  }\n";
     }
     s << "}\n";
   }
@@ -1536,7 +1540,8 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
     for (int o = 0; o < n_out; ++o) e.out_off.push_back(place(n_el, dtype_size(dt[(size_t)out_slots[o]]), e.out_chs));
     if (has_ext) {
       e.val_off = place(n_el / L, dtype_size(dt[(size_t)ext_slot]), e.win_chs);
-      e.idx_off = place(n_el / L, 8, e.win_chs);
+      if ((n_el / L) % 2 != 0 || (e.win_chs * 8) % 16 != 0) ok = false;
+      e.idx_off = place(n_el / L, 1, 16);     // one byte per window in LDS, 8 in memory
     }
     e.stage_bytes = off;
     Plan p3 = pl;
@@ -1545,6 +1550,10 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
     if (ok && off > 0 && finish_plan(p3, xp3, yp3, nullptr, 0, off) && p3.nbufs == pl.nbufs) { e.staged = true; pl = p3; }
     else e.stage_bytes = 0;
   }
+  // For measurements (HORDEAD_FOOTPRINT_BPC=2): two blocks to a CU when their LDS fits together.  The first
+  // CNN layer (784 rows x 16 x K 25 per chunk) runs 40 us that way against 34 us with one block per CU.
+  static const int bpc_env = getenv("HORDEAD_FOOTPRINT_BPC") ? atoi(getenv("HORDEAD_FOOTPRINT_BPC")) : 0;
+  pl.bpc = (pl.ks == 1 && 2 * (lds_bytes(pl) + e.stage_bytes + 512) <= 160 * 1024 && pl.nch >= 3 * (int64_t)ctx->num_cu && bpc_env == 2) ? 2 : 1;
 
   // ---- results
   std::vector<hgpu_array*> res((size_t)n_out, nullptr);
@@ -1585,7 +1594,7 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
   if (has_ext) { ea.push_back(data_ptr(v)); ea.push_back(data_ptr(ix)); }
   ea.push_back(nullptr);   // the int at the end, padded to a pointer
   void* args[] = {(void*)&xp, (void*)&yp, (void*)&cnull, (void*)&nch, (void*)&chx, (void*)&chy, (void*)&chc, (void*)&part_stride, (void*)ea.data()};
-  int64_t grid = pl.nch < ctx->num_cu ? pl.nch : ctx->num_cu;
+  int64_t grid = std::min<int64_t>(pl.nch, (int64_t)ctx->num_cu * pl.bpc);
   {
     const double M = (double)(swapped ? Nb : Ma), N = (double)(swapped ? Ma : Nb);
     double flops = 2.0 * M * N * K;

@@ -634,8 +634,8 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   if (n == 0) { *out = o; return HGPU_OK; }
   const bool fp = dtype_is_float(odt);
   const char* acc = fp ? "double" : "i64";
-  // Few elements: one block of 1024 threads sums them and writes the result, no second launch.
-  const bool single = (n + vec - 1) / vec <= 8192;
+  // Very few elements: one block of 1024 threads sums them and writes the result.
+  const bool single = (n + vec - 1) / vec <= 1024;
   const int NT = single ? 1024 : 256;
   const unsigned grid = single ? 1u : grid_for((n + vec - 1) / vec, 256, ctx->num_cu * 8);
   hgpu_buffer* part = nullptr;
@@ -644,6 +644,14 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     if (rc) { hgpu_release(o); return rc; }
   }
   auto drop_part = [&] { if (part) buffer_release(part); };
+  // Up to a million elements the block that finishes last adds the blocks' sums up; beyond, a second launch does
+  // (handing a sum over takes a fence per block, and the thousands of blocks of a large array would each pay it).
+  const bool ticketed = !single && n <= (1 << 20);
+  void* ticket = nullptr;
+  if (ticketed) {
+    rc = ticket_block(ctx, &ticket);
+    if (rc) { drop_part(); hgpu_release(o); return rc; }
+  }
 
   std::ostringstream s;
   s << kPrelude;
@@ -659,6 +667,7 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   s << "extern \"C\" __global__ void __launch_bounds__(" << NT << ") fused_sum(i64 n";
   for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
   if (single) s << ", " << ctype(odt) << "* __restrict__ out) {\n";
+  else if (ticketed) s << ", unsigned long long* part, unsigned int* ticket, " << ctype(odt) << "* __restrict__ out) {\n";
   else s << ", ACC* __restrict__ part) {\n";
   s << "  __shared__ ACC red[" << NT / 64 << "];\n";
   s << "  const i64 step = (i64)gridDim.x * " << NT << ";\n";
@@ -694,18 +703,37 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n";
   s << "  __syncthreads();\n";
   if (single) s << "  if (threadIdx.x == 0) {\n    ACC tot = 0;\n    for (int k = 0; k < " << NT / 64 << "; ++k) tot += red[k];\n    out[0] = (" << ctype(odt) << ")tot;\n  }\n";
-  else s << "  if (threadIdx.x == 0) part[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);\n";
+  else if (!ticketed) s << "  if (threadIdx.x == 0) part[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);\n";
+  else {
+    // The block that finishes last adds the blocks' sums up, always in the same order, and writes the result:
+    // every block hands its sum over (store, fence, ticket), the last one to draw a ticket sees them all.
+    s << "  __shared__ int last;\n";
+    s << "  if (threadIdx.x == 0) {\n    ACC tot = (red[0] + red[1]) + (red[2] + red[3]);\n";
+    s << "    __hip_atomic_store(part + blockIdx.x, *reinterpret_cast<unsigned long long*>(&tot), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+    s << "    __threadfence();\n    last = atomicAdd(ticket, 1u) == gridDim.x - 1;\n  }\n";
+    s << "  __syncthreads();\n  if (!last) return;\n  __threadfence();\n";
+    s << "  acc = 0;\n";
+    s << "  for (int i = threadIdx.x; i < (int)gridDim.x; i += 256) {\n";
+    s << "    unsigned long long u = __hip_atomic_load(part + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n    acc += *reinterpret_cast<ACC*>(&u);\n  }\n";
+    s << "  acc = wave_sum(acc);\n";
+    s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n";
+    s << "  __syncthreads();\n";
+    s << "  if (threadIdx.x == 0) {\n    out[0] = (" << ctype(odt) << ")((red[0] + red[1]) + (red[2] + red[3]));\n";
+    s << "    __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch\n  }\n";
+  }
   s << "}\n";
-  // second launch: one block adds the partial sums up, always in the same order
-  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_sum_final(int g, const ACC* __restrict__ part, " << ctype(odt) << "* __restrict__ out) {\n";
-  s << "  __shared__ ACC red[4];\n";
-  s << "  ACC acc = 0;\n";
-  s << "  for (int i = threadIdx.x; i < g; i += 256) acc += part[i];\n";
-  s << "  acc = wave_sum(acc);\n";
-  s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n";
-  s << "  __syncthreads();\n";
-  s << "  if (threadIdx.x == 0) out[0] = (" << ctype(odt) << ")((red[0] + red[1]) + (red[2] + red[3]));\n";
-  s << "}\n";
+  if (!single && !ticketed) {
+    // second launch: one block adds the partial sums up, in the same order
+    s << "extern \"C\" __global__ void __launch_bounds__(256) fused_sum_final(int g, const ACC* __restrict__ part, " << ctype(odt) << "* __restrict__ out) {\n";
+    s << "  __shared__ ACC red[4];\n";
+    s << "  ACC acc = 0;\n";
+    s << "  for (int i = threadIdx.x; i < g; i += 256) acc += part[i];\n";
+    s << "  acc = wave_sum(acc);\n";
+    s << "  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;\n";
+    s << "  __syncthreads();\n";
+    s << "  if (threadIdx.x == 0) out[0] = (" << ctype(odt) << ")((red[0] + red[1]) + (red[2] + red[3]));\n";
+    s << "}\n";
+  }
   std::string src = s.str();
 
   const char* label = "fused_sum";
@@ -733,20 +761,22 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     if (rc) { drop_part(); hgpu_release(o); return rc; }
     it = cache.emplace(src, c).first;
   }
-  hipFunction_t fin = nullptr;
-  hipError_t e = hipModuleGetFunction(&fin, it->second.mod, "fused_sum_final");
-  if (e != hipSuccess) { drop_part(); hgpu_release(o); return check_hip(ctx, e, "hipModuleGetFunction"); }
   std::vector<void*> args;
   int64_t nn = n;
   args.push_back(&nn);
   std::vector<const void*> ptrs((size_t)n_in);
   for (int i = 0; i < n_in; ++i) { ptrs[(size_t)i] = data_ptr(in[i]); args.push_back(&ptrs[(size_t)i]); }
-  void* pp = single ? data_ptr(o) : part->ptr;
-  args.push_back(&pp);
-  e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
-  if (e == hipSuccess && !single) {
+  void* po = data_ptr(o);
+  void* pp = single ? nullptr : part->ptr;
+  if (!single) args.push_back(&pp);
+  if (ticketed) args.push_back(&ticket);
+  if (single || ticketed) args.push_back(&po);
+  hipFunction_t fin = nullptr;
+  hipError_t e = hipSuccess;
+  if (!single && !ticketed) e = hipModuleGetFunction(&fin, it->second.mod, "fused_sum_final");
+  if (e == hipSuccess) e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e == hipSuccess && fin) {
     int g = (int)grid;
-    void* po = data_ptr(o);
     void* fargs[] = {&g, &pp, &po};
     e = hipModuleLaunchKernel(fin, 1, 1, 1, 256, 1, 1, 0, ctx->stream, fargs, nullptr);
   }
@@ -758,7 +788,7 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
 
 // hgpu_fused_map with sums: the map's outputs and the sums of some slots from
 // one pass over dense inputs.  Per-block partial sums (double / int64), added
-// up in a fixed order by a second, one-block launch.
+// up in a fixed order by the block that finishes last (by a second, one-block launch for large arrays).
 extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog, int n_out,
                                    const int* out_slots, hgpu_array** outs, int n_sum, const int* sum_slots, hgpu_array** sums) {
   if (!ctx || !in || !prog || (n_out > 0 && (!out_slots || !outs)) || (n_sum > 0 && (!sum_slots || !sums))) return HGPU_ERR_INVALID;
@@ -803,8 +833,8 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     widest = std::max(widest, dtype_size(dt[(size_t)sum_slots[j]]));
   }
   const int vec = (int)(16 / widest);
-  // Few elements: one block of 1024 threads writes the outputs and the finished sums, no second launch.
-  const bool single = (n + vec - 1) / vec <= 8192;
+  // Very few elements: one block of 1024 threads writes the outputs and the finished sums.
+  const bool single = (n + vec - 1) / vec <= 1024;
   const int NT = single ? 1024 : 256;
   const unsigned grid = single ? 1u : grid_for((n + vec - 1) / vec, 256, ctx->num_cu * 16);
   hgpu_buffer* part = nullptr;
@@ -814,6 +844,15 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     if (rc) { release_all(); return rc; }
   }
   auto drop_part = [&] { if (part) buffer_release(part); };
+  // Up to a million elements the block that finishes last adds the blocks' sums up; beyond, a second launch
+  // does (handing the sums over takes a fence per block, which also waits for the block's share of the outputs
+  // to leave the cache: 16.8 M elements with three outputs take 0.42 ms that way, 0.18 ms with two launches).
+  const bool ticketed = !single && n <= (1 << 20);
+  void* ticket = nullptr;
+  if (ticketed) {
+    rc = ticket_block(ctx, &ticket);
+    if (rc) { drop_part(); release_all(); return rc; }
+  }
 
   std::ostringstream s;
   s << kPrelude;
@@ -829,8 +868,9 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   s << "extern \"C\" __global__ void __launch_bounds__(" << NT << ") fused_map_sums(i64 n";
   for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
   for (int o = 0; o < n_out; ++o) s << ", " << ctype(res[(size_t)o]->dtype) << "* __restrict__ o" << o;
-  if (single) for (int j = 0; j < n_sum; ++j) s << ", " << ctype(dt[(size_t)sum_slots[j]]) << "* __restrict__ sum" << j;
-  else s << ", unsigned long long* __restrict__ part";
+  if (ticketed) s << ", unsigned long long* part, unsigned int* ticket";
+  else if (!single) s << ", unsigned long long* __restrict__ part";
+  if (single || ticketed) for (int j = 0; j < n_sum; ++j) s << ", " << ctype(dt[(size_t)sum_slots[j]]) << "* __restrict__ sum" << j;
   s << ") {\n";
   s << "  __shared__ unsigned long long red[" << NT / 64 << "];\n";
   s << "  const i64 step = (i64)gridDim.x * " << NT << ";\n";
@@ -878,23 +918,42 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     } else {
       s << "  if (threadIdx.x == 0) {\n    " << acc_t(j) << " t4[4];\n    for (int k = 0; k < 4; ++k) t4[k] = *reinterpret_cast<" << acc_t(j) << "*>(&red[k]);\n";
       s << "    " << acc_t(j) << " tot = (t4[0] + t4[1]) + (t4[2] + t4[3]);\n";
-      s << "    part[(i64)" << j << " * gridDim.x + blockIdx.x] = *reinterpret_cast<unsigned long long*>(&tot);\n  }\n";
+      if (ticketed) s << "    __hip_atomic_store(part + ((i64)" << j << " * gridDim.x + blockIdx.x), *reinterpret_cast<unsigned long long*>(&tot), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n  }\n";
+      else s << "    part[(i64)" << j << " * gridDim.x + blockIdx.x] = *reinterpret_cast<unsigned long long*>(&tot);\n  }\n";
     }
     s << "  __syncthreads();\n";
   }
-  s << "}\n";
-  // second launch: block j adds the partial sums of sum j, always in the same order
-  s << "extern \"C\" __global__ void __launch_bounds__(256) fused_map_sums_final(int g, const unsigned long long* __restrict__ part";
-  for (int j = 0; j < n_sum; ++j) s << ", " << ctype(dt[(size_t)sum_slots[j]]) << "* __restrict__ out" << j;
-  s << ") {\n  __shared__ unsigned long long red[4];\n";
-  for (int j = 0; j < n_sum; ++j) {
-    s << "  if (blockIdx.x == " << j << ") {\n    " << acc_t(j) << " acc = 0;\n";
-    s << "    for (int i = threadIdx.x; i < g; i += 256) acc += *reinterpret_cast<const " << acc_t(j) << "*>(&part[(i64)" << j << " * g + i]);\n";
-    s << "    acc = wave_sum(acc);\n    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = *reinterpret_cast<unsigned long long*>(&acc);\n    __syncthreads();\n";
-    s << "    if (threadIdx.x == 0) {\n      " << acc_t(j) << " t4[4];\n      for (int k = 0; k < 4; ++k) t4[k] = *reinterpret_cast<" << acc_t(j) << "*>(&red[k]);\n";
-    s << "      out" << j << "[0] = (" << ctype(dt[(size_t)sum_slots[j]]) << ")((t4[0] + t4[1]) + (t4[2] + t4[3]));\n    }\n  }\n";
+  if (ticketed) {
+    // The block that finishes last adds the blocks' sums up, always in the same order, and writes the results:
+    // every block hands its sums over (stores, fence, ticket), the last one to draw a ticket sees them all.
+    s << "  __shared__ int last;\n";
+    s << "  if (threadIdx.x == 0) {\n    __threadfence();\n    last = atomicAdd(ticket, 1u) == gridDim.x - 1;\n  }\n";
+    s << "  __syncthreads();\n  if (!last) return;\n  __threadfence();\n  const int g = (int)gridDim.x;\n";
+    for (int j = 0; j < n_sum; ++j) {
+      s << "  {\n    " << acc_t(j) << " acc = 0;\n";
+      s << "    for (int i = threadIdx.x; i < g; i += 256) {\n";
+      s << "      unsigned long long u = __hip_atomic_load(part + ((i64)" << j << " * g + i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n      acc += *reinterpret_cast<" << acc_t(j) << "*>(&u);\n    }\n";
+      s << "    acc = wave_sum(acc);\n    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = *reinterpret_cast<unsigned long long*>(&acc);\n    __syncthreads();\n";
+      s << "    if (threadIdx.x == 0) {\n      " << acc_t(j) << " t4[4];\n      for (int k = 0; k < 4; ++k) t4[k] = *reinterpret_cast<" << acc_t(j) << "*>(&red[k]);\n";
+      s << "      sum" << j << "[0] = (" << ctype(dt[(size_t)sum_slots[j]]) << ")((t4[0] + t4[1]) + (t4[2] + t4[3]));\n    }\n    __syncthreads();\n  }\n";
+    }
+    s << "  if (threadIdx.x == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch\n";
   }
   s << "}\n";
+  if (!single && !ticketed) {
+    // second launch: block j adds the partial sums of sum j, in the same order
+    s << "extern \"C\" __global__ void __launch_bounds__(256) fused_map_sums_final(int g, const unsigned long long* __restrict__ part";
+    for (int j = 0; j < n_sum; ++j) s << ", " << ctype(dt[(size_t)sum_slots[j]]) << "* __restrict__ out" << j;
+    s << ") {\n  __shared__ unsigned long long red[4];\n";
+    for (int j = 0; j < n_sum; ++j) {
+      s << "  if (blockIdx.x == " << j << ") {\n    " << acc_t(j) << " acc = 0;\n";
+      s << "    for (int i = threadIdx.x; i < g; i += 256) acc += *reinterpret_cast<const " << acc_t(j) << "*>(&part[(i64)" << j << " * g + i]);\n";
+      s << "    acc = wave_sum(acc);\n    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = *reinterpret_cast<unsigned long long*>(&acc);\n    __syncthreads();\n";
+      s << "    if (threadIdx.x == 0) {\n      " << acc_t(j) << " t4[4];\n      for (int k = 0; k < 4; ++k) t4[k] = *reinterpret_cast<" << acc_t(j) << "*>(&red[k]);\n";
+      s << "      out" << j << "[0] = (" << ctype(dt[(size_t)sum_slots[j]]) << ")((t4[0] + t4[1]) + (t4[2] + t4[3]));\n    }\n  }\n";
+    }
+    s << "}\n";
+  }
   std::string src = s.str();
 
   const char* label = "fused_map_sums";
@@ -923,9 +982,6 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     if (rc) { drop_part(); release_all(); return rc; }
     it = cache.emplace(src, c).first;
   }
-  hipFunction_t fin = nullptr;
-  hipError_t e = hipModuleGetFunction(&fin, it->second.mod, "fused_map_sums_final");
-  if (e != hipSuccess) { drop_part(); release_all(); return check_hip(ctx, e, "hipModuleGetFunction"); }
   std::vector<void*> args;
   int64_t nn = n;
   args.push_back(&nn);
@@ -935,10 +991,14 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   for (int o = 0; o < n_out; ++o) { optrs[(size_t)o] = data_ptr(res[(size_t)o]); args.push_back(&optrs[(size_t)o]); }
   for (int j = 0; j < n_sum; ++j) sptrs[(size_t)j] = data_ptr(sres[(size_t)j]);
   void* pp = part ? part->ptr : nullptr;
-  if (single) for (int j = 0; j < n_sum; ++j) args.push_back(&sptrs[(size_t)j]);
-  else args.push_back(&pp);
-  e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
-  if (e == hipSuccess && !single) {
+  if (!single) args.push_back(&pp);
+  if (ticketed) args.push_back(&ticket);
+  if (single || ticketed) for (int j = 0; j < n_sum; ++j) args.push_back(&sptrs[(size_t)j]);
+  hipFunction_t fin = nullptr;
+  hipError_t e = hipSuccess;
+  if (!single && !ticketed) e = hipModuleGetFunction(&fin, it->second.mod, "fused_map_sums_final");
+  if (e == hipSuccess) e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e == hipSuccess && fin) {
     int g = (int)grid;
     std::vector<void*> fargs = {&g, &pp};
     for (int j = 0; j < n_sum; ++j) fargs.push_back(&sptrs[(size_t)j]);

@@ -272,6 +272,20 @@ int zero_block(hgpu_ctx* ctx, const void** out) {
   *out = ctx->zero_block->ptr;
   return HGPU_OK;
 }
+
+int ticket_block(hgpu_ctx* ctx, void** out) {
+  if (!ctx->ticket_block) {
+    if (int rc0 = no_capture(ctx, "the first reduction that draws tickets")) return rc0;
+    hgpu_buffer* b = nullptr;
+    int rc = buffer_alloc(ctx, 256, &b);
+    if (rc) return rc;
+    rc = zero_fill(ctx, b->ptr, 256);
+    if (rc) { buffer_release(b); return rc; }
+    ctx->ticket_block = b;
+  }
+  *out = ctx->ticket_block->ptr;
+  return HGPU_OK;
+}
 }  // namespace hg
 
 extern "C" {
@@ -295,6 +309,8 @@ int hgpu_init(int device, hgpu_ctx** out) {
   if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->num_cu = prop.multiProcessorCount;
   const void* z = nullptr;
   (void)zero_block(ctx, &z);     // made now, so that no capture ever owns it
+  void* tk = nullptr;
+  (void)ticket_block(ctx, &tk);
   *out = ctx;
   return HGPU_OK;
 }
@@ -398,6 +414,7 @@ int hgpu_shutdown(hgpu_ctx* ctx) {
   (void)hipStreamSynchronize(ctx->stream);
   forget_remembered_sums(ctx);
   if (ctx->zero_block) { buffer_release(ctx->zero_block); ctx->zero_block = nullptr; }
+  if (ctx->ticket_block) { buffer_release(ctx->ticket_block); ctx->ticket_block = nullptr; }
   {
     std::lock_guard<std::mutex> g(ctx->mu);
     drop_cache_locked(ctx);
