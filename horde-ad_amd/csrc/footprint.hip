@@ -85,6 +85,7 @@ struct Plan {
   int addr_regs;   // per-lane address registers of the kernel
   int nbufs;   // LDS chunk buffers: 2, or 1 when two do not fit (the prefetch then waits in registers)
   int ks = 1;  // wavefronts per SIMD: the block's 4 ks wavefronts split the K groups of a chunk ks ways
+  int64_t colsum_at = -1;   // >= 0: the kernel also sums the columns operand over K, into these elements of its partial result (mode 0)
   int bpc = 1; // blocks that share a CU (their LDS fits together): one's loads and stores run under the other's multiplications
   bool cvec;   // groups of four rows are adjacent in C and 16-byte aligned: vector stores
 };
@@ -250,7 +251,8 @@ constexpr int rem_slots_before(int g) {
 constexpr int RGB = REM > 0 ? (4 / REM > 1 ? 4 / REM : 1) : 1;     // slots per batch of LDS reads
 struct RemOps { T a[RGB][REM > 0 ? REM : 1], b[RGB][REM > 0 ? REM : 1]; };
 constexpr int RED0 = NBUFS * BUF + (MODE == 0 ? 0 : LY);    // scratch for adding up split row blocks
-constexpr int LDS_ELEMS = RED0 + (REM > 0 && KS == 1 ? REM * 4 * 256 : 0);
+constexpr int CS0 = RED0 + (REM > 0 && KS == 1 ? REM * 4 * 256 : 0);   // where the parts' column sums meet
+constexpr int LDS_ELEMS = CS0 + (COLSUM && KS > 1 ? 16 * KS : 0);
 // where the parts' partial products meet (KS > 1): a chunk buffer that has been multiplied; the whole
 // row blocks first, the split ones behind them
 constexpr int XCH = 4 * NBF * (KS - 1) * 256;
@@ -403,6 +405,9 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   // (xch: an area of LDS nobody reads any more); the partial products of the split row blocks, of all
   // 4 KS wavefronts, are added by wavefronts 0 .. REM - 1 of the last part into srem.
   T srem[4] = {T(0), T(0), T(0), T(0)};
+  // COLSUM: wavefront 0 of every part adds up the column operand's fragments as it reads them: lane (r, q4)
+  // the elements k = 4 g + q4 of column r, over the part's K groups g and all the block's chunks
+  T colacc = T(0);
   auto meet = [&](T* xch) {
     if (KS > 1) {
 #pragma unroll
@@ -533,6 +538,9 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
           constexpr bool tail = gi == NG - 1 && KVALID < 4;
           T bv = LYp[by[p] + gy];
           if (tail && tail_lane) bv = T(0);
+#if COLSUM
+          if (wave == 0) colacc += bv;
+#endif
 #pragma unroll
           for (int t = 0; t < NBF; ++t) {
             T av = L[ax[t][p] + gx];
@@ -670,9 +678,24 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   }
 #if !EPI
   if (MODE == 0) {
+#if COLSUM
+    if (wave == 0) {
+      colacc += __shfl_xor(colacc, 16);
+      colacc += __shfl_xor(colacc, 32);
+      if (KS > 1 && q4 == 0) lds[CS0 + KH * 16 + r] = colacc;
+    }
+#endif
     if (KS > 1 || REM > 0) __syncthreads();      // all multiplications are done: the chunk buffers are free
     meet(lds);
     T* out = C + (i64)blockIdx.x * part_stride;
+#if COLSUM
+    if (KH == 0 && wave == 0 && q4 == 0 && r < NIN) {
+      T tot = colacc;
+#pragma unroll
+      for (int h = 1; h < KS; ++h) tot += lds[CS0 + h * 16 + r];
+      out[COLSUM + r - 1] = tot;       // COLSUM - 1: where the column sums start in a block's partial result
+    }
+#endif
 #pragma unroll
     for (int t = 0; t < NBF; ++t)
       if (t % KS == KH) store_rows(out, out_pos((wave + 4 * t) * 16 + 4 * q4, r), (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
@@ -715,7 +738,7 @@ std::string generate(const Plan& pl, const std::string& kname, const std::string
   s << "#define VIRT_Y " << (virt_y.empty() ? 0 : 1) << "\n#define YBASE " << ybase << "ll\n";
   s << "#define EPI " << (epilogue.empty() ? 0 : 1) << "\n#define EPI_STAGE " << stage_bytes << "\n#define BPC " << pl.bpc << "\n";
   const int es = pl.f64 ? 8 : 4;
-  s << "#define F64 " << (pl.f64 ? 1 : 0) << "\n#define KS " << pl.ks << "\n";
+  s << "#define F64 " << (pl.f64 ? 1 : 0) << "\n#define KS " << pl.ks << "\n#define COLSUM " << (pl.colsum_at >= 0 ? pl.colsum_at + 1 : 0) << "\n";
   s << "#define MODE " << pl.mode << "\n";
   s << "#define MIN " << pl.min_rows << "\n#define NIN " << pl.nin << "\n#define NG " << pl.gx.size() << "\n";
   s << "#define NPAT " << pl.px.size() << "\n#define KVALID " << pl.kvalid << "\n";
@@ -1042,6 +1065,10 @@ bool finish_plan(Plan& pl, const char* xp, const char* yp, const char* cp, int64
 
 }  // namespace
 
+namespace {
+void remember_sum(hgpu_ctx* ctx, const VirtualOp& v, const std::vector<int>& kept, hgpu_array* sum);
+}
+
 namespace hg {
 
 // gemm.hip: out[i] = sum over the `parts` partial outputs of part[s * n + i], in a fixed order.
@@ -1104,11 +1131,40 @@ int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const v
     }
   }
   if (!found) return HGPU_OK;
-  const Plan& pl = best;
+  Plan& pl = best;
   // the kernel's name tells a profiler which product it is
   char kname[128];
   const VirtualOp* vx = best_swapped ? vb : va;
   const VirtualOp* vy = best_swapped ? va : vb;
+  // The columns operand an expression, summed over K by the same kernel: the sum of the expression over
+  // every merged dim but the columns' (a bias's cotangent next to the kernel's), for the caller who asks next.
+  std::vector<int> colsum_dims;
+  std::vector<int64_t> colsum_shape;
+  if (vy && pl.mode == 0 && (pl.min_rows + 15) / 16 >= 4 && (best_swapped ? pa : pb) == nullptr && !vy->padded) {
+    const std::vector<Dim> cd = dims(best_swapped ? p.m : p.n, best_swapped), kd = dims(p.k, best_swapped);
+    const size_t rm = vy->M.size();
+    std::vector<int64_t> DM(rm, 1);
+    for (size_t k = rm; k-- > 1;) DM[k - 1] = DM[k] * vy->M[k];
+    std::vector<char> covered(rm, 0);
+    bool ok = true;
+    auto match = [&](const std::vector<Dim>& ds, bool keep) {
+      for (auto& d : ds) {
+        if (d.e == 1) continue;
+        int hit = -1;
+        for (size_t k = 0; k < rm; ++k)
+          if (vy->M[k] > 1 && !covered[k] && DM[k] == d.sy && vy->M[k] == d.e) { hit = (int)k; break; }
+        if (hit < 0) { ok = false; return; }
+        covered[(size_t)hit] = 1;
+        if (keep) { colsum_dims.push_back(hit); colsum_shape.push_back(d.e); }
+      }
+    };
+    match(cd, true);
+    if (ok) match(kd, false);
+    for (size_t k = 0; k < rm && ok; ++k)
+      if (vy->M[k] > 1 && !covered[k]) ok = false;
+    if (ok && !colsum_dims.empty()) pl.colsum_at = nelem(out);
+    else { colsum_dims.clear(); colsum_shape.clear(); }
+  }
   snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_%s%s%s%s%s", f64 ? "f64" : "f32", (long long)p.M, (long long)p.N, (long long)p.K,
            pl.mode == 0 ? "chunkK" : "chunkM", best_swapped ? "_swapped" : "", vx ? "_xmap" : "", vy ? "_ymap" : "", pl.ks == 2 ? "_w8" : "");
   const int64_t xbase = (int64_t)((uintptr_t)((const char*)(best_swapped ? pb : pa) + pl.shift_x * es) / (uintptr_t)es);
@@ -1134,11 +1190,17 @@ int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const v
   hgpu_buffer* part = nullptr;
   void* cdst = data_ptr(out);
   int64_t part_stride = 0;
+  const int64_t n_colsum = pl.colsum_at >= 0 ? pl.nin : 0;
+  hgpu_array* colsum = nullptr;
   if (pl.mode == 0) {
-    int rc = buffer_alloc(ctx, (size_t)out_n * (size_t)grid * es, &part);
-    if (rc) return rc;
+    if (n_colsum > 0) {
+      int rc = new_dense(ctx, dtype, (int)colsum_shape.size(), colsum_shape.data(), &colsum);
+      if (rc) return rc;
+    }
+    int rc = buffer_alloc(ctx, (size_t)(out_n + n_colsum) * (size_t)grid * es, &part);
+    if (rc) { if (colsum) hgpu_release(colsum); return rc; }
     cdst = part->ptr;
-    part_stride = out_n;
+    part_stride = out_n + n_colsum;
   }
   int64_t nch = pl.nch, chx = pl.chx, chy = pl.chy, chc = pl.chc;
   // the inputs of an expression operand follow as one struct of pointers each
@@ -1162,12 +1224,14 @@ int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const v
     {
       LaunchGuard lg(ctx, label, bytes, flops);
       hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256u * (unsigned)pl.ks, 1, 1, 0, ctx->stream, args.data(), nullptr);
-      if (e != hipSuccess) { if (part) buffer_release(part); return check_hip(ctx, e, "footprint gemm launch"); }
+      if (e != hipSuccess) { if (part) buffer_release(part); if (colsum) hgpu_release(colsum); return check_hip(ctx, e, "footprint gemm launch"); }
     }
     if (pl.mode == 0) {
-      int rc = sum_partials(ctx, dtype, out_n, (int)grid, (const void*)part->ptr, data_ptr(out));
+      int rc = colsum ? sum_partials_split(ctx, dtype, out_n, n_colsum, (int)grid, (const void*)part->ptr, data_ptr(out), data_ptr(colsum))
+                      : sum_partials(ctx, dtype, out_n, (int)grid, (const void*)part->ptr, data_ptr(out));
       buffer_release(part);
-      if (rc) return rc;
+      if (rc) { if (colsum) hgpu_release(colsum); return rc; }
+      if (colsum) remember_sum(ctx, *vy, colsum_dims, colsum);
     }
   }
   *handled = true;
