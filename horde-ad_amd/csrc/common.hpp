@@ -87,7 +87,7 @@ struct hgpu_ctx {
   std::mutex label_mu;                    // guards label_pool: labels are made on any calling thread
   std::vector<ProfRec> prof;
   hgpu_buffer* zero_block = nullptr;     // 256 zero bytes, for kernels that want a dummy table
-  hgpu_buffer* ticket_block = nullptr;   // a counter (zero between launches) for kernels whose last block finishes a reduction
+  hgpu_buffer* ticket_block = nullptr;   // counters (zero between launches) for kernels whose last block finishes a reduction
   hgpu_cap_pool* cap = nullptr;          // non-null while the stream is capturing into a graph
   // Small products whose launch is held back until something else needs the
   // stream: those that do not depend on one another then go out as one kernel.
@@ -123,8 +123,9 @@ int check_hip(hgpu_ctx* ctx, hipError_t e, const char* what);
 // Allocator (runtime.hip).
 int buffer_alloc(hgpu_ctx* ctx, size_t bytes, hgpu_buffer** out);
 int zero_block(hgpu_ctx* ctx, const void** out);   // a context-lifetime block of 256 zero bytes
-// A context-lifetime counter for kernels whose blocks draw tickets (the last one finishes the reduction and sets the
-// counter back to zero).  Launches on the context's stream follow one another, so one counter serves them all.
+// Context-lifetime counters (1024 of 32 bits, zero between launches) for kernels whose blocks draw tickets: the
+// last one finishes the reduction and sets its counter back to zero.  Launches on the context's stream follow one
+// another, so the same counters serve them all.
 int ticket_block(hgpu_ctx* ctx, void** out);
 // Fails (HGPU_ERR_UNSUPPORTED) when the stream is capturing: for entry points that must talk to the host.
 int no_capture(hgpu_ctx* ctx, const char* what);

@@ -277,9 +277,9 @@ int ticket_block(hgpu_ctx* ctx, void** out) {
   if (!ctx->ticket_block) {
     if (int rc0 = no_capture(ctx, "the first reduction that draws tickets")) return rc0;
     hgpu_buffer* b = nullptr;
-    int rc = buffer_alloc(ctx, 256, &b);
+    int rc = buffer_alloc(ctx, 4096, &b);
     if (rc) return rc;
-    rc = zero_fill(ctx, b->ptr, 256);
+    rc = zero_fill(ctx, b->ptr, 4096);
     if (rc) { buffer_release(b); return rc; }
     ctx->ticket_block = b;
   }

@@ -108,6 +108,10 @@ struct Spec {
   std::vector<int64_t> in_sp, in_sq;
   std::vector<int> out_slots;
   int x_elems, y_elems;    // LDS elements of the largest X / Y tile
+  // K shared out between `splits` blocks per tile (few tiles, long K: the blocks of one tile run side by side
+  // instead of one block walking all of K); each block writes its partial tile, and a second launch of one block
+  // per tile adds the partial tiles up in the order of K and runs the program
+  int splits = 1, chunks_per_split = 0;
 };
 
 // LDS pitch of a tile: the fragment reads of 16 rows x 4 k must not collide.
@@ -196,7 +200,8 @@ std::string generate_body(const Spec& sp) {
   std::ostringstream s;
   const int TP = sp.BP / (16 * sp.WP), TQ = sp.BQ / (16 * sp.WQ);
   const int64_t nbp = (sp.P + sp.BP - 1) / sp.BP, nbq = (sp.Q + sp.BQ - 1) / sp.BQ;
-  const int64_t nblk = nbp * nbq, per_xcd = (nblk + 7) / 8;
+  const int S = sp.splits;
+  const int64_t nblk = nbp * nbq, per_xcd = (nblk * S + 7) / 8;
   const bool vec_epi = !sp.f64 && sp.P % 4 == 0;
   s << "typedef " << (sp.f64 ? "double" : "float") << " T;\n";
   s << "typedef T V2 __attribute__((ext_vector_type(2), aligned(" << (sp.f64 ? 8 : 4) << ")));\n";
@@ -210,6 +215,7 @@ std::string generate_body(const Spec& sp) {
   for (int i = 0; i < sp.n_in; ++i)
     if (i != sp.c_slot) s << "  const " << ctype(sp.dt[(size_t)i]) << "* i" << i << ";\n";
   for (size_t o = 0; o < sp.out_slots.size(); ++o) s << "  " << ctype(sp.dt[(size_t)sp.out_slots[o]]) << "* o" << o << ";\n";
+  if (sp.splits > 1) s << "  T* part;\n";
   s << "};\n";
   for (size_t c = 0; c < sp.chunks.size(); ++c) {
     emit_stage_fn(s, ("x" + std::to_string(c)).c_str(), sp.chunks[c].x, sp.chunks[c], "", "");
@@ -321,8 +327,14 @@ std::string generate_body(const Spec& sp) {
   s << "__device__ __forceinline__ void body(const Args& ar, unsigned bid, T* __restrict__ lds) {\n";
   s << "  T* const xs = lds;\n  T* const ys = lds + " << sp.x_elems << ";\n";
   // consecutive block ids go round the eight XCDs: blocks that share operand tiles get ids of one XCD
-  s << "  const i64 blk = (i64)(bid % 8) * " << per_xcd << "LL + bid / 8;\n";
-  s << "  if (blk >= " << nblk << "LL) return;\n";
+  if (S == 1) {
+    s << "  const i64 blk = (i64)(bid % 8) * " << per_xcd << "LL + bid / 8;\n";
+    s << "  if (blk >= " << nblk << "LL) return;\n";
+  } else {
+    s << "  const i64 blk_all = (i64)(bid % 8) * " << per_xcd << "LL + bid / 8;\n";
+    s << "  if (blk_all >= " << nblk * S << "LL) return;\n";
+    s << "  const i64 blk = blk_all / " << S << ";\n  const int sidx = (int)(blk_all % " << S << ");\n";
+  }
   s << "  const i64 q0 = (blk % " << nbq << "LL) * " << sp.BQ << ", p0 = (blk / " << nbq << "LL) * " << sp.BP << ";\n";
   s << "  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r = lane & 15, g = lane >> 4;\n";
   s << "  const int wp = w % " << sp.WP << ", wq = w / " << sp.WP << ";\n";
@@ -334,22 +346,53 @@ std::string generate_body(const Spec& sp) {
     int t = sp.chunks[c].term;
     s << "  load_x" << c << "(rx" << c << ", ar.x" << t << ", p0, tid);\n  load_y" << c << "(ry" << c << ", ar.y" << t << ", q0, tid);\n";
   };
-  load(0);
   int n_read = 0;
   for (int i = 0; i < sp.n_in; ++i) n_read += i != sp.c_slot;
-  const bool prefetch = n_read > 0 && n_read * TP * TQ <= 16;
+  const bool prefetch = S == 1 && n_read > 0 && n_read * TP * TQ <= 16;
   if (n_read > 0) s << "  EpiIn ei[" << TP << "][" << TQ << "];\n";
   auto epi_loads = [&]() {
     s << "#pragma unroll\n  for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n    for (int b = 0; b < " << TQ << "; ++b)\n";
     s << "      ei[a][b] = epi_load(ar, p0 + (wp * " << TP << " + a) * 16, q0 + (wq * " << TQ << " + b) * 16, r, g);\n";
   };
-  if (prefetch) epi_loads();
-  for (size_t c = 0; c < nc; ++c) {
-    const Chunk& ch = sp.chunks[c];
-    s << "  store_x" << c << "(rx" << c << ", xs, tid);\n  store_y" << c << "(ry" << c << ", ys, tid);\n  __syncthreads();\n";
-    if (c + 1 < nc) load(c + 1);
-    s << "  compute<" << ch.kcp << ", " << ch.x.layout << ", " << ch.x.pitch << ", " << ch.y.layout << ", " << ch.y.pitch << ">(xs, ys, acc, r, g, wp, wq);\n";
-    if (c + 1 < nc) s << "  __syncthreads();\n";
+  auto run_chunks = [&](size_t c0, size_t c1) {
+    load(c0);
+    if (prefetch) epi_loads();
+    for (size_t c = c0; c < c1; ++c) {
+      const Chunk& ch = sp.chunks[c];
+      s << "  store_x" << c << "(rx" << c << ", xs, tid);\n  store_y" << c << "(ry" << c << ", ys, tid);\n  __syncthreads();\n";
+      if (c + 1 < c1) load(c + 1);
+      s << "  compute<" << ch.kcp << ", " << ch.x.layout << ", " << ch.x.pitch << ", " << ch.y.layout << ", " << ch.y.pitch << ">(xs, ys, acc, r, g, wp, wq);\n";
+      if (c + 1 < c1) s << "  __syncthreads();\n";
+    }
+  };
+  if (S == 1) {
+    run_chunks(0, nc);
+  } else {
+    for (int sp_i = 0; sp_i < S; ++sp_i) {
+      const size_t c0 = (size_t)sp_i * (size_t)sp.chunks_per_split, c1 = std::min(nc, c0 + (size_t)sp.chunks_per_split);
+      s << (sp_i ? "  else if" : "  if") << " (sidx == " << sp_i << ") {\n";
+      run_chunks(c0, c1);
+      s << "  }\n";
+    }
+    // hand the partial tile over: the registers of a lane side by side for the block's 256 lanes
+    const int nreg = TP * TQ * 4;
+    s << "  {\n    T* mine = ar.part + ((blk * " << S << " + sidx) * " << nreg << "LL) * 256 + tid;\n";
+    s << "#pragma unroll\n    for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n      for (int b = 0; b < " << TQ << "; ++b)\n#pragma unroll\n        for (int e = 0; e < 4; ++e) {\n";
+    s << "          mine[((a * " << TQ << " + b) * 4 + e) * 256] = acc[a][b][e];\n        }\n  }\n";
+    s << "}\n";
+    // The second launch: one block per tile adds the partial tiles up, in the order of K, and runs the program.
+    s << "__device__ __forceinline__ void finish(const Args& ar, unsigned bid) {\n";
+    s << "  const i64 blk = (i64)(bid % 8) * " << (nblk + 7) / 8 << "LL + bid / 8;\n";
+    s << "  if (blk >= " << nblk << "LL) return;\n";
+    s << "  const i64 q0 = (blk % " << nbq << "LL) * " << sp.BQ << ", p0 = (blk / " << nbq << "LL) * " << sp.BP << ";\n";
+    s << "  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r = lane & 15, g = lane >> 4;\n";
+    s << "  const int wp = w % " << sp.WP << ", wq = w / " << sp.WP << ";\n";
+    s << "  Acc acc[" << TP << "][" << TQ << "];\n";
+    if (n_read > 0) s << "  EpiIn ei[" << TP << "][" << TQ << "];\n";
+    s << "#pragma unroll\n  for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n    for (int b = 0; b < " << TQ << "; ++b) acc[a][b] = Acc{0, 0, 0, 0};\n";
+    s << "  for (int sj = 0; sj < " << S << "; ++sj) {\n    const T* theirs = ar.part + ((blk * " << S << " + sj) * " << nreg << "LL) * 256 + tid;\n";
+    s << "#pragma unroll\n    for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n      for (int b = 0; b < " << TQ << "; ++b)\n#pragma unroll\n        for (int e = 0; e < 4; ++e)\n";
+    s << "          acc[a][b][e] += theirs[((a * " << TQ << " + b) * 4 + e) * 256];\n  }\n";
   }
   if (n_read > 0 && !prefetch) epi_loads();
   s << "#pragma unroll\n  for (int a = 0; a < " << TP << "; ++a)\n#pragma unroll\n    for (int b = 0; b < " << TQ << "; ++b)\n";
@@ -363,7 +406,8 @@ std::string generate_body(const Spec& sp) {
 // first blocks run problem 0, the next ones problem 1, ...  (`grids[k]` blocks
 // each, multiples of 8 so that every problem's block ids keep their place in
 // the round of the XCDs).  A single problem gives the kernel of that problem.
-std::string kernel_source(const std::vector<const std::string*>& bodies, const std::vector<unsigned>& grids, const std::vector<int>& lds_bytes, const std::string& kname) {
+std::string kernel_source(const std::vector<const std::string*>& bodies, const std::vector<unsigned>& grids, const std::vector<int>& lds_bytes, const std::string& kname,
+                          bool with_finish = false) {
   std::ostringstream s;
   s << kPrelude;
   int lds = 16;
@@ -384,6 +428,8 @@ std::string kernel_source(const std::vector<const std::string*>& bodies, const s
     first += grids[k];
   }
   s << "}\n";
+  // a single problem whose K is shared out between blocks: the launch that adds the partial tiles up
+  if (with_finish) s << "extern \"C\" __global__ void __launch_bounds__(256) " << kname << "_finish(GroupArgs ar) { g0::finish(ar.a0, blockIdx.x); }\n";
   return s.str();
 }
 
@@ -504,8 +550,8 @@ bool fits_int(int64_t v) { return v > -(1LL << 40) && v < (1LL << 40); }
 
 // The kernel over the given problems, compiled once per source text; nullptr when the compiler refuses it.
 hipFunction_t compiled_kernel(hgpu_ctx* ctx, const std::vector<const std::string*>& bodies, const std::vector<unsigned>& grids, const std::vector<int>& lds_bytes,
-                              const std::string& kname) {
-  std::string src = kernel_source(bodies, grids, lds_bytes, kname);
+                              const std::string& kname, hipFunction_t* finish_fn = nullptr) {
+  std::string src = kernel_source(bodies, grids, lds_bytes, kname, finish_fn != nullptr);
   auto& cache = cache_of(ctx);
   auto it = cache.find(src);
   if (it == cache.end()) {
@@ -519,6 +565,10 @@ hipFunction_t compiled_kernel(hgpu_ctx* ctx, const std::vector<const std::string
       if (e != hipSuccess) c = Compiled{nullptr, nullptr};
     }
     it = cache.emplace(src, c).first;
+  }
+  if (finish_fn) {
+    *finish_fn = nullptr;
+    if (it->second.fn && hipModuleGetFunction(finish_fn, it->second.mod, (kname + "_finish").c_str()) != hipSuccess) return nullptr;
   }
   return it->second.fn;
 }
@@ -604,21 +654,37 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
   sp.out_slots.assign(out_slots, out_slots + n_out);
   choose_tile(ctx, sp, ktot);
   if (!plan_chunks(sp)) return HGPU_OK;
+  const int64_t ntiles = ((sp.P + sp.BP - 1) / sp.BP) * ((sp.Q + sp.BQ - 1) / sp.BQ);
+  {
+    // Fewer tiles than three quarters of the CUs and a long K (a dense layer's weight gradient, 784 x 128 over
+    // a batch of 1000: 98 tiles of 16 chunks): K is shared out so that about two blocks per CU run.  Short K
+    // (the steps of a recurrence) stays whole: those products are held back and grouped instead.
+    static const bool no_split = getenv("HORDEAD_SMALLK_NOSPLIT") != nullptr;
+    const int nc = (int)sp.chunks.size();
+    if (!no_split && ntiles * 4 < (int64_t)ctx->num_cu * 3 && nc >= 8) {
+      int want = (int)std::min<int64_t>(nc / 2, (2 * (int64_t)ctx->num_cu + ntiles - 1) / ntiles);
+      if (want >= 2) {
+        sp.chunks_per_split = (nc + want - 1) / want;
+        sp.splits = (nc + sp.chunks_per_split - 1) / sp.chunks_per_split;
+      }
+    }
+  }
 
   char kname[96];
   snprintf(kname, sizeof kname, "smallk_%s_p%lld_q%lld_k%lld_t%d_in%d_instr%d_out%d", sp.f64 ? "f64" : "f32", (long long)sp.P, (long long)sp.Q, (long long)ktot, n_terms, n_in - 1,
            n_instr, n_out);
   Deferred d;
+  hipFunction_t finish_fn = nullptr;
   d.body = generate_body(sp);
   d.kname = kname;
-  const int64_t nblk = ((sp.P + sp.BP - 1) / sp.BP) * ((sp.Q + sp.BQ - 1) / sp.BQ);
+  const int64_t nblk = ntiles * sp.splits;
   const int64_t grid = (nblk + 7) / 8 * 8;
   if (grid > 0x7fffffff) return HGPU_OK;
   d.grid = (unsigned)grid;
   d.lds_bytes = (sp.x_elems + sp.y_elems) * (sp.f64 ? 8 : 4);
   {
     std::lock_guard<std::mutex> lk(ctx->launch_mu);   // the kernel cache is shared with the thread that launches what is held back
-    d.fn = compiled_kernel(ctx, {&d.body}, {d.grid}, {d.lds_bytes}, d.kname);
+    d.fn = compiled_kernel(ctx, {&d.body}, {d.grid}, {d.lds_bytes}, d.kname, sp.splits > 1 ? &finish_fn : nullptr);
   }
   if (!d.fn) return HGPU_OK;
 
@@ -627,6 +693,12 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
     if (i != c_slot) d.args.push_back(data_ptr(in[i]));
   for (int o = 0; o < n_out; ++o) d.args.push_back(data_ptr(outs[o]));
   const double es = sp.f64 ? 8 : 4;
+  hgpu_buffer* part = nullptr;
+  if (sp.splits > 1) {
+    int rc = buffer_alloc(ctx, (size_t)nblk * (size_t)sp.BP * (size_t)sp.BQ * (size_t)es, &part);
+    if (rc) return rc;
+    d.args.push_back(part->ptr);
+  }
   d.flops = 2.0 * (double)sp.P * sp.Q * ktot;
   d.bytes = ((double)sp.P + sp.Q) * ktot * es;
   for (int i = 0; i < n_in; ++i)
@@ -637,12 +709,14 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
     char buf[200];
     std::string ks;
     for (auto& tm : sp.terms) ks += (ks.empty() ? "" : "+") + std::to_string(tm.K);
-    snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%sxB1,wholeK,t%dx%d,chunks%d,lds%dK,map(in%d,instr%d,out%d)]", d.label, (long long)sp.Q, (long long)sp.P, ks.c_str(), sp.BQ,
-             sp.BP, (int)sp.chunks.size(), (int)((sp.x_elems + sp.y_elems) * (int)es / 1024), n_in - 1, n_instr, n_out);
+    char splits[24] = "";
+    if (sp.splits > 1) snprintf(splits, sizeof splits, ",splits%d", sp.splits);
+    snprintf(buf, sizeof buf, "%s[M%lldxN%lldxK%sxB1,wholeK,t%dx%d,chunks%d%s,lds%dK,map(in%d,instr%d,out%d)]", d.label, (long long)sp.Q, (long long)sp.P, ks.c_str(), sp.BQ,
+             sp.BP, (int)sp.chunks.size(), splits, (int)((sp.x_elems + sp.y_elems) * (int)es / 1024), n_in - 1, n_instr, n_out);
     d.label = intern_label(ctx, buf);
   }
   static const bool hold = getenv("HORDEAD_NO_GROUPED_LAUNCH") == nullptr;
-  if (hold && nblk <= kGroupBlocksPerCu * ctx->num_cu) {
+  if (hold && sp.splits == 1 && nblk <= kGroupBlocksPerCu * ctx->num_cu) {
     // held back: the next small products may be independent of this one
     for (int t = 0; t < n_terms; ++t) { d.reads.push_back(as[t]->buf); d.reads.push_back(bs[t]->buf); }
     for (int i = 0; i < n_in; ++i)
@@ -661,6 +735,8 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
   LaunchGuard lg(ctx, d.label, d.bytes, d.flops);
   void* args[] = {(void*)d.args.data()};
   hipError_t err = hipModuleLaunchKernel(d.fn, d.grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+  if (err == hipSuccess && finish_fn) err = hipModuleLaunchKernel(finish_fn, (unsigned)((ntiles + 7) / 8 * 8), 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+  if (part) buffer_release(part);
   if (err != hipSuccess) return check_hip(ctx, err, "small-K product launch");
   *handled = true;
   return HGPU_OK;
