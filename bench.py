@@ -223,6 +223,51 @@ def cpu_baseline(pkg, key, mk):
             "sample": f"{wl.name} at {CPU_SAMPLE[key]} ({wl.batch} samples per gradient, {n} gradients, {dt:.3f} s each)"}
 
 
+def index_micro(capi, which, steps, warmup):
+    """One index kernel at a stated size, through the array-level entry points.
+
+    gather_units: 100 MB of 1 KiB slices picked by a data-dependent index vector (the general gather, 16-byte units).
+    scatter_sorted: 12.5 M single elements added into 3.1 M cells, four to a cell as in the adjoint of 2 x 2 pooling
+    over [1000, 16, 28, 28], the cells given as data (the general path: sort by destination, add each run in order).
+    Algorithmic bytes: what is read plus what is written, the index vector included."""
+    import numpy as np
+    ctx = capi.Lib().context(0)
+    rng = np.random.default_rng(3)
+    if which == "gather_units":
+        rows, width = 100_000, 128                    # 1 KiB slices of doubles
+        src = ctx.upload(rng.standard_normal((rows, width)))
+        ix = [ctx.upload(rng.integers(0, rows, rows).astype(np.int64))]
+        call = lambda: ctx.gather(src, ix, [rows])
+        alg = 2.0 * rows * width * 8 + 8.0 * rows
+        what = "gather of 100000 slices of 1 KiB from [100000, 128] f64 by an index vector"
+    else:
+        b, c, h, w = 1000, 16, 28, 28
+        m = b * c * h * w
+        pos = np.arange(m, dtype=np.int64).reshape(b, c, h // 2, 2, w // 2, 2)
+        cells_np = np.broadcast_to(np.arange(m // 4, dtype=np.int64).reshape(b, c, h // 2, 1, w // 2, 1), pos.shape).reshape(-1).copy()
+        src = ctx.upload(rng.standard_normal(m))
+        ix = [ctx.upload(cells_np)]
+        call = lambda: ctx.scatter_add(src, ix, 1, [m // 4])
+        alg = 8.0 * m + 8.0 * m + 8.0 * (m // 4)
+        what = "scatter-add of 12544000 f64 into 3136000 cells (four to a cell), cells given as an index vector"
+    for _ in range(max(1, warmup)):
+        o = call()
+        del o
+    ctx.sync()
+    ctx.profile(2)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = call()
+        del o
+    ctx.sync()
+    sec = (time.perf_counter() - t0) / steps
+    rep = ctx.profile_report()
+    ctx.profile(0)
+    kernels = {k: {"launches_per_call": v[0] / steps, "avg_us": v[1] / v[0] * 1e3} for k, v in rep.items() if v[0]}
+    return {"micro": which, "what": what, "ms_per_call": sec * 1e3, "algorithmic_mb": alg / 1e6, "achieved_gbs": alg / sec / 1e9,
+            "frac_of_hbm_peak": alg / sec / 1e9 / HBM_PEAK_GBS, "kernels": kernels}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -238,6 +283,8 @@ def main():
                     help="time loops of single matrix-core instructions (the ceiling of the product kernels) and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run plain dense copies of 1 GiB (for scaling hardware traffic counters) and exit")
+    ap.add_argument("--micro", choices=["gather_units", "scatter_sorted", "riders"],
+                    help="time one index kernel at a stated size (its algorithmic bytes over its launch time) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus,
@@ -272,7 +319,22 @@ def main():
         ctx.sync()
         print(json.dumps({"calibration": "5 dense copies", "bytes_read_per_copy": 1 << 30, "bytes_written_per_copy": 1 << 30}))
         return
+    if args.micro in ("gather_units", "scatter_sorted"):
+        print(json.dumps(index_micro(capi, args.micro, args.steps, args.warmup)))
+        return
     host = H.Host()      # raises when the HIP library is missing or no device is usable
+    if args.micro == "riders":
+        out = {}
+        for key, make in W.RIDERS.items():
+            if key == "c3_artifact_form":
+                continue
+            wl = make()
+            ps, ds = wl.upload(host)
+            eager_sec, loss = time_steps(host, wl, ps, ds, args.steps, args.warmup)
+            rep = profile(capi, host, wl, ps, ds)
+            out[key] = {"workload": wl.name, "ms_per_call_eager": eager_sec * 1e3, "algorithmic_mb": wl.bytes / 1e6, "kernels": kernel_table(rep, DTYPE_NAME[wl.dtype])}
+        print(json.dumps({"micro": "riders", "results": out}))
+        return
 
     keys = [args.workload] if args.only else [args.workload] + [k for k in W.CONFIGS if k != args.workload]
     results = {}
