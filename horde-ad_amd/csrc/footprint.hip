@@ -2390,8 +2390,7 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   emit_program(s, v.n_in, v.n_instr, v.prog, v.dt, "          ", "_");
   s << "          const T val = ok[it] ? v" << v.slot << "_ : T(0);\n";
   s << "          const T* xp = xs + kGX[gg[it]] + kOhX[ee[it]];\n";
-  static const int knob_nofma = getenv("HORDEAD_ONEHOT_NOFMA") ? atoi(getenv("HORDEAD_ONEHOT_NOFMA")) : 0;
-  for (int m = 0; m < (knob_nofma ? 1 : MR); ++m) s << "          acc[" << m << "] += val * xp[" << rx[(size_t)m] - rlo << "];\n";
+  for (int m = 0; m < MR; ++m) s << "          acc[" << m << "] += val * xp[" << rx[(size_t)m] - rlo << "];\n";
   s << "          acc[" << MR << "] += val;\n";
   s << "        }\n      }\n    }\n  }\n";
   // the threads of a column add up, a few rows of the result per round; thread (row, column) writes the block's partial result
