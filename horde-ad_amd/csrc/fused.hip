@@ -644,9 +644,9 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     if (rc) { hgpu_release(o); return rc; }
   }
   auto drop_part = [&] { if (part) buffer_release(part); };
-  // Up to a million elements the block that finishes last adds the blocks' sums up; beyond, a second launch does
+  // Up to 131072 elements (at most a few hundred blocks) the block that finishes last adds the blocks' sums up; beyond, a second launch does
   // (handing a sum over takes a fence per block, and the thousands of blocks of a large array would each pay it).
-  const bool ticketed = !single && n <= (1 << 20);
+  const bool ticketed = !single && n <= (1 << 17);
   void* ticket = nullptr;
   if (ticketed) {
     rc = ticket_block(ctx, &ticket);
@@ -844,10 +844,10 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     if (rc) { release_all(); return rc; }
   }
   auto drop_part = [&] { if (part) buffer_release(part); };
-  // Up to a million elements the block that finishes last adds the blocks' sums up; beyond, a second launch
+  // Up to 131072 elements (at most a few hundred blocks) the block that finishes last adds the blocks' sums up; beyond, a second launch
   // does (handing the sums over takes a fence per block, which also waits for the block's share of the outputs
   // to leave the cache: 16.8 M elements with three outputs take 0.42 ms that way, 0.18 ms with two launches).
-  const bool ticketed = !single && n <= (1 << 20);
+  const bool ticketed = !single && n <= (1 << 17);
   void* ticket = nullptr;
   if (ticketed) {
     rc = ticket_block(ctx, &ticket);

@@ -305,6 +305,27 @@ def test_fused_sum_equals_program_then_sum(gpu, dt):
     assert e.value.code == 4
 
 
+def test_fused_sum_is_finished_three_ways(gpu):
+    """Up to 1024 vectors one block writes the sum; up to 131072 elements the block that draws the last
+    ticket adds the blocks' sums; beyond, a second launch does.  Every size is summed twice in a row and
+    again after the others (the ticket counter must be back at zero): the same bits each time, and the
+    exact integer sum."""
+    O2 = capi.OP2
+    prog = [(1, O2["mul"], 0, 0, 1, 0)]
+    sizes = [2048, 2049, 60000, 131072, 131073, 600000]
+    data = {n: (rnd((n,), np.float64), rnd((n,), np.float64)) for n in sizes}
+    first = {}
+    for rnd_no in range(3):
+        for n in sizes if rnd_no != 1 else reversed(sizes):
+            a, b = data[n]
+            ins = [gpu.upload(a), gpu.upload(b)]
+            got = float(gpu.fused_sum(ins, prog, 2).numpy())
+            assert abs(got - float((a * b).sum())) <= 1e-10 * float(np.abs(a * b).sum())
+            assert first.setdefault(n, got) == got, (n, rnd_no)
+            ia, ib = (a * 1000).astype(np.int64), (b * 1000).astype(np.int64)
+            assert int(gpu.fused_sum([gpu.upload(ia), gpu.upload(ib)], prog, 2).numpy()) == int((ia * ib).sum())
+
+
 @pytest.mark.parametrize("dt", [np.float64, np.float32, np.int32])
 def test_fused_extremum_equals_program_then_extremum(gpu, dt):
     """The extremum of a program's result over its trailing dims, taken on the

@@ -103,6 +103,39 @@ def test_sorted_scatter_inside_a_recording(host):
         graph.free()
 
 
+def test_sums_finished_by_the_last_block_inside_a_recording(host):
+    """An objective's value and its cotangent from one pass over [10, 5000] (the sums of that pass are added up
+    by the block that draws the last ticket, and the counter goes back to zero in the same kernel): every replay
+    against the eager result, with eager sums of other sizes between the replays."""
+    rng = np.random.default_rng(33)
+    u = host.concrete(rng.uniform(-2, 2, (10, 5000)))
+    t = host.concrete(rng.uniform(0, 1, (10, 5000)))
+    other = host.concrete(rng.uniform(-1, 1, (300, 77)))
+
+    def program():
+        e = (u - 0.5).op1("exp")
+        r = e.ssum0().op1("recip")
+        soft = r.sreplicate0N(u.shape) * e
+        return (soft - t) * 2.0, -(soft.op1("log").sdot0(t))     # the cotangent first: its pass takes the value's sum along
+
+    def eager():
+        cot, loss = program()
+        c = cot.numpy()
+        return loss.numpy(), c
+
+    want = eager()
+    graph, (cot, loss) = host.capture(program)
+    try:
+        for replay in range(3):
+            graph.launch()
+            host.sync()
+            assert np.array_equal(cot.numpy(), want[1]) and np.array_equal(loss.numpy(), want[0]), replay
+            (other * other).ssum0().numpy()
+            (other.op1("sin")).ssum0().numpy()
+    finally:
+        graph.free()
+
+
 def test_host_calls_refused_while_recording(host):
     x = host.concrete(np.arange(6.0).reshape(2, 3))
     y = (x * x).ssum0()
