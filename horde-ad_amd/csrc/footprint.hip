@@ -2352,23 +2352,34 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
     else if (rep[(size_t)i] == i) s << "  const int c" << i << " = kCol" << i << "[cq];\n";
   }
   s << "  T acc[" << MA << "];\n#pragma unroll\n  for (int m = 0; m < " << MA << "; ++m) acc[m] = T(0);\n";
+  // A thread's positions of a chunk are taken a batch at a time: all the loads of `where`, then all the loads
+  // of the expression's inputs at the places they name, then the multiplications -- each step's trips to memory overlap.
+  // When one batch holds all of a thread's positions, its loads of `where` are issued before the chunk's footprint
+  // is copied to LDS: that trip to memory then runs under the copy's.
+  const int NI = (int)((G + TPC - 1) / TPC);
+  const int BATCH = NI < knob_batch ? NI : knob_batch;
+  const bool early_where = BATCH == NI;
+  const int rw = rep[(size_t)where_in];
+  auto where_loads = [&](const char* g0) {
+    s << "        int gg[" << BATCH << "], ee[" << BATCH << "];\n        bool ok[" << BATCH << "];\n        i64 wv[" << BATCH << "];\n";
+    s << "#pragma unroll\n        for (int it = 0; it < " << BATCH << "; ++it) {\n";
+    s << "          const int g = " << g0 << " + it * " << TPC << ";\n          ok[it] = g < " << G << ";\n          gg[it] = ok[it] ? g : 0;\n";
+    s << "          wv[it] = ins.i" << where_in << "[ch * " << chs[(size_t)rw] << "ll + (c" << rw << " + kG" << rw << "[gg[it]])];\n        }\n";
+  };
   s << "  for (i64 ch = blockIdx.x; ch < " << nch << "ll; ch += gridDim.x) {\n";
+  if (early_where) where_loads("li");
   s << "    __syncthreads();\n";
   s << "    for (int u = tid; u < " << span << "; u += 256) xs[u] = X[ch * " << chx << "ll + u];\n";
   s << "    __syncthreads();\n";
-  // A thread's positions of a chunk are taken a batch at a time: all the loads of `where`, then all the loads
-  // of the expression's inputs at the places they name, then the multiplications -- each step's trips to memory overlap.
-  const int NI = (int)((G + TPC - 1) / TPC);
-  const int BATCH = NI < knob_batch ? NI : knob_batch;
-  const int rw = rep[(size_t)where_in];
   s << "    if (col < " << NC << ") {\n";
-  s << "      for (int g0 = li; g0 < " << G << "; g0 += " << TPC * BATCH << ") {\n";
-  s << "        int gg[" << BATCH << "], ee[" << BATCH << "];\n        bool ok[" << BATCH << "];\n        i64 wv[" << BATCH << "];\n";
+  if (early_where) {
+    s << "      {\n";
+  } else {
+    s << "      for (int g0 = li; g0 < " << G << "; g0 += " << TPC * BATCH << ") {\n";
+    where_loads("g0");
+  }
   for (int i = 0; i < v.n_in; ++i)
     if (!scalar[(size_t)i] && i != which_in && i != where_in) s << "        " << ctype(v.dt[(size_t)i]) << " r" << i << "[" << BATCH << "];\n";
-  s << "#pragma unroll\n        for (int it = 0; it < " << BATCH << "; ++it) {\n";
-  s << "          const int g = g0 + it * " << TPC << ";\n          ok[it] = g < " << G << ";\n          gg[it] = ok[it] ? g : 0;\n";
-  s << "          wv[it] = ins.i" << where_in << "[ch * " << chs[(size_t)rw] << "ll + (c" << rw << " + kG" << rw << "[gg[it]])];\n        }\n";
   s << "#pragma unroll\n        for (int it = 0; it < " << BATCH << "; ++it) {\n";
   s << "          const i64 e = wv[it] - " << wh->offset << "ll;\n";
   s << "          ok[it] = ok[it] && e >= 0 && e < " << EH << ";\n          ee[it] = ok[it] ? (int)e : 0;\n";
