@@ -157,6 +157,27 @@ struct Dims {
   int64_t st[4][HG_KDIMS];
 };
 
+// One single-launch reduction of hgpu_contract (contract.hip) with every argument of its kernel: such a launch
+// can be held back like a small product, and reductions that do not read one another's results then go out as
+// one kernel (the bias and readout gradients at the end of a reverse pass).
+struct RedJob {
+  int dtype = 0;              // element type of operands and result
+  int variant = 0;            // 0: a block per output, 1: a wavefront per output, 2: a lane per output
+  int hasb = 0;
+  Dims keep, red;
+  int64_t n_out = 0, R = 0, Q = 0, Lin = 0, sa = 0, sb = 0, chunk = 0;
+  unsigned grid = 0;
+  const void* a = nullptr;
+  const void* b = nullptr;
+  void* out = nullptr;
+  const char* label = nullptr;
+  double bytes = 0, flops = 0;
+};
+// contract.hip: launches up to four such reductions of one element type as one kernel (the caller holds launch_mu)
+hipError_t launch_reduction_group(hgpu_ctx* ctx, const RedJob* const* jobs, int n);
+// smallk.hip: holds the launch back (retaining the buffers it reads and writes); false: the caller launches it now
+bool hold_reduction(hgpu_ctx* ctx, const RedJob& job, hgpu_buffer* const* reads, int n_reads, hgpu_buffer* write);
+
 // Builds the merged iteration space of `nops` operands that share `shape`.
 // Size-1 dims vanish; adjacent dims merge when every operand's strides allow.
 // Returns false when more than HG_KDIMS dims remain.

@@ -63,22 +63,24 @@ __device__ __forceinline__ A wave_sum(A v) {
 
 // Work item = (output o, chunk s); s-th chunk covers reduced linear indices
 // [s*chunk, min(R, (s+1)*chunk)).  out is dense [n_out, S].
+// (`bid` of `nb` blocks: the kernels below pass their own block index; the grouped kernel at the end of this
+// file passes a block's place among the blocks of its problem.  tp == nullptr: one product.)
 template <typename TI, typename TO, bool HASB>
-__global__ void __launch_bounds__(kBlock) k_contract_lane(Dims keep, Dims red, int64_t n_out, int64_t R, int S, int64_t chunk,
-                                                           const TI* __restrict__ a0, const TI* __restrict__ b0, TO* __restrict__ out, TermPtrs tp) {
+__device__ __forceinline__ void lane_body(const Dims& keep, const Dims& red, int64_t n_out, int64_t R, int S, int64_t chunk,
+                                          const TI* __restrict__ a0, const TI* __restrict__ b0, TO* __restrict__ out, const TermPtrs* tp, unsigned bid, unsigned nb) {
   using A = typename acc_of<TI>::type;
   int64_t items = n_out * S;
-  int64_t step = (int64_t)gridDim.x * kBlock;
-  for (int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x; item < items; item += step) {
+  int64_t step = (int64_t)nb * kBlock;
+  for (int64_t item = (int64_t)bid * kBlock + threadIdx.x; item < items; item += step) {
     int64_t o = item % n_out, s = item / n_out;
     const int64_t s_all = s;
     const TI* a = a0;
     const TI* b = b0;
-    if (tp.n) {
-      int term = (int)(s / tp.s_per);
-      s -= (int64_t)term * tp.s_per;
-      a = (const TI*)tp.a[term];
-      b = (const TI*)tp.b[term];
+    if (tp && tp->n) {
+      int term = (int)(s / tp->s_per);
+      s -= (int64_t)term * tp->s_per;
+      a = (const TI*)tp->a[term];
+      b = (const TI*)tp->b[term];
     }
     int64_t ko[2];
     decompose<2>(keep, o, ko);
@@ -122,6 +124,11 @@ __global__ void __launch_bounds__(kBlock) k_contract_lane(Dims keep, Dims red, i
     out[o * S + s_all] = (TO)acc;
   }
 }
+template <typename TI, typename TO, bool HASB>
+__global__ void __launch_bounds__(kBlock) k_contract_lane(Dims keep, Dims red, int64_t n_out, int64_t R, int S, int64_t chunk,
+                                                           const TI* __restrict__ a0, const TI* __restrict__ b0, TO* __restrict__ out, TermPtrs tp) {
+  lane_body<TI, TO, HASB>(keep, red, n_out, R, S, chunk, a0, b0, out, &tp, blockIdx.x, gridDim.x);
+}
 
 // Sum over j = j_first, j_first + 64, ... < j_end of a[j * sa] (* b[j * sb]): four
 // independent accumulators keep four loads per operand in flight.
@@ -154,23 +161,23 @@ __device__ __forceinline__ A lane_strided_sum(const TI* __restrict__ pa, const T
 // Lin = extent, (sa_in, sb_in) = strides; `red` keeps the outer reduced dims
 // with Q = their product.  Chunks split Q when Q > 1, else Lin.
 template <typename TI, typename TO, bool HASB>
-__global__ void __launch_bounds__(kBlock) k_contract_wave(Dims keep, Dims red, int64_t n_out, int64_t Q, int64_t Lin, int64_t sa_in, int64_t sb_in,
-                                                           int S, int64_t chunk, const TI* __restrict__ a0, const TI* __restrict__ b0, TO* __restrict__ out, TermPtrs tp) {
+__device__ __forceinline__ void wave_body(const Dims& keep, const Dims& red, int64_t n_out, int64_t Q, int64_t Lin, int64_t sa_in, int64_t sb_in,
+                                          int S, int64_t chunk, const TI* __restrict__ a0, const TI* __restrict__ b0, TO* __restrict__ out, const TermPtrs* tp, unsigned bid, unsigned nb) {
   using A = typename acc_of<TI>::type;
   const int lane = threadIdx.x & 63;
-  int64_t wave = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> 6;
-  int64_t nwaves = ((int64_t)gridDim.x * kBlock) >> 6;
+  int64_t wave = ((int64_t)bid * kBlock + threadIdx.x) >> 6;
+  int64_t nwaves = ((int64_t)nb * kBlock) >> 6;
   int64_t items = n_out * S;
   for (int64_t item = wave; item < items; item += nwaves) {
     int64_t o = item / S;
     int s = (int)(item - o * S);
     const TI* a = a0;
     const TI* b = b0;
-    if (tp.n) {
-      int term = s / tp.s_per;
-      s -= term * tp.s_per;
-      a = (const TI*)tp.a[term];
-      b = (const TI*)tp.b[term];
+    if (tp && tp->n) {
+      int term = s / tp->s_per;
+      s -= term * tp->s_per;
+      a = (const TI*)tp->a[term];
+      b = (const TI*)tp->b[term];
     }
     int64_t ko[2];
     decompose<2>(keep, o, ko);
@@ -218,6 +225,11 @@ __global__ void __launch_bounds__(kBlock) k_contract_wave(Dims keep, Dims red, i
     if (lane == 0) out[item] = (TO)acc;
   }
 }
+template <typename TI, typename TO, bool HASB>
+__global__ void __launch_bounds__(kBlock) k_contract_wave(Dims keep, Dims red, int64_t n_out, int64_t Q, int64_t Lin, int64_t sa_in, int64_t sb_in,
+                                                           int S, int64_t chunk, const TI* __restrict__ a0, const TI* __restrict__ b0, TO* __restrict__ out, TermPtrs tp) {
+  wave_body<TI, TO, HASB>(keep, red, n_out, Q, Lin, sa_in, sb_in, S, chunk, a0, b0, out, &tp, blockIdx.x, gridDim.x);
+}
 
 // One block of four wavefronts per output: for a few hundred outputs with a few
 // thousand reduced elements each, where one wavefront per output leaves most of
@@ -225,13 +237,13 @@ __global__ void __launch_bounds__(kBlock) k_contract_wave(Dims keep, Dims red, i
 // wavefronts take every fourth outer reduced index (or a quarter of the inner
 // dim when there is no outer one) and combine through LDS in a fixed order.
 template <typename TI, typename TO, bool HASB>
-__global__ void __launch_bounds__(kBlock) k_contract_block(Dims keep, Dims red, int64_t n_out, int64_t Q, int64_t Lin, int64_t sa_in, int64_t sb_in,
-                                                            const TI* __restrict__ a, const TI* __restrict__ b, TO* __restrict__ out) {
+__device__ __forceinline__ void block_body(const Dims& keep, const Dims& red, int64_t n_out, int64_t Q, int64_t Lin, int64_t sa_in, int64_t sb_in,
+                                           const TI* __restrict__ a, const TI* __restrict__ b, TO* __restrict__ out, unsigned bid, unsigned nb) {
   using A = typename acc_of<TI>::type;
   __shared__ A part[kBlock / 64];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   constexpr int NW = kBlock / 64;
-  for (int64_t o = blockIdx.x; o < n_out; o += gridDim.x) {
+  for (int64_t o = bid; o < n_out; o += nb) {
     int64_t ko[2];
     decompose<2>(keep, o, ko);
     A acc = 0;
@@ -256,6 +268,49 @@ __global__ void __launch_bounds__(kBlock) k_contract_block(Dims keep, Dims red, 
       out[o] = (TO)t;
     }
     __syncthreads();
+  }
+}
+template <typename TI, typename TO, bool HASB>
+__global__ void __launch_bounds__(kBlock) k_contract_block(Dims keep, Dims red, int64_t n_out, int64_t Q, int64_t Lin, int64_t sa_in, int64_t sb_in,
+                                                            const TI* __restrict__ a, const TI* __restrict__ b, TO* __restrict__ out) {
+  block_body<TI, TO, HASB>(keep, red, n_out, Q, Lin, sa_in, sb_in, a, b, out, blockIdx.x, gridDim.x);
+}
+
+// Up to four single-launch reductions of one element type as one kernel: the first blocks are problem 0's, the
+// next ones problem 1's, ...; every block runs the code of the kernel its problem would have been launched with.
+struct RedArgs {
+  Dims keep, red;
+  int64_t n_out, R, Q, Lin, sa, sb, chunk;
+  int variant, hasb;
+  unsigned grid, pad_;
+  const void* a;
+  const void* b;
+  void* out;
+};
+struct RedGroup {
+  int n, pad_;
+  RedArgs j[4];
+};
+static_assert(sizeof(RedGroup) <= 4000, "the grouped reduction's arguments must fit the kernel argument block");
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) k_contract_group(RedGroup g) {
+  unsigned bid = blockIdx.x;
+  int k = 0;
+  while (k < g.n - 1 && bid >= g.j[k].grid) { bid -= g.j[k].grid; ++k; }
+  const RedArgs& r = g.j[k];
+  const T* a = (const T*)r.a;
+  const T* b = (const T*)r.b;
+  T* out = (T*)r.out;
+  if (r.variant == 0) {
+    if (r.hasb) block_body<T, T, true>(r.keep, r.red, r.n_out, r.Q, r.Lin, r.sa, r.sb, a, b, out, bid, r.grid);
+    else block_body<T, T, false>(r.keep, r.red, r.n_out, r.Q, r.Lin, r.sa, r.sb, a, b, out, bid, r.grid);
+  } else if (r.variant == 1) {
+    if (r.hasb) wave_body<T, T, true>(r.keep, r.red, r.n_out, r.Q, r.Lin, r.sa, r.sb, 1, r.chunk, a, b, out, nullptr, bid, r.grid);
+    else wave_body<T, T, false>(r.keep, r.red, r.n_out, r.Q, r.Lin, r.sa, r.sb, 1, r.chunk, a, b, out, nullptr, bid, r.grid);
+  } else {
+    if (r.hasb) lane_body<T, T, true>(r.keep, r.red, r.n_out, r.R, 1, r.chunk, a, b, out, nullptr, bid, r.grid);
+    else lane_body<T, T, false>(r.keep, r.red, r.n_out, r.R, 1, r.chunk, a, b, out, nullptr, bid, r.grid);
   }
 }
 
@@ -457,9 +512,12 @@ __global__ void __launch_bounds__(64) k_argminmax_pick(int G, int want_max, cons
   }
 }
 
+// The buffers of a reduction whose launch may be held back (see RedJob): what it reads and what it writes.
+struct HoldBufs { hgpu_buffer* a; hgpu_buffer* b; hgpu_buffer* out; };
+
 template <typename TI, typename TO>
 int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red_full, int64_t n_out, int64_t R, int S, const void* a, const void* b, void* out,
-                 const TermPtrs* terms = nullptr) {
+                 const TermPtrs* terms = nullptr, const HoldBufs* hold = nullptr, int dtype = -1) {
   // with terms, S counts the chunks of all of them; each term is cut into s_per
   TermPtrs tp;
   tp.n = 0;
@@ -479,9 +537,47 @@ int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red
     label = intern_label(ctx, buf);
   }
   const double nterms = tp.n ? tp.n : 1;
-  LaunchGuard lg(ctx, label,
-                 (double)n_out * R * sizeof(TI) * (b ? 2 : 1) * nterms + (double)n_out * S * sizeof(TO), (double)n_out * R * (b ? 2 : 1) * nterms);
+  const double bytes = (double)n_out * R * sizeof(TI) * (b ? 2 : 1) * nterms + (double)n_out * S * sizeof(TO), flops = (double)n_out * R * (b ? 2 : 1) * nterms;
   int maxb = ctx->num_cu * 8;
+  // A single-launch reduction of at most eight million terms is held back: the next ones that do not read its result share its launch.
+  if (hold && !terms && S <= 1 && std::is_same<TI, TO>::value && (double)n_out * (double)R <= 8.0e6) {
+    RedJob j;
+    j.dtype = dtype;
+    j.hasb = b ? 1 : 0;
+    j.keep = keep;
+    j.red = red_full;
+    j.n_out = n_out;
+    j.R = R;
+    j.a = a;
+    j.b = b;
+    j.out = out;
+    j.label = label;
+    j.bytes = bytes;
+    j.flops = flops;
+    if (use_wave) {
+      int last = j.red.nd - 1;
+      j.Lin = j.red.shape[last];
+      j.sa = j.red.st[0][last];
+      j.sb = j.red.st[1][last];
+      j.Q = R / j.Lin;
+      if (j.red.nd > 1) { j.red.nd -= 1; } else { j.red.shape[0] = 1; j.red.st[0][0] = j.red.st[1][0] = 0; }
+      if (S == 0) {
+        j.variant = 0;
+        j.grid = (unsigned)(n_out < (int64_t)maxb ? n_out : maxb);
+      } else {
+        j.variant = 1;
+        j.chunk = j.Q > 1 ? j.Q : j.Lin;
+        j.grid = grid_for(n_out * 64, kBlock, maxb);
+      }
+    } else {
+      j.variant = 2;
+      j.chunk = R;
+      j.grid = grid_for(n_out, kBlock, maxb);
+    }
+    hgpu_buffer* reads[2] = {hold->a, hold->b};
+    if (hold_reduction(ctx, j, reads, hold->b ? 2 : 1, hold->out)) return HGPU_OK;
+  }
+  LaunchGuard lg(ctx, label, bytes, flops);
   if (use_wave && S == 0) {       // one block per output, no partials
     Dims red = red_full;
     int last = red.nd - 1;
@@ -513,6 +609,42 @@ int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red
   return HGPU_OK;
 }
 
+}  // namespace
+
+namespace hg {
+hipError_t launch_reduction_group(hgpu_ctx* ctx, const RedJob* const* jobs, int n) {
+  RedGroup g;
+  memset(&g, 0, sizeof g);
+  g.n = n;
+  unsigned grid = 0;
+  for (int i = 0; i < n; ++i) {
+    const RedJob& j = *jobs[i];
+    RedArgs& r = g.j[i];
+    r.keep = j.keep;
+    r.red = j.red;
+    r.n_out = j.n_out;
+    r.R = j.R;
+    r.Q = j.Q;
+    r.Lin = j.Lin;
+    r.sa = j.sa;
+    r.sb = j.sb;
+    r.chunk = j.chunk;
+    r.variant = j.variant;
+    r.hasb = j.hasb;
+    r.grid = j.grid;
+    r.a = j.a;
+    r.b = j.b;
+    r.out = j.out;
+    grid += j.grid;
+  }
+  if (jobs[0]->dtype == HGPU_F64) hipLaunchKernelGGL((k_contract_group<double>), dim3(grid), dim3(kBlock), 0, ctx->stream, g);
+  else hipLaunchKernelGGL((k_contract_group<float>), dim3(grid), dim3(kBlock), 0, ctx->stream, g);
+  return hipGetLastError();
+}
+}  // namespace hg
+
+namespace {
+
 int64_t min_abs_nonzero(const Dims& d, int dim) {
   int64_t m = INT64_MAX;
   for (int k = 0; k < 2; ++k) {
@@ -529,7 +661,7 @@ int64_t min_abs_nonzero(const Dims& d, int dim) {
 // live in `scratch` when the caller brings one (then nothing is allocated here,
 // and a request whose partial sums exceed scratch_bytes is refused), else in a
 // block from the context's allocator.
-int reduce_views(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, void* out, void* scratch, size_t scratch_bytes) {
+int reduce_views(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, void* out, void* scratch, size_t scratch_bytes, hgpu_buffer* out_buf = nullptr) {
   int64_t n_out = 1, R = 1;
   for (int i = 0; i < n_keep; ++i) n_out *= a->shape[i];
   for (int i = n_keep; i < a->rank; ++i) R *= a->shape[i];
@@ -570,11 +702,14 @@ int reduce_views(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_
   const void* pa = data_ptr(a);
   const void* pb = b ? data_ptr(b) : nullptr;
   int rc = HGPU_OK;
+  // (a caller that brings its own scratch wants its result written by the time the call returns to the stream: not held)
+  HoldBufs hb{a->buf, b ? b->buf : nullptr, out_buf};
+  const HoldBufs* hold = (out_buf && !scratch && a->buf && (!b || b->buf) && (a->dtype == HGPU_F64 || a->dtype == HGPU_F32)) ? &hb : nullptr;
   if (use_wave && n_out >= 64 && n_out <= 1024 && R >= 1024 && R <= 65536) {
     // a few hundred outputs of a few thousand elements: a block per output, one launch
-    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, true, keep, red, n_out, R, 0, pa, pb, out)));
+    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, true, keep, red, n_out, R, 0, pa, pb, out, nullptr, hold, a->dtype)));
   } else if (S == 1) {
-    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, use_wave, keep, red, n_out, R, 1, pa, pb, out)));
+    HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, use_wave, keep, red, n_out, R, 1, pa, pb, out, nullptr, hold, a->dtype)));
   } else {
     // stage 1: partials [n_out, S] in the accumulator type; stage 2 sums them.
     const size_t need = (size_t)n_out * (size_t)S * 8;
@@ -804,7 +939,7 @@ int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n
   if (rc) { hgpu_release(o); return rc; }
   if (handled) { *out = o; return HGPU_OK; }
 
-  rc = reduce_views(ctx, a, b, n_keep, data_ptr(o), nullptr, 0);
+  rc = reduce_views(ctx, a, b, n_keep, data_ptr(o), nullptr, 0, o->buf);
   if (rc) { hgpu_release(o); return rc; }
   *out = o;
   return HGPU_OK;

@@ -583,6 +583,8 @@ namespace hg {
 // A launch that is held back: everything the kernel needs, and the buffers it
 // reads and writes (retained, so that none is handed out again before the launch).
 struct Deferred {
+  bool is_reduction = false;   // a reduction of contract.hip (`red`) instead of a small product
+  RedJob red;
   std::string body, kname;
   hipFunction_t fn = nullptr;
   unsigned grid = 0;
@@ -784,9 +786,50 @@ void flush_deferred_locked(hgpu_ctx* ctx) {
     }
   };
   for (int lv = 0; lv <= top; ++lv) {
+    // the level's reductions: those of one element type go out together, four at a time
+    {
+      std::vector<Deferred*> reds;
+      for (auto& d : items)
+        if (d.level == lv && d.is_reduction) reds.push_back(&d);
+      std::stable_sort(reds.begin(), reds.end(), [](const Deferred* a, const Deferred* b) { return a->red.dtype < b->red.dtype; });
+      for (size_t g0 = 0; g0 < reds.size();) {
+        size_t g1 = g0 + 1;
+        while (g1 < reds.size() && g1 - g0 < 4 && reds[g1]->red.dtype == reds[g0]->red.dtype) ++g1;
+        const RedJob* jobs[4];
+        double bytes = 0, flops = 0;
+        for (size_t i = g0; i < g1; ++i) { jobs[i - g0] = &reds[i]->red; bytes += reds[i]->bytes; flops += reds[i]->flops; }
+        const char* label = reds[g0]->label;
+        if (g1 - g0 > 1) {
+          label = "contract_group";
+          if (ctx->profiling && ctx->profile_shapes) {
+            std::string lab = "contract_group[";
+            for (size_t i = g0; i < g1; ++i) lab += (i > g0 ? "|" : "") + std::string(reds[i]->label);
+            label = intern_label(ctx, lab + "]");
+          }
+        }
+        bool timed = false;
+        if (ctx->profiling && !ctx->cap) {
+          hgpu_ctx::ProfRec r{label, nullptr, nullptr, bytes, flops};
+          if (hipEventCreate(&r.a) == hipSuccess && hipEventCreate(&r.b) == hipSuccess) {
+            (void)hipEventRecord(r.a, ctx->stream);
+            ctx->prof.push_back(r);
+            timed = true;
+          }
+        }
+        hipError_t err = launch_reduction_group(ctx, jobs, (int)(g1 - g0));
+        if (timed) (void)hipEventRecord(ctx->prof.back().b, ctx->stream);
+        if (err != hipSuccess) {
+          int rc = check_hip(ctx, err, "grouped reduction launch");
+          if (!ctx->deferred_rc) ctx->deferred_rc = rc;
+        }
+        ctx->dq->n_launches += 1;
+        if (g1 - g0 > 1) ctx->dq->n_grouped += (long)(g1 - g0);
+        g0 = g1;
+      }
+    }
     std::vector<Deferred*> here;
     for (auto& d : items)
-      if (d.level == lv) here.push_back(&d);
+      if (d.level == lv && !d.is_reduction) here.push_back(&d);
     for (size_t g0 = 0; g0 < here.size(); g0 += kMaxGroup) {
       std::vector<Deferred*> grp(here.begin() + (long)g0, here.begin() + (long)std::min(here.size(), g0 + kMaxGroup));
       hipFunction_t fn = nullptr;
@@ -835,6 +878,30 @@ void flush_deferred_locked(hgpu_ctx* ctx) {
     for (auto* b : d.reads) buffer_release(b);
     for (auto* b : d.writes) buffer_release(b);
   }
+}
+
+// A single-launch reduction joins the queue: held back until something else needs the stream, levelled with
+// the held products by who reads whose results, and launched together with the other reductions of its level.
+bool hold_reduction(hgpu_ctx* ctx, const RedJob& job, hgpu_buffer* const* reads, int n_reads, hgpu_buffer* write) {
+  static const bool hold = getenv("HORDEAD_NO_GROUPED_LAUNCH") == nullptr;
+  if (!hold || !write) return false;
+  Deferred d;
+  d.is_reduction = true;
+  d.red = job;
+  d.label = job.label;
+  d.bytes = job.bytes;
+  d.flops = job.flops;
+  for (int i = 0; i < n_reads; ++i)
+    if (reads[i]) d.reads.push_back(reads[i]);
+  d.writes.push_back(write);
+  for (auto* b : d.reads) buffer_retain(b);
+  for (auto* b : d.writes) buffer_retain(b);
+  std::lock_guard<std::mutex> lk(ctx->launch_mu);
+  if (!ctx->dq) ctx->dq = new DeferredQueue;
+  if (ctx->dq->items.size() >= kMaxHeld) flush_deferred_locked(ctx);
+  ctx->dq->items.push_back(std::move(d));
+  ctx->dq_pending = true;
+  return true;
 }
 
 void flush_deferred(hgpu_ctx* ctx) {

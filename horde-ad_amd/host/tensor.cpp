@@ -883,6 +883,14 @@ void force_many(const std::vector<T>& ts) {
   for (auto& t : ts)
     if (t.valid() && t.pending_expr()) groups[{t.be(), t.shape()}].push_back(t.holder().get());
   for (auto& g : groups) force_roots(g.first.first, g.second);
+  // Small pending contractions (the bias and readout gradients at the end of a reverse pass) are asked for last,
+  // one after another: a provider that holds such launches back then sends them out as one kernel.
+  auto small_reduction = [](const T& t) {
+    const ArrHolder* p = t.holder().get();
+    return !p->h && p->ekind < 0 && p->fa && p->fb && p->keep >= 0 && p->more.empty() && !p->origin && t.size() <= 16384;
+  };
+  for (auto& t : ts)
+    if (t.valid() && !small_reduction(t)) (void)t.h();
   for (auto& t : ts)
     if (t.valid()) (void)t.h();
 }
