@@ -705,8 +705,9 @@ int reduce_views(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_
   // (a caller that brings its own scratch wants its result written by the time the call returns to the stream: not held)
   HoldBufs hb{a->buf, b ? b->buf : nullptr, out_buf};
   const HoldBufs* hold = (out_buf && !scratch && a->buf && (!b || b->buf) && (a->dtype == HGPU_F64 || a->dtype == HGPU_F32)) ? &hb : nullptr;
-  if (use_wave && n_out >= 64 && n_out <= 1024 && R >= 1024 && R <= 65536) {
-    // a few hundred outputs of a few thousand elements: a block per output, one launch
+  if (use_wave && ((n_out >= 64 && n_out <= 1024 && R >= 1024 && R <= 65536) || (n_out < 64 && S > 1 && R >= 1024 && R <= 16384))) {
+    // a few hundred outputs of a few thousand elements (or a handful of outputs that would otherwise take a
+    // launch for partial sums and a second one to add them): a block per output, one launch
     HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, true, keep, red, n_out, R, 0, pa, pb, out, nullptr, hold, a->dtype)));
   } else if (S == 1) {
     HG_DISPATCH_DTYPE(a->dtype, T, rc = (launch_stage<T, T>(ctx, use_wave, keep, red, n_out, R, 1, pa, pb, out, nullptr, hold, a->dtype)));
