@@ -62,6 +62,8 @@ SHAPES = [
     (np.float32, 128, 1000, [600], ["mk"]),                 # up to 1024 contracted elements when the result is small ...
     (np.float64, 128, 1000, [784], ["mk"]),                 # ... (a dense layer over a flattened image: 13 chunks)
     (np.float64, 128, 784, [1000], ["km"]),                 # its weight gradient: 16 chunks
+    (np.float64, 70, 333, [900], ["mk"]),                   # few tiles, long K, ragged everywhere: K shared out between blocks, a second launch adds the partial tiles
+    (np.float32, 50, 90, [1000], ["km"]),                   # the same in fp32 with the weights transposed (6 tiles of 16 chunks)
     (np.float32, 128, 1000, [1100], ["mk"]),                # too long for the kernel: the entry points one after another
     (np.float32, 300, 1000, [600], ["mk"]),                 # too long for a result of this size
     (np.float64, 300, 5000, [784], ["mk"]),                 # ... a dense layer over a flattened image at batch 5000: split in two along K, the program adds the halves

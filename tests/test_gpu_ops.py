@@ -305,6 +305,35 @@ def test_fused_sum_equals_program_then_sum(gpu, dt):
     assert e.value.code == 4
 
 
+def test_small_reductions_leave_together(gpu):
+    """Single-launch reductions that do not read one another's results are held back and go out as one kernel
+    (the bias and readout gradients at the end of a reverse pass); one that reads another's result runs after it.
+    Results against numpy, and bit-equal to the same reductions asked for one at a time."""
+    import os
+    if os.environ.get("HORDEAD_NO_GROUPED_LAUNCH"):
+        pytest.skip("grouped launches are switched off in this environment")
+    a, b, b2, c = rnd((300, 5000), np.float64), rnd((100, 5000), np.float64), rnd((100, 5000), np.float64), rnd((10, 1000), np.float64)
+    A, B, B2, Cc = gpu.upload(a), gpu.upload(b), gpu.upload(b2), gpu.upload(c)
+    alone = []
+    for x, y in ((A, None), (B, B2), (Cc, None)):
+        r = x.contract(y, 1)
+        alone.append(r.numpy())                      # the read-back sends each one out by itself
+    gpu.sync()
+    gpu.profile(2)
+    ra, rb, rc = A.contract(None, 1), B.contract(B2, 1), Cc.contract(None, 1)
+    rd = ra.contract(None, 0)                        # reads ra: the next level
+    got = [r.numpy() for r in (ra, rb, rc)]
+    total = float(rd.numpy())
+    rep = gpu.profile_report()
+    gpu.profile(0)
+    groups = {k: v for k, v in rep.items() if k.startswith("contract_group[") and v[0]}
+    assert len(groups) == 1 and list(groups.values())[0][0] == 1 and list(groups)[0].count("|") == 2, rep
+    for g, w, al in zip(got, (a.sum(1), (b * b2).sum(1), c.sum(1)), alone):
+        np.testing.assert_allclose(g, w, rtol=1e-10, atol=1e-9)
+        assert np.array_equal(g, al)
+    assert abs(total - float(a.sum())) <= 1e-10 * float(np.abs(a).sum())
+
+
 def test_fused_sum_is_finished_three_ways(gpu):
     """Up to 1024 vectors one block writes the sum; up to 131072 elements the block that draws the last
     ticket adds the blocks' sums; beyond, a second launch does.  Every size is summed twice in a row and
