@@ -537,7 +537,15 @@ int launch_stage(hgpu_ctx* ctx, bool use_wave, const Dims& keep, const Dims& red
     label = intern_label(ctx, buf);
   }
   const double nterms = tp.n ? tp.n : 1;
-  const double bytes = (double)n_out * R * sizeof(TI) * (b ? 2 : 1) * nterms + (double)n_out * S * sizeof(TO), flops = (double)n_out * R * (b ? 2 : 1) * nterms;
+  // algorithmic bytes: every operand's distinct elements once (an operand that stands still along a dim is not read again along it)
+  auto distinct = [&](int k) {
+    double n = 1;
+    for (int i = 0; i < keep.nd; ++i) if (keep.st[k][i] != 0) n *= (double)keep.shape[i];
+    for (int i = 0; i < red_full.nd; ++i) if (red_full.st[k][i] != 0) n *= (double)red_full.shape[i];
+    return n;
+  };
+  const double bytes = (distinct(0) + (b ? distinct(1) : 0.0)) * sizeof(TI) * nterms + (double)n_out * (S > 0 ? S : 1) * sizeof(TO),
+               flops = (double)n_out * R * (b ? 2 : 1) * nterms;
   int maxb = ctx->num_cu * 8;
   // A single-launch reduction of at most eight million terms is held back: the next ones that do not read its result share its launch.
   if (hold && !terms && S <= 1 && std::is_same<TI, TO>::value && (double)n_out * (double)R <= 8.0e6) {
