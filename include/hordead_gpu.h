@@ -278,7 +278,10 @@ int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, in
  * transposed behind), tsdot0 (:231-232), tsdot1In (:233-235), tsmatvecmul
  * (:236) and tsmatmul2 (:237-242, which the reference itself defines as
  * dot1In over replicated and transposed views).  Floating-point summation
- * order is unspecified (as it is in ox-arrays); integers are exact. */
+ * order is unspecified (as it is in ox-arrays) but fixed by the shapes;
+ * integers are exact.  The launch of a small reduction may be held back like
+ * that of a small product (see hgpu_contract_sum_map): reductions that do not
+ * read one another's results then leave as one kernel. */
 int hgpu_contract(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep, hgpu_array** out);
 
 /* out = sum_t contract(a[t], b[t], n_keep): the same contraction of n pairs of
