@@ -26,7 +26,6 @@
 
 #include <array>
 #include <map>
-#include <sstream>
 #include <string>
 #include <vector>
 
@@ -198,7 +197,7 @@ bool make_plan(bool f64, std::vector<Dim> rows, std::vector<Dim> cols, std::vect
 }
 
 std::string table(const char* qual, const char* name, const std::vector<int>& v) {
-  std::ostringstream s;
+  hg::fusedgen::Src s;
   s << qual << " int " << name << "[" << (v.empty() ? 1 : v.size()) << "] = {";
   for (size_t i = 0; i < v.size(); ++i) s << (i ? "," : "") << v[i];
   if (v.empty()) s << "0";
@@ -732,7 +731,7 @@ int lds_bytes(const Plan& pl) {
 
 std::string generate(const Plan& pl, const std::string& kname, const std::string& epilogue = std::string(), int stage_bytes = 0,
                      const std::string& virt_x = std::string(), int64_t xbase = 0, const std::string& virt_y = std::string(), int64_t ybase = 0) {
-  std::ostringstream s;
+  hg::fusedgen::Src s;
   s << "#define KNAME " << kname << "\n";
   s << "#define VIRT_X " << (virt_x.empty() ? 0 : 1) << "\n#define XBASE " << xbase << "ll\n";
   s << "#define VIRT_Y " << (virt_y.empty() ? 0 : 1) << "\n#define YBASE " << ybase << "ll\n";
@@ -806,7 +805,7 @@ bool vector_ok(const VirtualOp& v, int V) {
 // offset is decoded for every chunk.  Divisors are constants of the kernel.
 std::string vops_source(const VirtualOp& v, const char* tag_, int V, int64_t chunk_stride, int64_t max_elem = INT64_MAX) {
   using namespace hg::fusedgen;
-  std::ostringstream s;
+  Src s;
   const std::string tag = tag_;
   const std::string T_ = ctype(v.dtype);
   const size_t rm = v.M.size(), re = v.E.size();
@@ -1274,7 +1273,7 @@ struct EpiSpec {
 };
 
 std::string epilogue_source(const Plan& pl, const EpiSpec& e) {
-  std::ostringstream s;
+  Src s;
   s << kPrelude;
   const int WPL = 4 / e.L;
   for (int i = 0; i < e.n_in; ++i) {
@@ -1993,7 +1992,7 @@ int try_mapped_sum(hgpu_ctx* ctx, const VirtualOp& v, const hgpu_operand* o, int
   if (S < 1) S = 1;
   int64_t CH = ((R + S - 1) / S + W - 1) / W * W;
   S = (R + CH - 1) / CH;
-  std::ostringstream s;
+  Src s;
   s << "typedef long long i64;\n";
   s << "typedef " << (es == 8 ? "double" : "float") << " T;\n";
   s << "template <int N> struct VT { typedef T type __attribute__((ext_vector_type(N))); };\ntemplate <> struct VT<1> { typedef T type; };\ntemplate <int N> using Vec = typename VT<N>::type;\n";
@@ -2313,7 +2312,7 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
     fits32 = fits32 && reach < (1LL << 31);
   }
   if (!fits32) return HGPU_OK;
-  std::ostringstream s;
+  Src s;
   char kname[160];
   snprintf(kname, sizeof kname, "onehot_contract_%s_m%d_n%d_k%lldx%lld_onehot%lld", es == 8 ? "f64" : "f32", MR, NC, (long long)nch, (long long)G, (long long)EH);
   s << "typedef long long i64;\n";

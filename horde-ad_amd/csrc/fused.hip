@@ -17,7 +17,6 @@
 #include <hip/hiprtc.h>
 
 #include <memory>
-#include <sstream>
 
 #include "common.hpp"
 #include "fused_gen.hpp"
@@ -201,7 +200,7 @@ static int fused_map_impl(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, 
   }
 
   // ---- source
-  std::ostringstream s;
+  Src s;
   s << kPrelude;
   if (!all_simple) s << "struct FDims { int nd; i64 shape[" << HG_KDIMS << "]; i64 st[" << kMaxIn << "][" << HG_KDIMS << "]; };\n";
   s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
@@ -510,7 +509,7 @@ extern "C" int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     }
   }
   // ---- source: shapes and strides are constants of the kernel
-  std::ostringstream s;
+  Src s;
   s << kPrelude;
   s << "extern \"C\" __global__ void __launch_bounds__(256) fused_extremum(i64 n";
   for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
@@ -653,7 +652,7 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     if (rc) { drop_part(); hgpu_release(o); return rc; }
   }
 
-  std::ostringstream s;
+  Src s;
   s << kPrelude;
   s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
   s << "typedef " << acc << " ACC;\n";
@@ -854,7 +853,7 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     if (rc) { drop_part(); release_all(); return rc; }
   }
 
-  std::ostringstream s;
+  Src s;
   s << kPrelude;
   s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
   s << "template <typename A> __device__ __forceinline__ A wave_sum(A v) {\n"

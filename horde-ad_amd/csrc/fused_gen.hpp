@@ -4,14 +4,61 @@
 // straight-line code.  Shared by the fused maps and by the matrix-product
 // kernels that run a program over their result or their operands.
 #pragma once
-#include <sstream>
+#include <charconv>
+#include <cstdlib>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "common.hpp"
 
 namespace hg {
 namespace fusedgen {
+
+// The text of a generated kernel, appended to piece by piece: the interface of
+// an output stream for text and integers, without a stream's locale and virtual
+// calls (the generators run on every call, and a call's kernel is looked up by
+// its text).
+struct Src {
+  std::string text;
+  Src() { text.reserve(16384); }
+  Src& operator<<(const char* t) { text.append(t); return *this; }
+  Src& operator<<(const std::string& t) { text.append(t); return *this; }
+  Src& operator<<(char c) { text.push_back(c); return *this; }
+  template <typename I, typename std::enable_if<std::is_integral<I>::value && !std::is_same<I, char>::value && !std::is_same<I, bool>::value &&
+                                                    !std::is_same<I, signed char>::value && !std::is_same<I, unsigned char>::value, int>::type = 0>
+  Src& operator<<(I v) {
+    char buf[24];
+    auto r = std::to_chars(buf, buf + sizeof buf, v);
+    text.append(buf, (size_t)(r.ptr - buf));
+    return *this;
+  }
+  Src& operator<<(bool v) { text.push_back(v ? '1' : '0'); return *this; }
+  const std::string& str() const { return text; }
+};
+
+// What a generator's text depends on, as bytes: the key under which a call
+// finds the kernel that the same call generated before, without writing the
+// text again.  With HORDEAD_GPU_CHECK_KEYS set, every such find writes the text
+// anyway and compares it with the one kept (a key that leaves out something the
+// text depends on then shows as an error instead of a wrong kernel).
+struct Key {
+  std::string bytes;
+  template <typename X, typename std::enable_if<std::is_arithmetic<X>::value, int>::type = 0>
+  Key& put(X x) { bytes.append(reinterpret_cast<const char*>(&x), sizeof x); return *this; }
+  template <typename X> Key& put(const std::vector<X>& v) { put(v.size()); for (const X& x : v) put(x); return *this; }
+  Key& put(int n, const int64_t* v) { put(n); for (int i = 0; i < n; ++i) put(v[i]); return *this; }
+  Key& put(const std::string& t) { put(t.size()); bytes.append(t); return *this; }
+  Key& put(int n, const hgpu_fused_instr* prog) {
+    put(n);
+    for (int k = 0; k < n; ++k) put(prog[k].kind).put(prog[k].op).put(prog[k].dtype).put(prog[k].a).put(prog[k].b).put(prog[k].c);
+    return *this;
+  }
+};
+inline bool check_keys() {
+  static const bool on = getenv("HORDEAD_GPU_CHECK_KEYS") != nullptr;
+  return on;
+}
 
 inline const char* ctype(int dt) {
   switch (dt) {
@@ -147,7 +194,7 @@ inline int check_program(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, i
 }
 
 // One instruction per line: `const T v<slot><suffix> = ...;`
-inline void emit_program(std::ostringstream& s, int n_in, int n_instr, const hgpu_fused_instr* prog, const std::vector<int>& dt, const char* ind, const std::string& lane_suffix) {
+inline void emit_program(Src& s, int n_in, int n_instr, const hgpu_fused_instr* prog, const std::vector<int>& dt, const char* ind, const std::string& lane_suffix) {
   for (int k = 0; k < n_instr; ++k) {
     const hgpu_fused_instr& q = prog[k];
     int self = n_in + k;

@@ -44,8 +44,8 @@
 #include <cmath>
 #include <cstdlib>
 #include <map>
-#include <sstream>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "common.hpp"
@@ -75,6 +75,25 @@ std::map<std::string, Compiled>& cache_of(hgpu_ctx* ctx) {
   auto it = ctx->jit_cache.find("__smallk__");
   if (it == ctx->jit_cache.end()) it = ctx->jit_cache.emplace("__smallk__", new std::map<std::string, Compiled>()).first;
   return *static_cast<std::map<std::string, Compiled>*>(it->second);
+}
+
+// A problem's kernel, found again by what its text depends on (the text itself
+// is only written the first time), and the kernels over sets of problems, found
+// by their members.
+struct Known {
+  std::string body;    // the problem's device code
+  int id = 0;          // stands for the body where sets of problems are keyed
+  std::string kname;
+  hipFunction_t fn = nullptr, finish_fn = nullptr;
+};
+struct KnownKernels {
+  std::unordered_map<std::string, Known> problems;
+  std::unordered_map<std::string, hipFunction_t> groups;   // by the members' ids, grids and LDS bytes in the order of the kernel's text
+};
+KnownKernels& known_of(hgpu_ctx* ctx) {
+  auto it = ctx->jit_cache.find("__smallk_known__");
+  if (it == ctx->jit_cache.end()) it = ctx->jit_cache.emplace("__smallk_known__", new KnownKernels()).first;
+  return *static_cast<KnownKernels*>(it->second);
 }
 
 struct Term {
@@ -150,7 +169,7 @@ Operand make_operand(bool f64, int rows, int64_t extent, int64_t sr, int64_t sk,
 
 int tile_elems(const Operand& o, int kcp) { return o.layout == 0 ? kcp * o.pitch : o.rows * o.pitch; }
 
-void emit_stage_fn(std::ostringstream& s, const char* name, const Operand& o, const Chunk& c, const char* ptr, const char* r0) {
+void emit_stage_fn(Src& s, const char* name, const Operand& o, const Chunk& c, const char* ptr, const char* r0) {
   // registers of the next chunk's tile: load_<name>() issues the loads, store_<name>() puts them into LDS
   const int slots = o.rows * c.kcp / o.V;
   const int ns = (slots + 255) / 256;
@@ -197,7 +216,7 @@ void emit_stage_fn(std::ostringstream& s, const char* name, const Operand& o, co
 // does.  It names nothing outside itself but the prelude, so several problems'
 // code can sit in one source file, each in a namespace of its own.
 std::string generate_body(const Spec& sp) {
-  std::ostringstream s;
+  Src s;
   const int TP = sp.BP / (16 * sp.WP), TQ = sp.BQ / (16 * sp.WQ);
   const int64_t nbp = (sp.P + sp.BP - 1) / sp.BP, nbq = (sp.Q + sp.BQ - 1) / sp.BQ;
   const int S = sp.splits;
@@ -408,7 +427,7 @@ std::string generate_body(const Spec& sp) {
 // the round of the XCDs).  A single problem gives the kernel of that problem.
 std::string kernel_source(const std::vector<const std::string*>& bodies, const std::vector<unsigned>& grids, const std::vector<int>& lds_bytes, const std::string& kname,
                           bool with_finish = false) {
-  std::ostringstream s;
+  Src s;
   s << kPrelude;
   int lds = 16;
   for (size_t k = 0; k < bodies.size(); ++k) {
@@ -499,6 +518,21 @@ bool plan_chunks(Spec& sp) {
   return (size_t)(sp.x_elems + sp.y_elems) * (sp.f64 ? 8 : 4) <= 150 * 1024;
 }
 
+// Everything generate_body reads.
+Key spec_key(const Spec& sp) {
+  Key k;
+  k.put(sp.f64).put(sp.P).put(sp.Q).put(sp.BP).put(sp.BQ).put(sp.WP).put(sp.WQ).put(sp.terms.size());
+  for (const Term& t : sp.terms) k.put(t.K).put(t.sxp).put(t.sxk).put(t.syq).put(t.syk);
+  k.put(sp.chunks.size());
+  for (const Chunk& c : sp.chunks) {
+    k.put(c.term).put(c.k0).put(c.kc).put(c.kcp);
+    for (const Operand* o : {&c.x, &c.y}) k.put(o->rows).put(o->layout).put(o->V).put(o->pitch).put(o->sr).put(o->sk).put(o->extent);
+  }
+  k.put(sp.n_in).put(sp.c_slot).put(sp.n_instr, sp.prog).put(sp.dt).put(sp.in_sp).put(sp.in_sq).put(sp.out_slots);
+  k.put(sp.x_elems).put(sp.y_elems).put(sp.splits).put(sp.chunks_per_split);
+  return k;
+}
+
 // The non-unit kept dims of the terms must be two: P (contiguous in a dense
 // result: the later one) and Q.
 struct KeptDims { int dp, dq; int64_t P, Q; };
@@ -585,7 +619,9 @@ namespace hg {
 struct Deferred {
   bool is_reduction = false;   // a reduction of contract.hip (`red`) instead of a small product
   RedJob red;
-  std::string body, kname;
+  const std::string* body = nullptr;   // the problem's device code (kept with the known kernels) and the number that stands for it
+  int body_id = -1;
+  std::string kname;
   hipFunction_t fn = nullptr;
   unsigned grid = 0;
   int lds_bytes = 0;
@@ -598,7 +634,7 @@ struct Deferred {
 
 struct DeferredQueue {
   std::vector<Deferred> items;
-  std::map<size_t, int> seen;        // how often a set of problems came up together, by the hash of their code
+  std::map<size_t, int> seen;        // how often a set of problems came up together, by the hash of their ids, grids and LDS bytes
   long n_launches = 0, n_grouped = 0;
 };
 }  // namespace hg
@@ -677,7 +713,6 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
            n_instr, n_out);
   Deferred d;
   hipFunction_t finish_fn = nullptr;
-  d.body = generate_body(sp);
   d.kname = kname;
   const int64_t nblk = ntiles * sp.splits;
   const int64_t grid = (nblk + 7) / 8 * 8;
@@ -685,8 +720,24 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
   d.grid = (unsigned)grid;
   d.lds_bytes = (sp.x_elems + sp.y_elems) * (sp.f64 ? 8 : 4);
   {
-    std::lock_guard<std::mutex> lk(ctx->launch_mu);   // the kernel cache is shared with the thread that launches what is held back
-    d.fn = compiled_kernel(ctx, {&d.body}, {d.grid}, {d.lds_bytes}, d.kname, sp.splits > 1 ? &finish_fn : nullptr);
+    std::lock_guard<std::mutex> lk(ctx->launch_mu);   // the kernel caches are shared with the thread that launches what is held back
+    auto& known = known_of(ctx).problems;
+    const Key key = spec_key(sp);
+    auto it = known.find(key.bytes);
+    if (it == known.end()) {
+      Known kn;
+      kn.body = generate_body(sp);
+      kn.id = (int)known.size();
+      kn.kname = kname;
+      kn.fn = compiled_kernel(ctx, {&kn.body}, {d.grid}, {d.lds_bytes}, kn.kname, sp.splits > 1 ? &kn.finish_fn : nullptr);
+      it = known.emplace(key.bytes, std::move(kn)).first;
+    } else if (check_keys() && (it->second.body != generate_body(sp) || it->second.kname != kname)) {
+      return fail(ctx, HGPU_ERR_DEVICE, "small-K product: two different kernels under one key (%s)", kname);
+    }
+    d.body = &it->second.body;
+    d.body_id = it->second.id;
+    d.fn = it->second.fn;
+    finish_fn = it->second.finish_fn;
   }
   if (!d.fn) return HGPU_OK;
 
@@ -836,17 +887,29 @@ void flush_deferred_locked(hgpu_ctx* ctx) {
       std::string gname;
       if (grp.size() > 1) {
         // one order for a set of problems, whichever way round they were issued
-        std::stable_sort(grp.begin(), grp.end(), [](const Deferred* a, const Deferred* b) { return a->kname != b->kname ? a->kname < b->kname : a->body < b->body; });
-        gname = "smallk_x" + std::to_string(grp.size());
-        std::string key;
-        for (auto* d : grp) { gname += "__" + d->kname.substr(7); key += d->body + "\x1f"; }
+        std::stable_sort(grp.begin(), grp.end(), [](const Deferred* a, const Deferred* b) {
+          return a->kname != b->kname ? a->kname < b->kname : (a->body_id != b->body_id && *a->body < *b->body);
+        });
+        Key key;
+        for (auto* d : grp) key.put(d->body_id).put(d->grid).put(d->lds_bytes);
         // a set seen once may never come again (a second or so of compilation): the second time pays
-        if (++ctx->dq->seen[std::hash<std::string>()(key)] >= 2) {
-          std::vector<const std::string*> bodies;
-          std::vector<unsigned> grids;
-          std::vector<int> lds;
-          for (auto* d : grp) { bodies.push_back(&d->body); grids.push_back(d->grid); lds.push_back(d->lds_bytes); }
-          fn = compiled_kernel(ctx, bodies, grids, lds, gname);
+        if (++ctx->dq->seen[std::hash<std::string>()(key.bytes)] >= 2) {
+          auto& groups = known_of(ctx).groups;
+          auto it = groups.find(key.bytes);
+          if (it == groups.end() || check_keys()) {
+            gname = "smallk_x" + std::to_string(grp.size());
+            std::vector<const std::string*> bodies;
+            std::vector<unsigned> grids;
+            std::vector<int> lds;
+            for (auto* d : grp) { gname += "__" + d->kname.substr(7); bodies.push_back(d->body); grids.push_back(d->grid); lds.push_back(d->lds_bytes); }
+            hipFunction_t f = compiled_kernel(ctx, bodies, grids, lds, gname);
+            if (it != groups.end() && it->second != f) {
+              fprintf(stderr, "hordead_gpu: two different kernels under one key (%s)\n", gname.c_str());
+              if (!ctx->deferred_rc) ctx->deferred_rc = HGPU_ERR_DEVICE;
+            }
+            if (it == groups.end()) it = groups.emplace(key.bytes, f).first;
+          }
+          fn = it->second;
         }
       }
       if (fn) {
