@@ -54,6 +54,11 @@ struct hgpu_array {
   int64_t shape[HGPU_MAX_RANK];
   int64_t strides[HGPU_MAX_RANK];  // in elements
   int64_t offset;                  // in elements, from buf->ptr
+  // Arrays (views included) come and go by the thousand in a training step, most of them freed together
+  // when the step's tape goes: their blocks are kept on a list per thread instead of going back to the
+  // allocator, whose per-thread cache holds only a few blocks of one size.
+  static void* operator new(size_t n);
+  static void operator delete(void* p);
 };
 
 namespace hg {

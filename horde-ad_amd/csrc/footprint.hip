@@ -27,6 +27,7 @@
 #include <array>
 #include <map>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 using namespace hg;
@@ -63,6 +64,35 @@ int compile(hgpu_ctx* ctx, const std::string& src, const std::string& kname, Com
   return HGPU_OK;
 }
 
+// A kernel found again by what its text depends on; the text is written (and
+// looked up, and compiled) the first time only.  source() writes it.
+struct KnownKernel { Compiled c; std::string text; };
+template <typename F>
+int known_kernel(hgpu_ctx* ctx, const hg::fusedgen::Key& key, const std::string& kname, F&& source, Compiled* out) {
+  auto kit = ctx->jit_cache.find("__footprint_known__");
+  if (kit == ctx->jit_cache.end()) kit = ctx->jit_cache.emplace("__footprint_known__", new std::unordered_map<std::string, KnownKernel>()).first;
+  auto& known = *static_cast<std::unordered_map<std::string, KnownKernel>*>(kit->second);
+  auto it = known.find(key.bytes);
+  if (it != known.end() && !hg::fusedgen::check_keys()) { *out = it->second.c; return HGPU_OK; }
+  std::string src = source();
+  if (it != known.end()) {
+    if (it->second.text != src) return fail(ctx, HGPU_ERR_DEVICE, "%s: two different kernels under one key", kname.c_str());
+    *out = it->second.c;
+    return HGPU_OK;
+  }
+  auto& cache = cache_of(ctx);
+  auto ct = cache.find(src);
+  if (ct == cache.end()) {
+    Compiled c{nullptr, nullptr};
+    // a shape the compiler rejects is remembered and left to the other kernels
+    if (compile(ctx, src, kname, &c) != HGPU_OK) c = Compiled{nullptr, nullptr};
+    ct = cache.emplace(src, c).first;
+  }
+  *out = ct->second;
+  known.emplace(key.bytes, KnownKernel{ct->second, hg::fusedgen::check_keys() ? src : std::string()});
+  return HGPU_OK;
+}
+
 struct Dim { int64_t e, sx, sy, sc; };
 
 // The rows operand is X, the columns operand Y (A and B, or swapped).
@@ -88,6 +118,16 @@ struct Plan {
   int bpc = 1; // blocks that share a CU (their LDS fits together): one's loads and stores run under the other's multiplications
   bool cvec;   // groups of four rows are adjacent in C and 16-byte aligned: vector stores
 };
+
+void put_plan(hg::fusedgen::Key& k, const Plan& pl) {
+  k.put(pl.f64).put(pl.mode).put(pl.nch).put(pl.chx).put(pl.chy).put(pl.chc).put(pl.min_rows).put(pl.nin);
+  k.put(pl.row_x).put(pl.row_c).put(pl.col_y).put(pl.col_c).put(pl.gx).put(pl.gy).put(pl.gp);
+  k.put(pl.px.size());
+  for (size_t p = 0; p < pl.px.size(); ++p)
+    for (int q = 0; q < 4; ++q) k.put(pl.px[p][(size_t)q]).put(pl.py[p][(size_t)q]);
+  k.put(pl.kvalid).put(pl.span_x).put(pl.span_y).put(pl.shift_x).put(pl.shift_y).put(pl.vx).put(pl.vy).put(pl.ys).put(pl.ypad);
+  k.put(pl.addr_regs).put(pl.nbufs).put(pl.ks).put(pl.colsum_at).put(pl.bpc).put(pl.cvec);
+}
 
 int64_t prod(const std::vector<Dim>& d) {
   int64_t p = 1;
@@ -791,6 +831,16 @@ bool vector_ok(const VirtualOp& v, int V) {
   return v.E.back() % V == 0 && v.P.back() % V == 0 && v.lo.back() % V == 0 && v.total % V == 0;
 }
 
+// Everything vops_source reads.
+void put_virtual(hg::fusedgen::Key& k, const VirtualOp& v, int V, int64_t chunk_stride, int64_t max_elem) {
+  k.put(v.n_in).put(v.n_instr, v.prog).put(v.slot).put(v.dtype).put(v.dt).put(v.E).put(v.M).put(v.lo).put(v.hi).put(v.P).put(v.total).put(v.padded);
+  for (int i = 0; i < v.n_in; ++i) {
+    const hgpu_array* a = v.in[i];
+    k.put(a->dtype).put(a->rank, a->shape).put(a->rank, a->strides).put((int)((uintptr_t)data_ptr(a) & 63));
+  }
+  k.put(V).put(chunk_stride).put(max_elem);
+}
+
 // Source of the three steps that stand in for the load of V consecutive
 // elements of an expression operand (tag "x" or "y"):
 //   VPre  vpre(w)                the place of element offset w (the chunk's own
@@ -1171,17 +1221,21 @@ int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const v
   // the last staging vector of the last chunk may reach past its footprint: how far at most
   const int64_t xmax = xbase + (pl.nch - 1) * pl.chx + (pl.span_x + pl.vx - 1) / pl.vx * pl.vx;
   const int64_t ymax = ybase + (pl.nch - 1) * pl.chy + (pl.span_y + pl.vy - 1) / pl.vy * pl.vy;
-  std::string src = generate(pl, kname, std::string(), 0, vx ? vops_source(*vx, "x", pl.vx, pl.chx, xmax) : std::string(), vx ? xbase : 0,
-                             vy ? vops_source(*vy, "y", pl.vy, pl.chy, ymax) : std::string(), vy ? ybase : 0);
-  auto& cache = cache_of(ctx);
-  auto it = cache.find(src);
-  if (it == cache.end()) {
-    Compiled c{nullptr, nullptr};
-    // a shape the compiler rejects is remembered and left to the other kernels
-    if (compile(ctx, src, kname, &c) != HGPU_OK) c = Compiled{nullptr, nullptr};
-    it = cache.emplace(src, c).first;
+  Compiled kernel{nullptr, nullptr};
+  {
+    fusedgen::Key key;
+    key.put(std::string(kname));
+    put_plan(key, pl);
+    key.put(vx != nullptr).put(vy != nullptr);
+    if (vx) { put_virtual(key, *vx, pl.vx, pl.chx, xmax); key.put(xbase); }
+    if (vy) { put_virtual(key, *vy, pl.vy, pl.chy, ymax); key.put(ybase); }
+    int rc = known_kernel(ctx, key, kname, [&] {
+      return generate(pl, kname, std::string(), 0, vx ? vops_source(*vx, "x", pl.vx, pl.chx, xmax) : std::string(), vx ? xbase : 0,
+                      vy ? vops_source(*vy, "y", pl.vy, pl.chy, ymax) : std::string(), vy ? ybase : 0);
+    }, &kernel);
+    if (rc) return rc;
   }
-  if (!it->second.fn) return HGPU_OK;
+  if (!kernel.fn) return HGPU_OK;
   const char* xp = (const char*)(best_swapped ? pb : pa) + pl.shift_x * es;
   const char* yp = (const char*)(best_swapped ? pa : pb) + pl.shift_y * es;
   int64_t out_n = nelem(out);
@@ -1222,7 +1276,7 @@ int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const v
     }
     {
       LaunchGuard lg(ctx, label, bytes, flops);
-      hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256u * (unsigned)pl.ks, 1, 1, 0, ctx->stream, args.data(), nullptr);
+      hipError_t e = hipModuleLaunchKernel(kernel.fn, (unsigned)grid, 1, 1, 256u * (unsigned)pl.ks, 1, 1, 0, ctx->stream, args.data(), nullptr);
       if (e != hipSuccess) { if (part) buffer_release(part); if (colsum) hgpu_release(colsum); return check_hip(ctx, e, "footprint gemm launch"); }
     }
     if (pl.mode == 0) {
@@ -1271,6 +1325,12 @@ struct EpiSpec {
   std::vector<int> out_off;            // per output: byte offset of its block in the stage buffer
   int val_off = 0, idx_off = 0, stage_bytes = 0;
 };
+
+void put_epilogue(hg::fusedgen::Key& k, const EpiSpec& e) {
+  k.put(e.n_in).put(e.c_slot).put(e.n_instr, e.prog).put(e.dt).put(e.cls).put(e.in_row).put(e.in_col).put(e.in_chs).put(e.out_slots);
+  k.put(e.has_ext).put(e.want_max).put(e.ext_slot).put(e.L).put(e.win_row).put(e.win_col).put(e.win_chs).put(e.out_chs);
+  k.put(e.staged).put(e.out_off).put(e.val_off).put(e.idx_off).put(e.stage_bytes);
+}
 
 std::string epilogue_source(const Plan& pl, const EpiSpec& e) {
   Src s;
@@ -1635,15 +1695,16 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
   char kname[160];
   snprintf(kname, sizeof kname, "footprint_gemm_%s_m%lld_n%lld_k%lld_chunkM%s_map%d%s%s", f64 ? "f64" : "f32", (long long)(swapped ? Nb : Ma), (long long)(swapped ? Ma : Nb),
            (long long)K, swapped ? "_swapped" : "", n_instr, has_ext ? (want_max ? "_max" : "_min") : "", pl.ks == 2 ? "_w8" : "");
-  std::string src = generate(pl, kname, epilogue_source(pl, e), e.staged ? e.stage_bytes : 0);
-  auto& cache = cache_of(ctx);
-  auto it = cache.find(src);
-  if (it == cache.end()) {
-    Compiled c{nullptr, nullptr};
-    if (compile(ctx, src, kname, &c) != HGPU_OK) c = Compiled{nullptr, nullptr};
-    it = cache.emplace(src, c).first;
+  Compiled kernel{nullptr, nullptr};
+  {
+    Key key;
+    key.put(std::string(kname));
+    put_plan(key, pl);
+    put_epilogue(key, e);
+    int rc = known_kernel(ctx, key, kname, [&] { return generate(pl, kname, epilogue_source(pl, e), e.staged ? e.stage_bytes : 0); }, &kernel);
+    if (rc) { release_all(); return rc; }
   }
-  if (!it->second.fn) { release_all(); return HGPU_OK; }
+  if (!kernel.fn) { release_all(); return HGPU_OK; }
 
   // kernel arguments: the footprint kernel's own, then the EpiArgs struct (pointers in declaration order)
   const char* xp = (swapped ? pb : pa) + pl.shift_x * es;
@@ -1673,7 +1734,7 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
       label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, bytes, flops);
-    hipError_t err = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256u * (unsigned)pl.ks, 1, 1, 0, ctx->stream, args, nullptr);
+    hipError_t err = hipModuleLaunchKernel(kernel.fn, (unsigned)grid, 1, 1, 256u * (unsigned)pl.ks, 1, 1, 0, ctx->stream, args, nullptr);
     if (err != hipSuccess) { release_all(); return check_hip(ctx, err, "contract_map launch"); }
   }
   for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
@@ -2131,15 +2192,20 @@ bool onehot_gate(const VirtualOp& v, int slot, int* which_in, int* where_in) {
   }
 }
 
-// x: the operand that is an array; y: the expression operand.  Both seen through views of `rank` dims of one shape.
-int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, const hgpu_operand* yo, int n_keep, hgpu_array* out, bool* handled) {
-  *handled = false;
-  static const bool disabled = getenv("HORDEAD_NO_ONEHOT") != nullptr;
-  if (disabled) return HGPU_OK;
-  if (v.dtype != HGPU_F64 && v.dtype != HGPU_F32) return HGPU_OK;
-  if (v.padded || yo->offset != 0 || v.total >= (1LL << 31)) return HGPU_OK;
-  int which_in = -1, where_in = -1;
-  if (!onehot_gate(v, v.slot, &which_in, &where_in)) return HGPU_OK;
+// What a call of the one-hot kernel needs besides its operands: worked out once per kind of call
+// (shapes, strides, program), found again by those.
+struct OnehotKnown {
+  bool taken = false;      // false: the kernel does not take this kind of call
+  Compiled c{nullptr, nullptr};
+  std::string kname, text; // (the text is kept with HORDEAD_GPU_CHECK_KEYS only)
+  int which_in = -1, MR = 0, NC = 0;
+  int64_t nch = 0, G = 0, EH = 0, span = 0, lo = 0;
+  std::vector<int64_t> colshape;   // the column sums' shape, and the merged dims of the expression they keep
+  std::vector<int> colk;
+};
+
+// The plan and the kernel's text for x (an array) times the expression v seen through yo; kn->taken stays false when the kernel does not fit.
+void plan_onehot(const hgpu_array* x, const VirtualOp& v, const hgpu_operand* yo, int n_keep, int64_t out_n, int which_in, int where_in, OnehotKnown* kn, std::string* text) {
   const int rank = yo->rank;
   const size_t re = v.E.size(), rm = v.M.size();
   // ---- the one-hot dims of the inputs' shape: where `which` moves; `where` must stand still there
@@ -2149,18 +2215,18 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   std::vector<std::pair<int64_t, size_t>> digits;      // (stride of which, dim)
   for (size_t j = 0; j < re; ++j) {
     if (v.E[j] == 1 || wh->strides[j] == 0) continue;
-    if (wh->strides[j] < 0 || wr->strides[j] != 0) return HGPU_OK;
+    if (wh->strides[j] < 0 || wr->strides[j] != 0) return;
     oh[j] = 1;
     digits.push_back({wh->strides[j], j});
   }
-  if (digits.empty()) return HGPU_OK;
+  if (digits.empty()) return;
   std::sort(digits.begin(), digits.end());
   int64_t EH = 1;                                        // values `which` takes: which.offset + 0 .. EH - 1, as a mixed-radix number of the one-hot dims
   for (auto& d : digits) {
-    if (d.first != EH) return HGPU_OK;
+    if (d.first != EH) return;
     EH *= v.E[d.second];
   }
-  if (EH < 2 || EH > 64) return HGPU_OK;
+  if (EH < 2 || EH > 64) return;
   // ---- the inputs' dims as parts of the merged dims; one-hot dims must be the innermost parts of theirs
   std::vector<int> group_of(re, -1);
   std::vector<int64_t> inner_oh(rm, 1);                  // product of the one-hot parts of merged dim k
@@ -2171,18 +2237,18 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
       int64_t got = 1;
       const size_t j_first = j;
       while (j < re && (got < v.M[k] || (j < re && v.E[j] == 1))) { group_of[j] = (int)k; got *= v.E[j]; ++j; }
-      if (got != v.M[k]) return HGPU_OK;
+      if (got != v.M[k]) return;
       int64_t u = 1;
       bool below_all_onehot = true;
       for (size_t q = j; q-- > j_first;) {
         unit[q] = u;
         u *= v.E[q];
         if (v.E[q] == 1) continue;
-        if (oh[q]) { if (!below_all_onehot) return HGPU_OK; inner_oh[k] *= v.E[q]; }
+        if (oh[q]) { if (!below_all_onehot) return; inner_oh[k] *= v.E[q]; }
         else below_all_onehot = false;
       }
     }
-    for (; j < re; ++j) if (v.E[j] != 1) return HGPU_OK;
+    for (; j < re; ++j) if (v.E[j] != 1) return;
   }
   // ---- the view's dims: each walks one whole merged dim (or none: the operand stands still)
   std::vector<int64_t> DM(rm, 1);
@@ -2198,11 +2264,11 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
     if (q.sy != 0) {
       for (size_t k = 0; k < rm; ++k)
         if (v.M[k] > 1 && DM[k] == q.sy && v.M[k] == q.e && !covered[k]) { q.k = (int)k; covered[k] = 1; break; }
-      if (q.k < 0) return HGPU_OK;
+      if (q.k < 0) return;
     }
     vd.push_back(q);
   }
-  for (size_t k = 0; k < rm; ++k) if (v.M[k] > 1 && !covered[k]) return HGPU_OK;
+  for (size_t k = 0; k < rm; ++k) if (v.M[k] > 1 && !covered[k]) return;
   // ---- rows (the array's kept dims), columns (the expression's), contracted dims; the chunk dim
   std::vector<int64_t> rx{0}, rco{0}, cy{0}, cco{0};
   auto extend = [](std::vector<int64_t>& a, std::vector<int64_t>& b, int64_t e, int64_t sa, int64_t sb) {
@@ -2215,11 +2281,11 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   for (size_t i = 0; i < vd.size(); ++i) {
     const VD& q = vd[i];
     if (q.kept) {
-      if (q.sx != 0 && q.sy == 0) { if ((int64_t)rx.size() * q.e > 32) return HGPU_OK; extend(rx, rco, q.e, q.sx, q.so); }
-      else if (q.sx == 0 && q.sy != 0) { if (inner_oh[(size_t)q.k] != 1 || (int64_t)cy.size() * q.e > 64) return HGPU_OK; extend(cy, cco, q.e, q.sy, q.so); }
-      else return HGPU_OK;
+      if (q.sx != 0 && q.sy == 0) { if ((int64_t)rx.size() * q.e > 32) return; extend(rx, rco, q.e, q.sx, q.so); }
+      else if (q.sx == 0 && q.sy != 0) { if (inner_oh[(size_t)q.k] != 1 || (int64_t)cy.size() * q.e > 64) return; extend(cy, cco, q.e, q.sy, q.so); }
+      else return;
     } else {
-      if (q.sx == 0 || q.sy == 0) return HGPU_OK;
+      if (q.sx == 0 || q.sy == 0) return;
       if (inner_oh[(size_t)q.k] == 1 && (chunk < 0 || q.e > vd[(size_t)chunk].e)) chunk = (int)i;
     }
   }
@@ -2227,11 +2293,11 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
     if (inner_oh[k] == 1) continue;
     bool contracted = false;
     for (auto& q : vd) contracted = contracted || (q.k == (int)k && !q.kept);
-    if (!contracted) return HGPU_OK;                     // a one-hot dim that is kept: nothing to skip
+    if (!contracted) return;                     // a one-hot dim that is kept: nothing to skip
   }
-  if (chunk < 0 || vd[(size_t)chunk].e < 64) return HGPU_OK;
+  if (chunk < 0 || vd[(size_t)chunk].e < 64) return;
   const int MR = (int)rx.size(), NC = (int)cy.size();
-  if (MR < 2) return HGPU_OK;
+  if (MR < 2) return;
   // ---- the other contracted positions of a chunk (one-hot parts left out), and where the one-hot parts lead
   std::vector<int64_t> gx{0}, gy{0};
   std::vector<int64_t> ohx((size_t)EH, 0), ohy((size_t)EH, 0);
@@ -2240,7 +2306,7 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
     if (q.kept || (int)i == chunk) continue;
     const int64_t io = inner_oh[(size_t)q.k];
     if (q.e / io > 1) {
-      if ((int64_t)gx.size() * (q.e / io) > 65536) return HGPU_OK;
+      if ((int64_t)gx.size() * (q.e / io) > 65536) return;
       extend(gx, gy, q.e / io, q.sx * io, q.sy * io);
     }
   }
@@ -2255,7 +2321,7 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
     }
   }
   const int64_t G = (int64_t)gx.size();
-  if ((double)G * NC * (double)vd[(size_t)chunk].e * MR < 1.0e7) return HGPU_OK;     // too little work for a kernel of its own
+  if ((double)G * NC * (double)vd[(size_t)chunk].e * MR < 1.0e7) return;     // too little work for a kernel of its own
   int64_t lo = 0, hi = 0;
   {
     int64_t rlo = rx[0], rhi = rx[0], glo = gx[0], ghi = gx[0], olo = ohx[0], ohi = ohx[0];
@@ -2267,14 +2333,14 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   }
   const int64_t span = hi - lo + 1;
   const int es = v.dtype == HGPU_F64 ? 8 : 4;
-  if (span * es > 64 * 1024 || span < 1) return HGPU_OK;
-  for (int64_t a : gy) if (a < 0 || a > INT32_MAX) return HGPU_OK;
+  if (span * es > 64 * 1024 || span < 1) return;
+  for (int64_t a : gy) if (a < 0 || a > INT32_MAX) return;
   const VD& chd = vd[(size_t)chunk];
   const int64_t nch = chd.e, chx = chd.sx, chy = chd.sy;
   // threads per column, a power of two: 256 threads share the columns out
   int TPC = 256;
   while (TPC * NC > 256) TPC >>= 1;
-  if (TPC < 1) return HGPU_OK;
+  if (TPC < 1) return;
   // ---- where every input of the expression is read: the offset of (chunk, column, position, one-hot place)
   // is a sum of four parts, tabulated here from the inputs' strides; nothing is decoded in the kernel
   std::vector<char> scalar((size_t)v.n_in, 0);
@@ -2306,12 +2372,12 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   for (int i = 0; i < v.n_in; ++i) {
     if (scalar[(size_t)i] || rep[(size_t)i] != i) continue;
     chs[(size_t)i] = in_off(i, chy);
-    if (in_off(i, chy * (nch - 1)) != chs[(size_t)i] * (nch - 1)) return HGPU_OK;     // the chunk dim is one dim of the inputs
+    if (in_off(i, chy * (nch - 1)) != chs[(size_t)i] * (nch - 1)) return;     // the chunk dim is one dim of the inputs
     int64_t reach = 0;
     for (size_t j = 0; j < re; ++j) reach += (v.E[j] - 1) * (v.in[i]->strides[j] < 0 ? -v.in[i]->strides[j] : v.in[i]->strides[j]);
     fits32 = fits32 && reach < (1LL << 31);
   }
-  if (!fits32) return HGPU_OK;
+  if (!fits32) return;
   Src s;
   char kname[160];
   snprintf(kname, sizeof kname, "onehot_contract_%s_m%d_n%d_k%lldx%lld_onehot%lld", es == 8 ? "f64" : "f32", MR, NC, (long long)nch, (long long)G, (long long)EH);
@@ -2410,28 +2476,77 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   s << "      if (m < " << MA << ") {\n        T sum = T(0);\n";
   s << "        for (int l = 0; l < " << TPC << "; ++l) sum += red[(m - m0) * 256 + c * " << TPC << " + l];\n";
   // a block's partial result: the rows of the product, then the columns' plain sums
-  s << "        if (m < " << MR << ") part[(i64)blockIdx.x * " << (int64_t)nelem(out) + NC << "ll + kRowC[m] + kColC[c]] = sum;\n";
-  s << "        else part[(i64)blockIdx.x * " << (int64_t)nelem(out) + NC << "ll + " << (int64_t)nelem(out) << " + c] = sum;\n      }\n    }\n  }\n}\n";
-  std::string src = s.str();
-  auto& cache = cache_of(ctx);
-  auto it = cache.find(src);
-  if (it == cache.end()) {
-    Compiled c{nullptr, nullptr};
-    if (compile(ctx, src, kname, &c) != HGPU_OK) c = Compiled{nullptr, nullptr};
-    it = cache.emplace(src, c).first;
+  s << "        if (m < " << MR << ") part[(i64)blockIdx.x * " << out_n + NC << "ll + kRowC[m] + kColC[c]] = sum;\n";
+  s << "        else part[(i64)blockIdx.x * " << out_n + NC << "ll + " << out_n << " + c] = sum;\n      }\n    }\n  }\n}\n";
+  *text = s.str();
+  kn->taken = true;
+  kn->kname = kname;
+  kn->which_in = which_in;
+  kn->MR = MR;
+  kn->NC = NC;
+  kn->nch = nch;
+  kn->G = G;
+  kn->EH = EH;
+  kn->span = span;
+  kn->lo = lo;
+  // the column sums: an array of the columns' shape, kept for a caller that asks for exactly that sum next
+  for (auto& q : vd)
+    if (q.kept && q.sx == 0) { kn->colshape.push_back(q.e); kn->colk.push_back(q.k); }
+}
+
+// x: the operand that is an array; y: the expression operand.  Both seen through views of `rank` dims of one shape.
+int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, const hgpu_operand* yo, int n_keep, hgpu_array* out, bool* handled) {
+  *handled = false;
+  static const bool disabled = getenv("HORDEAD_NO_ONEHOT") != nullptr;
+  if (disabled) return HGPU_OK;
+  if (v.dtype != HGPU_F64 && v.dtype != HGPU_F32) return HGPU_OK;
+  if (v.padded || yo->offset != 0 || v.total >= (1LL << 31)) return HGPU_OK;
+  int which_in = -1, where_in = -1;
+  if (!onehot_gate(v, v.slot, &which_in, &where_in)) return HGPU_OK;
+  const int64_t out_n = nelem(out);
+  Key key;
+  key.put(which_in).put(where_in).put(x->dtype).put(x->rank, x->shape).put(x->rank, x->strides).put((int)((uintptr_t)data_ptr(x) & 63));
+  put_virtual(key, v, 0, 0, 0);
+  for (int i = 0; i < v.n_in; ++i) key.put(v.in[i]->offset);
+  key.put(yo->rank, yo->shape).put(yo->rank, yo->strides).put(yo->offset).put(n_keep).put(out_n);
+  auto kit = ctx->jit_cache.find("__onehot_known__");
+  if (kit == ctx->jit_cache.end()) kit = ctx->jit_cache.emplace("__onehot_known__", new std::unordered_map<std::string, OnehotKnown>()).first;
+  auto& known = *static_cast<std::unordered_map<std::string, OnehotKnown>*>(kit->second);
+  auto found = known.find(key.bytes);
+  if (found == known.end() || check_keys()) {
+    OnehotKnown fresh;
+    std::string text;
+    plan_onehot(x, v, yo, n_keep, out_n, which_in, where_in, &fresh, &text);
+    if (found != known.end()) {
+      if (fresh.taken != found->second.taken || (fresh.taken && text != found->second.text)) return fail(ctx, HGPU_ERR_DEVICE, "onehot_contract: two different kernels under one key");
+    } else {
+      if (fresh.taken) {
+        auto& cache = cache_of(ctx);
+        auto it = cache.find(text);
+        if (it == cache.end()) {
+          Compiled c{nullptr, nullptr};
+          if (compile(ctx, text, fresh.kname, &c) != HGPU_OK) c = Compiled{nullptr, nullptr};
+          it = cache.emplace(text, c).first;
+        }
+        fresh.c = it->second;
+        if (check_keys()) fresh.text = text;
+      }
+      found = known.emplace(key.bytes, std::move(fresh)).first;
+    }
   }
-  if (!it->second.fn) return HGPU_OK;
+  const OnehotKnown& kn = found->second;
+  if (!kn.taken || !kn.c.fn) return HGPU_OK;
+  const hgpu_array* wh = v.in[kn.which_in];
+  const int es = v.dtype == HGPU_F64 ? 8 : 4;
+  const int MR = kn.MR, NC = kn.NC;
+  const int64_t nch = kn.nch, G = kn.G, EH = kn.EH, span = kn.span, lo = kn.lo;
+  const std::vector<int64_t>& colshape = kn.colshape;
+  const std::vector<int>& colk = kn.colk;
   wh->buf->known_relied_on = true;
   for (int i = 0; i < v.n_in; ++i)
     if (v.in[i]->buf && v.in[i]->buf->known == hgpu_buffer::kZeroScalar) v.in[i]->buf->known_relied_on = true;
   static const int knob_grid = getenv("HORDEAD_ONEHOT_GRID") ? atoi(getenv("HORDEAD_ONEHOT_GRID")) : 2;
   const int64_t grid = std::min<int64_t>(nch, (int64_t)ctx->num_cu * knob_grid);
-  const int64_t out_n = nelem(out);
-  // the column sums: an array of the columns' shape, kept for a caller that asks for exactly that sum next
-  std::vector<int64_t> colshape;
-  std::vector<int> colk;
-  for (auto& q : vd)
-    if (q.kept && q.sx == 0) { colshape.push_back(q.e); colk.push_back(q.k); }
   hgpu_array* colsum = nullptr;
   int rc = new_dense(ctx, v.dtype, (int)colshape.size(), colshape.data(), &colsum);
   if (rc) return rc;
@@ -2446,7 +2561,7 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
   {
     double bytes = (double)nch * span * es;
     for (int i = 0; i < v.n_in; ++i) {
-      if (i == which_in) continue;
+      if (i == kn.which_in) continue;
       int64_t distinct = 1;
       for (int d = 0; d < v.in[i]->rank; ++d)
         if (v.in[i]->strides[d] != 0) distinct *= v.in[i]->shape[d];
@@ -2459,7 +2574,7 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
       label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, bytes, 2.0 * MR * NC * (double)G * (double)nch);
-    hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+    hipError_t e = hipModuleLaunchKernel(kn.c.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
     if (e != hipSuccess) { buffer_release(part); hgpu_release(colsum); return check_hip(ctx, e, "onehot_contract launch"); }
   }
   rc = hg::sum_partials_split(ctx, v.dtype, out_n, NC, (int)grid, part->ptr, data_ptr(out), data_ptr(colsum));

@@ -132,6 +132,42 @@ void buffer_release(hgpu_buffer* b) {
   }
 }
 
+}  // namespace hg
+
+namespace {
+struct ArrayBlocks {
+  struct Node { Node* next; };
+  Node* head = nullptr;
+  size_t n = 0;
+  ~ArrayBlocks() {
+    while (head) { Node* x = head; head = head->next; ::operator delete(x); }
+  }
+};
+thread_local ArrayBlocks array_blocks;
+constexpr size_t kArrayBlocksKept = 16384;
+}  // namespace
+
+void* hgpu_array::operator new(size_t n) {
+  ArrayBlocks& ab = array_blocks;
+  if (n == sizeof(hgpu_array) && ab.head) {
+    ArrayBlocks::Node* x = ab.head;
+    ab.head = x->next;
+    --ab.n;
+    return x;
+  }
+  return ::operator new(n < sizeof(hgpu_array) ? sizeof(hgpu_array) : n);
+}
+void hgpu_array::operator delete(void* p) {
+  if (!p) return;
+  ArrayBlocks& ab = array_blocks;
+  if (ab.n >= kArrayBlocksKept) { ::operator delete(p); return; }
+  auto* x = static_cast<ArrayBlocks::Node*>(p);
+  x->next = ab.head;
+  ab.head = x;
+  ++ab.n;
+}
+
+namespace hg {
 hgpu_array* new_view(hgpu_ctx* ctx, hgpu_buffer* buf, int dtype, int rank, const int64_t* shape,
                      const int64_t* strides, int64_t offset) {
   hgpu_array* a = new hgpu_array;

@@ -7,7 +7,10 @@
 // library, so the same object code drives the gfx950 library in production and
 // any other provider of the ABI a test hands in.
 #pragma once
+#include <algorithm>
 #include <cstdint>
+#include <initializer_list>
+#include <iterator>
 #include <functional>
 #include <map>
 #include <memory>
@@ -19,7 +22,110 @@
 
 namespace hordead {
 
-using Shape = std::vector<int64_t>;
+// A shape, or the strides that go with one: a vector of a few extents that sits in
+// place up to kInPlace of them (no allocation: shapes are made, copied and dropped
+// at every operation) and on the heap beyond.  The part of std::vector's interface
+// that the layer uses.
+class Shape {
+ public:
+  using value_type = int64_t;
+  using iterator = int64_t*;
+  using const_iterator = const int64_t*;
+  static constexpr size_t kInPlace = 8;
+  Shape() {}
+  explicit Shape(size_t n, int64_t v = 0) { grow(n); n_ = n; std::fill(p_, p_ + n, v); }
+  Shape(std::initializer_list<int64_t> l) { grow(l.size()); n_ = l.size(); std::copy(l.begin(), l.end(), p_); }
+  template <typename It, typename = typename std::iterator_traits<It>::iterator_category>
+  Shape(It a, It b) { const size_t n = (size_t)std::distance(a, b); grow(n); n_ = n; std::copy(a, b, p_); }
+  Shape(const Shape& o) { grow(o.n_); n_ = o.n_; std::copy(o.p_, o.p_ + n_, p_); }
+  Shape(Shape&& o) noexcept { steal(o); }
+  Shape(const std::vector<int64_t>& v) : Shape(v.begin(), v.end()) {}
+  ~Shape() { if (p_ != in_) delete[] p_; }
+  Shape& operator=(const Shape& o) {
+    if (this != &o) { n_ = 0; grow(o.n_); n_ = o.n_; std::copy(o.p_, o.p_ + n_, p_); }
+    return *this;
+  }
+  Shape& operator=(Shape&& o) noexcept {
+    if (this != &o) { if (p_ != in_) delete[] p_; p_ = in_; cap_ = kInPlace; steal(o); }
+    return *this;
+  }
+  size_t size() const { return n_; }
+  bool empty() const { return n_ == 0; }
+  int64_t* data() { return p_; }
+  const int64_t* data() const { return p_; }
+  iterator begin() { return p_; }
+  iterator end() { return p_ + n_; }
+  const_iterator begin() const { return p_; }
+  const_iterator end() const { return p_ + n_; }
+  std::reverse_iterator<iterator> rbegin() { return std::reverse_iterator<iterator>(end()); }
+  std::reverse_iterator<iterator> rend() { return std::reverse_iterator<iterator>(begin()); }
+  std::reverse_iterator<const_iterator> rbegin() const { return std::reverse_iterator<const_iterator>(end()); }
+  std::reverse_iterator<const_iterator> rend() const { return std::reverse_iterator<const_iterator>(begin()); }
+  int64_t& operator[](size_t i) { return p_[i]; }
+  const int64_t& operator[](size_t i) const { return p_[i]; }
+  int64_t& at(size_t i) { if (i >= n_) throw std::out_of_range("Shape::at"); return p_[i]; }
+  const int64_t& at(size_t i) const { if (i >= n_) throw std::out_of_range("Shape::at"); return p_[i]; }
+  int64_t& front() { return p_[0]; }
+  const int64_t& front() const { return p_[0]; }
+  int64_t& back() { return p_[n_ - 1]; }
+  const int64_t& back() const { return p_[n_ - 1]; }
+  void clear() { n_ = 0; }
+  void reserve(size_t n) { grow(n); }
+  void push_back(int64_t v) { grow(n_ + 1); p_[n_++] = v; }
+  void emplace_back(int64_t v) { push_back(v); }
+  void pop_back() { --n_; }
+  void resize(size_t n, int64_t v = 0) { grow(n); if (n > n_) std::fill(p_ + n_, p_ + n, v); n_ = n; }
+  void assign(size_t n, int64_t v) { n_ = 0; grow(n); n_ = n; std::fill(p_, p_ + n, v); }
+  template <typename It, typename = typename std::iterator_traits<It>::iterator_category>
+  void assign(It a, It b) { Shape t(a, b); *this = std::move(t); }
+  iterator insert(const_iterator at, int64_t v) { return insert(at, &v, &v + 1); }
+  template <typename It, typename = typename std::iterator_traits<It>::iterator_category>
+  iterator insert(const_iterator at, It a, It b) {
+    const size_t i = (size_t)(at - p_), k = (size_t)std::distance(a, b);
+    if (k == 0) return p_ + i;
+    int64_t tmp_in[kInPlace];   // the range may lie in this very object
+    std::vector<int64_t> tmp_big;
+    int64_t* src = tmp_in;
+    if (k > kInPlace) { tmp_big.assign(a, b); src = tmp_big.data(); } else std::copy(a, b, tmp_in);
+    grow(n_ + k);
+    std::copy_backward(p_ + i, p_ + n_, p_ + n_ + k);
+    std::copy(src, src + k, p_ + i);
+    n_ += k;
+    return p_ + i;
+  }
+  iterator erase(const_iterator at) { return erase(at, at + 1); }
+  iterator erase(const_iterator a, const_iterator b) {
+    const size_t i = (size_t)(a - p_), j = (size_t)(b - p_);
+    std::copy(p_ + j, p_ + n_, p_ + i);
+    n_ -= j - i;
+    return p_ + i;
+  }
+  void swap(Shape& o) { Shape t(std::move(o)); o = std::move(*this); *this = std::move(t); }
+  friend bool operator==(const Shape& a, const Shape& b) { return a.n_ == b.n_ && std::equal(a.p_, a.p_ + a.n_, b.p_); }
+  friend bool operator!=(const Shape& a, const Shape& b) { return !(a == b); }
+  friend bool operator<(const Shape& a, const Shape& b) { return std::lexicographical_compare(a.begin(), a.end(), b.begin(), b.end()); }
+  operator std::vector<int64_t>() const { return std::vector<int64_t>(begin(), end()); }
+
+ private:
+  void grow(size_t n) {
+    if (n <= cap_) return;
+    size_t c = cap_ * 2 > n ? cap_ * 2 : n;
+    int64_t* q = new int64_t[c];
+    std::copy(p_, p_ + n_, q);
+    if (p_ != in_) delete[] p_;
+    p_ = q;
+    cap_ = c;
+  }
+  void steal(Shape& o) {
+    n_ = o.n_;
+    if (o.p_ == o.in_) { std::copy(o.in_, o.in_ + n_, in_); }
+    else { p_ = o.p_; cap_ = o.cap_; o.p_ = o.in_; o.cap_ = kInPlace; }
+    o.n_ = 0;
+  }
+  int64_t in_[kInPlace];
+  int64_t* p_ = in_;
+  size_t n_ = 0, cap_ = kInPlace;
+};
 
 struct HostError : std::runtime_error {
   int code;
@@ -146,12 +252,58 @@ struct ArrHolder {
   bool view_of_written_source();
 };
 
+// Memory for the holders: a training step makes thousands of them and frees most together when its
+// tape goes, more than the allocator's per-thread cache of one block size holds, so freed blocks are
+// kept on a list per thread (and per block size) and handed out again.
+template <size_t N>
+struct BlockList {
+  struct Node { Node* next; };
+  Node* head = nullptr;
+  size_t n = 0;
+  ~BlockList() {
+    while (head) { Node* x = head; head = head->next; ::operator delete(x); }
+  }
+  static BlockList& mine() {
+    static thread_local BlockList l;
+    return l;
+  }
+};
+template <typename U>
+struct BlockAlloc {
+  using value_type = U;
+  BlockAlloc() = default;
+  template <typename V> BlockAlloc(const BlockAlloc<V>&) {}
+  U* allocate(size_t k) {
+    if (k == 1) {
+      auto& l = BlockList<sizeof(U)>::mine();
+      if (l.head) {
+        auto* x = l.head;
+        l.head = x->next;
+        --l.n;
+        return reinterpret_cast<U*>(x);
+      }
+    }
+    return static_cast<U*>(::operator new(k * sizeof(U)));
+  }
+  void deallocate(U* p, size_t k) {
+    auto& l = BlockList<sizeof(U)>::mine();
+    if (k != 1 || l.n >= 16384) { ::operator delete(p); return; }
+    auto* x = reinterpret_cast<typename BlockList<sizeof(U)>::Node*>(p);
+    x->next = l.head;
+    l.head = x;
+    ++l.n;
+  }
+  template <typename V> bool operator==(const BlockAlloc<V>&) const { return true; }
+  template <typename V> bool operator!=(const BlockAlloc<V>&) const { return false; }
+};
+inline std::shared_ptr<ArrHolder> new_holder(Backend* be, hgpu_array* h) { return std::allocate_shared<ArrHolder>(BlockAlloc<ArrHolder>(), be, h); }
+
 // `Gpu (TKS sh r)`: an immutable strided view on the device.  Scalars
 // (`TKScalar r`) are rank-0 views, so that they never force a device sync.
 class T {
  public:
   T() {}
-  T(Backend* be, hgpu_array* h) : p_(std::make_shared<ArrHolder>(be, h)) {}
+  T(Backend* be, hgpu_array* h) : p_(new_holder(be, h)) {}
   explicit T(std::shared_ptr<ArrHolder> p) : p_(std::move(p)) {}
   const std::shared_ptr<ArrHolder>& holder() const { return p_; }
   bool valid() const { return (bool)p_; }

@@ -236,7 +236,7 @@ bool meta_as_strided(const Meta& a, const Shape& shape, const Shape& strides, in
 }  // namespace
 
 static T make_probe(Backend* be, const Meta& m, int dtype) {
-  auto p = std::make_shared<ArrHolder>(be, nullptr);
+  auto p = new_holder(be, nullptr);
   p->probe = true;
   p->probe_dtype = dtype;
   p->vmeta = m;
@@ -244,7 +244,7 @@ static T make_probe(Backend* be, const Meta& m, int dtype) {
 }
 // The view m over the dense result of the pending value src.
 static T make_view(const std::shared_ptr<ArrHolder>& src, const Meta& m) {
-  auto p = std::make_shared<ArrHolder>(src->be, nullptr);
+  auto p = new_holder(src->be, nullptr);
   p->vsrc = src;
   p->vmeta = m;
   return T(p);
@@ -384,7 +384,7 @@ static void note_common_view(ArrHolder* p, int kind, int op, int dtype, const T&
 }
 
 static T make_expr(int kind, int op, int dtype, const T& a, const T* b, const T* c) {
-  auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
+  auto p = new_holder(a.be(), nullptr);
   p->ekind = kind;
   p->eop = op;
   p->edtype = dtype;
@@ -1060,7 +1060,7 @@ static bool sums_with(const T& a, const T& b) {
 T add_cotangents(const T& a, const T& b) {
   if (a.contraction_like() && b.contraction_like() && a.be() == b.be() && a.holder()->keep == b.holder()->keep &&
       a.dtype() == b.dtype() && sums_with(a, b)) {
-    auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
+    auto p = new_holder(a.be(), nullptr);
     const ArrHolder* x = a.holder().get();
     const ArrHolder* y = b.holder().get();
     p->fa = x->fa;
@@ -1102,7 +1102,7 @@ T add_cotangents(const T& a, const T& b) {
 T lazy_mul(const T& a, const T& b) { return ewise2(HGPU_MUL, a, b); }
 
 T lazy_contract(const T& a, const T& b, int n_keep) {
-  auto p = std::make_shared<ArrHolder>(a.be(), nullptr);
+  auto p = new_holder(a.be(), nullptr);
   p->fa = a.holder();
   p->fb = b.holder();
   p->keep = n_keep;
@@ -1131,7 +1131,7 @@ static T map_leaves(const T& a, const std::function<T(const T&)>& view) {
       else if (!p->h && !leaf.pending_view()) p->force();
       r = view(leaf).holder();
     } else {
-      r = std::make_shared<ArrHolder>(p->be, nullptr);
+      r = new_holder(p->be, nullptr);
       r->ekind = p->ekind;
       r->eop = p->eop;
       r->edtype = p->edtype;
@@ -1181,7 +1181,7 @@ static bool refines(const Shape& fine, const Shape& coarse, std::vector<int>* gr
 
 static T make_merged(const T& inner, const Shape& shape, const std::vector<int>& groups) {
   if (!inner.pending_expr()) return reshape(inner, shape);   // already an array: merge its dims now
-  auto p = std::make_shared<ArrHolder>(inner.be(), nullptr);
+  auto p = new_holder(inner.be(), nullptr);
   p->mv_inner = inner.holder();
   p->mv_shape = shape;
   p->mv_groups = groups;
@@ -1491,7 +1491,7 @@ T contract(const T& a, const T* b, int n_keep) {
     // of this shape, the sum waits for such a pass (the gradient's)
     if (be->fuse && api->struct_size >= offsetof(hgpu_api, fused_map_sums) + sizeof(api->fused_map_sums) && api->fused_map_sums && pending_size(a.holder()) <= 40 &&
         a.size() >= 4096) {
-      auto p = std::make_shared<ArrHolder>(be, nullptr);
+      auto p = new_holder(be, nullptr);
       p->ssrc = a.holder();
       auto& ps = be->pending_sums;
       ps.erase(std::remove_if(ps.begin(), ps.end(), [](const std::weak_ptr<ArrHolder>& w) { auto q = w.lock(); return !q || q->h || !q->ssrc; }), ps.end());
@@ -1518,7 +1518,7 @@ T contract(const T& a, const T* b, int n_keep) {
     const hgpu_api* api = a.be()->api;
     if (api->struct_size >= offsetof(hgpu_api, fused_map_sums) + sizeof(api->fused_map_sums) && api->fused_map_sums) {
       Backend* be = a.be();
-      auto p = std::make_shared<ArrHolder>(be, nullptr);
+      auto p = new_holder(be, nullptr);
       p->ssrc = make_expr(HGPU_FUSED_OP2, HGPU_MUL, a.dtype(), a, b, nullptr).holder();
       auto& ps = be->pending_sums;
       ps.erase(std::remove_if(ps.begin(), ps.end(), [](const std::weak_ptr<ArrHolder>& w) { auto q = w.lock(); return !q || q->h || !q->ssrc; }), ps.end());
@@ -1625,7 +1625,7 @@ static T from_pieces(Backend* be, std::vector<ArrHolder::Piece> pcs, const Shape
   }
   if (m.size() == 1 && m[0].v) return T(m[0].v);
   if (m.empty()) return zeros(be, dtype, shape);
-  auto p = std::make_shared<ArrHolder>(be, nullptr);
+  auto p = new_holder(be, nullptr);
   p->pieces = std::move(m);
   p->pshape = shape;
   p->pdtype = dtype;
