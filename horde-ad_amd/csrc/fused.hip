@@ -17,6 +17,7 @@
 #include <hip/hiprtc.h>
 
 #include <memory>
+#include <unordered_map>
 
 #include "common.hpp"
 #include "fused_gen.hpp"
@@ -47,6 +48,39 @@ int compile(hgpu_ctx* ctx, const std::string& src, Compiled* out, const char* kn
   if (e != hipSuccess) return check_hip(ctx, e, "hipModuleLoadData");
   e = hipModuleGetFunction(&out->fn, out->mod, kname);
   if (e != hipSuccess) return check_hip(ctx, e, "hipModuleGetFunction");
+  return HGPU_OK;
+}
+
+// Kernels found again by what their text depends on (the inputs' layouts and the program).
+struct Known { Compiled c; std::string text; };
+const Known* find_known(hgpu_ctx* ctx, const Key& key) {
+  std::lock_guard<std::mutex> lk(ctx->launch_mu);
+  auto kit = ctx->jit_cache.find("__fused_known__");
+  if (kit == ctx->jit_cache.end()) return nullptr;
+  auto& known = *static_cast<std::unordered_map<std::string, Known>*>(kit->second);
+  auto it = known.find(key.bytes);
+  return it == known.end() ? nullptr : &it->second;
+}
+// The kernel of a call: the known one (`hit`; with HORDEAD_GPU_CHECK_KEYS its text is compared with the one just written),
+// else the one with the text `src`, compiled if need be and remembered under the key.  Call with launch_mu held.
+int kernel_for(hgpu_ctx* ctx, const Key& key, const Known* hit, const std::string& src, const char* kname, Compiled* out) {
+  if (hit) {
+    if (check_keys() && hit->text != src) return fail(ctx, HGPU_ERR_DEVICE, "%s: two different kernels under one key", kname);
+    *out = hit->c;
+    return HGPU_OK;
+  }
+  auto& cache = cache_of(ctx);
+  auto it = cache.find(src);
+  if (it == cache.end()) {
+    Compiled c;
+    int rc = compile(ctx, src, &c, kname);
+    if (rc) return rc;
+    it = cache.emplace(src, c).first;
+  }
+  auto kit = ctx->jit_cache.find("__fused_known__");
+  if (kit == ctx->jit_cache.end()) kit = ctx->jit_cache.emplace("__fused_known__", new std::unordered_map<std::string, Known>()).first;
+  static_cast<std::unordered_map<std::string, Known>*>(kit->second)->emplace(key.bytes, Known{it->second, check_keys() ? src : std::string()});
+  *out = it->second;
   return HGPU_OK;
 }
 
@@ -200,11 +234,16 @@ static int fused_map_impl(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, 
   }
 
   // ---- source
-  Src s;
+  const char* kernel_name = sum_slot >= 0 ? "fused_map_dimsum" : "fused_map";
+  Key key;
+  key.put(std::string(kernel_name)).put(n_out).put(sum_slot).put(keep_dim);
+  for (int o = 0; o < n_out; ++o) key.put(out_slots[o]);
+  put_inputs(key, n_in, in, n_instr, prog);
+  const Known* hit = find_known(ctx, key);
+  Src s(!hit || check_keys());
   s << kPrelude;
   if (!all_simple) s << "struct FDims { int nd; i64 shape[" << HG_KDIMS << "]; i64 st[" << kMaxIn << "][" << HG_KDIMS << "]; };\n";
   s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
-  const char* kernel_name = sum_slot >= 0 ? "fused_map_dimsum" : "fused_map";
   s << "extern \"C\" __global__ void __launch_bounds__(256) " << kernel_name << "(i64 n";
   if (!all_simple && !bake) s << ", FDims d";
   for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
@@ -379,14 +418,8 @@ static int fused_map_impl(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, 
   }
   std::unique_ptr<LaunchGuard> guard(new LaunchGuard(ctx, label, 0, 0));   // ends before the partial sums' own launch
   LaunchGuard& lg = *guard;
-  auto& cache = cache_of(ctx);
-  auto it = cache.find(src);
-  if (it == cache.end()) {
-    Compiled c;
-    int rc = compile(ctx, src, &c, kernel_name);
-    if (rc) { release_all(); return rc; }
-    it = cache.emplace(src, c).first;
-  }
+  Compiled kernel;
+  if (int rc = kernel_for(ctx, key, hit, src, kernel_name, &kernel)) { release_all(); return rc; }
   // algorithmic traffic: every distinct non-broadcast input once, every output once
   double bytes = 0;
   for (int i = 0; i < n_in; ++i) {
@@ -423,7 +456,7 @@ static int fused_map_impl(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, 
     args.push_back(&part_ptr);
     grid = (unsigned)(dsC * ds_chunks);
   }
-  hipError_t e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  hipError_t e = hipModuleLaunchKernel(kernel.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
   if (e != hipSuccess) { if (part) buffer_release(part); if (sums) hgpu_release(sums); release_all(); return check_hip(ctx, e, "fused_map launch"); }
   guard.reset();
   if (part) {
@@ -509,7 +542,11 @@ extern "C" int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     }
   }
   // ---- source: shapes and strides are constants of the kernel
-  Src s;
+  Key key;
+  key.put(std::string("fused_extremum")).put(slot).put(n_reduce).put(want_max);
+  put_inputs(key, n_in, in, n_instr, prog);
+  const Known* hit = find_known(ctx, key);
+  Src s(!hit || check_keys());
   s << kPrelude;
   s << "extern \"C\" __global__ void __launch_bounds__(256) fused_extremum(i64 n";
   for (int i = 0; i < n_in; ++i) s << ", const " << ctype(in[i]->dtype) << "* __restrict__ i" << i;
@@ -570,14 +607,9 @@ extern "C" int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     bytes += (double)distinct * dtype_size(in[i]->dtype);
   }
   LaunchGuard lg(ctx, label, bytes, (double)n_out * L * (n_instr + 1));
-  auto& cache = cache_of(ctx);
-  auto it = cache.find(src);
-  if (it == cache.end()) {
-    Compiled c;
-    rc = compile(ctx, src, &c, "fused_extremum");
-    if (rc) { hgpu_release(v); hgpu_release(ix); return rc; }
-    it = cache.emplace(src, c).first;
-  }
+  Compiled kernel;
+  rc = kernel_for(ctx, key, hit, src, "fused_extremum", &kernel);
+  if (rc) { hgpu_release(v); hgpu_release(ix); return rc; }
   std::vector<void*> args;
   int64_t nn = n_out;
   args.push_back(&nn);
@@ -588,7 +620,7 @@ extern "C" int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   args.push_back(&pv);
   args.push_back(&pi);
   unsigned grid = grid_for(n_out, 256, ctx->num_cu * 16);
-  hipError_t e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  hipError_t e = hipModuleLaunchKernel(kernel.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
   if (e != hipSuccess) { hgpu_release(v); hgpu_release(ix); return check_hip(ctx, e, "fused_extremum launch"); }
   *values = v;
   *indices = ix;
@@ -652,7 +684,11 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     if (rc) { drop_part(); hgpu_release(o); return rc; }
   }
 
-  Src s;
+  Key key;
+  key.put(std::string("fused_sum")).put(slot);
+  put_inputs(key, n_in, in, n_instr, prog);
+  const Known* hit = find_known(ctx, key);
+  Src s(!hit || check_keys());
   s << kPrelude;
   s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
   s << "typedef " << acc << " ACC;\n";
@@ -752,14 +788,9 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
     if (!dup) bytes += (double)n * dtype_size(in[i]->dtype);
   }
   LaunchGuard lg(ctx, label, bytes, (double)n * (n_instr + 1));
-  auto& cache = cache_of(ctx);
-  auto it = cache.find(src);
-  if (it == cache.end()) {
-    Compiled c;
-    rc = compile(ctx, src, &c, "fused_sum");
-    if (rc) { drop_part(); hgpu_release(o); return rc; }
-    it = cache.emplace(src, c).first;
-  }
+  Compiled kernel;
+  rc = kernel_for(ctx, key, hit, src, "fused_sum", &kernel);
+  if (rc) { drop_part(); hgpu_release(o); return rc; }
   std::vector<void*> args;
   int64_t nn = n;
   args.push_back(&nn);
@@ -772,8 +803,8 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   if (single || ticketed) args.push_back(&po);
   hipFunction_t fin = nullptr;
   hipError_t e = hipSuccess;
-  if (!single && !ticketed) e = hipModuleGetFunction(&fin, it->second.mod, "fused_sum_final");
-  if (e == hipSuccess) e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (!single && !ticketed) e = hipModuleGetFunction(&fin, kernel.mod, "fused_sum_final");
+  if (e == hipSuccess) e = hipModuleLaunchKernel(kernel.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
   if (e == hipSuccess && fin) {
     int g = (int)grid;
     void* fargs[] = {&g, &pp, &po};
@@ -853,7 +884,13 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
     if (rc) { drop_part(); release_all(); return rc; }
   }
 
-  Src s;
+  Key key;
+  key.put(std::string("fused_map_sums")).put(n_out).put(n_sum);
+  for (int o = 0; o < n_out; ++o) key.put(out_slots[o]);
+  for (int j = 0; j < n_sum; ++j) key.put(sum_slots[j]);
+  put_inputs(key, n_in, in, n_instr, prog);
+  const Known* hit = find_known(ctx, key);
+  Src s(!hit || check_keys());
   s << kPrelude;
   s << "template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };\n";
   s << "template <typename A> __device__ __forceinline__ A wave_sum(A v) {\n"
@@ -973,14 +1010,9 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   }
   for (int o = 0; o < n_out; ++o) bytes += (double)n * dtype_size(res[(size_t)o]->dtype);
   LaunchGuard lg(ctx, label, bytes, (double)n * n_instr);
-  auto& cache = cache_of(ctx);
-  auto it = cache.find(src);
-  if (it == cache.end()) {
-    Compiled c;
-    rc = compile(ctx, src, &c, "fused_map_sums");
-    if (rc) { drop_part(); release_all(); return rc; }
-    it = cache.emplace(src, c).first;
-  }
+  Compiled kernel;
+  rc = kernel_for(ctx, key, hit, src, "fused_map_sums", &kernel);
+  if (rc) { drop_part(); release_all(); return rc; }
   std::vector<void*> args;
   int64_t nn = n;
   args.push_back(&nn);
@@ -995,8 +1027,8 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   if (single || ticketed) for (int j = 0; j < n_sum; ++j) args.push_back(&sptrs[(size_t)j]);
   hipFunction_t fin = nullptr;
   hipError_t e = hipSuccess;
-  if (!single && !ticketed) e = hipModuleGetFunction(&fin, it->second.mod, "fused_map_sums_final");
-  if (e == hipSuccess) e = hipModuleLaunchKernel(it->second.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (!single && !ticketed) e = hipModuleGetFunction(&fin, kernel.mod, "fused_map_sums_final");
+  if (e == hipSuccess) e = hipModuleLaunchKernel(kernel.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
   if (e == hipSuccess && fin) {
     int g = (int)grid;
     std::vector<void*> fargs = {&g, &pp};

@@ -21,19 +21,22 @@ namespace fusedgen {
 // its text).
 struct Src {
   std::string text;
+  bool on = true;   // false: the kernel is known already, nothing is written (the generator still runs: it also works out how to launch)
   Src() { text.reserve(16384); }
-  Src& operator<<(const char* t) { text.append(t); return *this; }
-  Src& operator<<(const std::string& t) { text.append(t); return *this; }
-  Src& operator<<(char c) { text.push_back(c); return *this; }
+  explicit Src(bool write) : on(write) { if (on) text.reserve(16384); }
+  Src& operator<<(const char* t) { if (on) text.append(t); return *this; }
+  Src& operator<<(const std::string& t) { if (on) text.append(t); return *this; }
+  Src& operator<<(char c) { if (on) text.push_back(c); return *this; }
   template <typename I, typename std::enable_if<std::is_integral<I>::value && !std::is_same<I, char>::value && !std::is_same<I, bool>::value &&
                                                     !std::is_same<I, signed char>::value && !std::is_same<I, unsigned char>::value, int>::type = 0>
   Src& operator<<(I v) {
+    if (!on) return *this;
     char buf[24];
     auto r = std::to_chars(buf, buf + sizeof buf, v);
     text.append(buf, (size_t)(r.ptr - buf));
     return *this;
   }
-  Src& operator<<(bool v) { text.push_back(v ? '1' : '0'); return *this; }
+  Src& operator<<(bool v) { if (on) text.push_back(v ? '1' : '0'); return *this; }
   const std::string& str() const { return text; }
 };
 
@@ -55,6 +58,12 @@ struct Key {
     return *this;
   }
 };
+// The arrays and the program of a fused call, as far as a kernel's text can depend on them.
+inline void put_inputs(Key& k, int n_in, const hgpu_array* const* in, int n_instr, const hgpu_fused_instr* prog) {
+  k.put(n_in);
+  for (int i = 0; i < n_in; ++i) k.put(in[i]->dtype).put(in[i]->rank, in[i]->shape).put(in[i]->rank, in[i]->strides).put((int)((uintptr_t)data_ptr(in[i]) & 63));
+  k.put(n_instr, prog);
+}
 inline bool check_keys() {
   static const bool on = getenv("HORDEAD_GPU_CHECK_KEYS") != nullptr;
   return on;
