@@ -9,6 +9,10 @@ GPU half: the same programs on the gfx950 library against the checker on the
 same seeded inputs: fp64 to 1e-10, fp32 to 1e-5 (normwise relative; device
 reductions associate differently from the checker's sequential double sums).
 """
+import os
+import subprocess
+import sys
+
 import numpy as np
 import pytest
 
@@ -211,6 +215,55 @@ def test_gpu_matches_checker(host_gpu, host_cpu, name, size):
         assert g.shape == c.shape and g.dtype == c.dtype
         record_error("%s %s gradient %d" % (name, size, i), float(np.max(np.abs(g - c))) / max(float(np.max(np.abs(c))), 1e-300), tol)
         assert close(g, c, tol), (name, size, i, float(np.max(np.abs(g - c))) / max(float(np.max(np.abs(c))), 1e-300))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(MEDIUM))
+def test_gpu_later_calls_repeat_the_first(host_gpu, name):
+    """The first call of a kind writes its kernels' text and compiles them; later
+    calls find the kernels by shapes, strides and programs alone.  They must be the
+    same kernels: every repetition gives the bits of the first."""
+    mk, kw = MEDIUM[name]
+    wl = mk(**kw)
+    l0, g0 = run(host_gpu, wl)
+    for _ in range(2):
+        l, g = run(host_gpu, wl)
+        assert l == l0
+        for a, b in zip(g, g0):
+            assert np.array_equal(a, b)
+
+
+KEY_CHECK = """
+import sys
+sys.path.insert(0, %r)
+from __graft_entry__ import load_package
+pkg = load_package()
+H, W = pkg.hostapi, pkg.workloads
+host = H.Host()
+cases = [(W.c0_elementwise, dict(n=301, m=257)), (W.c1_fcnn, dict(batch=130)), (W.c3_cnn, dict(batch=6)), (W.c3_cnn, dict(batch=10)),
+         (W.c4_rnn, dict(batch=70)), (W.c4_rnn, dict(batch=4, steps=5, n_in=5, width=6, n_classes=3))]
+for mk, kw in cases:
+    wl = mk(**kw)
+    first = None
+    for rep in range(3):
+        ps, ds = wl.upload(host)
+        loss, grads = wl.gradient(host, ps, ds)
+        got = (float(loss.numpy()), [g.numpy().tobytes() for g in grads])
+        first = first or got
+        assert got == first, (wl.name, rep)
+print("ok")
+"""
+
+
+@pytest.mark.gpu
+def test_gpu_kernels_found_by_key_are_the_ones_their_text_gives():
+    """With HORDEAD_GPU_CHECK_KEYS set (read once per process, hence the child
+    process) every kernel found by its key has its text written anyway and compared
+    with the text kept under that key; a difference fails the call."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, HORDEAD_GPU_CHECK_KEYS="1")
+    r = subprocess.run([sys.executable, "-c", KEY_CHECK % root], env=env, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), (r.stdout[-500:], r.stderr[-2000:])
 
 
 @pytest.mark.gpu
