@@ -17,8 +17,8 @@ namespace fusedgen {
 
 // The text of a generated kernel, appended to piece by piece: the interface of
 // an output stream for text and integers, without a stream's locale and virtual
-// calls (the generators run on every call, and a call's kernel is looked up by
-// its text).
+// calls.  A compiled kernel is kept under its text; calls find it under a Key
+// (below) without writing the text again.
 struct Src {
   std::string text;
   bool on = true;   // false: the kernel is known already, nothing is written (the generator still runs: it also works out how to launch)
