@@ -119,6 +119,8 @@ struct Plan {
   bool cvec;   // groups of four rows are adjacent in C and 16-byte aligned: vector stores
 };
 
+// (a field added to Plan changes its size: it belongs in put_plan too)
+static_assert(sizeof(Plan) == 352, "put_plan must cover every field of Plan");
 void put_plan(hg::fusedgen::Key& k, const Plan& pl) {
   k.put(pl.f64).put(pl.mode).put(pl.nch).put(pl.chx).put(pl.chy).put(pl.chc).put(pl.min_rows).put(pl.nin);
   k.put(pl.row_x).put(pl.row_c).put(pl.col_y).put(pl.col_c).put(pl.gx).put(pl.gy).put(pl.gp);
@@ -832,6 +834,7 @@ bool vector_ok(const VirtualOp& v, int V) {
 }
 
 // Everything vops_source reads.
+static_assert(sizeof(VirtualOp) == 192, "put_virtual must cover every field of VirtualOp");
 void put_virtual(hg::fusedgen::Key& k, const VirtualOp& v, int V, int64_t chunk_stride, int64_t max_elem) {
   k.put(v.n_in).put(v.n_instr, v.prog).put(v.slot).put(v.dtype).put(v.dt).put(v.E).put(v.M).put(v.lo).put(v.hi).put(v.P).put(v.total).put(v.padded);
   for (int i = 0; i < v.n_in; ++i) {
@@ -1326,6 +1329,7 @@ struct EpiSpec {
   int val_off = 0, idx_off = 0, stage_bytes = 0;
 };
 
+static_assert(sizeof(EpiSpec) == 296, "put_epilogue must cover every field of EpiSpec");
 void put_epilogue(hg::fusedgen::Key& k, const EpiSpec& e) {
   k.put(e.n_in).put(e.c_slot).put(e.n_instr, e.prog).put(e.dt).put(e.cls).put(e.in_row).put(e.in_col).put(e.in_chs).put(e.out_slots);
   k.put(e.has_ext).put(e.want_max).put(e.ext_slot).put(e.L).put(e.win_row).put(e.win_col).put(e.win_chs).put(e.out_chs);

@@ -519,6 +519,7 @@ bool plan_chunks(Spec& sp) {
 }
 
 // Everything generate_body reads.
+static_assert(sizeof(Spec) == 224 && sizeof(Chunk) == 96 && sizeof(Term) == 56, "spec_key must cover every field of Spec, Chunk, Operand and Term");
 Key spec_key(const Spec& sp) {
   Key k;
   k.put(sp.f64).put(sp.P).put(sp.Q).put(sp.BP).put(sp.BQ).put(sp.WP).put(sp.WQ).put(sp.terms.size());
