@@ -2,6 +2,7 @@
 // view, dimension collapsing and launch helpers.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <atomic>
 #include <cstdarg>
@@ -237,10 +238,29 @@ struct LaunchGuard {
     }
   }
   ~LaunchGuard() {
-    if (timed) (void)hipEventRecord(ctx->prof.back().b, ctx->stream);
+    if (timed && !stop_carried) (void)hipEventRecord(ctx->prof.back().b, ctx->stream);
     ctx->launch_mu.unlock();
   }
+  // The guard's events for a launch that carries them itself (hipExtModuleLaunchKernel, hipExtLaunchKernel): they
+  // then hold the kernel's own begin and end, which is what a profiler's kernel trace reports.  Events recorded
+  // around a launch also time its dispatch and the cache write-back after it, 3-4 us more on this device.  The
+  // first launch under the guard takes start_event(), the last one stop_event(); both are null while nothing is timed.
+  bool stop_carried = false;
+  hipEvent_t start_event() { return timed ? ctx->prof.back().a : nullptr; }
+  hipEvent_t stop_event() {
+    if (!timed) return nullptr;
+    stop_carried = true;
+    return ctx->prof.back().b;
+  }
 };
+
+// Launch of a run-time compiled kernel under a guard: `first` / `last` say whether this is the first / last
+// launch the guard's record is to cover.
+inline hipError_t launch_module(LaunchGuard& lg, hipFunction_t fn, unsigned grid, unsigned block, void** args, bool first = true, bool last = true) {
+  if (!lg.timed || (uint64_t)grid * block > 0xffffffffull) return hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, 0, lg.ctx->stream, args, nullptr);
+  return hipExtModuleLaunchKernel(fn, grid * block, 1, 1, block, 1, 1, 0, lg.ctx->stream, args, nullptr, first ? lg.start_event() : nullptr,
+                                  last ? lg.stop_event() : nullptr, 0);
+}
 
 // A label with the lifetime of the context (profiling records keep the pointer).
 inline const char* intern_label(hgpu_ctx* c, const std::string& s) {

@@ -1279,7 +1279,7 @@ int try_footprint_virtual(hgpu_ctx* ctx, const GemmParams& p, int dtype, const v
     }
     {
       LaunchGuard lg(ctx, label, bytes, flops);
-      hipError_t e = hipModuleLaunchKernel(kernel.fn, (unsigned)grid, 1, 1, 256u * (unsigned)pl.ks, 1, 1, 0, ctx->stream, args.data(), nullptr);
+      hipError_t e = launch_module(lg, kernel.fn, (unsigned)grid, 256u * (unsigned)pl.ks, args.data());
       if (e != hipSuccess) { if (part) buffer_release(part); if (colsum) hgpu_release(colsum); return check_hip(ctx, e, "footprint gemm launch"); }
     }
     if (pl.mode == 0) {
@@ -1738,7 +1738,7 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
       label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, bytes, flops);
-    hipError_t err = hipModuleLaunchKernel(kernel.fn, (unsigned)grid, 1, 1, 256u * (unsigned)pl.ks, 1, 1, 0, ctx->stream, args, nullptr);
+    hipError_t err = launch_module(lg, kernel.fn, (unsigned)grid, 256u * (unsigned)pl.ks, args);
     if (err != hipSuccess) { release_all(); return check_hip(ctx, err, "contract_map launch"); }
   }
   for (int o = 0; o < n_out; ++o) outs[o] = res[(size_t)o];
@@ -2126,7 +2126,7 @@ int try_mapped_sum(hgpu_ctx* ctx, const VirtualOp& v, const hgpu_operand* o, int
       label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, bytes, (double)n_out * R * (v.n_instr + 1));
-    hipError_t e = hipModuleLaunchKernel(it->second.fn, (unsigned)(n_out * S), 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+    hipError_t e = launch_module(lg, it->second.fn, (unsigned)(n_out * S), 256, args);
     if (e != hipSuccess) { if (part) buffer_release(part); return check_hip(ctx, e, "mapped_sum launch"); }
   }
   if (part) {
@@ -2578,7 +2578,7 @@ int try_onehot_contract(hgpu_ctx* ctx, const hgpu_array* x, const VirtualOp& v, 
       label = intern_label(ctx, buf);
     }
     LaunchGuard lg(ctx, label, bytes, 2.0 * MR * NC * (double)G * (double)nch);
-    hipError_t e = hipModuleLaunchKernel(kn.c.fn, (unsigned)grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+    hipError_t e = launch_module(lg, kn.c.fn, (unsigned)grid, 256, args);
     if (e != hipSuccess) { buffer_release(part); hgpu_release(colsum); return check_hip(ctx, e, "onehot_contract launch"); }
   }
   rc = hg::sum_partials_split(ctx, v.dtype, out_n, NC, (int)grid, part->ptr, data_ptr(out), data_ptr(colsum));

@@ -456,7 +456,7 @@ static int fused_map_impl(hgpu_ctx* ctx, int n_in, const hgpu_array* const* in, 
     args.push_back(&part_ptr);
     grid = (unsigned)(dsC * ds_chunks);
   }
-  hipError_t e = hipModuleLaunchKernel(kernel.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  hipError_t e = launch_module(lg, kernel.fn, grid, 256, args.data());
   if (e != hipSuccess) { if (part) buffer_release(part); if (sums) hgpu_release(sums); release_all(); return check_hip(ctx, e, "fused_map launch"); }
   guard.reset();
   if (part) {
@@ -620,7 +620,7 @@ extern "C" int hgpu_fused_extremum(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   args.push_back(&pv);
   args.push_back(&pi);
   unsigned grid = grid_for(n_out, 256, ctx->num_cu * 16);
-  hipError_t e = hipModuleLaunchKernel(kernel.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  hipError_t e = launch_module(lg, kernel.fn, grid, 256, args.data());
   if (e != hipSuccess) { hgpu_release(v); hgpu_release(ix); return check_hip(ctx, e, "fused_extremum launch"); }
   *values = v;
   *indices = ix;
@@ -804,11 +804,11 @@ extern "C" int hgpu_fused_sum(hgpu_ctx* ctx, int n_in, const hgpu_array* const* 
   hipFunction_t fin = nullptr;
   hipError_t e = hipSuccess;
   if (!single && !ticketed) e = hipModuleGetFunction(&fin, kernel.mod, "fused_sum_final");
-  if (e == hipSuccess) e = hipModuleLaunchKernel(kernel.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e == hipSuccess) e = launch_module(lg, kernel.fn, grid, (unsigned)NT, args.data(), true, fin == nullptr);
   if (e == hipSuccess && fin) {
     int g = (int)grid;
     void* fargs[] = {&g, &pp, &po};
-    e = hipModuleLaunchKernel(fin, 1, 1, 1, 256, 1, 1, 0, ctx->stream, fargs, nullptr);
+    e = launch_module(lg, fin, 1, 256, fargs, false, true);
   }
   drop_part();
   if (e != hipSuccess) { hgpu_release(o); return check_hip(ctx, e, "fused_sum launch"); }
@@ -1028,12 +1028,12 @@ extern "C" int hgpu_fused_map_sums(hgpu_ctx* ctx, int n_in, const hgpu_array* co
   hipFunction_t fin = nullptr;
   hipError_t e = hipSuccess;
   if (!single && !ticketed) e = hipModuleGetFunction(&fin, kernel.mod, "fused_map_sums_final");
-  if (e == hipSuccess) e = hipModuleLaunchKernel(kernel.fn, grid, 1, 1, (unsigned)NT, 1, 1, 0, ctx->stream, args.data(), nullptr);
+  if (e == hipSuccess) e = launch_module(lg, kernel.fn, grid, (unsigned)NT, args.data(), true, fin == nullptr);
   if (e == hipSuccess && fin) {
     int g = (int)grid;
     std::vector<void*> fargs = {&g, &pp};
     for (int j = 0; j < n_sum; ++j) fargs.push_back(&sptrs[(size_t)j]);
-    e = hipModuleLaunchKernel(fin, (unsigned)n_sum, 1, 1, 256, 1, 1, 0, ctx->stream, fargs.data(), nullptr);
+    e = launch_module(lg, fin, (unsigned)n_sum, 256, fargs.data(), false, true);
   }
   drop_part();
   if (e != hipSuccess) { release_all(); return check_hip(ctx, e, "fused_map_sums launch"); }

@@ -263,6 +263,8 @@ int gemm_direct(hgpu_ctx* ctx, GemmParams p, int dtype, const void* pa, const vo
     LaunchArgs la{ctx->stream, -1, tm, tn, va, vb, grid, pa, pb, cdst, ka, kb};
     {
       LaunchGuard lg(ctx, label, bytes, flops);
+      la.ev_start = lg.start_event();
+      la.ev_stop = lg.stop_event();
       if (dtype == HGPU_F64) launch_f64(p, la);
       else launch_f32(p, la);
     }
@@ -581,6 +583,8 @@ int try_gemm(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, int n_keep
     LaunchArgs la{ctx->stream, cfg, 0, 0, va, vb, grid, data_ptr(a), data_ptr(b), cdst, ka, kb};
     {
       LaunchGuard lg(ctx, label, bytes, flops);
+      la.ev_start = lg.start_event();
+      la.ev_stop = lg.stop_event();
       if (a->dtype == HGPU_F64) launch_f64(p, la);
       else launch_f32(p, la);
     }

@@ -659,6 +659,7 @@ struct LaunchArgs {
   const void *A, *B;
   void* C;
   const int64_t *ka, *kb;
+  hipEvent_t ev_start = nullptr, ev_stop = nullptr;   // while the profiler is on: events that the launch carries (the kernel's own begin and end)
 };
 
 // Blocks that walk the terms of a sum themselves exist for tiles up to 64 x 64
@@ -667,6 +668,13 @@ constexpr bool term_loop_tile(int wgm, int wgn, int tm, int tn) { return wgm * t
 
 // The MFMA flavour a tile runs on: fp32 tiles whose wavefronts hold whole
 // 32 x 32 blocks take the 32x32x2 instruction.
+// One launch: plain, or carrying the profiler's events (then they hold the kernel's own begin and end).
+template <typename F, typename... Args>
+inline void launch_kernel(const LaunchArgs& a, F kernel, Args... args) {
+  if (a.ev_start || a.ev_stop) hipExtLaunchKernelGGL(kernel, a.grid, dim3(NT), 0, a.stream, a.ev_start, a.ev_stop, 0, args...);
+  else hipLaunchKernelGGL(kernel, a.grid, dim3(NT), 0, a.stream, args...);
+}
+
 template <typename X0, int TM, int TN> struct FlavourOf { using type = X0; };
 template <int TM, int TN> struct FlavourOf<MfmaF32, TM, TN> {
   using type = typename std::conditional<TM % 2 == 0 && TN % 2 == 0, MfmaF32W, MfmaF32>::type;
@@ -689,15 +697,15 @@ void launch_cfg(const GemmParams& p, const LaunchArgs& a) {
       constexpr bool CA = BM >= 64, CB = BN >= 64;
       const bool va = CA && a.va, vb = CB && a.vb;
       if constexpr (CA && CB) {
-        if (va && vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, V, 1, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+        if (va && vb) { launch_kernel(a, (k_gemm<X, WGM, WGN, TM, TN, V, V, 1, true>), p, A, B, C, a.ka, a.kb); return; }
       }
       if constexpr (CA) {
-        if (va) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, 1, 1, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+        if (va) { launch_kernel(a, (k_gemm<X, WGM, WGN, TM, TN, V, 1, 1, true>), p, A, B, C, a.ka, a.kb); return; }
       }
       if constexpr (CB) {
-        if (vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, V, 1, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+        if (vb) { launch_kernel(a, (k_gemm<X, WGM, WGN, TM, TN, 1, V, 1, true>), p, A, B, C, a.ka, a.kb); return; }
       }
-      hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, 1, 1, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+      launch_kernel(a, (k_gemm<X, WGM, WGN, TM, TN, 1, 1, 1, true>), p, A, B, C, a.ka, a.kb);
       return;
     }
   }
@@ -708,15 +716,15 @@ void launch_cfg(const GemmParams& p, const LaunchArgs& a) {
   constexpr bool CA = BM >= 64, CB = BN >= 64;
   const bool va = CA && a.va, vb = CB && a.vb;
   if constexpr (CA && CB) {
-    if (va && vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, V, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+    if (va && vb) { launch_kernel(a, (k_gemm<X, WGM, WGN, TM, TN, V, V, NBUF>), p, A, B, C, a.ka, a.kb); return; }
   }
   if constexpr (CA) {
-    if (va) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, V, 1, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+    if (va) { launch_kernel(a, (k_gemm<X, WGM, WGN, TM, TN, V, 1, NBUF>), p, A, B, C, a.ka, a.kb); return; }
   }
   if constexpr (CB) {
-    if (vb) { hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, V, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb); return; }
+    if (vb) { launch_kernel(a, (k_gemm<X, WGM, WGN, TM, TN, 1, V, NBUF>), p, A, B, C, a.ka, a.kb); return; }
   }
-  hipLaunchKernelGGL((k_gemm<X, WGM, WGN, TM, TN, 1, 1, NBUF>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+  launch_kernel(a, (k_gemm<X, WGM, WGN, TM, TN, 1, 1, NBUF>), p, A, B, C, a.ka, a.kb);
 }
 
 template <typename X, int TM, int TN>
@@ -725,10 +733,10 @@ void launch_direct_cfg(const GemmParams& p, const LaunchArgs& a) {
   const T* A = (const T*)a.A;
   const T* B = (const T*)a.B;
   T* C = (T*)a.C;
-  if (a.va && a.vb) hipLaunchKernelGGL((k_gemm_direct<X, TM, TN, true, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
-  else if (a.va) hipLaunchKernelGGL((k_gemm_direct<X, TM, TN, true, false>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
-  else if (a.vb) hipLaunchKernelGGL((k_gemm_direct<X, TM, TN, false, true>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
-  else hipLaunchKernelGGL((k_gemm_direct<X, TM, TN, false, false>), a.grid, dim3(NT), 0, a.stream, p, A, B, C, a.ka, a.kb);
+  if (a.va && a.vb) launch_kernel(a, (k_gemm_direct<X, TM, TN, true, true>), p, A, B, C, a.ka, a.kb);
+  else if (a.va) launch_kernel(a, (k_gemm_direct<X, TM, TN, true, false>), p, A, B, C, a.ka, a.kb);
+  else if (a.vb) launch_kernel(a, (k_gemm_direct<X, TM, TN, false, true>), p, A, B, C, a.ka, a.kb);
+  else launch_kernel(a, (k_gemm_direct<X, TM, TN, false, false>), p, A, B, C, a.ka, a.kb);
 }
 
 template <typename X>

@@ -788,8 +788,8 @@ int try_smallk(hgpu_ctx* ctx, int n_terms, const hgpu_array* const* as, const hg
   }
   LaunchGuard lg(ctx, d.label, d.bytes, d.flops);
   void* args[] = {(void*)d.args.data()};
-  hipError_t err = hipModuleLaunchKernel(d.fn, d.grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
-  if (err == hipSuccess && finish_fn) err = hipModuleLaunchKernel(finish_fn, (unsigned)((ntiles + 7) / 8 * 8), 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
+  hipError_t err = launch_module(lg, d.fn, d.grid, 256, args, true, finish_fn == nullptr);
+  if (err == hipSuccess && finish_fn) err = launch_module(lg, finish_fn, (unsigned)((ntiles + 7) / 8 * 8), 256, args, false, true);
   if (part) buffer_release(part);
   if (err != hipSuccess) return check_hip(ctx, err, "small-K product launch");
   *handled = true;
@@ -820,18 +820,19 @@ void flush_deferred_locked(hgpu_ctx* ctx) {
     top = std::max(top, d.level);
   }
   auto timed_launch = [&](hipFunction_t fn, unsigned grid, const std::vector<const void*>& ar, const char* label, double bytes, double flops) {
-    bool timed = false;
-    if (ctx->profiling && !ctx->cap) {
+    // (timed: the launch carries its record's two events, which then hold the kernel's own begin and end)
+    hipEvent_t ea = nullptr, eb = nullptr;
+    if (ctx->profiling && !ctx->cap && (uint64_t)grid * 256 <= 0xffffffffull) {
       hgpu_ctx::ProfRec r{label, nullptr, nullptr, bytes, flops};
       if (hipEventCreate(&r.a) == hipSuccess && hipEventCreate(&r.b) == hipSuccess) {
-        (void)hipEventRecord(r.a, ctx->stream);
         ctx->prof.push_back(r);
-        timed = true;
+        ea = r.a;
+        eb = r.b;
       }
     }
     void* args[] = {(void*)ar.data()};
-    hipError_t err = hipModuleLaunchKernel(fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
-    if (timed) (void)hipEventRecord(ctx->prof.back().b, ctx->stream);
+    hipError_t err = ea ? hipExtModuleLaunchKernel(fn, grid * 256, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr, ea, eb, 0)
+                        : hipModuleLaunchKernel(fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args, nullptr);
     if (err != hipSuccess) {
       int rc = check_hip(ctx, err, "small-K product launch");
       if (!ctx->deferred_rc) ctx->deferred_rc = rc;

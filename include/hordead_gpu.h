@@ -117,8 +117,11 @@ void* hgpu_stream(hgpu_ctx* ctx);
  * path); a negative value switches it off. */
 int hgpu_inject_alloc_failure(hgpu_ctx* ctx, int64_t limit);
 
-/* Per-launch timing for benchmarks: while enabled every kernel launch is
- * bracketed by a HIP event pair on the context's stream.  The report has one
+/* Per-launch timing for benchmarks: while enabled every kernel launch has a
+ * HIP event pair on the context's stream.  The run-time compiled kernels and
+ * the staged matrix products carry their pair (it holds the kernel's own begin
+ * and end); the other kernels are bracketed by theirs, which also times the
+ * dispatch (a few microseconds more per launch).  The report has one
  * line per kernel family: "name launches total_ms algorithmic_bytes
  * algorithmic_flops".  Enabling (or disabling) clears the records.  on = 2
  * makes the matrix-product labels carry the problem shape. */
