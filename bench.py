@@ -128,14 +128,19 @@ def time_train_graph(pkg, host, wl, steps, warmup):
         graph.free()
 
 
-def profile(capi, host, wl, ps, ds, reps=2):
+def profile(capi, host, wl, ps, ds, reps=10):
     """Per-launch HIP-event timing by the library, one label per kernel and
-    problem shape: {label: (launches, ms, bytes, flops)} per gradient."""
+    problem shape: {label: (launches, ms, bytes, flops)} per gradient.  The
+    gradients are submitted one after another without waiting in between, as
+    in the timed region (a device left idle between steps clocks down, and its
+    kernels then take a few per cent longer)."""
     actx = array_ctx(capi, host)
+    for _ in range(2):
+        wl.gradient(host, ps, ds)
     actx.check(actx.lib.profile_enable(actx.h, 2))
     for _ in range(reps):
         wl.gradient(host, ps, ds)
-        host.sync()
+    host.sync()
     rep = actx.profile_report()
     actx.check(actx.lib.profile_enable(actx.h, 0))
     return {k: (v[0] / reps, v[1] / reps, v[2] / reps, v[3] / reps) for k, v in rep.items()}
