@@ -390,6 +390,44 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   if constexpr (KH < KS) {
   constexpr int GA = NG * KH / KS, GB = NG * (KH + 1) / KS;        // this part's K groups
   constexpr bool kRemOwner = KH == KS - 1;                          // its wavefronts 0 .. REM - 1 finish the split row blocks
+  // j-th staging vector of this thread; the tail repeats the last vector.  The last vector of a footprint may reach up to
+  // VX - 1 elements past it: still inside the operand's block, which the allocator ends with 16 spare bytes.
+  auto vidx = [&](int j) -> int { int v = tid + NT * (j < NLX ? j : j - NLX); int lim = (j < NLX ? XV : YV) - 1; return v < lim ? v : lim; };
+  // The first chunk, and the columns operand of mode 1, go to LDS up to 32
+  // vectors at a time: the loads in flight together, then the stores.  Copied
+  // one by one, every vector would wait out its own trip to memory.  The first
+  // batch of each is asked for here, before the address tables below are looked
+  // up: the three trips to memory (tables, first chunk, columns operand) then
+  // run side by side instead of one after the other.
+  constexpr int kFill = NLD < 32 ? (NLD > 0 ? NLD : 1) : 32;
+#if VIRT_X
+  VPre_x vpx[NLX];
+#pragma unroll
+  for (int j = 0; j < NLX; ++j) vpx[j] = vpre_x(XBASE + (i64)vidx(j) * VX);
+#endif
+#if VIRT_Y
+  VPre_y vpy[NLY];
+#pragma unroll
+  for (int j = 0; j < NLY; ++j) vpy[j] = vpre_y(YBASE + (i64)vidx(NLX + j) * VY);
+#endif
+  i64 ch = blockIdx.x;
+  RawX fx0[kFill];
+  RawY fy0[kFill];
+  if (ch < nch) {
+#pragma unroll
+    for (int j = 0; j < kFill && j < NLD; ++j) {
+      if (j < NLX) fx0[j] = LOAD_X(ch, j);
+      else fy0[j] = LOAD_Y(ch, j);
+    }
+  }
+  Vec<VY> fyc0[MODE == 1 ? kFill : 1];
+  if (MODE == 1) {
+#pragma unroll
+    for (int u = 0; u < kFill; ++u) {
+      const int v = tid + NT * u;
+      fyc0[u] = reinterpret_cast<const Vec<VY>*>(Y)[v < YV ? v : YV - 1];
+    }
+  }
   // per-lane addresses: row base + lane offset of each K pattern
   int ax[NBF > 0 ? NBF : 1][NPAT];
 #pragma unroll
@@ -490,27 +528,15 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
     }
   };
 
-  // j-th staging vector of this thread; the tail repeats the last vector.  The last vector of a footprint may reach up to
-  // VX - 1 elements past it: still inside the operand's block, which the allocator ends with 16 spare bytes.
-  auto vidx = [&](int j) -> int { int v = tid + NT * (j < NLX ? j : j - NLX); int lim = (j < NLX ? XV : YV) - 1; return v < lim ? v : lim; };
-  // The first chunk, and the columns operand of mode 1, go to LDS up to 32
-  // vectors at a time: the loads in flight together, then the stores.  Copied
-  // one by one, every vector would wait out its own trip to memory.
-  constexpr int kFill = NLD < 32 ? (NLD > 0 ? NLD : 1) : 32;
-#if VIRT_X
-  VPre_x vpx[NLX];
-#pragma unroll
-  for (int j = 0; j < NLX; ++j) vpx[j] = vpre_x(XBASE + (i64)vidx(j) * VX);
-#endif
-#if VIRT_Y
-  VPre_y vpy[NLY];
-#pragma unroll
-  for (int j = 0; j < NLY; ++j) vpy[j] = vpre_y(YBASE + (i64)vidx(NLX + j) * VY);
-#endif
-  i64 ch = blockIdx.x;
+  // the first batches arrive in LDS; what is left of the first chunk and of the columns operand follows, a batch at a time
   if (ch < nch) {
 #pragma unroll
-    for (int j0 = 0; j0 < NLD; j0 += kFill) {
+    for (int j = 0; j < kFill && j < NLD; ++j) {
+      if (j < NLX) reinterpret_cast<Vec<VX>*>(lds)[vidx(j)] = FIN_X(j, fx0[j]);
+      else reinterpret_cast<Vec<VY>*>(lds + LX)[ypos(vidx(j))] = FIN_Y(j, fy0[j]);
+    }
+#pragma unroll
+    for (int j0 = kFill; j0 < NLD; j0 += kFill) {
       RawX fx[kFill];
       RawY fy[kFill];
 #pragma unroll
@@ -526,7 +552,12 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
     }
   }
   if (MODE == 1) {   // the columns operand does not change with the chunk
-    for (int v0 = tid; v0 < YV; v0 += NT * kFill) {
+#pragma unroll
+    for (int u = 0; u < kFill; ++u) {
+      const int v = tid + NT * u;
+      if (v < YV) reinterpret_cast<Vec<VY>*>(lds + NBUFS * BUF)[ypos(v)] = fyc0[u];
+    }
+    for (int v0 = tid + NT * kFill; v0 < YV; v0 += NT * kFill) {
       Vec<VY> fy[kFill];
 #pragma unroll
       for (int u = 0; u < kFill; ++u) {
