@@ -149,7 +149,7 @@ class Ctx:
         self.check(self.lib.profile_report(self.h, buf, len(buf)))
         out = {}
         for line in buf.value.decode().splitlines():
-            name, cnt, ms, by, fl = line.split()
+            name, cnt, ms, by, fl = line.rsplit(None, 4)   # (a label may hold blanks)
             out[name] = (int(cnt), float(ms), float(by), float(fl))
         return out
 
