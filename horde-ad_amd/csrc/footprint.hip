@@ -428,7 +428,19 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
       fyc0[u] = reinterpret_cast<const Vec<VY>*>(Y)[v < YV ? v : YV - 1];
     }
   }
-  // per-lane addresses: row base + lane offset of each K pattern
+  // per-lane addresses: row base + lane offset of each K pattern.  Two blocks on a CU (BPC 2) have half the
+  // registers each: the sums are then made where they are used, from NBF + NPAT registers instead of NBF * NPAT.
+#if BPC == 2
+  int axr[NBF > 0 ? NBF : 1], axp[NPAT];
+#pragma unroll
+  for (int t = 0; t < NBF; ++t) {
+    int m = (wave + 4 * t) * 16 + ROW_OF(r);
+    axr[t] = kRowX[m < MIN ? m : MIN - 1];
+  }
+#pragma unroll
+  for (int p = 0; p < NPAT; ++p) axp[p] = kPatX[p * 4 + q4];
+#define AX(t_, p_) (axr[t_] + axp[p_])
+#else
   int ax[NBF > 0 ? NBF : 1][NPAT];
 #pragma unroll
   for (int t = 0; t < NBF; ++t) {
@@ -437,6 +449,8 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
 #pragma unroll
     for (int p = 0; p < NPAT; ++p) ax[t][p] = ro + kPatX[p * 4 + q4];
   }
+#define AX(t_, p_) ax[t_][p_]
+#endif
   const int cn = r < NIN ? r : NIN - 1;
   int by[NPAT];
 #pragma unroll
@@ -462,11 +476,19 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
   const bool tail_lane = q4 >= KVALID;
 #if EPI
   // where a lane's rows and windows go, and the program inputs that do not change with the row
+#if BPC == 2
+  // (half the registers: the places are looked up when a chunk is finished, in copies of the tables in LDS --
+  // a lookup in memory would wait for every store issued before it)
+  epi_tables_to_lds(tid);
+#define EPOS(t_, m0_) epi_pos(m0_, r)
+#else
   EPos epos[NACC];
 #pragma unroll
   for (int t = 0; t < NBF; ++t)
     if (t % KS == KH) epos[t] = epi_pos((wave + 4 * t) * 16 + 4 * q4, r);     // row block t is finished by part t % KS
   if (REM > 0 && kRemOwner) epos[NBF] = epi_pos((4 * NBF + (wave < REM ? wave : 0)) * 16 + 4 * q4, r);
+#define EPOS(t_, m0_) epos[t_]
+#endif
   const Hoist hz = epi_hoist(ea, r < NIN ? r : NIN - 1);
 #else
   OutPos pos[MODE == 1 ? NACC : 1];
@@ -615,7 +637,7 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
 #endif
 #pragma unroll
           for (int t = 0; t < NBF; ++t) {
-            T av = L[ax[t][p] + gx];
+            T av = L[AX(t, p) + gx];
             if (tail && tail_lane) av = T(0);
             acc[t] = MFMA(av, bv, acc[t]);
           }
@@ -733,8 +755,8 @@ KNAME(const T* __restrict__ X, const T* __restrict__ Y, T* __restrict__ C, i64 n
 #if EPI
 #pragma unroll
       for (int t = 0; t < NBF; ++t)
-        if (t % KS == KH) epi_tile(ea, hz, epos[t], stage, ch, (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
-      if (REM > 0 && kRemOwner && wave < REM) epi_tile(ea, hz, epos[NBF], stage, ch, (4 * NBF + wave) * 16 + 4 * q4, r, srem[0], srem[1], srem[2], srem[3]);
+        if (t % KS == KH) epi_tile(ea, hz, EPOS(t, (wave + 4 * t) * 16 + 4 * q4), stage, ch, (wave + 4 * t) * 16 + 4 * q4, r, acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      if (REM > 0 && kRemOwner && wave < REM) epi_tile(ea, hz, EPOS(NBF, (4 * NBF + wave) * 16 + 4 * q4), stage, ch, (4 * NBF + wave) * 16 + 4 * q4, r, srem[0], srem[1], srem[2], srem[3]);
 #else
       T* out = C + ch * chc;
 #pragma unroll
@@ -1397,15 +1419,23 @@ std::string epilogue_source(const Plan& pl, const EpiSpec& e) {
   for (int i = 0; i < e.n_in; ++i)
     if (e.cls[(size_t)i] == 'g') s << "  int g" << i << "[4];\n";
   s << "};\n";
+  // Two blocks on a CU: the tables epi_pos reads are copied to LDS when the block starts (E_ROWC ... name the copies).
+  s << "#if BPC == 2\n__shared__ int sRowC[MIN], sColC[NIN];\n";
+  if (e.has_ext) s << "__shared__ int sWinO[MIN / " << e.L << "], sColO[NIN];\n";
+  s << "__device__ __forceinline__ void epi_tables_to_lds(int tid) {\n";
+  s << "  for (int i = tid; i < MIN; i += NT) sRowC[i] = kRowC[i];\n  if (tid < NIN) sColC[tid] = kColC[tid];\n";
+  if (e.has_ext) s << "  for (int i = tid; i < MIN / " << e.L << "; i += NT) sWinO[i] = kWinO[i];\n  if (tid < NIN) sColO[tid] = kColO[tid];\n";
+  s << "}\n#define E_ROWC sRowC\n#define E_COLC sColC\n#define E_WINO sWinO\n#define E_COLO sColO\n";
+  s << "#else\n#define E_ROWC kRowC\n#define E_COLC kColC\n#define E_WINO kWinO\n#define E_COLO kColO\n#endif\n";
   s << "__device__ __forceinline__ EPos epi_pos(int m0, int col) {\n  EPos p;\n";
   s << "  const int cc = col < NIN ? col : NIN - 1;\n";
   s << "#pragma unroll\n  for (int j = 0; j < 4; ++j) {\n    const int m = m0 + j < MIN ? m0 + j : MIN - 1;\n";
-  s << "    p.o[j] = kRowC[m] + kColC[cc];\n";
+  s << "    p.o[j] = E_ROWC[m] + E_COLC[cc];\n";
   for (int i = 0; i < e.n_in; ++i)
     if (e.cls[(size_t)i] == 'g') s << "    p.g" << i << "[j] = kRowI" << i << "[m] + kColI" << i << "[cc];\n";
   s << "  }\n";
   s << "#pragma unroll\n  for (int w = 0; w < " << WPL << "; ++w) {\n";
-  if (e.has_ext) s << "    const int wi = m0 / " << e.L << " + w;\n    p.w[w] = kWinO[wi < MIN / " << e.L << " ? wi : MIN / " << e.L << " - 1] + kColO[cc];\n";
+  if (e.has_ext) s << "    const int wi = m0 / " << e.L << " + w;\n    p.w[w] = E_WINO[wi < MIN / " << e.L << " ? wi : MIN / " << e.L << " - 1] + E_COLO[cc];\n";
   else s << "    p.w[w] = 0;\n";
   s << "  }\n  return p;\n}\n";
   s << "__device__ __forceinline__ void epi_tile(const EpiArgs& ea, const Hoist& hz, const EPos& ep, unsigned char* stage, i64 ch, int m0, int col, T c0, T c1, T c2, T c3) {\n";
@@ -1710,8 +1740,15 @@ int try_contract_map(hgpu_ctx* ctx, const hgpu_array* a, const hgpu_array* b, in
   }
   // For measurements (HORDEAD_FOOTPRINT_BPC=2): two blocks to a CU when their LDS fits together.  The first
   // CNN layer (784 rows x 16 x K 25 per chunk) runs 40 us that way against 34 us with one block per CU.
+  // Two blocks on a CU where their LDS fits twice (with the copies of the epilogue's tables) and no input of the
+  // program is looked up per row: one block's loads, stores and program then run under the other's multiplications.
+  // (HORDEAD_FOOTPRINT_BPC=1: one block per CU.)
   static const int bpc_env = getenv("HORDEAD_FOOTPRINT_BPC") ? atoi(getenv("HORDEAD_FOOTPRINT_BPC")) : 0;
-  pl.bpc = (pl.ks == 1 && 2 * (lds_bytes(pl) + e.stage_bytes + 512) <= 160 * 1024 && pl.nch >= 3 * (int64_t)ctx->num_cu && bpc_env == 2) ? 2 : 1;
+  bool rows_looked_up = false;
+  for (char c : e.cls) rows_looked_up = rows_looked_up || c == 'g';
+  const int64_t tables_lds = 4 * ((int64_t)pl.min_rows + pl.nin + (e.has_ext ? pl.min_rows / e.L + pl.nin : 0));
+  pl.bpc = (pl.ks == 1 && e.staged && !rows_looked_up && 2 * (lds_bytes(pl) + e.stage_bytes + tables_lds + 512) <= 160 * 1024 &&
+            pl.nch >= 3 * (int64_t)ctx->num_cu && bpc_env != 1) ? 2 : 1;
 
   // ---- results
   std::vector<hgpu_array*> res((size_t)n_out, nullptr);
